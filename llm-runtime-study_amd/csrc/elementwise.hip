@@ -1,0 +1,220 @@
+// Memory-bound parts of the step: embedding gather, RMSNorm, rotary tables, the fused
+// per-head q/k norm + rotation + cache write, and the gated activation.
+// The residual stream is float32 in every precision mode; `T` below is the dtype of
+// weights and activations (float or bf16).  All statistics are computed in float32.
+#include "common.h"
+
+// ------------------------------------------------------------------ embedding
+template <typename T>
+__global__ void embed_kernel(float* __restrict__ out, const T* __restrict__ table,
+                             const int* __restrict__ ids, int hidden, float multiplier) {
+  const int64_t row = ids[blockIdx.x];
+  const T* src = table + row * hidden;
+  float* dst = out + (int64_t)blockIdx.x * hidden;
+  for (int i = threadIdx.x; i < hidden; i += blockDim.x) dst[i] = to_float(src[i]) * multiplier;
+}
+
+LRS_API int lrs_embed(float* out, const void* table, int dtype, const int* ids, int tokens,
+                      int hidden, float multiplier, void* stream) {
+  LRS_REQUIRE(tokens > 0 && hidden > 0, "embed: tokens=%d hidden=%d must be positive", tokens, hidden);
+  dim3 grid(tokens), block(256);
+  if (dtype == LRS_F32)
+    embed_kernel<float><<<grid, block, 0, (hipStream_t)stream>>>(out, (const float*)table, ids, hidden, multiplier);
+  else if (dtype == LRS_BF16)
+    embed_kernel<bf16><<<grid, block, 0, (hipStream_t)stream>>>(out, (const bf16*)table, ids, hidden, multiplier);
+  else
+    return lrs_fail("embed: unknown dtype %d", dtype);
+  return lrs_check_launch("embed");
+}
+
+// -------------------------------------------------------------------- RMSNorm
+// y = w * x * rsqrt(mean(x^2) + eps); x is a float32 row (optionally picked through `rows`),
+// the result is rounded once to the output dtype.
+template <typename TW, typename TO>
+__global__ void rmsnorm_kernel(TO* __restrict__ out, const float* __restrict__ x,
+                               const TW* __restrict__ weight, const int* __restrict__ rows,
+                               int hidden, float eps) {
+  __shared__ float scratch[16];
+  const int64_t src_row = rows ? rows[blockIdx.x] : blockIdx.x;
+  const float* src = x + src_row * hidden;
+  TO* dst = out + (int64_t)blockIdx.x * hidden;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
+    const float v = src[i];
+    ss += v * v;
+  }
+  ss = block_sum(ss, scratch);
+  const float inv = 1.0f / sqrtf(ss / (float)hidden + eps);
+  for (int i = threadIdx.x; i < hidden; i += blockDim.x)
+    dst[i] = from_float<TO>(to_float(weight[i]) * (src[i] * inv));
+}
+
+LRS_API int lrs_rmsnorm(void* out, int out_dtype, const float* x, const void* weight, int w_dtype,
+                        const int* rows, int n_rows, int hidden, float eps, void* stream) {
+  LRS_REQUIRE(n_rows > 0 && hidden > 0, "rmsnorm: rows=%d hidden=%d must be positive", n_rows, hidden);
+  LRS_REQUIRE(eps > 0.f, "rmsnorm: eps must be positive");
+  dim3 grid(n_rows), block(hidden >= 2048 ? 512 : 256);
+  hipStream_t s = (hipStream_t)stream;
+#define LAUNCH(TW, TO) \
+  rmsnorm_kernel<TW, TO><<<grid, block, 0, s>>>((TO*)out, x, (const TW*)weight, rows, hidden, eps)
+  if (w_dtype == LRS_F32 && out_dtype == LRS_F32) LAUNCH(float, float);
+  else if (w_dtype == LRS_BF16 && out_dtype == LRS_BF16) LAUNCH(bf16, bf16);
+  else if (w_dtype == LRS_F32 && out_dtype == LRS_BF16) LAUNCH(float, bf16);
+  else if (w_dtype == LRS_BF16 && out_dtype == LRS_F32) LAUNCH(bf16, float);
+  else return lrs_fail("rmsnorm: unknown dtypes %d/%d", w_dtype, out_dtype);
+#undef LAUNCH
+  return lrs_check_launch("rmsnorm");
+}
+
+// ------------------------------------------------------------- rotary tables
+// cos/sin [tokens, half] of angle = float(position) * inv_freq[i], all in float32.
+__global__ void rope_table_kernel(float* __restrict__ cosv, float* __restrict__ sinv,
+                                  const int* __restrict__ positions,
+                                  const float* __restrict__ inv_freq, int half) {
+  const float p = (float)positions[blockIdx.x];
+  for (int i = threadIdx.x; i < half; i += blockDim.x) {
+    const float angle = p * inv_freq[i];
+    cosv[(int64_t)blockIdx.x * half + i] = cosf(angle);
+    sinv[(int64_t)blockIdx.x * half + i] = sinf(angle);
+  }
+}
+
+LRS_API int lrs_rope_table(float* cosv, float* sinv, const int* positions, const float* inv_freq,
+                           int tokens, int half, void* stream) {
+  LRS_REQUIRE(tokens > 0 && half > 0, "rope_table: tokens=%d half=%d must be positive", tokens, half);
+  rope_table_kernel<<<dim3(tokens), dim3(64), 0, (hipStream_t)stream>>>(cosv, sinv, positions, inv_freq, half);
+  return lrs_check_launch("rope_table");
+}
+
+// ------------------------------------- per-head norm + rotation + cache write
+// One wave per (token, head) of the fused projection row [q heads | k heads | v heads].
+// q heads: optional RMSNorm over head_dim, optional half-split rotation of the first
+// 2*rot_half dims, written back in place.  k heads: the same, written into the paged key
+// cache; v heads: copied into the paged value cache.  Pages are [page, kv_head, slot, dim];
+// `slots[t]` is page * page_size + offset of token t (negative: do not store).
+template <typename T, typename TW>
+__global__ void qk_prep_kernel(T* __restrict__ qkv, int row_stride, int nq, int nkv, int d,
+                               const TW* __restrict__ q_weight, const TW* __restrict__ k_weight,
+                               float eps, const float* __restrict__ cosv,
+                               const float* __restrict__ sinv, int rot_half,
+                               T* __restrict__ k_pages, T* __restrict__ v_pages,
+                               const int* __restrict__ slots, int page_size) {
+  const int token = blockIdx.x, head = blockIdx.y, lane = threadIdx.x;
+  T* src = qkv + (int64_t)token * row_stride + (int64_t)head * d;
+  const bool is_q = head < nq, is_k = !is_q && head < nq + nkv;
+  T* dst = src;
+  if (!is_q) {
+    const int slot = slots[token];
+    if (slot < 0) return;
+    const int kv_head = is_k ? head - nq : head - nq - nkv;
+    const int64_t page = slot / page_size, off = slot % page_size;
+    dst = (is_k ? k_pages : v_pages) + ((page * nkv + kv_head) * page_size + off) * d;
+    if (!is_k) {
+      for (int i = lane; i < d; i += WAVE) dst[i] = src[i];
+      return;
+    }
+  }
+  const TW* weight = is_q ? q_weight : k_weight;
+  float inv = 1.f;
+  if (weight) {
+    float ss = 0.f;
+    for (int i = lane; i < d; i += WAVE) {
+      const float v = to_float(src[i]);
+      ss += v * v;
+    }
+    ss = wave_sum(ss);
+    inv = 1.0f / sqrtf(ss / (float)d + eps);
+  }
+  // pairs (i, i + rot_half) rotate together; dims >= 2*rot_half pass through
+  for (int i = lane; i < rot_half; i += WAVE) {
+    float a = to_float(src[i]) * inv, b = to_float(src[i + rot_half]) * inv;
+    if (weight) {
+      a *= to_float(weight[i]);
+      b *= to_float(weight[i + rot_half]);
+    }
+    const float c = cosv[(int64_t)token * rot_half + i], s = sinv[(int64_t)token * rot_half + i];
+    dst[i] = from_float<T>(a * c - b * s);
+    dst[i + rot_half] = from_float<T>(b * c + a * s);
+  }
+  for (int i = 2 * rot_half + lane; i < d; i += WAVE) {
+    float a = to_float(src[i]) * inv;
+    if (weight) a *= to_float(weight[i]);
+    dst[i] = from_float<T>(a);
+  }
+}
+
+LRS_API int lrs_qk_prep(void* qkv, int dtype, int tokens, int row_stride, int nq, int nkv, int d,
+                        const void* q_weight, const void* k_weight, int w_dtype, float eps,
+                        const float* cosv, const float* sinv, int rot_half, void* k_pages,
+                        void* v_pages, const int* slots, int page_size, void* stream) {
+  LRS_REQUIRE(tokens > 0 && nq > 0 && nkv >= 0 && d > 0, "qk_prep: bad sizes tokens=%d nq=%d nkv=%d d=%d", tokens, nq, nkv, d);
+  LRS_REQUIRE(rot_half >= 0 && 2 * rot_half <= d, "qk_prep: rotary width %d exceeds head_dim %d", 2 * rot_half, d);
+  LRS_REQUIRE(rot_half == 0 || (cosv && sinv), "qk_prep: rotation asked for without tables");
+  LRS_REQUIRE((q_weight == nullptr) == (k_weight == nullptr), "qk_prep: q and k norm weights must come together");
+  LRS_REQUIRE(nkv == 0 || (k_pages && v_pages && slots && page_size > 0), "qk_prep: cache write needs pages, slots and a page size");
+  LRS_REQUIRE(row_stride >= (nq + 2 * nkv) * d, "qk_prep: row stride %d too small", row_stride);
+  dim3 grid(tokens, nq + 2 * nkv), block(WAVE);
+  hipStream_t s = (hipStream_t)stream;
+#define LAUNCH(T, TW)                                                                          \
+  qk_prep_kernel<T, TW><<<grid, block, 0, s>>>((T*)qkv, row_stride, nq, nkv, d, (const TW*)q_weight, \
+                                               (const TW*)k_weight, eps, cosv, sinv, rot_half,  \
+                                               (T*)k_pages, (T*)v_pages, slots, page_size)
+  if (dtype == LRS_F32 && w_dtype == LRS_F32) LAUNCH(float, float);
+  else if (dtype == LRS_BF16 && w_dtype == LRS_BF16) LAUNCH(bf16, bf16);
+  else if (dtype == LRS_BF16 && w_dtype == LRS_F32) LAUNCH(bf16, float);
+  else if (dtype == LRS_F32 && w_dtype == LRS_BF16) LAUNCH(float, bf16);
+  else return lrs_fail("qk_prep: unknown dtypes %d/%d", dtype, w_dtype);
+#undef LAUNCH
+  return lrs_check_launch("qk_prep");
+}
+
+// ----------------------------------------------------------- gated activation
+// out[t, i] = silu(gu[t, i]) * gu[t, inter + i], silu evaluated in float32.
+template <typename T>
+__global__ void silu_mul_kernel(T* __restrict__ out, const T* __restrict__ gu, int inter, int64_t total) {
+  for (int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total;
+       idx += (int64_t)gridDim.x * blockDim.x) {
+    const int64_t t = idx / inter, i = idx % inter;
+    const float g = to_float(gu[t * 2 * inter + i]);
+    const float u = to_float(gu[t * 2 * inter + inter + i]);
+    out[idx] = from_float<T>(g / (1.0f + expf(-g)) * u);
+  }
+}
+
+LRS_API int lrs_silu_mul(void* out, const void* gu, int dtype, int tokens, int inter, void* stream) {
+  LRS_REQUIRE(tokens > 0 && inter > 0, "silu_mul: tokens=%d inter=%d must be positive", tokens, inter);
+  const int64_t total = (int64_t)tokens * inter;
+  const int blocks = (int)((total + 255) / 256 < 65536 ? (total + 255) / 256 : 65536);
+  hipStream_t s = (hipStream_t)stream;
+  if (dtype == LRS_F32)
+    silu_mul_kernel<float><<<blocks, 256, 0, s>>>((float*)out, (const float*)gu, inter, total);
+  else if (dtype == LRS_BF16)
+    silu_mul_kernel<bf16><<<blocks, 256, 0, s>>>((bf16*)out, (const bf16*)gu, inter, total);
+  else
+    return lrs_fail("silu_mul: unknown dtype %d", dtype);
+  return lrs_check_launch("silu_mul");
+}
+
+// ------------------------------------------------------------------ utilities
+__global__ void fill_i32_kernel(int* dst, int value, int64_t n) {
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x)
+    dst[i] = value;
+}
+LRS_API int lrs_fill_i32(int* dst, int value, int64_t n, void* stream) {
+  LRS_REQUIRE(n > 0, "fill: n must be positive");
+  const int blocks = (int)((n + 255) / 256 < 4096 ? (n + 255) / 256 : 4096);
+  fill_i32_kernel<<<blocks, 256, 0, (hipStream_t)stream>>>(dst, value, n);
+  return lrs_check_launch("fill_i32");
+}
+
+// Copies picked float32 rows: out[i] = x[rows[i]].
+__global__ void gather_rows_kernel(float* __restrict__ out, const float* __restrict__ x,
+                                   const int* __restrict__ rows, int hidden) {
+  const float* src = x + (int64_t)rows[blockIdx.x] * hidden;
+  for (int i = threadIdx.x; i < hidden; i += blockDim.x) out[(int64_t)blockIdx.x * hidden + i] = src[i];
+}
+LRS_API int lrs_gather_rows(float* out, const float* x, const int* rows, int n_rows, int hidden, void* stream) {
+  LRS_REQUIRE(n_rows > 0 && hidden > 0, "gather_rows: bad sizes");
+  gather_rows_kernel<<<n_rows, 256, 0, (hipStream_t)stream>>>(out, x, rows, hidden);
+  return lrs_check_launch("gather_rows");
+}

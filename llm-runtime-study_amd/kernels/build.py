@@ -1,0 +1,106 @@
+"""Compiles the HIP sources under csrc/ into one shared library for gfx950.
+
+The library is kept inside the package folder next to a file holding the hash of the
+sources it was built from.  `ensure_built()` compiles only when no library matching
+the sources exists, printing a line as each file starts and finishes, so that a first
+call in a fresh checkout shows progress.  Files are compiled in parallel.
+"""
+
+from __future__ import annotations
+
+import hashlib
+import os
+import shutil
+import subprocess
+import sys
+import time
+from concurrent.futures import ThreadPoolExecutor
+from pathlib import Path
+
+PACKAGE_DIR = Path(__file__).resolve().parent.parent
+SOURCE_DIR = PACKAGE_DIR / "csrc"
+LIBRARY = Path(__file__).resolve().parent / "liblrs_kernels.so"
+HASH_FILE = LIBRARY.with_suffix(".so.hash")
+ARCH = "gfx950"
+# -packed-fp32-ops: keep the compiler from forming packed float32 instructions.
+DEVICE_FLAGS = ["-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
+FLAGS = [f"--offload-arch={ARCH}", "-O3", "-std=c++17", "-fPIC", "-fvisibility=hidden", "-Wno-unused-command-line-argument"] + DEVICE_FLAGS
+
+
+class BuildError(RuntimeError):
+    """Raised when the kernel library cannot be compiled."""
+
+
+def sources() -> list[Path]:
+    return sorted(SOURCE_DIR.glob("*.hip"))
+
+
+def source_hash() -> str:
+    digest = hashlib.sha256()
+    for path in sorted(SOURCE_DIR.glob("*.hip")) + sorted(SOURCE_DIR.glob("*.h")):
+        digest.update(path.name.encode())
+        digest.update(path.read_bytes())
+    digest.update(" ".join(FLAGS).encode())
+    return digest.hexdigest()
+
+
+def is_current() -> bool:
+    return LIBRARY.is_file() and HASH_FILE.is_file() and HASH_FILE.read_text().strip() == source_hash()
+
+
+def _hipcc() -> str:
+    found = shutil.which("hipcc") or ("/opt/rocm/bin/hipcc" if os.path.exists("/opt/rocm/bin/hipcc") else None)
+    if found is None:
+        raise BuildError("hipcc was not found: the kernel library cannot be built")
+    return found
+
+
+def _say(message: str) -> None:
+    print(f"[kernels] {message}", file=sys.stderr, flush=True)
+
+
+def _compile_one(hipcc: str, src: Path, obj: Path) -> None:
+    _say(f"compiling {src.name} ...")
+    started = time.time()
+    proc = subprocess.run([hipcc, *FLAGS, "-c", str(src), "-o", str(obj)], capture_output=True, text=True)
+    if proc.returncode != 0:
+        raise BuildError(f"hipcc failed on {src.name}:\n{proc.stderr}")
+    _say(f"compiled {src.name} in {time.time() - started:.1f} s")
+
+
+def build(force: bool = True) -> Path:
+    """Compile every source and link the library; returns its path."""
+    if not force and is_current():
+        return LIBRARY
+    hipcc = _hipcc()
+    build_dir = SOURCE_DIR / "_build"
+    build_dir.mkdir(exist_ok=True)
+    srcs = sources()
+    if not srcs:
+        raise BuildError(f"no HIP sources under {SOURCE_DIR}")
+    objects = [build_dir / (src.stem + ".o") for src in srcs]
+    started = time.time()
+    workers = max(1, min(len(srcs), int(os.environ.get("MAX_JOBS", os.cpu_count() or 4)), 16))
+    with ThreadPoolExecutor(max_workers=workers) as pool:
+        for future in [pool.submit(_compile_one, hipcc, s, o) for s, o in zip(srcs, objects)]:
+            future.result()
+    tmp = LIBRARY.with_suffix(f".so.tmp{os.getpid()}")
+    proc = subprocess.run(
+        [hipcc, f"--offload-arch={ARCH}", "-shared", "-fPIC", *map(str, objects), "-o", str(tmp)],
+        capture_output=True, text=True,
+    )
+    if proc.returncode != 0:
+        raise BuildError(f"linking the kernel library failed:\n{proc.stderr}")
+    os.replace(tmp, LIBRARY)
+    HASH_FILE.write_text(source_hash() + "\n")
+    _say(f"built {LIBRARY.name} in {time.time() - started:.1f} s")
+    return LIBRARY
+
+
+def ensure_built() -> Path:
+    """Return the library, compiling it first if none matches the sources."""
+    return build(force=False)
+
+
+if __name__ == "__main__":
+    build(force=True)

@@ -1,0 +1,277 @@
+"""Python face of the gfx950 kernel library.
+
+Every function checks on the host that the operand shapes, dtypes and strides are what
+its kernel assumes, then launches on the current torch stream.  Nothing here computes
+with torch: tensors are only containers of device memory.  Loading fails loudly when
+the library is missing or cannot be built; there is no fallback.
+"""
+
+from __future__ import annotations
+
+import ctypes
+from ctypes import c_char_p, c_float, c_int, c_int64, c_void_p, POINTER, byref
+
+import torch
+
+from ..errors import KernelError
+from . import build as _build
+
+_lib = None
+
+F32, BF16 = 0, 1
+OUT_STORE, OUT_STORE_F32, OUT_ADD_F32 = 0, 1, 2
+
+_SIGNATURES = {
+    "lrs_last_error": (c_char_p, []),
+    "lrs_device_arch": (c_int, [c_int, c_char_p, c_int, POINTER(c_int)]),
+    "lrs_graph_begin": (c_int, [c_void_p]),
+    "lrs_graph_end": (c_int, [c_void_p, POINTER(c_void_p)]),
+    "lrs_graph_launch": (c_int, [c_void_p, c_void_p]),
+    "lrs_graph_destroy": (c_int, [c_void_p]),
+    "lrs_copy_h2d": (c_int, [c_void_p, c_void_p, c_int64, c_void_p]),
+    "lrs_embed": (c_int, [c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_float, c_void_p]),
+    "lrs_rmsnorm": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_float, c_void_p]),
+    "lrs_rope_table": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p]),
+    "lrs_qk_prep": (c_int, [c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_int, c_float,
+                            c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p]),
+    "lrs_silu_mul": (c_int, [c_void_p, c_void_p, c_int, c_int, c_int, c_void_p]),
+    "lrs_fill_i32": (c_int, [c_void_p, c_int, c_int64, c_void_p]),
+    "lrs_gather_rows": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p]),
+    "lrs_gemm": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p]),
+    "lrs_attention": (c_int, [c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p,
+                              c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_void_p]),
+    "lrs_choose_tokens": (c_int, [c_void_p, c_void_p, c_int64, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p]),
+    "lrs_filter_logits": (c_int, [c_void_p, c_int64, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p]),
+}
+
+
+def library():
+    """Load (building first if needed) the kernel library; raises KernelError if impossible."""
+    global _lib
+    if _lib is None:
+        try:
+            path = _build.ensure_built()
+            lib = ctypes.CDLL(str(path))
+        except (_build.BuildError, OSError) as exc:
+            raise KernelError(f"the HIP kernel library is not available: {exc}") from exc
+        for name, (restype, argtypes) in _SIGNATURES.items():
+            fn = getattr(lib, name)
+            fn.restype, fn.argtypes = restype, argtypes
+        _lib = lib
+    return _lib
+
+
+def loaded_library_path() -> str:
+    library()
+    return str(_build.LIBRARY)
+
+
+def _check(code: int) -> None:
+    if code != 0:
+        raise KernelError(library().lrs_last_error().decode())
+
+
+def _stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def dtype_code(dtype: torch.dtype) -> int:
+    if dtype == torch.float32:
+        return F32
+    if dtype == torch.bfloat16:
+        return BF16
+    raise KernelError(f"kernels take float32 or bfloat16, got {dtype}")
+
+
+def _need(cond: bool, message: str) -> None:
+    if not cond:
+        raise KernelError(message)
+
+
+def _dev(t: torch.Tensor, name: str, dtype=None) -> int:
+    _need(isinstance(t, torch.Tensor) and t.is_cuda, f"{name} must be a device tensor")
+    if dtype is not None:
+        _need(t.dtype == dtype, f"{name} must be {dtype}, got {t.dtype}")
+    return t.data_ptr()
+
+
+def _rows(t: torch.Tensor, name: str) -> int:
+    """Row stride of a 2-D tensor whose rows are contiguous."""
+    _need(t.dim() == 2 and t.stride(1) == 1, f"{name} must be 2-D with contiguous rows, got shape {tuple(t.shape)} strides {t.stride()}")
+    return t.stride(0)
+
+
+def device_arch(device: int = 0) -> tuple[str, int]:
+    buf = ctypes.create_string_buffer(256)
+    cus = c_int(0)
+    _check(library().lrs_device_arch(device, buf, 256, byref(cus)))
+    return buf.value.decode(), cus.value
+
+
+# ----------------------------------------------------------------- graphs
+def graph_begin() -> None:
+    _check(library().lrs_graph_begin(_stream()))
+
+
+def graph_end() -> int:
+    handle = c_void_p()
+    _check(library().lrs_graph_end(_stream(), byref(handle)))
+    return handle.value
+
+
+def graph_launch(handle: int) -> None:
+    _check(library().lrs_graph_launch(handle, _stream()))
+
+
+def graph_destroy(handle: int) -> None:
+    library().lrs_graph_destroy(handle)
+
+
+def copy_h2d(dst: torch.Tensor, src: torch.Tensor, count: int) -> None:
+    """Asynchronous copy of the first `count` elements of pinned `src` into device `dst`."""
+    _need(src.is_pinned() and src.is_contiguous() and dst.is_contiguous(), "copy_h2d needs pinned contiguous source and contiguous destination")
+    _need(src.dtype == dst.dtype and 0 < count <= src.numel() and count <= dst.numel(), "copy_h2d: size or dtype mismatch")
+    _check(library().lrs_copy_h2d(_dev(dst, "dst"), src.data_ptr(), count * src.element_size(), _stream()))
+
+
+# ------------------------------------------------------------ elementwise
+def embed(out: torch.Tensor, table: torch.Tensor, ids: torch.Tensor, multiplier: float = 1.0) -> None:
+    tokens, hidden = out.shape
+    _need(out.is_contiguous() and table.is_contiguous() and table.dim() == 2 and table.shape[1] == hidden, "embed: out [T,H] and table [V,H] must agree")
+    _need(ids.dtype == torch.int32 and ids.numel() >= tokens and ids.is_contiguous(), "embed: ids must be int32 [T]")
+    _check(library().lrs_embed(_dev(out, "out", torch.float32), _dev(table, "table"), dtype_code(table.dtype),
+                               _dev(ids, "ids"), tokens, hidden, multiplier, _stream()))
+
+
+def rmsnorm(out: torch.Tensor, x: torch.Tensor, weight: torch.Tensor, eps: float, rows: torch.Tensor | None = None) -> None:
+    n_rows, hidden = out.shape
+    _need(out.is_contiguous() and x.is_contiguous() and x.dim() == 2 and x.shape[1] == hidden, "rmsnorm: out and x must be contiguous [*, H]")
+    _need(weight.is_contiguous() and weight.numel() == hidden, f"rmsnorm: weight must hold {hidden} values")
+    if rows is None:
+        _need(x.shape[0] >= n_rows, "rmsnorm: x has fewer rows than out")
+    else:
+        _need(rows.dtype == torch.int32 and rows.numel() >= n_rows and rows.is_contiguous(), "rmsnorm: rows must be int32")
+    _check(library().lrs_rmsnorm(_dev(out, "out"), dtype_code(out.dtype), _dev(x, "x", torch.float32), _dev(weight, "weight"),
+                                 dtype_code(weight.dtype), None if rows is None else _dev(rows, "rows"), n_rows, hidden, eps, _stream()))
+
+
+def rope_table(cos: torch.Tensor, sin: torch.Tensor, positions: torch.Tensor, inv_freq: torch.Tensor) -> None:
+    tokens, half = cos.shape
+    _need(cos.is_contiguous() and sin.is_contiguous() and sin.shape == cos.shape, "rope_table: cos and sin must be contiguous [T, half]")
+    _need(inv_freq.numel() == half and inv_freq.is_contiguous(), "rope_table: inv_freq must hold `half` values")
+    _need(positions.dtype == torch.int32 and positions.numel() >= tokens and positions.is_contiguous(), "rope_table: positions must be int32 [T]")
+    _check(library().lrs_rope_table(_dev(cos, "cos", torch.float32), _dev(sin, "sin", torch.float32), _dev(positions, "positions"),
+                                    _dev(inv_freq, "inv_freq", torch.float32), tokens, half, _stream()))
+
+
+def qk_prep(qkv: torch.Tensor, nq: int, nkv: int, d: int, q_weight, k_weight, eps: float, cos, sin,
+            k_pages, v_pages, slots, page_size: int) -> None:
+    """Normalise and rotate the q and k heads of `qkv` [T, (nq+2*nkv)*d]; q in place, k and v into pages."""
+    tokens = qkv.shape[0]
+    stride = _rows(qkv, "qkv")
+    _need(qkv.shape[1] == (nq + 2 * nkv) * d, f"qk_prep: qkv width {qkv.shape[1]} is not (nq+2nkv)*d = {(nq + 2 * nkv) * d}")
+    rot_half = 0
+    if cos is not None:
+        rot_half = cos.shape[1]
+        _need(cos.shape[0] >= tokens and sin.shape == cos.shape and cos.is_contiguous() and sin.is_contiguous(), "qk_prep: rotary tables must be [T, half]")
+        _need(cos.dtype == torch.float32 and sin.dtype == torch.float32, "qk_prep: rotary tables must be float32")
+    w_dtype = qkv.dtype
+    if q_weight is not None:
+        _need(k_weight is not None and q_weight.numel() == d and k_weight.numel() == d and q_weight.dtype == k_weight.dtype, "qk_prep: q/k norm weights must both hold head_dim values")
+        w_dtype = q_weight.dtype
+    if nkv > 0:
+        _need(k_pages.dim() == 4 and k_pages.shape[1:] == (nkv, page_size, d) and v_pages.shape == k_pages.shape, f"qk_prep: pages must be [pages, {nkv}, {page_size}, {d}]")
+        _need(k_pages.is_contiguous() and v_pages.is_contiguous() and k_pages.dtype == qkv.dtype and v_pages.dtype == qkv.dtype, "qk_prep: pages must be contiguous and of the activation dtype")
+        _need(slots.dtype == torch.int32 and slots.numel() >= tokens and slots.is_contiguous(), "qk_prep: slots must be int32 [T]")
+    _check(library().lrs_qk_prep(
+        _dev(qkv, "qkv"), dtype_code(qkv.dtype), tokens, stride, nq, nkv, d,
+        None if q_weight is None else _dev(q_weight, "q_weight"), None if k_weight is None else _dev(k_weight, "k_weight"),
+        dtype_code(w_dtype), eps, None if cos is None else cos.data_ptr(), None if sin is None else sin.data_ptr(), rot_half,
+        None if nkv == 0 else _dev(k_pages, "k_pages"), None if nkv == 0 else _dev(v_pages, "v_pages"),
+        None if nkv == 0 else _dev(slots, "slots"), page_size, _stream()))
+
+
+def silu_mul(out: torch.Tensor, gate_up: torch.Tensor) -> None:
+    tokens, inter = out.shape
+    _need(out.is_contiguous() and gate_up.is_contiguous() and gate_up.shape == (tokens, 2 * inter) and gate_up.dtype == out.dtype, "silu_mul: gate_up must be [T, 2I] and out [T, I], same dtype")
+    _check(library().lrs_silu_mul(_dev(out, "out"), _dev(gate_up, "gate_up"), dtype_code(out.dtype), tokens, inter, _stream()))
+
+
+def fill_i32(dst: torch.Tensor, value: int) -> None:
+    _need(dst.dtype == torch.int32 and dst.is_contiguous(), "fill_i32: int32 contiguous tensor needed")
+    _check(library().lrs_fill_i32(_dev(dst, "dst"), value, dst.numel(), _stream()))
+
+
+def gather_rows(out: torch.Tensor, x: torch.Tensor, rows: torch.Tensor) -> None:
+    n_rows, hidden = out.shape
+    _need(out.is_contiguous() and x.is_contiguous() and x.shape[1] == hidden, "gather_rows: shapes disagree")
+    _need(rows.dtype == torch.int32 and rows.numel() >= n_rows, "gather_rows: rows must be int32")
+    _check(library().lrs_gather_rows(_dev(out, "out", torch.float32), _dev(x, "x", torch.float32), _dev(rows, "rows"), n_rows, hidden, _stream()))
+
+
+# ------------------------------------------------------------------- gemm
+def gemm(out: torch.Tensor, a: torch.Tensor, w: torch.Tensor, bias: torch.Tensor | None = None, accumulate: bool = False) -> None:
+    """out = a @ w.T (+ bias).  `accumulate` adds into a float32 `out` instead of storing."""
+    m, k = a.shape
+    n = w.shape[0]
+    lda, ldc = _rows(a, "a"), _rows(out, "out")
+    _need(w.dim() == 2 and w.is_contiguous() and w.shape[1] == k, f"gemm: weight must be contiguous [N, {k}], got {tuple(w.shape)}")
+    _need(out.shape == (m, n), f"gemm: out must be [{m}, {n}], got {tuple(out.shape)}")
+    _need(a.dtype == w.dtype, f"gemm: a is {a.dtype} but w is {w.dtype}")
+    if accumulate:
+        _need(out.dtype == torch.float32, "gemm: accumulation needs a float32 output")
+        mode = OUT_ADD_F32
+    elif out.dtype == a.dtype:
+        mode = OUT_STORE
+    else:
+        _need(out.dtype == torch.float32, "gemm: output must be of the input dtype or float32")
+        mode = OUT_STORE_F32
+    if bias is not None:
+        _need(bias.numel() == n and bias.dtype == a.dtype and bias.is_contiguous(), "gemm: bias must hold N values of the input dtype")
+    _check(library().lrs_gemm(_dev(out, "out"), mode, _dev(a, "a"), _dev(w, "w"), None if bias is None else _dev(bias, "bias"),
+                              dtype_code(a.dtype), m, n, k, lda, ldc, _stream()))
+
+
+# -------------------------------------------------------------- attention
+def attention(out: torch.Tensor, q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, block_table: torch.Tensor,
+              token_request: torch.Tensor, positions: torch.Tensor, nq: int, scale: float, window: int = 0) -> None:
+    """out [T, nq*d]; q [T, >= nq*d] (leading nq*d columns of each row); pages [P, nkv, page, d]."""
+    tokens = out.shape[0]
+    _need(k_pages.dim() == 4 and v_pages.shape == k_pages.shape and k_pages.is_contiguous() and v_pages.is_contiguous(), "attention: pages must be contiguous [P, nkv, page, d]")
+    _, nkv, page_size, d = k_pages.shape
+    _need(out.shape[1] == nq * d and q.shape[0] == tokens and q.shape[1] >= nq * d, "attention: q/out widths do not match nq*d")
+    _need(q.dtype == k_pages.dtype == v_pages.dtype == out.dtype, "attention: q, pages and out must share a dtype")
+    _need(block_table.dim() == 2 and block_table.dtype == torch.int32 and block_table.stride(1) == 1, "attention: block_table must be int32 [R, blocks]")
+    for name, t in (("token_request", token_request), ("positions", positions)):
+        _need(t.dtype == torch.int32 and t.numel() >= tokens and t.is_contiguous(), f"attention: {name} must be int32 [T]")
+    _check(library().lrs_attention(
+        _dev(out, "out"), _rows(out, "out"), _dev(q, "q"), _rows(q, "q"), _dev(k_pages, "k_pages"), _dev(v_pages, "v_pages"),
+        _dev(block_table, "block_table"), block_table.stride(0), _dev(token_request, "token_request"), _dev(positions, "positions"),
+        dtype_code(q.dtype), tokens, nq, nkv, d, page_size, scale, window, _stream()))
+
+
+# --------------------------------------------------------------- sampling
+def choose_tokens(out: torch.Tensor, logits: torch.Tensor, temperature=None, seeds=None, counters=None) -> None:
+    rows, vocab = logits.shape
+    _need(out.dtype == torch.int32 and out.numel() >= rows and out.is_contiguous(), "choose_tokens: out must be int32 [R]")
+    stride = _rows(logits, "logits")
+    if temperature is not None:
+        _need(temperature.dtype == torch.float32 and temperature.numel() >= rows, "choose_tokens: temperature must be float32 [R]")
+        _need(seeds is not None and seeds.dtype == torch.int64 and seeds.numel() >= rows, "choose_tokens: seeds must be int64 [R]")
+        _need(counters is not None and counters.dtype == torch.int32 and counters.numel() >= rows, "choose_tokens: counters must be int32 [R]")
+    _check(library().lrs_choose_tokens(
+        _dev(out, "out"), _dev(logits, "logits", torch.float32), stride, rows, vocab,
+        None if temperature is None else _dev(temperature, "temperature"), None if temperature is None else _dev(seeds, "seeds"),
+        None if temperature is None else _dev(counters, "counters"), _stream()))
+
+
+def filter_logits(logits: torch.Tensor, temperature: torch.Tensor, top_k: torch.Tensor | None, top_p: torch.Tensor | None) -> None:
+    rows, vocab = logits.shape
+    stride = _rows(logits, "logits")
+    _need(temperature.dtype == torch.float32 and temperature.numel() >= rows, "filter_logits: temperature must be float32 [R]")
+    if top_k is not None:
+        _need(top_k.dtype == torch.int32 and top_k.numel() >= rows, "filter_logits: top_k must be int32 [R]")
+    if top_p is not None:
+        _need(top_p.dtype == torch.float32 and top_p.numel() >= rows, "filter_logits: top_p must be float32 [R]")
+    _check(library().lrs_filter_logits(_dev(logits, "logits", torch.float32), stride, rows, vocab, _dev(temperature, "temperature"),
+                                       None if top_k is None else _dev(top_k, "top_k"), None if top_p is None else _dev(top_p, "top_p"), _stream()))

@@ -1,0 +1,337 @@
+"""Each HIP kernel alone against a plain float32 torch computation of the same op,
+at sizes other than the engine's: widths and vocabularies that are no power of two,
+head sizes in steps of 16, odd head and group counts, page edges."""
+
+import math
+
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+DTYPES = [torch.float32, torch.bfloat16]
+
+
+def tol(dtype, f32=1e-5, bf16=2e-2):
+    return dict(rtol=f32, atol=f32) if dtype == torch.float32 else dict(rtol=bf16, atol=bf16)
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from llm_runtime_study_amd.kernels import ops as _ops
+
+    _ops.library()
+    return _ops
+
+
+def dev(t):
+    return t.to("cuda")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("tokens,hidden,vocab", [(1, 64, 256), (7, 96, 331), (33, 4096, 1000)])
+def test_embed(ops, dtype, tokens, hidden, vocab):
+    g = torch.Generator().manual_seed(0)
+    table = torch.randn(vocab, hidden, generator=g).to(dtype)
+    ids = torch.randint(0, vocab, (tokens,), generator=g, dtype=torch.int32)
+    ids[0] = vocab - 1
+    out = torch.empty(tokens, hidden, device="cuda")
+    ops.embed(out, dev(table), dev(ids))
+    torch.testing.assert_close(out.cpu(), table.float()[ids.long()], rtol=0, atol=0)
+
+
+@pytest.mark.parametrize("out_dtype", DTYPES)
+@pytest.mark.parametrize("w_dtype", DTYPES)
+@pytest.mark.parametrize("rows,hidden,eps", [(1, 64, 1e-6), (5, 96, 1e-5), (3, 4096, 1e-6), (2, 5120 + 16, 1e-3)])
+def test_rmsnorm(ops, out_dtype, w_dtype, rows, hidden, eps):
+    g = torch.Generator().manual_seed(1)
+    x = torch.randn(rows + 2, hidden, generator=g) * 3
+    w = (1 + 0.1 * torch.randn(hidden, generator=g)).to(w_dtype)
+    want = w.float() * (x * torch.rsqrt(x.square().mean(-1, keepdim=True) + eps))
+    out = torch.empty(rows, hidden, device="cuda", dtype=out_dtype)
+    ops.rmsnorm(out, dev(x), dev(w), eps)
+    torch.testing.assert_close(out.cpu().float(), want[:rows], **tol(out_dtype, 2e-6, 1e-2))
+    pick = torch.tensor([rows + 1, 0, rows][:rows] + [1] * max(0, rows - 3), dtype=torch.int32)
+    ops.rmsnorm(out, dev(x), dev(w), eps, rows=dev(pick))
+    torch.testing.assert_close(out.cpu().float(), want[pick.long()], **tol(out_dtype, 2e-6, 1e-2))
+
+
+@pytest.mark.parametrize("half,theta", [(8, 1e4), (16, 1e6), (64, 1e6), (24, 5e5)])
+def test_rope_table(ops, half, theta):
+    positions = torch.tensor([0, 1, 2, 17, 511, 4095, 40959], dtype=torch.int32)
+    inv = 1.0 / (theta ** (torch.arange(0, 2 * half, 2, dtype=torch.float32) / (2 * half)))
+    cos = torch.empty(len(positions), half, device="cuda")
+    sin = torch.empty_like(cos)
+    ops.rope_table(cos, sin, dev(positions), dev(inv))
+    angles = positions.float().unsqueeze(-1) * inv
+    torch.testing.assert_close(cos.cpu(), angles.cos(), rtol=0, atol=2e-7)
+    torch.testing.assert_close(sin.cpu(), angles.sin(), rtol=0, atol=2e-7)
+    # against float64 angles: what float32 tables can give at position 40959
+    exact = (positions.double().unsqueeze(-1) * inv.double()).cos()
+    assert (cos.cpu().double() - exact).abs().max() < 3e-3
+
+
+def _qk_prep_reference(qkv, nq, nkv, d, qw, kw, eps, positions, inv, rot_half):
+    t = qkv.shape[0]
+    heads = qkv.float().view(t, nq + 2 * nkv, d)
+    q, k, v = heads[:, :nq], heads[:, nq:nq + nkv], heads[:, nq + nkv:]
+
+    def norm(x, w):
+        if w is None:
+            return x
+        return w.float() * (x * torch.rsqrt(x.square().mean(-1, keepdim=True) + eps))
+
+    def rotate(x):
+        if rot_half == 0:
+            return x
+        ang = positions.float().view(t, 1, 1) * inv.view(1, 1, -1)
+        c, s = ang.cos(), ang.sin()
+        a, b, rest = x[..., :rot_half], x[..., rot_half:2 * rot_half], x[..., 2 * rot_half:]
+        return torch.cat((a * c - b * s, b * c + a * s, rest), -1)
+
+    return rotate(norm(q, qw)), rotate(norm(k, kw)), v
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("nq,nkv,d,rot,normed,page", [
+    (4, 2, 16, 16, True, 4), (8, 2, 32, 32, True, 16), (3, 3, 48, 32, False, 8),
+    (32, 8, 128, 128, True, 16), (5, 1, 80, 0, True, 16), (6, 2, 256, 256, True, 64),
+])
+def test_qk_prep(ops, dtype, nq, nkv, d, rot, normed, page):
+    g = torch.Generator().manual_seed(2)
+    t, pages = 19, 12
+    qkv = torch.randn(t, (nq + 2 * nkv) * d, generator=g).to(dtype)
+    qw = (1 + 0.1 * torch.randn(d, generator=g)).to(dtype) if normed else None
+    kw = (1 + 0.1 * torch.randn(d, generator=g)).to(dtype) if normed else None
+    positions = torch.randint(0, 3000, (t,), generator=g, dtype=torch.int32)
+    rot_half = rot // 2
+    inv = 1.0 / (1e4 ** (torch.arange(0, rot, 2, dtype=torch.float32) / max(rot, 1)))
+    slots = torch.randperm(pages * page, generator=g)[:t].to(torch.int32)
+    slots[3] = -1  # a token that must not be stored
+    want_q, want_k, want_v = _qk_prep_reference(qkv, nq, nkv, d, qw, kw, 1e-6, positions, inv, rot_half)
+
+    d_qkv = dev(qkv)
+    kp = torch.full((pages, nkv, page, d), 7.0, device="cuda", dtype=dtype)
+    vp = torch.full((pages, nkv, page, d), 7.0, device="cuda", dtype=dtype)
+    cos = sin = None
+    if rot_half:
+        cos = torch.empty(t, rot_half, device="cuda")
+        sin = torch.empty_like(cos)
+        ops.rope_table(cos, sin, dev(positions), dev(inv))
+    ops.qk_prep(d_qkv, nq, nkv, d, None if qw is None else dev(qw), None if kw is None else dev(kw), 1e-6,
+                cos, sin, kp, vp, dev(slots), page)
+    got = d_qkv.cpu().float().view(t, nq + 2 * nkv, d)
+    torch.testing.assert_close(got[:, :nq], want_q, **tol(dtype, 1e-5, 2e-2))
+    kp, vp = kp.cpu().float(), vp.cpu().float()
+    touched = torch.zeros(pages, page, dtype=torch.bool)
+    for i in range(t):
+        s = int(slots[i])
+        if s < 0:
+            continue
+        touched[s // page, s % page] = True
+        torch.testing.assert_close(kp[s // page, :, s % page], want_k[i], **tol(dtype, 1e-5, 2e-2))
+        torch.testing.assert_close(vp[s // page, :, s % page], want_v[i], rtol=0, atol=0)
+    # nothing else was written
+    assert (kp.permute(0, 2, 1, 3)[~touched] == 7.0).all() and (vp.permute(0, 2, 1, 3)[~touched] == 7.0).all()
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("tokens,inter", [(1, 128), (9, 160), (4, 12288), (300, 331)])
+def test_silu_mul(ops, dtype, tokens, inter):
+    g = torch.Generator().manual_seed(3)
+    gu = (torch.randn(tokens, 2 * inter, generator=g) * 2).to(dtype)
+    out = torch.empty(tokens, inter, device="cuda", dtype=dtype)
+    ops.silu_mul(out, dev(gu))
+    gate, up = gu.float()[:, :inter], gu.float()[:, inter:]
+    torch.testing.assert_close(out.cpu().float(), torch.nn.functional.silu(gate) * up, **tol(dtype, 1e-6, 1e-2))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("m,n,k", [
+    (1, 64, 64), (5, 331, 96), (17, 160, 96), (64, 256, 160), (130, 200, 264), (3, 129, 40),
+    (2, 70, 36), (1, 1000, 4096), (257, 384, 512),
+])
+@pytest.mark.parametrize("mode", ["store", "store_f32", "add"])
+def test_gemm(ops, dtype, m, n, k, mode):
+    g = torch.Generator().manual_seed(4)
+    a = torch.randn(m, k, generator=g).to(dtype)
+    w = (torch.randn(n, k, generator=g) / math.sqrt(k)).to(dtype)
+    bias = torch.randn(n, generator=g).to(dtype) if n % 2 else None
+    want = a.double() @ w.double().T + (0 if bias is None else bias.double())
+    if mode == "store":
+        out = torch.empty(m, n, device="cuda", dtype=dtype)
+    else:
+        out = torch.full((m, n), 0.5, device="cuda")
+    ops.gemm(out, dev(a), dev(w), None if bias is None else dev(bias), accumulate=(mode == "add"))
+    if mode == "add":
+        want = want + 0.5
+    if dtype == torch.float32:
+        torch.testing.assert_close(out.cpu().double(), want, rtol=1e-5, atol=1e-5)
+    elif mode == "store":
+        torch.testing.assert_close(out.cpu().double(), want, rtol=1e-2, atol=1e-2)
+    else:  # bf16 inputs, float32 accumulation and output: only the summation order differs
+        torch.testing.assert_close(out.cpu().double(), want, rtol=1e-4, atol=1e-4)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_gemm_row_does_not_depend_on_batch(ops, dtype):
+    g = torch.Generator().manual_seed(5)
+    a = torch.randn(70, 96, generator=g).to(dtype)
+    w = torch.randn(200, 96, generator=g).to(dtype)
+    full = torch.empty(70, 200, device="cuda")
+    ops.gemm(full, dev(a), dev(w))
+    one = torch.empty(1, 200, device="cuda")
+    ops.gemm(one, dev(a[41:42]), dev(w))
+    torch.testing.assert_close(one.cpu(), full.cpu()[41:42], rtol=0, atol=0)
+    # strided input and output rows
+    wide_in = dev(torch.cat((a, a), 1))
+    wide_out = torch.zeros(70, 300, device="cuda")
+    ops.gemm(wide_out[:, :200], wide_in[:, 96:], dev(w))
+    torch.testing.assert_close(wide_out.cpu()[:, :200], full.cpu(), rtol=0, atol=0)
+    assert (wide_out[:, 200:] == 0).all()
+
+
+def _attention_reference(q, k_all, v_all, positions, lengths_before, nq, nkv, d, scale, window):
+    """q [T, nq, d]; k_all/v_all: per request [len, nkv, d]; returns [T, nq*d] float64."""
+    outs = []
+    for t, (r, p) in enumerate(positions):
+        k = k_all[r][: p + 1].double()
+        v = v_all[r][: p + 1].double()
+        lo = max(0, p - window + 1) if window else 0
+        k, v = k[lo:], v[lo:]
+        row = []
+        for h in range(nq):
+            gi = h // (nq // nkv)
+            s = (k[:, gi] @ q[t, h].double()) * scale
+            row.append(torch.softmax(s, 0) @ v[:, gi])
+        outs.append(torch.cat(row))
+    return torch.stack(outs)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("nq,nkv,d,page,window", [
+    (4, 2, 16, 4, 0), (8, 2, 32, 16, 0), (3, 1, 48, 8, 0), (6, 3, 80, 16, 0), (32, 8, 128, 16, 0),
+    (4, 4, 256, 64, 0), (8, 2, 32, 16, 7), (4, 2, 64, 16, 33),
+])
+def test_attention_ragged_batch(ops, dtype, nq, nkv, d, page, window):
+    g = torch.Generator().manual_seed(6)
+    # request: (cached length before the step, new tokens in the step)
+    requests = [(0, 19), (37, 1), (150, 1), (5, 6), (page * 3 - 1, 2)]
+    scale = 1 / math.sqrt(d)
+    max_blocks = max((a + b + page - 1) // page for a, b in requests)
+    n_pages = sum((a + b + page - 1) // page for a, b in requests) + 3
+    perm = torch.randperm(n_pages, generator=g).tolist()
+    kp = torch.zeros(n_pages, nkv, page, d)
+    vp = torch.zeros(n_pages, nkv, page, d)
+    table = torch.zeros(len(requests), max_blocks, dtype=torch.int32)
+    k_all, v_all, q_rows, tok_req, tok_pos, meta = [], [], [], [], [], []
+    for r, (before, new) in enumerate(requests):
+        total = before + new
+        k = torch.randn(total, nkv, d, generator=g).to(dtype)
+        v = torch.randn(total, nkv, d, generator=g).to(dtype)
+        k_all.append(k.float())
+        v_all.append(v.float())
+        for b in range((total + page - 1) // page):
+            pg = perm.pop()
+            table[r, b] = pg
+            n = min(page, total - b * page)
+            kp[pg, :, :n] = k[b * page: b * page + n].float().transpose(0, 1)
+            vp[pg, :, :n] = v[b * page: b * page + n].float().transpose(0, 1)
+        for i in range(new):
+            q_rows.append((torch.randn(nq, d, generator=g) * 2).to(dtype))
+            tok_req.append(r)
+            tok_pos.append(before + i)
+            meta.append((r, before + i))
+    q = torch.stack(q_rows)
+    t = q.shape[0]
+    want = _attention_reference(q.float(), k_all, v_all, meta, None, nq, nkv, d, scale, window)
+    # q sits in the leading columns of a wider row, as in the fused projection output
+    q_wide = torch.zeros(t, nq * d + 2 * nkv * d, dtype=dtype)
+    q_wide[:, : nq * d] = q.view(t, nq * d)
+    out = torch.empty(t, nq * d, device="cuda", dtype=dtype)
+    ops.attention(out, dev(q_wide), dev(kp.to(dtype)), dev(vp.to(dtype)), dev(table),
+                  dev(torch.tensor(tok_req, dtype=torch.int32)), dev(torch.tensor(tok_pos, dtype=torch.int32)),
+                  nq, scale, window)
+    torch.testing.assert_close(out.cpu().double(), want, **tol(dtype, 2e-5, 2e-2))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_attention_finds_a_far_key(ops, dtype):
+    """One key among 700 is made to dominate: the output must be its value, wherever it lies."""
+    nq, nkv, d, page = 2, 1, 32, 16
+    g = torch.Generator().manual_seed(7)
+    length = 700
+    for far in (0, 15, 16, 127, 128, 511, 698, 699):
+        k = torch.randn(length, nkv, d, generator=g) * 0.1
+        v = torch.randn(length, nkv, d, generator=g)
+        q = torch.randn(1, nq, d, generator=g)
+        q = q / q.norm(dim=-1, keepdim=True)
+        k[far, 0] = q[0, 0] * 60  # score 60/sqrt(32)*... dominates head 0
+        n_pages = (length + page - 1) // page
+        kp = torch.zeros(n_pages, nkv, page, d)
+        vp = torch.zeros(n_pages, nkv, page, d)
+        order = torch.randperm(n_pages, generator=g)
+        table = order.to(torch.int32).view(1, -1)
+        for b in range(n_pages):
+            n = min(page, length - b * page)
+            kp[order[b], :, :n] = k[b * page: b * page + n].transpose(0, 1)
+            vp[order[b], :, :n] = v[b * page: b * page + n].transpose(0, 1)
+        out = torch.empty(1, nq * d, device="cuda", dtype=dtype)
+        ops.attention(out, dev(q.view(1, -1).to(dtype)), dev(kp.to(dtype)), dev(vp.to(dtype)), dev(table),
+                      dev(torch.zeros(1, dtype=torch.int32)), dev(torch.tensor([length - 1], dtype=torch.int32)), nq, 1.0, 0)
+        torch.testing.assert_close(out.cpu().float()[0, :d], v[far, 0].to(dtype).float(), rtol=2e-2, atol=2e-2)
+
+
+@pytest.mark.parametrize("rows,vocab", [(1, 256), (5, 331), (3, 151936)])
+def test_choose_tokens_greedy(ops, rows, vocab):
+    g = torch.Generator().manual_seed(8)
+    logits = torch.randn(rows, vocab, generator=g)
+    logits[0, vocab - 1] = 50.0
+    if rows > 1:
+        logits[1, 5] = logits[1, 77] = 40.0  # tie: the lowest index wins
+    out = torch.empty(rows, dtype=torch.int32, device="cuda")
+    ops.choose_tokens(out, dev(logits))
+    assert out.cpu().tolist() == [int(torch.argmax(r)) if i != 1 else 5 for i, r in enumerate(logits)]
+
+
+def test_choose_tokens_temperature_statistics(ops):
+    vocab, draws = 11, 20000
+    probs = torch.tensor([0.3, 0.2, 0.15, 0.1, 0.08, 0.07, 0.05, 0.03, 0.01, 0.01, 0.0])
+    temperature = 0.7
+    logits = (torch.log(probs) * temperature).repeat(draws, 1)  # softmax(logits / T) = probs
+    out = torch.empty(draws, dtype=torch.int32, device="cuda")
+    temps = torch.full((draws,), temperature, device="cuda")
+    seeds = torch.full((draws,), 1234, dtype=torch.int64, device="cuda")
+    counters = torch.arange(draws, dtype=torch.int32, device="cuda")
+    ops.choose_tokens(out, dev(logits), temps, seeds, counters)
+    freq = torch.bincount(out.cpu().long(), minlength=vocab).float() / draws
+    assert freq[-1] == 0  # a -inf logit is never drawn
+    assert (freq - probs).abs().max() < 0.012
+    # reproducible, and a row's draw does not depend on its neighbours
+    again = torch.empty(7, dtype=torch.int32, device="cuda")
+    ops.choose_tokens(again, dev(logits[:7]), temps[:7], seeds[:7], counters[100:107].contiguous())
+    assert again.cpu().tolist() == out.cpu()[100:107].tolist()
+    other = torch.empty(draws, dtype=torch.int32, device="cuda")
+    ops.choose_tokens(other, dev(logits), temps, seeds + 1, counters)
+    assert (other != out).float().mean() > 0.3
+
+
+def test_filter_logits_matches_sort_based_rule(ops):
+    from tests.plain.model import filter_logits as plain_filter
+
+    g = torch.Generator().manual_seed(9)
+    cases = [(0.8, 5, 1.0), (1.3, None, 0.7), (0.5, 40, 0.9), (1.0, 1, 0.5), (2.0, None, 0.05), (1.0, 331, 1.0)]
+    logits = torch.randn(len(cases), 331, generator=g) * 3
+    logits[1, :4] = torch.log(torch.tensor([0.60, 0.25, 0.10, 0.05])) + 30  # reference vector: p=.70 keeps two
+    work = dev(logits.clone())
+    temps = dev(torch.tensor([c[0] for c in cases]))
+    ks = dev(torch.tensor([c[1] or 0 for c in cases], dtype=torch.int32))
+    ps = dev(torch.tensor([c[2] for c in cases]))
+    ops.filter_logits(work, temps, ks, ps)
+    got = work.cpu()
+    for i, (temp, k, p) in enumerate(cases):
+        want = plain_filter(logits[i], temp, k, p)
+        assert torch.equal(torch.isfinite(got[i]), torch.isfinite(want)), f"case {i}"
+        kept = torch.isfinite(want)
+        torch.testing.assert_close(got[i][kept], logits[i][kept], rtol=0, atol=0)
+    assert torch.isfinite(got[1]).sum() == 2

@@ -1,0 +1,201 @@
+"""Pins of the plain implementation: vectors held by the reference's own tests,
+special cases that reduce to a library routine, and invariants.  Each is chosen
+so that one plausible misreading (a sign, a pairing, a norm in the wrong place)
+fails it.  CPU only.
+"""
+
+import math
+
+import pytest
+import torch
+import torch.nn.functional as F
+
+from tests.plain import model as plain
+
+from tests.helpers import random_qwen3_weights, TINY_A, TINY_B
+
+
+def test_rms_norm_equation_vector():
+    # reference tests/test_norm.py:11-27
+    x = torch.tensor([[1.0, 2.0, 3.0, 4.0], [-2.0, 0.5, 1.5, 3.0]])
+    w = torch.tensor([1.0, 0.5, 1.5, 2.0])
+    got = plain.rms_norm(x, w, 1e-6)
+    row0 = torch.tensor([1.0, 2.0, 3.0, 4.0]) / math.sqrt(7.5 + 1e-6) * w
+    torch.testing.assert_close(got[0], row0)
+    torch.testing.assert_close(got, F.rms_norm(x, (4,), w, 1e-6))
+
+
+def test_rms_norm_half_precision_vector():
+    # reference tests/test_norm.py:29-38: [300, 400] -> [0.8486, 1.1314]
+    got = plain.rms_norm(torch.tensor([[300.0, 400.0]]), torch.ones(2), 1e-6)
+    torch.testing.assert_close(got, torch.tensor([[0.8486, 1.1314]]), rtol=1e-3, atol=1e-3)
+
+
+def test_rms_norm_invariants():
+    x = torch.randn(5, 24)
+    unit = plain.rms_norm(x, torch.ones(24), 1e-12)
+    torch.testing.assert_close(unit.square().mean(-1), torch.ones(5))
+    torch.testing.assert_close(plain.rms_norm(7.0 * x, torch.ones(24), 1e-12), unit)
+    # no mean subtraction: a constant vector maps to +-1, not to 0
+    torch.testing.assert_close(plain.rms_norm(torch.full((1, 8), 3.0), torch.ones(8), 1e-12), torch.ones(1, 8))
+
+
+def test_qk_norm_shared_weight_vector():
+    # reference tests/test_norm.py:64-85: weights 2 and 3 => k = 1.5 q
+    base = torch.tensor([1.0, 2.0, 3.0, 4.0])
+    q = plain.rms_norm(base.repeat(4, 3, 1), torch.full((4,), 2.0), 1e-6)
+    k = plain.rms_norm(base.repeat(2, 3, 1), torch.full((4,), 3.0), 1e-6)
+    torch.testing.assert_close(k[0, 0], 1.5 * q[0, 0])
+
+
+def test_rope_hand_rotation_vector():
+    # reference tests/test_rope.py:16-42: d=4, theta=1e4, pairs (0,2) and (1,3)
+    cos, sin = plain.rope_tables(torch.tensor([0, 1]), 4, 10000.0)
+    for vec in (torch.tensor([1.0, 2.0, 3.0, 4.0]), torch.tensor([-0.5, 1.5, 2.5, -3.0])):
+        out = plain.apply_rope(vec.expand(1, 2, 4), cos, sin)
+        torch.testing.assert_close(out[0, 0], vec)
+        a, b = 1.0, 0.01
+        want = torch.tensor([
+            vec[0] * math.cos(a) - vec[2] * math.sin(a),
+            vec[1] * math.cos(b) - vec[3] * math.sin(b),
+            vec[2] * math.cos(a) + vec[0] * math.sin(a),
+            vec[3] * math.cos(b) + vec[1] * math.sin(b),
+        ])
+        torch.testing.assert_close(out[0, 1], want)
+
+
+def test_rope_invariants():
+    d, theta = 16, 1e4
+    q, k = torch.randn(1, 1, d, dtype=torch.float64), torch.randn(1, 1, d, dtype=torch.float64)
+
+    def dot(p, s):
+        cp, sp = plain.rope_tables(torch.tensor([p]), d, theta, torch.float64)
+        cs, ss = plain.rope_tables(torch.tensor([s]), d, theta, torch.float64)
+        return (plain.apply_rope(q, cp, sp) * plain.apply_rope(k, cs, ss)).sum()
+
+    # only distances count
+    torch.testing.assert_close(dot(9, 4), dot(105, 100))
+    assert abs(dot(9, 4) - dot(9, 5)) > 1e-6
+    # norm preserving (reference tests/test_rope.py:44-58)
+    c, s = plain.rope_tables(torch.arange(7), d, theta, torch.float64)
+    x = torch.randn(3, 7, d, dtype=torch.float64)
+    torch.testing.assert_close(plain.apply_rope(x, c, s).norm(dim=-1), x.norm(dim=-1))
+    # inverse frequencies: first is 1, last is theta^-(d-2)/d
+    inv = plain.rope_inverse_frequencies(d, theta, torch.float64)
+    assert inv[0] == 1.0 and abs(inv[-1] - theta ** (-(d - 2) / d)) < 1e-15
+
+
+def test_attention_reduces_to_library():
+    heads, t, d = 3, 9, 8
+    q, k, v = (torch.randn(heads, t, d) for _ in range(3))
+    pos = torch.arange(t)
+    got = plain.masked_attention(q, k, v, 1 / math.sqrt(d), pos, pos)
+    want = F.scaled_dot_product_attention(q[None], k[None], v[None], is_causal=True)[0]
+    torch.testing.assert_close(got, want, rtol=1e-5, atol=1e-6)
+    # no mask at all: every query sits after every key
+    got = plain.masked_attention(q, k, v, 0.3, torch.full((t,), 100), pos)
+    want = torch.softmax(q @ k.transpose(-1, -2) * 0.3, -1) @ v
+    torch.testing.assert_close(got, want, rtol=1e-5, atol=1e-6)
+
+
+def test_attention_special_cases():
+    d = 4
+    q = torch.randn(2, 1, d)
+    v = torch.randn(2, 5, d)
+    # one key => output is its value
+    out = plain.masked_attention(q, torch.randn(2, 1, d), v[:, :1], 0.5, torch.tensor([0]), torch.tensor([0]))
+    torch.testing.assert_close(out, v[:, :1])
+    # identical keys => mean of the values
+    k = torch.randn(2, 1, d).expand(2, 5, d)
+    out = plain.masked_attention(q, k, v, 0.5, torch.tensor([4]), torch.arange(5))
+    torch.testing.assert_close(out, v.mean(1, keepdim=True), rtol=1e-5, atol=1e-6)
+    # window 2 at position 4 sees keys 3 and 4 only
+    out = plain.masked_attention(q, k, v, 0.5, torch.tensor([4]), torch.arange(5), window=2)
+    torch.testing.assert_close(out, v[:, 3:].mean(1, keepdim=True), rtol=1e-5, atol=1e-6)
+
+
+def test_gqa_head_map():
+    # reference tests/test_attention.py:88-96: kv heads [1, 2] serve query heads [1, 1, 2, 2]
+    states = torch.tensor([[[1.0]], [[2.0]]])
+    torch.testing.assert_close(plain.repeat_kv(states, 2)[:, 0, 0], torch.tensor([1.0, 1.0, 2.0, 2.0]))
+
+
+def test_qwen3_attention_matches_manual_reference():
+    # the recipe of reference tests/test_attention.py:47-84 at position 0..2 with theta so
+    # large that the rotation is the identity on all but the first pair
+    torch.manual_seed(11)
+    cfg = dict(num_attention_heads=2, num_key_value_heads=1, head_dim=2, rms_norm_eps=1e-6, rope_theta=1e4)
+    w = {
+        "a.q_proj.weight": torch.randn(4, 2), "a.k_proj.weight": torch.randn(2, 2),
+        "a.v_proj.weight": torch.randn(2, 2), "a.o_proj.weight": torch.randn(2, 4),
+        "a.q_norm.weight": torch.ones(2), "a.k_norm.weight": torch.ones(2),
+    }
+    x = torch.tensor([[1.0, 2.0], [-1.0, 0.5], [0.25, -0.75]])
+    # all positions equal => rotation cancels in q.k, so the no-rope manual recipe applies
+    got, _ = plain.qwen3_attention(x, w, "a", cfg, torch.zeros(3, dtype=torch.long))
+    q = (x @ w["a.q_proj.weight"].T).view(3, 2, 2).transpose(0, 1)
+    k = (x @ w["a.k_proj.weight"].T).view(3, 1, 2).transpose(0, 1)
+    v = (x @ w["a.v_proj.weight"].T).view(3, 1, 2).transpose(0, 1)
+    q = q * torch.rsqrt(q.square().mean(-1, keepdim=True) + 1e-6)
+    k = k * torch.rsqrt(k.square().mean(-1, keepdim=True) + 1e-6)
+    s = (q @ k.repeat_interleave(2, 0).transpose(-1, -2)) / math.sqrt(2)
+    # equal positions: the mask key_pos <= query_pos lets every key through
+    o = torch.softmax(s, -1) @ v.repeat_interleave(2, 0)
+    want = o.transpose(0, 1).reshape(3, 4) @ w["a.o_proj.weight"].T
+    torch.testing.assert_close(got, want, rtol=1e-5, atol=1e-6)
+
+
+def test_swiglu_vector():
+    # reference tests/test_mlp.py:12-30
+    x = torch.tensor([[1.0, -2.0], [0.5, 3.0]])
+    g = torch.tensor([[1.0, 0.5], [-0.5, 2.0], [1.5, -1.0]])
+    u = torch.tensor([[0.25, 1.0], [2.0, -0.5], [-1.0, 0.75]])
+    dn = torch.tensor([[1.0, -0.5, 0.25], [-0.25, 0.75, 1.5]])
+    want = F.linear(F.silu(F.linear(x, g)) * F.linear(x, u), dn)
+    torch.testing.assert_close(plain.swiglu(x, g, u, dn), want)
+    torch.testing.assert_close(plain.swiglu(x, g, torch.zeros_like(u), dn), torch.zeros(2, 2))
+
+
+@pytest.mark.parametrize("cfg", [TINY_A, TINY_B])
+def test_model_invariants(cfg):
+    w = random_qwen3_weights(cfg, seed=3, dtype=torch.float64)
+    ids = torch.randint(0, cfg["vocab_size"], (13,))
+    logits = plain.qwen3_forward(w, cfg, ids)
+    assert logits.shape == (13, cfg["vocab_size"])
+    # causality: changing token j leaves logits before j untouched
+    ids2 = ids.clone()
+    ids2[8] = (ids2[8] + 1) % cfg["vocab_size"]
+    logits2 = plain.qwen3_forward(w, cfg, ids2)
+    torch.testing.assert_close(logits2[:8], logits[:8], rtol=0, atol=0)
+    assert not torch.allclose(logits2[8:], logits[8:])
+    # only distances count: shifting all positions changes nothing
+    shifted = plain.qwen3_forward(w, cfg, ids, positions=torch.arange(13) + 29)
+    torch.testing.assert_close(shifted, logits, rtol=1e-9, atol=1e-9)
+    # zeroed o_proj and down_proj => logits = head(norm(embed))
+    wz = dict(w)
+    for i in range(cfg["num_hidden_layers"]):
+        wz[f"model.layers.{i}.self_attn.o_proj.weight"] = torch.zeros_like(w[f"model.layers.{i}.self_attn.o_proj.weight"])
+        wz[f"model.layers.{i}.mlp.down_proj.weight"] = torch.zeros_like(w[f"model.layers.{i}.mlp.down_proj.weight"])
+    head = wz.get("lm_head.weight", wz["model.embed_tokens.weight"])
+    want = plain.rms_norm(wz["model.embed_tokens.weight"][ids], wz["model.norm.weight"], cfg["rms_norm_eps"]) @ head.T
+    torch.testing.assert_close(plain.qwen3_forward(wz, cfg, ids), want)
+
+
+def test_tied_head_uses_embedding():
+    w = random_qwen3_weights(TINY_A, seed=1, dtype=torch.float64)
+    assert "lm_head.weight" not in w
+    untied = dict(w)
+    untied["lm_head.weight"] = w["model.embed_tokens.weight"].clone()
+    cfg2 = dict(TINY_A, tie_word_embeddings=False)
+    ids = [3, 9, 200, 17]
+    torch.testing.assert_close(plain.qwen3_forward(w, TINY_A, ids), plain.qwen3_forward(untied, cfg2, ids))
+
+
+def test_filter_logits_vectors():
+    # reference tests/test_generation.py top-p: probs .60 .25 .10 .05, p=.70 keeps two
+    logits = torch.log(torch.tensor([0.60, 0.25, 0.10, 0.05]))
+    kept = plain.filter_logits(logits, 1.0, None, 0.70)
+    assert torch.isfinite(kept).tolist() == [True, True, False, False]
+    kept = plain.filter_logits(torch.tensor([1.0, 4.0, 2.0, 3.0]), 2.0, 2, 1.0)
+    assert torch.isfinite(kept).tolist() == [False, True, False, True]
+    torch.testing.assert_close(kept[1], torch.tensor(2.0))
