@@ -1,0 +1,309 @@
+"""Cache manager: paged keys and values with a block table per request, and slots of
+fixed-size per-request state.
+
+What each schedule entry of the model keeps between steps is declared by its mixer:
+  PagedKVNeed(nkv, d, window)  keys and values of every position, or of a sliding window;
+  StateNeed(shape, dtype)      a state of fixed size;
+  ("from", j)                  nothing of its own: it reads the cache of entry j;
+  None                         nothing.
+Entries whose paged needs are equal form a group.  A group has a page pool of its own, one
+K and one V tensor [pages + 1, nkv, page_size, d] per entry (a page id addresses the same
+page in every entry of the group; the extra last page absorbs the writes of padding rows),
+and one block table per request.  Pages are taken when a request grows into them and given
+back when the request ends, is rolled back, or (windowed groups) when every position in
+the page has left the window of all future queries.
+
+Every admitted request also holds one state slot out of `max_requests`; StateNeed entries
+keep a tensor [max_requests, *shape], zeroed for the slot at admission.  The slot is also
+the request's row in the per-group host block tables.
+
+Lengths are host integers (reference mini_llm/cache/lengths.py:8-43): extend() before the
+forward, rollback() if it fails.  The reference reserves a request's whole lifetime at
+admission (mini_llm/cache/paged/cache.py:257-352); here pages are taken on demand and a
+reservation count gives the scheduler the same guarantee.
+"""
+
+from __future__ import annotations
+
+import heapq
+from dataclasses import dataclass, field
+
+import numpy as np
+import torch
+
+from ..errors import KVCacheError
+from ..parts import PagedKVNeed, StateNeed
+from .pages import PagePool
+
+
+@dataclass
+class LayerCache:
+    """What a mixer is handed for one schedule entry."""
+
+    group: int | None = None          # index of the paged group (ctx.group(i) has table and slots)
+    k_pages: torch.Tensor | None = None
+    v_pages: torch.Tensor | None = None
+    state: torch.Tensor | None = None  # [max_requests, *shape] for StateNeed entries
+    window: int | None = None
+
+
+@dataclass
+class RequestCache:
+    """Pages, slot and length of one live request."""
+
+    request_id: object
+    slot: int
+    length: int = 0
+    tables: list = field(default_factory=list)      # per group: page id per logical block, -1 = given back
+    first_live: list = field(default_factory=list)  # per group: first logical block still held
+    reserved: list = field(default_factory=list)    # per group: pages promised to this request
+    released: bool = False
+
+
+class PagedGroup:
+    def __init__(self, need: PagedKVNeed, entries: list[int], num_pages: int):
+        self.need, self.entries = need, entries
+        self.pool = PagePool(num_pages)
+        self.reserved_pages = 0
+        self.k: dict[int, torch.Tensor] = {}
+        self.v: dict[int, torch.Tensor] = {}
+        self.host_table: np.ndarray | None = None   # [max_requests, max_blocks] int32
+
+
+class CacheManager:
+    def __init__(self, needs: list, *, page_size: int, num_pages: int, max_requests: int, max_seq_len: int,
+                 dtype: torch.dtype = torch.float32, device="cpu", allocate_storage: bool = True):
+        if page_size <= 0:
+            raise KVCacheError(f"page_size must be positive, got {page_size}")
+        if max_requests <= 0:
+            raise KVCacheError(f"max_requests must be positive, got {max_requests}")
+        if max_seq_len <= 0:
+            raise KVCacheError(f"max_seq_len must be positive, got {max_seq_len}")
+        self.page_size, self.max_requests, self.max_seq_len = page_size, max_requests, max_seq_len
+        self.dtype, self.device = dtype, torch.device(device)
+        self.max_blocks = -(-max_seq_len // page_size)
+        self.groups: list[PagedGroup] = []
+        self.layer_caches: list[LayerCache] = []
+        self.state_entries: list[int] = []
+        self._free_slots = list(range(max_requests))
+        heapq.heapify(self._free_slots)
+        self._active: dict[int, RequestCache] = {}   # slot -> request
+        self.last_allocation_tokens = 0
+
+        by_need: dict[PagedKVNeed, PagedGroup] = {}
+        for position, need in enumerate(needs):
+            cache = LayerCache()
+            if isinstance(need, PagedKVNeed):
+                if need not in by_need:
+                    by_need[need] = PagedGroup(need, [], num_pages)
+                    self.groups.append(by_need[need])
+                group = by_need[need]
+                group.entries.append(position)
+                cache.group, cache.window = self.groups.index(group), need.window
+            elif isinstance(need, StateNeed):
+                self.state_entries.append(position)
+                if allocate_storage:
+                    cache.state = torch.zeros((max_requests, *need.shape), dtype=need.dtype, device=self.device)
+            elif isinstance(need, tuple) and len(need) == 2 and need[0] == "from":
+                source = need[1]
+                if not 0 <= source < position or self.layer_caches[source].group is None:
+                    raise KVCacheError(f"entry {position} reads the cache of entry {source}, which keeps no pages")
+                cache = self.layer_caches[source]
+            elif need is not None:
+                raise KVCacheError(f"entry {position} declares an unknown cache need: {need!r}")
+            self.layer_caches.append(cache)
+
+        for index, group in enumerate(self.groups):
+            group.host_table = np.full((max_requests, self.max_blocks), -1, dtype=np.int32)
+            if allocate_storage:
+                shape = (num_pages + 1, group.need.num_kv_heads, page_size, group.need.head_dim)
+                for position in group.entries:
+                    group.k[position] = torch.empty(shape, dtype=dtype, device=self.device)
+                    group.v[position] = torch.empty(shape, dtype=dtype, device=self.device)
+                    self.layer_caches[position].k_pages = group.k[position]
+                    self.layer_caches[position].v_pages = group.v[position]
+
+    # ------------------------------------------------------------------ sizes
+    @property
+    def capacity(self) -> int:
+        """Tokens the smallest pool can hold."""
+        return min((g.pool.num_pages for g in self.groups), default=0) * self.page_size
+
+    @property
+    def active_requests(self) -> int:
+        return len(self._active)
+
+    @property
+    def free_slots(self) -> int:
+        return len(self._free_slots)
+
+    def free_pages(self, group: int = 0) -> int:
+        return self.groups[group].pool.free_pages
+
+    def used_pages(self, group: int = 0) -> int:
+        return self.groups[group].pool.used_pages
+
+    @property
+    def used_tokens(self) -> int:
+        return max((g.pool.used_pages for g in self.groups), default=0) * self.page_size
+
+    def bytes_per_token(self) -> int:
+        size = torch.empty(0, dtype=self.dtype).element_size()
+        return sum(2 * len(g.entries) * g.need.num_kv_heads * g.need.head_dim * size for g in self.groups)
+
+    def trash_page(self, group: int = 0) -> int:
+        """Page that no request owns; padding rows of a padded batch write there."""
+        return self.groups[group].pool.num_pages
+
+    def pages_for(self, group: int, tokens: int, max_step_tokens: int | None = None) -> int:
+        """Pages a request of `tokens` positions can hold at once in `group`."""
+        blocks = -(-tokens // self.page_size)
+        window = self.groups[group].need.window
+        if window is None:
+            return blocks
+        step = tokens if max_step_tokens is None else max_step_tokens
+        return min(blocks, -(-window // self.page_size) + -(-step // self.page_size) + 2)
+
+    # -------------------------------------------------------------- admission
+    def can_admit(self, tokens: int, max_step_tokens: int | None = None) -> bool:
+        """Whether a slot is free and every pool can promise the pages of a `tokens`-long request."""
+        if not self._free_slots or tokens > self.max_seq_len:
+            return False
+        return all(g.reserved_pages + self.pages_for(i, tokens, max_step_tokens) <= g.pool.num_pages
+                   for i, g in enumerate(self.groups))
+
+    def admit(self, request_id=None, reserve_tokens: int = 0, max_step_tokens: int | None = None) -> RequestCache:
+        """Give a new request a state slot (zeroed) and, if asked, a promise of pages."""
+        if reserve_tokens < 0:
+            raise KVCacheError(f"reserve_tokens must not be negative, got {reserve_tokens}")
+        if reserve_tokens > self.max_seq_len:
+            raise KVCacheError(f"cache capacity {reserve_tokens} exceeds the context length {self.max_seq_len}")
+        if not self._free_slots:
+            raise KVCacheError(f"all {self.max_requests} request slots are in use")
+        reserved = [self.pages_for(i, reserve_tokens, max_step_tokens) if reserve_tokens else 0 for i in range(len(self.groups))]
+        for group, pages in zip(self.groups, reserved):
+            if group.reserved_pages + pages > group.pool.num_pages:
+                raise KVCacheError(
+                    f"KV block pool exhausted: need {pages} blocks but only "
+                    f"{group.pool.num_pages - group.reserved_pages} are unreserved")
+        slot = heapq.heappop(self._free_slots)
+        for group, pages in zip(self.groups, reserved):
+            group.reserved_pages += pages
+            group.host_table[slot, :] = -1
+        for position in self.state_entries:
+            state = self.layer_caches[position].state
+            if state is not None:
+                state[slot].zero_()
+        request = RequestCache(request_id, slot, 0, [[] for _ in self.groups], [0 for _ in self.groups], reserved)
+        self._active[slot] = request
+        self.last_allocation_tokens = reserve_tokens
+        return request
+
+    def _check_live(self, request: RequestCache) -> None:
+        if request.released or self._active.get(request.slot) is not request:
+            raise KVCacheError("cache has been released")
+
+    # ----------------------------------------------------------------- growth
+    def extend(self, request: RequestCache, tokens: int) -> None:
+        """Make room for `tokens` more positions and count them in; call before the forward."""
+        self._check_live(request)
+        if tokens <= 0:
+            raise KVCacheError(f"token_count must be positive, got {tokens}")
+        required = request.length + tokens
+        if required > self.max_seq_len:
+            raise KVCacheError(f"KV cache capacity exceeded: need {required} positions but capacity is {self.max_seq_len}")
+        blocks = -(-required // self.page_size)
+        wanted = [blocks - len(table) for table in request.tables]
+        for group, count in zip(self.groups, wanted):
+            if count > group.pool.free_pages:
+                raise KVCacheError(f"KV block pool exhausted: need {count} blocks but only {group.pool.free_pages} are free")
+        for index, (group, count) in enumerate(zip(self.groups, wanted)):
+            if count > 0:
+                table = request.tables[index]
+                pages = group.pool.allocate(count)
+                group.host_table[request.slot, len(table):len(table) + count] = pages
+                table.extend(pages)
+        request.length = required
+
+    def rollback(self, request: RequestCache, length: int) -> None:
+        """Forget positions from `length` on and give back the pages only they used."""
+        self._check_live(request)
+        if length < 0 or length > request.length:
+            raise KVCacheError(f"cannot roll cache back to length {length}")
+        blocks = -(-length // self.page_size)
+        for index, group in enumerate(self.groups):
+            table = request.tables[index]
+            if blocks < request.first_live[index]:
+                raise KVCacheError(f"cannot roll back to length {length}: its pages have left the window and were given back")
+            extra = [page for page in table[blocks:] if page >= 0]
+            group.pool.free(extra)
+            del table[blocks:]
+            group.host_table[request.slot, blocks:] = -1
+        request.length = length
+
+    def trim(self, request: RequestCache) -> int:
+        """Give back pages whose every position is outside the window of all future queries."""
+        self._check_live(request)
+        freed = 0
+        for index, group in enumerate(self.groups):
+            window = group.need.window
+            if window is None:
+                continue
+            # the next query sits at position `length` and sees keys j > length - window
+            dead_blocks = max(0, (request.length - window + 1) // self.page_size)
+            table = request.tables[index]
+            dead_blocks = min(dead_blocks, len(table))
+            pages = [table[b] for b in range(request.first_live[index], dead_blocks) if table[b] >= 0]
+            for b in range(request.first_live[index], dead_blocks):
+                table[b] = -1
+            if dead_blocks > request.first_live[index]:
+                group.host_table[request.slot, request.first_live[index]:dead_blocks] = -1
+                request.first_live[index] = dead_blocks
+            group.pool.free(pages)
+            freed += len(pages)
+        return freed
+
+    def release(self, request: RequestCache) -> None:
+        """Give back everything the request holds; releasing twice is harmless."""
+        if request.released:
+            return
+        if self._active.get(request.slot) is not request:
+            raise KVCacheError("cache is not owned by this cache manager")
+        for index, group in enumerate(self.groups):
+            group.pool.free([page for page in request.tables[index] if page >= 0])
+            group.reserved_pages -= request.reserved[index]
+            group.host_table[request.slot, :] = -1
+            request.tables[index] = []
+        request.released = True
+        request.length = 0
+        del self._active[request.slot]
+        heapq.heappush(self._free_slots, request.slot)
+
+    # ------------------------------------------------------------ step support
+    def slot_of_position(self, request: RequestCache, group: int, position: int) -> int:
+        """Physical slot (page * page_size + offset) of a logical position."""
+        page = request.tables[group][position // self.page_size]
+        if page < 0:
+            raise KVCacheError(f"position {position} lies in a page that was given back")
+        return page * self.page_size + position % self.page_size
+
+    def check_invariants(self) -> None:
+        """No page lost, held twice or free while held; used by tests."""
+        for index, group in enumerate(self.groups):
+            held = [page for request in self._active.values() for page in request.tables[index] if page >= 0]
+            if len(held) != len(set(held)):
+                raise AssertionError(f"group {index}: a page is held twice")
+            if len(held) != group.pool.used_pages:
+                raise AssertionError(f"group {index}: {group.pool.used_pages} pages are out but requests hold {len(held)}")
+            if set(held) & set(group.pool._free):
+                raise AssertionError(f"group {index}: a held page is on the free list")
+            for request in self._active.values():
+                row = group.host_table[request.slot]
+                table = request.tables[index]
+                if list(row[:len(table)]) != table or (row[len(table):] != -1).any():
+                    raise AssertionError(f"group {index}: host block table of slot {request.slot} is stale")
+        slots = [request.slot for request in self._active.values()]
+        if len(slots) != len(set(slots)) or set(slots) & set(self._free_slots):
+            raise AssertionError("a state slot is held twice or free while held")
+        if len(slots) + len(self._free_slots) != self.max_requests:
+            raise AssertionError("a state slot was lost")

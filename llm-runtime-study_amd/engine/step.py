@@ -1,0 +1,257 @@
+"""The step function: one batch of (request, its next tokens) through the model.
+
+A step is a list of StepEntry(cache, tokens, want).  A prompt portion and a decoded token
+are the same thing with different lengths; entries may be cut anywhere.  The runner
+
+  1. extends every request's cache by its tokens (taking pages as needed),
+  2. writes the step's metadata into one pinned host buffer and copies it to the device once,
+  3. runs the model on exactly the step's tokens as one ragged batch, reading earlier
+     positions from the paged cache,
+  4. returns float32 logits at the wanted places, in entry order then `want` order,
+  5. on failure rolls every cache back to its length before the step.
+
+Device metadata (all int32): token ids, positions, request row of each token, rows whose
+logits are wanted, per request cumulative query starts, context lengths and state slots,
+and per cache group the physical slot of each token and the block table rows of the batch.
+The layout has fixed offsets given the capacities, so a captured graph can be replayed
+after only the buffer's content has changed.
+
+Reference: mini_llm/model/base.py:161-248 (prefill/decode as extend -> forward -> logits,
+rollback on failure); the reference runs whole prompts alone and decode tokens as a second
+kind of call, here both are one call.
+"""
+
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import Sequence
+
+import numpy as np
+import torch
+
+from ..cache import CacheManager, RequestCache
+from ..errors import GenerationError, KVCacheError
+from ..kernels import ops
+from ..models import DecoderModel
+
+
+@dataclass
+class StepEntry:
+    cache: RequestCache
+    tokens: Sequence[int]
+    want: Sequence[int] = ()
+
+
+class GroupStep:
+    """Per cache group view of the step metadata on the device."""
+
+    def __init__(self, slots: torch.Tensor, block_table: torch.Tensor, page_size: int):
+        self.slots, self.block_table, self.page_size = slots, block_table, page_size
+
+
+class ScratchArena:
+    """Named device buffers that live across steps, so that a step allocates nothing once warm."""
+
+    def __init__(self, device):
+        self.device = device
+        self._buffers: dict = {}
+
+    def get(self, name: str, shape: tuple, dtype: torch.dtype) -> torch.Tensor:
+        rows, rest = shape[0], tuple(shape[1:])
+        key = (name, rest, dtype)
+        buf = self._buffers.get(key)
+        if buf is None or buf.shape[0] < rows:
+            capacity = max(rows, 1 if buf is None else buf.shape[0] * 2)
+            buf = torch.empty((capacity, *rest), dtype=dtype, device=self.device)
+            self._buffers[key] = buf
+        return buf[:rows]
+
+    def reserve(self, name: str, shape: tuple, dtype: torch.dtype) -> None:
+        self.get(name, shape, dtype)
+
+    def bytes(self) -> int:
+        return sum(b.numel() * b.element_size() for b in self._buffers.values())
+
+
+class StepContext:
+    """What the parts see of one step."""
+
+    def __init__(self, runner: "ModelRunner"):
+        self._runner = runner
+        self.dtype = runner.dtype
+        self.device = runner.device
+        self.memo: dict = {}
+        self.T = self.R = self.num_logit_rows = 0
+        self.max_q = self.max_k = 0
+        self.all_decode = False
+        self.host_q_lens: list[int] = []
+        self.host_slots: list[int] = []
+        self.host_positions: list[int] = []   # first position of each request's tokens in this step
+        self.token_ids = self.positions = self.token_request = self.logit_rows = None
+        self.cu_seqlens_q = self.seq_lens_k = self.slot_ids = None
+        self._groups: list[GroupStep] = []
+
+    def scratch(self, name: str, shape: tuple, dtype: torch.dtype) -> torch.Tensor:
+        return self._runner.arena.get(name, shape, dtype)
+
+    def group(self, index: int) -> GroupStep:
+        return self._groups[index]
+
+    def layer_cache(self, schedule_position: int):
+        return self._runner.cache.layer_caches[schedule_position]
+
+
+class ModelRunner:
+    def __init__(self, model: DecoderModel, cache: CacheManager, *, max_step_tokens: int, dtype: torch.dtype, device):
+        if max_step_tokens <= 0:
+            raise GenerationError(f"max_step_tokens must be positive, got {max_step_tokens}")
+        self.model, self.cache, self.dtype, self.device = model, cache, dtype, torch.device(device)
+        self.max_step_tokens = max_step_tokens
+        self.max_requests = cache.max_requests
+        self.arena = ScratchArena(self.device)
+        t, r, g, mb = max_step_tokens, self.max_requests, len(cache.groups), cache.max_blocks
+        # layout of the metadata buffer (int32 elements)
+        self._off = {}
+        cursor = 0
+        for name, size in (("token_ids", t), ("positions", t), ("token_request", t), ("logit_rows", t),
+                           ("cu_seqlens_q", r + 1), ("seq_lens_k", r), ("slot_ids", r)):
+            self._off[name] = (cursor, size)
+            cursor += size
+        for index in range(g):
+            self._off[f"slots{index}"] = (cursor, t)
+            cursor += t
+            self._off[f"table{index}"] = (cursor, r * mb)
+            cursor += r * mb
+        self._meta_size = cursor
+        # two pinned staging buffers used in turn: a buffer is rewritten only after the copy
+        # that read it has finished
+        pin = self.device.type == "cuda"
+        self._hosts = [torch.zeros(cursor, dtype=torch.int32, pin_memory=pin) for _ in range(2)]
+        self._copied = [None, None]
+        self._turn = 0
+        self._host = self._hosts[0]
+        self._host_np = self._host.numpy()
+        self._dev = torch.zeros(cursor, dtype=torch.int32, device=self.device)
+        self.steps_run = 0
+
+    def _next_staging(self) -> None:
+        self._turn ^= 1
+        if self._copied[self._turn] is not None:
+            self._copied[self._turn].synchronize()
+        self._host = self._hosts[self._turn]
+        self._host_np = self._host.numpy()
+
+    def _upload(self) -> None:
+        ops.copy_h2d(self._dev, self._host, self._meta_size)
+        if self.device.type == "cuda":
+            event = self._copied[self._turn] or torch.cuda.Event()
+            event.record()
+            self._copied[self._turn] = event
+
+    def _view(self, name: str, count: int | None = None) -> torch.Tensor:
+        start, size = self._off[name]
+        return self._dev[start:start + (size if count is None else count)]
+
+    def _host_view(self, name: str) -> np.ndarray:
+        start, size = self._off[name]
+        return self._host_np[start:start + size]
+
+    # -------------------------------------------------------------------- step
+    def validate(self, entries: Sequence[StepEntry]) -> None:
+        if not entries:
+            raise GenerationError("a step needs at least one entry")
+        if len(entries) > self.max_requests:
+            raise GenerationError(f"a step holds {len(entries)} requests but at most {self.max_requests} fit")
+        total = 0
+        seen = set()
+        vocab = self.model.spec.vocab_size
+        for entry in entries:
+            n = len(entry.tokens)
+            if n == 0:
+                raise GenerationError("every entry of a step needs at least one token")
+            if id(entry.cache) in seen:
+                raise GenerationError("a request may appear only once in a step")
+            seen.add(id(entry.cache))
+            for token in entry.tokens:
+                if not 0 <= token < vocab:
+                    raise GenerationError(f"input_ids must be within vocabulary [0, {vocab})")
+            for place in entry.want:
+                if not 0 <= place < n:
+                    raise GenerationError(f"wanted place {place} is outside the entry's {n} tokens")
+            total += n
+        if total > self.max_step_tokens:
+            raise GenerationError(f"a step holds {total} tokens but at most {self.max_step_tokens} fit")
+
+    def prepare(self, entries: Sequence[StepEntry]) -> StepContext:
+        """Fill the host metadata for `entries` (caches already extended) and copy it over."""
+        cache, page = self.cache, self.cache.page_size
+        ctx = StepContext(self)
+        self._next_staging()
+        ids, pos, req, rows = (self._host_view(n) for n in ("token_ids", "positions", "token_request", "logit_rows"))
+        cu, lens, slots = (self._host_view(n) for n in ("cu_seqlens_q", "seq_lens_k", "slot_ids"))
+        cursor = n_rows = 0
+        cu[0] = 0
+        for r, entry in enumerate(entries):
+            n = len(entry.tokens)
+            start = entry.cache.length - n
+            ids[cursor:cursor + n] = entry.tokens
+            pos[cursor:cursor + n] = np.arange(start, start + n, dtype=np.int32)
+            req[cursor:cursor + n] = r
+            for place in entry.want:
+                rows[n_rows] = cursor + place
+                n_rows += 1
+            cu[r + 1] = cursor + n
+            lens[r] = entry.cache.length
+            slots[r] = entry.cache.slot
+            ctx.host_q_lens.append(n)
+            ctx.host_slots.append(entry.cache.slot)
+            ctx.host_positions.append(start)
+            cursor += n
+        ctx.T, ctx.R, ctx.num_logit_rows = cursor, len(entries), n_rows
+        ctx.max_q = max(ctx.host_q_lens)
+        ctx.max_k = max(e.cache.length for e in entries)
+        ctx.all_decode = ctx.max_q == 1
+        mb = cache.max_blocks
+        for index, group in enumerate(cache.groups):
+            table = self._host_view(f"table{index}").reshape(self.max_requests, mb)
+            table[:len(entries)] = group.host_table[ctx.host_slots]
+            gslots = self._host_view(f"slots{index}")
+            p = pos[:cursor]
+            pages = table[req[:cursor], p // page]
+            gslots[:cursor] = np.where(pages >= 0, pages * page + p % page, -1)
+        self._upload()
+        self.bind_views(ctx)
+        return ctx
+
+    def bind_views(self, ctx: StepContext) -> None:
+        mb = self.cache.max_blocks
+        ctx.token_ids, ctx.positions = self._view("token_ids", ctx.T), self._view("positions", ctx.T)
+        ctx.token_request, ctx.logit_rows = self._view("token_request", ctx.T), self._view("logit_rows", max(ctx.num_logit_rows, 1))
+        ctx.cu_seqlens_q, ctx.seq_lens_k = self._view("cu_seqlens_q", ctx.R + 1), self._view("seq_lens_k", ctx.R)
+        ctx.slot_ids = self._view("slot_ids", ctx.R)
+        ctx._groups = [
+            GroupStep(self._view(f"slots{i}", ctx.T), self._view(f"table{i}").view(self.max_requests, mb)[:ctx.R], self.cache.page_size)
+            for i in range(len(self.cache.groups))
+        ]
+
+    def step(self, entries: Sequence[StepEntry]) -> torch.Tensor | None:
+        """Run one step; returns float32 logits [wanted, vocab] on the device, or None if none is wanted."""
+        self.validate(entries)
+        before = [entry.cache.length for entry in entries]
+        extended = []
+        try:
+            for entry in entries:
+                self.cache.extend(entry.cache, len(entry.tokens))
+                extended.append(entry)
+            ctx = self.prepare(entries)
+            h = self.model.forward_hidden(ctx)
+            logits = self.model.logits(ctx, h) if ctx.num_logit_rows else None
+        except Exception:
+            for entry, length in zip(extended, before):
+                if not entry.cache.released:
+                    self.cache.rollback(entry.cache, length)
+            raise
+        for entry in entries:
+            self.cache.trim(entry.cache)
+        self.steps_run += 1
+        return logits

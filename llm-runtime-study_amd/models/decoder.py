@@ -1,0 +1,85 @@
+"""Decoder-only language model assembled from a ModelSpec.
+
+Embedding, the scheduled layers, final norm, LM head (reference mini_llm/model/base.py:72-89
+for the stack, mini_llm/model/qwen.py:109-112 for the head; a tied head reuses the embedding
+table).  The forward runs only the tokens of the step it is given, reading and writing the
+caches that the step context carries; it holds no per-request state itself.
+"""
+
+from __future__ import annotations
+
+import torch
+
+from ..kernels import ops
+from ..parts import TensorSpec, create
+from .spec import ModelSpec
+
+
+class DecoderModel:
+    def __init__(self, spec: ModelSpec):
+        spec.validate()
+        self.spec = spec
+        self.layers = [create("block", block) for block in spec.layers]
+        self.final_norm = create("norm", spec.final_norm)
+        self.embedding = self.head = None
+        self.dtype = None
+
+    # ------------------------------------------------------------------ weights
+    def tensors(self) -> dict[str, TensorSpec]:
+        """Every checkpoint tensor by full name."""
+        spec = self.spec
+        out = {spec.embedding_name: TensorSpec((spec.vocab_size, spec.hidden_size), role="embedding")}
+        for index, layer in enumerate(self.layers):
+            prefix = spec.layer_prefix.format(index=index)
+            out.update({f"{prefix}.{name}": t for name, t in layer.tensors().items()})
+        out.update({f"{spec.final_norm_prefix}.{name}": t for name, t in self.final_norm.tensors().items()})
+        out[spec.head_name] = TensorSpec((spec.vocab_size, spec.hidden_size), role="matrix", optional=spec.tie_head)
+        return out
+
+    def bind(self, weights: dict[str, torch.Tensor], dtype: torch.dtype) -> None:
+        """Hand every part its tensors; `dtype` is the activation (and matrix) dtype of the run."""
+        spec = self.spec
+        self.dtype = dtype
+        self.embedding = weights[spec.embedding_name].to(dtype).contiguous()
+        head = weights.get(spec.head_name)
+        self.head = self.embedding if head is None else head.to(dtype).contiguous()
+        for index, layer in enumerate(self.layers):
+            prefix = spec.layer_prefix.format(index=index) + "."
+            layer.bind({n[len(prefix):]: t for n, t in weights.items() if n.startswith(prefix)}, dtype)
+        prefix = spec.final_norm_prefix + "."
+        self.final_norm.bind({n[len(prefix):]: t for n, t in weights.items() if n.startswith(prefix)}, dtype)
+
+    def cache_needs(self) -> list:
+        """What each schedule entry keeps between steps: a need, ("from", entry) or None."""
+        needs = []
+        for entry in self.spec.schedule:
+            if entry.cache_from is not None:
+                needs.append(("from", entry.cache_from))
+            else:
+                needs.append(self.layers[entry.layer].cache_need())
+        return needs
+
+    def weight_bytes(self, with_embedding: bool = False) -> int:
+        """Bytes of weights one decode step reads: every scheduled layer once, and the head."""
+        total = sum(self.layers[e.layer].weight_bytes() for e in self.spec.schedule)
+        total += self.head.numel() * self.head.element_size()
+        if with_embedding and self.head is not self.embedding:
+            total += self.embedding.numel() * self.embedding.element_size()
+        return total
+
+    # ------------------------------------------------------------------ forward
+    def forward_hidden(self, ctx) -> torch.Tensor:
+        """Residual stream [T, H] float32 after the last layer (before the final norm)."""
+        h = ctx.scratch("residual", (ctx.T, self.spec.hidden_size), torch.float32)
+        ops.embed(h, self.embedding, ctx.token_ids, self.spec.embedding_multiplier)
+        for position, entry in enumerate(self.spec.schedule):
+            self.layers[entry.layer].forward(ctx, h, ctx.layer_cache(position))
+        return h
+
+    def logits(self, ctx, h: torch.Tensor) -> torch.Tensor:
+        """float32 logits [n_wanted, V] at the rows of `h` listed in ctx.logit_rows."""
+        n = ctx.num_logit_rows
+        x = self.final_norm.forward(ctx, h, rows=ctx.logit_rows, count=n)
+        out = ctx.scratch("logits", (n, self.spec.vocab_size), torch.float32)
+        ops.gemm(out, x, self.head)
+        return out

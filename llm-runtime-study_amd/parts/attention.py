@@ -1,0 +1,99 @@
+"""Grouped-query causal attention over the paged cache.
+
+Reference mini_llm/nn/attention.py:141-254: q/k/v projections of the normed input, head
+split (head h owns columns h*d..(h+1)*d), optional per-head RMSNorm of q and k over head_dim
+with one weight for all q heads and one for all k heads (Qwen3, 291-302), rotation of q and k
+by the token's absolute position, write of k and v into the cache, softmax(q k^T * scale) v
+over cached positions j <= p (mask rule 231-235; scale 1/sqrt(d) unless given, 95-99), kv head
+h // (nq/nkv) for query head h (18-33), then the output projection without bias.
+
+q, k and v come from one stacked [nq*d + 2*nkv*d, H] product.  When `kv_shared` is set the
+layer owns no keys or values: it projects queries only and attends to the cache of the layer
+it is told to read.  `window` keeps keys with p - window < j <= p.
+"""
+
+from __future__ import annotations
+
+import math
+
+import torch
+
+from ..kernels import ops
+from .base import PagedKVNeed, Part, PartSpec, TensorSpec, create, register
+
+
+class GQAAttention(Part):
+    def __init__(self, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int, *,
+                 position: PartSpec = PartSpec("none"), qk_norm: bool = False, qk_norm_eps: float = 1e-6,
+                 bias: bool = False, scale: float | None = None, window: int | None = None,
+                 kv_shared: bool = False):
+        for name, value in (("hidden_size", hidden_size), ("num_heads", num_heads), ("num_kv_heads", num_kv_heads), ("head_dim", head_dim)):
+            if value <= 0:
+                raise ValueError(f"{name} must be positive, got {value}")
+        if num_heads % num_kv_heads != 0:
+            raise ValueError(f"num_heads must be divisible by num_kv_heads, got {num_heads} and {num_kv_heads}")
+        if scale is not None and (not math.isfinite(scale) or scale <= 0):
+            raise ValueError(f"scale must be finite and positive, got {scale}")
+        if window is not None and window <= 0:
+            raise ValueError(f"window must be positive when given, got {window}")
+        if qk_norm and qk_norm_eps <= 0:
+            raise ValueError(f"qk_norm_eps must be positive, got {qk_norm_eps}")
+        self.hidden_size, self.num_heads, self.num_kv_heads, self.head_dim = hidden_size, num_heads, num_kv_heads, head_dim
+        self.position = create("position", position)
+        self.qk_norm, self.qk_norm_eps, self.bias = qk_norm, qk_norm_eps, bias
+        self.scale = 1.0 / math.sqrt(head_dim) if scale is None else scale
+        self.window, self.kv_shared = window, kv_shared
+        self.w_qkv = self.b_qkv = self.w_o = self.q_norm = self.k_norm = None
+
+    # ------------------------------------------------------------------ weights
+    def tensors(self):
+        h, d = self.hidden_size, self.head_dim
+        names = ("q_proj",) if self.kv_shared else ("q_proj", "k_proj", "v_proj")
+        widths = {"q_proj": self.num_heads * d, "k_proj": self.num_kv_heads * d, "v_proj": self.num_kv_heads * d}
+        specs = {f"{n}.weight": TensorSpec((widths[n], h)) for n in names}
+        if self.bias:
+            specs.update({f"{n}.bias": TensorSpec((widths[n],), role="bias") for n in names})
+        specs["o_proj.weight"] = TensorSpec((h, self.num_heads * d))
+        if self.qk_norm:
+            specs["q_norm.weight"] = TensorSpec((d,), role="norm")
+            if not self.kv_shared:
+                specs["k_norm.weight"] = TensorSpec((d,), role="norm")
+        return specs
+
+    def bind(self, weights, dtype):
+        names = ("q_proj",) if self.kv_shared else ("q_proj", "k_proj", "v_proj")
+        self.w_qkv = torch.cat([weights[f"{n}.weight"] for n in names], 0).to(dtype).contiguous()
+        self.b_qkv = torch.cat([weights[f"{n}.bias"] for n in names], 0).to(dtype).contiguous() if self.bias else None
+        self.w_o = weights["o_proj.weight"].to(dtype).contiguous()
+        if self.qk_norm:
+            self.q_norm = weights["q_norm.weight"]
+            self.k_norm = weights["k_norm.weight"] if not self.kv_shared else self.q_norm
+
+    def weight_bytes(self):
+        return (self.w_qkv.numel() + self.w_o.numel()) * self.w_o.element_size()
+
+    def cache_need(self):
+        if self.kv_shared:
+            return None
+        return PagedKVNeed(self.num_kv_heads, self.head_dim, self.window)
+
+    # ------------------------------------------------------------------ forward
+    def forward(self, ctx, x, residual, cache):
+        if cache is None:
+            raise ValueError("attention needs a paged cache (its own, or the one it is told to read)")
+        t, d, nq = x.shape[0], self.head_dim, self.num_heads
+        nkv = 0 if self.kv_shared else self.num_kv_heads
+        group = ctx.group(cache.group)
+        qkv = ctx.scratch("attn_qkv", (t, (nq + 2 * nkv) * d), ctx.dtype)
+        ops.gemm(qkv, x, self.w_qkv, self.b_qkv)
+        tables = self.position.tables(ctx)
+        cos, sin = tables if tables is not None else (None, None)
+        ops.qk_prep(qkv, nq, nkv, d, self.q_norm, self.k_norm, self.qk_norm_eps, cos, sin,
+                    cache.k_pages, cache.v_pages, group.slots, group.page_size)
+        out = ctx.scratch("attn_out", (t, nq * d), ctx.dtype)
+        ops.attention(out, qkv, cache.k_pages, cache.v_pages, group.block_table, ctx.token_request, ctx.positions,
+                      nq, self.scale, self.window or 0)
+        ops.gemm(residual, out, self.w_o, accumulate=True)
+
+
+register("mixer", "gqa_attention", GQAAttention)

@@ -1,0 +1,101 @@
+"""Interfaces of the parts a layer is put together from, and the registry that builds them.
+
+A part is created from plain parameters (sizes and constants, never a model configuration),
+then told which tensors it wants (`tensors()`), then given them (`bind()`).  It never learns
+which model it is in.  Kinds are looked up by name in one registry per role, so a test or a
+new architecture adds a kind with `register(role, name, cls)` and nothing else changes.
+
+Roles and what each must provide:
+
+  norm           forward(ctx, h, rows=None) -> x        h float32 [T, H] -> activation dtype
+  position       tables(ctx) -> (cos, sin) | None       float32 [T, rot/2] for this step's tokens
+  mixer          cache_need() -> PagedKVNeed | StateNeed | None
+                 forward(ctx, x, residual, cache)       adds its output into residual (float32)
+  feed_forward   forward(ctx, x, residual)              adds its output into residual (float32)
+  block          forward(ctx, h, cache)                 one layer: norms, mixer, feed-forward
+
+`ctx` is the StepContext of engine/step.py: the step's token metadata on the device and a
+scratch arena.  The residual stream `h` is float32 in every precision mode.
+"""
+
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Any, Mapping
+
+import torch
+
+ROLES = ("norm", "position", "mixer", "feed_forward", "block")
+_REGISTRY: dict[str, dict[str, type]] = {role: {} for role in ROLES}
+
+
+def register(role: str, kind: str, cls: type) -> None:
+    """Make `kind` available for `role`; registering a name twice replaces it."""
+    if role not in _REGISTRY:
+        raise KeyError(f"unknown part role {role!r}; roles are {ROLES}")
+    _REGISTRY[role][kind] = cls
+
+
+def create(role: str, spec: "PartSpec"):
+    """Build the part that `spec` names, passing its parameters as keyword arguments."""
+    try:
+        cls = _REGISTRY[role][spec.kind]
+    except KeyError:
+        known = ", ".join(sorted(_REGISTRY.get(role, {}))) or "none"
+        raise KeyError(f"no {role} of kind {spec.kind!r} is registered (known: {known})") from None
+    return cls(**spec.params)
+
+
+@dataclass(frozen=True)
+class PartSpec:
+    """Kind and parameters of one part, as data."""
+
+    kind: str
+    params: Mapping[str, Any] = field(default_factory=dict)
+
+
+@dataclass(frozen=True)
+class TensorSpec:
+    """Shape and role of one checkpoint tensor a part wants.
+
+    role: "matrix" ([out, in] projection), "embedding", "norm" (scale around 1), "bias";
+    the random-weights mode draws each role differently.  dtype "float" follows the
+    checkpoint (bfloat16 stays bfloat16, a tensor stored in 32-bit stays so); "int32"
+    marks integer tables.
+    """
+
+    shape: tuple[int, ...]
+    role: str = "matrix"
+    dtype: str = "float"
+    optional: bool = False
+
+
+@dataclass(frozen=True)
+class PagedKVNeed:
+    """A mixer that keeps keys and values of every position (or of a window) in pages."""
+
+    num_kv_heads: int
+    head_dim: int
+    window: int | None = None
+
+
+@dataclass(frozen=True)
+class StateNeed:
+    """A mixer that keeps a state of fixed size per request."""
+
+    shape: tuple[int, ...]
+    dtype: torch.dtype = torch.float32
+
+
+class Part:
+    """Common behaviour: a part owns no tensor until bind() hands it the ones it asked for."""
+
+    def tensors(self) -> dict[str, TensorSpec]:
+        return {}
+
+    def bind(self, weights: Mapping[str, torch.Tensor], dtype: torch.dtype) -> None:
+        """Take the device tensors named by tensors(); `dtype` is the activation dtype."""
+
+    def weight_bytes(self) -> int:
+        """Bytes of weights that one step reads (for roofline accounting)."""
+        return 0

@@ -1,0 +1,47 @@
+"""Arrangement of norms, mixer and feed-forward in one layer.
+
+PreNormBlock (reference mini_llm/model/qwen.py:58-72):
+    h = h + mixer(norm1(h));  h = h + feed_forward(norm2(h))
+The two sums happen inside the parts, which add into the float32 residual stream.
+"""
+
+from __future__ import annotations
+
+from .base import Part, PartSpec, create, register
+
+
+class PreNormBlock(Part):
+    def __init__(self, mixer: PartSpec, feed_forward: PartSpec, mixer_norm: PartSpec, ff_norm: PartSpec,
+                 names: dict | None = None):
+        self.mixer = create("mixer", mixer)
+        self.feed_forward = create("feed_forward", feed_forward)
+        self.mixer_norm = create("norm", mixer_norm)
+        self.ff_norm = create("norm", ff_norm)
+        self.names = {"mixer": "mixer", "feed_forward": "feed_forward", "mixer_norm": "mixer_norm", "ff_norm": "ff_norm"}
+        self.names.update(names or {})
+
+    def _children(self):
+        return [(self.names[k], getattr(self, k)) for k in ("mixer_norm", "mixer", "ff_norm", "feed_forward")]
+
+    def tensors(self):
+        return {f"{prefix}.{name}": spec for prefix, part in self._children() for name, spec in part.tensors().items()}
+
+    def bind(self, weights, dtype):
+        for prefix, part in self._children():
+            own = {name[len(prefix) + 1:]: t for name, t in weights.items() if name.startswith(prefix + ".")}
+            part.bind(own, dtype)
+
+    def weight_bytes(self):
+        return sum(part.weight_bytes() for _, part in self._children())
+
+    def cache_need(self):
+        return self.mixer.cache_need()
+
+    def forward(self, ctx, h, cache):
+        x = self.mixer_norm.forward(ctx, h)
+        self.mixer.forward(ctx, x, h, cache)
+        x = self.ff_norm.forward(ctx, h)
+        self.feed_forward.forward(ctx, x, h)
+
+
+register("block", "prenorm", PreNormBlock)

@@ -1,0 +1,36 @@
+"""RMSNorm over the last dimension of the float32 residual stream.
+
+Formula (reference mini_llm/nn/norm.py:42-46): y = w * x * rsqrt(mean(x^2) + eps), statistics
+in float32.  The kernel rounds once, at the output, to the activation dtype.
+"""
+
+from __future__ import annotations
+
+from ..kernels import ops
+from .base import Part, TensorSpec, register
+
+
+class RMSNorm(Part):
+    def __init__(self, size: int, eps: float):
+        if size <= 0:
+            raise ValueError(f"size must be positive, got {size}")
+        if eps <= 0:
+            raise ValueError(f"eps must be positive, got {eps}")
+        self.size, self.eps = size, eps
+        self.weight = None
+
+    def tensors(self):
+        return {"weight": TensorSpec((self.size,), role="norm")}
+
+    def bind(self, weights, dtype):
+        self.weight = weights["weight"]
+
+    def forward(self, ctx, h, rows=None, count=None):
+        """Normalise rows of h [*, size] (all, or the `count` rows listed in `rows`)."""
+        n = h.shape[0] if rows is None else count
+        out = ctx.scratch("norm_out", (n, self.size), ctx.dtype)
+        ops.rmsnorm(out, h, self.weight, self.eps, rows=rows)
+        return out
+
+
+register("norm", "rmsnorm", RMSNorm)

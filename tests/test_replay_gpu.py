@@ -1,0 +1,140 @@
+"""Replays the same requests under every way of cutting them and compares each logits row
+with the plain whole-sequence implementation: alone and whole; most in one step and the
+last 32 tokens one by one; portions of changing size down to two tokens; and mixed, up to
+four live requests with so few pages that they are used again.  float32 and bfloat16."""
+
+import subprocess
+import sys
+from pathlib import Path
+
+import numpy as np
+import pytest
+import torch
+
+from tests import traces
+from tests.helpers import TINY_A, TINY_B
+from tests.plain import model as plain
+
+pytestmark = pytest.mark.gpu
+
+ROOT = Path(__file__).resolve().parents[1]
+LENGTHS = {"a": [5, 11, 17, 64, 65, 127, 33, 90], "b": [1, 23, 40, 64, 200, 331, 129, 77, 16]}
+
+
+@pytest.fixture(scope="module")
+def models(tmp_path_factory):
+    """Model folders of both tiny configurations, their requests and the plain logits."""
+    from llm_runtime_study_amd.config import config_from_dict
+    from llm_runtime_study_amd.weights import write_model_dir
+
+    out = {}
+    for name, raw in (("a", TINY_A), ("b", TINY_B)):
+        folder = tmp_path_factory.mktemp(f"model_{name}")
+        write_model_dir(config_from_dict(raw), seed=11 if name == "a" else 12, model_dir=folder, init="scaled")
+        cfg, weights = plain.load_model_dir(folder, torch.float64)
+        rng = np.random.default_rng(5)
+        requests = {f"{name}{i}": rng.integers(0, raw["vocab_size"], n).tolist() for i, n in enumerate(LENGTHS[name])}
+        want = {key: plain.qwen3_forward(weights, cfg, toks) for key, toks in requests.items()}
+        out[name] = (folder, raw, requests, want)
+    return out
+
+
+def run_replay(folder, dtype, steps, max_tokens, tmp_path, page_size=16):
+    from llm_runtime_study_amd.engine import trace
+
+    runner = trace.make_runner(folder, dtype, max_tokens, page_size)
+    out_dir = tmp_path / "logits"
+    trace.replay(runner, traces.strip(steps).splitlines(), out_dir, echo=lambda _: None)
+    runner.cache.check_invariants()
+    assert runner.cache.active_requests == 0 and runner.cache.used_pages() == 0
+    return out_dir
+
+
+def compare(got, want, dtype):
+    """Every row that was asked for, against the plain logits of the same position."""
+    checked = 0
+    for key, rows in got.items():
+        for position, row in rows.items():
+            ref = want[key][position]
+            if dtype == "float32":
+                torch.testing.assert_close(row.double(), ref, rtol=1e-4, atol=1e-4, msg=lambda m: f"{key}@{position}: {m}")
+            else:
+                err = (row.double() - ref).norm() / ref.norm()
+                assert err < 3e-2, f"{key}@{position}: relative error {err:.3g}"
+            checked += 1
+    return checked
+
+
+def round64(n):
+    return -(-n // 64) * 64
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["a", "b"])
+def test_whole(models, name, dtype, tmp_path):
+    folder, raw, requests, want = models[name]
+    steps = traces.whole(requests)
+    out = run_replay(folder, dtype, steps, max(round64(len(t)) for t in requests.values()), tmp_path)
+    got = traces.collect(steps, out, raw["vocab_size"])
+    assert compare(got, want, dtype) == sum(len(t) for t in requests.values())
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["a", "b"])
+def test_prefill_then_last_32_one_by_one(models, name, dtype, tmp_path):
+    folder, raw, requests, want = models[name]
+    steps = traces.prefill_then_decode(requests, tail=32)
+    out = run_replay(folder, dtype, steps, max(round64(len(t)) for t in requests.values()), tmp_path)
+    compare(traces.collect(steps, out, raw["vocab_size"]), want, dtype)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name,page", [("a", 16), ("b", 16), ("b", 4), ("a", 64)])
+def test_portions_of_changing_size(models, name, page, dtype, tmp_path):
+    folder, raw, requests, want = models[name]
+    steps = traces.portions(requests)
+    out = run_replay(folder, dtype, steps, max(round64(len(t)) for t in requests.values()), tmp_path, page)
+    compare(traces.collect(steps, out, raw["vocab_size"]), want, dtype)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name,seed", [("a", 0), ("b", 1), ("b", 2)])
+def test_mixed_with_reused_pages(models, name, seed, dtype, tmp_path):
+    folder, raw, requests, want = models[name]
+    budget = 2 * max(round64(len(t)) for t in requests.values())
+    steps, peak = traces.mixed(requests, seed=seed, max_live=4, max_tokens=budget)
+    assert max(len(s["entries"]) for s in steps) >= 3
+    out = run_replay(folder, dtype, steps, peak, tmp_path)
+    got = traces.collect(steps, out, raw["vocab_size"])
+    assert compare(got, want, dtype) > 50
+    # the pool was smaller than what all requests together need: pages were used again
+    assert peak < sum(round64(len(t)) for t in requests.values())
+
+
+def test_cuts_agree_bit_for_bit_in_float32(models, tmp_path):
+    """In float32 the order of every sum depends on the position alone, so whole, portioned and
+    mixed replays give identical bits."""
+    folder, raw, requests, _ = models["b"]
+    a = traces.whole(requests)
+    b = traces.portions(requests)
+    ga = traces.collect(a, run_replay(folder, "float32", a, 384, tmp_path / "w"), raw["vocab_size"])
+    gb = traces.collect(b, run_replay(folder, "float32", b, 384, tmp_path / "p"), raw["vocab_size"])
+    for key in ga:
+        for position in ga[key]:
+            assert torch.equal(ga[key][position], gb[key][position]), f"{key}@{position}"
+
+
+def test_trace_run_program(models, tmp_path):
+    """The program itself: reads steps on stdin, prints `done <step>` after each, exits 0."""
+    folder, raw, requests, want = models["a"]
+    few = dict(list(requests.items())[:3])
+    steps, peak = traces.mixed(few, seed=3, max_live=3)
+    out = tmp_path / "o"
+    proc = subprocess.run(
+        [sys.executable, str(ROOT / "bin" / "trace_run"), "--model", str(folder), "--dtype", "float32",
+         "--out", str(out), "--max-tokens", str(peak)],
+        input=traces.strip(steps), capture_output=True, text=True, timeout=300)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    done = [line for line in proc.stdout.splitlines() if line.startswith("done ")]
+    assert done == [f"done {s['step']}" for s in steps]
+    compare(traces.collect(steps, out, raw["vocab_size"]), want, "float32")
