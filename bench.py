@@ -1,0 +1,198 @@
+"""Decode and prefill throughput of the Qwen3-8B shape with random weights on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--context 2048] [--layers L]
+
+A step is one decode step of the whole engine (scheduler, step function, sampling) at the
+given batch; `value` is decoded tokens per second.  The same line carries the prefill rate
+of one 2,048-token prompt, the decode step's achieved HBM bandwidth (bytes it must read:
+every weight once plus the cache of the live requests) and decode rates at batch 1 and 64.
+Peaks are MI355X's published ones: HBM 8 TB/s; dense bf16 MFMA 2.5 PFLOP/s.
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import statistics
+import sys
+import time
+from pathlib import Path
+
+ROOT = Path(__file__).resolve().parent
+if str(ROOT) not in sys.path:
+    sys.path.insert(0, str(ROOT))
+
+HBM_PEAK = 8.0e12
+FLOP_PEAK = {"bf16": 2.5e15, "fp32": 157.3e12}
+
+# layer sizes of the Qwen3-8B shape
+QWEN3_8B = {
+    "architectures": ["Qwen3ForCausalLM"], "model_type": "qwen3", "vocab_size": 151936, "hidden_size": 4096,
+    "intermediate_size": 12288, "num_hidden_layers": 36, "num_attention_heads": 32, "num_key_value_heads": 8,
+    "head_dim": 128, "max_position_embeddings": 40960, "rms_norm_eps": 1e-6, "rope_theta": 1000000.0,
+    "hidden_act": "silu", "attention_bias": False, "attention_dropout": 0.0, "tie_word_embeddings": False,
+    "torch_dtype": "bfloat16", "bos_token_id": 151643, "eos_token_id": 151645,
+}
+FULL_LAYERS = QWEN3_8B["num_hidden_layers"]
+
+
+def parse_args():
+    parser = argparse.ArgumentParser()
+    parser.add_argument("--gpus", type=int, default=1)
+    parser.add_argument("--steps", type=int, default=128)
+    parser.add_argument("--warmup", type=int, default=8)
+    parser.add_argument("--batch", type=int, default=8)
+    parser.add_argument("--context", type=int, default=2048)
+    parser.add_argument("--prefill-tokens", type=int, default=2048)
+    parser.add_argument("--layers", type=int, default=FULL_LAYERS, help="fewer layers than the shape has (reported in config)")
+    parser.add_argument("--dtype", choices=("bfloat16", "float32"), default="bfloat16")
+    parser.add_argument("--no-points", action="store_true", help="skip the batch 1 and 64 decode points")
+    parser.add_argument("--no-graph", action="store_true")
+    return parser.parse_args()
+
+
+def matrix_params_per_layer(c) -> int:
+    qkv = (c.num_attention_heads + 2 * c.num_key_value_heads) * c.head_dim * c.hidden_size
+    return qkv + c.hidden_size * c.num_attention_heads * c.head_dim + 3 * c.hidden_size * c.intermediate_size
+
+
+def prefill_flops(c, tokens: int) -> float:
+    """Matrix products of every layer for all tokens, the head for one row, causal attention."""
+    linear = 2.0 * tokens * matrix_params_per_layer(c) * c.num_hidden_layers + 2.0 * c.hidden_size * c.vocab_size
+    attention = 4.0 * (tokens * (tokens + 1) / 2) * c.num_attention_heads * c.head_dim * c.num_hidden_layers
+    return linear + attention
+
+
+def measure_decode(engine, batch: int, context: int, steps: int, warmup: int, seed: int):
+    """Prefill `batch` prompts of `context` random tokens through the scheduler, then time `steps`
+    decode steps.  Returns (seconds per step list, mean context length over the timed steps)."""
+    import numpy as np
+    import torch
+
+    from llm_runtime_study_amd import SamplingConfig
+
+    rng = np.random.default_rng(seed)
+    vocab = engine.config.vocab_size
+    scheduler = engine.create_scheduler()
+    # eos can never end a request early here: random weights make every token about equally likely
+    scheduler._eos = frozenset()
+    for _ in range(batch):
+        scheduler.add_request(rng.integers(0, vocab, context).tolist(), max_new_tokens=warmup + steps + 2 * batch + 8,
+                              sampling=SamplingConfig())
+    times = []
+    with torch.cuda.device(engine.device), torch.cuda.stream(engine.stream):
+        # prefill phase: until every request has sampled its first token
+        produced = 0
+        while produced < batch:
+            produced += sum(1 for _, e in scheduler.step() if e.prompt_token_count is not None)
+        for _ in range(warmup):
+            scheduler.step()
+        engine.synchronize()
+        for _ in range(steps):
+            started = time.perf_counter()
+            events = scheduler.step()
+            engine.synchronize()
+            times.append(time.perf_counter() - started)
+            assert len(events) == batch
+        scheduler.abort_all()
+    # requests entered one step apart, so they are up to `batch` tokens apart in length
+    mean_context = context + 1 + warmup + (batch - 1) / 2 + (steps - 1) / 2
+    return times, mean_context
+
+
+def measure_prefill(engine, tokens: int, repeats: int, seed: int):
+    import numpy as np
+    import torch
+
+    from llm_runtime_study_amd.engine.step import StepEntry
+
+    rng = np.random.default_rng(seed)
+    runner = engine.runner
+    times = []
+    with torch.cuda.device(engine.device), torch.cuda.stream(engine.stream):
+        for i in range(repeats + 1):
+            prompt = rng.integers(0, engine.config.vocab_size, tokens).tolist()
+            cache = runner.cache.admit(f"prefill{i}")
+            engine.synchronize()
+            started = time.perf_counter()
+            runner.step([StepEntry(cache, prompt, [tokens - 1])])
+            engine.synchronize()
+            times.append(time.perf_counter() - started)
+            runner.cache.release(cache)
+    return times[1:]  # the first run warms up buffers
+
+
+def main() -> int:
+    args = parse_args()
+    if args.gpus != 1:
+        print(f"bench.py measures one GPU only: --gpus {args.gpus} is not supported by this single-GPU engine")
+        return 2
+    import torch
+
+    from llm_runtime_study_amd import Engine
+    from llm_runtime_study_amd.config import config_from_dict
+
+    raw = dict(QWEN3_8B, num_hidden_layers=args.layers)
+    config = config_from_dict(raw)
+    max_batch = args.batch if args.no_points else max(args.batch, 64)
+    max_seq_len = args.context + args.steps + args.warmup + 2 * max_batch + 64
+    max_seq_len = max(max_seq_len, args.prefill_tokens)
+    engine = Engine.from_config(config, seed=0, dtype=args.dtype, max_seq_len=max_seq_len, max_batch_size=max_batch,
+                                max_num_batched_tokens=max(2048, args.prefill_tokens), use_cuda_graph=not args.no_graph)
+    dtype_name = "bf16" if args.dtype == "bfloat16" else "fp32"
+
+    prefill_times = measure_prefill(engine, args.prefill_tokens, repeats=3, seed=1)
+    prefill_s = statistics.median(prefill_times)
+    flops = prefill_flops(config, args.prefill_tokens)
+
+    times, mean_context = measure_decode(engine, args.batch, args.context, args.steps, args.warmup, seed=2)
+    total = sum(times)
+    step_s = total / len(times)
+    weight_bytes = engine.model.weight_bytes()
+    kv_bytes = args.batch * mean_context * engine.cache_manager.bytes_per_token()
+    achieved = (weight_bytes + kv_bytes) / step_s
+
+    points = {}
+    if not args.no_points:
+        for batch in (1, 64):
+            point_steps = min(args.steps, 64)
+            t, _ = measure_decode(engine, batch, args.context, point_steps, min(args.warmup, 4), seed=3 + batch)
+            points[f"decode_b{batch}"] = round(batch * len(t) / sum(t), 2)
+
+    line = {
+        "metric": f"decode tok/s at batch {args.batch} (Qwen3-8B shape)",
+        "value": round(args.batch * len(times) / total, 2),
+        "unit": "tok/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(step_s * 1e3, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": dtype_name,
+        "data": "synthetic (seeded uniform random token ids, random weights N(0, 0.02))",
+        "config": {
+            "model": "Qwen3-8B shape", "layers": args.layers, "layers_of_shape": FULL_LAYERS,
+            "hidden_size": config.hidden_size, "intermediate_size": config.intermediate_size,
+            "num_attention_heads": config.num_attention_heads, "num_key_value_heads": config.num_key_value_heads,
+            "head_dim": config.head_dim, "vocab_size": config.vocab_size, "global_batch": args.batch,
+            "seq_len": args.context, "new_tokens": args.steps + args.warmup, "page_size": engine.page_size,
+            "prefill_tokens": args.prefill_tokens, "hip_graph": bool(engine.runner.use_graph), "parallelism": "single GPU",
+        },
+        "prefill": {
+            "value": round(args.prefill_tokens / prefill_s, 1), "tokens": args.prefill_tokens,
+            "ms": round(prefill_s * 1e3, 3), "frac": round(flops / prefill_s / FLOP_PEAK[dtype_name], 4),
+        },
+        "roofline": {
+            "bound": "hbm", "achieved": round(achieved / 1e9, 1), "peak": HBM_PEAK / 1e9, "unit": "GB/s",
+            "frac": round(achieved / HBM_PEAK, 4),
+        },
+        "points": points,
+    }
+    print(json.dumps(line))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

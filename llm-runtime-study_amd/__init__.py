@@ -1,1 +1,27 @@
-"""MI355X-native one-GPU inference runtime for Qwen3 dense models."""
+"""MI355X-native one-GPU inference runtime for Qwen3 dense models.
+
+    from llm_runtime_study_amd import Engine, SamplingConfig
+    engine = Engine.from_model_dir("model_dir", max_batch_size=8)
+    for index, event in engine.generate([[1, 2, 3]], max_new_tokens=16):
+        ...
+"""
+
+from .errors import (CheckpointError, CheckpointValidationError, ConfigError, EngineError, GenerationError,
+                     KernelError, KVCacheError, SamplingError, TokenizerError)
+from .sampling.config import SamplingConfig
+from .text.chat import ChatMessage
+
+__all__ = ["ChatMessage", "CheckpointError", "CheckpointValidationError", "ConfigError", "Engine", "EngineError",
+           "GenerationError", "GenerationEvent", "KVCacheError", "KernelError", "SamplingConfig", "SamplingError",
+           "TokenizerError"]
+
+
+def __getattr__(name):
+    # the engine pulls in torch and the kernel library; load it on first use
+    if name == "Engine":
+        from .engine.engine import Engine
+        return Engine
+    if name == "GenerationEvent":
+        from .engine.scheduler import GenerationEvent
+        return GenerationEvent
+    raise AttributeError(name)

@@ -1,0 +1,148 @@
+"""Engine: a loaded model, its cache pool, the step function and the generation entry points.
+
+Reference mini_llm/engine.py:144-352 (`Engine.from_model_dir(...)`, `.generate(...)`,
+`.create_scheduler()`, cache accounting, `.synchronize()`); names and defaults of the
+options are the reference's.  Differences: the device is the GPU only, `auto` precision is
+bfloat16, prompts may be token ids as well as chat messages, and prompts are prefilled in
+portions under `max_num_batched_tokens` next to decoding requests.
+"""
+
+from __future__ import annotations
+
+import time
+from pathlib import Path
+from typing import Iterator, Sequence
+
+import torch
+
+from ..cache import CacheManager
+from ..errors import EngineError
+from ..sampling import Sampler, SamplingConfig
+from ..text import TextTokenizer
+from ..config import load_config
+from .loading import load_model, random_model, resolve_device, resolve_dtype
+from .scheduler import BatchScheduler, GenerationEvent, generate as _generate
+from .step import ModelRunner
+
+DEFAULT_PAGE_SIZE = 16
+DEFAULT_STEP_TOKENS = 2048
+
+
+class Engine:
+    def __init__(self, config, model, *, device, dtype, max_seq_len: int = 4096, max_batch_size: int = 1,
+                 cache_backend: str = "paged", use_cuda_graph: bool = True, page_size: int = DEFAULT_PAGE_SIZE,
+                 max_num_batched_tokens: int | None = None, num_pages: int | None = None, tokenizer=None,
+                 load_seconds: float = 0.0):
+        if max_batch_size <= 0:
+            raise EngineError("max_batch_size must be positive")
+        if cache_backend != "paged":
+            raise EngineError(f"unsupported cache backend {cache_backend!r}; this runtime has the 'paged' cache only")
+        config.validate_context_length(max_seq_len)
+        self.config, self.model, self.device, self.dtype = config, model, device, dtype
+        self.max_seq_len, self.max_batch_size = max_seq_len, max_batch_size
+        self.cache_backend, self.use_cuda_graph = cache_backend, use_cuda_graph
+        self.page_size = page_size
+        self.max_num_batched_tokens = max(max_batch_size, max_num_batched_tokens or min(DEFAULT_STEP_TOKENS, max_seq_len))
+        self.num_pages = num_pages
+        self.tokenizer = tokenizer
+        self.load_seconds = load_seconds
+        self.quantization = "dense"
+        self.stream = torch.cuda.Stream(device)
+        self._runner: ModelRunner | None = None
+        self._sampler = Sampler(device)
+
+    # ---------------------------------------------------------------- loading
+    @classmethod
+    def from_model_dir(cls, model_dir, *, device="auto", dtype="auto", max_seq_len: int = 4096, max_batch_size: int = 1,
+                       cache_backend: str = "paged", use_cuda_graph: bool = True, **options) -> "Engine":
+        """Load config.json and the safetensors weights of `model_dir` onto the GPU."""
+        started = time.perf_counter()
+        config = load_config(model_dir)
+        config.validate_context_length(max_seq_len)
+        selected_device, selected_dtype = resolve_device(device), resolve_dtype(dtype)
+        config, model = load_model(model_dir, selected_dtype, selected_device, config)
+        tokenizer = TextTokenizer.from_model_dir(model_dir, config.vocab_size)
+        engine = cls(config, model, device=selected_device, dtype=selected_dtype, max_seq_len=max_seq_len,
+                     max_batch_size=max_batch_size, cache_backend=cache_backend, use_cuda_graph=use_cuda_graph,
+                     tokenizer=tokenizer, **options)
+        engine.synchronize()
+        engine.load_seconds = time.perf_counter() - started
+        return engine
+
+    @classmethod
+    def from_config(cls, config, *, seed: int = 0, init: str = "normal", device="auto", dtype="auto", **options) -> "Engine":
+        """Random weights made on the device for `config` (a typed configuration)."""
+        started = time.perf_counter()
+        selected_device, selected_dtype = resolve_device(device), resolve_dtype(dtype)
+        model = random_model(config, seed, selected_dtype, selected_device, init)
+        engine = cls(config, model, device=selected_device, dtype=selected_dtype, **options)
+        engine.synchronize()
+        engine.load_seconds = time.perf_counter() - started
+        return engine
+
+    # ------------------------------------------------------------------ cache
+    @property
+    def runner(self) -> ModelRunner:
+        """The step function over this engine's cache pool, made on first use: the pool holds
+        max_seq_len * max_batch_size tokens unless `num_pages` says otherwise."""
+        if self._runner is None:
+            pages = self.num_pages or -(-self.max_seq_len // self.page_size) * self.max_batch_size
+            cache = CacheManager(self.model.cache_needs(), page_size=self.page_size, num_pages=pages,
+                                 max_requests=self.max_batch_size, max_seq_len=self.max_seq_len,
+                                 dtype=self.dtype, device=self.device)
+            self._runner = ModelRunner(self.model, cache, max_step_tokens=self.max_num_batched_tokens,
+                                       dtype=self.dtype, device=self.device, use_graph=self.use_cuda_graph)
+        return self._runner
+
+    @property
+    def cache_manager(self) -> CacheManager:
+        return self.runner.cache
+
+    @property
+    def last_cache_capacity(self) -> int:
+        return self.cache_manager.last_allocation_tokens
+
+    @property
+    def last_cache_num_bytes(self) -> int:
+        return self.cache_manager.last_allocation_tokens * self.cache_manager.bytes_per_token()
+
+    # ------------------------------------------------------------- generation
+    def create_scheduler(self) -> BatchScheduler:
+        return BatchScheduler(
+            self.runner, self._sampler, max_batch_size=self.max_batch_size, max_seq_len=self.max_seq_len,
+            max_step_tokens=self.max_num_batched_tokens, eos_token_ids=self.config.eos_token_ids,
+            vocab_size=self.config.vocab_size, tokenizer=self.tokenizer, synchronize=self.synchronize)
+
+    def generate(self, message_batches: Sequence, *, max_new_tokens: int, sampling: SamplingConfig = SamplingConfig(),
+                 enable_thinking: bool = False) -> Iterator[tuple[int, GenerationEvent]]:
+        """Events (request index, GenerationEvent) of the given prompts, each a list of ChatMessage
+        or of token ids; requests beyond max_batch_size wait for a free slot."""
+        scheduler = self.create_scheduler()
+        inner = _generate(scheduler, message_batches, max_new_tokens=max_new_tokens, sampling=sampling,
+                          enable_thinking=enable_thinking)
+
+        def on_stream():
+            try:
+                while True:
+                    with torch.cuda.device(self.device), torch.cuda.stream(self.stream):
+                        try:
+                            item = next(inner)
+                        except StopIteration:
+                            return
+                    yield item
+            finally:
+                inner.close()
+
+        return on_stream()
+
+    def generate_tokens(self, prompts: Sequence[Sequence[int]], *, max_new_tokens: int,
+                        sampling: SamplingConfig = SamplingConfig()) -> list[list[int]]:
+        """Token ids generated for each prompt (a convenience over generate())."""
+        out = [[] for _ in prompts]
+        for index, event in self.generate([list(p) for p in prompts], max_new_tokens=max_new_tokens, sampling=sampling):
+            if event.token_id is not None:
+                out[index].append(event.token_id)
+        return out
+
+    def synchronize(self) -> None:
+        torch.cuda.synchronize(self.device)

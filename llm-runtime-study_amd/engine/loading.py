@@ -45,9 +45,9 @@ def resolve_dtype(requested="auto") -> torch.dtype:
     raise EngineError(f"unsupported dtype {requested!r}; expected auto, {', '.join(DTYPES)}")
 
 
-def load_model(model_dir, dtype: torch.dtype, device) -> tuple:
+def load_model(model_dir, dtype: torch.dtype, device, config=None) -> tuple:
     """(typed configuration, bound DecoderModel) of a model folder."""
-    config = load_config(model_dir)
+    config = load_config(model_dir) if config is None else config
     spec = spec_for(config)
     model = DecoderModel(spec)
     checkpoint = Checkpoint.from_model_dir(model_dir)

@@ -55,6 +55,7 @@ class ScratchArena:
     def __init__(self, device):
         self.device = device
         self._buffers: dict = {}
+        self.generation = 0   # bumped whenever a buffer is (re)allocated: captured graphs then hold stale addresses
 
     def get(self, name: str, shape: tuple, dtype: torch.dtype) -> torch.Tensor:
         rows, rest = shape[0], tuple(shape[1:])
@@ -64,6 +65,7 @@ class ScratchArena:
             capacity = max(rows, 1 if buf is None else buf.shape[0] * 2)
             buf = torch.empty((capacity, *rest), dtype=dtype, device=self.device)
             self._buffers[key] = buf
+            self.generation += 1
         return buf[:rows]
 
     def reserve(self, name: str, shape: tuple, dtype: torch.dtype) -> None:
@@ -102,13 +104,18 @@ class StepContext:
 
 
 class ModelRunner:
-    def __init__(self, model: DecoderModel, cache: CacheManager, *, max_step_tokens: int, dtype: torch.dtype, device):
+    def __init__(self, model: DecoderModel, cache: CacheManager, *, max_step_tokens: int, dtype: torch.dtype, device,
+                 use_graph: bool = False):
         if max_step_tokens <= 0:
             raise GenerationError(f"max_step_tokens must be positive, got {max_step_tokens}")
         self.model, self.cache, self.dtype, self.device = model, cache, dtype, torch.device(device)
         self.max_step_tokens = max_step_tokens
         self.max_requests = cache.max_requests
         self.arena = ScratchArena(self.device)
+        # decode-only steps are captured in a HIP graph per padded batch size and replayed
+        self.use_graph = use_graph and model.graph_safe()
+        self._graphs: dict[int, tuple] = {}   # bucket -> (handle, arena generation, logits tensor)
+        self.graph_replays = 0
         t, r, g, mb = max_step_tokens, self.max_requests, len(cache.groups), cache.max_blocks
         # layout of the metadata buffer (int32 elements)
         self._off = {}
@@ -182,8 +189,12 @@ class ModelRunner:
         if total > self.max_step_tokens:
             raise GenerationError(f"a step holds {total} tokens but at most {self.max_step_tokens} fit")
 
-    def prepare(self, entries: Sequence[StepEntry]) -> StepContext:
-        """Fill the host metadata for `entries` (caches already extended) and copy it over."""
+    def prepare(self, entries: Sequence[StepEntry], pad_to: int = 0) -> StepContext:
+        """Fill the host metadata for `entries` (caches already extended) and copy it over.
+
+        With `pad_to` (decode-only steps) the batch is filled up to that many rows with rows that
+        belong to no request: token 0 at position 0, written to and read from the trash page, and
+        logits are produced for every row, so that the step's shape depends on `pad_to` alone."""
         cache, page = self.cache, self.cache.page_size
         ctx = StepContext(self)
         self._next_staging()
@@ -207,14 +218,30 @@ class ModelRunner:
             ctx.host_slots.append(entry.cache.slot)
             ctx.host_positions.append(start)
             cursor += n
-        ctx.T, ctx.R, ctx.num_logit_rows = cursor, len(entries), n_rows
+        real = len(entries)
         ctx.max_q = max(ctx.host_q_lens)
         ctx.max_k = max(e.cache.length for e in entries)
         ctx.all_decode = ctx.max_q == 1
+        if pad_to > real:
+            extra = pad_to - real
+            ids[cursor:cursor + extra] = 0
+            pos[cursor:cursor + extra] = 0
+            req[cursor:cursor + extra] = np.arange(real, pad_to, dtype=np.int32)
+            cu[real + 1:pad_to + 1] = np.arange(cursor + 1, cursor + extra + 1, dtype=np.int32)
+            lens[real:pad_to] = 1
+            slots[real:pad_to] = 0
+            cursor += extra
+        if pad_to:
+            rows[:cursor] = np.arange(cursor, dtype=np.int32)
+            n_rows = cursor
+        ctx.T, ctx.R, ctx.num_logit_rows = cursor, max(real, pad_to), n_rows
         mb = cache.max_blocks
         for index, group in enumerate(cache.groups):
             table = self._host_view(f"table{index}").reshape(self.max_requests, mb)
-            table[:len(entries)] = group.host_table[ctx.host_slots]
+            table[:real] = group.host_table[ctx.host_slots]
+            if pad_to > real:
+                table[real:pad_to] = -1
+                table[real:pad_to, 0] = cache.trash_page(index)
             gslots = self._host_view(f"slots{index}")
             p = pos[:cursor]
             pages = table[req[:cursor], p // page]
@@ -243,9 +270,13 @@ class ModelRunner:
             for entry in entries:
                 self.cache.extend(entry.cache, len(entry.tokens))
                 extended.append(entry)
-            ctx = self.prepare(entries)
-            h = self.model.forward_hidden(ctx)
-            logits = self.model.logits(ctx, h) if ctx.num_logit_rows else None
+            bucket = self._graph_bucket(entries)
+            if bucket:
+                logits = self._step_graph(entries, bucket)
+            else:
+                ctx = self.prepare(entries)
+                h = self.model.forward_hidden(ctx)
+                logits = self.model.logits(ctx, h) if ctx.num_logit_rows else None
         except Exception:
             for entry, length in zip(extended, before):
                 if not entry.cache.released:
@@ -255,3 +286,54 @@ class ModelRunner:
             self.cache.trim(entry.cache)
         self.steps_run += 1
         return logits
+
+    # ------------------------------------------------------------------ graphs
+    def _graph_bucket(self, entries: Sequence[StepEntry]) -> int:
+        """Padded batch size for a decode-only step that may run as a graph, else 0."""
+        if not self.use_graph or any(len(e.tokens) != 1 for e in entries):
+            return 0
+        if torch.cuda.current_stream(self.device).cuda_stream == 0:
+            return 0  # the default stream cannot be captured
+        bucket = 1
+        while bucket < len(entries):
+            bucket *= 2
+        bucket = min(bucket, self.max_requests)
+        return bucket if bucket <= self.max_step_tokens else 0
+
+    def _step_graph(self, entries: Sequence[StepEntry], bucket: int) -> torch.Tensor | None:
+        """Replay (capturing first if needed) the graph of a decode step padded to `bucket` rows.
+
+        Logits come back for the wanted rows of the real entries only."""
+        ctx = self.prepare(entries, pad_to=bucket)
+        graph = self._graphs.get(bucket)
+        if graph is None or graph[1] != self.arena.generation:
+            if graph is not None:
+                ops.graph_destroy(graph[0])
+                del self._graphs[bucket]
+            # an eager run first: it sizes every scratch buffer, so that capture allocates nothing
+            h = self.model.forward_hidden(ctx)
+            logits = self.model.logits(ctx, h)
+            generation = self.arena.generation
+            ctx.memo.clear()
+            ops.graph_begin()
+            try:
+                h = self.model.forward_hidden(ctx)
+                logits = self.model.logits(ctx, h)
+            finally:
+                handle = ops.graph_end()
+            if self.arena.generation != generation:
+                ops.graph_destroy(handle)
+                raise GenerationError("scratch buffers moved during graph capture")
+            graph = self._graphs[bucket] = (handle, generation, logits)
+        ops.graph_launch(graph[0])
+        self.graph_replays += 1
+        wanted = [r for r, entry in enumerate(entries) if len(entry.want)]
+        if not wanted:
+            return None
+        logits = graph[2]
+        return logits[:len(entries)] if len(wanted) == len(entries) else logits[wanted]
+
+    def drop_graphs(self) -> None:
+        for handle, _, _ in self._graphs.values():
+            ops.graph_destroy(handle)
+        self._graphs.clear()

@@ -59,6 +59,11 @@ class DecoderModel:
                 needs.append(self.layers[entry.layer].cache_need())
         return needs
 
+    def graph_safe(self) -> bool:
+        """Whether a step launches only this library's kernels on preallocated buffers, so that it
+        can be captured in a HIP graph: every part must say so itself."""
+        return all(getattr(layer, "graph_safe", False) for layer in self.layers)
+
     def weight_bytes(self, with_embedding: bool = False) -> int:
         """Bytes of weights one decode step reads: every scheduled layer once, and the head."""
         total = sum(self.layers[e.layer].weight_bytes() for e in self.spec.schedule)

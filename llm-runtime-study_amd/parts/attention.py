@@ -23,6 +23,8 @@ from .base import PagedKVNeed, Part, PartSpec, TensorSpec, create, register
 
 
 class GQAAttention(Part):
+    graph_safe = True  # launches only library kernels on arena buffers
+
     def __init__(self, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int, *,
                  position: PartSpec = PartSpec("none"), qk_norm: bool = False, qk_norm_eps: float = 1e-6,
                  bias: bool = False, scale: float | None = None, window: int | None = None,

@@ -37,6 +37,10 @@ class PreNormBlock(Part):
     def cache_need(self):
         return self.mixer.cache_need()
 
+    @property
+    def graph_safe(self) -> bool:
+        return all(getattr(part, "graph_safe", False) for _, part in self._children())
+
     def forward(self, ctx, h, cache):
         x = self.mixer_norm.forward(ctx, h)
         self.mixer.forward(ctx, x, h, cache)

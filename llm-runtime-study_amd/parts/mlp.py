@@ -14,6 +14,8 @@ from .base import Part, TensorSpec, register
 
 
 class SwiGLU(Part):
+    graph_safe = True  # launches only library kernels on arena buffers
+
     def __init__(self, hidden_size: int, intermediate_size: int):
         if hidden_size <= 0 or intermediate_size <= 0:
             raise ValueError("hidden_size and intermediate_size must be positive")

@@ -11,6 +11,8 @@ from .base import Part, TensorSpec, register
 
 
 class RMSNorm(Part):
+    graph_safe = True  # launches only library kernels on arena buffers
+
     def __init__(self, size: int, eps: float):
         if size <= 0:
             raise ValueError(f"size must be positive, got {size}")

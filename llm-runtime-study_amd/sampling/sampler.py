@@ -1,0 +1,61 @@
+"""Token choice for a batch of logits rows, on the device.
+
+Greedy rows take the lowest index among the largest logits.  Other rows are filtered by
+top-k and top-p (rule of the reference, mini_llm/sampling.py:40-69) and drawn from
+softmax(logits / temperature) (89-91).  The reference draws on the CPU with a torch
+generator per request; here the draw is a device kernel keyed by (request seed, number of
+tokens the request has drawn), so a request's tokens depend on its own seed only, not on
+its batch mates; the stream of numbers is not torch's.  A request without a seed gets one
+from the operating system when it is admitted.
+"""
+
+from __future__ import annotations
+
+import random
+from dataclasses import dataclass
+
+import torch
+
+from ..errors import SamplingError
+from ..kernels import ops
+from .config import SamplingConfig
+
+_system_random = random.SystemRandom()
+
+
+def request_seed(config: SamplingConfig) -> int:
+    return config.seed if config.seed is not None else _system_random.getrandbits(62)
+
+
+@dataclass
+class SamplingRow:
+    config: SamplingConfig
+    seed: int
+    counter: int  # tokens this request has drawn so far
+
+
+class Sampler:
+    def __init__(self, device):
+        self.device = torch.device(device)
+
+    def choose(self, logits: torch.Tensor, rows: list[SamplingRow]) -> list[int]:
+        """One token per row of `logits` [R, V] float32 (filters the sampled rows in place)."""
+        if logits.dim() != 2 or logits.shape[0] != len(rows) or logits.dtype != torch.float32:
+            raise SamplingError(f"logits must be float32 [rows, vocabulary] with {len(rows)} rows, got {tuple(logits.shape)} {logits.dtype}")
+        vocab = logits.shape[1]
+        for row in rows:
+            if row.config.top_k is not None and row.config.top_k > vocab:
+                raise SamplingError(f"top_k {row.config.top_k} exceeds vocabulary size {vocab}")
+        out = torch.empty(len(rows), dtype=torch.int32, device=self.device)
+        if all(row.config.greedy for row in rows):
+            ops.choose_tokens(out, logits)
+            return out.cpu().tolist()
+        temperature = torch.tensor([row.config.temperature for row in rows], dtype=torch.float32, device=self.device)
+        seeds = torch.tensor([row.seed for row in rows], dtype=torch.int64, device=self.device)
+        counters = torch.tensor([row.counter for row in rows], dtype=torch.int32, device=self.device)
+        if any((row.config.top_k is not None and row.config.top_k < vocab) or row.config.top_p < 1.0 for row in rows if not row.config.greedy):
+            top_k = torch.tensor([row.config.top_k or 0 for row in rows], dtype=torch.int32, device=self.device)
+            top_p = torch.tensor([row.config.top_p for row in rows], dtype=torch.float32, device=self.device)
+            ops.filter_logits(logits, temperature, top_k, top_p)
+        ops.choose_tokens(out, logits, temperature, seeds, counters)
+        return out.cpu().tolist()
