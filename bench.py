@@ -73,9 +73,7 @@ def measure_decode(engine, batch: int, context: int, steps: int, warmup: int, se
 
     rng = np.random.default_rng(seed)
     vocab = engine.config.vocab_size
-    scheduler = engine.create_scheduler()
-    # eos can never end a request early here: random weights make every token about equally likely
-    scheduler._eos = frozenset()
+    scheduler = engine.create_scheduler(ignore_eos=True)   # every request runs to its length limit
     for _ in range(batch):
         scheduler.add_request(rng.integers(0, vocab, context).tolist(), max_new_tokens=warmup + steps + 2 * batch + 8,
                               sampling=SamplingConfig())

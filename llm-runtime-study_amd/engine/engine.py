@@ -107,17 +107,19 @@ class Engine:
         return self.cache_manager.last_allocation_tokens * self.cache_manager.bytes_per_token()
 
     # ------------------------------------------------------------- generation
-    def create_scheduler(self) -> BatchScheduler:
+    def create_scheduler(self, ignore_eos: bool = False) -> BatchScheduler:
+        """A continuous-batching scheduler over this engine's cache and step function; with
+        `ignore_eos` requests run to their length limits (benchmarks with random weights)."""
         return BatchScheduler(
             self.runner, self._sampler, max_batch_size=self.max_batch_size, max_seq_len=self.max_seq_len,
-            max_step_tokens=self.max_num_batched_tokens, eos_token_ids=self.config.eos_token_ids,
+            max_step_tokens=self.max_num_batched_tokens, eos_token_ids=() if ignore_eos else self.config.eos_token_ids,
             vocab_size=self.config.vocab_size, tokenizer=self.tokenizer, synchronize=self.synchronize)
 
     def generate(self, message_batches: Sequence, *, max_new_tokens: int, sampling: SamplingConfig = SamplingConfig(),
-                 enable_thinking: bool = False) -> Iterator[tuple[int, GenerationEvent]]:
+                 enable_thinking: bool = False, ignore_eos: bool = False) -> Iterator[tuple[int, GenerationEvent]]:
         """Events (request index, GenerationEvent) of the given prompts, each a list of ChatMessage
         or of token ids; requests beyond max_batch_size wait for a free slot."""
-        scheduler = self.create_scheduler()
+        scheduler = self.create_scheduler(ignore_eos)
         inner = _generate(scheduler, message_batches, max_new_tokens=max_new_tokens, sampling=sampling,
                           enable_thinking=enable_thinking)
 
@@ -136,10 +138,11 @@ class Engine:
         return on_stream()
 
     def generate_tokens(self, prompts: Sequence[Sequence[int]], *, max_new_tokens: int,
-                        sampling: SamplingConfig = SamplingConfig()) -> list[list[int]]:
+                        sampling: SamplingConfig = SamplingConfig(), ignore_eos: bool = False) -> list[list[int]]:
         """Token ids generated for each prompt (a convenience over generate())."""
         out = [[] for _ in prompts]
-        for index, event in self.generate([list(p) for p in prompts], max_new_tokens=max_new_tokens, sampling=sampling):
+        for index, event in self.generate([list(p) for p in prompts], max_new_tokens=max_new_tokens, sampling=sampling,
+                                          ignore_eos=ignore_eos):
             if event.token_id is not None:
                 out[index].append(event.token_id)
         return out

@@ -68,3 +68,28 @@ def device_weights(model: DecoderModel, seed: int, dtype: torch.dtype, device, i
     expected = model.tensors()
     return {name: _draw(expected[name], init, generator, device).to(torch.int32 if expected[name].dtype == "int32" else dtype)
             for name in sorted(expected) if not expected[name].optional}
+
+
+def main(argv=None) -> int:
+    """`python -m llm_runtime_study_amd.weights.random_init --config config.json --seed 0 --out DIR`"""
+    import argparse
+
+    from ..config import config_from_dict
+
+    parser = argparse.ArgumentParser(description="Write a model folder with random weights for a config.json.")
+    parser.add_argument("--config", type=Path, required=True, help="a config.json (or a folder holding one)")
+    parser.add_argument("--seed", type=int, default=0)
+    parser.add_argument("--out", type=Path, required=True)
+    parser.add_argument("--init", choices=("normal", "scaled"), default="normal")
+    args = parser.parse_args(argv)
+    path = args.config / "config.json" if args.config.is_dir() else args.config
+    config = config_from_dict(json.loads(path.read_text()))
+    write_model_dir(config, args.seed, args.out, args.init)
+    print(f"wrote {args.out}/config.json and model.safetensors")
+    return 0
+
+
+if __name__ == "__main__":
+    import sys
+
+    sys.exit(main())

@@ -1,0 +1,85 @@
+"""Command line: options, streaming, metrics and error exit code, with a fake engine (CPU)."""
+
+import io
+from types import SimpleNamespace
+
+import pytest
+
+from llm_runtime_study_amd import cli
+from llm_runtime_study_amd.engine.scheduler import GenerationEvent
+from llm_runtime_study_amd.errors import ConfigError
+from llm_runtime_study_amd.sampling import SamplingConfig
+from llm_runtime_study_amd.errors import SamplingError
+
+
+def test_parser_has_the_reference_options_and_defaults():
+    # reference mini_llm/cli.py:32-64
+    args = cli.build_parser().parse_args(["--model", "m", "--prompt", "hi"])
+    assert (args.max_new_tokens, args.max_seq_len, args.temperature, args.top_k, args.top_p, args.seed) == (128, 4096, 0.0, None, 1.0, None)
+    assert (args.device, args.dtype, args.interactive, args.thinking, args.no_stream, args.no_metrics) == ("auto", "auto", False, False, False, False)
+    with pytest.raises(SystemExit):
+        cli.build_parser().parse_args(["--prompt", "hi"])
+
+
+def fake_engine(events):
+    calls = {}
+
+    def generate(prompts, **options):
+        calls["prompts"], calls["options"] = prompts, options
+        return iter([(0, e) for e in events])
+
+    return SimpleNamespace(generate=generate, tokenizer=object(), device="cuda:0", dtype="torch.bfloat16", load_seconds=1.5,
+                           last_cache_capacity=48, last_cache_num_bytes=48 * 1024), calls
+
+
+def test_streams_text_and_prints_metrics(monkeypatch):
+    events = [GenerationEvent(5, 0, "Hel", "Hel", None, 0.5, 7), GenerationEvent(6, 1, "lo", "Hello", "max_new_tokens", 0.25, None)]
+    engine, calls = fake_engine(events)
+    monkeypatch.setattr(cli, "_engine_from_args", lambda args: engine)
+    out = io.StringIO()
+    code = cli.main(["--model", "m", "--prompt", "hi", "--max-new-tokens", "2", "--temperature", "0.7", "--top-k", "5", "--seed", "3"], output=out)
+    text = out.getvalue()
+    assert code == 0 and text.startswith("Hello\n")
+    assert "prompt tokens:       7" in text and "generated tokens:    2" in text and "stop reason:         max_new_tokens" in text
+    assert "decode throughput:   4.00 tokens/s" in text and "(48 positions)" in text
+    assert calls["options"]["sampling"] == SamplingConfig(temperature=0.7, top_k=5, top_p=1.0, seed=3)
+    assert calls["options"]["max_new_tokens"] == 2 and calls["prompts"][0][0].content == "hi"
+
+
+def test_prompt_ids_and_no_stream(monkeypatch):
+    engine, calls = fake_engine([GenerationEvent(9, 0, "", "", "eos", None, 3)])
+    engine.tokenizer = None
+    monkeypatch.setattr(cli, "_engine_from_args", lambda args: engine)
+    out = io.StringIO()
+    assert cli.main(["--model", "m", "--prompt-ids", "4, 5,6", "--no-stream", "--no-metrics"], output=out) == 0
+    assert calls["prompts"][0] == [4, 5, 6] and out.getvalue() == "9\n"
+
+
+def test_typed_errors_exit_with_2(monkeypatch):
+    def boom(args):
+        raise ConfigError("model directory does not exist: m")
+
+    monkeypatch.setattr(cli, "_engine_from_args", boom)
+    err = io.StringIO()
+    assert cli.main(["--model", "m", "--prompt", "hi"], error=err) == 2
+    assert err.getvalue() == "error: model directory does not exist: m\n"
+    err = io.StringIO()
+    assert cli.main(["--model", "m"], error=err) == 2 and "--prompt is required" in err.getvalue()
+    err = io.StringIO()
+    assert cli.main(["--model", "m", "--prompt", "x", "--temperature", "-1"], error=err) == 2 and "temperature" in err.getvalue()
+
+
+def test_sampling_config_validation():
+    # reference tests/test_generation.py:69-80
+    for bad in (dict(temperature=-1), dict(top_k=0), dict(top_p=0), dict(top_p=1.5), dict(seed=-1), dict(temperature=float("nan"))):
+        with pytest.raises(SamplingError):
+            SamplingConfig(**bad)
+    assert SamplingConfig().greedy and not SamplingConfig(temperature=0.3).greedy
+
+
+def test_interactive_reads_until_quit(monkeypatch):
+    engine, calls = fake_engine([GenerationEvent(5, 0, "ok", "ok", "eos", None, 2)])
+    monkeypatch.setattr(cli, "_engine_from_args", lambda args: engine)
+    out = io.StringIO()
+    code = cli.main(["--model", "m", "--interactive", "--no-metrics"], input_stream=io.StringIO("hello\n\n/quit\n"), output=out)
+    assert code == 0 and "assistant> ok" in out.getvalue() and out.getvalue().count("you> ") == 3

@@ -1,0 +1,217 @@
+"""The engine as a user meets it: greedy generation through the entry point, long decoding,
+the first tokens of a sequence, graph replay against eager steps, seeded sampling, a pool so
+small that requests wait, and the command line."""
+
+import subprocess
+import sys
+from pathlib import Path
+
+import numpy as np
+import pytest
+import torch
+
+from tests import traces
+from tests.helpers import TINY_A, TINY_B
+from tests.plain import model as plain
+
+pytestmark = pytest.mark.gpu
+ROOT = Path(__file__).resolve().parents[1]
+
+
+@pytest.fixture(scope="module")
+def folders(tmp_path_factory):
+    from llm_runtime_study_amd.config import config_from_dict
+    from llm_runtime_study_amd.weights import write_model_dir
+
+    out = {}
+    for name, raw, seed in (("a", TINY_A, 31), ("b", TINY_B, 32)):
+        folder = tmp_path_factory.mktemp(f"engine_{name}")
+        write_model_dir(config_from_dict(raw), seed=seed, model_dir=folder, init="scaled")
+        cfg, weights = plain.load_model_dir(folder, torch.float64)
+        out[name] = (folder, cfg, weights)
+    return out
+
+
+def plain_greedy(cfg, weights, prompt, new_tokens, stop=()):
+    ids = list(prompt)
+    for _ in range(new_tokens):
+        ids.append(int(plain.qwen3_forward(weights, cfg, ids)[-1].argmax()))
+        if ids[-1] in stop:
+            break
+    return ids[len(prompt):]
+
+
+@pytest.mark.parametrize("name", ["a", "b"])
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_greedy_generation_through_the_entry_point(folders, name, dtype):
+    from llm_runtime_study_amd import Engine, SamplingConfig
+
+    folder, cfg, weights = folders[name]
+    rng = np.random.default_rng(4)
+    prompts = [rng.integers(0, cfg["vocab_size"], n).tolist() for n in (5, 11, 17, 1, 40)]
+    eos = cfg["eos_token_id"] if isinstance(cfg["eos_token_id"], list) else [cfg["eos_token_id"]]
+    expected = [plain_greedy(cfg, weights, p, 8, eos) for p in prompts]
+    engine = Engine.from_model_dir(folder, dtype=dtype, max_seq_len=96, max_batch_size=3, max_num_batched_tokens=16)
+    events = list(engine.generate(prompts, max_new_tokens=8, sampling=SamplingConfig()))
+    got = [[e.token_id for i, e in events if i == r] for r in range(len(prompts))]
+    if dtype == "float32":
+        assert got == expected
+    else:
+        same = sum(a == b for g, e in zip(got, expected) for a, b in zip(g, e))
+        assert same >= 0.85 * sum(len(e) for e in expected)
+    firsts = [e for _, e in events if e.prompt_token_count is not None]
+    assert sorted(e.prompt_token_count for e in firsts) == sorted(len(p) for p in prompts)
+    for r in range(len(prompts)):
+        last = [e for i, e in events if i == r][-1]
+        assert last.finish_reason == ("eos" if last.token_id in eos else "max_new_tokens")
+    assert all(e.model_seconds is not None and e.model_seconds > 0 for _, e in events)
+    manager = engine.cache_manager
+    manager.check_invariants()
+    assert manager.active_requests == 0 and manager.used_pages() == 0
+    assert engine.last_cache_capacity == len(prompts[-1]) + 8 and engine.last_cache_num_bytes > 0
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_long_decoding_token_by_token(folders, dtype, tmp_path):
+    """8 prompt tokens, then 400 tokens one by one: every logits row against the plain model."""
+    from llm_runtime_study_amd.engine import trace
+
+    folder, cfg, weights = folders["b"]
+    ids = np.random.default_rng(6).integers(0, cfg["vocab_size"], 408).tolist()
+    want = plain.qwen3_forward(weights, cfg, ids)
+    steps = traces.prefill_then_decode({"r": ids}, tail=400)
+    runner = trace.make_runner(folder, dtype, 448)
+    trace.replay(runner, traces.strip(steps).splitlines(), tmp_path, echo=lambda _: None)
+    got = traces.collect(steps, tmp_path, cfg["vocab_size"])["r"]
+    assert len(got) == 408
+    for position, row in got.items():
+        if dtype == "float32":
+            torch.testing.assert_close(row.double(), want[position], rtol=1e-4, atol=1e-4, msg=lambda m: f"position {position}: {m}")
+        else:
+            err = (row.double() - want[position]).norm() / want[position].norm()
+            assert err < 3e-2, f"position {position}: relative error {err:.3g}"
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_first_tokens_of_a_sequence_one_by_one(folders, dtype, tmp_path):
+    from llm_runtime_study_amd.engine import trace
+
+    folder, cfg, weights = folders["a"]
+    ids = [9, 200, 3, 77, 150, 4]
+    want = plain.qwen3_forward(weights, cfg, ids)
+    steps = [{"step": i, "entries": [{"id": "r", "tokens": [t], "want": [0]}], "end": ["r"] if i == 5 else []} for i, t in enumerate(ids)]
+    runner = trace.make_runner(folder, dtype, 64)
+    trace.replay(runner, traces.strip(steps).splitlines(), tmp_path, echo=lambda _: None)
+    got = traces.collect(steps, tmp_path, cfg["vocab_size"])["r"]
+    for position in range(6):
+        err = (got[position].double() - want[position]).norm() / want[position].norm()
+        assert err < (1e-5 if dtype == "float32" else 3e-2), f"position {position}: {err:.3g}"
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_graph_replay_equals_eager_steps(folders, dtype):
+    """Decode steps through captured graphs, with eager prefill work and synchronisations between the
+    replays; every replay's logits must equal those of the same step run eagerly."""
+    from llm_runtime_study_amd.cache import CacheManager
+    from llm_runtime_study_amd.engine.loading import load_model
+    from llm_runtime_study_amd.engine.step import ModelRunner, StepEntry
+
+    folder, cfg, _ = folders["b"]
+    device = torch.device("cuda", 0)
+    _, model = load_model(folder, dtype, device)
+    rng = np.random.default_rng(8)
+
+    def make(use_graph):
+        cache = CacheManager(model.cache_needs(), page_size=16, num_pages=40, max_requests=8, max_seq_len=256, dtype=dtype, device=device)
+        return ModelRunner(model, cache, max_step_tokens=128, dtype=dtype, device=device, use_graph=use_graph)
+
+    eager, graphed = make(False), make(True)
+    assert graphed.use_graph
+    prompts = [rng.integers(0, cfg["vocab_size"], n).tolist() for n in (3, 30, 17, 45, 9)]
+    stream = torch.cuda.Stream(device)
+    with torch.cuda.stream(stream):
+        live = {}
+        for step in range(24):
+            if step in (0, 1, 5, 9, 13):       # a new request joins: an eager prefill step between replays
+                index = len(live)
+                caches = (eager.cache.admit(index), graphed.cache.admit(index))
+                a = eager.step([StepEntry(caches[0], prompts[index], [len(prompts[index]) - 1])]).clone()
+                b = graphed.step([StepEntry(caches[1], prompts[index], [len(prompts[index]) - 1])]).clone()
+                assert torch.equal(a, b)
+                live[index] = (caches, int(a[0].argmax()))
+            if step == 17:                      # a request leaves: the batch shrinks to another bucket
+                caches, _ = live.pop(1)
+                eager.cache.release(caches[0])
+                graphed.cache.release(caches[1])
+            order = sorted(live)
+            a = eager.step([StepEntry(live[i][0][0], [live[i][1]], [0]) for i in order]).clone()
+            b = graphed.step([StepEntry(live[i][0][1], [live[i][1]], [0]) for i in order]).clone()
+            torch.cuda.synchronize()
+            assert torch.equal(a, b), f"step {step}: graph replay differs from the eager step"
+            for row, i in enumerate(order):
+                live[i] = (live[i][0], int(a[row].argmax()))
+    assert graphed.graph_replays == 24 and len(graphed._graphs) >= 3
+    graphed.drop_graphs()
+
+
+def test_seeded_sampling_is_reproducible_and_independent_of_batch_mates(folders):
+    from llm_runtime_study_amd import Engine, SamplingConfig
+
+    folder, cfg, _ = folders["b"]
+    rng = np.random.default_rng(9)
+    prompts = [rng.integers(0, cfg["vocab_size"], n).tolist() for n in (23, 40, 1, 64)]
+    sampling = SamplingConfig(temperature=0.8, seed=0)
+    engine = Engine.from_model_dir(folder, dtype="float32", max_seq_len=128, max_batch_size=4, max_num_batched_tokens=16)
+    together = engine.generate_tokens(prompts, max_new_tokens=12, sampling=sampling, ignore_eos=True)
+    again = engine.generate_tokens(prompts, max_new_tokens=12, sampling=sampling, ignore_eos=True)
+    assert together == again and all(len(t) == 12 for t in together)
+    alone = [engine.generate_tokens([p], max_new_tokens=12, sampling=sampling, ignore_eos=True)[0] for p in prompts]
+    assert alone == together
+    other = engine.generate_tokens(prompts, max_new_tokens=12, sampling=SamplingConfig(temperature=0.8, seed=1), ignore_eos=True)
+    assert other != together
+    greedy = engine.generate_tokens(prompts, max_new_tokens=12, ignore_eos=True)
+    assert greedy != together
+    top1 = engine.generate_tokens(prompts, max_new_tokens=12, sampling=SamplingConfig(temperature=0.8, top_k=1, seed=5), ignore_eos=True)
+    assert top1 == greedy      # only the largest logit survives the filter
+
+
+def test_small_pool_makes_requests_wait_and_reuses_pages(folders):
+    from llm_runtime_study_amd import Engine
+
+    folder, cfg, weights = folders["a"]
+    rng = np.random.default_rng(10)
+    prompts = [rng.integers(0, cfg["vocab_size"], n).tolist() for n in (30, 25, 28, 12, 31, 5)]
+    expected = [plain_greedy(cfg, weights, p, 6, [cfg["eos_token_id"]]) for p in prompts]
+    # 6 pages of 16 tokens: two requests of up to 37 tokens (3 pages each) at a time
+    engine = Engine.from_model_dir(folder, dtype="float32", max_seq_len=48, max_batch_size=4, num_pages=6, max_num_batched_tokens=24)
+    scheduler = engine.create_scheduler()
+    for p in prompts:
+        scheduler.add_request(p, max_new_tokens=6)
+    got = {i: [] for i in range(len(prompts))}
+    most_running, waited_for_pages = 0, False
+    with torch.cuda.stream(engine.stream):
+        while scheduler.has_unfinished:
+            for i, e in scheduler.step():
+                got[i].append(e.token_id)
+            most_running = max(most_running, scheduler.num_running)
+            waited_for_pages |= scheduler.num_waiting > 0 and scheduler.num_running < 4
+            engine.cache_manager.check_invariants()
+    assert [got[i] for i in range(len(prompts))] == expected
+    assert 2 <= most_running <= 3 and waited_for_pages and engine.cache_manager.used_pages() == 0
+
+
+def test_command_line_on_the_gpu(folders):
+    folder, cfg, weights = folders["a"]
+    expected = plain_greedy(cfg, weights, [5, 6, 7], 4, [cfg["eos_token_id"]])
+    proc = subprocess.run([sys.executable, "-m", "llm_runtime_study_amd", "--model", str(folder), "--prompt-ids", "5,6,7",
+                           "--max-new-tokens", "4", "--max-seq-len", "64", "--dtype", "float32"],
+                          cwd=ROOT, capture_output=True, text=True, timeout=300)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    assert proc.stdout.split("\n")[0].split() == [str(t) for t in expected]
+    assert "prompt tokens:       3" in proc.stdout and "stop reason:" in proc.stdout
+    proc = subprocess.run([sys.executable, "-m", "llm_runtime_study_amd", "--model", str(folder), "--prompt", "hello", "--max-seq-len", "64"],
+                          cwd=ROOT, capture_output=True, text=True, timeout=300)
+    assert proc.returncode == 2 and "error: a text prompt needs a tokenizer" in proc.stderr
+    proc = subprocess.run([sys.executable, "-m", "llm_runtime_study_amd", "--model", str(folder), "--prompt-ids", "1", "--max-seq-len", "4096"],
+                          cwd=ROOT, capture_output=True, text=True, timeout=300)
+    assert proc.returncode == 2 and "exceeds the model limit" in proc.stderr

@@ -1,0 +1,209 @@
+"""Scheduler decisions with a fake step function: admission, portions under the token budget,
+decoding, finishing, freeing, waiting for pages, failure (CPU)."""
+
+import pytest
+import torch
+
+from llm_runtime_study_amd.cache import CacheManager
+from llm_runtime_study_amd.engine.scheduler import BatchScheduler, generate
+from llm_runtime_study_amd.errors import GenerationError, KVCacheError, SamplingError
+from llm_runtime_study_amd.parts import PagedKVNeed
+from llm_runtime_study_amd.sampling import SamplingConfig
+
+VOCAB = 50
+
+
+class FakeRunner:
+    """Extends caches like the real step function and returns logits that make request i's
+    k-th token equal `script[i][k]`; the request is known by its cache's request_id."""
+
+    def __init__(self, script, num_pages=16, page_size=4, max_requests=4, max_seq_len=64):
+        self.cache = CacheManager([PagedKVNeed(1, 8)], page_size=page_size, num_pages=num_pages, max_requests=max_requests,
+                                  max_seq_len=max_seq_len, dtype=torch.float32, device="cpu", allocate_storage=False)
+        self.script, self.produced, self.calls, self.fail_at = script, {}, [], None
+
+    def step(self, entries):
+        if self.fail_at is not None and len(self.calls) == self.fail_at:
+            raise RuntimeError("injected failure")
+        self.calls.append([(e.cache.request_id, list(e.tokens), list(e.want)) for e in entries])
+        rows = []
+        for e in entries:
+            self.cache.extend(e.cache, len(e.tokens))
+            for _ in e.want:
+                k = self.produced.get(e.cache.request_id, 0)
+                self.produced[e.cache.request_id] = k + 1
+                row = torch.zeros(VOCAB)
+                row[self.script[e.cache.request_id][k]] = 1.0
+                rows.append(row)
+        self.cache.check_invariants()
+        return torch.stack(rows) if rows else None
+
+
+class FakeSampler:
+    def choose(self, logits, rows):
+        assert logits.shape[0] == len(rows)
+        return logits.argmax(-1).tolist()
+
+
+def scheduler(runner, **options):
+    defaults = dict(max_batch_size=2, max_seq_len=64, max_step_tokens=8, eos_token_ids=(1,), vocab_size=VOCAB)
+    defaults.update(options)
+    return BatchScheduler(runner, FakeSampler(), **defaults)
+
+
+def drain(s):
+    events = []
+    while s.has_unfinished:
+        events += s.step()
+    return events
+
+
+def test_prompt_is_cut_under_the_budget_and_samples_only_on_its_last_portion():
+    runner = FakeRunner({0: [7, 8, 1]})
+    s = scheduler(runner, max_step_tokens=8)
+    s.add_request(list(range(10, 30)), max_new_tokens=5)
+    events = drain(s)
+    assert [len(c[0][1]) for c in runner.calls] == [8, 8, 4, 1, 1]
+    assert [c[0][2] for c in runner.calls] == [[], [], [3], [0], [0]]
+    assert runner.calls[3][0][1] == [7] and runner.calls[4][0][1] == [8]
+    assert [(i, e.token_id, e.token_index, e.finish_reason) for i, e in events] == [(0, 7, 0, None), (0, 8, 1, None), (0, 1, 2, "eos")]
+    assert events[0][1].prompt_token_count == 20 and events[1][1].prompt_token_count is None
+    assert runner.cache.used_pages() == 0 and runner.cache.active_requests == 0
+
+
+def test_decodes_come_first_and_portions_share_the_step():
+    runner = FakeRunner({0: [5, 6, 7, 8, 9, 9, 9], 1: [4, 4, 4, 4]})
+    s = scheduler(runner, max_step_tokens=6, max_batch_size=2)
+    s.add_request([2] * 3, max_new_tokens=6)
+    s.add_request([3] * 11, max_new_tokens=3)
+    drain(s)
+    # (request, tokens run) per step: request 1's prompt fills what request 0 leaves of the budget
+    assert s.step_log[:4] == [[(0, 3), (1, 3)], [(0, 1), (1, 5)], [(0, 1), (1, 3)], [(0, 1), (1, 1)]]
+    first_mixed = runner.calls[1]
+    assert first_mixed[0] == (0, [5], [0]) and first_mixed[1][2] == []   # decode row first, portion wants nothing yet
+
+
+def test_finish_reasons_and_compaction():
+    # reference tests/test_generation.py:387-400, 464-496
+    runner = FakeRunner({0: [9, 9, 9], 1: [9, 1], 2: [9, 9, 9, 9]}, max_seq_len=8)
+    s = scheduler(runner, max_batch_size=3, max_seq_len=8, max_step_tokens=16)
+    s.add_request([2, 2], max_new_tokens=3)            # ends by max_new_tokens
+    s.add_request([2, 2], max_new_tokens=5)            # ends by eos
+    s.add_request([2] * 5, max_new_tokens=10)          # context clips the output to 3
+    events = drain(s)
+    last = {i: e for i, e in events}
+    assert last[0].finish_reason == "max_new_tokens" and last[0].token_index == 2
+    assert last[1].finish_reason == "eos" and last[1].token_index == 1
+    assert last[2].finish_reason == "context_length" and last[2].token_index == 2
+    # after request 1 ended, the decode batch holds the survivors in their old order
+    assert [[r for r, _, _ in call] for call in runner.calls] == [[0, 1, 2], [0, 1, 2], [0, 2]]
+
+
+def test_zero_room_prompt_ends_without_a_forward():
+    runner = FakeRunner({1: [9]}, max_seq_len=8)
+    s = scheduler(runner, max_seq_len=8)
+    s.add_request([2] * 8, max_new_tokens=4)
+    s.add_request([2] * 3, max_new_tokens=1)
+    events = s.step()
+    assert (events[0][0], events[0][1].finish_reason, events[0][1].token_id, events[0][1].prompt_token_count) == (0, "context_length", None, 8)
+    assert events[1][0] == 1 and events[1][1].finish_reason == "max_new_tokens"
+    assert len(runner.calls) == 1 and runner.calls[0][0][0] == 1
+
+
+def test_requests_wait_for_a_slot_first_come_first_served():
+    # reference tests/test_generation.py:515-550
+    runner = FakeRunner({0: [9, 9, 9], 1: [9], 2: [9, 9]})
+    s = scheduler(runner, max_batch_size=2)
+    for n in (3, 1, 2):
+        s.add_request([2, 2], max_new_tokens=n)
+    s.step()
+    assert (s.num_running, s.num_waiting) == (1, 1)   # request 1 finished at once, request 2 still waits
+    s.step()
+    assert (s.num_running, s.num_waiting) == (2, 0)
+    drain(s)
+    assert [[r for r, _, _ in call] for call in runner.calls] == [[0, 1], [0, 2], [0, 2]]
+
+
+def test_head_of_queue_waits_for_pages_and_nothing_jumps_it():
+    # pool of 6 pages of 4 tokens; reference tests/test_generation.py:552-568
+    runner = FakeRunner({0: [9, 9, 9, 9], 1: [9, 9], 2: [9]}, num_pages=6)
+    s = scheduler(runner, max_batch_size=3)
+    s.add_request([2] * 12, max_new_tokens=4)     # lifetime 16 tokens = 4 pages
+    s.add_request([2] * 10, max_new_tokens=2)     # 3 pages: does not fit beside request 0
+    s.add_request([2] * 2, max_new_tokens=1)      # 1 page: would fit, but must not jump the queue
+    s.step()
+    assert (s.num_running, s.num_waiting) == (1, 2)
+    events = drain(s)
+    order = [i for i, e in events if e.prompt_token_count is not None]
+    assert order == [0, 1, 2]
+    first_step_of = {}
+    for n, call in enumerate(runner.calls):
+        for r, _, _ in call:
+            first_step_of.setdefault(r, n)
+    last_step_of_0 = max(n for n, call in enumerate(runner.calls) if any(r == 0 for r, _, _ in call))
+    assert first_step_of[1] > last_step_of_0 and first_step_of[2] >= first_step_of[1]
+    assert runner.cache.used_pages() == 0
+
+
+def test_requests_that_can_never_run_are_refused_when_added():
+    runner = FakeRunner({}, num_pages=4)      # 16 tokens of cache
+    s = scheduler(runner, max_seq_len=32)
+    with pytest.raises(GenerationError, match="max_new_tokens must be positive"):
+        s.add_request([2], max_new_tokens=0)
+    with pytest.raises(GenerationError, match="prompt has 33 tokens but model context limit is 32"):
+        s.add_request([2] * 33, max_new_tokens=1)
+    with pytest.raises(GenerationError, match="needs 20 cache tokens but the KV cache holds 16"):
+        s.add_request([2] * 12, max_new_tokens=8)
+    with pytest.raises(SamplingError, match="top_k 51 exceeds vocabulary size 50"):
+        s.add_request([2], max_new_tokens=1, sampling=SamplingConfig(temperature=1.0, top_k=51))
+    with pytest.raises(GenerationError, match="within vocabulary"):
+        s.add_request([2, 50], max_new_tokens=1)
+    with pytest.raises(GenerationError, match="needs a tokenizer"):
+        from llm_runtime_study_amd import ChatMessage
+        s.add_request([ChatMessage("user", "hi")], max_new_tokens=1)
+    with pytest.raises(GenerationError, match="must hold one token of each"):
+        scheduler(runner, max_batch_size=4, max_step_tokens=3)
+    assert not s.has_unfinished
+
+
+def test_failure_frees_every_request_and_reraises():
+    # reference tests/test_generation.py:592-610
+    runner = FakeRunner({0: [9] * 5, 1: [9] * 5})
+    s = scheduler(runner)
+    s.add_request([2] * 5, max_new_tokens=5)
+    s.add_request([2] * 5, max_new_tokens=5)
+    s.add_request([2] * 5, max_new_tokens=5)
+    s.step()
+    runner.fail_at = len(runner.calls)
+    with pytest.raises(RuntimeError, match="injected failure"):
+        s.step()
+    assert not s.has_unfinished and runner.cache.used_pages() == 0 and runner.cache.active_requests == 0
+    runner.cache.check_invariants()
+
+
+def test_closing_the_iterator_frees_everything():
+    runner = FakeRunner({0: [9] * 9})
+    s = scheduler(runner)
+    stream = generate(s, [[2, 2, 2]], max_new_tokens=9)
+    assert next(stream)[1].token_id == 9
+    assert runner.cache.used_pages() > 0
+    stream.close()
+    assert runner.cache.used_pages() == 0 and not s.has_unfinished
+    with pytest.raises(GenerationError, match="at least one request"):
+        generate(s, [], max_new_tokens=1)
+
+
+def test_sampling_rows_carry_each_requests_own_seed_and_counter():
+    seen = []
+
+    class RecordingSampler(FakeSampler):
+        def choose(self, logits, rows):
+            seen.append([(r.seed, r.counter, r.config.temperature) for r in rows])
+            return super().choose(logits, rows)
+
+    runner = FakeRunner({0: [9, 9, 9], 1: [9, 9]})
+    s = BatchScheduler(runner, RecordingSampler(), max_batch_size=2, max_seq_len=64, max_step_tokens=8, vocab_size=VOCAB)
+    s.add_request([2, 2], max_new_tokens=3, sampling=SamplingConfig(temperature=0.8, seed=11))
+    s.add_request([2, 2], max_new_tokens=2, sampling=SamplingConfig(temperature=0.5, seed=12))
+    drain(s)
+    assert seen == [[(11, 0, 0.8), (12, 0, 0.5)], [(11, 1, 0.8), (12, 1, 0.5)], [(11, 2, 0.8)]]

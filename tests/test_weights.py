@@ -1,0 +1,119 @@
+"""Safetensors reading, checkpoint validation and random weights (CPU)."""
+
+import json
+
+import pytest
+import torch
+
+from llm_runtime_study_amd.config import config_from_dict, spec_for
+from llm_runtime_study_amd.errors import CheckpointError, CheckpointValidationError
+from llm_runtime_study_amd.models import DecoderModel
+from llm_runtime_study_amd.weights import Checkpoint, load, random_tensors, validate, write_model_dir, write_safetensors
+from tests.helpers import TINY_A, TINY_B, qwen3_tensor_shapes
+
+
+def expected_for(raw):
+    return DecoderModel(spec_for(config_from_dict(raw))).tensors()
+
+
+def test_schema_names_and_count():
+    # 11 tensors a layer + embedding, final norm, head (reference tests/test_checkpoint.py: 11 L + 3)
+    raw = dict(TINY_B, attention_bias=False)
+    expected = expected_for(raw)
+    assert len(expected) == 11 * raw["num_hidden_layers"] + 3
+    assert {k: v.shape for k, v in expected_for(TINY_B).items()} == qwen3_tensor_shapes(TINY_B)
+    tied = expected_for(TINY_A)
+    assert tied["lm_head.weight"].optional and not tied["model.embed_tokens.weight"].optional
+
+
+def test_written_folder_reads_back_identically_with_both_readers(tmp_path):
+    from safetensors.torch import load_file
+
+    config = config_from_dict(TINY_B)
+    write_model_dir(config, 3, tmp_path, init="scaled")
+    checkpoint = Checkpoint.from_model_dir(tmp_path)
+    theirs = load_file(str(tmp_path / "model.safetensors"))
+    assert set(theirs) == set(checkpoint.manifest)
+    for name, tensor in theirs.items():
+        assert torch.equal(tensor, checkpoint.tensor(name)) and tensor.dtype == torch.bfloat16
+    weights = load(checkpoint, expected_for(TINY_B), "qwen3", "cpu")
+    assert all(t.dtype == torch.bfloat16 for t in weights.values())
+    # same seed, same folder; another seed, other weights
+    again = random_tensors(expected_for(TINY_B), 3, torch.bfloat16, "scaled")
+    other = random_tensors(expected_for(TINY_B), 4, torch.bfloat16, "scaled")
+    assert torch.equal(again["lm_head.weight"], weights["lm_head.weight"])
+    assert not torch.equal(other["lm_head.weight"], weights["lm_head.weight"])
+
+
+def test_all_problems_are_reported_in_one_error(tmp_path):
+    expected = expected_for(TINY_A)
+    tensors = random_tensors(expected, 0, torch.bfloat16)
+    del tensors["model.layers.1.mlp.up_proj.weight"]
+    del tensors["model.norm.weight"]
+    tensors["model.layers.0.self_attn.rotary.inv_freq"] = torch.zeros(8)
+    tensors["model.layers.0.self_attn.q_proj.weight"] = torch.zeros(64, 63, dtype=torch.bfloat16)
+    tensors["model.layers.0.input_layernorm.weight"] = torch.zeros(64, dtype=torch.int32)
+    write_safetensors(tmp_path / "model.safetensors", tensors)
+    with pytest.raises(CheckpointValidationError) as info:
+        validate(Checkpoint.from_model_dir(tmp_path), expected, "qwen3")
+    text = str(info.value)
+    assert text.startswith("checkpoint does not match qwen3 configuration:")
+    assert "missing tensors: model.layers.1.mlp.up_proj.weight, model.norm.weight" in text
+    assert "unexpected tensors: model.layers.0.self_attn.rotary.inv_freq" in text
+    assert "shape mismatch for model.layers.0.self_attn.q_proj.weight: expected (64, 64), got (64, 63)" in text
+    assert "dtype mismatch for model.layers.0.input_layernorm.weight" in text
+
+
+def test_tied_head_is_optional_and_untied_head_is_required(tmp_path):
+    tied = expected_for(TINY_A)
+    write_safetensors(tmp_path / "model.safetensors", random_tensors(tied, 0, torch.bfloat16))
+    validate(Checkpoint.from_model_dir(tmp_path), tied, "qwen3")
+    untied = expected_for(dict(TINY_A, tie_word_embeddings=False))
+    with pytest.raises(CheckpointValidationError, match="missing tensors: lm_head.weight"):
+        validate(Checkpoint.from_model_dir(tmp_path), untied, "qwen3")
+
+
+def test_stored_precision_is_kept(tmp_path):
+    expected = expected_for(TINY_A)
+    tensors = random_tensors(expected, 0, torch.bfloat16)
+    tensors["model.norm.weight"] = tensors["model.norm.weight"].float() + 1e-4   # stored in 32-bit: stays so
+    tensors["model.layers.0.mlp.down_proj.weight"] = tensors["model.layers.0.mlp.down_proj.weight"].half()
+    write_safetensors(tmp_path / "model.safetensors", tensors)
+    weights = load(Checkpoint.from_model_dir(tmp_path), expected, "qwen3", "cpu")
+    assert weights["model.norm.weight"].dtype == torch.float32
+    assert torch.equal(weights["model.norm.weight"], tensors["model.norm.weight"])
+    assert weights["model.layers.0.mlp.down_proj.weight"].dtype == torch.float32   # float16 is widened
+    assert weights["model.embed_tokens.weight"].dtype == torch.bfloat16
+
+
+def test_sharded_checkpoint_merges_headers(tmp_path):
+    expected = expected_for(TINY_A)
+    tensors = random_tensors(expected, 5, torch.bfloat16)
+    names = sorted(tensors)
+    first, second = names[: len(names) // 2], names[len(names) // 2:]
+    write_safetensors(tmp_path / "model-00001-of-00002.safetensors", {n: tensors[n] for n in first})
+    write_safetensors(tmp_path / "model-00002-of-00002.safetensors", {n: tensors[n] for n in second})
+    weight_map = {n: "model-00001-of-00002.safetensors" for n in first}
+    weight_map.update({n: "model-00002-of-00002.safetensors" for n in second})
+    (tmp_path / "model.safetensors.index.json").write_text(json.dumps({"weight_map": weight_map}))
+    checkpoint = Checkpoint.from_model_dir(tmp_path)
+    assert list(checkpoint.manifest) == names
+    weights = load(checkpoint, expected, "qwen3", "cpu")
+    assert all(torch.equal(weights[n], tensors[n]) for n in names)
+    (tmp_path / "model-00002-of-00002.safetensors").unlink()
+    with pytest.raises(CheckpointError, match="checkpoint shard does not exist"):
+        Checkpoint.from_model_dir(tmp_path)
+
+
+def test_file_errors(tmp_path):
+    with pytest.raises(CheckpointError, match="neither model.safetensors nor model.safetensors.index.json"):
+        Checkpoint.from_model_dir(tmp_path)
+    (tmp_path / "model.safetensors").write_bytes(b"\x05\x00\x00")
+    with pytest.raises(CheckpointError, match="too short"):
+        Checkpoint.from_model_dir(tmp_path)
+    (tmp_path / "model.safetensors").write_bytes((10**9).to_bytes(8, "little") + b"{}")
+    with pytest.raises(CheckpointError, match="bad header length"):
+        Checkpoint.from_model_dir(tmp_path)
+    write_safetensors(tmp_path / "model.safetensors", {"a": torch.zeros(2)})
+    with pytest.raises(CheckpointError, match="tensor is not in the checkpoint: b"):
+        Checkpoint.from_model_dir(tmp_path).tensor("b")
