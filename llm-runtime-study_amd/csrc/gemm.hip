@@ -137,6 +137,90 @@ __global__ __launch_bounds__(256) void gemm_bf16_mfma_kernel(void* __restrict__ 
     }
 }
 
+// ------------------------------------------------- bf16 kernel for few rows
+// Decode-sized products (M <= 64): the weight matrix is streamed exactly once and the time
+// is the time to read it.  One workgroup owns 16 weight rows; its waves split K between them
+// and add their partial sums through LDS in a fixed order.  Weights are the MFMA A operand
+// (16 rows x 32 k, each lane one 16-byte load of a row), the activations the B operand
+// (32 k x 16 tokens, read from L2); MT is the number of 16-token blocks.  UNROLL steps of 32 k
+// are loaded before any is used, so each wave keeps UNROLL KB of weights in flight.
+template <int MT, int WAVES, int UNROLL>
+__global__ __launch_bounds__(WAVES * 64) void gemm_bf16_skinny_kernel(
+    void* __restrict__ out, int mode, const bf16* __restrict__ x, const bf16* __restrict__ w,
+    const bf16* __restrict__ bias, int m, int n, int k, int lda, int ldc) {
+  __shared__ floatx4 partial[WAVES][MT][WAVE];
+  const int tid = threadIdx.x, lane = tid % WAVE, wave = tid / WAVE;
+  const int r = lane & 15, g = lane >> 4;
+  const int n0 = blockIdx.x * 16;
+  const int row = n0 + r < n ? n0 + r : n - 1;
+  const bf16* wp = w + (int64_t)row * k + g * 8;
+  const bf16* xp[MT];
+  bool live[MT];
+#pragma unroll
+  for (int t = 0; t < MT; ++t) {
+    const int token = t * 16 + r;
+    live[t] = token < m;
+    xp[t] = x + (int64_t)(live[t] ? token : 0) * lda + g * 8;
+  }
+  floatx4 acc[MT];
+#pragma unroll
+  for (int t = 0; t < MT; ++t) acc[t] = floatx4{0.f, 0.f, 0.f, 0.f};
+  const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
+
+  const int steps = (k + 31) / 32;
+  const int per_wave = (steps + WAVES - 1) / WAVES;
+  int s = wave * per_wave;
+  const int s_end = s + per_wave < steps ? s + per_wave : steps;
+  const int full_end = k / 32 < s_end ? k / 32 : s_end;   // steps whose 32 k are all inside K
+  for (; s + UNROLL <= full_end; s += UNROLL) {
+    bf16x8 a[UNROLL], b[UNROLL][MT];
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) a[u] = *(const bf16x8*)(wp + (s + u) * 32);
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u)
+#pragma unroll
+      for (int t = 0; t < MT; ++t) b[u][t] = live[t] ? *(const bf16x8*)(xp[t] + (s + u) * 32) : zero;
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u)
+#pragma unroll
+      for (int t = 0; t < MT; ++t) acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[u], b[u][t], acc[t], 0, 0, 0);
+  }
+  for (; s < s_end; ++s) {
+    const bool inside = s * 32 + g * 8 < k;
+    const bf16x8 a = inside ? *(const bf16x8*)(wp + s * 32) : zero;
+#pragma unroll
+    for (int t = 0; t < MT; ++t) {
+      const bf16x8 b = (inside && live[t]) ? *(const bf16x8*)(xp[t] + s * 32) : zero;
+      acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, acc[t], 0, 0, 0);
+    }
+  }
+#pragma unroll
+  for (int t = 0; t < MT; ++t) partial[wave][t][lane] = acc[t];
+  __syncthreads();
+  // accumulator layout: token = t*16 + lane % 16, weight row = n0 + 4 * (lane / 16) + i
+  for (int e = tid; e < MT * WAVE * 4; e += WAVES * WAVE) {
+    const int t = e / (WAVE * 4), l = (e / 4) % WAVE, i = e % 4;
+    const int token = t * 16 + (l & 15), gn = n0 + 4 * (l >> 4) + i;
+    if (token >= m || gn >= n) continue;
+    float v = 0.f;
+#pragma unroll
+    for (int wv = 0; wv < WAVES; ++wv) v += partial[wv][t][l][i];
+    if (bias) v += (float)bias[gn];
+    emit<bf16>(out, mode, (int64_t)token * ldc + gn, v);
+  }
+}
+
+template <int MT>
+static void launch_skinny(void* out, int mode, const bf16* a, const bf16* w, const bf16* bias, int m, int n,
+                          int k, int lda, int ldc, hipStream_t s) {
+  const int tiles = (n + 15) / 16;
+  constexpr int UNROLL = MT == 1 ? 8 : (MT == 2 ? 4 : 2);
+  if (tiles <= 2048)
+    gemm_bf16_skinny_kernel<MT, 8, UNROLL><<<tiles, 8 * 64, 0, s>>>(out, mode, a, w, bias, m, n, k, lda, ldc);
+  else
+    gemm_bf16_skinny_kernel<MT, 4, UNROLL><<<tiles, 4 * 64, 0, s>>>(out, mode, a, w, bias, m, n, k, lda, ldc);
+}
+
 // out [M, N] (row stride ldc) = a [M, K] (row stride lda) times w[N, K]^T.
 LRS_API int lrs_gemm(void* out, int mode, const void* a, const void* w, const void* bias, int dtype,
                      int m, int n, int k, int lda, int ldc, void* stream) {
@@ -150,7 +234,13 @@ LRS_API int lrs_gemm(void* out, int mode, const void* a, const void* w, const vo
                                                   (const float*)bias, m, n, k, lda, ldc);
   } else if (dtype == LRS_BF16) {
     const bool aligned = k % 8 == 0 && lda % 8 == 0 && ((uintptr_t)a % 16 == 0) && ((uintptr_t)w % 16 == 0);
-    if (aligned) {
+    if (aligned && m <= 64) {
+      const bf16 *ap = (const bf16*)a, *wp = (const bf16*)w, *bp = (const bf16*)bias;
+      if (m <= 16) launch_skinny<1>(out, mode, ap, wp, bp, m, n, k, lda, ldc, s);
+      else if (m <= 32) launch_skinny<2>(out, mode, ap, wp, bp, m, n, k, lda, ldc, s);
+      else if (m <= 48) launch_skinny<3>(out, mode, ap, wp, bp, m, n, k, lda, ldc, s);
+      else launch_skinny<4>(out, mode, ap, wp, bp, m, n, k, lda, ldc, s);
+    } else if (aligned) {
       dim3 grid((n + 127) / 128, (m + 127) / 128);
       gemm_bf16_mfma_kernel<<<grid, 256, 0, s>>>(out, mode, (const bf16*)a, (const bf16*)w,
                                                  (const bf16*)bias, m, n, k, lda, ldc);
