@@ -7,8 +7,10 @@ What each schedule entry of the model keeps between steps is declared by its mix
   ("from", j)                  nothing of its own: it reads the cache of entry j;
   None                         nothing.
 Entries whose paged needs are equal form a group.  A group has a page pool of its own, one
-K and one V tensor [pages + 1, nkv, page_size, d] per entry (a page id addresses the same
-page in every entry of the group; the extra last page absorbs the writes of padding rows),
+K tensor [pages + 1, nkv, page_size, d] and one V tensor [pages + 1, nkv, d, page_size] per
+entry (values are kept transposed inside a page, so that the keys of one value column are
+contiguous, which is what the matrix-core kernels read; a page id addresses the same page
+in every entry of the group; the extra last page absorbs the writes of padding rows),
 and one block table per request.  Pages are taken when a request grows into them and given
 back when the request ends, is rolled back, or (windowed groups) when every position in
 the page has left the window of all future queries.
@@ -116,10 +118,11 @@ class CacheManager:
         for index, group in enumerate(self.groups):
             group.host_table = np.full((max_requests, self.max_blocks), -1, dtype=np.int32)
             if allocate_storage:
-                shape = (num_pages + 1, group.need.num_kv_heads, page_size, group.need.head_dim)
+                k_shape = (num_pages + 1, group.need.num_kv_heads, page_size, group.need.head_dim)
+                v_shape = (num_pages + 1, group.need.num_kv_heads, group.need.head_dim, page_size)
                 for position in group.entries:
-                    group.k[position] = torch.empty(shape, dtype=dtype, device=self.device)
-                    group.v[position] = torch.empty(shape, dtype=dtype, device=self.device)
+                    group.k[position] = torch.zeros(k_shape, dtype=dtype, device=self.device)
+                    group.v[position] = torch.zeros(v_shape, dtype=dtype, device=self.device)
                     self.layer_caches[position].k_pages = group.k[position]
                     self.layer_caches[position].v_pages = group.v[position]
 

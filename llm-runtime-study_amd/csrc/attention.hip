@@ -3,8 +3,9 @@
 // position and lo = max(0, p - window + 1) when a window is given.  Keys and values of this
 // step's tokens are already in the cache when these kernels run.
 //
-// Pages are [page, kv_head, slot, dim]; block_table[r, i] is the page holding positions
-// i*page_size .. (i+1)*page_size-1 of request r.  Scores, softmax and the weighted sum are
+// Key pages are [page, kv_head, slot, dim], value pages [page, kv_head, dim, slot] (transposed
+// inside a page); block_table[r, i] is the page holding positions i*page_size ..
+// (i+1)*page_size-1 of request r.  Scores, softmax and the weighted sum are
 // float32.  Key tiles start at multiples of the tile size counted from position 0, so the
 // rounding of a query's result depends on its position only, never on how the sequence
 // was cut into steps.
@@ -19,10 +20,11 @@ __global__ __launch_bounds__(THREADS) void attention_generic_kernel(
     const int* __restrict__ block_table, int table_stride, const int* __restrict__ token_request,
     const int* __restrict__ positions, int nq, int nkv, int d, int page_size, float scale,
     int window) {
-  extern __shared__ float smem[];
+  extern __shared__ __attribute__((aligned(16))) float smem[];
   float* qs = smem;                           // [d]
-  float* probs = qs + d;                      // [THREADS]
-  int64_t* bases = (int64_t*)(probs + THREADS);  // [THREADS] element offset of each key row
+  float* probs = qs + d + d % 2;              // [THREADS]
+  int64_t* bases = (int64_t*)(probs + THREADS);  // [THREADS] element offset of each key's (page, kv head) block
+  int* offsets = (int*)(bases + THREADS);        // [THREADS] slot of each key inside its page
   __shared__ float scratch[16];
 
   const int token = blockIdx.x, head = blockIdx.y, tid = threadIdx.x;
@@ -42,10 +44,11 @@ __global__ __launch_bounds__(THREADS) void attention_generic_kernel(
     const bool valid = key >= lo && key <= pos;
     float score = -INFINITY;
     int64_t base = 0;
+    const int off = key % page_size;
     if (valid) {
       const int64_t page = table[key / page_size];
-      base = ((page * nkv + kv_head) * page_size + key % page_size) * d;
-      const T* kr = k_pages + base;
+      base = (page * nkv + kv_head) * page_size * d;
+      const T* kr = k_pages + base + (int64_t)off * d;
       float dot = 0.f;
       for (int i = 0; i < d; ++i) dot = fmaf(qs[i], to_float(kr[i]), dot);
       score = dot * scale;
@@ -59,6 +62,7 @@ __global__ __launch_bounds__(THREADS) void attention_generic_kernel(
     running_max = new_max;
     probs[tid] = p;
     bases[tid] = base;
+    offsets[tid] = off;
     __syncthreads();
     const int count = (pos - tile + 1 < THREADS) ? pos - tile + 1 : THREADS;
 #pragma unroll
@@ -68,7 +72,7 @@ __global__ __launch_bounds__(THREADS) void attention_generic_kernel(
         float a = acc[c] * alpha;
         for (int j = 0; j < count; ++j) {
           const float pj = probs[j];
-          if (pj != 0.f) a = fmaf(pj, to_float(v_pages[bases[j] + dim]), a);
+          if (pj != 0.f) a = fmaf(pj, to_float(v_pages[bases[j] + (int64_t)dim * page_size + offsets[j]]), a);
         }
         acc[c] = a;
       }
@@ -83,6 +87,207 @@ __global__ __launch_bounds__(THREADS) void attention_generic_kernel(
   }
 }
 
+// ------------------------------------------------- bf16 decode kernel
+// One query token per request (a decode step).  A workgroup of four waves owns one
+// (token, kv head, split): the query heads that share the kv head (at most 16) sit in the
+// columns of the matrix-core tiles, so every key and value is loaded once for the whole
+// group.  Keys are walked in tiles of 32; the tiles of a token are divided between `splits`
+// workgroups (so that few long requests still fill the chip) and, inside a workgroup,
+// dealt to the waves in turn.  Per tile:
+//     S[key, head]   = K[key, :] . Q[head, :]          A = K rows (16 keys x 32 dims per MFMA)
+//     P              = exp2(S * scale*log2(e) - max)   online softmax per head column
+//     O^T[dim, head] += V^T[dim, key] . P[key, head]   A = V^T rows, read from the transposed page
+// S comes out of the first product with a head per lane column and four keys per lane, which
+// is exactly the operand layout the second product wants for P, so P never leaves registers.
+// Waves are merged through LDS, splits by attention_merge_kernel.
+template <int D>
+__global__ __launch_bounds__(256) void attention_decode_bf16_kernel(
+    bf16* __restrict__ out, int out_stride, float* __restrict__ part_o, float* __restrict__ part_ml,
+    const bf16* __restrict__ q, int q_stride, const bf16* __restrict__ k_pages,
+    const bf16* __restrict__ v_pages, const int* __restrict__ block_table, int table_stride,
+    const int* __restrict__ token_request, const int* __restrict__ positions, int nq, int nkv,
+    int page_size, float scale, int window, int splits) {
+  constexpr int DS = D / 32, DB = D / 16, WAVES = 4;
+  __shared__ float sm_m[WAVES][16], sm_l[WAVES][16];
+  __shared__ float sm_o[WAVES][D][16];
+  const int tid = threadIdx.x, lane = tid % WAVE, wave = tid / WAVE;
+  const int col = lane & 15, g = lane >> 4;
+  const int split = blockIdx.x, kvh = blockIdx.y, token = blockIdx.z;
+  const int group = nq / nkv;
+  const int pos = positions[token];
+  const int lo = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
+  const int* table = block_table + (int64_t)token_request[token] * table_stride;
+  const int first_tile = lo / 32, last_tile = pos / 32;
+  const int per_split = (last_tile - first_tile + splits) / splits;
+  const int tile_begin = first_tile + split * per_split;
+  const int tile_end = tile_begin + per_split <= last_tile + 1 ? tile_begin + per_split : last_tile + 1;
+
+  const bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
+  bf16x8 qf[DS];
+#pragma unroll
+  for (int c = 0; c < DS; ++c)
+    qf[c] = col < group ? *(const bf16x8*)(q + (int64_t)token * q_stride + (int64_t)(kvh * group + col) * D + c * 32 + g * 8) : zero8;
+
+  floatx4 o[DB];
+#pragma unroll
+  for (int b = 0; b < DB; ++b) o[b] = floatx4{0.f, 0.f, 0.f, 0.f};
+  float run_max = -INFINITY, run_sum = 0.f;
+  const float scale2 = scale * 1.4426950408889634f;
+
+  for (int tile = tile_begin + wave; tile < tile_end; tile += WAVES) {
+    floatx4 s[2];
+    int64_t vbase[2];
+    bool present[2];
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      const int key0 = tile * 32 + h * 16;
+      present[h] = key0 <= pos && key0 + 15 >= lo;
+      s[h] = floatx4{0.f, 0.f, 0.f, 0.f};
+      vbase[h] = 0;
+      if (present[h]) {
+        const int64_t page = table[key0 / page_size];
+        const int off = key0 % page_size;
+        const bf16* kp = k_pages + ((page * nkv + kvh) * page_size + off + col) * D + g * 8;
+        vbase[h] = (page * nkv + kvh) * (int64_t)D * page_size + off;
+#pragma unroll
+        for (int c = 0; c < DS; ++c)
+          s[h] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(*(const bf16x8*)(kp + c * 32), qf[c], s[h], 0, 0, 0);
+      }
+    }
+    float tile_max = -INFINITY;
+#pragma unroll
+    for (int h = 0; h < 2; ++h)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int key = tile * 32 + h * 16 + g * 4 + i;
+        const bool valid = present[h] && key <= pos && key >= lo;
+        s[h][i] = valid ? s[h][i] * scale2 : -INFINITY;
+        tile_max = fmaxf(tile_max, s[h][i]);
+      }
+    tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 16, WAVE));
+    tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32, WAVE));
+    const float new_max = fmaxf(run_max, tile_max);
+    const float alpha = exp2f(run_max - new_max);
+    run_max = new_max;
+    bf16x8 pf;
+    float tile_sum = 0.f;
+#pragma unroll
+    for (int h = 0; h < 2; ++h)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const float p = exp2f(s[h][i] - new_max);
+        tile_sum += p;
+        pf[h * 4 + i] = (bf16)p;
+      }
+    run_sum = run_sum * alpha + tile_sum;
+#pragma unroll
+    for (int b = 0; b < DB; ++b) {
+      bf16x4 v0 = {0, 0, 0, 0}, v1 = {0, 0, 0, 0};
+      if (present[0]) v0 = *(const bf16x4*)(v_pages + vbase[0] + (int64_t)(b * 16 + col) * page_size + g * 4);
+      if (present[1]) v1 = *(const bf16x4*)(v_pages + vbase[1] + (int64_t)(b * 16 + col) * page_size + g * 4);
+      const bf16x8 vf = {v0[0], v0[1], v0[2], v0[3], v1[0], v1[1], v1[2], v1[3]};
+      o[b] *= alpha;
+      o[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf, o[b], 0, 0, 0);
+    }
+  }
+  run_sum += __shfl_xor(run_sum, 16, WAVE);
+  run_sum += __shfl_xor(run_sum, 32, WAVE);
+  if (g == 0) {
+    sm_m[wave][col] = run_max;
+    sm_l[wave][col] = run_sum;
+  }
+#pragma unroll
+  for (int b = 0; b < DB; ++b)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) sm_o[wave][b * 16 + g * 4 + i][col] = o[b][i];
+  __syncthreads();
+  for (int e = tid; e < D * 16; e += 256) {
+    const int dim = e / 16, h = e % 16;
+    if (h >= group) continue;
+    float top = sm_m[0][h];
+#pragma unroll
+    for (int w = 1; w < WAVES; ++w) top = fmaxf(top, sm_m[w][h]);
+    float acc = 0.f, total = 0.f;
+#pragma unroll
+    for (int w = 0; w < WAVES; ++w) {
+      const float weight = top == -INFINITY ? 0.f : exp2f(sm_m[w][h] - top);
+      acc += sm_o[w][dim][h] * weight;
+      total += sm_l[w][h] * weight;
+    }
+    const int head = kvh * group + h;
+    if (splits == 1) {
+      out[(int64_t)token * out_stride + (int64_t)head * D + dim] = (bf16)(acc / total);
+    } else {
+      const int64_t slot = ((int64_t)token * nq + head) * splits + split;
+      part_o[slot * D + dim] = acc;
+      if (dim == 0) {
+        part_ml[slot * 2] = top;
+        part_ml[slot * 2 + 1] = total;
+      }
+    }
+  }
+}
+
+// Merges the partial results of the splits of one (token, head): out = sum_s o_s 2^(m_s - m) / sum_s l_s 2^(m_s - m).
+__global__ void attention_merge_kernel(bf16* __restrict__ out, int out_stride, const float* __restrict__ part_o,
+                                       const float* __restrict__ part_ml, int nq, int d, int splits) {
+  const int token = blockIdx.x, head = blockIdx.y;
+  const int64_t base = ((int64_t)token * nq + head) * splits;
+  float top = -INFINITY;
+  for (int s = 0; s < splits; ++s) top = fmaxf(top, part_ml[(base + s) * 2]);
+  float total = 0.f;
+  for (int s = 0; s < splits; ++s) {
+    const float m = part_ml[(base + s) * 2];
+    if (m > -INFINITY) total += part_ml[(base + s) * 2 + 1] * exp2f(m - top);
+  }
+  for (int dim = threadIdx.x; dim < d; dim += blockDim.x) {
+    float acc = 0.f;
+    for (int s = 0; s < splits; ++s) {
+      const float m = part_ml[(base + s) * 2];
+      if (m > -INFINITY) acc += part_o[(base + s) * d + dim] * exp2f(m - top);
+    }
+    out[(int64_t)token * out_stride + (int64_t)head * d + dim] = (bf16)(acc / total);
+  }
+}
+
+// Decode step in bf16: one query token per request.  part_o [tokens, nq, splits, d] and part_ml
+// [tokens, nq, splits, 2] float32 are needed when splits > 1.  Returns an error for shapes the
+// matrix-core kernel does not take (the caller then uses lrs_attention).
+LRS_API int lrs_attention_decode(void* out, int out_stride, float* part_o, float* part_ml, const void* q,
+                                 int q_stride, const void* k_pages, const void* v_pages,
+                                 const int* block_table, int table_stride, const int* token_request,
+                                 const int* positions, int tokens, int nq, int nkv, int d, int page_size,
+                                 float scale, int window, int splits, void* stream) {
+  LRS_REQUIRE(tokens > 0 && nq > 0 && nkv > 0 && nq % nkv == 0, "attention_decode: bad sizes tokens=%d nq=%d nkv=%d", tokens, nq, nkv);
+  LRS_REQUIRE(nq / nkv <= 16, "attention_decode: %d query heads per kv head, at most 16 fit a tile", nq / nkv);
+  LRS_REQUIRE(page_size % 16 == 0, "attention_decode: page size %d is not a multiple of 16", page_size);
+  LRS_REQUIRE(splits >= 1 && (splits == 1 || (part_o && part_ml)), "attention_decode: splits=%d needs partial buffers", splits);
+  LRS_REQUIRE(window >= 0, "attention_decode: window must be >= 0 (0 = none)");
+  LRS_REQUIRE(q_stride % 8 == 0 && ((uintptr_t)q % 16) == 0, "attention_decode: q rows must be 16-byte aligned");
+  dim3 grid(splits, nkv, tokens);
+  hipStream_t s = (hipStream_t)stream;
+#define LAUNCH(D)                                                                                                   \
+  attention_decode_bf16_kernel<D><<<grid, 256, 0, s>>>((bf16*)out, out_stride, part_o, part_ml, (const bf16*)q, q_stride, \
+                                                       (const bf16*)k_pages, (const bf16*)v_pages, block_table,      \
+                                                       table_stride, token_request, positions, nq, nkv, page_size,   \
+                                                       scale, window, splits)
+  switch (d) {
+    case 32: LAUNCH(32); break;
+    case 64: LAUNCH(64); break;
+    case 96: LAUNCH(96); break;
+    case 128: LAUNCH(128); break;
+    case 192: LAUNCH(192); break;
+    default: return lrs_fail("attention_decode: head_dim %d has no matrix-core kernel (32, 64, 96, 128, 192)", d);
+  }
+#undef LAUNCH
+  if (lrs_check_launch("attention_decode")) return 1;
+  if (splits > 1) {
+    attention_merge_kernel<<<dim3(tokens, nq), d < 64 ? 64 : d, 0, s>>>((bf16*)out, out_stride, part_o, part_ml, nq, d, splits);
+    return lrs_check_launch("attention_merge");
+  }
+  return 0;
+}
+
 // out [tokens, nq*d] (row stride out_stride); q rows are [nq*d] with row stride q_stride.
 LRS_API int lrs_attention(void* out, int out_stride, const void* q, int q_stride, const void* k_pages,
                           const void* v_pages, const int* block_table, int table_stride,
@@ -95,7 +300,7 @@ LRS_API int lrs_attention(void* out, int out_stride, const void* q, int q_stride
   LRS_REQUIRE(window >= 0, "attention: window must be >= 0 (0 = none)");
   constexpr int THREADS = 128;
   dim3 grid(tokens, nq);
-  const size_t lds = sizeof(float) * (d + THREADS) + sizeof(int64_t) * THREADS + 16;
+  const size_t lds = sizeof(float) * (d + d % 2 + THREADS) + (sizeof(int64_t) + sizeof(int)) * THREADS + 16;
   hipStream_t s = (hipStream_t)stream;
   if (dtype == LRS_F32)
     attention_generic_kernel<float, THREADS><<<grid, THREADS, lds, s>>>(

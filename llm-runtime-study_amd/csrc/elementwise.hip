@@ -90,7 +90,8 @@ LRS_API int lrs_rope_table(float* cosv, float* sinv, const int* positions, const
 // One wave per (token, head) of the fused projection row [q heads | k heads | v heads].
 // q heads: optional RMSNorm over head_dim, optional half-split rotation of the first
 // 2*rot_half dims, written back in place.  k heads: the same, written into the paged key
-// cache; v heads: copied into the paged value cache.  Pages are [page, kv_head, slot, dim];
+// cache [page, kv_head, slot, dim]; v heads: copied into the paged value cache, which is
+// transposed inside a page: [page, kv_head, dim, slot].
 // `slots[t]` is page * page_size + offset of token t (negative: do not store).
 template <typename T, typename TW>
 __global__ void qk_prep_kernel(T* __restrict__ qkv, int row_stride, int nq, int nkv, int d,
@@ -108,11 +109,12 @@ __global__ void qk_prep_kernel(T* __restrict__ qkv, int row_stride, int nq, int 
     if (slot < 0) return;
     const int kv_head = is_k ? head - nq : head - nq - nkv;
     const int64_t page = slot / page_size, off = slot % page_size;
-    dst = (is_k ? k_pages : v_pages) + ((page * nkv + kv_head) * page_size + off) * d;
     if (!is_k) {
-      for (int i = lane; i < d; i += WAVE) dst[i] = src[i];
+      T* vdst = v_pages + (page * nkv + kv_head) * d * page_size + off;
+      for (int i = lane; i < d; i += WAVE) vdst[(int64_t)i * page_size] = src[i];
       return;
     }
+    dst = k_pages + ((page * nkv + kv_head) * page_size + off) * d;
   }
   const TW* weight = is_q ? q_weight : k_weight;
   float inv = 1.f;

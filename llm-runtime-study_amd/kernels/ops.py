@@ -40,6 +40,8 @@ _SIGNATURES = {
     "lrs_gemm": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p]),
     "lrs_attention": (c_int, [c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p,
                               c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_void_p]),
+    "lrs_attention_decode": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p,
+                                     c_void_p, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_int, c_void_p]),
     "lrs_choose_tokens": (c_int, [c_void_p, c_void_p, c_int64, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p]),
     "lrs_filter_logits": (c_int, [c_void_p, c_int64, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p]),
 }
@@ -180,7 +182,8 @@ def qk_prep(qkv: torch.Tensor, nq: int, nkv: int, d: int, q_weight, k_weight, ep
         _need(k_weight is not None and q_weight.numel() == d and k_weight.numel() == d and q_weight.dtype == k_weight.dtype, "qk_prep: q/k norm weights must both hold head_dim values")
         w_dtype = q_weight.dtype
     if nkv > 0:
-        _need(k_pages.dim() == 4 and k_pages.shape[1:] == (nkv, page_size, d) and v_pages.shape == k_pages.shape, f"qk_prep: pages must be [pages, {nkv}, {page_size}, {d}]")
+        _need(k_pages.dim() == 4 and k_pages.shape[1:] == (nkv, page_size, d) and v_pages.shape == (k_pages.shape[0], nkv, d, page_size),
+              f"qk_prep: key pages must be [pages, {nkv}, {page_size}, {d}] and value pages [pages, {nkv}, {d}, {page_size}]")
         _need(k_pages.is_contiguous() and v_pages.is_contiguous() and k_pages.dtype == qkv.dtype and v_pages.dtype == qkv.dtype, "qk_prep: pages must be contiguous and of the activation dtype")
         _need(slots.dtype == torch.int32 and slots.numel() >= tokens and slots.is_contiguous(), "qk_prep: slots must be int32 [T]")
     _check(library().lrs_qk_prep(
@@ -235,10 +238,12 @@ def gemm(out: torch.Tensor, a: torch.Tensor, w: torch.Tensor, bias: torch.Tensor
 # -------------------------------------------------------------- attention
 def attention(out: torch.Tensor, q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, block_table: torch.Tensor,
               token_request: torch.Tensor, positions: torch.Tensor, nq: int, scale: float, window: int = 0) -> None:
-    """out [T, nq*d]; q [T, >= nq*d] (leading nq*d columns of each row); pages [P, nkv, page, d]."""
+    """out [T, nq*d]; q [T, >= nq*d] (leading nq*d columns of each row); key pages [P, nkv, page, d],
+    value pages [P, nkv, d, page]."""
     tokens = out.shape[0]
-    _need(k_pages.dim() == 4 and v_pages.shape == k_pages.shape and k_pages.is_contiguous() and v_pages.is_contiguous(), "attention: pages must be contiguous [P, nkv, page, d]")
+    _need(k_pages.dim() == 4 and k_pages.is_contiguous() and v_pages.is_contiguous(), "attention: pages must be contiguous")
     _, nkv, page_size, d = k_pages.shape
+    _need(v_pages.shape == (k_pages.shape[0], nkv, d, page_size), "attention: key pages must be [P, nkv, page, d] and value pages [P, nkv, d, page]")
     _need(out.shape[1] == nq * d and q.shape[0] == tokens and q.shape[1] >= nq * d, "attention: q/out widths do not match nq*d")
     _need(q.dtype == k_pages.dtype == v_pages.dtype == out.dtype, "attention: q, pages and out must share a dtype")
     _need(block_table.dim() == 2 and block_table.dtype == torch.int32 and block_table.stride(1) == 1, "attention: block_table must be int32 [R, blocks]")
@@ -248,6 +253,38 @@ def attention(out: torch.Tensor, q: torch.Tensor, k_pages: torch.Tensor, v_pages
         _dev(out, "out"), _rows(out, "out"), _dev(q, "q"), _rows(q, "q"), _dev(k_pages, "k_pages"), _dev(v_pages, "v_pages"),
         _dev(block_table, "block_table"), block_table.stride(0), _dev(token_request, "token_request"), _dev(positions, "positions"),
         dtype_code(q.dtype), tokens, nq, nkv, d, page_size, scale, window, _stream()))
+
+
+DECODE_HEAD_DIMS = (32, 64, 96, 128, 192)
+
+
+def attention_decode_supported(dtype: torch.dtype, nq: int, nkv: int, d: int, page_size: int) -> bool:
+    """Whether the matrix-core decode kernel takes this shape (else use attention())."""
+    return dtype == torch.bfloat16 and d in DECODE_HEAD_DIMS and page_size % 16 == 0 and nq // nkv <= 16
+
+
+def attention_decode(out: torch.Tensor, q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, block_table: torch.Tensor,
+                     token_request: torch.Tensor, positions: torch.Tensor, nq: int, scale: float, window: int = 0, splits: int = 1,
+                     part_o: torch.Tensor | None = None, part_ml: torch.Tensor | None = None) -> None:
+    """attention() for a step with one query token per request, bfloat16 only; the keys of a token
+    are divided between `splits` workgroups whose partial results meet in part_o / part_ml."""
+    tokens = out.shape[0]
+    _need(k_pages.dim() == 4 and k_pages.is_contiguous() and v_pages.is_contiguous(), "attention_decode: pages must be contiguous")
+    _, nkv, page_size, d = k_pages.shape
+    _need(v_pages.shape == (k_pages.shape[0], nkv, d, page_size), "attention_decode: key pages must be [P, nkv, page, d] and value pages [P, nkv, d, page]")
+    _need(attention_decode_supported(q.dtype, nq, nkv, d, page_size), f"attention_decode: unsupported shape nq={nq} nkv={nkv} d={d} page={page_size} {q.dtype}")
+    _need(out.shape[1] == nq * d and q.shape[0] == tokens and q.shape[1] >= nq * d, "attention_decode: q/out widths do not match nq*d")
+    _need(q.dtype == k_pages.dtype == v_pages.dtype == out.dtype, "attention_decode: q, pages and out must share a dtype")
+    _need(block_table.dim() == 2 and block_table.dtype == torch.int32 and block_table.stride(1) == 1, "attention_decode: block_table must be int32 [R, blocks]")
+    for name, t in (("token_request", token_request), ("positions", positions)):
+        _need(t.dtype == torch.int32 and t.numel() >= tokens and t.is_contiguous(), f"attention_decode: {name} must be int32 [T]")
+    if splits > 1:
+        _need(part_o is not None and part_o.dtype == torch.float32 and part_o.is_contiguous() and part_o.numel() >= tokens * nq * splits * d, "attention_decode: part_o too small")
+        _need(part_ml is not None and part_ml.dtype == torch.float32 and part_ml.is_contiguous() and part_ml.numel() >= tokens * nq * splits * 2, "attention_decode: part_ml too small")
+    _check(library().lrs_attention_decode(
+        _dev(out, "out"), _rows(out, "out"), None if splits == 1 else _dev(part_o, "part_o"), None if splits == 1 else _dev(part_ml, "part_ml"),
+        _dev(q, "q"), _rows(q, "q"), _dev(k_pages, "k_pages"), _dev(v_pages, "v_pages"), _dev(block_table, "block_table"), block_table.stride(0),
+        _dev(token_request, "token_request"), _dev(positions, "positions"), tokens, nq, nkv, d, page_size, scale, window, splits, _stream()))
 
 
 # --------------------------------------------------------------- sampling

@@ -79,6 +79,13 @@ class GQAAttention(Part):
             return None
         return PagedKVNeed(self.num_kv_heads, self.head_dim, self.window)
 
+    @staticmethod
+    def _decode_splits(workgroups: int, longest: int) -> int:
+        """Into how many workgroups the keys of one decode token are divided: enough to fill the
+        chip twice over when the batch alone does not, but at least 256 keys each."""
+        wanted = -(-512 // workgroups)
+        return max(1, min(wanted, longest // 256, 64))
+
     # ------------------------------------------------------------------ forward
     def forward(self, ctx, x, residual, cache):
         if cache is None:
@@ -93,8 +100,18 @@ class GQAAttention(Part):
         ops.qk_prep(qkv, nq, nkv, d, self.q_norm, self.k_norm, self.qk_norm_eps, cos, sin,
                     cache.k_pages, cache.v_pages, group.slots, group.page_size)
         out = ctx.scratch("attn_out", (t, nq * d), ctx.dtype)
-        ops.attention(out, qkv, cache.k_pages, cache.v_pages, group.block_table, ctx.token_request, ctx.positions,
-                      nq, self.scale, self.window or 0)
+        kv_heads = cache.k_pages.shape[1]
+        if ctx.all_decode and ops.attention_decode_supported(ctx.dtype, nq, kv_heads, d, group.page_size):
+            splits = self._decode_splits(t * kv_heads, ctx.max_k if self.window is None else min(ctx.max_k, self.window + 32))
+            part_o = part_ml = None
+            if splits > 1:
+                part_o = ctx.scratch("attn_part_o", (t, nq * splits * d), torch.float32)
+                part_ml = ctx.scratch("attn_part_ml", (t, nq * splits * 2), torch.float32)
+            ops.attention_decode(out, qkv, cache.k_pages, cache.v_pages, group.block_table, ctx.token_request, ctx.positions,
+                                 nq, self.scale, self.window or 0, splits, part_o, part_ml)
+        else:
+            ops.attention(out, qkv, cache.k_pages, cache.v_pages, group.block_table, ctx.token_request, ctx.positions,
+                          nq, self.scale, self.window or 0)
         ops.gemm(residual, out, self.w_o, accumulate=True)
 
 

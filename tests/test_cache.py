@@ -138,6 +138,7 @@ def test_groups_share_needs_and_follow_cache_sources():
     caches = m.layer_caches
     assert caches[3] is caches[0] and caches[0].group == 0 and caches[1].group == 1 and caches[5].group is None
     assert caches[0].k_pages.shape == (5, 2, 4, 16)          # one extra page for padding rows
+    assert caches[0].v_pages.shape == (5, 2, 16, 4)          # values are transposed inside a page
     assert caches[0].k_pages.data_ptr() != caches[2].k_pages.data_ptr()
     assert caches[4].state.shape == (3, 3, 5)
     a = m.admit("a")

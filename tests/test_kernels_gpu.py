@@ -112,7 +112,7 @@ def test_qk_prep(ops, dtype, nq, nkv, d, rot, normed, page):
 
     d_qkv = dev(qkv)
     kp = torch.full((pages, nkv, page, d), 7.0, device="cuda", dtype=dtype)
-    vp = torch.full((pages, nkv, page, d), 7.0, device="cuda", dtype=dtype)
+    vp = torch.full((pages, nkv, d, page), 7.0, device="cuda", dtype=dtype)   # values: transposed inside a page
     cos = sin = None
     if rot_half:
         cos = torch.empty(t, rot_half, device="cuda")
@@ -130,9 +130,9 @@ def test_qk_prep(ops, dtype, nq, nkv, d, rot, normed, page):
             continue
         touched[s // page, s % page] = True
         torch.testing.assert_close(kp[s // page, :, s % page], want_k[i], **tol(dtype, 1e-5, 2e-2))
-        torch.testing.assert_close(vp[s // page, :, s % page], want_v[i], rtol=0, atol=0)
+        torch.testing.assert_close(vp[s // page, :, :, s % page], want_v[i], rtol=0, atol=0)
     # nothing else was written
-    assert (kp.permute(0, 2, 1, 3)[~touched] == 7.0).all() and (vp.permute(0, 2, 1, 3)[~touched] == 7.0).all()
+    assert (kp.permute(0, 2, 1, 3)[~touched] == 7.0).all() and (vp.permute(0, 3, 1, 2)[~touched] == 7.0).all()
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
@@ -225,7 +225,7 @@ def test_attention_ragged_batch(ops, dtype, nq, nkv, d, page, window):
     n_pages = sum((a + b + page - 1) // page for a, b in requests) + 3
     perm = torch.randperm(n_pages, generator=g).tolist()
     kp = torch.zeros(n_pages, nkv, page, d)
-    vp = torch.zeros(n_pages, nkv, page, d)
+    vp = torch.zeros(n_pages, nkv, d, page)
     table = torch.zeros(len(requests), max_blocks, dtype=torch.int32)
     k_all, v_all, q_rows, tok_req, tok_pos, meta = [], [], [], [], [], []
     for r, (before, new) in enumerate(requests):
@@ -239,7 +239,7 @@ def test_attention_ragged_batch(ops, dtype, nq, nkv, d, page, window):
             table[r, b] = pg
             n = min(page, total - b * page)
             kp[pg, :, :n] = k[b * page: b * page + n].float().transpose(0, 1)
-            vp[pg, :, :n] = v[b * page: b * page + n].float().transpose(0, 1)
+            vp[pg, :, :, :n] = v[b * page: b * page + n].float().permute(1, 2, 0)
         for i in range(new):
             q_rows.append((torch.randn(nq, d, generator=g) * 2).to(dtype))
             tok_req.append(r)
@@ -258,6 +258,52 @@ def test_attention_ragged_batch(ops, dtype, nq, nkv, d, page, window):
     torch.testing.assert_close(out.cpu().double(), want, **tol(dtype, 2e-5, 2e-2))
 
 
+@pytest.mark.parametrize("nq,nkv,d,page,window,splits", [
+    (8, 2, 32, 16, 0, 1), (32, 8, 128, 16, 0, 1), (32, 8, 128, 16, 0, 5), (4, 4, 64, 32, 0, 3), (16, 1, 96, 16, 0, 2),
+    (6, 2, 192, 64, 0, 4), (8, 2, 32, 16, 40, 1), (8, 2, 64, 16, 100, 3), (8, 2, 32, 16, 0, 64),
+])
+def test_attention_decode_kernel(ops, nq, nkv, d, page, window, splits):
+    """One query token per request at context lengths around tile and page edges."""
+    g = torch.Generator().manual_seed(16)
+    lengths = [1, 15, 16, 17, 31, 32, 33, 64, 257, 700]
+    scale = 1 / math.sqrt(d)
+    blocks = [(n + page - 1) // page for n in lengths]
+    n_pages = sum(blocks) + 2
+    perm = torch.randperm(n_pages, generator=g).tolist()
+    kp = torch.randn(n_pages, nkv, page, d, generator=g)      # slots never written hold finite junk
+    vp = torch.randn(n_pages, nkv, d, page, generator=g)
+    table = torch.full((len(lengths), max(blocks) + 1), -1, dtype=torch.int32)
+    k_all, v_all, meta = [], [], []
+    for r, n in enumerate(lengths):
+        k = torch.randn(n, nkv, d, generator=g).bfloat16()
+        v = torch.randn(n, nkv, d, generator=g).bfloat16()
+        k_all.append(k.float())
+        v_all.append(v.float())
+        for b in range(blocks[r]):
+            pg = perm.pop()
+            table[r, b] = pg
+            m = min(page, n - b * page)
+            kp[pg, :, :m] = k[b * page: b * page + m].float().transpose(0, 1)
+            vp[pg, :, :, :m] = v[b * page: b * page + m].float().permute(1, 2, 0)
+        meta.append((r, n - 1))
+    t = len(lengths)
+    q = (torch.randn(t, nq, d, generator=g) * 2).bfloat16()
+    want = _attention_reference(q.float(), k_all, v_all, meta, None, nq, nkv, d, scale, window)
+    q_wide = torch.zeros(t, nq * d + 2 * nkv * d, dtype=torch.bfloat16)
+    q_wide[:, : nq * d] = q.view(t, nq * d)
+    out = torch.empty(t, nq * d, device="cuda", dtype=torch.bfloat16)
+    part_o = torch.empty(t, nq * splits * d, device="cuda")
+    part_ml = torch.empty(t, nq * splits * 2, device="cuda")
+    assert ops.attention_decode_supported(torch.bfloat16, nq, nkv, d, page)
+    # requests sit in another order in the block table than the tokens in the batch
+    order = torch.randperm(t, generator=g)
+    shuffled = torch.empty_like(table)
+    shuffled[order] = table
+    ops.attention_decode(out, dev(q_wide), dev(kp.bfloat16()), dev(vp.bfloat16()), dev(shuffled), dev(order.to(torch.int32)),
+                         dev(torch.tensor([n - 1 for n in lengths], dtype=torch.int32)), nq, scale, window, splits, part_o, part_ml)
+    torch.testing.assert_close(out.cpu().double(), want, rtol=2e-2, atol=2e-2)
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_attention_finds_a_far_key(ops, dtype):
     """One key among 700 is made to dominate: the output must be its value, wherever it lies."""
@@ -272,13 +318,13 @@ def test_attention_finds_a_far_key(ops, dtype):
         k[far, 0] = q[0, 0] * 60  # score 60/sqrt(32)*... dominates head 0
         n_pages = (length + page - 1) // page
         kp = torch.zeros(n_pages, nkv, page, d)
-        vp = torch.zeros(n_pages, nkv, page, d)
+        vp = torch.zeros(n_pages, nkv, d, page)
         order = torch.randperm(n_pages, generator=g)
         table = order.to(torch.int32).view(1, -1)
         for b in range(n_pages):
             n = min(page, length - b * page)
             kp[order[b], :, :n] = k[b * page: b * page + n].transpose(0, 1)
-            vp[order[b], :, :n] = v[b * page: b * page + n].transpose(0, 1)
+            vp[order[b], :, :, :n] = v[b * page: b * page + n].permute(1, 2, 0)
         out = torch.empty(1, nq * d, device="cuda", dtype=dtype)
         ops.attention(out, dev(q.view(1, -1).to(dtype)), dev(kp.to(dtype)), dev(vp.to(dtype)), dev(table),
                       dev(torch.zeros(1, dtype=torch.int32)), dev(torch.tensor([length - 1], dtype=torch.int32)), nq, 1.0, 0)
