@@ -288,6 +288,150 @@ LRS_API int lrs_attention_decode(void* out, int out_stride, float* part_o, float
   return 0;
 }
 
+// ------------------------------------------------- bf16 kernel for any step
+// Ragged batch of prompt portions and single tokens.  The step's tokens are cut on the host into
+// blocks of at most 16 consecutive tokens of one request; a workgroup owns one (block, kv head)
+// and each of its waves one query head of the group, so the waves of a workgroup read the same
+// keys and values at about the same time.  The arithmetic is that of the decode kernel with the
+// 16 queries of the block in the tile columns instead of the heads: S[key, query] = K Q^T,
+// online softmax per query column with the causal (and window) mask of that query's position,
+// O^T[dim, query] += V^T P.  Every query is finished by one wave, so nothing is merged.
+template <int D>
+__global__ void attention_prefill_bf16_kernel(
+    bf16* __restrict__ out, int out_stride, const bf16* __restrict__ q, int q_stride,
+    const bf16* __restrict__ k_pages, const bf16* __restrict__ v_pages,
+    const int* __restrict__ block_table, int table_stride, const int* __restrict__ token_request,
+    const int* __restrict__ positions, const int* __restrict__ qblock_token0,
+    const int* __restrict__ qblock_count, int nq, int nkv, int page_size, float scale, int window) {
+  constexpr int DS = D / 32, DB = D / 16;
+  const int lane = threadIdx.x % WAVE, wave = threadIdx.x / WAVE;
+  const int col = lane & 15, g = lane >> 4;
+  const int kvh = blockIdx.y, group = nq / nkv;
+  const int head = kvh * group + wave;
+  const int token0 = qblock_token0[blockIdx.x], count = qblock_count[blockIdx.x];
+  const bool live = col < count;
+  const int token = token0 + (live ? col : 0);
+  const int pos = positions[token];
+  const int lo = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
+  const int pos_last = positions[token0 + count - 1];        // positions rise inside a block
+  const int pos_first = positions[token0];
+  const int lo_first = (window > 0 && pos_first - window + 1 > 0) ? pos_first - window + 1 : 0;
+  const int* table = block_table + (int64_t)token_request[token0] * table_stride;
+
+  const bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
+  bf16x8 qf[DS];
+#pragma unroll
+  for (int c = 0; c < DS; ++c)
+    qf[c] = live ? *(const bf16x8*)(q + (int64_t)token * q_stride + (int64_t)head * D + c * 32 + g * 8) : zero8;
+  floatx4 o[DB];
+#pragma unroll
+  for (int b = 0; b < DB; ++b) o[b] = floatx4{0.f, 0.f, 0.f, 0.f};
+  float run_max = -INFINITY, run_sum = 0.f;
+  const float scale2 = scale * 1.4426950408889634f;
+
+  for (int tile = lo_first / 32; tile <= pos_last / 32; ++tile) {
+    floatx4 s[2];
+    int64_t vbase[2];
+    bool present[2];
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      const int key0 = tile * 32 + h * 16;
+      present[h] = key0 <= pos_last && key0 + 15 >= lo_first;
+      s[h] = floatx4{0.f, 0.f, 0.f, 0.f};
+      vbase[h] = 0;
+      if (present[h]) {
+        const int64_t page = table[key0 / page_size];
+        const int off = key0 % page_size;
+        const bf16* kp = k_pages + ((page * nkv + kvh) * page_size + off + col) * D + g * 8;
+        vbase[h] = (page * nkv + kvh) * (int64_t)D * page_size + off;
+#pragma unroll
+        for (int c = 0; c < DS; ++c)
+          s[h] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(*(const bf16x8*)(kp + c * 32), qf[c], s[h], 0, 0, 0);
+      }
+    }
+    float tile_max = -INFINITY;
+#pragma unroll
+    for (int h = 0; h < 2; ++h)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int key = tile * 32 + h * 16 + g * 4 + i;
+        const bool valid = present[h] && key <= pos && key >= lo;
+        s[h][i] = valid ? s[h][i] * scale2 : -INFINITY;
+        tile_max = fmaxf(tile_max, s[h][i]);
+      }
+    tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 16, WAVE));
+    tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32, WAVE));
+    const float new_max = fmaxf(run_max, tile_max);
+    // a query whose window or position leaves it no key in this tile keeps its state
+    const float alpha = new_max == -INFINITY ? 1.f : exp2f(run_max - new_max);
+    const float shift = new_max == -INFINITY ? 0.f : new_max;
+    run_max = new_max;
+    bf16x8 pf;
+    float tile_sum = 0.f;
+#pragma unroll
+    for (int h = 0; h < 2; ++h)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const float p = exp2f(s[h][i] - shift);
+        tile_sum += p;
+        pf[h * 4 + i] = (bf16)p;
+      }
+    run_sum = run_sum * alpha + tile_sum;
+#pragma unroll
+    for (int b = 0; b < DB; ++b) {
+      bf16x4 v0 = {0, 0, 0, 0}, v1 = {0, 0, 0, 0};
+      if (present[0]) v0 = *(const bf16x4*)(v_pages + vbase[0] + (int64_t)(b * 16 + col) * page_size + g * 4);
+      if (present[1]) v1 = *(const bf16x4*)(v_pages + vbase[1] + (int64_t)(b * 16 + col) * page_size + g * 4);
+      const bf16x8 vf = {v0[0], v0[1], v0[2], v0[3], v1[0], v1[1], v1[2], v1[3]};
+      o[b] *= alpha;
+      o[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf, o[b], 0, 0, 0);
+    }
+  }
+  run_sum += __shfl_xor(run_sum, 16, WAVE);
+  run_sum += __shfl_xor(run_sum, 32, WAVE);
+  if (live) {
+    const float inv = 1.0f / run_sum;
+    bf16* dst = out + (int64_t)token * out_stride + (int64_t)head * D + g * 4;
+#pragma unroll
+    for (int b = 0; b < DB; ++b) {
+      const bf16x4 packed = {(bf16)(o[b][0] * inv), (bf16)(o[b][1] * inv), (bf16)(o[b][2] * inv), (bf16)(o[b][3] * inv)};
+      *(bf16x4*)(dst + b * 16) = packed;
+    }
+  }
+}
+
+// Any step in bf16.  qblock_token0 / qblock_count [n_blocks]: first token and number of tokens
+// (1..16) of each block of consecutive tokens of one request.
+LRS_API int lrs_attention_prefill(void* out, int out_stride, const void* q, int q_stride, const void* k_pages,
+                                  const void* v_pages, const int* block_table, int table_stride,
+                                  const int* token_request, const int* positions, const int* qblock_token0,
+                                  const int* qblock_count, int n_blocks, int nq, int nkv, int d, int page_size,
+                                  float scale, int window, void* stream) {
+  LRS_REQUIRE(n_blocks > 0 && nq > 0 && nkv > 0 && nq % nkv == 0, "attention_prefill: bad sizes blocks=%d nq=%d nkv=%d", n_blocks, nq, nkv);
+  LRS_REQUIRE(nq / nkv <= 16, "attention_prefill: %d query heads per kv head, at most 16 waves fit a workgroup", nq / nkv);
+  LRS_REQUIRE(page_size % 16 == 0, "attention_prefill: page size %d is not a multiple of 16", page_size);
+  LRS_REQUIRE(window >= 0, "attention_prefill: window must be >= 0 (0 = none)");
+  LRS_REQUIRE(q_stride % 8 == 0 && ((uintptr_t)q % 16) == 0 && out_stride % 4 == 0 && ((uintptr_t)out % 8) == 0,
+              "attention_prefill: q rows must be 16-byte and out rows 8-byte aligned");
+  dim3 grid(n_blocks, nkv), block((nq / nkv) * WAVE);
+  hipStream_t s = (hipStream_t)stream;
+#define LAUNCH(D)                                                                                                    \
+  attention_prefill_bf16_kernel<D><<<grid, block, 0, s>>>((bf16*)out, out_stride, (const bf16*)q, q_stride,          \
+                                                          (const bf16*)k_pages, (const bf16*)v_pages, block_table,   \
+                                                          table_stride, token_request, positions, qblock_token0,     \
+                                                          qblock_count, nq, nkv, page_size, scale, window)
+  switch (d) {
+    case 32: LAUNCH(32); break;
+    case 64: LAUNCH(64); break;
+    case 96: LAUNCH(96); break;
+    case 128: LAUNCH(128); break;
+    case 192: LAUNCH(192); break;
+    default: return lrs_fail("attention_prefill: head_dim %d has no matrix-core kernel (32, 64, 96, 128, 192)", d);
+  }
+#undef LAUNCH
+  return lrs_check_launch("attention_prefill");
+}
+
 // out [tokens, nq*d] (row stride out_stride); q rows are [nq*d] with row stride q_stride.
 LRS_API int lrs_attention(void* out, int out_stride, const void* q, int q_stride, const void* k_pages,
                           const void* v_pages, const int* block_table, int table_stride,

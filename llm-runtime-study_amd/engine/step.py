@@ -83,7 +83,8 @@ class StepContext:
         self.dtype = runner.dtype
         self.device = runner.device
         self.memo: dict = {}
-        self.T = self.R = self.num_logit_rows = 0
+        self.T = self.R = self.num_logit_rows = self.num_qblocks = 0
+        self.qblock_token0 = self.qblock_count = None
         self.max_q = self.max_k = 0
         self.all_decode = False
         self.host_q_lens: list[int] = []
@@ -120,8 +121,10 @@ class ModelRunner:
         # layout of the metadata buffer (int32 elements)
         self._off = {}
         cursor = 0
+        self._max_qblocks = -(-t // 16) + r
         for name, size in (("token_ids", t), ("positions", t), ("token_request", t), ("logit_rows", t),
-                           ("cu_seqlens_q", r + 1), ("seq_lens_k", r), ("slot_ids", r)):
+                           ("cu_seqlens_q", r + 1), ("seq_lens_k", r), ("slot_ids", r),
+                           ("qblock_token0", self._max_qblocks), ("qblock_count", self._max_qblocks)):
             self._off[name] = (cursor, size)
             cursor += size
         for index in range(g):
@@ -235,6 +238,14 @@ class ModelRunner:
             rows[:cursor] = np.arange(cursor, dtype=np.int32)
             n_rows = cursor
         ctx.T, ctx.R, ctx.num_logit_rows = cursor, max(real, pad_to), n_rows
+        # blocks of at most 16 consecutive tokens of one request, the longest contexts first
+        starts = cu[:ctx.R + 1]
+        blocks = [(int(pos[min(t0 + 16, int(starts[i + 1])) - 1]), t0, min(16, int(starts[i + 1]) - t0))
+                  for i in range(ctx.R) for t0 in range(int(starts[i]), int(starts[i + 1]), 16)]
+        blocks.sort(key=lambda b: -b[0])
+        ctx.num_qblocks = len(blocks)
+        self._host_view("qblock_token0")[:len(blocks)] = [b[1] for b in blocks]
+        self._host_view("qblock_count")[:len(blocks)] = [b[2] for b in blocks]
         mb = cache.max_blocks
         for index, group in enumerate(cache.groups):
             table = self._host_view(f"table{index}").reshape(self.max_requests, mb)
@@ -256,6 +267,8 @@ class ModelRunner:
         ctx.token_request, ctx.logit_rows = self._view("token_request", ctx.T), self._view("logit_rows", max(ctx.num_logit_rows, 1))
         ctx.cu_seqlens_q, ctx.seq_lens_k = self._view("cu_seqlens_q", ctx.R + 1), self._view("seq_lens_k", ctx.R)
         ctx.slot_ids = self._view("slot_ids", ctx.R)
+        ctx.qblock_token0 = self._view("qblock_token0", ctx.num_qblocks)
+        ctx.qblock_count = self._view("qblock_count", ctx.num_qblocks)
         ctx._groups = [
             GroupStep(self._view(f"slots{i}", ctx.T), self._view(f"table{i}").view(self.max_requests, mb)[:ctx.R], self.cache.page_size)
             for i in range(len(self.cache.groups))

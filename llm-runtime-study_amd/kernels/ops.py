@@ -42,6 +42,8 @@ _SIGNATURES = {
                               c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_void_p]),
     "lrs_attention_decode": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p,
                                      c_void_p, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_int, c_void_p]),
+    "lrs_attention_prefill": (c_int, [c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p,
+                                      c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_void_p]),
     "lrs_choose_tokens": (c_int, [c_void_p, c_void_p, c_int64, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p]),
     "lrs_filter_logits": (c_int, [c_void_p, c_int64, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p]),
 }
@@ -285,6 +287,30 @@ def attention_decode(out: torch.Tensor, q: torch.Tensor, k_pages: torch.Tensor, 
         _dev(out, "out"), _rows(out, "out"), None if splits == 1 else _dev(part_o, "part_o"), None if splits == 1 else _dev(part_ml, "part_ml"),
         _dev(q, "q"), _rows(q, "q"), _dev(k_pages, "k_pages"), _dev(v_pages, "v_pages"), _dev(block_table, "block_table"), block_table.stride(0),
         _dev(token_request, "token_request"), _dev(positions, "positions"), tokens, nq, nkv, d, page_size, scale, window, splits, _stream()))
+
+
+def attention_prefill(out: torch.Tensor, q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, block_table: torch.Tensor,
+                      token_request: torch.Tensor, positions: torch.Tensor, qblock_token0: torch.Tensor, qblock_count: torch.Tensor,
+                      nq: int, scale: float, window: int = 0) -> None:
+    """attention() on matrix cores for any bfloat16 step.  qblock_token0 / qblock_count list blocks of at
+    most 16 consecutive tokens of one request that together cover every token of the step once."""
+    tokens = out.shape[0]
+    _need(k_pages.dim() == 4 and k_pages.is_contiguous() and v_pages.is_contiguous(), "attention_prefill: pages must be contiguous")
+    _, nkv, page_size, d = k_pages.shape
+    _need(v_pages.shape == (k_pages.shape[0], nkv, d, page_size), "attention_prefill: key pages must be [P, nkv, page, d] and value pages [P, nkv, d, page]")
+    _need(attention_decode_supported(q.dtype, nq, nkv, d, page_size), f"attention_prefill: unsupported shape nq={nq} nkv={nkv} d={d} page={page_size} {q.dtype}")
+    _need(out.shape[1] == nq * d and q.shape[0] == tokens and q.shape[1] >= nq * d, "attention_prefill: q/out widths do not match nq*d")
+    _need(q.dtype == k_pages.dtype == v_pages.dtype == out.dtype, "attention_prefill: q, pages and out must share a dtype")
+    _need(block_table.dim() == 2 and block_table.dtype == torch.int32 and block_table.stride(1) == 1, "attention_prefill: block_table must be int32 [R, blocks]")
+    for name, t in (("token_request", token_request), ("positions", positions)):
+        _need(t.dtype == torch.int32 and t.numel() >= tokens and t.is_contiguous(), f"attention_prefill: {name} must be int32 [T]")
+    n_blocks = qblock_token0.numel()
+    _need(n_blocks > 0 and qblock_count.numel() == n_blocks and qblock_token0.dtype == qblock_count.dtype == torch.int32
+          and qblock_token0.is_contiguous() and qblock_count.is_contiguous(), "attention_prefill: query blocks must be two int32 vectors of one length")
+    _check(library().lrs_attention_prefill(
+        _dev(out, "out"), _rows(out, "out"), _dev(q, "q"), _rows(q, "q"), _dev(k_pages, "k_pages"), _dev(v_pages, "v_pages"),
+        _dev(block_table, "block_table"), block_table.stride(0), _dev(token_request, "token_request"), _dev(positions, "positions"),
+        _dev(qblock_token0, "qblock_token0"), _dev(qblock_count, "qblock_count"), n_blocks, nq, nkv, d, page_size, scale, window, _stream()))
 
 
 # --------------------------------------------------------------- sampling

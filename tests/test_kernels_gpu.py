@@ -214,7 +214,7 @@ def _attention_reference(q, k_all, v_all, positions, lengths_before, nq, nkv, d,
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("nq,nkv,d,page,window", [
     (4, 2, 16, 4, 0), (8, 2, 32, 16, 0), (3, 1, 48, 8, 0), (6, 3, 80, 16, 0), (32, 8, 128, 16, 0),
-    (4, 4, 256, 64, 0), (8, 2, 32, 16, 7), (4, 2, 64, 16, 33),
+    (4, 4, 256, 64, 0), (8, 2, 32, 16, 7), (4, 2, 64, 16, 33), (16, 1, 96, 32, 0), (12, 4, 192, 16, 21),
 ])
 def test_attention_ragged_batch(ops, dtype, nq, nkv, d, page, window):
     g = torch.Generator().manual_seed(6)
@@ -256,6 +256,19 @@ def test_attention_ragged_batch(ops, dtype, nq, nkv, d, page, window):
                   dev(torch.tensor(tok_req, dtype=torch.int32)), dev(torch.tensor(tok_pos, dtype=torch.int32)),
                   nq, scale, window)
     torch.testing.assert_close(out.cpu().double(), want, **tol(dtype, 2e-5, 2e-2))
+    if ops.attention_decode_supported(dtype, nq, nkv, d, page):
+        # the matrix-core kernel for ragged steps: blocks of at most 16 tokens of one request, in any order
+        blocks, at = [], 0
+        for before, new in requests:
+            blocks += [(at + i, min(16, new - i)) for i in range(0, new, 16)]
+            at += new
+        blocks = blocks[::-1]
+        fast = torch.empty_like(out)
+        ops.attention_prefill(fast, dev(q_wide), dev(kp.to(dtype)), dev(vp.to(dtype)), dev(table),
+                              dev(torch.tensor(tok_req, dtype=torch.int32)), dev(torch.tensor(tok_pos, dtype=torch.int32)),
+                              dev(torch.tensor([b[0] for b in blocks], dtype=torch.int32)),
+                              dev(torch.tensor([b[1] for b in blocks], dtype=torch.int32)), nq, scale, window)
+        torch.testing.assert_close(fast.cpu().double(), want, rtol=2e-2, atol=2e-2)
 
 
 @pytest.mark.parametrize("nq,nkv,d,page,window,splits", [
