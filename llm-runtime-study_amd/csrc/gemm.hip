@@ -71,6 +71,7 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(void* __restrict__ out,
 // 32x32x16 tiles.  K is walked in slices of 32 through LDS.  Needs K % 8 == 0 so that
 // every 8-element chunk is a 16-byte aligned load; rows past M or N and chunks past K
 // are zero-filled.
+template <bool SWIGLU>
 __global__ __launch_bounds__(256) void gemm_bf16_mfma_kernel(void* __restrict__ out, int mode,
                                                              const bf16* __restrict__ a,
                                                              const bf16* __restrict__ w,
@@ -127,6 +128,20 @@ __global__ __launch_bounds__(256) void gemm_bf16_mfma_kernel(void* __restrict__ 
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
       const int gn = n0 + wn + j * 32 + lane % 32;
+      if (SWIGLU) {
+        // columns come in groups of 8 gate rows followed by the 8 up rows of the same features:
+        // the up value of a gate column sits 8 lanes further on
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const float up = __shfl(acc[i][j][r], (lane + 8) % WAVE, WAVE);
+          const int gm = m0 + wm + i * 32 + 8 * (r / 4) + 4 * (lane / 32) + r % 4;
+          if (gn % 16 < 8 && gn + 8 < n && gm < m) {
+            const float gate = acc[i][j][r];
+            emit<bf16>(out, mode, (int64_t)gm * ldc + (gn / 16) * 8 + gn % 8, gate / (1.0f + __expf(-gate)) * up);
+          }
+        }
+        continue;
+      }
       if (gn >= n) continue;
       const float b = bias ? (float)bias[gn] : 0.f;
 #pragma unroll
@@ -144,28 +159,83 @@ __global__ __launch_bounds__(256) void gemm_bf16_mfma_kernel(void* __restrict__ 
 // (16 rows x 32 k, each lane one 16-byte load of a row), the activations the B operand
 // (32 k x 16 tokens, read from L2); MT is the number of 16-token blocks.  UNROLL steps of 32 k
 // are loaded before any is used, so each wave keeps UNROLL KB of weights in flight.
-template <int MT, int WAVES, int UNROLL>
+//
+// NORM: the input is the float32 residual stream and the product is taken of its RMSNorm:
+//   y[m, n] = rsqrt(mean_k h[m,k]^2 + eps) * sum_k (h[m,k] * g[k]) W[n,k]
+// The row factor leaves the sum, so the B operand is bf16(h * g) and the factor is applied in
+// the epilogue; the waves of a workgroup read all of K between them, so the sum of squares
+// falls out of the loads they do anyway.  `rows` optionally picks the rows of h.
+// SWIGLU: the 16 weight rows of a workgroup are 8 gate rows followed by the 8 up rows of the
+// same features (the matrix is stored interleaved like that); the epilogue writes
+// silu(gate) * up, 8 columns per workgroup, into out [M, N/2].
+struct NormInput {
+  const float* h;        // [*, K] float32, row stride lda
+  const int* rows;       // optional: row of h for each of the m inputs
+  const void* weight;    // [K] norm weight
+  int weight_is_f32;
+  float eps;
+};
+
+__device__ __forceinline__ float silu(float g) { return g / (1.0f + __expf(-g)); }
+
+template <int MT, int WAVES, int UNROLL, bool NORM, bool SWIGLU>
 __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_skinny_kernel(
-    void* __restrict__ out, int mode, const bf16* __restrict__ x, const bf16* __restrict__ w,
-    const bf16* __restrict__ bias, int m, int n, int k, int lda, int ldc) {
+    void* __restrict__ out, int mode, const bf16* __restrict__ x, NormInput norm,
+    const bf16* __restrict__ w, const bf16* __restrict__ bias, int m, int n, int k, int lda, int ldc) {
   __shared__ floatx4 partial[WAVES][MT][WAVE];
+  __shared__ float sumsq[WAVES][MT][16];
   const int tid = threadIdx.x, lane = tid % WAVE, wave = tid / WAVE;
   const int r = lane & 15, g = lane >> 4;
   const int n0 = blockIdx.x * 16;
   const int row = n0 + r < n ? n0 + r : n - 1;
   const bf16* wp = w + (int64_t)row * k + g * 8;
   const bf16* xp[MT];
+  const float* hp[MT];
   bool live[MT];
+  float ss[MT];
 #pragma unroll
   for (int t = 0; t < MT; ++t) {
     const int token = t * 16 + r;
     live[t] = token < m;
-    xp[t] = x + (int64_t)(live[t] ? token : 0) * lda + g * 8;
+    ss[t] = 0.f;
+    if (NORM) {
+      const int64_t src = live[t] ? (norm.rows ? norm.rows[token] : token) : 0;
+      hp[t] = norm.h + src * lda + g * 8;
+    } else {
+      xp[t] = x + (int64_t)(live[t] ? token : 0) * lda + g * 8;
+    }
   }
   floatx4 acc[MT];
 #pragma unroll
   for (int t = 0; t < MT; ++t) acc[t] = floatx4{0.f, 0.f, 0.f, 0.f};
   const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
+
+  // B operand of one k step for token block t: 8 consecutive k of one token
+  auto load_b = [&](int t, int step) -> bf16x8 {
+    if (!live[t]) return zero;
+    if (!NORM) return *(const bf16x8*)(xp[t] + step * 32);
+    const floatx4 h0 = *(const floatx4*)(hp[t] + step * 32), h1 = *(const floatx4*)(hp[t] + step * 32 + 4);
+    float gw[8];
+    if (norm.weight_is_f32) {
+      const floatx4 g0 = *(const floatx4*)((const float*)norm.weight + step * 32 + g * 8);
+      const floatx4 g1 = *(const floatx4*)((const float*)norm.weight + step * 32 + g * 8 + 4);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) { gw[i] = g0[i]; gw[4 + i] = g1[i]; }
+    } else {
+      const bf16x8 gb = *(const bf16x8*)((const bf16*)norm.weight + step * 32 + g * 8);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) gw[i] = (float)gb[i];
+    }
+    bf16x8 b;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      ss[t] = fmaf(h0[i], h0[i], ss[t]);
+      ss[t] = fmaf(h1[i], h1[i], ss[t]);
+      b[i] = (bf16)(h0[i] * gw[i]);
+      b[4 + i] = (bf16)(h1[i] * gw[4 + i]);
+    }
+    return b;
+  };
 
   const int steps = (k + 31) / 32;
   const int per_wave = (steps + WAVES - 1) / WAVES;
@@ -179,7 +249,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_skinny_kernel(
 #pragma unroll
     for (int u = 0; u < UNROLL; ++u)
 #pragma unroll
-      for (int t = 0; t < MT; ++t) b[u][t] = live[t] ? *(const bf16x8*)(xp[t] + (s + u) * 32) : zero;
+      for (int t = 0; t < MT; ++t) b[u][t] = load_b(t, s + u);
 #pragma unroll
     for (int u = 0; u < UNROLL; ++u)
 #pragma unroll
@@ -190,60 +260,118 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_skinny_kernel(
     const bf16x8 a = inside ? *(const bf16x8*)(wp + s * 32) : zero;
 #pragma unroll
     for (int t = 0; t < MT; ++t) {
-      const bf16x8 b = (inside && live[t]) ? *(const bf16x8*)(xp[t] + s * 32) : zero;
+      const bf16x8 b = inside ? load_b(t, s) : zero;
       acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, acc[t], 0, 0, 0);
     }
   }
 #pragma unroll
-  for (int t = 0; t < MT; ++t) partial[wave][t][lane] = acc[t];
+  for (int t = 0; t < MT; ++t) {
+    partial[wave][t][lane] = acc[t];
+    if (NORM) {
+      float v = ss[t];
+      v += __shfl_xor(v, 16, WAVE);
+      v += __shfl_xor(v, 32, WAVE);
+      if (g == 0) sumsq[wave][t][r] = v;
+    }
+  }
   __syncthreads();
   // accumulator layout: token = t*16 + lane % 16, weight row = n0 + 4 * (lane / 16) + i
-  for (int e = tid; e < MT * WAVE * 4; e += WAVES * WAVE) {
-    const int t = e / (WAVE * 4), l = (e / 4) % WAVE, i = e % 4;
-    const int token = t * 16 + (l & 15), gn = n0 + 4 * (l >> 4) + i;
-    if (token >= m || gn >= n) continue;
+  auto total = [&](int t, int l, int i) -> float {
     float v = 0.f;
 #pragma unroll
     for (int wv = 0; wv < WAVES; ++wv) v += partial[wv][t][l][i];
-    if (bias) v += (float)bias[gn];
-    emit<bf16>(out, mode, (int64_t)token * ldc + gn, v);
+    if (NORM) {
+      float q = 0.f;
+#pragma unroll
+      for (int wv = 0; wv < WAVES; ++wv) q += sumsq[wv][t][l & 15];
+      v *= 1.0f / sqrtf(q / (float)k + norm.eps);
+    }
+    return v;
+  };
+  if (SWIGLU) {
+    for (int e = tid; e < MT * 16 * 8; e += WAVES * WAVE) {
+      const int t = e / 128, c = (e / 8) % 16, j = e % 8;
+      const int token = t * 16 + c, feature = blockIdx.x * 8 + j;
+      if (token >= m || n0 + 8 + j >= n) continue;
+      const float gate = total(t, ((j / 4) << 4) | c, j % 4), up = total(t, ((2 + j / 4) << 4) | c, j % 4);
+      emit<bf16>(out, mode, (int64_t)token * ldc + feature, silu(gate) * up);
+    }
+  } else {
+    for (int e = tid; e < MT * WAVE * 4; e += WAVES * WAVE) {
+      const int t = e / (WAVE * 4), l = (e / 4) % WAVE, i = e % 4;
+      const int token = t * 16 + (l & 15), gn = n0 + 4 * (l >> 4) + i;
+      if (token >= m || gn >= n) continue;
+      float v = total(t, l, i);
+      if (bias) v += (float)bias[gn];
+      emit<bf16>(out, mode, (int64_t)token * ldc + gn, v);
+    }
   }
 }
 
-template <int MT>
-static void launch_skinny(void* out, int mode, const bf16* a, const bf16* w, const bf16* bias, int m, int n,
-                          int k, int lda, int ldc, hipStream_t s) {
+template <int MT, bool NORM, bool SWIGLU>
+static void launch_skinny(void* out, int mode, const bf16* a, NormInput norm, const bf16* w, const bf16* bias,
+                          int m, int n, int k, int lda, int ldc, hipStream_t s) {
   const int tiles = (n + 15) / 16;
-  constexpr int UNROLL = MT == 1 ? 8 : (MT == 2 ? 4 : 2);
+  constexpr int UNROLL = NORM ? (MT == 1 ? 4 : 2) : (MT == 1 ? 8 : (MT == 2 ? 4 : 2));
   if (tiles <= 2048)
-    gemm_bf16_skinny_kernel<MT, 8, UNROLL><<<tiles, 8 * 64, 0, s>>>(out, mode, a, w, bias, m, n, k, lda, ldc);
+    gemm_bf16_skinny_kernel<MT, 8, UNROLL, NORM, SWIGLU><<<tiles, 8 * 64, 0, s>>>(out, mode, a, norm, w, bias, m, n, k, lda, ldc);
   else
-    gemm_bf16_skinny_kernel<MT, 4, UNROLL><<<tiles, 4 * 64, 0, s>>>(out, mode, a, w, bias, m, n, k, lda, ldc);
+    gemm_bf16_skinny_kernel<MT, 4, UNROLL, NORM, SWIGLU><<<tiles, 4 * 64, 0, s>>>(out, mode, a, norm, w, bias, m, n, k, lda, ldc);
 }
 
+template <bool NORM, bool SWIGLU>
+static void launch_skinny_m(void* out, int mode, const bf16* a, NormInput norm, const bf16* w, const bf16* bias,
+                            int m, int n, int k, int lda, int ldc, hipStream_t s) {
+  if (m <= 16) launch_skinny<1, NORM, SWIGLU>(out, mode, a, norm, w, bias, m, n, k, lda, ldc, s);
+  else if (m <= 32) launch_skinny<2, NORM, SWIGLU>(out, mode, a, norm, w, bias, m, n, k, lda, ldc, s);
+  else if (m <= 48) launch_skinny<3, NORM, SWIGLU>(out, mode, a, norm, w, bias, m, n, k, lda, ldc, s);
+  else launch_skinny<4, NORM, SWIGLU>(out, mode, a, norm, w, bias, m, n, k, lda, ldc, s);
+}
+
+// Largest M for which the few-rows kernel (and with it the fused RMSNorm input) is used.
+LRS_API int lrs_gemm_skinny_max_m() { return 64; }
+
 // out [M, N] (row stride ldc) = a [M, K] (row stride lda) times w[N, K]^T.
+//   norm_weight != null: `a` is the float32 residual stream [*, K]; its rows (picked through
+//     `rows` if given) are RMS-normalised with norm_weight and eps on the way in.  bf16 weights,
+//     M <= lrs_gemm_skinny_max_m() only.
+//   swiglu != 0: w holds gate and up rows interleaved in groups of 8 and out is [M, N/2] with
+//     silu(gate) * up.  bf16, K % 8 == 0, no bias.
 LRS_API int lrs_gemm(void* out, int mode, const void* a, const void* w, const void* bias, int dtype,
-                     int m, int n, int k, int lda, int ldc, void* stream) {
+                     int m, int n, int k, int lda, int ldc, const int* rows, const void* norm_weight,
+                     int norm_weight_dtype, float eps, int swiglu, void* stream) {
   LRS_REQUIRE(m > 0 && n > 0 && k > 0, "gemm: sizes m=%d n=%d k=%d must be positive", m, n, k);
-  LRS_REQUIRE(lda >= k && ldc >= n, "gemm: strides lda=%d ldc=%d too small for k=%d n=%d", lda, ldc, k, n);
+  LRS_REQUIRE(lda >= k && ldc >= (swiglu ? n / 2 : n), "gemm: strides lda=%d ldc=%d too small for k=%d n=%d", lda, ldc, k, n);
   LRS_REQUIRE(mode >= OUT_STORE && mode <= OUT_ADD_F32, "gemm: unknown output mode %d", mode);
   hipStream_t s = (hipStream_t)stream;
+  const bool normed = norm_weight != nullptr;
+  const bool aligned = k % 8 == 0 && lda % 8 == 0 && ((uintptr_t)a % 16 == 0) && ((uintptr_t)w % 16 == 0);
+  if (normed || swiglu) {
+    LRS_REQUIRE(dtype == LRS_BF16 && aligned, "gemm: fused norm / swiglu need bf16 weights and 16-byte aligned rows (k=%d lda=%d)", k, lda);
+    LRS_REQUIRE(!swiglu || (n % 16 == 0 && bias == nullptr && mode == OUT_STORE), "gemm: swiglu needs n %% 16 == 0, no bias and a stored output (n=%d)", n);
+    LRS_REQUIRE(!normed || m <= 64, "gemm: the fused norm input takes at most 64 rows, got %d", m);
+    LRS_REQUIRE(!normed || eps > 0.f, "gemm: eps must be positive");
+  }
+  LRS_REQUIRE(normed || rows == nullptr, "gemm: a row gather needs the fused norm input");
   if (dtype == LRS_F32) {
     dim3 grid((n + 63) / 64, (m + 63) / 64);
     gemm_tiled_kernel<float><<<grid, 256, 0, s>>>(out, mode, (const float*)a, (const float*)w,
                                                   (const float*)bias, m, n, k, lda, ldc);
   } else if (dtype == LRS_BF16) {
-    const bool aligned = k % 8 == 0 && lda % 8 == 0 && ((uintptr_t)a % 16 == 0) && ((uintptr_t)w % 16 == 0);
     if (aligned && m <= 64) {
-      const bf16 *ap = (const bf16*)a, *wp = (const bf16*)w, *bp = (const bf16*)bias;
-      if (m <= 16) launch_skinny<1>(out, mode, ap, wp, bp, m, n, k, lda, ldc, s);
-      else if (m <= 32) launch_skinny<2>(out, mode, ap, wp, bp, m, n, k, lda, ldc, s);
-      else if (m <= 48) launch_skinny<3>(out, mode, ap, wp, bp, m, n, k, lda, ldc, s);
-      else launch_skinny<4>(out, mode, ap, wp, bp, m, n, k, lda, ldc, s);
+      const bf16 *wp = (const bf16*)w, *bp = (const bf16*)bias;
+      const NormInput norm{(const float*)a, rows, norm_weight, norm_weight_dtype == LRS_F32, eps};
+      const bf16* ap = normed ? nullptr : (const bf16*)a;
+      if (normed && swiglu) launch_skinny_m<true, true>(out, mode, ap, norm, wp, bp, m, n, k, lda, ldc, s);
+      else if (normed) launch_skinny_m<true, false>(out, mode, ap, norm, wp, bp, m, n, k, lda, ldc, s);
+      else if (swiglu) launch_skinny_m<false, true>(out, mode, ap, norm, wp, bp, m, n, k, lda, ldc, s);
+      else launch_skinny_m<false, false>(out, mode, ap, norm, wp, bp, m, n, k, lda, ldc, s);
     } else if (aligned) {
       dim3 grid((n + 127) / 128, (m + 127) / 128);
-      gemm_bf16_mfma_kernel<<<grid, 256, 0, s>>>(out, mode, (const bf16*)a, (const bf16*)w,
-                                                 (const bf16*)bias, m, n, k, lda, ldc);
+      if (swiglu)
+        gemm_bf16_mfma_kernel<true><<<grid, 256, 0, s>>>(out, mode, (const bf16*)a, (const bf16*)w, (const bf16*)bias, m, n, k, lda, ldc);
+      else
+        gemm_bf16_mfma_kernel<false><<<grid, 256, 0, s>>>(out, mode, (const bf16*)a, (const bf16*)w, (const bf16*)bias, m, n, k, lda, ldc);
     } else {
       dim3 grid((n + 63) / 64, (m + 63) / 64);
       gemm_tiled_kernel<bf16><<<grid, 256, 0, s>>>(out, mode, (const bf16*)a, (const bf16*)w,

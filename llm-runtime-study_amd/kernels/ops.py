@@ -37,7 +37,9 @@ _SIGNATURES = {
     "lrs_silu_mul": (c_int, [c_void_p, c_void_p, c_int, c_int, c_int, c_void_p]),
     "lrs_fill_i32": (c_int, [c_void_p, c_int, c_int64, c_void_p]),
     "lrs_gather_rows": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p]),
-    "lrs_gemm": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p]),
+    "lrs_gemm": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p,
+                         c_int, c_float, c_int, c_void_p]),
+    "lrs_gemm_skinny_max_m": (c_int, []),
     "lrs_attention": (c_int, [c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p,
                               c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_void_p]),
     "lrs_attention_decode": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p,
@@ -215,26 +217,53 @@ def gather_rows(out: torch.Tensor, x: torch.Tensor, rows: torch.Tensor) -> None:
 
 
 # ------------------------------------------------------------------- gemm
-def gemm(out: torch.Tensor, a: torch.Tensor, w: torch.Tensor, bias: torch.Tensor | None = None, accumulate: bool = False) -> None:
-    """out = a @ w.T (+ bias).  `accumulate` adds into a float32 `out` instead of storing."""
-    m, k = a.shape
-    n = w.shape[0]
+def gemm_fuses_norm(dtype: torch.dtype, m: int, k: int) -> bool:
+    """Whether gemm() can take the float32 residual stream and normalise it on the way in."""
+    return dtype == torch.bfloat16 and m <= library().lrs_gemm_skinny_max_m() and k % 8 == 0
+
+
+def gemm(out: torch.Tensor, a: torch.Tensor, w: torch.Tensor, bias: torch.Tensor | None = None, accumulate: bool = False,
+         swiglu: bool = False, norm_weight: torch.Tensor | None = None, eps: float = 0.0, rows: torch.Tensor | None = None,
+         count: int | None = None) -> None:
+    """out = a @ w.T (+ bias).  `accumulate` adds into a float32 `out` instead of storing.
+
+    norm_weight: `a` is the float32 residual stream [*, K]; the product is taken of its RMSNorm
+    (weight norm_weight, eps), of the `count` rows listed in `rows` if given, else of its first rows.
+    swiglu: `w` holds gate and up rows interleaved in groups of 8; out [M, N/2] = silu(gate) * up.
+    """
+    n, k = w.shape
     lda, ldc = _rows(a, "a"), _rows(out, "out")
-    _need(w.dim() == 2 and w.is_contiguous() and w.shape[1] == k, f"gemm: weight must be contiguous [N, {k}], got {tuple(w.shape)}")
-    _need(out.shape == (m, n), f"gemm: out must be [{m}, {n}], got {tuple(out.shape)}")
-    _need(a.dtype == w.dtype, f"gemm: a is {a.dtype} but w is {w.dtype}")
+    _need(w.dim() == 2 and w.is_contiguous() and a.shape[1] == k, f"gemm: weight must be contiguous [N, {a.shape[1]}], got {tuple(w.shape)}")
+    normed = norm_weight is not None
+    if normed:
+        m = count if rows is not None else out.shape[0]
+        _need(a.dtype == torch.float32 and gemm_fuses_norm(w.dtype, m, k), f"gemm: the fused norm input needs a float32 input, bf16 weights and at most {library().lrs_gemm_skinny_max_m()} rows")
+        _need(norm_weight.numel() == k and norm_weight.is_contiguous() and eps > 0, "gemm: norm weight must hold K values and eps be positive")
+        if rows is None:
+            _need(a.shape[0] >= m, "gemm: input has fewer rows than the output")
+        else:
+            _need(rows.dtype == torch.int32 and rows.numel() >= m and rows.is_contiguous(), "gemm: rows must be int32")
+    else:
+        m = a.shape[0]
+        _need(rows is None, "gemm: a row gather needs the fused norm input")
+        _need(a.dtype == w.dtype, f"gemm: a is {a.dtype} but w is {w.dtype}")
+    _need(out.shape == (m, n // 2 if swiglu else n), f"gemm: out must be [{m}, {n // 2 if swiglu else n}], got {tuple(out.shape)}")
     if accumulate:
         _need(out.dtype == torch.float32, "gemm: accumulation needs a float32 output")
         mode = OUT_ADD_F32
-    elif out.dtype == a.dtype:
+    elif out.dtype == w.dtype:
         mode = OUT_STORE
     else:
-        _need(out.dtype == torch.float32, "gemm: output must be of the input dtype or float32")
+        _need(out.dtype == torch.float32, "gemm: output must be of the weight dtype or float32")
         mode = OUT_STORE_F32
     if bias is not None:
-        _need(bias.numel() == n and bias.dtype == a.dtype and bias.is_contiguous(), "gemm: bias must hold N values of the input dtype")
+        _need(bias.numel() == n and bias.dtype == w.dtype and bias.is_contiguous(), "gemm: bias must hold N values of the weight dtype")
+    if swiglu:
+        _need(w.dtype == torch.bfloat16 and n % 16 == 0 and k % 8 == 0 and bias is None and mode == OUT_STORE, "gemm: swiglu needs bf16, N % 16 == 0, K % 8 == 0, no bias, a stored output")
     _check(library().lrs_gemm(_dev(out, "out"), mode, _dev(a, "a"), _dev(w, "w"), None if bias is None else _dev(bias, "bias"),
-                              dtype_code(a.dtype), m, n, k, lda, ldc, _stream()))
+                              dtype_code(w.dtype), m, n, k, lda, ldc, None if rows is None else _dev(rows, "rows"),
+                              None if not normed else _dev(norm_weight, "norm_weight"), dtype_code(norm_weight.dtype) if normed else 0,
+                              eps, 1 if swiglu else 0, _stream()))
 
 
 # -------------------------------------------------------------- attention

@@ -12,6 +12,7 @@ import torch
 
 from ..kernels import ops
 from ..parts import TensorSpec, create
+from ..parts.linear import linear
 from .spec import ModelSpec
 
 
@@ -84,7 +85,10 @@ class DecoderModel:
     def logits(self, ctx, h: torch.Tensor) -> torch.Tensor:
         """float32 logits [n_wanted, V] at the rows of `h` listed in ctx.logit_rows."""
         n = ctx.num_logit_rows
-        x = self.final_norm.forward(ctx, h, rows=ctx.logit_rows, count=n)
+        try:
+            x = self.final_norm.forward(ctx, h, rows=ctx.logit_rows, count=n, lazy=True)
+        except TypeError:      # a norm kind without the lazy form
+            x = self.final_norm.forward(ctx, h, rows=ctx.logit_rows, count=n)
         out = ctx.scratch("logits", (n, self.spec.vocab_size), torch.float32)
-        ops.gemm(out, x, self.head)
+        linear(ctx, out, x, self.head)
         return out

@@ -20,10 +20,12 @@ import torch
 
 from ..kernels import ops
 from .base import PagedKVNeed, Part, PartSpec, TensorSpec, create, register
+from .linear import linear, rows_of
 
 
 class GQAAttention(Part):
     graph_safe = True  # launches only library kernels on arena buffers
+    takes_lazy_norm = True
 
     def __init__(self, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int, *,
                  position: PartSpec = PartSpec("none"), qk_norm: bool = False, qk_norm_eps: float = 1e-6,
@@ -90,11 +92,11 @@ class GQAAttention(Part):
     def forward(self, ctx, x, residual, cache):
         if cache is None:
             raise ValueError("attention needs a paged cache (its own, or the one it is told to read)")
-        t, d, nq = x.shape[0], self.head_dim, self.num_heads
+        t, d, nq = rows_of(x), self.head_dim, self.num_heads
         nkv = 0 if self.kv_shared else self.num_kv_heads
         group = ctx.group(cache.group)
         qkv = ctx.scratch("attn_qkv", (t, (nq + 2 * nkv) * d), ctx.dtype)
-        ops.gemm(qkv, x, self.w_qkv, self.b_qkv)
+        linear(ctx, qkv, x, self.w_qkv, self.b_qkv)
         tables = self.position.tables(ctx)
         cos, sin = tables if tables is not None else (None, None)
         ops.qk_prep(qkv, nq, nkv, d, self.q_norm, self.k_norm, self.qk_norm_eps, cos, sin,

@@ -42,10 +42,21 @@ class PreNormBlock(Part):
         return all(getattr(part, "graph_safe", False) for _, part in self._children())
 
     def forward(self, ctx, h, cache):
-        x = self.mixer_norm.forward(ctx, h)
+        # a consumer that says `takes_lazy_norm` gets the norm as a description to fold into its
+        # first matrix product; any other gets the normalised tensor
+        x = self._normed(ctx, self.mixer_norm, self.mixer, h)
         self.mixer.forward(ctx, x, h, cache)
-        x = self.ff_norm.forward(ctx, h)
+        x = self._normed(ctx, self.ff_norm, self.feed_forward, h)
         self.feed_forward.forward(ctx, x, h)
+
+    @staticmethod
+    def _normed(ctx, norm, consumer, h):
+        if getattr(consumer, "takes_lazy_norm", False):
+            try:
+                return norm.forward(ctx, h, lazy=True)
+            except TypeError:      # a norm kind without the lazy form
+                pass
+        return norm.forward(ctx, h)
 
 
 register("block", "prenorm", PreNormBlock)

@@ -8,6 +8,7 @@ from __future__ import annotations
 
 from ..kernels import ops
 from .base import Part, TensorSpec, register
+from .linear import LazyNorm
 
 
 class RMSNorm(Part):
@@ -27,12 +28,13 @@ class RMSNorm(Part):
     def bind(self, weights, dtype):
         self.weight = weights["weight"]
 
-    def forward(self, ctx, h, rows=None, count=None):
-        """Normalise rows of h [*, size] (all, or the `count` rows listed in `rows`)."""
+    def forward(self, ctx, h, rows=None, count=None, lazy: bool = False):
+        """Normalise rows of h [*, size] (all, or the `count` rows listed in `rows`).
+
+        With `lazy` the work is left to the consumer's matrix product (see parts/linear.py)."""
         n = h.shape[0] if rows is None else count
-        out = ctx.scratch("norm_out", (n, self.size), ctx.dtype)
-        ops.rmsnorm(out, h, self.weight, self.eps, rows=rows)
-        return out
+        pending = LazyNorm(h, self.weight, self.eps, rows, n)
+        return pending if lazy else pending.materialize(ctx)
 
 
 register("norm", "rmsnorm", RMSNorm)

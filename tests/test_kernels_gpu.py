@@ -28,6 +28,14 @@ def dev(t):
     return t.to("cuda")
 
 
+def close_in_norm(got, want, rel=1e-2):
+    """bfloat16 results of long sums: the error is a small part of the whole (relative L2 norm) and
+    no single element strays by more than a few units of the largest one's rounding."""
+    got, want = got.cpu().double(), want.double()
+    assert (got - want).norm() <= rel * want.norm(), f"relative error {(got - want).norm() / want.norm():.3g}"
+    assert (got - want).abs().max() <= 2e-2 * want.abs().max() + 2e-2, f"largest error {(got - want).abs().max():.3g}"
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("tokens,hidden,vocab", [(1, 64, 256), (7, 96, 331), (33, 4096, 1000)])
 def test_embed(ops, dtype, tokens, hidden, vocab):
@@ -171,6 +179,53 @@ def test_gemm(ops, dtype, m, n, k, mode):
         torch.testing.assert_close(out.cpu().double(), want, rtol=1e-2, atol=1e-2)
     else:  # bf16 inputs, float32 accumulation and output: only the summation order differs
         torch.testing.assert_close(out.cpu().double(), want, rtol=1e-4, atol=1e-4)
+
+
+@pytest.mark.parametrize("w_dtype", DTYPES)
+@pytest.mark.parametrize("m,n,k", [(1, 64, 96), (8, 331, 160), (17, 200, 96), (64, 6144, 4096), (33, 48, 264)])
+def test_gemm_with_fused_rmsnorm_input(ops, w_dtype, m, n, k):
+    """The product of the RMSNorm of float32 rows, picked through a row list, in one kernel."""
+    g = torch.Generator().manual_seed(14)
+    h = torch.randn(m + 3, k, generator=g) * 4
+    gamma = (1 + 0.2 * torch.randn(k, generator=g)).to(w_dtype)
+    w = (torch.randn(n, k, generator=g) / math.sqrt(k)).bfloat16()
+    rows = torch.randperm(m + 3, generator=g)[:m].to(torch.int32)
+    eps = 1e-5
+    assert ops.gemm_fuses_norm(torch.bfloat16, m, k)
+    normed = gamma.double() * (h.double() * torch.rsqrt(h.double().square().mean(-1, keepdim=True) + eps))
+    want = normed[rows.long()] @ w.double().T
+    out = torch.empty(m, n, device="cuda")
+    ops.gemm(out, dev(h), dev(w), norm_weight=dev(gamma), eps=eps, rows=dev(rows), count=m)
+    close_in_norm(out, want, 5e-3)
+    # without a row list the first m rows are taken; against the two-kernel path the only
+    # difference is where the input is rounded to bfloat16
+    x = torch.empty(m, k, device="cuda", dtype=torch.bfloat16)
+    ops.rmsnorm(x, dev(h), dev(gamma), eps)
+    two = torch.empty(m, n, device="cuda")
+    ops.gemm(two, x, dev(w))
+    ops.gemm(out, dev(h), dev(w), norm_weight=dev(gamma), eps=eps)
+    close_in_norm(out, two.cpu(), 5e-3)
+
+
+@pytest.mark.parametrize("m,inter,k", [(1, 128, 64), (9, 160, 96), (64, 12288, 4096), (65, 160, 96), (300, 136, 264)])
+def test_gemm_with_swiglu_epilogue(ops, m, inter, k):
+    """Gate and up rows interleaved in groups of 8; the product writes silu(gate) * up."""
+    g = torch.Generator().manual_seed(15)
+    x = torch.randn(m, k, generator=g).bfloat16()
+    gate = (torch.randn(inter, k, generator=g) / math.sqrt(k) * 2).bfloat16()
+    up = (torch.randn(inter, k, generator=g) / math.sqrt(k) * 2).bfloat16()
+    mixed = torch.stack((gate.view(inter // 8, 8, k), up.view(inter // 8, 8, k)), 1).reshape(2 * inter, k).contiguous()
+    want = torch.nn.functional.silu(x.double() @ gate.double().T) * (x.double() @ up.double().T)
+    out = torch.empty(m, inter, device="cuda", dtype=torch.bfloat16)
+    ops.gemm(out, dev(x), dev(mixed), swiglu=True)
+    close_in_norm(out, want)
+    if m <= 64:   # with the normalisation folded in as well
+        h = torch.randn(m, k, generator=g) * 3
+        gamma = (1 + 0.1 * torch.randn(k, generator=g)).bfloat16()
+        xn = gamma.double() * (h.double() * torch.rsqrt(h.double().square().mean(-1, keepdim=True) + 1e-6))
+        want = torch.nn.functional.silu(xn @ gate.double().T) * (xn @ up.double().T)
+        ops.gemm(out, dev(h), dev(mixed), swiglu=True, norm_weight=dev(gamma), eps=1e-6)
+        close_in_norm(out, want)
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
