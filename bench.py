@@ -48,6 +48,7 @@ def parse_args():
     parser.add_argument("--dtype", choices=("bfloat16", "float32"), default="bfloat16")
     parser.add_argument("--no-points", action="store_true", help="skip the batch 1 and 64 decode points")
     parser.add_argument("--no-graph", action="store_true")
+    parser.add_argument("--own-gemm", action="store_true", help="this package's kernel also for products of many rows (default: vendor library)")
     return parser.parse_args()
 
 
@@ -136,7 +137,7 @@ def main() -> int:
     max_seq_len = args.context + args.steps + args.warmup + 2 * max_batch + 64
     max_seq_len = max(max_seq_len, args.prefill_tokens)
     engine = Engine.from_config(config, seed=0, dtype=args.dtype, max_seq_len=max_seq_len, max_batch_size=max_batch,
-                                max_num_batched_tokens=max(2048, args.prefill_tokens), use_cuda_graph=not args.no_graph)
+                                max_num_batched_tokens=max(2048, args.prefill_tokens), use_cuda_graph=not args.no_graph, library_gemm=not args.own_gemm)
     dtype_name = "bf16" if args.dtype == "bfloat16" else "fp32"
 
     prefill_times = measure_prefill(engine, args.prefill_tokens, repeats=3, seed=1)
@@ -176,7 +177,8 @@ def main() -> int:
             "num_attention_heads": config.num_attention_heads, "num_key_value_heads": config.num_key_value_heads,
             "head_dim": config.head_dim, "vocab_size": config.vocab_size, "global_batch": args.batch,
             "seq_len": args.context, "new_tokens": args.steps + args.warmup, "page_size": engine.page_size,
-            "prefill_tokens": args.prefill_tokens, "hip_graph": bool(engine.runner.use_graph), "parallelism": "single GPU",
+            "prefill_tokens": args.prefill_tokens, "hip_graph": bool(engine.runner.use_graph), "prefill_gemm": "own" if args.own_gemm else "hipBLASLt",
+            "parallelism": "single GPU",
         },
         "prefill": {
             "value": round(args.prefill_tokens / prefill_s, 1), "tokens": args.prefill_tokens,

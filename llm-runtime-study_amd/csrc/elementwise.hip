@@ -171,30 +171,55 @@ LRS_API int lrs_qk_prep(void* qkv, int dtype, int tokens, int row_stride, int nq
 }
 
 // ----------------------------------------------------------- gated activation
-// out[t, i] = silu(gu[t, i]) * gu[t, inter + i], silu evaluated in float32.
+// out[t, i] = silu(gate) * up, silu evaluated in float32.  Plain layout: gate = gu[t, i],
+// up = gu[t, inter + i].  Interleaved layout (groups of 8 gate columns followed by the 8 up
+// columns of the same features): gate = gu[t, 16*(i/8) + i%8], up = the column 8 further on.
 template <typename T>
-__global__ void silu_mul_kernel(T* __restrict__ out, const T* __restrict__ gu, int inter, int64_t total) {
+__global__ void silu_mul_kernel(T* __restrict__ out, const T* __restrict__ gu, int inter, int64_t total,
+                                int interleaved) {
   for (int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total;
        idx += (int64_t)gridDim.x * blockDim.x) {
     const int64_t t = idx / inter, i = idx % inter;
-    const float g = to_float(gu[t * 2 * inter + i]);
-    const float u = to_float(gu[t * 2 * inter + inter + i]);
+    const int64_t gate_at = interleaved ? t * 2 * inter + 16 * (i / 8) + i % 8 : t * 2 * inter + i;
+    const float g = to_float(gu[gate_at]);
+    const float u = to_float(gu[gate_at + (interleaved ? 8 : inter)]);
     out[idx] = from_float<T>(g / (1.0f + expf(-g)) * u);
   }
 }
 
-LRS_API int lrs_silu_mul(void* out, const void* gu, int dtype, int tokens, int inter, void* stream) {
+LRS_API int lrs_silu_mul(void* out, const void* gu, int dtype, int tokens, int inter, int interleaved, void* stream) {
   LRS_REQUIRE(tokens > 0 && inter > 0, "silu_mul: tokens=%d inter=%d must be positive", tokens, inter);
+  LRS_REQUIRE(!interleaved || inter % 8 == 0, "silu_mul: the interleaved layout needs inter %% 8 == 0, got %d", inter);
   const int64_t total = (int64_t)tokens * inter;
   const int blocks = (int)((total + 255) / 256 < 65536 ? (total + 255) / 256 : 65536);
   hipStream_t s = (hipStream_t)stream;
   if (dtype == LRS_F32)
-    silu_mul_kernel<float><<<blocks, 256, 0, s>>>((float*)out, (const float*)gu, inter, total);
+    silu_mul_kernel<float><<<blocks, 256, 0, s>>>((float*)out, (const float*)gu, inter, total, interleaved);
   else if (dtype == LRS_BF16)
-    silu_mul_kernel<bf16><<<blocks, 256, 0, s>>>((bf16*)out, (const bf16*)gu, inter, total);
+    silu_mul_kernel<bf16><<<blocks, 256, 0, s>>>((bf16*)out, (const bf16*)gu, inter, total, interleaved);
   else
     return lrs_fail("silu_mul: unknown dtype %d", dtype);
   return lrs_check_launch("silu_mul");
+}
+
+// -------------------------------------------------------------- residual add
+// residual[i] += y[i]: the float32 residual stream takes the output of a product that was
+// computed into the activation dtype.
+template <typename T>
+__global__ void add_into_kernel(float* __restrict__ residual, const T* __restrict__ y, int64_t total) {
+  for (int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total;
+       idx += (int64_t)gridDim.x * blockDim.x)
+    residual[idx] += to_float(y[idx]);
+}
+
+LRS_API int lrs_add_into(float* residual, const void* y, int dtype, int64_t total, void* stream) {
+  LRS_REQUIRE(total > 0, "add_into: nothing to add");
+  const int blocks = (int)((total + 255) / 256 < 65536 ? (total + 255) / 256 : 65536);
+  hipStream_t s = (hipStream_t)stream;
+  if (dtype == LRS_F32) add_into_kernel<float><<<blocks, 256, 0, s>>>(residual, (const float*)y, total);
+  else if (dtype == LRS_BF16) add_into_kernel<bf16><<<blocks, 256, 0, s>>>(residual, (const bf16*)y, total);
+  else return lrs_fail("add_into: unknown dtype %d", dtype);
+  return lrs_check_launch("add_into");
 }
 
 // ------------------------------------------------------------------ utilities

@@ -178,17 +178,22 @@ struct NormInput {
 
 __device__ __forceinline__ float silu(float g) { return g / (1.0f + __expf(-g)); }
 
-template <int MT, int WAVES, int UNROLL, bool NORM, bool SWIGLU>
+template <int MT, int RT, int WAVES, int UNROLL, bool NORM, bool SWIGLU>
 __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_skinny_kernel(
     void* __restrict__ out, int mode, const bf16* __restrict__ x, NormInput norm,
     const bf16* __restrict__ w, const bf16* __restrict__ bias, int m, int n, int k, int lda, int ldc) {
+  // RT: row tiles of 16 weight rows per workgroup; every activation fragment is used RT times
   __shared__ floatx4 partial[WAVES][MT][WAVE];
   __shared__ float sumsq[WAVES][MT][16];
   const int tid = threadIdx.x, lane = tid % WAVE, wave = tid / WAVE;
   const int r = lane & 15, g = lane >> 4;
-  const int n0 = blockIdx.x * 16;
-  const int row = n0 + r < n ? n0 + r : n - 1;
-  const bf16* wp = w + (int64_t)row * k + g * 8;
+  const int n0 = blockIdx.x * 16 * RT;
+  const bf16* wp[RT];
+#pragma unroll
+  for (int q = 0; q < RT; ++q) {
+    const int row = n0 + q * 16 + r < n ? n0 + q * 16 + r : n - 1;
+    wp[q] = w + (int64_t)row * k + g * 8;
+  }
   const bf16* xp[MT];
   const float* hp[MT];
   bool live[MT];
@@ -205,9 +210,11 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_skinny_kernel(
       xp[t] = x + (int64_t)(live[t] ? token : 0) * lda + g * 8;
     }
   }
-  floatx4 acc[MT];
+  floatx4 acc[RT][MT];
 #pragma unroll
-  for (int t = 0; t < MT; ++t) acc[t] = floatx4{0.f, 0.f, 0.f, 0.f};
+  for (int q = 0; q < RT; ++q)
+#pragma unroll
+    for (int t = 0; t < MT; ++t) acc[q][t] = floatx4{0.f, 0.f, 0.f, 0.f};
   const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
 
   // B operand of one k step for token block t: 8 consecutive k of one token
@@ -243,9 +250,11 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_skinny_kernel(
   const int s_end = s + per_wave < steps ? s + per_wave : steps;
   const int full_end = k / 32 < s_end ? k / 32 : s_end;   // steps whose 32 k are all inside K
   for (; s + UNROLL <= full_end; s += UNROLL) {
-    bf16x8 a[UNROLL], b[UNROLL][MT];
+    bf16x8 a[UNROLL][RT], b[UNROLL][MT];
 #pragma unroll
-    for (int u = 0; u < UNROLL; ++u) a[u] = *(const bf16x8*)(wp + (s + u) * 32);
+    for (int u = 0; u < UNROLL; ++u)
+#pragma unroll
+      for (int q = 0; q < RT; ++q) a[u][q] = *(const bf16x8*)(wp[q] + (s + u) * 32);
 #pragma unroll
     for (int u = 0; u < UNROLL; ++u)
 #pragma unroll
@@ -253,29 +262,33 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_skinny_kernel(
 #pragma unroll
     for (int u = 0; u < UNROLL; ++u)
 #pragma unroll
-      for (int t = 0; t < MT; ++t) acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[u], b[u][t], acc[t], 0, 0, 0);
+      for (int q = 0; q < RT; ++q)
+#pragma unroll
+        for (int t = 0; t < MT; ++t)
+          acc[q][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[u][q], b[u][t], acc[q][t], 0, 0, 0);
   }
   for (; s < s_end; ++s) {
     const bool inside = s * 32 + g * 8 < k;
-    const bf16x8 a = inside ? *(const bf16x8*)(wp + s * 32) : zero;
+    bf16x8 b[MT];
 #pragma unroll
-    for (int t = 0; t < MT; ++t) {
-      const bf16x8 b = inside ? load_b(t, s) : zero;
-      acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, acc[t], 0, 0, 0);
+    for (int t = 0; t < MT; ++t) b[t] = inside ? load_b(t, s) : zero;
+#pragma unroll
+    for (int q = 0; q < RT; ++q) {
+      const bf16x8 a = inside ? *(const bf16x8*)(wp[q] + s * 32) : zero;
+#pragma unroll
+      for (int t = 0; t < MT; ++t) acc[q][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b[t], acc[q][t], 0, 0, 0);
     }
   }
+  if (NORM) {
 #pragma unroll
-  for (int t = 0; t < MT; ++t) {
-    partial[wave][t][lane] = acc[t];
-    if (NORM) {
+    for (int t = 0; t < MT; ++t) {
       float v = ss[t];
       v += __shfl_xor(v, 16, WAVE);
       v += __shfl_xor(v, 32, WAVE);
       if (g == 0) sumsq[wave][t][r] = v;
     }
   }
-  __syncthreads();
-  // accumulator layout: token = t*16 + lane % 16, weight row = n0 + 4 * (lane / 16) + i
+  // accumulator layout: token = t*16 + lane % 16, weight row = tile row 4 * (lane / 16) + i
   auto total = [&](int t, int l, int i) -> float {
     float v = 0.f;
 #pragma unroll
@@ -288,35 +301,56 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_skinny_kernel(
     }
     return v;
   };
-  if (SWIGLU) {
-    for (int e = tid; e < MT * 16 * 8; e += WAVES * WAVE) {
-      const int t = e / 128, c = (e / 8) % 16, j = e % 8;
-      const int token = t * 16 + c, feature = blockIdx.x * 8 + j;
-      if (token >= m || n0 + 8 + j >= n) continue;
-      const float gate = total(t, ((j / 4) << 4) | c, j % 4), up = total(t, ((2 + j / 4) << 4) | c, j % 4);
-      emit<bf16>(out, mode, (int64_t)token * ldc + feature, silu(gate) * up);
-    }
-  } else {
-    for (int e = tid; e < MT * WAVE * 4; e += WAVES * WAVE) {
-      const int t = e / (WAVE * 4), l = (e / 4) % WAVE, i = e % 4;
-      const int token = t * 16 + (l & 15), gn = n0 + 4 * (l >> 4) + i;
-      if (token >= m || gn >= n) continue;
-      float v = total(t, l, i);
-      if (bias) v += (float)bias[gn];
-      emit<bf16>(out, mode, (int64_t)token * ldc + gn, v);
+#pragma unroll
+  for (int q = 0; q < RT; ++q) {
+    if (q) __syncthreads();
+#pragma unroll
+    for (int t = 0; t < MT; ++t) partial[wave][t][lane] = acc[q][t];
+    __syncthreads();
+    const int nq0 = n0 + q * 16;
+    if (SWIGLU) {
+      for (int e = tid; e < MT * 16 * 8; e += WAVES * WAVE) {
+        const int t = e / 128, c = (e / 8) % 16, j = e % 8;
+        const int token = t * 16 + c, feature = nq0 / 2 + j;
+        if (token >= m || nq0 + 8 + j >= n) continue;
+        const float gate = total(t, ((j / 4) << 4) | c, j % 4), up = total(t, ((2 + j / 4) << 4) | c, j % 4);
+        emit<bf16>(out, mode, (int64_t)token * ldc + feature, silu(gate) * up);
+      }
+    } else {
+      for (int e = tid; e < MT * WAVE * 4; e += WAVES * WAVE) {
+        const int t = e / (WAVE * 4), l = (e / 4) % WAVE, i = e % 4;
+        const int token = t * 16 + (l & 15), gn = nq0 + 4 * (l >> 4) + i;
+        if (token >= m || gn >= n) continue;
+        float v = total(t, l, i);
+        if (bias) v += (float)bias[gn];
+        emit<bf16>(out, mode, (int64_t)token * ldc + gn, v);
+      }
     }
   }
+}
+
+// Row tiles per workgroup: more of them means each activation fragment read from L2 serves more
+// weight rows, which matters once there are several token blocks; fewer means more workgroups.
+template <int MT, int RT, bool NORM, bool SWIGLU>
+static void launch_skinny_rt(void* out, int mode, const bf16* a, NormInput norm, const bf16* w, const bf16* bias,
+                             int m, int n, int k, int lda, int ldc, hipStream_t s) {
+  const int groups = (n + 16 * RT - 1) / (16 * RT);
+  constexpr int UNROLL = (NORM ? 4 : 8) / (MT * RT > 4 ? 4 : (MT * RT > 1 ? 2 : 1));
+  if (groups <= 2048)
+    gemm_bf16_skinny_kernel<MT, RT, 8, UNROLL, NORM, SWIGLU><<<groups, 8 * 64, 0, s>>>(out, mode, a, norm, w, bias, m, n, k, lda, ldc);
+  else
+    gemm_bf16_skinny_kernel<MT, RT, 4, UNROLL, NORM, SWIGLU><<<groups, 4 * 64, 0, s>>>(out, mode, a, norm, w, bias, m, n, k, lda, ldc);
 }
 
 template <int MT, bool NORM, bool SWIGLU>
 static void launch_skinny(void* out, int mode, const bf16* a, NormInput norm, const bf16* w, const bf16* bias,
                           int m, int n, int k, int lda, int ldc, hipStream_t s) {
-  const int tiles = (n + 15) / 16;
-  constexpr int UNROLL = NORM ? (MT == 1 ? 4 : 2) : (MT == 1 ? 8 : (MT == 2 ? 4 : 2));
-  if (tiles <= 2048)
-    gemm_bf16_skinny_kernel<MT, 8, UNROLL, NORM, SWIGLU><<<tiles, 8 * 64, 0, s>>>(out, mode, a, norm, w, bias, m, n, k, lda, ldc);
+  if (MT == 1 || n <= 32 * 128)
+    launch_skinny_rt<MT, 1, NORM, SWIGLU>(out, mode, a, norm, w, bias, m, n, k, lda, ldc, s);
+  else if (n < 64 * 256)
+    launch_skinny_rt<MT, 2, NORM, SWIGLU>(out, mode, a, norm, w, bias, m, n, k, lda, ldc, s);
   else
-    gemm_bf16_skinny_kernel<MT, 4, UNROLL, NORM, SWIGLU><<<tiles, 4 * 64, 0, s>>>(out, mode, a, norm, w, bias, m, n, k, lda, ldc);
+    launch_skinny_rt<MT, (MT > 1 ? 4 : 1), NORM, SWIGLU>(out, mode, a, norm, w, bias, m, n, k, lda, ldc, s);
 }
 
 template <bool NORM, bool SWIGLU>

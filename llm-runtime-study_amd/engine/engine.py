@@ -32,7 +32,7 @@ class Engine:
     def __init__(self, config, model, *, device, dtype, max_seq_len: int = 4096, max_batch_size: int = 1,
                  cache_backend: str = "paged", use_cuda_graph: bool = True, page_size: int = DEFAULT_PAGE_SIZE,
                  max_num_batched_tokens: int | None = None, num_pages: int | None = None, tokenizer=None,
-                 load_seconds: float = 0.0):
+                 load_seconds: float = 0.0, library_gemm: bool = True):
         if max_batch_size <= 0:
             raise EngineError("max_batch_size must be positive")
         if cache_backend != "paged":
@@ -44,6 +44,7 @@ class Engine:
         self.page_size = page_size
         self.max_num_batched_tokens = max(max_batch_size, max_num_batched_tokens or min(DEFAULT_STEP_TOKENS, max_seq_len))
         self.num_pages = num_pages
+        self.library_gemm = library_gemm
         self.tokenizer = tokenizer
         self.load_seconds = load_seconds
         self.quantization = "dense"
@@ -91,7 +92,8 @@ class Engine:
                                  max_requests=self.max_batch_size, max_seq_len=self.max_seq_len,
                                  dtype=self.dtype, device=self.device)
             self._runner = ModelRunner(self.model, cache, max_step_tokens=self.max_num_batched_tokens,
-                                       dtype=self.dtype, device=self.device, use_graph=self.use_cuda_graph)
+                                       dtype=self.dtype, device=self.device, use_graph=self.use_cuda_graph,
+                                       library_gemm=self.library_gemm)
         return self._runner
 
     @property

@@ -80,6 +80,7 @@ class StepContext:
 
     def __init__(self, runner: "ModelRunner"):
         self._runner = runner
+        self.library_gemm = runner.library_gemm
         self.dtype = runner.dtype
         self.device = runner.device
         self.memo: dict = {}
@@ -106,13 +107,15 @@ class StepContext:
 
 class ModelRunner:
     def __init__(self, model: DecoderModel, cache: CacheManager, *, max_step_tokens: int, dtype: torch.dtype, device,
-                 use_graph: bool = False):
+                 use_graph: bool = False, library_gemm: bool = True):
         if max_step_tokens <= 0:
             raise GenerationError(f"max_step_tokens must be positive, got {max_step_tokens}")
         self.model, self.cache, self.dtype, self.device = model, cache, dtype, torch.device(device)
         self.max_step_tokens = max_step_tokens
         self.max_requests = cache.max_requests
         self.arena = ScratchArena(self.device)
+        # bfloat16 products of more rows than the few-rows kernel takes go to the vendor library
+        self.library_gemm = library_gemm
         # decode-only steps are captured in a HIP graph per padded batch size and replayed
         self.use_graph = use_graph and model.graph_safe()
         self._graphs: dict[int, tuple] = {}   # bucket -> (handle, arena generation, logits tensor)
@@ -311,7 +314,8 @@ class ModelRunner:
         while bucket < len(entries):
             bucket *= 2
         bucket = min(bucket, self.max_requests)
-        return bucket if bucket <= self.max_step_tokens else 0
+        # a graph holds this package's kernels only: batches the few-rows kernels do not take run eagerly
+        return bucket if bucket <= min(self.max_step_tokens, ops.skinny_max_m()) else 0
 
     def _step_graph(self, entries: Sequence[StepEntry], bucket: int) -> torch.Tensor | None:
         """Replay (capturing first if needed) the graph of a decode step padded to `bucket` rows.

@@ -34,7 +34,8 @@ _SIGNATURES = {
     "lrs_rope_table": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p]),
     "lrs_qk_prep": (c_int, [c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_int, c_float,
                             c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p]),
-    "lrs_silu_mul": (c_int, [c_void_p, c_void_p, c_int, c_int, c_int, c_void_p]),
+    "lrs_silu_mul": (c_int, [c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p]),
+    "lrs_add_into": (c_int, [c_void_p, c_void_p, c_int, c_int64, c_void_p]),
     "lrs_fill_i32": (c_int, [c_void_p, c_int, c_int64, c_void_p]),
     "lrs_gather_rows": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p]),
     "lrs_gemm": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p,
@@ -198,10 +199,22 @@ def qk_prep(qkv: torch.Tensor, nq: int, nkv: int, d: int, q_weight, k_weight, ep
         None if nkv == 0 else _dev(slots, "slots"), page_size, _stream()))
 
 
-def silu_mul(out: torch.Tensor, gate_up: torch.Tensor) -> None:
+def silu_mul(out: torch.Tensor, gate_up: torch.Tensor, interleaved: bool = False) -> None:
+    """out = silu(gate) * up; gate_up holds [gate | up], or groups of 8 gate then 8 up columns if `interleaved`."""
     tokens, inter = out.shape
     _need(out.is_contiguous() and gate_up.is_contiguous() and gate_up.shape == (tokens, 2 * inter) and gate_up.dtype == out.dtype, "silu_mul: gate_up must be [T, 2I] and out [T, I], same dtype")
-    _check(library().lrs_silu_mul(_dev(out, "out"), _dev(gate_up, "gate_up"), dtype_code(out.dtype), tokens, inter, _stream()))
+    _check(library().lrs_silu_mul(_dev(out, "out"), _dev(gate_up, "gate_up"), dtype_code(out.dtype), tokens, inter, 1 if interleaved else 0, _stream()))
+
+
+def add_into(residual: torch.Tensor, y: torch.Tensor) -> None:
+    """residual (float32) += y, same shape, both contiguous."""
+    _need(residual.dtype == torch.float32 and residual.shape == y.shape and residual.is_contiguous() and y.is_contiguous(), "add_into: float32 residual and y of one contiguous shape needed")
+    _check(library().lrs_add_into(_dev(residual, "residual"), _dev(y, "y"), dtype_code(y.dtype), residual.numel(), _stream()))
+
+
+def skinny_max_m() -> int:
+    """Most rows the few-rows product kernel takes."""
+    return library().lrs_gemm_skinny_max_m()
 
 
 def fill_i32(dst: torch.Tensor, value: int) -> None:
@@ -220,6 +233,13 @@ def gather_rows(out: torch.Tensor, x: torch.Tensor, rows: torch.Tensor) -> None:
 def gemm_fuses_norm(dtype: torch.dtype, m: int, k: int) -> bool:
     """Whether gemm() can take the float32 residual stream and normalise it on the way in."""
     return dtype == torch.bfloat16 and m <= library().lrs_gemm_skinny_max_m() and k % 8 == 0
+
+
+def gemm_norm_fusion_pays(n: int) -> bool:
+    """Every workgroup of the fused kernel normalises the whole input again, so the fusion costs
+    more than the norm kernel it saves once the weight matrix has many rows (measured on MI355X:
+    even at 6144 rows it only breaks even)."""
+    return n <= 4096
 
 
 def gemm(out: torch.Tensor, a: torch.Tensor, w: torch.Tensor, bias: torch.Tensor | None = None, accumulate: bool = False,

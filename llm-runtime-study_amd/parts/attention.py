@@ -117,7 +117,7 @@ class GQAAttention(Part):
         else:
             ops.attention(out, qkv, cache.k_pages, cache.v_pages, group.block_table, ctx.token_request, ctx.positions,
                           nq, self.scale, self.window or 0)
-        ops.gemm(residual, out, self.w_o, accumulate=True)
+        linear(ctx, residual, out, self.w_o, accumulate=True)
 
 
 register("mixer", "gqa_attention", GQAAttention)

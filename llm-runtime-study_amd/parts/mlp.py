@@ -57,7 +57,7 @@ class SwiGLU(Part):
             gate_up = ctx.scratch("ffn_gate_up", (t, 2 * self.intermediate_size), ctx.dtype)
             linear(ctx, gate_up, x, self.gate_up)
             ops.silu_mul(act, gate_up)
-        ops.gemm(residual, act, self.down, accumulate=True)
+        linear(ctx, residual, act, self.down, accumulate=True)
 
 
 register("feed_forward", "swiglu", SwiGLU)

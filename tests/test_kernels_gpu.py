@@ -152,6 +152,20 @@ def test_silu_mul(ops, dtype, tokens, inter):
     ops.silu_mul(out, dev(gu))
     gate, up = gu.float()[:, :inter], gu.float()[:, inter:]
     torch.testing.assert_close(out.cpu().float(), torch.nn.functional.silu(gate) * up, **tol(dtype, 1e-6, 1e-2))
+    if inter % 8 == 0:   # groups of 8 gate columns followed by their 8 up columns
+        mixed = torch.stack((gu[:, :inter].view(tokens, inter // 8, 8), gu[:, inter:].view(tokens, inter // 8, 8)), 2).reshape(tokens, 2 * inter)
+        ops.silu_mul(out, dev(mixed.contiguous()), interleaved=True)
+        torch.testing.assert_close(out.cpu().float(), torch.nn.functional.silu(gate) * up, **tol(dtype, 1e-6, 1e-2))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_add_into(ops, dtype):
+    g = torch.Generator().manual_seed(13)
+    residual = torch.randn(37, 331, generator=g)
+    y = torch.randn(37, 331, generator=g).to(dtype)
+    out = dev(residual.clone())
+    ops.add_into(out, dev(y))
+    torch.testing.assert_close(out.cpu(), residual + y.float(), rtol=0, atol=0)
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
