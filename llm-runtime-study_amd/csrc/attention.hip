@@ -134,25 +134,38 @@ __global__ __launch_bounds__(256) void attention_decode_bf16_kernel(
   float run_max = -INFINITY, run_sum = 0.f;
   const float scale2 = scale * 1.4426950408889634f;
 
+  // Every key and value fragment of a tile is requested before any is used, so a tile costs one
+  // trip to memory instead of two.
   for (int tile = tile_begin + wave; tile < tile_end; tile += WAVES) {
-    floatx4 s[2];
-    int64_t vbase[2];
     bool present[2];
+    bf16x8 kf[2][DS];
+    bf16x4 vf[2][DB];
 #pragma unroll
     for (int h = 0; h < 2; ++h) {
       const int key0 = tile * 32 + h * 16;
       present[h] = key0 <= pos && key0 + 15 >= lo;
-      s[h] = floatx4{0.f, 0.f, 0.f, 0.f};
-      vbase[h] = 0;
       if (present[h]) {
         const int64_t page = table[key0 / page_size];
         const int off = key0 % page_size;
         const bf16* kp = k_pages + ((page * nkv + kvh) * page_size + off + col) * D + g * 8;
-        vbase[h] = (page * nkv + kvh) * (int64_t)D * page_size + off;
+        const bf16* vp = v_pages + (page * nkv + kvh) * (int64_t)D * page_size + off + (int64_t)col * page_size + g * 4;
 #pragma unroll
-        for (int c = 0; c < DS; ++c)
-          s[h] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(*(const bf16x8*)(kp + c * 32), qf[c], s[h], 0, 0, 0);
+        for (int c = 0; c < DS; ++c) kf[h][c] = *(const bf16x8*)(kp + c * 32);
+#pragma unroll
+        for (int b = 0; b < DB; ++b) vf[h][b] = *(const bf16x4*)(vp + (int64_t)b * 16 * page_size);
+      } else {
+#pragma unroll
+        for (int c = 0; c < DS; ++c) kf[h][c] = zero8;
+#pragma unroll
+        for (int b = 0; b < DB; ++b) vf[h][b] = bf16x4{0, 0, 0, 0};
       }
+    }
+    floatx4 s[2];
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      s[h] = floatx4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int c = 0; c < DS; ++c) s[h] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[h][c], qf[c], s[h], 0, 0, 0);
     }
     float tile_max = -INFINITY;
 #pragma unroll
@@ -182,12 +195,10 @@ __global__ __launch_bounds__(256) void attention_decode_bf16_kernel(
     run_sum = run_sum * alpha + tile_sum;
 #pragma unroll
     for (int b = 0; b < DB; ++b) {
-      bf16x4 v0 = {0, 0, 0, 0}, v1 = {0, 0, 0, 0};
-      if (present[0]) v0 = *(const bf16x4*)(v_pages + vbase[0] + (int64_t)(b * 16 + col) * page_size + g * 4);
-      if (present[1]) v1 = *(const bf16x4*)(v_pages + vbase[1] + (int64_t)(b * 16 + col) * page_size + g * 4);
-      const bf16x8 vf = {v0[0], v0[1], v0[2], v0[3], v1[0], v1[1], v1[2], v1[3]};
+      const bf16x4 v0 = vf[0][b], v1 = vf[1][b];
+      const bf16x8 vv = {v0[0], v0[1], v0[2], v0[3], v1[0], v1[1], v1[2], v1[3]};
       o[b] *= alpha;
-      o[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf, o[b], 0, 0, 0);
+      o[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vv, pf, o[b], 0, 0, 0);
     }
   }
   run_sum += __shfl_xor(run_sum, 16, WAVE);

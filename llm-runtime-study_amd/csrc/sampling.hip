@@ -76,6 +76,98 @@ __global__ __launch_bounds__(1024) void choose_token_kernel(
   }
 }
 
+// The same choice in two passes for large vocabularies: `parts` workgroups per row each reduce a
+// slice to its best (value, index); one workgroup per row then takes the best of those.  The order
+// of preference (larger value, then lower index) makes the result equal to the one-pass kernel's.
+__global__ __launch_bounds__(256) void choose_token_part_kernel(
+    float* __restrict__ part_value, int* __restrict__ part_index, const float* __restrict__ logits,
+    int64_t row_stride, int vocab, int parts, const float* __restrict__ temperature,
+    const uint64_t* __restrict__ seeds, const uint32_t* __restrict__ counters) {
+  __shared__ float best_value[4];
+  __shared__ int best_index[4];
+  const int row = blockIdx.y, part = blockIdx.x, tid = threadIdx.x;
+  const float* src = logits + (int64_t)row * row_stride;
+  const float temp = temperature ? temperature[row] : 0.f;
+  const uint64_t seed = seeds ? seeds[row] : 0;
+  const uint32_t counter = counters ? counters[row] : 0;
+  const int per = (vocab + parts - 1) / parts;
+  const int begin = part * per, end = begin + per < vocab ? begin + per : vocab;
+  float value = -INFINITY;
+  int index = 0x7fffffff;
+  for (int i = begin + tid; i < end; i += 256) {
+    float v = src[i];
+    if (temp > 0.f && v > -INFINITY)
+      v = v / temp - logf(exponential_variate((uint32_t)seed, (uint32_t)(seed >> 32), counter, (uint32_t)i));
+    if (v > value || (v == value && i < index)) {
+      value = v;
+      index = i;
+    }
+  }
+#pragma unroll
+  for (int off = WAVE / 2; off > 0; off >>= 1) {
+    const float ov = __shfl_xor(value, off, WAVE);
+    const int oi = __shfl_xor(index, off, WAVE);
+    if (ov > value || (ov == value && oi < index)) {
+      value = ov;
+      index = oi;
+    }
+  }
+  if (tid % WAVE == 0) {
+    best_value[tid / WAVE] = value;
+    best_index[tid / WAVE] = index;
+  }
+  __syncthreads();
+  if (tid == 0) {
+    for (int i = 1; i < 4; ++i)
+      if (best_value[i] > value || (best_value[i] == value && best_index[i] < index)) {
+        value = best_value[i];
+        index = best_index[i];
+      }
+    part_value[(int64_t)row * parts + part] = value;
+    part_index[(int64_t)row * parts + part] = index;
+  }
+}
+
+__global__ void choose_token_final_kernel(int* __restrict__ out, const float* __restrict__ part_value,
+                                          const int* __restrict__ part_index, int parts) {
+  const int row = blockIdx.x, lane = threadIdx.x;
+  float value = -INFINITY;
+  int index = 0x7fffffff;
+  for (int i = lane; i < parts; i += WAVE) {
+    const float v = part_value[(int64_t)row * parts + i];
+    const int at = part_index[(int64_t)row * parts + i];
+    if (v > value || (v == value && at < index)) {
+      value = v;
+      index = at;
+    }
+  }
+#pragma unroll
+  for (int off = WAVE / 2; off > 0; off >>= 1) {
+    const float ov = __shfl_xor(value, off, WAVE);
+    const int oi = __shfl_xor(index, off, WAVE);
+    if (ov > value || (ov == value && oi < index)) {
+      value = ov;
+      index = oi;
+    }
+  }
+  if (lane == 0) out[row] = index;
+}
+
+// out[r] = chosen token of row r.  temperature == nullptr or temperature[r] == 0: greedy.
+// part_value / part_index [rows, parts] are scratch for the two-pass form (parts > 1).
+LRS_API int lrs_choose_tokens_split(int* out, const float* logits, int64_t row_stride, int rows, int vocab,
+                                    const float* temperature, const uint64_t* seeds, const uint32_t* counters,
+                                    float* part_value, int* part_index, int parts, void* stream) {
+  LRS_REQUIRE(rows > 0 && vocab > 0 && parts > 0, "choose_tokens: rows=%d vocab=%d parts=%d must be positive", rows, vocab, parts);
+  LRS_REQUIRE(row_stride >= vocab, "choose_tokens: row stride below vocab");
+  LRS_REQUIRE(part_value && part_index, "choose_tokens: the two-pass form needs its scratch buffers");
+  choose_token_part_kernel<<<dim3(parts, rows), 256, 0, (hipStream_t)stream>>>(part_value, part_index, logits, row_stride, vocab,
+                                                                               parts, temperature, seeds, counters);
+  if (lrs_check_launch("choose_tokens_part")) return 1;
+  choose_token_final_kernel<<<rows, WAVE, 0, (hipStream_t)stream>>>(out, part_value, part_index, parts);
+  return lrs_check_launch("choose_tokens_final");
+}
+
 // out[r] = chosen token of row r.  temperature == nullptr or temperature[r] == 0: greedy.
 LRS_API int lrs_choose_tokens(int* out, const float* logits, int64_t row_stride, int rows, int vocab,
                               const float* temperature, const uint64_t* seeds,

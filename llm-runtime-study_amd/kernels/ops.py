@@ -48,6 +48,7 @@ _SIGNATURES = {
     "lrs_attention_prefill": (c_int, [c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p,
                                       c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_void_p]),
     "lrs_choose_tokens": (c_int, [c_void_p, c_void_p, c_int64, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p]),
+    "lrs_choose_tokens_split": (c_int, [c_void_p, c_void_p, c_int64, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p]),
     "lrs_filter_logits": (c_int, [c_void_p, c_int64, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p]),
 }
 
@@ -363,6 +364,9 @@ def attention_prefill(out: torch.Tensor, q: torch.Tensor, k_pages: torch.Tensor,
 
 
 # --------------------------------------------------------------- sampling
+_choose_scratch: dict = {}
+
+
 def choose_tokens(out: torch.Tensor, logits: torch.Tensor, temperature=None, seeds=None, counters=None) -> None:
     rows, vocab = logits.shape
     _need(out.dtype == torch.int32 and out.numel() >= rows and out.is_contiguous(), "choose_tokens: out must be int32 [R]")
@@ -371,10 +375,19 @@ def choose_tokens(out: torch.Tensor, logits: torch.Tensor, temperature=None, see
         _need(temperature.dtype == torch.float32 and temperature.numel() >= rows, "choose_tokens: temperature must be float32 [R]")
         _need(seeds is not None and seeds.dtype == torch.int64 and seeds.numel() >= rows, "choose_tokens: seeds must be int64 [R]")
         _need(counters is not None and counters.dtype == torch.int32 and counters.numel() >= rows, "choose_tokens: counters must be int32 [R]")
-    _check(library().lrs_choose_tokens(
-        _dev(out, "out"), _dev(logits, "logits", torch.float32), stride, rows, vocab,
-        None if temperature is None else _dev(temperature, "temperature"), None if temperature is None else _dev(seeds, "seeds"),
-        None if temperature is None else _dev(counters, "counters"), _stream()))
+    args = (None if temperature is None else _dev(temperature, "temperature"), None if temperature is None else _dev(seeds, "seeds"),
+            None if temperature is None else _dev(counters, "counters"))
+    if vocab >= 16384:   # large vocabulary: many workgroups per row, then one to pick among their results
+        parts = -(-vocab // 4096)
+        key = (logits.device, rows, parts)
+        scratch = _choose_scratch.get(key)
+        if scratch is None:
+            scratch = _choose_scratch[key] = (torch.empty(rows * parts, dtype=torch.float32, device=logits.device),
+                                              torch.empty(rows * parts, dtype=torch.int32, device=logits.device))
+        _check(library().lrs_choose_tokens_split(_dev(out, "out"), _dev(logits, "logits", torch.float32), stride, rows, vocab, *args,
+                                                 _dev(scratch[0], "part_value"), _dev(scratch[1], "part_index"), parts, _stream()))
+        return
+    _check(library().lrs_choose_tokens(_dev(out, "out"), _dev(logits, "logits", torch.float32), stride, rows, vocab, *args, _stream()))
 
 
 def filter_logits(logits: torch.Tensor, temperature: torch.Tensor, top_k: torch.Tensor | None, top_p: torch.Tensor | None) -> None:

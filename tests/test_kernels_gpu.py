@@ -413,16 +413,36 @@ def test_attention_finds_a_far_key(ops, dtype):
         torch.testing.assert_close(out.cpu().float()[0, :d], v[far, 0].to(dtype).float(), rtol=2e-2, atol=2e-2)
 
 
-@pytest.mark.parametrize("rows,vocab", [(1, 256), (5, 331), (3, 151936)])
+@pytest.mark.parametrize("rows,vocab", [(1, 256), (5, 331), (3, 151936), (5, 20000)])
 def test_choose_tokens_greedy(ops, rows, vocab):
     g = torch.Generator().manual_seed(8)
     logits = torch.randn(rows, vocab, generator=g)
     logits[0, vocab - 1] = 50.0
     if rows > 1:
         logits[1, 5] = logits[1, 77] = 40.0  # tie: the lowest index wins
+    if rows > 2:
+        logits[2, 100] = logits[2, vocab - 7] = 45.0  # a tie between far-apart slices of the vocabulary
     out = torch.empty(rows, dtype=torch.int32, device="cuda")
     ops.choose_tokens(out, dev(logits))
-    assert out.cpu().tolist() == [int(torch.argmax(r)) if i != 1 else 5 for i, r in enumerate(logits)]
+    want = [vocab - 1, 5, 100] + [int(torch.argmax(logits[i])) for i in range(3, rows)]
+    assert out.cpu().tolist() == want[:rows]
+
+
+def test_choose_tokens_two_pass_equals_one_pass(ops):
+    """Large vocabularies take the two-pass kernels: same choice as the one-pass kernel, sampled rows included."""
+    rows, vocab = 6, 151936
+    g = torch.Generator().manual_seed(18)
+    logits = dev(torch.randn(rows, vocab, generator=g) * 2)
+    temps = dev(torch.tensor([0.0, 0.7, 1.0, 1.5, 0.0, 0.3]))
+    seeds = dev(torch.tensor([1, 2, 3, 4, 5, 6], dtype=torch.int64))
+    counters = dev(torch.tensor([0, 9, 2, 7, 1, 4], dtype=torch.int32))
+    two = torch.empty(rows, dtype=torch.int32, device="cuda")
+    ops.choose_tokens(two, logits, temps, seeds, counters)
+    one = torch.empty(rows, dtype=torch.int32, device="cuda")
+    code = ops.library().lrs_choose_tokens(one.data_ptr(), logits.data_ptr(), vocab, rows, vocab, temps.data_ptr(), seeds.data_ptr(),
+                                           counters.data_ptr(), torch.cuda.current_stream().cuda_stream)
+    assert code == 0 and one.cpu().tolist() == two.cpu().tolist()
+    assert two.cpu()[0] == logits[0].argmax().cpu() and two.cpu()[1] != logits[1].argmax().cpu()
 
 
 def test_choose_tokens_temperature_statistics(ops):
