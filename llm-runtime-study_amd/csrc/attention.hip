@@ -11,6 +11,10 @@
 // was cut into steps.
 #include "common.h"
 
+// 2^x by the hardware instruction alone (arguments here are <= 0 or -inf; results below the
+// smallest normal number may flush to zero, which a softmax weight can afford).
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
 // ---------------------------------------------------------- generic kernel
 // One workgroup per (query token, query head); any head_dim up to 4 * threads.
 template <typename T, int THREADS>
@@ -180,7 +184,7 @@ __global__ __launch_bounds__(256) void attention_decode_bf16_kernel(
     tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 16, WAVE));
     tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32, WAVE));
     const float new_max = fmaxf(run_max, tile_max);
-    const float alpha = exp2f(run_max - new_max);
+    const float alpha = fast_exp2(run_max - new_max);
     run_max = new_max;
     bf16x8 pf;
     float tile_sum = 0.f;
@@ -188,7 +192,7 @@ __global__ __launch_bounds__(256) void attention_decode_bf16_kernel(
     for (int h = 0; h < 2; ++h)
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        const float p = exp2f(s[h][i] - new_max);
+        const float p = fast_exp2(s[h][i] - new_max);
         tile_sum += p;
         pf[h * 4 + i] = (bf16)p;
       }
@@ -221,7 +225,7 @@ __global__ __launch_bounds__(256) void attention_decode_bf16_kernel(
     float acc = 0.f, total = 0.f;
 #pragma unroll
     for (int w = 0; w < WAVES; ++w) {
-      const float weight = top == -INFINITY ? 0.f : exp2f(sm_m[w][h] - top);
+      const float weight = top == -INFINITY ? 0.f : fast_exp2(sm_m[w][h] - top);
       acc += sm_o[w][dim][h] * weight;
       total += sm_l[w][h] * weight;
     }
@@ -249,13 +253,13 @@ __global__ void attention_merge_kernel(bf16* __restrict__ out, int out_stride, c
   float total = 0.f;
   for (int s = 0; s < splits; ++s) {
     const float m = part_ml[(base + s) * 2];
-    if (m > -INFINITY) total += part_ml[(base + s) * 2 + 1] * exp2f(m - top);
+    if (m > -INFINITY) total += part_ml[(base + s) * 2 + 1] * fast_exp2(m - top);
   }
   for (int dim = threadIdx.x; dim < d; dim += blockDim.x) {
     float acc = 0.f;
     for (int s = 0; s < splits; ++s) {
       const float m = part_ml[(base + s) * 2];
-      if (m > -INFINITY) acc += part_o[(base + s) * d + dim] * exp2f(m - top);
+      if (m > -INFINITY) acc += part_o[(base + s) * d + dim] * fast_exp2(m - top);
     }
     out[(int64_t)token * out_stride + (int64_t)head * d + dim] = (bf16)(acc / total);
   }
@@ -301,14 +305,16 @@ LRS_API int lrs_attention_decode(void* out, int out_stride, float* part_o, float
 
 // ------------------------------------------------- bf16 kernel for any step
 // Ragged batch of prompt portions and single tokens.  The step's tokens are cut on the host into
-// blocks of at most 16 consecutive tokens of one request; a workgroup owns one (block, kv head)
-// and each of its waves one query head of the group, so the waves of a workgroup read the same
-// keys and values at about the same time.  The arithmetic is that of the decode kernel with the
-// 16 queries of the block in the tile columns instead of the heads: S[key, query] = K Q^T,
-// online softmax per query column with the causal (and window) mask of that query's position,
+// groups of at most 16*QB consecutive tokens of one request; a workgroup owns one (group, kv head)
+// and each of its waves one query head of the kv group, so the waves of a workgroup read the same
+// keys and values at about the same time.  A wave holds QB blocks of 16 queries: every key and
+// value fragment it loads serves QB matrix products, and the fragments of the next tile are
+// requested before the current tile is worked on.  The arithmetic is that of the decode kernel
+// with 16 queries in the tile columns instead of the heads: S[key, query] = K Q^T, online softmax
+// per query column with the causal (and window) mask of that query's position,
 // O^T[dim, query] += V^T P.  Every query is finished by one wave, so nothing is merged.
-template <int D>
-__global__ void attention_prefill_bf16_kernel(
+template <int D, int QB>
+__global__ __launch_bounds__(256) void attention_prefill_bf16_kernel(
     bf16* __restrict__ out, int out_stride, const bf16* __restrict__ q, int q_stride,
     const bf16* __restrict__ k_pages, const bf16* __restrict__ v_pages,
     const int* __restrict__ block_table, int table_stride, const int* __restrict__ token_request,
@@ -318,119 +324,171 @@ __global__ void attention_prefill_bf16_kernel(
   const int lane = threadIdx.x % WAVE, wave = threadIdx.x / WAVE;
   const int col = lane & 15, g = lane >> 4;
   const int kvh = blockIdx.y, group = nq / nkv;
-  const int head = kvh * group + wave;
   const int token0 = qblock_token0[blockIdx.x], count = qblock_count[blockIdx.x];
-  const bool live = col < count;
-  const int token = token0 + (live ? col : 0);
-  const int pos = positions[token];
-  const int lo = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
-  const int pos_last = positions[token0 + count - 1];        // positions rise inside a block
-  const int pos_first = positions[token0];
+  const int blocks = (count + 15) / 16;                       // query blocks in use, 1..QB
+  const int pos_first = positions[token0], pos_last = positions[token0 + count - 1];
   const int lo_first = (window > 0 && pos_first - window + 1 > 0) ? pos_first - window + 1 : 0;
   const int* table = block_table + (int64_t)token_request[token0] * table_stride;
-
   const bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
-  bf16x8 qf[DS];
-#pragma unroll
-  for (int c = 0; c < DS; ++c)
-    qf[c] = live ? *(const bf16x8*)(q + (int64_t)token * q_stride + (int64_t)head * D + c * 32 + g * 8) : zero8;
-  floatx4 o[DB];
-#pragma unroll
-  for (int b = 0; b < DB; ++b) o[b] = floatx4{0.f, 0.f, 0.f, 0.f};
-  float run_max = -INFINITY, run_sum = 0.f;
   const float scale2 = scale * 1.4426950408889634f;
 
-  for (int tile = lo_first / 32; tile <= pos_last / 32; ++tile) {
-    floatx4 s[2];
-    int64_t vbase[2];
-    bool present[2];
+  // a workgroup has at most four waves; kv groups of more than four heads take several turns
+  for (int head = kvh * group + wave; head < (kvh + 1) * group; head += blockDim.x / WAVE) {
+    bf16x8 qf[QB][DS];
+    floatx4 o[QB][DB];
+    float run_max[QB], run_sum[QB];
+    int pos[QB], lo[QB], block_last[QB];
+    bool live[QB];
 #pragma unroll
-    for (int h = 0; h < 2; ++h) {
-      const int key0 = tile * 32 + h * 16;
-      present[h] = key0 <= pos_last && key0 + 15 >= lo_first;
-      s[h] = floatx4{0.f, 0.f, 0.f, 0.f};
-      vbase[h] = 0;
-      if (present[h]) {
-        const int64_t page = table[key0 / page_size];
-        const int off = key0 % page_size;
-        const bf16* kp = k_pages + ((page * nkv + kvh) * page_size + off + col) * D + g * 8;
-        vbase[h] = (page * nkv + kvh) * (int64_t)D * page_size + off;
+    for (int b = 0; b < QB; ++b) {
+      block_last[b] = b < blocks ? positions[token0 + (b * 16 + 15 < count ? b * 16 + 15 : count - 1)] : -1;
+      live[b] = b * 16 + col < count;
+      const int token = token0 + (live[b] ? b * 16 + col : 0);
+      pos[b] = live[b] ? positions[token] : -1;                // a dead column sees no key
+      lo[b] = (window > 0 && pos[b] - window + 1 > 0) ? pos[b] - window + 1 : 0;
+      run_max[b] = -INFINITY;
+      run_sum[b] = 0.f;
 #pragma unroll
-        for (int c = 0; c < DS; ++c)
-          s[h] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(*(const bf16x8*)(kp + c * 32), qf[c], s[h], 0, 0, 0);
+      for (int c = 0; c < DS; ++c)
+        qf[b][c] = live[b] ? *(const bf16x8*)(q + (int64_t)token * q_stride + (int64_t)head * D + c * 32 + g * 8) : zero8;
+#pragma unroll
+      for (int e = 0; e < DB; ++e) o[b][e] = floatx4{0.f, 0.f, 0.f, 0.f};
+    }
+
+    bf16x8 ka[2][DS], kb[2][DS];
+    bf16x4 va[2][DB], vb[2][DB];
+    bool pa[2], pb[2];
+    auto fetch = [&](int tile, bf16x8 (&kd)[2][DS], bf16x4 (&vd)[2][DB], bool (&pd)[2]) {
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        const int key0 = tile * 32 + h * 16;
+        pd[h] = key0 <= pos_last && key0 + 15 >= lo_first;
+        if (pd[h]) {
+          const int64_t page = table[key0 / page_size];
+          const int off = key0 % page_size;
+          const bf16* kp = k_pages + ((page * nkv + kvh) * page_size + off + col) * D + g * 8;
+          const bf16* vp = v_pages + (page * nkv + kvh) * (int64_t)D * page_size + off + (int64_t)col * page_size + g * 4;
+#pragma unroll
+          for (int c = 0; c < DS; ++c) kd[h][c] = *(const bf16x8*)(kp + c * 32);
+#pragma unroll
+          for (int e = 0; e < DB; ++e) vd[h][e] = *(const bf16x4*)(vp + (int64_t)e * 16 * page_size);
+        } else {
+#pragma unroll
+          for (int c = 0; c < DS; ++c) kd[h][c] = zero8;
+#pragma unroll
+          for (int e = 0; e < DB; ++e) vd[h][e] = bf16x4{0, 0, 0, 0};
+        }
+      }
+    };
+    auto work = [&](int tile, const bf16x8 (&kf)[2][DS], const bf16x4 (&vf)[2][DB], const bool (&present)[2]) {
+#pragma unroll
+      for (int b = 0; b < QB; ++b) {
+        // blocks are in rising position order: block b needs no tile past its own last query
+        if (b >= blocks || tile * 32 > block_last[b]) continue;
+        floatx4 s[2];
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+          s[h] = floatx4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+          for (int c = 0; c < DS; ++c) s[h] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[h][c], qf[b][c], s[h], 0, 0, 0);
+        }
+        float tile_max = -INFINITY;
+#pragma unroll
+        for (int h = 0; h < 2; ++h)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            const int key = tile * 32 + h * 16 + g * 4 + i;
+            const bool valid = present[h] && key <= pos[b] && key >= lo[b];
+            s[h][i] = valid ? s[h][i] * scale2 : -INFINITY;
+            tile_max = fmaxf(tile_max, s[h][i]);
+          }
+        tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 16, WAVE));
+        tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32, WAVE));
+        const float new_max = fmaxf(run_max[b], tile_max);
+        // a query whose window or position leaves it no key in this tile keeps its state
+        const float alpha = new_max == -INFINITY ? 1.f : fast_exp2(run_max[b] - new_max);
+        const float shift = new_max == -INFINITY ? 0.f : new_max;
+        run_max[b] = new_max;
+        bf16x8 pf;
+        float tile_sum = 0.f;
+#pragma unroll
+        for (int h = 0; h < 2; ++h)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            const float p = fast_exp2(s[h][i] - shift);
+            tile_sum += p;
+            pf[h * 4 + i] = (bf16)p;
+          }
+        run_sum[b] = run_sum[b] * alpha + tile_sum;
+        // once the running maxima have settled no column needs rescaling: skip the multiplies
+        const bool rescale = __any(alpha != 1.f);
+#pragma unroll
+        for (int e = 0; e < DB; ++e) {
+          const bf16x4 v0 = vf[0][e], v1 = vf[1][e];
+          const bf16x8 vv = {v0[0], v0[1], v0[2], v0[3], v1[0], v1[1], v1[2], v1[3]};
+          if (rescale) o[b][e] *= alpha;
+          o[b][e] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vv, pf, o[b][e], 0, 0, 0);
+        }
+      }
+    };
+
+    // two register sets take turns: while one tile is worked on, the next one is on its way
+    const int first_tile = lo_first / 32, last_tile = pos_last / 32;
+    fetch(first_tile, ka, va, pa);
+    for (int tile = first_tile; tile <= last_tile; tile += 2) {
+      if (tile + 1 <= last_tile) fetch(tile + 1, kb, vb, pb);
+      work(tile, ka, va, pa);
+      if (tile + 1 <= last_tile) {
+        if (tile + 2 <= last_tile) fetch(tile + 2, ka, va, pa);
+        work(tile + 1, kb, vb, pb);
       }
     }
-    float tile_max = -INFINITY;
 #pragma unroll
-    for (int h = 0; h < 2; ++h)
+    for (int b = 0; b < QB; ++b) {
+      float total = run_sum[b];
+      total += __shfl_xor(total, 16, WAVE);
+      total += __shfl_xor(total, 32, WAVE);
+      if (live[b]) {
+        const float inv = 1.0f / total;
+        bf16* dst = out + (int64_t)(token0 + b * 16 + col) * out_stride + (int64_t)head * D + g * 4;
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const int key = tile * 32 + h * 16 + g * 4 + i;
-        const bool valid = present[h] && key <= pos && key >= lo;
-        s[h][i] = valid ? s[h][i] * scale2 : -INFINITY;
-        tile_max = fmaxf(tile_max, s[h][i]);
+        for (int e = 0; e < DB; ++e) {
+          const bf16x4 packed = {(bf16)(o[b][e][0] * inv), (bf16)(o[b][e][1] * inv), (bf16)(o[b][e][2] * inv), (bf16)(o[b][e][3] * inv)};
+          *(bf16x4*)(dst + e * 16) = packed;
+        }
       }
-    tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 16, WAVE));
-    tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32, WAVE));
-    const float new_max = fmaxf(run_max, tile_max);
-    // a query whose window or position leaves it no key in this tile keeps its state
-    const float alpha = new_max == -INFINITY ? 1.f : exp2f(run_max - new_max);
-    const float shift = new_max == -INFINITY ? 0.f : new_max;
-    run_max = new_max;
-    bf16x8 pf;
-    float tile_sum = 0.f;
-#pragma unroll
-    for (int h = 0; h < 2; ++h)
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const float p = exp2f(s[h][i] - shift);
-        tile_sum += p;
-        pf[h * 4 + i] = (bf16)p;
-      }
-    run_sum = run_sum * alpha + tile_sum;
-#pragma unroll
-    for (int b = 0; b < DB; ++b) {
-      bf16x4 v0 = {0, 0, 0, 0}, v1 = {0, 0, 0, 0};
-      if (present[0]) v0 = *(const bf16x4*)(v_pages + vbase[0] + (int64_t)(b * 16 + col) * page_size + g * 4);
-      if (present[1]) v1 = *(const bf16x4*)(v_pages + vbase[1] + (int64_t)(b * 16 + col) * page_size + g * 4);
-      const bf16x8 vf = {v0[0], v0[1], v0[2], v0[3], v1[0], v1[1], v1[2], v1[3]};
-      o[b] *= alpha;
-      o[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf, o[b], 0, 0, 0);
-    }
-  }
-  run_sum += __shfl_xor(run_sum, 16, WAVE);
-  run_sum += __shfl_xor(run_sum, 32, WAVE);
-  if (live) {
-    const float inv = 1.0f / run_sum;
-    bf16* dst = out + (int64_t)token * out_stride + (int64_t)head * D + g * 4;
-#pragma unroll
-    for (int b = 0; b < DB; ++b) {
-      const bf16x4 packed = {(bf16)(o[b][0] * inv), (bf16)(o[b][1] * inv), (bf16)(o[b][2] * inv), (bf16)(o[b][3] * inv)};
-      *(bf16x4*)(dst + b * 16) = packed;
     }
   }
 }
 
+// Largest number of tokens in one query group of lrs_attention_prefill.
+LRS_API int lrs_attention_prefill_group() { return 64; }
+
 // Any step in bf16.  qblock_token0 / qblock_count [n_blocks]: first token and number of tokens
-// (1..16) of each block of consecutive tokens of one request.
+// (1..lrs_attention_prefill_group()) of each group of consecutive tokens of one request.
 LRS_API int lrs_attention_prefill(void* out, int out_stride, const void* q, int q_stride, const void* k_pages,
                                   const void* v_pages, const int* block_table, int table_stride,
                                   const int* token_request, const int* positions, const int* qblock_token0,
-                                  const int* qblock_count, int n_blocks, int nq, int nkv, int d, int page_size,
-                                  float scale, int window, void* stream) {
+                                  const int* qblock_count, int n_blocks, int max_count, int nq, int nkv, int d,
+                                  int page_size, float scale, int window, void* stream) {
   LRS_REQUIRE(n_blocks > 0 && nq > 0 && nkv > 0 && nq % nkv == 0, "attention_prefill: bad sizes blocks=%d nq=%d nkv=%d", n_blocks, nq, nkv);
-  LRS_REQUIRE(nq / nkv <= 16, "attention_prefill: %d query heads per kv head, at most 16 waves fit a workgroup", nq / nkv);
+  LRS_REQUIRE(max_count >= 1 && max_count <= 64, "attention_prefill: query groups hold 1..64 tokens, got %d", max_count);
   LRS_REQUIRE(page_size % 16 == 0, "attention_prefill: page size %d is not a multiple of 16", page_size);
   LRS_REQUIRE(window >= 0, "attention_prefill: window must be >= 0 (0 = none)");
   LRS_REQUIRE(q_stride % 8 == 0 && ((uintptr_t)q % 16) == 0 && out_stride % 4 == 0 && ((uintptr_t)out % 8) == 0,
               "attention_prefill: q rows must be 16-byte and out rows 8-byte aligned");
-  dim3 grid(n_blocks, nkv), block((nq / nkv) * WAVE);
+  const int heads = nq / nkv;
+  dim3 grid(n_blocks, nkv), block((heads < 4 ? heads : 4) * WAVE);
   hipStream_t s = (hipStream_t)stream;
-#define LAUNCH(D)                                                                                                    \
-  attention_prefill_bf16_kernel<D><<<grid, block, 0, s>>>((bf16*)out, out_stride, (const bf16*)q, q_stride,          \
-                                                          (const bf16*)k_pages, (const bf16*)v_pages, block_table,   \
-                                                          table_stride, token_request, positions, qblock_token0,     \
-                                                          qblock_count, nq, nkv, page_size, scale, window)
+#define LAUNCH2(D, QB)                                                                                               \
+  attention_prefill_bf16_kernel<D, QB><<<grid, block, 0, s>>>((bf16*)out, out_stride, (const bf16*)q, q_stride,      \
+                                                              (const bf16*)k_pages, (const bf16*)v_pages, block_table, \
+                                                              table_stride, token_request, positions, qblock_token0, \
+                                                              qblock_count, nq, nkv, page_size, scale, window)
+#define LAUNCH(D)                                \
+  if (max_count <= 16) LAUNCH2(D, 1);            \
+  else if (max_count <= 32) LAUNCH2(D, 2);       \
+  else LAUNCH2(D, 4)
   switch (d) {
     case 32: LAUNCH(32); break;
     case 64: LAUNCH(64); break;
@@ -440,6 +498,7 @@ LRS_API int lrs_attention_prefill(void* out, int out_stride, const void* q, int 
     default: return lrs_fail("attention_prefill: head_dim %d has no matrix-core kernel (32, 64, 96, 128, 192)", d);
   }
 #undef LAUNCH
+#undef LAUNCH2
   return lrs_check_launch("attention_prefill");
 }
 

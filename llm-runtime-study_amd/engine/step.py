@@ -84,7 +84,7 @@ class StepContext:
         self.dtype = runner.dtype
         self.device = runner.device
         self.memo: dict = {}
-        self.T = self.R = self.num_logit_rows = self.num_qblocks = 0
+        self.T = self.R = self.num_logit_rows = self.num_qblocks = self.max_qblock = 0
         self.qblock_token0 = self.qblock_count = None
         self.max_q = self.max_k = 0
         self.all_decode = False
@@ -124,6 +124,8 @@ class ModelRunner:
         # layout of the metadata buffer (int32 elements)
         self._off = {}
         cursor = 0
+        # query groups for the ragged attention kernel: at most `query_group` consecutive tokens of one request
+        self.query_group = 64
         self._max_qblocks = -(-t // 16) + r
         for name, size in (("token_ids", t), ("positions", t), ("token_request", t), ("logit_rows", t),
                            ("cu_seqlens_q", r + 1), ("seq_lens_k", r), ("slot_ids", r),
@@ -241,12 +243,13 @@ class ModelRunner:
             rows[:cursor] = np.arange(cursor, dtype=np.int32)
             n_rows = cursor
         ctx.T, ctx.R, ctx.num_logit_rows = cursor, max(real, pad_to), n_rows
-        # blocks of at most 16 consecutive tokens of one request, the longest contexts first
-        starts = cu[:ctx.R + 1]
-        blocks = [(int(pos[min(t0 + 16, int(starts[i + 1])) - 1]), t0, min(16, int(starts[i + 1]) - t0))
-                  for i in range(ctx.R) for t0 in range(int(starts[i]), int(starts[i + 1]), 16)]
+        # groups of consecutive tokens of one request, the longest contexts first
+        starts, size = cu[:ctx.R + 1], self.query_group
+        blocks = [(int(pos[min(t0 + size, int(starts[i + 1])) - 1]), t0, min(size, int(starts[i + 1]) - t0))
+                  for i in range(ctx.R) for t0 in range(int(starts[i]), int(starts[i + 1]), size)]
         blocks.sort(key=lambda b: -b[0])
         ctx.num_qblocks = len(blocks)
+        ctx.max_qblock = max(b[2] for b in blocks)
         self._host_view("qblock_token0")[:len(blocks)] = [b[1] for b in blocks]
         self._host_view("qblock_count")[:len(blocks)] = [b[2] for b in blocks]
         mb = cache.max_blocks

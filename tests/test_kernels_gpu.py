@@ -288,7 +288,7 @@ def _attention_reference(q, k_all, v_all, positions, lengths_before, nq, nkv, d,
 def test_attention_ragged_batch(ops, dtype, nq, nkv, d, page, window):
     g = torch.Generator().manual_seed(6)
     # request: (cached length before the step, new tokens in the step)
-    requests = [(0, 19), (37, 1), (150, 1), (5, 6), (page * 3 - 1, 2)]
+    requests = [(0, 19), (37, 1), (150, 1), (5, 6), (page * 3 - 1, 2), (9, 75)]
     scale = 1 / math.sqrt(d)
     max_blocks = max((a + b + page - 1) // page for a, b in requests)
     n_pages = sum((a + b + page - 1) // page for a, b in requests) + 3
@@ -326,18 +326,20 @@ def test_attention_ragged_batch(ops, dtype, nq, nkv, d, page, window):
                   nq, scale, window)
     torch.testing.assert_close(out.cpu().double(), want, **tol(dtype, 2e-5, 2e-2))
     if ops.attention_decode_supported(dtype, nq, nkv, d, page):
-        # the matrix-core kernel for ragged steps: blocks of at most 16 tokens of one request, in any order
-        blocks, at = [], 0
-        for before, new in requests:
-            blocks += [(at + i, min(16, new - i)) for i in range(0, new, 16)]
-            at += new
-        blocks = blocks[::-1]
-        fast = torch.empty_like(out)
-        ops.attention_prefill(fast, dev(q_wide), dev(kp.to(dtype)), dev(vp.to(dtype)), dev(table),
-                              dev(torch.tensor(tok_req, dtype=torch.int32)), dev(torch.tensor(tok_pos, dtype=torch.int32)),
-                              dev(torch.tensor([b[0] for b in blocks], dtype=torch.int32)),
-                              dev(torch.tensor([b[1] for b in blocks], dtype=torch.int32)), nq, scale, window)
-        torch.testing.assert_close(fast.cpu().double(), want, rtol=2e-2, atol=2e-2)
+        # the matrix-core kernel for ragged steps: groups of consecutive tokens of one request, in any order
+        assert ops.attention_prefill_group() == 64
+        for size in (16, 7, 32, 64):
+            blocks, at = [], 0
+            for before, new in requests:
+                blocks += [(at + i, min(size, new - i)) for i in range(0, new, size)]
+                at += new
+            blocks = blocks[::-1]
+            fast = torch.empty_like(out)
+            ops.attention_prefill(fast, dev(q_wide), dev(kp.to(dtype)), dev(vp.to(dtype)), dev(table),
+                                  dev(torch.tensor(tok_req, dtype=torch.int32)), dev(torch.tensor(tok_pos, dtype=torch.int32)),
+                                  dev(torch.tensor([b[0] for b in blocks], dtype=torch.int32)),
+                                  dev(torch.tensor([b[1] for b in blocks], dtype=torch.int32)), nq, scale, window, size)
+            torch.testing.assert_close(fast.cpu().double(), want, rtol=2e-2, atol=2e-2)
 
 
 @pytest.mark.parametrize("nq,nkv,d,page,window,splits", [
