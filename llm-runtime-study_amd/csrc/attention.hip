@@ -15,6 +15,10 @@
 // smallest normal number may flush to zero, which a softmax weight can afford).
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
+// How far (in powers of two) a new maximum must exceed the reference point of a running softmax
+// before the reference point moves and the accumulators are rescaled.
+constexpr float RESCALE_STEP = 8.0f;
+
 // ---------------------------------------------------------- generic kernel
 // One workgroup per (query token, query head); any head_dim up to 4 * threads.
 template <typename T, int THREADS>
@@ -183,7 +187,7 @@ __global__ __launch_bounds__(256) void attention_decode_bf16_kernel(
       }
     tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 16, WAVE));
     tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32, WAVE));
-    const float new_max = fmaxf(run_max, tile_max);
+    const float new_max = tile_max > run_max + RESCALE_STEP ? tile_max : run_max;   // see RESCALE_STEP
     const float alpha = fast_exp2(run_max - new_max);
     run_max = new_max;
     bf16x8 pf;
@@ -197,11 +201,12 @@ __global__ __launch_bounds__(256) void attention_decode_bf16_kernel(
         pf[h * 4 + i] = (bf16)p;
       }
     run_sum = run_sum * alpha + tile_sum;
+    const bool rescale = __any(alpha != 1.f);
 #pragma unroll
     for (int b = 0; b < DB; ++b) {
       const bf16x4 v0 = vf[0][b], v1 = vf[1][b];
       const bf16x8 vv = {v0[0], v0[1], v0[2], v0[3], v1[0], v1[1], v1[2], v1[3]};
-      o[b] *= alpha;
+      if (rescale) o[b] *= alpha;
       o[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vv, pf, o[b], 0, 0, 0);
     }
   }
@@ -306,12 +311,13 @@ LRS_API int lrs_attention_decode(void* out, int out_stride, float* part_o, float
 // ------------------------------------------------- bf16 kernel for any step
 // Ragged batch of prompt portions and single tokens.  The step's tokens are cut on the host into
 // groups of at most 16*QB consecutive tokens of one request; a workgroup owns one (group, kv head)
-// and each of its waves one query head of the kv group, so the waves of a workgroup read the same
-// keys and values at about the same time.  A wave holds QB blocks of 16 queries: every key and
-// value fragment it loads serves QB matrix products, and the fragments of the next tile are
-// requested before the current tile is worked on.  The arithmetic is that of the decode kernel
-// with 16 queries in the tile columns instead of the heads: S[key, query] = K Q^T, online softmax
-// per query column with the causal (and window) mask of that query's position,
+// and each of its (up to four) waves one query head of the kv group.  Keys are walked in tiles of
+// 32: the workgroup brings a tile's keys and (transposed) values into LDS once, all waves take
+// their matrix-core operands from there, and the next tile is on its way from memory while the
+// current one is worked on (two LDS buffers, one barrier a tile).  A wave holds QB blocks of 16
+// queries, so every fragment it reads serves QB products.  The arithmetic is that of the decode
+// kernel with 16 queries in the tile columns instead of the heads: S[key, query] = K Q^T, online
+// softmax per query column with the causal (and window) mask of that query's position,
 // O^T[dim, query] += V^T P.  Every query is finished by one wave, so nothing is merged.
 template <int D, int QB>
 __global__ __launch_bounds__(256) void attention_prefill_bf16_kernel(
@@ -321,28 +327,82 @@ __global__ __launch_bounds__(256) void attention_prefill_bf16_kernel(
     const int* __restrict__ positions, const int* __restrict__ qblock_token0,
     const int* __restrict__ qblock_count, int nq, int nkv, int page_size, float scale, int window) {
   constexpr int DS = D / 32, DB = D / 16;
-  const int lane = threadIdx.x % WAVE, wave = threadIdx.x / WAVE;
+  constexpr int KLD = D + 8, VLD = 32 + 8;                    // padded LDS rows
+  constexpr int KCHUNKS = 32 * D / 8, VCHUNKS = D * 4;        // 16-byte pieces of one tile
+  constexpr int KPT = (KCHUNKS + 255) / 256, VPT = (VCHUNKS + 255) / 256;
+  __shared__ __attribute__((aligned(16))) bf16 ks[2][32 * KLD];
+  __shared__ __attribute__((aligned(16))) bf16 vs[2][D * VLD];
+  const int tid = threadIdx.x, threads = blockDim.x;
+  const int lane = tid % WAVE, wave = tid / WAVE, waves = threads / WAVE;
   const int col = lane & 15, g = lane >> 4;
   const int kvh = blockIdx.y, group = nq / nkv;
   const int token0 = qblock_token0[blockIdx.x], count = qblock_count[blockIdx.x];
-  const int blocks = (count + 15) / 16;                       // query blocks in use, 1..QB
   const int pos_first = positions[token0], pos_last = positions[token0 + count - 1];
   const int lo_first = (window > 0 && pos_first - window + 1 > 0) ? pos_first - window + 1 : 0;
   const int* table = block_table + (int64_t)token_request[token0] * table_stride;
   const bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
   const float scale2 = scale * 1.4426950408889634f;
+  const int first_tile = lo_first / 32, last_tile = pos_last / 32;
+  // the part of the request's block table that the tiles need, in LDS: the address of a key must
+  // not wait for a trip to memory of its own
+  extern __shared__ int page_ids[];
+  const int first_block = first_tile * 32 / page_size;
+  for (int i = tid; i <= pos_last / page_size - first_block; i += threads) page_ids[i] = table[first_block + i];
+  __syncthreads();
 
-  // a workgroup has at most four waves; kv groups of more than four heads take several turns
-  for (int head = kvh * group + wave; head < (kvh + 1) * group; head += blockDim.x / WAVE) {
+  // pieces of a tile this thread brings in: keys [32, D] and transposed values [D, 32]
+  // two register sets in turn: a tile is asked for two tiles ahead of its use
+  bf16x8 kreg_a[KPT], vreg_a[VPT], kreg_b[KPT], vreg_b[VPT];
+  auto fetch = [&](int tile, bf16x8 (&kreg)[KPT], bf16x8 (&vreg)[VPT]) {
+    int64_t kbase[2], vbase[2];
+    bool present[2];
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      const int key0 = tile * 32 + h * 16;
+      present[h] = key0 <= pos_last && key0 + 15 >= lo_first;
+      const int64_t page = present[h] ? page_ids[key0 / page_size - first_block] : 0;
+      const int off = key0 % page_size;
+      kbase[h] = ((page * nkv + kvh) * page_size + off) * D;
+      vbase[h] = (page * nkv + kvh) * (int64_t)D * page_size + off;
+    }
+#pragma unroll
+    for (int i = 0; i < KPT; ++i) {
+      const int idx = tid + i * threads;
+      const int key = idx / (D / 8), piece = idx % (D / 8);
+      kreg[i] = (idx < KCHUNKS && present[key / 16]) ? *(const bf16x8*)(k_pages + kbase[key / 16] + (key % 16) * D + piece * 8) : zero8;
+    }
+#pragma unroll
+    for (int i = 0; i < VPT; ++i) {
+      const int idx = tid + i * threads;
+      const int dim = idx / 4, part = idx % 4;
+      vreg[i] = (idx < VCHUNKS && present[part / 2]) ? *(const bf16x8*)(v_pages + vbase[part / 2] + (int64_t)dim * page_size + (part % 2) * 8) : zero8;
+    }
+  };
+  auto stash = [&](int buffer, const bf16x8 (&kreg)[KPT], const bf16x8 (&vreg)[VPT]) {
+#pragma unroll
+    for (int i = 0; i < KPT; ++i) {
+      const int idx = tid + i * threads;
+      if (idx < KCHUNKS) *(bf16x8*)(ks[buffer] + (idx / (D / 8)) * KLD + (idx % (D / 8)) * 8) = kreg[i];
+    }
+#pragma unroll
+    for (int i = 0; i < VPT; ++i) {
+      const int idx = tid + i * threads;
+      if (idx < VCHUNKS) *(bf16x8*)(vs[buffer] + (idx / 4) * VLD + (idx % 4) * 8) = vreg[i];
+    }
+  };
+
+  // kv groups of more than four heads take several passes over the keys
+  for (int head0 = kvh * group; head0 < (kvh + 1) * group; head0 += waves) {
+    const int head = head0 + wave;
+    const bool active = head < (kvh + 1) * group;
     bf16x8 qf[QB][DS];
     floatx4 o[QB][DB];
     float run_max[QB], run_sum[QB];
-    int pos[QB], lo[QB], block_last[QB];
+    int pos[QB], lo[QB];
     bool live[QB];
 #pragma unroll
     for (int b = 0; b < QB; ++b) {
-      block_last[b] = b < blocks ? positions[token0 + (b * 16 + 15 < count ? b * 16 + 15 : count - 1)] : -1;
-      live[b] = b * 16 + col < count;
+      live[b] = active && b * 16 + col < count;
       const int token = token0 + (live[b] ? b * 16 + col : 0);
       pos[b] = live[b] ? positions[token] : -1;                // a dead column sees no key
       lo[b] = (window > 0 && pos[b] - window + 1 > 0) ? pos[b] - window + 1 : 0;
@@ -355,93 +415,91 @@ __global__ __launch_bounds__(256) void attention_prefill_bf16_kernel(
       for (int e = 0; e < DB; ++e) o[b][e] = floatx4{0.f, 0.f, 0.f, 0.f};
     }
 
-    bf16x8 ka[2][DS], kb[2][DS];
-    bf16x4 va[2][DB], vb[2][DB];
-    bool pa[2], pb[2];
-    auto fetch = [&](int tile, bf16x8 (&kd)[2][DS], bf16x4 (&vd)[2][DB], bool (&pd)[2]) {
+    auto work = [&](int tile, int buffer) {
+      const bf16* kt = ks[buffer];
+      const bf16* vt = vs[buffer];
+      // Three phases over all query blocks at once, without branches: blocks past the diagonal or
+      // without queries are masked like any other key a query may not see and add nothing.
+      floatx4 sc[QB][2];
 #pragma unroll
-      for (int h = 0; h < 2; ++h) {
-        const int key0 = tile * 32 + h * 16;
-        pd[h] = key0 <= pos_last && key0 + 15 >= lo_first;
-        if (pd[h]) {
-          const int64_t page = table[key0 / page_size];
-          const int off = key0 % page_size;
-          const bf16* kp = k_pages + ((page * nkv + kvh) * page_size + off + col) * D + g * 8;
-          const bf16* vp = v_pages + (page * nkv + kvh) * (int64_t)D * page_size + off + (int64_t)col * page_size + g * 4;
+      for (int b = 0; b < QB; ++b) sc[b][0] = sc[b][1] = floatx4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-          for (int c = 0; c < DS; ++c) kd[h][c] = *(const bf16x8*)(kp + c * 32);
+      for (int h = 0; h < 2; ++h)
 #pragma unroll
-          for (int e = 0; e < DB; ++e) vd[h][e] = *(const bf16x4*)(vp + (int64_t)e * 16 * page_size);
-        } else {
+        for (int c = 0; c < DS; ++c) {
+          const bf16x8 kfrag = *(const bf16x8*)(kt + (h * 16 + col) * KLD + c * 32 + g * 8);
 #pragma unroll
-          for (int c = 0; c < DS; ++c) kd[h][c] = zero8;
-#pragma unroll
-          for (int e = 0; e < DB; ++e) vd[h][e] = bf16x4{0, 0, 0, 0};
+          for (int b = 0; b < QB; ++b) sc[b][h] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kfrag, qf[b][c], sc[b][h], 0, 0, 0);
         }
-      }
-    };
-    auto work = [&](int tile, const bf16x8 (&kf)[2][DS], const bf16x4 (&vf)[2][DB], const bool (&present)[2]) {
+      bf16x8 pf[QB];
+      float alpha[QB];
+      bool rescale = false;
 #pragma unroll
       for (int b = 0; b < QB; ++b) {
-        // blocks are in rising position order: block b needs no tile past its own last query
-        if (b >= blocks || tile * 32 > block_last[b]) continue;
-        floatx4 s[2];
-#pragma unroll
-        for (int h = 0; h < 2; ++h) {
-          s[h] = floatx4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-          for (int c = 0; c < DS; ++c) s[h] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[h][c], qf[b][c], s[h], 0, 0, 0);
-        }
         float tile_max = -INFINITY;
 #pragma unroll
         for (int h = 0; h < 2; ++h)
 #pragma unroll
           for (int i = 0; i < 4; ++i) {
             const int key = tile * 32 + h * 16 + g * 4 + i;
-            const bool valid = present[h] && key <= pos[b] && key >= lo[b];
-            s[h][i] = valid ? s[h][i] * scale2 : -INFINITY;
-            tile_max = fmaxf(tile_max, s[h][i]);
+            const bool valid = key <= pos[b] && key >= lo[b];
+            sc[b][h][i] = valid ? sc[b][h][i] * scale2 : -INFINITY;
+            tile_max = fmaxf(tile_max, sc[b][h][i]);
           }
         tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 16, WAVE));
         tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32, WAVE));
-        const float new_max = fmaxf(run_max[b], tile_max);
+        // The reference point of the exponentials follows the maximum only when that has grown by
+        // more than 2^8: weights then stay below 256, well inside float32 and bfloat16, and the
+        // accumulators need rescaling a few times per sequence instead of at nearly every tile.
+        const float new_max = tile_max > run_max[b] + RESCALE_STEP ? tile_max : run_max[b];
         // a query whose window or position leaves it no key in this tile keeps its state
-        const float alpha = new_max == -INFINITY ? 1.f : fast_exp2(run_max[b] - new_max);
+        alpha[b] = new_max == -INFINITY ? 1.f : fast_exp2(run_max[b] - new_max);
         const float shift = new_max == -INFINITY ? 0.f : new_max;
         run_max[b] = new_max;
-        bf16x8 pf;
         float tile_sum = 0.f;
 #pragma unroll
         for (int h = 0; h < 2; ++h)
 #pragma unroll
           for (int i = 0; i < 4; ++i) {
-            const float p = fast_exp2(s[h][i] - shift);
+            const float p = fast_exp2(sc[b][h][i] - shift);
             tile_sum += p;
-            pf[h * 4 + i] = (bf16)p;
+            pf[b][h * 4 + i] = (bf16)p;
           }
-        run_sum[b] = run_sum[b] * alpha + tile_sum;
-        // once the running maxima have settled no column needs rescaling: skip the multiplies
-        const bool rescale = __any(alpha != 1.f);
+        run_sum[b] = run_sum[b] * alpha[b] + tile_sum;
+        rescale |= alpha[b] != 1.f;
+      }
+      // once the running maxima have settled no column needs rescaling: skip the multiplies
+      if (__any(rescale)) {
 #pragma unroll
-        for (int e = 0; e < DB; ++e) {
-          const bf16x4 v0 = vf[0][e], v1 = vf[1][e];
-          const bf16x8 vv = {v0[0], v0[1], v0[2], v0[3], v1[0], v1[1], v1[2], v1[3]};
-          if (rescale) o[b][e] *= alpha;
-          o[b][e] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vv, pf, o[b][e], 0, 0, 0);
-        }
+        for (int b = 0; b < QB; ++b)
+#pragma unroll
+          for (int e = 0; e < DB; ++e) o[b][e] *= alpha[b];
+      }
+#pragma unroll
+      for (int e = 0; e < DB; ++e) {
+        const bf16x4 v0 = *(const bf16x4*)(vt + (e * 16 + col) * VLD + g * 4);
+        const bf16x4 v1 = *(const bf16x4*)(vt + (e * 16 + col) * VLD + 16 + g * 4);
+        const bf16x8 vv = {v0[0], v0[1], v0[2], v0[3], v1[0], v1[1], v1[2], v1[3]};
+#pragma unroll
+        for (int b = 0; b < QB; ++b) o[b][e] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vv, pf[b], o[b][e], 0, 0, 0);
       }
     };
-
-    // two register sets take turns: while one tile is worked on, the next one is on its way
-    const int first_tile = lo_first / 32, last_tile = pos_last / 32;
-    fetch(first_tile, ka, va, pa);
-    for (int tile = first_tile; tile <= last_tile; tile += 2) {
-      if (tile + 1 <= last_tile) fetch(tile + 1, kb, vb, pb);
-      work(tile, ka, va, pa);
-      if (tile + 1 <= last_tile) {
-        if (tile + 2 <= last_tile) fetch(tile + 2, ka, va, pa);
-        work(tile + 1, kb, vb, pb);
-      }
+    __syncthreads();                                           // the buffers of an earlier pass are done with
+    fetch(first_tile, kreg_a, vreg_a);
+    if (first_tile < last_tile) fetch(first_tile + 1, kreg_b, vreg_b);
+    stash(0, kreg_a, vreg_a);
+    __syncthreads();
+    // invariant at the top of a turn: tile is in LDS buffer `buffer`, tile + 1 is on its way into set b
+    for (int tile = first_tile, buffer = 0; tile <= last_tile; tile += 2) {
+      if (tile + 2 <= last_tile) fetch(tile + 2, kreg_a, vreg_a);
+      work(tile, buffer);
+      if (tile + 1 <= last_tile) stash(buffer ^ 1, kreg_b, vreg_b);
+      __syncthreads();
+      if (tile + 1 > last_tile) break;
+      if (tile + 3 <= last_tile) fetch(tile + 3, kreg_b, vreg_b);
+      work(tile + 1, buffer ^ 1);
+      if (tile + 2 <= last_tile) stash(buffer, kreg_a, vreg_a);
+      __syncthreads();
     }
 #pragma unroll
     for (int b = 0; b < QB; ++b) {
@@ -469,19 +527,24 @@ LRS_API int lrs_attention_prefill_group() { return 64; }
 LRS_API int lrs_attention_prefill(void* out, int out_stride, const void* q, int q_stride, const void* k_pages,
                                   const void* v_pages, const int* block_table, int table_stride,
                                   const int* token_request, const int* positions, const int* qblock_token0,
-                                  const int* qblock_count, int n_blocks, int max_count, int nq, int nkv, int d,
-                                  int page_size, float scale, int window, void* stream) {
+                                  const int* qblock_count, int n_blocks, int max_count, int max_context, int nq,
+                                  int nkv, int d, int page_size, float scale, int window, void* stream) {
   LRS_REQUIRE(n_blocks > 0 && nq > 0 && nkv > 0 && nq % nkv == 0, "attention_prefill: bad sizes blocks=%d nq=%d nkv=%d", n_blocks, nq, nkv);
   LRS_REQUIRE(max_count >= 1 && max_count <= 64, "attention_prefill: query groups hold 1..64 tokens, got %d", max_count);
   LRS_REQUIRE(page_size % 16 == 0, "attention_prefill: page size %d is not a multiple of 16", page_size);
   LRS_REQUIRE(window >= 0, "attention_prefill: window must be >= 0 (0 = none)");
   LRS_REQUIRE(q_stride % 8 == 0 && ((uintptr_t)q % 16) == 0 && out_stride % 4 == 0 && ((uintptr_t)out % 8) == 0,
               "attention_prefill: q rows must be 16-byte and out rows 8-byte aligned");
-  const int heads = nq / nkv;
-  dim3 grid(n_blocks, nkv), block((heads < 4 ? heads : 4) * WAVE);
+  // always four waves: with fewer heads in a kv group the spare waves still help to bring tiles in
+  dim3 grid(n_blocks, nkv), block(4 * WAVE);
+  // LDS copy of the block table entries a workgroup walks: at most those of the longest context
+  LRS_REQUIRE(max_context >= 1, "attention_prefill: max_context must be the longest context length of the step");
+  const int span = window > 0 && window + 16 * 4 + 64 < max_context ? window + 16 * 4 + 64 : max_context;
+  const size_t table_lds = sizeof(int) * (size_t)(span / page_size + 2);
+  LRS_REQUIRE(table_lds <= 24 * 1024, "attention_prefill: a context of %d tokens needs more block table entries than fit LDS", max_context);
   hipStream_t s = (hipStream_t)stream;
 #define LAUNCH2(D, QB)                                                                                               \
-  attention_prefill_bf16_kernel<D, QB><<<grid, block, 0, s>>>((bf16*)out, out_stride, (const bf16*)q, q_stride,      \
+  attention_prefill_bf16_kernel<D, QB><<<grid, block, table_lds, s>>>((bf16*)out, out_stride, (const bf16*)q, q_stride, \
                                                               (const bf16*)k_pages, (const bf16*)v_pages, block_table, \
                                                               table_stride, token_request, positions, qblock_token0, \
                                                               qblock_count, nq, nkv, page_size, scale, window)

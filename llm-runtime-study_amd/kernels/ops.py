@@ -46,7 +46,7 @@ _SIGNATURES = {
     "lrs_attention_decode": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p,
                                      c_void_p, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_int, c_void_p]),
     "lrs_attention_prefill": (c_int, [c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p,
-                                      c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_void_p]),
+                                      c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_void_p]),
     "lrs_attention_prefill_group": (c_int, []),
     "lrs_choose_tokens": (c_int, [c_void_p, c_void_p, c_int64, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p]),
     "lrs_choose_tokens_split": (c_int, [c_void_p, c_void_p, c_int64, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p]),
@@ -342,10 +342,11 @@ def attention_decode(out: torch.Tensor, q: torch.Tensor, k_pages: torch.Tensor, 
 
 def attention_prefill(out: torch.Tensor, q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, block_table: torch.Tensor,
                       token_request: torch.Tensor, positions: torch.Tensor, qblock_token0: torch.Tensor, qblock_count: torch.Tensor,
-                      nq: int, scale: float, window: int = 0, max_count: int | None = None) -> None:
+                      nq: int, scale: float, window: int = 0, max_count: int | None = None, max_context: int | None = None) -> None:
     """attention() on matrix cores for any bfloat16 step.  qblock_token0 / qblock_count list groups of at
     most attention_prefill_group() consecutive tokens of one request that together cover every token of
-    the step once; `max_count` is the largest count among them (the group limit if not given)."""
+    the step once; `max_count` is the largest count among them (the group limit if not given) and
+    `max_context` the longest context (position + 1) of any token (what the block table can hold if not given)."""
     tokens = out.shape[0]
     _need(k_pages.dim() == 4 and k_pages.is_contiguous() and v_pages.is_contiguous(), "attention_prefill: pages must be contiguous")
     _, nkv, page_size, d = k_pages.shape
@@ -363,7 +364,8 @@ def attention_prefill(out: torch.Tensor, q: torch.Tensor, k_pages: torch.Tensor,
         _dev(out, "out"), _rows(out, "out"), _dev(q, "q"), _rows(q, "q"), _dev(k_pages, "k_pages"), _dev(v_pages, "v_pages"),
         _dev(block_table, "block_table"), block_table.stride(0), _dev(token_request, "token_request"), _dev(positions, "positions"),
         _dev(qblock_token0, "qblock_token0"), _dev(qblock_count, "qblock_count"), n_blocks,
-        attention_prefill_group() if max_count is None else max_count, nq, nkv, d, page_size, scale, window, _stream()))
+        attention_prefill_group() if max_count is None else max_count,
+        block_table.shape[1] * page_size if max_context is None else max_context, nq, nkv, d, page_size, scale, window, _stream()))
 
 
 def attention_prefill_group() -> int:

@@ -113,7 +113,7 @@ class GQAAttention(Part):
                                  nq, self.scale, self.window or 0, splits, part_o, part_ml)
         elif ops.attention_decode_supported(ctx.dtype, nq, kv_heads, d, group.page_size):
             ops.attention_prefill(out, qkv, cache.k_pages, cache.v_pages, group.block_table, ctx.token_request, ctx.positions,
-                                  ctx.qblock_token0, ctx.qblock_count, nq, self.scale, self.window or 0, ctx.max_qblock)
+                                  ctx.qblock_token0, ctx.qblock_count, nq, self.scale, self.window or 0, ctx.max_qblock, ctx.max_k)
         else:
             ops.attention(out, qkv, cache.k_pages, cache.v_pages, group.block_table, ctx.token_request, ctx.positions,
                           nq, self.scale, self.window or 0)
