@@ -181,8 +181,11 @@ __device__ __forceinline__ float silu(float g) { return g / (1.0f + __expf(-g));
 template <int MT, int RT, int WAVES, int UNROLL, bool NORM, bool SWIGLU>
 __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_skinny_kernel(
     void* __restrict__ out, int mode, const bf16* __restrict__ x, NormInput norm,
-    const bf16* __restrict__ w, const bf16* __restrict__ bias, int m, int n, int k, int lda, int ldc) {
-  // RT: row tiles of 16 weight rows per workgroup; every activation fragment is used RT times
+    const bf16* __restrict__ w, const bf16* __restrict__ bias, int m, int n, int k, int lda, int ldc,
+    float* __restrict__ split_sums) {
+  // RT: row tiles of 16 weight rows per workgroup; every activation fragment is used RT times.
+  // gridDim.y > 1: K is also divided between workgroups; each then leaves its sums in
+  // split_sums [gridDim.y, m, n] for gemm_split_finish_kernel instead of writing the output.
   __shared__ floatx4 partial[WAVES][MT][WAVE];
   __shared__ float sumsq[WAVES][MT][16];
   const int tid = threadIdx.x, lane = tid % WAVE, wave = tid / WAVE;
@@ -244,10 +247,13 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_skinny_kernel(
     return b;
   };
 
-  const int steps = (k + 31) / 32;
-  const int per_wave = (steps + WAVES - 1) / WAVES;
-  int s = wave * per_wave;
-  const int s_end = s + per_wave < steps ? s + per_wave : steps;
+  const int all_steps = (k + 31) / 32;
+  const int per_split = (all_steps + gridDim.y - 1) / gridDim.y;
+  const int split_begin = blockIdx.y * per_split;
+  const int split_end = split_begin + per_split < all_steps ? split_begin + per_split : all_steps;
+  const int per_wave = (per_split + WAVES - 1) / WAVES;
+  int s = split_begin + wave * per_wave;
+  const int s_end = s + per_wave < split_end ? s + per_wave : split_end;
   const int full_end = k / 32 < s_end ? k / 32 : s_end;   // steps whose 32 k are all inside K
   for (; s + UNROLL <= full_end; s += UNROLL) {
     bf16x8 a[UNROLL][RT], b[UNROLL][MT];
@@ -308,7 +314,13 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_skinny_kernel(
     for (int t = 0; t < MT; ++t) partial[wave][t][lane] = acc[q][t];
     __syncthreads();
     const int nq0 = n0 + q * 16;
-    if (SWIGLU) {
+    if (gridDim.y > 1) {
+      for (int e = tid; e < MT * WAVE * 4; e += WAVES * WAVE) {
+        const int t = e / (WAVE * 4), l = (e / 4) % WAVE, i = e % 4;
+        const int token = t * 16 + (l & 15), gn = nq0 + 4 * (l >> 4) + i;
+        if (token < m && gn < n) split_sums[((int64_t)blockIdx.y * m + token) * n + gn] = total(t, l, i);
+      }
+    } else if (SWIGLU) {
       for (int e = tid; e < MT * 16 * 8; e += WAVES * WAVE) {
         const int t = e / 128, c = (e / 8) % 16, j = e % 8;
         const int token = t * 16 + c, feature = nq0 / 2 + j;
@@ -329,23 +341,71 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_skinny_kernel(
   }
 }
 
+// Adds up what the K splits left in split_sums [splits, m, n], in split order, and writes the output
+// with the same epilogues as the product kernels.
+template <bool SWIGLU>
+__global__ void gemm_split_finish_kernel(void* __restrict__ out, int mode, const float* __restrict__ split_sums,
+                                         const bf16* __restrict__ bias, int m, int n, int ldc, int splits) {
+  const int columns = SWIGLU ? n / 2 : n;
+  for (int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; e < (int64_t)m * columns; e += (int64_t)gridDim.x * blockDim.x) {
+    const int token = e / columns, c = e % columns;
+    const int gn = SWIGLU ? 16 * (c / 8) + c % 8 : c;
+    float v = 0.f, up = 0.f;
+    for (int sp = 0; sp < splits; ++sp) {
+      v += split_sums[((int64_t)sp * m + token) * n + gn];
+      if (SWIGLU) up += split_sums[((int64_t)sp * m + token) * n + gn + 8];
+    }
+    if (SWIGLU) v = silu(v) * up;
+    else if (bias) v += (float)bias[gn];
+    emit<bf16>(out, mode, (int64_t)token * ldc + c, v);
+  }
+}
+
 // Row tiles per workgroup: more of them means each activation fragment read from L2 serves more
 // weight rows, which matters once there are several token blocks; fewer means more workgroups.
 template <int MT, int RT, bool NORM, bool SWIGLU>
 static void launch_skinny_rt(void* out, int mode, const bf16* a, NormInput norm, const bf16* w, const bf16* bias,
-                             int m, int n, int k, int lda, int ldc, hipStream_t s) {
+                             int m, int n, int k, int lda, int ldc, hipStream_t s, float* split_sums = nullptr, int splits = 1) {
   const int groups = (n + 16 * RT - 1) / (16 * RT);
   constexpr int UNROLL = (NORM ? 4 : 8) / (MT * RT > 4 ? 4 : (MT * RT > 1 ? 2 : 1));
   if (groups <= 2048)
-    gemm_bf16_skinny_kernel<MT, RT, 8, UNROLL, NORM, SWIGLU><<<groups, 8 * 64, 0, s>>>(out, mode, a, norm, w, bias, m, n, k, lda, ldc);
+    gemm_bf16_skinny_kernel<MT, RT, 8, UNROLL, NORM, SWIGLU><<<dim3(groups, splits), 8 * 64, 0, s>>>(out, mode, a, norm, w, bias, m, n, k, lda, ldc, split_sums);
   else
-    gemm_bf16_skinny_kernel<MT, RT, 4, UNROLL, NORM, SWIGLU><<<groups, 4 * 64, 0, s>>>(out, mode, a, norm, w, bias, m, n, k, lda, ldc);
+    gemm_bf16_skinny_kernel<MT, RT, 4, UNROLL, NORM, SWIGLU><<<dim3(groups, splits), 4 * 64, 0, s>>>(out, mode, a, norm, w, bias, m, n, k, lda, ldc, split_sums);
+  if (splits > 1) {
+    const int64_t total = (int64_t)m * (SWIGLU ? n / 2 : n);
+    const int blocks = (int)((total + 255) / 256 < 1024 ? (total + 255) / 256 : 1024);
+    gemm_split_finish_kernel<SWIGLU><<<blocks, 256, 0, s>>>(out, mode, split_sums, bias, m, n, ldc, splits);
+  }
+}
+
+// Device memory for the sums of K splits, made on first use and kept (one per process: one GPU).
+static float* g_split_sums = nullptr;
+constexpr size_t SPLIT_SUMS_BYTES = 64u << 20;
+static float* split_sums_buffer() {
+  if (!g_split_sums && hipMalloc((void**)&g_split_sums, SPLIT_SUMS_BYTES) != hipSuccess) g_split_sums = nullptr;
+  return g_split_sums;
 }
 
 template <int MT, bool NORM, bool SWIGLU>
 static void launch_skinny(void* out, int mode, const bf16* a, NormInput norm, const bf16* w, const bf16* bias,
                           int m, int n, int k, int lda, int ldc, hipStream_t s) {
-  if (MT == 1 || n <= 32 * 128)
+  if (MT > 1 && !NORM) {
+    // several token blocks: 64 weight rows per workgroup, so that an activation fragment read from
+    // L2 serves four weight fragments, and K divided between workgroups until there are enough
+    // of them to fill the chip
+    const int groups = (n + 63) / 64;
+    int splits = (383 + groups) / groups;
+    if (splits > 8) splits = 8;
+    while (splits > 1 && k / splits < 512) --splits;
+    float* sums = splits > 1 ? split_sums_buffer() : nullptr;
+    if (splits > 1 && (!sums || (size_t)splits * m * n * sizeof(float) > SPLIT_SUMS_BYTES)) splits = 1;
+    launch_skinny_rt<MT, (MT > 1 ? 4 : 1), NORM, SWIGLU>(out, mode, a, norm, w, bias, m, n, k, lda, ldc, s, sums, splits);
+    return;
+  }
+  if (MT == 1 && !NORM && n >= 16384)   // measured: two row tiles and four waves stream wide matrices a little faster
+    gemm_bf16_skinny_kernel<1, 2, 4, 4, NORM, SWIGLU><<<dim3((n + 31) / 32, 1), 4 * 64, 0, s>>>(out, mode, a, norm, w, bias, m, n, k, lda, ldc, nullptr);
+  else if (MT == 1 || n <= 32 * 128)
     launch_skinny_rt<MT, 1, NORM, SWIGLU>(out, mode, a, norm, w, bias, m, n, k, lda, ldc, s);
   else if (n < 64 * 256)
     launch_skinny_rt<MT, 2, NORM, SWIGLU>(out, mode, a, norm, w, bias, m, n, k, lda, ldc, s);
@@ -362,8 +422,23 @@ static void launch_skinny_m(void* out, int mode, const bf16* a, NormInput norm, 
   else launch_skinny<4, NORM, SWIGLU>(out, mode, a, norm, w, bias, m, n, k, lda, ldc, s);
 }
 
-// Largest M for which the few-rows kernel (and with it the fused RMSNorm input) is used.
-LRS_API int lrs_gemm_skinny_max_m() { return 64; }
+// Allocates the device memory the K-split products need, so that no later call has to (a call
+// under graph capture must not allocate).  Safe to call more than once.
+LRS_API int lrs_gemm_prepare() {
+  if (!split_sums_buffer()) return lrs_fail("gemm_prepare: could not allocate %zu bytes for split sums", SPLIT_SUMS_BYTES);
+  return 0;
+}
+
+// Largest M for which callers should use the few-rows kernel (and with it the fused RMSNorm input).
+// The kernel itself takes up to 64 rows, but measured on MI355X the vendor library's products are
+// faster from 17 rows on, so callers that may use the library send larger products there.
+static int g_skinny_max_m = 16;
+LRS_API int lrs_gemm_skinny_max_m() { return g_skinny_max_m; }
+LRS_API int lrs_gemm_set_skinny_max_m(int m) {
+  LRS_REQUIRE(m >= 1 && m <= 64, "gemm: the few-rows kernel takes 1..64 rows, got %d", m);
+  g_skinny_max_m = m;
+  return 0;
+}
 
 // out [M, N] (row stride ldc) = a [M, K] (row stride lda) times w[N, K]^T.
 //   norm_weight != null: `a` is the float32 residual stream [*, K]; its rows (picked through

@@ -41,6 +41,8 @@ _SIGNATURES = {
     "lrs_gemm": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p,
                          c_int, c_float, c_int, c_void_p]),
     "lrs_gemm_skinny_max_m": (c_int, []),
+    "lrs_gemm_prepare": (c_int, []),
+    "lrs_gemm_set_skinny_max_m": (c_int, [c_int]),
     "lrs_attention": (c_int, [c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p,
                               c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_void_p]),
     "lrs_attention_decode": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p,
@@ -67,6 +69,9 @@ def library():
             fn = getattr(lib, name)
             fn.restype, fn.argtypes = restype, argtypes
         _lib = lib
+        if torch.cuda.is_available():
+            torch.cuda.init()
+            _check(lib.lrs_gemm_prepare())   # device scratch is made now, never inside a step
     return _lib
 
 
@@ -215,8 +220,13 @@ def add_into(residual: torch.Tensor, y: torch.Tensor) -> None:
 
 
 def skinny_max_m() -> int:
-    """Most rows the few-rows product kernel takes."""
+    """Most rows for which the few-rows product kernel is the one to use."""
     return library().lrs_gemm_skinny_max_m()
+
+
+def set_skinny_max_m(m: int) -> None:
+    """Move the row count from which products go to the vendor library (1..64)."""
+    _check(library().lrs_gemm_set_skinny_max_m(m))
 
 
 def fill_i32(dst: torch.Tensor, value: int) -> None:
