@@ -192,6 +192,79 @@ __global__ void qk_prep_kernel(T* __restrict__ qkv, int row_stride, int nq, int 
   }
 }
 
+// The same for the common shape, with vector loads: head_dim a power of two times 8, rotation over
+// the whole head (or none).  A thread owns 4 consecutive dims of the first half of a head and
+// their 4 rotation partners in the second half; d/8 neighbouring threads share a head.
+template <typename T, typename TW>
+__global__ __launch_bounds__(256) void qk_prep_vec_kernel(T* __restrict__ qkv, int row_stride, int nq, int nkv, int d,
+                                                          const TW* __restrict__ q_weight, const TW* __restrict__ k_weight,
+                                                          float eps, const float* __restrict__ cosv,
+                                                          const float* __restrict__ sinv, int rot_half,
+                                                          T* __restrict__ k_pages, T* __restrict__ v_pages,
+                                                          const int* __restrict__ slots, int page_size) {
+  typedef T vec4 __attribute__((ext_vector_type(4)));
+  const int per_head = d / 8, half = d / 2;
+  const int token = blockIdx.x;
+  const int head = blockIdx.y * (256 / per_head) + threadIdx.x / per_head;
+  const int j = threadIdx.x % per_head;
+  if (head >= nq + 2 * nkv) return;   // whole groups of per_head lanes leave together
+  T* src = qkv + (int64_t)token * row_stride + (int64_t)head * d;
+  const bool is_q = head < nq, is_k = !is_q && head < nq + nkv;
+  const vec4 lo = *(const vec4*)(src + 4 * j), hi = *(const vec4*)(src + half + 4 * j);
+  int64_t page = 0, off = 0;
+  int kv_head = 0;
+  if (!is_q) {
+    const int slot = slots[token];
+    if (slot < 0) return;
+    kv_head = is_k ? head - nq : head - nq - nkv;
+    page = slot / page_size;
+    off = slot % page_size;
+    if (!is_k) {
+      T* vdst = v_pages + (page * nkv + kv_head) * d * page_size + off;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        vdst[(int64_t)(4 * j + e) * page_size] = lo[e];
+        vdst[(int64_t)(half + 4 * j + e) * page_size] = hi[e];
+      }
+      return;
+    }
+  }
+  const TW* weight = is_q ? q_weight : k_weight;
+  float a[4], b[4], inv = 1.f;
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    a[e] = to_float(lo[e]);
+    b[e] = to_float(hi[e]);
+  }
+  if (weight) {
+    float ss = 0.f;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) ss += a[e] * a[e] + b[e] * b[e];
+    for (int step = per_head / 2; step > 0; step >>= 1) ss += __shfl_xor(ss, step, WAVE);
+    inv = 1.0f / sqrtf(ss / (float)d + eps);
+  }
+  vec4 out_lo, out_hi;
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    float x = a[e] * inv, y = b[e] * inv;
+    if (weight) {
+      x *= to_float(weight[4 * j + e]);
+      y *= to_float(weight[half + 4 * j + e]);
+    }
+    if (rot_half) {
+      const float c = cosv[(int64_t)token * rot_half + 4 * j + e], sn = sinv[(int64_t)token * rot_half + 4 * j + e];
+      out_lo[e] = from_float<T>(x * c - y * sn);
+      out_hi[e] = from_float<T>(y * c + x * sn);
+    } else {
+      out_lo[e] = from_float<T>(x);
+      out_hi[e] = from_float<T>(y);
+    }
+  }
+  T* dst = is_q ? src : k_pages + ((page * nkv + kv_head) * page_size + off) * d;
+  *(vec4*)(dst + 4 * j) = out_lo;
+  *(vec4*)(dst + half + 4 * j) = out_hi;
+}
+
 LRS_API int lrs_qk_prep(void* qkv, int dtype, int tokens, int row_stride, int nq, int nkv, int d,
                         const void* q_weight, const void* k_weight, int w_dtype, float eps,
                         const float* cosv, const float* sinv, int rot_half, void* k_pages,
@@ -204,6 +277,24 @@ LRS_API int lrs_qk_prep(void* qkv, int dtype, int tokens, int row_stride, int nq
   LRS_REQUIRE(row_stride >= (nq + 2 * nkv) * d, "qk_prep: row stride %d too small", row_stride);
   dim3 grid(tokens, nq + 2 * nkv), block(WAVE);
   hipStream_t s = (hipStream_t)stream;
+  const int per_head = d / 8;
+  const bool vectors = d % 8 == 0 && per_head <= 64 && (per_head & (per_head - 1)) == 0 && (rot_half == 0 || 2 * rot_half == d) &&
+                       row_stride % 4 == 0 && ((uintptr_t)qkv % 16) == 0 && ((uintptr_t)k_pages % 16) == 0;
+  if (vectors) {
+    const int heads_per_block = 256 / per_head;
+    dim3 vgrid(tokens, (nq + 2 * nkv + heads_per_block - 1) / heads_per_block);
+#define LAUNCH_VEC(T, TW)                                                                              \
+  qk_prep_vec_kernel<T, TW><<<vgrid, 256, 0, s>>>((T*)qkv, row_stride, nq, nkv, d, (const TW*)q_weight,  \
+                                                  (const TW*)k_weight, eps, cosv, sinv, rot_half,      \
+                                                  (T*)k_pages, (T*)v_pages, slots, page_size)
+    if (dtype == LRS_F32 && w_dtype == LRS_F32) LAUNCH_VEC(float, float);
+    else if (dtype == LRS_BF16 && w_dtype == LRS_BF16) LAUNCH_VEC(bf16, bf16);
+    else if (dtype == LRS_BF16 && w_dtype == LRS_F32) LAUNCH_VEC(bf16, float);
+    else if (dtype == LRS_F32 && w_dtype == LRS_BF16) LAUNCH_VEC(float, bf16);
+    else return lrs_fail("qk_prep: unknown dtypes %d/%d", dtype, w_dtype);
+#undef LAUNCH_VEC
+    return lrs_check_launch("qk_prep");
+  }
 #define LAUNCH(T, TW)                                                                          \
   qk_prep_kernel<T, TW><<<grid, block, 0, s>>>((T*)qkv, row_stride, nq, nkv, d, (const TW*)q_weight, \
                                                (const TW*)k_weight, eps, cosv, sinv, rot_half,  \
@@ -234,12 +325,33 @@ __global__ void silu_mul_kernel(T* __restrict__ out, const T* __restrict__ gu, i
   }
 }
 
+// Interleaved bf16 layout, 8 features per thread: 16 bytes of gate and 16 bytes of up in, 16 bytes out.
+__global__ void silu_mul_interleaved_bf16_kernel(bf16* __restrict__ out, const bf16* __restrict__ gu, int64_t groups) {
+  for (int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; idx < groups;
+       idx += (int64_t)gridDim.x * blockDim.x) {
+    const bf16x8 g = *(const bf16x8*)(gu + idx * 16), u = *(const bf16x8*)(gu + idx * 16 + 8);
+    bf16x8 r;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const float gv = (float)g[i];
+      r[i] = (bf16)(gv / (1.0f + expf(-gv)) * (float)u[i]);
+    }
+    *(bf16x8*)(out + idx * 8) = r;
+  }
+}
+
 LRS_API int lrs_silu_mul(void* out, const void* gu, int dtype, int tokens, int inter, int interleaved, void* stream) {
   LRS_REQUIRE(tokens > 0 && inter > 0, "silu_mul: tokens=%d inter=%d must be positive", tokens, inter);
   LRS_REQUIRE(!interleaved || inter % 8 == 0, "silu_mul: the interleaved layout needs inter %% 8 == 0, got %d", inter);
   const int64_t total = (int64_t)tokens * inter;
   const int blocks = (int)((total + 255) / 256 < 65536 ? (total + 255) / 256 : 65536);
   hipStream_t s = (hipStream_t)stream;
+  if (interleaved && dtype == LRS_BF16 && ((uintptr_t)gu % 16) == 0 && ((uintptr_t)out % 16) == 0) {
+    const int64_t groups = total / 8;
+    const int vec_blocks = (int)((groups + 255) / 256 < 16384 ? (groups + 255) / 256 : 16384);
+    silu_mul_interleaved_bf16_kernel<<<vec_blocks, 256, 0, s>>>((bf16*)out, (const bf16*)gu, groups);
+    return lrs_check_launch("silu_mul");
+  }
   if (dtype == LRS_F32)
     silu_mul_kernel<float><<<blocks, 256, 0, s>>>((float*)out, (const float*)gu, inter, total, interleaved);
   else if (dtype == LRS_BF16)
@@ -259,10 +371,31 @@ __global__ void add_into_kernel(float* __restrict__ residual, const T* __restric
     residual[idx] += to_float(y[idx]);
 }
 
+__global__ void add_into_bf16x8_kernel(float* __restrict__ residual, const bf16* __restrict__ y, int64_t groups) {
+  for (int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; idx < groups;
+       idx += (int64_t)gridDim.x * blockDim.x) {
+    const bf16x8 v = *(const bf16x8*)(y + idx * 8);
+    floatx4 a = *(floatx4*)(residual + idx * 8), b = *(floatx4*)(residual + idx * 8 + 4);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      a[i] += (float)v[i];
+      b[i] += (float)v[4 + i];
+    }
+    *(floatx4*)(residual + idx * 8) = a;
+    *(floatx4*)(residual + idx * 8 + 4) = b;
+  }
+}
+
 LRS_API int lrs_add_into(float* residual, const void* y, int dtype, int64_t total, void* stream) {
   LRS_REQUIRE(total > 0, "add_into: nothing to add");
   const int blocks = (int)((total + 255) / 256 < 65536 ? (total + 255) / 256 : 65536);
   hipStream_t s = (hipStream_t)stream;
+  if (dtype == LRS_BF16 && total % 8 == 0 && ((uintptr_t)y % 16) == 0 && ((uintptr_t)residual % 16) == 0) {
+    const int64_t groups = total / 8;
+    const int vec_blocks = (int)((groups + 255) / 256 < 16384 ? (groups + 255) / 256 : 16384);
+    add_into_bf16x8_kernel<<<vec_blocks, 256, 0, s>>>(residual, (const bf16*)y, groups);
+    return lrs_check_launch("add_into");
+  }
   if (dtype == LRS_F32) add_into_kernel<float><<<blocks, 256, 0, s>>>(residual, (const float*)y, total);
   else if (dtype == LRS_BF16) add_into_kernel<bf16><<<blocks, 256, 0, s>>>(residual, (const bf16*)y, total);
   else return lrs_fail("add_into: unknown dtype %d", dtype);
