@@ -130,11 +130,20 @@ __global__ __launch_bounds__(256) void attention_decode_bf16_kernel(
   const int tile_begin = first_tile + split * per_split;
   const int tile_end = tile_begin + per_split <= last_tile + 1 ? tile_begin + per_split : last_tile + 1;
 
+  // the block table entries of this workgroup's tiles, in LDS: the address of a key must not
+  // wait for a trip to memory of its own
+  extern __shared__ int page_ids[];
+  const int first_block = tile_begin * 32 / page_size;
+  const int last_key = tile_end * 32 - 1 < pos ? tile_end * 32 - 1 : pos;
+  if (tile_begin < tile_end)
+    for (int i = tid; i <= last_key / page_size - first_block; i += 256) page_ids[i] = table[first_block + i];
+
   const bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
   bf16x8 qf[DS];
 #pragma unroll
   for (int c = 0; c < DS; ++c)
     qf[c] = col < group ? *(const bf16x8*)(q + (int64_t)token * q_stride + (int64_t)(kvh * group + col) * D + c * 32 + g * 8) : zero8;
+  __syncthreads();
 
   floatx4 o[DB];
 #pragma unroll
@@ -153,7 +162,7 @@ __global__ __launch_bounds__(256) void attention_decode_bf16_kernel(
       const int key0 = tile * 32 + h * 16;
       present[h] = key0 <= pos && key0 + 15 >= lo;
       if (present[h]) {
-        const int64_t page = table[key0 / page_size];
+        const int64_t page = page_ids[key0 / page_size - first_block];
         const int off = key0 % page_size;
         const bf16* kp = k_pages + ((page * nkv + kvh) * page_size + off + col) * D + g * 8;
         const bf16* vp = v_pages + (page * nkv + kvh) * (int64_t)D * page_size + off + (int64_t)col * page_size + g * 4;
@@ -276,8 +285,8 @@ __global__ void attention_merge_kernel(bf16* __restrict__ out, int out_stride, c
 LRS_API int lrs_attention_decode(void* out, int out_stride, float* part_o, float* part_ml, const void* q,
                                  int q_stride, const void* k_pages, const void* v_pages,
                                  const int* block_table, int table_stride, const int* token_request,
-                                 const int* positions, int tokens, int nq, int nkv, int d, int page_size,
-                                 float scale, int window, int splits, void* stream) {
+                                 const int* positions, int tokens, int max_context, int nq, int nkv, int d,
+                                 int page_size, float scale, int window, int splits, void* stream) {
   LRS_REQUIRE(tokens > 0 && nq > 0 && nkv > 0 && nq % nkv == 0, "attention_decode: bad sizes tokens=%d nq=%d nkv=%d", tokens, nq, nkv);
   LRS_REQUIRE(nq / nkv <= 16, "attention_decode: %d query heads per kv head, at most 16 fit a tile", nq / nkv);
   LRS_REQUIRE(page_size % 16 == 0, "attention_decode: page size %d is not a multiple of 16", page_size);
@@ -286,8 +295,13 @@ LRS_API int lrs_attention_decode(void* out, int out_stride, float* part_o, float
   LRS_REQUIRE(q_stride % 8 == 0 && ((uintptr_t)q % 16) == 0, "attention_decode: q rows must be 16-byte aligned");
   dim3 grid(splits, nkv, tokens);
   hipStream_t s = (hipStream_t)stream;
+  // LDS copy of the block table entries one workgroup walks
+  LRS_REQUIRE(max_context >= 1, "attention_decode: max_context must be the longest context length of the step");
+  const int span = window > 0 && window + 64 < max_context ? window + 64 : max_context;
+  const size_t table_lds = sizeof(int) * (size_t)((span / 32 + splits) / splits * 32 / page_size + 4);
+  LRS_REQUIRE(table_lds <= 24 * 1024, "attention_decode: a context of %d tokens in %d splits needs more block table entries than fit LDS", max_context, splits);
 #define LAUNCH(D)                                                                                                   \
-  attention_decode_bf16_kernel<D><<<grid, 256, 0, s>>>((bf16*)out, out_stride, part_o, part_ml, (const bf16*)q, q_stride, \
+  attention_decode_bf16_kernel<D><<<grid, 256, table_lds, s>>>((bf16*)out, out_stride, part_o, part_ml, (const bf16*)q, q_stride, \
                                                        (const bf16*)k_pages, (const bf16*)v_pages, block_table,      \
                                                        table_stride, token_request, positions, nq, nkv, page_size,   \
                                                        scale, window, splits)

@@ -33,6 +33,7 @@ from ..cache import CacheManager, RequestCache
 from ..errors import GenerationError, KVCacheError
 from ..kernels import ops
 from ..models import DecoderModel
+from ..parts.base import length_class
 
 
 @dataclass
@@ -86,7 +87,7 @@ class StepContext:
         self.memo: dict = {}
         self.T = self.R = self.num_logit_rows = self.num_qblocks = self.max_qblock = 0
         self.qblock_token0 = self.qblock_count = None
-        self.max_q = self.max_k = 0
+        self.max_q = self.max_k = self.max_k_bound = 0
         self.all_decode = False
         self.host_q_lens: list[int] = []
         self.host_slots: list[int] = []
@@ -118,7 +119,7 @@ class ModelRunner:
         self.library_gemm = library_gemm
         # decode-only steps are captured in a HIP graph per padded batch size and replayed
         self.use_graph = use_graph and model.graph_safe()
-        self._graphs: dict[int, tuple] = {}   # bucket -> (handle, arena generation, logits tensor)
+        self._graphs: dict[tuple, tuple] = {}   # (bucket, length class) -> (handle, arena generation, logits tensor)
         self.graph_replays = 0
         t, r, g, mb = max_step_tokens, self.max_requests, len(cache.groups), cache.max_blocks
         # layout of the metadata buffer (int32 elements)
@@ -228,7 +229,11 @@ class ModelRunner:
             cursor += n
         real = len(entries)
         ctx.max_q = max(ctx.host_q_lens)
-        ctx.max_k = max(e.cache.length for e in entries)
+        ctx.max_k = ctx.max_k_bound = max(e.cache.length for e in entries)
+        if pad_to:
+            # a graph outlives the step it is captured in: sizes that must hold for every replay are
+            # made for the longest context the cache can hold
+            ctx.max_k_bound = self.cache.max_seq_len
         ctx.all_decode = ctx.max_q == 1
         if pad_to > real:
             extra = pad_to - real
@@ -325,11 +330,12 @@ class ModelRunner:
 
         Logits come back for the wanted rows of the real entries only."""
         ctx = self.prepare(entries, pad_to=bucket)
-        graph = self._graphs.get(bucket)
+        key = (bucket, length_class(ctx.max_k))
+        graph = self._graphs.get(key)
         if graph is None or graph[1] != self.arena.generation:
             if graph is not None:
                 ops.graph_destroy(graph[0])
-                del self._graphs[bucket]
+                del self._graphs[key]
             # an eager run first: it sizes every scratch buffer, so that capture allocates nothing
             h = self.model.forward_hidden(ctx)
             logits = self.model.logits(ctx, h)
@@ -344,7 +350,7 @@ class ModelRunner:
             if self.arena.generation != generation:
                 ops.graph_destroy(handle)
                 raise GenerationError("scratch buffers moved during graph capture")
-            graph = self._graphs[bucket] = (handle, generation, logits)
+            graph = self._graphs[key] = (handle, generation, logits)
         ops.graph_launch(graph[0])
         self.graph_replays += 1
         wanted = [r for r, entry in enumerate(entries) if len(entry.want)]

@@ -19,7 +19,7 @@ import math
 import torch
 
 from ..kernels import ops
-from .base import PagedKVNeed, Part, PartSpec, TensorSpec, create, register
+from .base import PagedKVNeed, Part, PartSpec, TensorSpec, create, length_class, register
 from .linear import linear, rows_of
 
 
@@ -82,11 +82,13 @@ class GQAAttention(Part):
         return PagedKVNeed(self.num_kv_heads, self.head_dim, self.window)
 
     @staticmethod
-    def _decode_splits(workgroups: int, longest: int) -> int:
+    def _decode_splits(workgroups: int, longest: int, bound: int, page_size: int) -> int:
         """Into how many workgroups the keys of one decode token are divided: enough to fill the
-        chip twice over when the batch alone does not, but at least 256 keys each."""
+        chip twice over when the batch alone does not, but at least 256 keys each (a power of two that
+        follows the length's class, not the length); and enough that the block table entries of one
+        workgroup (at most 4,096) fit its LDS for contexts up to `bound`."""
         wanted = -(-512 // workgroups)
-        return max(1, min(wanted, longest // 256, 64))
+        return max(1, min(wanted, length_class(longest) // 256, 64), -(-bound // (4096 * page_size)))
 
     # ------------------------------------------------------------------ forward
     def forward(self, ctx, x, residual, cache):
@@ -104,13 +106,16 @@ class GQAAttention(Part):
         out = ctx.scratch("attn_out", (t, nq * d), ctx.dtype)
         kv_heads = cache.k_pages.shape[1]
         if ctx.all_decode and ops.attention_decode_supported(ctx.dtype, nq, kv_heads, d, group.page_size):
-            splits = self._decode_splits(t * kv_heads, ctx.max_k if self.window is None else min(ctx.max_k, self.window + 32))
+            longest, bound = ctx.max_k, ctx.max_k_bound
+            if self.window is not None:
+                longest, bound = min(longest, self.window + 32), min(bound, self.window + 64)
+            splits = self._decode_splits(t * kv_heads, longest, bound, group.page_size)
             part_o = part_ml = None
             if splits > 1:
                 part_o = ctx.scratch("attn_part_o", (t, nq * splits * d), torch.float32)
                 part_ml = ctx.scratch("attn_part_ml", (t, nq * splits * 2), torch.float32)
             ops.attention_decode(out, qkv, cache.k_pages, cache.v_pages, group.block_table, ctx.token_request, ctx.positions,
-                                 nq, self.scale, self.window or 0, splits, part_o, part_ml)
+                                 nq, self.scale, self.window or 0, splits, part_o, part_ml, ctx.max_k_bound)
         elif ops.attention_decode_supported(ctx.dtype, nq, kv_heads, d, group.page_size):
             ops.attention_prefill(out, qkv, cache.k_pages, cache.v_pages, group.block_table, ctx.token_request, ctx.positions,
                                   ctx.qblock_token0, ctx.qblock_count, nq, self.scale, self.window or 0, ctx.max_qblock, ctx.max_k)

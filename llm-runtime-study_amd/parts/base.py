@@ -99,3 +99,11 @@ class Part:
     def weight_bytes(self) -> int:
         """Bytes of weights that one step reads (for roofline accounting)."""
         return 0
+
+
+def length_class(length: int) -> int:
+    """`length` rounded down to 256 times a power of two (0 below 256). Choices that follow the
+    context length (how far decode attention is split) are made per class, so that eager steps and
+    graph replays agree bit for bit and a growing context recaptures a handful of times."""
+    blocks = length // 256
+    return 256 << (blocks.bit_length() - 1) if blocks else 0

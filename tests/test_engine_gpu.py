@@ -108,10 +108,13 @@ def test_first_tokens_of_a_sequence_one_by_one(folders, dtype, tmp_path):
         assert err < (1e-5 if dtype == "float32" else 3e-2), f"position {position}: {err:.3g}"
 
 
+@pytest.mark.parametrize("lengths", [(3, 30, 17, 45, 9), (3, 250, 17, 500, 9)], ids=["short", "crossing-split-classes"])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-def test_graph_replay_equals_eager_steps(folders, dtype):
+def test_graph_replay_equals_eager_steps(folders, dtype, lengths):
     """Decode steps through captured graphs, with eager prefill work and synchronisations between the
-    replays; every replay's logits must equal those of the same step run eagerly."""
+    replays; every replay's logits must equal those of the same step run eagerly. The longer prompts
+    grow past 256 and 512 tokens while decoding, where decode attention starts to divide the keys
+    among more workgroups and a graph captured for the shorter context must not be replayed."""
     from llm_runtime_study_amd.cache import CacheManager
     from llm_runtime_study_amd.engine.loading import load_model
     from llm_runtime_study_amd.engine.step import ModelRunner, StepEntry
@@ -122,12 +125,13 @@ def test_graph_replay_equals_eager_steps(folders, dtype):
     rng = np.random.default_rng(8)
 
     def make(use_graph):
-        cache = CacheManager(model.cache_needs(), page_size=16, num_pages=40, max_requests=8, max_seq_len=256, dtype=dtype, device=device)
-        return ModelRunner(model, cache, max_step_tokens=128, dtype=dtype, device=device, use_graph=use_graph)
+        cache = CacheManager(model.cache_needs(), page_size=16, num_pages=40 + sum(lengths) // 16, max_requests=8, max_seq_len=1024,
+                             dtype=dtype, device=device)
+        return ModelRunner(model, cache, max_step_tokens=512, dtype=dtype, device=device, use_graph=use_graph)
 
     eager, graphed = make(False), make(True)
     assert graphed.use_graph
-    prompts = [rng.integers(0, cfg["vocab_size"], n).tolist() for n in (3, 30, 17, 45, 9)]
+    prompts = [rng.integers(0, cfg["vocab_size"], n).tolist() for n in lengths]
     stream = torch.cuda.Stream(device)
     with torch.cuda.stream(stream):
         live = {}
