@@ -407,6 +407,29 @@ __global__ void fill_i32_kernel(int* dst, int value, int64_t n) {
   for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x)
     dst[i] = value;
 }
+// ------------------------------------------------------------ scale_rows
+// out[r, :] = x[r, :] * rsqrt(sum_p sumsq[p, r] / hidden + eps): finishes an RMSNorm whose input a
+// matrix product left as bf16(h * weight) together with partial sums of h^2 (see gemm.hip), for a
+// consumer that wants the normalised rows as a tensor.
+__global__ __launch_bounds__(256) void scale_rows_kernel(bf16* __restrict__ out, const bf16* __restrict__ x,
+                                                         const float* __restrict__ sumsq, int parts, int rows,
+                                                         int hidden, float eps) {
+  __shared__ float scratch[16];
+  const int row = blockIdx.x;
+  float q = 0.f;
+  for (int p = threadIdx.x; p < parts; p += blockDim.x) q += sumsq[(int64_t)p * rows + row];
+  const float scale = 1.0f / sqrtf(block_sum(q, scratch) / (float)hidden + eps);
+  for (int c = threadIdx.x; c < hidden; c += blockDim.x)
+    out[(int64_t)row * hidden + c] = (bf16)((float)x[(int64_t)row * hidden + c] * scale);
+}
+
+LRS_API int lrs_scale_rows(void* out, const void* x, const float* sumsq, int parts, int rows, int hidden, float eps,
+                           void* stream) {
+  LRS_REQUIRE(rows > 0 && hidden > 0 && parts > 0 && eps > 0.f, "scale_rows: rows=%d hidden=%d parts=%d eps=%g must be positive", rows, hidden, parts, (double)eps);
+  scale_rows_kernel<<<rows, 256, 0, (hipStream_t)stream>>>((bf16*)out, (const bf16*)x, sumsq, parts, rows, hidden, eps);
+  return lrs_check_launch("scale_rows");
+}
+
 LRS_API int lrs_fill_i32(int* dst, int value, int64_t n, void* stream) {
   LRS_REQUIRE(n > 0, "fill: n must be positive");
   const int blocks = (int)((n + 255) / 256 < 4096 ? (n + 255) / 256 : 4096);

@@ -176,18 +176,38 @@ struct NormInput {
   float eps;
 };
 
+// A product between two RMSNorms of the residual stream can take the norm apart (at most 16 rows):
+//   * the product that adds into the residual stream h also writes next_x = bf16(h_new * g), g the
+//     weight of the norm that follows, and for each of its workgroups the sum of h_new^2 over the
+//     workgroup's columns, next_sumsq [gridDim.x, m];
+//   * the product that consumes the norm reads next_x as its input and multiplies row r of its
+//     result by rsqrt(sum_p in_sumsq[p, r] / K + eps), the factor that is constant along K.
+// The sums are added in a fixed order, so the result does not depend on the batch.
+struct NormChain {
+  const float* in_sumsq;   // consumer side: [in_parts, m], or null
+  int in_parts;
+  float in_eps;
+  bf16* next_x;            // producer side: [m, n], or null
+  float* next_sumsq;       // [gridDim.x, m]
+  const void* next_weight; // [n]
+  int next_weight_is_f32;
+};
+
 __device__ __forceinline__ float silu(float g) { return g / (1.0f + __expf(-g)); }
 
 template <int MT, int RT, int WAVES, int UNROLL, bool NORM, bool SWIGLU>
 __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_skinny_kernel(
     void* __restrict__ out, int mode, const bf16* __restrict__ x, NormInput norm,
     const bf16* __restrict__ w, const bf16* __restrict__ bias, int m, int n, int k, int lda, int ldc,
-    float* __restrict__ split_sums) {
+    float* __restrict__ split_sums, NormChain chain) {
   // RT: row tiles of 16 weight rows per workgroup; every activation fragment is used RT times.
   // gridDim.y > 1: K is also divided between workgroups; each then leaves its sums in
   // split_sums [gridDim.y, m, n] for gemm_split_finish_kernel instead of writing the output.
   __shared__ floatx4 partial[WAVES][MT][WAVE];
   __shared__ float sumsq[WAVES][MT][16];
+  __shared__ float chain_parts[WAVES * 4][16];   // in_sumsq, added up by WAVES * 4 threads per row
+  __shared__ float chain_scale[16];
+  __shared__ float chain_squares[16][RT * 16 + 1];
   const int tid = threadIdx.x, lane = tid % WAVE, wave = tid / WAVE;
   const int r = lane & 15, g = lane >> 4;
   const int n0 = blockIdx.x * 16 * RT;
@@ -294,11 +314,28 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_skinny_kernel(
       if (g == 0) sumsq[wave][t][r] = v;
     }
   }
+  const bool scaled_input = MT == 1 && !NORM && chain.in_sumsq != nullptr;
+  const bool feeds_norm = MT == 1 && !SWIGLU && chain.next_x != nullptr && mode == OUT_ADD_F32 && gridDim.y == 1;
+  if (scaled_input) {
+    const int token = tid % 16, part = tid / 16;
+    float v = 0.f;
+    if (token < m)
+      for (int p = part; p < chain.in_parts; p += WAVES * 4) v += chain.in_sumsq[(int64_t)p * m + token];
+    chain_parts[part][token] = v;
+    __syncthreads();
+    if (tid < 16) {
+      float q = 0.f;
+#pragma unroll
+      for (int p = 0; p < WAVES * 4; ++p) q += chain_parts[p][tid];
+      chain_scale[tid] = 1.0f / sqrtf(q / (float)k + chain.in_eps);
+    }
+  }
   // accumulator layout: token = t*16 + lane % 16, weight row = tile row 4 * (lane / 16) + i
   auto total = [&](int t, int l, int i) -> float {
     float v = 0.f;
 #pragma unroll
     for (int wv = 0; wv < WAVES; ++wv) v += partial[wv][t][l][i];
+    if (scaled_input) v *= chain_scale[l & 15];
     if (NORM) {
       float q = 0.f;
 #pragma unroll
@@ -332,11 +369,31 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_skinny_kernel(
       for (int e = tid; e < MT * WAVE * 4; e += WAVES * WAVE) {
         const int t = e / (WAVE * 4), l = (e / 4) % WAVE, i = e % 4;
         const int token = t * 16 + (l & 15), gn = nq0 + 4 * (l >> 4) + i;
-        if (token >= m || gn >= n) continue;
+        const bool inside = token < m && gn < n;
+        if (feeds_norm && !inside) chain_squares[l & 15][q * 16 + 4 * (l >> 4) + i] = 0.f;
+        if (!inside) continue;
         float v = total(t, l, i);
         if (bias) v += (float)bias[gn];
-        emit<bf16>(out, mode, (int64_t)token * ldc + gn, v);
+        if (feeds_norm) {
+          float* h = (float*)out + (int64_t)token * ldc + gn;
+          const float updated = *h + v;
+          *h = updated;
+          const float weight = chain.next_weight_is_f32 ? ((const float*)chain.next_weight)[gn] : (float)((const bf16*)chain.next_weight)[gn];
+          chain.next_x[(int64_t)token * n + gn] = (bf16)(updated * weight);
+          chain_squares[l & 15][q * 16 + 4 * (l >> 4) + i] = updated * updated;
+        } else {
+          emit<bf16>(out, mode, (int64_t)token * ldc + gn, v);
+        }
       }
+    }
+  }
+  if (feeds_norm) {
+    __syncthreads();
+    if (tid < m) {
+      float q = 0.f;
+#pragma unroll
+      for (int c = 0; c < RT * 16; ++c) q += chain_squares[tid][c];
+      chain.next_sumsq[(int64_t)blockIdx.x * m + tid] = q;
     }
   }
 }
@@ -365,13 +422,14 @@ __global__ void gemm_split_finish_kernel(void* __restrict__ out, int mode, const
 // weight rows, which matters once there are several token blocks; fewer means more workgroups.
 template <int MT, int RT, bool NORM, bool SWIGLU>
 static void launch_skinny_rt(void* out, int mode, const bf16* a, NormInput norm, const bf16* w, const bf16* bias,
-                             int m, int n, int k, int lda, int ldc, hipStream_t s, float* split_sums = nullptr, int splits = 1) {
+                             int m, int n, int k, int lda, int ldc, hipStream_t s, float* split_sums = nullptr, int splits = 1,
+                             NormChain chain = NormChain{}) {
   const int groups = (n + 16 * RT - 1) / (16 * RT);
   constexpr int UNROLL = (NORM ? 4 : 8) / (MT * RT > 4 ? 4 : (MT * RT > 1 ? 2 : 1));
   if (groups <= 2048)
-    gemm_bf16_skinny_kernel<MT, RT, 8, UNROLL, NORM, SWIGLU><<<dim3(groups, splits), 8 * 64, 0, s>>>(out, mode, a, norm, w, bias, m, n, k, lda, ldc, split_sums);
+    gemm_bf16_skinny_kernel<MT, RT, 8, UNROLL, NORM, SWIGLU><<<dim3(groups, splits), 8 * 64, 0, s>>>(out, mode, a, norm, w, bias, m, n, k, lda, ldc, split_sums, chain);
   else
-    gemm_bf16_skinny_kernel<MT, RT, 4, UNROLL, NORM, SWIGLU><<<dim3(groups, splits), 4 * 64, 0, s>>>(out, mode, a, norm, w, bias, m, n, k, lda, ldc, split_sums);
+    gemm_bf16_skinny_kernel<MT, RT, 4, UNROLL, NORM, SWIGLU><<<dim3(groups, splits), 4 * 64, 0, s>>>(out, mode, a, norm, w, bias, m, n, k, lda, ldc, split_sums, chain);
   if (splits > 1) {
     const int64_t total = (int64_t)m * (SWIGLU ? n / 2 : n);
     const int blocks = (int)((total + 255) / 256 < 1024 ? (total + 255) / 256 : 1024);
@@ -389,7 +447,7 @@ static float* split_sums_buffer() {
 
 template <int MT, bool NORM, bool SWIGLU>
 static void launch_skinny(void* out, int mode, const bf16* a, NormInput norm, const bf16* w, const bf16* bias,
-                          int m, int n, int k, int lda, int ldc, hipStream_t s) {
+                          int m, int n, int k, int lda, int ldc, hipStream_t s, NormChain chain = NormChain{}) {
   if (MT > 1 && !NORM) {
     // several token blocks: 64 weight rows per workgroup, so that an activation fragment read from
     // L2 serves four weight fragments, and K divided between workgroups until there are enough
@@ -404,9 +462,9 @@ static void launch_skinny(void* out, int mode, const bf16* a, NormInput norm, co
     return;
   }
   if (MT == 1 && !NORM && n >= 16384)   // measured: two row tiles and four waves stream wide matrices a little faster
-    gemm_bf16_skinny_kernel<1, 2, 4, 4, NORM, SWIGLU><<<dim3((n + 31) / 32, 1), 4 * 64, 0, s>>>(out, mode, a, norm, w, bias, m, n, k, lda, ldc, nullptr);
+    gemm_bf16_skinny_kernel<1, 2, 4, 4, NORM, SWIGLU><<<dim3((n + 31) / 32, 1), 4 * 64, 0, s>>>(out, mode, a, norm, w, bias, m, n, k, lda, ldc, nullptr, chain);
   else if (MT == 1 || n <= 32 * 128)
-    launch_skinny_rt<MT, 1, NORM, SWIGLU>(out, mode, a, norm, w, bias, m, n, k, lda, ldc, s);
+    launch_skinny_rt<MT, 1, NORM, SWIGLU>(out, mode, a, norm, w, bias, m, n, k, lda, ldc, s, nullptr, 1, chain);
   else if (n < 64 * 256)
     launch_skinny_rt<MT, 2, NORM, SWIGLU>(out, mode, a, norm, w, bias, m, n, k, lda, ldc, s);
   else
@@ -438,6 +496,36 @@ LRS_API int lrs_gemm_set_skinny_max_m(int m) {
   LRS_REQUIRE(m >= 1 && m <= 64, "gemm: the few-rows kernel takes 1..64 rows, got %d", m);
   g_skinny_max_m = m;
   return 0;
+}
+
+// How many partial sums of squares a product of n output columns leaves for the norm that follows it
+// (the number of workgroups of the few-rows kernel for that width).
+LRS_API int lrs_gemm_norm_chain_parts(int n) { return n >= 16384 ? (n + 31) / 32 : (n + 15) / 16; }
+
+// The few-rows bf16 product (M <= 16) with an RMSNorm of the residual stream taken apart around it;
+// see NormChain.  in_sumsq != null: `a` is bf16(h * g) and row r of the result is scaled by
+// rsqrt(sum_p in_sumsq[p, r] / K + in_eps).  next_x != null (mode must add into the float32
+// residual, no swiglu): also writes next_x [M, N] = bf16(out_new * next_weight) and next_sumsq
+// [lrs_gemm_norm_chain_parts(N), M].
+LRS_API int lrs_gemm_norm_chain(void* out, int mode, const void* a, const void* w, const void* bias, int m, int n, int k,
+                                int lda, int ldc, int swiglu, const float* in_sumsq, int in_parts, float in_eps,
+                                void* next_x, float* next_sumsq, const void* next_weight, int next_weight_dtype,
+                                void* stream) {
+  LRS_REQUIRE(m > 0 && m <= 16 && n > 0 && k > 0, "gemm_norm_chain: takes 1..16 rows and positive sizes, got m=%d n=%d k=%d", m, n, k);
+  LRS_REQUIRE(lda >= k && ldc >= (swiglu ? n / 2 : n), "gemm_norm_chain: strides lda=%d ldc=%d too small for k=%d n=%d", lda, ldc, k, n);
+  LRS_REQUIRE(mode >= OUT_STORE && mode <= OUT_ADD_F32, "gemm_norm_chain: unknown output mode %d", mode);
+  LRS_REQUIRE(k % 8 == 0 && lda % 8 == 0 && ((uintptr_t)a % 16 == 0) && ((uintptr_t)w % 16 == 0),
+              "gemm_norm_chain: needs 16-byte aligned rows (k=%d lda=%d)", k, lda);
+  LRS_REQUIRE(!swiglu || (n % 16 == 0 && bias == nullptr && mode == OUT_STORE), "gemm_norm_chain: swiglu needs n %% 16 == 0, no bias and a stored output (n=%d)", n);
+  LRS_REQUIRE(in_sumsq == nullptr || (in_parts > 0 && in_eps > 0.f), "gemm_norm_chain: in_parts and in_eps must be positive");
+  LRS_REQUIRE(next_x == nullptr || (mode == OUT_ADD_F32 && !swiglu && next_sumsq && next_weight),
+              "gemm_norm_chain: the output for the next norm needs a product that adds into the float32 residual stream");
+  const NormChain chain{in_sumsq, in_parts, in_eps, (bf16*)next_x, next_sumsq, next_weight, next_weight_dtype == LRS_F32};
+  const NormInput none{nullptr, nullptr, nullptr, 0, 0.f};
+  hipStream_t s = (hipStream_t)stream;
+  if (swiglu) launch_skinny<1, false, true>(out, mode, (const bf16*)a, none, (const bf16*)w, nullptr, m, n, k, lda, ldc, s, chain);
+  else launch_skinny<1, false, false>(out, mode, (const bf16*)a, none, (const bf16*)w, (const bf16*)bias, m, n, k, lda, ldc, s, chain);
+  return lrs_check_launch("gemm_norm_chain");
 }
 
 // out [M, N] (row stride ldc) = a [M, K] (row stride lda) times w[N, K]^T.

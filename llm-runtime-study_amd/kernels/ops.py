@@ -40,6 +40,10 @@ _SIGNATURES = {
     "lrs_gather_rows": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p]),
     "lrs_gemm": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p,
                          c_int, c_float, c_int, c_void_p]),
+    "lrs_gemm_norm_chain": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,
+                                    c_void_p, c_int, c_float, c_void_p, c_void_p, c_void_p, c_int, c_void_p]),
+    "lrs_gemm_norm_chain_parts": (c_int, [c_int]),
+    "lrs_scale_rows": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_float, c_void_p]),
     "lrs_gemm_skinny_max_m": (c_int, []),
     "lrs_gemm_prepare": (c_int, []),
     "lrs_gemm_set_skinny_max_m": (c_int, [c_int]),
@@ -296,6 +300,76 @@ def gemm(out: torch.Tensor, a: torch.Tensor, w: torch.Tensor, bias: torch.Tensor
                               dtype_code(w.dtype), m, n, k, lda, ldc, None if rows is None else _dev(rows, "rows"),
                               None if not normed else _dev(norm_weight, "norm_weight"), dtype_code(norm_weight.dtype) if normed else 0,
                               eps, 1 if swiglu else 0, _stream()))
+
+
+NORM_CHAIN_MAX_ROWS = 16
+
+
+def gemm_chains_norm(dtype: torch.dtype, m: int, k: int) -> bool:
+    """Whether gemm_norm_chain() takes a product of m rows over k with weights of `dtype`."""
+    return dtype == torch.bfloat16 and m <= min(NORM_CHAIN_MAX_ROWS, library().lrs_gemm_skinny_max_m()) and k % 8 == 0
+
+
+def norm_chain_parts(n: int) -> int:
+    """Partial sums of squares per row that a product of n output columns leaves for the next norm."""
+    return library().lrs_gemm_norm_chain_parts(n)
+
+
+def gemm_norm_chain(out: torch.Tensor, a: torch.Tensor, w: torch.Tensor, bias: torch.Tensor | None = None,
+                    accumulate: bool = False, swiglu: bool = False,
+                    in_sumsq: torch.Tensor | None = None, in_eps: float = 0.0,
+                    next_x: torch.Tensor | None = None, next_sumsq: torch.Tensor | None = None,
+                    next_weight: torch.Tensor | None = None) -> None:
+    """out = a @ w.T (+ bias) for at most 16 bf16 rows, with an RMSNorm taken apart around it.
+
+    in_sumsq [parts, M] float32: `a` holds bf16(h * norm weight); row r of the product is multiplied
+    by rsqrt(sum_p in_sumsq[p, r] / K + in_eps), which completes the norm.
+    next_x [M, N] bf16, next_sumsq [norm_chain_parts(N), M] float32, next_weight [N] (needs
+    `accumulate`): besides adding into `out`, write bf16(out_new * next_weight) and the partial sums
+    of out_new^2, the input of the next product called with in_sumsq."""
+    n, k = w.shape
+    m = a.shape[0]
+    lda, ldc = _rows(a, "a"), _rows(out, "out")
+    _need(w.dim() == 2 and w.is_contiguous() and a.shape[1] == k, f"gemm_norm_chain: weight must be contiguous [N, {a.shape[1]}], got {tuple(w.shape)}")
+    _need(a.dtype == torch.bfloat16 and gemm_chains_norm(w.dtype, m, k), "gemm_norm_chain: needs bf16 input and weights, at most 16 rows, K % 8 == 0")
+    _need(out.shape == (m, n // 2 if swiglu else n), f"gemm_norm_chain: out must be [{m}, {n // 2 if swiglu else n}], got {tuple(out.shape)}")
+    if accumulate:
+        _need(out.dtype == torch.float32, "gemm_norm_chain: accumulation needs a float32 output")
+        mode = OUT_ADD_F32
+    elif out.dtype == w.dtype:
+        mode = OUT_STORE
+    else:
+        _need(out.dtype == torch.float32, "gemm_norm_chain: output must be bf16 or float32")
+        mode = OUT_STORE_F32
+    if bias is not None:
+        _need(bias.numel() == n and bias.dtype == w.dtype and bias.is_contiguous(), "gemm_norm_chain: bias must hold N values of the weight dtype")
+    if swiglu:
+        _need(n % 16 == 0 and bias is None and mode == OUT_STORE, "gemm_norm_chain: swiglu needs N % 16 == 0, no bias, a stored output")
+    parts = 0
+    if in_sumsq is not None:
+        _need(in_sumsq.dtype == torch.float32 and in_sumsq.dim() == 2 and in_sumsq.shape[1] == m and in_sumsq.is_contiguous() and in_eps > 0,
+              f"gemm_norm_chain: in_sumsq must be contiguous float32 [parts, {m}] and in_eps positive")
+        parts = in_sumsq.shape[0]
+    if next_x is not None:
+        _need(accumulate and not swiglu, "gemm_norm_chain: only a product that adds into the residual stream can feed the next norm")
+        _need(next_x.dtype == torch.bfloat16 and next_x.shape == (m, n) and next_x.is_contiguous(), f"gemm_norm_chain: next_x must be contiguous bf16 [{m}, {n}]")
+        _need(next_sumsq is not None and next_sumsq.dtype == torch.float32 and next_sumsq.shape == (norm_chain_parts(n), m) and next_sumsq.is_contiguous(),
+              f"gemm_norm_chain: next_sumsq must be contiguous float32 [{norm_chain_parts(n)}, {m}]")
+        _need(next_weight is not None and next_weight.numel() == n and next_weight.is_contiguous(), "gemm_norm_chain: next_weight must hold N values")
+    _check(library().lrs_gemm_norm_chain(
+        _dev(out, "out"), mode, _dev(a, "a"), _dev(w, "w"), None if bias is None else _dev(bias, "bias"), m, n, k, lda, ldc,
+        1 if swiglu else 0, None if in_sumsq is None else _dev(in_sumsq, "in_sumsq"), parts, in_eps,
+        None if next_x is None else _dev(next_x, "next_x"), None if next_x is None else _dev(next_sumsq, "next_sumsq"),
+        None if next_x is None else _dev(next_weight, "next_weight"), dtype_code(next_weight.dtype) if next_x is not None else 0, _stream()))
+
+
+def scale_rows(out: torch.Tensor, x: torch.Tensor, sumsq: torch.Tensor, eps: float) -> None:
+    """out[r] = x[r] * rsqrt(sum_p sumsq[p, r] / hidden + eps): completes a norm that gemm_norm_chain() began."""
+    m, hidden = x.shape
+    _need(x.dtype == torch.bfloat16 and out.dtype == torch.bfloat16 and out.shape == x.shape and x.is_contiguous() and out.is_contiguous(),
+          "scale_rows: x and out must be contiguous bf16 of one shape")
+    _need(sumsq.dtype == torch.float32 and sumsq.dim() == 2 and sumsq.shape[1] == m and sumsq.is_contiguous(), f"scale_rows: sumsq must be float32 [parts, {m}]")
+    _check(library().lrs_scale_rows(_dev(out, "out"), _dev(x, "x"), _dev(sumsq, "sumsq"), sumsq.shape[0], m, hidden, eps, _stream()))
 
 
 # -------------------------------------------------------------- attention

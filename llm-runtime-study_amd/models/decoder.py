@@ -78,8 +78,17 @@ class DecoderModel:
         """Residual stream [T, H] float32 after the last layer (before the final norm)."""
         h = ctx.scratch("residual", (ctx.T, self.spec.hidden_size), torch.float32)
         ops.embed(h, self.embedding, ctx.token_ids, self.spec.embedding_multiplier)
-        for position, entry in enumerate(self.spec.schedule):
-            self.layers[entry.layer].forward(ctx, h, ctx.layer_cache(position))
+        schedule = self.spec.schedule
+        begun = None   # the next layer's first norm, if the product that last updated h began it
+        for position, entry in enumerate(schedule):
+            layer = self.layers[entry.layer]
+            if not getattr(layer, "chains_norms", False):
+                layer.forward(ctx, h, ctx.layer_cache(position))
+                begun = None
+                continue
+            following = self.layers[schedule[position + 1].layer] if position + 1 < len(schedule) else None
+            then_norm = following.first_norm if getattr(following, "chains_norms", False) else None
+            begun = layer.forward(ctx, h, ctx.layer_cache(position), normed=begun, then_norm=then_norm)
         return h
 
     def logits(self, ctx, h: torch.Tensor) -> torch.Tensor:

@@ -26,6 +26,7 @@ from .linear import linear, rows_of
 class GQAAttention(Part):
     graph_safe = True  # launches only library kernels on arena buffers
     takes_lazy_norm = True
+    begins_next_norm = True
 
     def __init__(self, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int, *,
                  position: PartSpec = PartSpec("none"), qk_norm: bool = False, qk_norm_eps: float = 1e-6,
@@ -91,7 +92,7 @@ class GQAAttention(Part):
         return max(1, min(wanted, length_class(longest) // 256, 64), -(-bound // (4096 * page_size)))
 
     # ------------------------------------------------------------------ forward
-    def forward(self, ctx, x, residual, cache):
+    def forward(self, ctx, x, residual, cache, then_norm=None):
         if cache is None:
             raise ValueError("attention needs a paged cache (its own, or the one it is told to read)")
         t, d, nq = rows_of(x), self.head_dim, self.num_heads
@@ -122,7 +123,7 @@ class GQAAttention(Part):
         else:
             ops.attention(out, qkv, cache.k_pages, cache.v_pages, group.block_table, ctx.token_request, ctx.positions,
                           nq, self.scale, self.window or 0)
-        linear(ctx, residual, out, self.w_o, accumulate=True)
+        return linear(ctx, residual, out, self.w_o, accumulate=True, then_norm=then_norm)
 
 
 register("mixer", "gqa_attention", GQAAttention)

@@ -14,6 +14,16 @@ Roles and what each must provide:
   feed_forward   forward(ctx, x, residual)              adds its output into residual (float32)
   block          forward(ctx, h, cache)                 one layer: norms, mixer, feed-forward
 
+Optional, each announced by a class attribute (a part without it is simply given plain tensors):
+
+  takes_lazy_norm = True      mixer / feed_forward: `x` may be a description of the norm (LazyNorm or
+                              ScaledRows of parts/linear.py) that its first `linear()` completes
+  begins_next_norm = True     mixer / feed_forward: forward(..., then_norm=norm) may return ScaledRows,
+                              the norm of the updated residual begun by its last product, or None
+  chains_norms = True         block: forward(ctx, h, cache, normed=None, then_norm=None) takes the
+                              normalised input a previous block began and may return the next one;
+                              `first_norm` is the norm it applies to its input
+
 `ctx` is the StepContext of engine/step.py: the step's token metadata on the device and a
 scratch arena.  The residual stream `h` is float32 in every precision mode.
 """

@@ -8,6 +8,7 @@ The two sums happen inside the parts, which add into the float32 residual stream
 from __future__ import annotations
 
 from .base import Part, PartSpec, create, register
+from .linear import materialize
 
 
 class PreNormBlock(Part):
@@ -41,17 +42,36 @@ class PreNormBlock(Part):
     def graph_safe(self) -> bool:
         return all(getattr(part, "graph_safe", False) for _, part in self._children())
 
-    def forward(self, ctx, h, cache):
+    chains_norms = True
+
+    @property
+    def first_norm(self):
+        return self.mixer_norm
+
+    def forward(self, ctx, h, cache, normed=None, then_norm=None):
+        """Run the layer on the residual stream h.  `normed`: this layer's first norm of h, already
+        begun by the product that last updated h; `then_norm`: the norm that follows this layer.
+        Returns that norm of the updated h if the last product began it, else None."""
         # a consumer that says `takes_lazy_norm` gets the norm as a description to fold into its
         # first matrix product; any other gets the normalised tensor
-        x = self._normed(ctx, self.mixer_norm, self.mixer, h)
-        self.mixer.forward(ctx, x, h, cache)
-        x = self._normed(ctx, self.ff_norm, self.feed_forward, h)
+        x = self._normed(ctx, self.mixer_norm, self.mixer, h, normed)
+        if getattr(self.mixer, "begins_next_norm", False):
+            begun = self.mixer.forward(ctx, x, h, cache, then_norm=self.ff_norm)
+        else:
+            self.mixer.forward(ctx, x, h, cache)
+            begun = None
+        x = self._normed(ctx, self.ff_norm, self.feed_forward, h, begun)
+        if then_norm is not None and getattr(self.feed_forward, "begins_next_norm", False):
+            return self.feed_forward.forward(ctx, x, h, then_norm=then_norm)
         self.feed_forward.forward(ctx, x, h)
+        return None
 
     @staticmethod
-    def _normed(ctx, norm, consumer, h):
-        if getattr(consumer, "takes_lazy_norm", False):
+    def _normed(ctx, norm, consumer, h, begun=None):
+        lazy = getattr(consumer, "takes_lazy_norm", False)
+        if begun is not None:
+            return begun if lazy else materialize(ctx, begun)
+        if lazy:
             try:
                 return norm.forward(ctx, h, lazy=True)
             except TypeError:      # a norm kind without the lazy form

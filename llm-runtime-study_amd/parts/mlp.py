@@ -17,6 +17,7 @@ from .linear import linear, rows_of
 class SwiGLU(Part):
     graph_safe = True  # launches only library kernels on arena buffers
     takes_lazy_norm = True
+    begins_next_norm = True
 
     def __init__(self, hidden_size: int, intermediate_size: int):
         if hidden_size <= 0 or intermediate_size <= 0:
@@ -48,7 +49,7 @@ class SwiGLU(Part):
     def weight_bytes(self):
         return (self.gate_up.numel() + self.down.numel()) * self.down.element_size()
 
-    def forward(self, ctx, x, residual):
+    def forward(self, ctx, x, residual, then_norm=None):
         t = rows_of(x)
         act = ctx.scratch("ffn_act", (t, self.intermediate_size), ctx.dtype)
         if self.interleaved:
@@ -57,7 +58,7 @@ class SwiGLU(Part):
             gate_up = ctx.scratch("ffn_gate_up", (t, 2 * self.intermediate_size), ctx.dtype)
             linear(ctx, gate_up, x, self.gate_up)
             ops.silu_mul(act, gate_up)
-        linear(ctx, residual, act, self.down, accumulate=True)
+        return linear(ctx, residual, act, self.down, accumulate=True, then_norm=then_norm)
 
 
 register("feed_forward", "swiglu", SwiGLU)

@@ -28,6 +28,11 @@ class RMSNorm(Part):
     def bind(self, weights, dtype):
         self.weight = weights["weight"]
 
+    def rms_parameters(self):
+        """(weight, eps): says that this norm is w * x * rsqrt(mean(x^2) + eps), so that the matrix
+        product before it may begin it (see parts/linear.py)."""
+        return self.weight, self.eps
+
     def forward(self, ctx, h, rows=None, count=None, lazy: bool = False):
         """Normalise rows of h [*, size] (all, or the `count` rows listed in `rows`).
 

@@ -252,6 +252,65 @@ def test_gemm_with_swiglu_epilogue(ops, m, inter, k, all_rows_in_own_kernel):
         close_in_norm(out, want)
 
 
+@pytest.mark.parametrize("w_dtype", DTYPES)
+@pytest.mark.parametrize("m,h,n2,k,swiglu", [(1, 64, 96, 32, False), (8, 4096, 6144, 4096, False), (16, 4096, 24576, 12288, True),
+                                             (5, 104, 328, 72, False), (9, 96, 320, 160, True), (3, 16400, 48, 64, False)])
+def test_gemm_with_norm_taken_apart(ops, w_dtype, m, h, n2, k, swiglu):
+    """Two products with an RMSNorm of the residual stream between them: the first adds into the
+    stream and leaves bf16(h * weight) with partial sums of squares, the second finishes the norm
+    with a row factor in its epilogue.  Checked against residual add, norm and products in float32;
+    scale_rows() turns the same intermediate into the normalised rows."""
+    g = torch.Generator().manual_seed(m * 1000 + h)
+    a = (torch.randn(m, k, generator=g)).bfloat16()
+    w1 = (torch.randn(h, k, generator=g) / math.sqrt(k)).bfloat16()
+    residual = torch.randn(m, h, generator=g) * 3
+    gamma = (1 + 0.3 * torch.randn(h, generator=g)).to(w_dtype)
+    w2 = (torch.randn(n2, h, generator=g) / math.sqrt(h)).bfloat16()
+    bias = None if swiglu else (torch.randn(n2, generator=g)).bfloat16()
+    eps = 1e-5
+
+    stream = dev(residual.clone())
+    parts = ops.norm_chain_parts(h)
+    next_x = torch.empty(m, h, dtype=torch.bfloat16, device="cuda")
+    sumsq = torch.full((parts, m), float("nan"), device="cuda")
+    ops.gemm_norm_chain(stream, dev(a), dev(w1), accumulate=True, next_x=next_x, next_sumsq=sumsq, next_weight=dev(gamma))
+    want_stream = residual + a.float() @ w1.float().T
+    torch.testing.assert_close(stream.cpu(), want_stream, rtol=1e-4, atol=1e-4)
+    torch.testing.assert_close(sumsq.sum(0).cpu(), want_stream.pow(2).sum(1), rtol=1e-4, atol=1e-4)
+    torch.testing.assert_close(next_x.cpu().float(), (stream.cpu() * gamma.float()).bfloat16().float(), rtol=0, atol=0)
+
+    normed = want_stream * torch.rsqrt(want_stream.pow(2).mean(1, keepdim=True) + eps) * gamma.float()
+    rows = torch.empty(m, h, dtype=torch.bfloat16, device="cuda")
+    ops.scale_rows(rows, next_x, sumsq, eps)
+    torch.testing.assert_close(rows.cpu().float(), normed, rtol=2e-2, atol=2e-2)
+
+    if swiglu:
+        inter = n2 // 2
+        gate, up = w2[:inter], w2[inter:]
+        stacked = torch.stack((gate.view(inter // 8, 8, h), up.view(inter // 8, 8, h)), 1).reshape(n2, h).contiguous()
+        out = torch.empty(m, inter, dtype=torch.bfloat16, device="cuda")
+        ops.gemm_norm_chain(out, next_x, dev(stacked), swiglu=True, in_sumsq=sumsq, in_eps=eps)
+        want = torch.nn.functional.silu(normed @ gate.float().T) * (normed @ up.float().T)
+    else:
+        out = torch.empty(m, n2, dtype=torch.bfloat16, device="cuda")
+        ops.gemm_norm_chain(out, next_x, dev(w2), dev(bias), in_sumsq=sumsq, in_eps=eps)
+        want = normed @ w2.float().T + bias.float()
+    close_in_norm(out.float(), want, rel=1.5e-2)
+
+
+def test_gemm_with_norm_taken_apart_refuses_what_it_cannot_do(ops):
+    from llm_runtime_study_amd.errors import KernelError
+
+    a = torch.zeros(17, 64, dtype=torch.bfloat16, device="cuda")
+    w = torch.zeros(32, 64, dtype=torch.bfloat16, device="cuda")
+    with pytest.raises(KernelError, match="at most 16 rows"):
+        ops.gemm_norm_chain(torch.zeros(17, 32, device="cuda"), a, w, accumulate=True)
+    with pytest.raises(KernelError, match="adds into the residual"):
+        ops.gemm_norm_chain(torch.zeros(4, 32, dtype=torch.bfloat16, device="cuda"), a[:4], w,
+                            next_x=torch.zeros(4, 32, dtype=torch.bfloat16, device="cuda"),
+                            next_sumsq=torch.zeros(2, 4, device="cuda"), next_weight=torch.ones(32, device="cuda"))
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_gemm_row_does_not_depend_on_batch(ops, dtype):
     g = torch.Generator().manual_seed(5)
