@@ -96,6 +96,81 @@ __global__ __launch_bounds__(THREADS) void attention_generic_kernel(
 }
 
 // ------------------------------------------------- bf16 decode kernel
+// What the decode kernel does to raw q, k and v rows when it also does the work of qk_prep: the
+// per-head RMSNorm of q and k (weights null: none), the rotation of pairs (i, i + D/2) by the
+// step's cos/sin tables (null: none) and the write of the new key and value into the pages.
+struct DecodePrep {
+  const void* q_weight;   // [D]
+  const void* k_weight;   // [D]
+  int weight_is_f32;
+  float eps;
+  const float* cosv;      // [tokens, D/2]
+  const float* sinv;
+  int kv_columns;         // kv heads held in the qkv rows after the q heads: k, then v; 0: keys and
+                          // values are another layer's, already in the pages
+};
+
+// One head row, raw -> normalised and rotated, in the operand layout of the 16x16x32 products: the
+// lane holds dims c*32 + g*8 .. +8 of every 32-dim chunk c, the four lanes g = 0..3 with equal
+// lane % 16 hold one head between them.  All 64 lanes must call it together.
+template <int D>
+__device__ __forceinline__ void prepare_head(bf16x8 (&r)[D / 32], const bf16* __restrict__ head, int g,
+                                             const void* __restrict__ weight, int weight_is_f32, float eps,
+                                             const float* __restrict__ cosrow, const float* __restrict__ sinrow) {
+  constexpr int DS = D / 32;
+  float x[DS][8];
+#pragma unroll
+  for (int c = 0; c < DS; ++c) {
+    const bf16x8 raw = *(const bf16x8*)(head + c * 32 + g * 8);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) x[c][j] = (float)raw[j];
+  }
+  // weights and tables come in 16-byte loads (the host checks their alignment)
+  if (weight) {
+    float ss = 0.f;
+#pragma unroll
+    for (int c = 0; c < DS; ++c)
+#pragma unroll
+      for (int j = 0; j < 8; ++j) ss = fmaf(x[c][j], x[c][j], ss);
+    ss += __shfl_xor(ss, 16, WAVE);
+    ss += __shfl_xor(ss, 32, WAVE);
+    const float inv = 1.0f / sqrtf(ss / (float)D + eps);
+#pragma unroll
+    for (int c = 0; c < DS; ++c) {
+      float w[8];
+      if (weight_is_f32) {
+        const floatx4 w0 = *(const floatx4*)((const float*)weight + c * 32 + g * 8), w1 = *(const floatx4*)((const float*)weight + c * 32 + g * 8 + 4);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) { w[j] = w0[j]; w[4 + j] = w1[j]; }
+      } else {
+        const bf16x8 wb = *(const bf16x8*)((const bf16*)weight + c * 32 + g * 8);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) w[j] = (float)wb[j];
+      }
+#pragma unroll
+      for (int j = 0; j < 8; ++j) x[c][j] = x[c][j] * inv * w[j];
+    }
+  }
+  if (cosrow) {
+#pragma unroll
+    for (int c = 0; c < DS / 2; ++c) {
+      const floatx4 c0 = *(const floatx4*)(cosrow + c * 32 + g * 8), c1 = *(const floatx4*)(cosrow + c * 32 + g * 8 + 4);
+      const floatx4 s0 = *(const floatx4*)(sinrow + c * 32 + g * 8), s1 = *(const floatx4*)(sinrow + c * 32 + g * 8 + 4);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const float cs = j < 4 ? c0[j & 3] : c1[j & 3], sn = j < 4 ? s0[j & 3] : s1[j & 3];
+        const float a = x[c][j], b = x[c + DS / 2][j];
+        x[c][j] = a * cs - b * sn;
+        x[c + DS / 2][j] = b * cs + a * sn;
+      }
+    }
+  }
+#pragma unroll
+  for (int c = 0; c < DS; ++c)
+#pragma unroll
+    for (int j = 0; j < 8; ++j) r[c][j] = (bf16)x[c][j];
+}
+
 // One query token per request (a decode step).  A workgroup of four waves owns one
 // (token, kv head, split): the query heads that share the kv head (at most 16) sit in the
 // columns of the matrix-core tiles, so every key and value is loaded once for the whole
@@ -108,13 +183,16 @@ __global__ __launch_bounds__(THREADS) void attention_generic_kernel(
 // S comes out of the first product with a head per lane column and four keys per lane, which
 // is exactly the operand layout the second product wants for P, so P never leaves registers.
 // Waves are merged through LDS, splits by attention_merge_kernel.
-template <int D>
+// PREP: q holds the raw rows of the q/k/v product; the kernel prepares q itself, and the wave that
+// meets the token's own position prepares the new key, takes it and the new value in place of what
+// the pages hold there, and writes both into the pages (see DecodePrep).
+template <int D, bool PREP>
 __global__ __launch_bounds__(256) void attention_decode_bf16_kernel(
     bf16* __restrict__ out, int out_stride, float* __restrict__ part_o, float* __restrict__ part_ml,
-    const bf16* __restrict__ q, int q_stride, const bf16* __restrict__ k_pages,
-    const bf16* __restrict__ v_pages, const int* __restrict__ block_table, int table_stride,
+    const bf16* __restrict__ q, int q_stride, bf16* __restrict__ k_pages,
+    bf16* __restrict__ v_pages, const int* __restrict__ block_table, int table_stride,
     const int* __restrict__ token_request, const int* __restrict__ positions, int nq, int nkv,
-    int page_size, float scale, int window, int splits) {
+    int page_size, float scale, int window, int splits, DecodePrep prep) {
   constexpr int DS = D / 32, DB = D / 16, WAVES = 4;
   __shared__ float sm_m[WAVES][16], sm_l[WAVES][16];
   __shared__ float sm_o[WAVES][D][16];
@@ -140,9 +218,47 @@ __global__ __launch_bounds__(256) void attention_decode_bf16_kernel(
 
   const bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
   bf16x8 qf[DS];
+  const bf16* q_row = q + (int64_t)token * q_stride;
+  if (PREP) {
+    const float* cosrow = prep.cosv ? prep.cosv + (int64_t)token * (D / 2) : nullptr;
+    const float* sinrow = prep.sinv ? prep.sinv + (int64_t)token * (D / 2) : nullptr;
+    prepare_head<D>(qf, q_row + (int64_t)(kvh * group + (col < group ? col : 0)) * D, g, prep.q_weight, prep.weight_is_f32,
+                    prep.eps, cosrow, sinrow);
 #pragma unroll
-  for (int c = 0; c < DS; ++c)
-    qf[c] = col < group ? *(const bf16x8*)(q + (int64_t)token * q_stride + (int64_t)(kvh * group + col) * D + c * 32 + g * 8) : zero8;
+    for (int c = 0; c < DS; ++c) qf[c] = col < group ? qf[c] : zero8;
+  } else {
+#pragma unroll
+    for (int c = 0; c < DS; ++c)
+      qf[c] = col < group ? *(const bf16x8*)(q_row + (int64_t)(kvh * group + col) * D + c * 32 + g * 8) : zero8;
+  }
+  // The workgroup that walks the token's own position prepares the new key once (its last wave,
+  // which is dealt the fewest tiles), leaves it and the new value in LDS for the wave that meets
+  // the position, and writes both into the pages.
+  __shared__ __attribute__((aligned(16))) bf16 own_k[D];
+  __shared__ bf16 own_v[D];
+  const bool holds_own = PREP && prep.kv_columns > 0 && tile_begin <= last_tile && last_tile < tile_end;
+  if (holds_own && wave == WAVES - 1) {
+    bf16x8 kn[DS];
+    prepare_head<D>(kn, q_row + (int64_t)(nq + kvh) * D, g, prep.k_weight, prep.weight_is_f32, prep.eps,
+                    prep.cosv ? prep.cosv + (int64_t)token * (D / 2) : nullptr,
+                    prep.sinv ? prep.sinv + (int64_t)token * (D / 2) : nullptr);
+    const int64_t page = table[pos / page_size];
+    const int off = pos % page_size;
+    if (col == 0) {
+      bf16* kdst = k_pages + ((page * nkv + kvh) * page_size + off) * D + g * 8;
+#pragma unroll
+      for (int c = 0; c < DS; ++c) {
+        *(bf16x8*)&own_k[c * 32 + g * 8] = kn[c];
+        if (page >= 0) *(bf16x8*)(kdst + c * 32) = kn[c];
+      }
+    }
+    const bf16* v_row = q_row + (int64_t)(nq + prep.kv_columns + kvh) * D;
+    for (int i = lane; i < D; i += WAVE) {
+      const bf16 vn = v_row[i];
+      own_v[i] = vn;
+      if (page >= 0) v_pages[(page * nkv + kvh) * (int64_t)D * page_size + (int64_t)i * page_size + off] = vn;
+    }
+  }
   __syncthreads();
 
   floatx4 o[DB];
@@ -175,6 +291,24 @@ __global__ __launch_bounds__(256) void attention_decode_bf16_kernel(
         for (int c = 0; c < DS; ++c) kf[h][c] = zero8;
 #pragma unroll
         for (int b = 0; b < DB; ++b) vf[h][b] = bf16x4{0, 0, 0, 0};
+      }
+    }
+    if (holds_own && tile == last_tile) {
+      // the token's own key and value take the place of what the pages hold at its position
+      const int own_half = (pos % 32) / 16, own_col = pos % 16, own_g = (pos % 16) / 4, own_i = pos % 4;
+#pragma unroll
+      for (int h = 0; h < 2; ++h)
+#pragma unroll
+        for (int c = 0; c < DS; ++c)
+          if (h == own_half && col == own_col) kf[h][c] = *(const bf16x8*)&own_k[c * 32 + g * 8];
+#pragma unroll
+      for (int b = 0; b < DB; ++b) {
+        const bf16 vn = own_v[b * 16 + col];
+#pragma unroll
+        for (int h = 0; h < 2; ++h)
+#pragma unroll
+          for (int i = 0; i < 4; ++i)
+            if (h == own_half && g == own_g && i == own_i) vf[h][b][i] = vn;
       }
     }
     floatx4 s[2];
@@ -282,11 +416,16 @@ __global__ void attention_merge_kernel(bf16* __restrict__ out, int out_stride, c
 // Decode step in bf16: one query token per request.  part_o [tokens, nq, splits, d] and part_ml
 // [tokens, nq, splits, 2] float32 are needed when splits > 1.  Returns an error for shapes the
 // matrix-core kernel does not take (the caller then uses lrs_attention).
+// prepare != 0: q points at the raw rows [q heads | kv_columns k heads | kv_columns v heads] of the
+// q/k/v product and the kernel does the work of lrs_qk_prep as well (rotation over the whole head
+// or none; kv_columns is nkv, or 0 for a layer that reads another layer's pages).
 LRS_API int lrs_attention_decode(void* out, int out_stride, float* part_o, float* part_ml, const void* q,
-                                 int q_stride, const void* k_pages, const void* v_pages,
+                                 int q_stride, void* k_pages, void* v_pages,
                                  const int* block_table, int table_stride, const int* token_request,
                                  const int* positions, int tokens, int max_context, int nq, int nkv, int d,
-                                 int page_size, float scale, int window, int splits, void* stream) {
+                                 int page_size, float scale, int window, int splits, int prepare,
+                                 const void* q_weight, const void* k_weight, int w_dtype, float eps,
+                                 const float* cosv, const float* sinv, int kv_columns, void* stream) {
   LRS_REQUIRE(tokens > 0 && nq > 0 && nkv > 0 && nq % nkv == 0, "attention_decode: bad sizes tokens=%d nq=%d nkv=%d", tokens, nq, nkv);
   LRS_REQUIRE(nq / nkv <= 16, "attention_decode: %d query heads per kv head, at most 16 fit a tile", nq / nkv);
   LRS_REQUIRE(page_size % 16 == 0, "attention_decode: page size %d is not a multiple of 16", page_size);
@@ -300,11 +439,28 @@ LRS_API int lrs_attention_decode(void* out, int out_stride, float* part_o, float
   const int span = window > 0 && window + 64 < max_context ? window + 64 : max_context;
   const size_t table_lds = sizeof(int) * (size_t)((span / 32 + splits) / splits * 32 / page_size + 4);
   LRS_REQUIRE(table_lds <= 24 * 1024, "attention_decode: a context of %d tokens in %d splits needs more block table entries than fit LDS", max_context, splits);
+  if (prepare) {
+    LRS_REQUIRE((q_weight == nullptr) == (k_weight == nullptr), "attention_decode: q and k norm weights must come together");
+    LRS_REQUIRE(q_weight == nullptr || eps > 0.f, "attention_decode: eps must be positive");
+    LRS_REQUIRE((cosv == nullptr) == (sinv == nullptr), "attention_decode: cos and sin tables must come together");
+    LRS_REQUIRE(cosv == nullptr || d % 64 == 0, "attention_decode: the kernel rotates heads of 64, 128 or 192 dims only, got %d", d);
+    LRS_REQUIRE(kv_columns == 0 || kv_columns == nkv, "attention_decode: kv_columns must be 0 or the number of kv heads (%d), got %d", nkv, kv_columns);
+    LRS_REQUIRE(q_stride >= (nq + 2 * kv_columns) * d, "attention_decode: q row stride %d too small for q, k and v heads", q_stride);
+    LRS_REQUIRE((uintptr_t)q_weight % 16 == 0 && (uintptr_t)k_weight % 16 == 0 && (uintptr_t)cosv % 16 == 0 && (uintptr_t)sinv % 16 == 0,
+                "attention_decode: norm weights and rotation tables must be 16-byte aligned");
+  }
+  const DecodePrep prep{q_weight, k_weight, w_dtype == LRS_F32, eps, cosv, sinv, kv_columns};
 #define LAUNCH(D)                                                                                                   \
-  attention_decode_bf16_kernel<D><<<grid, 256, table_lds, s>>>((bf16*)out, out_stride, part_o, part_ml, (const bf16*)q, q_stride, \
-                                                       (const bf16*)k_pages, (const bf16*)v_pages, block_table,      \
-                                                       table_stride, token_request, positions, nq, nkv, page_size,   \
-                                                       scale, window, splits)
+  do {                                                                                                              \
+    if (prepare)                                                                                                    \
+      attention_decode_bf16_kernel<D, true><<<grid, 256, table_lds, s>>>(                                           \
+          (bf16*)out, out_stride, part_o, part_ml, (const bf16*)q, q_stride, (bf16*)k_pages, (bf16*)v_pages,        \
+          block_table, table_stride, token_request, positions, nq, nkv, page_size, scale, window, splits, prep);    \
+    else                                                                                                            \
+      attention_decode_bf16_kernel<D, false><<<grid, 256, table_lds, s>>>(                                          \
+          (bf16*)out, out_stride, part_o, part_ml, (const bf16*)q, q_stride, (bf16*)k_pages, (bf16*)v_pages,        \
+          block_table, table_stride, token_request, positions, nq, nkv, page_size, scale, window, splits, prep);    \
+  } while (0)
   switch (d) {
     case 32: LAUNCH(32); break;
     case 64: LAUNCH(64); break;

@@ -8,6 +8,7 @@ the library is missing or cannot be built; there is no fallback.
 
 from __future__ import annotations
 
+from dataclasses import dataclass
 import ctypes
 from ctypes import c_char_p, c_float, c_int, c_int64, c_void_p, POINTER, byref
 
@@ -50,7 +51,8 @@ _SIGNATURES = {
     "lrs_attention": (c_int, [c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p,
                               c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_void_p]),
     "lrs_attention_decode": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p,
-                                     c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_int, c_void_p]),
+                                     c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_int, c_int,
+                                     c_void_p, c_void_p, c_int, c_float, c_void_p, c_void_p, c_int, c_void_p]),
     "lrs_attention_prefill": (c_int, [c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p,
                                       c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_void_p]),
     "lrs_attention_prefill_group": (c_int, []),
@@ -400,11 +402,35 @@ def attention_decode_supported(dtype: torch.dtype, nq: int, nkv: int, d: int, pa
     return dtype == torch.bfloat16 and d in DECODE_HEAD_DIMS and page_size % 16 == 0 and nq // nkv <= 16
 
 
+@dataclass
+class DecodePrepare:
+    """What attention_decode() does to the raw q/k/v rows when it stands in for qk_prep(): per-head
+    RMSNorm of q and k (weights None: none), rotation of the whole head by cos/sin [T, d/2] (None:
+    none), and the write of the new key and value into the pages (kv_heads = the number of kv heads
+    held in the rows; 0 for a layer that reads another layer's pages)."""
+    q_weight: torch.Tensor | None
+    k_weight: torch.Tensor | None
+    eps: float
+    cos: torch.Tensor | None
+    sin: torch.Tensor | None
+    kv_heads: int
+
+
+def decode_prepare_supported(d: int, rotates: bool) -> bool:
+    """Whether attention_decode() can do qk_prep()'s work for heads of d dims (it rotates pairs that
+    lie 32-dim chunks apart: d a multiple of 64)."""
+    return not rotates or d % 64 == 0
+
+
 def attention_decode(out: torch.Tensor, q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, block_table: torch.Tensor,
                      token_request: torch.Tensor, positions: torch.Tensor, nq: int, scale: float, window: int = 0, splits: int = 1,
-                     part_o: torch.Tensor | None = None, part_ml: torch.Tensor | None = None, max_context: int | None = None) -> None:
+                     part_o: torch.Tensor | None = None, part_ml: torch.Tensor | None = None, max_context: int | None = None,
+                     prepare: "DecodePrepare | None" = None) -> None:
     """attention() for a step with one query token per request, bfloat16 only; the keys of a token
-    are divided between `splits` workgroups whose partial results meet in part_o / part_ml."""
+    are divided between `splits` workgroups whose partial results meet in part_o / part_ml.
+
+    prepare: `q` holds the raw rows of the q/k/v product and the kernel also does what qk_prep()
+    does (see DecodePrepare); without it q, and the pages, must have been through qk_prep()."""
     tokens = out.shape[0]
     _need(k_pages.dim() == 4 and k_pages.is_contiguous() and v_pages.is_contiguous(), "attention_decode: pages must be contiguous")
     _, nkv, page_size, d = k_pages.shape
@@ -418,11 +444,27 @@ def attention_decode(out: torch.Tensor, q: torch.Tensor, k_pages: torch.Tensor, 
     if splits > 1:
         _need(part_o is not None and part_o.dtype == torch.float32 and part_o.is_contiguous() and part_o.numel() >= tokens * nq * splits * d, "attention_decode: part_o too small")
         _need(part_ml is not None and part_ml.dtype == torch.float32 and part_ml.is_contiguous() and part_ml.numel() >= tokens * nq * splits * 2, "attention_decode: part_ml too small")
+    fused = [0, None, None, 0, 0.0, None, None, 0]
+    if prepare is not None:
+        _need(decode_prepare_supported(d, prepare.cos is not None), f"attention_decode: cannot rotate heads of {d} dims itself")
+        _need((prepare.q_weight is None) == (prepare.k_weight is None), "attention_decode: q and k norm weights must come together")
+        _need(prepare.kv_heads in (0, nkv) and q.shape[1] >= (nq + 2 * prepare.kv_heads) * d, "attention_decode: q rows must hold the q heads and kv_heads (0 or all) k and v heads")
+        for name, w in (("q_weight", prepare.q_weight), ("k_weight", prepare.k_weight)):
+            _need(w is None or (w.numel() == d and w.is_contiguous() and w.dtype == prepare.q_weight.dtype), f"attention_decode: {name} must hold head_dim values")
+        for name, t in (("cos", prepare.cos), ("sin", prepare.sin)):
+            _need((t is None) == (prepare.cos is None) and (t is None or (t.dtype == torch.float32 and t.shape == (tokens, d // 2) and t.is_contiguous())),
+                  f"attention_decode: {name} must be float32 [{tokens}, {d // 2}]")
+        normed = prepare.q_weight is not None
+        _need(not normed or prepare.eps > 0, "attention_decode: eps must be positive")
+        fused = [1, _dev(prepare.q_weight, "q_weight") if normed else None, _dev(prepare.k_weight, "k_weight") if normed else None,
+                 dtype_code(prepare.q_weight.dtype) if normed else 0, prepare.eps,
+                 None if prepare.cos is None else _dev(prepare.cos, "cos"), None if prepare.sin is None else _dev(prepare.sin, "sin"), prepare.kv_heads]
     _check(library().lrs_attention_decode(
         _dev(out, "out"), _rows(out, "out"), None if splits == 1 else _dev(part_o, "part_o"), None if splits == 1 else _dev(part_ml, "part_ml"),
         _dev(q, "q"), _rows(q, "q"), _dev(k_pages, "k_pages"), _dev(v_pages, "v_pages"), _dev(block_table, "block_table"), block_table.stride(0),
         _dev(token_request, "token_request"), _dev(positions, "positions"), tokens,
-        block_table.shape[1] * page_size if max_context is None else max_context, nq, nkv, d, page_size, scale, window, splits, _stream()))
+        block_table.shape[1] * page_size if max_context is None else max_context, nq, nkv, d, page_size, scale, window, splits,
+        *fused, _stream()))
 
 
 def attention_prefill(out: torch.Tensor, q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, block_table: torch.Tensor,

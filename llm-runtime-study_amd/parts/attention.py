@@ -102,11 +102,19 @@ class GQAAttention(Part):
         linear(ctx, qkv, x, self.w_qkv, self.b_qkv)
         tables = self.position.tables(ctx)
         cos, sin = tables if tables is not None else (None, None)
-        ops.qk_prep(qkv, nq, nkv, d, self.q_norm, self.k_norm, self.qk_norm_eps, cos, sin,
-                    cache.k_pages, cache.v_pages, group.slots, group.page_size)
         out = ctx.scratch("attn_out", (t, nq * d), ctx.dtype)
         kv_heads = cache.k_pages.shape[1]
-        if ctx.all_decode and ops.attention_decode_supported(ctx.dtype, nq, kv_heads, d, group.page_size):
+        decode = ctx.all_decode and ops.attention_decode_supported(ctx.dtype, nq, kv_heads, d, group.page_size)
+        # a decode step's attention kernel normalises and rotates q and k and writes the new key and
+        # value itself, when the rotation covers the whole head or there is none
+        whole_head = cos is None or cos.shape[1] * 2 == d
+        prepare = None
+        if decode and whole_head and ops.decode_prepare_supported(d, cos is not None):
+            prepare = ops.DecodePrepare(self.q_norm, self.k_norm, self.qk_norm_eps, cos, sin, nkv)
+        else:
+            ops.qk_prep(qkv, nq, nkv, d, self.q_norm, self.k_norm, self.qk_norm_eps, cos, sin,
+                        cache.k_pages, cache.v_pages, group.slots, group.page_size)
+        if decode:
             longest, bound = ctx.max_k, ctx.max_k_bound
             if self.window is not None:
                 longest, bound = min(longest, self.window + 32), min(bound, self.window + 64)
@@ -116,7 +124,7 @@ class GQAAttention(Part):
                 part_o = ctx.scratch("attn_part_o", (t, nq * splits * d), torch.float32)
                 part_ml = ctx.scratch("attn_part_ml", (t, nq * splits * 2), torch.float32)
             ops.attention_decode(out, qkv, cache.k_pages, cache.v_pages, group.block_table, ctx.token_request, ctx.positions,
-                                 nq, self.scale, self.window or 0, splits, part_o, part_ml, ctx.max_k_bound)
+                                 nq, self.scale, self.window or 0, splits, part_o, part_ml, ctx.max_k_bound, prepare)
         elif ops.attention_decode_supported(ctx.dtype, nq, kv_heads, d, group.page_size):
             ops.attention_prefill(out, qkv, cache.k_pages, cache.v_pages, group.block_table, ctx.token_request, ctx.positions,
                                   ctx.qblock_token0, ctx.qblock_count, nq, self.scale, self.window or 0, ctx.max_qblock, ctx.max_k)

@@ -1,4 +1,4 @@
-"""Test-only helpers: the two tiny configurations and a weight generator of the tests' own."""
+"""Test-only helpers: the tiny configurations and a weight generator of the tests' own."""
 
 from __future__ import annotations
 
@@ -20,6 +20,16 @@ TINY_B = {
     "max_position_embeddings": 512, "rms_norm_eps": 1e-5, "rope_theta": 1000000.0,
     "hidden_act": "silu", "attention_bias": True, "attention_dropout": 0.0,
     "tie_word_embeddings": False, "torch_dtype": "bfloat16", "bos_token_id": 0, "eos_token_id": [5, 7],
+}
+# Heads of 64 dims, the smallest the decode attention kernel rotates itself; three query heads per
+# kv head, and every other size unlike A and B again.
+TINY_C = {
+    "architectures": ["Qwen3ForCausalLM"], "model_type": "qwen3",
+    "vocab_size": 300, "hidden_size": 80, "intermediate_size": 176, "num_hidden_layers": 2,
+    "num_attention_heads": 6, "num_key_value_heads": 2, "head_dim": 64,
+    "max_position_embeddings": 640, "rms_norm_eps": 3e-6, "rope_theta": 500000.0,
+    "hidden_act": "silu", "attention_bias": False, "attention_dropout": 0.0,
+    "tie_word_embeddings": False, "torch_dtype": "bfloat16", "bos_token_id": 3, "eos_token_id": 4,
 }
 
 

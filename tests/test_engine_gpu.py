@@ -11,7 +11,7 @@ import pytest
 import torch
 
 from tests import traces
-from tests.helpers import TINY_A, TINY_B
+from tests.helpers import TINY_A, TINY_B, TINY_C
 from tests.plain import model as plain
 
 pytestmark = pytest.mark.gpu
@@ -24,7 +24,7 @@ def folders(tmp_path_factory):
     from llm_runtime_study_amd.weights import write_model_dir
 
     out = {}
-    for name, raw, seed in (("a", TINY_A, 31), ("b", TINY_B, 32)):
+    for name, raw, seed in (("a", TINY_A, 31), ("b", TINY_B, 32), ("c", TINY_C, 33)):
         folder = tmp_path_factory.mktemp(f"engine_{name}")
         write_model_dir(config_from_dict(raw), seed=seed, model_dir=folder, init="scaled")
         cfg, weights = plain.load_model_dir(folder, torch.float64)
@@ -41,7 +41,7 @@ def plain_greedy(cfg, weights, prompt, new_tokens, stop=()):
     return ids[len(prompt):]
 
 
-@pytest.mark.parametrize("name", ["a", "b"])
+@pytest.mark.parametrize("name", ["a", "b", "c"])
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_greedy_generation_through_the_entry_point(folders, name, dtype):
     from llm_runtime_study_amd import Engine, SamplingConfig
@@ -71,12 +71,13 @@ def test_greedy_generation_through_the_entry_point(folders, name, dtype):
     assert engine.last_cache_capacity == len(prompts[-1]) + 8 and engine.last_cache_num_bytes > 0
 
 
+@pytest.mark.parametrize("name", ["b", "c"])
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-def test_long_decoding_token_by_token(folders, dtype, tmp_path):
+def test_long_decoding_token_by_token(folders, name, dtype, tmp_path):
     """8 prompt tokens, then 400 tokens one by one: every logits row against the plain model."""
     from llm_runtime_study_amd.engine import trace
 
-    folder, cfg, weights = folders["b"]
+    folder, cfg, weights = folders[name]
     ids = np.random.default_rng(6).integers(0, cfg["vocab_size"], 408).tolist()
     want = plain.qwen3_forward(weights, cfg, ids)
     steps = traces.prefill_then_decode({"r": ids}, tail=400)
@@ -109,8 +110,9 @@ def test_first_tokens_of_a_sequence_one_by_one(folders, dtype, tmp_path):
 
 
 @pytest.mark.parametrize("lengths", [(3, 30, 17, 45, 9), (3, 250, 17, 500, 9)], ids=["short", "crossing-split-classes"])
+@pytest.mark.parametrize("name", ["b", "c"])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-def test_graph_replay_equals_eager_steps(folders, dtype, lengths):
+def test_graph_replay_equals_eager_steps(folders, name, dtype, lengths):
     """Decode steps through captured graphs, with eager prefill work and synchronisations between the
     replays; every replay's logits must equal those of the same step run eagerly. The longer prompts
     grow past 256 and 512 tokens while decoding, where decode attention starts to divide the keys
@@ -119,7 +121,7 @@ def test_graph_replay_equals_eager_steps(folders, dtype, lengths):
     from llm_runtime_study_amd.engine.loading import load_model
     from llm_runtime_study_amd.engine.step import ModelRunner, StepEntry
 
-    folder, cfg, _ = folders["b"]
+    folder, cfg, _ = folders[name]
     device = torch.device("cuda", 0)
     _, model = load_model(folder, dtype, device)
     rng = np.random.default_rng(8)

@@ -457,6 +457,77 @@ def test_attention_decode_kernel(ops, nq, nkv, d, page, window, splits):
     torch.testing.assert_close(out.cpu().double(), want, rtol=2e-2, atol=2e-2)
 
 
+@pytest.mark.parametrize("nq,nkv,d,page,window,splits,normed,rotated,shared", [
+    (32, 8, 128, 16, 0, 5, True, True, False), (4, 4, 64, 32, 0, 3, True, True, False), (6, 2, 192, 64, 0, 4, False, True, False),
+    (8, 2, 32, 16, 0, 2, True, False, False), (16, 1, 96, 16, 40, 1, False, False, False), (8, 2, 64, 16, 100, 3, True, True, True),
+    (8, 2, 128, 16, 0, 1, True, True, False),
+])
+def test_attention_decode_prepares_q_k_v_itself(ops, nq, nkv, d, page, window, splits, normed, rotated, shared):
+    """The decode kernel given raw q/k/v rows (it normalises, rotates and writes the new key and
+    value itself) against qk_prep() followed by the same kernel: equal outputs and equal pages."""
+    g = torch.Generator().manual_seed(23)
+    lengths = [1, 15, 16, 17, 31, 32, 33, 64, 257, 700, 48, 49]
+    t, scale, eps = len(lengths), 1 / math.sqrt(d), 1e-5
+    blocks = [(n + page - 1) // page for n in lengths]
+    n_pages = sum(blocks) + 2
+    perm = torch.randperm(n_pages, generator=g).tolist()
+    kp = torch.randn(n_pages, nkv, page, d, generator=g).bfloat16()   # the new token's slot holds junk
+    vp = torch.randn(n_pages, nkv, d, page, generator=g).bfloat16()
+    table = torch.full((t, max(blocks) + 1), -1, dtype=torch.int32)
+    for r in range(t):
+        for b in range(blocks[r]):
+            table[r, b] = perm.pop()
+    positions = torch.tensor([n - 1 for n in lengths], dtype=torch.int32)
+    slots = torch.tensor([int(table[r, (n - 1) // page]) * page + (n - 1) % page for r, n in enumerate(lengths)], dtype=torch.int32)
+    kv_heads = 0 if shared else nkv
+    raw = (torch.randn(t, (nq + 2 * kv_heads) * d, generator=g) * 2).bfloat16()
+    qw = (1 + 0.3 * torch.randn(d, generator=g)).bfloat16() if normed else None
+    kw = (1 + 0.3 * torch.randn(d, generator=g)).bfloat16() if normed else None
+    cos = sin = None
+    if rotated:
+        angle = torch.rand(t, d // 2, generator=g) * 6.28
+        cos, sin = dev(angle.cos()), dev(angle.sin())
+    request = dev(torch.arange(t, dtype=torch.int32))
+
+    def run(fused):
+        k_dev, v_dev, rows = dev(kp.clone()), dev(vp.clone()), dev(raw.clone())
+        out = torch.empty(t, nq * d, device="cuda", dtype=torch.bfloat16)
+        part_o = torch.empty(t, nq * splits * d, device="cuda")
+        part_ml = torch.empty(t, nq * splits * 2, device="cuda")
+        prepare = None
+        if fused:
+            prepare = ops.DecodePrepare(None if qw is None else dev(qw), None if kw is None else dev(kw), eps, cos, sin, kv_heads)
+        else:
+            ops.qk_prep(rows, nq, kv_heads, d, None if qw is None else dev(qw), None if kw is None else dev(kw), eps, cos, sin,
+                        k_dev, v_dev, dev(slots), page)
+        ops.attention_decode(out, rows, k_dev, v_dev, dev(table), request, dev(positions), nq, scale, window, splits,
+                             part_o, part_ml, prepare=prepare)
+        torch.cuda.synchronize()
+        return out.cpu().float(), k_dev.cpu().float(), v_dev.cpu().float()
+
+    assert ops.decode_prepare_supported(d, rotated)
+    out_two, k_two, v_two = run(False)
+    out_one, k_one, v_one = run(True)
+    assert torch.equal(v_one, v_two)
+    torch.testing.assert_close(k_one, k_two, rtol=1e-2, atol=1e-6)     # a last bit of bf16 at most
+    assert (k_one != kp.float()).any() != shared                        # keys were written, unless they are another layer's
+    torch.testing.assert_close(out_one, out_two, rtol=2e-2, atol=2e-2)
+    assert (out_one - out_two).norm() <= 4e-3 * out_two.norm()
+
+
+def test_attention_decode_refuses_to_rotate_odd_chunk_counts(ops):
+    from llm_runtime_study_amd.errors import KernelError
+
+    assert not ops.decode_prepare_supported(96, True) and ops.decode_prepare_supported(96, False)
+    kp = torch.zeros(2, 1, 16, 96, dtype=torch.bfloat16, device="cuda")
+    vp = torch.zeros(2, 1, 96, 16, dtype=torch.bfloat16, device="cuda")
+    with pytest.raises(KernelError, match="cannot rotate"):
+        ops.attention_decode(torch.zeros(1, 96, dtype=torch.bfloat16, device="cuda"), torch.zeros(1, 3 * 96, dtype=torch.bfloat16, device="cuda"),
+                             kp, vp, torch.zeros(1, 2, dtype=torch.int32, device="cuda"), torch.zeros(1, dtype=torch.int32, device="cuda"),
+                             torch.zeros(1, dtype=torch.int32, device="cuda"), 1, 0.1,
+                             prepare=ops.DecodePrepare(None, None, 1e-6, torch.zeros(1, 48, device="cuda"), torch.zeros(1, 48, device="cuda"), 1))
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_attention_finds_a_far_key(ops, dtype):
     """One key among 700 is made to dominate: the output must be its value, wherever it lies."""

@@ -12,25 +12,25 @@ import pytest
 import torch
 
 from tests import traces
-from tests.helpers import TINY_A, TINY_B
+from tests.helpers import TINY_A, TINY_B, TINY_C
 from tests.plain import model as plain
 
 pytestmark = pytest.mark.gpu
 
 ROOT = Path(__file__).resolve().parents[1]
-LENGTHS = {"a": [5, 11, 17, 64, 65, 127, 33, 90], "b": [1, 23, 40, 64, 200, 331, 129, 77, 16]}
+LENGTHS = {"a": [5, 11, 17, 64, 65, 127, 33, 90], "b": [1, 23, 40, 64, 200, 331, 129, 77, 16], "c": [2, 34, 64, 130, 300, 95, 600]}
 
 
 @pytest.fixture(scope="module")
 def models(tmp_path_factory):
-    """Model folders of both tiny configurations, their requests and the plain logits."""
+    """Model folders of the tiny configurations, their requests and the plain logits."""
     from llm_runtime_study_amd.config import config_from_dict
     from llm_runtime_study_amd.weights import write_model_dir
 
     out = {}
-    for name, raw in (("a", TINY_A), ("b", TINY_B)):
+    for name, raw in (("a", TINY_A), ("b", TINY_B), ("c", TINY_C)):
         folder = tmp_path_factory.mktemp(f"model_{name}")
-        write_model_dir(config_from_dict(raw), seed=11 if name == "a" else 12, model_dir=folder, init="scaled")
+        write_model_dir(config_from_dict(raw), seed={"a": 11, "b": 12, "c": 13}[name], model_dir=folder, init="scaled")
         cfg, weights = plain.load_model_dir(folder, torch.float64)
         rng = np.random.default_rng(5)
         requests = {f"{name}{i}": rng.integers(0, raw["vocab_size"], n).tolist() for i, n in enumerate(LENGTHS[name])}
@@ -70,7 +70,7 @@ def round64(n):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name", ["a", "b"])
+@pytest.mark.parametrize("name", ["a", "b", "c"])
 def test_whole(models, name, dtype, tmp_path):
     folder, raw, requests, want = models[name]
     steps = traces.whole(requests)
@@ -80,7 +80,7 @@ def test_whole(models, name, dtype, tmp_path):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name", ["a", "b"])
+@pytest.mark.parametrize("name", ["a", "b", "c"])
 def test_prefill_then_last_32_one_by_one(models, name, dtype, tmp_path):
     folder, raw, requests, want = models[name]
     steps = traces.prefill_then_decode(requests, tail=32)
@@ -89,7 +89,7 @@ def test_prefill_then_last_32_one_by_one(models, name, dtype, tmp_path):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name,page", [("a", 16), ("b", 16), ("b", 4), ("a", 64)])
+@pytest.mark.parametrize("name,page", [("a", 16), ("b", 16), ("b", 4), ("a", 64), ("c", 32)])
 def test_portions_of_changing_size(models, name, page, dtype, tmp_path):
     folder, raw, requests, want = models[name]
     steps = traces.portions(requests)
@@ -98,7 +98,7 @@ def test_portions_of_changing_size(models, name, page, dtype, tmp_path):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name,seed", [("a", 0), ("b", 1), ("b", 2)])
+@pytest.mark.parametrize("name,seed", [("a", 0), ("b", 1), ("b", 2), ("c", 3)])
 def test_mixed_with_reused_pages(models, name, seed, dtype, tmp_path):
     folder, raw, requests, want = models[name]
     budget = 2 * max(round64(len(t)) for t in requests.values())
