@@ -9,6 +9,8 @@
 // float32.  Key tiles start at multiples of the tile size counted from position 0, so the
 // rounding of a query's result depends on its position only, never on how the sequence
 // was cut into steps.
+#include <type_traits>
+
 #include "common.h"
 
 // 2^x by the hardware instruction alone (arguments here are <= 0 or -inf; results below the
@@ -489,13 +491,20 @@ LRS_API int lrs_attention_decode(void* out, int out_stride, float* part_o, float
 // kernel with 16 queries in the tile columns instead of the heads: S[key, query] = K Q^T, online
 // softmax per query column with the causal (and window) mask of that query's position,
 // O^T[dim, query] += V^T P.  Every query is finished by one wave, so nothing is merged.
+// Two workgroups share a compute unit (at most 256 registers a lane, which also keeps the
+// accumulators out of the AGPRs, where rescaling them would cost moves at every tile), so one
+// wave's exponentials run beside another's matrix products.  The grid is one-dimensional: groups
+// come longest first, and in every second chunk of `chunk` workgroups (one per compute unit) the
+// order is turned round, so that the two workgroups that meet on a compute unit are a long and a
+// short one; the kv head changes fastest, which keeps one kv head's keys in one XCD's L2.
 template <int D, int QB>
-__global__ __launch_bounds__(256) void attention_prefill_bf16_kernel(
+__global__ __launch_bounds__(256, D <= 128 ? 2 : 1) void attention_prefill_bf16_kernel(
     bf16* __restrict__ out, int out_stride, const bf16* __restrict__ q, int q_stride,
     const bf16* __restrict__ k_pages, const bf16* __restrict__ v_pages,
     const int* __restrict__ block_table, int table_stride, const int* __restrict__ token_request,
     const int* __restrict__ positions, const int* __restrict__ qblock_token0,
-    const int* __restrict__ qblock_count, int nq, int nkv, int page_size, float scale, int window) {
+    const int* __restrict__ qblock_count, int n_blocks, int chunk, int nq, int nkv, int page_size, float scale,
+    int window) {
   constexpr int DS = D / 32, DB = D / 16;
   constexpr int KLD = D + 8, VLD = 32 + 8;                    // padded LDS rows
   constexpr int KCHUNKS = 32 * D / 8, VCHUNKS = D * 4;        // 16-byte pieces of one tile
@@ -505,13 +514,20 @@ __global__ __launch_bounds__(256) void attention_prefill_bf16_kernel(
   const int tid = threadIdx.x, threads = blockDim.x;
   const int lane = tid % WAVE, wave = tid / WAVE, waves = threads / WAVE;
   const int col = lane & 15, g = lane >> 4;
-  const int kvh = blockIdx.y, group = nq / nkv;
-  const int token0 = qblock_token0[blockIdx.x], count = qblock_count[blockIdx.x];
+  const int group = nq / nkv;
+  const int which_chunk = blockIdx.x / chunk, in_chunk = blockIdx.x % chunk;
+  const int chunk_block0 = which_chunk * (chunk / nkv);
+  const int chunk_blocks = n_blocks - chunk_block0 < chunk / nkv ? n_blocks - chunk_block0 : chunk / nkv;
+  const int kvh = in_chunk % nkv;
+  const int qblock = chunk_block0 + ((which_chunk & 1) ? chunk_blocks - 1 - in_chunk / nkv : in_chunk / nkv);
+  const int token0 = qblock_token0[qblock], count = qblock_count[qblock];
   const int pos_first = positions[token0], pos_last = positions[token0 + count - 1];
   const int lo_first = (window > 0 && pos_first - window + 1 > 0) ? pos_first - window + 1 : 0;
+  const int lo_last = (window > 0 && pos_last - window + 1 > 0) ? pos_last - window + 1 : 0;
   const int* table = block_table + (int64_t)token_request[token0] * table_stride;
   const bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
   const float scale2 = scale * 1.4426950408889634f;
+  const float rescale_step = RESCALE_STEP / scale2;              // in units of the unscaled scores
   const int first_tile = lo_first / 32, last_tile = pos_last / 32;
   // the part of the request's block table that the tiles need, in LDS: the address of a key must
   // not wait for a trip to memory of its own
@@ -521,8 +537,7 @@ __global__ __launch_bounds__(256) void attention_prefill_bf16_kernel(
   __syncthreads();
 
   // pieces of a tile this thread brings in: keys [32, D] and transposed values [D, 32]
-  // two register sets in turn: a tile is asked for two tiles ahead of its use
-  bf16x8 kreg_a[KPT], vreg_a[VPT], kreg_b[KPT], vreg_b[VPT];
+  bf16x8 kreg_a[KPT], vreg_a[VPT];
   auto fetch = [&](int tile, bf16x8 (&kreg)[KPT], bf16x8 (&vreg)[VPT]) {
     int64_t kbase[2], vbase[2];
     bool present[2];
@@ -585,11 +600,13 @@ __global__ __launch_bounds__(256) void attention_prefill_bf16_kernel(
       for (int e = 0; e < DB; ++e) o[b][e] = floatx4{0.f, 0.f, 0.f, 0.f};
     }
 
-    auto work = [&](int tile, int buffer) {
+    // MASKED = false: every query of the group may see every key of the tile (it lies wholly before
+    // the group's first position and inside the last one's window), so no score needs a test.
+    // Scores stay unscaled; the scale enters with the exponent: p = 2^(s * scale2 - max * scale2).
+    auto work = [&](int tile, int buffer, auto masked) {
+      constexpr bool MASKED = decltype(masked)::value;
       const bf16* kt = ks[buffer];
       const bf16* vt = vs[buffer];
-      // Three phases over all query blocks at once, without branches: blocks past the diagonal or
-      // without queries are masked like any other key a query may not see and add nothing.
       floatx4 sc[QB][2];
 #pragma unroll
       for (int b = 0; b < QB; ++b) sc[b][0] = sc[b][1] = floatx4{0.f, 0.f, 0.f, 0.f};
@@ -611,9 +628,10 @@ __global__ __launch_bounds__(256) void attention_prefill_bf16_kernel(
         for (int h = 0; h < 2; ++h)
 #pragma unroll
           for (int i = 0; i < 4; ++i) {
-            const int key = tile * 32 + h * 16 + g * 4 + i;
-            const bool valid = key <= pos[b] && key >= lo[b];
-            sc[b][h][i] = valid ? sc[b][h][i] * scale2 : -INFINITY;
+            if (MASKED) {
+              const int key = tile * 32 + h * 16 + g * 4 + i;
+              sc[b][h][i] = (key <= pos[b] && key >= lo[b]) ? sc[b][h][i] : -INFINITY;
+            }
             tile_max = fmaxf(tile_max, sc[b][h][i]);
           }
         tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 16, WAVE));
@@ -621,17 +639,18 @@ __global__ __launch_bounds__(256) void attention_prefill_bf16_kernel(
         // The reference point of the exponentials follows the maximum only when that has grown by
         // more than 2^8: weights then stay below 256, well inside float32 and bfloat16, and the
         // accumulators need rescaling a few times per sequence instead of at nearly every tile.
-        const float new_max = tile_max > run_max[b] + RESCALE_STEP ? tile_max : run_max[b];
-        // a query whose window or position leaves it no key in this tile keeps its state
-        alpha[b] = new_max == -INFINITY ? 1.f : fast_exp2(run_max[b] - new_max);
-        const float shift = new_max == -INFINITY ? 0.f : new_max;
+        const float new_max = tile_max > run_max[b] + rescale_step ? tile_max : run_max[b];
+        // a query whose window or position leaves it no key so far keeps its state
+        const bool empty = MASKED && new_max == -INFINITY;
+        alpha[b] = empty ? 1.f : fast_exp2((run_max[b] - new_max) * scale2);
+        const float shift = empty ? 0.f : -new_max * scale2;
         run_max[b] = new_max;
         float tile_sum = 0.f;
 #pragma unroll
         for (int h = 0; h < 2; ++h)
 #pragma unroll
           for (int i = 0; i < 4; ++i) {
-            const float p = fast_exp2(sc[b][h][i] - shift);
+            const float p = fast_exp2(fmaf(sc[b][h][i], scale2, shift));
             tile_sum += p;
             pf[b][h * 4 + i] = (bf16)p;
           }
@@ -656,21 +675,27 @@ __global__ __launch_bounds__(256) void attention_prefill_bf16_kernel(
     };
     __syncthreads();                                           // the buffers of an earlier pass are done with
     fetch(first_tile, kreg_a, vreg_a);
-    if (first_tile < last_tile) fetch(first_tile + 1, kreg_b, vreg_b);
     stash(0, kreg_a, vreg_a);
     __syncthreads();
-    // invariant at the top of a turn: tile is in LDS buffer `buffer`, tile + 1 is on its way into set b
-    for (int tile = first_tile, buffer = 0; tile <= last_tile; tile += 2) {
-      if (tile + 2 <= last_tile) fetch(tile + 2, kreg_a, vreg_a);
-      work(tile, buffer);
-      if (tile + 1 <= last_tile) stash(buffer ^ 1, kreg_b, vreg_b);
-      __syncthreads();
-      if (tile + 1 > last_tile) break;
-      if (tile + 3 <= last_tile) fetch(tile + 3, kreg_b, vreg_b);
-      work(tile + 1, buffer ^ 1);
-      if (tile + 2 <= last_tile) stash(buffer, kreg_a, vreg_a);
-      __syncthreads();
-    }
+    // At the top of a turn `tile` is in LDS buffer (tile - first_tile) % 2; the next tile is asked
+    // for before the work on this one and put into the other buffer after it.  Three runs of tiles:
+    // those the last query's window cuts, those every query sees whole, those on the diagonal.
+    auto run = [&](int begin, int end, auto masked) {
+      for (int tile = begin; tile < end; ++tile) {
+        const int buffer = (tile - first_tile) & 1;
+        if (tile < last_tile) fetch(tile + 1, kreg_a, vreg_a);
+        work(tile, buffer, masked);
+        if (tile < last_tile) stash(buffer ^ 1, kreg_a, vreg_a);
+        __syncthreads();
+      }
+    };
+    int whole_begin = (lo_last + 31) / 32, whole_end = (pos_first + 1) / 32;   // tiles [whole_begin, whole_end) need no mask
+    if (whole_begin < first_tile) whole_begin = first_tile;
+    if (whole_end > last_tile + 1) whole_end = last_tile + 1;
+    if (whole_end < whole_begin) whole_end = whole_begin;
+    run(first_tile, whole_begin, std::true_type{});
+    run(whole_begin, whole_end, std::false_type{});
+    run(whole_end, last_tile + 1, std::true_type{});
 #pragma unroll
     for (int b = 0; b < QB; ++b) {
       float total = run_sum[b];
@@ -690,7 +715,19 @@ __global__ __launch_bounds__(256) void attention_prefill_bf16_kernel(
 }
 
 // Largest number of tokens in one query group of lrs_attention_prefill.
-LRS_API int lrs_attention_prefill_group() { return 64; }
+LRS_API int lrs_attention_prefill_group() { return 32; }
+
+// Compute units of the current device (asked once).
+static int compute_units() {
+  static int units = 0;
+  if (!units) {
+    int device = 0;
+    hipDeviceProp_t prop;
+    if (hipGetDevice(&device) == hipSuccess && hipGetDeviceProperties(&prop, device) == hipSuccess) units = prop.multiProcessorCount;
+    if (units <= 0) units = 256;
+  }
+  return units;
+}
 
 // Any step in bf16.  qblock_token0 / qblock_count [n_blocks]: first token and number of tokens
 // (1..lrs_attention_prefill_group()) of each group of consecutive tokens of one request.
@@ -700,16 +737,18 @@ LRS_API int lrs_attention_prefill(void* out, int out_stride, const void* q, int 
                                   const int* qblock_count, int n_blocks, int max_count, int max_context, int nq,
                                   int nkv, int d, int page_size, float scale, int window, void* stream) {
   LRS_REQUIRE(n_blocks > 0 && nq > 0 && nkv > 0 && nq % nkv == 0, "attention_prefill: bad sizes blocks=%d nq=%d nkv=%d", n_blocks, nq, nkv);
-  LRS_REQUIRE(max_count >= 1 && max_count <= 64, "attention_prefill: query groups hold 1..64 tokens, got %d", max_count);
+  LRS_REQUIRE(max_count >= 1 && max_count <= 32, "attention_prefill: query groups hold 1..32 tokens, got %d", max_count);
   LRS_REQUIRE(page_size % 16 == 0, "attention_prefill: page size %d is not a multiple of 16", page_size);
   LRS_REQUIRE(window >= 0, "attention_prefill: window must be >= 0 (0 = none)");
   LRS_REQUIRE(q_stride % 8 == 0 && ((uintptr_t)q % 16) == 0 && out_stride % 4 == 0 && ((uintptr_t)out % 8) == 0,
               "attention_prefill: q rows must be 16-byte and out rows 8-byte aligned");
   // always four waves: with fewer heads in a kv group the spare waves still help to bring tiles in
-  dim3 grid(n_blocks, nkv), block(4 * WAVE);
+  dim3 grid(n_blocks * nkv), block(4 * WAVE);
+  // workgroups that share a compute unit: see the kernel
+  const int chunk = nkv >= compute_units() ? nkv : compute_units() / nkv * nkv;
   // LDS copy of the block table entries a workgroup walks: at most those of the longest context
   LRS_REQUIRE(max_context >= 1, "attention_prefill: max_context must be the longest context length of the step");
-  const int span = window > 0 && window + 16 * 4 + 64 < max_context ? window + 16 * 4 + 64 : max_context;
+  const int span = window > 0 && window + 32 + 64 < max_context ? window + 32 + 64 : max_context;
   const size_t table_lds = sizeof(int) * (size_t)(span / page_size + 2);
   LRS_REQUIRE(table_lds <= 24 * 1024, "attention_prefill: a context of %d tokens needs more block table entries than fit LDS", max_context);
   hipStream_t s = (hipStream_t)stream;
@@ -717,11 +756,10 @@ LRS_API int lrs_attention_prefill(void* out, int out_stride, const void* q, int 
   attention_prefill_bf16_kernel<D, QB><<<grid, block, table_lds, s>>>((bf16*)out, out_stride, (const bf16*)q, q_stride, \
                                                               (const bf16*)k_pages, (const bf16*)v_pages, block_table, \
                                                               table_stride, token_request, positions, qblock_token0, \
-                                                              qblock_count, nq, nkv, page_size, scale, window)
+                                                              qblock_count, n_blocks, chunk, nq, nkv, page_size, scale, window)
 #define LAUNCH(D)                                \
   if (max_count <= 16) LAUNCH2(D, 1);            \
-  else if (max_count <= 32) LAUNCH2(D, 2);       \
-  else LAUNCH2(D, 4)
+  else LAUNCH2(D, 2)
   switch (d) {
     case 32: LAUNCH(32); break;
     case 64: LAUNCH(64); break;

@@ -126,7 +126,7 @@ class ModelRunner:
         self._off = {}
         cursor = 0
         # query groups for the ragged attention kernel: at most `query_group` consecutive tokens of one request
-        self.query_group = 64
+        self.query_group = ops.attention_prefill_group()
         self._max_qblocks = -(-t // 16) + r
         for name, size in (("token_ids", t), ("positions", t), ("token_request", t), ("logit_rows", t),
                            ("cu_seqlens_q", r + 1), ("seq_lens_k", r), ("slot_ids", r),

@@ -396,8 +396,8 @@ def test_attention_ragged_batch(ops, dtype, nq, nkv, d, page, window):
     torch.testing.assert_close(out.cpu().double(), want, **tol(dtype, 2e-5, 2e-2))
     if ops.attention_decode_supported(dtype, nq, nkv, d, page):
         # the matrix-core kernel for ragged steps: groups of consecutive tokens of one request, in any order
-        assert ops.attention_prefill_group() == 64
-        for size in (16, 7, 32, 64):
+        assert ops.attention_prefill_group() == 32
+        for size in (16, 7, 32, 25):
             blocks, at = [], 0
             for before, new in requests:
                 blocks += [(at + i, min(size, new - i)) for i in range(0, new, size)]
