@@ -506,7 +506,11 @@ __global__ __launch_bounds__(256, D <= 128 ? 2 : 1) void attention_prefill_bf16_
     const int* __restrict__ qblock_count, int n_blocks, int chunk, int nq, int nkv, int page_size, float scale,
     int window) {
   constexpr int DS = D / 32, DB = D / 16;
-  constexpr int KLD = D + 8, VLD = 32 + 8;                    // padded LDS rows
+  // Padded LDS rows (32 banks of 4 bytes).  Key rows are read 16 bytes a lane by 8 lanes a cycle: a
+  // stride of 4 banks more than a multiple of 32 spreads them over all banks.  Value rows are read
+  // 8 bytes a lane by 16 lanes a cycle: a stride of 18 banks (twice an odd number) does the same;
+  // such rows start at multiples of 8 bytes only, so they are written 8 bytes at a time.
+  constexpr int KLD = D + 8, VLD = 32 + 4;
   constexpr int KCHUNKS = 32 * D / 8, VCHUNKS = D * 4;        // 16-byte pieces of one tile
   constexpr int KPT = (KCHUNKS + 255) / 256, VPT = (VCHUNKS + 255) / 256;
   __shared__ __attribute__((aligned(16))) bf16 ks[2][32 * KLD];
@@ -572,7 +576,11 @@ __global__ __launch_bounds__(256, D <= 128 ? 2 : 1) void attention_prefill_bf16_
 #pragma unroll
     for (int i = 0; i < VPT; ++i) {
       const int idx = tid + i * threads;
-      if (idx < VCHUNKS) *(bf16x8*)(vs[buffer] + (idx / 4) * VLD + (idx % 4) * 8) = vreg[i];
+      if (idx < VCHUNKS) {
+        bf16* dst = vs[buffer] + (idx / 4) * VLD + (idx % 4) * 8;
+        *(bf16x4*)dst = bf16x4{vreg[i][0], vreg[i][1], vreg[i][2], vreg[i][3]};
+        *(bf16x4*)(dst + 4) = bf16x4{vreg[i][4], vreg[i][5], vreg[i][6], vreg[i][7]};
+      }
     }
   };
 
@@ -714,9 +722,6 @@ __global__ __launch_bounds__(256, D <= 128 ? 2 : 1) void attention_prefill_bf16_
   }
 }
 
-// Largest number of tokens in one query group of lrs_attention_prefill.
-LRS_API int lrs_attention_prefill_group() { return 32; }
-
 // Compute units of the current device (asked once).
 static int compute_units() {
   static int units = 0;
@@ -728,6 +733,14 @@ static int compute_units() {
   }
   return units;
 }
+
+// Largest number of tokens in one query group of lrs_attention_prefill.
+LRS_API int lrs_attention_prefill_group() { return 32; }
+
+// The group size that serves a step of `tokens` tokens best: groups of 16 while those of 32 would
+// not give every compute unit its two workgroups several times over (measured on MI355X: 16 is
+// faster up to 2,048 tokens, 32 beyond).
+LRS_API int lrs_attention_prefill_group_for(int tokens) { return tokens <= 8 * compute_units() ? 16 : 32; }
 
 // Any step in bf16.  qblock_token0 / qblock_count [n_blocks]: first token and number of tokens
 // (1..lrs_attention_prefill_group()) of each group of consecutive tokens of one request.

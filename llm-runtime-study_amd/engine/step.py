@@ -126,7 +126,7 @@ class ModelRunner:
         self._off = {}
         cursor = 0
         # query groups for the ragged attention kernel: at most `query_group` consecutive tokens of one request
-        self.query_group = ops.attention_prefill_group()
+        self.query_group = ops.attention_prefill_group()   # the most; a step of few tokens uses smaller ones
         self._max_qblocks = -(-t // 16) + r
         for name, size in (("token_ids", t), ("positions", t), ("token_request", t), ("logit_rows", t),
                            ("cu_seqlens_q", r + 1), ("seq_lens_k", r), ("slot_ids", r),
@@ -249,7 +249,7 @@ class ModelRunner:
             n_rows = cursor
         ctx.T, ctx.R, ctx.num_logit_rows = cursor, max(real, pad_to), n_rows
         # groups of consecutive tokens of one request, the longest contexts first
-        starts, size = cu[:ctx.R + 1], self.query_group
+        starts, size = cu[:ctx.R + 1], min(self.query_group, ops.attention_prefill_group(cursor))
         blocks = [(int(pos[min(t0 + size, int(starts[i + 1])) - 1]), t0, min(size, int(starts[i + 1]) - t0))
                   for i in range(ctx.R) for t0 in range(int(starts[i]), int(starts[i + 1]), size)]
         blocks.sort(key=lambda b: -b[0])

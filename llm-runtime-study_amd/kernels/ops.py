@@ -56,6 +56,7 @@ _SIGNATURES = {
     "lrs_attention_prefill": (c_int, [c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p,
                                       c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_void_p]),
     "lrs_attention_prefill_group": (c_int, []),
+    "lrs_attention_prefill_group_for": (c_int, [c_int]),
     "lrs_choose_tokens": (c_int, [c_void_p, c_void_p, c_int64, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p]),
     "lrs_choose_tokens_split": (c_int, [c_void_p, c_void_p, c_int64, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p]),
     "lrs_filter_logits": (c_int, [c_void_p, c_int64, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p]),
@@ -495,9 +496,12 @@ def attention_prefill(out: torch.Tensor, q: torch.Tensor, k_pages: torch.Tensor,
         block_table.shape[1] * page_size if max_context is None else max_context, nq, nkv, d, page_size, scale, window, _stream()))
 
 
-def attention_prefill_group() -> int:
-    """Most tokens in one query group of attention_prefill()."""
-    return library().lrs_attention_prefill_group()
+def attention_prefill_group(tokens: int | None = None) -> int:
+    """Most tokens in one query group of attention_prefill(); with `tokens`, the group size that
+    serves a step of that many tokens best (smaller groups fill the chip when there are few)."""
+    if tokens is None:
+        return library().lrs_attention_prefill_group()
+    return library().lrs_attention_prefill_group_for(tokens)
 
 
 # --------------------------------------------------------------- sampling
