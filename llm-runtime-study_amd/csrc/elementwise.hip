@@ -29,18 +29,24 @@ LRS_API int lrs_embed(float* out, const void* table, int dtype, const int* ids, 
 
 // -------------------------------------------------------------------- RMSNorm
 // y = w * x * rsqrt(mean(x^2) + eps); x is a float32 row (optionally picked through `rows`),
-// the result is rounded once to the output dtype.
+// the result is rounded once to the output dtype.  With `add` (bf16 [rows, hidden], no row
+// picking) the row is first updated in place, x += add, and the norm is taken of the sum: the
+// residual add after a library matrix product and the norm that follows it in one pass.
 template <typename TW, typename TO>
-__global__ void rmsnorm_kernel(TO* __restrict__ out, const float* __restrict__ x,
+__global__ void rmsnorm_kernel(TO* __restrict__ out, float* __restrict__ x, const bf16* __restrict__ add,
                                const TW* __restrict__ weight, const int* __restrict__ rows,
                                int hidden, float eps) {
   __shared__ float scratch[16];
   const int64_t src_row = rows ? rows[blockIdx.x] : blockIdx.x;
-  const float* src = x + src_row * hidden;
+  float* src = x + src_row * hidden;
   TO* dst = out + (int64_t)blockIdx.x * hidden;
   float ss = 0.f;
   for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
-    const float v = src[i];
+    float v = src[i];
+    if (add) {
+      v += (float)add[src_row * hidden + i];
+      src[i] = v;                                   // read again below by the same thread only
+    }
     ss += v * v;
   }
   ss = block_sum(ss, scratch);
@@ -52,12 +58,12 @@ __global__ void rmsnorm_kernel(TO* __restrict__ out, const float* __restrict__ x
 // The same with the row held in registers: every thread owns up to VEC chunks of 4 values, read
 // once with 16-byte loads; for hidden % 4 == 0 and hidden <= 4 * VEC * threads.
 template <typename TW, typename TO, int VEC>
-__global__ void rmsnorm_vec_kernel(TO* __restrict__ out, const float* __restrict__ x,
+__global__ void rmsnorm_vec_kernel(TO* __restrict__ out, float* __restrict__ x, const bf16* __restrict__ add,
                                    const TW* __restrict__ weight, const int* __restrict__ rows,
                                    int hidden, float eps) {
   __shared__ float scratch[16];
   const int64_t src_row = rows ? rows[blockIdx.x] : blockIdx.x;
-  const floatx4* src = (const floatx4*)(x + src_row * hidden);
+  floatx4* src = (floatx4*)(x + src_row * hidden);
   const int chunks = hidden / 4;
   floatx4 v[VEC], w[VEC];
   float ss = 0.f;
@@ -66,6 +72,12 @@ __global__ void rmsnorm_vec_kernel(TO* __restrict__ out, const float* __restrict
     const int c = threadIdx.x + j * blockDim.x;
     if (c < chunks) {
       v[j] = src[c];
+      if (add) {
+        const bf16x4 y = *(const bf16x4*)(add + src_row * hidden + c * 4);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) v[j][i] += (float)y[i];
+        src[c] = v[j];
+      }
 #pragma unroll
       for (int i = 0; i < 4; ++i) w[j][i] = to_float(weight[c * 4 + i]);
       ss += v[j][0] * v[j][0] + v[j][1] * v[j][1] + v[j][2] * v[j][2] + v[j][3] * v[j][3];
@@ -84,16 +96,17 @@ __global__ void rmsnorm_vec_kernel(TO* __restrict__ out, const float* __restrict
   }
 }
 
-LRS_API int lrs_rmsnorm(void* out, int out_dtype, const float* x, const void* weight, int w_dtype,
-                        const int* rows, int n_rows, int hidden, float eps, void* stream) {
+static int launch_rmsnorm(void* out, int out_dtype, float* x, const bf16* add, const void* weight, int w_dtype,
+                          const int* rows, int n_rows, int hidden, float eps, void* stream) {
   LRS_REQUIRE(n_rows > 0 && hidden > 0, "rmsnorm: rows=%d hidden=%d must be positive", n_rows, hidden);
   LRS_REQUIRE(eps > 0.f, "rmsnorm: eps must be positive");
+  LRS_REQUIRE(add == nullptr || rows == nullptr, "rmsnorm: the fused residual add takes all rows in order");
   dim3 grid(n_rows), block(hidden >= 2048 ? 512 : 256);
   hipStream_t s = (hipStream_t)stream;
-  if (hidden % 4 == 0 && hidden <= 4 * 4 * 512 && ((uintptr_t)x % 16) == 0) {
+  if (hidden % 4 == 0 && hidden <= 4 * 4 * 512 && ((uintptr_t)x % 16) == 0 && ((uintptr_t)add % 8) == 0) {
     const int threads = hidden <= 1024 ? 64 : (hidden <= 4096 ? 256 : 512);
 #define LAUNCH_VEC(TW, TO) \
-  rmsnorm_vec_kernel<TW, TO, 4><<<grid, threads, 0, s>>>((TO*)out, x, (const TW*)weight, rows, hidden, eps)
+  rmsnorm_vec_kernel<TW, TO, 4><<<grid, threads, 0, s>>>((TO*)out, x, add, (const TW*)weight, rows, hidden, eps)
     if (w_dtype == LRS_F32 && out_dtype == LRS_F32) LAUNCH_VEC(float, float);
     else if (w_dtype == LRS_BF16 && out_dtype == LRS_BF16) LAUNCH_VEC(bf16, bf16);
     else if (w_dtype == LRS_F32 && out_dtype == LRS_BF16) LAUNCH_VEC(float, bf16);
@@ -103,7 +116,7 @@ LRS_API int lrs_rmsnorm(void* out, int out_dtype, const float* x, const void* we
     return lrs_check_launch("rmsnorm");
   }
 #define LAUNCH(TW, TO) \
-  rmsnorm_kernel<TW, TO><<<grid, block, 0, s>>>((TO*)out, x, (const TW*)weight, rows, hidden, eps)
+  rmsnorm_kernel<TW, TO><<<grid, block, 0, s>>>((TO*)out, x, add, (const TW*)weight, rows, hidden, eps)
   if (w_dtype == LRS_F32 && out_dtype == LRS_F32) LAUNCH(float, float);
   else if (w_dtype == LRS_BF16 && out_dtype == LRS_BF16) LAUNCH(bf16, bf16);
   else if (w_dtype == LRS_F32 && out_dtype == LRS_BF16) LAUNCH(float, bf16);
@@ -111,6 +124,18 @@ LRS_API int lrs_rmsnorm(void* out, int out_dtype, const float* x, const void* we
   else return lrs_fail("rmsnorm: unknown dtypes %d/%d", w_dtype, out_dtype);
 #undef LAUNCH
   return lrs_check_launch("rmsnorm");
+}
+
+LRS_API int lrs_rmsnorm(void* out, int out_dtype, const float* x, const void* weight, int w_dtype,
+                        const int* rows, int n_rows, int hidden, float eps, void* stream) {
+  return launch_rmsnorm(out, out_dtype, (float*)x, nullptr, weight, w_dtype, rows, n_rows, hidden, eps, stream);
+}
+
+// x [n_rows, hidden] float32 += y (bf16), then out = RMSNorm(x): see rmsnorm_kernel.
+LRS_API int lrs_add_rmsnorm(void* out, int out_dtype, float* x, const void* y, const void* weight, int w_dtype,
+                            int n_rows, int hidden, float eps, void* stream) {
+  LRS_REQUIRE(y != nullptr, "add_rmsnorm: nothing to add");
+  return launch_rmsnorm(out, out_dtype, x, (const bf16*)y, weight, w_dtype, nullptr, n_rows, hidden, eps, stream);
 }
 
 // ------------------------------------------------------------- rotary tables
@@ -147,6 +172,7 @@ __global__ void qk_prep_kernel(T* __restrict__ qkv, int row_stride, int nq, int 
                                const float* __restrict__ sinv, int rot_half,
                                T* __restrict__ k_pages, T* __restrict__ v_pages,
                                const int* __restrict__ slots, int page_size) {
+  // v_pages == null: the values are stored by values_to_pages_kernel instead
   const int token = blockIdx.x, head = blockIdx.y, lane = threadIdx.x;
   T* src = qkv + (int64_t)token * row_stride + (int64_t)head * d;
   const bool is_q = head < nq, is_k = !is_q && head < nq + nkv;
@@ -157,6 +183,7 @@ __global__ void qk_prep_kernel(T* __restrict__ qkv, int row_stride, int nq, int 
     const int kv_head = is_k ? head - nq : head - nq - nkv;
     const int64_t page = slot / page_size, off = slot % page_size;
     if (!is_k) {
+      if (!v_pages) return;
       T* vdst = v_pages + (page * nkv + kv_head) * d * page_size + off;
       for (int i = lane; i < d; i += WAVE) vdst[(int64_t)i * page_size] = src[i];
       return;
@@ -220,6 +247,7 @@ __global__ __launch_bounds__(256) void qk_prep_vec_kernel(T* __restrict__ qkv, i
     page = slot / page_size;
     off = slot % page_size;
     if (!is_k) {
+      if (!v_pages) return;
       T* vdst = v_pages + (page * nkv + kv_head) * d * page_size + off;
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
@@ -265,6 +293,53 @@ __global__ __launch_bounds__(256) void qk_prep_vec_kernel(T* __restrict__ qkv, i
   *(vec4*)(dst + half + 4 * j) = out_hi;
 }
 
+// The v heads of 16 consecutive tokens of the step and one kv head, through LDS into the value
+// pages [page, kv_head, dim, slot]: tokens that follow each other in one page land side by side,
+// so a thread writes the values of 16 / sizeof(T) such tokens for one dim with one 16-byte store
+// (and falls back to single stores where a run is broken by a page edge, another request or a
+// slot that is not to be stored).  For steps of many tokens: storing token by token scatters
+// 2-byte writes a page row apart.
+template <typename T>
+__global__ __launch_bounds__(256) void values_to_pages_kernel(const T* __restrict__ qkv, int row_stride, int v_offset,
+                                                              int tokens, int nkv, int d, T* __restrict__ v_pages,
+                                                              const int* __restrict__ slots, int page_size) {
+  constexpr int RUN = 16 / sizeof(T);
+  typedef T vec __attribute__((ext_vector_type(RUN)));
+  extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
+  T* tile = (T*)lds_raw;                            // [d][17]
+  __shared__ int slot_of[16];
+  const int token0 = blockIdx.x * 16, kvh = blockIdx.y, tid = threadIdx.x;
+  const int count = tokens - token0 < 16 ? tokens - token0 : 16;
+  if (tid < 16) slot_of[tid] = tid < count ? slots[token0 + tid] : -1;
+  for (int e = tid; e < 16 * d; e += 256) {
+    const int i = e / d, dim = e % d;
+    if (i < count) tile[dim * 17 + i] = qkv[(int64_t)(token0 + i) * row_stride + v_offset + (int64_t)kvh * d + dim];
+  }
+  __syncthreads();
+  for (int e = tid; e < d * (16 / RUN); e += 256) {
+    const int dim = e / (16 / RUN), first = (e % (16 / RUN)) * RUN;
+    const int slot0 = slot_of[first];
+    bool run = slot0 >= 0 && slot0 % RUN == 0 && slot0 % page_size + RUN <= page_size;
+#pragma unroll
+    for (int i = 1; i < RUN; ++i) run = run && slot_of[first + i] == slot0 + i;
+    if (run) {
+      vec v;
+#pragma unroll
+      for (int i = 0; i < RUN; ++i) v[i] = tile[dim * 17 + first + i];
+      const int64_t page = slot0 / page_size, off = slot0 % page_size;
+      *(vec*)(v_pages + ((page * nkv + kvh) * d + dim) * page_size + off) = v;
+    } else {
+#pragma unroll
+      for (int i = 0; i < RUN; ++i) {
+        const int slot = slot_of[first + i];
+        if (slot < 0) continue;
+        const int64_t page = slot / page_size, off = slot % page_size;
+        v_pages[((page * nkv + kvh) * d + dim) * page_size + off] = tile[dim * 17 + first + i];
+      }
+    }
+  }
+}
+
 LRS_API int lrs_qk_prep(void* qkv, int dtype, int tokens, int row_stride, int nq, int nkv, int d,
                         const void* q_weight, const void* k_weight, int w_dtype, float eps,
                         const float* cosv, const float* sinv, int rot_half, void* k_pages,
@@ -277,12 +352,30 @@ LRS_API int lrs_qk_prep(void* qkv, int dtype, int tokens, int row_stride, int nq
   LRS_REQUIRE(row_stride >= (nq + 2 * nkv) * d, "qk_prep: row stride %d too small", row_stride);
   dim3 grid(tokens, nq + 2 * nkv), block(WAVE);
   hipStream_t s = (hipStream_t)stream;
+  // many tokens: the values go through a kernel of their own that writes whole runs of slots
+  const size_t elem = dtype == LRS_F32 ? 4 : 2;
+  const bool values_apart = nkv > 0 && tokens >= 128 && page_size % (16 / elem) == 0 && ((uintptr_t)v_pages % 16) == 0 &&
+                            (size_t)d * 17 * elem <= 48 * 1024;
+  if (values_apart) {
+    dim3 vgrid((tokens + 15) / 16, nkv);
+    const size_t lds = (size_t)d * 17 * elem;
+    if (dtype == LRS_F32)
+      values_to_pages_kernel<float><<<vgrid, 256, lds, s>>>((const float*)qkv, row_stride, (nq + nkv) * d, tokens, nkv, d, (float*)v_pages, slots, page_size);
+    else if (dtype == LRS_BF16)
+      values_to_pages_kernel<bf16><<<vgrid, 256, lds, s>>>((const bf16*)qkv, row_stride, (nq + nkv) * d, tokens, nkv, d, (bf16*)v_pages, slots, page_size);
+    else
+      return lrs_fail("qk_prep: unknown dtype %d", dtype);
+    if (lrs_check_launch("values_to_pages")) return 1;
+    v_pages = nullptr;
+  }
+  const int heads = nq + (values_apart ? nkv : 2 * nkv);    // heads the kernels below have work for
+  grid.y = heads;
   const int per_head = d / 8;
   const bool vectors = d % 8 == 0 && per_head <= 64 && (per_head & (per_head - 1)) == 0 && (rot_half == 0 || 2 * rot_half == d) &&
                        row_stride % 4 == 0 && ((uintptr_t)qkv % 16) == 0 && ((uintptr_t)k_pages % 16) == 0;
   if (vectors) {
     const int heads_per_block = 256 / per_head;
-    dim3 vgrid(tokens, (nq + 2 * nkv + heads_per_block - 1) / heads_per_block);
+    dim3 vgrid(tokens, (heads + heads_per_block - 1) / heads_per_block);
 #define LAUNCH_VEC(T, TW)                                                                              \
   qk_prep_vec_kernel<T, TW><<<vgrid, 256, 0, s>>>((T*)qkv, row_stride, nq, nkv, d, (const TW*)q_weight,  \
                                                   (const TW*)k_weight, eps, cosv, sinv, rot_half,      \

@@ -32,6 +32,7 @@ _SIGNATURES = {
     "lrs_copy_h2d": (c_int, [c_void_p, c_void_p, c_int64, c_void_p]),
     "lrs_embed": (c_int, [c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_float, c_void_p]),
     "lrs_rmsnorm": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_float, c_void_p]),
+    "lrs_add_rmsnorm": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_float, c_void_p]),
     "lrs_rope_table": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p]),
     "lrs_qk_prep": (c_int, [c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_int, c_float,
                             c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p]),
@@ -174,6 +175,17 @@ def rmsnorm(out: torch.Tensor, x: torch.Tensor, weight: torch.Tensor, eps: float
         _need(rows.dtype == torch.int32 and rows.numel() >= n_rows and rows.is_contiguous(), "rmsnorm: rows must be int32")
     _check(library().lrs_rmsnorm(_dev(out, "out"), dtype_code(out.dtype), _dev(x, "x", torch.float32), _dev(weight, "weight"),
                                  dtype_code(weight.dtype), None if rows is None else _dev(rows, "rows"), n_rows, hidden, eps, _stream()))
+
+
+def add_rmsnorm(out: torch.Tensor, x: torch.Tensor, y: torch.Tensor, weight: torch.Tensor, eps: float) -> None:
+    """x += y (float32 residual stream, bf16 addend), then out = RMSNorm(x) with `weight`, in one pass."""
+    n_rows, hidden = x.shape
+    _need(x.dtype == torch.float32 and x.is_contiguous() and y.dtype == torch.bfloat16 and y.is_contiguous() and y.shape == x.shape,
+          "add_rmsnorm: x must be contiguous float32 [T, H] and y bf16 of the same shape")
+    _need(out.is_contiguous() and out.shape == x.shape, "add_rmsnorm: out must be contiguous [T, H]")
+    _need(weight.is_contiguous() and weight.numel() == hidden, f"add_rmsnorm: weight must hold {hidden} values")
+    _check(library().lrs_add_rmsnorm(_dev(out, "out"), dtype_code(out.dtype), _dev(x, "x"), _dev(y, "y"), _dev(weight, "weight"),
+                                     dtype_code(weight.dtype), n_rows, hidden, eps, _stream()))
 
 
 def rope_table(cos: torch.Tensor, sin: torch.Tensor, positions: torch.Tensor, inv_freq: torch.Tensor) -> None:

@@ -81,8 +81,9 @@ def linear(ctx, out, x, weight, bias=None, accumulate: bool = False, swiglu: boo
     """out = x @ weight.T (+ bias), x a tensor, a LazyNorm or ScaledRows.
 
     then_norm: the norm part that will be applied to `out` next (only meaningful with
-    `accumulate`).  Returns ScaledRows if the kernel began that norm, else None: the caller
-    then runs the norm as usual.
+    `accumulate`).  Returns that norm of the updated `out` if it was computed on the way, as
+    ScaledRows (begun by the few-rows kernel, finished by the next `linear()`) or as a plain
+    tensor (after a library product); else None: the caller then runs the norm as usual.
 
     Products of many rows in bfloat16 go to the vendor's matrix library (as the reference's
     nn.Linear does) when the step allows it (`ctx.library_gemm`); its result then reaches the
@@ -115,6 +116,13 @@ def linear(ctx, out, x, weight, bias=None, accumulate: bool = False, swiglu: boo
             y = ctx.scratch("library_gemm_out", (m, n), torch.bfloat16)
             torch.mm(x, weight.t(), out=y)
             if accumulate:
+                parameters = getattr(then_norm, "rms_parameters", None)
+                if parameters is not None and out.is_contiguous() and parameters()[0].numel() == n:
+                    # the residual add and the norm that follows it in one pass over the rows
+                    norm_weight, eps = parameters()
+                    normed = ctx.scratch("norm_after_add", (m, n), ctx.dtype)
+                    ops.add_rmsnorm(normed, out, y, norm_weight, eps)
+                    return normed
                 ops.add_into(out, y)
             else:
                 ops.silu_mul(out, y, interleaved=True)

@@ -74,6 +74,24 @@ def test_rmsnorm(ops, out_dtype, w_dtype, rows, hidden, eps):
     torch.testing.assert_close(out.cpu().float(), want[pick.long()], **tol(out_dtype, 2e-6, 1e-2))
 
 
+@pytest.mark.parametrize("out_dtype", DTYPES)
+@pytest.mark.parametrize("rows,hidden,eps", [(1, 64, 1e-6), (33, 96, 1e-5), (300, 4096, 1e-6), (2, 5120 + 16, 1e-3), (3, 9000, 1e-5), (4, 50, 1e-5)])
+def test_add_rmsnorm(ops, out_dtype, rows, hidden, eps):
+    """The residual add and the norm after it in one kernel: the stream is updated in place and
+    the norm is that of the updated rows."""
+    g = torch.Generator().manual_seed(rows + hidden)
+    x = torch.randn(rows, hidden, generator=g) * 3
+    y = torch.randn(rows, hidden, generator=g).bfloat16()
+    w = (1 + 0.2 * torch.randn(hidden, generator=g)).bfloat16()
+    stream = dev(x.clone())
+    out = torch.empty(rows, hidden, device="cuda", dtype=out_dtype)
+    ops.add_rmsnorm(out, stream, dev(y), dev(w), eps)
+    want_stream = x + y.float()
+    torch.testing.assert_close(stream.cpu(), want_stream, rtol=0, atol=0)
+    want = w.float() * want_stream * torch.rsqrt(want_stream.pow(2).mean(-1, keepdim=True) + eps)
+    torch.testing.assert_close(out.cpu().float(), want, **tol(out_dtype, 1e-5, 1e-2))
+
+
 @pytest.mark.parametrize("half,theta", [(8, 1e4), (16, 1e6), (64, 1e6), (24, 5e5)])
 def test_rope_table(ops, half, theta):
     positions = torch.tensor([0, 1, 2, 17, 511, 4095, 40959], dtype=torch.int32)
@@ -111,21 +129,33 @@ def _qk_prep_reference(qkv, nq, nkv, d, qw, kw, eps, positions, inv, rot_half):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("layout", ["scattered", "runs"])
 @pytest.mark.parametrize("nq,nkv,d,rot,normed,page", [
     (4, 2, 16, 16, True, 4), (8, 2, 32, 32, True, 16), (3, 3, 48, 32, False, 8),
     (32, 8, 128, 128, True, 16), (5, 1, 80, 0, True, 16), (6, 2, 256, 256, True, 64),
 ])
-def test_qk_prep(ops, dtype, nq, nkv, d, rot, normed, page):
+def test_qk_prep(ops, dtype, layout, nq, nkv, d, rot, normed, page):
+    """A few tokens with slots anywhere; and a step of many tokens (which stores the values through
+    a kernel of its own) whose requests occupy runs of slots that start and end inside pages."""
     g = torch.Generator().manual_seed(2)
-    t, pages = 19, 12
+    if layout == "scattered":
+        t, pages = 19, 12
+        slots = torch.randperm(pages * page, generator=g)[:t].to(torch.int32)
+    else:
+        runs, at, pieces = [1, 7, 16, 33, 64, 100, 79, 5], 3, []
+        for n in runs:                                   # each request starts somewhere inside a fresh page
+            pieces.append(torch.arange(at, at + n))
+            at = -(-(at + n) // page) * page + page + int(torch.randint(0, page, (1,), generator=g))
+        order = torch.randperm(len(pieces), generator=g).tolist()
+        slots = torch.cat([pieces[i] for i in order]).to(torch.int32)
+        t, pages = slots.numel(), -(-at // page) + 1
+    slots[3] = -1  # a token that must not be stored
     qkv = torch.randn(t, (nq + 2 * nkv) * d, generator=g).to(dtype)
     qw = (1 + 0.1 * torch.randn(d, generator=g)).to(dtype) if normed else None
     kw = (1 + 0.1 * torch.randn(d, generator=g)).to(dtype) if normed else None
     positions = torch.randint(0, 3000, (t,), generator=g, dtype=torch.int32)
     rot_half = rot // 2
     inv = 1.0 / (1e4 ** (torch.arange(0, rot, 2, dtype=torch.float32) / max(rot, 1)))
-    slots = torch.randperm(pages * page, generator=g)[:t].to(torch.int32)
-    slots[3] = -1  # a token that must not be stored
     want_q, want_k, want_v = _qk_prep_reference(qkv, nq, nkv, d, qw, kw, 1e-6, positions, inv, rot_half)
 
     d_qkv = dev(qkv)
