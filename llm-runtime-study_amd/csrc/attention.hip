@@ -394,6 +394,9 @@ __global__ __launch_bounds__(256) void attention_decode_bf16_kernel(
 }
 
 // Merges the partial results of the splits of one (token, head): out = sum_s o_s 2^(m_s - m) / sum_s l_s 2^(m_s - m).
+// A kernel of its own on purpose: letting the last workgroup to finish merge inside the decode
+// kernel needs a device-wide fence in every workgroup, and on this chip (eight L2s) those fences
+// write back and invalidate whole caches; measured, they cost many times what this kernel does.
 __global__ void attention_merge_kernel(bf16* __restrict__ out, int out_stride, const float* __restrict__ part_o,
                                        const float* __restrict__ part_ml, int nq, int d, int splits) {
   const int token = blockIdx.x, head = blockIdx.y;

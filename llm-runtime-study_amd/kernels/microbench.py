@@ -1,0 +1,139 @@
+"""Timings of single kernels at the shapes of a model, outside any model.
+
+    python -m llm_runtime_study_amd.kernels.microbench attention_prefill --tokens 2048,8192 --group 16,32
+    python -m llm_runtime_study_amd.kernels.microbench attention_decode --batch 1,8,64 --context 2048 --splits 1,4,8
+    python -m llm_runtime_study_amd.kernels.microbench gemm --rows 1,8,16,64,2048
+
+Head and matrix shapes default to those of Qwen3-8B and can be changed with options.  Weights and
+caches larger than the last-level cache are rotated between calls where a kernel streams them once
+(decode attention, products of few rows), so that a timing is one of reads from memory.  Prints one
+line per case; the profiler attaches to this program like to any other.
+"""
+
+from __future__ import annotations
+
+import argparse
+import math
+import sys
+
+import torch
+
+from . import ops
+
+
+def _ints(text: str) -> list[int]:
+    return [int(part) for part in text.split(",") if part]
+
+
+def _time(call, repeats: int) -> float:
+    """Seconds per call of `call(i)`, measured over `repeats` calls after three warm-up calls."""
+    for i in range(3):
+        call(i)
+    torch.cuda.synchronize()
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    start.record()
+    for i in range(repeats):
+        call(i)
+    stop.record()
+    torch.cuda.synchronize()
+    return start.elapsed_time(stop) / repeats * 1e-3
+
+
+def attention_prefill(args) -> None:
+    """One request's whole prompt: `tokens` queries over their own causal context."""
+    nq, nkv, d, page = args.heads, args.kv_heads, args.head_dim, args.page_size
+    for tokens in _ints(args.tokens):
+        pages = -(-tokens // page)
+        k_pages = torch.randn(pages + 1, nkv, page, d, device="cuda", dtype=torch.bfloat16)
+        v_pages = torch.randn(pages + 1, nkv, d, page, device="cuda", dtype=torch.bfloat16)
+        table = torch.randperm(pages, device="cuda").to(torch.int32).view(1, -1)
+        q = torch.randn(tokens, (nq + 2 * nkv) * d, device="cuda", dtype=torch.bfloat16)
+        out = torch.empty(tokens, nq * d, device="cuda", dtype=torch.bfloat16)
+        request = torch.zeros(tokens, dtype=torch.int32, device="cuda")
+        positions = torch.arange(tokens, dtype=torch.int32, device="cuda")
+        flops = 4 * (tokens * (tokens + 1) / 2) * nq * d
+        groups = _ints(args.group) if args.group else [ops.attention_prefill_group(tokens)]
+        for size in groups:
+            starts = list(range(0, tokens, size))[::-1]          # longest contexts first, as the engine orders them
+            token0 = torch.tensor(starts, dtype=torch.int32, device="cuda")
+            count = torch.tensor([min(size, tokens - s) for s in starts], dtype=torch.int32, device="cuda")
+            seconds = _time(lambda i: ops.attention_prefill(out, q, k_pages, v_pages, table, request, positions, token0, count,
+                                                            nq, 1 / math.sqrt(d), args.window, size, tokens), args.repeats)
+            print(f"attention_prefill tokens={tokens} group={size}: {seconds * 1e6:9.1f} us  {flops / seconds / 1e12:7.1f} TFLOP/s (causal half)", flush=True)
+
+
+def attention_decode(args) -> None:
+    """One query token per request over `context` cached tokens."""
+    nq, nkv, d, page, context = args.heads, args.kv_heads, args.head_dim, args.page_size, args.context
+    for batch in _ints(args.batch):
+        pages = batch * (context // page + 1)
+        cache_bytes = batch * context * nkv * d * 2 * 2
+        sets = max(1, min(8, int(3e9 / (pages * nkv * page * d * 2 * 2))))
+        caches = [(torch.randn(pages + 1, nkv, page, d, device="cuda", dtype=torch.bfloat16),
+                   torch.randn(pages + 1, nkv, d, page, device="cuda", dtype=torch.bfloat16)) for _ in range(sets)]
+        table = torch.randperm(pages, device="cuda").to(torch.int32).view(batch, -1)
+        q = torch.randn(batch, (nq + 2 * nkv) * d, device="cuda", dtype=torch.bfloat16)
+        out = torch.empty(batch, nq * d, device="cuda", dtype=torch.bfloat16)
+        request = torch.arange(batch, dtype=torch.int32, device="cuda")
+        positions = torch.full((batch,), context - 1, dtype=torch.int32, device="cuda")
+        for splits in _ints(args.splits):
+            part_o = torch.empty(batch, nq * splits * d, device="cuda")
+            part_ml = torch.empty(batch, nq * splits * 2, device="cuda")
+            seconds = _time(lambda i: ops.attention_decode(out, q, caches[i % sets][0], caches[i % sets][1], table, request, positions,
+                                                           nq, 1 / math.sqrt(d), args.window, splits, part_o, part_ml, context), args.repeats)
+            print(f"attention_decode batch={batch} context={context} splits={splits}: {seconds * 1e6:8.1f} us  "
+                  f"{cache_bytes / seconds / 1e9:7.0f} GB/s of cache", flush=True)
+
+
+def gemm(args) -> None:
+    """x [rows, K] times W[N, K]^T for the products of one layer: this package's kernel and torch.mm."""
+    hidden, inter = args.hidden_size, args.intermediate_size
+    qkv = (args.heads + 2 * args.kv_heads) * args.head_dim
+    shapes = [("qkv", qkv, hidden), ("o", hidden, args.heads * args.head_dim), ("gate_up", 2 * inter, hidden), ("down", hidden, inter)]
+    before = ops.skinny_max_m()
+    ops.set_skinny_max_m(64)            # time the few-rows kernel up to its own limit, not the caller's
+    try:
+        for name, n, k in shapes:
+            sets = max(2, min(16, int(1.2e9 / (n * k * 2))))
+            weights = [torch.randn(n, k, device="cuda", dtype=torch.bfloat16) for _ in range(sets)]
+            for rows in _ints(args.rows):
+                x = torch.randn(rows, k, device="cuda", dtype=torch.bfloat16)
+                out = torch.empty(rows, n, device="cuda", dtype=torch.bfloat16)
+                for which, call in (("own", lambda i: ops.gemm(out, x, weights[i % sets])),
+                                    ("library", lambda i: torch.mm(x, weights[i % sets].t(), out=out))):
+                    seconds = _time(call, max(args.repeats, 2 * sets))
+                    print(f"gemm {name:8s} rows={rows:5d} {which:8s} {seconds * 1e6:9.1f} us  {n * k * 2 / seconds / 1e9:8.0f} GB/s of weights  "
+                          f"{2 * rows * n * k / seconds / 1e12:8.1f} TFLOP/s", flush=True)
+            del weights
+    finally:
+        ops.set_skinny_max_m(before)
+
+
+def main(argv=None) -> int:
+    parser = argparse.ArgumentParser(prog="python -m llm_runtime_study_amd.kernels.microbench", description=__doc__.split("\n\n")[0])
+    parser.add_argument("kernel", choices=["attention_prefill", "attention_decode", "gemm"])
+    parser.add_argument("--heads", type=int, default=32)
+    parser.add_argument("--kv-heads", type=int, default=8)
+    parser.add_argument("--head-dim", type=int, default=128)
+    parser.add_argument("--hidden-size", type=int, default=4096)
+    parser.add_argument("--intermediate-size", type=int, default=12288)
+    parser.add_argument("--page-size", type=int, default=16)
+    parser.add_argument("--window", type=int, default=0)
+    parser.add_argument("--tokens", default="2048", help="attention_prefill: prompt lengths, comma separated")
+    parser.add_argument("--group", default="", help="attention_prefill: query group sizes (default: what the engine would choose)")
+    parser.add_argument("--batch", default="1,8,64", help="attention_decode: batch sizes")
+    parser.add_argument("--context", type=int, default=2048, help="attention_decode: cached tokens per request")
+    parser.add_argument("--splits", default="1,2,4,8,16", help="attention_decode: workgroups per (token, kv head)")
+    parser.add_argument("--rows", default="1,8,16,64,2048", help="gemm: numbers of rows")
+    parser.add_argument("--repeats", type=int, default=20)
+    args = parser.parse_args(argv)
+    if not torch.cuda.is_available():
+        print("microbench needs the GPU", file=sys.stderr)
+        return 2
+    ops.library()
+    {"attention_prefill": attention_prefill, "attention_decode": attention_decode, "gemm": gemm}[args.kernel](args)
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())
