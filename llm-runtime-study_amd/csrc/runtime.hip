@@ -64,9 +64,49 @@ LRS_API int lrs_graph_destroy(void* exec) {
   return 0;
 }
 
-// Asynchronous copy of step metadata from pinned host memory to the device.
+// The address under which kernels see pinned host memory (hipHostMalloc): results of a few bytes
+// (the chosen tokens) are written there directly, which spares a copy back and its latency.
+LRS_API int lrs_host_device_pointer(void* host, void** device) {
+  hipError_t err = hipHostGetDevicePointer(device, host, 0);
+  if (err != hipSuccess) return lrs_fail("hipHostGetDevicePointer: %s (is the memory pinned?)", hipGetErrorString(err));
+  return 0;
+}
+
+// Asynchronous copy of step metadata from pinned host memory to the device.  Small copies (a decode
+// step's few KB) are done by a kernel that reads the pinned memory through its device address:
+// launching it costs the host a fraction of what the runtime's copy path does, and it orders with
+// the step's kernels like any other.  `src` must be pinned (hipHostMalloc) memory.
+__global__ void copy_from_host_kernel(int4* __restrict__ dst, const int4* __restrict__ src, int64_t chunks) {
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < chunks; i += (int64_t)gridDim.x * blockDim.x) dst[i] = src[i];
+}
+
 LRS_API int lrs_copy_h2d(void* dst, const void* src, int64_t bytes, void* stream) {
-  hipError_t err = hipMemcpyAsync(dst, src, (size_t)bytes, hipMemcpyHostToDevice, (hipStream_t)stream);
+  hipStream_t s = (hipStream_t)stream;
+  if (bytes <= (256 << 10) && bytes % 16 == 0 && (uintptr_t)dst % 16 == 0 && (uintptr_t)src % 16 == 0) {
+    // device addresses of the (few) pinned buffers seen so far
+    static const void* known_host[8];
+    static void* known_device[8];
+    static int known = 0;
+    void* device_src = nullptr;
+    for (int i = 0; i < known; ++i)
+      if (known_host[i] == src) device_src = known_device[i];
+    if (!device_src) {
+      if (hipHostGetDevicePointer(&device_src, const_cast<void*>(src), 0) != hipSuccess) {
+        (void)hipGetLastError();
+        device_src = nullptr;
+      } else if (known < 8) {
+        known_host[known] = src;
+        known_device[known++] = device_src;
+      }
+    }
+    if (device_src) {
+      const int64_t chunks = bytes / 16;
+      const int blocks = (int)((chunks + 255) / 256 < 64 ? (chunks + 255) / 256 : 64);
+      copy_from_host_kernel<<<blocks, 256, 0, s>>>((int4*)dst, (const int4*)device_src, chunks);
+      return lrs_check_launch("copy_h2d");
+    }
+  }
+  hipError_t err = hipMemcpyAsync(dst, src, (size_t)bytes, hipMemcpyHostToDevice, s);
   if (err != hipSuccess) return lrs_fail("hipMemcpyAsync: %s", hipGetErrorString(err));
   return 0;
 }

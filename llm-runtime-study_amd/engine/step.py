@@ -121,34 +121,46 @@ class ModelRunner:
         self.use_graph = use_graph and model.graph_safe()
         self._graphs: dict[tuple, tuple] = {}   # (bucket, length class) -> (handle, arena generation, logits tensor)
         self.graph_replays = 0
-        t, r, g, mb = max_step_tokens, self.max_requests, len(cache.groups), cache.max_blocks
-        # layout of the metadata buffer (int32 elements)
-        self._off = {}
-        cursor = 0
         # query groups for the ragged attention kernel: at most `query_group` consecutive tokens of one request
         self.query_group = ops.attention_prefill_group()   # the most; a step of few tokens uses smaller ones
-        self._max_qblocks = -(-t // 16) + r
-        for name, size in (("token_ids", t), ("positions", t), ("token_request", t), ("logit_rows", t),
-                           ("cu_seqlens_q", r + 1), ("seq_lens_k", r), ("slot_ids", r),
-                           ("qblock_token0", self._max_qblocks), ("qblock_count", self._max_qblocks)):
-            self._off[name] = (cursor, size)
-            cursor += size
-        for index in range(g):
-            self._off[f"slots{index}"] = (cursor, t)
-            cursor += t
-            self._off[f"table{index}"] = (cursor, r * mb)
-            cursor += r * mb
-        self._meta_size = cursor
+        # The metadata of a step is one int32 buffer whose layout follows the step's own numbers of
+        # tokens and requests, so that a decode step uploads a few KB whatever the limits are.  A
+        # graph holds addresses inside it: steps of one padded batch size share one layout.
+        self._layouts: dict[tuple[int, int], tuple[dict, int]] = {}
+        self._off, self._meta_size = self._layout(max_step_tokens, self.max_requests)
+        cursor = self._meta_size
         # two pinned staging buffers used in turn: a buffer is rewritten only after the copy
         # that read it has finished
         pin = self.device.type == "cuda"
         self._hosts = [torch.zeros(cursor, dtype=torch.int32, pin_memory=pin) for _ in range(2)]
+        if pin and not all(host.is_pinned() for host in self._hosts):
+            raise GenerationError("could not allocate pinned host memory for the step metadata")
         self._copied = [None, None]
         self._turn = 0
         self._host = self._hosts[0]
         self._host_np = self._host.numpy()
         self._dev = torch.zeros(cursor, dtype=torch.int32, device=self.device)
+        self._views: dict[tuple, tuple] = {}
+        self._counting = np.arange(max(max_step_tokens, self.max_requests) + 1, dtype=np.int32)
         self.steps_run = 0
+
+    def _layout(self, tokens: int, requests: int) -> tuple[dict, int]:
+        """Where each array of a step of `tokens` tokens and `requests` requests lies in the metadata
+        buffer: name -> (first element, elements), and the elements in all (16-byte aligned parts)."""
+        known = self._layouts.get((tokens, requests))
+        if known is None:
+            offsets, cursor = {}, 0
+            qblocks = -(-tokens // 16) + requests
+            parts = [("token_ids", tokens), ("positions", tokens), ("token_request", tokens), ("logit_rows", tokens),
+                     ("cu_seqlens_q", requests + 1), ("seq_lens_k", requests), ("slot_ids", requests),
+                     ("qblock_token0", qblocks), ("qblock_count", qblocks)]
+            for index in range(len(self.cache.groups)):
+                parts += [(f"slots{index}", tokens), (f"table{index}", requests * self.cache.max_blocks)]
+            for name, size in parts:
+                offsets[name] = (cursor, size)
+                cursor += -(-size // 4) * 4
+            known = self._layouts[(tokens, requests)] = (offsets, cursor)
+        return known
 
     def _next_staging(self) -> None:
         self._turn ^= 1
@@ -207,29 +219,48 @@ class ModelRunner:
         cache, page = self.cache, self.cache.page_size
         ctx = StepContext(self)
         self._next_staging()
+        self._off, self._meta_size = self._layout(max(sum(len(e.tokens) for e in entries), pad_to), max(len(entries), pad_to))
         ids, pos, req, rows = (self._host_view(n) for n in ("token_ids", "positions", "token_request", "logit_rows"))
         cu, lens, slots = (self._host_view(n) for n in ("cu_seqlens_q", "seq_lens_k", "slot_ids"))
         cursor = n_rows = 0
         cu[0] = 0
-        for r, entry in enumerate(entries):
-            n = len(entry.tokens)
-            start = entry.cache.length - n
-            ids[cursor:cursor + n] = entry.tokens
-            pos[cursor:cursor + n] = np.arange(start, start + n, dtype=np.int32)
-            req[cursor:cursor + n] = r
-            for place in entry.want:
-                rows[n_rows] = cursor + place
-                n_rows += 1
-            cu[r + 1] = cursor + n
-            lens[r] = entry.cache.length
-            slots[r] = entry.cache.slot
-            ctx.host_q_lens.append(n)
-            ctx.host_slots.append(entry.cache.slot)
-            ctx.host_positions.append(start)
-            cursor += n
+        if all(len(entry.tokens) == 1 for entry in entries):
+            # one token per request (a decode step): whole arrays at once, no loop over tokens
+            cursor = len(entries)
+            count = self._counting[:cursor + 1]
+            lengths = np.fromiter((entry.cache.length for entry in entries), dtype=np.int32, count=cursor)
+            ctx.host_slots = [entry.cache.slot for entry in entries]
+            ids[:cursor] = [entry.tokens[0] for entry in entries]
+            pos[:cursor] = lengths - 1
+            req[:cursor] = count[:cursor]
+            cu[:cursor + 1] = count
+            lens[:cursor] = lengths
+            slots[:cursor] = ctx.host_slots
+            wanted = [r for r, entry in enumerate(entries) if len(entry.want)]
+            n_rows = len(wanted)
+            rows[:n_rows] = wanted
+            ctx.host_q_lens = [1] * cursor
+            ctx.host_positions = pos[:cursor].tolist()
+        else:
+            for r, entry in enumerate(entries):
+                n = len(entry.tokens)
+                start = entry.cache.length - n
+                ids[cursor:cursor + n] = entry.tokens
+                pos[cursor:cursor + n] = np.arange(start, start + n, dtype=np.int32)
+                req[cursor:cursor + n] = r
+                for place in entry.want:
+                    rows[n_rows] = cursor + place
+                    n_rows += 1
+                cu[r + 1] = cursor + n
+                lens[r] = entry.cache.length
+                slots[r] = entry.cache.slot
+                ctx.host_q_lens.append(n)
+                ctx.host_slots.append(entry.cache.slot)
+                ctx.host_positions.append(start)
+                cursor += n
         real = len(entries)
         ctx.max_q = max(ctx.host_q_lens)
-        ctx.max_k = ctx.max_k_bound = max(e.cache.length for e in entries)
+        ctx.max_k = ctx.max_k_bound = int(lens[:real].max())
         if pad_to:
             # a graph outlives the step it is captured in: sizes that must hold for every replay are
             # made for the longest context the cache can hold
@@ -249,17 +280,22 @@ class ModelRunner:
             n_rows = cursor
         ctx.T, ctx.R, ctx.num_logit_rows = cursor, max(real, pad_to), n_rows
         # groups of consecutive tokens of one request, the longest contexts first
-        starts, size = cu[:ctx.R + 1], min(self.query_group, ops.attention_prefill_group(cursor))
-        blocks = [(int(pos[min(t0 + size, int(starts[i + 1])) - 1]), t0, min(size, int(starts[i + 1]) - t0))
-                  for i in range(ctx.R) for t0 in range(int(starts[i]), int(starts[i + 1]), size)]
-        blocks.sort(key=lambda b: -b[0])
-        ctx.num_qblocks = len(blocks)
-        ctx.max_qblock = max(b[2] for b in blocks)
-        self._host_view("qblock_token0")[:len(blocks)] = [b[1] for b in blocks]
-        self._host_view("qblock_count")[:len(blocks)] = [b[2] for b in blocks]
+        if ctx.all_decode:
+            ctx.num_qblocks, ctx.max_qblock = cursor, 1
+            self._host_view("qblock_token0")[:cursor] = np.argsort(-pos[:cursor], kind="stable")
+            self._host_view("qblock_count")[:cursor] = 1
+        else:
+            starts, size = cu[:ctx.R + 1], min(self.query_group, ops.attention_prefill_group(cursor))
+            blocks = [(int(pos[min(t0 + size, int(starts[i + 1])) - 1]), t0, min(size, int(starts[i + 1]) - t0))
+                      for i in range(ctx.R) for t0 in range(int(starts[i]), int(starts[i + 1]), size)]
+            blocks.sort(key=lambda b: -b[0])
+            ctx.num_qblocks = len(blocks)
+            ctx.max_qblock = max(b[2] for b in blocks)
+            self._host_view("qblock_token0")[:len(blocks)] = [b[1] for b in blocks]
+            self._host_view("qblock_count")[:len(blocks)] = [b[2] for b in blocks]
         mb = cache.max_blocks
         for index, group in enumerate(cache.groups):
-            table = self._host_view(f"table{index}").reshape(self.max_requests, mb)
+            table = self._host_view(f"table{index}").reshape(max(real, pad_to), mb)
             table[:real] = group.host_table[ctx.host_slots]
             if pad_to > real:
                 table[real:pad_to] = -1
@@ -273,17 +309,22 @@ class ModelRunner:
         return ctx
 
     def bind_views(self, ctx: StepContext) -> None:
-        mb = self.cache.max_blocks
-        ctx.token_ids, ctx.positions = self._view("token_ids", ctx.T), self._view("positions", ctx.T)
-        ctx.token_request, ctx.logit_rows = self._view("token_request", ctx.T), self._view("logit_rows", max(ctx.num_logit_rows, 1))
-        ctx.cu_seqlens_q, ctx.seq_lens_k = self._view("cu_seqlens_q", ctx.R + 1), self._view("seq_lens_k", ctx.R)
-        ctx.slot_ids = self._view("slot_ids", ctx.R)
-        ctx.qblock_token0 = self._view("qblock_token0", ctx.num_qblocks)
-        ctx.qblock_count = self._view("qblock_count", ctx.num_qblocks)
-        ctx._groups = [
-            GroupStep(self._view(f"slots{i}", ctx.T), self._view(f"table{i}").view(self.max_requests, mb)[:ctx.R], self.cache.page_size)
-            for i in range(len(self.cache.groups))
-        ]
+        """The device views of the step's arrays; steps of one shape share them (slicing is slow)."""
+        key = (ctx.T, ctx.R, ctx.num_logit_rows, ctx.num_qblocks)
+        views = self._views.get(key)
+        if views is None:
+            mb = self.cache.max_blocks
+            if len(self._views) > 256:
+                self._views.clear()
+            views = self._views[key] = (
+                self._view("token_ids", ctx.T), self._view("positions", ctx.T), self._view("token_request", ctx.T),
+                self._view("logit_rows", max(ctx.num_logit_rows, 1)), self._view("cu_seqlens_q", ctx.R + 1),
+                self._view("seq_lens_k", ctx.R), self._view("slot_ids", ctx.R), self._view("qblock_token0", ctx.num_qblocks),
+                self._view("qblock_count", ctx.num_qblocks),
+                [GroupStep(self._view(f"slots{i}", ctx.T), self._view(f"table{i}").view(ctx.R, mb), self.cache.page_size)
+                 for i in range(len(self.cache.groups))])
+        (ctx.token_ids, ctx.positions, ctx.token_request, ctx.logit_rows, ctx.cu_seqlens_q, ctx.seq_lens_k, ctx.slot_ids,
+         ctx.qblock_token0, ctx.qblock_count, ctx._groups) = views
 
     def step(self, entries: Sequence[StepEntry]) -> torch.Tensor | None:
         """Run one step; returns float32 logits [wanted, vocab] on the device, or None if none is wanted."""

@@ -48,6 +48,7 @@ _SIGNATURES = {
     "lrs_scale_rows": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_float, c_void_p]),
     "lrs_gemm_skinny_max_m": (c_int, []),
     "lrs_gemm_prepare": (c_int, []),
+    "lrs_host_device_pointer": (c_int, [c_void_p, POINTER(c_void_p)]),
     "lrs_gemm_set_skinny_max_m": (c_int, [c_int]),
     "lrs_attention": (c_int, [c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p,
                               c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_void_p]),
@@ -117,6 +118,27 @@ def _dev(t: torch.Tensor, name: str, dtype=None) -> int:
     return t.data_ptr()
 
 
+_host_visible: dict[int, int] = {}
+
+
+def _dev_or_pinned(t: torch.Tensor, name: str, dtype=None) -> int:
+    """Device address of a device tensor, or of a pinned host tensor that a kernel is to write
+    (the caller allocated it pinned; its device address is asked for once)."""
+    if t.is_cuda:
+        return _dev(t, name, dtype)
+    if dtype is not None:
+        _need(t.dtype == dtype, f"{name} must be {dtype}, got {t.dtype}")
+    address = _host_visible.get(t.data_ptr())
+    if address is None:
+        _need(t.is_pinned(), f"{name} must be a device tensor or pinned host memory")
+        out = c_void_p()
+        _check(library().lrs_host_device_pointer(t.data_ptr(), byref(out)))
+        if len(_host_visible) > 64:
+            _host_visible.clear()
+        address = _host_visible[t.data_ptr()] = out.value
+    return address
+
+
 def _rows(t: torch.Tensor, name: str) -> int:
     """Row stride of a 2-D tensor whose rows are contiguous."""
     _need(t.dim() == 2 and t.stride(1) == 1, f"{name} must be 2-D with contiguous rows, got shape {tuple(t.shape)} strides {t.stride()}")
@@ -150,8 +172,9 @@ def graph_destroy(handle: int) -> None:
 
 
 def copy_h2d(dst: torch.Tensor, src: torch.Tensor, count: int) -> None:
-    """Asynchronous copy of the first `count` elements of pinned `src` into device `dst`."""
-    _need(src.is_pinned() and src.is_contiguous() and dst.is_contiguous(), "copy_h2d needs pinned contiguous source and contiguous destination")
+    """Asynchronous copy of the first `count` elements of `src` into device `dst`.  `src` must be
+    pinned host memory (the caller checks that once, when it allocates it: asking is slow)."""
+    _need(src.device.type == "cpu" and src.is_contiguous() and dst.is_contiguous(), "copy_h2d needs a contiguous host source and a contiguous destination")
     _need(src.dtype == dst.dtype and 0 < count <= src.numel() and count <= dst.numel(), "copy_h2d: size or dtype mismatch")
     _check(library().lrs_copy_h2d(_dev(dst, "dst"), src.data_ptr(), count * src.element_size(), _stream()))
 
@@ -521,6 +544,8 @@ _choose_scratch: dict = {}
 
 
 def choose_tokens(out: torch.Tensor, logits: torch.Tensor, temperature=None, seeds=None, counters=None) -> None:
+    """One token per row of logits into `out` (int32 [R]: on the device, or pinned host memory that
+    the kernel writes directly and the host reads after synchronising the stream)."""
     rows, vocab = logits.shape
     _need(out.dtype == torch.int32 and out.numel() >= rows and out.is_contiguous(), "choose_tokens: out must be int32 [R]")
     stride = _rows(logits, "logits")
@@ -537,10 +562,10 @@ def choose_tokens(out: torch.Tensor, logits: torch.Tensor, temperature=None, see
         if scratch is None:
             scratch = _choose_scratch[key] = (torch.empty(rows * parts, dtype=torch.float32, device=logits.device),
                                               torch.empty(rows * parts, dtype=torch.int32, device=logits.device))
-        _check(library().lrs_choose_tokens_split(_dev(out, "out"), _dev(logits, "logits", torch.float32), stride, rows, vocab, *args,
+        _check(library().lrs_choose_tokens_split(_dev_or_pinned(out, "out"), _dev(logits, "logits", torch.float32), stride, rows, vocab, *args,
                                                  _dev(scratch[0], "part_value"), _dev(scratch[1], "part_index"), parts, _stream()))
         return
-    _check(library().lrs_choose_tokens(_dev(out, "out"), _dev(logits, "logits", torch.float32), stride, rows, vocab, *args, _stream()))
+    _check(library().lrs_choose_tokens(_dev_or_pinned(out, "out"), _dev(logits, "logits", torch.float32), stride, rows, vocab, *args, _stream()))
 
 
 def filter_logits(logits: torch.Tensor, temperature: torch.Tensor, top_k: torch.Tensor | None, top_p: torch.Tensor | None) -> None:

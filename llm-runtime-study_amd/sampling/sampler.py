@@ -37,6 +37,16 @@ class SamplingRow:
 class Sampler:
     def __init__(self, device):
         self.device = torch.device(device)
+        self._chosen = None      # pinned host memory the kernel writes the tokens into
+
+    def _result(self, rows: int) -> torch.Tensor:
+        if self._chosen is None or self._chosen.numel() < rows:
+            self._chosen = torch.zeros(max(rows, 64), dtype=torch.int32, pin_memory=True)
+        return self._chosen[:rows]
+
+    def _read(self, out: torch.Tensor) -> list[int]:
+        torch.cuda.current_stream(self.device).synchronize()
+        return out.tolist()
 
     def choose(self, logits: torch.Tensor, rows: list[SamplingRow]) -> list[int]:
         """One token per row of `logits` [R, V] float32 (filters the sampled rows in place)."""
@@ -46,10 +56,10 @@ class Sampler:
         for row in rows:
             if row.config.top_k is not None and row.config.top_k > vocab:
                 raise SamplingError(f"top_k {row.config.top_k} exceeds vocabulary size {vocab}")
-        out = torch.empty(len(rows), dtype=torch.int32, device=self.device)
+        out = self._result(len(rows))
         if all(row.config.greedy for row in rows):
             ops.choose_tokens(out, logits)
-            return out.cpu().tolist()
+            return self._read(out)
         temperature = torch.tensor([row.config.temperature for row in rows], dtype=torch.float32, device=self.device)
         seeds = torch.tensor([row.seed for row in rows], dtype=torch.int64, device=self.device)
         counters = torch.tensor([row.counter for row in rows], dtype=torch.int32, device=self.device)
@@ -58,4 +68,4 @@ class Sampler:
             top_p = torch.tensor([row.config.top_p for row in rows], dtype=torch.float32, device=self.device)
             ops.filter_logits(logits, temperature, top_k, top_p)
         ops.choose_tokens(out, logits, temperature, seeds, counters)
-        return out.cpu().tolist()
+        return self._read(out)
