@@ -500,6 +500,9 @@ LRS_API int lrs_attention_decode(void* out, int out_stride, float* part_o, float
 // come longest first, and in every second chunk of `chunk` workgroups (one per compute unit) the
 // order is turned round, so that the two workgroups that meet on a compute unit are a long and a
 // short one; the kv head changes fastest, which keeps one kv head's keys in one XCD's L2.
+// splits > 1 (few queries over long contexts): the key tiles of every group are divided between
+// `splits` workgroups, which leave unnormalised sums, maxima and weights in part_o / part_ml
+// [tokens, heads, splits, ...] for attention_merge_kernel, as the decode kernel does.
 template <int D, int QB>
 __global__ __launch_bounds__(256, D <= 128 ? 2 : 1) void attention_prefill_bf16_kernel(
     bf16* __restrict__ out, int out_stride, const bf16* __restrict__ q, int q_stride,
@@ -507,7 +510,7 @@ __global__ __launch_bounds__(256, D <= 128 ? 2 : 1) void attention_prefill_bf16_
     const int* __restrict__ block_table, int table_stride, const int* __restrict__ token_request,
     const int* __restrict__ positions, const int* __restrict__ qblock_token0,
     const int* __restrict__ qblock_count, int n_blocks, int chunk, int nq, int nkv, int page_size, float scale,
-    int window) {
+    int window, int splits, float* __restrict__ part_o, float* __restrict__ part_ml) {
   constexpr int DS = D / 32, DB = D / 16;
   // Padded LDS rows (32 banks of 4 bytes).  Key rows are read 16 bytes a lane by 8 lanes a cycle: a
   // stride of 4 banks more than a multiple of 32 spreads them over all banks.  Value rows are read
@@ -522,7 +525,8 @@ __global__ __launch_bounds__(256, D <= 128 ? 2 : 1) void attention_prefill_bf16_
   const int lane = tid % WAVE, wave = tid / WAVE, waves = threads / WAVE;
   const int col = lane & 15, g = lane >> 4;
   const int group = nq / nkv;
-  const int which_chunk = blockIdx.x / chunk, in_chunk = blockIdx.x % chunk;
+  const int work = blockIdx.x % (n_blocks * nkv), split = blockIdx.x / (n_blocks * nkv);
+  const int which_chunk = work / chunk, in_chunk = work % chunk;
   const int chunk_block0 = which_chunk * (chunk / nkv);
   const int chunk_blocks = n_blocks - chunk_block0 < chunk / nkv ? n_blocks - chunk_block0 : chunk / nkv;
   const int kvh = in_chunk % nkv;
@@ -535,12 +539,19 @@ __global__ __launch_bounds__(256, D <= 128 ? 2 : 1) void attention_prefill_bf16_
   const bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
   const float scale2 = scale * 1.4426950408889634f;
   const float rescale_step = RESCALE_STEP / scale2;              // in units of the unscaled scores
-  const int first_tile = lo_first / 32, last_tile = pos_last / 32;
+  int first_tile = lo_first / 32, last_tile = pos_last / 32;
+  if (splits > 1) {                                              // this workgroup's share of the tiles (may be none)
+    const int per_split = (last_tile - first_tile + splits) / splits;
+    first_tile += split * per_split;
+    if (first_tile + per_split - 1 < last_tile) last_tile = first_tile + per_split - 1;
+  }
   // the part of the request's block table that the tiles need, in LDS: the address of a key must
   // not wait for a trip to memory of its own
   extern __shared__ int page_ids[];
   const int first_block = first_tile * 32 / page_size;
-  for (int i = tid; i <= pos_last / page_size - first_block; i += threads) page_ids[i] = table[first_block + i];
+  const int last_key = last_tile * 32 + 31 < pos_last ? last_tile * 32 + 31 : pos_last;
+  if (first_tile <= last_tile)
+    for (int i = tid; i <= last_key / page_size - first_block; i += threads) page_ids[i] = table[first_block + i];
   __syncthreads();
 
   // pieces of a tile this thread brings in: keys [32, D] and transposed values [D, 32]
@@ -685,8 +696,10 @@ __global__ __launch_bounds__(256, D <= 128 ? 2 : 1) void attention_prefill_bf16_
       }
     };
     __syncthreads();                                           // the buffers of an earlier pass are done with
-    fetch(first_tile, kreg_a, vreg_a);
-    stash(0, kreg_a, vreg_a);
+    if (first_tile <= last_tile) {
+      fetch(first_tile, kreg_a, vreg_a);
+      stash(0, kreg_a, vreg_a);
+    }
     __syncthreads();
     // At the top of a turn `tile` is in LDS buffer (tile - first_tile) % 2; the next tile is asked
     // for before the work on this one and put into the other buffer after it.  Three runs of tiles:
@@ -702,6 +715,7 @@ __global__ __launch_bounds__(256, D <= 128 ? 2 : 1) void attention_prefill_bf16_
     };
     int whole_begin = (lo_last + 31) / 32, whole_end = (pos_first + 1) / 32;   // tiles [whole_begin, whole_end) need no mask
     if (whole_begin < first_tile) whole_begin = first_tile;
+    if (whole_begin > last_tile + 1) whole_begin = last_tile + 1;
     if (whole_end > last_tile + 1) whole_end = last_tile + 1;
     if (whole_end < whole_begin) whole_end = whole_begin;
     run(first_tile, whole_begin, std::true_type{});
@@ -712,7 +726,15 @@ __global__ __launch_bounds__(256, D <= 128 ? 2 : 1) void attention_prefill_bf16_
       float total = run_sum[b];
       total += __shfl_xor(total, 16, WAVE);
       total += __shfl_xor(total, 32, WAVE);
-      if (live[b]) {
+      if (live[b] && splits > 1) {
+        const int64_t slot = ((int64_t)(token0 + b * 16 + col) * nq + head) * splits + split;
+#pragma unroll
+        for (int e = 0; e < DB; ++e) *(floatx4*)(part_o + slot * D + e * 16 + g * 4) = o[b][e];
+        if (g == 0) {
+          part_ml[slot * 2] = run_max[b] * scale2;               // -inf stays -inf: no key seen
+          part_ml[slot * 2 + 1] = total;
+        }
+      } else if (live[b]) {
         const float inv = 1.0f / total;
         bf16* dst = out + (int64_t)(token0 + b * 16 + col) * out_stride + (int64_t)head * D + g * 4;
 #pragma unroll
@@ -747,11 +769,14 @@ LRS_API int lrs_attention_prefill_group_for(int tokens) { return tokens <= 8 * c
 
 // Any step in bf16.  qblock_token0 / qblock_count [n_blocks]: first token and number of tokens
 // (1..lrs_attention_prefill_group()) of each group of consecutive tokens of one request.
+// splits > 1: every group's keys are divided between that many workgroups; needs part_o
+// [tokens, nq, splits, d] and part_ml [tokens, nq, splits, 2] float32 and `tokens`, the step's size.
 LRS_API int lrs_attention_prefill(void* out, int out_stride, const void* q, int q_stride, const void* k_pages,
                                   const void* v_pages, const int* block_table, int table_stride,
                                   const int* token_request, const int* positions, const int* qblock_token0,
                                   const int* qblock_count, int n_blocks, int max_count, int max_context, int nq,
-                                  int nkv, int d, int page_size, float scale, int window, void* stream) {
+                                  int nkv, int d, int page_size, float scale, int window, int tokens, int splits,
+                                  float* part_o, float* part_ml, void* stream) {
   LRS_REQUIRE(n_blocks > 0 && nq > 0 && nkv > 0 && nq % nkv == 0, "attention_prefill: bad sizes blocks=%d nq=%d nkv=%d", n_blocks, nq, nkv);
   LRS_REQUIRE(max_count >= 1 && max_count <= 32, "attention_prefill: query groups hold 1..32 tokens, got %d", max_count);
   LRS_REQUIRE(page_size % 16 == 0, "attention_prefill: page size %d is not a multiple of 16", page_size);
@@ -759,7 +784,10 @@ LRS_API int lrs_attention_prefill(void* out, int out_stride, const void* q, int 
   LRS_REQUIRE(q_stride % 8 == 0 && ((uintptr_t)q % 16) == 0 && out_stride % 4 == 0 && ((uintptr_t)out % 8) == 0,
               "attention_prefill: q rows must be 16-byte and out rows 8-byte aligned");
   // always four waves: with fewer heads in a kv group the spare waves still help to bring tiles in
-  dim3 grid(n_blocks * nkv), block(4 * WAVE);
+  LRS_REQUIRE(splits >= 1 && splits <= 64 && (splits == 1 || (part_o && part_ml && tokens > 0)),
+              "attention_prefill: splits=%d (1..64) need partial buffers and the number of tokens", splits);
+  LRS_REQUIRE(splits == 1 || ((uintptr_t)part_o % 16) == 0, "attention_prefill: part_o must be 16-byte aligned");
+  dim3 grid(n_blocks * nkv * splits), block(4 * WAVE);
   // workgroups that share a compute unit: see the kernel
   const int chunk = nkv >= compute_units() ? nkv : compute_units() / nkv * nkv;
   // LDS copy of the block table entries a workgroup walks: at most those of the longest context
@@ -772,7 +800,8 @@ LRS_API int lrs_attention_prefill(void* out, int out_stride, const void* q, int 
   attention_prefill_bf16_kernel<D, QB><<<grid, block, table_lds, s>>>((bf16*)out, out_stride, (const bf16*)q, q_stride, \
                                                               (const bf16*)k_pages, (const bf16*)v_pages, block_table, \
                                                               table_stride, token_request, positions, qblock_token0, \
-                                                              qblock_count, n_blocks, chunk, nq, nkv, page_size, scale, window)
+                                                              qblock_count, n_blocks, chunk, nq, nkv, page_size, scale, window, \
+                                                              splits, part_o, part_ml)
 #define LAUNCH(D)                                \
   if (max_count <= 16) LAUNCH2(D, 1);            \
   else LAUNCH2(D, 2)
@@ -786,8 +815,16 @@ LRS_API int lrs_attention_prefill(void* out, int out_stride, const void* q, int 
   }
 #undef LAUNCH
 #undef LAUNCH2
-  return lrs_check_launch("attention_prefill");
+  if (lrs_check_launch("attention_prefill")) return 1;
+  if (splits > 1) {
+    attention_merge_kernel<<<dim3(tokens, nq), d < 64 ? 64 : d, 0, s>>>((bf16*)out, out_stride, part_o, part_ml, nq, d, splits);
+    return lrs_check_launch("attention_merge");
+  }
+  return 0;
 }
+
+// Compute units of the device, for callers that size their launches by it.
+LRS_API int lrs_compute_units() { return compute_units(); }
 
 // out [tokens, nq*d] (row stride out_stride); q rows are [nq*d] with row stride q_stride.
 LRS_API int lrs_attention(void* out, int out_stride, const void* q, int q_stride, const void* k_pages,

@@ -1,6 +1,7 @@
 """Timings of single kernels at the shapes of a model, outside any model.
 
     python -m llm_runtime_study_amd.kernels.microbench attention_prefill --tokens 2048,8192 --group 16,32
+    python -m llm_runtime_study_amd.kernels.microbench attention_prefill --tokens 64 --before 32704 --key-splits 1,8,32
     python -m llm_runtime_study_amd.kernels.microbench attention_decode --batch 1,8,64 --context 2048 --splits 1,4,8
     python -m llm_runtime_study_amd.kernels.microbench gemm --rows 1,8,16,64,2048
 
@@ -40,26 +41,31 @@ def _time(call, repeats: int) -> float:
 
 
 def attention_prefill(args) -> None:
-    """One request's whole prompt: `tokens` queries over their own causal context."""
-    nq, nkv, d, page = args.heads, args.kv_heads, args.head_dim, args.page_size
+    """One request's prompt, or a later portion of it: `tokens` queries after `before` cached tokens."""
+    nq, nkv, d, page, before = args.heads, args.kv_heads, args.head_dim, args.page_size, args.before
     for tokens in _ints(args.tokens):
-        pages = -(-tokens // page)
+        pages = -(-(before + tokens) // page)
         k_pages = torch.randn(pages + 1, nkv, page, d, device="cuda", dtype=torch.bfloat16)
         v_pages = torch.randn(pages + 1, nkv, d, page, device="cuda", dtype=torch.bfloat16)
         table = torch.randperm(pages, device="cuda").to(torch.int32).view(1, -1)
         q = torch.randn(tokens, (nq + 2 * nkv) * d, device="cuda", dtype=torch.bfloat16)
         out = torch.empty(tokens, nq * d, device="cuda", dtype=torch.bfloat16)
         request = torch.zeros(tokens, dtype=torch.int32, device="cuda")
-        positions = torch.arange(tokens, dtype=torch.int32, device="cuda")
-        flops = 4 * (tokens * (tokens + 1) / 2) * nq * d
+        positions = torch.arange(before, before + tokens, dtype=torch.int32, device="cuda")
+        flops = 4 * (tokens * before + tokens * (tokens + 1) / 2) * nq * d
         groups = _ints(args.group) if args.group else [ops.attention_prefill_group(tokens)]
         for size in groups:
             starts = list(range(0, tokens, size))[::-1]          # longest contexts first, as the engine orders them
             token0 = torch.tensor(starts, dtype=torch.int32, device="cuda")
             count = torch.tensor([min(size, tokens - s) for s in starts], dtype=torch.int32, device="cuda")
-            seconds = _time(lambda i: ops.attention_prefill(out, q, k_pages, v_pages, table, request, positions, token0, count,
-                                                            nq, 1 / math.sqrt(d), args.window, size, tokens), args.repeats)
-            print(f"attention_prefill tokens={tokens} group={size}: {seconds * 1e6:9.1f} us  {flops / seconds / 1e12:7.1f} TFLOP/s (causal half)", flush=True)
+            for splits in _ints(args.key_splits):
+                part_o = torch.empty(tokens, nq * splits * d, device="cuda") if splits > 1 else None
+                part_ml = torch.empty(tokens, nq * splits * 2, device="cuda") if splits > 1 else None
+                seconds = _time(lambda i: ops.attention_prefill(out, q, k_pages, v_pages, table, request, positions, token0, count,
+                                                                nq, 1 / math.sqrt(d), args.window, size, before + tokens,
+                                                                splits, part_o, part_ml), args.repeats)
+                print(f"attention_prefill tokens={tokens} after={before} group={size} splits={splits}: {seconds * 1e6:9.1f} us  "
+                      f"{flops / seconds / 1e12:7.1f} TFLOP/s (keys a query may see)", flush=True)
 
 
 def attention_decode(args) -> None:
@@ -120,6 +126,8 @@ def main(argv=None) -> int:
     parser.add_argument("--page-size", type=int, default=16)
     parser.add_argument("--window", type=int, default=0)
     parser.add_argument("--tokens", default="2048", help="attention_prefill: prompt lengths, comma separated")
+    parser.add_argument("--before", type=int, default=0, help="attention_prefill: tokens of the request already in the cache (the queries are a later portion)")
+    parser.add_argument("--key-splits", default="1", help="attention_prefill: workgroups per query group")
     parser.add_argument("--group", default="", help="attention_prefill: query group sizes (default: what the engine would choose)")
     parser.add_argument("--batch", default="1,8,64", help="attention_decode: batch sizes")
     parser.add_argument("--context", type=int, default=2048, help="attention_decode: cached tokens per request")

@@ -56,7 +56,9 @@ _SIGNATURES = {
                                      c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_int, c_int,
                                      c_void_p, c_void_p, c_int, c_float, c_void_p, c_void_p, c_int, c_void_p]),
     "lrs_attention_prefill": (c_int, [c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p,
-                                      c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_void_p]),
+                                      c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int,
+                                      c_int, c_int, c_void_p, c_void_p, c_void_p]),
+    "lrs_compute_units": (c_int, []),
     "lrs_attention_prefill_group": (c_int, []),
     "lrs_attention_prefill_group_for": (c_int, [c_int]),
     "lrs_choose_tokens": (c_int, [c_void_p, c_void_p, c_int64, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p]),
@@ -505,11 +507,14 @@ def attention_decode(out: torch.Tensor, q: torch.Tensor, k_pages: torch.Tensor, 
 
 def attention_prefill(out: torch.Tensor, q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, block_table: torch.Tensor,
                       token_request: torch.Tensor, positions: torch.Tensor, qblock_token0: torch.Tensor, qblock_count: torch.Tensor,
-                      nq: int, scale: float, window: int = 0, max_count: int | None = None, max_context: int | None = None) -> None:
+                      nq: int, scale: float, window: int = 0, max_count: int | None = None, max_context: int | None = None,
+                      splits: int = 1, part_o: torch.Tensor | None = None, part_ml: torch.Tensor | None = None) -> None:
     """attention() on matrix cores for any bfloat16 step.  qblock_token0 / qblock_count list groups of at
     most attention_prefill_group() consecutive tokens of one request that together cover every token of
     the step once; `max_count` is the largest count among them (the group limit if not given) and
-    `max_context` the longest context (position + 1) of any token (what the block table can hold if not given)."""
+    `max_context` the longest context (position + 1) of any token (what the block table can hold if not given).
+    splits > 1 divides every group's keys between that many workgroups (few queries over long contexts);
+    their partial results meet in part_o [T, nq * splits * d] and part_ml [T, nq * splits * 2] float32."""
     tokens = out.shape[0]
     _need(k_pages.dim() == 4 and k_pages.is_contiguous() and v_pages.is_contiguous(), "attention_prefill: pages must be contiguous")
     _, nkv, page_size, d = k_pages.shape
@@ -523,12 +528,22 @@ def attention_prefill(out: torch.Tensor, q: torch.Tensor, k_pages: torch.Tensor,
     n_blocks = qblock_token0.numel()
     _need(n_blocks > 0 and qblock_count.numel() == n_blocks and qblock_token0.dtype == qblock_count.dtype == torch.int32
           and qblock_token0.is_contiguous() and qblock_count.is_contiguous(), "attention_prefill: query blocks must be two int32 vectors of one length")
+    _need(1 <= splits <= 64, f"attention_prefill: splits must be 1..64, got {splits}")
+    if splits > 1:
+        _need(part_o is not None and part_o.dtype == torch.float32 and part_o.is_contiguous() and part_o.numel() >= tokens * nq * splits * d, "attention_prefill: part_o too small")
+        _need(part_ml is not None and part_ml.dtype == torch.float32 and part_ml.is_contiguous() and part_ml.numel() >= tokens * nq * splits * 2, "attention_prefill: part_ml too small")
     _check(library().lrs_attention_prefill(
         _dev(out, "out"), _rows(out, "out"), _dev(q, "q"), _rows(q, "q"), _dev(k_pages, "k_pages"), _dev(v_pages, "v_pages"),
         _dev(block_table, "block_table"), block_table.stride(0), _dev(token_request, "token_request"), _dev(positions, "positions"),
         _dev(qblock_token0, "qblock_token0"), _dev(qblock_count, "qblock_count"), n_blocks,
         attention_prefill_group() if max_count is None else max_count,
-        block_table.shape[1] * page_size if max_context is None else max_context, nq, nkv, d, page_size, scale, window, _stream()))
+        block_table.shape[1] * page_size if max_context is None else max_context, nq, nkv, d, page_size, scale, window,
+        tokens, splits, None if splits == 1 else _dev(part_o, "part_o"), None if splits == 1 else _dev(part_ml, "part_ml"), _stream()))
+
+
+def compute_units() -> int:
+    """Compute units of the device (workgroups of one kernel that can start at the same time, per occupancy)."""
+    return library().lrs_compute_units()
 
 
 def attention_prefill_group(tokens: int | None = None) -> int:

@@ -34,3 +34,17 @@ def test_decode_splits_keep_a_workgroups_block_table_inside_lds():
     assert splits(512, 100, 4096 * 16 + 1, 16) == 2
     assert splits(512, 100, 1 << 20, 16) == 16
     assert splits(512, 100, 1 << 20, 64) == 4
+
+
+def test_prefill_splits_only_where_groups_leave_the_chip_idle(monkeypatch):
+    from llm_runtime_study_amd.kernels import ops
+
+    monkeypatch.setattr(ops, "compute_units", lambda: 256)
+    splits = GQAAttention._prefill_splits
+    assert splits(1024, 100000, 1 << 20) == 1           # enough groups already (a 2,048-token prompt, 8 kv heads)
+    assert splits(512, 1024, 1 << 20) == 1              # short contexts
+    assert splits(256, 33216, 1 << 20) == 8             # a 512-token portion after 32,704 tokens
+    assert splits(32, 32768, 1 << 20) == 32             # a 64-token portion
+    assert splits(8, 32768, 1 << 16) == 32              # one token: as many as allowed
+    assert splits(8, 2048, 1 << 16) == 2                # at least 1,024 keys each
+    assert splits(8, 1 << 20, 16 << 20) == 4            # partial results stay within 256 MB

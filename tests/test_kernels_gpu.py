@@ -427,17 +427,21 @@ def test_attention_ragged_batch(ops, dtype, nq, nkv, d, page, window):
     if ops.attention_decode_supported(dtype, nq, nkv, d, page):
         # the matrix-core kernel for ragged steps: groups of consecutive tokens of one request, in any order
         assert ops.attention_prefill_group() == 32
-        for size in (16, 7, 32, 25):
+        # ... and with the keys of every group divided between several workgroups (more than some groups have tiles)
+        for size, splits in ((16, 1), (7, 1), (32, 1), (25, 1), (16, 3), (32, 8), (7, 64)):
             blocks, at = [], 0
             for before, new in requests:
                 blocks += [(at + i, min(size, new - i)) for i in range(0, new, size)]
                 at += new
             blocks = blocks[::-1]
             fast = torch.empty_like(out)
+            part_o = torch.full((out.shape[0], nq * splits * d), float("nan"), device="cuda") if splits > 1 else None
+            part_ml = torch.full((out.shape[0], nq * splits * 2), float("nan"), device="cuda") if splits > 1 else None
             ops.attention_prefill(fast, dev(q_wide), dev(kp.to(dtype)), dev(vp.to(dtype)), dev(table),
                                   dev(torch.tensor(tok_req, dtype=torch.int32)), dev(torch.tensor(tok_pos, dtype=torch.int32)),
                                   dev(torch.tensor([b[0] for b in blocks], dtype=torch.int32)),
-                                  dev(torch.tensor([b[1] for b in blocks], dtype=torch.int32)), nq, scale, window, size)
+                                  dev(torch.tensor([b[1] for b in blocks], dtype=torch.int32)), nq, scale, window, size,
+                                  splits=splits, part_o=part_o, part_ml=part_ml)
             torch.testing.assert_close(fast.cpu().double(), want, rtol=2e-2, atol=2e-2)
 
 

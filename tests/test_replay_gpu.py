@@ -111,6 +111,38 @@ def test_mixed_with_reused_pages(models, name, seed, dtype, tmp_path):
     assert peak < sum(round64(len(t)) for t in requests.values())
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_late_portions_and_single_tokens_of_a_long_prompt(tmp_path, dtype):
+    """2,300 tokens: most in one step, then portions of 40, 16, 2 and 1 tokens and a step that holds a
+    portion of this request beside a single token of another.  With so few queries over more than a
+    thousand keys the bfloat16 attention kernel divides each group's keys between workgroups."""
+    from llm_runtime_study_amd.config import config_from_dict
+    from llm_runtime_study_amd.weights import write_model_dir
+
+    raw = dict(TINY_C, max_position_embeddings=4096)
+    folder = tmp_path / "model"
+    write_model_dir(config_from_dict(raw), seed=14, model_dir=folder, init="scaled")
+    cfg, weights = plain.load_model_dir(folder, torch.float64)
+    rng = np.random.default_rng(9)
+    long_ids = rng.integers(0, raw["vocab_size"], 2300).tolist()
+    other = rng.integers(0, raw["vocab_size"], 1200).tolist()
+    want = {"long": plain.qwen3_forward(weights, cfg, long_ids), "other": plain.qwen3_forward(weights, cfg, other)}
+    steps, at = [], 0
+    cuts = [2200, 40, 16, 2, 1, 30, 11]
+    for number, n in enumerate(cuts):
+        entries = [{"id": "long", "tokens": long_ids[at:at + n], "want": list(range(max(0, n - 48), n))}]
+        if number == 0:
+            entries.append({"id": "other", "tokens": other[:1199], "want": [1198]})
+        if number == 5:     # a single token of the other request beside a portion of this one
+            entries.insert(0, {"id": "other", "tokens": other[1199:], "want": [0]})
+        steps.append({"step": number, "entries": entries, "end": ["long", "other"] if number == len(cuts) - 1 else []})
+        at += n
+    assert at == len(long_ids)
+    out = run_replay(folder, dtype, steps, 2304 + 1216, tmp_path)
+    got = traces.collect(steps, out, raw["vocab_size"])
+    assert compare(got, want, dtype) == 48 + 40 + 16 + 2 + 1 + 30 + 11 + 2
+
+
 def test_cuts_agree_bit_for_bit_in_float32(models, tmp_path):
     """In float32 the order of every sum depends on the position alone, so whole, portioned and
     mixed replays give identical bits."""
