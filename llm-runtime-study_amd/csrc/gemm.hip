@@ -275,16 +275,22 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_skinny_kernel(
   int s = split_begin + wave * per_wave;
   const int s_end = s + per_wave < split_end ? s + per_wave : split_end;
   const int full_end = k / 32 < s_end ? k / 32 : s_end;   // steps whose 32 k are all inside K
-  for (; s + UNROLL <= full_end; s += UNROLL) {
+  // Workgroups walk their K slices from different starting points (the order of a column's sum
+  // depends on the column alone): all of them read the same activations, and in step they would
+  // all ask the same few cache lines of the L2 at the same moment.
+  const int batches = full_end > s ? (full_end - s) / UNROLL : 0;
+  const int s_first = s;
+  for (int j = 0; j < batches; ++j) {
+    const int sb = s_first + ((j + (int)blockIdx.x) % batches) * UNROLL;
     bf16x8 a[UNROLL][RT], b[UNROLL][MT];
 #pragma unroll
     for (int u = 0; u < UNROLL; ++u)
 #pragma unroll
-      for (int q = 0; q < RT; ++q) a[u][q] = *(const bf16x8*)(wp[q] + (s + u) * 32);
+      for (int q = 0; q < RT; ++q) a[u][q] = *(const bf16x8*)(wp[q] + (sb + u) * 32);
 #pragma unroll
     for (int u = 0; u < UNROLL; ++u)
 #pragma unroll
-      for (int t = 0; t < MT; ++t) b[u][t] = load_b(t, s + u);
+      for (int t = 0; t < MT; ++t) b[u][t] = load_b(t, sb + u);
 #pragma unroll
     for (int u = 0; u < UNROLL; ++u)
 #pragma unroll
@@ -293,6 +299,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_skinny_kernel(
         for (int t = 0; t < MT; ++t)
           acc[q][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[u][q], b[u][t], acc[q][t], 0, 0, 0);
   }
+  s = s_first + batches * UNROLL;
   for (; s < s_end; ++s) {
     const bool inside = s * 32 + g * 8 < k;
     bf16x8 b[MT];
