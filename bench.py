@@ -48,6 +48,7 @@ def parse_args():
     parser.add_argument("--dtype", choices=("bfloat16", "float32"), default="bfloat16")
     parser.add_argument("--no-points", action="store_true", help="skip the batch 1 and 64 decode points")
     parser.add_argument("--no-graph", action="store_true")
+    parser.add_argument("--decode-steps-per-launch", type=int, default=4, help="greedy decode steps run from one graph launch (1: one step a launch)")
     parser.add_argument("--own-gemm", action="store_true", help="this package's kernel also for products of many rows (default: vendor library)")
     return parser.parse_args()
 
@@ -84,15 +85,27 @@ def measure_decode(engine, batch: int, context: int, steps: int, warmup: int, se
         produced = 0
         while produced < batch:
             produced += sum(1 for _, e in scheduler.step() if e.prompt_token_count is not None)
-        for _ in range(warmup):
-            scheduler.step()
+        # one call of the scheduler may hold several decode steps (one graph launch): count steps, not calls
+        per_launch = scheduler.decode_steps_per_launch
+
+        def run(count: int, record: bool) -> None:
+            done = 0
+            while done < count:
+                scheduler.decode_steps_per_launch = min(per_launch, count - done)
+                started = time.perf_counter()
+                events = scheduler.step()
+                engine.synchronize()
+                elapsed = time.perf_counter() - started
+                assert len(events) % batch == 0 and len(events) > 0
+                held = len(events) // batch
+                if record:
+                    times.extend([elapsed / held] * held)
+                done += held
+
+        run(warmup, False)
         engine.synchronize()
-        for _ in range(steps):
-            started = time.perf_counter()
-            events = scheduler.step()
-            engine.synchronize()
-            times.append(time.perf_counter() - started)
-            assert len(events) == batch
+        run(steps, True)
+        assert len(times) == steps
         scheduler.abort_all()
     # requests entered one step apart, so they are up to `batch` tokens apart in length
     mean_context = context + 1 + warmup + (batch - 1) / 2 + (steps - 1) / 2
@@ -137,7 +150,8 @@ def main() -> int:
     max_seq_len = args.context + args.steps + args.warmup + 2 * max_batch + 64
     max_seq_len = max(max_seq_len, args.prefill_tokens)
     engine = Engine.from_config(config, seed=0, dtype=args.dtype, max_seq_len=max_seq_len, max_batch_size=max_batch,
-                                max_num_batched_tokens=max(2048, args.prefill_tokens), use_cuda_graph=not args.no_graph, library_gemm=not args.own_gemm)
+                                max_num_batched_tokens=max(2048, args.prefill_tokens), use_cuda_graph=not args.no_graph, library_gemm=not args.own_gemm,
+                                decode_steps_per_launch=args.decode_steps_per_launch)
     dtype_name = "bf16" if args.dtype == "bfloat16" else "fp32"
 
     prefill_times = measure_prefill(engine, args.prefill_tokens, repeats=3, seed=1)
@@ -177,7 +191,8 @@ def main() -> int:
             "num_attention_heads": config.num_attention_heads, "num_key_value_heads": config.num_key_value_heads,
             "head_dim": config.head_dim, "vocab_size": config.vocab_size, "global_batch": args.batch,
             "seq_len": args.context, "new_tokens": args.steps + args.warmup, "page_size": engine.page_size,
-            "prefill_tokens": args.prefill_tokens, "hip_graph": bool(engine.runner.use_graph), "prefill_gemm": "own" if args.own_gemm else "hipBLASLt",
+            "prefill_tokens": args.prefill_tokens, "hip_graph": bool(engine.runner.use_graph),
+            "decode_steps_per_launch": args.decode_steps_per_launch if engine.runner.use_graph else 1, "prefill_gemm": "own" if args.own_gemm else "hipBLASLt",
             "parallelism": "single GPU",
         },
         "prefill": {

@@ -3,7 +3,7 @@
 Options, defaults and output follow the reference's command line (mini_llm/cli.py:32-64
 parser, 101-158 one prompt, 161-210 interactive, 213-247 metrics, 250-284 error handling:
 typed errors print `error: ...` and exit with 2).  Added: --prompt-ids for models without
-a tokenizer, --max-batch-size, --page-size, --no-graph.
+a tokenizer, --max-batch-size, --page-size, --no-graph, --decode-steps-per-launch.
 """
 
 from __future__ import annotations
@@ -51,6 +51,8 @@ def build_parser() -> argparse.ArgumentParser:
     parser.add_argument("--max-batch-size", type=int, default=1)
     parser.add_argument("--page-size", type=int, default=16)
     parser.add_argument("--no-graph", action="store_true", help="run decode steps without HIP graph replay")
+    parser.add_argument("--decode-steps-per-launch", type=int, default=4,
+                        help="greedy decode steps run from one graph launch; tokens then arrive that many at a time (1: one by one)")
     return parser
 
 
@@ -63,7 +65,7 @@ def _engine_from_args(args):
 
     return Engine.from_model_dir(args.model, device=args.device, dtype=args.dtype, max_seq_len=args.max_seq_len,
                                  max_batch_size=args.max_batch_size, use_cuda_graph=not args.no_graph,
-                                 page_size=args.page_size)
+                                 page_size=args.page_size, decode_steps_per_launch=args.decode_steps_per_launch)
 
 
 def _prompt_from_args(args, text: str | None):

@@ -523,6 +523,45 @@ LRS_API int lrs_scale_rows(void* out, const void* x, const float* sumsq, int par
   return lrs_check_launch("scale_rows");
 }
 
+// ---------------------------------------------------- next decode step's metadata
+// Several decode steps can run from one launch: between two of them the step's metadata is moved
+// on by the device itself.  Each of the first *real_rows rows (the others pad the batch) takes the
+// token just chosen for it, moves one position on and lengthens its request by one ...
+__global__ void advance_decode_kernel(int* __restrict__ token_ids, int* __restrict__ positions,
+                                      const int* __restrict__ token_request, int* __restrict__ seq_lens,
+                                      const int* __restrict__ chosen, const int* __restrict__ real_rows, int rows) {
+  const int t = blockIdx.x * blockDim.x + threadIdx.x;
+  if (t >= rows || t >= *real_rows) return;
+  token_ids[t] = chosen[t];
+  positions[t] += 1;
+  seq_lens[token_request[t]] += 1;
+}
+
+// ... and, per cache group, finds the slot of its new position in its request's block table.
+__global__ void advance_slots_kernel(int* __restrict__ slots, const int* __restrict__ positions,
+                                     const int* __restrict__ token_request, const int* __restrict__ block_table,
+                                     int table_stride, int page_size, const int* __restrict__ real_rows, int rows) {
+  const int t = blockIdx.x * blockDim.x + threadIdx.x;
+  if (t >= rows || t >= *real_rows) return;
+  const int pos = positions[t];
+  const int page = block_table[(int64_t)token_request[t] * table_stride + pos / page_size];
+  slots[t] = page >= 0 ? page * page_size + pos % page_size : -1;
+}
+
+LRS_API int lrs_advance_decode(int* token_ids, int* positions, const int* token_request, int* seq_lens, const int* chosen,
+                               const int* real_rows, int rows, void* stream) {
+  LRS_REQUIRE(rows > 0 && token_ids && positions && token_request && seq_lens && chosen && real_rows, "advance_decode: missing arrays or no rows");
+  advance_decode_kernel<<<(rows + 255) / 256, 256, 0, (hipStream_t)stream>>>(token_ids, positions, token_request, seq_lens, chosen, real_rows, rows);
+  return lrs_check_launch("advance_decode");
+}
+
+LRS_API int lrs_advance_slots(int* slots, const int* positions, const int* token_request, const int* block_table,
+                              int table_stride, int page_size, const int* real_rows, int rows, void* stream) {
+  LRS_REQUIRE(rows > 0 && page_size > 0 && slots && positions && token_request && block_table && real_rows, "advance_slots: missing arrays or no rows");
+  advance_slots_kernel<<<(rows + 255) / 256, 256, 0, (hipStream_t)stream>>>(slots, positions, token_request, block_table, table_stride, page_size, real_rows, rows);
+  return lrs_check_launch("advance_slots");
+}
+
 LRS_API int lrs_fill_i32(int* dst, int value, int64_t n, void* stream) {
   LRS_REQUIRE(n > 0, "fill: n must be positive");
   const int blocks = (int)((n + 255) / 256 < 4096 ? (n + 255) / 256 : 4096);

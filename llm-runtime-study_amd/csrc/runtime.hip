@@ -76,8 +76,22 @@ LRS_API int lrs_host_device_pointer(void* host, void** device) {
 // step's few KB) are done by a kernel that reads the pinned memory through its device address:
 // launching it costs the host a fraction of what the runtime's copy path does, and it orders with
 // the step's kernels like any other.  `src` must be pinned (hipHostMalloc) memory.
-__global__ void copy_from_host_kernel(int4* __restrict__ dst, const int4* __restrict__ src, int64_t chunks) {
+__global__ void copy_from_host_kernel(int4* __restrict__ dst, const int4* __restrict__ src, int64_t chunks) {   // either side may be pinned host memory
   for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < chunks; i += (int64_t)gridDim.x * blockDim.x) dst[i] = src[i];
+}
+
+// A few bytes of results from the device into pinned host memory, written by a kernel through the
+// memory's device address (can be recorded in a graph, unlike a copy that may use a copy engine).
+LRS_API int lrs_copy_to_pinned(void* dst_host, const void* src, int64_t bytes, void* stream) {
+  LRS_REQUIRE(bytes > 0 && bytes % 16 == 0 && (uintptr_t)dst_host % 16 == 0 && (uintptr_t)src % 16 == 0,
+              "copy_to_pinned: %lld bytes and both addresses must be multiples of 16", (long long)bytes);
+  void* device_dst = nullptr;
+  hipError_t err = hipHostGetDevicePointer(&device_dst, dst_host, 0);
+  if (err != hipSuccess) return lrs_fail("hipHostGetDevicePointer: %s (is the memory pinned?)", hipGetErrorString(err));
+  const int64_t chunks = bytes / 16;
+  const int blocks = (int)((chunks + 255) / 256 < 64 ? (chunks + 255) / 256 : 64);
+  copy_from_host_kernel<<<blocks, 256, 0, (hipStream_t)stream>>>((int4*)device_dst, (const int4*)src, chunks);
+  return lrs_check_launch("copy_to_pinned");
 }
 
 LRS_API int lrs_copy_h2d(void* dst, const void* src, int64_t bytes, void* stream) {

@@ -32,7 +32,7 @@ class Engine:
     def __init__(self, config, model, *, device, dtype, max_seq_len: int = 4096, max_batch_size: int = 1,
                  cache_backend: str = "paged", use_cuda_graph: bool = True, page_size: int = DEFAULT_PAGE_SIZE,
                  max_num_batched_tokens: int | None = None, num_pages: int | None = None, tokenizer=None,
-                 load_seconds: float = 0.0, library_gemm: bool = True):
+                 load_seconds: float = 0.0, library_gemm: bool = True, decode_steps_per_launch: int = 4):
         if max_batch_size <= 0:
             raise EngineError("max_batch_size must be positive")
         if cache_backend != "paged":
@@ -44,6 +44,8 @@ class Engine:
         self.page_size = page_size
         self.max_num_batched_tokens = max(max_batch_size, max_num_batched_tokens or min(DEFAULT_STEP_TOKENS, max_seq_len))
         self.num_pages = num_pages
+        # greedy decoding runs up to this many steps from one graph launch (1: the host sees every step)
+        self.decode_steps_per_launch = decode_steps_per_launch
         self.library_gemm = library_gemm
         self.tokenizer = tokenizer
         self.load_seconds = load_seconds
@@ -115,7 +117,8 @@ class Engine:
         return BatchScheduler(
             self.runner, self._sampler, max_batch_size=self.max_batch_size, max_seq_len=self.max_seq_len,
             max_step_tokens=self.max_num_batched_tokens, eos_token_ids=() if ignore_eos else self.config.eos_token_ids,
-            vocab_size=self.config.vocab_size, tokenizer=self.tokenizer, synchronize=self.synchronize)
+            vocab_size=self.config.vocab_size, tokenizer=self.tokenizer, synchronize=self.synchronize,
+            decode_steps_per_launch=self.decode_steps_per_launch if self.use_cuda_graph else 1)
 
     def generate(self, message_batches: Sequence, *, max_new_tokens: int, sampling: SamplingConfig = SamplingConfig(),
                  enable_thinking: bool = False, ignore_eos: bool = False) -> Iterator[tuple[int, GenerationEvent]]:

@@ -78,7 +78,7 @@ class _Running:
 class BatchScheduler:
     def __init__(self, runner, sampler, *, max_batch_size: int, max_seq_len: int, max_step_tokens: int,
                  eos_token_ids: Sequence[int] = (), vocab_size: int | None = None, tokenizer=None,
-                 synchronize: Callable[[], None] | None = None):
+                 synchronize: Callable[[], None] | None = None, decode_steps_per_launch: int = 1):
         if max_batch_size <= 0:
             raise GenerationError("max_batch_size must be positive")
         if max_seq_len <= 0 or max_seq_len > runner.cache.max_seq_len:
@@ -92,6 +92,14 @@ class BatchScheduler:
         self.vocab_size = vocab_size
         self._eos = frozenset(eos_token_ids)
         self._synchronize = synchronize
+        if decode_steps_per_launch < 1:
+            raise GenerationError(f"decode_steps_per_launch must be at least 1, got {decode_steps_per_launch}")
+        # When every running request decodes greedily, up to this many steps run from one launch
+        # (the step function feeds each chosen token back in on the device): the host, which needs
+        # about a tenth of a millisecond between steps, is then out of the loop.  Tokens a request
+        # produced after its end-of-sequence token are dropped; a waiting request is admitted up
+        # to that many steps later than it could have been.
+        self.decode_steps_per_launch = decode_steps_per_launch
         self._ids = itertools.count()
         self._waiting: deque[_Waiting] = deque()
         self._running: list[_Running] = []
@@ -149,6 +157,10 @@ class BatchScheduler:
         events: list[tuple[int, GenerationEvent]] = []
         try:
             self._admit(events)
+            steps = self._decode_steps_ahead()
+            if steps > 1:
+                self._decode_several(steps, events)
+                return events
             entries, rows = self._build_batch()
             if entries:
                 started = self._now()
@@ -211,6 +223,37 @@ class BatchScheduler:
         if log:
             self.step_log.append(log)
         return entries, rows
+
+    def _decode_steps_ahead(self) -> int:
+        """How many decode steps the next launch may hold: more than one only if every running request
+        is decoding greedily and the step function can feed tokens back in by itself; never more than
+        any request has left to produce."""
+        if self.decode_steps_per_launch <= 1 or not self._running or not hasattr(self.runner, "decode_steps"):
+            return 1
+        if any(r.next_token is None or not r.sampling.greedy for r in self._running):
+            return 1
+        steps = min(self.decode_steps_per_launch, min(r.output_limit - r.produced for r in self._running))
+        if steps <= 1:
+            return 1
+        entries = [StepEntry(r.cache, [r.next_token], [0]) for r in self._running]
+        return steps if self.runner.can_decode_steps(entries) else 1
+
+    def _decode_several(self, steps: int, events) -> None:
+        running = list(self._running)
+        entries = [StepEntry(r.cache, [r.next_token], [0]) for r in running]
+        started = self._now()
+        chosen = self.runner.decode_steps(entries, steps)
+        seconds = (self._now() - started) / steps if started is not None else None
+        alive = running
+        for tokens in chosen:
+            if not alive:
+                break
+            by_request = dict(zip(map(id, running), tokens))
+            self.step_log.append([(r.index, 1) for r in alive])
+            rows = [(r, None) for r in alive]
+            self._finish_step(rows, [by_request[id(r)] for r in alive], seconds, events)
+            still = {id(r) for r in self._running}
+            alive = [r for r in alive if id(r) in still]
 
     def _finish_step(self, rows, tokens, seconds, events) -> None:
         finished = set()

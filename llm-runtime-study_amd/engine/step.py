@@ -93,7 +93,7 @@ class StepContext:
         self.host_slots: list[int] = []
         self.host_positions: list[int] = []   # first position of each request's tokens in this step
         self.token_ids = self.positions = self.token_request = self.logit_rows = None
-        self.cu_seqlens_q = self.seq_lens_k = self.slot_ids = None
+        self.cu_seqlens_q = self.seq_lens_k = self.slot_ids = self.counts = None
         self._groups: list[GroupStep] = []
 
     def scratch(self, name: str, shape: tuple, dtype: torch.dtype) -> torch.Tensor:
@@ -141,6 +141,7 @@ class ModelRunner:
         self._host_np = self._host.numpy()
         self._dev = torch.zeros(cursor, dtype=torch.int32, device=self.device)
         self._views: dict[tuple, tuple] = {}
+        self._chosen_dev = self._chosen_host = None   # tokens chosen on the device by decode_steps()
         self._counting = np.arange(max(max_step_tokens, self.max_requests) + 1, dtype=np.int32)
         self.steps_run = 0
 
@@ -153,7 +154,7 @@ class ModelRunner:
             qblocks = -(-tokens // 16) + requests
             parts = [("token_ids", tokens), ("positions", tokens), ("token_request", tokens), ("logit_rows", tokens),
                      ("cu_seqlens_q", requests + 1), ("seq_lens_k", requests), ("slot_ids", requests),
-                     ("qblock_token0", qblocks), ("qblock_count", qblocks)]
+                     ("qblock_token0", qblocks), ("qblock_count", qblocks), ("counts", 4)]
             for index in range(len(self.cache.groups)):
                 parts += [(f"slots{index}", tokens), (f"table{index}", requests * self.cache.max_blocks)]
             for name, size in parts:
@@ -279,6 +280,7 @@ class ModelRunner:
             rows[:cursor] = np.arange(cursor, dtype=np.int32)
             n_rows = cursor
         ctx.T, ctx.R, ctx.num_logit_rows = cursor, max(real, pad_to), n_rows
+        self._host_view("counts")[0] = real          # rows that belong to requests (the others pad a graph's batch)
         # groups of consecutive tokens of one request, the longest contexts first
         if ctx.all_decode:
             ctx.num_qblocks, ctx.max_qblock = cursor, 1
@@ -320,11 +322,11 @@ class ModelRunner:
                 self._view("token_ids", ctx.T), self._view("positions", ctx.T), self._view("token_request", ctx.T),
                 self._view("logit_rows", max(ctx.num_logit_rows, 1)), self._view("cu_seqlens_q", ctx.R + 1),
                 self._view("seq_lens_k", ctx.R), self._view("slot_ids", ctx.R), self._view("qblock_token0", ctx.num_qblocks),
-                self._view("qblock_count", ctx.num_qblocks),
+                self._view("qblock_count", ctx.num_qblocks), self._view("counts", 4),
                 [GroupStep(self._view(f"slots{i}", ctx.T), self._view(f"table{i}").view(ctx.R, mb), self.cache.page_size)
                  for i in range(len(self.cache.groups))])
         (ctx.token_ids, ctx.positions, ctx.token_request, ctx.logit_rows, ctx.cu_seqlens_q, ctx.seq_lens_k, ctx.slot_ids,
-         ctx.qblock_token0, ctx.qblock_count, ctx._groups) = views
+         ctx.qblock_token0, ctx.qblock_count, ctx.counts, ctx._groups) = views
 
     def step(self, entries: Sequence[StepEntry]) -> torch.Tensor | None:
         """Run one step; returns float32 logits [wanted, vocab] on the device, or None if none is wanted."""
@@ -351,6 +353,99 @@ class ModelRunner:
             self.cache.trim(entry.cache)
         self.steps_run += 1
         return logits
+
+    # ------------------------------------------------- several decode steps, one launch
+    MAX_DECODE_STEPS = 8
+
+    def can_decode_steps(self, entries: Sequence[StepEntry]) -> bool:
+        """Whether decode_steps() takes these entries: one token each, and a graph for their number."""
+        return self._graph_bucket(entries) > 0
+
+    def decode_steps(self, entries: Sequence[StepEntry], steps: int) -> list[list[int]]:
+        """`steps` greedy decode steps of the same requests from one graph launch.
+
+        Each entry brings the one token its request decodes next.  After every step the device itself
+        picks the largest logit of every row, feeds it in as the next token and moves the step's
+        metadata one position on, so the host is not in the loop between steps.  Returns the chosen
+        tokens [steps][entries]; every request's cache is `steps` tokens longer afterwards (the caller
+        rolls back what it does not keep)."""
+        if not 1 <= steps <= self.MAX_DECODE_STEPS:
+            raise GenerationError(f"decode_steps takes 1..{self.MAX_DECODE_STEPS} steps, got {steps}")
+        self.validate(entries)
+        bucket = self._graph_bucket(entries)
+        if not bucket:
+            raise GenerationError("decode_steps needs graphs and one token per entry")
+        before = [entry.cache.length for entry in entries]
+        extended = []
+        try:
+            for entry in entries:
+                self.cache.extend(entry.cache, 1)
+                extended.append(entry)
+            ctx = self.prepare(entries, pad_to=bucket)
+            if steps > 1:
+                for entry in entries:                           # pages of the later positions: the block tables must hold them
+                    self.cache.extend(entry.cache, steps - 1)
+                self._refresh_tables(entries, bucket)
+            chosen = self._run_decode_graph(ctx, bucket, steps)
+        except Exception:
+            for entry, length in zip(extended, before):
+                if not entry.cache.released:
+                    self.cache.rollback(entry.cache, length)
+            raise
+        for entry in entries:
+            self.cache.trim(entry.cache)
+        self.steps_run += steps
+        return [row[:len(entries)] for row in chosen]
+
+    def _refresh_tables(self, entries: Sequence[StepEntry], bucket: int) -> None:
+        """Block tables of the step's requests written again (after pages were added) and uploaded."""
+        mb = self.cache.max_blocks
+        slots = [entry.cache.slot for entry in entries]
+        for index, group in enumerate(self.cache.groups):
+            self._host_view(f"table{index}").reshape(bucket, mb)[:len(entries)] = group.host_table[slots]
+        self._upload()
+
+    def _run_decode_graph(self, ctx: StepContext, bucket: int, steps: int) -> list[list[int]]:
+        key = (bucket, length_class(ctx.max_k), steps)
+        if self._chosen_dev is None:
+            rows = self.MAX_DECODE_STEPS * (-(-self.max_requests // 4) * 4)
+            self._chosen_dev = torch.zeros(rows, dtype=torch.int32, device=self.device)
+            self._chosen_host = torch.zeros(rows, dtype=torch.int32, pin_memory=True)
+        stride = -(-self.max_requests // 4) * 4                    # rows of 16 bytes and more
+        graph = self._graphs.get(key)
+        if graph is None or graph[1] != self.arena.generation:
+            if graph is not None:
+                ops.graph_destroy(graph[0])
+                del self._graphs[key]
+            self._decode_steps_on_stream(ctx, steps, stride)       # an eager run first: it sizes every scratch buffer
+            generation = self.arena.generation
+            ops.graph_begin()
+            try:
+                self._decode_steps_on_stream(ctx, steps, stride)
+            finally:
+                handle = ops.graph_end()
+            if self.arena.generation != generation:
+                ops.graph_destroy(handle)
+                raise GenerationError("scratch buffers moved during graph capture")
+            graph = self._graphs[key] = (handle, generation, None)
+            self._upload()                                         # the eager run moved the metadata on: start again
+        ops.graph_launch(graph[0])
+        self.graph_replays += 1
+        torch.cuda.current_stream(self.device).synchronize()
+        return [self._chosen_host[i * stride:i * stride + bucket].tolist() for i in range(steps)]
+
+    def _decode_steps_on_stream(self, ctx: StepContext, steps: int, stride: int) -> None:
+        for i in range(steps):
+            ctx.memo.clear()                                       # position tables are made again for the new positions
+            h = self.model.forward_hidden(ctx)
+            logits = self.model.logits(ctx, h)
+            chosen = self._chosen_dev[i * stride:i * stride + ctx.T]
+            ops.choose_tokens(chosen, logits)
+            if i + 1 < steps:
+                ops.advance_decode(ctx.token_ids, ctx.positions, ctx.token_request, ctx.seq_lens_k, chosen, ctx.counts)
+                for group in ctx._groups:
+                    ops.advance_slots(group.slots, ctx.positions, ctx.token_request, group.block_table, group.page_size, ctx.counts)
+        ops.copy_to_pinned(self._chosen_host, self._chosen_dev, steps * stride)
 
     # ------------------------------------------------------------------ graphs
     def _graph_bucket(self, entries: Sequence[StepEntry]) -> int:
@@ -401,6 +496,6 @@ class ModelRunner:
         return logits[:len(entries)] if len(wanted) == len(entries) else logits[wanted]
 
     def drop_graphs(self) -> None:
-        for handle, _, _ in self._graphs.values():
+        for handle, *_ in self._graphs.values():
             ops.graph_destroy(handle)
         self._graphs.clear()

@@ -47,6 +47,9 @@ _SIGNATURES = {
     "lrs_gemm_norm_chain_parts": (c_int, [c_int]),
     "lrs_scale_rows": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_float, c_void_p]),
     "lrs_gemm_skinny_max_m": (c_int, []),
+    "lrs_advance_decode": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p]),
+    "lrs_advance_slots": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p, c_int, c_void_p]),
+    "lrs_copy_to_pinned": (c_int, [c_void_p, c_void_p, c_int64, c_void_p]),
     "lrs_gemm_prepare": (c_int, []),
     "lrs_host_device_pointer": (c_int, [c_void_p, POINTER(c_void_p)]),
     "lrs_gemm_set_skinny_max_m": (c_int, [c_int]),
@@ -181,6 +184,14 @@ def copy_h2d(dst: torch.Tensor, src: torch.Tensor, count: int) -> None:
     _check(library().lrs_copy_h2d(_dev(dst, "dst"), src.data_ptr(), count * src.element_size(), _stream()))
 
 
+def copy_to_pinned(dst: torch.Tensor, src: torch.Tensor, count: int) -> None:
+    """The first `count` elements of device `src` into pinned host `dst`, by a kernel (the host reads
+    them after synchronising the stream).  count * element size must be a multiple of 16."""
+    _need(dst.device.type == "cpu" and dst.is_contiguous() and src.is_contiguous(), "copy_to_pinned needs a contiguous pinned host destination and a contiguous source")
+    _need(src.dtype == dst.dtype and 0 < count <= src.numel() and count <= dst.numel(), "copy_to_pinned: size or dtype mismatch")
+    _check(library().lrs_copy_to_pinned(dst.data_ptr(), _dev(src, "src"), count * src.element_size(), _stream()))
+
+
 # ------------------------------------------------------------ elementwise
 def embed(out: torch.Tensor, table: torch.Tensor, ids: torch.Tensor, multiplier: float = 1.0) -> None:
     tokens, hidden = out.shape
@@ -271,6 +282,31 @@ def skinny_max_m() -> int:
 def set_skinny_max_m(m: int) -> None:
     """Move the row count from which products go to the vendor library (1..64)."""
     _check(library().lrs_gemm_set_skinny_max_m(m))
+
+
+def _int_vector(t: torch.Tensor, name: str, at_least: int) -> int:
+    _need(t.dtype == torch.int32 and t.is_contiguous() and t.numel() >= at_least, f"{name} must be contiguous int32 with at least {at_least} elements")
+    return _dev(t, name)
+
+
+def advance_decode(token_ids: torch.Tensor, positions: torch.Tensor, token_request: torch.Tensor, seq_lens: torch.Tensor,
+                   chosen: torch.Tensor, real_rows: torch.Tensor) -> None:
+    """A decode step's metadata moved on to the next step, on the device: the first real_rows[0] rows
+    take the tokens in `chosen`, move one position on and lengthen their requests by one."""
+    rows = token_ids.numel()
+    _check(library().lrs_advance_decode(_int_vector(token_ids, "token_ids", rows), _int_vector(positions, "positions", rows),
+                                        _int_vector(token_request, "token_request", rows), _int_vector(seq_lens, "seq_lens", 1),
+                                        _int_vector(chosen, "chosen", rows), _int_vector(real_rows, "real_rows", 1), rows, _stream()))
+
+
+def advance_slots(slots: torch.Tensor, positions: torch.Tensor, token_request: torch.Tensor, block_table: torch.Tensor,
+                  page_size: int, real_rows: torch.Tensor) -> None:
+    """The cache slots of the (already advanced) positions of the first real_rows[0] rows, from the block table."""
+    rows = slots.numel()
+    _need(block_table.dim() == 2 and block_table.dtype == torch.int32 and block_table.stride(1) == 1, "advance_slots: block_table must be int32 [R, blocks]")
+    _check(library().lrs_advance_slots(_int_vector(slots, "slots", rows), _int_vector(positions, "positions", rows),
+                                       _int_vector(token_request, "token_request", rows), _dev(block_table, "block_table"),
+                                       block_table.stride(0), page_size, _int_vector(real_rows, "real_rows", 1), rows, _stream()))
 
 
 def fill_i32(dst: torch.Tensor, value: int) -> None:

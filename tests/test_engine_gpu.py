@@ -160,6 +160,60 @@ def test_graph_replay_equals_eager_steps(folders, name, dtype, lengths):
     graphed.drop_graphs()
 
 
+@pytest.mark.parametrize("name", ["b", "c"])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_several_decode_steps_from_one_launch_equal_single_steps(folders, name, dtype):
+    """decode_steps(): the device chooses each token, feeds it back in and moves the metadata on by
+    itself.  Tokens and cache contents must equal those of single steps with the host in the loop,
+    across page edges (page size 16, contexts from 3 to 70) and with fewer requests than the padded batch."""
+    from llm_runtime_study_amd.cache import CacheManager
+    from llm_runtime_study_amd.engine.loading import load_model
+    from llm_runtime_study_amd.engine.step import ModelRunner, StepEntry
+
+    folder, cfg, _ = folders[name]
+    device = torch.device("cuda", 0)
+    _, model = load_model(folder, dtype, device)
+    rng = np.random.default_rng(12)
+    prompts = [rng.integers(0, cfg["vocab_size"], n).tolist() for n in (3, 30, 61)]
+
+    def make():
+        cache = CacheManager(model.cache_needs(), page_size=16, num_pages=40, max_requests=4, max_seq_len=256, dtype=dtype, device=device)
+        return ModelRunner(model, cache, max_step_tokens=128, dtype=dtype, device=device, use_graph=True)
+
+    single, several = make(), make()
+    with torch.cuda.stream(torch.cuda.Stream(device)):
+        state = []
+        for runner in (single, several):
+            caches, last = [], []
+            for i, prompt in enumerate(prompts):
+                caches.append(runner.cache.admit(i))
+                last.append(int(runner.step([StepEntry(caches[-1], prompt, [len(prompt) - 1])])[0].argmax()))
+            state.append((caches, last))
+        assert state[0][1] == state[1][1]
+        assert several.can_decode_steps([StepEntry(c, [t], [0]) for c, t in zip(*state[1])])
+        want, got = [], []
+        caches, last = state[0]
+        for _ in range(9):
+            logits = single.step([StepEntry(c, [t], [0]) for c, t in zip(caches, last)])
+            last = logits.argmax(-1).tolist()
+            want.append(last)
+        caches, last = state[1]
+        for steps in (4, 1, 4):
+            chosen = several.decode_steps([StepEntry(c, [t], [0]) for c, t in zip(caches, last)], steps)
+            assert len(chosen) == steps and all(len(row) == len(prompts) for row in chosen)
+            got += chosen
+            last = chosen[-1]
+        torch.cuda.synchronize()
+    assert got == want
+    assert [c.length for c in state[0][0]] == [c.length for c in state[1][0]] == [len(p) + 9 for p in prompts]
+    for a, b in zip(single.cache.layer_caches, several.cache.layer_caches):
+        for request_a, request_b in zip(state[0][0], state[1][0]):
+            pages_a, pages_b = request_a.tables[a.group], request_b.tables[b.group]
+            assert torch.equal(a.k_pages[pages_a], b.k_pages[pages_b]) and torch.equal(a.v_pages[pages_a], b.v_pages[pages_b])
+    several.drop_graphs()
+    single.drop_graphs()
+
+
 def test_seeded_sampling_is_reproducible_and_independent_of_batch_mates(folders):
     from llm_runtime_study_amd import Engine, SamplingConfig
 

@@ -207,3 +207,71 @@ def test_sampling_rows_carry_each_requests_own_seed_and_counter():
     s.add_request([2, 2], max_new_tokens=2, sampling=SamplingConfig(temperature=0.5, seed=12))
     drain(s)
     assert seen == [[(11, 0, 0.8), (12, 0, 0.5)], [(11, 1, 0.8), (12, 1, 0.5)], [(11, 2, 0.8)]]
+
+
+class SeveralStepsRunner(FakeRunner):
+    """A fake step function that can also run several greedy decode steps from one call, as the real
+    one does on the device: it extends every cache by that many tokens and reports what each step chose."""
+
+    def __init__(self, *args, **kwargs):
+        super().__init__(*args, **kwargs)
+        self.launches = []
+
+    def can_decode_steps(self, entries):
+        return all(len(e.tokens) == 1 for e in entries)
+
+    def decode_steps(self, entries, steps):
+        self.launches.append((steps, [e.cache.request_id for e in entries]))
+        chosen = []
+        for e in entries:
+            self.cache.extend(e.cache, steps)
+        for _ in range(steps):
+            row = []
+            for e in entries:
+                k = self.produced.get(e.cache.request_id, 0)
+                self.produced[e.cache.request_id] = k + 1
+                script = self.script[e.cache.request_id]
+                row.append(script[k] if k < len(script) else 0)
+            chosen.append(row)
+        self.cache.check_invariants()
+        return chosen
+
+
+def test_several_decode_steps_per_launch_give_the_same_events():
+    script = {0: [7, 8, 9, 10, 11, 12, 13], 1: [20, 21, 1, 22, 23, 24, 25]}     # request 1 meets eos (1) as its third token
+
+    def run(per_launch):
+        runner = SeveralStepsRunner(script)
+        s = scheduler(runner, decode_steps_per_launch=per_launch)
+        s.add_request([3, 4, 5], max_new_tokens=7)
+        s.add_request([6, 2], max_new_tokens=7)
+        events = [(i, e.token_id, e.token_index, e.finish_reason) for i, e in drain(s)]
+        assert runner.cache.active_requests == 0 and runner.cache.used_pages() == 0
+        return events, runner, s
+
+    single, _, log_single = run(1)
+    several, runner, log_several = run(4)
+    assert sorted(single) == sorted(several)
+    assert [t for i, t, _, _ in several if i == 1] == [20, 21, 1]               # nothing after the end-of-sequence token
+    assert [t for i, t, _, _ in several if i == 0] == [7, 8, 9, 10, 11, 12, 13]
+    # prompts run as ordinary steps; then launches of 4 steps for both, and what is left for request 0 alone
+    assert runner.launches == [(4, [0, 1]), (2, [0])]
+    assert log_single.step_log == log_several.step_log
+
+
+def test_several_decode_steps_need_greedy_requests_and_room():
+    script = {0: [7, 8, 9, 10], 1: [20, 21, 22, 23]}
+    runner = SeveralStepsRunner(script)
+    s = scheduler(runner, decode_steps_per_launch=4)
+    s.add_request([3, 4], max_new_tokens=4, sampling=SamplingConfig(temperature=0.7, seed=1))
+    s.add_request([5], max_new_tokens=4)
+    drain(s)
+    assert runner.launches == []                                                # a sampled request keeps the host in the loop
+    runner = SeveralStepsRunner(script)
+    s = scheduler(runner, decode_steps_per_launch=8)
+    s.add_request([3, 4], max_new_tokens=4)
+    s.add_request([5], max_new_tokens=3)
+    drain(s)
+    assert runner.launches == [(2, [0, 1])]                                     # never more steps than the shortest has left
+    with pytest.raises(GenerationError, match="decode_steps_per_launch"):
+        scheduler(FakeRunner(script), decode_steps_per_launch=0)
