@@ -111,7 +111,8 @@ def linear(ctx, out, x, weight, bias=None, accumulate: bool = False, swiglu: boo
         x = x.materialize(ctx)
     m, n = x.shape[0], weight.shape[0]
     if (getattr(ctx, "library_gemm", False) and weight.dtype == torch.bfloat16 and x.dtype == torch.bfloat16 and m > ops.skinny_max_m()
-            and bias is None and x.is_contiguous() and (accumulate or (out.dtype == torch.bfloat16 and out.is_contiguous()))):
+            and bias is None and x.is_contiguous() and (accumulate or (out.dtype in (torch.bfloat16, torch.float32) and out.is_contiguous()))
+            and not (swiglu and out.dtype != torch.bfloat16)):
         if accumulate or swiglu:
             y = ctx.scratch("library_gemm_out", (m, n), torch.bfloat16)
             torch.mm(x, weight.t(), out=y)
@@ -126,6 +127,8 @@ def linear(ctx, out, x, weight, bias=None, accumulate: bool = False, swiglu: boo
                 ops.add_into(out, y)
             else:
                 ops.silu_mul(out, y, interleaved=True)
+        elif out.dtype == torch.float32:
+            torch.mm(x, weight.t(), out_dtype=torch.float32, out=out)     # float32 logits of many rows
         else:
             torch.mm(x, weight.t(), out=out)
         return None
