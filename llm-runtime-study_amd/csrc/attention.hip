@@ -270,47 +270,54 @@ __global__ __launch_bounds__(256) void attention_decode_bf16_kernel(
   const float scale2 = scale * 1.4426950408889634f;
 
   // Every key and value fragment of a tile is requested before any is used, so a tile costs one
-  // trip to memory instead of two.
+  // trip to memory instead of two.  Which of the tile's 32 keys a row of the two key blocks stands
+  // for is chosen so that a lane ends up with the weights of eight consecutive keys, g*8 .. g*8+7:
+  // block h, row 4*r + i is key 8*r + 4*h + i.  The values of those eight keys lie side by side in
+  // the (transposed) page, one 16-byte load a dim.
+  const int key_of_row = (col >> 2) * 8 + (col & 3);           // + 4*h
   for (int tile = tile_begin + wave; tile < tile_end; tile += WAVES) {
-    bool present[2];
     bf16x8 kf[2][DS];
-    bf16x4 vf[2][DB];
+    bf16x8 vf[DB];
 #pragma unroll
     for (int h = 0; h < 2; ++h) {
-      const int key0 = tile * 32 + h * 16;
-      present[h] = key0 <= pos && key0 + 15 >= lo;
-      if (present[h]) {
-        const int64_t page = page_ids[key0 / page_size - first_block];
-        const int off = key0 % page_size;
-        const bf16* kp = k_pages + ((page * nkv + kvh) * page_size + off + col) * D + g * 8;
-        const bf16* vp = v_pages + (page * nkv + kvh) * (int64_t)D * page_size + off + (int64_t)col * page_size + g * 4;
+      const int key = tile * 32 + key_of_row + 4 * h;
+      if (key <= pos && key >= lo) {
+        const int64_t page = page_ids[key / page_size - first_block];
+        const bf16* kp = k_pages + ((page * nkv + kvh) * page_size + key % page_size) * D + g * 8;
 #pragma unroll
         for (int c = 0; c < DS; ++c) kf[h][c] = *(const bf16x8*)(kp + c * 32);
-#pragma unroll
-        for (int b = 0; b < DB; ++b) vf[h][b] = *(const bf16x4*)(vp + (int64_t)b * 16 * page_size);
       } else {
 #pragma unroll
         for (int c = 0; c < DS; ++c) kf[h][c] = zero8;
+      }
+    }
+    {
+      const int key8 = tile * 32 + g * 8;                      // this lane's eight keys; pages hold multiples of 16
+      if (key8 <= pos && key8 + 7 >= lo) {
+        const int64_t page = page_ids[key8 / page_size - first_block];
+        const bf16* vp = v_pages + (page * nkv + kvh) * (int64_t)D * page_size + (int64_t)col * page_size + key8 % page_size;
 #pragma unroll
-        for (int b = 0; b < DB; ++b) vf[h][b] = bf16x4{0, 0, 0, 0};
+        for (int b = 0; b < DB; ++b) vf[b] = *(const bf16x8*)(vp + (int64_t)b * 16 * page_size);
+      } else {
+#pragma unroll
+        for (int b = 0; b < DB; ++b) vf[b] = zero8;
       }
     }
     if (holds_own && tile == last_tile) {
       // the token's own key and value take the place of what the pages hold at its position
-      const int own_half = (pos % 32) / 16, own_col = pos % 16, own_g = (pos % 16) / 4, own_i = pos % 4;
+      const int own = pos % 32;
+      const int own_h = (own % 8) / 4, own_col = (own / 8) * 4 + own % 4, own_g = own / 8, own_j = own % 8;
 #pragma unroll
       for (int h = 0; h < 2; ++h)
 #pragma unroll
         for (int c = 0; c < DS; ++c)
-          if (h == own_half && col == own_col) kf[h][c] = *(const bf16x8*)&own_k[c * 32 + g * 8];
+          if (h == own_h && col == own_col) kf[h][c] = *(const bf16x8*)&own_k[c * 32 + g * 8];
 #pragma unroll
       for (int b = 0; b < DB; ++b) {
         const bf16 vn = own_v[b * 16 + col];
 #pragma unroll
-        for (int h = 0; h < 2; ++h)
-#pragma unroll
-          for (int i = 0; i < 4; ++i)
-            if (h == own_half && g == own_g && i == own_i) vf[h][b][i] = vn;
+        for (int j = 0; j < 8; ++j)
+          if (g == own_g && j == own_j) vf[b][j] = vn;
       }
     }
     floatx4 s[2];
@@ -325,8 +332,8 @@ __global__ __launch_bounds__(256) void attention_decode_bf16_kernel(
     for (int h = 0; h < 2; ++h)
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        const int key = tile * 32 + h * 16 + g * 4 + i;
-        const bool valid = present[h] && key <= pos && key >= lo;
+        const int key = tile * 32 + g * 8 + h * 4 + i;
+        const bool valid = key <= pos && key >= lo;
         s[h][i] = valid ? s[h][i] * scale2 : -INFINITY;
         tile_max = fmaxf(tile_max, s[h][i]);
       }
@@ -349,10 +356,8 @@ __global__ __launch_bounds__(256) void attention_decode_bf16_kernel(
     const bool rescale = __any(alpha != 1.f);
 #pragma unroll
     for (int b = 0; b < DB; ++b) {
-      const bf16x4 v0 = vf[0][b], v1 = vf[1][b];
-      const bf16x8 vv = {v0[0], v0[1], v0[2], v0[3], v1[0], v1[1], v1[2], v1[3]};
       if (rescale) o[b] *= alpha;
-      o[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vv, pf, o[b], 0, 0, 0);
+      o[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[b], pf, o[b], 0, 0, 0);
     }
   }
   run_sum += __shfl_xor(run_sum, 16, WAVE);
