@@ -526,15 +526,18 @@ LRS_API int lrs_scale_rows(void* out, const void* x, const float* sumsq, int par
 // ---------------------------------------------------- next decode step's metadata
 // Several decode steps can run from one launch: between two of them the step's metadata is moved
 // on by the device itself.  Each of the first *real_rows rows (the others pad the batch) takes the
-// token just chosen for it, moves one position on and lengthens its request by one ...
+// token just chosen for it, moves one position on, lengthens its request by one and counts the draw
+// (`draws`, optional: the per-row counters of seeded sampling) ...
 __global__ void advance_decode_kernel(int* __restrict__ token_ids, int* __restrict__ positions,
                                       const int* __restrict__ token_request, int* __restrict__ seq_lens,
-                                      const int* __restrict__ chosen, const int* __restrict__ real_rows, int rows) {
+                                      const int* __restrict__ chosen, int* __restrict__ draws,
+                                      const int* __restrict__ real_rows, int rows) {
   const int t = blockIdx.x * blockDim.x + threadIdx.x;
   if (t >= rows || t >= *real_rows) return;
   token_ids[t] = chosen[t];
   positions[t] += 1;
   seq_lens[token_request[t]] += 1;
+  if (draws) draws[t] += 1;
 }
 
 // ... and, per cache group, finds the slot of its new position in its request's block table.
@@ -549,9 +552,9 @@ __global__ void advance_slots_kernel(int* __restrict__ slots, const int* __restr
 }
 
 LRS_API int lrs_advance_decode(int* token_ids, int* positions, const int* token_request, int* seq_lens, const int* chosen,
-                               const int* real_rows, int rows, void* stream) {
+                               int* draws, const int* real_rows, int rows, void* stream) {
   LRS_REQUIRE(rows > 0 && token_ids && positions && token_request && seq_lens && chosen && real_rows, "advance_decode: missing arrays or no rows");
-  advance_decode_kernel<<<(rows + 255) / 256, 256, 0, (hipStream_t)stream>>>(token_ids, positions, token_request, seq_lens, chosen, real_rows, rows);
+  advance_decode_kernel<<<(rows + 255) / 256, 256, 0, (hipStream_t)stream>>>(token_ids, positions, token_request, seq_lens, chosen, draws, real_rows, rows);
   return lrs_check_launch("advance_decode");
 }
 

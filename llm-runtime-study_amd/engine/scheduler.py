@@ -94,8 +94,8 @@ class BatchScheduler:
         self._synchronize = synchronize
         if decode_steps_per_launch < 1:
             raise GenerationError(f"decode_steps_per_launch must be at least 1, got {decode_steps_per_launch}")
-        # When every running request decodes greedily, up to this many steps run from one launch
-        # (the step function feeds each chosen token back in on the device): the host, which needs
+        # When every running request decodes, up to this many steps run from one launch (the step
+        # function chooses each token and feeds it back in on the device): the host, which needs
         # about a tenth of a millisecond between steps, is then out of the loop.  Tokens a request
         # produced after its end-of-sequence token are dropped; a waiting request is admitted up
         # to that many steps later than it could have been.
@@ -226,11 +226,13 @@ class BatchScheduler:
 
     def _decode_steps_ahead(self) -> int:
         """How many decode steps the next launch may hold: more than one only if every running request
-        is decoding greedily and the step function can feed tokens back in by itself; never more than
-        any request has left to produce."""
+        is decoding and the step function can choose tokens and feed them back in by itself (all
+        greedy, unless it also samples); never more than any request has left to produce."""
         if self.decode_steps_per_launch <= 1 or not self._running or not hasattr(self.runner, "decode_steps"):
             return 1
-        if any(r.next_token is None or not r.sampling.greedy for r in self._running):
+        if any(r.next_token is None for r in self._running):
+            return 1
+        if not getattr(self.runner, "decode_steps_sample", False) and any(not r.sampling.greedy for r in self._running):
             return 1
         steps = min(self.decode_steps_per_launch, min(r.output_limit - r.produced for r in self._running))
         if steps <= 1:
@@ -242,7 +244,10 @@ class BatchScheduler:
         running = list(self._running)
         entries = [StepEntry(r.cache, [r.next_token], [0]) for r in running]
         started = self._now()
-        chosen = self.runner.decode_steps(entries, steps)
+        if getattr(self.runner, "decode_steps_sample", False):
+            chosen = self.runner.decode_steps(entries, steps, [SamplingRow(r.sampling, r.seed, r.produced) for r in running])
+        else:
+            chosen = self.runner.decode_steps(entries, steps)
         seconds = (self._now() - started) / steps if started is not None else None
         alive = running
         for tokens in chosen:

@@ -142,6 +142,7 @@ class ModelRunner:
         self._dev = torch.zeros(cursor, dtype=torch.int32, device=self.device)
         self._views: dict[tuple, tuple] = {}
         self._chosen_dev = self._chosen_host = None   # tokens chosen on the device by decode_steps()
+        self._sampling_dev = self._sampling_host = None
         self._counting = np.arange(max(max_step_tokens, self.max_requests) + 1, dtype=np.int32)
         self.steps_run = 0
 
@@ -361,14 +362,17 @@ class ModelRunner:
         """Whether decode_steps() takes these entries: one token each, and a graph for their number."""
         return self._graph_bucket(entries) > 0
 
-    def decode_steps(self, entries: Sequence[StepEntry], steps: int) -> list[list[int]]:
-        """`steps` greedy decode steps of the same requests from one graph launch.
+    decode_steps_sample = True     # decode_steps() also draws from filtered, tempered distributions
+
+    def decode_steps(self, entries: Sequence[StepEntry], steps: int, sampling: Sequence | None = None) -> list[list[int]]:
+        """`steps` decode steps of the same requests from one graph launch.
 
         Each entry brings the one token its request decodes next.  After every step the device itself
-        picks the largest logit of every row, feeds it in as the next token and moves the step's
-        metadata one position on, so the host is not in the loop between steps.  Returns the chosen
-        tokens [steps][entries]; every request's cache is `steps` tokens longer afterwards (the caller
-        rolls back what it does not keep)."""
+        chooses a token for every row (the largest logit; or, for the rows whose entry of `sampling`,
+        a list of sampling.SamplingRow, says so, a seeded draw after top-k / top-p filtering, exactly
+        as Sampler.choose would), feeds it in as the next token and moves the step's metadata one
+        position on, so the host is not in the loop between steps.  Returns the chosen tokens
+        [steps][entries]; every request's cache is `steps` tokens longer afterwards."""
         if not 1 <= steps <= self.MAX_DECODE_STEPS:
             raise GenerationError(f"decode_steps takes 1..{self.MAX_DECODE_STEPS} steps, got {steps}")
         self.validate(entries)
@@ -386,7 +390,12 @@ class ModelRunner:
                 for entry in entries:                           # pages of the later positions: the block tables must hold them
                     self.cache.extend(entry.cache, steps - 1)
                 self._refresh_tables(entries, bucket)
-            chosen = self._run_decode_graph(ctx, bucket, steps)
+            sampled = sampling is not None and any(not row.config.greedy for row in sampling)
+            if sampled:
+                if len(sampling) != len(entries):
+                    raise GenerationError("decode_steps needs one sampling row per entry")
+                self._upload_sampling(sampling)
+            chosen = self._run_decode_graph(ctx, bucket, steps, sampled)
         except Exception:
             for entry, length in zip(extended, before):
                 if not entry.cache.released:
@@ -405,8 +414,31 @@ class ModelRunner:
             self._host_view(f"table{index}").reshape(bucket, mb)[:len(entries)] = group.host_table[slots]
         self._upload()
 
-    def _run_decode_graph(self, ctx: StepContext, bucket: int, steps: int) -> list[list[int]]:
-        key = (bucket, length_class(ctx.max_k), steps)
+    def _upload_sampling(self, sampling: Sequence) -> None:
+        """Temperature, top-p, top-k, draws so far and seed of every row, in one buffer on the device
+        (rows beyond those given stay at temperature 0: the largest logit)."""
+        cap = -(-self.max_requests // 4) * 4
+        if self._sampling_host is None:
+            self._sampling_host = torch.zeros(6 * cap, dtype=torch.int32, pin_memory=True)
+            self._sampling_dev = torch.zeros(6 * cap, dtype=torch.int32, device=self.device)
+        host = self._sampling_host.numpy()
+        host[:] = 0
+        n = len(sampling)
+        host[:cap].view(np.float32)[:n] = [row.config.temperature for row in sampling]
+        host[cap:2 * cap].view(np.float32)[:n] = [row.config.top_p for row in sampling]
+        host[2 * cap:3 * cap][:n] = [row.config.top_k or 0 for row in sampling]
+        host[3 * cap:4 * cap][:n] = [row.counter for row in sampling]
+        host[4 * cap:6 * cap].view(np.int64)[:n] = [row.seed for row in sampling]
+        ops.copy_h2d(self._sampling_dev, self._sampling_host, 6 * cap)
+
+    def _sampling_views(self, rows: int):
+        cap = -(-self.max_requests // 4) * 4
+        dev = self._sampling_dev
+        return (dev[:cap].view(torch.float32)[:rows], dev[cap:2 * cap].view(torch.float32)[:rows], dev[2 * cap:3 * cap][:rows],
+                dev[3 * cap:4 * cap][:rows], dev[4 * cap:6 * cap].view(torch.int64)[:rows])
+
+    def _run_decode_graph(self, ctx: StepContext, bucket: int, steps: int, sampled: bool = False) -> list[list[int]]:
+        key = (bucket, length_class(ctx.max_k), steps, sampled)
         if self._chosen_dev is None:
             rows = self.MAX_DECODE_STEPS * (-(-self.max_requests // 4) * 4)
             self._chosen_dev = torch.zeros(rows, dtype=torch.int32, device=self.device)
@@ -417,11 +449,11 @@ class ModelRunner:
             if graph is not None:
                 ops.graph_destroy(graph[0])
                 del self._graphs[key]
-            self._decode_steps_on_stream(ctx, steps, stride)       # an eager run first: it sizes every scratch buffer
+            self._decode_steps_on_stream(ctx, steps, stride, sampled)   # an eager run first: it sizes every scratch buffer
             generation = self.arena.generation
             ops.graph_begin()
             try:
-                self._decode_steps_on_stream(ctx, steps, stride)
+                self._decode_steps_on_stream(ctx, steps, stride, sampled)
             finally:
                 handle = ops.graph_end()
             if self.arena.generation != generation:
@@ -429,20 +461,29 @@ class ModelRunner:
                 raise GenerationError("scratch buffers moved during graph capture")
             graph = self._graphs[key] = (handle, generation, None)
             self._upload()                                         # the eager run moved the metadata on: start again
+            if sampled:
+                ops.copy_h2d(self._sampling_dev, self._sampling_host, self._sampling_host.numel())
         ops.graph_launch(graph[0])
         self.graph_replays += 1
         torch.cuda.current_stream(self.device).synchronize()
         return [self._chosen_host[i * stride:i * stride + bucket].tolist() for i in range(steps)]
 
-    def _decode_steps_on_stream(self, ctx: StepContext, steps: int, stride: int) -> None:
+    def _decode_steps_on_stream(self, ctx: StepContext, steps: int, stride: int, sampled: bool) -> None:
+        draws = None
+        if sampled:
+            temperature, top_p, top_k, draws, seeds = self._sampling_views(ctx.T)
         for i in range(steps):
             ctx.memo.clear()                                       # position tables are made again for the new positions
             h = self.model.forward_hidden(ctx)
             logits = self.model.logits(ctx, h)
             chosen = self._chosen_dev[i * stride:i * stride + ctx.T]
-            ops.choose_tokens(chosen, logits)
+            if sampled:
+                ops.filter_logits(logits, temperature, top_k, top_p)
+                ops.choose_tokens(chosen, logits, temperature, seeds, draws)
+            else:
+                ops.choose_tokens(chosen, logits)
             if i + 1 < steps:
-                ops.advance_decode(ctx.token_ids, ctx.positions, ctx.token_request, ctx.seq_lens_k, chosen, ctx.counts)
+                ops.advance_decode(ctx.token_ids, ctx.positions, ctx.token_request, ctx.seq_lens_k, chosen, ctx.counts, draws)
                 for group in ctx._groups:
                     ops.advance_slots(group.slots, ctx.positions, ctx.token_request, group.block_table, group.page_size, ctx.counts)
         ops.copy_to_pinned(self._chosen_host, self._chosen_dev, steps * stride)

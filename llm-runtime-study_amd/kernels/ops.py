@@ -47,7 +47,7 @@ _SIGNATURES = {
     "lrs_gemm_norm_chain_parts": (c_int, [c_int]),
     "lrs_scale_rows": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_float, c_void_p]),
     "lrs_gemm_skinny_max_m": (c_int, []),
-    "lrs_advance_decode": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p]),
+    "lrs_advance_decode": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p]),
     "lrs_advance_slots": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p, c_int, c_void_p]),
     "lrs_copy_to_pinned": (c_int, [c_void_p, c_void_p, c_int64, c_void_p]),
     "lrs_gemm_prepare": (c_int, []),
@@ -290,13 +290,15 @@ def _int_vector(t: torch.Tensor, name: str, at_least: int) -> int:
 
 
 def advance_decode(token_ids: torch.Tensor, positions: torch.Tensor, token_request: torch.Tensor, seq_lens: torch.Tensor,
-                   chosen: torch.Tensor, real_rows: torch.Tensor) -> None:
+                   chosen: torch.Tensor, real_rows: torch.Tensor, draws: torch.Tensor | None = None) -> None:
     """A decode step's metadata moved on to the next step, on the device: the first real_rows[0] rows
-    take the tokens in `chosen`, move one position on and lengthen their requests by one."""
+    take the tokens in `chosen`, move one position on, lengthen their requests by one and (with
+    `draws`, the counters of seeded sampling) count one more draw."""
     rows = token_ids.numel()
     _check(library().lrs_advance_decode(_int_vector(token_ids, "token_ids", rows), _int_vector(positions, "positions", rows),
                                         _int_vector(token_request, "token_request", rows), _int_vector(seq_lens, "seq_lens", 1),
-                                        _int_vector(chosen, "chosen", rows), _int_vector(real_rows, "real_rows", 1), rows, _stream()))
+                                        _int_vector(chosen, "chosen", rows), None if draws is None else _int_vector(draws, "draws", rows),
+                                        _int_vector(real_rows, "real_rows", 1), rows, _stream()))
 
 
 def advance_slots(slots: torch.Tensor, positions: torch.Tensor, token_request: torch.Tensor, block_table: torch.Tensor,

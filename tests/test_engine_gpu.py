@@ -235,6 +235,38 @@ def test_seeded_sampling_is_reproducible_and_independent_of_batch_mates(folders)
     assert top1 == greedy      # only the largest logit survives the filter
 
 
+def test_sampled_tokens_do_not_depend_on_steps_per_launch(folders):
+    """Seeded draws with top-k and top-p, one request greedy beside them: four decode steps from one
+    launch (the device filters, draws and counts the draws itself) give the tokens of single steps."""
+    from llm_runtime_study_amd import Engine, SamplingConfig
+
+    folder, cfg, _ = folders["c"]
+    rng = np.random.default_rng(21)
+    prompts = [rng.integers(0, cfg["vocab_size"], n).tolist() for n in (9, 20, 4)]
+    configs = [SamplingConfig(temperature=0.9, top_k=40, top_p=0.9, seed=5), SamplingConfig(),
+               SamplingConfig(temperature=1.3, seed=77)]
+
+    def run(per_launch):
+        engine = Engine.from_model_dir(folder, dtype="bfloat16", max_seq_len=96, max_batch_size=3, decode_steps_per_launch=per_launch)
+        scheduler = engine.create_scheduler(ignore_eos=True)
+        for prompt, config in zip(prompts, configs):
+            scheduler.add_request(prompt, max_new_tokens=11, sampling=config)
+        tokens = {i: [] for i in range(len(prompts))}
+        with torch.cuda.device(engine.device), torch.cuda.stream(engine.stream):
+            while scheduler.has_unfinished:
+                for index, event in scheduler.step():
+                    tokens[index].append(event.token_id)
+        replays = engine.runner.graph_replays
+        engine.runner.drop_graphs()
+        return tokens, replays
+
+    single, replays_single = run(1)
+    several, replays_several = run(4)
+    assert single == several and all(len(t) == 11 for t in single.values())
+    assert len(set(single[0])) > 3 and len(set(single[2])) > 3        # draws, not a fixed point
+    assert replays_several < replays_single
+
+
 def test_small_pool_makes_requests_wait_and_reuses_pages(folders):
     from llm_runtime_study_amd import Engine
 

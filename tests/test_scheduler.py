@@ -215,13 +215,14 @@ class SeveralStepsRunner(FakeRunner):
 
     def __init__(self, *args, **kwargs):
         super().__init__(*args, **kwargs)
-        self.launches = []
+        self.launches, self.sampling_seen = [], []
 
     def can_decode_steps(self, entries):
         return all(len(e.tokens) == 1 for e in entries)
 
-    def decode_steps(self, entries, steps):
+    def decode_steps(self, entries, steps, sampling=None):
         self.launches.append((steps, [e.cache.request_id for e in entries]))
+        self.sampling_seen.append(None if sampling is None else [(row.config.temperature, row.seed, row.counter) for row in sampling])
         chosen = []
         for e in entries:
             self.cache.extend(e.cache, steps)
@@ -275,3 +276,13 @@ def test_several_decode_steps_need_greedy_requests_and_room():
     assert runner.launches == [(2, [0, 1])]                                     # never more steps than the shortest has left
     with pytest.raises(GenerationError, match="decode_steps_per_launch"):
         scheduler(FakeRunner(script), decode_steps_per_launch=0)
+    # a step function that also samples on the device is handed every request's temperature, seed and draws so far
+    runner = SeveralStepsRunner(script)
+    runner.decode_steps_sample = True
+    s = scheduler(runner, decode_steps_per_launch=2)
+    s.add_request([3, 4], max_new_tokens=4, sampling=SamplingConfig(temperature=0.7, seed=11))
+    s.add_request([5], max_new_tokens=4)
+    drain(s)
+    assert runner.launches == [(2, [0, 1])]
+    (first, second), = runner.sampling_seen
+    assert first == (0.7, 11, 1) and second[0] == 0.0 and second[2] == 1
