@@ -357,6 +357,7 @@ class ModelRunner:
 
     # ------------------------------------------------- several decode steps, one launch
     MAX_DECODE_STEPS = 8
+    LIBRARY_GRAPH_ROWS = 64     # largest padded batch whose step (with library matrix products) is captured
 
     def can_decode_steps(self, entries: Sequence[StepEntry]) -> bool:
         """Whether decode_steps() takes these entries: one token each, and a graph for their number."""
@@ -499,8 +500,10 @@ class ModelRunner:
         while bucket < len(entries):
             bucket *= 2
         bucket = min(bucket, self.max_requests)
-        # a graph holds this package's kernels only: batches the few-rows kernels do not take run eagerly
-        return bucket if bucket <= min(self.max_step_tokens, ops.skinny_max_m()) else 0
+        # Up to the rows the few-rows kernels take, a graph holds this package's kernels only; larger
+        # batches (up to 64 rows) bring the vendor library's products into the capture.
+        most = max(ops.skinny_max_m(), self.LIBRARY_GRAPH_ROWS) if self.library_gemm and self.dtype == torch.bfloat16 else ops.skinny_max_m()
+        return bucket if bucket <= min(self.max_step_tokens, most) else 0
 
     def _step_graph(self, entries: Sequence[StepEntry], bucket: int) -> torch.Tensor | None:
         """Replay (capturing first if needed) the graph of a decode step padded to `bucket` rows.

@@ -235,6 +235,56 @@ def test_seeded_sampling_is_reproducible_and_independent_of_batch_mates(folders)
     assert top1 == greedy      # only the largest logit survives the filter
 
 
+def test_graphs_of_large_batches_hold_library_products(folders):
+    """More rows than the few-rows kernels take: the vendor library's matrix products are captured
+    with the rest.  Every replay (24 of them, three padded sizes, eager prefill steps and
+    synchronisations between them) must give the logits of the same step run eagerly."""
+    from llm_runtime_study_amd.cache import CacheManager
+    from llm_runtime_study_amd.engine.loading import load_model
+    from llm_runtime_study_amd.engine.step import ModelRunner, StepEntry
+
+    folder, cfg, _ = folders["c"]
+    device, dtype = torch.device("cuda", 0), torch.bfloat16
+    _, model = load_model(folder, dtype, device)
+    rng = np.random.default_rng(31)
+
+    def make(use_graph):
+        cache = CacheManager(model.cache_needs(), page_size=16, num_pages=400, max_requests=64, max_seq_len=128, dtype=dtype, device=device)
+        return ModelRunner(model, cache, max_step_tokens=256, dtype=dtype, device=device, use_graph=use_graph)
+
+    eager, graphed = make(False), make(True)
+    live = {}
+
+    def admit(index):
+        prompt = rng.integers(0, cfg["vocab_size"], int(rng.integers(1, 40))).tolist()
+        caches = (eager.cache.admit(index), graphed.cache.admit(index))
+        a = eager.step([StepEntry(caches[0], prompt, [len(prompt) - 1])]).clone()
+        b = graphed.step([StepEntry(caches[1], prompt, [len(prompt) - 1])]).clone()
+        assert torch.equal(a, b)
+        live[index] = (caches, int(a[0].argmax()))
+
+    with torch.cuda.stream(torch.cuda.Stream(device)):
+        for index in range(20):
+            admit(index)
+        for step in range(24):
+            if step in (3, 4, 5, 9, 10, 11, 12, 13, 14, 15, 16, 17, 18, 19, 20):     # 20 -> 35 requests: buckets 32 and 64
+                admit(100 + step)
+            if step == 22:                                                           # ... and down to 15: the own kernels' graphs
+                for index in sorted(live)[:20]:
+                    caches, _ = live.pop(index)
+                    eager.cache.release(caches[0])
+                    graphed.cache.release(caches[1])
+            order = sorted(live)
+            a = eager.step([StepEntry(live[i][0][0], [live[i][1]], [0]) for i in order]).clone()
+            b = graphed.step([StepEntry(live[i][0][1], [live[i][1]], [0]) for i in order]).clone()
+            torch.cuda.synchronize()
+            assert torch.equal(a, b), f"step {step} with {len(order)} requests: graph replay differs from the eager step"
+            for row, i in enumerate(order):
+                live[i] = (live[i][0], int(a[row].argmax()))
+    assert graphed.graph_replays == 24 and {key[0] for key in graphed._graphs} == {16, 32, 64}
+    graphed.drop_graphs()
+
+
 def test_sampled_tokens_do_not_depend_on_steps_per_launch(folders):
     """Seeded draws with top-k and top-p, one request greedy beside them: four decode steps from one
     launch (the device filters, draws and counts the draws itself) give the tokens of single steps."""
