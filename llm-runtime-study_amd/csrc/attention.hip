@@ -188,14 +188,14 @@ __device__ __forceinline__ void prepare_head(bf16x8 (&r)[D / 32], const bf16* __
 // PREP: q holds the raw rows of the q/k/v product; the kernel prepares q itself, and the wave that
 // meets the token's own position prepares the new key, takes it and the new value in place of what
 // the pages hold there, and writes both into the pages (see DecodePrep).
-template <int D, bool PREP>
-__global__ __launch_bounds__(256) void attention_decode_bf16_kernel(
+template <int D, bool PREP, int WAVES, bool AHEAD>
+__global__ __launch_bounds__(WAVES * 64) void attention_decode_bf16_kernel(
     bf16* __restrict__ out, int out_stride, float* __restrict__ part_o, float* __restrict__ part_ml,
     const bf16* __restrict__ q, int q_stride, bf16* __restrict__ k_pages,
     bf16* __restrict__ v_pages, const int* __restrict__ block_table, int table_stride,
     const int* __restrict__ token_request, const int* __restrict__ positions, int nq, int nkv,
     int page_size, float scale, int window, int splits, DecodePrep prep) {
-  constexpr int DS = D / 32, DB = D / 16, WAVES = 4;
+  constexpr int DS = D / 32, DB = D / 16, THREADS = WAVES * 64;
   __shared__ float sm_m[WAVES][16], sm_l[WAVES][16];
   __shared__ float sm_o[WAVES][D][16];
   const int tid = threadIdx.x, lane = tid % WAVE, wave = tid / WAVE;
@@ -216,7 +216,7 @@ __global__ __launch_bounds__(256) void attention_decode_bf16_kernel(
   const int first_block = tile_begin * 32 / page_size;
   const int last_key = tile_end * 32 - 1 < pos ? tile_end * 32 - 1 : pos;
   if (tile_begin < tile_end)
-    for (int i = tid; i <= last_key / page_size - first_block; i += 256) page_ids[i] = table[first_block + i];
+    for (int i = tid; i <= last_key / page_size - first_block; i += THREADS) page_ids[i] = table[first_block + i];
 
   const bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
   bf16x8 qf[DS];
@@ -275,9 +275,7 @@ __global__ __launch_bounds__(256) void attention_decode_bf16_kernel(
   // block h, row 4*r + i is key 8*r + 4*h + i.  The values of those eight keys lie side by side in
   // the (transposed) page, one 16-byte load a dim.
   const int key_of_row = (col >> 2) * 8 + (col & 3);           // + 4*h
-  for (int tile = tile_begin + wave; tile < tile_end; tile += WAVES) {
-    bf16x8 kf[2][DS];
-    bf16x8 vf[DB];
+  auto fetch = [&](int tile, bf16x8 (&kf)[2][DS], bf16x8 (&vf)[DB]) {
 #pragma unroll
     for (int h = 0; h < 2; ++h) {
       const int key = tile * 32 + key_of_row + 4 * h;
@@ -291,18 +289,18 @@ __global__ __launch_bounds__(256) void attention_decode_bf16_kernel(
         for (int c = 0; c < DS; ++c) kf[h][c] = zero8;
       }
     }
-    {
-      const int key8 = tile * 32 + g * 8;                      // this lane's eight keys; pages hold multiples of 16
-      if (key8 <= pos && key8 + 7 >= lo) {
-        const int64_t page = page_ids[key8 / page_size - first_block];
-        const bf16* vp = v_pages + (page * nkv + kvh) * (int64_t)D * page_size + (int64_t)col * page_size + key8 % page_size;
+    const int key8 = tile * 32 + g * 8;                        // this lane's eight keys; pages hold multiples of 16
+    if (key8 <= pos && key8 + 7 >= lo) {
+      const int64_t page = page_ids[key8 / page_size - first_block];
+      const bf16* vp = v_pages + (page * nkv + kvh) * (int64_t)D * page_size + (int64_t)col * page_size + key8 % page_size;
 #pragma unroll
-        for (int b = 0; b < DB; ++b) vf[b] = *(const bf16x8*)(vp + (int64_t)b * 16 * page_size);
-      } else {
+      for (int b = 0; b < DB; ++b) vf[b] = *(const bf16x8*)(vp + (int64_t)b * 16 * page_size);
+    } else {
 #pragma unroll
-        for (int b = 0; b < DB; ++b) vf[b] = zero8;
-      }
+      for (int b = 0; b < DB; ++b) vf[b] = zero8;
     }
+  };
+  auto work = [&](int tile, bf16x8 (&kf)[2][DS], bf16x8 (&vf)[DB]) {
     if (holds_own && tile == last_tile) {
       // the token's own key and value take the place of what the pages hold at its position
       const int own = pos % 32;
@@ -359,6 +357,25 @@ __global__ __launch_bounds__(256) void attention_decode_bf16_kernel(
       if (rescale) o[b] *= alpha;
       o[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[b], pf, o[b], 0, 0, 0);
     }
+  };
+  if (AHEAD) {
+    // two register sets in turn: the next tile of this wave is on its way while this one is worked on
+    bf16x8 kf_a[2][DS], vf_a[DB], kf_b[2][DS], vf_b[DB];
+    int tile = tile_begin + wave;
+    if (tile < tile_end) fetch(tile, kf_a, vf_a);
+    for (; tile < tile_end; tile += 2 * WAVES) {
+      if (tile + WAVES < tile_end) fetch(tile + WAVES, kf_b, vf_b);
+      work(tile, kf_a, vf_a);
+      if (tile + WAVES >= tile_end) break;
+      if (tile + 2 * WAVES < tile_end) fetch(tile + 2 * WAVES, kf_a, vf_a);
+      work(tile + WAVES, kf_b, vf_b);
+    }
+  } else {
+    for (int tile = tile_begin + wave; tile < tile_end; tile += WAVES) {
+      bf16x8 kf[2][DS], vf[DB];
+      fetch(tile, kf, vf);
+      work(tile, kf, vf);
+    }
   }
   run_sum += __shfl_xor(run_sum, 16, WAVE);
   run_sum += __shfl_xor(run_sum, 32, WAVE);
@@ -371,7 +388,7 @@ __global__ __launch_bounds__(256) void attention_decode_bf16_kernel(
 #pragma unroll
     for (int i = 0; i < 4; ++i) sm_o[wave][b * 16 + g * 4 + i][col] = o[b][i];
   __syncthreads();
-  for (int e = tid; e < D * 16; e += 256) {
+  for (int e = tid; e < D * 16; e += THREADS) {
     const int dim = e / 16, h = e % 16;
     if (h >= group) continue;
     float top = sm_m[0][h];
@@ -433,7 +450,7 @@ LRS_API int lrs_attention_decode(void* out, int out_stride, float* part_o, float
                                  int q_stride, void* k_pages, void* v_pages,
                                  const int* block_table, int table_stride, const int* token_request,
                                  const int* positions, int tokens, int max_context, int nq, int nkv, int d,
-                                 int page_size, float scale, int window, int splits, int prepare,
+                                 int page_size, float scale, int window, int splits, int form, int prepare,
                                  const void* q_weight, const void* k_weight, int w_dtype, float eps,
                                  const float* cosv, const float* sinv, int kv_columns, void* stream) {
   LRS_REQUIRE(tokens > 0 && nq > 0 && nkv > 0 && nq % nkv == 0, "attention_decode: bad sizes tokens=%d nq=%d nkv=%d", tokens, nq, nkv);
@@ -441,6 +458,7 @@ LRS_API int lrs_attention_decode(void* out, int out_stride, float* part_o, float
   LRS_REQUIRE(page_size % 16 == 0, "attention_decode: page size %d is not a multiple of 16", page_size);
   LRS_REQUIRE(splits >= 1 && (splits == 1 || (part_o && part_ml)), "attention_decode: splits=%d needs partial buffers", splits);
   LRS_REQUIRE(window >= 0, "attention_decode: window must be >= 0 (0 = none)");
+  LRS_REQUIRE(form >= 0 && form <= 2, "attention_decode: form must be 0, 1 or 2, got %d", form);
   LRS_REQUIRE(q_stride % 8 == 0 && ((uintptr_t)q % 16) == 0, "attention_decode: q rows must be 16-byte aligned");
   dim3 grid(splits, nkv, tokens);
   hipStream_t s = (hipStream_t)stream;
@@ -460,16 +478,21 @@ LRS_API int lrs_attention_decode(void* out, int out_stride, float* part_o, float
                 "attention_decode: norm weights and rotation tables must be 16-byte aligned");
   }
   const DecodePrep prep{q_weight, k_weight, w_dtype == LRS_F32, eps, cosv, sinv, kv_columns};
-#define LAUNCH(D)                                                                                                   \
-  do {                                                                                                              \
-    if (prepare)                                                                                                    \
-      attention_decode_bf16_kernel<D, true><<<grid, 256, table_lds, s>>>(                                           \
-          (bf16*)out, out_stride, part_o, part_ml, (const bf16*)q, q_stride, (bf16*)k_pages, (bf16*)v_pages,        \
-          block_table, table_stride, token_request, positions, nq, nkv, page_size, scale, window, splits, prep);    \
-    else                                                                                                            \
-      attention_decode_bf16_kernel<D, false><<<grid, 256, table_lds, s>>>(                                          \
-          (bf16*)out, out_stride, part_o, part_ml, (const bf16*)q, q_stride, (bf16*)k_pages, (bf16*)v_pages,        \
-          block_table, table_stride, token_request, positions, nq, nkv, page_size, scale, window, splits, prep);    \
+  // `form`: 0 = four waves, a tile at a time; 1 = four waves, 2 = eight waves, each wave with its next
+  // tile on the way while it works (heads of 192 dims have no registers for that and stay with 0)
+#define ARGS                                                                                                 \
+  (bf16*)out, out_stride, part_o, part_ml, (const bf16*)q, q_stride, (bf16*)k_pages, (bf16*)v_pages, block_table, \
+      table_stride, token_request, positions, nq, nkv, page_size, scale, window, splits, prep
+#define LAUNCH_PREP(D, PREP)                                                                                 \
+  do {                                                                                                       \
+    if (form == 2 && D <= 128) attention_decode_bf16_kernel<D, PREP, 8, (D <= 128)><<<grid, 512, table_lds, s>>>(ARGS); \
+    else if (form == 1 && D <= 128) attention_decode_bf16_kernel<D, PREP, 4, (D <= 128)><<<grid, 256, table_lds, s>>>(ARGS); \
+    else attention_decode_bf16_kernel<D, PREP, 4, false><<<grid, 256, table_lds, s>>>(ARGS);                  \
+  } while (0)
+#define LAUNCH(D)                        \
+  do {                                   \
+    if (prepare) LAUNCH_PREP(D, true);   \
+    else LAUNCH_PREP(D, false);          \
   } while (0)
   switch (d) {
     case 32: LAUNCH(32); break;
@@ -480,6 +503,8 @@ LRS_API int lrs_attention_decode(void* out, int out_stride, float* part_o, float
     default: return lrs_fail("attention_decode: head_dim %d has no matrix-core kernel (32, 64, 96, 128, 192)", d);
   }
 #undef LAUNCH
+#undef LAUNCH_PREP
+#undef ARGS
   if (lrs_check_launch("attention_decode")) return 1;
   if (splits > 1) {
     attention_merge_kernel<<<dim3(tokens, nq), d < 64 ? 64 : d, 0, s>>>((bf16*)out, out_stride, part_o, part_ml, nq, d, splits);

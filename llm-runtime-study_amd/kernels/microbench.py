@@ -82,13 +82,15 @@ def attention_decode(args) -> None:
         out = torch.empty(batch, nq * d, device="cuda", dtype=torch.bfloat16)
         request = torch.arange(batch, dtype=torch.int32, device="cuda")
         positions = torch.full((batch,), context - 1, dtype=torch.int32, device="cuda")
-        for splits in _ints(args.splits):
-            part_o = torch.empty(batch, nq * splits * d, device="cuda")
-            part_ml = torch.empty(batch, nq * splits * 2, device="cuda")
-            seconds = _time(lambda i: ops.attention_decode(out, q, caches[i % sets][0], caches[i % sets][1], table, request, positions,
-                                                           nq, 1 / math.sqrt(d), args.window, splits, part_o, part_ml, context), args.repeats)
-            print(f"attention_decode batch={batch} context={context} splits={splits}: {seconds * 1e6:8.1f} us  "
-                  f"{cache_bytes / seconds / 1e9:7.0f} GB/s of cache", flush=True)
+        for form in _ints(args.form):
+            for splits in _ints(args.splits):
+                part_o = torch.empty(batch, nq * splits * d, device="cuda")
+                part_ml = torch.empty(batch, nq * splits * 2, device="cuda")
+                seconds = _time(lambda i: ops.attention_decode(out, q, caches[i % sets][0], caches[i % sets][1], table, request, positions,
+                                                               nq, 1 / math.sqrt(d), args.window, splits, part_o, part_ml, context,
+                                                               form=form), args.repeats)
+                print(f"attention_decode batch={batch} context={context} form={form} splits={splits}: {seconds * 1e6:8.1f} us  "
+                      f"{cache_bytes / seconds / 1e9:7.0f} GB/s of cache", flush=True)
 
 
 def gemm(args) -> None:
@@ -132,6 +134,7 @@ def main(argv=None) -> int:
     parser.add_argument("--batch", default="1,8,64", help="attention_decode: batch sizes")
     parser.add_argument("--context", type=int, default=2048, help="attention_decode: cached tokens per request")
     parser.add_argument("--splits", default="1,2,4,8,16", help="attention_decode: workgroups per (token, kv head)")
+    parser.add_argument("--form", default="0,1,2", help="attention_decode: 0 four waves, 1 four waves with the next tile on the way, 2 eight waves likewise")
     parser.add_argument("--rows", default="1,8,16,64,2048", help="gemm: numbers of rows")
     parser.add_argument("--repeats", type=int, default=20)
     args = parser.parse_args(argv)

@@ -56,7 +56,7 @@ _SIGNATURES = {
     "lrs_attention": (c_int, [c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p,
                               c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_void_p]),
     "lrs_attention_decode": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p,
-                                     c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_int, c_int,
+                                     c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_int, c_int, c_int,
                                      c_void_p, c_void_p, c_int, c_float, c_void_p, c_void_p, c_int, c_void_p]),
     "lrs_attention_prefill": (c_int, [c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p,
                                       c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int,
@@ -501,7 +501,7 @@ def decode_prepare_supported(d: int, rotates: bool) -> bool:
 def attention_decode(out: torch.Tensor, q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, block_table: torch.Tensor,
                      token_request: torch.Tensor, positions: torch.Tensor, nq: int, scale: float, window: int = 0, splits: int = 1,
                      part_o: torch.Tensor | None = None, part_ml: torch.Tensor | None = None, max_context: int | None = None,
-                     prepare: "DecodePrepare | None" = None) -> None:
+                     prepare: "DecodePrepare | None" = None, form: int = 0) -> None:
     """attention() for a step with one query token per request, bfloat16 only; the keys of a token
     are divided between `splits` workgroups whose partial results meet in part_o / part_ml.
 
@@ -540,7 +540,7 @@ def attention_decode(out: torch.Tensor, q: torch.Tensor, k_pages: torch.Tensor, 
         _dev(q, "q"), _rows(q, "q"), _dev(k_pages, "k_pages"), _dev(v_pages, "v_pages"), _dev(block_table, "block_table"), block_table.stride(0),
         _dev(token_request, "token_request"), _dev(positions, "positions"), tokens,
         block_table.shape[1] * page_size if max_context is None else max_context, nq, nkv, d, page_size, scale, window, splits,
-        *fused, _stream()))
+        form, *fused, _stream()))
 
 
 def attention_prefill(out: torch.Tensor, q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, block_table: torch.Tensor,

@@ -13,7 +13,10 @@ def test_length_class_is_256_times_a_power_of_two():
         assert c <= n and (c == 0 or (n < 2 * c and (c // 256) & (c // 256 - 1) == 0))
 
 
-def test_decode_splits_follow_the_class_not_the_length():
+def test_decode_splits_follow_the_class_not_the_length(monkeypatch):
+    from llm_runtime_study_amd.kernels import ops
+
+    monkeypatch.setattr(ops, "compute_units", lambda: 256)
     splits = GQAAttention._decode_splits
     # short contexts and large batches: one workgroup per (token, kv head)
     assert splits(64, 100, 4096, 16) == 1 and splits(512, 5000, 8192, 16) == 1
@@ -27,7 +30,10 @@ def test_decode_splits_follow_the_class_not_the_length():
             assert 1 <= n <= 64 and (n == 1 or length // n >= 256)
 
 
-def test_decode_splits_keep_a_workgroups_block_table_inside_lds():
+def test_decode_splits_keep_a_workgroups_block_table_inside_lds(monkeypatch):
+    from llm_runtime_study_amd.kernels import ops
+
+    monkeypatch.setattr(ops, "compute_units", lambda: 256)
     splits = GQAAttention._decode_splits
     # one workgroup can hold 4,096 block table entries: contexts beyond that are split even when the batch is large
     assert splits(512, 100, 4096 * 16, 16) == 1

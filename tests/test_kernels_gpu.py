@@ -486,9 +486,15 @@ def test_attention_decode_kernel(ops, nq, nkv, d, page, window, splits):
     order = torch.randperm(t, generator=g)
     shuffled = torch.empty_like(table)
     shuffled[order] = table
-    ops.attention_decode(out, dev(q_wide), dev(kp.bfloat16()), dev(vp.bfloat16()), dev(shuffled), dev(order.to(torch.int32)),
-                         dev(torch.tensor([n - 1 for n in lengths], dtype=torch.int32)), nq, scale, window, splits, part_o, part_ml)
-    torch.testing.assert_close(out.cpu().double(), want, rtol=2e-2, atol=2e-2)
+    results = []
+    for form in (0, 1, 2):      # a tile at a time; the next tile on its way, with four and with eight waves
+        out.fill_(float("nan"))
+        ops.attention_decode(out, dev(q_wide), dev(kp.bfloat16()), dev(vp.bfloat16()), dev(shuffled), dev(order.to(torch.int32)),
+                             dev(torch.tensor([n - 1 for n in lengths], dtype=torch.int32)), nq, scale, window, splits, part_o, part_ml,
+                             form=form)
+        torch.testing.assert_close(out.cpu().double(), want, rtol=2e-2, atol=2e-2)
+        results.append(out.cpu().clone())
+    assert torch.equal(results[0], results[1])      # the same sums in the same order
 
 
 @pytest.mark.parametrize("nq,nkv,d,page,window,splits,normed,rotated,shared", [
