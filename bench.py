@@ -77,7 +77,7 @@ def measure_decode(engine, batch: int, context: int, steps: int, warmup: int, se
     vocab = engine.config.vocab_size
     scheduler = engine.create_scheduler(ignore_eos=True)   # every request runs to its length limit
     for _ in range(batch):
-        scheduler.add_request(rng.integers(0, vocab, context).tolist(), max_new_tokens=warmup + steps + 2 * batch + 8,
+        scheduler.add_request(rng.integers(0, vocab, context).tolist(), max_new_tokens=warmup + steps + 2 * batch + 8 + 2 * scheduler.decode_steps_per_launch,
                               sampling=SamplingConfig())
     times = []
     with torch.cuda.device(engine.device), torch.cuda.stream(engine.stream):
@@ -102,13 +102,19 @@ def measure_decode(engine, batch: int, context: int, steps: int, warmup: int, se
                     times.extend([elapsed / held] * held)
                 done += held
 
-        run(warmup, False)
+        # warm-up: at least `warmup` steps, in whole launches, and one launch of every size the timed
+        # steps will use (a graph is captured at the first launch of its size)
+        warmed = -(-max(warmup, 1) // per_launch) * per_launch
+        run(warmed, False)
+        if steps % per_launch:
+            run(steps % per_launch, False)
+            warmed += steps % per_launch
         engine.synchronize()
         run(steps, True)
         assert len(times) == steps
         scheduler.abort_all()
     # requests entered one step apart, so they are up to `batch` tokens apart in length
-    mean_context = context + 1 + warmup + (batch - 1) / 2 + (steps - 1) / 2
+    mean_context = context + 1 + warmed + (batch - 1) / 2 + (steps - 1) / 2
     return times, mean_context
 
 
