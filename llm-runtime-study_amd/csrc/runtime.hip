@@ -97,21 +97,10 @@ LRS_API int lrs_copy_to_pinned(void* dst_host, const void* src, int64_t bytes, v
 LRS_API int lrs_copy_h2d(void* dst, const void* src, int64_t bytes, void* stream) {
   hipStream_t s = (hipStream_t)stream;
   if (bytes <= (256 << 10) && bytes % 16 == 0 && (uintptr_t)dst % 16 == 0 && (uintptr_t)src % 16 == 0) {
-    // device addresses of the (few) pinned buffers seen so far
-    static const void* known_host[8];
-    static void* known_device[8];
-    static int known = 0;
     void* device_src = nullptr;
-    for (int i = 0; i < known; ++i)
-      if (known_host[i] == src) device_src = known_device[i];
-    if (!device_src) {
-      if (hipHostGetDevicePointer(&device_src, const_cast<void*>(src), 0) != hipSuccess) {
-        (void)hipGetLastError();
-        device_src = nullptr;
-      } else if (known < 8) {
-        known_host[known] = src;
-        known_device[known++] = device_src;
-      }
+    if (hipHostGetDevicePointer(&device_src, const_cast<void*>(src), 0) != hipSuccess) {
+      (void)hipGetLastError();      // not pinned after all: the runtime's copy path takes it
+      device_src = nullptr;
     }
     if (device_src) {
       const int64_t chunks = bytes / 16;

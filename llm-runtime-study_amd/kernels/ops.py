@@ -123,25 +123,13 @@ def _dev(t: torch.Tensor, name: str, dtype=None) -> int:
     return t.data_ptr()
 
 
-_host_visible: dict[int, int] = {}
-
-
-def _dev_or_pinned(t: torch.Tensor, name: str, dtype=None) -> int:
-    """Device address of a device tensor, or of a pinned host tensor that a kernel is to write
-    (the caller allocated it pinned; its device address is asked for once)."""
-    if t.is_cuda:
-        return _dev(t, name, dtype)
-    if dtype is not None:
-        _need(t.dtype == dtype, f"{name} must be {dtype}, got {t.dtype}")
-    address = _host_visible.get(t.data_ptr())
-    if address is None:
-        _need(t.is_pinned(), f"{name} must be a device tensor or pinned host memory")
-        out = c_void_p()
-        _check(library().lrs_host_device_pointer(t.data_ptr(), byref(out)))
-        if len(_host_visible) > 64:
-            _host_visible.clear()
-        address = _host_visible[t.data_ptr()] = out.value
-    return address
+def pinned_device_address(t: torch.Tensor) -> int:
+    """The address under which kernels see the pinned host tensor `t`.  The owner of the tensor asks
+    once and keeps the answer with the tensor (asking whether memory is pinned is slow)."""
+    _need(not t.is_cuda and t.is_contiguous() and t.is_pinned(), "pinned_device_address needs a contiguous pinned host tensor")
+    out = c_void_p()
+    _check(library().lrs_host_device_pointer(t.data_ptr(), byref(out)))
+    return out.value
 
 
 def _rows(t: torch.Tensor, name: str) -> int:
@@ -596,12 +584,19 @@ def attention_prefill_group(tokens: int | None = None) -> int:
 _choose_scratch: dict = {}
 
 
-def choose_tokens(out: torch.Tensor, logits: torch.Tensor, temperature=None, seeds=None, counters=None) -> None:
-    """One token per row of logits into `out` (int32 [R]: on the device, or pinned host memory that
-    the kernel writes directly and the host reads after synchronising the stream)."""
+def choose_tokens(out: torch.Tensor, logits: torch.Tensor, temperature=None, seeds=None, counters=None,
+                  out_address: int | None = None) -> None:
+    """One token per row of logits into `out`, int32 [R] on the device; or, with `out_address` (from
+    pinned_device_address(out)), into pinned host memory that the kernel writes directly and the
+    host reads after synchronising the stream."""
     rows, vocab = logits.shape
     _need(out.dtype == torch.int32 and out.numel() >= rows and out.is_contiguous(), "choose_tokens: out must be int32 [R]")
     stride = _rows(logits, "logits")
+    if out_address is None:
+        out_pointer = _dev(out, "out")
+    else:
+        _need(not out.is_cuda, "choose_tokens: out_address goes with a pinned host tensor")
+        out_pointer = out_address + out.storage_offset() * out.element_size()
     if temperature is not None:
         _need(temperature.dtype == torch.float32 and temperature.numel() >= rows, "choose_tokens: temperature must be float32 [R]")
         _need(seeds is not None and seeds.dtype == torch.int64 and seeds.numel() >= rows, "choose_tokens: seeds must be int64 [R]")
@@ -615,10 +610,10 @@ def choose_tokens(out: torch.Tensor, logits: torch.Tensor, temperature=None, see
         if scratch is None:
             scratch = _choose_scratch[key] = (torch.empty(rows * parts, dtype=torch.float32, device=logits.device),
                                               torch.empty(rows * parts, dtype=torch.int32, device=logits.device))
-        _check(library().lrs_choose_tokens_split(_dev_or_pinned(out, "out"), _dev(logits, "logits", torch.float32), stride, rows, vocab, *args,
+        _check(library().lrs_choose_tokens_split(out_pointer, _dev(logits, "logits", torch.float32), stride, rows, vocab, *args,
                                                  _dev(scratch[0], "part_value"), _dev(scratch[1], "part_index"), parts, _stream()))
         return
-    _check(library().lrs_choose_tokens(_dev_or_pinned(out, "out"), _dev(logits, "logits", torch.float32), stride, rows, vocab, *args, _stream()))
+    _check(library().lrs_choose_tokens(out_pointer, _dev(logits, "logits", torch.float32), stride, rows, vocab, *args, _stream()))
 
 
 def filter_logits(logits: torch.Tensor, temperature: torch.Tensor, top_k: torch.Tensor | None, top_p: torch.Tensor | None) -> None:

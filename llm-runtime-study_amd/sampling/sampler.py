@@ -37,11 +37,13 @@ class SamplingRow:
 class Sampler:
     def __init__(self, device):
         self.device = torch.device(device)
-        self._chosen = None      # pinned host memory the kernel writes the tokens into
+        self._chosen = None      # pinned host memory the kernel writes the tokens into ...
+        self._chosen_address = 0  # ... and where the device sees it
 
     def _result(self, rows: int) -> torch.Tensor:
         if self._chosen is None or self._chosen.numel() < rows:
             self._chosen = torch.zeros(max(rows, 64), dtype=torch.int32, pin_memory=True)
+            self._chosen_address = ops.pinned_device_address(self._chosen)
         return self._chosen[:rows]
 
     def _read(self, out: torch.Tensor) -> list[int]:
@@ -58,7 +60,7 @@ class Sampler:
                 raise SamplingError(f"top_k {row.config.top_k} exceeds vocabulary size {vocab}")
         out = self._result(len(rows))
         if all(row.config.greedy for row in rows):
-            ops.choose_tokens(out, logits)
+            ops.choose_tokens(out, logits, out_address=self._chosen_address)
             return self._read(out)
         temperature = torch.tensor([row.config.temperature for row in rows], dtype=torch.float32, device=self.device)
         seeds = torch.tensor([row.seed for row in rows], dtype=torch.int64, device=self.device)
@@ -67,5 +69,5 @@ class Sampler:
             top_k = torch.tensor([row.config.top_k or 0 for row in rows], dtype=torch.int32, device=self.device)
             top_p = torch.tensor([row.config.top_p for row in rows], dtype=torch.float32, device=self.device)
             ops.filter_logits(logits, temperature, top_k, top_p)
-        ops.choose_tokens(out, logits, temperature, seeds, counters)
+        ops.choose_tokens(out, logits, temperature, seeds, counters, out_address=self._chosen_address)
         return self._read(out)
