@@ -1,0 +1,80 @@
+"""The kernels at the sizes of the model the benchmark runs (hidden 4096, 32/8 heads of 128 dims,
+feed-forward 12288, vocabulary 151936; two layers): the bfloat16 path with everything it uses at
+that size (graphs, fused norms, library products for many rows, key splits) against the float32
+path of the same weights, over prompts in portions, mixed steps and decode steps."""
+
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+SHAPE = {
+    "architectures": ["Qwen3ForCausalLM"], "model_type": "qwen3",
+    "vocab_size": 151936, "hidden_size": 4096, "intermediate_size": 12288, "num_hidden_layers": 2,
+    "num_attention_heads": 32, "num_key_value_heads": 8, "head_dim": 128,
+    "max_position_embeddings": 40960, "rms_norm_eps": 1e-6, "rope_theta": 1000000.0,
+    "hidden_act": "silu", "attention_bias": False, "attention_dropout": 0.0,
+    "tie_word_embeddings": False, "torch_dtype": "bfloat16", "bos_token_id": 151643, "eos_token_id": 151645,
+}
+
+
+def test_bfloat16_path_follows_float32_at_full_layer_sizes():
+    from llm_runtime_study_amd.cache import CacheManager
+    from llm_runtime_study_amd.config import config_from_dict, spec_for
+    from llm_runtime_study_amd.engine.step import ModelRunner, StepEntry
+    from llm_runtime_study_amd.models import DecoderModel
+    from llm_runtime_study_amd.weights import random_init
+
+    cfg = config_from_dict(SHAPE)
+    device = torch.device("cuda", 0)
+    weights = random_init.device_weights(DecoderModel(spec_for(cfg)), 0, torch.bfloat16, device, "scaled")
+    rng = np.random.default_rng(1)
+    prompts = [rng.integers(0, cfg.vocab_size, n).tolist() for n in (700, 33, 1500, 257, 64, 5, 1023, 90)]
+    logits_of, tokens_of = {}, {}
+    for dtype in (torch.float32, torch.bfloat16):
+        model = DecoderModel(spec_for(cfg))
+        model.bind(weights, dtype)
+        cache = CacheManager(model.cache_needs(), page_size=16, num_pages=400, max_requests=8, max_seq_len=2048, dtype=dtype, device=device)
+        runner = ModelRunner(model, cache, max_step_tokens=2048, dtype=dtype, device=device, use_graph=dtype == torch.bfloat16)
+        rows, fed = [], []          # every token fed comes from the float32 run, so both runs see the same sequences
+        with torch.cuda.stream(torch.cuda.Stream(device)):
+            caches = [cache.admit(i) for i in range(len(prompts))]
+            last = {}
+            for i, prompt in enumerate(prompts):
+                # the first half of the prompt beside one decode token of every earlier request, then the rest alone
+                half = len(prompt) // 2
+                decoding = [StepEntry(caches[j], [last[j]], [0]) for j in sorted(last)]
+                if half:
+                    mixed = runner.step(decoding + [StepEntry(caches[i], prompt[:half], [])])
+                    if decoding:
+                        rows.append(mixed.float().cpu())
+                        fed.append(mixed.argmax(-1).tolist())
+                        last = dict(zip(sorted(last), tokens_of[len(fed) - 1] if dtype == torch.bfloat16 else fed[-1]))
+                    final = runner.step([StepEntry(caches[i], prompt[half:], [len(prompt) - half - 1])])
+                else:
+                    final = runner.step(decoding + [StepEntry(caches[i], prompt, [len(prompt) - 1])])[-1:]
+                rows.append(final.float().cpu())
+                fed.append(final.argmax(-1).tolist())
+                last[i] = (tokens_of[len(fed) - 1] if dtype == torch.bfloat16 else fed[-1])[0]
+            for _ in range(6):
+                out = runner.step([StepEntry(caches[j], [last[j]], [0]) for j in sorted(last)])
+                rows.append(out.float().cpu())
+                fed.append(out.argmax(-1).tolist())
+                last = dict(zip(sorted(last), tokens_of[len(fed) - 1] if dtype == torch.bfloat16 else fed[-1]))
+            if dtype == torch.bfloat16:
+                assert runner.graph_replays >= 6
+                # the same continuation, four steps from one launch: the device's own choices
+                chosen = runner.decode_steps([StepEntry(caches[j], [last[j]], [0]) for j in sorted(last)], 4)
+                assert len(chosen) == 4 and all(0 <= t < cfg.vocab_size for row in chosen for t in row)
+                runner.drop_graphs()
+        if dtype == torch.float32:
+            tokens_of = dict(enumerate(fed))
+        logits_of[dtype] = torch.cat(rows)
+        cache.check_invariants()
+        del runner, cache, model
+    exact, fast = logits_of[torch.float32], logits_of[torch.bfloat16]
+    assert exact.shape == fast.shape and exact.shape[0] > 80
+    error = (exact - fast).norm(dim=1) / exact.norm(dim=1)
+    assert error.max() < 2e-2, f"largest relative error of a logits row {error.max():.3g}"
+    assert (exact.argmax(1) == fast.argmax(1)).float().mean() > 0.95
