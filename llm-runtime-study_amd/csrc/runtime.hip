@@ -113,3 +113,27 @@ LRS_API int lrs_copy_h2d(void* dst, const void* src, int64_t bytes, void* stream
   if (err != hipSuccess) return lrs_fail("hipMemcpyAsync: %s", hipGetErrorString(err));
   return 0;
 }
+
+// Probe of the rate at which a kernel can stream memory: reads `chunks` 16-byte pieces once (four
+// in flight per lane) and leaves one word per workgroup in `sink` so that nothing is optimised away.
+__global__ __launch_bounds__(256) void stream_read_kernel(const int4* __restrict__ src, int64_t chunks, int* __restrict__ sink) {
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  int acc = 0;
+  int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  for (; i + 3 * stride < chunks; i += 4 * stride) {
+    const int4 a = src[i], b = src[i + stride], c = src[i + 2 * stride], d = src[i + 3 * stride];
+    acc ^= a.x ^ a.y ^ a.z ^ a.w ^ b.x ^ b.y ^ b.z ^ b.w ^ c.x ^ c.y ^ c.z ^ c.w ^ d.x ^ d.y ^ d.z ^ d.w;
+  }
+  for (; i < chunks; i += stride) {
+    const int4 a = src[i];
+    acc ^= a.x ^ a.y ^ a.z ^ a.w;
+  }
+  acc ^= __shfl_xor(acc, 32, 64);
+  if (threadIdx.x == 0) sink[blockIdx.x] = acc;
+}
+
+LRS_API int lrs_stream_read(const void* src, int64_t bytes, int* sink, int blocks, void* stream) {
+  LRS_REQUIRE(bytes >= 16 && (uintptr_t)src % 16 == 0 && blocks > 0 && sink, "stream_read: needs 16-byte aligned memory, a sink and blocks");
+  stream_read_kernel<<<blocks, 256, 0, (hipStream_t)stream>>>((const int4*)src, bytes / 16, sink);
+  return lrs_check_launch("stream_read");
+}

@@ -4,6 +4,7 @@
     python -m llm_runtime_study_amd.kernels.microbench attention_prefill --tokens 64 --before 32704 --key-splits 1,8,32
     python -m llm_runtime_study_amd.kernels.microbench attention_decode --batch 1,8,64 --context 2048 --splits 1,4,8
     python -m llm_runtime_study_amd.kernels.microbench gemm --rows 1,8,16,64,2048
+    python -m llm_runtime_study_amd.kernels.microbench memory
 
 Head and matrix shapes default to those of Qwen3-8B and can be changed with options.  Weights and
 caches larger than the last-level cache are rotated between calls where a kernel streams them once
@@ -117,9 +118,20 @@ def gemm(args) -> None:
         ops.set_skinny_max_m(before)
 
 
+def memory(args) -> None:
+    """The rate at which a plain kernel streams memory once: what 'reads from memory' can mean on this GPU."""
+    for megabytes in _ints(args.megabytes):
+        buffers = [torch.randint(0, 1 << 30, (megabytes << 18,), dtype=torch.int32, device="cuda") for _ in range(max(2, min(6, 3072 // megabytes)))]
+        for blocks in _ints(args.blocks):
+            sink = torch.zeros(blocks, dtype=torch.int32, device="cuda")
+            seconds = _time(lambda i: ops.stream_read(buffers[i % len(buffers)], sink, blocks), args.repeats)
+            print(f"memory read {megabytes:5d} MB with {blocks:5d} workgroups: {seconds * 1e6:9.1f} us  {(megabytes << 20) / seconds / 1e9:7.0f} GB/s", flush=True)
+        del buffers
+
+
 def main(argv=None) -> int:
     parser = argparse.ArgumentParser(prog="python -m llm_runtime_study_amd.kernels.microbench", description=__doc__.split("\n\n")[0])
-    parser.add_argument("kernel", choices=["attention_prefill", "attention_decode", "gemm"])
+    parser.add_argument("kernel", choices=["attention_prefill", "attention_decode", "gemm", "memory"])
     parser.add_argument("--heads", type=int, default=32)
     parser.add_argument("--kv-heads", type=int, default=8)
     parser.add_argument("--head-dim", type=int, default=128)
@@ -136,13 +148,15 @@ def main(argv=None) -> int:
     parser.add_argument("--splits", default="1,2,4,8,16", help="attention_decode: workgroups per (token, kv head)")
     parser.add_argument("--form", default="0,1,2", help="attention_decode: 0 four waves, 1 four waves with the next tile on the way, 2 eight waves likewise")
     parser.add_argument("--rows", default="1,8,16,64,2048", help="gemm: numbers of rows")
+    parser.add_argument("--megabytes", default="32,200,1200", help="memory: sizes of the buffers read")
+    parser.add_argument("--blocks", default="512,2048,8192", help="memory: numbers of workgroups")
     parser.add_argument("--repeats", type=int, default=20)
     args = parser.parse_args(argv)
     if not torch.cuda.is_available():
         print("microbench needs the GPU", file=sys.stderr)
         return 2
     ops.library()
-    {"attention_prefill": attention_prefill, "attention_decode": attention_decode, "gemm": gemm}[args.kernel](args)
+    {"attention_prefill": attention_prefill, "attention_decode": attention_decode, "gemm": gemm, "memory": memory}[args.kernel](args)
     return 0
 
 

@@ -50,6 +50,7 @@ _SIGNATURES = {
     "lrs_advance_decode": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p]),
     "lrs_advance_slots": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p, c_int, c_void_p]),
     "lrs_copy_to_pinned": (c_int, [c_void_p, c_void_p, c_int64, c_void_p]),
+    "lrs_stream_read": (c_int, [c_void_p, c_int64, c_void_p, c_int, c_void_p]),
     "lrs_gemm_prepare": (c_int, []),
     "lrs_host_device_pointer": (c_int, [c_void_p, POINTER(c_void_p)]),
     "lrs_gemm_set_skinny_max_m": (c_int, [c_int]),
@@ -170,6 +171,12 @@ def copy_h2d(dst: torch.Tensor, src: torch.Tensor, count: int) -> None:
     _need(src.device.type == "cpu" and src.is_contiguous() and dst.is_contiguous(), "copy_h2d needs a contiguous host source and a contiguous destination")
     _need(src.dtype == dst.dtype and 0 < count <= src.numel() and count <= dst.numel(), "copy_h2d: size or dtype mismatch")
     _check(library().lrs_copy_h2d(_dev(dst, "dst"), src.data_ptr(), count * src.element_size(), _stream()))
+
+
+def stream_read(src: torch.Tensor, sink: torch.Tensor, blocks: int) -> None:
+    """Reads all of `src` once with `blocks` workgroups (a probe of the memory rate a kernel can reach)."""
+    _need(src.is_contiguous() and sink.dtype == torch.int32 and sink.numel() >= blocks, "stream_read: contiguous source and an int32 sink of `blocks` elements")
+    _check(library().lrs_stream_read(_dev(src, "src"), src.numel() * src.element_size(), _dev(sink, "sink"), blocks, _stream()))
 
 
 def copy_to_pinned(dst: torch.Tensor, src: torch.Tensor, count: int) -> None:
