@@ -145,6 +145,15 @@ class ModelRunner:
         self._sampling_dev = self._sampling_host = None
         self._counting = np.arange(max(max_step_tokens, self.max_requests) + 1, dtype=np.int32)
         self.steps_run = 0
+        # The weights, the cache pools and the buffers above were converted and cleared by work queued
+        # on the stream that is current now.  A step on another stream waits for that work once: streams
+        # made by torch do not wait for the default stream by themselves.
+        self._built = None
+        if self.device.type == "cuda":
+            stream = torch.cuda.current_stream(self.device)
+            self._built = torch.cuda.Event()
+            self._built.record(stream)
+            self._follows_construction = {stream.cuda_stream}
 
     def _layout(self, tokens: int, requests: int) -> tuple[dict, int]:
         """Where each array of a step of `tokens` tokens and `requests` requests lies in the metadata
@@ -163,6 +172,18 @@ class ModelRunner:
                 cursor += -(-size // 4) * 4
             known = self._layouts[(tokens, requests)] = (offsets, cursor)
         return known
+
+    def _follow_construction(self) -> None:
+        """Order the current stream after the work that built the model, the cache and this runner."""
+        if self._built is None:
+            return
+        if self._built.query():
+            self._built = None
+            return
+        stream = torch.cuda.current_stream(self.device)
+        if stream.cuda_stream not in self._follows_construction:
+            stream.wait_event(self._built)
+            self._follows_construction.add(stream.cuda_stream)
 
     def _next_staging(self) -> None:
         self._turn ^= 1
@@ -332,6 +353,7 @@ class ModelRunner:
     def step(self, entries: Sequence[StepEntry]) -> torch.Tensor | None:
         """Run one step; returns float32 logits [wanted, vocab] on the device, or None if none is wanted."""
         self.validate(entries)
+        self._follow_construction()
         before = [entry.cache.length for entry in entries]
         extended = []
         try:
@@ -377,6 +399,7 @@ class ModelRunner:
         if not 1 <= steps <= self.MAX_DECODE_STEPS:
             raise GenerationError(f"decode_steps takes 1..{self.MAX_DECODE_STEPS} steps, got {steps}")
         self.validate(entries)
+        self._follow_construction()
         bucket = self._graph_bucket(entries)
         if not bucket:
             raise GenerationError("decode_steps needs graphs and one token per entry")

@@ -214,6 +214,37 @@ def test_several_decode_steps_from_one_launch_equal_single_steps(folders, name, 
     single.drop_graphs()
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_first_step_on_another_stream_waits_for_the_work_that_built_the_runner(folders, dtype):
+    """Weights are converted and cache pools cleared on the stream that is current when they are
+    made; streams made by torch do not wait for that stream.  With the default stream kept busy
+    while the model is bound and the runner built, the first step on a new stream must still see
+    finished weights and cleared pools: its logits equal those of a run that waited for everything."""
+    from llm_runtime_study_amd.cache import CacheManager
+    from llm_runtime_study_amd.engine.loading import load_model
+    from llm_runtime_study_amd.engine.step import ModelRunner, StepEntry
+
+    folder, cfg, _ = folders["c"]
+    device = torch.device("cuda", 0)
+    prompt = np.random.default_rng(21).integers(0, cfg["vocab_size"], 90).tolist()
+    busy = torch.randn(4096, 4096, device=device)
+    results = []
+    for wait_first in (True, False):
+        if not wait_first:
+            for _ in range(40):                 # tens of milliseconds of work ahead of the model's own
+                busy = (busy @ busy).clamp_(-1, 1)
+        _, model = load_model(folder, dtype, device)
+        cache = CacheManager(model.cache_needs(), page_size=16, num_pages=12, max_requests=2, max_seq_len=128, dtype=dtype, device=device)
+        runner = ModelRunner(model, cache, max_step_tokens=128, dtype=dtype, device=device)
+        if wait_first:
+            torch.cuda.synchronize()
+        with torch.cuda.stream(torch.cuda.Stream(device)):
+            entry = cache.admit(0)
+            results.append(runner.step([StepEntry(entry, prompt, [0, len(prompt) - 1])]).float().cpu())
+        torch.cuda.synchronize()
+    assert torch.equal(results[0], results[1])
+
+
 def test_seeded_sampling_is_reproducible_and_independent_of_batch_mates(folders):
     from llm_runtime_study_amd import Engine, SamplingConfig
 
