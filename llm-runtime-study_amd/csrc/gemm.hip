@@ -275,6 +275,33 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_skinny_kernel(
   int s = split_begin + wave * per_wave;
   const int s_end = s + per_wave < split_end ? s + per_wave : split_end;
   const int full_end = k / 32 < s_end ? k / 32 : s_end;   // steps whose 32 k are all inside K
+  // What the epilogue will need from memory is asked for now, before the weights stream, so that it
+  // has long arrived by then: the partial sums of squares of the norm this product finishes, and
+  // the residual values and norm weights of the columns this thread will update.
+  const bool scaled_input = MT == 1 && !NORM && chain.in_sumsq != nullptr;
+  const bool feeds_norm = MT == 1 && !SWIGLU && chain.next_x != nullptr && mode == OUT_ADD_F32 && gridDim.y == 1;
+  constexpr int EARLY = 16;
+  const bool sums_early = scaled_input && chain.in_parts <= WAVES * 4 * EARLY;
+  float early_sums[EARLY];
+  if (sums_early) {
+    const int token = tid % 16, part = tid / 16;
+#pragma unroll
+    for (int j = 0; j < EARLY; ++j) {
+      const int p = part + j * WAVES * 4;
+      early_sums[j] = (token < m && p < chain.in_parts) ? chain.in_sumsq[(int64_t)p * m + token] : 0.f;
+    }
+  }
+  float early_h[RT], early_w[RT];
+  if (feeds_norm && tid < WAVE * 4) {
+    const int l = tid / 4, i = tid % 4, token = l & 15;
+#pragma unroll
+    for (int q = 0; q < RT; ++q) {
+      const int gn = n0 + q * 16 + 4 * (l >> 4) + i;
+      const bool inside = token < m && gn < n;
+      early_h[q] = inside ? ((const float*)out)[(int64_t)token * ldc + gn] : 0.f;
+      early_w[q] = !inside ? 0.f : chain.next_weight_is_f32 ? ((const float*)chain.next_weight)[gn] : (float)((const bf16*)chain.next_weight)[gn];
+    }
+  }
   // Workgroups walk their K slices from different starting points (the order of a column's sum
   // depends on the column alone): all of them read the same activations, and in step they would
   // all ask the same few cache lines of the L2 at the same moment.
@@ -321,13 +348,15 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_skinny_kernel(
       if (g == 0) sumsq[wave][t][r] = v;
     }
   }
-  const bool scaled_input = MT == 1 && !NORM && chain.in_sumsq != nullptr;
-  const bool feeds_norm = MT == 1 && !SWIGLU && chain.next_x != nullptr && mode == OUT_ADD_F32 && gridDim.y == 1;
   if (scaled_input) {
     const int token = tid % 16, part = tid / 16;
     float v = 0.f;
-    if (token < m)
+    if (sums_early) {
+#pragma unroll
+      for (int j = 0; j < EARLY; ++j) v += early_sums[j];      // the order of the loop below
+    } else if (token < m) {
       for (int p = part; p < chain.in_parts; p += WAVES * 4) v += chain.in_sumsq[(int64_t)p * m + token];
+    }
     chain_parts[part][token] = v;
     __syncthreads();
     if (tid < 16) {
@@ -381,12 +410,10 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_skinny_kernel(
         if (!inside) continue;
         float v = total(t, l, i);
         if (bias) v += (float)bias[gn];
-        if (feeds_norm) {
-          float* h = (float*)out + (int64_t)token * ldc + gn;
-          const float updated = *h + v;
-          *h = updated;
-          const float weight = chain.next_weight_is_f32 ? ((const float*)chain.next_weight)[gn] : (float)((const bf16*)chain.next_weight)[gn];
-          chain.next_x[(int64_t)token * n + gn] = (bf16)(updated * weight);
+        if (feeds_norm) {                                        // MT == 1: e == tid, the element asked for early
+          const float updated = early_h[q] + v;
+          ((float*)out)[(int64_t)token * ldc + gn] = updated;
+          chain.next_x[(int64_t)token * n + gn] = (bf16)(updated * early_w[q]);
           chain_squares[l & 15][q * 16 + 4 * (l >> 4) + i] = updated * updated;
         } else {
           emit<bf16>(out, mode, (int64_t)token * ldc + gn, v);
