@@ -65,6 +65,12 @@ def prefill_flops(c, tokens: int) -> float:
     return linear + attention
 
 
+def decode_lead(batch: int, context: int, step_tokens: int) -> int:
+    """Tokens the first request has decoded when the last one has read its prompt: prompts are read one
+    after the other, in portions of at most `step_tokens`, and whoever has finished decodes meanwhile."""
+    return (batch - 1) * -(-context // step_tokens)
+
+
 def measure_decode(engine, batch: int, context: int, steps: int, warmup: int, seed: int):
     """Prefill `batch` prompts of `context` random tokens through the scheduler, then time `steps`
     decode steps.  Returns (seconds per step list, mean context length over the timed steps)."""
@@ -76,8 +82,11 @@ def measure_decode(engine, batch: int, context: int, steps: int, warmup: int, se
     rng = np.random.default_rng(seed)
     vocab = engine.config.vocab_size
     scheduler = engine.create_scheduler(ignore_eos=True)   # every request runs to its length limit
+    # a request decodes while the prompts behind it are still read, one portion a step
+    lead = decode_lead(batch, context, engine.max_num_batched_tokens)
     for _ in range(batch):
-        scheduler.add_request(rng.integers(0, vocab, context).tolist(), max_new_tokens=warmup + steps + 2 * batch + 8 + 2 * scheduler.decode_steps_per_launch,
+        scheduler.add_request(rng.integers(0, vocab, context).tolist(),
+                              max_new_tokens=warmup + steps + lead + batch + 8 + 2 * scheduler.decode_steps_per_launch,
                               sampling=SamplingConfig())
     times = []
     with torch.cuda.device(engine.device), torch.cuda.stream(engine.stream):
@@ -113,8 +122,8 @@ def measure_decode(engine, batch: int, context: int, steps: int, warmup: int, se
         run(steps, True)
         assert len(times) == steps
         scheduler.abort_all()
-    # requests entered one step apart, so they are up to `batch` tokens apart in length
-    mean_context = context + 1 + warmed + (batch - 1) / 2 + (steps - 1) / 2
+    # requests finished their prompts `portions` steps apart, so they are up to `lead` tokens apart in length
+    mean_context = context + 1 + warmed + lead / 2 + (steps - 1) / 2
     return times, mean_context
 
 
@@ -153,7 +162,7 @@ def main() -> int:
     raw = dict(QWEN3_8B, num_hidden_layers=args.layers)
     config = config_from_dict(raw)
     max_batch = args.batch if args.no_points else max(args.batch, 64)
-    max_seq_len = args.context + args.steps + args.warmup + 2 * max_batch + 64
+    max_seq_len = args.context + args.steps + args.warmup + decode_lead(max_batch, args.context, max(2048, args.prefill_tokens)) + max_batch + 64
     max_seq_len = max(max_seq_len, args.prefill_tokens)
     engine = Engine.from_config(config, seed=0, dtype=args.dtype, max_seq_len=max_seq_len, max_batch_size=max_batch,
                                 max_num_batched_tokens=max(2048, args.prefill_tokens), use_cuda_graph=not args.no_graph, library_gemm=not args.own_gemm,
