@@ -219,25 +219,96 @@ __global__ void qk_prep_kernel(T* __restrict__ qkv, int row_stride, int nq, int 
   }
 }
 
-// The same for the common shape, with vector loads: head_dim a power of two times 8, rotation over
-// the whole head (or none).  A thread owns 4 consecutive dims of the first half of a head and
-// their 4 rotation partners in the second half; d/8 neighbouring threads share a head.
+// N values of type TW as floats, read in pieces of at most 16 bytes (p aligned to a piece).
+template <typename TW, int N>
+__device__ __forceinline__ void load_floats(const TW* __restrict__ p, float* out) {
+  constexpr int PER = (int)(16 / sizeof(TW)) < N ? (int)(16 / sizeof(TW)) : N;
+  typedef TW piece __attribute__((ext_vector_type(PER)));
+#pragma unroll
+  for (int c = 0; c < N / PER; ++c) {
+    const piece v = *(const piece*)(p + c * PER);
+#pragma unroll
+    for (int i = 0; i < PER; ++i) out[c * PER + i] = to_float(v[i]);
+  }
+}
+
+// The v heads of 16 consecutive tokens of the step and one kv head into the value pages
+// [page, kv_head, dim, slot]: tokens that follow each other in one page land side by side, so a
+// thread gathers the values of 16 / sizeof(T) such tokens for one dim (neighbouring lanes read
+// neighbouring dims of one token) and writes them with one 16-byte store; it falls back to single
+// stores where a run is broken by a page edge, another request or a slot that is not to be stored.
+// For steps of many tokens: storing token by token scatters 2-byte writes a page row apart.
+template <typename T>
+__device__ __forceinline__ void values_to_pages(const T* __restrict__ qkv, int row_stride, int v_offset, int tokens, int nkv,
+                                                int d, T* __restrict__ v_pages, const int* __restrict__ slots, int page_size,
+                                                int token0, int kvh, int* slot_of) {
+  constexpr int RUN = 16 / sizeof(T);
+  typedef T vec __attribute__((ext_vector_type(RUN)));
+  const int tid = threadIdx.x;
+  if (tid < 16) slot_of[tid] = token0 + tid < tokens ? slots[token0 + tid] : -1;
+  __syncthreads();
+  for (int e = tid; e < d * (16 / RUN); e += 256) {
+    const int dim = e % d, first = (e / d) * RUN;
+    const int slot0 = slot_of[first];
+    bool run = slot0 >= 0 && slot0 % RUN == 0 && slot0 % page_size + RUN <= page_size;
+#pragma unroll
+    for (int i = 1; i < RUN; ++i) run = run && slot_of[first + i] == slot0 + i;
+    const T* src = qkv + (int64_t)(token0 + first) * row_stride + v_offset + (int64_t)kvh * d + dim;
+    if (run) {
+      vec v;
+#pragma unroll
+      for (int i = 0; i < RUN; ++i) v[i] = src[(int64_t)i * row_stride];
+      const int64_t page = slot0 / page_size, off = slot0 % page_size;
+      *(vec*)(v_pages + ((page * nkv + kvh) * d + dim) * page_size + off) = v;
+    } else {
+#pragma unroll
+      for (int i = 0; i < RUN; ++i) {
+        const int slot = slot_of[first + i];
+        if (slot < 0) continue;
+        const int64_t page = slot / page_size, off = slot % page_size;
+        v_pages[((page * nkv + kvh) * d + dim) * page_size + off] = src[(int64_t)i * row_stride];
+      }
+    }
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void values_to_pages_kernel(const T* __restrict__ qkv, int row_stride, int v_offset,
+                                                              int tokens, int nkv, int d, T* __restrict__ v_pages,
+                                                              const int* __restrict__ slots, int page_size) {
+  __shared__ int slot_of[16];
+  values_to_pages<T>(qkv, row_stride, v_offset, tokens, nkv, d, v_pages, slots, page_size, blockIdx.x * 16, blockIdx.y, slot_of);
+}
+
+// qk_prep for the common shape, with 16-byte accesses: head_dim a power of two times 32 / sizeof(T),
+// rotation over the whole head (or none).  A thread owns VE = 16 / sizeof(T) consecutive dims of the
+// first half of a head and their VE rotation partners in the second half; d / (2 VE) neighbouring
+// threads share a head, and a workgroup takes 256 / that many consecutive (token, head) pairs of the
+// `heads` first heads of every token.  Workgroups from `prep_blocks` on (if any) store the v heads
+// instead, 16 tokens of one kv head each, as values_to_pages() does.
 template <typename T, typename TW>
-__global__ __launch_bounds__(256) void qk_prep_vec_kernel(T* __restrict__ qkv, int row_stride, int nq, int nkv, int d,
-                                                          const TW* __restrict__ q_weight, const TW* __restrict__ k_weight,
-                                                          float eps, const float* __restrict__ cosv,
-                                                          const float* __restrict__ sinv, int rot_half,
-                                                          T* __restrict__ k_pages, T* __restrict__ v_pages,
-                                                          const int* __restrict__ slots, int page_size) {
-  typedef T vec4 __attribute__((ext_vector_type(4)));
-  const int per_head = d / 8, half = d / 2;
-  const int token = blockIdx.x;
-  const int head = blockIdx.y * (256 / per_head) + threadIdx.x / per_head;
+__global__ __launch_bounds__(256) void qk_prep_vec_kernel(T* __restrict__ qkv, int row_stride, int tokens, int heads, int nq,
+                                                          int nkv, int d, const TW* __restrict__ q_weight,
+                                                          const TW* __restrict__ k_weight, float eps,
+                                                          const float* __restrict__ cosv, const float* __restrict__ sinv,
+                                                          int rot_half, T* __restrict__ k_pages, T* __restrict__ v_pages,
+                                                          const int* __restrict__ slots, int page_size, int prep_blocks) {
+  constexpr int VE = 16 / sizeof(T);
+  typedef T vec __attribute__((ext_vector_type(VE)));
+  __shared__ int slot_of[16];
+  if ((int)blockIdx.x >= prep_blocks) {      // the whole workgroup
+    const int vb = blockIdx.x - prep_blocks;
+    values_to_pages<T>(qkv, row_stride, (nq + nkv) * d, tokens, nkv, d, v_pages, slots, page_size, (vb / nkv) * 16, vb % nkv, slot_of);
+    return;
+  }
+  const int per_head = d / (2 * VE), half = d / 2;
+  const int64_t pair = (int64_t)blockIdx.x * (256 / per_head) + threadIdx.x / per_head;
   const int j = threadIdx.x % per_head;
-  if (head >= nq + 2 * nkv) return;   // whole groups of per_head lanes leave together
+  if (pair >= (int64_t)tokens * heads) return;   // whole groups of per_head lanes leave together
+  const int token = pair / heads, head = pair % heads;
   T* src = qkv + (int64_t)token * row_stride + (int64_t)head * d;
   const bool is_q = head < nq, is_k = !is_q && head < nq + nkv;
-  const vec4 lo = *(const vec4*)(src + 4 * j), hi = *(const vec4*)(src + half + 4 * j);
+  const vec lo = *(const vec*)(src + VE * j), hi = *(const vec*)(src + half + VE * j);
   int64_t page = 0, off = 0;
   int kv_head = 0;
   if (!is_q) {
@@ -247,97 +318,57 @@ __global__ __launch_bounds__(256) void qk_prep_vec_kernel(T* __restrict__ qkv, i
     page = slot / page_size;
     off = slot % page_size;
     if (!is_k) {
-      if (!v_pages) return;
       T* vdst = v_pages + (page * nkv + kv_head) * d * page_size + off;
 #pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        vdst[(int64_t)(4 * j + e) * page_size] = lo[e];
-        vdst[(int64_t)(half + 4 * j + e) * page_size] = hi[e];
+      for (int e = 0; e < VE; ++e) {
+        vdst[(int64_t)(VE * j + e) * page_size] = lo[e];
+        vdst[(int64_t)(half + VE * j + e) * page_size] = hi[e];
       }
       return;
     }
   }
   const TW* weight = is_q ? q_weight : k_weight;
-  float a[4], b[4], inv = 1.f;
+  float a[VE], b[VE], inv = 1.f;
 #pragma unroll
-  for (int e = 0; e < 4; ++e) {
+  for (int e = 0; e < VE; ++e) {
     a[e] = to_float(lo[e]);
     b[e] = to_float(hi[e]);
   }
   if (weight) {
     float ss = 0.f;
 #pragma unroll
-    for (int e = 0; e < 4; ++e) ss += a[e] * a[e] + b[e] * b[e];
+    for (int e = 0; e < VE; ++e) ss += a[e] * a[e] + b[e] * b[e];
     for (int step = per_head / 2; step > 0; step >>= 1) ss += __shfl_xor(ss, step, WAVE);
     inv = 1.0f / sqrtf(ss / (float)d + eps);
-  }
-  vec4 out_lo, out_hi;
+    float wa[VE], wb[VE];
+    load_floats<TW, VE>(weight + VE * j, wa);
+    load_floats<TW, VE>(weight + half + VE * j, wb);
 #pragma unroll
-  for (int e = 0; e < 4; ++e) {
-    float x = a[e] * inv, y = b[e] * inv;
-    if (weight) {
-      x *= to_float(weight[4 * j + e]);
-      y *= to_float(weight[half + 4 * j + e]);
+    for (int e = 0; e < VE; ++e) {
+      a[e] = a[e] * inv * wa[e];
+      b[e] = b[e] * inv * wb[e];
     }
-    if (rot_half) {
-      const float c = cosv[(int64_t)token * rot_half + 4 * j + e], sn = sinv[(int64_t)token * rot_half + 4 * j + e];
-      out_lo[e] = from_float<T>(x * c - y * sn);
-      out_hi[e] = from_float<T>(y * c + x * sn);
-    } else {
-      out_lo[e] = from_float<T>(x);
-      out_hi[e] = from_float<T>(y);
+  }
+  vec out_lo, out_hi;
+  if (rot_half) {
+    float c[VE], sn[VE];
+    load_floats<float, VE>(cosv + (int64_t)token * rot_half + VE * j, c);
+    load_floats<float, VE>(sinv + (int64_t)token * rot_half + VE * j, sn);
+#pragma unroll
+    for (int e = 0; e < VE; ++e) {
+      out_lo[e] = from_float<T>(a[e] * c[e] - b[e] * sn[e]);
+      out_hi[e] = from_float<T>(b[e] * c[e] + a[e] * sn[e]);
+    }
+  } else {
+#pragma unroll
+    for (int e = 0; e < VE; ++e) {
+      out_lo[e] = from_float<T>(a[e]);
+      out_hi[e] = from_float<T>(b[e]);
     }
   }
   T* dst = is_q ? src : k_pages + ((page * nkv + kv_head) * page_size + off) * d;
-  *(vec4*)(dst + 4 * j) = out_lo;
-  *(vec4*)(dst + half + 4 * j) = out_hi;
-}
-
-// The v heads of 16 consecutive tokens of the step and one kv head, through LDS into the value
-// pages [page, kv_head, dim, slot]: tokens that follow each other in one page land side by side,
-// so a thread writes the values of 16 / sizeof(T) such tokens for one dim with one 16-byte store
-// (and falls back to single stores where a run is broken by a page edge, another request or a
-// slot that is not to be stored).  For steps of many tokens: storing token by token scatters
-// 2-byte writes a page row apart.
-template <typename T>
-__global__ __launch_bounds__(256) void values_to_pages_kernel(const T* __restrict__ qkv, int row_stride, int v_offset,
-                                                              int tokens, int nkv, int d, T* __restrict__ v_pages,
-                                                              const int* __restrict__ slots, int page_size) {
-  constexpr int RUN = 16 / sizeof(T);
-  typedef T vec __attribute__((ext_vector_type(RUN)));
-  extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
-  T* tile = (T*)lds_raw;                            // [d][17]
-  __shared__ int slot_of[16];
-  const int token0 = blockIdx.x * 16, kvh = blockIdx.y, tid = threadIdx.x;
-  const int count = tokens - token0 < 16 ? tokens - token0 : 16;
-  if (tid < 16) slot_of[tid] = tid < count ? slots[token0 + tid] : -1;
-  for (int e = tid; e < 16 * d; e += 256) {
-    const int i = e / d, dim = e % d;
-    if (i < count) tile[dim * 17 + i] = qkv[(int64_t)(token0 + i) * row_stride + v_offset + (int64_t)kvh * d + dim];
-  }
-  __syncthreads();
-  for (int e = tid; e < d * (16 / RUN); e += 256) {
-    const int dim = e / (16 / RUN), first = (e % (16 / RUN)) * RUN;
-    const int slot0 = slot_of[first];
-    bool run = slot0 >= 0 && slot0 % RUN == 0 && slot0 % page_size + RUN <= page_size;
-#pragma unroll
-    for (int i = 1; i < RUN; ++i) run = run && slot_of[first + i] == slot0 + i;
-    if (run) {
-      vec v;
-#pragma unroll
-      for (int i = 0; i < RUN; ++i) v[i] = tile[dim * 17 + first + i];
-      const int64_t page = slot0 / page_size, off = slot0 % page_size;
-      *(vec*)(v_pages + ((page * nkv + kvh) * d + dim) * page_size + off) = v;
-    } else {
-#pragma unroll
-      for (int i = 0; i < RUN; ++i) {
-        const int slot = slot_of[first + i];
-        if (slot < 0) continue;
-        const int64_t page = slot / page_size, off = slot % page_size;
-        v_pages[((page * nkv + kvh) * d + dim) * page_size + off] = tile[dim * 17 + first + i];
-      }
-    }
-  }
+  *(vec*)(dst + VE * j) = out_lo;
+  *(vec*)(dst + half + VE * j) = out_hi;
 }
 
 LRS_API int lrs_qk_prep(void* qkv, int dtype, int tokens, int row_stride, int nq, int nkv, int d,
@@ -352,34 +383,27 @@ LRS_API int lrs_qk_prep(void* qkv, int dtype, int tokens, int row_stride, int nq
   LRS_REQUIRE(row_stride >= (nq + 2 * nkv) * d, "qk_prep: row stride %d too small", row_stride);
   dim3 grid(tokens, nq + 2 * nkv), block(WAVE);
   hipStream_t s = (hipStream_t)stream;
-  // many tokens: the values go through a kernel of their own that writes whole runs of slots
+  // many tokens: the values are written in whole runs of slots, by workgroups of their own
   const size_t elem = dtype == LRS_F32 ? 4 : 2;
-  const bool values_apart = nkv > 0 && tokens >= 128 && page_size % (16 / elem) == 0 && ((uintptr_t)v_pages % 16) == 0 &&
-                            (size_t)d * 17 * elem <= 48 * 1024;
-  if (values_apart) {
-    dim3 vgrid((tokens + 15) / 16, nkv);
-    const size_t lds = (size_t)d * 17 * elem;
-    if (dtype == LRS_F32)
-      values_to_pages_kernel<float><<<vgrid, 256, lds, s>>>((const float*)qkv, row_stride, (nq + nkv) * d, tokens, nkv, d, (float*)v_pages, slots, page_size);
-    else if (dtype == LRS_BF16)
-      values_to_pages_kernel<bf16><<<vgrid, 256, lds, s>>>((const bf16*)qkv, row_stride, (nq + nkv) * d, tokens, nkv, d, (bf16*)v_pages, slots, page_size);
-    else
-      return lrs_fail("qk_prep: unknown dtype %d", dtype);
-    if (lrs_check_launch("values_to_pages")) return 1;
-    v_pages = nullptr;
-  }
-  const int heads = nq + (values_apart ? nkv : 2 * nkv);    // heads the kernels below have work for
-  grid.y = heads;
-  const int per_head = d / 8;
-  const bool vectors = d % 8 == 0 && per_head <= 64 && (per_head & (per_head - 1)) == 0 && (rot_half == 0 || 2 * rot_half == d) &&
-                       row_stride % 4 == 0 && ((uintptr_t)qkv % 16) == 0 && ((uintptr_t)k_pages % 16) == 0;
+  const int ve = (int)(16 / elem);
+  const bool values_apart = nkv > 0 && tokens >= 128 && page_size % ve == 0 && ((uintptr_t)v_pages % 16) == 0;
+  const int per_head = d / (2 * ve);
+  const bool vectors = d % (2 * ve) == 0 && per_head <= 64 && (per_head & (per_head - 1)) == 0 && (rot_half == 0 || 2 * rot_half == d) &&
+                       row_stride % ve == 0 && ((uintptr_t)qkv % 16) == 0 && ((uintptr_t)k_pages % 16) == 0 &&
+                       ((uintptr_t)q_weight % 16) == 0 && ((uintptr_t)k_weight % 16) == 0 && ((uintptr_t)cosv % 16) == 0 &&
+                       ((uintptr_t)sinv % 16) == 0;
   if (vectors) {
-    const int heads_per_block = 256 / per_head;
-    dim3 vgrid(tokens, (heads + heads_per_block - 1) / heads_per_block);
-#define LAUNCH_VEC(T, TW)                                                                              \
-  qk_prep_vec_kernel<T, TW><<<vgrid, 256, 0, s>>>((T*)qkv, row_stride, nq, nkv, d, (const TW*)q_weight,  \
-                                                  (const TW*)k_weight, eps, cosv, sinv, rot_half,      \
-                                                  (T*)k_pages, (T*)v_pages, slots, page_size)
+    const int heads = nq + (values_apart ? nkv : 2 * nkv);    // heads the (token, head) pairs run over
+    const int64_t pairs = (int64_t)tokens * heads;
+    const int per_block = 256 / per_head;
+    const int64_t prep_blocks = (pairs + per_block - 1) / per_block;
+    const int64_t value_blocks = values_apart ? (int64_t)((tokens + 15) / 16) * nkv : 0;
+    LRS_REQUIRE(prep_blocks + value_blocks < (1ll << 31), "qk_prep: %d tokens are too many for one launch", tokens);
+    dim3 vgrid((unsigned)(prep_blocks + value_blocks));
+#define LAUNCH_VEC(T, TW)                                                                                        \
+  qk_prep_vec_kernel<T, TW><<<vgrid, 256, 0, s>>>((T*)qkv, row_stride, tokens, heads, nq, nkv, d, (const TW*)q_weight, \
+                                                  (const TW*)k_weight, eps, cosv, sinv, rot_half, (T*)k_pages,   \
+                                                  (T*)v_pages, slots, page_size, (int)prep_blocks)
     if (dtype == LRS_F32 && w_dtype == LRS_F32) LAUNCH_VEC(float, float);
     else if (dtype == LRS_BF16 && w_dtype == LRS_BF16) LAUNCH_VEC(bf16, bf16);
     else if (dtype == LRS_BF16 && w_dtype == LRS_F32) LAUNCH_VEC(bf16, float);
@@ -387,6 +411,18 @@ LRS_API int lrs_qk_prep(void* qkv, int dtype, int tokens, int row_stride, int nq
     else return lrs_fail("qk_prep: unknown dtypes %d/%d", dtype, w_dtype);
 #undef LAUNCH_VEC
     return lrs_check_launch("qk_prep");
+  }
+  if (values_apart) {
+    dim3 vgrid((tokens + 15) / 16, nkv);
+    if (dtype == LRS_F32)
+      values_to_pages_kernel<float><<<vgrid, 256, 0, s>>>((const float*)qkv, row_stride, (nq + nkv) * d, tokens, nkv, d, (float*)v_pages, slots, page_size);
+    else if (dtype == LRS_BF16)
+      values_to_pages_kernel<bf16><<<vgrid, 256, 0, s>>>((const bf16*)qkv, row_stride, (nq + nkv) * d, tokens, nkv, d, (bf16*)v_pages, slots, page_size);
+    else
+      return lrs_fail("qk_prep: unknown dtype %d", dtype);
+    if (lrs_check_launch("values_to_pages")) return 1;
+    v_pages = nullptr;
+    grid.y = nq + nkv;
   }
 #define LAUNCH(T, TW)                                                                          \
   qk_prep_kernel<T, TW><<<grid, block, 0, s>>>((T*)qkv, row_stride, nq, nkv, d, (const TW*)q_weight, \
