@@ -595,6 +595,67 @@ def test_attention_finds_a_far_key(ops, dtype):
         torch.testing.assert_close(out.cpu().float()[0, :d], v[far, 0].to(dtype).float(), rtol=2e-2, atol=2e-2)
 
 
+@pytest.mark.parametrize("window,planted", [(0, 0), (0, 17), (0, 527), (100, 600), (100, 599), (100, 595), (100, 689), (33, 660)])
+def test_one_key_stands_out_in_every_attention_kernel(ops, window, planted):
+    """Ten new tokens after 690 cached ones, every query pointing at one planted key whose score dwarfs the
+    rest.  Without a window every query must return that key's value, wherever it lies (first tile, a page
+    edge, deep in the cache); with a window the key counts for exactly the queries whose window still holds
+    it (595 with a window of 100: positions 690..694 yes, 695..699 no; 599: only 690..698) and a kernel
+    that is one off at the window's edge returns a different row.  All kernels: the general one, the
+    matrix-core decode kernel (last token; whole and split over keys) and the ragged prefill kernel."""
+    nq, nkv, d, page, before, new = 4, 2, 64, 16, 690, 10
+    length = before + new
+    g = torch.Generator().manual_seed(70 + planted)
+    k = (torch.randn(length, nkv, d, generator=g) * 0.1).bfloat16()
+    v = torch.randn(length, nkv, d, generator=g).bfloat16()
+    direction = torch.randn(d, generator=g)
+    direction = direction / direction.norm()
+    k[planted] = (direction * 40).bfloat16()
+    q = (direction * 2).bfloat16().expand(new, nq, d).contiguous()      # score 80 * scale at the planted key
+    scale = 1.0
+    n_pages = (length + page - 1) // page
+    order = torch.randperm(n_pages + 2, generator=g)[:n_pages]
+    kp = torch.randn(n_pages + 2, nkv, page, d, generator=g)
+    vp = torch.randn(n_pages + 2, nkv, d, page, generator=g)
+    for b in range(n_pages):
+        n = min(page, length - b * page)
+        kp[order[b], :, :n] = k[b * page: b * page + n].float().transpose(0, 1)
+        vp[order[b], :, :, :n] = v[b * page: b * page + n].float().permute(1, 2, 0)
+    table = order.to(torch.int32).view(1, -1)
+    meta = [(0, before + i) for i in range(new)]
+    want = _attention_reference(q.float(), [k.float()], [v.float()], meta, None, nq, nkv, d, scale, window)
+    for i, (_, pos) in enumerate(meta):     # the scenario is what the docstring says
+        seen = planted <= pos and (window == 0 or planted > pos - window)
+        close = torch.allclose(want[i, :d], v[planted, 0].double(), atol=1e-2)
+        assert close == seen, (pos, seen)
+    q_wide = torch.zeros(new, (nq + 2 * nkv) * d, dtype=torch.bfloat16)
+    q_wide[:, : nq * d] = q.view(new, nq * d)
+    request = dev(torch.zeros(new, dtype=torch.int32))
+    positions = dev(torch.tensor([pos for _, pos in meta], dtype=torch.int32))
+    pages = (dev(kp.bfloat16()), dev(vp.bfloat16()))
+    out = torch.full((new, nq * d), float("nan"), device="cuda", dtype=torch.bfloat16)
+    ops.attention(out, dev(q_wide), *pages, dev(table), request, positions, nq, scale, window)
+    torch.testing.assert_close(out.cpu().double(), want, rtol=2e-2, atol=2e-2)
+    for splits in (1, 4, 11):
+        last = torch.full((1, nq * d), float("nan"), device="cuda", dtype=torch.bfloat16)
+        part_o = torch.full((1, nq * splits * d), float("nan"), device="cuda")
+        part_ml = torch.full((1, nq * splits * 2), float("nan"), device="cuda")
+        for form in (0, 1, 2):
+            ops.attention_decode(last, dev(q_wide[-1:]), *pages, dev(table), request[:1], positions[-1:], nq, scale, window,
+                                 splits, part_o, part_ml, form=form)
+            torch.testing.assert_close(last.cpu().double(), want[-1:], rtol=2e-2, atol=2e-2)
+    for size, splits in ((16, 1), (32, 1), (4, 1), (16, 5), (32, 16)):
+        groups = [(i, min(size, new - i)) for i in range(0, new, size)]
+        fast = torch.full((new, nq * d), float("nan"), device="cuda", dtype=torch.bfloat16)
+        part_o = torch.full((new, nq * splits * d), float("nan"), device="cuda") if splits > 1 else None
+        part_ml = torch.full((new, nq * splits * 2), float("nan"), device="cuda") if splits > 1 else None
+        ops.attention_prefill(fast, dev(q_wide), *pages, dev(table), request, positions,
+                              dev(torch.tensor([b[0] for b in groups], dtype=torch.int32)),
+                              dev(torch.tensor([b[1] for b in groups], dtype=torch.int32)), nq, scale, window, size,
+                              splits=splits, part_o=part_o, part_ml=part_ml)
+        torch.testing.assert_close(fast.cpu().double(), want, rtol=2e-2, atol=2e-2)
+
+
 @pytest.mark.parametrize("rows,vocab", [(1, 256), (5, 331), (3, 151936), (5, 20000)])
 def test_choose_tokens_greedy(ops, rows, vocab):
     g = torch.Generator().manual_seed(8)
