@@ -3,7 +3,9 @@
 The library is kept inside the package folder next to a file holding the hash of the
 sources it was built from.  `ensure_built()` compiles only when no library matching
 the sources exists, printing a line as each file starts and finishes, so that a first
-call in a fresh checkout shows progress.  Files are compiled in parallel.
+call in a fresh checkout shows progress.  Files are compiled in parallel.  A checkout
+that the user cannot write to gets its library in a folder of the user's own under the
+temporary directory, named by the hash of the sources.
 """
 
 from __future__ import annotations
@@ -13,6 +15,7 @@ import os
 import shutil
 import subprocess
 import sys
+import tempfile
 import time
 from concurrent.futures import ThreadPoolExecutor
 from pathlib import Path
@@ -48,6 +51,15 @@ def is_current() -> bool:
     return LIBRARY.is_file() and HASH_FILE.is_file() and HASH_FILE.read_text().strip() == source_hash()
 
 
+def _outside_the_checkout() -> Path:
+    """Where the library goes when the checkout cannot be written to."""
+    return Path(tempfile.gettempdir()) / f"lrs_kernels_{os.getuid()}_{source_hash()[:16]}"
+
+
+def _writable(folder: Path) -> bool:
+    return os.access(folder, os.W_OK | os.X_OK)
+
+
 def _hipcc() -> str:
     found = shutil.which("hipcc") or ("/opt/rocm/bin/hipcc" if os.path.exists("/opt/rocm/bin/hipcc") else None)
     if found is None:
@@ -72,8 +84,15 @@ def build(force: bool = True) -> Path:
     """Compile every source and link the library; returns its path."""
     if not force and is_current():
         return LIBRARY
+    library, hash_file, build_dir = LIBRARY, HASH_FILE, SOURCE_DIR / "_build"
+    if not (_writable(LIBRARY.parent) and _writable(SOURCE_DIR)):
+        folder = _outside_the_checkout()
+        library, hash_file, build_dir = folder / LIBRARY.name, folder / HASH_FILE.name, folder / "_build"
+        if not force and library.is_file() and hash_file.is_file() and hash_file.read_text().strip() == source_hash():
+            return library
+        folder.mkdir(mode=0o700, exist_ok=True)
+        _say(f"{LIBRARY.parent} is not writable: building in {folder}")
     hipcc = _hipcc()
-    build_dir = SOURCE_DIR / "_build"
     build_dir.mkdir(exist_ok=True)
     srcs = sources()
     if not srcs:
@@ -84,17 +103,17 @@ def build(force: bool = True) -> Path:
     with ThreadPoolExecutor(max_workers=workers) as pool:
         for future in [pool.submit(_compile_one, hipcc, s, o) for s, o in zip(srcs, objects)]:
             future.result()
-    tmp = LIBRARY.with_suffix(f".so.tmp{os.getpid()}")
+    tmp = library.with_suffix(f".so.tmp{os.getpid()}")
     proc = subprocess.run(
         [hipcc, f"--offload-arch={ARCH}", "-shared", "-fPIC", *map(str, objects), "-o", str(tmp)],
         capture_output=True, text=True,
     )
     if proc.returncode != 0:
         raise BuildError(f"linking the kernel library failed:\n{proc.stderr}")
-    os.replace(tmp, LIBRARY)
-    HASH_FILE.write_text(source_hash() + "\n")
-    _say(f"built {LIBRARY.name} in {time.time() - started:.1f} s")
-    return LIBRARY
+    os.replace(tmp, library)
+    hash_file.write_text(source_hash() + "\n")
+    _say(f"built {library.name} in {time.time() - started:.1f} s")
+    return library
 
 
 def ensure_built() -> Path:

@@ -18,6 +18,7 @@ from ..errors import KernelError
 from . import build as _build
 
 _lib = None
+_lib_path = ""
 
 F32, BF16 = 0, 1
 OUT_STORE, OUT_STORE_F32, OUT_ADD_F32 = 0, 1, 2
@@ -73,11 +74,12 @@ _SIGNATURES = {
 
 def library():
     """Load (building first if needed) the kernel library; raises KernelError if impossible."""
-    global _lib
+    global _lib, _lib_path
     if _lib is None:
         try:
             path = _build.ensure_built()
             lib = ctypes.CDLL(str(path))
+            _lib_path = str(path)
         except (_build.BuildError, OSError) as exc:
             raise KernelError(f"the HIP kernel library is not available: {exc}") from exc
         for name, (restype, argtypes) in _SIGNATURES.items():
@@ -92,7 +94,7 @@ def library():
 
 def loaded_library_path() -> str:
     library()
-    return str(_build.LIBRARY)
+    return _lib_path
 
 
 def _check(code: int) -> None:
