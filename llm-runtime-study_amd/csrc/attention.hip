@@ -219,6 +219,44 @@ __global__ __launch_bounds__(WAVES * 64) void attention_decode_bf16_kernel(
     for (int i = tid; i <= last_key / page_size - first_block; i += THREADS) page_ids[i] = table[first_block + i];
 
   const bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
+  // Every key and value fragment of a tile is requested before any is used, so a tile costs one
+  // trip to memory instead of two.  Which of the tile's 32 keys a row of the two key blocks stands
+  // for is chosen so that a lane ends up with the weights of eight consecutive keys, g*8 .. g*8+7:
+  // block h, row 4*r + i is key 8*r + 4*h + i.  The values of those eight keys lie side by side in
+  // the (transposed) page, one 16-byte load a dim.
+  const int key_of_row = (col >> 2) * 8 + (col & 3);           // + 4*h
+  auto fetch = [&](int tile, bf16x8 (&kf)[2][DS], bf16x8 (&vf)[DB]) {
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      const int key = tile * 32 + key_of_row + 4 * h;
+      if (key <= pos && key >= lo) {
+        const int64_t page = page_ids[key / page_size - first_block];
+        const bf16* kp = k_pages + ((page * nkv + kvh) * page_size + key % page_size) * D + g * 8;
+#pragma unroll
+        for (int c = 0; c < DS; ++c) kf[h][c] = *(const bf16x8*)(kp + c * 32);
+      } else {
+#pragma unroll
+        for (int c = 0; c < DS; ++c) kf[h][c] = zero8;
+      }
+    }
+    const int key8 = tile * 32 + g * 8;                        // this lane's eight keys; pages hold multiples of 16
+    if (key8 <= pos && key8 + 7 >= lo) {
+      const int64_t page = page_ids[key8 / page_size - first_block];
+      const bf16* vp = v_pages + (page * nkv + kvh) * (int64_t)D * page_size + (int64_t)col * page_size + key8 % page_size;
+#pragma unroll
+      for (int b = 0; b < DB; ++b) vf[b] = *(const bf16x8*)(vp + (int64_t)b * 16 * page_size);
+    } else {
+#pragma unroll
+      for (int b = 0; b < DB; ++b) vf[b] = zero8;
+    }
+  };
+  // AHEAD: the wave's first tile is asked for as soon as the page ids are there, before the query (and
+  // the new key) are prepared, so that the first trip to memory runs beside that work.
+  bf16x8 kf_a[AHEAD ? 2 : 1][AHEAD ? DS : 1], vf_a[AHEAD ? DB : 1];
+  if constexpr (AHEAD) {
+    __syncthreads();
+    if (tile_begin + wave < tile_end) fetch(tile_begin + wave, (bf16x8(&)[2][DS])kf_a, (bf16x8(&)[DB])vf_a);
+  }
   bf16x8 qf[DS];
   const bf16* q_row = q + (int64_t)token * q_stride;
   if (PREP) {
@@ -269,37 +307,6 @@ __global__ __launch_bounds__(WAVES * 64) void attention_decode_bf16_kernel(
   float run_max = -INFINITY, run_sum = 0.f;
   const float scale2 = scale * 1.4426950408889634f;
 
-  // Every key and value fragment of a tile is requested before any is used, so a tile costs one
-  // trip to memory instead of two.  Which of the tile's 32 keys a row of the two key blocks stands
-  // for is chosen so that a lane ends up with the weights of eight consecutive keys, g*8 .. g*8+7:
-  // block h, row 4*r + i is key 8*r + 4*h + i.  The values of those eight keys lie side by side in
-  // the (transposed) page, one 16-byte load a dim.
-  const int key_of_row = (col >> 2) * 8 + (col & 3);           // + 4*h
-  auto fetch = [&](int tile, bf16x8 (&kf)[2][DS], bf16x8 (&vf)[DB]) {
-#pragma unroll
-    for (int h = 0; h < 2; ++h) {
-      const int key = tile * 32 + key_of_row + 4 * h;
-      if (key <= pos && key >= lo) {
-        const int64_t page = page_ids[key / page_size - first_block];
-        const bf16* kp = k_pages + ((page * nkv + kvh) * page_size + key % page_size) * D + g * 8;
-#pragma unroll
-        for (int c = 0; c < DS; ++c) kf[h][c] = *(const bf16x8*)(kp + c * 32);
-      } else {
-#pragma unroll
-        for (int c = 0; c < DS; ++c) kf[h][c] = zero8;
-      }
-    }
-    const int key8 = tile * 32 + g * 8;                        // this lane's eight keys; pages hold multiples of 16
-    if (key8 <= pos && key8 + 7 >= lo) {
-      const int64_t page = page_ids[key8 / page_size - first_block];
-      const bf16* vp = v_pages + (page * nkv + kvh) * (int64_t)D * page_size + (int64_t)col * page_size + key8 % page_size;
-#pragma unroll
-      for (int b = 0; b < DB; ++b) vf[b] = *(const bf16x8*)(vp + (int64_t)b * 16 * page_size);
-    } else {
-#pragma unroll
-      for (int b = 0; b < DB; ++b) vf[b] = zero8;
-    }
-  };
   auto work = [&](int tile, bf16x8 (&kf)[2][DS], bf16x8 (&vf)[DB]) {
     if (holds_own && tile == last_tile) {
       // the token's own key and value take the place of what the pages hold at its position
@@ -358,16 +365,16 @@ __global__ __launch_bounds__(WAVES * 64) void attention_decode_bf16_kernel(
       o[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[b], pf, o[b], 0, 0, 0);
     }
   };
-  if (AHEAD) {
+  if constexpr (AHEAD) {
     // two register sets in turn: the next tile of this wave is on its way while this one is worked on
-    bf16x8 kf_a[2][DS], vf_a[DB], kf_b[2][DS], vf_b[DB];
-    int tile = tile_begin + wave;
-    if (tile < tile_end) fetch(tile, kf_a, vf_a);
-    for (; tile < tile_end; tile += 2 * WAVES) {
+    bf16x8 (&kf_first)[2][DS] = (bf16x8(&)[2][DS])kf_a;
+    bf16x8 (&vf_first)[DB] = (bf16x8(&)[DB])vf_a;
+    bf16x8 kf_b[2][DS], vf_b[DB];
+    for (int tile = tile_begin + wave; tile < tile_end; tile += 2 * WAVES) {
       if (tile + WAVES < tile_end) fetch(tile + WAVES, kf_b, vf_b);
-      work(tile, kf_a, vf_a);
+      work(tile, kf_first, vf_first);
       if (tile + WAVES >= tile_end) break;
-      if (tile + 2 * WAVES < tile_end) fetch(tile + 2 * WAVES, kf_a, vf_a);
+      if (tile + 2 * WAVES < tile_end) fetch(tile + 2 * WAVES, kf_first, vf_first);
       work(tile + WAVES, kf_b, vf_b);
     }
   } else {

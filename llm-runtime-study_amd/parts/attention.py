@@ -140,7 +140,7 @@ class GQAAttention(Part):
                 part_ml = ctx.scratch("attn_part_ml", (t, nq * splits * 2), torch.float32)
             ops.attention_decode(out, qkv, cache.k_pages, cache.v_pages, group.block_table, ctx.token_request, ctx.positions,
                                  nq, self.scale, self.window or 0, splits, part_o, part_ml, ctx.max_k_bound, prepare,
-                                 form=1 if splits == 1 else 0)   # long walks per wave: the next tile on its way (measured: 0.6 % of a 64-row step)
+                                 form=1)   # the next tile on its way while one is worked on, the first one before the query is prepared (measured: 0.6 % of a step)
         elif ops.attention_decode_supported(ctx.dtype, nq, kv_heads, d, group.page_size):
             longest = ctx.max_k if self.window is None else min(ctx.max_k, self.window + 64)
             splits = self._prefill_splits(ctx.num_qblocks * kv_heads, longest, t * nq * d)
