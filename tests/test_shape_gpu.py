@@ -1,7 +1,8 @@
 """The kernels at the sizes of the model the benchmark runs (hidden 4096, 32/8 heads of 128 dims,
-feed-forward 12288, vocabulary 151936; two layers): the bfloat16 path with everything it uses at
-that size (graphs, fused norms, library products for many rows, key splits) against the float32
-path of the same weights, over prompts in portions, mixed steps and decode steps."""
+feed-forward 12288, vocabulary 151936; two layers) and at the layer sizes of the two larger dense
+models of the family (hidden 5120 with 40/8 and 64/8 heads): the bfloat16 path with everything it
+uses at that size (graphs, fused norms, library products for many rows, key splits) against the
+float32 path of the same weights, over prompts in portions, mixed steps and decode steps."""
 
 import numpy as np
 import pytest
@@ -19,14 +20,22 @@ SHAPE = {
 }
 
 
-def test_bfloat16_path_follows_float32_at_full_layer_sizes():
+LARGER = {
+    "8b": {},
+    "14b": {"hidden_size": 5120, "intermediate_size": 17408, "num_attention_heads": 40},
+    "32b": {"hidden_size": 5120, "intermediate_size": 25600, "num_attention_heads": 64},
+}
+
+
+@pytest.mark.parametrize("sizes", list(LARGER))
+def test_bfloat16_path_follows_float32_at_full_layer_sizes(sizes):
     from llm_runtime_study_amd.cache import CacheManager
     from llm_runtime_study_amd.config import config_from_dict, spec_for
     from llm_runtime_study_amd.engine.step import ModelRunner, StepEntry
     from llm_runtime_study_amd.models import DecoderModel
     from llm_runtime_study_amd.weights import random_init
 
-    cfg = config_from_dict(SHAPE)
+    cfg = config_from_dict(dict(SHAPE, **LARGER[sizes]))
     device = torch.device("cuda", 0)
     weights = random_init.device_weights(DecoderModel(spec_for(cfg)), 0, torch.bfloat16, device, "scaled")
     rng = np.random.default_rng(1)
