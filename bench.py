@@ -1,6 +1,6 @@
 """Decode and prefill throughput of the Qwen3-8B shape with random weights on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--context 2048] [--layers L]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--context 2048] [--layers L] [--shape 8b|14b|32b]
 
 A step is one decode step of the whole engine (scheduler, step function, sampling) at the
 given batch; `value` is decoded tokens per second.  The same line carries the prefill rate
@@ -34,6 +34,12 @@ QWEN3_8B = {
     "torch_dtype": "bfloat16", "bos_token_id": 151643, "eos_token_id": 151645,
 }
 FULL_LAYERS = QWEN3_8B["num_hidden_layers"]
+# the two larger dense models of the family, for runs at further sizes (--shape)
+SHAPES = {
+    "8b": QWEN3_8B,
+    "14b": dict(QWEN3_8B, hidden_size=5120, intermediate_size=17408, num_hidden_layers=40, num_attention_heads=40),
+    "32b": dict(QWEN3_8B, hidden_size=5120, intermediate_size=25600, num_hidden_layers=64, num_attention_heads=64),
+}
 
 
 def parse_args():
@@ -44,7 +50,8 @@ def parse_args():
     parser.add_argument("--batch", type=int, default=8)
     parser.add_argument("--context", type=int, default=2048)
     parser.add_argument("--prefill-tokens", type=int, default=2048)
-    parser.add_argument("--layers", type=int, default=FULL_LAYERS, help="fewer layers than the shape has (reported in config)")
+    parser.add_argument("--shape", choices=tuple(SHAPES), default="8b", help="layer sizes: Qwen3-8B (default), 14B or 32B")
+    parser.add_argument("--layers", type=int, default=None, help="fewer layers than the shape has (reported in config)")
     parser.add_argument("--dtype", choices=("bfloat16", "float32"), default="bfloat16")
     parser.add_argument("--no-points", action="store_true", help="skip the batch 1 and 64 decode points")
     parser.add_argument("--no-graph", action="store_true")
@@ -159,7 +166,10 @@ def main() -> int:
     from llm_runtime_study_amd import Engine
     from llm_runtime_study_amd.config import config_from_dict
 
-    raw = dict(QWEN3_8B, num_hidden_layers=args.layers)
+    full_layers = SHAPES[args.shape]["num_hidden_layers"]
+    if args.layers is None:
+        args.layers = full_layers
+    raw = dict(SHAPES[args.shape], num_hidden_layers=args.layers)
     config = config_from_dict(raw)
     max_batch = args.batch if args.no_points else max(args.batch, 64)
     max_seq_len = args.context + args.steps + args.warmup + decode_lead(max_batch, args.context, max(2048, args.prefill_tokens)) + max_batch + 64
@@ -188,7 +198,7 @@ def main() -> int:
             points[f"decode_b{batch}"] = round(batch * len(t) / sum(t), 2)
 
     line = {
-        "metric": f"decode tok/s at batch {args.batch} (Qwen3-8B shape)",
+        "metric": f"decode tok/s at batch {args.batch} (Qwen3-{args.shape.upper()} shape)",
         "value": round(args.batch * len(times) / total, 2),
         "unit": "tok/s",
         "n_gpus": 1,
@@ -201,7 +211,7 @@ def main() -> int:
         "dtype": dtype_name,
         "data": "synthetic (seeded uniform random token ids, random weights N(0, 0.02))",
         "config": {
-            "model": "Qwen3-8B shape", "layers": args.layers, "layers_of_shape": FULL_LAYERS,
+            "model": f"Qwen3-{args.shape.upper()} shape", "layers": args.layers, "layers_of_shape": full_layers,
             "hidden_size": config.hidden_size, "intermediate_size": config.intermediate_size,
             "num_attention_heads": config.num_attention_heads, "num_key_value_heads": config.num_key_value_heads,
             "head_dim": config.head_dim, "vocab_size": config.vocab_size, "global_batch": args.batch,
