@@ -7,6 +7,8 @@
 // else is in the batch.
 #include "common.h"
 
+#include <type_traits>
+
 enum { OUT_STORE = 0, OUT_STORE_F32 = 1, OUT_ADD_F32 = 2 };
 
 template <typename T>
@@ -302,31 +304,47 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_skinny_kernel(
       early_w[q] = !inside ? 0.f : chain.next_weight_is_f32 ? ((const float*)chain.next_weight)[gn] : (float)((const bf16*)chain.next_weight)[gn];
     }
   }
-  // Workgroups walk their K slices from different starting points (the order of a column's sum
-  // depends on the column alone): all of them read the same activations, and in step they would
-  // all ask the same few cache lines of the L2 at the same moment.
-  const int batches = full_end > s ? (full_end - s) / UNROLL : 0;
-  const int s_first = s;
-  for (int j = 0; j < batches; ++j) {
-    const int sb = s_first + ((j + (int)blockIdx.x) % batches) * UNROLL;
-    bf16x8 a[UNROLL][RT], b[UNROLL][MT];
+  // U steps of 32 k, all their loads asked for before any is used
+  auto steps_together = [&](int sb, auto count) {
+    constexpr int U = decltype(count)::value;
+    bf16x8 a[U][RT], b[U][MT];
 #pragma unroll
-    for (int u = 0; u < UNROLL; ++u)
+    for (int u = 0; u < U; ++u)
 #pragma unroll
       for (int q = 0; q < RT; ++q) a[u][q] = *(const bf16x8*)(wp[q] + (sb + u) * 32);
 #pragma unroll
-    for (int u = 0; u < UNROLL; ++u)
+    for (int u = 0; u < U; ++u)
 #pragma unroll
       for (int t = 0; t < MT; ++t) b[u][t] = load_b(t, sb + u);
 #pragma unroll
-    for (int u = 0; u < UNROLL; ++u)
+    for (int u = 0; u < U; ++u)
 #pragma unroll
       for (int q = 0; q < RT; ++q)
 #pragma unroll
         for (int t = 0; t < MT; ++t)
           acc[q][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[u][q], b[u][t], acc[q][t], 0, 0, 0);
-  }
+  };
+  // Workgroups walk their K slices from different starting points (the order of a column's sum
+  // depends on the column alone): all of them read the same activations, and in step they would
+  // all ask the same few cache lines of the L2 at the same moment.
+  const int batches = full_end > s ? (full_end - s) / UNROLL : 0;
+  const int s_first = s;
+  for (int j = 0; j < batches; ++j)
+    steps_together(s_first + ((j + (int)blockIdx.x) % batches) * UNROLL, std::integral_constant<int, UNROLL>{});
   s = s_first + batches * UNROLL;
+  // what is left of the whole steps, in shrinking groups (a step alone costs a trip to memory of its own)
+  if constexpr (UNROLL > 4) {
+    if (full_end - s >= 4) {
+      steps_together(s, std::integral_constant<int, 4>{});
+      s += 4;
+    }
+  }
+  if constexpr (UNROLL > 2) {
+    if (full_end - s >= 2) {
+      steps_together(s, std::integral_constant<int, 2>{});
+      s += 2;
+    }
+  }
   for (; s < s_end; ++s) {
     const bool inside = s * 32 + g * 8 < k;
     bf16x8 b[MT];
