@@ -197,12 +197,15 @@ struct NormChain {
 
 __device__ __forceinline__ float silu(float g) { return g / (1.0f + __expf(-g)); }
 
-template <int MT, int RT, int WAVES, int UNROLL, bool NORM, bool SWIGLU>
+template <int MT, int RT, int WAVES, int UNROLL, bool NORM, bool SWIGLU, bool PARTIAL = false>
 __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_skinny_kernel(
     void* __restrict__ out, int mode, const bf16* __restrict__ x, NormInput norm,
     const bf16* __restrict__ w, const bf16* __restrict__ bias, int m, int n, int k, int lda, int ldc,
-    float* __restrict__ split_sums, NormChain chain) {
+    float* __restrict__ split_sums, NormChain chain, int group_rows) {
   // RT: row tiles of 16 weight rows per workgroup; every activation fragment is used RT times.
+  // group_rows (16 * RT unless PARTIAL): the weight rows a workgroup owns; fewer than its tiles hold
+  // when that divides the matrix evenly between the compute units (rows past them are neither
+  // loaded nor written).
   // gridDim.y > 1: K is also divided between workgroups; each then leaves its sums in
   // split_sums [gridDim.y, m, n] for gemm_split_finish_kernel instead of writing the output.
   __shared__ floatx4 partial[WAVES][MT][WAVE];
@@ -212,11 +215,14 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_skinny_kernel(
   __shared__ float chain_squares[16][RT * 16 + 1];
   const int tid = threadIdx.x, lane = tid % WAVE, wave = tid / WAVE;
   const int r = lane & 15, g = lane >> 4;
-  const int n0 = blockIdx.x * 16 * RT;
+  const int n0 = blockIdx.x * group_rows;
+  const int n_end = n0 + group_rows < n ? n0 + group_rows : n;      // this workgroup's rows are [n0, n_end)
   const bf16* wp[RT];
+  bool wrow[RT];
 #pragma unroll
   for (int q = 0; q < RT; ++q) {
-    const int row = n0 + q * 16 + r < n ? n0 + q * 16 + r : n - 1;
+    wrow[q] = !PARTIAL || n0 + q * 16 + r < n_end;
+    const int row = PARTIAL ? (wrow[q] ? n0 + q * 16 + r : n0) : (n0 + q * 16 + r < n ? n0 + q * 16 + r : n - 1);
     wp[q] = w + (int64_t)row * k + g * 8;
   }
   const bf16* xp[MT];
@@ -299,7 +305,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_skinny_kernel(
 #pragma unroll
     for (int q = 0; q < RT; ++q) {
       const int gn = n0 + q * 16 + 4 * (l >> 4) + i;
-      const bool inside = token < m && gn < n;
+      const bool inside = token < m && gn < n_end;
       early_h[q] = inside ? ((const float*)out)[(int64_t)token * ldc + gn] : 0.f;
       early_w[q] = !inside ? 0.f : chain.next_weight_is_f32 ? ((const float*)chain.next_weight)[gn] : (float)((const bf16*)chain.next_weight)[gn];
     }
@@ -311,7 +317,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_skinny_kernel(
 #pragma unroll
     for (int u = 0; u < U; ++u)
 #pragma unroll
-      for (int q = 0; q < RT; ++q) a[u][q] = *(const bf16x8*)(wp[q] + (sb + u) * 32);
+      for (int q = 0; q < RT; ++q) a[u][q] = !PARTIAL || wrow[q] ? *(const bf16x8*)(wp[q] + (sb + u) * 32) : zero;
 #pragma unroll
     for (int u = 0; u < U; ++u)
 #pragma unroll
@@ -352,7 +358,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_skinny_kernel(
     for (int t = 0; t < MT; ++t) b[t] = inside ? load_b(t, s) : zero;
 #pragma unroll
     for (int q = 0; q < RT; ++q) {
-      const bf16x8 a = inside ? *(const bf16x8*)(wp[q] + s * 32) : zero;
+      const bf16x8 a = inside && (!PARTIAL || wrow[q]) ? *(const bf16x8*)(wp[q] + s * 32) : zero;
 #pragma unroll
       for (int t = 0; t < MT; ++t) acc[q][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b[t], acc[q][t], 0, 0, 0);
     }
@@ -409,7 +415,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_skinny_kernel(
       for (int e = tid; e < MT * WAVE * 4; e += WAVES * WAVE) {
         const int t = e / (WAVE * 4), l = (e / 4) % WAVE, i = e % 4;
         const int token = t * 16 + (l & 15), gn = nq0 + 4 * (l >> 4) + i;
-        if (token < m && gn < n) split_sums[((int64_t)blockIdx.y * m + token) * n + gn] = total(t, l, i);
+        if (token < m && gn < n_end) split_sums[((int64_t)blockIdx.y * m + token) * n + gn] = total(t, l, i);
       }
     } else if (SWIGLU) {
       for (int e = tid; e < MT * 16 * 8; e += WAVES * WAVE) {
@@ -423,7 +429,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_skinny_kernel(
       for (int e = tid; e < MT * WAVE * 4; e += WAVES * WAVE) {
         const int t = e / (WAVE * 4), l = (e / 4) % WAVE, i = e % 4;
         const int token = t * 16 + (l & 15), gn = nq0 + 4 * (l >> 4) + i;
-        const bool inside = token < m && gn < n;
+        const bool inside = token < m && gn < n_end;
         if (feeds_norm && !inside) chain_squares[l & 15][q * 16 + 4 * (l >> 4) + i] = 0.f;
         if (!inside) continue;
         float v = total(t, l, i);
@@ -475,18 +481,36 @@ __global__ void gemm_split_finish_kernel(void* __restrict__ out, int mode, const
 template <int MT, int RT, bool NORM, bool SWIGLU>
 static void launch_skinny_rt(void* out, int mode, const bf16* a, NormInput norm, const bf16* w, const bf16* bias,
                              int m, int n, int k, int lda, int ldc, hipStream_t s, float* split_sums = nullptr, int splits = 1,
-                             NormChain chain = NormChain{}) {
-  const int groups = (n + 16 * RT - 1) / (16 * RT);
+                             NormChain chain = NormChain{}, int group_rows = 16 * RT) {
+  const int groups = (n + group_rows - 1) / group_rows;
   constexpr int UNROLL = (NORM ? 4 : 8) / (MT * RT > 4 ? 4 : (MT * RT > 1 ? 2 : 1));
-  if (groups <= 2048)
-    gemm_bf16_skinny_kernel<MT, RT, 8, UNROLL, NORM, SWIGLU><<<dim3(groups, splits), 8 * 64, 0, s>>>(out, mode, a, norm, w, bias, m, n, k, lda, ldc, split_sums, chain);
+  if (group_rows != 16 * RT) {
+    if constexpr (MT == 1 && RT == 2 && !NORM && !SWIGLU)
+      gemm_bf16_skinny_kernel<MT, RT, 8, UNROLL, NORM, SWIGLU, true><<<dim3(groups, splits), 8 * 64, 0, s>>>(out, mode, a, norm, w, bias, m, n, k, lda, ldc, split_sums, chain, group_rows);
+  } else if (groups <= 2048)
+    gemm_bf16_skinny_kernel<MT, RT, 8, UNROLL, NORM, SWIGLU><<<dim3(groups, splits), 8 * 64, 0, s>>>(out, mode, a, norm, w, bias, m, n, k, lda, ldc, split_sums, chain, group_rows);
   else
-    gemm_bf16_skinny_kernel<MT, RT, 4, UNROLL, NORM, SWIGLU><<<dim3(groups, splits), 4 * 64, 0, s>>>(out, mode, a, norm, w, bias, m, n, k, lda, ldc, split_sums, chain);
+    gemm_bf16_skinny_kernel<MT, RT, 4, UNROLL, NORM, SWIGLU><<<dim3(groups, splits), 4 * 64, 0, s>>>(out, mode, a, norm, w, bias, m, n, k, lda, ldc, split_sums, chain, group_rows);
   if (splits > 1) {
     const int64_t total = (int64_t)m * (SWIGLU ? n / 2 : n);
     const int blocks = (int)((total + 255) / 256 < 1024 ? (total + 255) / 256 : 1024);
     gemm_split_finish_kernel<SWIGLU><<<blocks, 256, 0, s>>>(out, mode, split_sums, bias, m, n, ldc, splits);
   }
+}
+
+LRS_API int lrs_compute_units();
+
+// Weight rows per workgroup for a product of at most 16 rows and n output columns that is narrow
+// enough for one row tile per workgroup (n < 16384, no gated epilogue).  16, unless that leaves the
+// compute units unevenly loaded (n = 5120: 320 workgroups for 256 units, a quarter of them with twice
+// the work): then the rows are dealt out evenly over a whole multiple of the units, between 16 and 32
+// a workgroup (two tiles, the second partly empty).  Measured on MI355X at 8 rows: 6144 columns
+// 16.7 -> 14.5 us, 5120 columns (K 5120 and 17408) 19.9 -> 15.9 and 56.0 -> 39.6 us.  0: 16 rows.
+static int even_group_rows(int n) {
+  const int units = lrs_compute_units(), tiles = (n + 15) / 16;
+  if (units <= 0 || tiles <= units || tiles % units == 0) return 0;
+  const int rows = (n + units * (tiles / units) - 1) / (units * (tiles / units));
+  return rows <= 32 ? rows : 0;
 }
 
 // Device memory for the sums of K splits, made on first use and kept (one per process: one GPU).
@@ -514,8 +538,11 @@ static void launch_skinny(void* out, int mode, const bf16* a, NormInput norm, co
     return;
   }
   if (MT == 1 && !NORM && n >= 16384)   // measured: two row tiles and four waves stream wide matrices a little faster
-    gemm_bf16_skinny_kernel<1, 2, 4, 4, NORM, SWIGLU><<<dim3((n + 31) / 32, 1), 4 * 64, 0, s>>>(out, mode, a, norm, w, bias, m, n, k, lda, ldc, nullptr, chain);
-  else if (MT == 1 || n <= 32 * 128)
+    gemm_bf16_skinny_kernel<1, 2, 4, 4, NORM, SWIGLU><<<dim3((n + 31) / 32, 1), 4 * 64, 0, s>>>(out, mode, a, norm, w, bias, m, n, k, lda, ldc, nullptr, chain, 32);
+  else if (MT == 1 && !NORM && !SWIGLU && even_group_rows(n) > 0) {
+    if constexpr (MT == 1 && !NORM && !SWIGLU)
+      launch_skinny_rt<1, 2, false, false>(out, mode, a, norm, w, bias, m, n, k, lda, ldc, s, nullptr, 1, chain, even_group_rows(n));
+  } else if (MT == 1 || n <= 32 * 128)
     launch_skinny_rt<MT, 1, NORM, SWIGLU>(out, mode, a, norm, w, bias, m, n, k, lda, ldc, s, nullptr, 1, chain);
   else if (n < 64 * 256)
     launch_skinny_rt<MT, 2, NORM, SWIGLU>(out, mode, a, norm, w, bias, m, n, k, lda, ldc, s);
@@ -552,7 +579,11 @@ LRS_API int lrs_gemm_set_skinny_max_m(int m) {
 
 // How many partial sums of squares a product of n output columns leaves for the norm that follows it
 // (the number of workgroups of the few-rows kernel for that width).
-LRS_API int lrs_gemm_norm_chain_parts(int n) { return n >= 16384 ? (n + 31) / 32 : (n + 15) / 16; }
+LRS_API int lrs_gemm_norm_chain_parts(int n) {
+  if (n >= 16384) return (n + 31) / 32;
+  const int rows = even_group_rows(n);
+  return rows > 0 ? (n + rows - 1) / rows : (n + 15) / 16;
+}
 
 // The few-rows bf16 product (M <= 16) with an RMSNorm of the residual stream taken apart around it;
 // see NormChain.  in_sumsq != null: `a` is bf16(h * g) and row r of the result is scaled by

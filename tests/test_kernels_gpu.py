@@ -212,6 +212,7 @@ def test_add_into(ops, dtype):
 @pytest.mark.parametrize("m,n,k", [
     (1, 64, 64), (5, 331, 96), (17, 160, 96), (64, 256, 160), (130, 200, 264), (3, 129, 40),
     (2, 70, 36), (1, 1000, 4096), (257, 384, 512),
+    (8, 5120, 160), (3, 4112, 72), (16, 12290, 64),      # few rows, widths that are dealt out unevenly by 16-row tiles
 ])
 @pytest.mark.parametrize("mode", ["store", "store_f32", "add"])
 def test_gemm(ops, dtype, m, n, k, mode):
@@ -284,7 +285,8 @@ def test_gemm_with_swiglu_epilogue(ops, m, inter, k, all_rows_in_own_kernel):
 
 @pytest.mark.parametrize("w_dtype", DTYPES)
 @pytest.mark.parametrize("m,h,n2,k,swiglu", [(1, 64, 96, 32, False), (8, 4096, 6144, 4096, False), (16, 4096, 24576, 12288, True),
-                                             (5, 104, 328, 72, False), (9, 96, 320, 160, True), (3, 16400, 48, 64, False)])
+                                             (5, 104, 328, 72, False), (9, 96, 320, 160, True), (3, 16400, 48, 64, False),
+                                             (7, 5120, 7168, 640, False), (4, 4112, 4400, 96, False)])
 def test_gemm_with_norm_taken_apart(ops, w_dtype, m, h, n2, k, swiglu):
     """Two products with an RMSNorm of the residual stream between them: the first adds into the
     stream and leaves bf16(h * weight) with partial sums of squares, the second finishes the norm
