@@ -373,6 +373,42 @@ def test_small_pool_makes_requests_wait_and_reuses_pages(folders):
     assert 2 <= most_running <= 3 and waited_for_pages and engine.cache_manager.used_pages() == 0
 
 
+@pytest.mark.parametrize("steps_per_launch", [1, 4])
+def test_many_requests_through_the_scheduler_equal_each_alone(steps_per_launch):
+    """Forty requests of random lengths, two in three greedy and the others with seeded top-k / top-p
+    sampling, arriving a few at a time into continuous batching with portions of at most 48 tokens, a
+    pool of 40 pages and up to eight running: in float32 every request's tokens are exactly those it
+    produces alone, and the pool is empty at the end."""
+    from llm_runtime_study_amd import Engine, SamplingConfig
+    from llm_runtime_study_amd.config import config_from_dict
+
+    cfg = config_from_dict(TINY_C)
+    rng = np.random.default_rng(5)
+    requests = []
+    for i in range(40):
+        prompt = rng.integers(0, cfg.vocab_size, int(rng.integers(1, 120))).tolist()
+        sampling = SamplingConfig() if i % 3 else SamplingConfig(temperature=0.8, top_k=20, top_p=0.9, seed=i)
+        requests.append((prompt, int(rng.integers(1, 40)), sampling))
+    alone = Engine.from_config(cfg, seed=1, init="scaled", dtype="float32", max_seq_len=256, max_batch_size=1, decode_steps_per_launch=1)
+    want = [alone.generate_tokens([p], max_new_tokens=n, sampling=s, ignore_eos=True)[0] for p, n, s in requests]
+    engine = Engine.from_config(cfg, seed=1, init="scaled", dtype="float32", max_seq_len=256, max_batch_size=8,
+                                max_num_batched_tokens=48, num_pages=40, decode_steps_per_launch=steps_per_launch)
+    scheduler = engine.create_scheduler(ignore_eos=True)
+    got, pending = {}, list(requests)
+    with torch.cuda.device(engine.device), torch.cuda.stream(engine.stream):
+        while pending or scheduler.has_unfinished:
+            for _ in range(int(rng.integers(0, 3))):
+                if pending:
+                    prompt, n, sampling = pending.pop(0)
+                    got[scheduler.add_request(prompt, max_new_tokens=n, sampling=sampling)] = []
+            if scheduler.has_unfinished:
+                for index, event in scheduler.step():
+                    got[index].append(event.token_id)
+                engine.cache_manager.check_invariants()
+    assert [got[i] for i in range(len(requests))] == want
+    assert engine.cache_manager.used_pages() == 0
+
+
 def test_command_line_on_the_gpu(folders):
     folder, cfg, weights = folders["a"]
     expected = plain_greedy(cfg, weights, [5, 6, 7], 4, [cfg["eos_token_id"]])
