@@ -51,6 +51,7 @@ class Engine:
         self.load_seconds = load_seconds
         self.quantization = "dense"
         self.stream = torch.cuda.Stream(device)
+        self._reload = None        # makes the model again in another dtype: set by from_model_dir / from_config
         self._runner: ModelRunner | None = None
         self._sampler = Sampler(device)
 
@@ -68,6 +69,7 @@ class Engine:
         engine = cls(config, model, device=selected_device, dtype=selected_dtype, max_seq_len=max_seq_len,
                      max_batch_size=max_batch_size, cache_backend=cache_backend, use_cuda_graph=use_cuda_graph,
                      tokenizer=tokenizer, **options)
+        engine._reload = lambda dtype: load_model(model_dir, dtype, selected_device, config)[1]
         engine.synchronize()
         engine.load_seconds = time.perf_counter() - started
         return engine
@@ -79,6 +81,7 @@ class Engine:
         selected_device, selected_dtype = resolve_device(device), resolve_dtype(dtype)
         model = random_model(config, seed, selected_dtype, selected_device, init)
         engine = cls(config, model, device=selected_device, dtype=selected_dtype, **options)
+        engine._reload = lambda dtype: random_model(config, seed, dtype, selected_device, init)
         engine.synchronize()
         engine.load_seconds = time.perf_counter() - started
         return engine
@@ -151,6 +154,43 @@ class Engine:
             if event.token_id is not None:
                 out[index].append(event.token_id)
         return out
+
+    def allocate_cache(self, capacity: int):
+        """A request's cache with `capacity` tokens promised to it (reference Engine.allocate_cache,
+        mini_llm/engine.py:298-299): for callers that drive the step function themselves."""
+        if capacity <= 0 or capacity > self.max_seq_len:
+            raise EngineError(f"cache capacity must be within 1..{self.max_seq_len}, got {capacity}")
+        manager = self.cache_manager
+        if not manager.can_admit(capacity):
+            raise EngineError(f"the KV cache cannot promise {capacity} more tokens")
+        return manager.admit(reserve_tokens=capacity)
+
+    def release_cache(self, cache) -> None:
+        """Give a cache from allocate_cache() back (mini_llm/engine.py:301-302); idempotent."""
+        self.cache_manager.release(cache)
+
+    def to(self, *, device=None, dtype=None) -> "Engine":
+        """The same engine in another precision (reference Engine.to, mini_llm/engine.py:304-346).  The
+        weights are made again from their source (the model folder, or the configuration and seed)
+        rather than converted in place, so float32 after bfloat16 has the checkpoint's precision;
+        cache pool, graphs and step function are rebuilt on next use.  The device cannot change."""
+        if device is not None and resolve_device(device) != self.device:
+            raise EngineError(f"this runtime has one device, {self.device}; it cannot move to {device}")
+        selected = self.dtype if dtype is None else resolve_dtype(dtype)
+        if selected == self.dtype:
+            return self
+        if self._runner is not None and self._runner.cache.active_requests:
+            raise EngineError("cannot move an engine while request caches are active")
+        if self._reload is None:
+            raise EngineError("this engine was not made by from_model_dir or from_config and cannot make its weights again")
+        if self._runner is not None:
+            self._runner.drop_graphs()
+            self._runner = None
+        self.model = None                  # the old weights go before the new ones come
+        self.model = self._reload(selected)
+        self.dtype = selected
+        self.synchronize()
+        return self
 
     def synchronize(self) -> None:
         torch.cuda.synchronize(self.device)

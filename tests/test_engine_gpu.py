@@ -409,6 +409,41 @@ def test_many_requests_through_the_scheduler_equal_each_alone(steps_per_launch):
     assert engine.cache_manager.used_pages() == 0
 
 
+def test_engine_changes_precision_and_hands_out_caches(folders):
+    """Engine.to(dtype=...) makes the weights again in the other precision (float32 after bfloat16 is
+    the checkpoint's precision, not a widened bfloat16) and refuses while a cache is out;
+    allocate_cache / release_cache are the reference's calls for driving the step function by hand."""
+    from llm_runtime_study_amd import Engine
+    from llm_runtime_study_amd.engine.step import StepEntry
+    from llm_runtime_study_amd.errors import EngineError
+
+    folder, cfg, weights = folders["b"]
+    prompt = [5, 9, 200, 31, 7, 7, 120]
+    expected = plain_greedy(cfg, weights, prompt, 8, [cfg["eos_token_id"]])
+    engine = Engine.from_model_dir(folder, dtype="bfloat16", max_seq_len=64, max_batch_size=2)
+    first = engine.generate_tokens([prompt], max_new_tokens=8)[0]
+    assert sum(a == b for a, b in zip(first, expected)) >= 6
+    assert engine.to(dtype="bfloat16") is engine
+    engine.to(dtype="float32")
+    assert engine.dtype == torch.float32 and engine.cache_manager.dtype == torch.float32
+    assert engine.generate_tokens([prompt], max_new_tokens=8)[0] == expected
+    cache = engine.allocate_cache(32)
+    with pytest.raises(EngineError, match="while request caches are active"):
+        engine.to(dtype="bfloat16")
+    with torch.cuda.stream(engine.stream):
+        logits = engine.runner.step([StepEntry(cache, prompt, [len(prompt) - 1])])
+        assert int(logits[0].argmax()) == expected[0]
+    engine.release_cache(cache)
+    engine.release_cache(cache)
+    assert engine.cache_manager.used_pages() == 0
+    with pytest.raises(EngineError, match="capacity"):
+        engine.allocate_cache(65)
+    with pytest.raises(EngineError, match="runs on the GPU only"):
+        engine.to(device="cpu")
+    engine.to(dtype="bfloat16")
+    assert engine.generate_tokens([prompt], max_new_tokens=8)[0] == first
+
+
 def test_command_line_on_the_gpu(folders):
     folder, cfg, weights = folders["a"]
     expected = plain_greedy(cfg, weights, [5, 6, 7], 4, [cfg["eos_token_id"]])
