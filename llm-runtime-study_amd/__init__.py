@@ -12,8 +12,8 @@ from .sampling.config import SamplingConfig
 from .text.chat import ChatMessage
 
 __all__ = ["ChatMessage", "CheckpointError", "CheckpointValidationError", "ConfigError", "Engine", "EngineError",
-           "GenerationError", "GenerationEvent", "KVCacheError", "KernelError", "SamplingConfig", "SamplingError",
-           "TokenizerError"]
+           "GenerationError", "GenerationEvent", "KVCacheError", "KernelError", "Qwen3Config", "SamplingConfig",
+           "SamplingError", "TokenizerError", "load_config"]
 
 
 def __getattr__(name):
@@ -24,4 +24,7 @@ def __getattr__(name):
     if name == "GenerationEvent":
         from .engine.scheduler import GenerationEvent
         return GenerationEvent
+    if name in ("Qwen3Config", "load_config"):       # as the reference's package exports them (mini_llm/__init__.py)
+        from . import config
+        return getattr(config, name)
     raise AttributeError(name)
