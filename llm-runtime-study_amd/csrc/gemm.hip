@@ -68,6 +68,8 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(void* __restrict__ out,
   }
 }
 
+__device__ __forceinline__ float silu(float g) { return g / (1.0f + __expf(-g)); }
+
 // ------------------------------------------------------- bf16 MFMA kernel
 // 128x128 output tile per workgroup of 4 waves (2x2), each wave 64x64 as 2x2 MFMA
 // 32x32x16 tiles.  K is walked in slices of 32 through LDS.  Needs K % 8 == 0 so that
@@ -154,6 +156,146 @@ __global__ __launch_bounds__(256) void gemm_bf16_mfma_kernel(void* __restrict__ 
     }
 }
 
+// ------------------------------------------------- bf16 MFMA kernel for many rows
+// 128 tokens x 256 weight rows per workgroup of four waves (2 x 2: a wave owns 64 tokens x 128 weight
+// rows as 4 x 8 tiles of the 16x16x32 product), K walked in slices of BK.  Both operands pass through
+// LDS (two buffers, one barrier a slice); a slice is asked from memory three slices before it is
+// multiplied and waits in registers meanwhile (two register sets in turn), and with slices of 32 two
+// workgroups share a compute unit, so a trip to memory has several slices' worth of matrix
+// instructions to hide behind.  Every fragment a wave reads from LDS feeds four or eight matrix
+// instructions.  Workgroups are numbered so that the 32 that share an XCD (and its L2) cover 4 x 8
+// tiles.  Needs K % BK == 0, 16-byte aligned rows, no bias and matrices of fewer than 2^31 elements
+// (the 128 x 128 kernel above takes what this one does not).
+// Accumulator layout: weight row 4 * (lane / 16) + i, token lane % 16, i.e. four consecutive output
+// columns of one token per lane.
+constexpr int WIDE_BK = 32;   // measured on MI355X at 2,048 rows: slices of 32 (two workgroups a compute unit) 0.66-0.88 PFLOP/s, of 64 (one) 0.53-0.74
+template <bool SWIGLU, int MODE, int BK>
+__global__ __launch_bounds__(256, BK == 32 ? 2 : 1) void gemm_bf16_wide_kernel(void* __restrict__ out, const bf16* __restrict__ x,
+                                                             const bf16* __restrict__ w,
+                                                             int m, int n, int k, int lda, int ldc, int tiles_m, int tiles_n) {
+  constexpr int BM = 128, BN = 256, LD = BK == 32 ? 32 : BK + 8;
+  constexpr int CH = BK / 8;                                 // 16-byte pieces of one row of a slice
+  constexpr int XL = BM * CH / 256, WL = BN * CH / 256;      // pieces of a slice per thread
+  constexpr int RS = 256 / CH;                               // rows between two pieces of one thread
+  __shared__ __attribute__((aligned(16))) bf16 xs[2][BM * LD];
+  __shared__ __attribute__((aligned(16))) bf16 ws[2][BN * LD];
+  const int tid = threadIdx.x, lane = tid % WAVE, wave = tid / WAVE;
+  const int r = lane & 15, g = lane >> 4;
+  int id = blockIdx.x;
+  const int tiles = tiles_m * tiles_n;
+  if (tiles % 8 == 0) id = (id % 8) * (tiles / 8) + id / 8;        // consecutive workgroups go to different XCDs
+  const int band = id / (4 * tiles_n), within = id % (4 * tiles_n);
+  const int band_rows = tiles_m - band * 4 < 4 ? tiles_m - band * 4 : 4;
+  const int m0 = (band * 4 + within % band_rows) * BM, n0 = (within / band_rows) * BN;
+  const int wm = (wave >> 1) * 64, wn = (wave & 1) * 128;           // this wave's corner inside the tile
+  // piece i of a slice for this thread: row tid / CH + RS * i, k chunk tid % CH (CH lanes read one row's
+  // bytes of the slice).  Rows past the matrix are read from its last row (and never written), slices
+  // past K are read from the last slice (and not multiplied): no load in the loop is conditional.
+  const int prow = tid / CH, pchunk = (tid % CH) * 8;
+  int xoff[XL], woff[WL];
+#pragma unroll
+  for (int i = 0; i < XL; ++i) xoff[i] = (m0 + prow + RS * i < m ? m0 + prow + RS * i : m - 1) * lda + pchunk;
+#pragma unroll
+  for (int i = 0; i < WL; ++i) woff[i] = (n0 + prow + RS * i < n ? n0 + prow + RS * i : n - 1) * k + pchunk;
+  floatx4 acc[8][4];
+#pragma unroll
+  for (int it = 0; it < 8; ++it)
+#pragma unroll
+    for (int jt = 0; jt < 4; ++jt) acc[it][jt] = floatx4{0.f, 0.f, 0.f, 0.f};
+  const int steps = (k + BK - 1) / BK;
+  auto fetch = [&](int kt, bf16x8 (&xr)[XL], bf16x8 (&wr)[WL]) {
+    const int at = (kt < steps ? kt : steps - 1) * BK;
+#pragma unroll
+    for (int i = 0; i < XL; ++i) xr[i] = *(const bf16x8*)(x + xoff[i] + at);
+#pragma unroll
+    for (int i = 0; i < WL; ++i) wr[i] = *(const bf16x8*)(w + woff[i] + at);
+  };
+  // Where chunk `chunk` (8 k) of tile row `row` lies in a buffer.  Slices of 64: rows 144 bytes apart.
+  // Slices of 32: rows are 64 bytes, half a line of banks, packed without padding; rows swap places in
+  // pairs in the upper half of every 16 and chunks are turned round by the row number, so that the
+  // rows 0..7, 8..15, the even and the odd rows of a fragment each touch every bank once.
+  auto cell = [&](int row, int chunk) -> int {
+    if constexpr (BK == 32) return ((row ^ ((row >> 3) & 1)) * 4 + (chunk ^ ((row >> 1) & 3))) * 8;
+    else return row * LD + chunk * 8;
+  };
+  auto stash = [&](int buffer, const bf16x8 (&xr)[XL], const bf16x8 (&wr)[WL]) {
+#pragma unroll
+    for (int i = 0; i < XL; ++i) *(bf16x8*)(xs[buffer] + cell(prow + RS * i, tid % CH)) = xr[i];
+#pragma unroll
+    for (int i = 0; i < WL; ++i) *(bf16x8*)(ws[buffer] + cell(prow + RS * i, tid % CH)) = wr[i];
+  };
+  auto multiply = [&](int buffer) {
+#pragma unroll
+    for (int h = 0; h < BK / 32; ++h) {
+      bf16x8 xf[4];
+#pragma unroll
+      for (int jt = 0; jt < 4; ++jt) xf[jt] = *(const bf16x8*)(xs[buffer] + cell(wm + jt * 16 + r, h * 4 + g));
+#pragma unroll
+      for (int it = 0; it < 8; ++it) {
+        const bf16x8 wf = *(const bf16x8*)(ws[buffer] + cell(wn + it * 16 + r, h * 4 + g));
+#pragma unroll
+        for (int jt = 0; jt < 4; ++jt) acc[it][jt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf, xf[jt], acc[it][jt], 0, 0, 0);
+      }
+    }
+  };
+  int m0_opaque = m0;
+  bf16x8 xa[XL], wa[WL], xb[XL], wb[WL];
+  fetch(0, xa, wa);
+  fetch(1, xb, wb);
+  stash(0, xa, wa);
+  fetch(2, xa, wa);
+  __syncthreads();
+  for (int kt = 0; kt < steps; kt += 2) {
+    multiply(0);                       // slice kt; the registers hold kt + 1 (b) and kt + 2 (a)
+    if (kt + 1 >= steps) break;
+    stash(1, xb, wb);
+    fetch(kt + 3, xb, wb);
+    __syncthreads();
+    multiply(1);                       // slice kt + 1; the registers hold kt + 2 (a) and kt + 3 (b)
+    if (kt + 2 < steps) {
+      stash(0, xa, wa);
+      fetch(kt + 4, xa, wa);
+    }
+    __syncthreads();
+  }
+  // nothing of the epilogue's addresses may be worked out (and kept in registers) before the loop above ends
+  asm volatile("" : "+s"(ldc), "+s"(m0_opaque));
+  // jt outside: one token row's address is worked out once and its 8 pieces of 4 columns follow 16 apart;
+  // the fence after each piece keeps the compiler from working out all 32 addresses (64 registers) first
+#pragma unroll
+  for (int jt = 0; jt < 4; ++jt) {
+    const int token = m0_opaque + wm + jt * 16 + r;
+    const int64_t row_at = (int64_t)token * ldc;
+#pragma unroll
+    for (int it = 0; it < 8; ++it) {
+      const int tile0 = n0 + wn + it * 16, row0 = tile0 + 4 * g;     // this lane's four weight rows = output columns
+      if (SWIGLU) {
+        // a tile's 16 weight rows are 8 gate rows and the 8 up rows of the same features: the up
+        // values of a lane's gate rows are held by the lane 32 further on
+        floatx4 up;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) up[i] = __shfl(acc[it][jt][i], (lane + 32) % WAVE, WAVE);
+        if (g < 2 && token < m && tile0 + 15 < n) {
+          const floatx4 gate = acc[it][jt];
+          const bf16x4 y = {(bf16)(silu(gate[0]) * up[0]), (bf16)(silu(gate[1]) * up[1]), (bf16)(silu(gate[2]) * up[2]), (bf16)(silu(gate[3]) * up[3])};
+          *(bf16x4*)((bf16*)out + row_at + tile0 / 2 + 4 * g) = y;
+        }
+      } else if (token < m && row0 < n) {
+        floatx4 v = acc[it][jt];
+        // An identity move across lanes: with a convergent operation on the accumulators here the
+        // compiler keeps the loop above free of spills (222 registers); without one it spills about 300.
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          v[i] = __shfl(v[i], lane, WAVE);
+        if constexpr (MODE == OUT_STORE) *(bf16x4*)((bf16*)out + row_at + row0) = bf16x4{(bf16)v[0], (bf16)v[1], (bf16)v[2], (bf16)v[3]};
+        else if constexpr (MODE == OUT_STORE_F32) *(floatx4*)((float*)out + row_at + row0) = v;
+        else *(floatx4*)((float*)out + row_at + row0) = *(const floatx4*)((const float*)out + row_at + row0) + v;
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  }
+}
+
 // ------------------------------------------------- bf16 kernel for few rows
 // Decode-sized products (M <= 64): the weight matrix is streamed exactly once and the time
 // is the time to read it.  One workgroup owns 16 weight rows; its waves split K between them
@@ -195,7 +337,6 @@ struct NormChain {
   int next_weight_is_f32;
 };
 
-__device__ __forceinline__ float silu(float g) { return g / (1.0f + __expf(-g)); }
 
 template <int MT, int RT, int WAVES, int UNROLL, bool NORM, bool SWIGLU, bool PARTIAL = false>
 __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_skinny_kernel(
@@ -646,6 +787,15 @@ LRS_API int lrs_gemm(void* out, int mode, const void* a, const void* w, const vo
       else if (normed) launch_skinny_m<true, false>(out, mode, ap, norm, wp, bp, m, n, k, lda, ldc, s);
       else if (swiglu) launch_skinny_m<false, true>(out, mode, ap, norm, wp, bp, m, n, k, lda, ldc, s);
       else launch_skinny_m<false, false>(out, mode, ap, norm, wp, bp, m, n, k, lda, ldc, s);
+    } else if (aligned && k % WIDE_BK == 0 && n % 4 == 0 && ldc % 4 == 0 && (uintptr_t)out % 16 == 0 && !bias &&
+               (int64_t)m * lda < (1ll << 31) && (int64_t)n * k < (1ll << 31)) {
+      const int tiles_m = (m + 127) / 128, tiles_n = (n + 255) / 256;
+#define WIDE(SW, MODE) gemm_bf16_wide_kernel<SW, MODE, WIDE_BK><<<tiles_m * tiles_n, 256, 0, s>>>(out, (const bf16*)a, (const bf16*)w, m, n, k, lda, ldc, tiles_m, tiles_n)
+      if (swiglu) WIDE(true, OUT_STORE);
+      else if (mode == OUT_STORE) WIDE(false, OUT_STORE);
+      else if (mode == OUT_STORE_F32) WIDE(false, OUT_STORE_F32);
+      else WIDE(false, OUT_ADD_F32);
+#undef WIDE
     } else if (aligned) {
       dim3 grid((n + 127) / 128, (m + 127) / 128);
       if (swiglu)

@@ -213,6 +213,7 @@ def test_add_into(ops, dtype):
     (1, 64, 64), (5, 331, 96), (17, 160, 96), (64, 256, 160), (130, 200, 264), (3, 129, 40),
     (2, 70, 36), (1, 1000, 4096), (257, 384, 512),
     (8, 5120, 160), (3, 4112, 72), (16, 12290, 64),      # few rows, widths that are dealt out unevenly by 16-row tiles
+    (300, 516, 96), (1100, 4096, 1024),                  # many rows, K a multiple of 32: the kernel of 128 x 256 tiles, ragged edges and 8 XCDs' numbering
 ])
 @pytest.mark.parametrize("mode", ["store", "store_f32", "add"])
 def test_gemm(ops, dtype, m, n, k, mode):
@@ -262,7 +263,8 @@ def test_gemm_with_fused_rmsnorm_input(ops, w_dtype, m, n, k, all_rows_in_own_ke
     close_in_norm(out, two.cpu(), 5e-3)
 
 
-@pytest.mark.parametrize("m,inter,k", [(1, 128, 64), (9, 160, 96), (64, 12288, 4096), (65, 160, 96), (300, 136, 264)])
+@pytest.mark.parametrize("m,inter,k", [(1, 128, 64), (9, 160, 96), (64, 12288, 4096), (65, 160, 96), (300, 136, 264),
+                                       (300, 392, 160), (2048, 1024, 512)])      # K a multiple of 32 and more than 64 rows: the kernel of 128 x 256 tiles
 def test_gemm_with_swiglu_epilogue(ops, m, inter, k, all_rows_in_own_kernel):
     """Gate and up rows interleaved in groups of 8; the product writes silu(gate) * up."""
     g = torch.Generator().manual_seed(15)
