@@ -158,27 +158,29 @@ __global__ __launch_bounds__(256) void gemm_bf16_mfma_kernel(void* __restrict__ 
 
 // ------------------------------------------------- bf16 MFMA kernel for many rows
 // 128 tokens x 256 weight rows per workgroup of four waves (2 x 2: a wave owns 64 tokens x 128 weight
-// rows as 4 x 8 tiles of the 16x16x32 product), K walked in slices of BK.  Both operands pass through
+// rows as 4 x 8 tiles of the 16x16x32 product), K walked in slices of 32.  Both operands pass through
 // LDS (two buffers, one barrier a slice); a slice is asked from memory three slices before it is
-// multiplied and waits in registers meanwhile (two register sets in turn), and with slices of 32 two
+// multiplied and waits in registers meanwhile (two register sets in turn), and two
 // workgroups share a compute unit, so a trip to memory has several slices' worth of matrix
 // instructions to hide behind.  Every fragment a wave reads from LDS feeds four or eight matrix
 // instructions.  Workgroups are numbered so that the 32 that share an XCD (and its L2) cover 4 x 8
-// tiles.  Needs K % BK == 0, 16-byte aligned rows, no bias and matrices of fewer than 2^31 elements
+// tiles.  Needs K % 32 == 0, 16-byte aligned rows, no bias and matrices of fewer than 2^31 elements
 // (the 128 x 128 kernel above takes what this one does not).
+// What bounds it (measured at 2,048 x 24,576 x 4,096, 469 us): without the loads from memory inside the
+// loop 348 us, without the writes into LDS as well 252 us; the LDS moves about 64 bytes a cycle and unit
+// and a slice needs 72 KB of it per workgroup (48 KB of fragment reads, 24 KB of writes).  Weights
+// straight from memory into registers (only activations through LDS, 40 KB) were slower: 513 us.
 // Accumulator layout: weight row 4 * (lane / 16) + i, token lane % 16, i.e. four consecutive output
 // columns of one token per lane.
-constexpr int WIDE_BK = 32;   // measured on MI355X at 2,048 rows: slices of 32 (two workgroups a compute unit) 0.66-0.88 PFLOP/s, of 64 (one) 0.53-0.74
-template <bool SWIGLU, int MODE, int BK>
-__global__ __launch_bounds__(256, BK == 32 ? 2 : 1) void gemm_bf16_wide_kernel(void* __restrict__ out, const bf16* __restrict__ x,
-                                                             const bf16* __restrict__ w,
-                                                             int m, int n, int k, int lda, int ldc, int tiles_m, int tiles_n) {
-  constexpr int BM = 128, BN = 256, LD = BK == 32 ? 32 : BK + 8;
-  constexpr int CH = BK / 8;                                 // 16-byte pieces of one row of a slice
-  constexpr int XL = BM * CH / 256, WL = BN * CH / 256;      // pieces of a slice per thread
-  constexpr int RS = 256 / CH;                               // rows between two pieces of one thread
-  __shared__ __attribute__((aligned(16))) bf16 xs[2][BM * LD];
-  __shared__ __attribute__((aligned(16))) bf16 ws[2][BN * LD];
+constexpr int WIDE_BK = 32;   // measured on MI355X at 2,048 rows: slices of 32 (two workgroups a compute unit) beat slices of 64 (one) by a fifth
+template <bool SWIGLU, int MODE>
+__global__ __launch_bounds__(256, 2) void gemm_bf16_wide_kernel(void* __restrict__ out, const bf16* __restrict__ x,
+                                                                const bf16* __restrict__ w, int m, int n, int k, int lda,
+                                                                int ldc, int tiles_m, int tiles_n) {
+  constexpr int BM = 128, BN = 256, BK = WIDE_BK;
+  constexpr int XL = BM * 4 / 256, WL = BN * 4 / 256;        // 16-byte pieces of a slice per thread: 2 of x, 4 of w
+  __shared__ __attribute__((aligned(16))) bf16 xs[2][BM * BK];
+  __shared__ __attribute__((aligned(16))) bf16 ws[2][BN * BK];
   const int tid = threadIdx.x, lane = tid % WAVE, wave = tid / WAVE;
   const int r = lane & 15, g = lane >> 4;
   int id = blockIdx.x;
@@ -188,21 +190,29 @@ __global__ __launch_bounds__(256, BK == 32 ? 2 : 1) void gemm_bf16_wide_kernel(v
   const int band_rows = tiles_m - band * 4 < 4 ? tiles_m - band * 4 : 4;
   const int m0 = (band * 4 + within % band_rows) * BM, n0 = (within / band_rows) * BN;
   const int wm = (wave >> 1) * 64, wn = (wave & 1) * 128;           // this wave's corner inside the tile
-  // piece i of a slice for this thread: row tid / CH + RS * i, k chunk tid % CH (CH lanes read one row's
+  // piece i of a slice for this thread: row tid / 4 + 64 * i, k chunk tid % 4 (4 lanes read one row's 64
   // bytes of the slice).  Rows past the matrix are read from its last row (and never written), slices
   // past K are read from the last slice (and not multiplied): no load in the loop is conditional.
-  const int prow = tid / CH, pchunk = (tid % CH) * 8;
+  const int prow = tid / 4;
   int xoff[XL], woff[WL];
 #pragma unroll
-  for (int i = 0; i < XL; ++i) xoff[i] = (m0 + prow + RS * i < m ? m0 + prow + RS * i : m - 1) * lda + pchunk;
+  for (int i = 0; i < XL; ++i) xoff[i] = (m0 + prow + 64 * i < m ? m0 + prow + 64 * i : m - 1) * lda + (tid % 4) * 8;
 #pragma unroll
-  for (int i = 0; i < WL; ++i) woff[i] = (n0 + prow + RS * i < n ? n0 + prow + RS * i : n - 1) * k + pchunk;
+  for (int i = 0; i < WL; ++i) woff[i] = (n0 + prow + 64 * i < n ? n0 + prow + 64 * i : n - 1) * k + (tid % 4) * 8;
+  // Where chunk c (8 k) of tile row q lies in a buffer: rows are 64 bytes, half a line of banks, packed
+  // without padding; rows swap places in pairs in the upper half of every 16 and chunks are turned
+  // round by the row number, so that the rows 0..7, 8..15, the even and the odd rows of a fragment
+  // each touch every bank once (measured: no bank conflicts; with rows 80 bytes apart every second
+  // LDS cycle was one).  Element ((q ^ (q >> 3 & 1)) * 4 + (c ^ (q >> 1 & 3))) * 8; only the low four
+  // bits of q enter the swaps, so a tile row 16 * j + q lies 16 * j * 32 elements further on.
+  const int spot = ((prow ^ ((prow >> 3) & 1)) * 4 + ((tid % 4) ^ ((prow >> 1) & 3))) * 8;   // where this thread's pieces go
+  const int frag = ((r ^ ((r >> 3) & 1)) * 4 + (g ^ ((r >> 1) & 3))) * 8;                    // where its fragments come from
   floatx4 acc[8][4];
 #pragma unroll
   for (int it = 0; it < 8; ++it)
 #pragma unroll
     for (int jt = 0; jt < 4; ++jt) acc[it][jt] = floatx4{0.f, 0.f, 0.f, 0.f};
-  const int steps = (k + BK - 1) / BK;
+  const int steps = k / BK;
   auto fetch = [&](int kt, bf16x8 (&xr)[XL], bf16x8 (&wr)[WL]) {
     const int at = (kt < steps ? kt : steps - 1) * BK;
 #pragma unroll
@@ -210,34 +220,26 @@ __global__ __launch_bounds__(256, BK == 32 ? 2 : 1) void gemm_bf16_wide_kernel(v
 #pragma unroll
     for (int i = 0; i < WL; ++i) wr[i] = *(const bf16x8*)(w + woff[i] + at);
   };
-  // Where chunk `chunk` (8 k) of tile row `row` lies in a buffer.  Slices of 64: rows 144 bytes apart.
-  // Slices of 32: rows are 64 bytes, half a line of banks, packed without padding; rows swap places in
-  // pairs in the upper half of every 16 and chunks are turned round by the row number, so that the
-  // rows 0..7, 8..15, the even and the odd rows of a fragment each touch every bank once.
-  auto cell = [&](int row, int chunk) -> int {
-    if constexpr (BK == 32) return ((row ^ ((row >> 3) & 1)) * 4 + (chunk ^ ((row >> 1) & 3))) * 8;
-    else return row * LD + chunk * 8;
-  };
   auto stash = [&](int buffer, const bf16x8 (&xr)[XL], const bf16x8 (&wr)[WL]) {
 #pragma unroll
-    for (int i = 0; i < XL; ++i) *(bf16x8*)(xs[buffer] + cell(prow + RS * i, tid % CH)) = xr[i];
+    for (int i = 0; i < XL; ++i) *(bf16x8*)(xs[buffer] + spot + 64 * i * BK) = xr[i];
 #pragma unroll
-    for (int i = 0; i < WL; ++i) *(bf16x8*)(ws[buffer] + cell(prow + RS * i, tid % CH)) = wr[i];
+    for (int i = 0; i < WL; ++i) *(bf16x8*)(ws[buffer] + spot + 64 * i * BK) = wr[i];
   };
   auto multiply = [&](int buffer) {
+    bf16x8 xf[4];
 #pragma unroll
-    for (int h = 0; h < BK / 32; ++h) {
-      bf16x8 xf[4];
+    for (int jt = 0; jt < 4; ++jt) xf[jt] = *(const bf16x8*)(xs[buffer] + frag + (wm + jt * 16) * BK);
 #pragma unroll
-      for (int jt = 0; jt < 4; ++jt) xf[jt] = *(const bf16x8*)(xs[buffer] + cell(wm + jt * 16 + r, h * 4 + g));
+    for (int it = 0; it < 8; ++it) {
+      const bf16x8 wf = *(const bf16x8*)(ws[buffer] + frag + (wn + it * 16) * BK);
 #pragma unroll
-      for (int it = 0; it < 8; ++it) {
-        const bf16x8 wf = *(const bf16x8*)(ws[buffer] + cell(wn + it * 16 + r, h * 4 + g));
-#pragma unroll
-        for (int jt = 0; jt < 4; ++jt) acc[it][jt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf, xf[jt], acc[it][jt], 0, 0, 0);
-      }
+      for (int jt = 0; jt < 4; ++jt) acc[it][jt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf, xf[jt], acc[it][jt], 0, 0, 0);
     }
   };
+  // Slice kt is multiplied from buffer kt % 2 while slice kt + 1 goes from registers into the other
+  // buffer and slice kt + 3 is asked for from memory (two register sets in turn): the writes and the
+  // requests are issued before the slice's matrix instructions and run beside them.
   int m0_opaque = m0;
   bf16x8 xa[XL], wa[WL], xb[XL], wb[WL];
   fetch(0, xa, wa);
@@ -246,16 +248,14 @@ __global__ __launch_bounds__(256, BK == 32 ? 2 : 1) void gemm_bf16_wide_kernel(v
   fetch(2, xa, wa);
   __syncthreads();
   for (int kt = 0; kt < steps; kt += 2) {
-    multiply(0);                       // slice kt; the registers hold kt + 1 (b) and kt + 2 (a)
-    if (kt + 1 >= steps) break;
-    stash(1, xb, wb);
+    stash(1, xb, wb);                  // slice kt + 1
     fetch(kt + 3, xb, wb);
+    multiply(0);                       // slice kt
     __syncthreads();
-    multiply(1);                       // slice kt + 1; the registers hold kt + 2 (a) and kt + 3 (b)
-    if (kt + 2 < steps) {
-      stash(0, xa, wa);
-      fetch(kt + 4, xa, wa);
-    }
+    if (kt + 1 >= steps) break;
+    stash(0, xa, wa);                  // slice kt + 2
+    fetch(kt + 4, xa, wa);
+    multiply(1);                       // slice kt + 1
     __syncthreads();
   }
   // nothing of the epilogue's addresses may be worked out (and kept in registers) before the loop above ends
@@ -790,7 +790,7 @@ LRS_API int lrs_gemm(void* out, int mode, const void* a, const void* w, const vo
     } else if (aligned && k % WIDE_BK == 0 && n % 4 == 0 && ldc % 4 == 0 && (uintptr_t)out % 16 == 0 && !bias &&
                (int64_t)m * lda < (1ll << 31) && (int64_t)n * k < (1ll << 31)) {
       const int tiles_m = (m + 127) / 128, tiles_n = (n + 255) / 256;
-#define WIDE(SW, MODE) gemm_bf16_wide_kernel<SW, MODE, WIDE_BK><<<tiles_m * tiles_n, 256, 0, s>>>(out, (const bf16*)a, (const bf16*)w, m, n, k, lda, ldc, tiles_m, tiles_n)
+#define WIDE(SW, MODE) gemm_bf16_wide_kernel<SW, MODE><<<tiles_m * tiles_n, 256, 0, s>>>(out, (const bf16*)a, (const bf16*)w, m, n, k, lda, ldc, tiles_m, tiles_n)
       if (swiglu) WIDE(true, OUT_STORE);
       else if (mode == OUT_STORE) WIDE(false, OUT_STORE);
       else if (mode == OUT_STORE_F32) WIDE(false, OUT_STORE_F32);
