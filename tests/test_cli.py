@@ -83,3 +83,33 @@ def test_interactive_reads_until_quit(monkeypatch):
     out = io.StringIO()
     code = cli.main(["--model", "m", "--interactive", "--no-metrics"], input_stream=io.StringIO("hello\n\n/quit\n"), output=out)
     assert code == 0 and "assistant> ok" in out.getvalue() and out.getvalue().count("you> ") == 3
+
+
+def test_bench_refuses_more_than_one_gpu_with_one_line_and_exit_code_2():
+    """The benchmark's contract: this engine runs on one GPU; asked for more it says so in one line."""
+    import subprocess
+    import sys
+    from pathlib import Path
+
+    root = Path(__file__).resolve().parents[1]
+    proc = subprocess.run([sys.executable, str(root / "bench.py"), "--gpus", "2"], capture_output=True, text=True, timeout=120)
+    assert proc.returncode == 2
+    lines = [line for line in proc.stdout.splitlines() if line.strip()]
+    assert len(lines) == 1 and "one GPU" in lines[0]
+
+
+def test_bench_counts_the_flops_and_the_lead_of_early_requests():
+    import bench
+
+    from llm_runtime_study_amd.config import config_from_dict
+
+    c = config_from_dict(bench.QWEN3_8B)
+    per_layer = bench.matrix_params_per_layer(c)
+    assert per_layer == (32 + 16) * 128 * 4096 + 4096 * 4096 + 3 * 4096 * 12288
+    linear = 2.0 * 2048 * per_layer * 36 + 2.0 * 4096 * 151936
+    attention = 4.0 * (2048 * 2049 / 2) * 32 * 128 * 36
+    assert bench.prefill_flops(c, 2048) == linear + attention
+    # eight prompts of 2,048 tokens read one a step: the first request is seven tokens ahead of the last
+    assert bench.decode_lead(8, 2048, 2048) == 7
+    assert bench.decode_lead(8, 32768, 2048) == 7 * 16 and bench.decode_lead(1, 5000, 2048) == 0
+    assert set(bench.SHAPES) == {"8b", "14b", "32b"} and bench.SHAPES["32b"]["num_hidden_layers"] == 64
