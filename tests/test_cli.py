@@ -113,3 +113,21 @@ def test_bench_counts_the_flops_and_the_lead_of_early_requests():
     assert bench.decode_lead(8, 2048, 2048) == 7
     assert bench.decode_lead(8, 32768, 2048) == 7 * 16 and bench.decode_lead(1, 5000, 2048) == 0
     assert set(bench.SHAPES) == {"8b", "14b", "32b"} and bench.SHAPES["32b"]["num_hidden_layers"] == 64
+
+
+def test_staggered_benchmark_percentiles_and_drawn_requests():
+    """Nearest-rank percentiles as the reference takes them (benchmarks/common.py:91-95); the same
+    seed draws the same requests, inside the asked ranges."""
+    import numpy as np
+
+    from llm_runtime_study_amd.benchmarks import staggered
+
+    assert staggered.percentile([4.0, 1.0, 3.0, 2.0], 0.5) == 2.0
+    assert staggered.percentile([4.0, 1.0, 3.0, 2.0], 0.95) == 4.0
+    assert staggered.percentile([7.0], 0.95) == 7.0
+    assert staggered.span("128,2048") == (128, 2048) and staggered.span("64") == (64, 64)
+    first = staggered.draw_requests(np.random.default_rng(3), 331, 20, (5, 9), (2, 4))
+    again = staggered.draw_requests(np.random.default_rng(3), 331, 20, (5, 9), (2, 4))
+    assert first == again
+    assert all(5 <= len(p) <= 9 and 2 <= n <= 4 and all(0 <= t < 331 for t in p) for p, n in first)
+    assert {len(p) for p, _ in first} == {5, 6, 7, 8, 9}

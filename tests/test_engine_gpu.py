@@ -459,3 +459,25 @@ def test_command_line_on_the_gpu(folders):
     proc = subprocess.run([sys.executable, "-m", "llm_runtime_study_amd", "--model", str(folder), "--prompt-ids", "1", "--max-seq-len", "4096"],
                           cwd=ROOT, capture_output=True, text=True, timeout=300)
     assert proc.returncode == 2 and "exceeds the model limit" in proc.stderr
+
+
+@pytest.mark.gpu
+def test_staggered_benchmark_runs_every_request_to_its_limit(capsys):
+    """The staggered serving run on one layer of the 8B shape: six requests, a pool for four, portions of
+    32 tokens; every request produces exactly its output limit and the report holds the reference's figures."""
+    import json
+
+    from llm_runtime_study_amd.benchmarks import staggered
+
+    code = staggered.main(["--shape", "8b", "--layers", "1", "--requests", "6", "--interval-ms", "1", "--prompt-tokens", "16,64",
+                           "--new-tokens", "4,8", "--max-batch-size", "4", "--step-tokens", "32", "--max-seq-len", "128",
+                           "--warmups", "0", "--seed", "1"])
+    assert code == 0
+    report = json.loads(capsys.readouterr().out.strip().splitlines()[-1])
+    import numpy as np
+    drawn = staggered.draw_requests(np.random.default_rng(1), 151936, 6, (16, 64), (4, 8))
+    assert report["generated_tokens"] == sum(n for _, n in drawn)
+    assert report["prompt_tokens"] == sum(len(p) for p, _ in drawn)
+    assert report["makespan_s"] > 0 and report["output_tok_s"] > 0
+    assert 0 < report["ttft_ms_p50"] <= report["ttft_ms_p95"] <= report["latency_ms_p95"]
+    assert report["latency_ms_p50"] <= report["latency_ms_p95"] <= 1000.0 * report["makespan_s"] + 1e-6
