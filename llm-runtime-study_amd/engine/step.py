@@ -259,7 +259,7 @@ class ModelRunner:
             cu[:cursor + 1] = count
             lens[:cursor] = lengths
             slots[:cursor] = ctx.host_slots
-            wanted = [r for r, entry in enumerate(entries) if len(entry.want)]
+            wanted = [r for r, entry in enumerate(entries) for _ in entry.want]   # a place asked twice is given twice
             n_rows = len(wanted)
             rows[:n_rows] = wanted
             ctx.host_q_lens = [1] * cursor
@@ -351,7 +351,9 @@ class ModelRunner:
          ctx.qblock_token0, ctx.qblock_count, ctx.counts, ctx._groups) = views
 
     def step(self, entries: Sequence[StepEntry]) -> torch.Tensor | None:
-        """Run one step; returns float32 logits [wanted, vocab] on the device, or None if none is wanted."""
+        """Run one step; returns float32 logits [wanted, vocab] on the device, or None if none is wanted.
+
+        The logits lie in a buffer that the next step writes again: read or copy them before it."""
         self.validate(entries)
         self._follow_construction()
         before = [entry.cache.length for entry in entries]
@@ -556,11 +558,11 @@ class ModelRunner:
             graph = self._graphs[key] = (handle, generation, logits)
         ops.graph_launch(graph[0])
         self.graph_replays += 1
-        wanted = [r for r, entry in enumerate(entries) if len(entry.want)]
+        wanted = [r for r, entry in enumerate(entries) for _ in entry.want]   # a place asked twice is given twice
         if not wanted:
             return None
         logits = graph[2]
-        return logits[:len(entries)] if len(wanted) == len(entries) else logits[wanted]
+        return logits[:len(entries)] if wanted == list(range(len(entries))) else logits[wanted]
 
     def drop_graphs(self) -> None:
         for handle, *_ in self._graphs.values():
