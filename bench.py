@@ -44,6 +44,7 @@ def parse_args():
     parser.add_argument("--no-points", action="store_true", help="skip the batch 1 and 64 decode points")
     parser.add_argument("--no-graph", action="store_true")
     parser.add_argument("--decode-steps-per-launch", type=int, default=4, help="greedy decode steps run from one graph launch (1: one step a launch)")
+    parser.add_argument("--library-mid-gemm", action="store_true", help="products of 17..64 rows through the vendor library instead of this package's kernel for them")
     parser.add_argument("--own-gemm", action="store_true", help="this package's kernel also for products of many rows (default: vendor library)")
     return parser.parse_args()
 
@@ -165,6 +166,9 @@ def main() -> int:
     engine = Engine.from_config(config, seed=0, dtype=args.dtype, max_seq_len=max_seq_len, max_batch_size=max_batch,
                                 max_num_batched_tokens=max(2048, args.prefill_tokens), use_cuda_graph=not args.no_graph, library_gemm=not args.own_gemm,
                                 decode_steps_per_launch=args.decode_steps_per_launch)
+    if args.library_mid_gemm:
+        from llm_runtime_study_amd.kernels import ops
+        ops.gemm_mid_tune(False)
     dtype_name = "bf16" if args.dtype == "bfloat16" else "fp32"
 
     prefill_times = measure_prefill(engine, args.prefill_tokens, repeats=3, seed=1)

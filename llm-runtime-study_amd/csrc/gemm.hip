@@ -617,6 +617,167 @@ __global__ void gemm_split_finish_kernel(void* __restrict__ out, int mode, const
   }
 }
 
+// ------------------------------------------------- bf16 kernel for 17..64 rows
+// Between the few-rows kernel (every wave reads its activations from L2 itself) and the many-rows
+// kernel (both operands tiled through LDS): the weights are still streamed exactly once, as the MFMA A
+// operand straight from memory into registers, but with several 16-token blocks the activations are
+// as many bytes as the weights of a workgroup, so the waves of a workgroup (each with 16 weight rows
+// of its own) share them through LDS.  K is walked in slices of 256: while a slice is multiplied,
+// the weights of the next two slices are on their way into registers and the activations of the
+// next slice lie in the other LDS buffer, stored there in MFMA B-fragment order (a fragment is 1 KB,
+// lane l at byte 16 l: reads and writes are conflict-free).  gridDim.y > 1 divides K between
+// workgroups; with split_sums given every workgroup leaves its sums there ([gridDim.y, m, n]) for a
+// kernel that adds them up (gemm_split_finish_kernel, or the residual add and norm that follow).  K % 256 == 0.
+template <int MT, int WAVES, bool SWIGLU>
+__global__ __launch_bounds__(WAVES * 64) void gemm_bf16_mid_kernel(
+    void* __restrict__ out, int mode, const bf16* __restrict__ x, const bf16* __restrict__ w,
+    int m, int n, int k, int lda, int ldc, float* __restrict__ split_sums) {
+  constexpr int STEPS = 8;                         // k steps of 32 in a slice
+  constexpr int FRAGS = STEPS * MT;                // activation fragments of a slice
+  constexpr int MINE = (FRAGS + WAVES - 1) / WAVES;  // of which a wave brings this many
+  __shared__ bf16x8 acts[2][STEPS][MT][WAVE];
+  const int tid = threadIdx.x, lane = tid % WAVE, wave = __builtin_amdgcn_readfirstlane(tid / WAVE);
+  const int r = lane & 15, g = lane >> 4;
+  const int row0 = blockIdx.x * (16 * WAVES) + wave * 16;
+  const bf16* wp = w + (int64_t)(row0 + r < n ? row0 + r : n - 1) * k + g * 8;
+  const int slices = k / 256;
+  const int per_split = (slices + gridDim.y - 1) / gridDim.y;
+  const int s0 = blockIdx.y * per_split;
+  const int count = (s0 + per_split < slices ? s0 + per_split : slices) - s0;
+  // Workgroups walk their slices from different starting points (round the ring): all of them read the
+  // same activations, and in step they would all ask the same cache lines at the same moment.  The order
+  // of a column's sum then depends on the column's workgroup alone.
+  const int turn = count > 0 ? (int)(blockIdx.x % (unsigned)count) : 0;
+  auto slice_at = [&](int c) -> int { const int v = c + turn; return s0 + (v >= count ? v - count : v); };
+  // Every load and every LDS write below is unconditional, so that the compiler can count the loads
+  // in flight instead of waiting for all of them at a branch: a token past m reads the last token's
+  // row (its columns of the result are never written), and where the fragments do not divide evenly
+  // between the waves the spare turns bring the last fragment once more (same data, same place).
+  const bf16* xp[MINE];
+  bf16x8* spot[MINE];
+#pragma unroll
+  for (int i = 0; i < MINE; ++i) {
+    const int f = wave + i * WAVES < FRAGS ? wave + i * WAVES : FRAGS - 1;
+    const int step = f / MT, t = f % MT, token = t * 16 + r < m ? t * 16 + r : m - 1;
+    xp[i] = x + (int64_t)token * lda + step * 32 + g * 8;
+    spot[i] = &acts[0][step][t][lane];
+  }
+  floatx4 acc[MT];
+#pragma unroll
+  for (int t = 0; t < MT; ++t) acc[t] = floatx4{0.f, 0.f, 0.f, 0.f};
+  bf16x8 wa[STEPS], wb[STEPS], sa[MINE], sb[MINE];
+  auto load_w = [&](int slice, bf16x8 (&a)[STEPS]) {
+#pragma unroll
+    for (int j = 0; j < STEPS; ++j) a[j] = *(const bf16x8*)(wp + (int64_t)slice * 256 + j * 32);
+  };
+  auto load_acts = [&](int slice, bf16x8 (&st)[MINE]) {
+#pragma unroll
+    for (int i = 0; i < MINE; ++i) st[i] = *(const bf16x8*)(xp[i] + (int64_t)slice * 256);
+  };
+  auto store_acts = [&](int buf, const bf16x8 (&st)[MINE]) {
+#pragma unroll
+    for (int i = 0; i < MINE; ++i) spot[i][buf * (STEPS * MT * WAVE)] = st[i];
+  };
+  // Multiplies the slice in LDS buffer `buf` by the weights in a[].  RELOAD: every a[j] is asked again,
+  // for slice `next`, as soon as its products are issued (the scheduling barriers keep the compiler
+  // from gathering these loads at the end, where they would leave the memory idle meanwhile).  The
+  // activation fragments of a step are read from LDS while the step before is multiplied.
+  const bf16x8* frag = &acts[0][0][0][lane];
+  auto compute = [&](int buf, bf16x8 (&a)[STEPS], auto reload, int next) {
+    constexpr bool RELOAD = decltype(reload)::value;
+    const bf16x8* from = frag + buf * (STEPS * MT * WAVE);
+    bf16x8 b[2][MT];
+#pragma unroll
+    for (int t = 0; t < MT; ++t) b[0][t] = from[t * WAVE];
+#pragma unroll
+    for (int j = 0; j < STEPS; ++j) {
+      if (j + 1 < STEPS) {
+#pragma unroll
+        for (int t = 0; t < MT; ++t) b[(j + 1) & 1][t] = from[((j + 1) * MT + t) * WAVE];
+      }
+#pragma unroll
+      for (int t = 0; t < MT; ++t) acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[j], b[j & 1][t], acc[t], 0, 0, 0);
+      if constexpr (RELOAD) {
+        a[j] = *(const bf16x8*)(wp + (int64_t)next * 256 + j * 32);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+  };
+  const std::true_type again;
+  const std::false_type last;
+  // While slice c is multiplied, the weights of slice c + 1 are in registers or on their way and those of
+  // slice c + 2 are asked for as the products of c are issued; the activations of slices c + 2 and c + 3
+  // are on their way into two sets of staging registers (they come from L2, but a wait for them once a
+  // slice would show), and those of slice c + 1 go from registers into the LDS buffer that slice c - 1
+  // has left.
+  if (count > 0) {
+    load_w(slice_at(0), wa);
+    load_acts(slice_at(0), sa);
+  }
+  if (count > 1) {
+    load_w(slice_at(1), wb);
+    load_acts(slice_at(1), sb);
+  }
+  if (count > 0) store_acts(0, sa);
+  if (count > 2) load_acts(slice_at(2), sa);
+  // slice c: after the barrier LDS buffer c & 1 holds it and nobody reads the other buffer any more
+  auto steady = [&](int c, bf16x8 (&a)[STEPS], bf16x8 (&st)[MINE]) {
+    __syncthreads();
+    store_acts((c & 1) ^ 1, st);                       // slice c + 1
+    load_acts(slice_at(c + 3), st);
+    compute(c & 1, a, again, slice_at(c + 2));
+  };
+  auto ending = [&](int c, bf16x8 (&a)[STEPS], bf16x8 (&st)[MINE]) {
+    __syncthreads();
+    if (c + 1 < count) store_acts((c & 1) ^ 1, st);
+    if (c + 3 < count) load_acts(slice_at(c + 3), st);
+    if (c + 2 < count) compute(c & 1, a, again, slice_at(c + 2));
+    else compute(c & 1, a, last, 0);
+  };
+  int c = 0;
+  for (; c + 4 < count; c += 2) {            // no branch inside: slices up to c + 4 exist
+    steady(c, wa, sb);
+    steady(c + 1, wb, sa);
+  }
+  for (; c < count; c += 2) {                // the last one to four slices
+    ending(c, wa, sb);
+    if (c + 1 >= count) break;
+    ending(c + 1, wb, sa);
+  }
+  // accumulator layout: token = t * 16 + lane % 16, weight rows row0 + 4 * (lane / 16) + 0..3
+  const int gn = row0 + 4 * g;
+  if (split_sums) {
+#pragma unroll
+    for (int t = 0; t < MT; ++t) {
+      const int token = t * 16 + r;
+      if (token < m && gn < n) *(floatx4*)(split_sums + ((int64_t)blockIdx.y * m + token) * n + gn) = acc[t];
+    }
+    return;
+  }
+#pragma unroll
+  for (int t = 0; t < MT; ++t) {
+    const int token = t * 16 + r;
+    if constexpr (SWIGLU) {
+      // the 16 rows of a wave are 8 gate rows and the 8 up rows of the same features: the up values
+      // of a lane's gate rows sit 32 lanes further on
+      floatx4 up;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) up[i] = __shfl(acc[t][i], (lane + 32) & 63, WAVE);
+      if (g < 2 && token < m && row0 < n) {
+        bf16x4 y;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) y[i] = (bf16)(silu(acc[t][i]) * up[i]);
+        *(bf16x4*)((bf16*)out + (int64_t)token * ldc + row0 / 2 + 4 * g) = y;
+      }
+    } else if (token < m && gn < n) {
+      const floatx4 v = acc[t];
+      if (mode == OUT_STORE) *(bf16x4*)((bf16*)out + (int64_t)token * ldc + gn) = bf16x4{(bf16)v[0], (bf16)v[1], (bf16)v[2], (bf16)v[3]};
+      else if (mode == OUT_STORE_F32) *(floatx4*)((float*)out + (int64_t)token * ldc + gn) = v;
+      else *(floatx4*)((float*)out + (int64_t)token * ldc + gn) = *(const floatx4*)((const float*)out + (int64_t)token * ldc + gn) + v;
+    }
+  }
+}
+
 // Row tiles per workgroup: more of them means each activation fragment read from L2 serves more
 // weight rows, which matters once there are several token blocks; fewer means more workgroups.
 template <int MT, int RT, bool NORM, bool SWIGLU>
@@ -660,6 +821,68 @@ constexpr size_t SPLIT_SUMS_BYTES = 64u << 20;
 static float* split_sums_buffer() {
   if (!g_split_sums && hipMalloc((void**)&g_split_sums, SPLIT_SUMS_BYTES) != hipSuccess) g_split_sums = nullptr;
   return g_split_sums;
+}
+
+// The kernel for 17..64 rows: which of its workgroup shapes and how many K splits.  0 = chosen here:
+// the shape and split that fill a whole multiple of the compute units best, then the fewest splits.
+static int g_mid_waves = 0, g_mid_splits = 0, g_mid_enabled = 1;
+LRS_API int lrs_gemm_mid_tune(int enabled, int waves, int splits) {
+  LRS_REQUIRE(waves == 0 || waves == 4 || waves == 6 || waves == 8, "gemm_mid_tune: 4, 6 or 8 waves (0: automatic), got %d", waves);
+  LRS_REQUIRE(splits >= 0 && splits <= 16, "gemm_mid_tune: 0..16 splits, got %d", splits);
+  g_mid_enabled = enabled != 0, g_mid_waves = waves, g_mid_splits = splits;
+  return 0;
+}
+LRS_API int lrs_gemm_mid_enabled() { return g_mid_enabled; }
+
+static void choose_mid_shape(int n, int k, int& waves, int& splits) {
+  const int units = lrs_compute_units() > 0 ? lrs_compute_units() : 256, slices = k / 256;
+  double best = -1.0;
+  const int shapes[3] = {4, 6, 8};
+  for (int wi = 0; wi < 3; ++wi) {
+    const int wv = shapes[wi];
+    if (g_mid_waves && wv != g_mid_waves) continue;
+    const int tiles = (n + 16 * wv - 1) / (16 * wv);
+    for (int sp = 1; sp <= 8; ++sp) {
+      if (g_mid_splits && sp != g_mid_splits) continue;
+      if (sp > 1 && slices / sp < 2) continue;                  // at least two slices a workgroup
+      const int groups = tiles * sp;
+      const int rounds = (groups + units - 1) / units;
+      // share of the chip at work, less a little for every split (its sums are written and read again)
+      const double score = (double)groups / (rounds * units) - 0.02 * (sp - 1) - 0.01 * (rounds - 1);
+      if (score > best + 1e-9) best = score, waves = wv, splits = sp;
+    }
+  }
+  if (best < 0) waves = g_mid_waves ? g_mid_waves : 4, splits = 1;
+}
+
+// keep_sums: the sums of the K splits (of the one split, if K is not divided) stay in the split buffer for
+// the caller's own finishing kernel; returns their number, or 0 if the buffer cannot hold them.
+template <int MT, bool SWIGLU>
+static int launch_mid_mt(void* out, int mode, const bf16* a, const bf16* w, int m, int n, int k, int lda, int ldc, hipStream_t s, bool keep_sums) {
+  int waves = 4, splits = 1;
+  choose_mid_shape(n, k, waves, splits);
+  float* sums = splits > 1 || keep_sums ? split_sums_buffer() : nullptr;
+  if ((splits > 1 || keep_sums) && (!sums || (size_t)splits * m * n * sizeof(float) > SPLIT_SUMS_BYTES)) {
+    if (keep_sums) return 0;
+    splits = 1, sums = nullptr;
+  }
+  const dim3 grid((n + 16 * waves - 1) / (16 * waves), splits);
+  if (waves == 4) gemm_bf16_mid_kernel<MT, 4, SWIGLU><<<grid, 4 * 64, 0, s>>>(out, mode, a, w, m, n, k, lda, ldc, sums);
+  else if (waves == 6) gemm_bf16_mid_kernel<MT, 6, SWIGLU><<<grid, 6 * 64, 0, s>>>(out, mode, a, w, m, n, k, lda, ldc, sums);
+  else gemm_bf16_mid_kernel<MT, 8, SWIGLU><<<grid, 8 * 64, 0, s>>>(out, mode, a, w, m, n, k, lda, ldc, sums);
+  if (splits > 1 && !keep_sums) {
+    const int64_t total = (int64_t)m * (SWIGLU ? n / 2 : n);
+    const int blocks = (int)((total + 255) / 256 < 1024 ? (total + 255) / 256 : 1024);
+    gemm_split_finish_kernel<SWIGLU><<<blocks, 256, 0, s>>>(out, mode, sums, nullptr, m, n, ldc, splits);
+  }
+  return splits;
+}
+
+template <bool SWIGLU>
+static int launch_mid(void* out, int mode, const bf16* a, const bf16* w, int m, int n, int k, int lda, int ldc, hipStream_t s, bool keep_sums = false) {
+  if (m <= 32) return launch_mid_mt<2, SWIGLU>(out, mode, a, w, m, n, k, lda, ldc, s, keep_sums);
+  if (m <= 48) return launch_mid_mt<3, SWIGLU>(out, mode, a, w, m, n, k, lda, ldc, s, keep_sums);
+  return launch_mid_mt<4, SWIGLU>(out, mode, a, w, m, n, k, lda, ldc, s, keep_sums);
 }
 
 template <int MT, bool NORM, bool SWIGLU>
@@ -752,6 +975,28 @@ LRS_API int lrs_gemm_norm_chain(void* out, int mode, const void* a, const void* 
   return lrs_check_launch("gemm_norm_chain");
 }
 
+// Defined beside the norm kernels: x [rows, hidden] += the sum over `splits` of sums[split, rows, hidden],
+// then out = RMSNorm(x) with `weight`.
+extern "C" int lrs_split_add_rmsnorm(void* out, int out_dtype, float* x, const float* sums, int splits, const void* weight,
+                                     int w_dtype, int n_rows, int hidden, float eps, void* stream);
+
+// A product of 17..64 rows that adds into the float32 residual stream, with the RMSNorm that follows:
+// residual [M, N] += a [M, K] w[N, K]^T, then normed [M, N] = RMSNorm(residual) with norm_weight and eps.
+// The sums of the product's K splits go straight into the kernel that adds and normalises: one launch
+// less and no rounding of the product to bf16 on the way.
+LRS_API int lrs_gemm_mid_add_rmsnorm(void* normed, int normed_dtype, float* residual, const void* a, const void* w,
+                                     const void* norm_weight, int norm_weight_dtype, int m, int n, int k, int lda,
+                                     float eps, void* stream) {
+  LRS_REQUIRE(m > 16 && m <= 64 && n > 0 && k > 0, "gemm_mid_add_rmsnorm: takes 17..64 rows, got m=%d n=%d k=%d", m, n, k);
+  LRS_REQUIRE(k % 256 == 0 && n % 16 == 0 && lda >= k && lda % 8 == 0 && ((uintptr_t)a % 16 == 0) && ((uintptr_t)w % 16 == 0) && ((uintptr_t)residual % 16 == 0),
+              "gemm_mid_add_rmsnorm: needs K %% 256 == 0, N %% 16 == 0 and 16-byte aligned rows (n=%d k=%d lda=%d)", n, k, lda);
+  LRS_REQUIRE(eps > 0.f, "gemm_mid_add_rmsnorm: eps must be positive");
+  const int splits = launch_mid<false>(nullptr, OUT_STORE, (const bf16*)a, (const bf16*)w, m, n, k, lda, n, (hipStream_t)stream, true);
+  LRS_REQUIRE(splits > 0, "gemm_mid_add_rmsnorm: the buffer for the sums of the K splits cannot hold %d x %d values", m, n);
+  if (int rc = lrs_check_launch("gemm_mid_add_rmsnorm")) return rc;
+  return lrs_split_add_rmsnorm(normed, normed_dtype, residual, split_sums_buffer(), splits, norm_weight, norm_weight_dtype, m, n, eps, stream);
+}
+
 // out [M, N] (row stride ldc) = a [M, K] (row stride lda) times w[N, K]^T.
 //   norm_weight != null: `a` is the float32 residual stream [*, K]; its rows (picked through
 //     `rows` if given) are RMS-normalised with norm_weight and eps on the way in.  bf16 weights,
@@ -783,7 +1028,10 @@ LRS_API int lrs_gemm(void* out, int mode, const void* a, const void* w, const vo
       const bf16 *wp = (const bf16*)w, *bp = (const bf16*)bias;
       const NormInput norm{(const float*)a, rows, norm_weight, norm_weight_dtype == LRS_F32, eps};
       const bf16* ap = normed ? nullptr : (const bf16*)a;
-      if (normed && swiglu) launch_skinny_m<true, true>(out, mode, ap, norm, wp, bp, m, n, k, lda, ldc, s);
+      if (m > 16 && !normed && !bias && g_mid_enabled && k % 256 == 0 && n % 16 == 0 && ldc % 4 == 0 && (uintptr_t)out % 16 == 0) {
+        if (swiglu) launch_mid<true>(out, mode, ap, wp, m, n, k, lda, ldc, s);
+        else launch_mid<false>(out, mode, ap, wp, m, n, k, lda, ldc, s);
+      } else if (normed && swiglu) launch_skinny_m<true, true>(out, mode, ap, norm, wp, bp, m, n, k, lda, ldc, s);
       else if (normed) launch_skinny_m<true, false>(out, mode, ap, norm, wp, bp, m, n, k, lda, ldc, s);
       else if (swiglu) launch_skinny_m<false, true>(out, mode, ap, norm, wp, bp, m, n, k, lda, ldc, s);
       else launch_skinny_m<false, false>(out, mode, ap, norm, wp, bp, m, n, k, lda, ldc, s);

@@ -381,7 +381,7 @@ class ModelRunner:
 
     # ------------------------------------------------- several decode steps, one launch
     MAX_DECODE_STEPS = 8
-    LIBRARY_GRAPH_ROWS = 64     # largest padded batch whose step (with library matrix products) is captured
+    LIBRARY_GRAPH_ROWS = 64     # largest padded batch whose bfloat16 step is captured
 
     def can_decode_steps(self, entries: Sequence[StepEntry]) -> bool:
         """Whether decode_steps() takes these entries: one token each, and a graph for their number."""
@@ -525,9 +525,10 @@ class ModelRunner:
         while bucket < len(entries):
             bucket *= 2
         bucket = min(bucket, self.max_requests)
-        # Up to the rows the few-rows kernels take, a graph holds this package's kernels only; larger
-        # batches (up to 64 rows) bring the vendor library's products into the capture.
-        most = max(ops.skinny_max_m(), self.LIBRARY_GRAPH_ROWS) if self.library_gemm and self.dtype == torch.bfloat16 else ops.skinny_max_m()
+        # Up to 48 rows a bfloat16 graph holds this package's kernels only (the few-rows kernels, then the
+        # kernel for 17..64 rows); a batch padded to 64 rows brings the vendor library's products into the
+        # capture when the runner may use them.
+        most = max(ops.skinny_max_m(), self.LIBRARY_GRAPH_ROWS) if self.dtype == torch.bfloat16 else ops.skinny_max_m()
         return bucket if bucket <= min(self.max_step_tokens, most) else 0
 
     def _step_graph(self, entries: Sequence[StepEntry], bucket: int) -> torch.Tensor | None:

@@ -99,6 +99,8 @@ def gemm(args) -> None:
     hidden, inter = args.hidden_size, args.intermediate_size
     qkv = (args.heads + 2 * args.kv_heads) * args.head_dim
     shapes = [("qkv", qkv, hidden), ("o", hidden, args.heads * args.head_dim), ("gate_up", 2 * inter, hidden), ("down", hidden, inter)]
+    if args.vocab_size:
+        shapes.append(("lm_head", args.vocab_size, hidden))
     before = ops.skinny_max_m()
     ops.set_skinny_max_m(64)            # time the few-rows kernel up to its own limit, not the caller's
     try:
@@ -108,11 +110,19 @@ def gemm(args) -> None:
             for rows in _ints(args.rows):
                 x = torch.randn(rows, k, device="cuda", dtype=torch.bfloat16)
                 out = torch.empty(rows, n, device="cuda", dtype=torch.bfloat16)
-                for which, call in (("own", lambda i: ops.gemm(out, x, weights[i % sets])),
-                                    ("library", lambda i: torch.mm(x, weights[i % sets].t(), out=out))):
+                variants = [("own", 0, 0), ("library", 0, 0)]
+                if args.mid_sweep and 16 < rows <= 64:
+                    variants = [(f"mid w{wv} s{sp}", wv, sp) for wv in (4, 6, 8) for sp in _ints(args.mid_sweep)] + variants
+                for which, wv, sp in variants:
+                    if which == "library":
+                        call = lambda i: torch.mm(x, weights[i % sets].t(), out=out)
+                    else:
+                        ops.gemm_mid_tune(True, wv, sp)
+                        call = lambda i: ops.gemm(out, x, weights[i % sets])
                     seconds = _time(call, max(args.repeats, 2 * sets))
-                    print(f"gemm {name:8s} rows={rows:5d} {which:8s} {seconds * 1e6:9.1f} us  {n * k * 2 / seconds / 1e9:8.0f} GB/s of weights  "
+                    print(f"gemm {name:8s} rows={rows:5d} {which:10s} {seconds * 1e6:9.1f} us  {n * k * 2 / seconds / 1e9:8.0f} GB/s of weights  "
                           f"{2 * rows * n * k / seconds / 1e12:8.1f} TFLOP/s", flush=True)
+                ops.gemm_mid_tune(True, 0, 0)
             del weights
     finally:
         ops.set_skinny_max_m(before)
@@ -137,6 +147,7 @@ def main(argv=None) -> int:
     parser.add_argument("--head-dim", type=int, default=128)
     parser.add_argument("--hidden-size", type=int, default=4096)
     parser.add_argument("--intermediate-size", type=int, default=12288)
+    parser.add_argument("--vocab-size", type=int, default=0, help="gemm: also the LM head of this many rows")
     parser.add_argument("--page-size", type=int, default=16)
     parser.add_argument("--window", type=int, default=0)
     parser.add_argument("--tokens", default="2048", help="attention_prefill: prompt lengths, comma separated")
@@ -148,6 +159,7 @@ def main(argv=None) -> int:
     parser.add_argument("--splits", default="1,2,4,8,16", help="attention_decode: workgroups per (token, kv head)")
     parser.add_argument("--form", default="0,1,2", help="attention_decode: 0 four waves, 1 four waves with the next tile on the way, 2 eight waves likewise")
     parser.add_argument("--rows", default="1,8,16,64,2048", help="gemm: numbers of rows")
+    parser.add_argument("--mid-sweep", default="", help="gemm: also time the kernel for 17..64 rows with 4, 6 and 8 waves at these numbers of K splits")
     parser.add_argument("--megabytes", default="32,200,1200", help="memory: sizes of the buffers read")
     parser.add_argument("--blocks", default="512,2048,8192", help="memory: numbers of workgroups")
     parser.add_argument("--repeats", type=int, default=20)

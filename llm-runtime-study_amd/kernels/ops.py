@@ -55,6 +55,9 @@ _SIGNATURES = {
     "lrs_gemm_prepare": (c_int, []),
     "lrs_host_device_pointer": (c_int, [c_void_p, POINTER(c_void_p)]),
     "lrs_gemm_set_skinny_max_m": (c_int, [c_int]),
+    "lrs_gemm_mid_tune": (c_int, [c_int, c_int, c_int]),
+    "lrs_gemm_mid_enabled": (c_int, []),
+    "lrs_gemm_mid_add_rmsnorm": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_float, c_void_p]),
     "lrs_attention": (c_int, [c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p,
                               c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_void_p]),
     "lrs_attention_decode": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p,
@@ -281,6 +284,46 @@ def add_into(residual: torch.Tensor, y: torch.Tensor) -> None:
 def skinny_max_m() -> int:
     """Most rows for which the few-rows product kernel is the one to use."""
     return library().lrs_gemm_skinny_max_m()
+
+
+def gemm_mid_tune(enabled: bool = True, waves: int = 0, splits: int = 0) -> None:
+    """Whether bf16 products of 17..64 rows take this package's kernel for them, and (for measurements)
+    its workgroup shape (4, 6 or 8 waves) and number of K splits; 0 lets the library choose."""
+    _check(library().lrs_gemm_mid_tune(int(bool(enabled)), waves, splits))
+
+
+def gemm_mid_enabled() -> bool:
+    return bool(library().lrs_gemm_mid_enabled())
+
+
+# The kernel for 17..64 rows takes up to 64, but measured on MI355X in whole decode steps (Qwen3-8B shape)
+# it beats the vendor library's products up to 48 rows (4 % at 24, 3 % at 32, equal at 48) and loses 1 % at 64,
+# where its activation loads cost as much as a fifth of its time: callers that may use the library do so from 49 rows on.
+MID_ROWS_PREFERRED = 48
+
+
+def gemm_mid_takes(dtype: torch.dtype, m: int, n: int, k: int, most: int = 64) -> bool:
+    """Whether a product of m rows (at most `most`) can go to the kernel for 17..64 rows (weights streamed
+    once, activations shared through LDS), which also writes the gated activation itself."""
+    return dtype == torch.bfloat16 and 16 < m <= min(most, 64) and k % 256 == 0 and n % 16 == 0 and gemm_mid_enabled()
+
+
+def gemm_mid_add_rmsnorm(normed: torch.Tensor, residual: torch.Tensor, a: torch.Tensor, w: torch.Tensor,
+                         norm_weight: torch.Tensor, eps: float) -> None:
+    """residual (float32 [M, N]) += a @ w.T, then normed = RMSNorm(residual) with norm_weight: the product
+    of 17..64 bf16 rows, its residual add and the norm that follows, the sums of the product's K splits going
+    straight into the kernel that adds and normalises."""
+    m, k = a.shape
+    n = w.shape[0]
+    _need(gemm_mid_takes(w.dtype, m, n, k) and a.dtype == torch.bfloat16, "gemm_mid_add_rmsnorm: takes bf16 products of 17..64 rows, K % 256 == 0, N % 16 == 0")
+    _need(w.dim() == 2 and w.is_contiguous() and w.shape[1] == k, f"gemm_mid_add_rmsnorm: weight must be contiguous [N, {k}]")
+    _need(residual.dtype == torch.float32 and residual.is_contiguous() and residual.shape == (m, n), f"gemm_mid_add_rmsnorm: residual must be contiguous float32 [{m}, {n}]")
+    _need(normed.is_contiguous() and normed.shape == (m, n), f"gemm_mid_add_rmsnorm: normed must be contiguous [{m}, {n}]")
+    _need(norm_weight.is_contiguous() and norm_weight.numel() == n and eps > 0, f"gemm_mid_add_rmsnorm: norm weight must hold {n} values and eps be positive")
+    _need(n <= 8192, "gemm_mid_add_rmsnorm: rows of at most 8192 values")
+    _check(library().lrs_gemm_mid_add_rmsnorm(_dev(normed, "normed"), dtype_code(normed.dtype), _dev(residual, "residual"), _dev(a, "a"),
+                                              _dev(w, "w"), _dev(norm_weight, "norm_weight"), dtype_code(norm_weight.dtype), m, n, k,
+                                              _rows(a, "a"), eps, _stream()))
 
 
 def set_skinny_max_m(m: int) -> None:

@@ -237,6 +237,60 @@ def test_gemm(ops, dtype, m, n, k, mode):
         torch.testing.assert_close(out.cpu().double(), want, rtol=1e-4, atol=1e-4)
 
 
+@pytest.mark.parametrize("m", [17, 32, 40, 48, 49, 64])
+@pytest.mark.parametrize("n,k", [(64, 256), (208, 512), (4096, 1024), (6144, 4096), (1040, 3328)])
+@pytest.mark.parametrize("waves,splits", [(0, 0), (4, 1), (6, 2), (8, 3), (4, 8)])
+def test_gemm_of_17_to_64_rows(ops, m, n, k, waves, splits):
+    """The kernel for 17..64 rows (K a multiple of 256): every workgroup shape, K divided between
+    workgroups or not, ragged last tiles, all three output modes and the gated epilogue."""
+    g = torch.Generator().manual_seed(m * 131 + n + k)
+    a = torch.randn(m, k, generator=g).bfloat16()
+    w = (torch.randn(n, k, generator=g) / math.sqrt(k)).bfloat16()
+    want = a.double() @ w.double().T
+    ops.gemm_mid_tune(True, waves, splits)
+    try:
+        stored = torch.empty(m, n, device="cuda", dtype=torch.bfloat16)
+        ops.gemm(stored, dev(a), dev(w))
+        wide = torch.full((m, n), 0.5, device="cuda")
+        ops.gemm(wide, dev(a), dev(w), accumulate=True)
+        plain = torch.empty(m, n, device="cuda")
+        ops.gemm(plain, dev(a), dev(w))
+        inter = n // 2
+        gate, up = w[:inter], w[inter:]
+        mixed = torch.stack((gate.view(inter // 8, 8, k), up.view(inter // 8, 8, k)), 1).reshape(n, k).contiguous()
+        gated = torch.empty(m, inter, device="cuda", dtype=torch.bfloat16)
+        ops.gemm(gated, dev(a), dev(mixed), swiglu=True)
+    finally:
+        ops.gemm_mid_tune(True, 0, 0)
+    torch.testing.assert_close(stored.cpu().double(), want, rtol=1e-2, atol=1e-2)
+    torch.testing.assert_close(plain.cpu().double(), want, rtol=1e-4, atol=1e-4)
+    torch.testing.assert_close(wide.cpu().double(), want + 0.5, rtol=1e-4, atol=1e-4)
+    close_in_norm(gated, torch.nn.functional.silu(want[:, :inter]) * want[:, inter:])
+
+
+@pytest.mark.parametrize("w_dtype", DTYPES)
+@pytest.mark.parametrize("m,n,k,splits", [(17, 64, 256, 0), (40, 208, 1024, 2), (64, 4096, 4096, 0), (33, 1040, 3328, 3), (48, 5120, 512, 1)])
+def test_gemm_of_17_to_64_rows_with_residual_add_and_norm(ops, w_dtype, m, n, k, splits):
+    """residual += x W^T and the RMSNorm of the new residual, the K splits' sums added inside the norm kernel."""
+    g = torch.Generator().manual_seed(m + n + k)
+    a = torch.randn(m, k, generator=g).bfloat16()
+    w = (torch.randn(n, k, generator=g) / math.sqrt(k)).bfloat16()
+    residual = torch.randn(m, n, generator=g) * 2
+    gamma = (1 + 0.2 * torch.randn(n, generator=g)).to(w_dtype)
+    eps = 1e-5
+    updated = residual.double() + a.double() @ w.double().T
+    want = gamma.double() * updated * torch.rsqrt(updated.square().mean(-1, keepdim=True) + eps)
+    out = dev(residual.clone())
+    normed = torch.empty(m, n, device="cuda", dtype=torch.bfloat16)
+    ops.gemm_mid_tune(True, 0, splits)
+    try:
+        ops.gemm_mid_add_rmsnorm(normed, out, dev(a), dev(w), dev(gamma), eps)
+    finally:
+        ops.gemm_mid_tune(True, 0, 0)
+    torch.testing.assert_close(out.cpu().double(), updated, rtol=1e-4, atol=1e-4)
+    close_in_norm(normed, want, 5e-3)
+
+
 @pytest.mark.parametrize("w_dtype", DTYPES)
 @pytest.mark.parametrize("m,n,k", [(1, 64, 96), (8, 331, 160), (17, 200, 96), (64, 6144, 4096), (33, 48, 264)])
 def test_gemm_with_fused_rmsnorm_input(ops, w_dtype, m, n, k, all_rows_in_own_kernel):
