@@ -624,8 +624,8 @@ __global__ void gemm_split_finish_kernel(void* __restrict__ out, int mode, const
 // as many bytes as the weights of a workgroup, so the waves of a workgroup (each with 16 weight rows
 // of its own) share them through LDS.  K is walked in slices of 256: while a slice is multiplied,
 // the weights of the next two slices are on their way into registers and the activations of the
-// next slice lie in the other LDS buffer, stored there in MFMA B-fragment order (a fragment is 1 KB,
-// lane l at byte 16 l: reads and writes are conflict-free).  gridDim.y > 1 divides K between
+// next slice lie in the other LDS buffer, loaded as whole 128-byte lines and laid out so that fragment reads
+// meet no bank conflicts (see below).  gridDim.y > 1 divides K between
 // workgroups; with split_sums given every workgroup leaves its sums there ([gridDim.y, m, n]) for a
 // kernel that adds them up (gemm_split_finish_kernel, or the residual add and norm that follow).  K % 256 == 0.
 template <int MT, int WAVES, bool SWIGLU>
@@ -649,18 +649,33 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_mid_kernel(
   // of a column's sum then depends on the column's workgroup alone.
   const int turn = count > 0 ? (int)(blockIdx.x % (unsigned)count) : 0;
   auto slice_at = [&](int c) -> int { const int v = c + turn; return s0 + (v >= count ? v - count : v); };
+  // The activations of a slice come from memory as whole 128-byte lines: a load instruction brings 8 k
+  // chunks (16 bytes each) of 8 tokens, FRAGS such pieces a slice, dealt out over the waves.  (Loaded as
+  // B fragments, 64 bytes of 16 tokens an instruction, they cost a fifth of the kernel's time at 64 rows.)
+  // In LDS a slice is 8 panels (one per k step) of MT blocks of 16 tokens; a token's row in a block is
+  // its 4 chunks of that step, 64 bytes, and rows and chunks are permuted like this: rows swap places in
+  // pairs in the upper half of a block, chunks are turned round by the row number, and odd panels swap
+  // neighbouring rows once more.  A fragment read (lane = token % 16 + 16 * chunk) then touches every
+  // bank once in each of its quarter-waves, and the 8 chunks of a token that one lane group of a load
+  // writes fall into the two halves of a 128-byte bank line.  Address in 16-byte units:
+  //   panel * MT * 64 + block * 64 + (row ^ (row >> 3 & 1) ^ (panel & 1)) * 4 + (chunk ^ (row >> 1 & 3))
   // Every load and every LDS write below is unconditional, so that the compiler can count the loads
   // in flight instead of waiting for all of them at a branch: a token past m reads the last token's
-  // row (its columns of the result are never written), and where the fragments do not divide evenly
-  // between the waves the spare turns bring the last fragment once more (same data, same place).
+  // row (its columns of the result are never written), and where the pieces do not divide evenly
+  // between the waves the spare turns bring the last piece once more (same data, same place).
+  auto place = [&](int panel, int block, int row, int chunk) -> int {
+    return panel * (MT * 64) + block * 64 + ((row ^ ((row >> 3) & 1) ^ (panel & 1)) * 4 + (chunk ^ ((row >> 1) & 3)));
+  };
   const bf16* xp[MINE];
   bf16x8* spot[MINE];
+  bf16x8* const lds = &acts[0][0][0][0];
 #pragma unroll
   for (int i = 0; i < MINE; ++i) {
-    const int f = wave + i * WAVES < FRAGS ? wave + i * WAVES : FRAGS - 1;
-    const int step = f / MT, t = f % MT, token = t * 16 + r < m ? t * 16 + r : m - 1;
-    xp[i] = x + (int64_t)token * lda + step * 32 + g * 8;
-    spot[i] = &acts[0][step][t][lane];
+    const int piece = wave + i * WAVES < FRAGS ? wave + i * WAVES : FRAGS - 1;
+    const int oct = piece % (2 * MT), line = piece / (2 * MT);              // 8 tokens, 128 bytes of the slice
+    const int tok = oct * 8 + lane / 8, chunk = line * 8 + lane % 8;
+    xp[i] = x + (int64_t)(tok < m ? tok : m - 1) * lda + chunk * 8;
+    spot[i] = lds + place(chunk / 4, tok / 16, tok % 16, chunk % 4);
   }
   floatx4 acc[MT];
 #pragma unroll
@@ -682,18 +697,20 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_mid_kernel(
   // for slice `next`, as soon as its products are issued (the scheduling barriers keep the compiler
   // from gathering these loads at the end, where they would leave the memory idle meanwhile).  The
   // activation fragments of a step are read from LDS while the step before is multiplied.
-  const bf16x8* frag = &acts[0][0][0][lane];
+  const bf16x8* const frag_even = lds + place(0, 0, r, g);    // this lane's piece of a fragment in an even panel ...
+  const bf16x8* const frag_odd = lds + place(1, 0, r, g) - MT * 64;   // ... and in an odd one, less the panel's own offset
   auto compute = [&](int buf, bf16x8 (&a)[STEPS], auto reload, int next) {
     constexpr bool RELOAD = decltype(reload)::value;
-    const bf16x8* from = frag + buf * (STEPS * MT * WAVE);
+    const bf16x8* const even = frag_even + buf * (STEPS * MT * WAVE);
+    const bf16x8* const odd = frag_odd + buf * (STEPS * MT * WAVE);
     bf16x8 b[2][MT];
 #pragma unroll
-    for (int t = 0; t < MT; ++t) b[0][t] = from[t * WAVE];
+    for (int t = 0; t < MT; ++t) b[0][t] = even[t * WAVE];
 #pragma unroll
     for (int j = 0; j < STEPS; ++j) {
       if (j + 1 < STEPS) {
 #pragma unroll
-        for (int t = 0; t < MT; ++t) b[(j + 1) & 1][t] = from[((j + 1) * MT + t) * WAVE];
+        for (int t = 0; t < MT; ++t) b[(j + 1) & 1][t] = ((j + 1) & 1 ? odd : even)[((j + 1) * MT + t) * WAVE];
       }
 #pragma unroll
       for (int t = 0; t < MT; ++t) acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[j], b[j & 1][t], acc[t], 0, 0, 0);
@@ -826,6 +843,7 @@ static float* split_sums_buffer() {
 // The kernel for 17..64 rows: which of its workgroup shapes and how many K splits.  0 = chosen here:
 // the shape and split that fill a whole multiple of the compute units best, then the fewest splits.
 static int g_mid_waves = 0, g_mid_splits = 0, g_mid_enabled = 1;
+LRS_API int lrs_compute_units();
 LRS_API int lrs_gemm_mid_tune(int enabled, int waves, int splits) {
   LRS_REQUIRE(waves == 0 || waves == 4 || waves == 6 || waves == 8, "gemm_mid_tune: 4, 6 or 8 waves (0: automatic), got %d", waves);
   LRS_REQUIRE(splits >= 0 && splits <= 16, "gemm_mid_tune: 0..16 splits, got %d", splits);
@@ -836,23 +854,63 @@ LRS_API int lrs_gemm_mid_enabled() { return g_mid_enabled; }
 
 static void choose_mid_shape(int n, int k, int& waves, int& splits) {
   const int units = lrs_compute_units() > 0 ? lrs_compute_units() : 256, slices = k / 256;
-  double best = -1.0;
+  auto tiles_of = [&](int wv) { return (n + 16 * wv - 1) / (16 * wv); };
+  auto fill_of = [&](int groups) { return (double)groups / ((groups + units - 1) / units * units); };
+  if (g_mid_waves && g_mid_splits) {
+    waves = g_mid_waves, splits = g_mid_splits;
+    return;
+  }
+  // Measured on MI355X (Qwen3-8B shapes, 32..64 rows).  A matrix with enough rows to give every compute
+  // unit a workgroup is not divided along K: six waves (96 rows) a workgroup, or four where that fills the
+  // chip clearly better; eight waves walking many slices were a third slower (gate_up, the LM head).
+  if ((!g_mid_splits || g_mid_splits == 1) && tiles_of(6) >= units && (!g_mid_waves || g_mid_waves == 4 || g_mid_waves == 6)) {
+    splits = 1;
+    waves = g_mid_waves ? g_mid_waves : (fill_of(tiles_of(4)) > fill_of(tiles_of(6)) + 0.08 ? 4 : 6);
+    return;
+  }
+  // A narrower matrix: K is divided so that tiles x splits fills the units once (at least two slices a
+  // workgroup, at most 8 splits).  Of the choices within 3 % of the fullest: the one with the most waves
+  // among those whose workgroups still walk four slices or more (down: 8 waves x 8 splits, 6 slices each),
+  // else the one with the fewest waves (o_proj: 4 waves x 4 splits); then the fewest splits.
+  struct Choice { int waves, splits, len; double fill; };
+  Choice all[24];
+  int count = 0;
+  double fullest = -1.0;
   const int shapes[3] = {4, 6, 8};
   for (int wi = 0; wi < 3; ++wi) {
     const int wv = shapes[wi];
     if (g_mid_waves && wv != g_mid_waves) continue;
-    const int tiles = (n + 16 * wv - 1) / (16 * wv);
     for (int sp = 1; sp <= 8; ++sp) {
       if (g_mid_splits && sp != g_mid_splits) continue;
-      if (sp > 1 && slices / sp < 2) continue;                  // at least two slices a workgroup
-      const int groups = tiles * sp;
-      const int rounds = (groups + units - 1) / units;
-      // share of the chip at work, less a little for every split (its sums are written and read again)
-      const double score = (double)groups / (rounds * units) - 0.02 * (sp - 1) - 0.01 * (rounds - 1);
-      if (score > best + 1e-9) best = score, waves = wv, splits = sp;
+      if (sp > 1 && slices / sp < 2) continue;
+      const int groups = tiles_of(wv) * sp;
+      const double fill = groups <= units ? (double)groups / units : fill_of(groups) - 0.25;   // a second round costs more than its share
+      all[count++] = Choice{wv, sp, slices / sp, fill};
+      if (fill > fullest) fullest = fill;
     }
   }
-  if (best < 0) waves = g_mid_waves ? g_mid_waves : 4, splits = 1;
+  if (count == 0) {
+    waves = g_mid_waves ? g_mid_waves : 4, splits = g_mid_splits ? g_mid_splits : 1;
+    return;
+  }
+  const Choice* pick = nullptr;
+  for (int i = 0; i < count; ++i) {
+    const Choice& c = all[i];
+    if (c.fill < fullest - 0.03) continue;
+    if (!pick) { pick = &c; continue; }
+    const bool c_long = c.len >= 4, p_long = pick->len >= 4;
+    if (c_long != p_long) { if (c_long) pick = &c; continue; }
+    if (c.waves != pick->waves) { if ((c.waves > pick->waves) == c_long) pick = &c; continue; }
+    if (c.splits < pick->splits) pick = &c;
+  }
+  waves = pick->waves, splits = pick->splits;
+}
+
+// The shape the kernel for 17..64 rows takes for a matrix of n rows and k columns (for tests and reports).
+LRS_API int lrs_gemm_mid_shape(int n, int k, int* waves, int* splits) {
+  LRS_REQUIRE(n > 0 && k > 0 && k % 256 == 0 && waves && splits, "gemm_mid_shape: needs n > 0 and K %% 256 == 0, got n=%d k=%d", n, k);
+  choose_mid_shape(n, k, *waves, *splits);
+  return 0;
 }
 
 // keep_sums: the sums of the K splits (of the one split, if K is not divided) stay in the split buffer for

@@ -525,9 +525,9 @@ class ModelRunner:
         while bucket < len(entries):
             bucket *= 2
         bucket = min(bucket, self.max_requests)
-        # Up to 48 rows a bfloat16 graph holds this package's kernels only (the few-rows kernels, then the
-        # kernel for 17..64 rows); a batch padded to 64 rows brings the vendor library's products into the
-        # capture when the runner may use them.
+        # A bfloat16 graph of up to 64 rows holds this package's kernels (the few-rows kernels, then the
+        # kernel for 17..64 rows); where a shape does not suit that kernel (K no multiple of 256) and the runner
+        # may use the vendor library, its products are captured with them.
         most = max(ops.skinny_max_m(), self.LIBRARY_GRAPH_ROWS) if self.dtype == torch.bfloat16 else ops.skinny_max_m()
         return bucket if bucket <= min(self.max_step_tokens, most) else 0
 

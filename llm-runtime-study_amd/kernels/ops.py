@@ -57,6 +57,7 @@ _SIGNATURES = {
     "lrs_gemm_set_skinny_max_m": (c_int, [c_int]),
     "lrs_gemm_mid_tune": (c_int, [c_int, c_int, c_int]),
     "lrs_gemm_mid_enabled": (c_int, []),
+    "lrs_gemm_mid_shape": (c_int, [c_int, c_int, c_void_p, c_void_p]),
     "lrs_gemm_mid_add_rmsnorm": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_float, c_void_p]),
     "lrs_attention": (c_int, [c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p,
                               c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_void_p]),
@@ -292,14 +293,22 @@ def gemm_mid_tune(enabled: bool = True, waves: int = 0, splits: int = 0) -> None
     _check(library().lrs_gemm_mid_tune(int(bool(enabled)), waves, splits))
 
 
+def gemm_mid_shape(n: int, k: int) -> tuple[int, int]:
+    """(waves a workgroup, K splits) the kernel for 17..64 rows takes for a weight matrix [n, k]."""
+    import ctypes
+    waves, splits = ctypes.c_int(0), ctypes.c_int(0)
+    _check(library().lrs_gemm_mid_shape(n, k, ctypes.addressof(waves), ctypes.addressof(splits)))
+    return waves.value, splits.value
+
+
 def gemm_mid_enabled() -> bool:
     return bool(library().lrs_gemm_mid_enabled())
 
 
-# The kernel for 17..64 rows takes up to 64, but measured on MI355X in whole decode steps (Qwen3-8B shape)
-# it beats the vendor library's products up to 48 rows (4 % at 24, 3 % at 32, equal at 48) and loses 1 % at 64,
-# where its activation loads cost as much as a fifth of its time: callers that may use the library do so from 49 rows on.
-MID_ROWS_PREFERRED = 48
+# Rows up to which callers that may use the vendor library take this package's kernel for 17..64 rows instead.
+# Measured on MI355X in whole decode steps (Qwen3-8B shape): 4-6 % faster than the library's products at
+# batches of 24, 32, 48 and 64.
+MID_ROWS_PREFERRED = 64
 
 
 def gemm_mid_takes(dtype: torch.dtype, m: int, n: int, k: int, most: int = 64) -> bool:

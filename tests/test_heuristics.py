@@ -54,3 +54,20 @@ def test_prefill_splits_only_where_groups_leave_the_chip_idle(monkeypatch):
     assert splits(8, 32768, 1 << 16) == 32              # one token: as many as allowed
     assert splits(8, 2048, 1 << 16) == 2                # at least 1,024 keys each
     assert splits(8, 1 << 20, 16 << 20) == 4            # partial results stay within 256 MB
+
+
+def test_shapes_of_the_kernel_for_17_to_64_rows():
+    """Workgroup shape and K splits for the layer shapes it was measured on: wide matrices are not divided
+    (six waves), narrow ones are divided until every compute unit has a workgroup, short walks take the
+    smaller workgroup and long ones the larger."""
+    from llm_runtime_study_amd.kernels import ops
+
+    units = ops.compute_units()
+    if units not in (0, 256):
+        return
+    assert ops.gemm_mid_shape(24576, 4096) == (6, 1) and ops.gemm_mid_shape(151936, 4096) == (6, 1)
+    assert ops.gemm_mid_shape(6144, 4096) == (6, 4)
+    assert ops.gemm_mid_shape(4096, 4096) == (4, 4) and ops.gemm_mid_shape(4096, 12288) == (8, 8)
+    for n, k in ((64, 256), (208, 512), (5120, 5120), (5120, 17408), (7168, 5120), (51200, 5120), (1040, 3328)):
+        waves, splits = ops.gemm_mid_shape(n, k)
+        assert waves in (4, 6, 8) and 1 <= splits <= 8 and (splits == 1 or k // 256 // splits >= 2)
