@@ -338,7 +338,7 @@ struct NormChain {
 };
 
 
-template <int MT, int RT, int WAVES, int UNROLL, bool NORM, bool SWIGLU, bool PARTIAL = false>
+template <int MT, int RT, int WAVES, int UNROLL, bool NORM, bool SWIGLU, bool PARTIAL = false, bool LINES = false>
 __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_skinny_kernel(
     void* __restrict__ out, int mode, const bf16* __restrict__ x, NormInput norm,
     const bf16* __restrict__ w, const bf16* __restrict__ bias, int m, int n, int k, int lda, int ldc,
@@ -349,6 +349,14 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_skinny_kernel(
   // loaded nor written).
   // gridDim.y > 1: K is also divided between workgroups; each then leaves its sums in
   // split_sums [gridDim.y, m, n] for gemm_split_finish_kernel instead of writing the output.
+  // LINES: the weights come from memory as whole 128-byte lines (a load instruction brings 8 k chunks of
+  // 8 rows; as fragments, 64 bytes of 16 rows, the same kilobyte is twice as many requests, which is what
+  // these kernels are short of) and take their places in the fragments through a patch of LDS of the
+  // wave's own: two instructions fill 16 rows x 128 bytes, laid out as two panels (one per k step) of
+  // 16 rows x 64 bytes with rows and chunks permuted so that writes and fragment reads meet no bank
+  // conflicts; four steps go through the patch at a time.  No barrier: a wave's LDS instructions
+  // execute in order.
+  __shared__ bf16x8 patch_all[LINES ? WAVES : 1][2][128];
   __shared__ floatx4 partial[WAVES][MT][WAVE];
   __shared__ float sumsq[WAVES][MT][16];
   __shared__ float chain_parts[WAVES * 4][16];   // in_sumsq, added up by WAVES * 4 threads per row
@@ -365,6 +373,24 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_skinny_kernel(
     wrow[q] = !PARTIAL || n0 + q * 16 + r < n_end;
     const int row = PARTIAL ? (wrow[q] ? n0 + q * 16 + r : n0) : (n0 + q * 16 + r < n ? n0 + q * 16 + r : n - 1);
     wp[q] = w + (int64_t)row * k + g * 8;
+  }
+  const bf16* wl[RT][2];
+  int wr_off[2], rd_off[2];
+  bf16x8* const patch = &patch_all[LINES ? wave : 0][0][0];
+  if constexpr (LINES) {
+    auto place = [](int panel, int row, int chunk) -> int {
+      return panel * 64 + ((row ^ ((row >> 3) & 1) ^ (panel & 1)) * 4 + (chunk ^ ((row >> 1) & 3)));
+    };
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      wr_off[h] = place((lane % 8) / 4, 8 * h + lane / 8, lane % 4);
+      rd_off[h] = place(h, r, g);
+#pragma unroll
+      for (int q = 0; q < RT; ++q) {
+        const int row = n0 + q * 16 + 8 * h + lane / 8;
+        wl[q][h] = w + (int64_t)(row < n ? row : n - 1) * k + (lane % 8) * 8;
+      }
+    }
   }
   const bf16* xp[MT];
   const float* hp[MT];
@@ -454,6 +480,31 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_skinny_kernel(
   // U steps of 32 k, all their loads asked for before any is used
   auto steps_together = [&](int sb, auto count) {
     constexpr int U = decltype(count)::value;
+    if constexpr (LINES && U % 4 == 0) {
+      bf16x8 raw[U][RT], b[U][MT];
+#pragma unroll
+      for (int u = 0; u < U; ++u)
+#pragma unroll
+        for (int q = 0; q < RT; ++q) raw[u][q] = *(const bf16x8*)(wl[q][u & 1] + (sb + (u & ~1)) * 32);
+#pragma unroll
+      for (int u = 0; u < U; ++u)
+#pragma unroll
+        for (int t = 0; t < MT; ++t) b[u][t] = load_b(t, sb + u);
+#pragma unroll
+      for (int c4 = 0; c4 < U; c4 += 4)
+#pragma unroll
+        for (int q = 0; q < RT; ++q) {
+#pragma unroll
+          for (int i = 0; i < 4; ++i) patch[(i >> 1) * 128 + wr_off[i & 1]] = raw[c4 + i][q];
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            const bf16x8 a = patch[(i >> 1) * 128 + rd_off[i & 1]];
+#pragma unroll
+            for (int t = 0; t < MT; ++t) acc[q][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b[c4 + i][t], acc[q][t], 0, 0, 0);
+          }
+        }
+      return;
+    }
     bf16x8 a[U][RT], b[U][MT];
 #pragma unroll
     for (int u = 0; u < U; ++u)
@@ -795,6 +846,13 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_mid_kernel(
   }
 }
 
+// Whether the few-rows kernel loads its weights as whole 128-byte lines where the shape allows (for measurements).
+static int g_skinny_lines = 1;
+LRS_API int lrs_gemm_skinny_lines(int enabled) {
+  g_skinny_lines = enabled != 0;
+  return 0;
+}
+
 // Row tiles per workgroup: more of them means each activation fragment read from L2 serves more
 // weight rows, which matters once there are several token blocks; fewer means more workgroups.
 template <int MT, int RT, bool NORM, bool SWIGLU>
@@ -806,8 +864,15 @@ static void launch_skinny_rt(void* out, int mode, const bf16* a, NormInput norm,
   if (group_rows != 16 * RT) {
     if constexpr (MT == 1 && RT == 2 && !NORM && !SWIGLU)
       gemm_bf16_skinny_kernel<MT, RT, 8, UNROLL, NORM, SWIGLU, true><<<dim3(groups, splits), 8 * 64, 0, s>>>(out, mode, a, norm, w, bias, m, n, k, lda, ldc, split_sums, chain, group_rows);
-  } else if (groups <= 2048)
+  } else if (groups <= 2048) {
+    if constexpr (MT == 1 && !NORM && UNROLL % 4 == 0) {
+      if (g_skinny_lines && splits == 1 && k % 64 == 0 && (k / 32) % 16 == 0) {   // every wave starts at an even step
+        gemm_bf16_skinny_kernel<MT, RT, 8, UNROLL, NORM, SWIGLU, false, true><<<dim3(groups, 1), 8 * 64, 0, s>>>(out, mode, a, norm, w, bias, m, n, k, lda, ldc, split_sums, chain, group_rows);
+        return;
+      }
+    }
     gemm_bf16_skinny_kernel<MT, RT, 8, UNROLL, NORM, SWIGLU><<<dim3(groups, splits), 8 * 64, 0, s>>>(out, mode, a, norm, w, bias, m, n, k, lda, ldc, split_sums, chain, group_rows);
+  }
   else
     gemm_bf16_skinny_kernel<MT, RT, 4, UNROLL, NORM, SWIGLU><<<dim3(groups, splits), 4 * 64, 0, s>>>(out, mode, a, norm, w, bias, m, n, k, lda, ldc, split_sums, chain, group_rows);
   if (splits > 1) {
@@ -959,8 +1024,12 @@ static void launch_skinny(void* out, int mode, const bf16* a, NormInput norm, co
     launch_skinny_rt<MT, (MT > 1 ? 4 : 1), NORM, SWIGLU>(out, mode, a, norm, w, bias, m, n, k, lda, ldc, s, sums, splits);
     return;
   }
-  if (MT == 1 && !NORM && n >= 16384)   // measured: two row tiles and four waves stream wide matrices a little faster
-    gemm_bf16_skinny_kernel<1, 2, 4, 4, NORM, SWIGLU><<<dim3((n + 31) / 32, 1), 4 * 64, 0, s>>>(out, mode, a, norm, w, bias, m, n, k, lda, ldc, nullptr, chain, 32);
+  if (MT == 1 && !NORM && n >= 16384) {  // measured: two row tiles and four waves stream wide matrices a little faster
+    if (g_skinny_lines && k % 64 == 0 && (k / 32) % 8 == 0)
+      gemm_bf16_skinny_kernel<1, 2, 4, 4, NORM, SWIGLU, false, true><<<dim3((n + 31) / 32, 1), 4 * 64, 0, s>>>(out, mode, a, norm, w, bias, m, n, k, lda, ldc, nullptr, chain, 32);
+    else
+      gemm_bf16_skinny_kernel<1, 2, 4, 4, NORM, SWIGLU><<<dim3((n + 31) / 32, 1), 4 * 64, 0, s>>>(out, mode, a, norm, w, bias, m, n, k, lda, ldc, nullptr, chain, 32);
+  }
   else if (MT == 1 && !NORM && !SWIGLU && even_group_rows(n) > 0) {
     if constexpr (MT == 1 && !NORM && !SWIGLU)
       launch_skinny_rt<1, 2, false, false>(out, mode, a, norm, w, bias, m, n, k, lda, ldc, s, nullptr, 1, chain, even_group_rows(n));

@@ -57,6 +57,7 @@ _SIGNATURES = {
     "lrs_gemm_set_skinny_max_m": (c_int, [c_int]),
     "lrs_gemm_mid_tune": (c_int, [c_int, c_int, c_int]),
     "lrs_gemm_mid_enabled": (c_int, []),
+    "lrs_gemm_skinny_lines": (c_int, [c_int]),
     "lrs_gemm_mid_shape": (c_int, [c_int, c_int, c_void_p, c_void_p]),
     "lrs_gemm_mid_add_rmsnorm": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_float, c_void_p]),
     "lrs_attention": (c_int, [c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p,
@@ -291,6 +292,11 @@ def gemm_mid_tune(enabled: bool = True, waves: int = 0, splits: int = 0) -> None
     """Whether bf16 products of 17..64 rows take this package's kernel for them, and (for measurements)
     its workgroup shape (4, 6 or 8 waves) and number of K splits; 0 lets the library choose."""
     _check(library().lrs_gemm_mid_tune(int(bool(enabled)), waves, splits))
+
+
+def gemm_skinny_lines(enabled: bool) -> None:
+    """Whether the few-rows kernel loads its weights as whole 128-byte lines where the shape allows (for measurements)."""
+    _check(library().lrs_gemm_skinny_lines(int(bool(enabled))))
 
 
 def gemm_mid_shape(n: int, k: int) -> tuple[int, int]:
