@@ -375,6 +375,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_skinny_kernel(
     wp[q] = w + (int64_t)row * k + g * 8;
   }
   const bf16* wl[RT][2];
+  bool wl_ok[RT][2];
   int wr_off[2], rd_off[2];
   bf16x8* const patch = &patch_all[LINES ? wave : 0][0][0];
   if constexpr (LINES) {
@@ -388,6 +389,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_skinny_kernel(
 #pragma unroll
       for (int q = 0; q < RT; ++q) {
         const int row = n0 + q * 16 + 8 * h + lane / 8;
+        wl_ok[q][h] = !PARTIAL || row < n_end;                 // PARTIAL: rows past the workgroup's own are the next one's
         wl[q][h] = w + (int64_t)(row < n ? row : n - 1) * k + (lane % 8) * 8;
       }
     }
@@ -485,7 +487,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_skinny_kernel(
 #pragma unroll
       for (int u = 0; u < U; ++u)
 #pragma unroll
-        for (int q = 0; q < RT; ++q) raw[u][q] = *(const bf16x8*)(wl[q][u & 1] + (sb + (u & ~1)) * 32);
+        for (int q = 0; q < RT; ++q) raw[u][q] = wl_ok[q][u & 1] ? *(const bf16x8*)(wl[q][u & 1] + (sb + (u & ~1)) * 32) : zero;
 #pragma unroll
       for (int u = 0; u < U; ++u)
 #pragma unroll
@@ -862,8 +864,12 @@ static void launch_skinny_rt(void* out, int mode, const bf16* a, NormInput norm,
   const int groups = (n + group_rows - 1) / group_rows;
   constexpr int UNROLL = (NORM ? 4 : 8) / (MT * RT > 4 ? 4 : (MT * RT > 1 ? 2 : 1));
   if (group_rows != 16 * RT) {
-    if constexpr (MT == 1 && RT == 2 && !NORM && !SWIGLU)
-      gemm_bf16_skinny_kernel<MT, RT, 8, UNROLL, NORM, SWIGLU, true><<<dim3(groups, splits), 8 * 64, 0, s>>>(out, mode, a, norm, w, bias, m, n, k, lda, ldc, split_sums, chain, group_rows);
+    if constexpr (MT == 1 && RT == 2 && !NORM && !SWIGLU) {
+      if (g_skinny_lines && splits == 1 && k % 64 == 0 && (k / 32) % 16 == 0 && UNROLL % 4 == 0)
+        gemm_bf16_skinny_kernel<MT, RT, 8, UNROLL, NORM, SWIGLU, true, true><<<dim3(groups, 1), 8 * 64, 0, s>>>(out, mode, a, norm, w, bias, m, n, k, lda, ldc, split_sums, chain, group_rows);
+      else
+        gemm_bf16_skinny_kernel<MT, RT, 8, UNROLL, NORM, SWIGLU, true><<<dim3(groups, splits), 8 * 64, 0, s>>>(out, mode, a, norm, w, bias, m, n, k, lda, ldc, split_sums, chain, group_rows);
+    }
   } else if (groups <= 2048) {
     if constexpr (MT == 1 && !NORM && UNROLL % 4 == 0) {
       if (g_skinny_lines && splits == 1 && k % 64 == 0 && (k / 32) % 16 == 0) {   // every wave starts at an even step
