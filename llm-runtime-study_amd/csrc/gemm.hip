@@ -688,11 +688,26 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_mid_kernel(
   constexpr int STEPS = 8;                         // k steps of 32 in a slice
   constexpr int FRAGS = STEPS * MT;                // activation fragments of a slice
   constexpr int MINE = (FRAGS + WAVES - 1) / WAVES;  // of which a wave brings this many
-  __shared__ bf16x8 acts[2][STEPS][MT][WAVE];
+  // LDS (dynamic: more than the 64 KB a static array may have): two buffers of activations, then a patch of
+  // 4 KB for each wave through which its weights, loaded as whole 128-byte lines (8 k chunks of 8 rows an
+  // instruction), take their places in the A fragments (see gemm_bf16_skinny_kernel, LINES).
+  extern __shared__ __attribute__((aligned(16))) bf16x8 mid_lds[];
   const int tid = threadIdx.x, lane = tid % WAVE, wave = __builtin_amdgcn_readfirstlane(tid / WAVE);
   const int r = lane & 15, g = lane >> 4;
   const int row0 = blockIdx.x * (16 * WAVES) + wave * 16;
-  const bf16* wp = w + (int64_t)(row0 + r < n ? row0 + r : n - 1) * k + g * 8;
+  bf16x8* const patch = mid_lds + 2 * STEPS * MT * WAVE + wave * 256;
+  const bf16* wl[2];
+  int wr_off[2], rd_off[2];
+#pragma unroll
+  for (int h = 0; h < 2; ++h) {
+    auto spot_of = [](int panel, int row, int chunk) -> int {
+      return panel * 64 + ((row ^ ((row >> 3) & 1) ^ (panel & 1)) * 4 + (chunk ^ ((row >> 1) & 3)));
+    };
+    const int row = row0 + 8 * h + lane / 8;
+    wl[h] = w + (int64_t)(row < n ? row : n - 1) * k + (lane % 8) * 8;
+    wr_off[h] = spot_of((lane % 8) / 4, 8 * h + lane / 8, lane % 4);
+    rd_off[h] = spot_of(h, r, g);
+  }
   const int slices = k / 256;
   const int per_split = (slices + gridDim.y - 1) / gridDim.y;
   const int s0 = blockIdx.y * per_split;
@@ -721,7 +736,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_mid_kernel(
   };
   const bf16* xp[MINE];
   bf16x8* spot[MINE];
-  bf16x8* const lds = &acts[0][0][0][0];
+  bf16x8* const lds = mid_lds;
 #pragma unroll
   for (int i = 0; i < MINE; ++i) {
     const int piece = wave + i * WAVES < FRAGS ? wave + i * WAVES : FRAGS - 1;
@@ -734,9 +749,10 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_mid_kernel(
 #pragma unroll
   for (int t = 0; t < MT; ++t) acc[t] = floatx4{0.f, 0.f, 0.f, 0.f};
   bf16x8 wa[STEPS], wb[STEPS], sa[MINE], sb[MINE];
+  // a[2 p + h]: line p (k steps 2 p and 2 p + 1) of rows 8 h .. 8 h + 7
   auto load_w = [&](int slice, bf16x8 (&a)[STEPS]) {
 #pragma unroll
-    for (int j = 0; j < STEPS; ++j) a[j] = *(const bf16x8*)(wp + (int64_t)slice * 256 + j * 32);
+    for (int j = 0; j < STEPS; ++j) a[j] = *(const bf16x8*)(wl[j & 1] + (int64_t)slice * 256 + (j >> 1) * 64);
   };
   auto load_acts = [&](int slice, bf16x8 (&st)[MINE]) {
 #pragma unroll
@@ -760,17 +776,27 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_mid_kernel(
 #pragma unroll
     for (int t = 0; t < MT; ++t) b[0][t] = even[t * WAVE];
 #pragma unroll
-    for (int j = 0; j < STEPS; ++j) {
-      if (j + 1 < STEPS) {
-#pragma unroll
-        for (int t = 0; t < MT; ++t) b[(j + 1) & 1][t] = ((j + 1) & 1 ? odd : even)[((j + 1) * MT + t) * WAVE];
-      }
-#pragma unroll
-      for (int t = 0; t < MT; ++t) acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[j], b[j & 1][t], acc[t], 0, 0, 0);
+    for (int p = 0; p < STEPS / 2; ++p) {
+      // two load instructions' worth (16 rows x 128 bytes) through the wave's patch: the A fragments of two steps
+      bf16x8* const pp = patch + (p & 1) * 128;
+      pp[wr_off[0]] = a[2 * p];
+      pp[wr_off[1]] = a[2 * p + 1];
+      const bf16x8 f0 = pp[rd_off[0]], f1 = pp[rd_off[1]];
       if constexpr (RELOAD) {
-        a[j] = *(const bf16x8*)(wp + (int64_t)next * 256 + j * 32);
-        __builtin_amdgcn_sched_barrier(0);
+        a[2 * p] = *(const bf16x8*)(wl[0] + (int64_t)next * 256 + p * 64);
+        a[2 * p + 1] = *(const bf16x8*)(wl[1] + (int64_t)next * 256 + p * 64);
       }
+#pragma unroll
+      for (int t = 0; t < MT; ++t) b[1][t] = odd[((2 * p + 1) * MT + t) * WAVE];
+#pragma unroll
+      for (int t = 0; t < MT; ++t) acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(f0, b[0][t], acc[t], 0, 0, 0);
+      if (2 * p + 2 < STEPS) {
+#pragma unroll
+        for (int t = 0; t < MT; ++t) b[0][t] = even[((2 * p + 2) * MT + t) * WAVE];
+      }
+#pragma unroll
+      for (int t = 0; t < MT; ++t) acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(f1, b[1][t], acc[t], 0, 0, 0);
+      if constexpr (RELOAD) __builtin_amdgcn_sched_barrier(0);
     }
   };
   const std::true_type again;
@@ -996,9 +1022,21 @@ static int launch_mid_mt(void* out, int mode, const bf16* a, const bf16* w, int 
     splits = 1, sums = nullptr;
   }
   const dim3 grid((n + 16 * waves - 1) / (16 * waves), splits);
-  if (waves == 4) gemm_bf16_mid_kernel<MT, 4, SWIGLU><<<grid, 4 * 64, 0, s>>>(out, mode, a, w, m, n, k, lda, ldc, sums);
-  else if (waves == 6) gemm_bf16_mid_kernel<MT, 6, SWIGLU><<<grid, 6 * 64, 0, s>>>(out, mode, a, w, m, n, k, lda, ldc, sums);
-  else gemm_bf16_mid_kernel<MT, 8, SWIGLU><<<grid, 8 * 64, 0, s>>>(out, mode, a, w, m, n, k, lda, ldc, sums);
+  // dynamic LDS: two activation buffers of 8 x MT KB and 4 KB a wave; more than 64 KB has to be asked for once
+#define MID_LAUNCH(WV)                                                                                              \
+  do {                                                                                                              \
+    constexpr int bytes = (2 * 8 * MT * 64 + WV * 256) * 16;                                                        \
+    static bool asked = false;                                                                                      \
+    if (!asked) {                                                                                                   \
+      (void)hipFuncSetAttribute((const void*)gemm_bf16_mid_kernel<MT, WV, SWIGLU>, hipFuncAttributeMaxDynamicSharedMemorySize, bytes); \
+      asked = true;                                                                                                 \
+    }                                                                                                               \
+    gemm_bf16_mid_kernel<MT, WV, SWIGLU><<<grid, WV * 64, bytes, s>>>(out, mode, a, w, m, n, k, lda, ldc, sums);    \
+  } while (0)
+  if (waves == 4) MID_LAUNCH(4);
+  else if (waves == 6) MID_LAUNCH(6);
+  else MID_LAUNCH(8);
+#undef MID_LAUNCH
   if (splits > 1 && !keep_sums) {
     const int64_t total = (int64_t)m * (SWIGLU ? n / 2 : n);
     const int blocks = (int)((total + 255) / 256 < 1024 ? (total + 255) / 256 : 1024);
