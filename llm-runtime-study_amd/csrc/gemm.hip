@@ -357,6 +357,9 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_skinny_kernel(
   // conflicts; four steps go through the patch at a time.  No barrier: a wave's LDS instructions
   // execute in order.
   __shared__ bf16x8 patch_all[LINES ? WAVES : 1][2][128];
+  // the activations likewise (8 tokens x 128 bytes an instruction, the second one only if there are more
+  // than 8 tokens), through a patch of their own, two steps at a time
+  __shared__ bf16x8 act_patch_all[LINES ? WAVES : 1][128];
   __shared__ floatx4 partial[WAVES][MT][WAVE];
   __shared__ float sumsq[WAVES][MT][16];
   __shared__ float chain_parts[WAVES * 4][16];   // in_sumsq, added up by WAVES * 4 threads per row
@@ -392,6 +395,15 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_skinny_kernel(
         wl_ok[q][h] = !PARTIAL || row < n_end;                 // PARTIAL: rows past the workgroup's own are the next one's
         wl[q][h] = w + (int64_t)(row < n ? row : n - 1) * k + (lane % 8) * 8;
       }
+    }
+  }
+  const bf16* xl[2];
+  bf16x8* const act_patch = &act_patch_all[LINES ? wave : 0][0];
+  if constexpr (LINES) {
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      const int token = 8 * h + lane / 8;
+      xl[h] = x + (int64_t)(token < m ? token : m - 1) * lda + (lane % 8) * 8;   // tokens past m: the last one's row, never written
     }
   }
   const bf16* xp[MT];
@@ -483,17 +495,28 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_skinny_kernel(
   auto steps_together = [&](int sb, auto count) {
     constexpr int U = decltype(count)::value;
     if constexpr (LINES && U % 4 == 0) {
-      bf16x8 raw[U][RT], b[U][MT];
+      static_assert(MT == 1, "whole-line loads are for one block of tokens");
+      bf16x8 raw[U][RT], rawb[U / 2][2];
+      const bool second = m > 8;                       // the same for the whole grid
 #pragma unroll
       for (int u = 0; u < U; ++u)
 #pragma unroll
         for (int q = 0; q < RT; ++q) raw[u][q] = wl_ok[q][u & 1] ? *(const bf16x8*)(wl[q][u & 1] + (sb + (u & ~1)) * 32) : zero;
 #pragma unroll
-      for (int u = 0; u < U; ++u)
+      for (int p = 0; p < U / 2; ++p) {
+        rawb[p][0] = *(const bf16x8*)(xl[0] + (sb + 2 * p) * 32);
+        rawb[p][1] = second ? *(const bf16x8*)(xl[1] + (sb + 2 * p) * 32) : zero;
+      }
 #pragma unroll
-        for (int t = 0; t < MT; ++t) b[u][t] = load_b(t, sb + u);
+      for (int c4 = 0; c4 < U; c4 += 4) {
+        bf16x8 b[4];
 #pragma unroll
-      for (int c4 = 0; c4 < U; c4 += 4)
+        for (int p = 0; p < 2; ++p) {                  // two steps of activations through their patch at a time
+          act_patch[wr_off[0]] = rawb[c4 / 2 + p][0];
+          act_patch[wr_off[1]] = rawb[c4 / 2 + p][1];
+          b[2 * p] = act_patch[rd_off[0]];
+          b[2 * p + 1] = act_patch[rd_off[1]];
+        }
 #pragma unroll
         for (int q = 0; q < RT; ++q) {
 #pragma unroll
@@ -501,10 +524,10 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_skinny_kernel(
 #pragma unroll
           for (int i = 0; i < 4; ++i) {
             const bf16x8 a = patch[(i >> 1) * 128 + rd_off[i & 1]];
-#pragma unroll
-            for (int t = 0; t < MT; ++t) acc[q][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b[c4 + i][t], acc[q][t], 0, 0, 0);
+            acc[q][0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b[i], acc[q][0], 0, 0, 0);
           }
         }
+      }
       return;
     }
     bf16x8 a[U][RT], b[U][MT];
