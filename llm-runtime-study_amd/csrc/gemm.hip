@@ -350,8 +350,8 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_skinny_kernel(
   // gridDim.y > 1: K is also divided between workgroups; each then leaves its sums in
   // split_sums [gridDim.y, m, n] for gemm_split_finish_kernel instead of writing the output.
   // LINES: the weights come from memory as whole 128-byte lines (a load instruction brings 8 k chunks of
-  // 8 rows; as fragments, 64 bytes of 16 rows, the same kilobyte is twice as many requests, which is what
-  // these kernels are short of) and take their places in the fragments through a patch of LDS of the
+  // 8 rows; as fragments, 64 bytes of 16 rows, the same kilobyte touches 16 cache lines instead of 8, twice
+  // the work for the address and tag units in front of the L1, which is what these kernels are short of) and take their places in the fragments through a patch of LDS of the
   // wave's own: two instructions fill 16 rows x 128 bytes, laid out as two panels (one per k step) of
   // 16 rows x 64 bytes with rows and chunks permuted so that writes and fragment reads meet no bank
   // conflicts; four steps go through the patch at a time.  No barrier: a wave's LDS instructions

@@ -103,6 +103,7 @@ def gemm(args) -> None:
         shapes.append(("lm_head", args.vocab_size, hidden))
     before = ops.skinny_max_m()
     ops.set_skinny_max_m(64)            # time the few-rows kernel up to its own limit, not the caller's
+    ops.gemm_skinny_lines(not args.fragment_loads)
     try:
         for name, n, k in shapes:
             sets = max(2, min(16, int(1.2e9 / (n * k * 2))))
@@ -126,6 +127,7 @@ def gemm(args) -> None:
             del weights
     finally:
         ops.set_skinny_max_m(before)
+        ops.gemm_skinny_lines(True)
 
 
 def memory(args) -> None:
@@ -159,6 +161,7 @@ def main(argv=None) -> int:
     parser.add_argument("--splits", default="1,2,4,8,16", help="attention_decode: workgroups per (token, kv head)")
     parser.add_argument("--form", default="0,1,2", help="attention_decode: 0 four waves, 1 four waves with the next tile on the way, 2 eight waves likewise")
     parser.add_argument("--rows", default="1,8,16,64,2048", help="gemm: numbers of rows")
+    parser.add_argument("--fragment-loads", action="store_true", help="gemm: the few-rows kernel loads weights and activations as MFMA fragments (64 bytes of 16 rows), not as whole lines")
     parser.add_argument("--mid-sweep", default="", help="gemm: also time the kernel for 17..64 rows with 4, 6 and 8 waves at these numbers of K splits")
     parser.add_argument("--megabytes", default="32,200,1200", help="memory: sizes of the buffers read")
     parser.add_argument("--blocks", default="512,2048,8192", help="memory: numbers of workgroups")
