@@ -44,7 +44,7 @@ def parse_args():
     parser.add_argument("--no-points", action="store_true", help="skip the batch 1 and 64 decode points")
     parser.add_argument("--no-graph", action="store_true")
     parser.add_argument("--decode-steps-per-launch", type=int, default=4, help="greedy decode steps run from one graph launch (1: one step a launch)")
-    parser.add_argument("--library-mid-gemm", action="store_true", help="products of 17..64 rows through the vendor library instead of this package's kernel for them")
+    parser.add_argument("--library-mid-gemm", action="store_true", help="products of 17..128 rows through the vendor library instead of this package's kernel for them")
     parser.add_argument("--own-gemm", action="store_true", help="this package's kernel also for products of many rows (default: vendor library)")
     return parser.parse_args()
 

@@ -693,8 +693,8 @@ __global__ void gemm_split_finish_kernel(void* __restrict__ out, int mode, const
   }
 }
 
-// ------------------------------------------------- bf16 kernel for 17..64 rows
-// Between the few-rows kernel (every wave reads its activations from L2 itself) and the many-rows
+// ------------------------------------------------- bf16 kernel for 17..128 rows
+// (MT blocks of 16 tokens: 2, 3, 4, 6 or 8.)  Between the few-rows kernel (every wave reads its activations from L2 itself) and the many-rows
 // kernel (both operands tiled through LDS): the weights are still streamed exactly once, as the MFMA A
 // operand straight from memory into registers, but with several 16-token blocks the activations are
 // as many bytes as the weights of a workgroup, so the waves of a workgroup (each with 16 weight rows
@@ -825,43 +825,78 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_mid_kernel(
   const std::true_type again;
   const std::false_type last;
   // While slice c is multiplied, the weights of slice c + 1 are in registers or on their way and those of
-  // slice c + 2 are asked for as the products of c are issued; the activations of slices c + 2 and c + 3
-  // are on their way into two sets of staging registers (they come from L2, but a wait for them once a
-  // slice would show), and those of slice c + 1 go from registers into the LDS buffer that slice c - 1
-  // has left.
-  if (count > 0) {
-    load_w(slice_at(0), wa);
-    load_acts(slice_at(0), sa);
-  }
-  if (count > 1) {
-    load_w(slice_at(1), wb);
-    load_acts(slice_at(1), sb);
-  }
-  if (count > 0) store_acts(0, sa);
-  if (count > 2) load_acts(slice_at(2), sa);
-  // slice c: after the barrier LDS buffer c & 1 holds it and nobody reads the other buffer any more
-  auto steady = [&](int c, bf16x8 (&a)[STEPS], bf16x8 (&st)[MINE]) {
-    __syncthreads();
-    store_acts((c & 1) ^ 1, st);                       // slice c + 1
-    load_acts(slice_at(c + 3), st);
-    compute(c & 1, a, again, slice_at(c + 2));
-  };
-  auto ending = [&](int c, bf16x8 (&a)[STEPS], bf16x8 (&st)[MINE]) {
-    __syncthreads();
-    if (c + 1 < count) store_acts((c & 1) ^ 1, st);
-    if (c + 3 < count) load_acts(slice_at(c + 3), st);
-    if (c + 2 < count) compute(c & 1, a, again, slice_at(c + 2));
-    else compute(c & 1, a, last, 0);
-  };
+  // slice c + 2 are asked for as the products of c are issued; the activations of slice c + 1 go from
+  // staging registers into the LDS buffer that slice c - 1 has left, and those of the slices after it are on
+  // their way into the staging registers: two sets of them in turn (slices c + 2 and c + 3) up to 64 rows, one
+  // set (slice c + 2) beyond, where registers are short.
   int c = 0;
-  for (; c + 4 < count; c += 2) {            // no branch inside: slices up to c + 4 exist
-    steady(c, wa, sb);
-    steady(c + 1, wb, sa);
-  }
-  for (; c < count; c += 2) {                // the last one to four slices
-    ending(c, wa, sb);
-    if (c + 1 >= count) break;
-    ending(c + 1, wb, sa);
+  if constexpr (MT <= 4) {
+    if (count > 0) {
+      load_w(slice_at(0), wa);
+      load_acts(slice_at(0), sa);
+    }
+    if (count > 1) {
+      load_w(slice_at(1), wb);
+      load_acts(slice_at(1), sb);
+    }
+    if (count > 0) store_acts(0, sa);
+    if (count > 2) load_acts(slice_at(2), sa);
+    // slice c: after the barrier LDS buffer c & 1 holds it and nobody reads the other buffer any more
+    auto steady = [&](int c, bf16x8 (&a)[STEPS], bf16x8 (&st)[MINE]) {
+      __syncthreads();
+      store_acts((c & 1) ^ 1, st);                       // slice c + 1
+      load_acts(slice_at(c + 3), st);
+      compute(c & 1, a, again, slice_at(c + 2));
+    };
+    auto ending = [&](int c, bf16x8 (&a)[STEPS], bf16x8 (&st)[MINE]) {
+      __syncthreads();
+      if (c + 1 < count) store_acts((c & 1) ^ 1, st);
+      if (c + 3 < count) load_acts(slice_at(c + 3), st);
+      if (c + 2 < count) compute(c & 1, a, again, slice_at(c + 2));
+      else compute(c & 1, a, last, 0);
+    };
+    for (; c + 4 < count; c += 2) {            // no branch inside: slices up to c + 4 exist
+      steady(c, wa, sb);
+      steady(c + 1, wb, sa);
+    }
+    for (; c < count; c += 2) {                // the last one to four slices
+      ending(c, wa, sb);
+      if (c + 1 >= count) break;
+      ending(c + 1, wb, sa);
+    }
+  } else {
+    if (count > 0) {
+      load_w(slice_at(0), wa);
+      load_acts(slice_at(0), sa);
+    }
+    if (count > 1) load_w(slice_at(1), wb);
+    if (count > 0) store_acts(0, sa);
+    if (count > 1) load_acts(slice_at(1), sa);
+    auto steady = [&](int c, bf16x8 (&a)[STEPS]) {
+      __syncthreads();
+      store_acts((c & 1) ^ 1, sa);                       // slice c + 1
+      load_acts(slice_at(c + 2), sa);
+      compute(c & 1, a, again, slice_at(c + 2));
+    };
+    auto ending = [&](int c, bf16x8 (&a)[STEPS]) {
+      __syncthreads();
+      if (c + 1 < count) store_acts((c & 1) ^ 1, sa);
+      if (c + 2 < count) {
+        load_acts(slice_at(c + 2), sa);
+        compute(c & 1, a, again, slice_at(c + 2));
+      } else {
+        compute(c & 1, a, last, 0);
+      }
+    };
+    for (; c + 3 < count; c += 2) {            // no branch inside: slices up to c + 3 exist
+      steady(c, wa);
+      steady(c + 1, wb);
+    }
+    for (; c < count; c += 2) {                // the last one to three slices
+      ending(c, wa);
+      if (c + 1 >= count) break;
+      ending(c + 1, wb);
+    }
   }
   // accumulator layout: token = t * 16 + lane % 16, weight rows row0 + 4 * (lane / 16) + 0..3
   const int gn = row0 + 4 * g;
@@ -960,7 +995,7 @@ static float* split_sums_buffer() {
   return g_split_sums;
 }
 
-// The kernel for 17..64 rows: which of its workgroup shapes and how many K splits.  0 = chosen here:
+// The kernel for 17..128 rows: which of its workgroup shapes and how many K splits.  0 = chosen here:
 // the shape and split that fill a whole multiple of the compute units best, then the fewest splits.
 static int g_mid_waves = 0, g_mid_splits = 0, g_mid_enabled = 1;
 LRS_API int lrs_compute_units();
@@ -1026,7 +1061,7 @@ static void choose_mid_shape(int n, int k, int& waves, int& splits) {
   waves = pick->waves, splits = pick->splits;
 }
 
-// The shape the kernel for 17..64 rows takes for a matrix of n rows and k columns (for tests and reports).
+// The shape the kernel for 17..128 rows takes for a matrix of n rows and k columns (for tests and reports).
 LRS_API int lrs_gemm_mid_shape(int n, int k, int* waves, int* splits) {
   LRS_REQUIRE(n > 0 && k > 0 && k % 256 == 0 && waves && splits, "gemm_mid_shape: needs n > 0 and K %% 256 == 0, got n=%d k=%d", n, k);
   choose_mid_shape(n, k, *waves, *splits);
@@ -1072,7 +1107,9 @@ template <bool SWIGLU>
 static int launch_mid(void* out, int mode, const bf16* a, const bf16* w, int m, int n, int k, int lda, int ldc, hipStream_t s, bool keep_sums = false) {
   if (m <= 32) return launch_mid_mt<2, SWIGLU>(out, mode, a, w, m, n, k, lda, ldc, s, keep_sums);
   if (m <= 48) return launch_mid_mt<3, SWIGLU>(out, mode, a, w, m, n, k, lda, ldc, s, keep_sums);
-  return launch_mid_mt<4, SWIGLU>(out, mode, a, w, m, n, k, lda, ldc, s, keep_sums);
+  if (m <= 64) return launch_mid_mt<4, SWIGLU>(out, mode, a, w, m, n, k, lda, ldc, s, keep_sums);
+  if (m <= 96) return launch_mid_mt<6, SWIGLU>(out, mode, a, w, m, n, k, lda, ldc, s, keep_sums);
+  return launch_mid_mt<8, SWIGLU>(out, mode, a, w, m, n, k, lda, ldc, s, keep_sums);
 }
 
 template <int MT, bool NORM, bool SWIGLU>
@@ -1125,8 +1162,8 @@ LRS_API int lrs_gemm_prepare() {
 }
 
 // Largest M for which callers should use the few-rows kernel (and with it the fused RMSNorm input).
-// The kernel itself takes up to 64 rows, but measured on MI355X the vendor library's products are
-// faster from 17 rows on, so callers that may use the library send larger products there.
+// The kernel itself takes up to 64 rows, but from 17 rows on the kernel for 17..128 rows (or, where a
+// shape does not suit it, the vendor library) is faster, so callers send larger products there.
 static int g_skinny_max_m = 16;
 LRS_API int lrs_gemm_skinny_max_m() { return g_skinny_max_m; }
 LRS_API int lrs_gemm_set_skinny_max_m(int m) {
@@ -1174,14 +1211,14 @@ LRS_API int lrs_gemm_norm_chain(void* out, int mode, const void* a, const void* 
 extern "C" int lrs_split_add_rmsnorm(void* out, int out_dtype, float* x, const float* sums, int splits, const void* weight,
                                      int w_dtype, int n_rows, int hidden, float eps, void* stream);
 
-// A product of 17..64 rows that adds into the float32 residual stream, with the RMSNorm that follows:
+// A product of 17..128 rows that adds into the float32 residual stream, with the RMSNorm that follows:
 // residual [M, N] += a [M, K] w[N, K]^T, then normed [M, N] = RMSNorm(residual) with norm_weight and eps.
 // The sums of the product's K splits go straight into the kernel that adds and normalises: one launch
 // less and no rounding of the product to bf16 on the way.
 LRS_API int lrs_gemm_mid_add_rmsnorm(void* normed, int normed_dtype, float* residual, const void* a, const void* w,
                                      const void* norm_weight, int norm_weight_dtype, int m, int n, int k, int lda,
                                      float eps, void* stream) {
-  LRS_REQUIRE(m > 16 && m <= 64 && n > 0 && k > 0, "gemm_mid_add_rmsnorm: takes 17..64 rows, got m=%d n=%d k=%d", m, n, k);
+  LRS_REQUIRE(m > 16 && m <= 128 && n > 0 && k > 0, "gemm_mid_add_rmsnorm: takes 17..128 rows, got m=%d n=%d k=%d", m, n, k);
   LRS_REQUIRE(k % 256 == 0 && n % 16 == 0 && lda >= k && lda % 8 == 0 && ((uintptr_t)a % 16 == 0) && ((uintptr_t)w % 16 == 0) && ((uintptr_t)residual % 16 == 0),
               "gemm_mid_add_rmsnorm: needs K %% 256 == 0, N %% 16 == 0 and 16-byte aligned rows (n=%d k=%d lda=%d)", n, k, lda);
   LRS_REQUIRE(eps > 0.f, "gemm_mid_add_rmsnorm: eps must be positive");
@@ -1218,11 +1255,13 @@ LRS_API int lrs_gemm(void* out, int mode, const void* a, const void* w, const vo
     gemm_tiled_kernel<float><<<grid, 256, 0, s>>>(out, mode, (const float*)a, (const float*)w,
                                                   (const float*)bias, m, n, k, lda, ldc);
   } else if (dtype == LRS_BF16) {
-    if (aligned && m <= 64) {
+    const bool mid = aligned && m > 16 && m <= 128 && !normed && !bias && g_mid_enabled && k % 256 == 0 && n % 16 == 0 && ldc % 4 == 0 &&
+                     (uintptr_t)out % 16 == 0;
+    if (aligned && (m <= 64 || mid)) {
       const bf16 *wp = (const bf16*)w, *bp = (const bf16*)bias;
       const NormInput norm{(const float*)a, rows, norm_weight, norm_weight_dtype == LRS_F32, eps};
       const bf16* ap = normed ? nullptr : (const bf16*)a;
-      if (m > 16 && !normed && !bias && g_mid_enabled && k % 256 == 0 && n % 16 == 0 && ldc % 4 == 0 && (uintptr_t)out % 16 == 0) {
+      if (mid) {
         if (swiglu) launch_mid<true>(out, mode, ap, wp, m, n, k, lda, ldc, s);
         else launch_mid<false>(out, mode, ap, wp, m, n, k, lda, ldc, s);
       } else if (normed && swiglu) launch_skinny_m<true, true>(out, mode, ap, norm, wp, bp, m, n, k, lda, ldc, s);

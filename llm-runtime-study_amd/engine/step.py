@@ -381,7 +381,7 @@ class ModelRunner:
 
     # ------------------------------------------------- several decode steps, one launch
     MAX_DECODE_STEPS = 8
-    GRAPH_ROWS = 64     # largest padded batch whose bfloat16 step is captured
+    GRAPH_ROWS = 128    # largest padded batch whose bfloat16 step is captured
 
     def can_decode_steps(self, entries: Sequence[StepEntry]) -> bool:
         """Whether decode_steps() takes these entries: one token each, and a graph for their number."""
@@ -525,8 +525,8 @@ class ModelRunner:
         while bucket < len(entries):
             bucket *= 2
         bucket = min(bucket, self.max_requests)
-        # A bfloat16 graph of up to 64 rows holds this package's kernels (the few-rows kernels, then the
-        # kernel for 17..64 rows); where a shape does not suit that kernel (K no multiple of 256) and the runner
+        # A bfloat16 graph of up to 128 rows holds this package's kernels (the few-rows kernels, then the
+        # kernel for 17..128 rows); where a shape does not suit that kernel (K no multiple of 256) and the runner
         # may use the vendor library, its products are captured with them.
         most = max(ops.skinny_max_m(), self.GRAPH_ROWS) if self.dtype == torch.bfloat16 else ops.skinny_max_m()
         return bucket if bucket <= min(self.max_step_tokens, most) else 0

@@ -112,7 +112,7 @@ def gemm(args) -> None:
                 x = torch.randn(rows, k, device="cuda", dtype=torch.bfloat16)
                 out = torch.empty(rows, n, device="cuda", dtype=torch.bfloat16)
                 variants = [("own", 0, 0), ("library", 0, 0)]
-                if args.mid_sweep and 16 < rows <= 64:
+                if args.mid_sweep and 16 < rows <= 128:
                     variants = [(f"mid w{wv} s{sp}", wv, sp) for wv in (4, 6, 8) for sp in _ints(args.mid_sweep)] + variants
                 for which, wv, sp in variants:
                     if which == "library":
@@ -162,7 +162,7 @@ def main(argv=None) -> int:
     parser.add_argument("--form", default="0,1,2", help="attention_decode: 0 four waves, 1 four waves with the next tile on the way, 2 eight waves likewise")
     parser.add_argument("--rows", default="1,8,16,64,2048", help="gemm: numbers of rows")
     parser.add_argument("--fragment-loads", action="store_true", help="gemm: the few-rows kernel loads weights and activations as MFMA fragments (64 bytes of 16 rows), not as whole lines")
-    parser.add_argument("--mid-sweep", default="", help="gemm: also time the kernel for 17..64 rows with 4, 6 and 8 waves at these numbers of K splits")
+    parser.add_argument("--mid-sweep", default="", help="gemm: also time the kernel for 17..128 rows with 4, 6 and 8 waves at these numbers of K splits")
     parser.add_argument("--megabytes", default="32,200,1200", help="memory: sizes of the buffers read")
     parser.add_argument("--blocks", default="512,2048,8192", help="memory: numbers of workgroups")
     parser.add_argument("--repeats", type=int, default=20)

@@ -289,7 +289,7 @@ def skinny_max_m() -> int:
 
 
 def gemm_mid_tune(enabled: bool = True, waves: int = 0, splits: int = 0) -> None:
-    """Whether bf16 products of 17..64 rows take this package's kernel for them, and (for measurements)
+    """Whether bf16 products of 17..128 rows take this package's kernel for them, and (for measurements)
     its workgroup shape (4, 6 or 8 waves) and number of K splits; 0 lets the library choose."""
     _check(library().lrs_gemm_mid_tune(int(bool(enabled)), waves, splits))
 
@@ -300,7 +300,7 @@ def gemm_skinny_lines(enabled: bool) -> None:
 
 
 def gemm_mid_shape(n: int, k: int) -> tuple[int, int]:
-    """(waves a workgroup, K splits) the kernel for 17..64 rows takes for a weight matrix [n, k]."""
+    """(waves a workgroup, K splits) the kernel for 17..128 rows takes for a weight matrix [n, k]."""
     import ctypes
     waves, splits = ctypes.c_int(0), ctypes.c_int(0)
     _check(library().lrs_gemm_mid_shape(n, k, ctypes.addressof(waves), ctypes.addressof(splits)))
@@ -311,26 +311,27 @@ def gemm_mid_enabled() -> bool:
     return bool(library().lrs_gemm_mid_enabled())
 
 
-# Rows up to which callers that may use the vendor library take this package's kernel for 17..64 rows instead.
+# Rows up to which callers that may use the vendor library take this package's kernel for 17..128 rows instead.
 # Measured on MI355X in whole decode steps (Qwen3-8B shape): 4-6 % faster than the library's products at
-# batches of 24, 32, 48 and 64.
-MID_ROWS_PREFERRED = 64
+# batches of 24..64; at 128 rows a layer's four products take 141 us against 169 us (and a separate gated
+# activation), only the LM head is slower (320 against 279 us).
+MID_ROWS_PREFERRED = 128
 
 
-def gemm_mid_takes(dtype: torch.dtype, m: int, n: int, k: int, most: int = 64) -> bool:
-    """Whether a product of m rows (at most `most`) can go to the kernel for 17..64 rows (weights streamed
+def gemm_mid_takes(dtype: torch.dtype, m: int, n: int, k: int, most: int = 128) -> bool:
+    """Whether a product of m rows (at most `most`) can go to the kernel for 17..128 rows (weights streamed
     once, activations shared through LDS), which also writes the gated activation itself."""
-    return dtype == torch.bfloat16 and 16 < m <= min(most, 64) and k % 256 == 0 and n % 16 == 0 and gemm_mid_enabled()
+    return dtype == torch.bfloat16 and 16 < m <= min(most, 128) and k % 256 == 0 and n % 16 == 0 and gemm_mid_enabled()
 
 
 def gemm_mid_add_rmsnorm(normed: torch.Tensor, residual: torch.Tensor, a: torch.Tensor, w: torch.Tensor,
                          norm_weight: torch.Tensor, eps: float) -> None:
     """residual (float32 [M, N]) += a @ w.T, then normed = RMSNorm(residual) with norm_weight: the product
-    of 17..64 bf16 rows, its residual add and the norm that follows, the sums of the product's K splits going
+    of 17..128 bf16 rows, its residual add and the norm that follows, the sums of the product's K splits going
     straight into the kernel that adds and normalises."""
     m, k = a.shape
     n = w.shape[0]
-    _need(gemm_mid_takes(w.dtype, m, n, k) and a.dtype == torch.bfloat16, "gemm_mid_add_rmsnorm: takes bf16 products of 17..64 rows, K % 256 == 0, N % 16 == 0")
+    _need(gemm_mid_takes(w.dtype, m, n, k) and a.dtype == torch.bfloat16, "gemm_mid_add_rmsnorm: takes bf16 products of 17..128 rows, K % 256 == 0, N % 16 == 0")
     _need(w.dim() == 2 and w.is_contiguous() and w.shape[1] == k, f"gemm_mid_add_rmsnorm: weight must be contiguous [N, {k}]")
     _need(residual.dtype == torch.float32 and residual.is_contiguous() and residual.shape == (m, n), f"gemm_mid_add_rmsnorm: residual must be contiguous float32 [{m}, {n}]")
     _need(normed.is_contiguous() and normed.shape == (m, n), f"gemm_mid_add_rmsnorm: normed must be contiguous [{m}, {n}]")

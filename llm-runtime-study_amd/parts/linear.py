@@ -85,10 +85,10 @@ def linear(ctx, out, x, weight, bias=None, accumulate: bool = False, swiglu: boo
     ScaledRows (begun by the few-rows kernel, finished by the next `linear()`) or as a plain
     tensor (after a library product); else None: the caller then runs the norm as usual.
 
-    Products of more than 64 rows in bfloat16 go to the vendor's matrix library (as the reference's
+    Products of more than 128 rows in bfloat16 go to the vendor's matrix library (as the reference's
     nn.Linear does) when the step allows it (`ctx.library_gemm`); its result then reaches the
     residual stream or the gated activation through one more small kernel.  Everything else,
-    and every float32 product, runs in this package's own kernels (17..64 rows: the kernel that
+    and every float32 product, runs in this package's own kernels (17..128 rows: the kernel that
     shares the activations through LDS, when the shape suits it: K a multiple of 256)."""
     scaled = None
     if isinstance(x, ScaledRows):
@@ -114,7 +114,7 @@ def linear(ctx, out, x, weight, bias=None, accumulate: bool = False, swiglu: boo
     if (getattr(ctx, "library_gemm", False) and weight.dtype == torch.bfloat16 and x.dtype == torch.bfloat16 and m > ops.skinny_max_m()
             and bias is None and x.is_contiguous() and (accumulate or (out.dtype in (torch.bfloat16, torch.float32) and out.is_contiguous()))
             and not (swiglu and out.dtype != torch.bfloat16)):
-        own = ops.gemm_mid_takes(weight.dtype, m, n, weight.shape[1], ops.MID_ROWS_PREFERRED)   # 17..64 rows: this package's kernel, not the library's
+        own = ops.gemm_mid_takes(weight.dtype, m, n, weight.shape[1], ops.MID_ROWS_PREFERRED)   # 17..128 rows: this package's kernel, not the library's
         if own and not accumulate:
             ops.gemm(out, x, weight, None, False, swiglu)
             return None

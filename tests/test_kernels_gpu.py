@@ -237,7 +237,7 @@ def test_gemm(ops, dtype, m, n, k, mode):
         torch.testing.assert_close(out.cpu().double(), want, rtol=1e-4, atol=1e-4)
 
 
-@pytest.mark.parametrize("m", [17, 32, 40, 48, 49, 64])
+@pytest.mark.parametrize("m", [17, 32, 40, 48, 49, 64, 65, 96, 100, 128])
 @pytest.mark.parametrize("n,k", [(64, 256), (208, 512), (4096, 1024), (6144, 4096), (1040, 3328)])
 @pytest.mark.parametrize("waves,splits", [(0, 0), (4, 1), (6, 2), (8, 3), (4, 8)])
 def test_gemm_of_17_to_64_rows(ops, m, n, k, waves, splits):
@@ -269,7 +269,7 @@ def test_gemm_of_17_to_64_rows(ops, m, n, k, waves, splits):
 
 
 @pytest.mark.parametrize("w_dtype", DTYPES)
-@pytest.mark.parametrize("m,n,k,splits", [(17, 64, 256, 0), (40, 208, 1024, 2), (64, 4096, 4096, 0), (33, 1040, 3328, 3), (48, 5120, 512, 1)])
+@pytest.mark.parametrize("m,n,k,splits", [(17, 64, 256, 0), (40, 208, 1024, 2), (64, 4096, 4096, 0), (33, 1040, 3328, 3), (48, 5120, 512, 1), (90, 208, 1024, 2), (128, 4096, 4096, 0)])
 def test_gemm_of_17_to_64_rows_with_residual_add_and_norm(ops, w_dtype, m, n, k, splits):
     """residual += x W^T and the RMSNorm of the new residual, the K splits' sums added inside the norm kernel."""
     g = torch.Generator().manual_seed(m + n + k)
