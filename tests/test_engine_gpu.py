@@ -316,6 +316,62 @@ def test_graphs_of_large_batches_hold_library_products(folders):
     graphed.drop_graphs()
 
 
+def test_graphs_of_up_to_128_rows_hold_this_packages_kernels(tmp_path):
+    """A model whose matrices suit the kernel for 17..128 rows (every K a multiple of 256): batches of 40 to 100
+    requests run as graphs of 64 and 128 rows of this package's kernels alone, and every replay gives the
+    logits of the same step run eagerly, bit for bit; the logits agree with the float32 path."""
+    from llm_runtime_study_amd.cache import CacheManager
+    from llm_runtime_study_amd.config import config_from_dict
+    from llm_runtime_study_amd.engine.loading import load_model
+    from llm_runtime_study_amd.engine.step import ModelRunner, StepEntry
+    from llm_runtime_study_amd.kernels import ops
+    from llm_runtime_study_amd.weights import write_model_dir
+
+    raw = dict(TINY_C, vocab_size=352, hidden_size=256, intermediate_size=512, num_attention_heads=4, num_key_value_heads=2, head_dim=64)
+    write_model_dir(config_from_dict(raw), seed=41, model_dir=tmp_path, init="scaled")
+    device = torch.device("cuda", 0)
+    _, model = load_model(tmp_path, torch.bfloat16, device)
+    _, model32 = load_model(tmp_path, torch.float32, device)
+    for n, k in ((4 * 64 + 2 * 2 * 64, 256), (256, 256), (1024, 256), (256, 512), (352, 256)):
+        assert ops.gemm_mid_takes(torch.bfloat16, 100, n, k)
+    rng = np.random.default_rng(32)
+
+    def make(use_graph, m=model, dtype=torch.bfloat16):
+        cache = CacheManager(m.cache_needs(), page_size=16, num_pages=500, max_requests=128, max_seq_len=96, dtype=dtype, device=device)
+        return ModelRunner(m, cache, max_step_tokens=256, dtype=dtype, device=device, use_graph=use_graph, library_gemm=False)
+
+    eager, graphed, exact = make(False), make(True), make(False, model32, torch.float32)
+    live = {}
+
+    def admit(index):
+        prompt = rng.integers(0, raw["vocab_size"], int(rng.integers(2, 30))).tolist()
+        caches = (eager.cache.admit(index), graphed.cache.admit(index), exact.cache.admit(index))
+        a = eager.step([StepEntry(caches[0], prompt, [len(prompt) - 1])]).clone()
+        b = graphed.step([StepEntry(caches[1], prompt, [len(prompt) - 1])]).clone()
+        exact.step([StepEntry(caches[2], prompt, [])])
+        assert torch.equal(a, b)
+        live[index] = (caches, int(a[0].argmax()))
+
+    with torch.cuda.stream(torch.cuda.Stream(device)):
+        for index in range(40):
+            admit(index)
+        for step in range(12):
+            for extra in range(6 if step < 10 else 0):                 # 40 -> 100 requests: buckets 64 and 128
+                admit(1000 + step * 10 + extra)
+            order = sorted(live)
+            a = eager.step([StepEntry(live[i][0][0], [live[i][1]], [0]) for i in order]).clone()
+            b = graphed.step([StepEntry(live[i][0][1], [live[i][1]], [0]) for i in order]).clone()
+            c = exact.step([StepEntry(live[i][0][2], [live[i][1]], [0]) for i in order]).clone()
+            torch.cuda.synchronize()
+            assert torch.equal(a, b), f"step {step} with {len(order)} requests: graph replay differs from the eager step"
+            error = (a - c).norm() / c.norm()
+            assert error < 0.03, f"step {step}: bfloat16 logits are {float(error):.3f} of the float32 logits away"
+            for row, i in enumerate(order):
+                live[i] = (live[i][0], int(c[row].argmax()))
+    assert graphed.graph_replays == 12 and {key[0] for key in graphed._graphs} == {64, 128}
+    graphed.drop_graphs()
+
+
 def test_sampled_tokens_do_not_depend_on_steps_per_launch(folders):
     """Seeded draws with top-k and top-p, one request greedy beside them: four decode steps from one
     launch (the device filters, draws and counts the draws itself) give the tokens of single steps."""
