@@ -7,8 +7,11 @@ QWEN3_8B = {
     "hidden_act": "silu", "attention_bias": False, "attention_dropout": 0.0, "tie_word_embeddings": False,
     "torch_dtype": "bfloat16", "bos_token_id": 151643, "eos_token_id": 151645,
 }
-# the two larger dense models of the family
+# the other dense models of the family (the reference's own published figures are for the smallest)
 SHAPES = {
+    "0.6b": dict(QWEN3_8B, hidden_size=1024, intermediate_size=3072, num_hidden_layers=28, num_attention_heads=16, tie_word_embeddings=True),
+    "1.7b": dict(QWEN3_8B, hidden_size=2048, intermediate_size=6144, num_hidden_layers=28, num_attention_heads=16, tie_word_embeddings=True),
+    "4b": dict(QWEN3_8B, hidden_size=2560, intermediate_size=9728, num_hidden_layers=36, num_attention_heads=32, tie_word_embeddings=True),
     "8b": QWEN3_8B,
     "14b": dict(QWEN3_8B, hidden_size=5120, intermediate_size=17408, num_hidden_layers=40, num_attention_heads=40),
     "32b": dict(QWEN3_8B, hidden_size=5120, intermediate_size=25600, num_hidden_layers=64, num_attention_heads=64),

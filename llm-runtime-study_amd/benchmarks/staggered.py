@@ -21,6 +21,8 @@ import statistics
 import sys
 import time
 
+from .shapes import SHAPES
+
 
 def percentile(values, fraction: float) -> float:
     """Nearest-rank percentile, as the reference takes it (benchmarks/common.py:91-95)."""
@@ -41,7 +43,7 @@ def span(text: str) -> tuple[int, int]:
 
 def build_parser() -> argparse.ArgumentParser:
     parser = argparse.ArgumentParser(prog="staggered", description=__doc__.splitlines()[0])
-    parser.add_argument("--shape", choices=("8b", "14b", "32b"), default="14b")
+    parser.add_argument("--shape", choices=tuple(SHAPES), default="14b")
     parser.add_argument("--layers", type=int, default=None, help="fewer layers than the shape has (reported)")
     parser.add_argument("--requests", type=int, default=64)
     parser.add_argument("--interval-ms", type=float, default=50.0)
@@ -112,7 +114,6 @@ def main(argv=None) -> int:
 
     from .. import Engine
     from ..config import config_from_dict
-    from .shapes import SHAPES
 
     raw = dict(SHAPES[args.shape])
     full_layers = raw["num_hidden_layers"]

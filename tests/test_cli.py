@@ -112,7 +112,7 @@ def test_bench_counts_the_flops_and_the_lead_of_early_requests():
     # eight prompts of 2,048 tokens read one a step: the first request is seven tokens ahead of the last
     assert bench.decode_lead(8, 2048, 2048) == 7
     assert bench.decode_lead(8, 32768, 2048) == 7 * 16 and bench.decode_lead(1, 5000, 2048) == 0
-    assert set(bench.SHAPES) == {"8b", "14b", "32b"} and bench.SHAPES["32b"]["num_hidden_layers"] == 64
+    assert set(bench.SHAPES) == {"0.6b", "1.7b", "4b", "8b", "14b", "32b"} and bench.SHAPES["32b"]["num_hidden_layers"] == 64
 
 
 def test_staggered_benchmark_percentiles_and_drawn_requests():
