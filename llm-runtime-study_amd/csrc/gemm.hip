@@ -704,10 +704,19 @@ __global__ void gemm_split_finish_kernel(void* __restrict__ out, int mode, const
 // meet no bank conflicts (see below).  gridDim.y > 1 divides K between
 // workgroups; with split_sums given every workgroup leaves its sums there ([gridDim.y, m, n]) for a
 // kernel that adds them up (gemm_split_finish_kernel, or the residual add and norm that follow).  K % 256 == 0.
+// The input may be an RMSNorm that the kernel before began (see NormChain): x = bf16(h * norm weight) and partial
+// sums of h^2 per row, sumsq [parts, m]; row r of the result (of every K split's sums alike: the factor is
+// constant along K) is then multiplied by rsqrt(sum_p sumsq[p, r] / K + eps).
+struct MidScale {
+  const float* sumsq;   // null: the input is what it is
+  int parts;
+  float eps;
+};
+
 template <int MT, int WAVES, bool SWIGLU>
 __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_mid_kernel(
     void* __restrict__ out, int mode, const bf16* __restrict__ x, const bf16* __restrict__ w,
-    int m, int n, int k, int lda, int ldc, float* __restrict__ split_sums) {
+    int m, int n, int k, int lda, int ldc, float* __restrict__ split_sums, MidScale scale) {
   constexpr int STEPS = 8;                         // k steps of 32 in a slice
   constexpr int FRAGS = STEPS * MT;                // activation fragments of a slice
   constexpr int MINE = (FRAGS + WAVES - 1) / WAVES;  // of which a wave brings this many
@@ -767,6 +776,14 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_mid_kernel(
     const int tok = oct * 8 + lane / 8, chunk = line * 8 + lane % 8;
     xp[i] = x + (int64_t)(tok < m ? tok : m - 1) * lda + chunk * 8;
     spot[i] = lds + place(chunk / 4, tok / 16, tok % 16, chunk % 4);
+  }
+  // the factors of a norm begun before this product: one thread a token adds up the parts now (the loads run
+  // beside the weights') and keeps the factor; after the last slice they go through LDS to the lanes that need them
+  float my_scale = 1.f;
+  if (scale.sumsq && tid < m) {
+    float q = 0.f;
+    for (int p = 0; p < scale.parts; ++p) q += scale.sumsq[(int64_t)p * m + tid];
+    my_scale = 1.0f / sqrtf(q / (float)k + scale.eps);
   }
   floatx4 acc[MT];
 #pragma unroll
@@ -899,6 +916,14 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_mid_kernel(
     }
   }
   // accumulator layout: token = t * 16 + lane % 16, weight rows row0 + 4 * (lane / 16) + 0..3
+  if (scale.sumsq) {
+    float* const row_scales = (float*)mid_lds;     // the activation buffers have done their work
+    __syncthreads();
+    if (tid < m) row_scales[tid] = my_scale;
+    __syncthreads();
+#pragma unroll
+    for (int t = 0; t < MT; ++t) acc[t] *= row_scales[t * 16 + r < m ? t * 16 + r : 0];
+  }
   const int gn = row0 + 4 * g;
   if (split_sums) {
 #pragma unroll
@@ -1071,7 +1096,7 @@ LRS_API int lrs_gemm_mid_shape(int n, int k, int* waves, int* splits) {
 // keep_sums: the sums of the K splits (of the one split, if K is not divided) stay in the split buffer for
 // the caller's own finishing kernel; returns their number, or 0 if the buffer cannot hold them.
 template <int MT, bool SWIGLU>
-static int launch_mid_mt(void* out, int mode, const bf16* a, const bf16* w, int m, int n, int k, int lda, int ldc, hipStream_t s, bool keep_sums) {
+static int launch_mid_mt(void* out, int mode, const bf16* a, const bf16* w, int m, int n, int k, int lda, int ldc, hipStream_t s, bool keep_sums, MidScale scale) {
   int waves = 4, splits = 1;
   choose_mid_shape(n, k, waves, splits);
   float* sums = splits > 1 || keep_sums ? split_sums_buffer() : nullptr;
@@ -1089,7 +1114,7 @@ static int launch_mid_mt(void* out, int mode, const bf16* a, const bf16* w, int 
       (void)hipFuncSetAttribute((const void*)gemm_bf16_mid_kernel<MT, WV, SWIGLU>, hipFuncAttributeMaxDynamicSharedMemorySize, bytes); \
       asked = true;                                                                                                 \
     }                                                                                                               \
-    gemm_bf16_mid_kernel<MT, WV, SWIGLU><<<grid, WV * 64, bytes, s>>>(out, mode, a, w, m, n, k, lda, ldc, sums);    \
+    gemm_bf16_mid_kernel<MT, WV, SWIGLU><<<grid, WV * 64, bytes, s>>>(out, mode, a, w, m, n, k, lda, ldc, sums, scale);    \
   } while (0)
   if (waves == 4) MID_LAUNCH(4);
   else if (waves == 6) MID_LAUNCH(6);
@@ -1104,12 +1129,13 @@ static int launch_mid_mt(void* out, int mode, const bf16* a, const bf16* w, int 
 }
 
 template <bool SWIGLU>
-static int launch_mid(void* out, int mode, const bf16* a, const bf16* w, int m, int n, int k, int lda, int ldc, hipStream_t s, bool keep_sums = false) {
-  if (m <= 32) return launch_mid_mt<2, SWIGLU>(out, mode, a, w, m, n, k, lda, ldc, s, keep_sums);
-  if (m <= 48) return launch_mid_mt<3, SWIGLU>(out, mode, a, w, m, n, k, lda, ldc, s, keep_sums);
-  if (m <= 64) return launch_mid_mt<4, SWIGLU>(out, mode, a, w, m, n, k, lda, ldc, s, keep_sums);
-  if (m <= 96) return launch_mid_mt<6, SWIGLU>(out, mode, a, w, m, n, k, lda, ldc, s, keep_sums);
-  return launch_mid_mt<8, SWIGLU>(out, mode, a, w, m, n, k, lda, ldc, s, keep_sums);
+static int launch_mid(void* out, int mode, const bf16* a, const bf16* w, int m, int n, int k, int lda, int ldc, hipStream_t s, bool keep_sums = false,
+                      MidScale scale = MidScale{nullptr, 0, 0.f}) {
+  if (m <= 32) return launch_mid_mt<2, SWIGLU>(out, mode, a, w, m, n, k, lda, ldc, s, keep_sums, scale);
+  if (m <= 48) return launch_mid_mt<3, SWIGLU>(out, mode, a, w, m, n, k, lda, ldc, s, keep_sums, scale);
+  if (m <= 64) return launch_mid_mt<4, SWIGLU>(out, mode, a, w, m, n, k, lda, ldc, s, keep_sums, scale);
+  if (m <= 96) return launch_mid_mt<6, SWIGLU>(out, mode, a, w, m, n, k, lda, ldc, s, keep_sums, scale);
+  return launch_mid_mt<8, SWIGLU>(out, mode, a, w, m, n, k, lda, ldc, s, keep_sums, scale);
 }
 
 template <int MT, bool NORM, bool SWIGLU>
@@ -1226,6 +1252,47 @@ LRS_API int lrs_gemm_mid_add_rmsnorm(void* normed, int normed_dtype, float* resi
   LRS_REQUIRE(splits > 0, "gemm_mid_add_rmsnorm: the buffer for the sums of the K splits cannot hold %d x %d values", m, n);
   if (int rc = lrs_check_launch("gemm_mid_add_rmsnorm")) return rc;
   return lrs_split_add_rmsnorm(normed, normed_dtype, residual, split_sums_buffer(), splits, norm_weight, norm_weight_dtype, m, n, eps, stream);
+}
+
+static bool mid_shape_ok(const void* a, const void* w, int m, int n, int k, int lda) {
+  return m > 16 && m <= 128 && n > 0 && k > 0 && k % 256 == 0 && n % 16 == 0 && lda >= k && lda % 8 == 0 && ((uintptr_t)a % 16 == 0) &&
+         ((uintptr_t)w % 16 == 0);
+}
+
+// The product of 17..128 rows whose input is a norm that the kernel before began: a = bf16(h * norm weight)
+// [M, K], in_sumsq [in_parts, M] partial sums of h^2; row r of the result is multiplied by
+// rsqrt(sum_p in_sumsq[p, r] / K + in_eps).  swiglu as in lrs_gemm.
+LRS_API int lrs_gemm_mid_scaled(void* out, int mode, const void* a, const void* w, int m, int n, int k, int lda, int ldc,
+                                int swiglu, const float* in_sumsq, int in_parts, float in_eps, void* stream) {
+  LRS_REQUIRE(mid_shape_ok(a, w, m, n, k, lda), "gemm_mid_scaled: takes 17..128 rows, K %% 256 == 0, N %% 16 == 0, 16-byte aligned rows (m=%d n=%d k=%d lda=%d)", m, n, k, lda);
+  LRS_REQUIRE(mode >= OUT_STORE && mode <= OUT_ADD_F32 && ldc >= (swiglu ? n / 2 : n) && ldc % 4 == 0 && (uintptr_t)out % 16 == 0,
+              "gemm_mid_scaled: unknown output mode %d, or an output that is not 16-byte aligned (ldc=%d)", mode, ldc);
+  LRS_REQUIRE(!swiglu || mode == OUT_STORE, "gemm_mid_scaled: swiglu needs a stored output");
+  LRS_REQUIRE(in_sumsq != nullptr && in_parts > 0 && in_eps > 0.f, "gemm_mid_scaled: needs the partial sums of squares, their number and eps");
+  const MidScale scale{in_sumsq, in_parts, in_eps};
+  if (swiglu) launch_mid<true>(out, mode, (const bf16*)a, (const bf16*)w, m, n, k, lda, ldc, (hipStream_t)stream, false, scale);
+  else launch_mid<false>(out, mode, (const bf16*)a, (const bf16*)w, m, n, k, lda, ldc, (hipStream_t)stream, false, scale);
+  return lrs_check_launch("gemm_mid_scaled");
+}
+
+// Defined beside the norm kernels: x [rows, hidden] += the sum over `splits` of sums[split, rows, hidden]; next_x =
+// bf16(x * weight); next_sumsq [lrs_norm_begin_parts(hidden), rows] = partial sums of x^2.
+extern "C" int lrs_split_add_norm_begin(float* x, const float* sums, int splits, const void* weight, int w_dtype, void* next_x,
+                                        float* next_sumsq, int n_rows, int hidden, void* stream);
+
+// A product of 17..128 rows that adds into the float32 residual stream and begins the RMSNorm that follows:
+// residual [M, N] += a [M, K] w[N, K]^T; next_x [M, N] = bf16(residual * norm_weight); next_sumsq
+// [lrs_norm_begin_parts(N), M] = partial sums of residual^2, for the product that finishes the norm
+// (lrs_gemm_mid_scaled) or for scale_rows.  The kernel that adds the K splits' sums spreads over rows x 256
+// columns, where a whole norm would have one workgroup a row.
+LRS_API int lrs_gemm_mid_add_norm_begin(float* residual, const void* a, const void* w, const void* norm_weight, int norm_weight_dtype,
+                                        void* next_x, float* next_sumsq, int m, int n, int k, int lda, void* stream) {
+  LRS_REQUIRE(mid_shape_ok(a, w, m, n, k, lda) && ((uintptr_t)residual % 16 == 0), "gemm_mid_add_norm_begin: takes 17..128 rows, K %% 256 == 0, N %% 16 == 0, 16-byte aligned rows (m=%d n=%d k=%d lda=%d)", m, n, k, lda);
+  LRS_REQUIRE(next_x && next_sumsq && norm_weight, "gemm_mid_add_norm_begin: needs the norm weight and the two outputs for the next norm");
+  const int splits = launch_mid<false>(nullptr, OUT_STORE, (const bf16*)a, (const bf16*)w, m, n, k, lda, n, (hipStream_t)stream, true);
+  LRS_REQUIRE(splits > 0, "gemm_mid_add_norm_begin: the buffer for the sums of the K splits cannot hold %d x %d values", m, n);
+  if (int rc = lrs_check_launch("gemm_mid_add_norm_begin")) return rc;
+  return lrs_split_add_norm_begin(residual, split_sums_buffer(), splits, norm_weight, norm_weight_dtype, next_x, next_sumsq, m, n, stream);
 }
 
 // out [M, N] (row stride ldc) = a [M, K] (row stride lda) times w[N, K]^T.

@@ -59,6 +59,9 @@ _SIGNATURES = {
     "lrs_gemm_mid_enabled": (c_int, []),
     "lrs_gemm_skinny_lines": (c_int, [c_int]),
     "lrs_gemm_mid_shape": (c_int, [c_int, c_int, c_void_p, c_void_p]),
+    "lrs_gemm_mid_scaled": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_int, c_float, c_void_p]),
+    "lrs_gemm_mid_add_norm_begin": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p]),
+    "lrs_norm_begin_parts": (c_int, [c_int]),
     "lrs_gemm_mid_add_rmsnorm": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_float, c_void_p]),
     "lrs_attention": (c_int, [c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p,
                               c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_void_p]),
@@ -340,6 +343,46 @@ def gemm_mid_add_rmsnorm(normed: torch.Tensor, residual: torch.Tensor, a: torch.
     _check(library().lrs_gemm_mid_add_rmsnorm(_dev(normed, "normed"), dtype_code(normed.dtype), _dev(residual, "residual"), _dev(a, "a"),
                                               _dev(w, "w"), _dev(norm_weight, "norm_weight"), dtype_code(norm_weight.dtype), m, n, k,
                                               _rows(a, "a"), eps, _stream()))
+
+
+def norm_begin_parts(n: int) -> int:
+    """Partial sums of squares per row that gemm_mid_add_norm_begin() leaves for a norm over n columns."""
+    return library().lrs_norm_begin_parts(n)
+
+
+def gemm_mid_add_norm_begin(residual: torch.Tensor, a: torch.Tensor, w: torch.Tensor, norm_weight: torch.Tensor,
+                            next_x: torch.Tensor, next_sumsq: torch.Tensor) -> None:
+    """residual (float32 [M, N]) += a @ w.T for 17..128 bf16 rows, and the first half of the RMSNorm that follows:
+    next_x [M, N] = bf16(residual * norm_weight), next_sumsq [norm_begin_parts(N), M] = partial sums of residual^2.
+    gemm_mid_scaled() (or scale_rows()) finishes the norm."""
+    m, k = a.shape
+    n = w.shape[0]
+    _need(gemm_mid_takes(w.dtype, m, n, k) and a.dtype == torch.bfloat16, "gemm_mid_add_norm_begin: takes bf16 products of 17..128 rows, K % 256 == 0, N % 16 == 0")
+    _need(w.dim() == 2 and w.is_contiguous() and w.shape[1] == k, f"gemm_mid_add_norm_begin: weight must be contiguous [N, {k}]")
+    _need(residual.dtype == torch.float32 and residual.is_contiguous() and residual.shape == (m, n), f"gemm_mid_add_norm_begin: residual must be contiguous float32 [{m}, {n}]")
+    _need(next_x.dtype == torch.bfloat16 and next_x.is_contiguous() and next_x.shape == (m, n), f"gemm_mid_add_norm_begin: next_x must be contiguous bf16 [{m}, {n}]")
+    _need(next_sumsq.dtype == torch.float32 and next_sumsq.is_contiguous() and next_sumsq.shape == (norm_begin_parts(n), m),
+          f"gemm_mid_add_norm_begin: next_sumsq must be contiguous float32 [{norm_begin_parts(n)}, {m}]")
+    _need(norm_weight.is_contiguous() and norm_weight.numel() == n, f"gemm_mid_add_norm_begin: norm weight must hold {n} values")
+    _check(library().lrs_gemm_mid_add_norm_begin(_dev(residual, "residual"), _dev(a, "a"), _dev(w, "w"), _dev(norm_weight, "norm_weight"),
+                                                 dtype_code(norm_weight.dtype), _dev(next_x, "next_x"), _dev(next_sumsq, "next_sumsq"),
+                                                 m, n, k, _rows(a, "a"), _stream()))
+
+
+def gemm_mid_scaled(out: torch.Tensor, a: torch.Tensor, w: torch.Tensor, sumsq: torch.Tensor, eps: float, swiglu: bool = False) -> None:
+    """out = (the RMSNorm that `a` and `sumsq` stand for) @ w.T for 17..128 rows: a = bf16(h * norm weight) [M, K],
+    sumsq [parts, M] partial sums of h^2; row r of the product is multiplied by rsqrt(sum_p sumsq[p, r] / K + eps).
+    swiglu as in gemm()."""
+    m, k = a.shape
+    n = w.shape[0]
+    _need(gemm_mid_takes(w.dtype, m, n, k) and a.dtype == torch.bfloat16, "gemm_mid_scaled: takes bf16 products of 17..128 rows, K % 256 == 0, N % 16 == 0")
+    _need(w.dim() == 2 and w.is_contiguous() and w.shape[1] == k, f"gemm_mid_scaled: weight must be contiguous [N, {k}]")
+    _need(out.shape == (m, n // 2 if swiglu else n), f"gemm_mid_scaled: out must be [{m}, {n // 2 if swiglu else n}], got {tuple(out.shape)}")
+    _need(out.dtype in (torch.bfloat16, torch.float32) and not (swiglu and out.dtype != torch.bfloat16), "gemm_mid_scaled: output must be bf16, or float32 without swiglu")
+    _need(sumsq.dtype == torch.float32 and sumsq.dim() == 2 and sumsq.shape[1] == m and sumsq.is_contiguous() and eps > 0, f"gemm_mid_scaled: sumsq must be float32 [parts, {m}] and eps positive")
+    mode = OUT_STORE if out.dtype == torch.bfloat16 else OUT_STORE_F32
+    _check(library().lrs_gemm_mid_scaled(_dev(out, "out"), mode, _dev(a, "a"), _dev(w, "w"), m, n, k, _rows(a, "a"), _rows(out, "out"),
+                                         int(swiglu), _dev(sumsq, "sumsq"), sumsq.shape[0], eps, _stream()))
 
 
 def set_skinny_max_m(m: int) -> None:

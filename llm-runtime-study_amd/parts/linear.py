@@ -94,6 +94,11 @@ def linear(ctx, out, x, weight, bias=None, accumulate: bool = False, swiglu: boo
     if isinstance(x, ScaledRows):
         if ops.gemm_chains_norm(weight.dtype, x.count, weight.shape[1]):
             scaled, x = x, x.x
+        elif (ops.gemm_mid_takes(weight.dtype, x.count, weight.shape[0], weight.shape[1], ops.MID_ROWS_PREFERRED) and bias is None
+              and not accumulate and out.dtype in (torch.bfloat16, torch.float32) and not (swiglu and out.dtype != torch.bfloat16)):
+            # 17..128 rows: the product finishes the norm that the product before it began
+            ops.gemm_mid_scaled(out, x.x, weight, x.sumsq, x.eps, swiglu)
+            return None
         else:
             x = x.materialize(ctx)
     if not isinstance(x, LazyNorm) and x.dtype == torch.bfloat16:
@@ -111,27 +116,29 @@ def linear(ctx, out, x, weight, bias=None, accumulate: bool = False, swiglu: boo
             return None
         x = x.materialize(ctx)
     m, n = x.shape[0], weight.shape[0]
-    if (getattr(ctx, "library_gemm", False) and weight.dtype == torch.bfloat16 and x.dtype == torch.bfloat16 and m > ops.skinny_max_m()
+    library = getattr(ctx, "library_gemm", False)
+    # 17..128 rows: this package's kernel for them, whether or not the step may use the vendor library
+    if (x.dtype == torch.bfloat16 and bias is None and x.is_contiguous() and (accumulate or out.dtype in (torch.bfloat16, torch.float32))
+            and not (swiglu and out.dtype != torch.bfloat16)
+            and ops.gemm_mid_takes(weight.dtype, m, n, weight.shape[1], ops.MID_ROWS_PREFERRED if library else 128)):
+        parameters = getattr(then_norm, "rms_parameters", None) if accumulate else None
+        if parameters is not None and out.is_contiguous() and out.dtype == torch.float32 and parameters()[0].numel() == n:
+            # product, residual add and the first half of the norm that follows: the kernel that adds the K
+            # splits' sums leaves bf16(h * norm weight) and partial sums of squares, the next product finishes
+            norm_weight, eps = parameters()
+            turn = ctx.memo["norm_ahead_turn"] = 1 - ctx.memo.get("norm_ahead_turn", 0)
+            begun = ScaledRows(ctx.scratch(f"norm_ahead_x{turn}", (m, n), torch.bfloat16),
+                               ctx.scratch(f"norm_begin_sumsq{turn}", (ops.norm_begin_parts(n), m), torch.float32), eps, m)
+            ops.gemm_mid_add_norm_begin(out, x, weight, norm_weight, begun.x, begun.sumsq)
+            return begun
+        ops.gemm(out, x, weight, None, accumulate, swiglu)
+        return None
+    if (library and weight.dtype == torch.bfloat16 and x.dtype == torch.bfloat16 and m > ops.skinny_max_m()
             and bias is None and x.is_contiguous() and (accumulate or (out.dtype in (torch.bfloat16, torch.float32) and out.is_contiguous()))
             and not (swiglu and out.dtype != torch.bfloat16)):
-        own = ops.gemm_mid_takes(weight.dtype, m, n, weight.shape[1], ops.MID_ROWS_PREFERRED)   # 17..128 rows: this package's kernel, not the library's
-        if own and not accumulate:
-            ops.gemm(out, x, weight, None, False, swiglu)
-            return None
-        if own and accumulate and out.is_contiguous() and out.dtype == torch.float32 and n <= 8192:
-            parameters = getattr(then_norm, "rms_parameters", None)
-            if parameters is not None and parameters()[0].numel() == n:
-                # product, residual add and the norm that follows: the sums of the K splits go straight into the norm kernel
-                norm_weight, eps = parameters()
-                normed = ctx.scratch("norm_after_add", (m, n), ctx.dtype)
-                ops.gemm_mid_add_rmsnorm(normed, out, x, weight, norm_weight, eps)
-                return normed
         if accumulate or swiglu:
             y = ctx.scratch("library_gemm_out", (m, n), torch.bfloat16)
-            if own:
-                ops.gemm(y, x, weight)
-            else:
-                torch.mm(x, weight.t(), out=y)
+            torch.mm(x, weight.t(), out=y)
             if accumulate:
                 parameters = getattr(then_norm, "rms_parameters", None)
                 if parameters is not None and out.is_contiguous() and parameters()[0].numel() == n:

@@ -292,6 +292,47 @@ def test_gemm_of_17_to_64_rows_with_residual_add_and_norm(ops, w_dtype, m, n, k,
 
 
 @pytest.mark.parametrize("w_dtype", DTYPES)
+@pytest.mark.parametrize("m,h,n2,k,swiglu,splits", [(17, 256, 64, 256, False, 0), (40, 512, 208, 1024, True, 2), (64, 4096, 6144, 4096, False, 0),
+                                                     (100, 1024, 2048, 3328, True, 3), (128, 4096, 24576, 512, True, 0)])
+def test_gemm_of_17_to_128_rows_with_norm_taken_apart(ops, w_dtype, m, h, n2, k, swiglu, splits):
+    """residual += x W1^T begins the RMSNorm of the new residual (bf16(h * weight) and partial sums of squares, left by
+    the kernel that adds the K splits' sums); the next product finishes it in its epilogue, or scale_rows does."""
+    g = torch.Generator().manual_seed(m + h + n2 + k)
+    a = torch.randn(m, k, generator=g).bfloat16()
+    w1 = (torch.randn(h, k, generator=g) / math.sqrt(k)).bfloat16()
+    w2 = (torch.randn(n2, h, generator=g) / math.sqrt(h)).bfloat16()
+    residual = torch.randn(m, h, generator=g) * 2
+    gamma = (1 + 0.2 * torch.randn(h, generator=g)).to(w_dtype)
+    eps = 1e-5
+    updated = residual.double() + a.double() @ w1.double().T
+    normed = gamma.double() * updated * torch.rsqrt(updated.square().mean(-1, keepdim=True) + eps)
+    out = dev(residual.clone())
+    next_x = torch.empty(m, h, device="cuda", dtype=torch.bfloat16)
+    sumsq = torch.empty(ops.norm_begin_parts(h), m, device="cuda")
+    ops.gemm_mid_tune(True, 0, splits)
+    try:
+        ops.gemm_mid_add_norm_begin(out, dev(a), dev(w1), dev(gamma), next_x, sumsq)
+        torch.testing.assert_close(out.cpu().double(), updated, rtol=1e-4, atol=1e-4)
+        torch.testing.assert_close(sumsq.sum(0).cpu().double(), updated.square().sum(-1), rtol=1e-4, atol=1e-4)
+        finished = torch.empty(m, h, device="cuda", dtype=torch.bfloat16)
+        ops.scale_rows(finished, next_x, sumsq, eps)
+        close_in_norm(finished, normed, 5e-3)
+        if swiglu:
+            inter = n2 // 2
+            mixed = torch.stack((w2[:inter].view(inter // 8, 8, h), w2[inter:].view(inter // 8, 8, h)), 1).reshape(n2, h).contiguous()
+            got = torch.empty(m, inter, device="cuda", dtype=torch.bfloat16)
+            ops.gemm_mid_scaled(got, next_x, dev(mixed), sumsq, eps, swiglu=True)
+            y = normed @ w2.double().T
+            close_in_norm(got, torch.nn.functional.silu(y[:, :inter]) * y[:, inter:], 1e-2)
+        else:
+            got = torch.empty(m, n2, device="cuda")
+            ops.gemm_mid_scaled(got, next_x, dev(w2), sumsq, eps)
+            close_in_norm(got, normed @ w2.double().T, 5e-3)
+    finally:
+        ops.gemm_mid_tune(True, 0, 0)
+
+
+@pytest.mark.parametrize("w_dtype", DTYPES)
 @pytest.mark.parametrize("m,n,k", [(1, 64, 96), (8, 331, 160), (17, 200, 96), (64, 6144, 4096), (33, 48, 264)])
 def test_gemm_with_fused_rmsnorm_input(ops, w_dtype, m, n, k, all_rows_in_own_kernel):
     """The product of the RMSNorm of float32 rows, picked through a row list, in one kernel."""
