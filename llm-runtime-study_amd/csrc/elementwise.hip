@@ -159,15 +159,17 @@ LRS_API int lrs_split_add_rmsnorm(void* out, int out_dtype, float* x, const floa
   return lrs_check_launch("split_add_rmsnorm");
 }
 
-// The first half of "add the K splits' sums to the residual stream, then RMSNorm", spread over rows x 256 columns
-// (one wave each) instead of one workgroup a row: x += sum of the splits; next_x = bf16(x * weight); the wave's
-// sum of x^2 goes to next_sumsq [gridDim.x, rows].  The product that reads next_x multiplies its rows by
-// rsqrt(sum of the parts / hidden + eps): the factor is constant along a row.
+// The first half of "add the K splits' sums to the residual stream, then RMSNorm", spread over rows x 1,024
+// columns (a workgroup of four waves each) instead of one workgroup a row: x += sum of the splits; next_x =
+// bf16(x * weight); the workgroup's sum of x^2 goes to next_sumsq [gridDim.x, rows].  The product that reads
+// next_x multiplies its rows by rsqrt(sum of the parts / hidden + eps): the factor is constant along a row.
+constexpr int NORM_BEGIN_COLUMNS = 1024;
 template <typename TW>
-__global__ void split_add_norm_begin_kernel(float* __restrict__ x, const float* __restrict__ sums, int splits,
-                                            const TW* __restrict__ weight, bf16* __restrict__ next_x,
-                                            float* __restrict__ next_sumsq, int hidden) {
-  const int row = blockIdx.y, rows = gridDim.y, c = (blockIdx.x * WAVE + threadIdx.x) * 4;
+__global__ __launch_bounds__(NORM_BEGIN_COLUMNS / 4) void split_add_norm_begin_kernel(
+    float* __restrict__ x, const float* __restrict__ sums, int splits, const TW* __restrict__ weight,
+    bf16* __restrict__ next_x, float* __restrict__ next_sumsq, int hidden) {
+  __shared__ float scratch[16];
+  const int row = blockIdx.y, rows = gridDim.y, c = (blockIdx.x * (NORM_BEGIN_COLUMNS / 4) + threadIdx.x) * 4;
   float ss = 0.f;
   if (c < hidden) {
     const int64_t at = (int64_t)row * hidden + c;
@@ -184,11 +186,11 @@ __global__ void split_add_norm_begin_kernel(float* __restrict__ x, const float* 
     }
     *(bf16x4*)(next_x + at) = nx;
   }
-  ss = wave_sum(ss);
+  ss = block_sum(ss, scratch);
   if (threadIdx.x == 0) next_sumsq[(int64_t)blockIdx.x * rows + row] = ss;
 }
 
-LRS_API int lrs_norm_begin_parts(int hidden) { return (hidden + 4 * WAVE - 1) / (4 * WAVE); }
+LRS_API int lrs_norm_begin_parts(int hidden) { return (hidden + NORM_BEGIN_COLUMNS - 1) / NORM_BEGIN_COLUMNS; }
 
 LRS_API int lrs_split_add_norm_begin(float* x, const float* sums, int splits, const void* weight, int w_dtype, void* next_x,
                                      float* next_sumsq, int n_rows, int hidden, void* stream) {
@@ -197,9 +199,10 @@ LRS_API int lrs_split_add_norm_begin(float* x, const float* sums, int splits, co
   LRS_REQUIRE(hidden % 4 == 0 && ((uintptr_t)x % 16) == 0 && ((uintptr_t)sums % 16) == 0 && ((uintptr_t)next_x % 8) == 0,
               "split_add_norm_begin: needs hidden %% 4 == 0 and aligned rows (hidden=%d)", hidden);
   const dim3 grid(lrs_norm_begin_parts(hidden), n_rows);
+  constexpr int threads = NORM_BEGIN_COLUMNS / 4;
   hipStream_t s = (hipStream_t)stream;
-  if (w_dtype == LRS_F32) split_add_norm_begin_kernel<float><<<grid, WAVE, 0, s>>>(x, sums, splits, (const float*)weight, (bf16*)next_x, next_sumsq, hidden);
-  else if (w_dtype == LRS_BF16) split_add_norm_begin_kernel<bf16><<<grid, WAVE, 0, s>>>(x, sums, splits, (const bf16*)weight, (bf16*)next_x, next_sumsq, hidden);
+  if (w_dtype == LRS_F32) split_add_norm_begin_kernel<float><<<grid, threads, 0, s>>>(x, sums, splits, (const float*)weight, (bf16*)next_x, next_sumsq, hidden);
+  else if (w_dtype == LRS_BF16) split_add_norm_begin_kernel<bf16><<<grid, threads, 0, s>>>(x, sums, splits, (const bf16*)weight, (bf16*)next_x, next_sumsq, hidden);
   else return lrs_fail("split_add_norm_begin: unknown weight dtype %d", w_dtype);
   return lrs_check_launch("split_add_norm_begin");
 }

@@ -782,7 +782,13 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_mid_kernel(
   float my_scale = 1.f;
   if (scale.sumsq && tid < m) {
     float q = 0.f;
-    for (int p = 0; p < scale.parts; ++p) q += scale.sumsq[(int64_t)p * m + tid];
+    for (int p0 = 0; p0 < scale.parts; p0 += 8) {      // eight parts asked for at a time (usually all there are)
+      float part[8];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) part[j] = p0 + j < scale.parts ? scale.sumsq[(int64_t)(p0 + j) * m + tid] : 0.f;
+#pragma unroll
+      for (int j = 0; j < 8; ++j) q += part[j];
+    }
     my_scale = 1.0f / sqrtf(q / (float)k + scale.eps);
   }
   floatx4 acc[MT];
@@ -1283,7 +1289,7 @@ extern "C" int lrs_split_add_norm_begin(float* x, const float* sums, int splits,
 // A product of 17..128 rows that adds into the float32 residual stream and begins the RMSNorm that follows:
 // residual [M, N] += a [M, K] w[N, K]^T; next_x [M, N] = bf16(residual * norm_weight); next_sumsq
 // [lrs_norm_begin_parts(N), M] = partial sums of residual^2, for the product that finishes the norm
-// (lrs_gemm_mid_scaled) or for scale_rows.  The kernel that adds the K splits' sums spreads over rows x 256
+// (lrs_gemm_mid_scaled) or for scale_rows.  The kernel that adds the K splits' sums spreads over rows x 1,024
 // columns, where a whole norm would have one workgroup a row.
 LRS_API int lrs_gemm_mid_add_norm_begin(float* residual, const void* a, const void* w, const void* norm_weight, int norm_weight_dtype,
                                         void* next_x, float* next_sumsq, int m, int n, int k, int lda, void* stream) {
