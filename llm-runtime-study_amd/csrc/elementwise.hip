@@ -368,7 +368,11 @@ __global__ __launch_bounds__(256) void qk_prep_vec_kernel(T* __restrict__ qkv, i
                                                           const TW* __restrict__ k_weight, float eps,
                                                           const float* __restrict__ cosv, const float* __restrict__ sinv,
                                                           int rot_half, T* __restrict__ k_pages, T* __restrict__ v_pages,
-                                                          const int* __restrict__ slots, int page_size, int prep_blocks) {
+                                                          const int* __restrict__ slots, int page_size, int prep_blocks,
+                                                          const float* __restrict__ sums = nullptr, int splits = 0,
+                                                          int sum_columns = 0) {
+  // sums != null: the heads come as the float32 sums that the K splits of the q/k/v product left,
+  // [splits, tokens, sum_columns], added up here in split order; qkv only receives the prepared q heads.
   constexpr int VE = 16 / sizeof(T);
   typedef T vec __attribute__((ext_vector_type(VE)));
   __shared__ int slot_of[16];
@@ -384,7 +388,29 @@ __global__ __launch_bounds__(256) void qk_prep_vec_kernel(T* __restrict__ qkv, i
   const int token = pair / heads, head = pair % heads;
   T* src = qkv + (int64_t)token * row_stride + (int64_t)head * d;
   const bool is_q = head < nq, is_k = !is_q && head < nq + nkv;
-  const vec lo = *(const vec*)(src + VE * j), hi = *(const vec*)(src + half + VE * j);
+  float a[VE], b[VE], inv = 1.f;
+  if (sums) {
+#pragma unroll
+    for (int e = 0; e < VE; ++e) a[e] = b[e] = 0.f;
+    const float* from = sums + (int64_t)token * sum_columns + (int64_t)head * d;
+    for (int sp = 0; sp < splits; ++sp, from += (int64_t)tokens * sum_columns) {
+      float pa[VE], pb[VE];
+      load_floats<float, VE>(from + VE * j, pa);
+      load_floats<float, VE>(from + half + VE * j, pb);
+#pragma unroll
+      for (int e = 0; e < VE; ++e) {
+        a[e] += pa[e];
+        b[e] += pb[e];
+      }
+    }
+  } else {
+    const vec lo = *(const vec*)(src + VE * j), hi = *(const vec*)(src + half + VE * j);
+#pragma unroll
+    for (int e = 0; e < VE; ++e) {
+      a[e] = to_float(lo[e]);
+      b[e] = to_float(hi[e]);
+    }
+  }
   int64_t page = 0, off = 0;
   int kv_head = 0;
   if (!is_q) {
@@ -397,19 +423,13 @@ __global__ __launch_bounds__(256) void qk_prep_vec_kernel(T* __restrict__ qkv, i
       T* vdst = v_pages + (page * nkv + kv_head) * d * page_size + off;
 #pragma unroll
       for (int e = 0; e < VE; ++e) {
-        vdst[(int64_t)(VE * j + e) * page_size] = lo[e];
-        vdst[(int64_t)(half + VE * j + e) * page_size] = hi[e];
+        vdst[(int64_t)(VE * j + e) * page_size] = from_float<T>(a[e]);
+        vdst[(int64_t)(half + VE * j + e) * page_size] = from_float<T>(b[e]);
       }
       return;
     }
   }
   const TW* weight = is_q ? q_weight : k_weight;
-  float a[VE], b[VE], inv = 1.f;
-#pragma unroll
-  for (int e = 0; e < VE; ++e) {
-    a[e] = to_float(lo[e]);
-    b[e] = to_float(hi[e]);
-  }
   if (weight) {
     float ss = 0.f;
 #pragma unroll
@@ -447,10 +467,11 @@ __global__ __launch_bounds__(256) void qk_prep_vec_kernel(T* __restrict__ qkv, i
   *(vec*)(dst + half + VE * j) = out_hi;
 }
 
-LRS_API int lrs_qk_prep(void* qkv, int dtype, int tokens, int row_stride, int nq, int nkv, int d,
-                        const void* q_weight, const void* k_weight, int w_dtype, float eps,
-                        const float* cosv, const float* sinv, int rot_half, void* k_pages,
-                        void* v_pages, const int* slots, int page_size, void* stream) {
+static int qk_prep_launch(void* qkv, int dtype, int tokens, int row_stride, int nq, int nkv, int d,
+                          const void* q_weight, const void* k_weight, int w_dtype, float eps,
+                          const float* cosv, const float* sinv, int rot_half, void* k_pages,
+                          void* v_pages, const int* slots, int page_size, void* stream,
+                          const float* sums, int splits, int sum_columns) {
   LRS_REQUIRE(tokens > 0 && nq > 0 && nkv >= 0 && d > 0, "qk_prep: bad sizes tokens=%d nq=%d nkv=%d d=%d", tokens, nq, nkv, d);
   LRS_REQUIRE(rot_half >= 0 && 2 * rot_half <= d, "qk_prep: rotary width %d exceeds head_dim %d", 2 * rot_half, d);
   LRS_REQUIRE(rot_half == 0 || (cosv && sinv), "qk_prep: rotation asked for without tables");
@@ -462,7 +483,7 @@ LRS_API int lrs_qk_prep(void* qkv, int dtype, int tokens, int row_stride, int nq
   // many tokens: the values are written in whole runs of slots, by workgroups of their own
   const size_t elem = dtype == LRS_F32 ? 4 : 2;
   const int ve = (int)(16 / elem);
-  const bool values_apart = nkv > 0 && tokens >= 128 && page_size % ve == 0 && ((uintptr_t)v_pages % 16) == 0;
+  const bool values_apart = !sums && nkv > 0 && tokens >= 128 && page_size % ve == 0 && ((uintptr_t)v_pages % 16) == 0;
   const int per_head = d / (2 * ve);
   const bool vectors = d % (2 * ve) == 0 && per_head <= 64 && (per_head & (per_head - 1)) == 0 && (rot_half == 0 || 2 * rot_half == d) &&
                        row_stride % ve == 0 && ((uintptr_t)qkv % 16) == 0 && ((uintptr_t)k_pages % 16) == 0 &&
@@ -479,7 +500,7 @@ LRS_API int lrs_qk_prep(void* qkv, int dtype, int tokens, int row_stride, int nq
 #define LAUNCH_VEC(T, TW)                                                                                        \
   qk_prep_vec_kernel<T, TW><<<vgrid, 256, 0, s>>>((T*)qkv, row_stride, tokens, heads, nq, nkv, d, (const TW*)q_weight, \
                                                   (const TW*)k_weight, eps, cosv, sinv, rot_half, (T*)k_pages,   \
-                                                  (T*)v_pages, slots, page_size, (int)prep_blocks)
+                                                  (T*)v_pages, slots, page_size, (int)prep_blocks, sums, splits, sum_columns)
     if (dtype == LRS_F32 && w_dtype == LRS_F32) LAUNCH_VEC(float, float);
     else if (dtype == LRS_BF16 && w_dtype == LRS_BF16) LAUNCH_VEC(bf16, bf16);
     else if (dtype == LRS_BF16 && w_dtype == LRS_F32) LAUNCH_VEC(bf16, float);
@@ -488,6 +509,7 @@ LRS_API int lrs_qk_prep(void* qkv, int dtype, int tokens, int row_stride, int nq
 #undef LAUNCH_VEC
     return lrs_check_launch("qk_prep");
   }
+  LRS_REQUIRE(!sums, "qk_prep: the sums of K splits need the shape the vector kernel takes (head_dim %d, rotation over %d)", d, 2 * rot_half);
   if (values_apart) {
     dim3 vgrid((tokens + 15) / 16, nkv);
     if (dtype == LRS_F32)
@@ -511,6 +533,25 @@ LRS_API int lrs_qk_prep(void* qkv, int dtype, int tokens, int row_stride, int nq
   else return lrs_fail("qk_prep: unknown dtypes %d/%d", dtype, w_dtype);
 #undef LAUNCH
   return lrs_check_launch("qk_prep");
+}
+
+LRS_API int lrs_qk_prep(void* qkv, int dtype, int tokens, int row_stride, int nq, int nkv, int d,
+                        const void* q_weight, const void* k_weight, int w_dtype, float eps,
+                        const float* cosv, const float* sinv, int rot_half, void* k_pages,
+                        void* v_pages, const int* slots, int page_size, void* stream) {
+  return qk_prep_launch(qkv, dtype, tokens, row_stride, nq, nkv, d, q_weight, k_weight, w_dtype, eps, cosv, sinv, rot_half, k_pages,
+                        v_pages, slots, page_size, stream, nullptr, 0, 0);
+}
+
+// The same from the float32 sums that the K splits of the q/k/v product left, sums [splits, tokens, (nq + 2 nkv) d]:
+// they are added up on the way, so no kernel of its own has to.  qkv receives the prepared q heads.
+LRS_API int lrs_qk_prep_from_sums(void* qkv, int dtype, int tokens, int row_stride, int nq, int nkv, int d,
+                                  const void* q_weight, const void* k_weight, int w_dtype, float eps,
+                                  const float* cosv, const float* sinv, int rot_half, void* k_pages,
+                                  void* v_pages, const int* slots, int page_size, const float* sums, int splits, void* stream) {
+  LRS_REQUIRE(sums != nullptr && splits > 0 && ((uintptr_t)sums % 16) == 0, "qk_prep_from_sums: needs the sums and their number");
+  return qk_prep_launch(qkv, dtype, tokens, row_stride, nq, nkv, d, q_weight, k_weight, w_dtype, eps, cosv, sinv, rot_half, k_pages,
+                        v_pages, slots, page_size, stream, sums, splits, (nq + 2 * nkv) * d);
 }
 
 // ----------------------------------------------------------- gated activation

@@ -1301,6 +1301,31 @@ LRS_API int lrs_gemm_mid_add_norm_begin(float* residual, const void* a, const vo
   return lrs_split_add_norm_begin(residual, split_sums_buffer(), splits, norm_weight, norm_weight_dtype, next_x, next_sumsq, m, n, stream);
 }
 
+// Defined beside qk_prep: see there.
+extern "C" int lrs_qk_prep_from_sums(void* qkv, int dtype, int tokens, int row_stride, int nq, int nkv, int d, const void* q_weight,
+                                     const void* k_weight, int w_dtype, float eps, const float* cosv, const float* sinv,
+                                     int rot_half, void* k_pages, void* v_pages, const int* slots, int page_size,
+                                     const float* sums, int splits, void* stream);
+
+// The q/k/v product of 17..128 rows (its input possibly a norm begun before it: in_sumsq as in lrs_gemm_mid_scaled, or
+// null) and what follows it: per-head norm and rotation of q and k, q into qkv [M, row_stride], k and v into the
+// pages.  The kernel that prepares the heads adds up the K splits' sums itself.
+LRS_API int lrs_gemm_mid_qk_prep(void* qkv, int row_stride, const void* a, const void* w, int m, int k, int lda,
+                                 const float* in_sumsq, int in_parts, float in_eps, int nq, int nkv, int d,
+                                 const void* q_weight, const void* k_weight, int w_dtype, float eps, const float* cosv,
+                                 const float* sinv, int rot_half, void* k_pages, void* v_pages, const int* slots,
+                                 int page_size, void* stream) {
+  const int n = (nq + 2 * nkv) * d;
+  LRS_REQUIRE(mid_shape_ok(a, w, m, n, k, lda), "gemm_mid_qk_prep: takes 17..128 rows, K %% 256 == 0, N %% 16 == 0, 16-byte aligned rows (m=%d n=%d k=%d lda=%d)", m, n, k, lda);
+  LRS_REQUIRE(in_sumsq == nullptr || (in_parts > 0 && in_eps > 0.f), "gemm_mid_qk_prep: in_parts and in_eps must be positive");
+  const MidScale scale{in_sumsq, in_parts, in_eps};
+  const int splits = launch_mid<false>(nullptr, OUT_STORE, (const bf16*)a, (const bf16*)w, m, n, k, lda, n, (hipStream_t)stream, true, scale);
+  LRS_REQUIRE(splits > 0, "gemm_mid_qk_prep: the buffer for the sums of the K splits cannot hold %d x %d values", m, n);
+  if (int rc = lrs_check_launch("gemm_mid_qk_prep")) return rc;
+  return lrs_qk_prep_from_sums(qkv, LRS_BF16, m, row_stride, nq, nkv, d, q_weight, k_weight, w_dtype, eps, cosv, sinv, rot_half, k_pages,
+                               v_pages, slots, page_size, split_sums_buffer(), splits, stream);
+}
+
 // out [M, N] (row stride ldc) = a [M, K] (row stride lda) times w[N, K]^T.
 //   norm_weight != null: `a` is the float32 residual stream [*, K]; its rows (picked through
 //     `rows` if given) are RMS-normalised with norm_weight and eps on the way in.  bf16 weights,

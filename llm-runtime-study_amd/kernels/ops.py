@@ -37,6 +37,8 @@ _SIGNATURES = {
     "lrs_rope_table": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p]),
     "lrs_qk_prep": (c_int, [c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_int, c_float,
                             c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p]),
+    "lrs_gemm_mid_qk_prep": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p, c_int, c_float, c_int, c_int, c_int,
+                                     c_void_p, c_void_p, c_int, c_float, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p]),
     "lrs_silu_mul": (c_int, [c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p]),
     "lrs_add_into": (c_int, [c_void_p, c_void_p, c_int, c_int64, c_void_p]),
     "lrs_fill_i32": (c_int, [c_void_p, c_int, c_int64, c_void_p]),
@@ -271,6 +273,46 @@ def qk_prep(qkv: torch.Tensor, nq: int, nkv: int, d: int, q_weight, k_weight, ep
         dtype_code(w_dtype), eps, None if cos is None else cos.data_ptr(), None if sin is None else sin.data_ptr(), rot_half,
         None if nkv == 0 else _dev(k_pages, "k_pages"), None if nkv == 0 else _dev(v_pages, "v_pages"),
         None if nkv == 0 else _dev(slots, "slots"), page_size, _stream()))
+
+
+def gemm_mid_qk_prep_takes(dtype: torch.dtype, m: int, nq: int, nkv: int, d: int, k: int, rot_half: int) -> bool:
+    """Whether gemm_mid_qk_prep() takes the shape: bf16, 17..128 rows, heads the vector form of qk_prep takes
+    (head_dim 16, 32, 64, ... 1024, rotation over the whole head or none), cache written by this layer."""
+    per_head = d // 16
+    return (gemm_mid_takes(dtype, m, (nq + 2 * nkv) * d, k, MID_ROWS_PREFERRED) and nkv > 0 and d % 16 == 0 and 0 < per_head <= 64
+            and per_head & (per_head - 1) == 0 and rot_half in (0, d // 2))
+
+
+def gemm_mid_qk_prep(qkv: torch.Tensor, a: torch.Tensor, w: torch.Tensor, sumsq: torch.Tensor | None, in_eps: float, nq: int, nkv: int,
+                     d: int, q_weight, k_weight, eps: float, cos, sin, k_pages, v_pages, slots, page_size: int) -> None:
+    """The q/k/v product of 17..128 bf16 rows (a @ w.T; with `sumsq` the input is a norm begun before it, as in
+    gemm_mid_scaled) and qk_prep() of its result in two kernels: the one that prepares the heads adds up the sums of
+    the product's K splits itself.  q goes into `qkv` [M, (nq+2*nkv)*d], k and v into the pages."""
+    m, k = a.shape
+    n = (nq + 2 * nkv) * d
+    rot_half = 0 if cos is None else cos.shape[1]
+    _need(a.dtype == torch.bfloat16 and gemm_mid_qk_prep_takes(w.dtype, m, nq, nkv, d, k, rot_half), "gemm_mid_qk_prep: shape not taken (see gemm_mid_qk_prep_takes)")
+    _need(w.shape == (n, k) and w.is_contiguous(), f"gemm_mid_qk_prep: weight must be contiguous [{n}, {k}]")
+    _need(qkv.dtype == torch.bfloat16 and qkv.shape == (m, n), f"gemm_mid_qk_prep: qkv must be bf16 [{m}, {n}]")
+    if sumsq is not None:
+        _need(sumsq.dtype == torch.float32 and sumsq.dim() == 2 and sumsq.shape[1] == m and sumsq.is_contiguous() and in_eps > 0, f"gemm_mid_qk_prep: sumsq must be float32 [parts, {m}] and its eps positive")
+    if cos is not None:
+        _need(cos.shape[0] >= m and sin.shape == cos.shape and cos.is_contiguous() and sin.is_contiguous() and cos.dtype == torch.float32 and sin.dtype == torch.float32,
+              "gemm_mid_qk_prep: rotary tables must be float32 [T, half]")
+    w_dtype = torch.bfloat16
+    if q_weight is not None:
+        _need(k_weight is not None and q_weight.numel() == d and k_weight.numel() == d and q_weight.dtype == k_weight.dtype, "gemm_mid_qk_prep: q/k norm weights must both hold head_dim values")
+        w_dtype = q_weight.dtype
+    _need(k_pages.dim() == 4 and k_pages.shape[1:] == (nkv, page_size, d) and v_pages.shape == (k_pages.shape[0], nkv, d, page_size),
+          f"gemm_mid_qk_prep: key pages must be [pages, {nkv}, {page_size}, {d}] and value pages [pages, {nkv}, {d}, {page_size}]")
+    _need(k_pages.is_contiguous() and v_pages.is_contiguous() and k_pages.dtype == torch.bfloat16 and v_pages.dtype == torch.bfloat16, "gemm_mid_qk_prep: pages must be contiguous bf16")
+    _need(slots.dtype == torch.int32 and slots.numel() >= m and slots.is_contiguous(), "gemm_mid_qk_prep: slots must be int32 [T]")
+    _check(library().lrs_gemm_mid_qk_prep(
+        _dev(qkv, "qkv"), _rows(qkv, "qkv"), _dev(a, "a"), _dev(w, "w"), m, k, _rows(a, "a"),
+        None if sumsq is None else _dev(sumsq, "sumsq"), 0 if sumsq is None else sumsq.shape[0], in_eps if sumsq is not None else 0.0,
+        nq, nkv, d, None if q_weight is None else _dev(q_weight, "q_weight"), None if k_weight is None else _dev(k_weight, "k_weight"),
+        dtype_code(w_dtype), eps, None if cos is None else cos.data_ptr(), None if sin is None else sin.data_ptr(), rot_half,
+        _dev(k_pages, "k_pages"), _dev(v_pages, "v_pages"), _dev(slots, "slots"), page_size, _stream()))
 
 
 def silu_mul(out: torch.Tensor, gate_up: torch.Tensor, interleaved: bool = False) -> None:

@@ -20,7 +20,7 @@ import torch
 
 from ..kernels import ops
 from .base import PagedKVNeed, Part, PartSpec, TensorSpec, create, length_class, register
-from .linear import linear, rows_of
+from .linear import ScaledRows, linear, materialize, rows_of
 
 
 class GQAAttention(Part):
@@ -106,6 +106,8 @@ class GQAAttention(Part):
             return 1
         return max(1, min(-(-8 * units // workgroups), longest // 1024, 32, (64 << 20) // max(outputs, 1)))
 
+    PREPARE_INSIDE_ROWS = 16     # rows of a decode step up to which the attention kernel prepares q, k and v itself
+
     # ------------------------------------------------------------------ forward
     def forward(self, ctx, x, residual, cache, then_norm=None):
         if cache is None:
@@ -114,17 +116,34 @@ class GQAAttention(Part):
         nkv = 0 if self.kv_shared else self.num_kv_heads
         group = ctx.group(cache.group)
         qkv = ctx.scratch("attn_qkv", (t, (nq + 2 * nkv) * d), ctx.dtype)
-        linear(ctx, qkv, x, self.w_qkv, self.b_qkv)
         tables = self.position.tables(ctx)
         cos, sin = tables if tables is not None else (None, None)
+        # 17..128 rows of a decode step: the q/k/v product and the preparation of its heads as two kernels, the
+        # second adding up the sums of the product's K splits (no kernel of its own for that)
+        together = (ctx.all_decode and self.b_qkv is None and ctx.dtype == torch.bfloat16 and t > self.PREPARE_INSIDE_ROWS
+                    and ops.gemm_mid_qk_prep_takes(self.w_qkv.dtype, t, nq, nkv, d, self.w_qkv.shape[1], 0 if cos is None else cos.shape[1]))
+        begun = plain = None
+        if together:
+            begun = x if isinstance(x, ScaledRows) else None          # a norm that the product before began
+            plain = begun.x if begun is not None else materialize(ctx, x)
+            together = plain.dtype == torch.bfloat16 and plain.is_contiguous()
+        if together:
+            ops.gemm_mid_qk_prep(qkv, plain, self.w_qkv, None if begun is None else begun.sumsq, 0.0 if begun is None else begun.eps,
+                                 nq, nkv, d, self.q_norm, self.k_norm, self.qk_norm_eps, cos, sin, cache.k_pages, cache.v_pages,
+                                 group.slots, group.page_size)
+        else:
+            linear(ctx, qkv, x if plain is None or begun is not None else plain, self.w_qkv, self.b_qkv)
         out = ctx.scratch("attn_out", (t, nq * d), ctx.dtype)
         kv_heads = cache.k_pages.shape[1]
         decode = ctx.all_decode and ops.attention_decode_supported(ctx.dtype, nq, kv_heads, d, group.page_size)
         # a decode step's attention kernel normalises and rotates q and k and writes the new key and
-        # value itself, when the rotation covers the whole head or there is none
+        # value itself, when the rotation covers the whole head or there is none; beyond 16 rows a kernel
+        # before it does that once a token (measured: 98 against 108 us for the attention kernel at 64 rows)
         whole_head = cos is None or cos.shape[1] * 2 == d
         prepare = None
-        if decode and whole_head and ops.decode_prepare_supported(d, cos is not None):
+        if together:
+            pass
+        elif decode and whole_head and ops.decode_prepare_supported(d, cos is not None) and t <= self.PREPARE_INSIDE_ROWS:
             prepare = ops.DecodePrepare(self.q_norm, self.k_norm, self.qk_norm_eps, cos, sin, nkv)
         else:
             ops.qk_prep(qkv, nq, nkv, d, self.q_norm, self.k_norm, self.qk_norm_eps, cos, sin,

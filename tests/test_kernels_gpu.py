@@ -332,6 +332,59 @@ def test_gemm_of_17_to_128_rows_with_norm_taken_apart(ops, w_dtype, m, h, n2, k,
         ops.gemm_mid_tune(True, 0, 0)
 
 
+@pytest.mark.parametrize("m,nq,nkv,d,k,splits,begun", [(17, 4, 2, 64, 256, 0, False), (64, 32, 8, 128, 4096, 0, True), (100, 6, 2, 32, 1024, 2, True),
+                                                       (128, 8, 8, 128, 512, 1, False)])
+def test_qkv_product_of_17_to_128_rows_with_head_preparation(ops, m, nq, nkv, d, k, splits, begun):
+    """The q/k/v product whose K splits' sums are added up by the kernel that normalises and rotates the heads
+    and writes k and v into the pages, against the product, qk_prep and the plain formulas one after the other."""
+    g = torch.Generator().manual_seed(m + nq + d + k)
+    n, page, pages = (nq + 2 * nkv) * d, 16, 12
+    h = torch.randn(m, k, generator=g) * 2
+    gamma = 1 + 0.2 * torch.randn(k, generator=g)
+    w = (torch.randn(n, k, generator=g) / math.sqrt(k)).bfloat16()
+    qw, kw = (1 + 0.2 * torch.randn(d, generator=g)).bfloat16(), (1 + 0.2 * torch.randn(d, generator=g)).bfloat16()
+    positions = torch.randint(0, 500, (m,), generator=g)
+    inv_freq = 1.0 / (10000.0 ** (torch.arange(0, d, 2).float() / d))
+    angle = positions.float()[:, None] * inv_freq[None, :]
+    cos, sin = dev(angle.cos().contiguous()), dev(angle.sin().contiguous())
+    slots = torch.randperm(pages * page, generator=g)[:m].to(torch.int32)
+    eps, norm_eps = 1e-6, 1e-5
+    if begun:     # the input is a norm begun before: x = bf16(h * gamma) and partial sums of h^2
+        x = (h * gamma).bfloat16()
+        parts = 3
+        sumsq = torch.stack([h[:, i::parts].square().sum(-1) for i in range(parts)]).contiguous()
+        source = x.double() * torch.rsqrt(h.double().square().mean(-1, keepdim=True) + norm_eps)
+    else:
+        x, sumsq = h.bfloat16(), None
+        source = x.double()
+    y = source @ w.double().T
+
+    def rms(v, weight):
+        return weight.double() * v * torch.rsqrt(v.square().mean(-1, keepdim=True) + eps)
+
+    def rotate(v):
+        c, s_ = angle.cos().double()[:, None, :], angle.sin().double()[:, None, :]
+        a, b = v[..., : d // 2], v[..., d // 2:]
+        return torch.cat((a * c - b * s_, b * c + a * s_), -1)
+
+    q_want = rotate(rms(y[:, : nq * d].view(m, nq, d), qw))
+    k_want = rotate(rms(y[:, nq * d: (nq + nkv) * d].view(m, nkv, d), kw))
+    v_want = y[:, (nq + nkv) * d:].view(m, nkv, d)
+    qkv = torch.zeros(m, n, device="cuda", dtype=torch.bfloat16)
+    k_pages = torch.zeros(pages, nkv, page, d, device="cuda", dtype=torch.bfloat16)
+    v_pages = torch.zeros(pages, nkv, d, page, device="cuda", dtype=torch.bfloat16)
+    ops.gemm_mid_tune(True, 0, splits)
+    try:
+        ops.gemm_mid_qk_prep(qkv, dev(x), dev(w), None if sumsq is None else dev(sumsq), norm_eps, nq, nkv, d, dev(qw), dev(kw), eps,
+                             cos, sin, k_pages, v_pages, dev(slots), page)
+    finally:
+        ops.gemm_mid_tune(True, 0, 0)
+    close_in_norm(qkv[:, : nq * d], q_want.reshape(m, nq * d), 1e-2)
+    pg, off = (slots // page).long(), (slots % page).long()
+    close_in_norm(k_pages.cpu()[pg, :, off, :], k_want, 1e-2)
+    close_in_norm(v_pages.cpu()[pg, :, :, off], v_want, 1e-2)
+
+
 @pytest.mark.parametrize("w_dtype", DTYPES)
 @pytest.mark.parametrize("m,n,k", [(1, 64, 96), (8, 331, 160), (17, 200, 96), (64, 6144, 4096), (33, 48, 264)])
 def test_gemm_with_fused_rmsnorm_input(ops, w_dtype, m, n, k, all_rows_in_own_kernel):
