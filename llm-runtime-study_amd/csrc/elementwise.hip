@@ -174,8 +174,15 @@ __global__ __launch_bounds__(NORM_BEGIN_COLUMNS / 4) void split_add_norm_begin_k
   if (c < hidden) {
     const int64_t at = (int64_t)row * hidden + c;
     floatx4 v = *(const floatx4*)(x + at);
-    floatx4 y = *(const floatx4*)(sums + at);
-    for (int sp = 1; sp < splits; ++sp) y += *(const floatx4*)(sums + ((int64_t)sp * rows) * hidden + at);
+    floatx4 y = floatx4{0.f, 0.f, 0.f, 0.f};
+    for (int sp0 = 0; sp0 < splits; sp0 += 8) {       // eight splits asked for at a time (usually all there are)
+      floatx4 part[8];
+#pragma unroll
+      for (int i = 0; i < 8; ++i)
+        part[i] = sp0 + i < splits ? *(const floatx4*)(sums + ((int64_t)(sp0 + i) * rows) * hidden + at) : floatx4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int i = 0; i < 8; ++i) y += part[i];
+    }
     v += y;
     *(floatx4*)(x + at) = v;
     bf16x4 nx;
@@ -393,14 +400,25 @@ __global__ __launch_bounds__(256) void qk_prep_vec_kernel(T* __restrict__ qkv, i
 #pragma unroll
     for (int e = 0; e < VE; ++e) a[e] = b[e] = 0.f;
     const float* from = sums + (int64_t)token * sum_columns + (int64_t)head * d;
-    for (int sp = 0; sp < splits; ++sp, from += (int64_t)tokens * sum_columns) {
-      float pa[VE], pb[VE];
-      load_floats<float, VE>(from + VE * j, pa);
-      load_floats<float, VE>(from + half + VE * j, pb);
+    const int64_t apart = (int64_t)tokens * sum_columns;
+    for (int sp0 = 0; sp0 < splits; sp0 += 4) {       // four splits asked for at a time: one trip to memory, not four
+      float pa[4][VE], pb[4][VE];
 #pragma unroll
-      for (int e = 0; e < VE; ++e) {
-        a[e] += pa[e];
-        b[e] += pb[e];
+      for (int i = 0; i < 4; ++i) {
+        if (sp0 + i < splits) {
+          load_floats<float, VE>(from + (sp0 + i) * apart + VE * j, pa[i]);
+          load_floats<float, VE>(from + (sp0 + i) * apart + half + VE * j, pb[i]);
+        }
+      }
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        if (sp0 + i < splits) {
+#pragma unroll
+          for (int e = 0; e < VE; ++e) {
+            a[e] += pa[i][e];
+            b[e] += pb[i][e];
+          }
+        }
       }
     }
   } else {
