@@ -57,12 +57,10 @@ __global__ void rmsnorm_kernel(TO* __restrict__ out, float* __restrict__ x, cons
 
 // The same with the row held in registers: every thread owns up to VEC chunks of 4 values, read
 // once with 16-byte loads; for hidden % 4 == 0 and hidden <= 4 * VEC * threads.
-// sums != null: the addend is the sum over `splits` float32 matrices [splits, gridDim.x, hidden] (what the K
-// splits of a matrix product left), added in split order.
 template <typename TW, typename TO, int VEC>
 __global__ void rmsnorm_vec_kernel(TO* __restrict__ out, float* __restrict__ x, const bf16* __restrict__ add,
                                    const TW* __restrict__ weight, const int* __restrict__ rows,
-                                   int hidden, float eps, const float* __restrict__ sums = nullptr, int splits = 0) {
+                                   int hidden, float eps) {
   __shared__ float scratch[16];
   const int64_t src_row = rows ? rows[blockIdx.x] : blockIdx.x;
   floatx4* src = (floatx4*)(x + src_row * hidden);
@@ -78,11 +76,6 @@ __global__ void rmsnorm_vec_kernel(TO* __restrict__ out, float* __restrict__ x, 
         const bf16x4 y = *(const bf16x4*)(add + src_row * hidden + c * 4);
 #pragma unroll
         for (int i = 0; i < 4; ++i) v[j][i] += (float)y[i];
-        src[c] = v[j];
-      } else if (sums) {
-        floatx4 y = *(const floatx4*)(sums + src_row * hidden + c * 4);
-        for (int sp = 1; sp < splits; ++sp) y += *(const floatx4*)(sums + ((int64_t)sp * gridDim.x + src_row) * hidden + c * 4);
-        v[j] += y;
         src[c] = v[j];
       }
 #pragma unroll
@@ -136,27 +129,6 @@ static int launch_rmsnorm(void* out, int out_dtype, float* x, const bf16* add, c
 LRS_API int lrs_rmsnorm(void* out, int out_dtype, const float* x, const void* weight, int w_dtype,
                         const int* rows, int n_rows, int hidden, float eps, void* stream) {
   return launch_rmsnorm(out, out_dtype, (float*)x, nullptr, weight, w_dtype, rows, n_rows, hidden, eps, stream);
-}
-
-// x [n_rows, hidden] float32 += sums[0] + ... + sums[splits - 1] (each [n_rows, hidden] float32), then
-// out = RMSNorm(x).  For rows the register-resident kernel takes: hidden % 4 == 0 and at most 8192.
-LRS_API int lrs_split_add_rmsnorm(void* out, int out_dtype, float* x, const float* sums, int splits, const void* weight,
-                                  int w_dtype, int n_rows, int hidden, float eps, void* stream) {
-  LRS_REQUIRE(n_rows > 0 && hidden > 0 && splits > 0 && sums != nullptr, "split_add_rmsnorm: rows=%d hidden=%d splits=%d must be positive", n_rows, hidden, splits);
-  LRS_REQUIRE(eps > 0.f, "split_add_rmsnorm: eps must be positive");
-  LRS_REQUIRE(hidden % 4 == 0 && hidden <= 4 * 4 * 512 && ((uintptr_t)x % 16) == 0 && ((uintptr_t)sums % 16) == 0,
-              "split_add_rmsnorm: needs hidden %% 4 == 0, hidden <= 8192 and 16-byte aligned rows (hidden=%d)", hidden);
-  const int threads = hidden <= 1024 ? 64 : (hidden <= 4096 ? 256 : 512);
-  hipStream_t s = (hipStream_t)stream;
-#define LAUNCH_SPLIT(TW, TO) \
-  rmsnorm_vec_kernel<TW, TO, 4><<<n_rows, threads, 0, s>>>((TO*)out, x, nullptr, (const TW*)weight, nullptr, hidden, eps, sums, splits)
-  if (w_dtype == LRS_F32 && out_dtype == LRS_F32) LAUNCH_SPLIT(float, float);
-  else if (w_dtype == LRS_BF16 && out_dtype == LRS_BF16) LAUNCH_SPLIT(bf16, bf16);
-  else if (w_dtype == LRS_F32 && out_dtype == LRS_BF16) LAUNCH_SPLIT(float, bf16);
-  else if (w_dtype == LRS_BF16 && out_dtype == LRS_F32) LAUNCH_SPLIT(bf16, float);
-  else return lrs_fail("split_add_rmsnorm: unknown dtypes %d/%d", w_dtype, out_dtype);
-#undef LAUNCH_SPLIT
-  return lrs_check_launch("split_add_rmsnorm");
 }
 
 // The first half of "add the K splits' sums to the residual stream, then RMSNorm", spread over rows x 1,024

@@ -1238,28 +1238,6 @@ LRS_API int lrs_gemm_norm_chain(void* out, int mode, const void* a, const void* 
   return lrs_check_launch("gemm_norm_chain");
 }
 
-// Defined beside the norm kernels: x [rows, hidden] += the sum over `splits` of sums[split, rows, hidden],
-// then out = RMSNorm(x) with `weight`.
-extern "C" int lrs_split_add_rmsnorm(void* out, int out_dtype, float* x, const float* sums, int splits, const void* weight,
-                                     int w_dtype, int n_rows, int hidden, float eps, void* stream);
-
-// A product of 17..128 rows that adds into the float32 residual stream, with the RMSNorm that follows:
-// residual [M, N] += a [M, K] w[N, K]^T, then normed [M, N] = RMSNorm(residual) with norm_weight and eps.
-// The sums of the product's K splits go straight into the kernel that adds and normalises: one launch
-// less and no rounding of the product to bf16 on the way.
-LRS_API int lrs_gemm_mid_add_rmsnorm(void* normed, int normed_dtype, float* residual, const void* a, const void* w,
-                                     const void* norm_weight, int norm_weight_dtype, int m, int n, int k, int lda,
-                                     float eps, void* stream) {
-  LRS_REQUIRE(m > 16 && m <= 128 && n > 0 && k > 0, "gemm_mid_add_rmsnorm: takes 17..128 rows, got m=%d n=%d k=%d", m, n, k);
-  LRS_REQUIRE(k % 256 == 0 && n % 16 == 0 && lda >= k && lda % 8 == 0 && ((uintptr_t)a % 16 == 0) && ((uintptr_t)w % 16 == 0) && ((uintptr_t)residual % 16 == 0),
-              "gemm_mid_add_rmsnorm: needs K %% 256 == 0, N %% 16 == 0 and 16-byte aligned rows (n=%d k=%d lda=%d)", n, k, lda);
-  LRS_REQUIRE(eps > 0.f, "gemm_mid_add_rmsnorm: eps must be positive");
-  const int splits = launch_mid<false>(nullptr, OUT_STORE, (const bf16*)a, (const bf16*)w, m, n, k, lda, n, (hipStream_t)stream, true);
-  LRS_REQUIRE(splits > 0, "gemm_mid_add_rmsnorm: the buffer for the sums of the K splits cannot hold %d x %d values", m, n);
-  if (int rc = lrs_check_launch("gemm_mid_add_rmsnorm")) return rc;
-  return lrs_split_add_rmsnorm(normed, normed_dtype, residual, split_sums_buffer(), splits, norm_weight, norm_weight_dtype, m, n, eps, stream);
-}
-
 static bool mid_shape_ok(const void* a, const void* w, int m, int n, int k, int lda) {
   return m > 16 && m <= 128 && n > 0 && k > 0 && k % 256 == 0 && n % 16 == 0 && lda >= k && lda % 8 == 0 && ((uintptr_t)a % 16 == 0) &&
          ((uintptr_t)w % 16 == 0);

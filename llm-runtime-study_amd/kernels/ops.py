@@ -64,7 +64,6 @@ _SIGNATURES = {
     "lrs_gemm_mid_scaled": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_int, c_float, c_void_p]),
     "lrs_gemm_mid_add_norm_begin": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p]),
     "lrs_norm_begin_parts": (c_int, [c_int]),
-    "lrs_gemm_mid_add_rmsnorm": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_float, c_void_p]),
     "lrs_attention": (c_int, [c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p,
                               c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_void_p]),
     "lrs_attention_decode": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p,
@@ -367,24 +366,6 @@ def gemm_mid_takes(dtype: torch.dtype, m: int, n: int, k: int, most: int = 128) 
     """Whether a product of m rows (at most `most`) can go to the kernel for 17..128 rows (weights streamed
     once, activations shared through LDS), which also writes the gated activation itself."""
     return dtype == torch.bfloat16 and 16 < m <= min(most, 128) and k % 256 == 0 and n % 16 == 0 and gemm_mid_enabled()
-
-
-def gemm_mid_add_rmsnorm(normed: torch.Tensor, residual: torch.Tensor, a: torch.Tensor, w: torch.Tensor,
-                         norm_weight: torch.Tensor, eps: float) -> None:
-    """residual (float32 [M, N]) += a @ w.T, then normed = RMSNorm(residual) with norm_weight: the product
-    of 17..128 bf16 rows, its residual add and the norm that follows, the sums of the product's K splits going
-    straight into the kernel that adds and normalises."""
-    m, k = a.shape
-    n = w.shape[0]
-    _need(gemm_mid_takes(w.dtype, m, n, k) and a.dtype == torch.bfloat16, "gemm_mid_add_rmsnorm: takes bf16 products of 17..128 rows, K % 256 == 0, N % 16 == 0")
-    _need(w.dim() == 2 and w.is_contiguous() and w.shape[1] == k, f"gemm_mid_add_rmsnorm: weight must be contiguous [N, {k}]")
-    _need(residual.dtype == torch.float32 and residual.is_contiguous() and residual.shape == (m, n), f"gemm_mid_add_rmsnorm: residual must be contiguous float32 [{m}, {n}]")
-    _need(normed.is_contiguous() and normed.shape == (m, n), f"gemm_mid_add_rmsnorm: normed must be contiguous [{m}, {n}]")
-    _need(norm_weight.is_contiguous() and norm_weight.numel() == n and eps > 0, f"gemm_mid_add_rmsnorm: norm weight must hold {n} values and eps be positive")
-    _need(n <= 8192, "gemm_mid_add_rmsnorm: rows of at most 8192 values")
-    _check(library().lrs_gemm_mid_add_rmsnorm(_dev(normed, "normed"), dtype_code(normed.dtype), _dev(residual, "residual"), _dev(a, "a"),
-                                              _dev(w, "w"), _dev(norm_weight, "norm_weight"), dtype_code(norm_weight.dtype), m, n, k,
-                                              _rows(a, "a"), eps, _stream()))
 
 
 def norm_begin_parts(n: int) -> int:

@@ -269,29 +269,6 @@ def test_gemm_of_17_to_64_rows(ops, m, n, k, waves, splits):
 
 
 @pytest.mark.parametrize("w_dtype", DTYPES)
-@pytest.mark.parametrize("m,n,k,splits", [(17, 64, 256, 0), (40, 208, 1024, 2), (64, 4096, 4096, 0), (33, 1040, 3328, 3), (48, 5120, 512, 1), (90, 208, 1024, 2), (128, 4096, 4096, 0)])
-def test_gemm_of_17_to_64_rows_with_residual_add_and_norm(ops, w_dtype, m, n, k, splits):
-    """residual += x W^T and the RMSNorm of the new residual, the K splits' sums added inside the norm kernel."""
-    g = torch.Generator().manual_seed(m + n + k)
-    a = torch.randn(m, k, generator=g).bfloat16()
-    w = (torch.randn(n, k, generator=g) / math.sqrt(k)).bfloat16()
-    residual = torch.randn(m, n, generator=g) * 2
-    gamma = (1 + 0.2 * torch.randn(n, generator=g)).to(w_dtype)
-    eps = 1e-5
-    updated = residual.double() + a.double() @ w.double().T
-    want = gamma.double() * updated * torch.rsqrt(updated.square().mean(-1, keepdim=True) + eps)
-    out = dev(residual.clone())
-    normed = torch.empty(m, n, device="cuda", dtype=torch.bfloat16)
-    ops.gemm_mid_tune(True, 0, splits)
-    try:
-        ops.gemm_mid_add_rmsnorm(normed, out, dev(a), dev(w), dev(gamma), eps)
-    finally:
-        ops.gemm_mid_tune(True, 0, 0)
-    torch.testing.assert_close(out.cpu().double(), updated, rtol=1e-4, atol=1e-4)
-    close_in_norm(normed, want, 5e-3)
-
-
-@pytest.mark.parametrize("w_dtype", DTYPES)
 @pytest.mark.parametrize("m,h,n2,k,swiglu,splits", [(17, 256, 64, 256, False, 0), (40, 512, 208, 1024, True, 2), (64, 4096, 6144, 4096, False, 0),
                                                      (100, 1024, 2048, 3328, True, 3), (128, 4096, 24576, 512, True, 0)])
 def test_gemm_of_17_to_128_rows_with_norm_taken_apart(ops, w_dtype, m, h, n2, k, swiglu, splits):
