@@ -6,6 +6,9 @@
 //   seed and on how many tokens it has drawn, never on the other rows of the batch.
 //   Entries equal to -inf (filtered out beforehand) are never chosen.
 #include "common.h"
+#include "no_alloc.h"
+
+#include <mutex>
 
 __device__ __forceinline__ uint32_t mix32(uint32_t x) {
   x ^= x >> 16;
@@ -166,6 +169,62 @@ LRS_API int lrs_choose_tokens_split(int* out, const float* logits, int64_t row_s
   if (lrs_check_launch("choose_tokens_part")) return 1;
   choose_token_final_kernel<<<rows, WAVE, 0, (hipStream_t)stream>>>(out, part_value, part_index, parts);
   return lrs_check_launch("choose_tokens_final");
+}
+
+// ---- The two-pass choice for callers that cannot allocate (declared in no_alloc.h).
+// Its scratch, the best (value, index) of every slice of every row, lies in a file-scope device array
+// instead of a buffer that the caller brings.  Every GPU of the process holds a copy of the array, at
+// an address of its own, until the process ends; host code never uses the array's name as an address
+// but asks the runtime once per device (choose_scratch_of) and passes the answer to the kernels.
+// Nothing in the array has to start at zero: the first pass writes every element the second reads.
+// Calls that overlap on one GPU (two streams, two threads) share the array and race.
+static __device__ __align__(256) unsigned char choose_scratch[LRS_CHOOSE_STATIC_MAX_PARTS * 8];
+
+constexpr int CHOOSE_MAX_DEVICES = 64;
+static void* g_choose_scratch[CHOOSE_MAX_DEVICES] = {};
+static std::mutex g_choose_scratch_lock;
+
+// The address of the current device's copy of choose_scratch, asked from the runtime the first time.
+static int choose_scratch_of(void** address) {
+  int device = -1;
+  hipError_t err = hipGetDevice(&device);
+  if (err != hipSuccess) return lrs_fail("choose_tokens_static: hipGetDevice: %s", hipGetErrorString(err));
+  if (device < 0 || device >= CHOOSE_MAX_DEVICES) return lrs_fail("choose_tokens_static: device %d is beyond the %d this library keeps scratch for", device, CHOOSE_MAX_DEVICES);
+  std::lock_guard<std::mutex> hold(g_choose_scratch_lock);
+  if (!g_choose_scratch[device]) {
+    void* found = nullptr;
+    err = hipGetSymbolAddress(&found, HIP_SYMBOL(choose_scratch));
+    if (err != hipSuccess || !found) return lrs_fail("choose_tokens_static: hipGetSymbolAddress: %s", hipGetErrorString(err));
+    g_choose_scratch[device] = found;
+  }
+  *address = g_choose_scratch[device];
+  return 0;
+}
+
+LRS_API int lrs_choose_tokens_static_init() {
+  void* unused = nullptr;
+  return choose_scratch_of(&unused);
+}
+
+LRS_API int lrs_choose_tokens_static_max_parts() { return LRS_CHOOSE_STATIC_MAX_PARTS; }
+
+LRS_API int lrs_choose_tokens_static(int* out, const float* logits, int64_t row_stride, int rows, int vocab,
+                                     const float* temperature, const uint64_t* seeds, const uint32_t* counters,
+                                     int parts, void* stream) {
+  LRS_REQUIRE(rows > 0 && vocab > 0 && parts > 0, "choose_tokens_static: rows=%d vocab=%d parts=%d must be positive", rows, vocab, parts);
+  LRS_REQUIRE(row_stride >= vocab, "choose_tokens_static: row stride below vocab");
+  LRS_REQUIRE(out && logits, "choose_tokens_static: out and logits are required");
+  LRS_REQUIRE((int64_t)rows * parts <= LRS_CHOOSE_STATIC_MAX_PARTS,
+              "choose_tokens_static: rows x parts = %d x %d is more than the %d slices the static scratch holds", rows, parts, LRS_CHOOSE_STATIC_MAX_PARTS);
+  void* scratch = nullptr;
+  if (int rc = choose_scratch_of(&scratch)) return rc;
+  float* part_value = (float*)scratch;
+  int* part_index = (int*)((unsigned char*)scratch + (size_t)LRS_CHOOSE_STATIC_MAX_PARTS * 4);
+  choose_token_part_kernel<<<dim3(parts, rows), 256, 0, (hipStream_t)stream>>>(part_value, part_index, logits, row_stride, vocab,
+                                                                               parts, temperature, seeds, counters);
+  if (lrs_check_launch("choose_tokens_static_part")) return 1;
+  choose_token_final_kernel<<<rows, WAVE, 0, (hipStream_t)stream>>>(out, part_value, part_index, parts);
+  return lrs_check_launch("choose_tokens_static_final");
 }
 
 // out[r] = chosen token of row r.  temperature == nullptr or temperature[r] == 0: greedy.

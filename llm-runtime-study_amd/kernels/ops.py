@@ -77,6 +77,9 @@ _SIGNATURES = {
     "lrs_attention_prefill_group_for": (c_int, [c_int]),
     "lrs_choose_tokens": (c_int, [c_void_p, c_void_p, c_int64, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p]),
     "lrs_choose_tokens_split": (c_int, [c_void_p, c_void_p, c_int64, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p]),
+    "lrs_choose_tokens_static": (c_int, [c_void_p, c_void_p, c_int64, c_int, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p]),
+    "lrs_choose_tokens_static_init": (c_int, []),
+    "lrs_choose_tokens_static_max_parts": (c_int, []),
     "lrs_filter_logits": (c_int, [c_void_p, c_int64, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p]),
 }
 
@@ -98,6 +101,7 @@ def library():
         if torch.cuda.is_available():
             torch.cuda.init()
             _check(lib.lrs_gemm_prepare())   # device scratch is made now, never inside a step
+            _check(lib.lrs_choose_tokens_static_init())
     return _lib
 
 
@@ -755,6 +759,23 @@ def choose_tokens(out: torch.Tensor, logits: torch.Tensor, temperature=None, see
                                                  _dev(scratch[0], "part_value"), _dev(scratch[1], "part_index"), parts, _stream()))
         return
     _check(library().lrs_choose_tokens(out_pointer, _dev(logits, "logits", torch.float32), stride, rows, vocab, *args, _stream()))
+
+
+def choose_tokens_static(out: torch.Tensor, logits: torch.Tensor, parts: int, temperature=None, seeds=None, counters=None) -> None:
+    """choose_tokens() in its two-pass form (`parts` slices a row) for callers that must not allocate: the
+    slices' results go to a fixed array inside the library (rows * parts at most
+    lrs_choose_tokens_static_max_parts()), so nothing is allocated here or there.  Calls that overlap on
+    one GPU share that array and race."""
+    rows, vocab = logits.shape
+    _need(out.dtype == torch.int32 and out.numel() >= rows and out.is_contiguous(), "choose_tokens_static: out must be int32 [R]")
+    if temperature is not None:
+        _need(temperature.dtype == torch.float32 and temperature.numel() >= rows, "choose_tokens_static: temperature must be float32 [R]")
+        _need(seeds is not None and seeds.dtype == torch.int64 and seeds.numel() >= rows, "choose_tokens_static: seeds must be int64 [R]")
+        _need(counters is not None and counters.dtype == torch.int32 and counters.numel() >= rows, "choose_tokens_static: counters must be int32 [R]")
+    _check(library().lrs_choose_tokens_static(
+        _dev(out, "out"), _dev(logits, "logits", torch.float32), _rows(logits, "logits"), rows, vocab,
+        None if temperature is None else _dev(temperature, "temperature"), None if temperature is None else _dev(seeds, "seeds"),
+        None if temperature is None else _dev(counters, "counters"), parts, _stream()))
 
 
 def filter_logits(logits: torch.Tensor, temperature: torch.Tensor, top_k: torch.Tensor | None, top_p: torch.Tensor | None) -> None:
