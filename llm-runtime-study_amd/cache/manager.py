@@ -16,8 +16,12 @@ back when the request ends, is rolled back, or (windowed groups) when every posi
 the page has left the window of all future queries.
 
 Every admitted request also holds one state slot out of `max_requests`; StateNeed entries
-keep a tensor [max_requests, *shape], zeroed for the slot at admission.  The slot is also
-the request's row in the per-group host block tables.
+keep a tensor [max_requests + 1, *shape], zeroed for the slot at admission.  The slot is also
+the request's row in the per-group host block tables.  The extra last row is the trash slot:
+rows that pad a batch (graph replays) point there, as their keys and values go to the trash
+page, so no request's state is touched by them.  A step that fails must leave no trace:
+snapshot_state() before the forward and restore_state() after a failure put the touched
+rows back, as rollback() does for lengths and pages.
 
 Lengths are host integers (reference mini_llm/cache/lengths.py:8-43): extend() before the
 forward, rollback() if it fails.  The reference reserves a request's whole lifetime at
@@ -45,7 +49,7 @@ class LayerCache:
     group: int | None = None          # index of the paged group (ctx.group(i) has table and slots)
     k_pages: torch.Tensor | None = None
     v_pages: torch.Tensor | None = None
-    state: torch.Tensor | None = None  # [max_requests, *shape] for StateNeed entries
+    state: torch.Tensor | None = None  # [max_requests + 1, *shape] for StateNeed entries (last row: trash slot)
     window: int | None = None
 
 
@@ -105,7 +109,7 @@ class CacheManager:
             elif isinstance(need, StateNeed):
                 self.state_entries.append(position)
                 if allocate_storage:
-                    cache.state = torch.zeros((max_requests, *need.shape), dtype=need.dtype, device=self.device)
+                    cache.state = torch.zeros((max_requests + 1, *need.shape), dtype=need.dtype, device=self.device)
             elif isinstance(need, tuple) and len(need) == 2 and need[0] == "from":
                 source = need[1]
                 if not 0 <= source < position or self.layer_caches[source].group is None:
@@ -157,6 +161,29 @@ class CacheManager:
     def trash_page(self, group: int = 0) -> int:
         """Page that no request owns; padding rows of a padded batch write there."""
         return self.groups[group].pool.num_pages
+
+    @property
+    def trash_slot(self) -> int:
+        """State row that no request owns; padding rows of a padded batch point there."""
+        return self.max_requests
+
+    def snapshot_state(self, requests) -> list:
+        """Copies of the state rows of `requests` (every StateNeed entry), to put back with restore_state()
+        if the step that is about to run fails.  Empty, and free, for a model without such entries."""
+        if not self.state_entries:
+            return []
+        slots = [request.slot for request in requests]
+        kept = []
+        for position in self.state_entries:
+            state = self.layer_caches[position].state
+            if state is not None:
+                kept.append((state, slots, state[slots].clone()))
+        return kept
+
+    @staticmethod
+    def restore_state(snapshot: list) -> None:
+        for state, slots, rows in snapshot:
+            state[slots] = rows
 
     def pages_for(self, group: int, tokens: int, max_step_tokens: int | None = None) -> int:
         """Pages a request of `tokens` positions can hold at once in `group`."""

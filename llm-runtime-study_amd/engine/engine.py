@@ -19,7 +19,7 @@ from ..cache import CacheManager
 from ..errors import EngineError
 from ..sampling import Sampler, SamplingConfig
 from ..text import TextTokenizer
-from ..config import load_config
+from ..config import chat_template_for, load_config
 from .loading import load_model, random_model, resolve_device, resolve_dtype
 from .scheduler import BatchScheduler, GenerationEvent, generate as _generate
 from .step import ModelRunner
@@ -58,18 +58,20 @@ class Engine:
     # ---------------------------------------------------------------- loading
     @classmethod
     def from_model_dir(cls, model_dir, *, device="auto", dtype="auto", max_seq_len: int = 4096, max_batch_size: int = 1,
-                       cache_backend: str = "paged", use_cuda_graph: bool = True, **options) -> "Engine":
-        """Load config.json and the safetensors weights of `model_dir` onto the GPU."""
+                       cache_backend: str = "paged", use_cuda_graph: bool = True, stored_precision: bool = False,
+                       **options) -> "Engine":
+        """Load config.json and the safetensors weights of `model_dir` onto the GPU.  The tensors must be
+        stored in the configuration's `torch_dtype` unless `stored_precision` is set (see load_model)."""
         started = time.perf_counter()
         config = load_config(model_dir)
         config.validate_context_length(max_seq_len)
         selected_device, selected_dtype = resolve_device(device), resolve_dtype(dtype)
-        config, model = load_model(model_dir, selected_dtype, selected_device, config)
-        tokenizer = TextTokenizer.from_model_dir(model_dir, config.vocab_size)
+        config, model = load_model(model_dir, selected_dtype, selected_device, config, stored_precision)
+        tokenizer = TextTokenizer.from_model_dir(model_dir, config.vocab_size, chat_template_for(config))
         engine = cls(config, model, device=selected_device, dtype=selected_dtype, max_seq_len=max_seq_len,
                      max_batch_size=max_batch_size, cache_backend=cache_backend, use_cuda_graph=use_cuda_graph,
                      tokenizer=tokenizer, **options)
-        engine._reload = lambda dtype: load_model(model_dir, dtype, selected_device, config)[1]
+        engine._reload = lambda dtype: load_model(model_dir, dtype, selected_device, config, stored_precision)[1]
         engine.synchronize()
         engine.load_seconds = time.perf_counter() - started
         return engine

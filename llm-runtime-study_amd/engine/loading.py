@@ -45,13 +45,17 @@ def resolve_dtype(requested="auto") -> torch.dtype:
     raise EngineError(f"unsupported dtype {requested!r}; expected auto, {', '.join(DTYPES)}")
 
 
-def load_model(model_dir, dtype: torch.dtype, device, config=None) -> tuple:
-    """(typed configuration, bound DecoderModel) of a model folder."""
+def load_model(model_dir, dtype: torch.dtype, device, config=None, stored_precision: bool = False) -> tuple:
+    """(typed configuration, bound DecoderModel) of a model folder.
+
+    The checkpoint's floating tensors must be stored in the configuration's dtype, as in the reference
+    (mini_llm/checkpoint.py:478-481); `stored_precision=True` takes them in whatever floating dtype they
+    are stored (a bfloat16 model with 32-bit norm weights, say) and keeps that precision."""
     config = load_config(model_dir) if config is None else config
     spec = spec_for(config)
     model = DecoderModel(spec)
     checkpoint = Checkpoint.from_model_dir(model_dir)
-    weights = load(checkpoint, model.tensors(), config.model_type, device)
+    weights = load(checkpoint, model.tensors(), config.model_type, device, None if stored_precision else spec.checkpoint_dtype)
     checkpoint.close()
     model.bind(weights, dtype)
     return config, model

@@ -33,7 +33,7 @@ from typing import Callable, Sequence
 
 from ..errors import GenerationError, SamplingError
 from ..sampling import SamplingConfig, SamplingRow, request_seed
-from ..text import ChatMessage, IncrementalTextDecoder
+from ..text import ChatMessage, TextStream
 from .step import StepEntry
 
 
@@ -68,7 +68,7 @@ class _Running:
     sampling: SamplingConfig
     seed: int
     cache: object
-    decoder: IncrementalTextDecoder
+    decoder: TextStream
     fed: int = 0                      # prompt tokens already run
     produced: int = 0                 # tokens sampled so far
     next_token: int | None = None     # sampled, not yet run
@@ -199,7 +199,7 @@ class BatchScheduler:
             self._waiting.popleft()
             cache = self.cache.admit(head.index, reserve_tokens=lifetime, max_step_tokens=self.max_step_tokens)
             self._running.append(_Running(head.index, head.prompt, head.output_limit, head.max_new_tokens, head.sampling,
-                                          request_seed(head.sampling), cache, IncrementalTextDecoder(self.tokenizer)))
+                                          request_seed(head.sampling), cache, TextStream(self.tokenizer)))
 
     def _build_batch(self):
         budget = self.max_step_tokens
@@ -263,7 +263,7 @@ class BatchScheduler:
     def _finish_step(self, rows, tokens, seconds, events) -> None:
         finished = set()
         for (request, _), token in zip(rows, tokens):
-            delta = request.decoder.add(token)
+            delta = request.decoder.push(token)
             request.produced += 1
             request.tokens.append(token)
             reason = None

@@ -120,7 +120,8 @@ class ModelRunner:
         # decode-only steps are captured in a HIP graph per padded batch size and replayed
         self.use_graph = use_graph and model.graph_safe()
         self._graphs: dict[tuple, tuple] = {}   # (bucket, length class) -> (handle, arena generation, logits tensor)
-        self.graph_replays = 0
+        self.graph_replays = 0     # steps (or launches of several steps) served by replaying a graph
+        self.graph_captures = 0    # ... and those that ran eagerly and were captured on the way
         # query groups for the ragged attention kernel: at most `query_group` consecutive tokens of one request
         self.query_group = ops.attention_prefill_group()   # the most; a step of few tokens uses smaller ones
         # The metadata of a step is one int32 buffer whose layout follows the step's own numbers of
@@ -233,12 +234,15 @@ class ModelRunner:
         if total > self.max_step_tokens:
             raise GenerationError(f"a step holds {total} tokens but at most {self.max_step_tokens} fit")
 
-    def prepare(self, entries: Sequence[StepEntry], pad_to: int = 0) -> StepContext:
+    def prepare(self, entries: Sequence[StepEntry], pad_to: int = 0, ahead: int = 0) -> StepContext:
         """Fill the host metadata for `entries` (caches already extended) and copy it over.
 
         With `pad_to` (decode-only steps) the batch is filled up to that many rows with rows that
         belong to no request: token 0 at position 0, written to and read from the trash page, and
-        logits are produced for every row, so that the step's shape depends on `pad_to` alone."""
+        logits are produced for every row, so that the step's shape depends on `pad_to` alone.
+        `ahead` (decode-only steps): the caches were extended by that many positions more than this
+        step's one, for the steps that follow it in the same launch; positions and context lengths are
+        this step's, the block tables hold the later pages too."""
         cache, page = self.cache, self.cache.page_size
         ctx = StepContext(self)
         self._next_staging()
@@ -251,7 +255,7 @@ class ModelRunner:
             # one token per request (a decode step): whole arrays at once, no loop over tokens
             cursor = len(entries)
             count = self._counting[:cursor + 1]
-            lengths = np.fromiter((entry.cache.length for entry in entries), dtype=np.int32, count=cursor)
+            lengths = np.fromiter((entry.cache.length - ahead for entry in entries), dtype=np.int32, count=cursor)
             ctx.host_slots = [entry.cache.slot for entry in entries]
             ids[:cursor] = [entry.tokens[0] for entry in entries]
             pos[:cursor] = lengths - 1
@@ -265,6 +269,8 @@ class ModelRunner:
             ctx.host_q_lens = [1] * cursor
             ctx.host_positions = pos[:cursor].tolist()
         else:
+            if ahead:
+                raise GenerationError("only a decode-only step can be prepared ahead of later steps")
             for r, entry in enumerate(entries):
                 n = len(entry.tokens)
                 start = entry.cache.length - n
@@ -296,7 +302,7 @@ class ModelRunner:
             req[cursor:cursor + extra] = np.arange(real, pad_to, dtype=np.int32)
             cu[real + 1:pad_to + 1] = np.arange(cursor + 1, cursor + extra + 1, dtype=np.int32)
             lens[real:pad_to] = 1
-            slots[real:pad_to] = 0
+            slots[real:pad_to] = cache.trash_slot        # their state, like their keys and values, goes where no request reads
             cursor += extra
         if pad_to:
             rows[:cursor] = np.arange(cursor, dtype=np.int32)
@@ -358,6 +364,7 @@ class ModelRunner:
         self._follow_construction()
         before = [entry.cache.length for entry in entries]
         extended = []
+        states = self.cache.snapshot_state([entry.cache for entry in entries])
         try:
             for entry in entries:
                 self.cache.extend(entry.cache, len(entry.tokens))
@@ -370,14 +377,20 @@ class ModelRunner:
                 h = self.model.forward_hidden(ctx)
                 logits = self.model.logits(ctx, h) if ctx.num_logit_rows else None
         except Exception:
-            for entry, length in zip(extended, before):
-                if not entry.cache.released:
-                    self.cache.rollback(entry.cache, length)
+            self._undo(extended, before, states)
             raise
         for entry in entries:
             self.cache.trim(entry.cache)
         self.steps_run += 1
         return logits
+
+    def _undo(self, extended: Sequence[StepEntry], before: Sequence[int], states: list) -> None:
+        """After a failed step: every cache that was extended back to its length before the step (pages
+        that only the step took go back to the pool) and every per-request state row as it was."""
+        for entry, length in zip(extended, before):
+            if not entry.cache.released:
+                self.cache.rollback(entry.cache, length)
+        self.cache.restore_state(states)
 
     # ------------------------------------------------- several decode steps, one launch
     MAX_DECODE_STEPS = 8
@@ -390,14 +403,19 @@ class ModelRunner:
     decode_steps_sample = True     # decode_steps() also draws from filtered, tempered distributions
 
     def decode_steps(self, entries: Sequence[StepEntry], steps: int, sampling: Sequence | None = None) -> list[list[int]]:
-        """`steps` decode steps of the same requests from one graph launch.
+        """`steps` decode steps of the same requests, the host out of the loop between them.
 
         Each entry brings the one token its request decodes next.  After every step the device itself
         chooses a token for every row (the largest logit; or, for the rows whose entry of `sampling`,
         a list of sampling.SamplingRow, says so, a seeded draw after top-k / top-p filtering, exactly
         as Sampler.choose would), feeds it in as the next token and moves the step's metadata one
-        position on, so the host is not in the loop between steps.  Returns the chosen tokens
-        [steps][entries]; every request's cache is `steps` tokens longer afterwards."""
+        position on.  Returns the chosen tokens [steps][entries]; every request's cache is `steps`
+        tokens longer afterwards, or, after a failure, as long as before.
+
+        The steps run from one graph launch, unless the longest context crosses into another length
+        class on the way (256, 512, 1024, ...): how far decode attention divides the keys follows the
+        class, so the launch ends at the edge and another begins there.  Every step thus runs exactly
+        as it would alone, and the tokens do not depend on how many steps a launch holds."""
         if not 1 <= steps <= self.MAX_DECODE_STEPS:
             raise GenerationError(f"decode_steps takes 1..{self.MAX_DECODE_STEPS} steps, got {steps}")
         self.validate(entries)
@@ -405,40 +423,41 @@ class ModelRunner:
         bucket = self._graph_bucket(entries)
         if not bucket:
             raise GenerationError("decode_steps needs graphs and one token per entry")
+        if sampling is not None and len(sampling) != len(entries):
+            raise GenerationError("decode_steps needs one sampling row per entry")
         before = [entry.cache.length for entry in entries]
-        extended = []
+        states = self.cache.snapshot_state([entry.cache for entry in entries])
+        chosen: list[list[int]] = []
+        current, rows = list(entries), sampling
         try:
-            for entry in entries:
-                self.cache.extend(entry.cache, 1)
-                extended.append(entry)
-            ctx = self.prepare(entries, pad_to=bucket)
-            if steps > 1:
-                for entry in entries:                           # pages of the later positions: the block tables must hold them
-                    self.cache.extend(entry.cache, steps - 1)
-                self._refresh_tables(entries, bucket)
-            sampled = sampling is not None and any(not row.config.greedy for row in sampling)
-            if sampled:
-                if len(sampling) != len(entries):
-                    raise GenerationError("decode_steps needs one sampling row per entry")
-                self._upload_sampling(sampling)
-            chosen = self._run_decode_graph(ctx, bucket, steps, sampled)
+            while len(chosen) < steps:
+                longest = max(entry.cache.length for entry in entries) + 1     # the longest context of the launch's first step
+                reach = length_class(longest)
+                edge = 2 * reach if reach else 256
+                count = min(steps - len(chosen), edge - longest)
+                if chosen:
+                    current = [StepEntry(entry.cache, [token], entry.want) for entry, token in zip(entries, chosen[-1])]
+                    if sampling is not None:
+                        rows = [type(row)(row.config, row.seed, row.counter + len(chosen)) for row in sampling]
+                chosen += self._decode_launch(current, count, rows, bucket)
         except Exception:
-            for entry, length in zip(extended, before):
-                if not entry.cache.released:
-                    self.cache.rollback(entry.cache, length)
+            self._undo(entries, before, states)
             raise
         for entry in entries:
             self.cache.trim(entry.cache)
         self.steps_run += steps
-        return [row[:len(entries)] for row in chosen]
+        return chosen
 
-    def _refresh_tables(self, entries: Sequence[StepEntry], bucket: int) -> None:
-        """Block tables of the step's requests written again (after pages were added) and uploaded."""
-        mb = self.cache.max_blocks
-        slots = [entry.cache.slot for entry in entries]
-        for index, group in enumerate(self.cache.groups):
-            self._host_view(f"table{index}").reshape(bucket, mb)[:len(entries)] = group.host_table[slots]
-        self._upload()
+    def _decode_launch(self, entries: Sequence[StepEntry], steps: int, sampling: Sequence | None, bucket: int) -> list[list[int]]:
+        """One graph launch of `steps` decode steps.  Every cache is lengthened by all `steps` positions
+        first, so the block tables that the launch uploads already hold the pages of the later ones."""
+        for entry in entries:
+            self.cache.extend(entry.cache, steps)
+        ctx = self.prepare(entries, pad_to=bucket, ahead=steps - 1)
+        sampled = sampling is not None and any(not row.config.greedy for row in sampling)
+        if sampled:
+            self._upload_sampling(sampling)
+        return [row[:len(entries)] for row in self._run_decode_graph(ctx, bucket, steps, sampled)]
 
     def _upload_sampling(self, sampling: Sequence) -> None:
         """Temperature, top-p, top-k, draws so far and seed of every row, in one buffer on the device
@@ -486,11 +505,13 @@ class ModelRunner:
                 ops.graph_destroy(handle)
                 raise GenerationError("scratch buffers moved during graph capture")
             graph = self._graphs[key] = (handle, generation, None)
-            self._upload()                                         # the eager run moved the metadata on: start again
-            if sampled:
-                ops.copy_h2d(self._sampling_dev, self._sampling_host, self._sampling_host.numel())
-        ops.graph_launch(graph[0])
-        self.graph_replays += 1
+            # The eager run above was this launch: its tokens are on their way to the host.  Replaying the graph as
+            # well would run every step twice, which keys and values bear (the same values land in the same slots)
+            # but a mixer with state of its own does not.
+            self.graph_captures += 1
+        else:
+            ops.graph_launch(graph[0])
+            self.graph_replays += 1
         torch.cuda.current_stream(self.device).synchronize()
         return [self._chosen_host[i * stride:i * stride + bucket].tolist() for i in range(steps)]
 
@@ -557,8 +578,10 @@ class ModelRunner:
                 ops.graph_destroy(handle)
                 raise GenerationError("scratch buffers moved during graph capture")
             graph = self._graphs[key] = (handle, generation, logits)
-        ops.graph_launch(graph[0])
-        self.graph_replays += 1
+            self.graph_captures += 1     # the eager run was this step (see _run_decode_graph): no replay on top of it
+        else:
+            ops.graph_launch(graph[0])
+            self.graph_replays += 1
         wanted = [r for r, entry in enumerate(entries) for _ in entry.want]   # a place asked twice is given twice
         if not wanted:
             return None
@@ -566,6 +589,9 @@ class ModelRunner:
         return logits[:len(entries)] if wanted == list(range(len(entries))) else logits[wanted]
 
     def drop_graphs(self) -> None:
+        """Destroy every captured graph, after the device has finished with them."""
+        if self._graphs and self.device.type == "cuda":
+            torch.cuda.synchronize(self.device)
         for handle, *_ in self._graphs.values():
             ops.graph_destroy(handle)
         self._graphs.clear()

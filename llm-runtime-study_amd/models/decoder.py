@@ -94,9 +94,9 @@ class DecoderModel:
     def logits(self, ctx, h: torch.Tensor) -> torch.Tensor:
         """float32 logits [n_wanted, V] at the rows of `h` listed in ctx.logit_rows."""
         n = ctx.num_logit_rows
-        try:
+        if getattr(self.final_norm, "has_lazy_form", False):   # the head's product normalises its own input
             x = self.final_norm.forward(ctx, h, rows=ctx.logit_rows, count=n, lazy=True)
-        except TypeError:      # a norm kind without the lazy form
+        else:
             x = self.final_norm.forward(ctx, h, rows=ctx.logit_rows, count=n)
         out = ctx.scratch("logits", (n, self.spec.vocab_size), torch.float32)
         linear(ctx, out, x, self.head)

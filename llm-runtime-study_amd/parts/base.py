@@ -7,7 +7,8 @@ new architecture adds a kind with `register(role, name, cls)` and nothing else c
 
 Roles and what each must provide:
 
-  norm           forward(ctx, h, rows=None) -> x        h float32 [T, H] -> activation dtype
+  norm           forward(ctx, h, rows=None, count=None) -> x    h float32 [T, H] -> activation dtype; with `rows`
+                                                        (int32 on the device) only the `count` rows listed there
   position       tables(ctx) -> (cos, sin) | None       float32 [T, rot/2] for this step's tokens
   mixer          cache_need() -> PagedKVNeed | StateNeed | None
                  forward(ctx, x, residual, cache)       adds its output into residual (float32)
@@ -16,6 +17,8 @@ Roles and what each must provide:
 
 Optional, each announced by a class attribute (a part without it is simply given plain tensors):
 
+  has_lazy_form = True        norm: forward(..., lazy=True) may return a description of the norm (LazyNorm of
+                              parts/linear.py) instead of a tensor; asked for only when the consumer takes one
   takes_lazy_norm = True      mixer / feed_forward: `x` may be a description of the norm (LazyNorm or
                               ScaledRows of parts/linear.py) that its first `linear()` completes
   begins_next_norm = True     mixer / feed_forward: forward(..., then_norm=norm) may return ScaledRows,

@@ -71,11 +71,8 @@ class PreNormBlock(Part):
         lazy = getattr(consumer, "takes_lazy_norm", False)
         if begun is not None:
             return begun if lazy else materialize(ctx, begun)
-        if lazy:
-            try:
-                return norm.forward(ctx, h, lazy=True)
-            except TypeError:      # a norm kind without the lazy form
-                pass
+        if lazy and getattr(norm, "has_lazy_form", False):
+            return norm.forward(ctx, h, lazy=True)
         return norm.forward(ctx, h)
 
 

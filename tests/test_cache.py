@@ -140,7 +140,7 @@ def test_groups_share_needs_and_follow_cache_sources():
     assert caches[0].k_pages.shape == (5, 2, 4, 16)          # one extra page for padding rows
     assert caches[0].v_pages.shape == (5, 2, 16, 4)          # values are transposed inside a page
     assert caches[0].k_pages.data_ptr() != caches[2].k_pages.data_ptr()
-    assert caches[4].state.shape == (3, 3, 5)
+    assert caches[4].state.shape == (3 + 1, 3, 5) and m.trash_slot == 3   # one row beyond the requests' slots: the trash slot
     a = m.admit("a")
     caches[4].state[a.slot] += 1.0
     m.release(a)
@@ -150,6 +150,24 @@ def test_groups_share_needs_and_follow_cache_sources():
         manager(needs=(state, ("from", 0)))
     with pytest.raises(KVCacheError, match="unknown cache need"):
         manager(needs=("pages",))
+
+
+def test_state_rows_are_put_back_after_a_failed_step():
+    state = StateNeed((4,))
+    m = manager(needs=(FULL, state, state), storage=True, page_size=4, num_pages=8)
+    a, b, c = m.admit("a"), m.admit("b"), m.admit("c")
+    for position in (1, 2):
+        m.layer_caches[position].state[:] = torch.arange(4 * 4, dtype=torch.float32).view(4, 4) + 100 * position
+    kept = m.snapshot_state([a, c])
+    before = [m.layer_caches[position].state.clone() for position in (1, 2)]
+    for position in (1, 2):
+        m.layer_caches[position].state[[a.slot, c.slot]] -= 7.0          # what a step's mixers did before the step failed
+        m.layer_caches[position].state[b.slot] += 1.0                    # another request's row: not the failed step's business
+    m.restore_state(kept)
+    for position, old in zip((1, 2), before):
+        now = m.layer_caches[position].state
+        assert torch.equal(now[[a.slot, c.slot]], old[[a.slot, c.slot]]) and torch.equal(now[b.slot], old[b.slot] + 1.0)
+    assert manager(needs=(FULL,)).snapshot_state([]) == []               # a model without state pays nothing
 
 
 @pytest.mark.parametrize("seed", range(6))

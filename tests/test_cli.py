@@ -17,6 +17,7 @@ def test_parser_has_the_reference_options_and_defaults():
     args = cli.build_parser().parse_args(["--model", "m", "--prompt", "hi"])
     assert (args.max_new_tokens, args.max_seq_len, args.temperature, args.top_k, args.top_p, args.seed) == (128, 4096, 0.0, None, 1.0, None)
     assert (args.device, args.dtype, args.interactive, args.thinking, args.no_stream, args.no_metrics) == ("auto", "auto", False, False, False, False)
+    assert args.random_weights is None and cli.build_parser().parse_args(["--model", "m", "--random-weights", "7", "--device", "hip"]).random_weights == 7
     with pytest.raises(SystemExit):
         cli.build_parser().parse_args(["--prompt", "hi"])
 
@@ -35,7 +36,7 @@ def fake_engine(events):
 def test_streams_text_and_prints_metrics(monkeypatch):
     events = [GenerationEvent(5, 0, "Hel", "Hel", None, 0.5, 7), GenerationEvent(6, 1, "lo", "Hello", "max_new_tokens", 0.25, None)]
     engine, calls = fake_engine(events)
-    monkeypatch.setattr(cli, "_engine_from_args", lambda args: engine)
+    monkeypatch.setattr(cli, "open_engine", lambda args: engine)
     out = io.StringIO()
     code = cli.main(["--model", "m", "--prompt", "hi", "--max-new-tokens", "2", "--temperature", "0.7", "--top-k", "5", "--seed", "3"], output=out)
     text = out.getvalue()
@@ -49,7 +50,7 @@ def test_streams_text_and_prints_metrics(monkeypatch):
 def test_prompt_ids_and_no_stream(monkeypatch):
     engine, calls = fake_engine([GenerationEvent(9, 0, "", "", "eos", None, 3)])
     engine.tokenizer = None
-    monkeypatch.setattr(cli, "_engine_from_args", lambda args: engine)
+    monkeypatch.setattr(cli, "open_engine", lambda args: engine)
     out = io.StringIO()
     assert cli.main(["--model", "m", "--prompt-ids", "4, 5,6", "--no-stream", "--no-metrics"], output=out) == 0
     assert calls["prompts"][0] == [4, 5, 6] and out.getvalue() == "9\n"
@@ -59,7 +60,7 @@ def test_typed_errors_exit_with_2(monkeypatch):
     def boom(args):
         raise ConfigError("model directory does not exist: m")
 
-    monkeypatch.setattr(cli, "_engine_from_args", boom)
+    monkeypatch.setattr(cli, "open_engine", boom)
     err = io.StringIO()
     assert cli.main(["--model", "m", "--prompt", "hi"], error=err) == 2
     assert err.getvalue() == "error: model directory does not exist: m\n"
@@ -67,6 +68,56 @@ def test_typed_errors_exit_with_2(monkeypatch):
     assert cli.main(["--model", "m"], error=err) == 2 and "--prompt is required" in err.getvalue()
     err = io.StringIO()
     assert cli.main(["--model", "m", "--prompt", "x", "--temperature", "-1"], error=err) == 2 and "temperature" in err.getvalue()
+
+
+def test_metrics_block_has_the_reference_layout(monkeypatch):
+    """Every line of the block as the reference prints it (mini_llm/cli.py:213-247): two spaces, the name with
+    its colon padded to 21 columns, the value."""
+    events = [GenerationEvent(5, 0, "a", "a", None, 0.5, 3), GenerationEvent(6, 1, "b", "ab", None, 0.5, None),
+              GenerationEvent(7, 2, "c", "abc", "eos", 0.5, None)]
+    engine, _ = fake_engine(events)
+    monkeypatch.setattr(cli, "open_engine", lambda args: engine)
+    out = io.StringIO()
+    assert cli.main(["--model", "m", "--prompt", "hi"], output=out) == 0
+    lines = out.getvalue().split("\n")
+    assert lines[:3] == ["abc", "", "metrics"]
+    assert lines[3:6] == ["  device:              cuda:0", "  dtype:               torch.bfloat16", "  load time:           1.50 s"]
+    assert lines[6:9] == ["  prompt tokens:       3", "  generated tokens:    3", "  cache:               0.05 MiB (48 positions)"]
+    assert lines[9].startswith("  time to first token: ") and lines[9].endswith(" ms")
+    assert lines[10:12] == ["  decode throughput:   2.00 tokens/s", "  stop reason:         eos"]
+
+
+def test_an_answer_without_events_or_without_a_prompt_count_is_an_error(monkeypatch):
+    engine, _ = fake_engine([])
+    monkeypatch.setattr(cli, "open_engine", lambda args: engine)
+    err = io.StringIO()
+    assert cli.main(["--model", "m", "--prompt", "hi"], output=io.StringIO(), error=err) == 2 and "without a terminal event" in err.getvalue()
+    engine, _ = fake_engine([GenerationEvent(5, 0, "a", "a", "eos", 0.5, None)])
+    monkeypatch.setattr(cli, "open_engine", lambda args: engine)
+    err = io.StringIO()
+    assert cli.main(["--model", "m", "--prompt", "hi"], output=io.StringIO(), error=err) == 2 and "prompt-token count" in err.getvalue()
+    err = io.StringIO()
+    assert cli.main(["--model", "m", "--prompt-ids", "4,x"], output=io.StringIO(), error=err) == 2 and "comma-separated integers" in err.getvalue()
+
+
+def test_interactive_goes_on_after_a_failed_prompt(monkeypatch):
+    from llm_runtime_study_amd.errors import GenerationError
+
+    answers = iter([GenerationError("prompt has 9 tokens but model context limit is 4"), [GenerationEvent(5, 0, "fine", "fine", "eos", None, 2)]])
+
+    def generate(prompts, **options):
+        item = next(answers)
+        if isinstance(item, Exception):
+            raise item
+        return iter([(0, e) for e in item])
+
+    engine, _ = fake_engine([])
+    engine.generate = generate
+    monkeypatch.setattr(cli, "open_engine", lambda args: engine)
+    out, err = io.StringIO(), io.StringIO()
+    code = cli.main(["--model", "m", "--interactive", "--no-metrics", "--prompt", "first"], input_stream=io.StringIO("second\n"), output=out, error=err)
+    assert code == 0 and err.getvalue() == "error: prompt has 9 tokens but model context limit is 4\n"
+    assert "you> first" in out.getvalue() and "assistant> fine" in out.getvalue()
 
 
 def test_sampling_config_validation():
@@ -79,7 +130,7 @@ def test_sampling_config_validation():
 
 def test_interactive_reads_until_quit(monkeypatch):
     engine, calls = fake_engine([GenerationEvent(5, 0, "ok", "ok", "eos", None, 2)])
-    monkeypatch.setattr(cli, "_engine_from_args", lambda args: engine)
+    monkeypatch.setattr(cli, "open_engine", lambda args: engine)
     out = io.StringIO()
     code = cli.main(["--model", "m", "--interactive", "--no-metrics"], input_stream=io.StringIO("hello\n\n/quit\n"), output=out)
     assert code == 0 and "assistant> ok" in out.getvalue() and out.getvalue().count("you> ") == 3

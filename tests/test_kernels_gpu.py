@@ -92,6 +92,54 @@ def test_add_rmsnorm(ops, out_dtype, rows, hidden, eps):
     torch.testing.assert_close(out.cpu().float(), want, **tol(out_dtype, 1e-5, 1e-2))
 
 
+@pytest.mark.parametrize("hidden", [64, 4096])
+def test_every_norm_kernel_has_eps_under_the_square_root(ops, hidden):
+    """eps = 0.5 beside a mean of squares of 0.25: x * rsqrt(mean + eps) is x / 0.866, while x / (sqrt(mean) + eps)
+    would be x / 1.0.  The norm kernel, the add-and-norm kernel, the norm folded into a product's input, and the
+    norm taken apart around products of few rows and of 17..128 rows."""
+    g = torch.Generator().manual_seed(hidden)
+    rows, eps = 3, 0.5
+    x = 0.5 * torch.sign(torch.randn(rows, hidden, generator=g))
+    w = (1 + 0.25 * torch.randn(hidden, generator=g)).bfloat16()
+    want = w.float() * x / math.sqrt(0.75)
+    assert ((want - w.float() * x).abs() / want.abs()).min() > 0.13          # the misreading is 13 % away, the tolerances below 1-2 %
+    for out_dtype in DTYPES:
+        out = torch.empty(rows, hidden, device="cuda", dtype=out_dtype)
+        ops.rmsnorm(out, dev(x), dev(w), eps)
+        torch.testing.assert_close(out.cpu().float(), want, **tol(out_dtype, 2e-6, 1e-2))
+        stream = dev(x - 1.0)
+        ops.add_rmsnorm(out, stream, dev(torch.ones(rows, hidden).bfloat16()), dev(w), eps)
+        torch.testing.assert_close(out.cpu().float(), want, **tol(out_dtype, 2e-6, 1e-2))
+    # folded into a product's input: the product with the identity gives the normalised rows back
+    eye = torch.eye(hidden).bfloat16()
+    out = torch.empty(rows, hidden, device="cuda", dtype=torch.float32)
+    ops.gemm(out, dev(x), dev(eye), norm_weight=dev(w), eps=eps)
+    torch.testing.assert_close(out.cpu(), want, rtol=1e-2, atol=1e-2)
+    # taken apart: a product that adds zero into the stream begins the norm, scale_rows or the next product finishes it
+    for m in (rows, 24):
+        if m > 16 and hidden % 256:
+            continue
+        xs = x[torch.arange(m) % rows]
+        stream = dev(xs.clone())
+        zeros_a, zeros_w = torch.zeros(m, hidden, dtype=torch.bfloat16, device="cuda"), torch.zeros(hidden, hidden, dtype=torch.bfloat16, device="cuda")
+        next_x = torch.empty(m, hidden, dtype=torch.bfloat16, device="cuda")
+        if m <= 16:
+            sumsq = torch.empty(ops.norm_chain_parts(hidden), m, device="cuda")
+            ops.gemm_norm_chain(stream, zeros_a, zeros_w, accumulate=True, next_x=next_x, next_sumsq=sumsq, next_weight=dev(w))
+        else:
+            sumsq = torch.empty(ops.norm_begin_parts(hidden), m, device="cuda")
+            ops.gemm_mid_add_norm_begin(stream, zeros_a, zeros_w, dev(w), next_x, sumsq)
+        finished = torch.empty(m, hidden, dtype=torch.bfloat16, device="cuda")
+        ops.scale_rows(finished, next_x, sumsq, eps)
+        torch.testing.assert_close(finished.cpu().float(), want[torch.arange(m) % rows], rtol=1e-2, atol=1e-2)
+        out = torch.empty(m, hidden, dtype=torch.float32, device="cuda")
+        if m <= 16:
+            ops.gemm_norm_chain(out, next_x, dev(eye), in_sumsq=sumsq, in_eps=eps)
+        else:
+            ops.gemm_mid_scaled(out, next_x, dev(eye), sumsq, eps)
+        torch.testing.assert_close(out.cpu(), want[torch.arange(m) % rows], rtol=1e-2, atol=1e-2)
+
+
 @pytest.mark.parametrize("half,theta", [(8, 1e4), (16, 1e6), (64, 1e6), (24, 5e5)])
 def test_rope_table(ops, half, theta):
     positions = torch.tensor([0, 1, 2, 17, 511, 4095, 40959], dtype=torch.int32)

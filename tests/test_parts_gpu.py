@@ -23,7 +23,7 @@ def close(got, want, dtype, f32=2e-5, bf16=3e-2):
         assert err < bf16, f"relative error {err:.3g}"
 
 
-def build_runner(spec, weights, dtype, *, page_size=16, num_pages=64, max_requests=4, max_seq_len=512, max_step_tokens=512):
+def build_runner(spec, weights, dtype, *, page_size=16, num_pages=64, max_requests=4, max_seq_len=512, max_step_tokens=512, use_graph=False):
     from llm_runtime_study_amd.cache import CacheManager
     from llm_runtime_study_amd.engine.step import ModelRunner
     from llm_runtime_study_amd.models import DecoderModel
@@ -32,7 +32,7 @@ def build_runner(spec, weights, dtype, *, page_size=16, num_pages=64, max_reques
     model.bind({k: v.to("cuda") for k, v in weights.items()}, dtype)
     cache = CacheManager(model.cache_needs(), page_size=page_size, num_pages=num_pages, max_requests=max_requests,
                          max_seq_len=max_seq_len, dtype=dtype, device="cuda")
-    return ModelRunner(model, cache, max_step_tokens=max_step_tokens, dtype=dtype, device="cuda")
+    return ModelRunner(model, cache, max_step_tokens=max_step_tokens, dtype=dtype, device="cuda", use_graph=use_graph)
 
 
 def spec_and_weights(raw, seed, edit=None):
@@ -324,3 +324,123 @@ def test_toy_mixer_with_state_is_registered_built_and_stepped(dtype):
     assert caches["c"].slot == caches["a"].slot
     for key in requests:
         close(torch.cat(got[key]), want[key], dtype, f32=1e-4)
+
+
+class GraphSafeRunningMean(RunningMeanMixer):
+    """The same toy mixer, able to run inside a captured decode step: there it finds its state rows through
+    the slot ids on the device (a replay sees the slots of its own step, and the rows that pad the batch
+    point at the trash slot), works in place on scratch buffers and leaves the product to the package."""
+
+    graph_safe = True
+
+    def bind(self, weights, dtype):
+        super().bind(weights, dtype)
+        self.weight_run = weights["mix.weight"].to(dtype).contiguous()
+
+    def forward(self, ctx, x, residual, cache):
+        from llm_runtime_study_amd.parts.linear import linear
+
+        if not ctx.all_decode:
+            return super().forward(ctx, x, residual, cache)
+        rows_n, hidden = ctx.T, self.hidden_size
+        index = ctx.scratch("toy_index", (rows_n,), torch.int64)
+        index.copy_(ctx.slot_ids)
+        rows = ctx.scratch("toy_rows", (rows_n, hidden + 1), torch.float32)
+        torch.index_select(cache.state, 0, index, out=rows)
+        rows[:, :-1].add_(x)
+        rows[:, -1].add_(1.0)
+        mean32 = ctx.scratch("toy_mean32", (rows_n, hidden), torch.float32)
+        torch.div(rows[:, :-1], rows[:, -1:], out=mean32)
+        mean = ctx.scratch("toy_mean", (rows_n, hidden), ctx.dtype)
+        mean.copy_(mean32)
+        linear(ctx, residual, mean, self.weight_run, accumulate=True)
+        cache.state.index_copy_(0, index, rows)
+
+
+def toy_state_model(kind, cls):
+    from llm_runtime_study_amd.models import DecoderModel, ModelSpec, ScheduleEntry
+    from llm_runtime_study_amd.parts import PartSpec, register
+    from llm_runtime_study_amd.weights import random_tensors
+
+    register("mixer", kind, cls)
+    hidden, vocab, eps = 48, 97, 1e-5
+    norm = PartSpec("rmsnorm", {"size": hidden, "eps": eps})
+    block = PartSpec("prenorm", {
+        "mixer": PartSpec(kind, {"hidden_size": hidden}),
+        "feed_forward": PartSpec("swiglu", {"hidden_size": hidden, "intermediate_size": 80}),
+        "mixer_norm": norm, "ff_norm": norm,
+        "names": {"mixer": "mixer", "feed_forward": "mlp", "mixer_norm": "input_layernorm", "ff_norm": "post_attention_layernorm"},
+    })
+    spec = ModelSpec(architecture="ToyRunningMean", vocab_size=vocab, hidden_size=hidden, layers=(block, block),
+                     schedule=(ScheduleEntry(0), ScheduleEntry(1)), final_norm=norm, max_positions=256)
+    weights = random_tensors(DecoderModel(spec).tensors(), 5, torch.bfloat16, "scaled")
+    return spec, weights, vocab, eps
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_rows_that_pad_a_graph_batch_leave_every_request_state_alone(dtype):
+    """Three requests decode as a captured batch of four rows: the fourth row belongs to no request.  Its
+    state goes to the trash slot, so the request in slot 0 keeps its own."""
+    from llm_runtime_study_amd.engine.step import StepEntry
+
+    spec, weights, vocab, eps = toy_state_model("toy_running_mean_graph", GraphSafeRunningMean)
+    runner = build_runner(spec, weights, dtype, use_graph=True)
+    assert runner.use_graph
+    cache = runner.cache
+    assert cache.layer_caches[0].state.shape == (cache.max_requests + 1, 49) and cache.trash_slot == cache.max_requests
+    rng = np.random.default_rng(3)
+    requests = {k: rng.integers(0, vocab, n).tolist() for k, n in (("a", 18), ("b", 13), ("c", 20))}
+    double = {k: v.double() for k, v in weights.items()}
+    want = {k: plain_running_mean_model(double, {"rms_norm_eps": eps}, ids, 2) for k, ids in requests.items()}
+    prompt = {"a": 10, "b": 5, "c": 12}
+    got = {k: [] for k in requests}
+    with torch.cuda.stream(torch.cuda.Stream("cuda")):
+        caches = {k: cache.admit(k) for k in requests}
+        assert caches["a"].slot == 0
+        runner.step([StepEntry(caches[k], requests[k][:n], []) for k, n in prompt.items()])
+        for step in range(8):
+            logits = runner.step([StepEntry(caches[k], [requests[k][prompt[k] + step]], [0]) for k in requests])
+            for row, k in enumerate(requests):
+                got[k].append(logits[row].clone())
+        torch.cuda.synchronize()
+        assert runner.graph_captures == 1 and runner.graph_replays == 7       # the capturing step runs once, eagerly
+        trash = cache.layer_caches[0].state[cache.trash_slot]
+        assert trash[-1].item() > 0          # the padding row counted its tokens there
+        runner.drop_graphs()
+    for k in requests:
+        close(torch.stack(got[k]), want[k][prompt[k]:prompt[k] + 8], dtype, f32=1e-4)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_a_failing_step_puts_per_request_state_back(dtype):
+    """The mixers of both layers have moved their state on when the second layer's feed-forward raises:
+    the rows of the step's requests are as before, and the step run again gives the right logits."""
+    from llm_runtime_study_amd.engine.step import StepEntry
+
+    spec, weights, vocab, eps = toy_state_model("toy_running_mean", RunningMeanMixer)
+    runner = build_runner(spec, weights, dtype)
+    cache = runner.cache
+    rng = np.random.default_rng(4)
+    ids = {k: rng.integers(0, vocab, 24).tolist() for k in ("a", "b")}
+    double = {k: v.double() for k, v in weights.items()}
+    want = {k: plain_running_mean_model(double, {"rms_norm_eps": eps}, v, 2) for k, v in ids.items()}
+    caches = {k: cache.admit(k) for k in ids}
+    runner.step([StepEntry(caches["a"], ids["a"][:9], []), StepEntry(caches["b"], ids["b"][:16], [])])
+    states = [cache.layer_caches[i].state.clone() for i in (0, 1)]
+    entries = [StepEntry(caches["a"], ids["a"][9:], list(range(15))), StepEntry(caches["b"], ids["b"][16:17], [0])]
+    feed_forward = runner.model.layers[1].feed_forward
+    original = feed_forward.forward
+
+    def broken(*args, **kwargs):
+        raise RuntimeError("the feed-forward fails")
+
+    feed_forward.forward = broken
+    with pytest.raises(RuntimeError, match="feed-forward fails"):
+        runner.step(entries)
+    feed_forward.forward = original
+    assert [caches[k].length for k in ids] == [9, 16]
+    for i in (0, 1):
+        assert torch.equal(cache.layer_caches[i].state, states[i])
+    logits = runner.step(entries)
+    close(logits[:15], want["a"][9:], dtype, f32=1e-4)
+    close(logits[15:], want["b"][16:17], dtype, f32=1e-4)

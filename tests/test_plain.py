@@ -25,6 +25,18 @@ def test_rms_norm_equation_vector():
     torch.testing.assert_close(got, F.rms_norm(x, (4,), w, 1e-6))
 
 
+def test_rms_norm_eps_sits_under_the_square_root():
+    """reference mini_llm/nn/norm.py:42-46: x * rsqrt(mean(x^2) + eps).  With eps = 0.5 the other readings are far
+    off: x / (sqrt(mean) + eps) gives 1/1.0, eps added to the sum instead of the mean gives 1/sqrt(0.375)."""
+    x = torch.tensor([[0.5, -0.5, 0.5, -0.5]])           # mean of squares 0.25
+    got = plain.rms_norm(x, torch.ones(4), 0.5)
+    torch.testing.assert_close(got, x / math.sqrt(0.75))
+    assert not torch.allclose(got, x / (0.5 + 0.5), rtol=0.05) and not torch.allclose(got, x / math.sqrt(0.25 + 0.5 / 4), rtol=0.05)
+    torch.testing.assert_close(got, F.rms_norm(x, (4,), torch.ones(4), 0.5))
+    w = torch.tensor([2.0, 1.0, 0.5, 3.0])                # the weight multiplies after the normalisation
+    torch.testing.assert_close(plain.rms_norm(x, w, 0.5), w * x / math.sqrt(0.75))
+
+
 def test_rms_norm_half_precision_vector():
     # reference tests/test_norm.py:29-38: [300, 400] -> [0.8486, 1.1314]
     got = plain.rms_norm(torch.tensor([[300.0, 400.0]]), torch.ones(2), 1e-6)
@@ -121,8 +133,9 @@ def test_gqa_head_map():
 
 
 def test_qwen3_attention_matches_manual_reference():
-    # the recipe of reference tests/test_attention.py:47-84 at position 0..2 with theta so
-    # large that the rotation is the identity on all but the first pair
+    # the recipe of reference tests/test_attention.py:47-84 with unit norm weights and all tokens at one
+    # position: pins projections, head split, grouping, scale and the output projection; the order of norm
+    # and rotation and the mask are pinned by the next test
     torch.manual_seed(11)
     cfg = dict(num_attention_heads=2, num_key_value_heads=1, head_dim=2, rms_norm_eps=1e-6, rope_theta=1e4)
     w = {
@@ -143,6 +156,47 @@ def test_qwen3_attention_matches_manual_reference():
     o = torch.softmax(s, -1) @ v.repeat_interleave(2, 0)
     want = o.transpose(0, 1).reshape(3, 4) @ w["a.o_proj.weight"].T
     torch.testing.assert_close(got, want, rtol=1e-5, atol=1e-6)
+
+
+def test_qwen3_attention_normalises_before_it_rotates_and_masks_later_keys():
+    """Heads of two dims are one rotary pair, so the rotation is a plain 2-D rotation by the position (theta plays
+    no part).  With norm weights (2, 0.5) rotating before normalising gives other numbers, and with positions
+    0, 1, 2 a key after the query must not count (reference mini_llm/nn/attention.py:231-248, 286-302)."""
+    torch.manual_seed(12)
+    cfg = dict(num_attention_heads=2, num_key_value_heads=1, head_dim=2, rms_norm_eps=1e-6, rope_theta=1e4)
+    w = {
+        "a.q_proj.weight": torch.randn(4, 2), "a.k_proj.weight": torch.randn(2, 2),
+        "a.v_proj.weight": torch.randn(2, 2), "a.o_proj.weight": torch.randn(2, 4),
+        "a.q_norm.weight": torch.tensor([2.0, 0.5]), "a.k_norm.weight": torch.tensor([0.25, 3.0]),
+    }
+    x = torch.tensor([[1.0, 2.0], [-1.0, 0.5], [0.25, -0.75]])
+    positions = torch.tensor([0, 1, 2])
+    got, _ = plain.qwen3_attention(x, w, "a", cfg, positions)
+
+    def rotate(t, swap_order=False):          # t [heads, tokens, 2]
+        c, s_ = torch.cos(positions.float()), torch.sin(positions.float())
+        return torch.stack((t[..., 0] * c - t[..., 1] * s_, t[..., 1] * c + t[..., 0] * s_), -1)
+
+    def norm(t, weight):
+        return t * torch.rsqrt(t.square().mean(-1, keepdim=True) + 1e-6) * weight
+
+    def recipe(norm_first: bool, causal: bool):
+        q = (x @ w["a.q_proj.weight"].T).view(3, 2, 2).transpose(0, 1)
+        k = (x @ w["a.k_proj.weight"].T).view(3, 1, 2).transpose(0, 1)
+        v = (x @ w["a.v_proj.weight"].T).view(3, 1, 2).transpose(0, 1)
+        if norm_first:
+            q, k = rotate(norm(q, w["a.q_norm.weight"])), rotate(norm(k, w["a.k_norm.weight"]))
+        else:
+            q, k = norm(rotate(q), w["a.q_norm.weight"]), norm(rotate(k), w["a.k_norm.weight"])
+        scores = (q @ k.repeat_interleave(2, 0).transpose(-1, -2)) / math.sqrt(2)
+        if causal:
+            scores = scores.masked_fill(torch.triu(torch.ones(3, 3, dtype=torch.bool), 1), -torch.inf)
+        o = torch.softmax(scores, -1) @ v.repeat_interleave(2, 0)
+        return o.transpose(0, 1).reshape(3, 4) @ w["a.o_proj.weight"].T
+
+    torch.testing.assert_close(got, recipe(True, True), rtol=1e-5, atol=1e-6)
+    assert not torch.allclose(got, recipe(False, True), rtol=1e-2, atol=1e-3)      # norm after the rotation: other numbers
+    assert not torch.allclose(got, recipe(True, False), rtol=1e-2, atol=1e-3)      # no mask: other numbers
 
 
 def test_swiglu_vector():

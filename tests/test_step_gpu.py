@@ -1,0 +1,295 @@
+"""The step function's own promises: what it refuses, that a failing forward leaves no trace in the
+caches (reference tests/test_cache.py:306-324, mini_llm/model/base.py:136-156,180-190), that decode
+launches of several steps give the tokens of single steps also across a length class's edge, the
+package's own many-rows product inside whole steps, and one layer at the benchmark's sizes against
+the plain implementation directly."""
+
+import numpy as np
+import pytest
+import torch
+
+from tests import traces
+from tests.helpers import TINY_B, TINY_C
+from tests.plain import model as plain
+
+pytestmark = pytest.mark.gpu
+DTYPES = [torch.float32, torch.bfloat16]
+
+
+@pytest.fixture(scope="module")
+def folder_b(tmp_path_factory):
+    from llm_runtime_study_amd.config import config_from_dict
+    from llm_runtime_study_amd.weights import write_model_dir
+
+    folder = tmp_path_factory.mktemp("step_b")
+    write_model_dir(config_from_dict(TINY_B), seed=41, model_dir=folder, init="scaled")
+    return folder
+
+
+def make_runner(folder, dtype, *, pages=40, requests=4, seq=256, step_tokens=64, graph=False, page_size=16):
+    from llm_runtime_study_amd.cache import CacheManager
+    from llm_runtime_study_amd.engine.loading import load_model
+    from llm_runtime_study_amd.engine.step import ModelRunner
+
+    device = torch.device("cuda", 0)
+    _, model = load_model(folder, dtype, device)
+    cache = CacheManager(model.cache_needs(), page_size=page_size, num_pages=pages, max_requests=requests, max_seq_len=seq, dtype=dtype, device=device)
+    return ModelRunner(model, cache, max_step_tokens=step_tokens, dtype=dtype, device=device, use_graph=graph)
+
+
+def snapshot(cache, requests):
+    """Everything a failed step must leave as it was."""
+    return ([r.length for r in requests], [[list(t) for t in r.tables] for r in requests],
+            [cache.used_pages(g) for g in range(len(cache.groups))], [cache.free_pages(g) for g in range(len(cache.groups))],
+            [g.host_table.copy() for g in cache.groups], cache.active_requests)
+
+
+def same(a, b):
+    return a[:4] == b[:4] and all((x == y).all() for x, y in zip(a[4], b[4])) and a[5] == b[5]
+
+
+class Failing(RuntimeError):
+    pass
+
+
+# ------------------------------------------------------------------ refusals
+def test_every_refusal_of_the_step_function_leaves_the_cache_alone(folder_b):
+    from llm_runtime_study_amd.engine.step import StepEntry
+    from llm_runtime_study_amd.errors import GenerationError
+
+    runner = make_runner(folder_b, torch.float32, requests=2, step_tokens=12)
+    cache = runner.cache
+    a, b = cache.admit("a"), cache.admit("b")
+    runner.step([StepEntry(a, [1, 2, 3], [])])
+    outsider = make_runner(folder_b, torch.float32, requests=3).cache.admit("c")
+    vocab = TINY_B["vocab_size"]
+    cases = [
+        ([], "at least one entry"),
+        ([StepEntry(a, [1]), StepEntry(b, [2]), StepEntry(outsider, [3])], "3 requests but at most 2"),
+        ([StepEntry(a, [1]), StepEntry(b, [])], "at least one token"),
+        ([StepEntry(a, [1]), StepEntry(a, [2])], "only once"),
+        ([StepEntry(a, [1, vocab])], rf"within vocabulary \[0, {vocab}\)"),
+        ([StepEntry(a, [1, -1])], "within vocabulary"),
+        ([StepEntry(a, [1, 2], [2])], "wanted place 2 is outside the entry's 2 tokens"),
+        ([StepEntry(a, [1, 2], [-1])], "wanted place -1"),
+        ([StepEntry(a, [1] * 7), StepEntry(b, [2] * 6)], "13 tokens but at most 12"),
+    ]
+    before = snapshot(cache, [a, b])
+    for entries, message in cases:
+        with pytest.raises(GenerationError, match=message):
+            runner.step(entries)
+        assert same(snapshot(cache, [a, b]), before)
+    with pytest.raises(GenerationError, match="1..8 steps"):
+        runner.decode_steps([StepEntry(a, [1])], 9)
+    with pytest.raises(GenerationError, match="needs graphs"):
+        runner.decode_steps([StepEntry(a, [1])], 2)       # this runner was built without graphs
+    assert same(snapshot(cache, [a, b]), before)
+    cache.check_invariants()
+    # a cache that was given back is refused by the cache manager, and the other entry's growth is undone
+    cache.release(b)
+    from llm_runtime_study_amd.errors import KVCacheError
+    with pytest.raises(KVCacheError, match="released"):
+        runner.step([StepEntry(a, [4]), StepEntry(b, [5])])
+    assert a.length == 3
+    cache.check_invariants()
+
+
+# ------------------------------------------------------- a forward that fails
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_a_failing_forward_leaves_no_trace_in_a_mixed_step(folder_b, dtype):
+    """Two running requests decode beside a new request's first portion; the second layer raises.
+    Lengths, page lists, pool counts and host block tables are as before, the new request holds
+    nothing, and the same step run again gives what a runner that never failed gives."""
+    from llm_runtime_study_amd.engine.step import StepEntry
+
+    rng = np.random.default_rng(3)
+    prompts = [rng.integers(0, TINY_B["vocab_size"], n).tolist() for n in (31, 16, 20)]
+
+    def drive(fail: bool):
+        runner = make_runner(folder_b, dtype, pages=12)
+        cache = runner.cache
+        r0, r1 = cache.admit(0), cache.admit(1)
+        runner.step([StepEntry(r0, prompts[0], []), StepEntry(r1, prompts[1], [])])     # r1 ends exactly at a page's edge
+        r2 = cache.admit(2)
+        entries = [StepEntry(r0, [7], [0]), StepEntry(r1, [9], [0]), StepEntry(r2, prompts[2], [19])]
+        if fail:
+            before = snapshot(cache, [r0, r1, r2])
+            layer = runner.model.layers[1]
+            original = layer.forward
+
+            def broken(*args, **kwargs):
+                raise Failing("the second layer fails")
+
+            layer.forward = broken
+            with pytest.raises(Failing):
+                runner.step(entries)
+            layer.forward = original
+            assert same(snapshot(cache, [r0, r1, r2]), before)
+            assert r2.length == 0 and r2.tables == [[]] and cache.used_pages() == 3
+            cache.check_invariants()
+        first = runner.step(entries).clone()
+        second = runner.step([StepEntry(r0, [1], [0]), StepEntry(r1, [2], [0]), StepEntry(r2, [3], [0])]).clone()
+        cache.check_invariants()
+        return first, second
+
+    for got, want in zip(drive(True), drive(False)):
+        assert torch.equal(got, want)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_a_failing_launch_of_several_decode_steps_leaves_no_trace(folder_b, dtype):
+    """decode_steps(4) takes the pages of all four positions before it runs; the third step's forward
+    raises.  One request sits two tokens before a page's edge, so the launch had taken a page for it."""
+    from llm_runtime_study_amd.engine.step import StepEntry
+
+    rng = np.random.default_rng(4)
+    prompts = [rng.integers(0, TINY_B["vocab_size"], n).tolist() for n in (30, 9, 17)]
+
+    def drive(fail: bool):
+        runner = make_runner(folder_b, dtype, pages=12, graph=True)
+        cache = runner.cache
+        with torch.cuda.stream(torch.cuda.Stream(runner.device)):
+            requests = [cache.admit(i) for i in range(3)]
+            runner.step([StepEntry(r, p, []) for r, p in zip(requests, prompts)])
+            entries = [StepEntry(r, [5 + i], [0]) for i, r in enumerate(requests)]
+            assert runner.can_decode_steps(entries)
+            if fail:
+                before = snapshot(cache, requests)
+                original, calls = runner.model.forward_hidden, []
+
+                def broken(ctx):
+                    calls.append(1)
+                    if len(calls) == 3:
+                        raise Failing("the third step fails")
+                    return original(ctx)
+
+                runner.model.forward_hidden = broken
+                with pytest.raises(Failing):
+                    runner.decode_steps(entries, 4)
+                runner.model.forward_hidden = original
+                assert len(calls) == 3 and same(snapshot(cache, requests), before)
+                assert [r.length for r in requests] == [30, 9, 17] and cache.used_pages() == 2 + 1 + 2
+                cache.check_invariants()
+            chosen = runner.decode_steps(entries, 4)
+            assert [r.length for r in requests] == [34, 13, 21]
+            after = runner.step([StepEntry(r, [row], [0]) for r, row in zip(requests, chosen[-1])]).clone()
+            torch.cuda.synchronize()          # the comparison below runs on another stream
+            runner.drop_graphs()
+        cache.check_invariants()
+        return chosen, after
+
+    (chosen, after), (chosen_ok, after_ok) = drive(True), drive(False)
+    assert chosen == chosen_ok and torch.equal(after, after_ok)
+
+
+# ------------------------------------------- launches that cross a class's edge
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_tokens_do_not_depend_on_steps_per_launch_across_a_length_class_edge(tmp_path, dtype):
+    """From a context of 254 tokens on, eight tokens in launches of 4, of 3 and one by one: the contexts
+    cross 256, where decode attention begins to divide the keys.  Same tokens, same logits afterwards,
+    same keys and values in the pages."""
+    from llm_runtime_study_amd.config import config_from_dict
+    from llm_runtime_study_amd.engine.step import StepEntry
+    from llm_runtime_study_amd.weights import write_model_dir
+
+    folder = tmp_path / "c"
+    write_model_dir(config_from_dict(TINY_C), seed=42, model_dir=folder, init="scaled")
+    rng = np.random.default_rng(6)
+    prompts = [rng.integers(0, TINY_C["vocab_size"], n).tolist() for n in (253, 120)]
+    outcomes = []
+    for per_launch in (4, 3, 1):
+        runner = make_runner(folder, dtype, pages=40, seq=320, step_tokens=512, graph=True)
+        cache = runner.cache
+        with torch.cuda.stream(torch.cuda.Stream(runner.device)):
+            requests = [cache.admit(i) for i in range(2)]
+            runner.step([StepEntry(r, p, []) for r, p in zip(requests, prompts)])
+            tokens, last = [], [11, 12]
+            while len(tokens) < 8:
+                n = min(per_launch, 8 - len(tokens))
+                chosen = runner.decode_steps([StepEntry(r, [t], [0]) for r, t in zip(requests, last)], n)
+                tokens += chosen
+                last = chosen[-1]
+            final = runner.step([StepEntry(r, [t], [0]) for r, t in zip(requests, last)]).clone()
+            torch.cuda.synchronize()
+            layer = cache.layer_caches[1]
+            pages = [p for r in requests for p in r.tables[0]]
+            outcomes.append((tokens, final, layer.k_pages[pages].clone(), layer.v_pages[pages].clone(), pages))
+            assert requests[0].length == 253 + 9 and runner.graph_replays + runner.graph_captures >= 8 // per_launch
+            runner.drop_graphs()
+    for tokens, final, keys, values, pages in outcomes[1:]:
+        assert tokens == outcomes[0][0] and pages == outcomes[0][4]
+        assert torch.equal(final, outcomes[0][1]) and torch.equal(keys, outcomes[0][2]) and torch.equal(values, outcomes[0][3])
+
+
+# ---------------------------------------- the package's own many-rows product
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_whole_prompts_through_the_own_many_rows_product(folder_b, dtype, tmp_path):
+    """Replay with `library_gemm=False`: a 300-token prompt whole (more rows than the kernels for few
+    rows take) and the same prompt in two portions, against the plain implementation."""
+    from llm_runtime_study_amd.engine import trace
+
+    cfg, weights = plain.load_model_dir(folder_b, torch.float64)
+    rng = np.random.default_rng(8)
+    requests = {"long": rng.integers(0, cfg["vocab_size"], 300).tolist(), "mid": rng.integers(0, cfg["vocab_size"], 150).tolist()}
+    want = {key: plain.qwen3_forward(weights, cfg, ids) for key, ids in requests.items()}
+    steps = traces.whole(requests)
+    ids = requests["long"]
+    steps += [{"step": len(steps), "entries": [{"id": "again", "tokens": ids[:170], "want": [0, 169]}], "end": []},
+              {"step": len(steps) + 1, "entries": [{"id": "again", "tokens": ids[170:], "want": list(range(130))}], "end": ["again"]}]
+    want["again"] = want["long"]
+    runner = trace.make_runner(folder_b, dtype, 320, library_gemm=False)
+    assert runner.library_gemm is False
+    out = tmp_path / "logits"
+    trace.replay(runner, traces.strip(steps).splitlines(), out, echo=lambda _: None)
+    got = traces.collect(steps, out, cfg["vocab_size"])
+    checked = 0
+    for key, rows in got.items():
+        for position, row in rows.items():
+            ref = want[key][position]
+            if dtype == "float32":
+                torch.testing.assert_close(row.double(), ref, rtol=1e-4, atol=1e-4, msg=lambda m: f"{key}@{position}: {m}")
+            else:
+                err = (row.double() - ref).norm() / ref.norm()
+                assert err < 3e-2, f"{key}@{position}: relative error {err:.3g}"
+            checked += 1
+    assert checked == 300 + 150 + 2 + 130
+
+
+# ------------------------------- one layer at the benchmark's sizes, against plain
+def test_one_layer_at_the_benchmark_sizes_against_the_plain_implementation():
+    """Hidden 4096, 32 query and 8 kv heads of 128 dims, feed-forward 12288, vocabulary 151936, float32,
+    100 tokens in portions of 60, 39 and 1: the engine against the plain implementation itself, not against
+    another precision of the engine.  The plain side computes the logits of three slices of the vocabulary
+    (its first, a middle and its last rows) to keep the float64 work small."""
+    from llm_runtime_study_amd.cache import CacheManager
+    from llm_runtime_study_amd.config import config_from_dict, spec_for
+    from llm_runtime_study_amd.engine.step import ModelRunner, StepEntry
+    from llm_runtime_study_amd.models import DecoderModel
+    from llm_runtime_study_amd.weights import random_init
+    from tests.test_shape_gpu import SHAPE
+
+    raw = dict(SHAPE, num_hidden_layers=1)
+    cfg = config_from_dict(raw)
+    device = torch.device("cuda", 0)
+    model = DecoderModel(spec_for(cfg))
+    weights = random_init.device_weights(model, 3, torch.bfloat16, device, "scaled")
+    model.bind(weights, torch.float32)
+    cache = CacheManager(model.cache_needs(), page_size=16, num_pages=8, max_requests=1, max_seq_len=128, dtype=torch.float32, device=device)
+    runner = ModelRunner(model, cache, max_step_tokens=128, dtype=torch.float32, device=device)
+    rng = np.random.default_rng(9)
+    ids = rng.integers(0, cfg.vocab_size, 100).tolist()
+    request = cache.admit("r")
+    rows = []
+    for portion in (ids[:60], ids[60:99], ids[99:]):
+        rows.append(runner.step([StepEntry(request, portion, list(range(len(portion))))]).cpu())
+    got = torch.cat(rows)
+    # the plain side: only the embedding rows and head rows it needs, in float64
+    vocab = cfg.vocab_size
+    columns = torch.cat([torch.arange(0, 700), torch.arange(70000, 70700), torch.arange(vocab - 700, vocab)])
+    used = sorted(set(ids))
+    small = {name: t.cpu().double() for name, t in weights.items() if name not in ("model.embed_tokens.weight", "lm_head.weight")}
+    small["model.embed_tokens.weight"] = weights["model.embed_tokens.weight"][torch.tensor(used, device=device)].cpu().double()
+    small["lm_head.weight"] = weights["lm_head.weight"][columns.to(device)].cpu().double()
+    want = plain.qwen3_forward(small, raw, [used.index(t) for t in ids])
+    torch.testing.assert_close(got[:, columns].double(), want, rtol=1e-4, atol=1e-4)
+    assert want.abs().max() > 1.0

@@ -53,10 +53,15 @@ def test_all_problems_are_reported_in_one_error(tmp_path):
     tensors["model.layers.0.self_attn.rotary.inv_freq"] = torch.zeros(8)
     tensors["model.layers.0.self_attn.q_proj.weight"] = torch.zeros(64, 63, dtype=torch.bfloat16)
     tensors["model.layers.0.input_layernorm.weight"] = torch.zeros(64, dtype=torch.int32)
+    tensors["model.layers.1.mlp.down_proj.weight"] = tensors["model.layers.1.mlp.down_proj.weight"].half()
     write_safetensors(tmp_path / "model.safetensors", tensors)
     with pytest.raises(CheckpointValidationError) as info:
-        validate(Checkpoint.from_model_dir(tmp_path), expected, "qwen3")
+        validate(Checkpoint.from_model_dir(tmp_path), expected, "qwen3", "bfloat16")
     text = str(info.value)
+    # the configuration's dtype is the one every floating tensor must have (reference checkpoint.py:478-481)
+    assert "dtype mismatch for model.layers.1.mlp.down_proj.weight: expected BF16, got F16" in text
+    assert "dtype mismatch for model.layers.0.input_layernorm.weight: expected BF16, got I32" in text
+    assert text.count("\n  - ") == 5   # one line for each kind of problem and each tensor at fault: nothing is reported twice
     assert text.startswith("checkpoint does not match qwen3 configuration:")
     assert "missing tensors: model.layers.1.mlp.up_proj.weight, model.norm.weight" in text
     assert "unexpected tensors: model.layers.0.self_attn.rotary.inv_freq" in text
@@ -73,13 +78,45 @@ def test_tied_head_is_optional_and_untied_head_is_required(tmp_path):
         validate(Checkpoint.from_model_dir(tmp_path), untied, "qwen3")
 
 
-def test_stored_precision_is_kept(tmp_path):
+def test_dtype_follows_the_configuration(tmp_path):
+    """BF16 for torch_dtype bfloat16, F32 for float32, F16 for float16; anything else is named in the error."""
+    expected = expected_for(TINY_A)
+    for stored, config_dtype, container in ((torch.bfloat16, "bfloat16", "BF16"), (torch.float32, "float32", "F32"), (torch.float16, "float16", "F16")):
+        write_safetensors(tmp_path / "model.safetensors", random_tensors(expected, 0, stored))
+        checkpoint = Checkpoint.from_model_dir(tmp_path)
+        validate(checkpoint, expected, "qwen3", config_dtype)
+        for other in {"bfloat16", "float32", "float16"} - {config_dtype}:
+            with pytest.raises(CheckpointValidationError, match=f"dtype mismatch for lm_head.weight: expected .*, got {container}|dtype mismatch for model.embed_tokens.weight: expected .*, got {container}"):
+                validate(checkpoint, expected, "qwen3", other)
+        checkpoint.close()
+    with pytest.raises(CheckpointValidationError, match="unsupported checkpoint dtype 'float64'"):
+        validate(Checkpoint.from_model_dir(tmp_path), expected, "qwen3", "float64")
+
+
+def test_a_model_folder_is_checked_against_its_own_torch_dtype(tmp_path):
+    """Through the path Engine.from_model_dir takes: a folder whose tensors are not in the configuration's
+    dtype is refused, unless the caller asks for the stored precision."""
+    from llm_runtime_study_amd.engine.loading import load_model
+
+    config = config_from_dict(TINY_A)
+    write_model_dir(config, 1, tmp_path)
+    expected = expected_for(TINY_A)
+    tensors = random_tensors(expected, 1, torch.bfloat16)
+    tensors["model.norm.weight"] = tensors["model.norm.weight"].float()
+    write_safetensors(tmp_path / "model.safetensors", tensors)
+    with pytest.raises(CheckpointValidationError, match="dtype mismatch for model.norm.weight: expected BF16, got F32"):
+        load_model(tmp_path, torch.float32, "cpu")
+
+
+def test_stored_precision_is_kept_when_asked_for(tmp_path):
     expected = expected_for(TINY_A)
     tensors = random_tensors(expected, 0, torch.bfloat16)
     tensors["model.norm.weight"] = tensors["model.norm.weight"].float() + 1e-4   # stored in 32-bit: stays so
     tensors["model.layers.0.mlp.down_proj.weight"] = tensors["model.layers.0.mlp.down_proj.weight"].half()
     write_safetensors(tmp_path / "model.safetensors", tensors)
-    weights = load(Checkpoint.from_model_dir(tmp_path), expected, "qwen3", "cpu")
+    with pytest.raises(CheckpointValidationError, match="expected BF16, got F32"):
+        load(Checkpoint.from_model_dir(tmp_path), expected, "qwen3", "cpu", "bfloat16")
+    weights = load(Checkpoint.from_model_dir(tmp_path), expected, "qwen3", "cpu", checkpoint_dtype=None)
     assert weights["model.norm.weight"].dtype == torch.float32
     assert torch.equal(weights["model.norm.weight"], tensors["model.norm.weight"])
     assert weights["model.layers.0.mlp.down_proj.weight"].dtype == torch.float32   # float16 is widened
