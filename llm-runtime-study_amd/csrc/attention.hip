@@ -554,8 +554,6 @@ __global__ __launch_bounds__(256, D <= 128 ? 2 : 1) void attention_prefill_bf16_
   // 8 bytes a lane by 16 lanes a cycle: a stride of 18 banks (twice an odd number) does the same;
   // such rows start at multiples of 8 bytes only, so they are written 8 bytes at a time.
   constexpr int KLD = D + 8, VLD = 32 + 4;
-  constexpr int KCHUNKS = 32 * D / 8, VCHUNKS = D * 4;        // 16-byte pieces of one tile
-  constexpr int KPT = (KCHUNKS + 255) / 256, VPT = (VCHUNKS + 255) / 256;
   __shared__ __attribute__((aligned(16))) bf16 ks[2][32 * KLD];
   __shared__ __attribute__((aligned(16))) bf16 vs[2][D * VLD];
   const int tid = threadIdx.x, threads = blockDim.x;
@@ -585,50 +583,61 @@ __global__ __launch_bounds__(256, D <= 128 ? 2 : 1) void attention_prefill_bf16_
   // the part of the request's block table that the tiles need, in LDS: the address of a key must
   // not wait for a trip to memory of its own
   extern __shared__ int page_ids[];
-  const int first_block = first_tile * 32 / page_size;
   const int last_key = last_tile * 32 + 31 < pos_last ? last_tile * 32 + 31 : pos_last;
-  if (first_tile <= last_tile)
-    for (int i = tid; i <= last_key / page_size - first_block; i += threads) page_ids[i] = table[first_block + i];
+  {
+    const int first = first_tile * 32 / page_size;
+    if (first_tile <= last_tile)
+      for (int i = tid; i <= last_key / page_size - first; i += threads) page_ids[i] = table[first + i];
+  }
   __syncthreads();
 
-  // pieces of a tile this thread brings in: keys [32, D] and transposed values [D, 32]
+  // Pieces of a tile this thread brings in: keys [32, D] and transposed values [D, 32].  A run of 16 keys
+  // lies in one page, and a wave serves one run (waves 0 and 1 the tile's first, 2 and 3 its second), so
+  // everything about the run's place in memory is the same for the whole wave and is worked out in
+  // scalar registers: one block table entry, one base address; a lane adds a distance that never changes.
+  constexpr int KPIECES = D / 8, RUN_CHUNKS = 16 * KPIECES, TPR = 128, KPT = (RUN_CHUNKS + TPR - 1) / TPR;
+  constexpr int VRUN_CHUNKS = 2 * D, VPT = (VRUN_CHUNKS + TPR - 1) / TPR;
   bf16x8 kreg_a[KPT], vreg_a[VPT];
+  const int wrun = __builtin_amdgcn_readfirstlane(tid / TPR), t1 = tid % TPR;
+  const int pages16 = page_size / 16;                            // runs of 16 keys in a page
+  const unsigned magic = pages16 > 1 ? 0xFFFFFFFFu / (unsigned)pages16 + 1u : 0u;   // run / pages16 = umulhi(run, magic)
+  const int first_block = pages16 > 1 ? (int)__umulhi((unsigned)(first_tile * 2), magic) : first_tile * 2;
+  unsigned koff[KPT], voff[VPT];
+#pragma unroll
+  for (int i = 0; i < KPT; ++i) koff[i] = (unsigned)(((t1 + i * TPR) / KPIECES) * D + ((t1 + i * TPR) % KPIECES) * 8);
+#pragma unroll
+  for (int i = 0; i < VPT; ++i) voff[i] = (unsigned)(((t1 + i * TPR) / 2) * page_size + ((t1 + i * TPR) % 2) * 8);
   auto fetch = [&](int tile, bf16x8 (&kreg)[KPT], bf16x8 (&vreg)[VPT]) {
-    int64_t kbase[2], vbase[2];
-    bool present[2];
+    const int run = tile * 2 + wrun, key0 = run * 16;
+    const bool present = key0 <= pos_last && key0 + 15 >= lo_first;
+    if (present) {
+      const int block = pages16 > 1 ? (int)__umulhi((unsigned)run, magic) : run;
+      const int64_t page = __builtin_amdgcn_readfirstlane(page_ids[block - first_block]);
+      const int off = (run - block * pages16) * 16;
+      const bf16* kbase = k_pages + ((page * nkv + kvh) * page_size + off) * D;
+      const bf16* vbase = v_pages + (page * nkv + kvh) * (int64_t)D * page_size + off;
 #pragma unroll
-    for (int h = 0; h < 2; ++h) {
-      const int key0 = tile * 32 + h * 16;
-      present[h] = key0 <= pos_last && key0 + 15 >= lo_first;
-      const int64_t page = present[h] ? page_ids[key0 / page_size - first_block] : 0;
-      const int off = key0 % page_size;
-      kbase[h] = ((page * nkv + kvh) * page_size + off) * D;
-      vbase[h] = (page * nkv + kvh) * (int64_t)D * page_size + off;
-    }
+      for (int i = 0; i < KPT; ++i) kreg[i] = t1 + i * TPR < RUN_CHUNKS ? *(const bf16x8*)(kbase + koff[i]) : zero8;
 #pragma unroll
-    for (int i = 0; i < KPT; ++i) {
-      const int idx = tid + i * threads;
-      const int key = idx / (D / 8), piece = idx % (D / 8);
-      kreg[i] = (idx < KCHUNKS && present[key / 16]) ? *(const bf16x8*)(k_pages + kbase[key / 16] + (key % 16) * D + piece * 8) : zero8;
-    }
+      for (int i = 0; i < VPT; ++i) vreg[i] = t1 + i * TPR < VRUN_CHUNKS ? *(const bf16x8*)(vbase + voff[i]) : zero8;
+    } else {
 #pragma unroll
-    for (int i = 0; i < VPT; ++i) {
-      const int idx = tid + i * threads;
-      const int dim = idx / 4, part = idx % 4;
-      vreg[i] = (idx < VCHUNKS && present[part / 2]) ? *(const bf16x8*)(v_pages + vbase[part / 2] + (int64_t)dim * page_size + (part % 2) * 8) : zero8;
+      for (int i = 0; i < KPT; ++i) kreg[i] = zero8;
+#pragma unroll
+      for (int i = 0; i < VPT; ++i) vreg[i] = zero8;
     }
   };
   auto stash = [&](int buffer, const bf16x8 (&kreg)[KPT], const bf16x8 (&vreg)[VPT]) {
 #pragma unroll
     for (int i = 0; i < KPT; ++i) {
-      const int idx = tid + i * threads;
-      if (idx < KCHUNKS) *(bf16x8*)(ks[buffer] + (idx / (D / 8)) * KLD + (idx % (D / 8)) * 8) = kreg[i];
+      const int c = t1 + i * TPR;
+      if (c < RUN_CHUNKS) *(bf16x8*)(ks[buffer] + (wrun * 16 + c / KPIECES) * KLD + (c % KPIECES) * 8) = kreg[i];
     }
 #pragma unroll
     for (int i = 0; i < VPT; ++i) {
-      const int idx = tid + i * threads;
-      if (idx < VCHUNKS) {
-        bf16* dst = vs[buffer] + (idx / 4) * VLD + (idx % 4) * 8;
+      const int c = t1 + i * TPR;
+      if (c < VRUN_CHUNKS) {
+        bf16* dst = vs[buffer] + (c / 2) * VLD + wrun * 16 + (c % 2) * 8;
         *(bf16x4*)dst = bf16x4{vreg[i][0], vreg[i][1], vreg[i][2], vreg[i][3]};
         *(bf16x4*)(dst + 4) = bf16x4{vreg[i][4], vreg[i][5], vreg[i][6], vreg[i][7]};
       }
@@ -659,14 +668,10 @@ __global__ __launch_bounds__(256, D <= 128 ? 2 : 1) void attention_prefill_bf16_
       for (int e = 0; e < DB; ++e) o[b][e] = floatx4{0.f, 0.f, 0.f, 0.f};
     }
 
-    // MASKED = false: every query of the group may see every key of the tile (it lies wholly before
-    // the group's first position and inside the last one's window), so no score needs a test.
-    // Scores stay unscaled; the scale enters with the exponent: p = 2^(s * scale2 - max * scale2).
-    auto work = [&](int tile, int buffer, auto masked) {
-      constexpr bool MASKED = decltype(masked)::value;
+    // The three parts of a tile's work.
+    // scores: S[key, query] = K Q^T, unscaled (the scale enters with the exponent).
+    auto scores = [&](int buffer, floatx4 (&sc)[QB][2]) {
       const bf16* kt = ks[buffer];
-      const bf16* vt = vs[buffer];
-      floatx4 sc[QB][2];
 #pragma unroll
       for (int b = 0; b < QB; ++b) sc[b][0] = sc[b][1] = floatx4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
@@ -677,7 +682,17 @@ __global__ __launch_bounds__(256, D <= 128 ? 2 : 1) void attention_prefill_bf16_
 #pragma unroll
           for (int b = 0; b < QB; ++b) sc[b][h] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kfrag, qf[b][c], sc[b][h], 0, 0, 0);
         }
-      bf16x8 pf[QB];
+    };
+    // weights: one step of the running softmax, p = 2^(s * scale2 - reference * scale2) as bfloat16 operands.
+    // The reference point of a query's exponentials need not be its maximum: any value that keeps the
+    // weights inside float32 and bfloat16 gives the same result up to rounding.  So a tile that needs no
+    // mask first tries the reference it has, without looking for the tile's maximum at all (`weights`,
+    // which changes nothing if it fails); only if a weight sum comes out above 2^60 (or the query has no
+    // reference yet) is the tile done the long way (`weights_with_maximum`), which moves the reference to
+    // the tile's maximum when that exceeds it by more than 2^8 and rescales the accumulators.  That
+    // happens a few times per sequence.
+    auto weights_with_maximum = [&](int tile, floatx4 (&sc)[QB][2], auto masked, bf16x8 (&pf)[QB]) {
+      constexpr bool MASKED = decltype(masked)::value;
       float alpha[QB];
       bool rescale = false;
 #pragma unroll
@@ -695,9 +710,6 @@ __global__ __launch_bounds__(256, D <= 128 ? 2 : 1) void attention_prefill_bf16_
           }
         tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 16, WAVE));
         tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32, WAVE));
-        // The reference point of the exponentials follows the maximum only when that has grown by
-        // more than 2^8: weights then stay below 256, well inside float32 and bfloat16, and the
-        // accumulators need rescaling a few times per sequence instead of at nearly every tile.
         const float new_max = tile_max > run_max[b] + rescale_step ? tile_max : run_max[b];
         // a query whose window or position leaves it no key so far keeps its state
         const bool empty = MASKED && new_max == -INFINITY;
@@ -716,13 +728,40 @@ __global__ __launch_bounds__(256, D <= 128 ? 2 : 1) void attention_prefill_bf16_
         run_sum[b] = run_sum[b] * alpha[b] + tile_sum;
         rescale |= alpha[b] != 1.f;
       }
-      // once the running maxima have settled no column needs rescaling: skip the multiplies
+      // once the reference points have settled no column needs rescaling: skip the multiplies
       if (__any(rescale)) {
 #pragma unroll
         for (int b = 0; b < QB; ++b)
 #pragma unroll
           for (int e = 0; e < DB; ++e) o[b][e] *= alpha[b];
       }
+    };
+    auto weights = [&](floatx4 (&sc)[QB][2], bf16x8 (&pf)[QB]) -> bool {
+      float sums[QB];
+      bool again = false;
+#pragma unroll
+      for (int b = 0; b < QB; ++b) {
+        const float shift = -run_max[b] * scale2;                // +inf before the query's first tile: the sum then says "again"
+        float tile_sum = 0.f;
+#pragma unroll
+        for (int h = 0; h < 2; ++h)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            const float p = fast_exp2(fmaf(sc[b][h][i], scale2, shift));
+            tile_sum += p;
+            pf[b][h * 4 + i] = (bf16)p;
+          }
+        sums[b] = tile_sum;
+        again |= !(tile_sum <= 0x1p60f);                         // too large, infinite or not a number
+      }
+      if (__any(again)) return false;
+#pragma unroll
+      for (int b = 0; b < QB; ++b) run_sum[b] += sums[b];
+      return true;
+    };
+    // values: O^T[dim, query] += V^T P
+    auto values = [&](int buffer, const bf16x8 (&pf)[QB]) {
+      const bf16* vt = vs[buffer];
 #pragma unroll
       for (int e = 0; e < DB; ++e) {
         const bf16x4 v0 = *(const bf16x4*)(vt + (e * 16 + col) * VLD + g * 4);
@@ -732,32 +771,52 @@ __global__ __launch_bounds__(256, D <= 128 ? 2 : 1) void attention_prefill_bf16_
         for (int b = 0; b < QB; ++b) o[b][e] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vv, pf[b], o[b][e], 0, 0, 0);
       }
     };
+
+    // Tiles [whole_begin, whole_end) need no mask: every query of the group sees every key of theirs.
+    int whole_begin = (lo_last + 31) / 32, whole_end = (pos_first + 1) / 32;
+    if (whole_begin < first_tile) whole_begin = first_tile;
+    if (whole_begin > last_tile + 1) whole_begin = last_tile + 1;
+    if (whole_end > last_tile + 1) whole_end = last_tile + 1;
+    if (whole_end < whole_begin) whole_end = whole_begin;
+
+    // The walk over the tiles.  At the top of a turn `tile` is in LDS buffer (tile - first_tile) % 2; the
+    // next tile is asked for before the work on this one and put into the other buffer after it.  Most
+    // turns take the short way through the weights; the inner loop holds only those, so that nothing in it
+    // touches the accumulators but the matrix products.  A tile that needs the mask, or whose weights
+    // came out too large for the reference point it was tried with, leaves the inner loop, is finished
+    // the long way and the inner loop begins again behind it.
     __syncthreads();                                           // the buffers of an earlier pass are done with
     if (first_tile <= last_tile) {
       fetch(first_tile, kreg_a, vreg_a);
       stash(0, kreg_a, vreg_a);
     }
     __syncthreads();
-    // At the top of a turn `tile` is in LDS buffer (tile - first_tile) % 2; the next tile is asked
-    // for before the work on this one and put into the other buffer after it.  Three runs of tiles:
-    // those the last query's window cuts, those every query sees whole, those on the diagonal.
-    auto run = [&](int begin, int end, auto masked) {
-      for (int tile = begin; tile < end; ++tile) {
+    floatx4 sc[QB][2];
+    bf16x8 pf[QB];
+    int tile = first_tile;
+    for (;;) {
+      bool unfinished = false;
+      for (; tile <= last_tile; ++tile) {
         const int buffer = (tile - first_tile) & 1;
         if (tile < last_tile) fetch(tile + 1, kreg_a, vreg_a);
-        work(tile, buffer, masked);
+        scores(buffer, sc);
+        if (tile < whole_begin || tile >= whole_end || !weights(sc, pf)) {
+          unfinished = true;
+          break;
+        }
+        values(buffer, pf);
         if (tile < last_tile) stash(buffer ^ 1, kreg_a, vreg_a);
         __syncthreads();
       }
-    };
-    int whole_begin = (lo_last + 31) / 32, whole_end = (pos_first + 1) / 32;   // tiles [whole_begin, whole_end) need no mask
-    if (whole_begin < first_tile) whole_begin = first_tile;
-    if (whole_begin > last_tile + 1) whole_begin = last_tile + 1;
-    if (whole_end > last_tile + 1) whole_end = last_tile + 1;
-    if (whole_end < whole_begin) whole_end = whole_begin;
-    run(first_tile, whole_begin, std::true_type{});
-    run(whole_begin, whole_end, std::false_type{});
-    run(whole_end, last_tile + 1, std::true_type{});
+      if (!unfinished) break;
+      const int buffer = (tile - first_tile) & 1;
+      if (tile < whole_begin || tile >= whole_end) weights_with_maximum(tile, sc, std::true_type{}, pf);
+      else weights_with_maximum(tile, sc, std::false_type{}, pf);
+      values(buffer, pf);
+      if (tile < last_tile) stash(buffer ^ 1, kreg_a, vreg_a);
+      __syncthreads();
+      ++tile;
+    }
 #pragma unroll
     for (int b = 0; b < QB; ++b) {
       float total = run_sum[b];
