@@ -163,12 +163,12 @@ def main() -> int:
     max_batch = args.batch if args.no_points else max(args.batch, 64)
     max_seq_len = args.context + args.steps + args.warmup + decode_lead(max_batch, args.context, max(2048, args.prefill_tokens)) + max_batch + 64
     max_seq_len = max(max_seq_len, args.prefill_tokens)
+    from llm_runtime_study_amd.kernels.ops import KernelChoice
+
     engine = Engine.from_config(config, seed=0, dtype=args.dtype, max_seq_len=max_seq_len, max_batch_size=max_batch,
-                                max_num_batched_tokens=max(2048, args.prefill_tokens), use_cuda_graph=not args.no_graph, library_gemm=not args.own_gemm,
+                                max_num_batched_tokens=max(2048, args.prefill_tokens), use_cuda_graph=not args.no_graph,
+                                kernels=KernelChoice(library=not args.own_gemm, mid=not args.library_mid_gemm),
                                 decode_steps_per_launch=args.decode_steps_per_launch)
-    if args.library_mid_gemm:
-        from llm_runtime_study_amd.kernels import ops
-        ops.gemm_mid_tune(False)
     dtype_name = "bf16" if args.dtype == "bfloat16" else "fp32"
 
     prefill_times = measure_prefill(engine, args.prefill_tokens, repeats=3, seed=1)

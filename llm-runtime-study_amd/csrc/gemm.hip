@@ -963,31 +963,41 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_mid_kernel(
   }
 }
 
-// Whether the few-rows kernel loads its weights as whole 128-byte lines where the shape allows (for measurements).
-static int g_skinny_lines = 1;
-LRS_API int lrs_gemm_skinny_lines(int enabled) {
-  g_skinny_lines = enabled != 0;
-  return 0;
+// Choices a caller may make for the products (measurements and tests; a step carries its runner's).  They
+// travel with every call as one word, so that nothing about them is kept in the library:
+//   bit 0      the kernel for 17..128 rows may be used (else such products take the kernels for other row counts)
+//   bit 1      the few-rows kernel loads its weights as whole 128-byte lines where the shape allows
+//   bits 4-7   workgroup shape of the kernel for 17..128 rows: 4, 6 or 8 waves (0: chosen here)
+//   bits 8-12  its number of K splits, 1..16 (0: chosen here)
+struct GemmTune {
+  bool mid, lines;
+  int waves, splits;
+};
+constexpr int TUNE_DEFAULT = 3;
+static bool tune_ok(int word) {
+  const int waves = (word >> 4) & 15, splits = (word >> 8) & 31;
+  return word >= 0 && (word >> 13) == 0 && (waves == 0 || waves == 4 || waves == 6 || waves == 8) && splits <= 16;
 }
+static GemmTune tune_of(int word) { return GemmTune{(word & 1) != 0, (word & 2) != 0, (word >> 4) & 15, (word >> 8) & 31}; }
 
 // Row tiles per workgroup: more of them means each activation fragment read from L2 serves more
 // weight rows, which matters once there are several token blocks; fewer means more workgroups.
 template <int MT, int RT, bool NORM, bool SWIGLU>
 static void launch_skinny_rt(void* out, int mode, const bf16* a, NormInput norm, const bf16* w, const bf16* bias,
-                             int m, int n, int k, int lda, int ldc, hipStream_t s, float* split_sums = nullptr, int splits = 1,
+                             int m, int n, int k, int lda, int ldc, hipStream_t s, GemmTune tune, float* split_sums = nullptr, int splits = 1,
                              NormChain chain = NormChain{}, int group_rows = 16 * RT) {
   const int groups = (n + group_rows - 1) / group_rows;
   constexpr int UNROLL = (NORM ? 4 : 8) / (MT * RT > 4 ? 4 : (MT * RT > 1 ? 2 : 1));
   if (group_rows != 16 * RT) {
     if constexpr (MT == 1 && RT == 2 && !NORM && !SWIGLU) {
-      if (g_skinny_lines && splits == 1 && k % 64 == 0 && (k / 32) % 16 == 0 && UNROLL % 4 == 0)
+      if (tune.lines && splits == 1 && k % 64 == 0 && (k / 32) % 16 == 0 && UNROLL % 4 == 0)
         gemm_bf16_skinny_kernel<MT, RT, 8, UNROLL, NORM, SWIGLU, true, true><<<dim3(groups, 1), 8 * 64, 0, s>>>(out, mode, a, norm, w, bias, m, n, k, lda, ldc, split_sums, chain, group_rows);
       else
         gemm_bf16_skinny_kernel<MT, RT, 8, UNROLL, NORM, SWIGLU, true><<<dim3(groups, splits), 8 * 64, 0, s>>>(out, mode, a, norm, w, bias, m, n, k, lda, ldc, split_sums, chain, group_rows);
     }
   } else if (groups <= 2048) {
     if constexpr (MT == 1 && !NORM && UNROLL % 4 == 0) {
-      if (g_skinny_lines && splits == 1 && k % 64 == 0 && (k / 32) % 16 == 0) {   // every wave starts at an even step
+      if (tune.lines && splits == 1 && k % 64 == 0 && (k / 32) % 16 == 0) {   // every wave starts at an even step
         gemm_bf16_skinny_kernel<MT, RT, 8, UNROLL, NORM, SWIGLU, false, true><<<dim3(groups, 1), 8 * 64, 0, s>>>(out, mode, a, norm, w, bias, m, n, k, lda, ldc, split_sums, chain, group_rows);
         return;
       }
@@ -1026,32 +1036,26 @@ static float* split_sums_buffer() {
   return g_split_sums;
 }
 
-// The kernel for 17..128 rows: which of its workgroup shapes and how many K splits.  0 = chosen here:
-// the shape and split that fill a whole multiple of the compute units best, then the fewest splits.
-static int g_mid_waves = 0, g_mid_splits = 0, g_mid_enabled = 1;
+// The kernel for 17..128 rows: which of its workgroup shapes and how many K splits.  Unless the caller's
+// choices say otherwise: the shape and split that fill a whole multiple of the compute units best, then the
+// fewest splits.
 LRS_API int lrs_compute_units();
-LRS_API int lrs_gemm_mid_tune(int enabled, int waves, int splits) {
-  LRS_REQUIRE(waves == 0 || waves == 4 || waves == 6 || waves == 8, "gemm_mid_tune: 4, 6 or 8 waves (0: automatic), got %d", waves);
-  LRS_REQUIRE(splits >= 0 && splits <= 16, "gemm_mid_tune: 0..16 splits, got %d", splits);
-  g_mid_enabled = enabled != 0, g_mid_waves = waves, g_mid_splits = splits;
-  return 0;
-}
-LRS_API int lrs_gemm_mid_enabled() { return g_mid_enabled; }
 
-static void choose_mid_shape(int n, int k, int& waves, int& splits) {
+static void choose_mid_shape(int n, int k, GemmTune tune, int& waves, int& splits) {
+  const int want_waves = tune.waves, want_splits = tune.splits;
   const int units = lrs_compute_units() > 0 ? lrs_compute_units() : 256, slices = k / 256;
   auto tiles_of = [&](int wv) { return (n + 16 * wv - 1) / (16 * wv); };
   auto fill_of = [&](int groups) { return (double)groups / ((groups + units - 1) / units * units); };
-  if (g_mid_waves && g_mid_splits) {
-    waves = g_mid_waves, splits = g_mid_splits;
+  if (want_waves && want_splits) {
+    waves = want_waves, splits = want_splits;
     return;
   }
   // Measured on MI355X (Qwen3-8B shapes, 32..64 rows).  A matrix with enough rows to give every compute
   // unit a workgroup is not divided along K: six waves (96 rows) a workgroup, or four where that fills the
   // chip clearly better; eight waves walking many slices were a third slower (gate_up, the LM head).
-  if ((!g_mid_splits || g_mid_splits == 1) && tiles_of(6) >= units && (!g_mid_waves || g_mid_waves == 4 || g_mid_waves == 6)) {
+  if ((!want_splits || want_splits == 1) && tiles_of(6) >= units && (!want_waves || want_waves == 4 || want_waves == 6)) {
     splits = 1;
-    waves = g_mid_waves ? g_mid_waves : (fill_of(tiles_of(4)) > fill_of(tiles_of(6)) + 0.08 ? 4 : 6);
+    waves = want_waves ? want_waves : (fill_of(tiles_of(4)) > fill_of(tiles_of(6)) + 0.08 ? 4 : 6);
     return;
   }
   // A narrower matrix: K is divided so that tiles x splits fills the units once (at least two slices a
@@ -1065,9 +1069,9 @@ static void choose_mid_shape(int n, int k, int& waves, int& splits) {
   const int shapes[3] = {4, 6, 8};
   for (int wi = 0; wi < 3; ++wi) {
     const int wv = shapes[wi];
-    if (g_mid_waves && wv != g_mid_waves) continue;
+    if (want_waves && wv != want_waves) continue;
     for (int sp = 1; sp <= 8; ++sp) {
-      if (g_mid_splits && sp != g_mid_splits) continue;
+      if (want_splits && sp != want_splits) continue;
       if (sp > 1 && slices / sp < 2) continue;
       const int groups = tiles_of(wv) * sp;
       const double fill = groups <= units ? (double)groups / units : fill_of(groups) - 0.25;   // a second round costs more than its share
@@ -1076,7 +1080,7 @@ static void choose_mid_shape(int n, int k, int& waves, int& splits) {
     }
   }
   if (count == 0) {
-    waves = g_mid_waves ? g_mid_waves : 4, splits = g_mid_splits ? g_mid_splits : 1;
+    waves = want_waves ? want_waves : 4, splits = want_splits ? want_splits : 1;
     return;
   }
   const Choice* pick = nullptr;
@@ -1093,18 +1097,19 @@ static void choose_mid_shape(int n, int k, int& waves, int& splits) {
 }
 
 // The shape the kernel for 17..128 rows takes for a matrix of n rows and k columns (for tests and reports).
-LRS_API int lrs_gemm_mid_shape(int n, int k, int* waves, int* splits) {
+LRS_API int lrs_gemm_mid_shape(int n, int k, int tune, int* waves, int* splits) {
   LRS_REQUIRE(n > 0 && k > 0 && k % 256 == 0 && waves && splits, "gemm_mid_shape: needs n > 0 and K %% 256 == 0, got n=%d k=%d", n, k);
-  choose_mid_shape(n, k, *waves, *splits);
+  LRS_REQUIRE(tune_ok(tune), "gemm_mid_shape: unknown choices %d", tune);
+  choose_mid_shape(n, k, tune_of(tune), *waves, *splits);
   return 0;
 }
 
 // keep_sums: the sums of the K splits (of the one split, if K is not divided) stay in the split buffer for
 // the caller's own finishing kernel; returns their number, or 0 if the buffer cannot hold them.
 template <int MT, bool SWIGLU>
-static int launch_mid_mt(void* out, int mode, const bf16* a, const bf16* w, int m, int n, int k, int lda, int ldc, hipStream_t s, bool keep_sums, MidScale scale) {
+static int launch_mid_mt(void* out, int mode, const bf16* a, const bf16* w, int m, int n, int k, int lda, int ldc, hipStream_t s, GemmTune tune, bool keep_sums, MidScale scale) {
   int waves = 4, splits = 1;
-  choose_mid_shape(n, k, waves, splits);
+  choose_mid_shape(n, k, tune, waves, splits);
   float* sums = splits > 1 || keep_sums ? split_sums_buffer() : nullptr;
   if ((splits > 1 || keep_sums) && (!sums || (size_t)splits * m * n * sizeof(float) > SPLIT_SUMS_BYTES)) {
     if (keep_sums) return 0;
@@ -1135,18 +1140,18 @@ static int launch_mid_mt(void* out, int mode, const bf16* a, const bf16* w, int 
 }
 
 template <bool SWIGLU>
-static int launch_mid(void* out, int mode, const bf16* a, const bf16* w, int m, int n, int k, int lda, int ldc, hipStream_t s, bool keep_sums = false,
-                      MidScale scale = MidScale{nullptr, 0, 0.f}) {
-  if (m <= 32) return launch_mid_mt<2, SWIGLU>(out, mode, a, w, m, n, k, lda, ldc, s, keep_sums, scale);
-  if (m <= 48) return launch_mid_mt<3, SWIGLU>(out, mode, a, w, m, n, k, lda, ldc, s, keep_sums, scale);
-  if (m <= 64) return launch_mid_mt<4, SWIGLU>(out, mode, a, w, m, n, k, lda, ldc, s, keep_sums, scale);
-  if (m <= 96) return launch_mid_mt<6, SWIGLU>(out, mode, a, w, m, n, k, lda, ldc, s, keep_sums, scale);
-  return launch_mid_mt<8, SWIGLU>(out, mode, a, w, m, n, k, lda, ldc, s, keep_sums, scale);
+static int launch_mid(void* out, int mode, const bf16* a, const bf16* w, int m, int n, int k, int lda, int ldc, hipStream_t s, GemmTune tune,
+                      bool keep_sums = false, MidScale scale = MidScale{nullptr, 0, 0.f}) {
+  if (m <= 32) return launch_mid_mt<2, SWIGLU>(out, mode, a, w, m, n, k, lda, ldc, s, tune, keep_sums, scale);
+  if (m <= 48) return launch_mid_mt<3, SWIGLU>(out, mode, a, w, m, n, k, lda, ldc, s, tune, keep_sums, scale);
+  if (m <= 64) return launch_mid_mt<4, SWIGLU>(out, mode, a, w, m, n, k, lda, ldc, s, tune, keep_sums, scale);
+  if (m <= 96) return launch_mid_mt<6, SWIGLU>(out, mode, a, w, m, n, k, lda, ldc, s, tune, keep_sums, scale);
+  return launch_mid_mt<8, SWIGLU>(out, mode, a, w, m, n, k, lda, ldc, s, tune, keep_sums, scale);
 }
 
 template <int MT, bool NORM, bool SWIGLU>
 static void launch_skinny(void* out, int mode, const bf16* a, NormInput norm, const bf16* w, const bf16* bias,
-                          int m, int n, int k, int lda, int ldc, hipStream_t s, NormChain chain = NormChain{}) {
+                          int m, int n, int k, int lda, int ldc, hipStream_t s, GemmTune tune, NormChain chain = NormChain{}) {
   if (MT > 1 && !NORM) {
     // several token blocks: 64 weight rows per workgroup, so that an activation fragment read from
     // L2 serves four weight fragments, and K divided between workgroups until there are enough
@@ -1157,33 +1162,33 @@ static void launch_skinny(void* out, int mode, const bf16* a, NormInput norm, co
     while (splits > 1 && k / splits < 512) --splits;
     float* sums = splits > 1 ? split_sums_buffer() : nullptr;
     if (splits > 1 && (!sums || (size_t)splits * m * n * sizeof(float) > SPLIT_SUMS_BYTES)) splits = 1;
-    launch_skinny_rt<MT, (MT > 1 ? 4 : 1), NORM, SWIGLU>(out, mode, a, norm, w, bias, m, n, k, lda, ldc, s, sums, splits);
+    launch_skinny_rt<MT, (MT > 1 ? 4 : 1), NORM, SWIGLU>(out, mode, a, norm, w, bias, m, n, k, lda, ldc, s, tune, sums, splits);
     return;
   }
   if (MT == 1 && !NORM && n >= 16384) {  // measured: two row tiles and four waves stream wide matrices a little faster
-    if (g_skinny_lines && k % 64 == 0 && (k / 32) % 8 == 0)
+    if (tune.lines && k % 64 == 0 && (k / 32) % 8 == 0)
       gemm_bf16_skinny_kernel<1, 2, 4, 4, NORM, SWIGLU, false, true><<<dim3((n + 31) / 32, 1), 4 * 64, 0, s>>>(out, mode, a, norm, w, bias, m, n, k, lda, ldc, nullptr, chain, 32);
     else
       gemm_bf16_skinny_kernel<1, 2, 4, 4, NORM, SWIGLU><<<dim3((n + 31) / 32, 1), 4 * 64, 0, s>>>(out, mode, a, norm, w, bias, m, n, k, lda, ldc, nullptr, chain, 32);
   }
   else if (MT == 1 && !NORM && !SWIGLU && even_group_rows(n) > 0) {
     if constexpr (MT == 1 && !NORM && !SWIGLU)
-      launch_skinny_rt<1, 2, false, false>(out, mode, a, norm, w, bias, m, n, k, lda, ldc, s, nullptr, 1, chain, even_group_rows(n));
+      launch_skinny_rt<1, 2, false, false>(out, mode, a, norm, w, bias, m, n, k, lda, ldc, s, tune, nullptr, 1, chain, even_group_rows(n));
   } else if (MT == 1 || n <= 32 * 128)
-    launch_skinny_rt<MT, 1, NORM, SWIGLU>(out, mode, a, norm, w, bias, m, n, k, lda, ldc, s, nullptr, 1, chain);
+    launch_skinny_rt<MT, 1, NORM, SWIGLU>(out, mode, a, norm, w, bias, m, n, k, lda, ldc, s, tune, nullptr, 1, chain);
   else if (n < 64 * 256)
-    launch_skinny_rt<MT, 2, NORM, SWIGLU>(out, mode, a, norm, w, bias, m, n, k, lda, ldc, s);
+    launch_skinny_rt<MT, 2, NORM, SWIGLU>(out, mode, a, norm, w, bias, m, n, k, lda, ldc, s, tune);
   else
-    launch_skinny_rt<MT, (MT > 1 ? 4 : 1), NORM, SWIGLU>(out, mode, a, norm, w, bias, m, n, k, lda, ldc, s);
+    launch_skinny_rt<MT, (MT > 1 ? 4 : 1), NORM, SWIGLU>(out, mode, a, norm, w, bias, m, n, k, lda, ldc, s, tune);
 }
 
 template <bool NORM, bool SWIGLU>
 static void launch_skinny_m(void* out, int mode, const bf16* a, NormInput norm, const bf16* w, const bf16* bias,
-                            int m, int n, int k, int lda, int ldc, hipStream_t s) {
-  if (m <= 16) launch_skinny<1, NORM, SWIGLU>(out, mode, a, norm, w, bias, m, n, k, lda, ldc, s);
-  else if (m <= 32) launch_skinny<2, NORM, SWIGLU>(out, mode, a, norm, w, bias, m, n, k, lda, ldc, s);
-  else if (m <= 48) launch_skinny<3, NORM, SWIGLU>(out, mode, a, norm, w, bias, m, n, k, lda, ldc, s);
-  else launch_skinny<4, NORM, SWIGLU>(out, mode, a, norm, w, bias, m, n, k, lda, ldc, s);
+                            int m, int n, int k, int lda, int ldc, hipStream_t s, GemmTune tune) {
+  if (m <= 16) launch_skinny<1, NORM, SWIGLU>(out, mode, a, norm, w, bias, m, n, k, lda, ldc, s, tune);
+  else if (m <= 32) launch_skinny<2, NORM, SWIGLU>(out, mode, a, norm, w, bias, m, n, k, lda, ldc, s, tune);
+  else if (m <= 48) launch_skinny<3, NORM, SWIGLU>(out, mode, a, norm, w, bias, m, n, k, lda, ldc, s, tune);
+  else launch_skinny<4, NORM, SWIGLU>(out, mode, a, norm, w, bias, m, n, k, lda, ldc, s, tune);
 }
 
 // Allocates the device memory the K-split products need, so that no later call has to (a call
@@ -1193,16 +1198,10 @@ LRS_API int lrs_gemm_prepare() {
   return 0;
 }
 
-// Largest M for which callers should use the few-rows kernel (and with it the fused RMSNorm input).
-// The kernel itself takes up to 64 rows, but from 17 rows on the kernel for 17..128 rows (or, where a
-// shape does not suit it, the vendor library) is faster, so callers send larger products there.
-static int g_skinny_max_m = 16;
-LRS_API int lrs_gemm_skinny_max_m() { return g_skinny_max_m; }
-LRS_API int lrs_gemm_set_skinny_max_m(int m) {
-  LRS_REQUIRE(m >= 1 && m <= 64, "gemm: the few-rows kernel takes 1..64 rows, got %d", m);
-  g_skinny_max_m = m;
-  return 0;
-}
+// Most rows the few-rows kernel takes (and with it the fused RMSNorm input).  From 17 rows on the kernel for
+// 17..128 rows (or, where a shape does not suit it, the vendor library) is faster, so callers send larger
+// products there unless they are told otherwise.
+LRS_API int lrs_gemm_skinny_capacity() { return 64; }
 
 // How many partial sums of squares a product of n output columns leaves for the norm that follows it
 // (the number of workgroups of the few-rows kernel for that width).
@@ -1220,8 +1219,9 @@ LRS_API int lrs_gemm_norm_chain_parts(int n) {
 LRS_API int lrs_gemm_norm_chain(void* out, int mode, const void* a, const void* w, const void* bias, int m, int n, int k,
                                 int lda, int ldc, int swiglu, const float* in_sumsq, int in_parts, float in_eps,
                                 void* next_x, float* next_sumsq, const void* next_weight, int next_weight_dtype,
-                                void* stream) {
+                                int tune, void* stream) {
   LRS_REQUIRE(m > 0 && m <= 16 && n > 0 && k > 0, "gemm_norm_chain: takes 1..16 rows and positive sizes, got m=%d n=%d k=%d", m, n, k);
+  LRS_REQUIRE(tune_ok(tune), "gemm_norm_chain: unknown choices %d", tune);
   LRS_REQUIRE(lda >= k && ldc >= (swiglu ? n / 2 : n), "gemm_norm_chain: strides lda=%d ldc=%d too small for k=%d n=%d", lda, ldc, k, n);
   LRS_REQUIRE(mode >= OUT_STORE && mode <= OUT_ADD_F32, "gemm_norm_chain: unknown output mode %d", mode);
   LRS_REQUIRE(k % 8 == 0 && lda % 8 == 0 && ((uintptr_t)a % 16 == 0) && ((uintptr_t)w % 16 == 0),
@@ -1233,8 +1233,8 @@ LRS_API int lrs_gemm_norm_chain(void* out, int mode, const void* a, const void* 
   const NormChain chain{in_sumsq, in_parts, in_eps, (bf16*)next_x, next_sumsq, next_weight, next_weight_dtype == LRS_F32};
   const NormInput none{nullptr, nullptr, nullptr, 0, 0.f};
   hipStream_t s = (hipStream_t)stream;
-  if (swiglu) launch_skinny<1, false, true>(out, mode, (const bf16*)a, none, (const bf16*)w, nullptr, m, n, k, lda, ldc, s, chain);
-  else launch_skinny<1, false, false>(out, mode, (const bf16*)a, none, (const bf16*)w, (const bf16*)bias, m, n, k, lda, ldc, s, chain);
+  if (swiglu) launch_skinny<1, false, true>(out, mode, (const bf16*)a, none, (const bf16*)w, nullptr, m, n, k, lda, ldc, s, tune_of(tune), chain);
+  else launch_skinny<1, false, false>(out, mode, (const bf16*)a, none, (const bf16*)w, (const bf16*)bias, m, n, k, lda, ldc, s, tune_of(tune), chain);
   return lrs_check_launch("gemm_norm_chain");
 }
 
@@ -1247,15 +1247,16 @@ static bool mid_shape_ok(const void* a, const void* w, int m, int n, int k, int 
 // [M, K], in_sumsq [in_parts, M] partial sums of h^2; row r of the result is multiplied by
 // rsqrt(sum_p in_sumsq[p, r] / K + in_eps).  swiglu as in lrs_gemm.
 LRS_API int lrs_gemm_mid_scaled(void* out, int mode, const void* a, const void* w, int m, int n, int k, int lda, int ldc,
-                                int swiglu, const float* in_sumsq, int in_parts, float in_eps, void* stream) {
+                                int swiglu, const float* in_sumsq, int in_parts, float in_eps, int tune, void* stream) {
+  LRS_REQUIRE(tune_ok(tune), "gemm_mid_scaled: unknown choices %d", tune);
   LRS_REQUIRE(mid_shape_ok(a, w, m, n, k, lda), "gemm_mid_scaled: takes 17..128 rows, K %% 256 == 0, N %% 16 == 0, 16-byte aligned rows (m=%d n=%d k=%d lda=%d)", m, n, k, lda);
   LRS_REQUIRE(mode >= OUT_STORE && mode <= OUT_ADD_F32 && ldc >= (swiglu ? n / 2 : n) && ldc % 4 == 0 && (uintptr_t)out % 16 == 0,
               "gemm_mid_scaled: unknown output mode %d, or an output that is not 16-byte aligned (ldc=%d)", mode, ldc);
   LRS_REQUIRE(!swiglu || mode == OUT_STORE, "gemm_mid_scaled: swiglu needs a stored output");
   LRS_REQUIRE(in_sumsq != nullptr && in_parts > 0 && in_eps > 0.f, "gemm_mid_scaled: needs the partial sums of squares, their number and eps");
   const MidScale scale{in_sumsq, in_parts, in_eps};
-  if (swiglu) launch_mid<true>(out, mode, (const bf16*)a, (const bf16*)w, m, n, k, lda, ldc, (hipStream_t)stream, false, scale);
-  else launch_mid<false>(out, mode, (const bf16*)a, (const bf16*)w, m, n, k, lda, ldc, (hipStream_t)stream, false, scale);
+  if (swiglu) launch_mid<true>(out, mode, (const bf16*)a, (const bf16*)w, m, n, k, lda, ldc, (hipStream_t)stream, tune_of(tune), false, scale);
+  else launch_mid<false>(out, mode, (const bf16*)a, (const bf16*)w, m, n, k, lda, ldc, (hipStream_t)stream, tune_of(tune), false, scale);
   return lrs_check_launch("gemm_mid_scaled");
 }
 
@@ -1270,10 +1271,11 @@ extern "C" int lrs_split_add_norm_begin(float* x, const float* sums, int splits,
 // (lrs_gemm_mid_scaled) or for scale_rows.  The kernel that adds the K splits' sums spreads over rows x 1,024
 // columns, where a whole norm would have one workgroup a row.
 LRS_API int lrs_gemm_mid_add_norm_begin(float* residual, const void* a, const void* w, const void* norm_weight, int norm_weight_dtype,
-                                        void* next_x, float* next_sumsq, int m, int n, int k, int lda, void* stream) {
+                                        void* next_x, float* next_sumsq, int m, int n, int k, int lda, int tune, void* stream) {
+  LRS_REQUIRE(tune_ok(tune), "gemm_mid_add_norm_begin: unknown choices %d", tune);
   LRS_REQUIRE(mid_shape_ok(a, w, m, n, k, lda) && ((uintptr_t)residual % 16 == 0), "gemm_mid_add_norm_begin: takes 17..128 rows, K %% 256 == 0, N %% 16 == 0, 16-byte aligned rows (m=%d n=%d k=%d lda=%d)", m, n, k, lda);
   LRS_REQUIRE(next_x && next_sumsq && norm_weight, "gemm_mid_add_norm_begin: needs the norm weight and the two outputs for the next norm");
-  const int splits = launch_mid<false>(nullptr, OUT_STORE, (const bf16*)a, (const bf16*)w, m, n, k, lda, n, (hipStream_t)stream, true);
+  const int splits = launch_mid<false>(nullptr, OUT_STORE, (const bf16*)a, (const bf16*)w, m, n, k, lda, n, (hipStream_t)stream, tune_of(tune), true);
   LRS_REQUIRE(splits > 0, "gemm_mid_add_norm_begin: the buffer for the sums of the K splits cannot hold %d x %d values", m, n);
   if (int rc = lrs_check_launch("gemm_mid_add_norm_begin")) return rc;
   return lrs_split_add_norm_begin(residual, split_sums_buffer(), splits, norm_weight, norm_weight_dtype, next_x, next_sumsq, m, n, stream);
@@ -1292,12 +1294,13 @@ LRS_API int lrs_gemm_mid_qk_prep(void* qkv, int row_stride, const void* a, const
                                  const float* in_sumsq, int in_parts, float in_eps, int nq, int nkv, int d,
                                  const void* q_weight, const void* k_weight, int w_dtype, float eps, const float* cosv,
                                  const float* sinv, int rot_half, void* k_pages, void* v_pages, const int* slots,
-                                 int page_size, void* stream) {
+                                 int page_size, int tune, void* stream) {
   const int n = (nq + 2 * nkv) * d;
+  LRS_REQUIRE(tune_ok(tune), "gemm_mid_qk_prep: unknown choices %d", tune);
   LRS_REQUIRE(mid_shape_ok(a, w, m, n, k, lda), "gemm_mid_qk_prep: takes 17..128 rows, K %% 256 == 0, N %% 16 == 0, 16-byte aligned rows (m=%d n=%d k=%d lda=%d)", m, n, k, lda);
   LRS_REQUIRE(in_sumsq == nullptr || (in_parts > 0 && in_eps > 0.f), "gemm_mid_qk_prep: in_parts and in_eps must be positive");
   const MidScale scale{in_sumsq, in_parts, in_eps};
-  const int splits = launch_mid<false>(nullptr, OUT_STORE, (const bf16*)a, (const bf16*)w, m, n, k, lda, n, (hipStream_t)stream, true, scale);
+  const int splits = launch_mid<false>(nullptr, OUT_STORE, (const bf16*)a, (const bf16*)w, m, n, k, lda, n, (hipStream_t)stream, tune_of(tune), true, scale);
   LRS_REQUIRE(splits > 0, "gemm_mid_qk_prep: the buffer for the sums of the K splits cannot hold %d x %d values", m, n);
   if (int rc = lrs_check_launch("gemm_mid_qk_prep")) return rc;
   return lrs_qk_prep_from_sums(qkv, LRS_BF16, m, row_stride, nq, nkv, d, q_weight, k_weight, w_dtype, eps, cosv, sinv, rot_half, k_pages,
@@ -1307,13 +1310,15 @@ LRS_API int lrs_gemm_mid_qk_prep(void* qkv, int row_stride, const void* a, const
 // out [M, N] (row stride ldc) = a [M, K] (row stride lda) times w[N, K]^T.
 //   norm_weight != null: `a` is the float32 residual stream [*, K]; its rows (picked through
 //     `rows` if given) are RMS-normalised with norm_weight and eps on the way in.  bf16 weights,
-//     M <= lrs_gemm_skinny_max_m() only.
+//     at most 64 rows.
 //   swiglu != 0: w holds gate and up rows interleaved in groups of 8 and out is [M, N/2] with
 //     silu(gate) * up.  bf16, K % 8 == 0, no bias.
 LRS_API int lrs_gemm(void* out, int mode, const void* a, const void* w, const void* bias, int dtype,
                      int m, int n, int k, int lda, int ldc, const int* rows, const void* norm_weight,
-                     int norm_weight_dtype, float eps, int swiglu, void* stream) {
+                     int norm_weight_dtype, float eps, int swiglu, int tune_word, void* stream) {
   LRS_REQUIRE(m > 0 && n > 0 && k > 0, "gemm: sizes m=%d n=%d k=%d must be positive", m, n, k);
+  LRS_REQUIRE(tune_ok(tune_word), "gemm: unknown choices %d", tune_word);
+  const GemmTune tune = tune_of(tune_word);
   LRS_REQUIRE(lda >= k && ldc >= (swiglu ? n / 2 : n), "gemm: strides lda=%d ldc=%d too small for k=%d n=%d", lda, ldc, k, n);
   LRS_REQUIRE(mode >= OUT_STORE && mode <= OUT_ADD_F32, "gemm: unknown output mode %d", mode);
   hipStream_t s = (hipStream_t)stream;
@@ -1331,19 +1336,19 @@ LRS_API int lrs_gemm(void* out, int mode, const void* a, const void* w, const vo
     gemm_tiled_kernel<float><<<grid, 256, 0, s>>>(out, mode, (const float*)a, (const float*)w,
                                                   (const float*)bias, m, n, k, lda, ldc);
   } else if (dtype == LRS_BF16) {
-    const bool mid = aligned && m > 16 && m <= 128 && !normed && !bias && g_mid_enabled && k % 256 == 0 && n % 16 == 0 && ldc % 4 == 0 &&
+    const bool mid = aligned && m > 16 && m <= 128 && !normed && !bias && tune.mid && k % 256 == 0 && n % 16 == 0 && ldc % 4 == 0 &&
                      (uintptr_t)out % 16 == 0;
     if (aligned && (m <= 64 || mid)) {
       const bf16 *wp = (const bf16*)w, *bp = (const bf16*)bias;
       const NormInput norm{(const float*)a, rows, norm_weight, norm_weight_dtype == LRS_F32, eps};
       const bf16* ap = normed ? nullptr : (const bf16*)a;
       if (mid) {
-        if (swiglu) launch_mid<true>(out, mode, ap, wp, m, n, k, lda, ldc, s);
-        else launch_mid<false>(out, mode, ap, wp, m, n, k, lda, ldc, s);
-      } else if (normed && swiglu) launch_skinny_m<true, true>(out, mode, ap, norm, wp, bp, m, n, k, lda, ldc, s);
-      else if (normed) launch_skinny_m<true, false>(out, mode, ap, norm, wp, bp, m, n, k, lda, ldc, s);
-      else if (swiglu) launch_skinny_m<false, true>(out, mode, ap, norm, wp, bp, m, n, k, lda, ldc, s);
-      else launch_skinny_m<false, false>(out, mode, ap, norm, wp, bp, m, n, k, lda, ldc, s);
+        if (swiglu) launch_mid<true>(out, mode, ap, wp, m, n, k, lda, ldc, s, tune);
+        else launch_mid<false>(out, mode, ap, wp, m, n, k, lda, ldc, s, tune);
+      } else if (normed && swiglu) launch_skinny_m<true, true>(out, mode, ap, norm, wp, bp, m, n, k, lda, ldc, s, tune);
+      else if (normed) launch_skinny_m<true, false>(out, mode, ap, norm, wp, bp, m, n, k, lda, ldc, s, tune);
+      else if (swiglu) launch_skinny_m<false, true>(out, mode, ap, norm, wp, bp, m, n, k, lda, ldc, s, tune);
+      else launch_skinny_m<false, false>(out, mode, ap, norm, wp, bp, m, n, k, lda, ldc, s, tune);
     } else if (aligned && k % WIDE_BK == 0 && n % 4 == 0 && ldc % 4 == 0 && (uintptr_t)out % 16 == 0 && !bias &&
                (int64_t)m * lda < (1ll << 31) && (int64_t)n * k < (1ll << 31)) {
       const int tiles_m = (m + 127) / 128, tiles_n = (n + 255) / 256;

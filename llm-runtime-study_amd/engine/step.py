@@ -81,7 +81,7 @@ class StepContext:
 
     def __init__(self, runner: "ModelRunner"):
         self._runner = runner
-        self.library_gemm = runner.library_gemm
+        self.kernels = runner.kernels          # which matrix-product kernels this runner's steps use (ops.KernelChoice)
         self.dtype = runner.dtype
         self.device = runner.device
         self.memo: dict = {}
@@ -108,15 +108,18 @@ class StepContext:
 
 class ModelRunner:
     def __init__(self, model: DecoderModel, cache: CacheManager, *, max_step_tokens: int, dtype: torch.dtype, device,
-                 use_graph: bool = False, library_gemm: bool = True):
+                 use_graph: bool = False, library_gemm: bool = True, kernels: "ops.KernelChoice | None" = None):
         if max_step_tokens <= 0:
             raise GenerationError(f"max_step_tokens must be positive, got {max_step_tokens}")
         self.model, self.cache, self.dtype, self.device = model, cache, dtype, torch.device(device)
         self.max_step_tokens = max_step_tokens
         self.max_requests = cache.max_requests
         self.arena = ScratchArena(self.device)
-        # bfloat16 products of more rows than the few-rows kernel takes go to the vendor library
-        self.library_gemm = library_gemm
+        # Which matrix-product kernels this runner's steps use: a property of the runner, carried by every step's
+        # context, never of the process.  Unless `kernels` says otherwise: bfloat16 products of more rows than this
+        # package's kernels for few rows take go to the vendor library, if `library_gemm` allows it.
+        self.kernels = kernels if kernels is not None else ops.KernelChoice(library=library_gemm)
+        self.library_gemm = self.kernels.library
         # decode-only steps are captured in a HIP graph per padded batch size and replayed
         self.use_graph = use_graph and model.graph_safe()
         self._graphs: dict[tuple, tuple] = {}   # (bucket, length class) -> (handle, arena generation, logits tensor)
@@ -549,7 +552,7 @@ class ModelRunner:
         # A bfloat16 graph of up to 128 rows holds this package's kernels (the few-rows kernels, then the
         # kernel for 17..128 rows); where a shape does not suit that kernel (K no multiple of 256) and the runner
         # may use the vendor library, its products are captured with them.
-        most = max(ops.skinny_max_m(), self.GRAPH_ROWS) if self.dtype == torch.bfloat16 else ops.skinny_max_m()
+        most = max(self.kernels.few_rows_max, self.GRAPH_ROWS) if self.dtype == torch.bfloat16 else self.kernels.few_rows_max
         return bucket if bucket <= min(self.max_step_tokens, most) else 0
 
     def _step_graph(self, entries: Sequence[StepEntry], bucket: int) -> torch.Tensor | None:

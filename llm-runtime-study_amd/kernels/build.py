@@ -28,6 +28,9 @@ ARCH = "gfx950"
 # -packed-fp32-ops: keep the compiler from forming packed float32 instructions.
 DEVICE_FLAGS = ["-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
 FLAGS = [f"--offload-arch={ARCH}", "-O3", "-std=c++17", "-fPIC", "-fvisibility=hidden", "-Wno-unused-command-line-argument"] + DEVICE_FLAGS
+# the vendor's matrix library, for bfloat16 products of many rows (csrc/library_gemm.hip)
+ROCM_LIB = Path(os.environ.get("ROCM_PATH", "/opt/rocm")) / "lib"
+LINK_FLAGS = [f"-L{ROCM_LIB}", "-lhipblaslt", f"-Wl,-rpath,{ROCM_LIB}"]
 
 
 class BuildError(RuntimeError):
@@ -43,7 +46,7 @@ def source_hash() -> str:
     for path in sorted(SOURCE_DIR.glob("*.hip")) + sorted(SOURCE_DIR.glob("*.h")):
         digest.update(path.name.encode())
         digest.update(path.read_bytes())
-    digest.update(" ".join(FLAGS).encode())
+    digest.update(" ".join(FLAGS + LINK_FLAGS).encode())
     return digest.hexdigest()
 
 
@@ -105,7 +108,7 @@ def build(force: bool = True) -> Path:
             future.result()
     tmp = library.with_suffix(f".so.tmp{os.getpid()}")
     proc = subprocess.run(
-        [hipcc, f"--offload-arch={ARCH}", "-shared", "-fPIC", *map(str, objects), "-o", str(tmp)],
+        [hipcc, f"--offload-arch={ARCH}", "-shared", "-fPIC", *map(str, objects), *LINK_FLAGS, "-o", str(tmp)],
         capture_output=True, text=True,
     )
     if proc.returncode != 0:

@@ -101,33 +101,30 @@ def gemm(args) -> None:
     shapes = [("qkv", qkv, hidden), ("o", hidden, args.heads * args.head_dim), ("gate_up", 2 * inter, hidden), ("down", hidden, inter)]
     if args.vocab_size:
         shapes.append(("lm_head", args.vocab_size, hidden))
-    before = ops.skinny_max_m()
-    ops.set_skinny_max_m(64)            # time the few-rows kernel up to its own limit, not the caller's
-    ops.gemm_skinny_lines(not args.fragment_loads)
-    try:
+    # the few-rows kernel is timed up to its own limit, not the one steps use
+    base = dict(few_rows_max=ops.few_rows_capacity(), whole_lines=not args.fragment_loads)
+    if True:
         for name, n, k in shapes:
             sets = max(2, min(16, int(1.2e9 / (n * k * 2))))
             weights = [torch.randn(n, k, device="cuda", dtype=torch.bfloat16) for _ in range(sets)]
             for rows in _ints(args.rows):
                 x = torch.randn(rows, k, device="cuda", dtype=torch.bfloat16)
                 out = torch.empty(rows, n, device="cuda", dtype=torch.bfloat16)
-                variants = [("own", 0, 0), ("library", 0, 0)]
+                variants = [("own", 0, 0), ("library", 0, 0), ("torch.mm", 0, 0)]
                 if args.mid_sweep and 16 < rows <= 128:
                     variants = [(f"mid w{wv} s{sp}", wv, sp) for wv in (4, 6, 8) for sp in _ints(args.mid_sweep)] + variants
                 for which, wv, sp in variants:
                     if which == "library":
+                        call = lambda i: ops.library_gemm(out, x, weights[i % sets])
+                    elif which == "torch.mm":
                         call = lambda i: torch.mm(x, weights[i % sets].t(), out=out)
                     else:
-                        ops.gemm_mid_tune(True, wv, sp)
-                        call = lambda i: ops.gemm(out, x, weights[i % sets])
+                        choice = ops.KernelChoice(mid_waves=wv, mid_splits=sp, **base)
+                        call = lambda i: ops.gemm(out, x, weights[i % sets], choice=choice)
                     seconds = _time(call, max(args.repeats, 2 * sets))
                     print(f"gemm {name:8s} rows={rows:5d} {which:10s} {seconds * 1e6:9.1f} us  {n * k * 2 / seconds / 1e9:8.0f} GB/s of weights  "
                           f"{2 * rows * n * k / seconds / 1e12:8.1f} TFLOP/s", flush=True)
-                ops.gemm_mid_tune(True, 0, 0)
             del weights
-    finally:
-        ops.set_skinny_max_m(before)
-        ops.gemm_skinny_lines(True)
 
 
 def memory(args) -> None:

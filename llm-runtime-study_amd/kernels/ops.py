@@ -23,6 +23,42 @@ _lib_path = ""
 F32, BF16 = 0, 1
 OUT_STORE, OUT_STORE_F32, OUT_ADD_F32 = 0, 1, 2
 
+
+@dataclass(frozen=True)
+class KernelChoice:
+    """Which matrix-product kernels a caller wants where there is a choice.  A step carries its runner's
+    (`ctx.kernels`); measurements and tests make their own.  Nothing of it is kept in the kernel library:
+    the parts that concern a kernel travel with every call.
+
+    few_rows_max   rows up to which the few-rows kernels (and the norms folded into them) are used: 16 in
+                   steps, since from 17 rows on other kernels are faster; the kernels themselves take 64
+    mid            the kernel for 17..128 rows may be used
+    mid_waves, mid_splits   its workgroup shape (4, 6 or 8 waves) and number of K splits (0: its own choice)
+    whole_lines    the few-rows kernel loads its weights as whole 128-byte lines where the shape allows
+    library        bfloat16 products of more rows than these kernels are made for go to the vendor's matrix
+                   library (as the reference leaves them to nn.Linear); else to this package's own kernel"""
+
+    few_rows_max: int = 16
+    mid: bool = True
+    mid_waves: int = 0
+    mid_splits: int = 0
+    whole_lines: bool = True
+    library: bool = True
+
+    def __post_init__(self):
+        if not 1 <= self.few_rows_max <= 64:
+            raise KernelError(f"the few-rows kernel takes 1..64 rows, got few_rows_max={self.few_rows_max}")
+        if self.mid_waves not in (0, 4, 6, 8) or not 0 <= self.mid_splits <= 16:
+            raise KernelError(f"the kernel for 17..128 rows has 4, 6 or 8 waves and 1..16 K splits (0: its own choice), got {self.mid_waves} and {self.mid_splits}")
+
+    @property
+    def word(self) -> int:
+        """The choices a kernel launch needs, as the one integer the entry points take."""
+        return int(self.mid) | int(self.whole_lines) << 1 | self.mid_waves << 4 | self.mid_splits << 8
+
+
+DEFAULT_CHOICE = KernelChoice()
+
 _SIGNATURES = {
     "lrs_last_error": (c_char_p, []),
     "lrs_device_arch": (c_int, [c_int, c_char_p, c_int, POINTER(c_int)]),
@@ -38,31 +74,29 @@ _SIGNATURES = {
     "lrs_qk_prep": (c_int, [c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_int, c_float,
                             c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p]),
     "lrs_gemm_mid_qk_prep": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p, c_int, c_float, c_int, c_int, c_int,
-                                     c_void_p, c_void_p, c_int, c_float, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p]),
+                                     c_void_p, c_void_p, c_int, c_float, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p]),
     "lrs_silu_mul": (c_int, [c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p]),
     "lrs_add_into": (c_int, [c_void_p, c_void_p, c_int, c_int64, c_void_p]),
     "lrs_fill_i32": (c_int, [c_void_p, c_int, c_int64, c_void_p]),
     "lrs_gather_rows": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p]),
     "lrs_gemm": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p,
-                         c_int, c_float, c_int, c_void_p]),
+                         c_int, c_float, c_int, c_int, c_void_p]),
     "lrs_gemm_norm_chain": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,
-                                    c_void_p, c_int, c_float, c_void_p, c_void_p, c_void_p, c_int, c_void_p]),
+                                    c_void_p, c_int, c_float, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p]),
     "lrs_gemm_norm_chain_parts": (c_int, [c_int]),
     "lrs_scale_rows": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_float, c_void_p]),
-    "lrs_gemm_skinny_max_m": (c_int, []),
+    "lrs_gemm_skinny_capacity": (c_int, []),
     "lrs_advance_decode": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p]),
     "lrs_advance_slots": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p, c_int, c_void_p]),
     "lrs_copy_to_pinned": (c_int, [c_void_p, c_void_p, c_int64, c_void_p]),
     "lrs_stream_read": (c_int, [c_void_p, c_int64, c_void_p, c_int, c_void_p]),
     "lrs_gemm_prepare": (c_int, []),
+    "lrs_library_gemm_prepare": (c_int, []),
+    "lrs_library_gemm": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p]),
     "lrs_host_device_pointer": (c_int, [c_void_p, POINTER(c_void_p)]),
-    "lrs_gemm_set_skinny_max_m": (c_int, [c_int]),
-    "lrs_gemm_mid_tune": (c_int, [c_int, c_int, c_int]),
-    "lrs_gemm_mid_enabled": (c_int, []),
-    "lrs_gemm_skinny_lines": (c_int, [c_int]),
-    "lrs_gemm_mid_shape": (c_int, [c_int, c_int, c_void_p, c_void_p]),
-    "lrs_gemm_mid_scaled": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_int, c_float, c_void_p]),
-    "lrs_gemm_mid_add_norm_begin": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p]),
+    "lrs_gemm_mid_shape": (c_int, [c_int, c_int, c_int, c_void_p, c_void_p]),
+    "lrs_gemm_mid_scaled": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_int, c_float, c_int, c_void_p]),
+    "lrs_gemm_mid_add_norm_begin": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p]),
     "lrs_norm_begin_parts": (c_int, [c_int]),
     "lrs_attention": (c_int, [c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p,
                               c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_void_p]),
@@ -102,6 +136,7 @@ def library():
             torch.cuda.init()
             _check(lib.lrs_gemm_prepare())   # device scratch is made now, never inside a step
             _check(lib.lrs_choose_tokens_static_init())
+            _check(lib.lrs_library_gemm_prepare())
     return _lib
 
 
@@ -278,23 +313,25 @@ def qk_prep(qkv: torch.Tensor, nq: int, nkv: int, d: int, q_weight, k_weight, ep
         None if nkv == 0 else _dev(slots, "slots"), page_size, _stream()))
 
 
-def gemm_mid_qk_prep_takes(dtype: torch.dtype, m: int, nq: int, nkv: int, d: int, k: int, rot_half: int) -> bool:
+def gemm_mid_qk_prep_takes(dtype: torch.dtype, m: int, nq: int, nkv: int, d: int, k: int, rot_half: int,
+                           choice: KernelChoice = DEFAULT_CHOICE) -> bool:
     """Whether gemm_mid_qk_prep() takes the shape: bf16, 17..128 rows, heads the vector form of qk_prep takes
     (head_dim 16, 32, 64, ... 1024, rotation over the whole head or none), cache written by this layer."""
     per_head = d // 16
-    return (gemm_mid_takes(dtype, m, (nq + 2 * nkv) * d, k, MID_ROWS_PREFERRED) and nkv > 0 and d % 16 == 0 and 0 < per_head <= 64
+    return (gemm_mid_takes(dtype, m, (nq + 2 * nkv) * d, k, MID_ROWS_PREFERRED, choice) and nkv > 0 and d % 16 == 0 and 0 < per_head <= 64
             and per_head & (per_head - 1) == 0 and rot_half in (0, d // 2))
 
 
 def gemm_mid_qk_prep(qkv: torch.Tensor, a: torch.Tensor, w: torch.Tensor, sumsq: torch.Tensor | None, in_eps: float, nq: int, nkv: int,
-                     d: int, q_weight, k_weight, eps: float, cos, sin, k_pages, v_pages, slots, page_size: int) -> None:
+                     d: int, q_weight, k_weight, eps: float, cos, sin, k_pages, v_pages, slots, page_size: int,
+                     choice: KernelChoice = DEFAULT_CHOICE) -> None:
     """The q/k/v product of 17..128 bf16 rows (a @ w.T; with `sumsq` the input is a norm begun before it, as in
     gemm_mid_scaled) and qk_prep() of its result in two kernels: the one that prepares the heads adds up the sums of
     the product's K splits itself.  q goes into `qkv` [M, (nq+2*nkv)*d], k and v into the pages."""
     m, k = a.shape
     n = (nq + 2 * nkv) * d
     rot_half = 0 if cos is None else cos.shape[1]
-    _need(a.dtype == torch.bfloat16 and gemm_mid_qk_prep_takes(w.dtype, m, nq, nkv, d, k, rot_half), "gemm_mid_qk_prep: shape not taken (see gemm_mid_qk_prep_takes)")
+    _need(a.dtype == torch.bfloat16 and gemm_mid_qk_prep_takes(w.dtype, m, nq, nkv, d, k, rot_half, choice), "gemm_mid_qk_prep: shape not taken (see gemm_mid_qk_prep_takes)")
     _need(w.shape == (n, k) and w.is_contiguous(), f"gemm_mid_qk_prep: weight must be contiguous [{n}, {k}]")
     _need(qkv.dtype == torch.bfloat16 and qkv.shape == (m, n), f"gemm_mid_qk_prep: qkv must be bf16 [{m}, {n}]")
     if sumsq is not None:
@@ -315,7 +352,7 @@ def gemm_mid_qk_prep(qkv: torch.Tensor, a: torch.Tensor, w: torch.Tensor, sumsq:
         None if sumsq is None else _dev(sumsq, "sumsq"), 0 if sumsq is None else sumsq.shape[0], in_eps if sumsq is not None else 0.0,
         nq, nkv, d, None if q_weight is None else _dev(q_weight, "q_weight"), None if k_weight is None else _dev(k_weight, "k_weight"),
         dtype_code(w_dtype), eps, None if cos is None else cos.data_ptr(), None if sin is None else sin.data_ptr(), rot_half,
-        _dev(k_pages, "k_pages"), _dev(v_pages, "v_pages"), _dev(slots, "slots"), page_size, _stream()))
+        _dev(k_pages, "k_pages"), _dev(v_pages, "v_pages"), _dev(slots, "slots"), page_size, choice.word, _stream()))
 
 
 def silu_mul(out: torch.Tensor, gate_up: torch.Tensor, interleaved: bool = False) -> None:
@@ -331,32 +368,16 @@ def add_into(residual: torch.Tensor, y: torch.Tensor) -> None:
     _check(library().lrs_add_into(_dev(residual, "residual"), _dev(y, "y"), dtype_code(y.dtype), residual.numel(), _stream()))
 
 
-def skinny_max_m() -> int:
-    """Most rows for which the few-rows product kernel is the one to use."""
-    return library().lrs_gemm_skinny_max_m()
+def few_rows_capacity() -> int:
+    """Most rows the few-rows product kernel takes at all (callers use it up to KernelChoice.few_rows_max)."""
+    return library().lrs_gemm_skinny_capacity()
 
 
-def gemm_mid_tune(enabled: bool = True, waves: int = 0, splits: int = 0) -> None:
-    """Whether bf16 products of 17..128 rows take this package's kernel for them, and (for measurements)
-    its workgroup shape (4, 6 or 8 waves) and number of K splits; 0 lets the library choose."""
-    _check(library().lrs_gemm_mid_tune(int(bool(enabled)), waves, splits))
-
-
-def gemm_skinny_lines(enabled: bool) -> None:
-    """Whether the few-rows kernel loads its weights as whole 128-byte lines where the shape allows (for measurements)."""
-    _check(library().lrs_gemm_skinny_lines(int(bool(enabled))))
-
-
-def gemm_mid_shape(n: int, k: int) -> tuple[int, int]:
+def gemm_mid_shape(n: int, k: int, choice: KernelChoice = DEFAULT_CHOICE) -> tuple[int, int]:
     """(waves a workgroup, K splits) the kernel for 17..128 rows takes for a weight matrix [n, k]."""
-    import ctypes
-    waves, splits = ctypes.c_int(0), ctypes.c_int(0)
-    _check(library().lrs_gemm_mid_shape(n, k, ctypes.addressof(waves), ctypes.addressof(splits)))
+    waves, splits = c_int(0), c_int(0)
+    _check(library().lrs_gemm_mid_shape(n, k, choice.word, ctypes.addressof(waves), ctypes.addressof(splits)))
     return waves.value, splits.value
-
-
-def gemm_mid_enabled() -> bool:
-    return bool(library().lrs_gemm_mid_enabled())
 
 
 # Rows up to which callers that may use the vendor library take this package's kernel for 17..128 rows instead.
@@ -366,10 +387,10 @@ def gemm_mid_enabled() -> bool:
 MID_ROWS_PREFERRED = 128
 
 
-def gemm_mid_takes(dtype: torch.dtype, m: int, n: int, k: int, most: int = 128) -> bool:
+def gemm_mid_takes(dtype: torch.dtype, m: int, n: int, k: int, most: int = 128, choice: KernelChoice = DEFAULT_CHOICE) -> bool:
     """Whether a product of m rows (at most `most`) can go to the kernel for 17..128 rows (weights streamed
     once, activations shared through LDS), which also writes the gated activation itself."""
-    return dtype == torch.bfloat16 and 16 < m <= min(most, 128) and k % 256 == 0 and n % 16 == 0 and gemm_mid_enabled()
+    return dtype == torch.bfloat16 and 16 < m <= min(most, 128) and k % 256 == 0 and n % 16 == 0 and choice.mid
 
 
 def norm_begin_parts(n: int) -> int:
@@ -378,13 +399,13 @@ def norm_begin_parts(n: int) -> int:
 
 
 def gemm_mid_add_norm_begin(residual: torch.Tensor, a: torch.Tensor, w: torch.Tensor, norm_weight: torch.Tensor,
-                            next_x: torch.Tensor, next_sumsq: torch.Tensor) -> None:
+                            next_x: torch.Tensor, next_sumsq: torch.Tensor, choice: KernelChoice = DEFAULT_CHOICE) -> None:
     """residual (float32 [M, N]) += a @ w.T for 17..128 bf16 rows, and the first half of the RMSNorm that follows:
     next_x [M, N] = bf16(residual * norm_weight), next_sumsq [norm_begin_parts(N), M] = partial sums of residual^2.
     gemm_mid_scaled() (or scale_rows()) finishes the norm."""
     m, k = a.shape
     n = w.shape[0]
-    _need(gemm_mid_takes(w.dtype, m, n, k) and a.dtype == torch.bfloat16, "gemm_mid_add_norm_begin: takes bf16 products of 17..128 rows, K % 256 == 0, N % 16 == 0")
+    _need(gemm_mid_takes(w.dtype, m, n, k, 128, choice) and a.dtype == torch.bfloat16, "gemm_mid_add_norm_begin: takes bf16 products of 17..128 rows, K % 256 == 0, N % 16 == 0")
     _need(w.dim() == 2 and w.is_contiguous() and w.shape[1] == k, f"gemm_mid_add_norm_begin: weight must be contiguous [N, {k}]")
     _need(residual.dtype == torch.float32 and residual.is_contiguous() and residual.shape == (m, n), f"gemm_mid_add_norm_begin: residual must be contiguous float32 [{m}, {n}]")
     _need(next_x.dtype == torch.bfloat16 and next_x.is_contiguous() and next_x.shape == (m, n), f"gemm_mid_add_norm_begin: next_x must be contiguous bf16 [{m}, {n}]")
@@ -393,28 +414,24 @@ def gemm_mid_add_norm_begin(residual: torch.Tensor, a: torch.Tensor, w: torch.Te
     _need(norm_weight.is_contiguous() and norm_weight.numel() == n, f"gemm_mid_add_norm_begin: norm weight must hold {n} values")
     _check(library().lrs_gemm_mid_add_norm_begin(_dev(residual, "residual"), _dev(a, "a"), _dev(w, "w"), _dev(norm_weight, "norm_weight"),
                                                  dtype_code(norm_weight.dtype), _dev(next_x, "next_x"), _dev(next_sumsq, "next_sumsq"),
-                                                 m, n, k, _rows(a, "a"), _stream()))
+                                                 m, n, k, _rows(a, "a"), choice.word, _stream()))
 
 
-def gemm_mid_scaled(out: torch.Tensor, a: torch.Tensor, w: torch.Tensor, sumsq: torch.Tensor, eps: float, swiglu: bool = False) -> None:
+def gemm_mid_scaled(out: torch.Tensor, a: torch.Tensor, w: torch.Tensor, sumsq: torch.Tensor, eps: float, swiglu: bool = False,
+                    choice: KernelChoice = DEFAULT_CHOICE) -> None:
     """out = (the RMSNorm that `a` and `sumsq` stand for) @ w.T for 17..128 rows: a = bf16(h * norm weight) [M, K],
     sumsq [parts, M] partial sums of h^2; row r of the product is multiplied by rsqrt(sum_p sumsq[p, r] / K + eps).
     swiglu as in gemm()."""
     m, k = a.shape
     n = w.shape[0]
-    _need(gemm_mid_takes(w.dtype, m, n, k) and a.dtype == torch.bfloat16, "gemm_mid_scaled: takes bf16 products of 17..128 rows, K % 256 == 0, N % 16 == 0")
+    _need(gemm_mid_takes(w.dtype, m, n, k, 128, choice) and a.dtype == torch.bfloat16, "gemm_mid_scaled: takes bf16 products of 17..128 rows, K % 256 == 0, N % 16 == 0")
     _need(w.dim() == 2 and w.is_contiguous() and w.shape[1] == k, f"gemm_mid_scaled: weight must be contiguous [N, {k}]")
     _need(out.shape == (m, n // 2 if swiglu else n), f"gemm_mid_scaled: out must be [{m}, {n // 2 if swiglu else n}], got {tuple(out.shape)}")
     _need(out.dtype in (torch.bfloat16, torch.float32) and not (swiglu and out.dtype != torch.bfloat16), "gemm_mid_scaled: output must be bf16, or float32 without swiglu")
     _need(sumsq.dtype == torch.float32 and sumsq.dim() == 2 and sumsq.shape[1] == m and sumsq.is_contiguous() and eps > 0, f"gemm_mid_scaled: sumsq must be float32 [parts, {m}] and eps positive")
     mode = OUT_STORE if out.dtype == torch.bfloat16 else OUT_STORE_F32
     _check(library().lrs_gemm_mid_scaled(_dev(out, "out"), mode, _dev(a, "a"), _dev(w, "w"), m, n, k, _rows(a, "a"), _rows(out, "out"),
-                                         int(swiglu), _dev(sumsq, "sumsq"), sumsq.shape[0], eps, _stream()))
-
-
-def set_skinny_max_m(m: int) -> None:
-    """Move the row count from which products go to the vendor library (1..64)."""
-    _check(library().lrs_gemm_set_skinny_max_m(m))
+                                         int(swiglu), _dev(sumsq, "sumsq"), sumsq.shape[0], eps, choice.word, _stream()))
 
 
 def _int_vector(t: torch.Tensor, name: str, at_least: int) -> int:
@@ -457,9 +474,9 @@ def gather_rows(out: torch.Tensor, x: torch.Tensor, rows: torch.Tensor) -> None:
 
 
 # ------------------------------------------------------------------- gemm
-def gemm_fuses_norm(dtype: torch.dtype, m: int, k: int) -> bool:
+def gemm_fuses_norm(dtype: torch.dtype, m: int, k: int, choice: KernelChoice = DEFAULT_CHOICE) -> bool:
     """Whether gemm() can take the float32 residual stream and normalise it on the way in."""
-    return dtype == torch.bfloat16 and m <= library().lrs_gemm_skinny_max_m() and k % 8 == 0
+    return dtype == torch.bfloat16 and m <= choice.few_rows_max and k % 8 == 0
 
 
 def gemm_norm_fusion_pays(n: int) -> bool:
@@ -471,7 +488,7 @@ def gemm_norm_fusion_pays(n: int) -> bool:
 
 def gemm(out: torch.Tensor, a: torch.Tensor, w: torch.Tensor, bias: torch.Tensor | None = None, accumulate: bool = False,
          swiglu: bool = False, norm_weight: torch.Tensor | None = None, eps: float = 0.0, rows: torch.Tensor | None = None,
-         count: int | None = None) -> None:
+         count: int | None = None, choice: KernelChoice = DEFAULT_CHOICE) -> None:
     """out = a @ w.T (+ bias).  `accumulate` adds into a float32 `out` instead of storing.
 
     norm_weight: `a` is the float32 residual stream [*, K]; the product is taken of its RMSNorm
@@ -484,7 +501,7 @@ def gemm(out: torch.Tensor, a: torch.Tensor, w: torch.Tensor, bias: torch.Tensor
     normed = norm_weight is not None
     if normed:
         m = count if rows is not None else out.shape[0]
-        _need(a.dtype == torch.float32 and gemm_fuses_norm(w.dtype, m, k), f"gemm: the fused norm input needs a float32 input, bf16 weights and at most {library().lrs_gemm_skinny_max_m()} rows")
+        _need(a.dtype == torch.float32 and gemm_fuses_norm(w.dtype, m, k, choice), f"gemm: the fused norm input needs a float32 input, bf16 weights and at most {choice.few_rows_max} rows")
         _need(norm_weight.numel() == k and norm_weight.is_contiguous() and eps > 0, "gemm: norm weight must hold K values and eps be positive")
         if rows is None:
             _need(a.shape[0] >= m, "gemm: input has fewer rows than the output")
@@ -510,15 +527,27 @@ def gemm(out: torch.Tensor, a: torch.Tensor, w: torch.Tensor, bias: torch.Tensor
     _check(library().lrs_gemm(_dev(out, "out"), mode, _dev(a, "a"), _dev(w, "w"), None if bias is None else _dev(bias, "bias"),
                               dtype_code(w.dtype), m, n, k, lda, ldc, None if rows is None else _dev(rows, "rows"),
                               None if not normed else _dev(norm_weight, "norm_weight"), dtype_code(norm_weight.dtype) if normed else 0,
-                              eps, 1 if swiglu else 0, _stream()))
+                              eps, 1 if swiglu else 0, choice.word, _stream()))
+
+
+def library_gemm(out: torch.Tensor, a: torch.Tensor, w: torch.Tensor) -> None:
+    """out [M, N] = a [M, K] @ w[N, K].T by the vendor's matrix library (bfloat16 inputs, float32 sums; out bfloat16
+    or float32): for products of more rows than this package's own kernels are made for."""
+    m, k = a.shape
+    n = w.shape[0]
+    _need(a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and w.dim() == 2 and w.shape[1] == k and w.is_contiguous(),
+          f"library_gemm: a and w must be bfloat16, w contiguous [N, {k}]")
+    _need(out.shape == (m, n) and out.dtype in (torch.bfloat16, torch.float32), f"library_gemm: out must be bfloat16 or float32 [{m}, {n}]")
+    _check(library().lrs_library_gemm(_dev(out, "out"), 1 if out.dtype == torch.float32 else 0, _dev(a, "a"), _dev(w, "w"), m, n, k,
+                                      _rows(a, "a"), _rows(out, "out"), _stream()))
 
 
 NORM_CHAIN_MAX_ROWS = 16
 
 
-def gemm_chains_norm(dtype: torch.dtype, m: int, k: int) -> bool:
+def gemm_chains_norm(dtype: torch.dtype, m: int, k: int, choice: KernelChoice = DEFAULT_CHOICE) -> bool:
     """Whether gemm_norm_chain() takes a product of m rows over k with weights of `dtype`."""
-    return dtype == torch.bfloat16 and m <= min(NORM_CHAIN_MAX_ROWS, library().lrs_gemm_skinny_max_m()) and k % 8 == 0
+    return dtype == torch.bfloat16 and m <= min(NORM_CHAIN_MAX_ROWS, choice.few_rows_max) and k % 8 == 0
 
 
 def norm_chain_parts(n: int) -> int:
@@ -530,7 +559,7 @@ def gemm_norm_chain(out: torch.Tensor, a: torch.Tensor, w: torch.Tensor, bias: t
                     accumulate: bool = False, swiglu: bool = False,
                     in_sumsq: torch.Tensor | None = None, in_eps: float = 0.0,
                     next_x: torch.Tensor | None = None, next_sumsq: torch.Tensor | None = None,
-                    next_weight: torch.Tensor | None = None) -> None:
+                    next_weight: torch.Tensor | None = None, choice: KernelChoice = DEFAULT_CHOICE) -> None:
     """out = a @ w.T (+ bias) for at most 16 bf16 rows, with an RMSNorm taken apart around it.
 
     in_sumsq [parts, M] float32: `a` holds bf16(h * norm weight); row r of the product is multiplied
@@ -542,7 +571,7 @@ def gemm_norm_chain(out: torch.Tensor, a: torch.Tensor, w: torch.Tensor, bias: t
     m = a.shape[0]
     lda, ldc = _rows(a, "a"), _rows(out, "out")
     _need(w.dim() == 2 and w.is_contiguous() and a.shape[1] == k, f"gemm_norm_chain: weight must be contiguous [N, {a.shape[1]}], got {tuple(w.shape)}")
-    _need(a.dtype == torch.bfloat16 and gemm_chains_norm(w.dtype, m, k), "gemm_norm_chain: needs bf16 input and weights, at most 16 rows, K % 8 == 0")
+    _need(a.dtype == torch.bfloat16 and gemm_chains_norm(w.dtype, m, k, choice), "gemm_norm_chain: needs bf16 input and weights, at most 16 rows, K % 8 == 0")
     _need(out.shape == (m, n // 2 if swiglu else n), f"gemm_norm_chain: out must be [{m}, {n // 2 if swiglu else n}], got {tuple(out.shape)}")
     if accumulate:
         _need(out.dtype == torch.float32, "gemm_norm_chain: accumulation needs a float32 output")
@@ -571,7 +600,8 @@ def gemm_norm_chain(out: torch.Tensor, a: torch.Tensor, w: torch.Tensor, bias: t
         _dev(out, "out"), mode, _dev(a, "a"), _dev(w, "w"), None if bias is None else _dev(bias, "bias"), m, n, k, lda, ldc,
         1 if swiglu else 0, None if in_sumsq is None else _dev(in_sumsq, "in_sumsq"), parts, in_eps,
         None if next_x is None else _dev(next_x, "next_x"), None if next_x is None else _dev(next_sumsq, "next_sumsq"),
-        None if next_x is None else _dev(next_weight, "next_weight"), dtype_code(next_weight.dtype) if next_x is not None else 0, _stream()))
+        None if next_x is None else _dev(next_weight, "next_weight"), dtype_code(next_weight.dtype) if next_x is not None else 0,
+        choice.word, _stream()))
 
 
 def scale_rows(out: torch.Tensor, x: torch.Tensor, sumsq: torch.Tensor, eps: float) -> None:

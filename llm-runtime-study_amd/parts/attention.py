@@ -20,7 +20,7 @@ import torch
 
 from ..kernels import ops
 from .base import PagedKVNeed, Part, PartSpec, TensorSpec, create, length_class, register
-from .linear import ScaledRows, linear, materialize, rows_of
+from .linear import ScaledRows, kernels_of, linear, materialize, rows_of
 
 
 class GQAAttention(Part):
@@ -121,7 +121,8 @@ class GQAAttention(Part):
         # 17..128 rows of a decode step: the q/k/v product and the preparation of its heads as two kernels, the
         # second adding up the sums of the product's K splits (no kernel of its own for that)
         together = (ctx.all_decode and self.b_qkv is None and ctx.dtype == torch.bfloat16 and t > self.PREPARE_INSIDE_ROWS
-                    and ops.gemm_mid_qk_prep_takes(self.w_qkv.dtype, t, nq, nkv, d, self.w_qkv.shape[1], 0 if cos is None else cos.shape[1]))
+                    and ops.gemm_mid_qk_prep_takes(self.w_qkv.dtype, t, nq, nkv, d, self.w_qkv.shape[1], 0 if cos is None else cos.shape[1],
+                                                   kernels_of(ctx)))
         begun = plain = None
         if together:
             begun = x if isinstance(x, ScaledRows) else None          # a norm that the product before began
@@ -130,7 +131,7 @@ class GQAAttention(Part):
         if together:
             ops.gemm_mid_qk_prep(qkv, plain, self.w_qkv, None if begun is None else begun.sumsq, 0.0 if begun is None else begun.eps,
                                  nq, nkv, d, self.q_norm, self.k_norm, self.qk_norm_eps, cos, sin, cache.k_pages, cache.v_pages,
-                                 group.slots, group.page_size)
+                                 group.slots, group.page_size, choice=kernels_of(ctx))
         else:
             linear(ctx, qkv, x if plain is None or begun is not None else plain, self.w_qkv, self.b_qkv)
         out = ctx.scratch("attn_out", (t, nq * d), ctx.dtype)

@@ -8,8 +8,22 @@ never needs to know which happened.  Parts that want a plain tensor call `materi
 
 Between two layers the norm can also be started by the product before it: `linear(..., then_norm=
 norm)` on a product that adds into the residual stream returns ScaledRows when the kernel took it
-(bfloat16, at most 16 rows: decoding), which the next `linear()` completes in its epilogue.  That
+(bfloat16, at most 128 rows: decoding), which the next `linear()` completes in its epilogue.  That
 saves the norm kernel between every two products of a decode step.
+
+Which kernel serves a product is decided in one place, `plan()`, from the product's shape, the
+dtypes, the form its input arrives in and the step's KernelChoice (`ctx.kernels`); it returns the
+name of a route and `linear()` runs it.  The routes:
+
+  chain      at most 16 bfloat16 rows: the few-rows kernel finishing a norm begun before it and / or
+             beginning the one that follows (gemm_norm_chain)
+  mid_scaled 17..128 rows whose norm was begun before: the kernel for them finishes it (gemm_mid_scaled)
+  fused_norm few rows of the float32 residual stream, normalised on the way in (gemm with norm_weight)
+  mid_begin  17..128 rows adding into the residual stream and beginning the norm that follows
+  mid        17..128 rows, nothing folded in (gemm picks the kernel for them)
+  library    more rows than these kernels are made for, if the step may use the vendor library; the
+             residual add (with the norm that follows) or the gated activation take one more small kernel
+  own        everything else, and every float32 product (gemm picks the kernel by shape)
 """
 
 from __future__ import annotations
@@ -58,23 +72,63 @@ def rows_of(x) -> int:
     return x.count if isinstance(x, (LazyNorm, ScaledRows)) else x.shape[0]
 
 
-def _norm_ahead(ctx, then_norm, out, weight, m: int, accumulate: bool, swiglu: bool):
-    """Buffers for the norm that follows a product, if the kernel can begin it: the norm must be
-    an RMSNorm (it says so through `rms_parameters()`), the product must add into the residual."""
+def kernels_of(ctx) -> ops.KernelChoice:
+    return getattr(ctx, "kernels", None) or ops.DEFAULT_CHOICE
+
+
+ROUTES = ("chain", "mid_scaled", "fused_norm", "mid_begin", "mid", "library", "own")
+
+
+def plan(m: int, n: int, k: int, *, weight_dtype: torch.dtype, run_dtype: torch.dtype, out_dtype: torch.dtype, arrives: str,
+         accumulate: bool = False, swiglu: bool = False, bias: bool = False, norm_follows: int = 0,
+         contiguous: bool = True, out_contiguous: bool = True, choice: ops.KernelChoice = ops.DEFAULT_CHOICE) -> tuple[str, str]:
+    """(route, what to do with the input first) for out [m, n] = x [m, k] @ w[n, k].T.
+
+    arrives: "tensor" (activation dtype), "lazy" (LazyNorm) or "scaled" (ScaledRows); norm_follows: the size
+    of the RMSNorm the caller will apply to `out` next (0: none, or not an RMSNorm).  The second value says
+    whether the input has to be turned into a plain tensor before the route runs: "" or "materialize"."""
+    bf16 = weight_dtype == torch.bfloat16 and run_dtype == torch.bfloat16
+    stores = out_dtype in (torch.bfloat16, torch.float32) and not (swiglu and out_dtype != torch.bfloat16)
+    follows = bool(norm_follows) and norm_follows == n and accumulate and not swiglu and out_dtype == torch.float32
+    if arrives == "scaled":
+        if ops.gemm_chains_norm(weight_dtype, m, k, choice):
+            return "chain", ""
+        if ops.gemm_mid_takes(weight_dtype, m, n, k, ops.MID_ROWS_PREFERRED, choice) and not bias and not accumulate and stores:
+            return "mid_scaled", ""
+        arrives, first = "tensor", "materialize"
+    elif arrives == "lazy":
+        if ops.gemm_fuses_norm(weight_dtype, m, k, choice) and ops.gemm_norm_fusion_pays(n):
+            return "fused_norm", ""
+        arrives, first = "tensor", "materialize"
+    else:
+        first = ""
+    if bf16 and follows and ops.gemm_chains_norm(weight_dtype, m, k, choice):
+        return "chain", first
+    mid_most = ops.MID_ROWS_PREFERRED if choice.library else 128
+    if (bf16 and not bias and contiguous and (accumulate or stores)
+            and ops.gemm_mid_takes(weight_dtype, m, n, k, mid_most, choice)):
+        return ("mid_begin" if follows and out_contiguous else "mid"), first
+    if (choice.library and bf16 and m > choice.few_rows_max and not bias and contiguous
+            and (accumulate or (stores and out_contiguous))):
+        return "library", first
+    return "own", first
+
+
+def _next_norm(then_norm, n: int):
+    """(weight, eps) of the norm that follows if it is an RMSNorm over n columns (it says so through
+    `rms_parameters()`), else None."""
     parameters = getattr(then_norm, "rms_parameters", None)
-    if parameters is None or not accumulate or swiglu or ctx.dtype != torch.bfloat16 or out.dtype != torch.float32:
+    if parameters is None:
         return None
-    n, k = weight.shape
-    if not ops.gemm_chains_norm(weight.dtype, m, k) or out.shape != (m, n):
-        return None
-    norm_weight, eps = parameters()
-    if norm_weight.numel() != n:
-        return None
+    weight, eps = parameters()
+    return (weight, eps) if weight.numel() == n else None
+
+
+def _ahead_buffers(ctx, m: int, n: int, parts: int, eps: float, tag: str) -> ScaledRows:
     # two sets of buffers in turn: the one a product reads may not be the one it writes
     turn = ctx.memo["norm_ahead_turn"] = 1 - ctx.memo.get("norm_ahead_turn", 0)
-    x = ctx.scratch(f"norm_ahead_x{turn}", (m, n), torch.bfloat16)
-    sumsq = ctx.scratch(f"norm_ahead_sumsq{turn}", (ops.norm_chain_parts(n), m), torch.float32)
-    return ScaledRows(x, sumsq, eps, m), norm_weight
+    return ScaledRows(ctx.scratch(f"norm_ahead_x{turn}", (m, n), torch.bfloat16),
+                      ctx.scratch(f"{tag}{turn}", (parts, m), torch.float32), eps, m)
 
 
 def linear(ctx, out, x, weight, bias=None, accumulate: bool = False, swiglu: bool = False, then_norm=None):
@@ -82,78 +136,61 @@ def linear(ctx, out, x, weight, bias=None, accumulate: bool = False, swiglu: boo
 
     then_norm: the norm part that will be applied to `out` next (only meaningful with
     `accumulate`).  Returns that norm of the updated `out` if it was computed on the way, as
-    ScaledRows (begun by the few-rows kernel, finished by the next `linear()`) or as a plain
-    tensor (after a library product); else None: the caller then runs the norm as usual.
-
-    Products of more than 128 rows in bfloat16 go to the vendor's matrix library (as the reference's
-    nn.Linear does) when the step allows it (`ctx.library_gemm`); its result then reaches the
-    residual stream or the gated activation through one more small kernel.  Everything else,
-    and every float32 product, runs in this package's own kernels (17..128 rows: the kernel that
-    shares the activations through LDS, when the shape suits it: K a multiple of 256)."""
-    scaled = None
-    if isinstance(x, ScaledRows):
-        if ops.gemm_chains_norm(weight.dtype, x.count, weight.shape[1]):
-            scaled, x = x, x.x
-        elif (ops.gemm_mid_takes(weight.dtype, x.count, weight.shape[0], weight.shape[1], ops.MID_ROWS_PREFERRED) and bias is None
-              and not accumulate and out.dtype in (torch.bfloat16, torch.float32) and not (swiglu and out.dtype != torch.bfloat16)):
-            # 17..128 rows: the product finishes the norm that the product before it began
-            ops.gemm_mid_scaled(out, x.x, weight, x.sumsq, x.eps, swiglu)
-            return None
-        else:
-            x = x.materialize(ctx)
-    if not isinstance(x, LazyNorm) and x.dtype == torch.bfloat16:
-        ahead = _norm_ahead(ctx, then_norm, out, weight, x.shape[0], accumulate, swiglu) if then_norm is not None else None
-        if scaled is not None or ahead is not None:
-            following, norm_weight = ahead if ahead is not None else (None, None)
-            ops.gemm_norm_chain(out, x, weight, bias, accumulate, swiglu,
-                                in_sumsq=None if scaled is None else scaled.sumsq, in_eps=0.0 if scaled is None else scaled.eps,
-                                next_x=None if following is None else following.x,
-                                next_sumsq=None if following is None else following.sumsq, next_weight=norm_weight)
-            return following
-    if isinstance(x, LazyNorm):
-        if ops.gemm_fuses_norm(weight.dtype, x.count, weight.shape[1]) and ops.gemm_norm_fusion_pays(weight.shape[0]):
-            ops.gemm(out, x.h, weight, bias, accumulate, swiglu, norm_weight=x.weight, eps=x.eps, rows=x.rows, count=x.count)
-            return None
+    ScaledRows (begun by the product, finished by the next `linear()`) or as a plain tensor (after a
+    library product); else None: the caller then runs the norm as usual."""
+    choice = kernels_of(ctx)
+    n, k = weight.shape
+    m = rows_of(x)
+    following = _next_norm(then_norm, n) if then_norm is not None and accumulate else None
+    arrives = "scaled" if isinstance(x, ScaledRows) else "lazy" if isinstance(x, LazyNorm) else "tensor"
+    route, first = plan(m, n, k, weight_dtype=weight.dtype, run_dtype=ctx.dtype, out_dtype=out.dtype, arrives=arrives,
+                        accumulate=accumulate, swiglu=swiglu, bias=bias is not None, norm_follows=n if following else 0,
+                        contiguous=arrives != "tensor" or x.is_contiguous(), out_contiguous=out.is_contiguous(), choice=choice)
+    scaled = x if arrives == "scaled" and not first else None
+    if first:
         x = x.materialize(ctx)
-    m, n = x.shape[0], weight.shape[0]
-    library = getattr(ctx, "library_gemm", False)
-    # 17..128 rows: this package's kernel for them, whether or not the step may use the vendor library
-    if (x.dtype == torch.bfloat16 and bias is None and x.is_contiguous() and (accumulate or out.dtype in (torch.bfloat16, torch.float32))
-            and not (swiglu and out.dtype != torch.bfloat16)
-            and ops.gemm_mid_takes(weight.dtype, m, n, weight.shape[1], ops.MID_ROWS_PREFERRED if library else 128)):
-        parameters = getattr(then_norm, "rms_parameters", None) if accumulate else None
-        if parameters is not None and out.is_contiguous() and out.dtype == torch.float32 and parameters()[0].numel() == n:
-            # product, residual add and the first half of the norm that follows: the kernel that adds the K
-            # splits' sums leaves bf16(h * norm weight) and partial sums of squares, the next product finishes
-            norm_weight, eps = parameters()
-            turn = ctx.memo["norm_ahead_turn"] = 1 - ctx.memo.get("norm_ahead_turn", 0)
-            begun = ScaledRows(ctx.scratch(f"norm_ahead_x{turn}", (m, n), torch.bfloat16),
-                               ctx.scratch(f"norm_begin_sumsq{turn}", (ops.norm_begin_parts(n), m), torch.float32), eps, m)
-            ops.gemm_mid_add_norm_begin(out, x, weight, norm_weight, begun.x, begun.sumsq)
-            return begun
-        ops.gemm(out, x, weight, None, accumulate, swiglu)
+        # a plain tensor now: its dtype and layout may send it elsewhere than was planned for the norm's own form
+        if route in ("mid", "mid_begin", "library") and not (x.dtype == torch.bfloat16 and x.is_contiguous()):
+            route = "own"
+    elif arrives == "tensor" and route != "own" and x.dtype != torch.bfloat16:
+        route = "own"
+
+    if route == "chain":
+        begun = None
+        if following is not None and not swiglu and out.dtype == torch.float32 and out.shape == (m, n):
+            begun = _ahead_buffers(ctx, m, n, ops.norm_chain_parts(n), following[1], "norm_ahead_sumsq")
+        ops.gemm_norm_chain(out, x.x if scaled is not None else x, weight, bias, accumulate, swiglu,
+                            in_sumsq=None if scaled is None else scaled.sumsq, in_eps=0.0 if scaled is None else scaled.eps,
+                            next_x=None if begun is None else begun.x, next_sumsq=None if begun is None else begun.sumsq,
+                            next_weight=None if begun is None else following[0], choice=choice)
+        return begun
+    if route == "mid_scaled":
+        ops.gemm_mid_scaled(out, scaled.x, weight, scaled.sumsq, scaled.eps, swiglu, choice=choice)
         return None
-    if (library and weight.dtype == torch.bfloat16 and x.dtype == torch.bfloat16 and m > ops.skinny_max_m()
-            and bias is None and x.is_contiguous() and (accumulate or (out.dtype in (torch.bfloat16, torch.float32) and out.is_contiguous()))
-            and not (swiglu and out.dtype != torch.bfloat16)):
-        if accumulate or swiglu:
-            y = ctx.scratch("library_gemm_out", (m, n), torch.bfloat16)
-            torch.mm(x, weight.t(), out=y)
-            if accumulate:
-                parameters = getattr(then_norm, "rms_parameters", None)
-                if parameters is not None and out.is_contiguous() and parameters()[0].numel() == n:
-                    # the residual add and the norm that follows it in one pass over the rows
-                    norm_weight, eps = parameters()
-                    normed = ctx.scratch("norm_after_add", (m, n), ctx.dtype)
-                    ops.add_rmsnorm(normed, out, y, norm_weight, eps)
-                    return normed
-                ops.add_into(out, y)
-            else:
-                ops.silu_mul(out, y, interleaved=True)
-        elif out.dtype == torch.float32:
-            torch.mm(x, weight.t(), out_dtype=torch.float32, out=out)     # float32 logits of many rows
-        else:
-            torch.mm(x, weight.t(), out=out)
+    if route == "fused_norm":
+        ops.gemm(out, x.h, weight, bias, accumulate, swiglu, norm_weight=x.weight, eps=x.eps, rows=x.rows, count=x.count, choice=choice)
         return None
-    ops.gemm(out, x, weight, bias, accumulate, swiglu)
+    if route == "mid_begin":
+        # product, residual add and the first half of the norm that follows: the kernel that adds the K splits'
+        # sums leaves bf16(h * norm weight) and partial sums of squares, the next product finishes
+        begun = _ahead_buffers(ctx, m, n, ops.norm_begin_parts(n), following[1], "norm_begin_sumsq")
+        ops.gemm_mid_add_norm_begin(out, x, weight, following[0], begun.x, begun.sumsq, choice=choice)
+        return begun
+    if route == "library":
+        if not (accumulate or swiglu):
+            ops.library_gemm(out, x, weight)                      # bfloat16, or the float32 logits of many rows
+            return None
+        y = ctx.scratch("library_gemm_out", (m, n), torch.bfloat16)
+        ops.library_gemm(y, x, weight)
+        if swiglu:
+            ops.silu_mul(out, y, interleaved=True)
+            return None
+        if following is not None and out.is_contiguous():
+            # the residual add and the norm that follows it in one pass over the rows
+            normed = ctx.scratch("norm_after_add", (m, n), ctx.dtype)
+            ops.add_rmsnorm(normed, out, y, following[0], following[1])
+            return normed
+        ops.add_into(out, y)
+        return None
+    ops.gemm(out, x, weight, bias, accumulate, swiglu, choice=choice)     # "mid" and "own": gemm picks the kernel by shape
     return None

@@ -71,3 +71,67 @@ def test_shapes_of_the_kernel_for_17_to_64_rows():
     for n, k in ((64, 256), (208, 512), (5120, 5120), (5120, 17408), (7168, 5120), (51200, 5120), (1040, 3328)):
         waves, splits = ops.gemm_mid_shape(n, k)
         assert waves in (4, 6, 8) and 1 <= splits <= 8 and (splits == 1 or k // 256 // splits >= 2)
+
+
+def test_the_route_of_a_product_follows_rows_dtype_and_the_runners_choices():
+    """`plan()` of parts/linear.py: one decision per class of (rows, shape, dtype, form of the input), and the
+    choices a runner carries move it; nothing in the process does."""
+    import torch
+
+    from llm_runtime_study_amd.kernels.ops import KernelChoice
+    from llm_runtime_study_amd.parts.linear import ROUTES, plan
+
+    bf16, f32 = torch.bfloat16, torch.float32
+
+    def route(m, n, k, arrives="tensor", dtype=bf16, out=bf16, **more):
+        got = plan(m, n, k, weight_dtype=dtype, run_dtype=dtype, out_dtype=out, arrives=arrives, **more)
+        assert got[0] in ROUTES
+        return got
+
+    # decode, at most 16 rows: the norm arrives begun and the next one is begun (o_proj, down), or only finished (qkv, gate_up)
+    assert route(8, 4096, 4096, "scaled", out=f32, accumulate=True, norm_follows=4096) == ("chain", "")
+    assert route(8, 24576, 4096, "scaled", swiglu=True) == ("chain", "")
+    assert route(8, 4096, 4096, out=f32, accumulate=True, norm_follows=4096) == ("chain", "")     # a plain input, the next norm begun
+    assert route(8, 4096, 4096, out=f32, accumulate=True) == ("own", "")                          # nothing to fold in: the few-rows kernel by shape
+    # the first product of a step: the residual stream, normalised on the way in where that pays (narrow matrices)
+    assert route(8, 4096, 4096, "lazy") == ("fused_norm", "")
+    assert route(8, 24576, 4096, "lazy", swiglu=True) == ("own", "materialize")
+    assert route(1, 151936, 4096, "lazy", out=f32) == ("own", "materialize")
+    # 17..128 rows
+    assert route(64, 6144, 4096, "scaled") == ("mid_scaled", "")
+    assert route(64, 4096, 12288, out=f32, accumulate=True, norm_follows=4096) == ("mid_begin", "")
+    assert route(64, 4096, 12288, out=f32, accumulate=True, norm_follows=4096, out_contiguous=False) == ("mid", "")
+    assert route(128, 24576, 4096, swiglu=True) == ("mid", "")
+    assert route(64, 4096, 4000) == ("library", "")                                               # K no multiple of 256: not that kernel's
+    assert route(64, 4096, 4000, choice=KernelChoice(library=False)) == ("own", "")
+    assert route(64, 6144, 4096, "scaled", choice=KernelChoice(mid=False)) == ("library", "materialize")
+    assert route(64, 6144, 4096, "scaled", choice=KernelChoice(mid=False, library=False)) == ("own", "materialize")
+    assert route(64, 6144, 4096, "lazy", choice=KernelChoice(few_rows_max=64)) == ("mid", "materialize")   # 6,144 rows: folding the norm in does not pay
+    assert route(64, 4096, 4096, "lazy", choice=KernelChoice(few_rows_max=64)) == ("fused_norm", "")
+    # many rows
+    assert route(2048, 24576, 4096, swiglu=True) == ("library", "")
+    assert route(2048, 4096, 4096, out=f32, accumulate=True, norm_follows=4096) == ("library", "")
+    assert route(2048, 4096, 4096, bias=True) == ("own", "")
+    assert route(2048, 4096, 4096, contiguous=False) == ("own", "")
+    assert route(2048, 24576, 4096, swiglu=True, choice=KernelChoice(library=False)) == ("own", "")
+    assert route(129, 4096, 4096) == ("library", "") and route(128, 4096, 4096) == ("mid", "")
+    # float32 runs: this package's own kernels whatever the rows
+    for m in (1, 8, 64, 2048):
+        assert route(m, 4096, 4096, dtype=f32, out=f32) == ("own", "")
+        assert route(m, 4096, 4096, "lazy", dtype=f32, out=f32) == ("own", "materialize")
+
+
+def test_kernel_choices_travel_with_the_call():
+    from llm_runtime_study_amd.errors import KernelError
+    from llm_runtime_study_amd.kernels import ops
+    import pytest
+
+    assert ops.DEFAULT_CHOICE.word == 3 and ops.KernelChoice(mid=False, whole_lines=False).word == 0
+    assert ops.KernelChoice(mid_waves=6, mid_splits=4).word == 3 | 6 << 4 | 4 << 8
+    for bad in (dict(few_rows_max=0), dict(few_rows_max=65), dict(mid_waves=5), dict(mid_splits=17)):
+        with pytest.raises(KernelError):
+            ops.KernelChoice(**bad)
+    assert not hasattr(ops, "gemm_mid_tune") and not hasattr(ops, "set_skinny_max_m") and not hasattr(ops, "gemm_skinny_lines")
+    if ops.compute_units() in (0, 256):
+        assert ops.gemm_mid_shape(4096, 4096, ops.KernelChoice(mid_waves=8, mid_splits=2)) == (8, 2)
+        assert ops.gemm_mid_shape(4096, 4096) == (4, 4)

@@ -26,12 +26,10 @@ def ops():
 
 @pytest.fixture
 def all_rows_in_own_kernel(ops):
-    """The few-rows kernel takes up to 64 rows; by default callers hand over to the vendor library
-    from 17 rows on.  Lift that for tests of the kernel itself."""
-    before = ops.skinny_max_m()
-    ops.set_skinny_max_m(64)
-    yield
-    ops.set_skinny_max_m(before)
+    """The few-rows kernel takes up to 64 rows; in steps callers hand over to other kernels from 17 rows
+    on.  The choice that lifts that, for tests of the kernel itself (passed with the call: nothing is set
+    in the library)."""
+    return ops.KernelChoice(few_rows_max=ops.few_rows_capacity())
 
 
 def dev(t):
@@ -295,21 +293,18 @@ def test_gemm_of_17_to_64_rows(ops, m, n, k, waves, splits):
     a = torch.randn(m, k, generator=g).bfloat16()
     w = (torch.randn(n, k, generator=g) / math.sqrt(k)).bfloat16()
     want = a.double() @ w.double().T
-    ops.gemm_mid_tune(True, waves, splits)
-    try:
-        stored = torch.empty(m, n, device="cuda", dtype=torch.bfloat16)
-        ops.gemm(stored, dev(a), dev(w))
-        wide = torch.full((m, n), 0.5, device="cuda")
-        ops.gemm(wide, dev(a), dev(w), accumulate=True)
-        plain = torch.empty(m, n, device="cuda")
-        ops.gemm(plain, dev(a), dev(w))
-        inter = n // 2
-        gate, up = w[:inter], w[inter:]
-        mixed = torch.stack((gate.view(inter // 8, 8, k), up.view(inter // 8, 8, k)), 1).reshape(n, k).contiguous()
-        gated = torch.empty(m, inter, device="cuda", dtype=torch.bfloat16)
-        ops.gemm(gated, dev(a), dev(mixed), swiglu=True)
-    finally:
-        ops.gemm_mid_tune(True, 0, 0)
+    choice = ops.KernelChoice(mid_waves=waves, mid_splits=splits)
+    stored = torch.empty(m, n, device="cuda", dtype=torch.bfloat16)
+    ops.gemm(stored, dev(a), dev(w), choice=choice)
+    wide = torch.full((m, n), 0.5, device="cuda")
+    ops.gemm(wide, dev(a), dev(w), accumulate=True, choice=choice)
+    plain = torch.empty(m, n, device="cuda")
+    ops.gemm(plain, dev(a), dev(w), choice=choice)
+    inter = n // 2
+    gate, up = w[:inter], w[inter:]
+    mixed = torch.stack((gate.view(inter // 8, 8, k), up.view(inter // 8, 8, k)), 1).reshape(n, k).contiguous()
+    gated = torch.empty(m, inter, device="cuda", dtype=torch.bfloat16)
+    ops.gemm(gated, dev(a), dev(mixed), swiglu=True, choice=choice)
     torch.testing.assert_close(stored.cpu().double(), want, rtol=1e-2, atol=1e-2)
     torch.testing.assert_close(plain.cpu().double(), want, rtol=1e-4, atol=1e-4)
     torch.testing.assert_close(wide.cpu().double(), want + 0.5, rtol=1e-4, atol=1e-4)
@@ -334,27 +329,24 @@ def test_gemm_of_17_to_128_rows_with_norm_taken_apart(ops, w_dtype, m, h, n2, k,
     out = dev(residual.clone())
     next_x = torch.empty(m, h, device="cuda", dtype=torch.bfloat16)
     sumsq = torch.empty(ops.norm_begin_parts(h), m, device="cuda")
-    ops.gemm_mid_tune(True, 0, splits)
-    try:
-        ops.gemm_mid_add_norm_begin(out, dev(a), dev(w1), dev(gamma), next_x, sumsq)
-        torch.testing.assert_close(out.cpu().double(), updated, rtol=1e-4, atol=1e-4)
-        torch.testing.assert_close(sumsq.sum(0).cpu().double(), updated.square().sum(-1), rtol=1e-4, atol=1e-4)
-        finished = torch.empty(m, h, device="cuda", dtype=torch.bfloat16)
-        ops.scale_rows(finished, next_x, sumsq, eps)
-        close_in_norm(finished, normed, 5e-3)
-        if swiglu:
-            inter = n2 // 2
-            mixed = torch.stack((w2[:inter].view(inter // 8, 8, h), w2[inter:].view(inter // 8, 8, h)), 1).reshape(n2, h).contiguous()
-            got = torch.empty(m, inter, device="cuda", dtype=torch.bfloat16)
-            ops.gemm_mid_scaled(got, next_x, dev(mixed), sumsq, eps, swiglu=True)
-            y = normed @ w2.double().T
-            close_in_norm(got, torch.nn.functional.silu(y[:, :inter]) * y[:, inter:], 1e-2)
-        else:
-            got = torch.empty(m, n2, device="cuda")
-            ops.gemm_mid_scaled(got, next_x, dev(w2), sumsq, eps)
-            close_in_norm(got, normed @ w2.double().T, 5e-3)
-    finally:
-        ops.gemm_mid_tune(True, 0, 0)
+    choice = ops.KernelChoice(mid_splits=splits)
+    ops.gemm_mid_add_norm_begin(out, dev(a), dev(w1), dev(gamma), next_x, sumsq, choice=choice)
+    torch.testing.assert_close(out.cpu().double(), updated, rtol=1e-4, atol=1e-4)
+    torch.testing.assert_close(sumsq.sum(0).cpu().double(), updated.square().sum(-1), rtol=1e-4, atol=1e-4)
+    finished = torch.empty(m, h, device="cuda", dtype=torch.bfloat16)
+    ops.scale_rows(finished, next_x, sumsq, eps)
+    close_in_norm(finished, normed, 5e-3)
+    if swiglu:
+        inter = n2 // 2
+        mixed = torch.stack((w2[:inter].view(inter // 8, 8, h), w2[inter:].view(inter // 8, 8, h)), 1).reshape(n2, h).contiguous()
+        got = torch.empty(m, inter, device="cuda", dtype=torch.bfloat16)
+        ops.gemm_mid_scaled(got, next_x, dev(mixed), sumsq, eps, swiglu=True, choice=choice)
+        y = normed @ w2.double().T
+        close_in_norm(got, torch.nn.functional.silu(y[:, :inter]) * y[:, inter:], 1e-2)
+    else:
+        got = torch.empty(m, n2, device="cuda")
+        ops.gemm_mid_scaled(got, next_x, dev(w2), sumsq, eps, choice=choice)
+        close_in_norm(got, normed @ w2.double().T, 5e-3)
 
 
 @pytest.mark.parametrize("m,nq,nkv,d,k,splits,begun", [(17, 4, 2, 64, 256, 0, False), (64, 32, 8, 128, 4096, 0, True), (100, 6, 2, 32, 1024, 2, True),
@@ -398,12 +390,8 @@ def test_qkv_product_of_17_to_128_rows_with_head_preparation(ops, m, nq, nkv, d,
     qkv = torch.zeros(m, n, device="cuda", dtype=torch.bfloat16)
     k_pages = torch.zeros(pages, nkv, page, d, device="cuda", dtype=torch.bfloat16)
     v_pages = torch.zeros(pages, nkv, d, page, device="cuda", dtype=torch.bfloat16)
-    ops.gemm_mid_tune(True, 0, splits)
-    try:
-        ops.gemm_mid_qk_prep(qkv, dev(x), dev(w), None if sumsq is None else dev(sumsq), norm_eps, nq, nkv, d, dev(qw), dev(kw), eps,
-                             cos, sin, k_pages, v_pages, dev(slots), page)
-    finally:
-        ops.gemm_mid_tune(True, 0, 0)
+    ops.gemm_mid_qk_prep(qkv, dev(x), dev(w), None if sumsq is None else dev(sumsq), norm_eps, nq, nkv, d, dev(qw), dev(kw), eps,
+                         cos, sin, k_pages, v_pages, dev(slots), page, choice=ops.KernelChoice(mid_splits=splits))
     close_in_norm(qkv[:, : nq * d], q_want.reshape(m, nq * d), 1e-2)
     pg, off = (slots // page).long(), (slots % page).long()
     close_in_norm(k_pages.cpu()[pg, :, off, :], k_want, 1e-2)
@@ -420,11 +408,11 @@ def test_gemm_with_fused_rmsnorm_input(ops, w_dtype, m, n, k, all_rows_in_own_ke
     w = (torch.randn(n, k, generator=g) / math.sqrt(k)).bfloat16()
     rows = torch.randperm(m + 3, generator=g)[:m].to(torch.int32)
     eps = 1e-5
-    assert ops.gemm_fuses_norm(torch.bfloat16, m, k)
+    assert ops.gemm_fuses_norm(torch.bfloat16, m, k, all_rows_in_own_kernel) and ops.gemm_fuses_norm(torch.bfloat16, m, k) == (m <= 16)
     normed = gamma.double() * (h.double() * torch.rsqrt(h.double().square().mean(-1, keepdim=True) + eps))
     want = normed[rows.long()] @ w.double().T
     out = torch.empty(m, n, device="cuda")
-    ops.gemm(out, dev(h), dev(w), norm_weight=dev(gamma), eps=eps, rows=dev(rows), count=m)
+    ops.gemm(out, dev(h), dev(w), norm_weight=dev(gamma), eps=eps, rows=dev(rows), count=m, choice=all_rows_in_own_kernel)
     close_in_norm(out, want, 5e-3)
     # without a row list the first m rows are taken; against the two-kernel path the only
     # difference is where the input is rounded to bfloat16
@@ -432,7 +420,7 @@ def test_gemm_with_fused_rmsnorm_input(ops, w_dtype, m, n, k, all_rows_in_own_ke
     ops.rmsnorm(x, dev(h), dev(gamma), eps)
     two = torch.empty(m, n, device="cuda")
     ops.gemm(two, x, dev(w))
-    ops.gemm(out, dev(h), dev(w), norm_weight=dev(gamma), eps=eps)
+    ops.gemm(out, dev(h), dev(w), norm_weight=dev(gamma), eps=eps, choice=all_rows_in_own_kernel)
     close_in_norm(out, two.cpu(), 5e-3)
 
 
@@ -454,7 +442,7 @@ def test_gemm_with_swiglu_epilogue(ops, m, inter, k, all_rows_in_own_kernel):
         gamma = (1 + 0.1 * torch.randn(k, generator=g)).bfloat16()
         xn = gamma.double() * (h.double() * torch.rsqrt(h.double().square().mean(-1, keepdim=True) + 1e-6))
         want = torch.nn.functional.silu(xn @ gate.double().T) * (xn @ up.double().T)
-        ops.gemm(out, dev(h), dev(mixed), swiglu=True, norm_weight=dev(gamma), eps=1e-6)
+        ops.gemm(out, dev(h), dev(mixed), swiglu=True, norm_weight=dev(gamma), eps=1e-6, choice=all_rows_in_own_kernel)
         close_in_norm(out, want)
 
 
