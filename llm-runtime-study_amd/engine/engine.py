@@ -32,7 +32,8 @@ class Engine:
     def __init__(self, config, model, *, device, dtype, max_seq_len: int = 4096, max_batch_size: int = 1,
                  cache_backend: str = "paged", use_cuda_graph: bool = True, page_size: int = DEFAULT_PAGE_SIZE,
                  max_num_batched_tokens: int | None = None, num_pages: int | None = None, tokenizer=None,
-                 load_seconds: float = 0.0, library_gemm: bool = True, decode_steps_per_launch: int = 4, kernels=None):
+                 load_seconds: float = 0.0, library_gemm: bool = True, decode_steps_per_launch: int = 4, kernels=None,
+                 use_launch_plans: bool = True):
         if max_batch_size <= 0:
             raise EngineError("max_batch_size must be positive")
         if cache_backend != "paged":
@@ -50,6 +51,8 @@ class Engine:
         # for bfloat16 products of many rows if `library_gemm`, this package's own kernels for everything else
         self.kernels = kernels
         self.library_gemm = library_gemm if kernels is None else kernels.library
+        # steps outside graphs are recorded once per shape and made again from the record (see engine/step.py)
+        self.use_launch_plans = use_launch_plans
         self.tokenizer = tokenizer
         self.load_seconds = load_seconds
         self.quantization = "dense"
@@ -103,7 +106,7 @@ class Engine:
                                  dtype=self.dtype, device=self.device)
             self._runner = ModelRunner(self.model, cache, max_step_tokens=self.max_num_batched_tokens,
                                        dtype=self.dtype, device=self.device, use_graph=self.use_cuda_graph,
-                                       library_gemm=self.library_gemm, kernels=self.kernels)
+                                       library_gemm=self.library_gemm, kernels=self.kernels, use_plans=self.use_launch_plans)
         return self._runner
 
     @property

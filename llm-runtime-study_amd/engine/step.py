@@ -56,17 +56,23 @@ class ScratchArena:
     def __init__(self, device):
         self.device = device
         self._buffers: dict = {}
-        self.generation = 0   # bumped whenever a buffer is (re)allocated: captured graphs then hold stale addresses
+        # bumped whenever a buffer that was handed out before is replaced by a larger one: whoever wrote its
+        # address down (a captured graph, a recorded plan) then holds a stale address.  A buffer made for
+        # the first time moves nothing.
+        self.generation = 0
 
-    def get(self, name: str, shape: tuple, dtype: torch.dtype) -> torch.Tensor:
+    def get(self, name: str, shape: tuple, dtype: torch.dtype, zeroed: bool = False) -> torch.Tensor:
+        """The buffer `name` with at least shape[0] rows.  zeroed: all zero when it is made (for buffers whose
+        users leave them as they found them, such as arrival counters); never cleared again."""
         rows, rest = shape[0], tuple(shape[1:])
         key = (name, rest, dtype)
         buf = self._buffers.get(key)
         if buf is None or buf.shape[0] < rows:
             capacity = max(rows, 1 if buf is None else buf.shape[0] * 2)
-            buf = torch.empty((capacity, *rest), dtype=dtype, device=self.device)
+            if buf is not None:
+                self.generation += 1
+            buf = (torch.zeros if zeroed else torch.empty)((capacity, *rest), dtype=dtype, device=self.device)
             self._buffers[key] = buf
-            self.generation += 1
         return buf[:rows]
 
     def reserve(self, name: str, shape: tuple, dtype: torch.dtype) -> None:
@@ -108,7 +114,8 @@ class StepContext:
 
 class ModelRunner:
     def __init__(self, model: DecoderModel, cache: CacheManager, *, max_step_tokens: int, dtype: torch.dtype, device,
-                 use_graph: bool = False, library_gemm: bool = True, kernels: "ops.KernelChoice | None" = None):
+                 use_graph: bool = False, library_gemm: bool = True, kernels: "ops.KernelChoice | None" = None,
+                 use_plans: bool = True):
         if max_step_tokens <= 0:
             raise GenerationError(f"max_step_tokens must be positive, got {max_step_tokens}")
         self.model, self.cache, self.dtype, self.device = model, cache, dtype, torch.device(device)
@@ -123,6 +130,16 @@ class ModelRunner:
         # decode-only steps are captured in a HIP graph per padded batch size and replayed
         self.use_graph = use_graph and model.graph_safe()
         self._graphs: dict[tuple, tuple] = {}   # (bucket, length class) -> (handle, arena generation, logits tensor)
+        # Steps that are not replayed from a graph (prompt portions, mixed steps) are recorded as launch plans:
+        # the first step of a shape runs through the parts as usual while every launch is written down; later
+        # steps of that shape fill in the metadata and make the same launches from one call into the library.
+        # A shape is what the launches' arguments depend on (see _plan_key); a plan also names addresses, so it
+        # is good only while the scratch buffers stay where they are (the arena's generation).  Only models
+        # whose every part launches through this package's kernels alone (`plan_safe`) are recorded.
+        self.use_plans = use_plans and getattr(model, "plan_safe", lambda: False)()
+        self._plans: dict[tuple, tuple] = {}    # key -> (ops.Plan, arena generation, logits tensor or None)
+        self.plan_replays = 0
+        self.plan_recordings = 0
         self.graph_replays = 0     # steps (or launches of several steps) served by replaying a graph
         self.graph_captures = 0    # ... and those that ran eagerly and were captured on the way
         # query groups for the ragged attention kernel: at most `query_group` consecutive tokens of one request
@@ -292,7 +309,10 @@ class ModelRunner:
                 cursor += n
         real = len(entries)
         ctx.max_q = max(ctx.host_q_lens)
-        ctx.max_k = ctx.max_k_bound = int(lens[:real].max())
+        ctx.max_k = int(lens[:real].max())
+        # what kernels size their tables and choose their key splits by: an upper bound of the longest context that is
+        # the same for every step of one shape (a recorded plan holds it), the next multiple of 256
+        ctx.max_k_bound = min(-(-ctx.max_k // 256) * 256, max(self.cache.max_seq_len, ctx.max_k))
         if pad_to:
             # a graph outlives the step it is captured in: sizes that must hold for every replay are
             # made for the longest context the cache can hold
@@ -376,16 +396,52 @@ class ModelRunner:
             if bucket:
                 logits = self._step_graph(entries, bucket)
             else:
-                ctx = self.prepare(entries)
-                h = self.model.forward_hidden(ctx)
-                logits = self.model.logits(ctx, h) if ctx.num_logit_rows else None
+                logits = self._step_eager(self.prepare(entries))
         except Exception:
+            ops.record_drop()
             self._undo(extended, before, states)
             raise
         for entry in entries:
             self.cache.trim(entry.cache)
         self.steps_run += 1
         return logits
+
+    def _plan_key(self, ctx: StepContext) -> tuple:
+        """Everything the launches of a step depend on besides the contents of the metadata buffer: the numbers
+        of tokens, requests, wanted rows and query groups (sizes and grids, and where the metadata arrays lie),
+        the largest query group, whether every request brings one token, and the two coarse measures of the
+        longest context that kernels size tables and choose key splits by."""
+        return (ctx.T, ctx.R, ctx.num_logit_rows, ctx.num_qblocks, ctx.max_qblock, ctx.all_decode, ctx.max_k_bound, length_class(ctx.max_k))
+
+    def _step_eager(self, ctx: StepContext) -> torch.Tensor | None:
+        """The model on a prepared step, outside any graph: from a recorded plan if one fits, else through
+        the parts (recording a plan on the way, if plans are in use)."""
+        if not self.use_plans:
+            h = self.model.forward_hidden(ctx)
+            return self.model.logits(ctx, h) if ctx.num_logit_rows else None
+        key = self._plan_key(ctx)
+        known = self._plans.get(key)
+        if known is not None and known[1] == self.arena.generation:
+            ops.plan_run(known[0])
+            self.plan_replays += 1
+            return known[2]
+        generation = self.arena.generation
+        ops.record_begin()
+        try:
+            h = self.model.forward_hidden(ctx)
+            logits = self.model.logits(ctx, h) if ctx.num_logit_rows else None
+        except Exception:
+            ops.record_drop()
+            raise
+        plan = ops.record_end()
+        if self.arena.generation == generation:          # else a buffer moved on the way: addresses written down before are stale
+            if len(self._plans) >= self.MAX_PLANS:
+                self._plans.pop(next(iter(self._plans)))
+            self._plans[key] = (plan, generation, logits)
+            self.plan_recordings += 1
+        return logits
+
+    MAX_PLANS = 512      # plans kept (each a few hundred launches of a few dozen words); the oldest goes first
 
     def _undo(self, extended: Sequence[StepEntry], before: Sequence[int], states: list) -> None:
         """After a failed step: every cache that was extended back to its length before the step (pages

@@ -43,7 +43,7 @@ def sources() -> list[Path]:
 
 def source_hash() -> str:
     digest = hashlib.sha256()
-    for path in sorted(SOURCE_DIR.glob("*.hip")) + sorted(SOURCE_DIR.glob("*.h")):
+    for path in sorted(SOURCE_DIR.glob("*.hip")) + sorted(SOURCE_DIR.glob("*.h")) + sorted(SOURCE_DIR.glob("*.inc")):
         digest.update(path.name.encode())
         digest.update(path.read_bytes())
     digest.update(" ".join(FLAGS + LINK_FLAGS).encode())

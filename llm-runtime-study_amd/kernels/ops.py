@@ -10,6 +10,7 @@ from __future__ import annotations
 
 from dataclasses import dataclass
 import ctypes
+import struct
 from ctypes import c_char_p, c_float, c_int, c_int64, c_void_p, POINTER, byref
 
 import torch
@@ -61,6 +62,7 @@ DEFAULT_CHOICE = KernelChoice()
 
 _SIGNATURES = {
     "lrs_last_error": (c_char_p, []),
+    "lrs_plan_run": (c_int, [c_void_p, c_int64, c_int, c_void_p]),
     "lrs_device_arch": (c_int, [c_int, c_char_p, c_int, POINTER(c_int)]),
     "lrs_graph_begin": (c_int, [c_void_p]),
     "lrs_graph_end": (c_int, [c_void_p, POINTER(c_void_p)]),
@@ -138,6 +140,83 @@ def library():
             _check(lib.lrs_choose_tokens_static_init())
             _check(lib.lrs_library_gemm_prepare())
     return _lib
+
+
+# ------------------------------------------------------------ launch plans
+# Every kernel launch goes through _launch().  While a recording is open, the launch (entry point and
+# arguments, without the stream) is also written down; the recording becomes a Plan, an array of 64-bit words
+# that lrs_plan_run() walks in one call, making the same launches with the same arguments on the stream it
+# is given.  A step whose shape has been seen before is then one call into the library instead of some
+# hundreds of Python calls.  What is written down are addresses and sizes: a plan is good for as long as
+# every buffer it names lives where it lived (the caller's business: see engine/step.py).
+#
+# PLAN_OPS fixes the number of each entry point inside a plan; csrc/plan_dispatch.inc, made from this list
+# and _SIGNATURES by kernels/plan_codegen.py, is the other side (a test keeps the two in step).
+PLAN_OPS = ("lrs_add_into", "lrs_add_rmsnorm", "lrs_advance_decode", "lrs_advance_slots", "lrs_attention", "lrs_attention_decode",
+            "lrs_attention_prefill", "lrs_choose_tokens", "lrs_choose_tokens_split", "lrs_copy_to_pinned", "lrs_embed", "lrs_fill_i32",
+            "lrs_filter_logits", "lrs_gather_rows", "lrs_gemm", "lrs_gemm_mid_add_norm_begin", "lrs_gemm_mid_qk_prep", "lrs_gemm_mid_scaled",
+            "lrs_gemm_norm_chain", "lrs_library_gemm", "lrs_qk_prep", "lrs_rmsnorm", "lrs_rope_table", "lrs_scale_rows", "lrs_silu_mul")
+_PLAN_INDEX = {name: index for index, name in enumerate(PLAN_OPS)}
+_recording: list | None = None
+
+
+class Plan:
+    """A recorded sequence of launches, ready for plan_run()."""
+
+    def __init__(self, calls: list):
+        words: list[int] = []
+        for name, args in calls:
+            argtypes = _SIGNATURES[name][1][:-1]
+            words.append(_PLAN_INDEX[name])
+            for kind, value in zip(argtypes, args):
+                if kind is c_float:
+                    words.append(int.from_bytes(struct.pack("<f", value), "little"))
+                elif value is None:
+                    words.append(0)
+                else:
+                    words.append(int(value) & 0xFFFFFFFFFFFFFFFF)
+        self.launches = len(calls)
+        self.words = (ctypes.c_uint64 * max(len(words), 1))(*words)
+        self.length = len(words)
+
+
+def record_begin() -> None:
+    """Start writing launches down (they still run as they are made)."""
+    global _recording
+    if _recording is not None:
+        raise KernelError("a recording of launches is already open")
+    _recording = []
+
+
+def record_end() -> Plan:
+    """Stop writing launches down; returns the plan of those made since record_begin()."""
+    global _recording
+    if _recording is None:
+        raise KernelError("no recording of launches is open")
+    calls, _recording = _recording, None
+    return Plan(calls)
+
+
+def record_drop() -> None:
+    """Stop writing launches down and forget them (after a failure)."""
+    global _recording
+    _recording = None
+
+
+def plan_run(plan: Plan) -> None:
+    """Make the plan's launches, in order, on the current stream."""
+    if plan.launches:
+        _check(library().lrs_plan_run(plan.words, plan.length, plan.launches, _stream()))
+
+
+def _launch(name: str, *args) -> None:
+    code = getattr(_lib or library(), name)(*args)
+    if code != 0:
+        raise KernelError(library().lrs_last_error().decode())
+    if _recording is not None:
+        if name not in _PLAN_INDEX:
+            raise KernelError(f"{name} cannot be part of a recorded plan")
+        _recording.append((name, args[:-1]))
 
 
 def loaded_library_path() -> str:
@@ -227,13 +306,13 @@ def copy_h2d(dst: torch.Tensor, src: torch.Tensor, count: int) -> None:
     pinned host memory (the caller checks that once, when it allocates it: asking is slow)."""
     _need(src.device.type == "cpu" and src.is_contiguous() and dst.is_contiguous(), "copy_h2d needs a contiguous host source and a contiguous destination")
     _need(src.dtype == dst.dtype and 0 < count <= src.numel() and count <= dst.numel(), "copy_h2d: size or dtype mismatch")
-    _check(library().lrs_copy_h2d(_dev(dst, "dst"), src.data_ptr(), count * src.element_size(), _stream()))
+    _launch("lrs_copy_h2d", _dev(dst, "dst"), src.data_ptr(), count * src.element_size(), _stream())
 
 
 def stream_read(src: torch.Tensor, sink: torch.Tensor, blocks: int) -> None:
     """Reads all of `src` once with `blocks` workgroups (a probe of the memory rate a kernel can reach)."""
     _need(src.is_contiguous() and sink.dtype == torch.int32 and sink.numel() >= blocks, "stream_read: contiguous source and an int32 sink of `blocks` elements")
-    _check(library().lrs_stream_read(_dev(src, "src"), src.numel() * src.element_size(), _dev(sink, "sink"), blocks, _stream()))
+    _launch("lrs_stream_read", _dev(src, "src"), src.numel() * src.element_size(), _dev(sink, "sink"), blocks, _stream())
 
 
 def copy_to_pinned(dst: torch.Tensor, src: torch.Tensor, count: int) -> None:
@@ -241,7 +320,7 @@ def copy_to_pinned(dst: torch.Tensor, src: torch.Tensor, count: int) -> None:
     them after synchronising the stream).  count * element size must be a multiple of 16."""
     _need(dst.device.type == "cpu" and dst.is_contiguous() and src.is_contiguous(), "copy_to_pinned needs a contiguous pinned host destination and a contiguous source")
     _need(src.dtype == dst.dtype and 0 < count <= src.numel() and count <= dst.numel(), "copy_to_pinned: size or dtype mismatch")
-    _check(library().lrs_copy_to_pinned(dst.data_ptr(), _dev(src, "src"), count * src.element_size(), _stream()))
+    _launch("lrs_copy_to_pinned", dst.data_ptr(), _dev(src, "src"), count * src.element_size(), _stream())
 
 
 # ------------------------------------------------------------ elementwise
@@ -249,8 +328,8 @@ def embed(out: torch.Tensor, table: torch.Tensor, ids: torch.Tensor, multiplier:
     tokens, hidden = out.shape
     _need(out.is_contiguous() and table.is_contiguous() and table.dim() == 2 and table.shape[1] == hidden, "embed: out [T,H] and table [V,H] must agree")
     _need(ids.dtype == torch.int32 and ids.numel() >= tokens and ids.is_contiguous(), "embed: ids must be int32 [T]")
-    _check(library().lrs_embed(_dev(out, "out", torch.float32), _dev(table, "table"), dtype_code(table.dtype),
-                               _dev(ids, "ids"), tokens, hidden, multiplier, _stream()))
+    _launch("lrs_embed", _dev(out, "out", torch.float32), _dev(table, "table"), dtype_code(table.dtype),
+                               _dev(ids, "ids"), tokens, hidden, multiplier, _stream())
 
 
 def rmsnorm(out: torch.Tensor, x: torch.Tensor, weight: torch.Tensor, eps: float, rows: torch.Tensor | None = None) -> None:
@@ -261,8 +340,8 @@ def rmsnorm(out: torch.Tensor, x: torch.Tensor, weight: torch.Tensor, eps: float
         _need(x.shape[0] >= n_rows, "rmsnorm: x has fewer rows than out")
     else:
         _need(rows.dtype == torch.int32 and rows.numel() >= n_rows and rows.is_contiguous(), "rmsnorm: rows must be int32")
-    _check(library().lrs_rmsnorm(_dev(out, "out"), dtype_code(out.dtype), _dev(x, "x", torch.float32), _dev(weight, "weight"),
-                                 dtype_code(weight.dtype), None if rows is None else _dev(rows, "rows"), n_rows, hidden, eps, _stream()))
+    _launch("lrs_rmsnorm", _dev(out, "out"), dtype_code(out.dtype), _dev(x, "x", torch.float32), _dev(weight, "weight"),
+                                 dtype_code(weight.dtype), None if rows is None else _dev(rows, "rows"), n_rows, hidden, eps, _stream())
 
 
 def add_rmsnorm(out: torch.Tensor, x: torch.Tensor, y: torch.Tensor, weight: torch.Tensor, eps: float) -> None:
@@ -272,8 +351,8 @@ def add_rmsnorm(out: torch.Tensor, x: torch.Tensor, y: torch.Tensor, weight: tor
           "add_rmsnorm: x must be contiguous float32 [T, H] and y bf16 of the same shape")
     _need(out.is_contiguous() and out.shape == x.shape, "add_rmsnorm: out must be contiguous [T, H]")
     _need(weight.is_contiguous() and weight.numel() == hidden, f"add_rmsnorm: weight must hold {hidden} values")
-    _check(library().lrs_add_rmsnorm(_dev(out, "out"), dtype_code(out.dtype), _dev(x, "x"), _dev(y, "y"), _dev(weight, "weight"),
-                                     dtype_code(weight.dtype), n_rows, hidden, eps, _stream()))
+    _launch("lrs_add_rmsnorm", _dev(out, "out"), dtype_code(out.dtype), _dev(x, "x"), _dev(y, "y"), _dev(weight, "weight"),
+                                     dtype_code(weight.dtype), n_rows, hidden, eps, _stream())
 
 
 def rope_table(cos: torch.Tensor, sin: torch.Tensor, positions: torch.Tensor, inv_freq: torch.Tensor) -> None:
@@ -281,8 +360,8 @@ def rope_table(cos: torch.Tensor, sin: torch.Tensor, positions: torch.Tensor, in
     _need(cos.is_contiguous() and sin.is_contiguous() and sin.shape == cos.shape, "rope_table: cos and sin must be contiguous [T, half]")
     _need(inv_freq.numel() == half and inv_freq.is_contiguous(), "rope_table: inv_freq must hold `half` values")
     _need(positions.dtype == torch.int32 and positions.numel() >= tokens and positions.is_contiguous(), "rope_table: positions must be int32 [T]")
-    _check(library().lrs_rope_table(_dev(cos, "cos", torch.float32), _dev(sin, "sin", torch.float32), _dev(positions, "positions"),
-                                    _dev(inv_freq, "inv_freq", torch.float32), tokens, half, _stream()))
+    _launch("lrs_rope_table", _dev(cos, "cos", torch.float32), _dev(sin, "sin", torch.float32), _dev(positions, "positions"),
+                                    _dev(inv_freq, "inv_freq", torch.float32), tokens, half, _stream())
 
 
 def qk_prep(qkv: torch.Tensor, nq: int, nkv: int, d: int, q_weight, k_weight, eps: float, cos, sin,
@@ -305,12 +384,12 @@ def qk_prep(qkv: torch.Tensor, nq: int, nkv: int, d: int, q_weight, k_weight, ep
               f"qk_prep: key pages must be [pages, {nkv}, {page_size}, {d}] and value pages [pages, {nkv}, {d}, {page_size}]")
         _need(k_pages.is_contiguous() and v_pages.is_contiguous() and k_pages.dtype == qkv.dtype and v_pages.dtype == qkv.dtype, "qk_prep: pages must be contiguous and of the activation dtype")
         _need(slots.dtype == torch.int32 and slots.numel() >= tokens and slots.is_contiguous(), "qk_prep: slots must be int32 [T]")
-    _check(library().lrs_qk_prep(
+    _launch("lrs_qk_prep", 
         _dev(qkv, "qkv"), dtype_code(qkv.dtype), tokens, stride, nq, nkv, d,
         None if q_weight is None else _dev(q_weight, "q_weight"), None if k_weight is None else _dev(k_weight, "k_weight"),
         dtype_code(w_dtype), eps, None if cos is None else cos.data_ptr(), None if sin is None else sin.data_ptr(), rot_half,
         None if nkv == 0 else _dev(k_pages, "k_pages"), None if nkv == 0 else _dev(v_pages, "v_pages"),
-        None if nkv == 0 else _dev(slots, "slots"), page_size, _stream()))
+        None if nkv == 0 else _dev(slots, "slots"), page_size, _stream())
 
 
 def gemm_mid_qk_prep_takes(dtype: torch.dtype, m: int, nq: int, nkv: int, d: int, k: int, rot_half: int,
@@ -347,25 +426,25 @@ def gemm_mid_qk_prep(qkv: torch.Tensor, a: torch.Tensor, w: torch.Tensor, sumsq:
           f"gemm_mid_qk_prep: key pages must be [pages, {nkv}, {page_size}, {d}] and value pages [pages, {nkv}, {d}, {page_size}]")
     _need(k_pages.is_contiguous() and v_pages.is_contiguous() and k_pages.dtype == torch.bfloat16 and v_pages.dtype == torch.bfloat16, "gemm_mid_qk_prep: pages must be contiguous bf16")
     _need(slots.dtype == torch.int32 and slots.numel() >= m and slots.is_contiguous(), "gemm_mid_qk_prep: slots must be int32 [T]")
-    _check(library().lrs_gemm_mid_qk_prep(
+    _launch("lrs_gemm_mid_qk_prep", 
         _dev(qkv, "qkv"), _rows(qkv, "qkv"), _dev(a, "a"), _dev(w, "w"), m, k, _rows(a, "a"),
         None if sumsq is None else _dev(sumsq, "sumsq"), 0 if sumsq is None else sumsq.shape[0], in_eps if sumsq is not None else 0.0,
         nq, nkv, d, None if q_weight is None else _dev(q_weight, "q_weight"), None if k_weight is None else _dev(k_weight, "k_weight"),
         dtype_code(w_dtype), eps, None if cos is None else cos.data_ptr(), None if sin is None else sin.data_ptr(), rot_half,
-        _dev(k_pages, "k_pages"), _dev(v_pages, "v_pages"), _dev(slots, "slots"), page_size, choice.word, _stream()))
+        _dev(k_pages, "k_pages"), _dev(v_pages, "v_pages"), _dev(slots, "slots"), page_size, choice.word, _stream())
 
 
 def silu_mul(out: torch.Tensor, gate_up: torch.Tensor, interleaved: bool = False) -> None:
     """out = silu(gate) * up; gate_up holds [gate | up], or groups of 8 gate then 8 up columns if `interleaved`."""
     tokens, inter = out.shape
     _need(out.is_contiguous() and gate_up.is_contiguous() and gate_up.shape == (tokens, 2 * inter) and gate_up.dtype == out.dtype, "silu_mul: gate_up must be [T, 2I] and out [T, I], same dtype")
-    _check(library().lrs_silu_mul(_dev(out, "out"), _dev(gate_up, "gate_up"), dtype_code(out.dtype), tokens, inter, 1 if interleaved else 0, _stream()))
+    _launch("lrs_silu_mul", _dev(out, "out"), _dev(gate_up, "gate_up"), dtype_code(out.dtype), tokens, inter, 1 if interleaved else 0, _stream())
 
 
 def add_into(residual: torch.Tensor, y: torch.Tensor) -> None:
     """residual (float32) += y, same shape, both contiguous."""
     _need(residual.dtype == torch.float32 and residual.shape == y.shape and residual.is_contiguous() and y.is_contiguous(), "add_into: float32 residual and y of one contiguous shape needed")
-    _check(library().lrs_add_into(_dev(residual, "residual"), _dev(y, "y"), dtype_code(y.dtype), residual.numel(), _stream()))
+    _launch("lrs_add_into", _dev(residual, "residual"), _dev(y, "y"), dtype_code(y.dtype), residual.numel(), _stream())
 
 
 def few_rows_capacity() -> int:
@@ -412,9 +491,9 @@ def gemm_mid_add_norm_begin(residual: torch.Tensor, a: torch.Tensor, w: torch.Te
     _need(next_sumsq.dtype == torch.float32 and next_sumsq.is_contiguous() and next_sumsq.shape == (norm_begin_parts(n), m),
           f"gemm_mid_add_norm_begin: next_sumsq must be contiguous float32 [{norm_begin_parts(n)}, {m}]")
     _need(norm_weight.is_contiguous() and norm_weight.numel() == n, f"gemm_mid_add_norm_begin: norm weight must hold {n} values")
-    _check(library().lrs_gemm_mid_add_norm_begin(_dev(residual, "residual"), _dev(a, "a"), _dev(w, "w"), _dev(norm_weight, "norm_weight"),
+    _launch("lrs_gemm_mid_add_norm_begin", _dev(residual, "residual"), _dev(a, "a"), _dev(w, "w"), _dev(norm_weight, "norm_weight"),
                                                  dtype_code(norm_weight.dtype), _dev(next_x, "next_x"), _dev(next_sumsq, "next_sumsq"),
-                                                 m, n, k, _rows(a, "a"), choice.word, _stream()))
+                                                 m, n, k, _rows(a, "a"), choice.word, _stream())
 
 
 def gemm_mid_scaled(out: torch.Tensor, a: torch.Tensor, w: torch.Tensor, sumsq: torch.Tensor, eps: float, swiglu: bool = False,
@@ -430,8 +509,8 @@ def gemm_mid_scaled(out: torch.Tensor, a: torch.Tensor, w: torch.Tensor, sumsq: 
     _need(out.dtype in (torch.bfloat16, torch.float32) and not (swiglu and out.dtype != torch.bfloat16), "gemm_mid_scaled: output must be bf16, or float32 without swiglu")
     _need(sumsq.dtype == torch.float32 and sumsq.dim() == 2 and sumsq.shape[1] == m and sumsq.is_contiguous() and eps > 0, f"gemm_mid_scaled: sumsq must be float32 [parts, {m}] and eps positive")
     mode = OUT_STORE if out.dtype == torch.bfloat16 else OUT_STORE_F32
-    _check(library().lrs_gemm_mid_scaled(_dev(out, "out"), mode, _dev(a, "a"), _dev(w, "w"), m, n, k, _rows(a, "a"), _rows(out, "out"),
-                                         int(swiglu), _dev(sumsq, "sumsq"), sumsq.shape[0], eps, choice.word, _stream()))
+    _launch("lrs_gemm_mid_scaled", _dev(out, "out"), mode, _dev(a, "a"), _dev(w, "w"), m, n, k, _rows(a, "a"), _rows(out, "out"),
+                                         int(swiglu), _dev(sumsq, "sumsq"), sumsq.shape[0], eps, choice.word, _stream())
 
 
 def _int_vector(t: torch.Tensor, name: str, at_least: int) -> int:
@@ -445,10 +524,10 @@ def advance_decode(token_ids: torch.Tensor, positions: torch.Tensor, token_reque
     take the tokens in `chosen`, move one position on, lengthen their requests by one and (with
     `draws`, the counters of seeded sampling) count one more draw."""
     rows = token_ids.numel()
-    _check(library().lrs_advance_decode(_int_vector(token_ids, "token_ids", rows), _int_vector(positions, "positions", rows),
+    _launch("lrs_advance_decode", _int_vector(token_ids, "token_ids", rows), _int_vector(positions, "positions", rows),
                                         _int_vector(token_request, "token_request", rows), _int_vector(seq_lens, "seq_lens", 1),
                                         _int_vector(chosen, "chosen", rows), None if draws is None else _int_vector(draws, "draws", rows),
-                                        _int_vector(real_rows, "real_rows", 1), rows, _stream()))
+                                        _int_vector(real_rows, "real_rows", 1), rows, _stream())
 
 
 def advance_slots(slots: torch.Tensor, positions: torch.Tensor, token_request: torch.Tensor, block_table: torch.Tensor,
@@ -456,21 +535,21 @@ def advance_slots(slots: torch.Tensor, positions: torch.Tensor, token_request: t
     """The cache slots of the (already advanced) positions of the first real_rows[0] rows, from the block table."""
     rows = slots.numel()
     _need(block_table.dim() == 2 and block_table.dtype == torch.int32 and block_table.stride(1) == 1, "advance_slots: block_table must be int32 [R, blocks]")
-    _check(library().lrs_advance_slots(_int_vector(slots, "slots", rows), _int_vector(positions, "positions", rows),
+    _launch("lrs_advance_slots", _int_vector(slots, "slots", rows), _int_vector(positions, "positions", rows),
                                        _int_vector(token_request, "token_request", rows), _dev(block_table, "block_table"),
-                                       block_table.stride(0), page_size, _int_vector(real_rows, "real_rows", 1), rows, _stream()))
+                                       block_table.stride(0), page_size, _int_vector(real_rows, "real_rows", 1), rows, _stream())
 
 
 def fill_i32(dst: torch.Tensor, value: int) -> None:
     _need(dst.dtype == torch.int32 and dst.is_contiguous(), "fill_i32: int32 contiguous tensor needed")
-    _check(library().lrs_fill_i32(_dev(dst, "dst"), value, dst.numel(), _stream()))
+    _launch("lrs_fill_i32", _dev(dst, "dst"), value, dst.numel(), _stream())
 
 
 def gather_rows(out: torch.Tensor, x: torch.Tensor, rows: torch.Tensor) -> None:
     n_rows, hidden = out.shape
     _need(out.is_contiguous() and x.is_contiguous() and x.shape[1] == hidden, "gather_rows: shapes disagree")
     _need(rows.dtype == torch.int32 and rows.numel() >= n_rows, "gather_rows: rows must be int32")
-    _check(library().lrs_gather_rows(_dev(out, "out", torch.float32), _dev(x, "x", torch.float32), _dev(rows, "rows"), n_rows, hidden, _stream()))
+    _launch("lrs_gather_rows", _dev(out, "out", torch.float32), _dev(x, "x", torch.float32), _dev(rows, "rows"), n_rows, hidden, _stream())
 
 
 # ------------------------------------------------------------------- gemm
@@ -524,10 +603,10 @@ def gemm(out: torch.Tensor, a: torch.Tensor, w: torch.Tensor, bias: torch.Tensor
         _need(bias.numel() == n and bias.dtype == w.dtype and bias.is_contiguous(), "gemm: bias must hold N values of the weight dtype")
     if swiglu:
         _need(w.dtype == torch.bfloat16 and n % 16 == 0 and k % 8 == 0 and bias is None and mode == OUT_STORE, "gemm: swiglu needs bf16, N % 16 == 0, K % 8 == 0, no bias, a stored output")
-    _check(library().lrs_gemm(_dev(out, "out"), mode, _dev(a, "a"), _dev(w, "w"), None if bias is None else _dev(bias, "bias"),
+    _launch("lrs_gemm", _dev(out, "out"), mode, _dev(a, "a"), _dev(w, "w"), None if bias is None else _dev(bias, "bias"),
                               dtype_code(w.dtype), m, n, k, lda, ldc, None if rows is None else _dev(rows, "rows"),
                               None if not normed else _dev(norm_weight, "norm_weight"), dtype_code(norm_weight.dtype) if normed else 0,
-                              eps, 1 if swiglu else 0, choice.word, _stream()))
+                              eps, 1 if swiglu else 0, choice.word, _stream())
 
 
 def library_gemm(out: torch.Tensor, a: torch.Tensor, w: torch.Tensor) -> None:
@@ -538,8 +617,8 @@ def library_gemm(out: torch.Tensor, a: torch.Tensor, w: torch.Tensor) -> None:
     _need(a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and w.dim() == 2 and w.shape[1] == k and w.is_contiguous(),
           f"library_gemm: a and w must be bfloat16, w contiguous [N, {k}]")
     _need(out.shape == (m, n) and out.dtype in (torch.bfloat16, torch.float32), f"library_gemm: out must be bfloat16 or float32 [{m}, {n}]")
-    _check(library().lrs_library_gemm(_dev(out, "out"), 1 if out.dtype == torch.float32 else 0, _dev(a, "a"), _dev(w, "w"), m, n, k,
-                                      _rows(a, "a"), _rows(out, "out"), _stream()))
+    _launch("lrs_library_gemm", _dev(out, "out"), 1 if out.dtype == torch.float32 else 0, _dev(a, "a"), _dev(w, "w"), m, n, k,
+                                      _rows(a, "a"), _rows(out, "out"), _stream())
 
 
 NORM_CHAIN_MAX_ROWS = 16
@@ -596,12 +675,12 @@ def gemm_norm_chain(out: torch.Tensor, a: torch.Tensor, w: torch.Tensor, bias: t
         _need(next_sumsq is not None and next_sumsq.dtype == torch.float32 and next_sumsq.shape == (norm_chain_parts(n), m) and next_sumsq.is_contiguous(),
               f"gemm_norm_chain: next_sumsq must be contiguous float32 [{norm_chain_parts(n)}, {m}]")
         _need(next_weight is not None and next_weight.numel() == n and next_weight.is_contiguous(), "gemm_norm_chain: next_weight must hold N values")
-    _check(library().lrs_gemm_norm_chain(
+    _launch("lrs_gemm_norm_chain", 
         _dev(out, "out"), mode, _dev(a, "a"), _dev(w, "w"), None if bias is None else _dev(bias, "bias"), m, n, k, lda, ldc,
         1 if swiglu else 0, None if in_sumsq is None else _dev(in_sumsq, "in_sumsq"), parts, in_eps,
         None if next_x is None else _dev(next_x, "next_x"), None if next_x is None else _dev(next_sumsq, "next_sumsq"),
         None if next_x is None else _dev(next_weight, "next_weight"), dtype_code(next_weight.dtype) if next_x is not None else 0,
-        choice.word, _stream()))
+        choice.word, _stream())
 
 
 def scale_rows(out: torch.Tensor, x: torch.Tensor, sumsq: torch.Tensor, eps: float) -> None:
@@ -610,7 +689,7 @@ def scale_rows(out: torch.Tensor, x: torch.Tensor, sumsq: torch.Tensor, eps: flo
     _need(x.dtype == torch.bfloat16 and out.dtype == torch.bfloat16 and out.shape == x.shape and x.is_contiguous() and out.is_contiguous(),
           "scale_rows: x and out must be contiguous bf16 of one shape")
     _need(sumsq.dtype == torch.float32 and sumsq.dim() == 2 and sumsq.shape[1] == m and sumsq.is_contiguous(), f"scale_rows: sumsq must be float32 [parts, {m}]")
-    _check(library().lrs_scale_rows(_dev(out, "out"), _dev(x, "x"), _dev(sumsq, "sumsq"), sumsq.shape[0], m, hidden, eps, _stream()))
+    _launch("lrs_scale_rows", _dev(out, "out"), _dev(x, "x"), _dev(sumsq, "sumsq"), sumsq.shape[0], m, hidden, eps, _stream())
 
 
 # -------------------------------------------------------------- attention
@@ -627,10 +706,10 @@ def attention(out: torch.Tensor, q: torch.Tensor, k_pages: torch.Tensor, v_pages
     _need(block_table.dim() == 2 and block_table.dtype == torch.int32 and block_table.stride(1) == 1, "attention: block_table must be int32 [R, blocks]")
     for name, t in (("token_request", token_request), ("positions", positions)):
         _need(t.dtype == torch.int32 and t.numel() >= tokens and t.is_contiguous(), f"attention: {name} must be int32 [T]")
-    _check(library().lrs_attention(
+    _launch("lrs_attention", 
         _dev(out, "out"), _rows(out, "out"), _dev(q, "q"), _rows(q, "q"), _dev(k_pages, "k_pages"), _dev(v_pages, "v_pages"),
         _dev(block_table, "block_table"), block_table.stride(0), _dev(token_request, "token_request"), _dev(positions, "positions"),
-        dtype_code(q.dtype), tokens, nq, nkv, d, page_size, scale, window, _stream()))
+        dtype_code(q.dtype), tokens, nq, nkv, d, page_size, scale, window, _stream())
 
 
 DECODE_HEAD_DIMS = (32, 64, 96, 128, 192)
@@ -698,12 +777,12 @@ def attention_decode(out: torch.Tensor, q: torch.Tensor, k_pages: torch.Tensor, 
         fused = [1, _dev(prepare.q_weight, "q_weight") if normed else None, _dev(prepare.k_weight, "k_weight") if normed else None,
                  dtype_code(prepare.q_weight.dtype) if normed else 0, prepare.eps,
                  None if prepare.cos is None else _dev(prepare.cos, "cos"), None if prepare.sin is None else _dev(prepare.sin, "sin"), prepare.kv_heads]
-    _check(library().lrs_attention_decode(
+    _launch("lrs_attention_decode", 
         _dev(out, "out"), _rows(out, "out"), None if splits == 1 else _dev(part_o, "part_o"), None if splits == 1 else _dev(part_ml, "part_ml"),
         _dev(q, "q"), _rows(q, "q"), _dev(k_pages, "k_pages"), _dev(v_pages, "v_pages"), _dev(block_table, "block_table"), block_table.stride(0),
         _dev(token_request, "token_request"), _dev(positions, "positions"), tokens,
         block_table.shape[1] * page_size if max_context is None else max_context, nq, nkv, d, page_size, scale, window, splits,
-        form, *fused, _stream()))
+        form, *fused, _stream())
 
 
 def attention_prefill(out: torch.Tensor, q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, block_table: torch.Tensor,
@@ -733,13 +812,13 @@ def attention_prefill(out: torch.Tensor, q: torch.Tensor, k_pages: torch.Tensor,
     if splits > 1:
         _need(part_o is not None and part_o.dtype == torch.float32 and part_o.is_contiguous() and part_o.numel() >= tokens * nq * splits * d, "attention_prefill: part_o too small")
         _need(part_ml is not None and part_ml.dtype == torch.float32 and part_ml.is_contiguous() and part_ml.numel() >= tokens * nq * splits * 2, "attention_prefill: part_ml too small")
-    _check(library().lrs_attention_prefill(
+    _launch("lrs_attention_prefill", 
         _dev(out, "out"), _rows(out, "out"), _dev(q, "q"), _rows(q, "q"), _dev(k_pages, "k_pages"), _dev(v_pages, "v_pages"),
         _dev(block_table, "block_table"), block_table.stride(0), _dev(token_request, "token_request"), _dev(positions, "positions"),
         _dev(qblock_token0, "qblock_token0"), _dev(qblock_count, "qblock_count"), n_blocks,
         attention_prefill_group() if max_count is None else max_count,
         block_table.shape[1] * page_size if max_context is None else max_context, nq, nkv, d, page_size, scale, window,
-        tokens, splits, None if splits == 1 else _dev(part_o, "part_o"), None if splits == 1 else _dev(part_ml, "part_ml"), _stream()))
+        tokens, splits, None if splits == 1 else _dev(part_o, "part_o"), None if splits == 1 else _dev(part_ml, "part_ml"), _stream())
 
 
 def compute_units() -> int:
@@ -785,10 +864,10 @@ def choose_tokens(out: torch.Tensor, logits: torch.Tensor, temperature=None, see
         if scratch is None:
             scratch = _choose_scratch[key] = (torch.empty(rows * parts, dtype=torch.float32, device=logits.device),
                                               torch.empty(rows * parts, dtype=torch.int32, device=logits.device))
-        _check(library().lrs_choose_tokens_split(out_pointer, _dev(logits, "logits", torch.float32), stride, rows, vocab, *args,
-                                                 _dev(scratch[0], "part_value"), _dev(scratch[1], "part_index"), parts, _stream()))
+        _launch("lrs_choose_tokens_split", out_pointer, _dev(logits, "logits", torch.float32), stride, rows, vocab, *args,
+                                                 _dev(scratch[0], "part_value"), _dev(scratch[1], "part_index"), parts, _stream())
         return
-    _check(library().lrs_choose_tokens(out_pointer, _dev(logits, "logits", torch.float32), stride, rows, vocab, *args, _stream()))
+    _launch("lrs_choose_tokens", out_pointer, _dev(logits, "logits", torch.float32), stride, rows, vocab, *args, _stream())
 
 
 def choose_tokens_static(out: torch.Tensor, logits: torch.Tensor, parts: int, temperature=None, seeds=None, counters=None) -> None:
@@ -802,10 +881,10 @@ def choose_tokens_static(out: torch.Tensor, logits: torch.Tensor, parts: int, te
         _need(temperature.dtype == torch.float32 and temperature.numel() >= rows, "choose_tokens_static: temperature must be float32 [R]")
         _need(seeds is not None and seeds.dtype == torch.int64 and seeds.numel() >= rows, "choose_tokens_static: seeds must be int64 [R]")
         _need(counters is not None and counters.dtype == torch.int32 and counters.numel() >= rows, "choose_tokens_static: counters must be int32 [R]")
-    _check(library().lrs_choose_tokens_static(
+    _launch("lrs_choose_tokens_static", 
         _dev(out, "out"), _dev(logits, "logits", torch.float32), _rows(logits, "logits"), rows, vocab,
         None if temperature is None else _dev(temperature, "temperature"), None if temperature is None else _dev(seeds, "seeds"),
-        None if temperature is None else _dev(counters, "counters"), parts, _stream()))
+        None if temperature is None else _dev(counters, "counters"), parts, _stream())
 
 
 def filter_logits(logits: torch.Tensor, temperature: torch.Tensor, top_k: torch.Tensor | None, top_p: torch.Tensor | None) -> None:
@@ -816,5 +895,5 @@ def filter_logits(logits: torch.Tensor, temperature: torch.Tensor, top_k: torch.
         _need(top_k.dtype == torch.int32 and top_k.numel() >= rows, "filter_logits: top_k must be int32 [R]")
     if top_p is not None:
         _need(top_p.dtype == torch.float32 and top_p.numel() >= rows, "filter_logits: top_p must be float32 [R]")
-    _check(library().lrs_filter_logits(_dev(logits, "logits", torch.float32), stride, rows, vocab, _dev(temperature, "temperature"),
-                                       None if top_k is None else _dev(top_k, "top_k"), None if top_p is None else _dev(top_p, "top_p"), _stream()))
+    _launch("lrs_filter_logits", _dev(logits, "logits", torch.float32), stride, rows, vocab, _dev(temperature, "temperature"),
+                                       None if top_k is None else _dev(top_k, "top_k"), None if top_p is None else _dev(top_p, "top_p"), _stream())

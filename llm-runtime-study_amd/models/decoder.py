@@ -65,6 +65,11 @@ class DecoderModel:
         can be captured in a HIP graph: every part must say so itself."""
         return all(getattr(layer, "graph_safe", False) for layer in self.layers)
 
+    def plan_safe(self) -> bool:
+        """Whether a step's launches can be written down once and made again from the record: every part must
+        launch through this package's kernels alone, with arguments that follow from the step's shape."""
+        return all(getattr(layer, "plan_safe", False) for layer in self.layers) and getattr(self.final_norm, "plan_safe", False)
+
     def weight_bytes(self, with_embedding: bool = False) -> int:
         """Bytes of weights one decode step reads: every scheduled layer once, and the head."""
         total = sum(self.layers[e.layer].weight_bytes() for e in self.spec.schedule)

@@ -25,6 +25,7 @@ from .linear import ScaledRows, kernels_of, linear, materialize, rows_of
 
 class GQAAttention(Part):
     graph_safe = True  # launches only library kernels on arena buffers
+    plan_safe = True   # ... and nothing but this package's kernels, with arguments that follow the step's shape alone
     takes_lazy_norm = True
     begins_next_norm = True
 
@@ -162,14 +163,15 @@ class GQAAttention(Part):
                                  nq, self.scale, self.window or 0, splits, part_o, part_ml, ctx.max_k_bound, prepare,
                                  form=1)   # the next tile on its way while one is worked on, the first one before the query is prepared (measured: 0.6 % of a step)
         elif ops.attention_decode_supported(ctx.dtype, nq, kv_heads, d, group.page_size):
-            longest = ctx.max_k if self.window is None else min(ctx.max_k, self.window + 64)
+            # sized by the step's coarse bound of the longest context, the same for every step of one shape
+            longest = ctx.max_k_bound if self.window is None else min(ctx.max_k_bound, self.window + 64)
             splits = self._prefill_splits(ctx.num_qblocks * kv_heads, longest, t * nq * d)
             part_o = part_ml = None
             if splits > 1:
                 part_o = ctx.scratch("attn_part_o", (t, nq * splits * d), torch.float32)
                 part_ml = ctx.scratch("attn_part_ml", (t, nq * splits * 2), torch.float32)
             ops.attention_prefill(out, qkv, cache.k_pages, cache.v_pages, group.block_table, ctx.token_request, ctx.positions,
-                                  ctx.qblock_token0, ctx.qblock_count, nq, self.scale, self.window or 0, ctx.max_qblock, ctx.max_k,
+                                  ctx.qblock_token0, ctx.qblock_count, nq, self.scale, self.window or 0, ctx.max_qblock, ctx.max_k_bound,
                                   splits, part_o, part_ml)
         else:
             ops.attention(out, qkv, cache.k_pages, cache.v_pages, group.block_table, ctx.token_request, ctx.positions,

@@ -27,6 +27,14 @@ Optional, each announced by a class attribute (a part without it is simply given
                               normalised input a previous block began and may return the next one;
                               `first_norm` is the norm it applies to its input
 
+A part may also say how its steps can be run again without it (both default to no):
+
+  graph_safe = True           it launches only kernels on preallocated buffers, and reads the step's data from
+                              the device (never from ctx.host_*): decode steps can be captured in a HIP graph
+  plan_safe = True            it launches through this package's kernels (kernels/ops.py) alone, with arguments that
+                              follow from the step's shape: a step's launches can be recorded and made again by
+                              one call (engine/step.py), without running the part
+
 `ctx` is the StepContext of engine/step.py: the step's token metadata on the device and a
 scratch arena.  The residual stream `h` is float32 in every precision mode.
 """

@@ -42,6 +42,10 @@ class PreNormBlock(Part):
     def graph_safe(self) -> bool:
         return all(getattr(part, "graph_safe", False) for _, part in self._children())
 
+    @property
+    def plan_safe(self) -> bool:
+        return all(getattr(part, "plan_safe", False) for _, part in self._children())
+
     chains_norms = True
 
     @property

@@ -16,6 +16,7 @@ from .linear import linear, rows_of
 
 class SwiGLU(Part):
     graph_safe = True  # launches only library kernels on arena buffers
+    plan_safe = True
     takes_lazy_norm = True
     begins_next_norm = True
 

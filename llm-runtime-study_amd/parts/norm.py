@@ -13,6 +13,7 @@ from .linear import LazyNorm
 
 class RMSNorm(Part):
     graph_safe = True  # launches only library kernels on arena buffers
+    plan_safe = True
     has_lazy_form = True
 
     def __init__(self, size: int, eps: float):

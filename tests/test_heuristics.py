@@ -135,3 +135,24 @@ def test_kernel_choices_travel_with_the_call():
     if ops.compute_units() in (0, 256):
         assert ops.gemm_mid_shape(4096, 4096, ops.KernelChoice(mid_waves=8, mid_splits=2)) == (8, 2)
         assert ops.gemm_mid_shape(4096, 4096) == (4, 4)
+
+
+def test_the_generated_plan_dispatch_is_in_step_with_the_entry_point_table():
+    """csrc/plan_dispatch.inc is made from ops.PLAN_OPS and ops._SIGNATURES; whoever changes an entry point's
+    arguments has to make it again (python -m llm_runtime_study_amd.kernels.plan_codegen)."""
+    from llm_runtime_study_amd.kernels import ops, plan_codegen
+
+    assert plan_codegen.TARGET.read_text() == plan_codegen.generate()
+    assert len(set(ops.PLAN_OPS)) == len(ops.PLAN_OPS) and all(ops._SIGNATURES[name][1][-1] is not None for name in ops.PLAN_OPS)
+
+
+def test_a_plan_packs_one_word_per_argument():
+    from llm_runtime_study_amd.kernels import ops
+
+    plan = ops.Plan([("lrs_add_into", (0x7F0000001000, 0x7F0000002000, 1, 1 << 33)),
+                     ("lrs_scale_rows", (1, 2, 3, 4, 5, 6, 0.5)), ("lrs_fill_i32", (None, -7, 12))])
+    words = list(plan.words)[:plan.length]
+    assert plan.launches == 3 and plan.length == 5 + 8 + 4
+    assert words[:5] == [ops.PLAN_OPS.index("lrs_add_into"), 0x7F0000001000, 0x7F0000002000, 1, 1 << 33]
+    assert words[5] == ops.PLAN_OPS.index("lrs_scale_rows") and words[12] == 0x3F000000        # 0.5 as its 32 bits
+    assert words[13:] == [ops.PLAN_OPS.index("lrs_fill_i32"), 0, (1 << 64) - 7, 12]               # None: a null pointer; -7: two's complement

@@ -293,3 +293,71 @@ def test_one_layer_at_the_benchmark_sizes_against_the_plain_implementation():
     want = plain.qwen3_forward(small, raw, [used.index(t) for t in ids])
     torch.testing.assert_close(got[:, columns].double(), want, rtol=1e-4, atol=1e-4)
     assert want.abs().max() > 1.0
+
+
+# ---------------------------------------------------------------- launch plans
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_steps_made_again_from_a_recorded_plan_equal_steps_through_the_parts(folder_b, dtype):
+    """Two runners over the same weights, one recording launch plans, one not, through the same steps: prompt
+    portions, mixed steps and eager decode steps whose shapes come back with other tokens, other pages and
+    other (longer) contexts.  Every logits row and the pages are bit for bit the same; the second time a
+    shape comes, it is served from the plan; a shape whose longest context has left its 256-token class is
+    recorded anew."""
+    from llm_runtime_study_amd.engine.step import StepEntry
+
+    rng = np.random.default_rng(11)
+    vocab = TINY_B["vocab_size"]
+    runners = [make_runner(folder_b, dtype, pages=80, requests=4, seq=400, step_tokens=96) for _ in range(2)]
+    runners[1].use_plans = False
+    assert runners[0].use_plans
+    caches = [[r.cache.admit(i) for i in range(4)] for r in runners]
+
+    def both(plan):
+        """plan: list of (request, tokens, want); runs it on both runners and compares."""
+        outs = []
+        for runner, mine in zip(runners, caches):
+            outs.append(runner.step([StepEntry(mine[i], tokens, want) for i, tokens, want in plan]))
+        if outs[0] is None:
+            assert outs[1] is None
+        else:
+            assert torch.equal(outs[0], outs[1])
+
+    def portion(n):
+        return rng.integers(0, vocab, n).tolist()
+
+    # rounds one and two: every shape is new; a step during which a scratch buffer was made or grown is not kept
+    # (addresses written down before the buffer moved are stale), so a shape may be recorded twice
+    for first, second, third in ((0, 1, 2), (3, 2, 1)):
+        both([(first, portion(40), [39]), (second, portion(33), [0, 32])])
+        both([(first, portion(1), [0]), (second, portion(1), [0]), (third, portion(20), [19])])
+        both([(0, portion(1), [0]), (1, portion(1), [0]), (2, portion(1), [0])])
+    recorded, replayed = runners[0].plan_recordings, runners[0].plan_replays
+    assert recorded == 3 and 1 <= replayed <= 3 and len(runners[0]._plans) == 3      # a recording that was not kept counts as neither
+    # round three: the same shapes with other tokens, requests in other places and longer contexts (still below 256)
+    both([(2, portion(40), [39]), (3, portion(33), [0, 32])])
+    both([(2, portion(1), [0]), (3, portion(1), [0]), (0, portion(20), [19])])
+    for _ in range(5):
+        both([(0, portion(1), [0]), (1, portion(1), [0]), (2, portion(1), [0])])
+    assert runners[0].plan_recordings == recorded and runners[0].plan_replays == replayed + 7
+    # request 1 grows past 256 tokens: the same three-token decode shape, another class of context, a new plan
+    both([(1, portion(96), [])])
+    both([(1, portion(96), [95])])
+    both([(1, portion(30), [])])
+    assert caches[0][1].length > 256
+    before = runners[0].plan_recordings
+    both([(0, portion(1), [0]), (1, portion(1), [0]), (2, portion(1), [0])])
+    both([(0, portion(1), [0]), (1, portion(1), [0]), (2, portion(1), [0])])
+    assert runners[0].plan_recordings == before + 1
+    torch.cuda.synchronize()
+    for a, b in zip(runners[0].cache.layer_caches, runners[1].cache.layer_caches):
+        assert torch.equal(a.k_pages, b.k_pages) and torch.equal(a.v_pages, b.v_pages)
+    # a model with a part that is not known to be safe to record runs through its parts every time
+    runners[0].cache.check_invariants()
+
+
+def test_a_model_with_parts_of_unknown_habits_is_never_recorded():
+    from tests.test_parts_gpu import RunningMeanMixer, build_runner, toy_state_model
+
+    spec, weights, _, _ = toy_state_model("toy_running_mean", RunningMeanMixer)
+    runner = build_runner(spec, weights, torch.float32)
+    assert not runner.use_plans
