@@ -82,6 +82,17 @@ class ScratchArena:
         return sum(b.numel() * b.element_size() for b in self._buffers.values())
 
 
+@dataclass
+class RecordedStep:
+    """The launches of one step shape, written down (see ModelRunner._step_eager)."""
+
+    plan: "ops.Plan"
+    generation: int                      # of the scratch arena when it was recorded
+    logits: torch.Tensor | None          # where the step's logits come out
+    uses: int = 0
+    graph: int | None = None             # the plan captured in a HIP graph, once the shape has come back often enough
+
+
 class StepContext:
     """What the parts see of one step."""
 
@@ -137,7 +148,7 @@ class ModelRunner:
         # is good only while the scratch buffers stay where they are (the arena's generation).  Only models
         # whose every part launches through this package's kernels alone (`plan_safe`) are recorded.
         self.use_plans = use_plans and getattr(model, "plan_safe", lambda: False)()
-        self._plans: dict[tuple, tuple] = {}    # key -> (ops.Plan, arena generation, logits tensor or None)
+        self._plans: dict[tuple, RecordedStep] = {}
         self.plan_replays = 0
         self.plan_recordings = 0
         self.graph_replays = 0     # steps (or launches of several steps) served by replaying a graph
@@ -421,10 +432,27 @@ class ModelRunner:
             return self.model.logits(ctx, h) if ctx.num_logit_rows else None
         key = self._plan_key(ctx)
         known = self._plans.get(key)
-        if known is not None and known[1] == self.arena.generation:
-            ops.plan_run(known[0])
+        if known is not None and known.generation == self.arena.generation:
+            known.uses += 1
+            stream = torch.cuda.current_stream(self.device).cuda_stream
+            if known.graph is None and known.uses >= self.PLAN_GRAPH_AFTER and stream != 0:
+                # a shape that keeps coming back: its launches go into a HIP graph, made by running the plan under
+                # capture (nothing runs then), and from now on the step is one graph launch
+                ops.graph_begin()
+                try:
+                    ops.plan_run(known.plan)
+                except Exception:
+                    ops.graph_destroy(ops.graph_end())
+                    raise
+                known.graph = ops.graph_end()
+            if known.graph is not None and stream != 0:
+                ops.graph_launch(known.graph)
+            else:
+                ops.plan_run(known.plan)
             self.plan_replays += 1
-            return known[2]
+            return known.logits
+        if known is not None:
+            self._forget_plan(key)
         generation = self.arena.generation
         ops.record_begin()
         try:
@@ -436,11 +464,19 @@ class ModelRunner:
         plan = ops.record_end()
         if self.arena.generation == generation:          # else a buffer moved on the way: addresses written down before are stale
             if len(self._plans) >= self.MAX_PLANS:
-                self._plans.pop(next(iter(self._plans)))
-            self._plans[key] = (plan, generation, logits)
+                self._forget_plan(next(iter(self._plans)))
+            self._plans[key] = RecordedStep(plan, generation, logits)
             self.plan_recordings += 1
         return logits
 
+    def _forget_plan(self, key: tuple) -> None:
+        known = self._plans.pop(key, None)
+        if known is not None and known.graph is not None:
+            if self.device.type == "cuda":
+                torch.cuda.synchronize(self.device)
+            ops.graph_destroy(known.graph)
+
+    PLAN_GRAPH_AFTER = 3     # replays of a plan after which it is captured in a graph
     MAX_PLANS = 512      # plans kept (each a few hundred launches of a few dozen words); the oldest goes first
 
     def _undo(self, extended: Sequence[StepEntry], before: Sequence[int], states: list) -> None:
@@ -649,6 +685,8 @@ class ModelRunner:
 
     def drop_graphs(self) -> None:
         """Destroy every captured graph, after the device has finished with them."""
+        for key in list(self._plans):
+            self._forget_plan(key)
         if self._graphs and self.device.type == "cuda":
             torch.cuda.synchronize(self.device)
         for handle, *_ in self._graphs.values():
