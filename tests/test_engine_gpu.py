@@ -537,3 +537,21 @@ def test_staggered_benchmark_runs_every_request_to_its_limit(capsys):
     assert report["makespan_s"] > 0 and report["output_tok_s"] > 0
     assert 0 < report["ttft_ms_p50"] <= report["ttft_ms_p95"] <= report["latency_ms_p95"]
     assert report["latency_ms_p50"] <= report["latency_ms_p95"] <= 1000.0 * report["makespan_s"] + 1e-6
+
+
+@pytest.mark.gpu
+def test_host_cost_benchmark_times_the_three_ways_of_launching_a_step(capsys):
+    """One layer of the 8B shape, a 64-token portion beside two decoding requests: the report holds the three
+    ways of launching, the plan is recorded once and replayed for every timed step, and the graph of the plan
+    costs the host less than the parts do."""
+    import json
+
+    from llm_runtime_study_amd.benchmarks import host_cost
+
+    code = host_cost.main(["--shape", "8b", "--layers", "1", "--tokens", "64", "--decoding", "2", "--context", "40", "--repeats", "3"])
+    assert code == 0
+    report = json.loads(capsys.readouterr().out.strip().splitlines()[-1])
+    for way in ("through_parts", "from_plan", "from_graph_of_plan"):
+        assert 0 < report[way]["host_ms"] <= report[way]["total_ms"]
+    assert report["from_plan"]["replays"] >= 3 and report["from_graph_of_plan"]["replays"] >= 3
+    assert report["from_graph_of_plan"]["host_ms"] < report["through_parts"]["host_ms"]
