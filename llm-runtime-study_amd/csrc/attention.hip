@@ -549,11 +549,13 @@ __global__ __launch_bounds__(256, D <= 128 ? 2 : 1) void attention_prefill_bf16_
     const int* __restrict__ qblock_count, int n_blocks, int chunk, int nq, int nkv, int page_size, float scale,
     int window, int splits, float* __restrict__ part_o, float* __restrict__ part_ml) {
   constexpr int DS = D / 32, DB = D / 16;
-  // Padded LDS rows (32 banks of 4 bytes).  Key rows are read 16 bytes a lane by 8 lanes a cycle: a
-  // stride of 4 banks more than a multiple of 32 spreads them over all banks.  Value rows are read
-  // 8 bytes a lane by 16 lanes a cycle: a stride of 18 banks (twice an odd number) does the same;
-  // such rows start at multiples of 8 bytes only, so they are written 8 bytes at a time.
-  constexpr int KLD = D + 8, VLD = 32 + 4;
+  // Padded LDS rows.  Every fragment is read 16 bytes a lane, 16 rows at a time (the lane's row is col, its
+  // piece g), which the LDS serves at its full 256 bytes a cycle when rows lie 32 bytes more than a multiple
+  // of 64 apart, and at half of that, or worse, otherwise (measured for every stride; 8-byte reads reach
+  // half at best).  Key rows are D elements long; a row of the transposed value tile holds a dimension's 32
+  // keys in the order the second product wants them, so that a lane's eight are one 16-byte piece: position
+  // g * 8 + h * 4 + i for key h * 16 + g * 4 + i, which is where the first product leaves that key's weight.
+  constexpr int KLD = D + 16, VLD = 32 + 16;
   __shared__ __attribute__((aligned(16))) bf16 ks[2][32 * KLD];
   __shared__ __attribute__((aligned(16))) bf16 vs[2][D * VLD];
   const int tid = threadIdx.x, threads = blockDim.x;
@@ -637,9 +639,10 @@ __global__ __launch_bounds__(256, D <= 128 ? 2 : 1) void attention_prefill_bf16_
     for (int i = 0; i < VPT; ++i) {
       const int c = t1 + i * TPR;
       if (c < VRUN_CHUNKS) {
-        bf16* dst = vs[buffer] + (c / 2) * VLD + wrun * 16 + (c % 2) * 8;
+        // keys wrun * 16 + (c % 2) * 8 + 0..7 of dimension c / 2: h = wrun, g = (c % 2) * 2 and the next
+        bf16* dst = vs[buffer] + (c / 2) * VLD + (c % 2) * 16 + wrun * 4;
         *(bf16x4*)dst = bf16x4{vreg[i][0], vreg[i][1], vreg[i][2], vreg[i][3]};
-        *(bf16x4*)(dst + 4) = bf16x4{vreg[i][4], vreg[i][5], vreg[i][6], vreg[i][7]};
+        *(bf16x4*)(dst + 8) = bf16x4{vreg[i][4], vreg[i][5], vreg[i][6], vreg[i][7]};
       }
     }
   };
@@ -764,9 +767,7 @@ __global__ __launch_bounds__(256, D <= 128 ? 2 : 1) void attention_prefill_bf16_
       const bf16* vt = vs[buffer];
 #pragma unroll
       for (int e = 0; e < DB; ++e) {
-        const bf16x4 v0 = *(const bf16x4*)(vt + (e * 16 + col) * VLD + g * 4);
-        const bf16x4 v1 = *(const bf16x4*)(vt + (e * 16 + col) * VLD + 16 + g * 4);
-        const bf16x8 vv = {v0[0], v0[1], v0[2], v0[3], v1[0], v1[1], v1[2], v1[3]};
+        const bf16x8 vv = *(const bf16x8*)(vt + (e * 16 + col) * VLD + g * 8);
 #pragma unroll
         for (int b = 0; b < QB; ++b) o[b][e] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vv, pf[b], o[b][e], 0, 0, 0);
       }
@@ -843,6 +844,399 @@ __global__ __launch_bounds__(256, D <= 128 ? 2 : 1) void attention_prefill_bf16_
   }
 }
 
+// ------------------------------------- bf16 kernel for any step, head size 128
+// The same walk as attention_prefill_bf16_kernel with the tiles brought in differently: memory
+// writes them straight into LDS (global_load_lds_dwordx4: a wave's 64 lanes fetch 16 bytes each,
+// from addresses of their own choice, and the 1,024 bytes land in lane order at the address in m0),
+// so a tile passes through no registers, three tiles are in flight instead of one, nothing is written
+// to LDS by the waves, and where a piece lies in LDS is decided by which lane fetches it.
+//
+// LDS serves 16-byte reads at its full 256 bytes a cycle when the lanes it takes together (eight
+// consecutive rows of the fragment, pieces g and g + 1) fall on 64 different banks; measured, and
+// that is what the layout is made for:
+//   keys    eight blocks of 1,024 bytes (four rows of 256), block j at j * 1,056; row (h, col) of
+//           the first product's fragments lies in block col % 8 as its row 2 h + col / 8, so eight
+//           consecutive columns meet eight blocks, each 8 banks further on than the one before.
+//   values  transposed, a half for each run of 16 keys: [half][dim][16 keys], the second half 16
+//           bytes out of step; lanes g = 0, 2 read the first half's two pieces, g = 1, 3 the second's.
+// A block is one fetch of one wave and comes from one page.  Which key a fragment row holds is free
+// as long as the second product meets the weights where the first left them: lanes of group g hold
+// the scores of keys 8 m + 4 h + i (m = 0, 2, 1, 3 for g = 0..3; h the fragment, i the register), and
+// read the values of keys 8 m .. 8 m + 7 as one piece.
+// The wave that fetched a tile waits for its own fetches (vmcnt) before the barrier that opens the
+// tile to the others; the fetches of the tile after it stay in flight.  The fetches are written in
+// assembly because the compiler would wait for all of them before any LDS read it cannot tell apart.
+__device__ __forceinline__ void fetch_to_lds(const void* base, unsigned lane_offset, unsigned lds_address) {
+  const unsigned lo = __builtin_amdgcn_readfirstlane((unsigned)(uintptr_t)base);
+  const unsigned hi = __builtin_amdgcn_readfirstlane((unsigned)((uintptr_t)base >> 32));
+  const unsigned long long uniform_base = ((unsigned long long)hi << 32) | lo;
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+               :: "s"(__builtin_amdgcn_readfirstlane(lds_address)), "v"(lane_offset), "s"(uniform_base) : "memory");
+}
+// Waits until at most `pending` of this wave's fetches are still on their way, then for the workgroup.
+template <int PENDING>
+__device__ __forceinline__ void fetched_then_barrier() {
+  asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" :: "n"(PENDING) : "memory");
+}
+
+template <int QB>
+__global__ __launch_bounds__(256, 2) void attention_prefill_d128_bf16_kernel(
+    bf16* __restrict__ out, int out_stride, const bf16* __restrict__ q, int q_stride,
+    const bf16* __restrict__ k_pages, const bf16* __restrict__ v_pages,
+    const int* __restrict__ block_table, int table_stride, const int* __restrict__ token_request,
+    const int* __restrict__ positions, const int* __restrict__ qblock_token0,
+    const int* __restrict__ qblock_count, int n_blocks, int chunk, int nq, int nkv, int page_size, float scale,
+    int window, int splits, float* __restrict__ part_o, float* __restrict__ part_ml) {
+  constexpr int D = 128, DS = D / 32, DB = D / 16, STAGES = 3;
+  constexpr int KBLOCK = 1024 + 32, KBYTES = 8 * KBLOCK, VHALF = 16 * D * 2 + 16, VBYTES = 2 * VHALF;
+  constexpr int VSTAGE = (VBYTES + 63) / 64 * 64;
+  __shared__ __attribute__((aligned(64))) unsigned char key_tiles[STAGES * KBYTES];
+  __shared__ __attribute__((aligned(64))) unsigned char value_tiles[STAGES * VSTAGE];
+  const int tid = threadIdx.x;
+  const int lane = tid % WAVE, wave = __builtin_amdgcn_readfirstlane(tid / WAVE);
+  const int col = lane & 15, g = lane >> 4;
+  const int key_chunk = ((g & 1) << 1) | (g >> 1);                 // m: the eight keys this lane group holds weights of
+  const int group = nq / nkv;
+  const int work = blockIdx.x % (n_blocks * nkv), split = blockIdx.x / (n_blocks * nkv);
+  const int which_chunk = work / chunk, in_chunk = work % chunk;
+  const int chunk_block0 = which_chunk * (chunk / nkv);
+  const int chunk_blocks = n_blocks - chunk_block0 < chunk / nkv ? n_blocks - chunk_block0 : chunk / nkv;
+  const int kvh = in_chunk % nkv;
+  const int qblock = chunk_block0 + ((which_chunk & 1) ? chunk_blocks - 1 - in_chunk / nkv : in_chunk / nkv);
+  const int token0 = qblock_token0[qblock], count = qblock_count[qblock];
+  const int pos_first = positions[token0], pos_last = positions[token0 + count - 1];
+  const int lo_first = (window > 0 && pos_first - window + 1 > 0) ? pos_first - window + 1 : 0;
+  const int lo_last = (window > 0 && pos_last - window + 1 > 0) ? pos_last - window + 1 : 0;
+  const int* table = block_table + (int64_t)token_request[token0] * table_stride;
+  const bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
+  const float scale2 = scale * 1.4426950408889634f;
+  const float rescale_step = RESCALE_STEP / scale2;              // in units of the unscaled scores
+  int first_tile = lo_first / 32, last_tile = pos_last / 32;
+  if (splits > 1) {                                              // this workgroup's share of the tiles (may be none)
+    const int per_split = (last_tile - first_tile + splits) / splits;
+    first_tile += split * per_split;
+    if (first_tile + per_split - 1 < last_tile) last_tile = first_tile + per_split - 1;
+  }
+  const int first_run = lo_first / 16, last_run = pos_last / 16;   // runs of 16 keys that hold a key some query sees
+
+  // What this wave fetches of a tile: key blocks `wave` (first run) and `wave + 4` (second run), and the
+  // dimensions 32 wave .. 32 wave + 31 of both value halves.  A lane's distance from the run's first key
+  // (or first slot) never changes; the run's page is looked up once a wave.
+  const int pages16 = page_size / 16;                            // runs of 16 keys in a page
+  const unsigned magic = pages16 > 1 ? 0xFFFFFFFFu / (unsigned)pages16 + 1u : 0u;   // run / pages16 = umulhi(run, magic)
+  // lane l of a key block brings row l / 16 (h = row / 2, k = row % 2), piece l % 16: key 8 k + 4 h + wave of its run
+  const unsigned key_offset = (unsigned)(((((lane >> 4) & 1) * 8 + (lane >> 5) * 4 + wave) * D + (lane & 15) * 8) * 2);
+  // lane l of a value block brings dimension 32 wave + l / 2, keys 8 (l % 2) .. + 7 of the run
+  const unsigned value_offset = (unsigned)((((wave * 32 + (lane >> 1)) * page_size) + (lane & 1) * 8) * 2);
+  const unsigned keys_address = (unsigned)(uintptr_t)(__attribute__((address_space(3))) unsigned char*)key_tiles;
+  const unsigned values_address = (unsigned)(uintptr_t)(__attribute__((address_space(3))) unsigned char*)value_tiles;
+  // Where a run of 16 keys lies in memory.  Everything about it is the same for the whole workgroup, so the
+  // page comes from the block table by a scalar load and the rest is a handful of scalar instructions; a
+  // tile's two pages are asked for a turn before its addresses are wanted.  A run no query sees is masked:
+  // any page with numbers in it will do, so runs are clamped to those the queries do see.
+  const unsigned page_bytes = (unsigned)(nkv * page_size * D * 2);   // from page to page, keys and values alike
+  const char* const k_head = (const char*)(k_pages + (int64_t)kvh * page_size * D);
+  const char* const v_head = (const char*)(v_pages + (int64_t)kvh * page_size * D);
+  // INSIDE: the tile lies behind the first of the walk, so that only the far end needs the clamp
+  auto run_in_reach = [&](auto inside, int tile, int half) {
+    const int run = tile * 2 + half;
+    if (decltype(inside)::value) return run > last_run ? last_run : run;
+    return run < first_run ? first_run : run > last_run ? last_run : run;
+  };
+  auto pages_of = [&](auto inside, int tile, int (&pages)[2]) {
+#pragma unroll
+    for (int half = 0; half < 2; ++half) {
+      const int run = run_in_reach(inside, tile, half);
+      pages[half] = table[pages16 > 1 ? (int)__umulhi((unsigned)run, magic) : run];
+    }
+  };
+  auto locate = [&](auto inside, int tile, const int (&pages)[2], const char* (&kbase)[2], const char* (&vbase)[2]) {
+#pragma unroll
+    for (int half = 0; half < 2; ++half) {
+      const uint64_t at = (uint64_t)(unsigned)pages[half] * page_bytes;
+      if (pages16 > 1) {
+        const int run = run_in_reach(inside, tile, half);
+        const unsigned off = (unsigned)(run - (int)__umulhi((unsigned)run, magic) * pages16) * 16u;
+        kbase[half] = k_head + at + off * (unsigned)(D * 2);
+        vbase[half] = v_head + at + off * 2u;
+      } else {
+        kbase[half] = k_head + at;
+        vbase[half] = v_head + at;
+      }
+    }
+  };
+  auto fetch_keys = [&](const char* const (&kbase)[2], int stage) {      // two fetches a wave
+#pragma unroll
+    for (int half = 0; half < 2; ++half)
+      fetch_to_lds(kbase[half], key_offset, keys_address + (unsigned)(stage * KBYTES + (wave + 4 * half) * KBLOCK));
+  };
+  auto fetch_values = [&](const char* const (&vbase)[2], int stage) {    // two fetches a wave
+#pragma unroll
+    for (int half = 0; half < 2; ++half)
+      fetch_to_lds(vbase[half], value_offset, values_address + (unsigned)(stage * VSTAGE + half * VHALF + wave * 1024));
+  };
+  // where this lane's fragments lie in a stage
+  const int key_fragment = (col & 7) * KBLOCK + (col >> 3) * 256 + g * 16;              // + h * 512 + c * 64
+  const int value_fragment = (g & 1) * VHALF + col * 32 + (g >> 1) * 16;                // + e * 512
+
+  // kv groups of more than four heads take several passes over the keys
+  const int waves = blockDim.x / WAVE;
+  for (int head0 = kvh * group; head0 < (kvh + 1) * group; head0 += waves) {
+    const int head = head0 + wave;
+    const bool active = head < (kvh + 1) * group;
+    bf16x8 qf[QB][DS];
+    floatx4 o[QB][DB];
+    float run_max[QB], run_sum[QB];
+    int pos[QB], lo[QB];
+    bool live[QB];
+#pragma unroll
+    for (int b = 0; b < QB; ++b) {
+      live[b] = active && b * 16 + col < count;
+      const int token = token0 + (live[b] ? b * 16 + col : 0);
+      pos[b] = live[b] ? positions[token] : -1;                // a dead column sees no key
+      lo[b] = (window > 0 && pos[b] - window + 1 > 0) ? pos[b] - window + 1 : 0;
+      run_max[b] = -INFINITY;
+      run_sum[b] = 0.f;
+#pragma unroll
+      for (int c = 0; c < DS; ++c)
+        qf[b][c] = live[b] ? *(const bf16x8*)(q + (int64_t)token * q_stride + (int64_t)head * D + c * 32 + g * 8) : zero8;
+#pragma unroll
+      for (int e = 0; e < DB; ++e) o[b][e] = floatx4{0.f, 0.f, 0.f, 0.f};
+    }
+
+    // scores: S[key, query] = K Q^T, unscaled (the scale enters with the exponent)
+    auto scores = [&](int stage, floatx4 (&sc)[QB][2]) {
+      const unsigned char* kt = key_tiles + stage * KBYTES + key_fragment;
+#pragma unroll
+      for (int b = 0; b < QB; ++b) sc[b][0] = sc[b][1] = floatx4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int h = 0; h < 2; ++h)
+#pragma unroll
+        for (int c = 0; c < DS; ++c) {
+          const bf16x8 kfrag = *(const bf16x8*)(kt + h * 512 + c * 64);
+#pragma unroll
+          for (int b = 0; b < QB; ++b) sc[b][h] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kfrag, qf[b][c], sc[b][h], 0, 0, 0);
+        }
+    };
+    // weights: as in attention_prefill_bf16_kernel; sc[b][h][i] belongs to key tile * 32 + 8 m + 4 h + i
+    auto weights_with_maximum = [&](int tile, floatx4 (&sc)[QB][2], auto masked, bf16x8 (&pf)[QB]) {
+      constexpr bool MASKED = decltype(masked)::value;
+      float alpha[QB];
+      bool rescale = false;
+#pragma unroll
+      for (int b = 0; b < QB; ++b) {
+        float tile_max = -INFINITY;
+#pragma unroll
+        for (int h = 0; h < 2; ++h)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            if (MASKED) {
+              const int key = tile * 32 + key_chunk * 8 + h * 4 + i;
+              sc[b][h][i] = (key <= pos[b] && key >= lo[b]) ? sc[b][h][i] : -INFINITY;
+            }
+            tile_max = fmaxf(tile_max, sc[b][h][i]);
+          }
+        tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 16, WAVE));
+        tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32, WAVE));
+        const float new_max = tile_max > run_max[b] + rescale_step ? tile_max : run_max[b];
+        // a query whose window or position leaves it no key so far keeps its state
+        const bool empty = MASKED && new_max == -INFINITY;
+        alpha[b] = empty ? 1.f : fast_exp2((run_max[b] - new_max) * scale2);
+        const float shift = empty ? 0.f : -new_max * scale2;
+        run_max[b] = new_max;
+        float tile_sum = 0.f;
+#pragma unroll
+        for (int h = 0; h < 2; ++h)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            const float p = fast_exp2(fmaf(sc[b][h][i], scale2, shift));
+            tile_sum += p;
+            pf[b][h * 4 + i] = (bf16)p;
+          }
+        run_sum[b] = run_sum[b] * alpha[b] + tile_sum;
+        rescale |= alpha[b] != 1.f;
+      }
+      if (__any(rescale)) {
+#pragma unroll
+        for (int b = 0; b < QB; ++b)
+#pragma unroll
+          for (int e = 0; e < DB; ++e) o[b][e] *= alpha[b];
+      }
+    };
+    // The short way through the weights of the tile whose scores are in `sc`, and beside it the scores of the
+    // tile after it (keys in `stage`) into `next`: the matrix cores work on the next tile's products while the
+    // vector units turn this tile's scores into weights.  The two are independent and are written here one
+    // product, one weight at a time, with a fence for the instruction scheduler after each pair, so that this
+    // is the order the wave issues them in: a product keeps the matrix core busy for 16 cycles, in which the
+    // three or four vector instructions of a weight cost nothing.  A head of 128 has as many products a tile
+    // (8 for every 16 queries) as a lane has weights.  Returns false, and has changed nothing but pf and
+    // next, if a weight sum says the reference point will not do.
+    auto weights_beside_scores = [&](int stage, floatx4 (&sc)[QB][2], floatx4 (&next)[QB][2], bf16x8 (&pf)[QB]) -> bool {
+      const unsigned char* kt = key_tiles + stage * KBYTES + key_fragment;
+      constexpr int FRAGMENTS = 2 * DS, READ_AHEAD = 3;
+      static_assert(FRAGMENTS * QB == QB * 8, "one weight for every product");
+      bf16x8 kf[FRAGMENTS];
+#pragma unroll
+      for (int f = 0; f < READ_AHEAD; ++f) kf[f] = *(const bf16x8*)(kt + (f / DS) * 512 + (f % DS) * 64);
+      float shift[QB], tile_sum[QB], weight[QB * 8];
+#pragma unroll
+      for (int b = 0; b < QB; ++b) {
+        next[b][0] = next[b][1] = floatx4{0.f, 0.f, 0.f, 0.f};
+        shift[b] = -run_max[b] * scale2;                         // +inf before the query's first tile: the sum then says "again"
+        tile_sum[b] = 0.f;
+      }
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int n = 0; n < FRAGMENTS * QB; ++n) {
+        const int f = n / QB, b = n % QB;
+        if (b == 0 && f + READ_AHEAD < FRAGMENTS)
+          kf[f + READ_AHEAD] = *(const bf16x8*)(kt + ((f + READ_AHEAD) / DS) * 512 + ((f + READ_AHEAD) % DS) * 64);
+        next[b][f / DS] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[f], qf[b][f % DS], next[b][f / DS], 0, 0, 0);
+        const int wb = n / 8, wh = (n / 4) % 2, wi = n % 4;      // the n-th weight of the lane
+        weight[n] = fast_exp2(fmaf(sc[wb][wh][wi], scale2, shift[wb]));
+        tile_sum[wb] += weight[n];
+        if (n % 2 == 1) {
+          pf[wb][wh * 4 + wi - 1] = (bf16)weight[n - 1];
+          pf[wb][wh * 4 + wi] = (bf16)weight[n];
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      bool again = false;
+#pragma unroll
+      for (int b = 0; b < QB; ++b) again |= !(tile_sum[b] <= 0x1p60f);   // too large, infinite or not a number
+      if (__any(again)) return false;
+#pragma unroll
+      for (int b = 0; b < QB; ++b) run_sum[b] += tile_sum[b];
+      return true;
+    };
+    // values: O^T[dim, query] += V^T P
+    auto values = [&](int stage, const bf16x8 (&pf)[QB]) {
+      const unsigned char* vt = value_tiles + stage * VSTAGE + value_fragment;
+#pragma unroll
+      for (int e = 0; e < DB; ++e) {
+        const bf16x8 vv = *(const bf16x8*)(vt + e * 512);
+#pragma unroll
+        for (int b = 0; b < QB; ++b) o[b][e] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vv, pf[b], o[b][e], 0, 0, 0);
+      }
+    };
+
+    // Tiles [whole_begin, whole_end) need no mask: every query of the group sees every key of theirs.
+    int whole_begin = (lo_last + 31) / 32, whole_end = (pos_first + 1) / 32;
+    if (whole_begin < first_tile) whole_begin = first_tile;
+    if (whole_begin > last_tile + 1) whole_begin = last_tile + 1;
+    if (whole_end > last_tile + 1) whole_end = last_tile + 1;
+    if (whole_end < whole_begin) whole_end = whole_begin;
+
+    // The walk.  Keys and values of tile t lie in stage (t - first_tile) % 3 of their rings.  A turn works on
+    // tile t, whose scores the turn before has left in registers: it asks memory for the keys of t + 3 (their
+    // stage was last read a turn ago, for the scores of t) and the values of t + 2 (likewise), computes the
+    // scores of t + 1 beside the weights of t, adds the values of t, and before the barrier waits until only
+    // what it asked for itself is still on its way: the keys of t + 2 and the values of t + 1 are then in LDS.
+    __syncthreads();                                           // the stages of an earlier pass are done with
+    floatx4 sa[QB][2], sb[QB][2];
+    bf16x8 pf[QB];
+    int pages_ahead[2];                                        // the pages of tile + 3 at the top of a turn
+    const char* values_ahead[2];                               // where the values of tile + 2 lie
+    if (first_tile <= last_tile) {
+      int pages[2];
+      const char *kbase[2], *vbase[2];
+      pages_of(std::false_type{}, first_tile, pages);
+      locate(std::false_type{}, first_tile, pages, kbase, vbase);
+      fetch_keys(kbase, 0);
+      fetch_values(vbase, 0);
+      pages_of(std::false_type{}, first_tile + 1, pages);
+      locate(std::false_type{}, first_tile + 1, pages, kbase, values_ahead);
+      if (first_tile + 1 <= last_tile) fetch_keys(kbase, 1);
+      int pending = 0;
+      pages_of(std::false_type{}, first_tile + 2, pages);
+      locate(std::false_type{}, first_tile + 2, pages, kbase, vbase);
+      if (first_tile + 2 <= last_tile) fetch_keys(kbase, 2), pending += 2;
+      if (first_tile + 1 <= last_tile) fetch_values(values_ahead, 1), pending += 2;
+      values_ahead[0] = vbase[0], values_ahead[1] = vbase[1];
+      pages_of(std::false_type{}, first_tile + 3, pages_ahead);
+      if (pending == 4) fetched_then_barrier<4>();
+      else if (pending == 2) fetched_then_barrier<2>();
+      else fetched_then_barrier<0>();
+      scores(0, sa);
+      asm volatile("s_barrier" ::: "memory");                  // everyone has read the first keys: their stage may be filled again
+    }
+    int tile = first_tile, stage = 0;                          // stage = (tile - first_tile) % 3
+    // the turn's fetches, and how many they are; EVERY: tile + 3 is not past the last, so all of them happen
+    auto ask_ahead = [&](auto every) -> int {
+      constexpr bool EVERY = decltype(every)::value;
+      int pending = 0;
+      const char *kbase[2], *vbase[2];
+      locate(std::true_type{}, tile + 3, pages_ahead, kbase, vbase);
+      if (EVERY || tile + 3 <= last_tile) fetch_keys(kbase, stage), pending += 2;
+      if (EVERY || tile + 2 <= last_tile) fetch_values(values_ahead, stage == 0 ? STAGES - 1 : stage - 1), pending += 2;
+      values_ahead[0] = vbase[0], values_ahead[1] = vbase[1];
+      pages_of(std::true_type{}, tile + 4, pages_ahead);        // wanted a turn from now
+      return pending;
+    };
+    auto turn_over = [&](int pending) {
+      if (pending == 4) fetched_then_barrier<4>();
+      else if (pending == 2) fetched_then_barrier<2>();
+      else fetched_then_barrier<0>();
+      stage = stage == STAGES - 1 ? 0 : stage + 1;
+      ++tile;
+    };
+    // Most turns take the short way and have three tiles behind them: the inner loop holds only those, with
+    // every count fixed, so that nothing in it touches the accumulators but the matrix products.  A tile
+    // that needs the mask, or whose weights came out too large, or one of the last three, leaves it and takes
+    // the long way.  The scores of the tile at hand are in sa at the top of every turn.
+    const int fast_begin = whole_begin, fast_end = whole_end < last_tile - 2 ? whole_end : last_tile - 2;
+    for (;;) {
+      bool asked = false;                                      // the turn's fetches have been asked for already
+      // one way out of the inner loop only, at its top, before anything of the turn has happened to the accumulators
+      for (;;) {
+        if (asked || tile < fast_begin || tile >= fast_end) break;
+        ask_ahead(std::true_type{});
+        if (!weights_beside_scores(stage == STAGES - 1 ? 0 : stage + 1, sa, sb, pf)) {
+          asked = true;
+          continue;
+        }
+        values(stage, pf);
+        turn_over(4);
+#pragma unroll
+        for (int b = 0; b < QB; ++b) sa[b][0] = sb[b][0], sa[b][1] = sb[b][1];
+      }
+      const bool unfinished = tile <= last_tile;
+      if (!unfinished) break;
+      const int pending = asked ? 4 : ask_ahead(std::false_type{});
+      if (tile < last_tile) scores(stage == STAGES - 1 ? 0 : stage + 1, sb);
+      if (tile >= whole_begin && tile < whole_end) weights_with_maximum(tile, sa, std::false_type{}, pf);
+      else weights_with_maximum(tile, sa, std::true_type{}, pf);
+      values(stage, pf);
+      turn_over(pending);
+#pragma unroll
+      for (int b = 0; b < QB; ++b) sa[b][0] = sb[b][0], sa[b][1] = sb[b][1];
+    }
+#pragma unroll
+    for (int b = 0; b < QB; ++b) {
+      float total = run_sum[b];
+      total += __shfl_xor(total, 16, WAVE);
+      total += __shfl_xor(total, 32, WAVE);
+      if (live[b] && splits > 1) {
+        const int64_t slot = ((int64_t)(token0 + b * 16 + col) * nq + head) * splits + split;
+#pragma unroll
+        for (int e = 0; e < DB; ++e) *(floatx4*)(part_o + slot * D + e * 16 + g * 4) = o[b][e];
+        if (g == 0) {
+          part_ml[slot * 2] = run_max[b] * scale2;               // -inf stays -inf: no key seen
+          part_ml[slot * 2 + 1] = total;
+        }
+      } else if (live[b]) {
+        const float inv = 1.0f / total;
+        bf16* dst = out + (int64_t)(token0 + b * 16 + col) * out_stride + (int64_t)head * D + g * 4;
+#pragma unroll
+        for (int e = 0; e < DB; ++e) {
+          const bf16x4 packed = {(bf16)(o[b][e][0] * inv), (bf16)(o[b][e][1] * inv), (bf16)(o[b][e][2] * inv), (bf16)(o[b][e][3] * inv)};
+          *(bf16x4*)(dst + e * 16) = packed;
+        }
+      }
+    }
+  }
+}
+
 // Compute units of the current device (asked once).
 static int compute_units() {
   static int units = 0;
@@ -890,7 +1284,8 @@ LRS_API int lrs_attention_prefill(void* out, int out_stride, const void* q, int 
   LRS_REQUIRE(max_context >= 1, "attention_prefill: max_context must be the longest context length of the step");
   const int span = window > 0 && window + 32 + 64 < max_context ? window + 32 + 64 : max_context;
   const size_t table_lds = sizeof(int) * (size_t)(span / page_size + 2);
-  LRS_REQUIRE(table_lds <= 24 * 1024, "attention_prefill: a context of %d tokens needs more block table entries than fit LDS", max_context);
+  // (the kernel for heads of 128 reads the block table with scalar loads and keeps no copy)
+  LRS_REQUIRE(d == 128 || table_lds <= 24 * 1024, "attention_prefill: a context of %d tokens needs more block table entries than fit LDS", max_context);
   hipStream_t s = (hipStream_t)stream;
 #define LAUNCH2(D, QB)                                                                                               \
   attention_prefill_bf16_kernel<D, QB><<<grid, block, table_lds, s>>>((bf16*)out, out_stride, (const bf16*)q, q_stride, \
@@ -905,7 +1300,17 @@ LRS_API int lrs_attention_prefill(void* out, int out_stride, const void* q, int 
     case 32: LAUNCH(32); break;
     case 64: LAUNCH(64); break;
     case 96: LAUNCH(96); break;
-    case 128: LAUNCH(128); break;
+    case 128:
+      // head size 128 has a kernel of its own, whose tiles go from memory straight into LDS
+      if (max_count <= 16)
+        attention_prefill_d128_bf16_kernel<1><<<grid, block, 0, s>>>(
+            (bf16*)out, out_stride, (const bf16*)q, q_stride, (const bf16*)k_pages, (const bf16*)v_pages, block_table, table_stride,
+            token_request, positions, qblock_token0, qblock_count, n_blocks, chunk, nq, nkv, page_size, scale, window, splits, part_o, part_ml);
+      else
+        attention_prefill_d128_bf16_kernel<2><<<grid, block, 0, s>>>(
+            (bf16*)out, out_stride, (const bf16*)q, q_stride, (const bf16*)k_pages, (const bf16*)v_pages, block_table, table_stride,
+            token_request, positions, qblock_token0, qblock_count, n_blocks, chunk, nq, nkv, page_size, scale, window, splits, part_o, part_ml);
+      break;
     case 192: LAUNCH(192); break;
     default: return lrs_fail("attention_prefill: head_dim %d has no matrix-core kernel (32, 64, 96, 128, 192)", d);
   }
