@@ -866,19 +866,6 @@ __global__ __launch_bounds__(256, D <= 128 ? 2 : 1) void attention_prefill_bf16_
 // The wave that fetched a tile waits for its own fetches (vmcnt) before the barrier that opens the
 // tile to the others; the fetches of the tile after it stay in flight.  The fetches are written in
 // assembly because the compiler would wait for all of them before any LDS read it cannot tell apart.
-__device__ __forceinline__ void fetch_to_lds(const void* base, unsigned lane_offset, unsigned lds_address) {
-  const unsigned lo = __builtin_amdgcn_readfirstlane((unsigned)(uintptr_t)base);
-  const unsigned hi = __builtin_amdgcn_readfirstlane((unsigned)((uintptr_t)base >> 32));
-  const unsigned long long uniform_base = ((unsigned long long)hi << 32) | lo;
-  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
-               :: "s"(__builtin_amdgcn_readfirstlane(lds_address)), "v"(lane_offset), "s"(uniform_base) : "memory");
-}
-// Waits until at most `pending` of this wave's fetches are still on their way, then for the workgroup.
-template <int PENDING>
-__device__ __forceinline__ void fetched_then_barrier() {
-  asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" :: "n"(PENDING) : "memory");
-}
-
 template <int QB>
 __global__ __launch_bounds__(256, 2) void attention_prefill_d128_bf16_kernel(
     bf16* __restrict__ out, int out_stride, const bf16* __restrict__ q, int q_stride,

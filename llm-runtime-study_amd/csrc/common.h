@@ -68,3 +68,22 @@ __device__ __forceinline__ float block_max(float v, float* scratch) {
   for (int i = 0; i < waves; ++i) total = fmaxf(total, scratch[i]);
   return total;
 }
+
+// Memory straight into LDS (global_load_lds_dwordx4): lane l of the wave fetches the 16 bytes at
+// base + lane_offset (base the same for the whole wave) and they land at LDS byte address lds_address +
+// 16 l; nothing passes through registers and the wave goes on at once.  The compiler does not know these
+// fetches: whoever reads the LDS they fill waits for them with fetched_then_barrier (they finish in the
+// order they were asked for, and count in vmcnt).  LDS that only they write must still be named as an
+// address here, which is what tells the compiler that its contents change.
+__device__ __forceinline__ void fetch_to_lds(const void* base, unsigned lane_offset, unsigned lds_address) {
+  const unsigned lo = __builtin_amdgcn_readfirstlane((unsigned)(uintptr_t)base);
+  const unsigned hi = __builtin_amdgcn_readfirstlane((unsigned)((uintptr_t)base >> 32));
+  const unsigned long long uniform_base = ((unsigned long long)hi << 32) | lo;
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+               :: "s"(__builtin_amdgcn_readfirstlane(lds_address)), "v"(lane_offset), "s"(uniform_base) : "memory");
+}
+// Waits until at most `PENDING` of this wave's fetches are still on their way, then for the workgroup.
+template <int PENDING>
+__device__ __forceinline__ void fetched_then_barrier() {
+  asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" :: "n"(PENDING) : "memory");
+}

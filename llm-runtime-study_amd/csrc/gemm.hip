@@ -159,17 +159,17 @@ __global__ __launch_bounds__(256) void gemm_bf16_mfma_kernel(void* __restrict__ 
 // ------------------------------------------------- bf16 MFMA kernel for many rows
 // 128 tokens x 256 weight rows per workgroup of four waves (2 x 2: a wave owns 64 tokens x 128 weight
 // rows as 4 x 8 tiles of the 16x16x32 product), K walked in slices of 32.  Both operands pass through
-// LDS (two buffers, one barrier a slice); a slice is asked from memory three slices before it is
-// multiplied and waits in registers meanwhile (two register sets in turn), and two
-// workgroups share a compute unit, so a trip to memory has several slices' worth of matrix
-// instructions to hide behind.  Every fragment a wave reads from LDS feeds four or eight matrix
-// instructions.  Workgroups are numbered so that the 32 that share an XCD (and its L2) cover 4 x 8
-// tiles.  Needs K % 32 == 0, 16-byte aligned rows, no bias and matrices of fewer than 2^31 elements
-// (the 128 x 128 kernel above takes what this one does not).
-// What bounds it (measured at 2,048 x 24,576 x 4,096, 469 us): without the loads from memory inside the
-// loop 348 us, without the writes into LDS as well 252 us; the LDS moves about 64 bytes a cycle and unit
-// and a slice needs 72 KB of it per workgroup (48 KB of fragment reads, 24 KB of writes).  Weights
-// straight from memory into registers (only activations through LDS, 40 KB) were slower: 513 us.
+// LDS, and memory writes them there itself (fetch_to_lds: no staging registers, no LDS write
+// instructions): three stages of 24 KB, the slice two ahead asked for before a slice is multiplied, one
+// barrier a slice, before which a wave waits for its own six fetches of the next slice.  Two workgroups
+// share a compute unit.  Every fragment a wave reads from LDS feeds four or eight matrix instructions.
+// Workgroups are numbered so that the 32 that share an XCD (and its L2) cover 4 x 8 tiles.  Needs
+// K % 32 == 0, 16-byte aligned rows, no bias and matrices of fewer than 2^31 elements (the 128 x 128
+// kernel above takes what this one does not).
+// Before, a slice went through registers (asked for three slices ahead) and was written to LDS by the
+// waves; measured then at 2,048 x 24,576 x 4,096: 469 us, without the loads from memory inside the loop
+// 348 us, without the writes into LDS as well 252 us.  Weights straight from memory into registers (only
+// activations through LDS) were slower: 513 us.
 // Accumulator layout: weight row 4 * (lane / 16) + i, token lane % 16, i.e. four consecutive output
 // columns of one token per lane.
 constexpr int WIDE_BK = 32;   // measured on MI355X at 2,048 rows: slices of 32 (two workgroups a compute unit) beat slices of 64 (one) by a fifth
@@ -177,11 +177,11 @@ template <bool SWIGLU, int MODE>
 __global__ __launch_bounds__(256, 2) void gemm_bf16_wide_kernel(void* __restrict__ out, const bf16* __restrict__ x,
                                                                 const bf16* __restrict__ w, int m, int n, int k, int lda,
                                                                 int ldc, int tiles_m, int tiles_n) {
-  constexpr int BM = 128, BN = 256, BK = WIDE_BK;
-  constexpr int XL = BM * 4 / 256, WL = BN * 4 / 256;        // 16-byte pieces of a slice per thread: 2 of x, 4 of w
-  __shared__ __attribute__((aligned(16))) bf16 xs[2][BM * BK];
-  __shared__ __attribute__((aligned(16))) bf16 ws[2][BN * BK];
-  const int tid = threadIdx.x, lane = tid % WAVE, wave = tid / WAVE;
+  constexpr int BM = 128, BN = 256, BK = WIDE_BK, STAGES = 3;
+  constexpr int XL = BM / 16 / 4, WL = BN / 16 / 4;           // blocks of 16 rows (1,024 bytes of a slice) per wave: 2 of x, 4 of w
+  constexpr int STAGE_ELEMENTS = (BM + BN) * BK;
+  __shared__ __attribute__((aligned(64))) bf16 slices[STAGES * STAGE_ELEMENTS];   // a stage: the tokens' slice, then the weights'
+  const int tid = threadIdx.x, lane = tid % WAVE, wave = __builtin_amdgcn_readfirstlane(tid / WAVE);
   const int r = lane & 15, g = lane >> 4;
   int id = blockIdx.x;
   const int tiles = tiles_m * tiles_n;
@@ -190,74 +190,71 @@ __global__ __launch_bounds__(256, 2) void gemm_bf16_wide_kernel(void* __restrict
   const int band_rows = tiles_m - band * 4 < 4 ? tiles_m - band * 4 : 4;
   const int m0 = (band * 4 + within % band_rows) * BM, n0 = (within / band_rows) * BN;
   const int wm = (wave >> 1) * 64, wn = (wave & 1) * 128;           // this wave's corner inside the tile
-  // piece i of a slice for this thread: row tid / 4 + 64 * i, k chunk tid % 4 (4 lanes read one row's 64
-  // bytes of the slice).  Rows past the matrix are read from its last row (and never written), slices
-  // past K are read from the last slice (and not multiplied): no load in the loop is conditional.
-  const int prow = tid / 4;
-  int xoff[XL], woff[WL];
-#pragma unroll
-  for (int i = 0; i < XL; ++i) xoff[i] = (m0 + prow + 64 * i < m ? m0 + prow + 64 * i : m - 1) * lda + (tid % 4) * 8;
-#pragma unroll
-  for (int i = 0; i < WL; ++i) woff[i] = (n0 + prow + 64 * i < n ? n0 + prow + 64 * i : n - 1) * k + (tid % 4) * 8;
-  // Where chunk c (8 k) of tile row q lies in a buffer: rows are 64 bytes, half a line of banks, packed
+  // Where chunk c (8 k) of tile row q lies in a stage: rows are 64 bytes, half a line of banks, packed
   // without padding; rows swap places in pairs in the upper half of every 16 and chunks are turned
-  // round by the row number, so that the rows 0..7, 8..15, the even and the odd rows of a fragment
-  // each touch every bank once (measured: no bank conflicts; with rows 80 bytes apart every second
-  // LDS cycle was one).  Element ((q ^ (q >> 3 & 1)) * 4 + (c ^ (q >> 1 & 3))) * 8; only the low four
-  // bits of q enter the swaps, so a tile row 16 * j + q lies 16 * j * 32 elements further on.
-  const int spot = ((prow ^ ((prow >> 3) & 1)) * 4 + ((tid % 4) ^ ((prow >> 1) & 3))) * 8;   // where this thread's pieces go
-  const int frag = ((r ^ ((r >> 3) & 1)) * 4 + (g ^ ((r >> 1) & 3))) * 8;                    // where its fragments come from
+  // round by the row number, so that the lanes LDS serves together (eight consecutive rows of a fragment,
+  // chunks g and g + 1) each touch every bank once.  Element ((q ^ (q >> 3 & 1)) * 4 + (c ^ (q >> 1 & 3))) * 8;
+  // only the low four bits of q enter the swaps, so a tile row 16 * j + q lies 16 * j * 32 elements further on.
+  // A block of 16 rows is one fetch of one wave, whose lane l fills place l: it asks for the row and chunk
+  // that belong there.  Rows past the matrix are read from its last row (and never written), slices past K
+  // from the last slice (and not multiplied): no fetch in the loop is conditional.
+  const int place_row = (lane >> 2) ^ ((lane >> 5) & 1);            // the row whose piece lies at place l = row' * 4 + chunk'
+  const int place_chunk = (lane & 3) ^ ((place_row >> 1) & 3);
+  unsigned xoff[XL], woff[WL];                                      // bytes from the matrix's first element
+#pragma unroll
+  for (int i = 0; i < XL; ++i) {
+    const int row = m0 + 16 * (wave + 4 * i) + place_row;
+    xoff[i] = (unsigned)(((row < m ? row : m - 1) * lda + place_chunk * 8) * 2);
+  }
+#pragma unroll
+  for (int i = 0; i < WL; ++i) {
+    const int row = n0 + 16 * (wave + 4 * i) + place_row;
+    woff[i] = (unsigned)(((row < n ? row : n - 1) * k + place_chunk * 8) * 2);
+  }
+  const int frag = ((r ^ ((r >> 3) & 1)) * 4 + (g ^ ((r >> 1) & 3))) * 8;                    // where this lane's fragments come from
   floatx4 acc[8][4];
 #pragma unroll
   for (int it = 0; it < 8; ++it)
 #pragma unroll
     for (int jt = 0; jt < 4; ++jt) acc[it][jt] = floatx4{0.f, 0.f, 0.f, 0.f};
   const int steps = k / BK;
-  auto fetch = [&](int kt, bf16x8 (&xr)[XL], bf16x8 (&wr)[WL]) {
-    const int at = (kt < steps ? kt : steps - 1) * BK;
+  const unsigned slices_address = (unsigned)(uintptr_t)(__attribute__((address_space(3))) bf16*)slices;
+  auto fetch = [&](int kt, int stage) {                             // six fetches a wave
+    const int at = (kt < steps ? kt : steps - 1) * BK * 2;
+    const unsigned to = slices_address + (unsigned)(stage * STAGE_ELEMENTS * 2 + wave * 1024);
 #pragma unroll
-    for (int i = 0; i < XL; ++i) xr[i] = *(const bf16x8*)(x + xoff[i] + at);
+    for (int i = 0; i < XL; ++i) fetch_to_lds((const char*)x + at, xoff[i], to + (unsigned)(i * 4096));
 #pragma unroll
-    for (int i = 0; i < WL; ++i) wr[i] = *(const bf16x8*)(w + woff[i] + at);
+    for (int i = 0; i < WL; ++i) fetch_to_lds((const char*)w + at, woff[i], to + (unsigned)(BM * BK * 2 + i * 4096));
   };
-  auto stash = [&](int buffer, const bf16x8 (&xr)[XL], const bf16x8 (&wr)[WL]) {
-#pragma unroll
-    for (int i = 0; i < XL; ++i) *(bf16x8*)(xs[buffer] + spot + 64 * i * BK) = xr[i];
-#pragma unroll
-    for (int i = 0; i < WL; ++i) *(bf16x8*)(ws[buffer] + spot + 64 * i * BK) = wr[i];
-  };
-  auto multiply = [&](int buffer) {
+  auto multiply = [&](int stage) {
+    const bf16* xs = slices + stage * STAGE_ELEMENTS;
+    const bf16* ws = xs + BM * BK;
     bf16x8 xf[4];
 #pragma unroll
-    for (int jt = 0; jt < 4; ++jt) xf[jt] = *(const bf16x8*)(xs[buffer] + frag + (wm + jt * 16) * BK);
+    for (int jt = 0; jt < 4; ++jt) xf[jt] = *(const bf16x8*)(xs + frag + (wm + jt * 16) * BK);
 #pragma unroll
     for (int it = 0; it < 8; ++it) {
-      const bf16x8 wf = *(const bf16x8*)(ws[buffer] + frag + (wn + it * 16) * BK);
+      const bf16x8 wf = *(const bf16x8*)(ws + frag + (wn + it * 16) * BK);
 #pragma unroll
       for (int jt = 0; jt < 4; ++jt) acc[it][jt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf, xf[jt], acc[it][jt], 0, 0, 0);
     }
   };
-  // Slice kt is multiplied from buffer kt % 2 while slice kt + 1 goes from registers into the other
-  // buffer and slice kt + 3 is asked for from memory (two register sets in turn): the writes and the
-  // requests are issued before the slice's matrix instructions and run beside them.
+  // Slice kt is multiplied from stage kt % 3 while slice kt + 1 arrives and slice kt + 2 is asked for (into
+  // the stage that slice kt - 1 was multiplied from a barrier ago).  Before the barrier a wave waits until only
+  // the six fetches it has just asked for are still on their way: slice kt + 1 is then in LDS.
   int m0_opaque = m0;
-  bf16x8 xa[XL], wa[WL], xb[XL], wb[WL];
-  fetch(0, xa, wa);
-  fetch(1, xb, wb);
-  stash(0, xa, wa);
-  fetch(2, xa, wa);
-  __syncthreads();
-  for (int kt = 0; kt < steps; kt += 2) {
-    stash(1, xb, wb);                  // slice kt + 1
-    fetch(kt + 3, xb, wb);
-    multiply(0);                       // slice kt
-    __syncthreads();
-    if (kt + 1 >= steps) break;
-    stash(0, xa, wa);                  // slice kt + 2
-    fetch(kt + 4, xa, wa);
-    multiply(1);                       // slice kt + 1
-    __syncthreads();
+  fetch(0, 0);
+  fetch(1, 1);
+  fetched_then_barrier<6>();
+  int stage = 0;
+  for (int kt = 0; kt < steps; ++kt) {
+    fetch(kt + 2, stage == 0 ? 2 : stage - 1);
+    multiply(stage);
+    fetched_then_barrier<6>();
+    stage = stage == STAGES - 1 ? 0 : stage + 1;
   }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");               // the fetches past K that nobody reads
   // nothing of the epilogue's addresses may be worked out (and kept in registers) before the loop above ends
   asm volatile("" : "+s"(ldc), "+s"(m0_opaque));
   // jt outside: one token row's address is worked out once and its 8 pieces of 4 columns follow 16 apart;
