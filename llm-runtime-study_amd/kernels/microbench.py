@@ -5,6 +5,8 @@
     python -m llm_runtime_study_amd.kernels.microbench attention_decode --batch 1,8,64 --context 2048 --splits 1,4,8
     python -m llm_runtime_study_amd.kernels.microbench gemm --rows 1,8,16,64,2048
     python -m llm_runtime_study_amd.kernels.microbench memory
+    python -m llm_runtime_study_amd.kernels.microbench lds          # LDS read rate by the distance between a fragment's rows
+    python -m llm_runtime_study_amd.kernels.microbench mfma         # matrix instructions with vector work beside them
 
 Head and matrix shapes default to those of Qwen3-8B and can be changed with options.  Weights and
 caches larger than the last-level cache are rotated between calls where a kernel streams them once
@@ -138,9 +140,31 @@ def memory(args) -> None:
         del buffers
 
 
+def lds(args) -> None:
+    """16-byte LDS reads in the shape of a matrix-core fragment (a lane's row is lane % 16, its piece lane / 16)
+    for every distance between rows: what the layout of a tile in LDS has to respect."""
+    units, iters = ops.compute_units(), 4096
+    sink = torch.zeros(256, dtype=torch.int32, device="cuda")
+    for stride in range(64, 321, 16):
+        seconds = _time(lambda i: ops.probe_lds(sink, 2 * units, iters, stride), 5)
+        per_cycle = 2 * 256 * iters * 8 * 16 / seconds / 2.4e9
+        print(f"lds rows {stride:3d} bytes apart: {seconds * 1e3:7.3f} ms  {per_cycle:6.1f} bytes a cycle and compute unit (at 2.4 GHz)", flush=True)
+
+
+def mfma(args) -> None:
+    """What the matrix cores sustain alone and with vector instructions of the same wave between the products."""
+    units, iters = ops.compute_units(), 4000
+    sink = torch.zeros(256, dtype=torch.float32, device="cuda")
+    for valu, exps in ((0, False), (1, False), (2, False), (3, False), (4, False), (6, False), (2, True), (3, True)):
+        seconds = _time(lambda i: ops.probe_mfma(sink, 8 * units, iters, valu, exps), 3)
+        rate = 8 * units * 4 * iters * 32 * 16384 / seconds / 1e12
+        print(f"mfma 16x16x32 bf16 with {valu} multiply-adds after each{' and an exponential after every second' if exps else ''}: "
+              f"{seconds * 1e3:7.3f} ms  {rate:7.1f} TFLOP/s", flush=True)
+
+
 def main(argv=None) -> int:
     parser = argparse.ArgumentParser(prog="python -m llm_runtime_study_amd.kernels.microbench", description=__doc__.split("\n\n")[0])
-    parser.add_argument("kernel", choices=["attention_prefill", "attention_decode", "gemm", "memory"])
+    parser.add_argument("kernel", choices=["attention_prefill", "attention_decode", "gemm", "memory", "lds", "mfma"])
     parser.add_argument("--heads", type=int, default=32)
     parser.add_argument("--kv-heads", type=int, default=8)
     parser.add_argument("--head-dim", type=int, default=128)
@@ -168,7 +192,7 @@ def main(argv=None) -> int:
         print("microbench needs the GPU", file=sys.stderr)
         return 2
     ops.library()
-    {"attention_prefill": attention_prefill, "attention_decode": attention_decode, "gemm": gemm, "memory": memory}[args.kernel](args)
+    {"attention_prefill": attention_prefill, "attention_decode": attention_decode, "gemm": gemm, "memory": memory, "lds": lds, "mfma": mfma}[args.kernel](args)
     return 0
 
 

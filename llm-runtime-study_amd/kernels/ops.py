@@ -92,6 +92,8 @@ _SIGNATURES = {
     "lrs_advance_slots": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p, c_int, c_void_p]),
     "lrs_copy_to_pinned": (c_int, [c_void_p, c_void_p, c_int64, c_void_p]),
     "lrs_stream_read": (c_int, [c_void_p, c_int64, c_void_p, c_int, c_void_p]),
+    "lrs_probe_lds": (c_int, [c_void_p, c_int, c_int, c_int, c_void_p]),
+    "lrs_probe_mfma": (c_int, [c_void_p, c_int, c_int, c_int, c_int, c_void_p]),
     "lrs_gemm_prepare": (c_int, []),
     "lrs_library_gemm_prepare": (c_int, []),
     "lrs_library_gemm": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p]),
@@ -314,6 +316,18 @@ def stream_read(src: torch.Tensor, sink: torch.Tensor, blocks: int) -> None:
     _need(src.is_contiguous() and sink.dtype == torch.int32 and sink.numel() >= blocks, "stream_read: contiguous source and an int32 sink of `blocks` elements")
     _launch("lrs_stream_read", _dev(src, "src"), src.numel() * src.element_size(), _dev(sink, "sink"), blocks, _stream())
 
+
+
+def probe_lds(sink: torch.Tensor, blocks: int, iters: int, stride: int) -> None:
+    """`blocks` workgroups read LDS `iters` x 8 times, 16 bytes a lane, rows `stride` bytes apart (microbench lds)."""
+    _need(sink.dtype == torch.int32 and sink.numel() >= 256, "probe_lds: an int32 sink of 256 elements")
+    _launch("lrs_probe_lds", _dev(sink, "sink"), blocks, iters, stride, _stream())
+
+
+def probe_mfma(sink: torch.Tensor, blocks: int, iters: int, valu: int, exps: bool) -> None:
+    """`blocks` workgroups issue `iters` x 32 matrix instructions with `valu` multiply-adds after each (microbench mfma)."""
+    _need(sink.dtype == torch.float32 and sink.numel() >= 256, "probe_mfma: a float32 sink of 256 elements")
+    _launch("lrs_probe_mfma", _dev(sink, "sink"), blocks, iters, valu, int(bool(exps)), _stream())
 
 def copy_to_pinned(dst: torch.Tensor, src: torch.Tensor, count: int) -> None:
     """The first `count` elements of device `src` into pinned host `dst`, by a kernel (the host reads

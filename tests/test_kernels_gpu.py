@@ -894,3 +894,22 @@ def test_filter_logits_matches_sort_based_rule(ops):
         kept = torch.isfinite(want)
         torch.testing.assert_close(got[i][kept], logits[i][kept], rtol=0, atol=0)
     assert torch.isfinite(got[1]).sum() == 2
+
+
+@pytest.mark.gpu
+def test_the_probes_of_lds_and_matrix_rates_run_and_refuse_what_they_cannot_do(ops):
+    """`microbench lds` and `microbench mfma` are measurements, not products: here only that they launch,
+    finish and refuse parameters outside what their kernels hold."""
+    from llm_runtime_study_amd.errors import KernelError
+
+    ints = torch.zeros(256, dtype=torch.int32, device="cuda")
+    floats = torch.zeros(256, dtype=torch.float32, device="cuda")
+    ops.probe_lds(ints, 8, 4, 96)
+    ops.probe_mfma(floats, 8, 4, 2, True)
+    ops.probe_mfma(floats, 8, 4, 0, False)
+    torch.cuda.synchronize()
+    for bad in (8, 100, 1024):
+        with pytest.raises(KernelError):
+            ops.probe_lds(ints, 8, 4, bad)
+    with pytest.raises(KernelError):
+        ops.probe_mfma(floats, 8, 4, 5, False)
