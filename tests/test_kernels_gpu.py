@@ -548,6 +548,9 @@ def _attention_reference(q, k_all, v_all, positions, lengths_before, nq, nkv, d,
 @pytest.mark.parametrize("nq,nkv,d,page,window", [
     (4, 2, 16, 4, 0), (8, 2, 32, 16, 0), (3, 1, 48, 8, 0), (6, 3, 80, 16, 0), (32, 8, 128, 16, 0),
     (4, 4, 256, 64, 0), (8, 2, 32, 16, 7), (4, 2, 64, 16, 33), (16, 1, 96, 32, 0), (12, 4, 192, 16, 21),
+    # heads of 128 have a kernel of their own for ragged steps: pages of several runs of 16 keys, kv groups of
+    # more heads than a workgroup has waves (several passes) and of fewer, windows
+    (8, 1, 128, 32, 0), (6, 2, 128, 64, 40), (16, 1, 128, 16, 21), (2, 2, 128, 48, 0), (5, 1, 128, 16, 70),
 ])
 def test_attention_ragged_batch(ops, dtype, nq, nkv, d, page, window):
     g = torch.Generator().manual_seed(6)
@@ -768,7 +771,13 @@ def test_one_key_stands_out_in_every_attention_kernel(ops, window, planted):
     it (595 with a window of 100: positions 690..694 yes, 695..699 no; 599: only 690..698) and a kernel
     that is one off at the window's edge returns a different row.  All kernels: the general one, the
     matrix-core decode kernel (last token; whole and split over keys) and the ragged prefill kernel."""
-    nq, nkv, d, page, before, new = 4, 2, 64, 16, 690, 10
+    run_one_key_stands_out(ops, window, planted, 64, 16)
+    run_one_key_stands_out(ops, window, planted, 128, 16)      # heads of 128: the ragged kernel is another one
+    run_one_key_stands_out(ops, window, planted, 128, 32)
+
+
+def run_one_key_stands_out(ops, window, planted, d, page):
+    nq, nkv, before, new = 4, 2, 690, 10
     length = before + new
     g = torch.Generator().manual_seed(70 + planted)
     k = (torch.randn(length, nkv, d, generator=g) * 0.1).bfloat16()
