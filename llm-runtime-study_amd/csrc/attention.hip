@@ -430,18 +430,34 @@ __global__ void attention_merge_kernel(bf16* __restrict__ out, int out_stride, c
                                        const float* __restrict__ part_ml, int nq, int d, int splits) {
   const int token = blockIdx.x, head = blockIdx.y;
   const int64_t base = ((int64_t)token * nq + head) * splits;
-  float top = -INFINITY;
-  for (int s = 0; s < splits; ++s) top = fmaxf(top, part_ml[(base + s) * 2]);
-  float total = 0.f;
-  for (int s = 0; s < splits; ++s) {
-    const float m = part_ml[(base + s) * 2];
-    if (m > -INFINITY) total += part_ml[(base + s) * 2 + 1] * fast_exp2(m - top);
-  }
+  // Everything is asked for before anything is used: the partial sums of a split do not wait for its maximum
+  // (a split that saw no key holds zeros and gets the weight zero), so the kernel is one trip to memory long.
+  constexpr int AT_ONCE = 8;
   for (int dim = threadIdx.x; dim < d; dim += blockDim.x) {
-    float acc = 0.f;
-    for (int s = 0; s < splits; ++s) {
-      const float m = part_ml[(base + s) * 2];
-      if (m > -INFINITY) acc += part_o[(base + s) * d + dim] * fast_exp2(m - top);
+    float top = -INFINITY, total = 0.f, acc = 0.f;
+    for (int s0 = 0; s0 < splits; s0 += AT_ONCE) {
+      float m[AT_ONCE], l[AT_ONCE], o[AT_ONCE];
+#pragma unroll
+      for (int i = 0; i < AT_ONCE; ++i) {
+        const int s = s0 + i < splits ? s0 + i : splits - 1;
+        m[i] = part_ml[(base + s) * 2];
+        l[i] = part_ml[(base + s) * 2 + 1];
+        o[i] = part_o[(base + s) * d + dim];
+      }
+      float chunk_top = top;
+#pragma unroll
+      for (int i = 0; i < AT_ONCE; ++i)
+        if (s0 + i < splits) chunk_top = fmaxf(chunk_top, m[i]);
+      const float keep = top == -INFINITY ? 0.f : fast_exp2(top - chunk_top);   // what was added up so far, against the new maximum
+      total *= keep;
+      acc *= keep;
+      top = chunk_top;
+#pragma unroll
+      for (int i = 0; i < AT_ONCE; ++i) {
+        const float weight = (s0 + i < splits && m[i] > -INFINITY) ? fast_exp2(m[i] - top) : 0.f;
+        total += l[i] * weight;
+        acc += o[i] * weight;
+      }
     }
     out[(int64_t)token * out_stride + (int64_t)head * d + dim] = (bf16)(acc / total);
   }
