@@ -293,6 +293,135 @@ __global__ __launch_bounds__(256, 2) void gemm_bf16_wide_kernel(void* __restrict
   }
 }
 
+// ------------------------------------------ bf16 MFMA kernel for many rows, slices of whole lines
+// 256 tokens x BN weight rows per workgroup of eight waves, K walked in slices of 64, one workgroup a
+// compute unit.  BN = 256 (2 x 4 waves: a wave owns 128 tokens x 64 weight rows as 8 x 4 tiles of the
+// 16x16x32 product; two stages of 64 KB), BN = 192 (2 x 4 waves of 128 x 48; two stages of 56 KB) or
+// BN = 128 (4 x 2 waves of 64 x 64; three stages of 48 KB): whichever leaves the compute units the least
+// idle in the launch's last round (6,144 columns are 256 tiles of 192, one a unit).  Against the kernel above: a
+// slice holds whole 128-byte lines of every row, so a fetch touches 8 lines instead of 16 halves (the address
+// units in front of the L1 were busy 62 % of that kernel's time), and at BN = 256 a third less traffic from
+// memory per product.  The slice after next (BN = 128) or the next (BN = 256) is asked for before a slice
+// is multiplied.  K % 64 == 0; the kernel above takes the rest.
+// Where chunk c (8 k, 16 bytes) of tile row q lies in a stage: rows are 128 bytes, eight to a block of
+// 1,024 bytes (one fetch of one wave, whose lane l fills place l), and the chunks of a row are turned round
+// by twice (q / 2) % 4, so that the lanes LDS serves together (eight consecutive rows, chunks g and g + 1)
+// meet every bank once: place (q % 8) * 8 + (c ^ ((q >> 1 & 3) << 1)) of block q / 8.
+template <int BN, bool SWIGLU, int MODE>
+__global__ __launch_bounds__(512, 1) void gemm_bf16_lines_kernel(void* __restrict__ out, const bf16* __restrict__ x,
+                                                                 const bf16* __restrict__ w, int m, int n, int k, int lda,
+                                                                 int ldc, int tiles_m, int tiles_n) {
+  static_assert(BN == 256 || BN == 192 || BN == 128, "256, 192 or 128 weight rows a workgroup");
+  constexpr int BM = 256, BK = 64, STAGES = BN == 128 ? 3 : 2;
+  constexpr int WAVES_N = BN == 128 ? 2 : 4;                   // waves side by side along the weight rows
+  constexpr int IT = BN / WAVES_N / 16, JT = BM / (8 / WAVES_N) / 16;   // a wave's tiles: 4 x 8, 3 x 8 or 4 x 4
+  constexpr int XL = BM / 8 / 8, WL = BN / 8 / 8;             // blocks of 8 rows per wave: 4 of x, 4, 3 or 2 of w
+  constexpr int PENDING = STAGES == 2 ? 0 : XL + WL;          // fetches that may still be on their way at a barrier
+  constexpr int STAGE_ELEMENTS = (BM + BN) * BK;
+  __shared__ __attribute__((aligned(64))) bf16 slices[STAGES * STAGE_ELEMENTS];
+  const int tid = threadIdx.x, lane = tid % WAVE, wave = __builtin_amdgcn_readfirstlane(tid / WAVE);
+  const int r = lane & 15, g = lane >> 4;
+  int id = blockIdx.x;
+  const int tiles = tiles_m * tiles_n;
+  if (tiles % 8 == 0) id = (id % 8) * (tiles / 8) + id / 8;        // consecutive workgroups go to different XCDs
+  const int band = id / (4 * tiles_n), within = id % (4 * tiles_n);
+  const int band_rows = tiles_m - band * 4 < 4 ? tiles_m - band * 4 : 4;
+  const int m0 = (band * 4 + within % band_rows) * BM, n0 = (within / band_rows) * BN;
+  const int wm = (wave / WAVES_N) * (JT * 16), wn = (wave % WAVES_N) * (IT * 16);   // this wave's corner inside the tile
+  const int place_row = lane >> 3;                                  // the row whose piece lies at place l of a block
+  const int place_chunk = (lane & 7) ^ (((place_row >> 1) & 3) << 1);
+  unsigned xoff[XL], woff[WL];                                      // bytes from the matrix's first element
+#pragma unroll
+  for (int i = 0; i < XL; ++i) {
+    const int row = m0 + 8 * (wave + 8 * i) + place_row;
+    xoff[i] = (unsigned)(((row < m ? row : m - 1) * lda + place_chunk * 8) * 2);
+  }
+#pragma unroll
+  for (int i = 0; i < WL; ++i) {
+    const int row = n0 + 8 * (wave + 8 * i) + place_row;
+    woff[i] = (unsigned)(((row < n ? row : n - 1) * k + place_chunk * 8) * 2);
+  }
+  // this lane's fragment of rows 16 j .. 16 j + 15, k half c: row r, chunk 4 c + g
+  const int frag_row = (r >> 3) * 512 + (r & 7) * 64;               // elements; + 16 j * 64
+  const int turn = ((r >> 1) & 3) << 1;
+  const int frag0 = frag_row + ((g ^ turn) * 8), frag1 = frag_row + (((4 + g) ^ turn) * 8);
+  floatx4 acc[IT][JT];
+#pragma unroll
+  for (int it = 0; it < IT; ++it)
+#pragma unroll
+    for (int jt = 0; jt < JT; ++jt) acc[it][jt] = floatx4{0.f, 0.f, 0.f, 0.f};
+  const int steps = k / BK;
+  const unsigned slices_address = (unsigned)(uintptr_t)(__attribute__((address_space(3))) bf16*)slices;
+  auto fetch = [&](int kt, int stage) {                             // XL + WL fetches a wave
+    const int at = (kt < steps ? kt : steps - 1) * BK * 2;
+    const unsigned to = slices_address + (unsigned)(stage * STAGE_ELEMENTS * 2 + wave * 1024);
+#pragma unroll
+    for (int i = 0; i < XL; ++i) fetch_to_lds((const char*)x + at, xoff[i], to + (unsigned)(i * 8192));
+#pragma unroll
+    for (int i = 0; i < WL; ++i) fetch_to_lds((const char*)w + at, woff[i], to + (unsigned)(BM * BK * 2 + i * 8192));
+  };
+  auto multiply = [&](int stage) {
+    const bf16* xs = slices + stage * STAGE_ELEMENTS;
+    const bf16* ws = xs + BM * BK;
+#pragma unroll
+    for (int c = 0; c < 2; ++c) {
+      const int frag = c ? frag1 : frag0;
+      bf16x8 xf[JT];
+#pragma unroll
+      for (int jt = 0; jt < JT; ++jt) xf[jt] = *(const bf16x8*)(xs + frag + (wm + jt * 16) * BK);
+#pragma unroll
+      for (int it = 0; it < IT; ++it) {
+        const bf16x8 wf = *(const bf16x8*)(ws + frag + (wn + it * 16) * BK);
+#pragma unroll
+        for (int jt = 0; jt < JT; ++jt) acc[it][jt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf, xf[jt], acc[it][jt], 0, 0, 0);
+      }
+    }
+  };
+  // Slice kt is multiplied from stage kt % STAGES while the slices after it arrive; a stage is filled again a
+  // barrier after it was last read.  Before the barrier a wave waits until only the fetches it asked for in
+  // this turn (none, with two stages) are still on their way: the next slice is then in LDS.
+  int m0_opaque = m0;
+  fetch(0, 0);
+  if (STAGES == 3) fetch(1, 1);
+  fetched_then_barrier<PENDING>();
+  int stage = 0;
+  for (int kt = 0; kt < steps; ++kt) {
+    fetch(kt + STAGES - 1, stage == 0 ? STAGES - 1 : stage - 1);
+    multiply(stage);
+    fetched_then_barrier<PENDING>();
+    stage = stage == STAGES - 1 ? 0 : stage + 1;
+  }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");               // the fetches past K that nobody reads
+  asm volatile("" : "+s"(ldc), "+s"(m0_opaque));
+#pragma unroll
+  for (int jt = 0; jt < JT; ++jt) {
+    const int token = m0_opaque + wm + jt * 16 + r;
+    const int64_t row_at = (int64_t)token * ldc;
+#pragma unroll
+    for (int it = 0; it < IT; ++it) {
+      const int tile0 = n0 + wn + it * 16, row0 = tile0 + 4 * g;     // this lane's four weight rows = output columns
+      if (SWIGLU) {
+        floatx4 up;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) up[i] = __shfl(acc[it][jt][i], (lane + 32) % WAVE, WAVE);
+        if (g < 2 && token < m && tile0 + 15 < n) {
+          const floatx4 gate = acc[it][jt];
+          const bf16x4 y = {(bf16)(silu(gate[0]) * up[0]), (bf16)(silu(gate[1]) * up[1]), (bf16)(silu(gate[2]) * up[2]), (bf16)(silu(gate[3]) * up[3])};
+          *(bf16x4*)((bf16*)out + row_at + tile0 / 2 + 4 * g) = y;
+        }
+      } else if (token < m && row0 < n) {
+        floatx4 v = acc[it][jt];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) v[i] = __shfl(v[i], lane, WAVE);    // as in the kernel above: keeps the loop free of spills
+        if constexpr (MODE == OUT_STORE) *(bf16x4*)((bf16*)out + row_at + row0) = bf16x4{(bf16)v[0], (bf16)v[1], (bf16)v[2], (bf16)v[3]};
+        else if constexpr (MODE == OUT_STORE_F32) *(floatx4*)((float*)out + row_at + row0) = v;
+        else *(floatx4*)((float*)out + row_at + row0) = *(const floatx4*)((const float*)out + row_at + row0) + v;
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  }
+}
+
 // ------------------------------------------------- bf16 kernel for few rows
 // Decode-sized products (M <= 64): the weight matrix is streamed exactly once and the time
 // is the time to read it.  One workgroup owns 16 weight rows; its waves split K between them
@@ -1348,13 +1477,41 @@ LRS_API int lrs_gemm(void* out, int mode, const void* a, const void* w, const vo
       else launch_skinny_m<false, false>(out, mode, ap, norm, wp, bp, m, n, k, lda, ldc, s, tune);
     } else if (aligned && k % WIDE_BK == 0 && n % 4 == 0 && ldc % 4 == 0 && (uintptr_t)out % 16 == 0 && !bias &&
                (int64_t)m * lda < (1ll << 31) && (int64_t)n * k < (1ll << 31)) {
-      const int tiles_m = (m + 127) / 128, tiles_n = (n + 255) / 256;
+      // Slices of whole lines (K % 64 == 0), once there is a tile of 256 x 128 for every compute unit: the tile
+      // width (256, 192 or 128 weight rows) whose launch takes the fewest rounds of the chip times its width;
+      // the wider of two that tie (less traffic per product).
+      const int units = lrs_compute_units() > 0 ? lrs_compute_units() : 256;
+      const int big_m = (m + 255) / 256;
+      int width = 0, tiles_w = 0;
+      if (k % 64 == 0 && big_m * ((n + 127) / 128) >= units) {
+        int64_t best = 0;
+        for (int candidate : {256, 192, 128}) {
+          const int across = (n + candidate - 1) / candidate;
+          const int64_t cost = (int64_t)((big_m * across + units - 1) / units) * candidate;
+          if (!width || cost < best) width = candidate, tiles_w = across, best = cost;
+        }
+      }
+      if (width) {
+#define LINES(BN, SW, MODE) gemm_bf16_lines_kernel<BN, SW, MODE><<<big_m * tiles_w, 512, 0, s>>>(out, (const bf16*)a, (const bf16*)w, m, n, k, lda, ldc, big_m, tiles_w)
+#define LINES_OF(BN)                                            \
+        if (swiglu) LINES(BN, true, OUT_STORE);                 \
+        else if (mode == OUT_STORE) LINES(BN, false, OUT_STORE); \
+        else if (mode == OUT_STORE_F32) LINES(BN, false, OUT_STORE_F32); \
+        else LINES(BN, false, OUT_ADD_F32)
+        if (width == 256) { LINES_OF(256); }
+        else if (width == 192) { LINES_OF(192); }
+        else { LINES_OF(128); }
+#undef LINES_OF
+#undef LINES
+      } else {
+        const int tiles_m = (m + 127) / 128, tiles_n = (n + 255) / 256;
 #define WIDE(SW, MODE) gemm_bf16_wide_kernel<SW, MODE><<<tiles_m * tiles_n, 256, 0, s>>>(out, (const bf16*)a, (const bf16*)w, m, n, k, lda, ldc, tiles_m, tiles_n)
-      if (swiglu) WIDE(true, OUT_STORE);
-      else if (mode == OUT_STORE) WIDE(false, OUT_STORE);
-      else if (mode == OUT_STORE_F32) WIDE(false, OUT_STORE_F32);
-      else WIDE(false, OUT_ADD_F32);
+        if (swiglu) WIDE(true, OUT_STORE);
+        else if (mode == OUT_STORE) WIDE(false, OUT_STORE);
+        else if (mode == OUT_STORE_F32) WIDE(false, OUT_STORE_F32);
+        else WIDE(false, OUT_ADD_F32);
 #undef WIDE
+      }
     } else if (aligned) {
       dim3 grid((n + 127) / 128, (m + 127) / 128);
       if (swiglu)
