@@ -1433,6 +1433,24 @@ LRS_API int lrs_gemm_mid_qk_prep(void* qkv, int row_stride, const void* a, const
                                v_pages, slots, page_size, split_sums_buffer(), splits, stream);
 }
 
+// Which tile width the kernel for many rows with slices of whole lines would take for this product, or 0 if
+// it does not take it: K a multiple of 64 and a tile of 256 x 128 for every compute unit; then the width
+// (256, 192 or 128 weight rows) whose launch takes the fewest rounds of the chip times its width, the wider
+// of two that tie (less traffic per product).
+LRS_API int lrs_gemm_lines_width(int m, int n, int k) {
+  const int units = lrs_compute_units() > 0 ? lrs_compute_units() : 256;
+  const int big_m = (m + 255) / 256;
+  if (m <= 0 || n <= 0 || k <= 0 || k % 64 != 0 || big_m * ((n + 127) / 128) < units) return 0;
+  int width = 0;
+  int64_t best = 0;
+  for (int candidate : {256, 192, 128}) {
+    const int across = (n + candidate - 1) / candidate;
+    const int64_t cost = (int64_t)((big_m * across + units - 1) / units) * candidate;
+    if (!width || cost < best) width = candidate, best = cost;
+  }
+  return width;
+}
+
 // out [M, N] (row stride ldc) = a [M, K] (row stride lda) times w[N, K]^T.
 //   norm_weight != null: `a` is the float32 residual stream [*, K]; its rows (picked through
 //     `rows` if given) are RMS-normalised with norm_weight and eps on the way in.  bf16 weights,
@@ -1477,20 +1495,7 @@ LRS_API int lrs_gemm(void* out, int mode, const void* a, const void* w, const vo
       else launch_skinny_m<false, false>(out, mode, ap, norm, wp, bp, m, n, k, lda, ldc, s, tune);
     } else if (aligned && k % WIDE_BK == 0 && n % 4 == 0 && ldc % 4 == 0 && (uintptr_t)out % 16 == 0 && !bias &&
                (int64_t)m * lda < (1ll << 31) && (int64_t)n * k < (1ll << 31)) {
-      // Slices of whole lines (K % 64 == 0), once there is a tile of 256 x 128 for every compute unit: the tile
-      // width (256, 192 or 128 weight rows) whose launch takes the fewest rounds of the chip times its width;
-      // the wider of two that tie (less traffic per product).
-      const int units = lrs_compute_units() > 0 ? lrs_compute_units() : 256;
-      const int big_m = (m + 255) / 256;
-      int width = 0, tiles_w = 0;
-      if (k % 64 == 0 && big_m * ((n + 127) / 128) >= units) {
-        int64_t best = 0;
-        for (int candidate : {256, 192, 128}) {
-          const int across = (n + candidate - 1) / candidate;
-          const int64_t cost = (int64_t)((big_m * across + units - 1) / units) * candidate;
-          if (!width || cost < best) width = candidate, tiles_w = across, best = cost;
-        }
-      }
+      const int big_m = (m + 255) / 256, width = lrs_gemm_lines_width(m, n, k), tiles_w = width ? (n + width - 1) / width : 0;
       if (width) {
 #define LINES(BN, SW, MODE) gemm_bf16_lines_kernel<BN, SW, MODE><<<big_m * tiles_w, 512, 0, s>>>(out, (const bf16*)a, (const bf16*)w, m, n, k, lda, ldc, big_m, tiles_w)
 #define LINES_OF(BN)                                            \

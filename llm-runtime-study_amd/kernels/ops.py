@@ -8,6 +8,8 @@ the library is missing or cannot be built; there is no fallback.
 
 from __future__ import annotations
 
+import functools
+
 from dataclasses import dataclass
 import ctypes
 import struct
@@ -111,6 +113,7 @@ _SIGNATURES = {
                                       c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int,
                                       c_int, c_int, c_void_p, c_void_p, c_void_p]),
     "lrs_compute_units": (c_int, []),
+    "lrs_gemm_lines_width": (c_int, [c_int, c_int, c_int]),
     "lrs_attention_prefill_group": (c_int, []),
     "lrs_attention_prefill_group_for": (c_int, [c_int]),
     "lrs_choose_tokens": (c_int, [c_void_p, c_void_p, c_int64, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p]),
@@ -459,6 +462,13 @@ def add_into(residual: torch.Tensor, y: torch.Tensor) -> None:
     """residual (float32) += y, same shape, both contiguous."""
     _need(residual.dtype == torch.float32 and residual.shape == y.shape and residual.is_contiguous() and y.is_contiguous(), "add_into: float32 residual and y of one contiguous shape needed")
     _launch("lrs_add_into", _dev(residual, "residual"), _dev(y, "y"), dtype_code(y.dtype), residual.numel(), _stream())
+
+
+@functools.lru_cache(maxsize=4096)
+def gemm_lines_width(m: int, n: int, k: int) -> int:
+    """The tile width (256, 192 or 128 weight rows) the many-rows kernel with slices of whole lines would take
+    for out [m, n] = x [m, k] w[n, k]^T, or 0 if that kernel does not take the product."""
+    return int(library().lrs_gemm_lines_width(m, n, k))
 
 
 def few_rows_capacity() -> int:

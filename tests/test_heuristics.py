@@ -156,3 +156,19 @@ def test_a_plan_packs_one_word_per_argument():
     assert words[:5] == [ops.PLAN_OPS.index("lrs_add_into"), 0x7F0000001000, 0x7F0000002000, 1, 1 << 33]
     assert words[5] == ops.PLAN_OPS.index("lrs_scale_rows") and words[12] == 0x3F000000        # 0.5 as its 32 bits
     assert words[13:] == [ops.PLAN_OPS.index("lrs_fill_i32"), 0, (1 << 64) - 7, 12]               # None: a null pointer; -7: two's complement
+
+
+def test_the_tile_width_of_the_many_rows_kernel_follows_the_rounds_of_the_chip():
+    """`lrs_gemm_lines_width`: K a multiple of 64 and a 256 x 128 tile for every compute unit, then the width
+    that needs the fewest rounds times its width (the shapes of the 8B layer at 2,048 rows: one round each)."""
+    from llm_runtime_study_amd.kernels import ops
+
+    if ops.compute_units() not in (0, 256):
+        return
+    assert ops.gemm_lines_width(2048, 24576, 4096) == 256      # 768 tiles: three rounds
+    assert ops.gemm_lines_width(2048, 6144, 4096) == 192       # 256 tiles of 192: one round
+    assert ops.gemm_lines_width(2048, 4096, 12288) == 128      # 256 tiles of 128
+    assert ops.gemm_lines_width(8192, 4096, 4096) == 256       # 512 tiles: two rounds of 256 tie with four of 128
+    assert ops.gemm_lines_width(1024, 4096, 4096) == 0         # not a tile for every compute unit
+    assert ops.gemm_lines_width(2048, 4096, 4000) == 0         # K no multiple of 64
+    assert ops.gemm_lines_width(129, 151936, 4096) == 256      # the LM head of a small step
