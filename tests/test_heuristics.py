@@ -171,4 +171,4 @@ def test_the_tile_width_of_the_many_rows_kernel_follows_the_rounds_of_the_chip()
     assert ops.gemm_lines_width(8192, 4096, 4096) == 256       # 512 tiles: two rounds of 256 tie with four of 128
     assert ops.gemm_lines_width(1024, 4096, 4096) == 0         # not a tile for every compute unit
     assert ops.gemm_lines_width(2048, 4096, 4000) == 0         # K no multiple of 64
-    assert ops.gemm_lines_width(129, 151936, 4096) == 256      # the LM head of a small step
+    assert ops.gemm_lines_width(129, 151936, 4096) == 128      # the LM head of a small step: five rounds of 128 against three of 256
