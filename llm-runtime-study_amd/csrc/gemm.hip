@@ -310,7 +310,7 @@ __global__ __launch_bounds__(256, 2) void gemm_bf16_wide_kernel(void* __restrict
 template <int BN, bool SWIGLU, int MODE>
 __global__ __launch_bounds__(512, 1) void gemm_bf16_lines_kernel(void* __restrict__ out, const bf16* __restrict__ x,
                                                                  const bf16* __restrict__ w, int m, int n, int k, int lda,
-                                                                 int ldc, int tiles_m, int tiles_n) {
+                                                                 int ldc, int tiles_m, int tiles_n, int splits) {
   static_assert(BN == 256 || BN == 192 || BN == 128, "256, 192 or 128 weight rows a workgroup");
   constexpr int BM = 256, BK = 64, STAGES = BN == 128 ? 3 : 2;
   constexpr int WAVES_N = BN == 128 ? 2 : 4;                   // waves side by side along the weight rows
@@ -321,8 +321,9 @@ __global__ __launch_bounds__(512, 1) void gemm_bf16_lines_kernel(void* __restric
   __shared__ __attribute__((aligned(64))) bf16 slices[STAGES * STAGE_ELEMENTS];
   const int tid = threadIdx.x, lane = tid % WAVE, wave = __builtin_amdgcn_readfirstlane(tid / WAVE);
   const int r = lane & 15, g = lane >> 4;
-  int id = blockIdx.x;
   const int tiles = tiles_m * tiles_n;
+  const int split = blockIdx.x / tiles;                            // which part of K (the launch is tiles x splits)
+  int id = blockIdx.x - split * tiles;
   if (tiles % 8 == 0) id = (id % 8) * (tiles / 8) + id / 8;        // consecutive workgroups go to different XCDs
   const int band = id / (4 * tiles_n), within = id % (4 * tiles_n);
   const int band_rows = tiles_m - band * 4 < 4 ? tiles_m - band * 4 : 4;
@@ -350,10 +351,13 @@ __global__ __launch_bounds__(512, 1) void gemm_bf16_lines_kernel(void* __restric
   for (int it = 0; it < IT; ++it)
 #pragma unroll
     for (int jt = 0; jt < JT; ++jt) acc[it][jt] = floatx4{0.f, 0.f, 0.f, 0.f};
-  const int steps = k / BK;
+  // with K divided between workgroups, this one walks the slices step0 .. step0 + steps - 1 and leaves its sums
+  // in part `split` of out [splits, m, ldc]
+  const int steps_of_k = k / BK, steps_each = (steps_of_k + splits - 1) / splits, step0 = split * steps_each;
+  const int steps = steps_of_k - step0 < steps_each ? steps_of_k - step0 : steps_each;
   const unsigned slices_address = (unsigned)(uintptr_t)(__attribute__((address_space(3))) bf16*)slices;
   auto fetch = [&](int kt, int stage) {                             // XL + WL fetches a wave
-    const int at = (kt < steps ? kt : steps - 1) * BK * 2;
+    const int at = (step0 + (kt < steps ? kt : steps - 1)) * BK * 2;
     const unsigned to = slices_address + (unsigned)(stage * STAGE_ELEMENTS * 2 + wave * 1024);
 #pragma unroll
     for (int i = 0; i < XL; ++i) fetch_to_lds((const char*)x + at, xoff[i], to + (unsigned)(i * 8192));
@@ -396,7 +400,7 @@ __global__ __launch_bounds__(512, 1) void gemm_bf16_lines_kernel(void* __restric
 #pragma unroll
   for (int jt = 0; jt < JT; ++jt) {
     const int token = m0_opaque + wm + jt * 16 + r;
-    const int64_t row_at = (int64_t)token * ldc;
+    const int64_t row_at = ((int64_t)split * m + token) * ldc;
 #pragma unroll
     for (int it = 0; it < IT; ++it) {
       const int tile0 = n0 + wn + it * 16, row0 = tile0 + 4 * g;     // this lane's four weight rows = output columns
@@ -1451,6 +1455,37 @@ LRS_API int lrs_gemm_lines_width(int m, int n, int k) {
   return width;
 }
 
+// Into how many parts that kernel divides K for a product with too few tiles of 256 x 128 to go round the
+// compute units, or 0 if it does not take the product that way (then lrs_gemm_lines_width says whether it takes
+// it whole): the number of parts, from 1 (just the tiles, if they fill half the units) to 8, that fills the
+// units best in one round, every part with 8 slices of 64 or more, and the parts' sums within the split buffer.
+LRS_API int lrs_gemm_lines_splits(int m, int n, int k) {
+  const int units = lrs_compute_units() > 0 ? lrs_compute_units() : 256;
+  if (m <= 128 || n <= 0 || k <= 0 || k % 64 != 0) return 0;
+  const int tiles = ((m + 255) / 256) * ((n + 127) / 128), steps = k / 64;
+  if (tiles >= units) return 0;
+  int splits = 0;
+  for (int parts = 1; parts <= 8 && tiles * parts <= units; ++parts) {
+    const int each = (steps + parts - 1) / parts;
+    if (parts > 1 && (each < 8 || (parts - 1) * each >= steps || (size_t)parts * m * n * sizeof(float) > SPLIT_SUMS_BYTES)) continue;
+    splits = parts;
+  }
+  return splits && 2 * tiles * splits >= units ? splits : 0;
+}
+
+// Whether that divided form is the faster way for a product that could also go to the vendor library.  Measured
+// on MI355X at 256..1024 rows with the layer sizes of the 8B and 14B models, against the library's first choice:
+// products with a long K (the feed-forward's second: K three times N or more) take 0.4 to 0.9 of the library's
+// time at every such row count (14B at 512 rows: 102 against 171 us; 8B: 61 against 82); square and wide ones only
+// up to 256 rows, when every part still has 12 slices (14B q/k/v 41 against 54 us, o_proj 35 against 49; with 8
+// slices a part, 8B o_proj, 31 against 23).  Elsewhere the library is as fast or faster.
+LRS_API int lrs_gemm_lines_split_pays(int m, int n, int k) {
+  const int splits = lrs_gemm_lines_splits(m, n, k);
+  if (splits < 1 || n % 4 != 0) return 0;
+  if (k >= 2 * n) return 1;
+  return m <= 256 && splits >= 2 && (k / 64 + splits - 1) / splits >= 12;
+}
+
 // out [M, N] (row stride ldc) = a [M, K] (row stride lda) times w[N, K]^T.
 //   norm_weight != null: `a` is the float32 residual stream [*, K]; its rows (picked through
 //     `rows` if given) are RMS-normalised with norm_weight and eps on the way in.  bf16 weights,
@@ -1495,14 +1530,26 @@ LRS_API int lrs_gemm(void* out, int mode, const void* a, const void* w, const vo
       else launch_skinny_m<false, false>(out, mode, ap, norm, wp, bp, m, n, k, lda, ldc, s, tune);
     } else if (aligned && k % WIDE_BK == 0 && n % 4 == 0 && ldc % 4 == 0 && (uintptr_t)out % 16 == 0 && !bias &&
                (int64_t)m * lda < (1ll << 31) && (int64_t)n * k < (1ll << 31)) {
-      const int big_m = (m + 255) / 256, width = lrs_gemm_lines_width(m, n, k), tiles_w = width ? (n + width - 1) / width : 0;
-      if (width) {
-#define LINES(BN, SW, MODE) gemm_bf16_lines_kernel<BN, SW, MODE><<<big_m * tiles_w, 512, 0, s>>>(out, (const bf16*)a, (const bf16*)w, m, n, k, lda, ldc, big_m, tiles_w)
-#define LINES_OF(BN)                                            \
-        if (swiglu) LINES(BN, true, OUT_STORE);                 \
-        else if (mode == OUT_STORE) LINES(BN, false, OUT_STORE); \
-        else if (mode == OUT_STORE_F32) LINES(BN, false, OUT_STORE_F32); \
-        else LINES(BN, false, OUT_ADD_F32)
+      const int big_m = (m + 255) / 256, splits = lrs_gemm_lines_splits(m, n, k);
+      const int width = splits ? 128 : lrs_gemm_lines_width(m, n, k), tiles_w = width ? (n + width - 1) / width : 0;
+#define LINES(BN, SW, MODE, OUT, LDC, SPLITS) \
+  gemm_bf16_lines_kernel<BN, SW, MODE><<<big_m * tiles_w * SPLITS, 512, 0, s>>>(OUT, (const bf16*)a, (const bf16*)w, m, n, k, lda, LDC, big_m, tiles_w, SPLITS)
+      if (splits > 1) {
+        // K divided between workgroups: their sums go to the split buffer, and the kernel that adds them up
+        // writes the output with the epilogue that was asked for
+        float* sums = split_sums_buffer();
+        LRS_REQUIRE(sums != nullptr, "gemm: no memory for the sums of %d K splits", splits);
+        LINES(128, false, OUT_STORE_F32, sums, n, splits);
+        const int64_t total = (int64_t)m * (swiglu ? n / 2 : n);
+        const int blocks = (int)((total + 1023) / 1024 < 2048 ? (total + 1023) / 1024 : 2048);
+        if (swiglu) gemm_split_finish_kernel<true><<<blocks, 256, 0, s>>>(out, mode, sums, nullptr, m, n, ldc, splits);
+        else gemm_split_finish_kernel<false><<<blocks, 256, 0, s>>>(out, mode, sums, nullptr, m, n, ldc, splits);
+      } else if (width) {
+#define LINES_OF(BN)                                                           \
+        if (swiglu) LINES(BN, true, OUT_STORE, out, ldc, 1);                    \
+        else if (mode == OUT_STORE) LINES(BN, false, OUT_STORE, out, ldc, 1);   \
+        else if (mode == OUT_STORE_F32) LINES(BN, false, OUT_STORE_F32, out, ldc, 1); \
+        else LINES(BN, false, OUT_ADD_F32, out, ldc, 1)
         if (width == 256) { LINES_OF(256); }
         else if (width == 192) { LINES_OF(192); }
         else { LINES_OF(128); }

@@ -114,6 +114,8 @@ _SIGNATURES = {
                                       c_int, c_int, c_void_p, c_void_p, c_void_p]),
     "lrs_compute_units": (c_int, []),
     "lrs_gemm_lines_width": (c_int, [c_int, c_int, c_int]),
+    "lrs_gemm_lines_splits": (c_int, [c_int, c_int, c_int]),
+    "lrs_gemm_lines_split_pays": (c_int, [c_int, c_int, c_int]),
     "lrs_attention_prefill_group": (c_int, []),
     "lrs_attention_prefill_group_for": (c_int, [c_int]),
     "lrs_choose_tokens": (c_int, [c_void_p, c_void_p, c_int64, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p]),
@@ -469,6 +471,21 @@ def gemm_lines_width(m: int, n: int, k: int) -> int:
     """The tile width (256, 192 or 128 weight rows) the many-rows kernel with slices of whole lines would take
     for out [m, n] = x [m, k] w[n, k]^T, or 0 if that kernel does not take the product."""
     return int(library().lrs_gemm_lines_width(m, n, k))
+
+
+@functools.lru_cache(maxsize=4096)
+def gemm_lines_splits(m: int, n: int, k: int) -> int:
+    """Into how many parts the many-rows kernel with slices of whole lines divides K for a product with too few
+    tiles of 256 x 128 to go round the compute units (1: the tiles as they are), or 0 if it does not take the
+    product that way."""
+    return int(library().lrs_gemm_lines_splits(m, n, k))
+
+
+@functools.lru_cache(maxsize=4096)
+def gemm_split_pays(m: int, n: int, k: int) -> bool:
+    """Whether a bfloat16 product of more than 128 rows is faster by this package's many-rows kernel with K divided
+    between workgroups than by the vendor library (a rule from measurements, see `lrs_gemm_lines_split_pays`)."""
+    return bool(library().lrs_gemm_lines_split_pays(m, n, k))
 
 
 def few_rows_capacity() -> int:

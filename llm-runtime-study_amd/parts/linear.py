@@ -110,6 +110,8 @@ def plan(m: int, n: int, k: int, *, weight_dtype: torch.dtype, run_dtype: torch.
         return ("mid_begin" if follows and out_contiguous else "mid"), first
     if (choice.library and bf16 and m > choice.few_rows_max and not bias and contiguous
             and (accumulate or (stores and out_contiguous))):
+        if m > 128 and out_contiguous and ops.gemm_split_pays(m, n, k):
+            return "own", first            # too few tiles for the chip and a long K: divided between workgroups here
         return "library", first
     return "own", first
 

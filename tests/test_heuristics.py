@@ -78,6 +78,7 @@ def test_the_route_of_a_product_follows_rows_dtype_and_the_runners_choices():
     choices a runner carries move it; nothing in the process does."""
     import torch
 
+    from llm_runtime_study_amd.kernels import ops
     from llm_runtime_study_amd.kernels.ops import KernelChoice
     from llm_runtime_study_amd.parts.linear import ROUTES, plan
 
@@ -115,6 +116,15 @@ def test_the_route_of_a_product_follows_rows_dtype_and_the_runners_choices():
     assert route(2048, 4096, 4096, contiguous=False) == ("own", "")
     assert route(2048, 24576, 4096, swiglu=True, choice=KernelChoice(library=False)) == ("own", "")
     assert route(129, 4096, 4096) == ("library", "") and route(128, 4096, 4096) == ("mid", "")
+    # a prompt portion of a few hundred rows: too few tiles for the chip; with a long K (or up to 256 rows) this
+    # package's kernel with K divided between workgroups, else the library
+    if ops.compute_units() in (0, 256):
+        assert route(512, 5120, 17408, out=f32, accumulate=True, norm_follows=5120) == ("own", "")
+        assert route(512, 4096, 12288, out=f32, accumulate=True, norm_follows=4096) == ("own", "")
+        assert route(256, 7168, 5120) == ("own", "") and route(512, 7168, 5120) == ("library", "")
+        assert route(512, 4096, 4096, out=f32, accumulate=True, norm_follows=4096) == ("library", "")
+        assert route(512, 34816, 5120, swiglu=True) == ("library", "")
+        assert route(512, 4096, 12288, out=f32, accumulate=True, out_contiguous=False) == ("library", "")
     # float32 runs: this package's own kernels whatever the rows
     for m in (1, 8, 64, 2048):
         assert route(m, 4096, 4096, dtype=f32, out=f32) == ("own", "")
@@ -172,3 +182,16 @@ def test_the_tile_width_of_the_many_rows_kernel_follows_the_rounds_of_the_chip()
     assert ops.gemm_lines_width(1024, 4096, 4096) == 0         # not a tile for every compute unit
     assert ops.gemm_lines_width(2048, 4096, 4000) == 0         # K no multiple of 64
     assert ops.gemm_lines_width(129, 151936, 4096) == 128      # the LM head of a small step: five rounds of 128 against three of 256
+    # too few tiles for the chip: K in as many parts as fill it in one round, each with 8 slices of 64 or more
+    assert ops.gemm_lines_splits(512, 4096, 4096) == 4         # 64 tiles x 4
+    assert ops.gemm_lines_splits(512, 5120, 17408) == 3        # 80 tiles x 3 = 240
+    assert ops.gemm_lines_splits(512, 7168, 5120) == 2         # 112 tiles x 2
+    assert ops.gemm_lines_splits(300, 9000, 1088) == 1         # 142 tiles, more than half the units: as they are
+    assert ops.gemm_lines_splits(512, 4096, 512) == 0          # one part of 8 slices, 64 tiles: under half the units
+    assert ops.gemm_lines_splits(2048, 4096, 4096) == 0        # a tile for every unit: not divided
+    assert ops.gemm_lines_splits(128, 4096, 4096) == 0         # the kernel for 17..128 rows' size
+    # ... and where that form is taken instead of the vendor library: a long K at any such row count, others up to 256 rows
+    assert ops.gemm_split_pays(512, 5120, 17408) and ops.gemm_split_pays(1024, 4096, 12288) and ops.gemm_split_pays(300, 4096, 12288)
+    assert ops.gemm_split_pays(256, 5120, 5120) and not ops.gemm_split_pays(512, 5120, 5120)
+    assert not ops.gemm_split_pays(256, 4096, 4096)            # 8 parts of 8 slices: too short
+    assert not ops.gemm_split_pays(2048, 4096, 12288) and not ops.gemm_split_pays(512, 34816, 5120)

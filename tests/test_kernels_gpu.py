@@ -263,6 +263,7 @@ def test_add_into(ops, dtype):
     (2000, 16648, 192), (2048, 16384, 64),               # many rows and wide, K a multiple of 64: the kernel of 256 x 256 tiles, ragged edges
     (2000, 4232, 192), (2048, 4096, 64),                 # ... and less wide: its form of 256 x 128 tiles
     (2000, 6100, 192), (2048, 6144, 64),                 # ... and 256 tiles of 256 x 192
+    (512, 4096, 2048), (520, 4232, 2048), (300, 9000, 1088),   # too few 256 x 128 tiles for the chip: K divided between workgroups (4, 2 and 1 parts)
 ])
 @pytest.mark.parametrize("mode", ["store", "store_f32", "add"])
 def test_gemm(ops, dtype, m, n, k, mode):
@@ -429,7 +430,8 @@ def test_gemm_with_fused_rmsnorm_input(ops, w_dtype, m, n, k, all_rows_in_own_ke
 
 @pytest.mark.parametrize("m,inter,k", [(1, 128, 64), (9, 160, 96), (64, 12288, 4096), (65, 160, 96), (300, 136, 264),
                                        (300, 392, 160), (2048, 1024, 512),       # K a multiple of 32 and more than 64 rows: the kernel of 128 x 256 tiles
-                                       (2040, 8200, 128), (2040, 2056, 128), (2040, 3072, 128)])    # wide enough for the kernel of 256 x 256 tiles, for its 256 x 128 and its 256 x 192 form
+                                       (2040, 8200, 128), (2040, 2056, 128), (2040, 3072, 128),     # wide enough for the kernel of 256 x 256 tiles, for its 256 x 128 and its 256 x 192 form
+                                       (500, 4104, 1024)])                       # K divided between workgroups of 256 x 128 tiles
 def test_gemm_with_swiglu_epilogue(ops, m, inter, k, all_rows_in_own_kernel):
     """Gate and up rows interleaved in groups of 8; the product writes silu(gate) * up."""
     g = torch.Generator().manual_seed(15)

@@ -51,7 +51,7 @@ def spec_and_weights(raw, seed, edit=None):
 class PartHarness:
     """A step context around one part: a runner whose model is never run."""
 
-    def __init__(self, needs, dtype, page_size=16):
+    def __init__(self, needs, dtype, page_size=16, max_step_tokens=256):
         from llm_runtime_study_amd.cache import CacheManager
         from llm_runtime_study_amd.engine.step import ModelRunner
 
@@ -59,8 +59,9 @@ class PartHarness:
             def graph_safe(self):
                 return False
 
-        self.cache = CacheManager(needs, page_size=page_size, num_pages=32, max_requests=4, max_seq_len=256, dtype=dtype, device="cuda")
-        self.runner = ModelRunner(NoModel(), self.cache, max_step_tokens=256, dtype=dtype, device="cuda")
+        self.cache = CacheManager(needs, page_size=page_size, num_pages=max(32, max_step_tokens // page_size + 1), max_requests=4,
+                                  max_seq_len=max_step_tokens, dtype=dtype, device="cuda")
+        self.runner = ModelRunner(NoModel(), self.cache, max_step_tokens=max_step_tokens, dtype=dtype, device="cuda")
 
     def context(self, entries):
         from llm_runtime_study_amd.engine.step import StepEntry
@@ -118,6 +119,33 @@ def test_swiglu_part_adds_into_the_residual(dtype):
     part.forward(ctx, x.cuda(), out)
     want = residual + plain.swiglu(x.float(), *(w[n].float() for n in ("gate_proj.weight", "up_proj.weight", "down_proj.weight")))
     close(out, want, dtype, bf16=1e-2)
+
+
+def test_swiglu_part_of_a_prompt_portion_divides_the_long_k_of_its_second_product():
+    """300 rows, 1,024 wide, 4,096 between: the second product has 16 tiles of 256 x 128 for 256 compute units and a
+    K four times its width, so it goes to this package's kernel with K in 8 parts (the first one to the library)."""
+    from llm_runtime_study_amd.kernels import ops
+    from llm_runtime_study_amd.parts import PartSpec, create
+    from llm_runtime_study_amd.parts.linear import plan
+
+    hidden, inter, rows = 1024, 4096, 300
+    if ops.compute_units() == 256:
+        assert ops.gemm_lines_splits(rows, hidden, inter) == 8
+        assert plan(rows, hidden, inter, weight_dtype=torch.bfloat16, run_dtype=torch.bfloat16, out_dtype=torch.float32,
+                    arrives="tensor", accumulate=True)[0] == "own"
+    part = create("feed_forward", PartSpec("swiglu", {"hidden_size": hidden, "intermediate_size": inter}))
+    g = torch.Generator().manual_seed(31)
+    w = {n: (torch.randn(s, generator=g) / math.sqrt(s[1])).to(torch.bfloat16) for n, s in
+         (("gate_proj.weight", (inter, hidden)), ("up_proj.weight", (inter, hidden)), ("down_proj.weight", (hidden, inter)))}
+    part.bind({k: v.cuda() for k, v in w.items()}, torch.bfloat16)
+    harness = PartHarness([], torch.bfloat16, max_step_tokens=512)
+    ctx = harness.context([(harness.cache.admit("a"), [1] * rows)])
+    x = torch.randn(rows, hidden, generator=g).to(torch.bfloat16)
+    residual = torch.randn(rows, hidden, generator=g)
+    out = residual.clone().cuda()
+    part.forward(ctx, x.cuda(), out)
+    want = residual + plain.swiglu(x.float(), *(w[n].float() for n in ("gate_proj.weight", "up_proj.weight", "down_proj.weight")))
+    close(out, want, torch.bfloat16, bf16=1e-2)
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
