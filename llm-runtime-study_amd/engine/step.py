@@ -106,6 +106,7 @@ class StepContext:
         self.qblock_token0 = self.qblock_count = None
         self.max_q = self.max_k = self.max_k_bound = 0
         self.all_decode = False
+        self.single_rows = 0          # a mixed step's leading requests that bring one token each (their tokens are its first rows)
         self.host_q_lens: list[int] = []
         self.host_slots: list[int] = []
         self.host_positions: list[int] = []   # first position of each request's tokens in this step
@@ -349,9 +350,14 @@ class ModelRunner:
             self._host_view("qblock_token0")[:cursor] = np.argsort(-pos[:cursor], kind="stable")
             self._host_view("qblock_count")[:cursor] = 1
         else:
-            starts, size = cu[:ctx.R + 1], min(self.query_group, ops.attention_prefill_group(cursor))
-            blocks = [(int(pos[min(t0 + size, int(starts[i + 1])) - 1]), t0, min(size, int(starts[i + 1]) - t0))
-                      for i in range(ctx.R) for t0 in range(int(starts[i]), int(starts[i + 1]), size)]
+            # The requests at the head of the step that bring one token each (a scheduler puts its decoding requests
+            # first) are left to the mixer as single rows, `single_rows` of them: the query groups cover the rows
+            # after them, and count their tokens from there.
+            singles = next(i for i, n in enumerate(ctx.host_q_lens) if n != 1)
+            ctx.single_rows = singles
+            starts, size = cu[:ctx.R + 1], min(self.query_group, ops.attention_prefill_group(cursor - singles))
+            blocks = [(int(pos[min(t0 + size, int(starts[i + 1])) - 1]), t0 - singles, min(size, int(starts[i + 1]) - t0))
+                      for i in range(singles, ctx.R) for t0 in range(int(starts[i]), int(starts[i + 1]), size)]
             blocks.sort(key=lambda b: -b[0])
             ctx.num_qblocks = len(blocks)
             ctx.max_qblock = max(b[2] for b in blocks)
@@ -420,9 +426,10 @@ class ModelRunner:
     def _plan_key(self, ctx: StepContext) -> tuple:
         """Everything the launches of a step depend on besides the contents of the metadata buffer: the numbers
         of tokens, requests, wanted rows and query groups (sizes and grids, and where the metadata arrays lie),
-        the largest query group, whether every request brings one token, and the two coarse measures of the
-        longest context that kernels size tables and choose key splits by."""
-        return (ctx.T, ctx.R, ctx.num_logit_rows, ctx.num_qblocks, ctx.max_qblock, ctx.all_decode, ctx.max_k_bound, length_class(ctx.max_k))
+        the largest query group, whether every request brings one token, how many at the head of a mixed step do,
+        and the two coarse measures of the longest context that kernels size tables and choose key splits by."""
+        return (ctx.T, ctx.R, ctx.num_logit_rows, ctx.num_qblocks, ctx.max_qblock, ctx.all_decode, ctx.single_rows, ctx.max_k_bound,
+                length_class(ctx.max_k))
 
     def _step_eager(self, ctx: StepContext) -> torch.Tensor | None:
         """The model on a prepared step, outside any graph: from a recorded plan if one fits, else through

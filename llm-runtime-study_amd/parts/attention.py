@@ -165,12 +165,27 @@ class GQAAttention(Part):
         elif ops.attention_decode_supported(ctx.dtype, nq, kv_heads, d, group.page_size):
             # sized by the step's coarse bound of the longest context, the same for every step of one shape
             longest = ctx.max_k_bound if self.window is None else min(ctx.max_k_bound, self.window + 64)
-            splits = self._prefill_splits(ctx.num_qblocks * kv_heads, longest, t * nq * d)
+            singles = ctx.single_rows
+            if singles:
+                # the single tokens at the head of a mixed step (decoding requests beside a prompt portion) go to the
+                # kernel of decode steps, which divides one token's keys between waves and workgroups; as rows of
+                # the other kernel each would walk its whole context in one workgroup
+                splits = self._decode_splits(singles * kv_heads, longest, ctx.max_k_bound, group.page_size)
+                part_o = part_ml = None
+                if splits > 1:
+                    part_o = ctx.scratch("attn_single_part_o", (singles, nq * splits * d), torch.float32)
+                    part_ml = ctx.scratch("attn_single_part_ml", (singles, nq * splits * 2), torch.float32)
+                ops.attention_decode(out[:singles], qkv[:singles], cache.k_pages, cache.v_pages, group.block_table, ctx.token_request,
+                                     ctx.positions, nq, self.scale, self.window or 0, splits, part_o, part_ml, ctx.max_k_bound, None, form=1)
+            rest = ctx.memo.get("rows_after_singles")
+            if rest is None:
+                rest = ctx.memo["rows_after_singles"] = (ctx.token_request[singles:], ctx.positions[singles:])
+            splits = self._prefill_splits(ctx.num_qblocks * kv_heads, longest, (t - singles) * nq * d)
             part_o = part_ml = None
             if splits > 1:
-                part_o = ctx.scratch("attn_part_o", (t, nq * splits * d), torch.float32)
-                part_ml = ctx.scratch("attn_part_ml", (t, nq * splits * 2), torch.float32)
-            ops.attention_prefill(out, qkv, cache.k_pages, cache.v_pages, group.block_table, ctx.token_request, ctx.positions,
+                part_o = ctx.scratch("attn_part_o", (t - singles, nq * splits * d), torch.float32)
+                part_ml = ctx.scratch("attn_part_ml", (t - singles, nq * splits * 2), torch.float32)
+            ops.attention_prefill(out[singles:], qkv[singles:], cache.k_pages, cache.v_pages, group.block_table, rest[0], rest[1],
                                   ctx.qblock_token0, ctx.qblock_count, nq, self.scale, self.window or 0, ctx.max_qblock, ctx.max_k_bound,
                                   splits, part_o, part_ml)
         else:

@@ -255,6 +255,49 @@ def test_whole_prompts_through_the_own_many_rows_product(folder_b, dtype, tmp_pa
     assert checked == 300 + 150 + 2 + 130
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_single_tokens_at_the_head_of_a_mixed_step_and_elsewhere_in_it(folder_b, dtype, tmp_path):
+    """Decoding requests beside a prompt portion: the single tokens that a step begins with go to the
+    attention kernel of decode steps, single tokens further back stay rows of the other kernel, and one
+    token that is a whole portion (a request's first) is a single token like any other.  Every asked row
+    against the plain implementation."""
+    from llm_runtime_study_amd.engine import trace
+
+    cfg, weights = plain.load_model_dir(folder_b, torch.float64)
+    rng = np.random.default_rng(21)
+    requests = {key: rng.integers(0, cfg["vocab_size"], n).tolist() for key, n in (("a", 45), ("b", 30), ("c", 64), ("d", 3))}
+    want = {key: plain.qwen3_forward(weights, cfg, ids) for key, ids in requests.items()}
+    a, b, c, d = (requests[key] for key in "abcd")
+
+    def entry(key, tokens, first):
+        return {"id": key, "tokens": tokens, "want": list(range(len(tokens)))}, [(key, first + i) for i in range(len(tokens))]
+
+    plan = [
+        [entry("a", a[:40], 0), entry("b", b[:25], 0)],
+        [entry("a", a[40:41], 40), entry("b", b[25:26], 25), entry("c", c[:50], 0), entry("d", d[:1], 0)],      # two at the head, one at the end
+        [entry("d", d[1:2], 1), entry("c", c[50:60], 50), entry("a", a[41:42], 41), entry("b", b[26:28], 26)],   # the head is a request's second token
+        [entry("b", b[28:29], 28), entry("a", a[42:43], 42), entry("d", d[2:3], 2), entry("c", c[60:64], 60)],   # three single tokens, then a portion
+    ]
+    steps = [{"step": i, "entries": [e for e, _ in row], "end": []} for i, row in enumerate(plan)]
+    runner = trace.make_runner(folder_b, dtype, 256)
+    out = tmp_path / "logits"
+    trace.replay(runner, traces.strip(steps).splitlines(), out, echo=lambda _: None)
+    checked = 0
+    for i, row in enumerate(plan):
+        got = torch.from_numpy(np.fromfile(out / f"{i}.f32", dtype="<f4").reshape(-1, cfg["vocab_size"]).copy())
+        places = [place for _, where in row for place in where]
+        assert got.shape[0] == len(places)
+        for logits, (key, position) in zip(got, places):
+            ref = want[key][position]
+            if dtype == "float32":
+                torch.testing.assert_close(logits.double(), ref, rtol=1e-4, atol=1e-4, msg=lambda m: f"step {i} {key}@{position}: {m}")
+            else:
+                err = (logits.double() - ref).norm() / ref.norm()
+                assert err < 3e-2, f"step {i} {key}@{position}: relative error {err:.3g}"
+            checked += 1
+    assert checked == 65 + 53 + 14 + 7
+
+
 # ------------------------------- one layer at the benchmark's sizes, against plain
 def test_one_layer_at_the_benchmark_sizes_against_the_plain_implementation():
     """Hidden 4096, 32 query and 8 kv heads of 128 dims, feed-forward 12288, vocabulary 151936, float32,
