@@ -809,6 +809,20 @@ template <bool SWIGLU>
 __global__ void gemm_split_finish_kernel(void* __restrict__ out, int mode, const float* __restrict__ split_sums,
                                          const bf16* __restrict__ bias, int m, int n, int ldc, int splits) {
   const int columns = SWIGLU ? n / 2 : n;
+  if (!SWIGLU && !bias && n % 4 == 0 && ldc % 4 == 0 && (uintptr_t)out % 16 == 0) {
+    // four columns a thread, 16 bytes a load
+    const int quads = n / 4;
+    for (int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; e < (int64_t)m * quads; e += (int64_t)gridDim.x * blockDim.x) {
+      const int token = e / quads, c = (e % quads) * 4;
+      floatx4 v = {0.f, 0.f, 0.f, 0.f};
+      for (int sp = 0; sp < splits; ++sp) v += *(const floatx4*)(split_sums + ((int64_t)sp * m + token) * n + c);
+      const int64_t at = (int64_t)token * ldc + c;
+      if (mode == OUT_STORE) *(bf16x4*)((bf16*)out + at) = bf16x4{(bf16)v[0], (bf16)v[1], (bf16)v[2], (bf16)v[3]};
+      else if (mode == OUT_STORE_F32) *(floatx4*)((float*)out + at) = v;
+      else *(floatx4*)((float*)out + at) = *(const floatx4*)((const float*)out + at) + v;
+    }
+    return;
+  }
   for (int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; e < (int64_t)m * columns; e += (int64_t)gridDim.x * blockDim.x) {
     const int token = e / columns, c = e % columns;
     const int gn = SWIGLU ? 16 * (c / 8) + c % 8 : c;
