@@ -348,8 +348,8 @@ __global__ __launch_bounds__(256) void qk_prep_vec_kernel(T* __restrict__ qkv, i
                                                           const float* __restrict__ cosv, const float* __restrict__ sinv,
                                                           int rot_half, T* __restrict__ k_pages, T* __restrict__ v_pages,
                                                           const int* __restrict__ slots, int page_size, int prep_blocks,
-                                                          const float* __restrict__ sums = nullptr, int splits = 0,
-                                                          int sum_columns = 0) {
+                                                          const float* __restrict__ sums, int splits,
+                                                          int sum_columns, int together) {
   // sums != null: the heads come as the float32 sums that the K splits of the q/k/v product left,
   // [splits, tokens, sum_columns], added up here in split order; qkv only receives the prepared q heads.
   constexpr int VE = 16 / sizeof(T);
@@ -361,100 +361,110 @@ __global__ __launch_bounds__(256) void qk_prep_vec_kernel(T* __restrict__ qkv, i
     return;
   }
   const int per_head = d / (2 * VE), half = d / 2;
+  // A group of per_head threads takes `together` consecutive heads of one token in turn (a whole number of
+  // them fill a token's heads), so the token's rotation tables and the norm weights, which every head needs
+  // again, are read once a group.
+  const int groups_per_token = heads / together;
   const int64_t pair = (int64_t)blockIdx.x * (256 / per_head) + threadIdx.x / per_head;
   const int j = threadIdx.x % per_head;
-  if (pair >= (int64_t)tokens * heads) return;   // whole groups of per_head lanes leave together
-  const int token = pair / heads, head = pair % heads;
-  T* src = qkv + (int64_t)token * row_stride + (int64_t)head * d;
-  const bool is_q = head < nq, is_k = !is_q && head < nq + nkv;
-  float a[VE], b[VE], inv = 1.f;
-  if (sums) {
+  if (pair >= (int64_t)tokens * groups_per_token) return;   // whole groups of per_head lanes leave together
+  const int token = pair / groups_per_token, head0 = (int)(pair % groups_per_token) * together;
+  float c[VE], sn[VE], wq[2][VE], wk[2][VE];
+  if (rot_half) {
+    load_floats<float, VE>(cosv + (int64_t)token * rot_half + VE * j, c);
+    load_floats<float, VE>(sinv + (int64_t)token * rot_half + VE * j, sn);
+  }
+  if (q_weight) {
+    load_floats<TW, VE>(q_weight + VE * j, wq[0]);
+    load_floats<TW, VE>(q_weight + half + VE * j, wq[1]);
+    load_floats<TW, VE>(k_weight + VE * j, wk[0]);
+    load_floats<TW, VE>(k_weight + half + VE * j, wk[1]);
+  }
+  const int slot = heads > nq ? slots[token] : -1;
+  for (int head = head0; head < head0 + together; ++head) {
+    T* src = qkv + (int64_t)token * row_stride + (int64_t)head * d;
+    const bool is_q = head < nq, is_k = !is_q && head < nq + nkv;
+    float a[VE], b[VE], inv = 1.f;
+    if (sums) {
 #pragma unroll
-    for (int e = 0; e < VE; ++e) a[e] = b[e] = 0.f;
-    const float* from = sums + (int64_t)token * sum_columns + (int64_t)head * d;
-    const int64_t apart = (int64_t)tokens * sum_columns;
-    for (int sp0 = 0; sp0 < splits; sp0 += 4) {       // four splits asked for at a time: one trip to memory, not four
-      float pa[4][VE], pb[4][VE];
+      for (int e = 0; e < VE; ++e) a[e] = b[e] = 0.f;
+      const float* from = sums + (int64_t)token * sum_columns + (int64_t)head * d;
+      const int64_t apart = (int64_t)tokens * sum_columns;
+      for (int sp0 = 0; sp0 < splits; sp0 += 4) {       // four splits asked for at a time: one trip to memory, not four
+        float pa[4][VE], pb[4][VE];
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        if (sp0 + i < splits) {
-          load_floats<float, VE>(from + (sp0 + i) * apart + VE * j, pa[i]);
-          load_floats<float, VE>(from + (sp0 + i) * apart + half + VE * j, pb[i]);
+        for (int i = 0; i < 4; ++i) {
+          if (sp0 + i < splits) {
+            load_floats<float, VE>(from + (sp0 + i) * apart + VE * j, pa[i]);
+            load_floats<float, VE>(from + (sp0 + i) * apart + half + VE * j, pb[i]);
+          }
         }
-      }
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        if (sp0 + i < splits) {
+        for (int i = 0; i < 4; ++i) {
+          if (sp0 + i < splits) {
 #pragma unroll
-          for (int e = 0; e < VE; ++e) {
-            a[e] += pa[i][e];
-            b[e] += pb[i][e];
+            for (int e = 0; e < VE; ++e) {
+              a[e] += pa[i][e];
+              b[e] += pb[i][e];
+            }
           }
         }
       }
-    }
-  } else {
-    const vec lo = *(const vec*)(src + VE * j), hi = *(const vec*)(src + half + VE * j);
-#pragma unroll
-    for (int e = 0; e < VE; ++e) {
-      a[e] = to_float(lo[e]);
-      b[e] = to_float(hi[e]);
-    }
-  }
-  int64_t page = 0, off = 0;
-  int kv_head = 0;
-  if (!is_q) {
-    const int slot = slots[token];
-    if (slot < 0) return;
-    kv_head = is_k ? head - nq : head - nq - nkv;
-    page = slot / page_size;
-    off = slot % page_size;
-    if (!is_k) {
-      T* vdst = v_pages + (page * nkv + kv_head) * d * page_size + off;
+    } else {
+      const vec lo = *(const vec*)(src + VE * j), hi = *(const vec*)(src + half + VE * j);
 #pragma unroll
       for (int e = 0; e < VE; ++e) {
-        vdst[(int64_t)(VE * j + e) * page_size] = from_float<T>(a[e]);
-        vdst[(int64_t)(half + VE * j + e) * page_size] = from_float<T>(b[e]);
+        a[e] = to_float(lo[e]);
+        b[e] = to_float(hi[e]);
       }
-      return;
     }
+    int64_t page = 0, off = 0;
+    int kv_head = 0;
+    if (!is_q) {
+      if (slot < 0) continue;
+      kv_head = is_k ? head - nq : head - nq - nkv;
+      page = slot / page_size;
+      off = slot % page_size;
+      if (!is_k) {
+        T* vdst = v_pages + (page * nkv + kv_head) * d * page_size + off;
+#pragma unroll
+        for (int e = 0; e < VE; ++e) {
+          vdst[(int64_t)(VE * j + e) * page_size] = from_float<T>(a[e]);
+          vdst[(int64_t)(half + VE * j + e) * page_size] = from_float<T>(b[e]);
+        }
+        continue;
+      }
+    }
+    if (q_weight) {
+      float ss = 0.f;
+#pragma unroll
+      for (int e = 0; e < VE; ++e) ss += a[e] * a[e] + b[e] * b[e];
+      for (int step = per_head / 2; step > 0; step >>= 1) ss += __shfl_xor(ss, step, WAVE);
+      inv = 1.0f / sqrtf(ss / (float)d + eps);
+#pragma unroll
+      for (int e = 0; e < VE; ++e) {
+        a[e] = a[e] * inv * (is_q ? wq[0][e] : wk[0][e]);
+        b[e] = b[e] * inv * (is_q ? wq[1][e] : wk[1][e]);
+      }
+    }
+    vec out_lo, out_hi;
+    if (rot_half) {
+#pragma unroll
+      for (int e = 0; e < VE; ++e) {
+        out_lo[e] = from_float<T>(a[e] * c[e] - b[e] * sn[e]);
+        out_hi[e] = from_float<T>(b[e] * c[e] + a[e] * sn[e]);
+      }
+    } else {
+#pragma unroll
+      for (int e = 0; e < VE; ++e) {
+        out_lo[e] = from_float<T>(a[e]);
+        out_hi[e] = from_float<T>(b[e]);
+      }
+    }
+    T* dst = is_q ? src : k_pages + ((page * nkv + kv_head) * page_size + off) * d;
+    *(vec*)(dst + VE * j) = out_lo;
+    *(vec*)(dst + half + VE * j) = out_hi;
   }
-  const TW* weight = is_q ? q_weight : k_weight;
-  if (weight) {
-    float ss = 0.f;
-#pragma unroll
-    for (int e = 0; e < VE; ++e) ss += a[e] * a[e] + b[e] * b[e];
-    for (int step = per_head / 2; step > 0; step >>= 1) ss += __shfl_xor(ss, step, WAVE);
-    inv = 1.0f / sqrtf(ss / (float)d + eps);
-    float wa[VE], wb[VE];
-    load_floats<TW, VE>(weight + VE * j, wa);
-    load_floats<TW, VE>(weight + half + VE * j, wb);
-#pragma unroll
-    for (int e = 0; e < VE; ++e) {
-      a[e] = a[e] * inv * wa[e];
-      b[e] = b[e] * inv * wb[e];
-    }
-  }
-  vec out_lo, out_hi;
-  if (rot_half) {
-    float c[VE], sn[VE];
-    load_floats<float, VE>(cosv + (int64_t)token * rot_half + VE * j, c);
-    load_floats<float, VE>(sinv + (int64_t)token * rot_half + VE * j, sn);
-#pragma unroll
-    for (int e = 0; e < VE; ++e) {
-      out_lo[e] = from_float<T>(a[e] * c[e] - b[e] * sn[e]);
-      out_hi[e] = from_float<T>(b[e] * c[e] + a[e] * sn[e]);
-    }
-  } else {
-#pragma unroll
-    for (int e = 0; e < VE; ++e) {
-      out_lo[e] = from_float<T>(a[e]);
-      out_hi[e] = from_float<T>(b[e]);
-    }
-  }
-  T* dst = is_q ? src : k_pages + ((page * nkv + kv_head) * page_size + off) * d;
-  *(vec*)(dst + VE * j) = out_lo;
-  *(vec*)(dst + half + VE * j) = out_hi;
 }
 
 static int qk_prep_launch(void* qkv, int dtype, int tokens, int row_stride, int nq, int nkv, int d,
@@ -481,7 +491,10 @@ static int qk_prep_launch(void* qkv, int dtype, int tokens, int row_stride, int 
                        ((uintptr_t)sinv % 16) == 0;
   if (vectors) {
     const int heads = nq + (values_apart ? nkv : 2 * nkv);    // heads the (token, head) pairs run over
-    const int64_t pairs = (int64_t)tokens * heads;
+    // heads of one token that a group of threads takes in turn: the largest of 5, 4, 2 that divides them, for
+    // steps of many tokens (a decode step has too few groups to fill the chip as it is)
+    const int together = tokens < 128 || sums ? 1 : heads % 5 == 0 ? 5 : heads % 4 == 0 ? 4 : heads % 2 == 0 ? 2 : 1;
+    const int64_t pairs = (int64_t)tokens * (heads / together);
     const int per_block = 256 / per_head;
     const int64_t prep_blocks = (pairs + per_block - 1) / per_block;
     const int64_t value_blocks = values_apart ? (int64_t)((tokens + 15) / 16) * nkv : 0;
@@ -490,7 +503,7 @@ static int qk_prep_launch(void* qkv, int dtype, int tokens, int row_stride, int 
 #define LAUNCH_VEC(T, TW)                                                                                        \
   qk_prep_vec_kernel<T, TW><<<vgrid, 256, 0, s>>>((T*)qkv, row_stride, tokens, heads, nq, nkv, d, (const TW*)q_weight, \
                                                   (const TW*)k_weight, eps, cosv, sinv, rot_half, (T*)k_pages,   \
-                                                  (T*)v_pages, slots, page_size, (int)prep_blocks, sums, splits, sum_columns)
+                                                  (T*)v_pages, slots, page_size, (int)prep_blocks, sums, splits, sum_columns, together)
     if (dtype == LRS_F32 && w_dtype == LRS_F32) LAUNCH_VEC(float, float);
     else if (dtype == LRS_BF16 && w_dtype == LRS_BF16) LAUNCH_VEC(bf16, bf16);
     else if (dtype == LRS_BF16 && w_dtype == LRS_F32) LAUNCH_VEC(bf16, float);
