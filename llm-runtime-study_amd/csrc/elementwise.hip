@@ -341,7 +341,7 @@ __global__ __launch_bounds__(256) void values_to_pages_kernel(const T* __restric
 // threads share a head, and a workgroup takes 256 / that many consecutive (token, head) pairs of the
 // `heads` first heads of every token.  Workgroups from `prep_blocks` on (if any) store the v heads
 // instead, 16 tokens of one kv head each, as values_to_pages() does.
-template <typename T, typename TW>
+template <typename T, typename TW, int TOGETHER>
 __global__ __launch_bounds__(256) void qk_prep_vec_kernel(T* __restrict__ qkv, int row_stride, int tokens, int heads, int nq,
                                                           int nkv, int d, const TW* __restrict__ q_weight,
                                                           const TW* __restrict__ k_weight, float eps,
@@ -349,7 +349,7 @@ __global__ __launch_bounds__(256) void qk_prep_vec_kernel(T* __restrict__ qkv, i
                                                           int rot_half, T* __restrict__ k_pages, T* __restrict__ v_pages,
                                                           const int* __restrict__ slots, int page_size, int prep_blocks,
                                                           const float* __restrict__ sums, int splits,
-                                                          int sum_columns, int together) {
+                                                          int sum_columns) {
   // sums != null: the heads come as the float32 sums that the K splits of the q/k/v product left,
   // [splits, tokens, sum_columns], added up here in split order; qkv only receives the prepared q heads.
   constexpr int VE = 16 / sizeof(T);
@@ -361,9 +361,10 @@ __global__ __launch_bounds__(256) void qk_prep_vec_kernel(T* __restrict__ qkv, i
     return;
   }
   const int per_head = d / (2 * VE), half = d / 2;
-  // A group of per_head threads takes `together` consecutive heads of one token in turn (a whole number of
-  // them fill a token's heads), so the token's rotation tables and the norm weights, which every head needs
-  // again, are read once a group.
+  // A group of per_head threads takes TOGETHER consecutive heads of one token (a whole number of such runs
+  // fill a token's heads): the token's rotation tables and the norm weights, which every head needs again, are
+  // read once a group, and all the heads' values are asked for before the first is worked on.
+  constexpr int together = TOGETHER;
   const int groups_per_token = heads / together;
   const int64_t pair = (int64_t)blockIdx.x * (256 / per_head) + threadIdx.x / per_head;
   const int j = threadIdx.x % per_head;
@@ -381,7 +382,18 @@ __global__ __launch_bounds__(256) void qk_prep_vec_kernel(T* __restrict__ qkv, i
     load_floats<TW, VE>(k_weight + half + VE * j, wk[1]);
   }
   const int slot = heads > nq ? slots[token] : -1;
-  for (int head = head0; head < head0 + together; ++head) {
+  vec lo[TOGETHER], hi[TOGETHER];
+  if (!sums) {
+#pragma unroll
+    for (int t = 0; t < TOGETHER; ++t) {
+      const T* from = qkv + (int64_t)token * row_stride + (int64_t)(head0 + t) * d;
+      lo[t] = *(const vec*)(from + VE * j);
+      hi[t] = *(const vec*)(from + half + VE * j);
+    }
+  }
+#pragma unroll
+  for (int t = 0; t < TOGETHER; ++t) {
+    const int head = head0 + t;
     T* src = qkv + (int64_t)token * row_stride + (int64_t)head * d;
     const bool is_q = head < nq, is_k = !is_q && head < nq + nkv;
     float a[VE], b[VE], inv = 1.f;
@@ -411,11 +423,10 @@ __global__ __launch_bounds__(256) void qk_prep_vec_kernel(T* __restrict__ qkv, i
         }
       }
     } else {
-      const vec lo = *(const vec*)(src + VE * j), hi = *(const vec*)(src + half + VE * j);
 #pragma unroll
       for (int e = 0; e < VE; ++e) {
-        a[e] = to_float(lo[e]);
-        b[e] = to_float(hi[e]);
+        a[e] = to_float(lo[t][e]);
+        b[e] = to_float(hi[t][e]);
       }
     }
     int64_t page = 0, off = 0;
@@ -500,16 +511,24 @@ static int qk_prep_launch(void* qkv, int dtype, int tokens, int row_stride, int 
     const int64_t value_blocks = values_apart ? (int64_t)((tokens + 15) / 16) * nkv : 0;
     LRS_REQUIRE(prep_blocks + value_blocks < (1ll << 31), "qk_prep: %d tokens are too many for one launch", tokens);
     dim3 vgrid((unsigned)(prep_blocks + value_blocks));
-#define LAUNCH_VEC(T, TW)                                                                                        \
-  qk_prep_vec_kernel<T, TW><<<vgrid, 256, 0, s>>>((T*)qkv, row_stride, tokens, heads, nq, nkv, d, (const TW*)q_weight, \
-                                                  (const TW*)k_weight, eps, cosv, sinv, rot_half, (T*)k_pages,   \
-                                                  (T*)v_pages, slots, page_size, (int)prep_blocks, sums, splits, sum_columns, together)
+#define LAUNCH_VEC_OF(T, TW, TOGETHER)                                                                                   \
+  qk_prep_vec_kernel<T, TW, TOGETHER><<<vgrid, 256, 0, s>>>((T*)qkv, row_stride, tokens, heads, nq, nkv, d, (const TW*)q_weight, \
+                                                            (const TW*)k_weight, eps, cosv, sinv, rot_half, (T*)k_pages,   \
+                                                            (T*)v_pages, slots, page_size, (int)prep_blocks, sums, splits, sum_columns)
+#define LAUNCH_VEC(T, TW)                        \
+  do {                                           \
+    if (together == 5) LAUNCH_VEC_OF(T, TW, 5);  \
+    else if (together == 4) LAUNCH_VEC_OF(T, TW, 4); \
+    else if (together == 2) LAUNCH_VEC_OF(T, TW, 2); \
+    else LAUNCH_VEC_OF(T, TW, 1);                \
+  } while (0)
     if (dtype == LRS_F32 && w_dtype == LRS_F32) LAUNCH_VEC(float, float);
     else if (dtype == LRS_BF16 && w_dtype == LRS_BF16) LAUNCH_VEC(bf16, bf16);
     else if (dtype == LRS_BF16 && w_dtype == LRS_F32) LAUNCH_VEC(bf16, float);
     else if (dtype == LRS_F32 && w_dtype == LRS_BF16) LAUNCH_VEC(float, bf16);
     else return lrs_fail("qk_prep: unknown dtypes %d/%d", dtype, w_dtype);
 #undef LAUNCH_VEC
+#undef LAUNCH_VEC_OF
     return lrs_check_launch("qk_prep");
   }
   LRS_REQUIRE(!sums, "qk_prep: the sums of K splits need the shape the vector kernel takes (head_dim %d, rotation over %d)", d, 2 * rot_half);
