@@ -42,6 +42,9 @@ def parse_args():
     parser.add_argument("--layers", type=int, default=None, help="fewer layers than the shape has (reported in config)")
     parser.add_argument("--dtype", choices=("bfloat16", "float32"), default="bfloat16")
     parser.add_argument("--no-points", action="store_true", help="skip the batch 1 and 64 decode points")
+    parser.add_argument("--temperature", type=float, default=0.0, help="draw the tokens at this temperature instead of taking the largest logit (reported in config)")
+    parser.add_argument("--top-k", type=int, default=None, help="with --temperature: keep the k likeliest tokens")
+    parser.add_argument("--top-p", type=float, default=1.0, help="with --temperature: keep the likeliest tokens up to this share of the mass")
     parser.add_argument("--no-graph", action="store_true")
     parser.add_argument("--decode-steps-per-launch", type=int, default=4, help="greedy decode steps run from one graph launch (1: one step a launch)")
     parser.add_argument("--library-mid-gemm", action="store_true", help="products of 17..128 rows through the vendor library instead of this package's kernel for them")
@@ -67,7 +70,7 @@ def decode_lead(batch: int, context: int, step_tokens: int) -> int:
     return (batch - 1) * -(-context // step_tokens)
 
 
-def measure_decode(engine, batch: int, context: int, steps: int, warmup: int, seed: int):
+def measure_decode(engine, batch: int, context: int, steps: int, warmup: int, seed: int, sampling=None):
     """Prefill `batch` prompts of `context` random tokens through the scheduler, then time `steps`
     decode steps.  Returns (seconds per step list, mean context length over the timed steps)."""
     import numpy as np
@@ -83,7 +86,7 @@ def measure_decode(engine, batch: int, context: int, steps: int, warmup: int, se
     for _ in range(batch):
         scheduler.add_request(rng.integers(0, vocab, context).tolist(),
                               max_new_tokens=warmup + steps + lead + batch + 8 + 2 * scheduler.decode_steps_per_launch,
-                              sampling=SamplingConfig())
+                              sampling=sampling if sampling is not None else SamplingConfig())
     times = []
     with torch.cuda.device(engine.device), torch.cuda.stream(engine.stream):
         # prefill phase: until every request has sampled its first token
@@ -175,7 +178,12 @@ def main() -> int:
     prefill_s = statistics.median(prefill_times)
     flops = prefill_flops(config, args.prefill_tokens)
 
-    times, mean_context = measure_decode(engine, args.batch, args.context, args.steps, args.warmup, seed=2)
+    sampling = None
+    if args.temperature > 0:
+        from llm_runtime_study_amd import SamplingConfig
+
+        sampling = SamplingConfig(temperature=args.temperature, top_k=args.top_k, top_p=args.top_p, seed=7)
+    times, mean_context = measure_decode(engine, args.batch, args.context, args.steps, args.warmup, seed=2, sampling=sampling)
     total = sum(times)
     step_s = total / len(times)
     weight_bytes = engine.model.weight_bytes()
@@ -186,7 +194,7 @@ def main() -> int:
     if not args.no_points:
         for batch in (1, 64):
             point_steps = min(args.steps, 64)
-            t, _ = measure_decode(engine, batch, args.context, point_steps, min(args.warmup, 4), seed=3 + batch)
+            t, _ = measure_decode(engine, batch, args.context, point_steps, min(args.warmup, 4), seed=3 + batch, sampling=sampling)
             points[f"decode_b{batch}"] = round(batch * len(t) / sum(t), 2)
 
     line = {
@@ -211,6 +219,7 @@ def main() -> int:
             "prefill_tokens": args.prefill_tokens, "hip_graph": bool(engine.runner.use_graph),
             "decode_steps_per_launch": args.decode_steps_per_launch if engine.runner.use_graph else 1, "prefill_gemm": "own" if args.own_gemm else "hipBLASLt",
             "parallelism": "single GPU",
+            "sampling": "greedy" if sampling is None else f"temperature {args.temperature} top_k {args.top_k} top_p {args.top_p}",
         },
         "prefill": {
             "value": round(args.prefill_tokens / prefill_s, 1), "tokens": args.prefill_tokens,

@@ -9,6 +9,7 @@
 #include "no_alloc.h"
 
 #include <mutex>
+#include <type_traits>
 
 __device__ __forceinline__ uint32_t mix32(uint32_t x) {
   x ^= x >> 16;
@@ -243,11 +244,49 @@ LRS_API int lrs_choose_tokens(int* out, const float* logits, int64_t row_stride,
 // others to -inf, in place.  One workgroup per row.  Rule (the reference's): after scaling
 // by 1/temperature keep the k largest; then, in descending order, drop a token once the
 // probability mass strictly before it reaches top_p, so the token that crosses stays.
-// Both thresholds are found by bisection over the ordered bit patterns of float32 (at most
-// 32 passes over the row each), which needs no sort.
+// Both thresholds are values of the row itself and are found without a sort, by selection over the
+// ordered bit patterns of float32, 11 + 11 + 10 bits at a time: a pass over the row counts (top-k) or
+// weighs (top-p) the values by the next digit of their pattern in LDS, the digit whose bin holds the
+// k-th largest value (the value at which the mass from the top reaches p of the whole) is fixed, and the
+// next pass looks inside that bin.  Three passes each instead of a bisection's thirty-two.  Masses are
+// added up as integers (exp(v - max) * 2^35), so the sums, and with them the tokens kept, do not depend on
+// the order in which the threads arrive.
 __device__ __forceinline__ uint32_t ordered_key(float v) {
   const uint32_t bits = __float_as_uint(v);
   return (bits & 0x80000000U) ? ~bits : (bits | 0x80000000U);
+}
+
+constexpr int FILTER_BINS = 2048;
+
+// The largest bin b whose own content and everything above it come to `need` or more, and what lies above it.
+// All threads call; the first wave works.  bins[] is complete (a barrier has passed) and may be cleared after.
+template <typename V>
+__device__ __forceinline__ void filter_find_bin(const V* bins, int nbins, double need, int* found_bin, double* found_above) {
+  const int lane = threadIdx.x % WAVE;
+  if (threadIdx.x < WAVE) {
+    const int per = nbins / WAVE;
+    double mine = 0.0;
+    for (int i = 0; i < per; ++i) mine += (double)bins[lane * per + i];
+    double with_mine = mine;                                   // this lane's bins and those of the lanes above
+    for (int step = 1; step < WAVE; step <<= 1) {
+      const double other = __shfl_down(with_mine, step, WAVE);
+      if (lane + step < WAVE) with_mine += other;
+    }
+    const unsigned long long reach = __ballot(with_mine >= need);
+    const int owner = reach ? 63 - __builtin_clzll(reach) : 0;   // the highest lane that reaches it (lane 0 if none: cannot happen)
+    if (lane == owner) {
+      double above = with_mine - mine;
+      int bin = lane * per;
+      for (int i = per - 1; i >= 0; --i) {
+        const double here = (double)bins[lane * per + i];
+        if (above + here >= need) { bin = lane * per + i; break; }
+        above += here;
+      }
+      *found_bin = bin;
+      *found_above = above;
+    }
+  }
+  __syncthreads();
 }
 
 __global__ __launch_bounds__(1024) void filter_logits_kernel(float* __restrict__ logits,
@@ -256,6 +295,9 @@ __global__ __launch_bounds__(1024) void filter_logits_kernel(float* __restrict__
                                                              const int* __restrict__ top_k,
                                                              const float* __restrict__ top_p) {
   __shared__ float scratch[16];
+  __shared__ unsigned long long bins[FILTER_BINS];             // counts or masses
+  __shared__ int found_bin;
+  __shared__ double found_above;
   const int row = blockIdx.x, tid = threadIdx.x;
   float* z = logits + (int64_t)row * row_stride;
   const float temp = temperature[row];
@@ -265,52 +307,92 @@ __global__ __launch_bounds__(1024) void filter_logits_kernel(float* __restrict__
   const bool use_k = k > 0 && k < vocab, use_p = p < 1.f;
   if (!use_k && !use_p) return;
 
-  float vmax = -INFINITY, vmin = INFINITY;
-  for (int i = tid; i < vocab; i += blockDim.x) {
-    const float v = z[i] / temp;
-    vmax = fmaxf(vmax, v);
-    if (v > -INFINITY) vmin = fminf(vmin, v);
-  }
-  vmax = block_max(vmax, scratch);
-  vmin = -block_max(-vmin, scratch);
-  const uint32_t key_min = ordered_key(vmin), key_max = ordered_key(vmax);
-
-  // largest key t with count(key >= t) >= k: the k-th largest value
-  uint32_t threshold = key_min;
-  if (use_k) {
-    uint32_t lo = key_min, hi = key_max;
-    while (lo < hi) {
-      const uint32_t mid = lo + (hi - lo + 1) / 2;
-      float count = 0.f;
-      for (int i = tid; i < vocab; i += blockDim.x) count += (ordered_key(z[i] / temp) >= mid) ? 1.f : 0.f;
-      count = block_sum(count, scratch);
-      if (count >= (float)k) lo = mid; else hi = mid - 1;
-    }
-    threshold = lo;
-  }
-  if (use_p) {
-    float total = 0.f;
-    for (int i = tid; i < vocab; i += blockDim.x) {
-      const float v = z[i] / temp;
-      if (ordered_key(v) >= threshold) total += expf(v - vmax);
-    }
-    total = block_sum(total, scratch);
-    // smallest key t with mass(keys > t) < p * total; mass above the maximum is 0, so it exists
-    uint32_t lo = threshold, hi = key_max;
-    while (lo < hi) {
-      const uint32_t mid = lo + (hi - lo) / 2;
-      float above = 0.f;
-      for (int i = tid; i < vocab; i += blockDim.x) {
-        const float v = z[i] / temp;
-        if (ordered_key(v) > mid) above += expf(v - vmax);
+  // A pass over the row: body(index, logit) for each of this thread's values.  Four loads of 16 bytes are asked
+  // for before any is used (a thread's loads one after the other, each waited for, were what a pass took its
+  // time for); rows that do not begin on 16 bytes go one value at a time.  Dividing by the temperature (positive)
+  // changes no order, so the patterns compared are those of the logits themselves, and only the masses are taken
+  // of the scaled values: exp((logit - largest logit) / temperature).
+  const bool in_fours = ((uintptr_t)z % 16) == 0;
+  auto walk = [&](auto&& body) {
+    const int fours = in_fours ? vocab / 4 : 0;
+    for (int first = tid; first < fours; first += 4 * (int)blockDim.x) {
+      floatx4 part[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int at = first + j * (int)blockDim.x;
+        part[j] = ((const floatx4*)z)[at < fours ? at : first];
       }
-      above = block_sum(above, scratch);
-      if (above < p * total) hi = mid; else lo = mid + 1;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int at = first + j * (int)blockDim.x;
+        if (at < fours) {
+#pragma unroll
+          for (int e = 0; e < 4; ++e) body(at * 4 + e, part[j][e]);
+        }
+      }
     }
-    threshold = lo;
-  }
-  for (int i = tid; i < vocab; i += blockDim.x)
-    if (ordered_key(z[i] / temp) < threshold) z[i] = -INFINITY;
+    for (int i = fours * 4 + tid; i < vocab; i += blockDim.x) body(i, z[i]);
+  };
+
+  float zmax = -INFINITY;
+  walk([&](int, float v) { zmax = fmaxf(zmax, v); });
+  zmax = block_max(zmax, scratch);
+  const float per_temp2 = 1.4426950408889634f / temp;          // exp(x / temp) = exp2(x * this)
+
+  // One selection: MASS false: the largest pattern t with count(pattern >= t) >= need; MASS true: the largest
+  // pattern t, among those >= floor, with mass(pattern >= t) >= share of the mass of all those >= floor.
+  auto select = [&](auto mass, double need, uint32_t floor, float share) -> uint32_t {
+    constexpr bool MASS = decltype(mass)::value;
+    uint32_t prefix = 0;
+#pragma unroll
+    for (int level = 0; level < 3; ++level) {
+      const int shift = level == 0 ? 21 : level == 1 ? 10 : 0, nbins = level == 2 ? 1024 : 2048;
+      for (int i = tid; i < nbins; i += blockDim.x) bins[i] = 0;
+      __syncthreads();
+      uint32_t run_bin = 0xFFFFFFFFu;                          // values that follow each other into one bin are added up first
+      unsigned long long run = 0;
+      walk([&](int, float v) {
+        const uint32_t key = ordered_key(v);
+        if (MASS && key < floor) return;
+        if (level == 1 && (key >> 21) != prefix) return;
+        if (level == 2 && (key >> 10) != prefix) return;
+        const uint32_t bin = (key >> shift) & (uint32_t)(nbins - 1);
+        const unsigned long long weight = MASS ? (unsigned long long)(__builtin_amdgcn_exp2f((v - zmax) * per_temp2) * 34359738368.f) : 1ull;
+        if (bin == run_bin) {
+          run += weight;
+        } else {
+          if (run_bin != 0xFFFFFFFFu) atomicAdd(&bins[run_bin], run);
+          run_bin = bin;
+          run = weight;
+        }
+      });
+      if (run_bin != 0xFFFFFFFFu) atomicAdd(&bins[run_bin], run);
+      __syncthreads();
+      if (MASS && level == 0) {                                // the whole mass: every bin of the first pass
+        double whole = 0.0;
+        if (tid < WAVE) {
+          for (int i = tid; i < nbins; i += WAVE) whole += (double)bins[i];
+          for (int step = WAVE / 2; step > 0; step >>= 1) whole += __shfl_xor(whole, step, WAVE);
+          if (tid == 0) found_above = whole;
+        }
+        __syncthreads();
+        need = (double)share * found_above;
+        __syncthreads();
+      }
+      filter_find_bin(bins, nbins, need, &found_bin, &found_above);
+      need -= found_above;
+      prefix = (prefix << (level == 2 ? 10 : 11)) | (uint32_t)found_bin;
+      __syncthreads();                                         // everyone has read the result before the bins are cleared
+    }
+    return prefix;
+  };
+
+  uint32_t threshold = 0;
+  if (use_k) threshold = select(std::false_type{}, (double)k, 0u, 0.f);
+  if (use_p) threshold = select(std::true_type{}, 0.0, threshold, p);
+  walk([&](int i, float v) {
+    if (ordered_key(v) < threshold) z[i] = -INFINITY;
+  });
 }
 
 LRS_API int lrs_filter_logits(float* logits, int64_t row_stride, int rows, int vocab,

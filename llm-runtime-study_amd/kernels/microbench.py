@@ -5,6 +5,7 @@
     python -m llm_runtime_study_amd.kernels.microbench attention_decode --batch 1,8,64 --context 2048 --splits 1,4,8
     python -m llm_runtime_study_amd.kernels.microbench gemm --rows 1,8,16,64,2048
     python -m llm_runtime_study_amd.kernels.microbench memory
+    python -m llm_runtime_study_amd.kernels.microbench sampling --batch 8,64   # top-k / top-p filtering and the draw, a vocabulary of 151,936
     python -m llm_runtime_study_amd.kernels.microbench lds          # LDS read rate by the distance between a fragment's rows
     python -m llm_runtime_study_amd.kernels.microbench mfma         # matrix instructions with vector work beside them
 
@@ -140,6 +141,33 @@ def memory(args) -> None:
         del buffers
 
 
+def sampling(args) -> None:
+    """Filtering the logits of a step (top-k, top-p, both) and choosing its tokens (greedy, drawn)."""
+    vocab = args.vocab_size or 151936
+    generator = torch.Generator().manual_seed(0)
+    for rows in _ints(args.batch):
+        base = (torch.randn(rows, vocab, generator=generator) * 3).cuda()
+        copies = [base.clone() for _ in range(8)]
+        temperature = torch.full((rows,), 0.8, device="cuda")
+        seeds = torch.arange(rows, dtype=torch.int64, device="cuda")
+        counters = torch.zeros(rows, dtype=torch.int32, device="cuda")
+        out = torch.zeros(rows, dtype=torch.int32, device="cuda")
+        for name, k, p in (("top_k 50", 50, 1.0), ("top_p 0.9", 0, 0.9), ("top_k 50, top_p 0.9", 50, 0.9)):
+            top_k = torch.full((rows,), k, dtype=torch.int32, device="cuda")
+            top_p = torch.full((rows,), p, device="cuda")
+
+            def call(i):
+                copies[i % 8].copy_(base)             # the filter writes into the logits: a fresh copy every time
+                ops.filter_logits(copies[i % 8], temperature, top_k, top_p)
+
+            copy_only = _time(lambda i: copies[i % 8].copy_(base), args.repeats)
+            seconds = _time(call, args.repeats) - copy_only
+            print(f"sampling rows={rows:3d} vocab={vocab} filter_logits {name:20s} {seconds * 1e6:8.1f} us", flush=True)
+        for name, drawn in (("greedy", False), ("drawn", True)):
+            seconds = _time(lambda i: ops.choose_tokens(out, base, *((temperature, seeds, counters) if drawn else ())), args.repeats)
+            print(f"sampling rows={rows:3d} vocab={vocab} choose_tokens {name:20s} {seconds * 1e6:8.1f} us", flush=True)
+
+
 def lds(args) -> None:
     """16-byte LDS reads in the shape of a matrix-core fragment (a lane's row is lane % 16, its piece lane / 16)
     for every distance between rows: what the layout of a tile in LDS has to respect."""
@@ -164,20 +192,20 @@ def mfma(args) -> None:
 
 def main(argv=None) -> int:
     parser = argparse.ArgumentParser(prog="python -m llm_runtime_study_amd.kernels.microbench", description=__doc__.split("\n\n")[0])
-    parser.add_argument("kernel", choices=["attention_prefill", "attention_decode", "gemm", "memory", "lds", "mfma"])
+    parser.add_argument("kernel", choices=["attention_prefill", "attention_decode", "gemm", "memory", "sampling", "lds", "mfma"])
     parser.add_argument("--heads", type=int, default=32)
     parser.add_argument("--kv-heads", type=int, default=8)
     parser.add_argument("--head-dim", type=int, default=128)
     parser.add_argument("--hidden-size", type=int, default=4096)
     parser.add_argument("--intermediate-size", type=int, default=12288)
-    parser.add_argument("--vocab-size", type=int, default=0, help="gemm: also the LM head of this many rows")
+    parser.add_argument("--vocab-size", type=int, default=0, help="gemm: also the LM head of this many rows; sampling: the vocabulary (default 151936)")
     parser.add_argument("--page-size", type=int, default=16)
     parser.add_argument("--window", type=int, default=0)
     parser.add_argument("--tokens", default="2048", help="attention_prefill: prompt lengths, comma separated")
     parser.add_argument("--before", type=int, default=0, help="attention_prefill: tokens of the request already in the cache (the queries are a later portion)")
     parser.add_argument("--key-splits", default="1", help="attention_prefill: workgroups per query group")
     parser.add_argument("--group", default="", help="attention_prefill: query group sizes (default: what the engine would choose)")
-    parser.add_argument("--batch", default="1,8,64", help="attention_decode: batch sizes")
+    parser.add_argument("--batch", default="1,8,64", help="attention_decode, sampling: batch sizes")
     parser.add_argument("--context", type=int, default=2048, help="attention_decode: cached tokens per request")
     parser.add_argument("--splits", default="1,2,4,8,16", help="attention_decode: workgroups per (token, kv head)")
     parser.add_argument("--form", default="0,1,2", help="attention_decode: 0 four waves, 1 four waves with the next tile on the way, 2 eight waves likewise")
@@ -192,7 +220,8 @@ def main(argv=None) -> int:
         print("microbench needs the GPU", file=sys.stderr)
         return 2
     ops.library()
-    {"attention_prefill": attention_prefill, "attention_decode": attention_decode, "gemm": gemm, "memory": memory, "lds": lds, "mfma": mfma}[args.kernel](args)
+    {"attention_prefill": attention_prefill, "attention_decode": attention_decode, "gemm": gemm, "memory": memory, "sampling": sampling, "lds": lds,
+     "mfma": mfma}[args.kernel](args)
     return 0
 
 

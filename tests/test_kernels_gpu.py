@@ -911,6 +911,57 @@ def test_filter_logits_matches_sort_based_rule(ops):
     assert torch.isfinite(got[1]).sum() == 2
 
 
+@pytest.mark.parametrize("vocab", [151936, 50257, 4099])
+def test_filter_logits_of_a_large_vocabulary_matches_the_sort_based_rule(ops, vocab):
+    """The selection by digits of the bit pattern, where it has something to select from: a vocabulary of the
+    real size, rows whose values crowd into one or two of its first bins (all between 16 and 20; all negative
+    and small), rows with the usual spread, a k beyond the first bin, a share that the largest value holds alone."""
+    from tests.plain.model import filter_logits as plain_filter
+
+    g = torch.Generator().manual_seed(vocab)
+    cases = [(0.8, 50, 1.0), (1.0, None, 0.9), (0.7, 50, 0.9), (1.0, 1000, 0.95), (1.5, 7, 0.3), (1.0, None, 0.999),
+             (1.0, 20, 0.9), (1.0, None, 0.5), (0.9, 3000, 1.0), (1.0, None, 0.2)]
+    logits = torch.randn(len(cases), vocab, generator=g) * 3
+    logits[6] = 16 + 4 * torch.rand(vocab, generator=g)          # one bin of the first digit holds them all
+    logits[7] = -1e-3 * torch.rand(vocab, generator=g) - 1e-4    # tiny negatives, close together
+    logits[9, 17] = 40.0                                         # one token has nearly all the mass
+    work = dev(logits.clone())
+    temps = dev(torch.tensor([c[0] for c in cases]))
+    ks = dev(torch.tensor([c[1] or 0 for c in cases], dtype=torch.int32))
+    ps = dev(torch.tensor([c[2] for c in cases]))
+    ops.filter_logits(work, temps, ks, ps)
+    got = work.cpu()
+    def rule_in_float64(row, temp, k, p):
+        # tests/plain/model.py:filter_logits with the masses added up in float64 (in float32 the running sum of
+        # 150,000 terms is itself uncertain by more than the tokens at the edge of a share of 0.999 weigh)
+        z = (row.float() / temp).double()
+        if k is not None and k < z.numel():
+            top, idx = torch.topk(z, k)
+            z = torch.full_like(z, -torch.inf).scatter(0, idx, top)
+        if p < 1.0:
+            ordered, idx = torch.sort(z, descending=True)
+            share = torch.softmax(ordered, -1)
+            before = torch.cumsum(share, -1) - share
+            z = torch.empty_like(z).scatter(0, idx, ordered.masked_fill(before >= p, -torch.inf))
+        return z
+
+    for i, (temp, k, p) in enumerate(cases):
+        if vocab == 4099:
+            assert torch.equal(torch.isfinite(plain_filter(logits[i], temp, k, p)), torch.isfinite(rule_in_float64(logits[i], temp, k, p)))
+        kept, wanted = torch.isfinite(got[i]), torch.isfinite(rule_in_float64(logits[i], temp, k, p))
+        # a token exactly at the edge may fall either way (the kernel's exponentials are float32); far down the tail
+        # (a share of 0.999) a few more, but never a mass that matters
+        share = torch.softmax(logits[i].double() / temp, -1)
+        assert share[kept != wanted].sum() < 2e-7, f"case {i}: {kept.sum()} kept, {wanted.sum()} wanted"
+        if p < 0.99:
+            assert (kept != wanted).sum() <= 1, f"case {i}: {kept.sum()} kept, {wanted.sum()} wanted"
+        both = kept & wanted
+        torch.testing.assert_close(got[i][both], logits[i][both], rtol=0, atol=0)
+        if k is not None and p == 1.0:
+            assert torch.equal(kept, wanted) and kept.sum() == k
+    assert torch.isfinite(got[9]).sum() == 1
+
+
 @pytest.mark.gpu
 def test_the_probes_of_lds_and_matrix_rates_run_and_refuse_what_they_cannot_do(ops):
     """`microbench lds` and `microbench mfma` are measurements, not products: here only that they launch,
