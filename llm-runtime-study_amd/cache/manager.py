@@ -119,6 +119,15 @@ class CacheManager:
                 raise KVCacheError(f"entry {position} declares an unknown cache need: {need!r}")
             self.layer_caches.append(cache)
 
+        if allocate_storage and self.device.type == "cuda" and self.groups:
+            # a pool the device cannot hold is refused before anything is allocated, with the numbers that decide it
+            element = torch.empty(0, dtype=dtype).element_size()
+            per_page = sum(2 * len(g.entries) * g.need.num_kv_heads * g.need.head_dim * page_size * element for g in self.groups)
+            free, _ = torch.cuda.mem_get_info(self.device)
+            if (num_pages + 1) * per_page > free:
+                fits = max(free // per_page - 1, 0)
+                raise KVCacheError(f"a cache pool of {num_pages} pages of {page_size} tokens needs {(num_pages + 1) * per_page / 2**30:.1f} GiB, "
+                                   f"{free / 2**30:.1f} GiB are free on {self.device}: {fits} pages ({fits * page_size} tokens) would fit")
         for index, group in enumerate(self.groups):
             group.host_table = np.full((max_requests, self.max_blocks), -1, dtype=np.int32)
             if allocate_storage:

@@ -555,3 +555,17 @@ def test_host_cost_benchmark_times_the_three_ways_of_launching_a_step(capsys):
         assert 0 < report[way]["host_ms"] <= report[way]["total_ms"]
     assert report["from_plan"]["replays"] >= 3 and report["from_graph_of_plan"]["replays"] >= 3
     assert report["from_graph_of_plan"]["host_ms"] < report["through_parts"]["host_ms"]
+
+
+def test_a_cache_pool_the_device_cannot_hold_is_refused_before_anything_is_allocated():
+    """64 requests of 1,048,576 tokens for 36 layers of 8 kv heads of 128: 9 TiB of pages.  The error says what
+    was asked for, what is free and what would fit; nothing was allocated."""
+    from llm_runtime_study_amd.cache import CacheManager
+    from llm_runtime_study_amd.parts import PagedKVNeed
+    from llm_runtime_study_amd.errors import KVCacheError
+
+    before = torch.cuda.memory_allocated()
+    with pytest.raises(KVCacheError, match=r"needs 9\d\d\d\.\d GiB.*GiB are free.*would fit"):
+        CacheManager([PagedKVNeed(8, 128, None)] * 36, page_size=16, num_pages=64 * 65536, max_requests=64, max_seq_len=1 << 20,
+                     dtype=torch.bfloat16, device="cuda")
+    assert torch.cuda.memory_allocated() == before
