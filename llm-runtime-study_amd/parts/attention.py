@@ -91,7 +91,11 @@ class GQAAttention(Part):
         256 keys each (a power of two that follows the length's class, not the length); and enough
         that the block table entries of one workgroup (at most 4,096) fit its LDS for contexts up
         to `bound`."""
-        wanted = -(-2 * ops.compute_units() // workgroups)
+        units = ops.compute_units()
+        # from five workgroups for every eight units on, the batch alone does as well or better, and there is nothing
+        # to merge (2,048 tokens of context, batch 20 / 24 / 32: 37.8 / 42.0 / 52.7 us undivided against 40.1 / 45 /
+        # 54.4 us with the 4 / 3 / 2 parts that two workgroups a unit would ask for; the same at 8,192 tokens)
+        wanted = 1 if 8 * workgroups >= 5 * units else -(-2 * units // workgroups)
         return max(1, min(wanted, length_class(longest) // 256, 64), -(-bound // (4096 * page_size)))
 
     @staticmethod

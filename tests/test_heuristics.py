@@ -23,6 +23,8 @@ def test_decode_splits_follow_the_class_not_the_length(monkeypatch):
     # few rows, long context: more workgroups, at least 256 keys each
     assert splits(8, 2048, 4096, 16) == 8 and splits(8, 2049, 4096, 16) == 8 and splits(8, 4095, 4096, 16) == 8
     assert splits(8, 4096, 8192, 16) == 16 and splits(64, 2048, 4096, 16) == 8 and splits(128, 2048, 4096, 16) == 4
+    # five workgroups for every eight compute units, or more: not divided
+    assert splits(152, 2048, 4096, 16) == 4 and splits(160, 2048, 4096, 16) == 1 and splits(192, 8192, 8192, 16) == 1
     for workgroups in (1, 8, 24, 64, 200):
         for length in range(1, 20000, 501):
             n = splits(workgroups, length, 32768, 16)
