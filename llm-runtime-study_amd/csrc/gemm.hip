@@ -1111,7 +1111,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_mid_kernel(
 // travel with every call as one word, so that nothing about them is kept in the library:
 //   bit 0      the kernel for 17..128 rows may be used (else such products take the kernels for other row counts)
 //   bit 1      the few-rows kernel loads its weights as whole 128-byte lines where the shape allows
-//   bits 4-7   workgroup shape of the kernel for 17..128 rows: 4, 6 or 8 waves (0: chosen here)
+//   bits 4-7   workgroup shape of the kernel for 17..128 rows: 4, 5, 6 or 8 waves (0: chosen here)
 //   bits 8-12  its number of K splits, 1..16 (0: chosen here)
 struct GemmTune {
   bool mid, lines;
@@ -1120,7 +1120,7 @@ struct GemmTune {
 constexpr int TUNE_DEFAULT = 3;
 static bool tune_ok(int word) {
   const int waves = (word >> 4) & 15, splits = (word >> 8) & 31;
-  return word >= 0 && (word >> 13) == 0 && (waves == 0 || waves == 4 || waves == 6 || waves == 8) && splits <= 16;
+  return word >= 0 && (word >> 13) == 0 && (waves == 0 || waves == 4 || waves == 5 || waves == 6 || waves == 8) && splits <= 16;
 }
 static GemmTune tune_of(int word) { return GemmTune{(word & 1) != 0, (word & 2) != 0, (word >> 4) & 15, (word >> 8) & 31}; }
 
@@ -1197,9 +1197,16 @@ static void choose_mid_shape(int n, int k, GemmTune tune, int& waves, int& split
   // Measured on MI355X (Qwen3-8B shapes, 32..64 rows).  A matrix with enough rows to give every compute
   // unit a workgroup is not divided along K: six waves (96 rows) a workgroup, or four where that fills the
   // chip clearly better; eight waves walking many slices were a third slower (gate_up, the LM head).
-  if ((!want_splits || want_splits == 1) && tiles_of(6) >= units && (!want_waves || want_waves == 4 || want_waves == 6)) {
+  // Five waves where the launch then takes a tenth fewer rows a compute unit (rounds of the chip times the
+  // rows of a workgroup) than with either: 34,816 rows are 363 workgroups of 96 rows or 544 of 64, two and
+  // three rounds, 192 rows a unit, but 436 of 80, two rounds, 160 (at 64 rows 89 -> 77 us).
+  if ((!want_splits || want_splits == 1) && tiles_of(6) >= units && (!want_waves || want_waves == 4 || want_waves == 5 || want_waves == 6)) {
     splits = 1;
     waves = want_waves ? want_waves : (fill_of(tiles_of(4)) > fill_of(tiles_of(6)) + 0.08 ? 4 : 6);
+    if (!want_waves) {
+      auto rows_a_unit = [&](int wv) { return (tiles_of(wv) + units - 1) / units * wv; };
+      if (10 * rows_a_unit(5) <= 9 * rows_a_unit(4) && 10 * rows_a_unit(5) <= 9 * rows_a_unit(6)) waves = 5;
+    }
     return;
   }
   // A narrower matrix: K is divided so that tiles x splits fills the units once (at least two slices a
@@ -1272,6 +1279,7 @@ static int launch_mid_mt(void* out, int mode, const bf16* a, const bf16* w, int 
     gemm_bf16_mid_kernel<MT, WV, SWIGLU><<<grid, WV * 64, bytes, s>>>(out, mode, a, w, m, n, k, lda, ldc, sums, scale);    \
   } while (0)
   if (waves == 4) MID_LAUNCH(4);
+  else if (waves == 5) MID_LAUNCH(5);
   else if (waves == 6) MID_LAUNCH(6);
   else MID_LAUNCH(8);
 #undef MID_LAUNCH

@@ -36,7 +36,7 @@ class KernelChoice:
     few_rows_max   rows up to which the few-rows kernels (and the norms folded into them) are used: 16 in
                    steps, since from 17 rows on other kernels are faster; the kernels themselves take 64
     mid            the kernel for 17..128 rows may be used
-    mid_waves, mid_splits   its workgroup shape (4, 6 or 8 waves) and number of K splits (0: its own choice)
+    mid_waves, mid_splits   its workgroup shape (4, 5, 6 or 8 waves) and number of K splits (0: its own choice)
     whole_lines    the few-rows kernel loads its weights as whole 128-byte lines where the shape allows
     library        bfloat16 products of more rows than these kernels are made for go to the vendor's matrix
                    library (as the reference leaves them to nn.Linear); else to this package's own kernel"""
@@ -51,8 +51,8 @@ class KernelChoice:
     def __post_init__(self):
         if not 1 <= self.few_rows_max <= 64:
             raise KernelError(f"the few-rows kernel takes 1..64 rows, got few_rows_max={self.few_rows_max}")
-        if self.mid_waves not in (0, 4, 6, 8) or not 0 <= self.mid_splits <= 16:
-            raise KernelError(f"the kernel for 17..128 rows has 4, 6 or 8 waves and 1..16 K splits (0: its own choice), got {self.mid_waves} and {self.mid_splits}")
+        if self.mid_waves not in (0, 4, 5, 6, 8) or not 0 <= self.mid_splits <= 16:
+            raise KernelError(f"the kernel for 17..128 rows has 4, 5, 6 or 8 waves and 1..16 K splits (0: its own choice), got {self.mid_waves} and {self.mid_splits}")
 
     @property
     def word(self) -> int:

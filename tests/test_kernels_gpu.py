@@ -289,7 +289,7 @@ def test_gemm(ops, dtype, m, n, k, mode):
 
 @pytest.mark.parametrize("m", [17, 32, 40, 48, 49, 64, 65, 96, 100, 128])
 @pytest.mark.parametrize("n,k", [(64, 256), (208, 512), (4096, 1024), (6144, 4096), (1040, 3328)])
-@pytest.mark.parametrize("waves,splits", [(0, 0), (4, 1), (6, 2), (8, 3), (4, 8)])
+@pytest.mark.parametrize("waves,splits", [(0, 0), (4, 1), (5, 1), (5, 3), (6, 2), (8, 3), (4, 8)])
 def test_gemm_of_17_to_64_rows(ops, m, n, k, waves, splits):
     """The kernel for 17..64 rows (K a multiple of 256): every workgroup shape, K divided between
     workgroups or not, ragged last tiles, all three output modes and the gated epilogue."""
