@@ -68,6 +68,86 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(void* __restrict__ out,
   }
 }
 
+// ------------------------------------------------- float32 FMA kernel for at most 16 rows
+// A decode step in float32: the tiled kernel above would fill one row of its 64 x 64 tiles in sixteen and walk K
+// sixteen values at a time.  Here a workgroup of 256 threads owns 256 / MR weight rows and all (at most MR) rows
+// of the input; a thread owns one output and adds its products up one after the other, k ascending from zero,
+// which is exactly the sum the tiled kernel makes: the two give the same bits, so a row's result still does not
+// depend on how many rows travel with it.  K is walked in slices of 64 through LDS (the weights as whole lines
+// of 256 bytes, the next slice on its way into registers while this one is multiplied).  K % 64 == 0.
+template <int MR>
+__global__ __launch_bounds__(256) void gemm_f32_few_rows_kernel(void* __restrict__ out, int mode, const float* __restrict__ a,
+                                                                 const float* __restrict__ w, const float* __restrict__ bias,
+                                                                 int m, int n, int k, int lda, int ldc) {
+  constexpr int CN = 256 / MR, BK = 64, PITCH = BK + 8;      // rows 288 bytes apart: 16-byte reads of consecutive rows at the full LDS rate
+  constexpr int W_LOADS = CN * BK / 4 / 256, A_LOADS = (MR * BK / 4 + 255) / 256;
+  static_assert(MR == 4 || MR == 8 || MR == 16, "4, 8 or 16 input rows a workgroup");
+  __shared__ __attribute__((aligned(16))) float ws[2][CN * PITCH];
+  __shared__ __attribute__((aligned(16))) float as[2][MR * PITCH];
+  const int tid = threadIdx.x;
+  const int n0 = blockIdx.x * CN;
+  const int col = tid % CN, row = tid / CN;                   // this thread's output: weight row n0 + col, input row `row`
+  // what this thread brings of a slice: 16 bytes of a weight row (and of an input row)
+  const float* wsrc[W_LOADS];
+  int wdst[W_LOADS];
+#pragma unroll
+  for (int i = 0; i < W_LOADS; ++i) {
+    const int piece = tid + i * 256, r = piece / (BK / 4), c = piece % (BK / 4);
+    const int gn = n0 + r < n ? n0 + r : n - 1;
+    wsrc[i] = w + (int64_t)gn * k + c * 4;
+    wdst[i] = r * PITCH + c * 4;
+  }
+  const float* asrc[A_LOADS];
+  int adst[A_LOADS];
+#pragma unroll
+  for (int i = 0; i < A_LOADS; ++i) {
+    const int piece = tid + i * 256, r = (piece / (BK / 4)) % MR, c = piece % (BK / 4);
+    asrc[i] = a + (int64_t)(r < m ? r : m - 1) * lda + c * 4;
+    adst[i] = r * PITCH + c * 4;
+  }
+  const bool brings_a = tid < MR * BK / 4 || A_LOADS > 1;
+  floatx4 wreg[W_LOADS], areg[A_LOADS];
+  auto load = [&](int k0) {
+#pragma unroll
+    for (int i = 0; i < W_LOADS; ++i) wreg[i] = *(const floatx4*)(wsrc[i] + k0);
+#pragma unroll
+    for (int i = 0; i < A_LOADS; ++i) areg[i] = *(const floatx4*)(asrc[i] + k0);
+  };
+  auto store = [&](int buf) {
+#pragma unroll
+    for (int i = 0; i < W_LOADS; ++i) *(floatx4*)(ws[buf] + wdst[i]) = wreg[i];
+    if (brings_a) {
+#pragma unroll
+      for (int i = 0; i < A_LOADS; ++i) *(floatx4*)(as[buf] + adst[i]) = areg[i];
+    }
+  };
+  float acc = 0.f;
+  load(0);
+  store(0);
+  const int slices = k / BK;
+  for (int slice = 0; slice < slices; ++slice) {
+    __syncthreads();                                           // slice `slice` is in its buffer; the other buffer is read by nobody
+    if (slice + 1 < slices) load((slice + 1) * BK);
+    const float* wr = ws[slice & 1] + col * PITCH;
+    const float* ar = as[slice & 1] + row * PITCH;
+#pragma unroll
+    for (int kk = 0; kk < BK; kk += 4) {
+      const floatx4 wv = *(const floatx4*)(wr + kk), av = *(const floatx4*)(ar + kk);
+      acc = fmaf(av[0], wv[0], acc);
+      acc = fmaf(av[1], wv[1], acc);
+      acc = fmaf(av[2], wv[2], acc);
+      acc = fmaf(av[3], wv[3], acc);
+    }
+    if (slice + 1 < slices) store((slice + 1) & 1);
+  }
+  const int gn = n0 + col;
+  if (row < m && gn < n) {
+    float v = acc;
+    if (bias) v += bias[gn];
+    emit<float>(out, mode, (int64_t)row * ldc + gn, v);
+  }
+}
+
 __device__ __forceinline__ float silu(float g) { return g / (1.0f + __expf(-g)); }
 
 // ------------------------------------------------------- bf16 MFMA kernel
@@ -1532,7 +1612,12 @@ LRS_API int lrs_gemm(void* out, int mode, const void* a, const void* w, const vo
     LRS_REQUIRE(!normed || eps > 0.f, "gemm: eps must be positive");
   }
   LRS_REQUIRE(normed || rows == nullptr, "gemm: a row gather needs the fused norm input");
-  if (dtype == LRS_F32) {
+  if (dtype == LRS_F32 && m <= 16 && k % 64 == 0 && lda % 4 == 0 && ((uintptr_t)a % 16) == 0 && ((uintptr_t)w % 16) == 0) {
+    // a decode step in float32: the same sums as the tiled kernel below makes, from a kernel made for few rows
+    if (m <= 4) gemm_f32_few_rows_kernel<4><<<(n + 63) / 64, 256, 0, s>>>(out, mode, (const float*)a, (const float*)w, (const float*)bias, m, n, k, lda, ldc);
+    else if (m <= 8) gemm_f32_few_rows_kernel<8><<<(n + 31) / 32, 256, 0, s>>>(out, mode, (const float*)a, (const float*)w, (const float*)bias, m, n, k, lda, ldc);
+    else gemm_f32_few_rows_kernel<16><<<(n + 15) / 16, 256, 0, s>>>(out, mode, (const float*)a, (const float*)w, (const float*)bias, m, n, k, lda, ldc);
+  } else if (dtype == LRS_F32) {
     dim3 grid((n + 63) / 64, (m + 63) / 64);
     gemm_tiled_kernel<float><<<grid, 256, 0, s>>>(out, mode, (const float*)a, (const float*)w,
                                                   (const float*)bias, m, n, k, lda, ldc);

@@ -525,6 +525,20 @@ def test_gemm_row_does_not_depend_on_batch(ops, dtype):
         torch.testing.assert_close(one.cpu(), full.cpu()[41:42], rtol=0, atol=0)
     else:                        # few rows take another kernel than many: equal beyond rounding only
         torch.testing.assert_close(one.cpu(), full.cpu()[41:42], rtol=1e-5, atol=1e-4)
+    if dtype == torch.float32:
+        # float32 steps of at most 16 rows have a kernel of their own (K a multiple of 64) that adds up in the
+        # tiled kernel's order: 3, 8 and 13 rows alone give the bits they have inside a batch of 70
+        a64 = torch.randn(70, 192, generator=g)
+        w64 = torch.randn(203, 192, generator=g)
+        bias = torch.randn(203, generator=g)
+        whole = torch.empty(70, 203, device="cuda")
+        ops.gemm(whole, dev(a64), dev(w64), dev(bias))
+        for first, rows in ((41, 3), (5, 8), (57, 13)):
+            few = torch.full((rows, 203), 0.25, device="cuda")
+            ops.gemm(few, dev(a64[first:first + rows]), dev(w64), dev(bias))
+            torch.testing.assert_close(few.cpu(), whole.cpu()[first:first + rows], rtol=0, atol=0)
+            ops.gemm(few, dev(a64[first:first + rows]), dev(w64), dev(bias), accumulate=True)
+            torch.testing.assert_close(few.cpu(), 2 * whole.cpu()[first:first + rows], rtol=0, atol=0)
     # strided input and output rows
     wide_in = dev(torch.cat((a, a), 1))
     wide_out = torch.zeros(70, 300, device="cuda")
