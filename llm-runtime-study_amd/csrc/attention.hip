@@ -60,7 +60,18 @@ __global__ __launch_bounds__(THREADS) void attention_generic_kernel(
       base = (page * nkv + kv_head) * page_size * d;
       const T* kr = k_pages + base + (int64_t)off * d;
       float dot = 0.f;
-      for (int i = 0; i < d; ++i) dot = fmaf(qs[i], to_float(kr[i]), dot);
+      if (sizeof(T) == 4 && d % 4 == 0 && ((uintptr_t)k_pages % 16) == 0) {
+        // float32 rows, 16 bytes a load; the products are added up in the same order as one by one
+        for (int i = 0; i < d; i += 4) {
+          const floatx4 kv = *(const floatx4*)((const float*)kr + i);
+          dot = fmaf(qs[i], kv[0], dot);
+          dot = fmaf(qs[i + 1], kv[1], dot);
+          dot = fmaf(qs[i + 2], kv[2], dot);
+          dot = fmaf(qs[i + 3], kv[3], dot);
+        }
+      } else {
+        for (int i = 0; i < d; ++i) dot = fmaf(qs[i], to_float(kr[i]), dot);
+      }
       score = dot * scale;
     }
     const float tile_max = block_max(score, scratch);
@@ -80,9 +91,34 @@ __global__ __launch_bounds__(THREADS) void attention_generic_kernel(
       const int dim = tid + c * THREADS;
       if (dim < d) {
         float a = acc[c] * alpha;
-        for (int j = 0; j < count; ++j) {
-          const float pj = probs[j];
-          if (pj != 0.f) a = fmaf(pj, to_float(v_pages[bases[j] + (int64_t)dim * page_size + offsets[j]]), a);
+        if (sizeof(T) == 4 && page_size % 4 == 0 && THREADS % 4 == 0 && ((uintptr_t)v_pages % 16) == 0) {
+          // four keys that lie side by side in a (transposed) page in one load of 16 bytes; added in key order as below
+          int j = 0;
+          for (; j + 4 <= count; j += 4) {
+            if (tile + j < lo) {                                 // keys before the window have no page to read from
+#pragma unroll
+              for (int e = 0; e < 4; ++e) {
+                const float pj = probs[j + e];
+                if (pj != 0.f) a = fmaf(pj, to_float(v_pages[bases[j + e] + (int64_t)dim * page_size + offsets[j + e]]), a);
+              }
+              continue;
+            }
+            const floatx4 vv = *(const floatx4*)((const float*)v_pages + bases[j] + (int64_t)dim * page_size + offsets[j]);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+              const float pj = probs[j + e];
+              if (pj != 0.f) a = fmaf(pj, vv[e], a);
+            }
+          }
+          for (; j < count; ++j) {
+            const float pj = probs[j];
+            if (pj != 0.f) a = fmaf(pj, to_float(v_pages[bases[j] + (int64_t)dim * page_size + offsets[j]]), a);
+          }
+        } else {
+          for (int j = 0; j < count; ++j) {
+            const float pj = probs[j];
+            if (pj != 0.f) a = fmaf(pj, to_float(v_pages[bases[j] + (int64_t)dim * page_size + offsets[j]]), a);
+          }
         }
         acc[c] = a;
       }
