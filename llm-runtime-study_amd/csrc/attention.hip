@@ -919,7 +919,7 @@ __global__ __launch_bounds__(256, D <= 128 ? 2 : 1) void attention_prefill_bf16_
 // tile to the others; the fetches of the tile after it stay in flight.  The fetches are written in
 // assembly because the compiler would wait for all of them before any LDS read it cannot tell apart.
 template <int QB>
-__global__ __launch_bounds__(256, 2) void attention_prefill_d128_bf16_kernel(
+__global__ __launch_bounds__(512) void attention_prefill_d128_bf16_kernel(
     bf16* __restrict__ out, int out_stride, const bf16* __restrict__ q, int q_stride,
     const bf16* __restrict__ k_pages, const bf16* __restrict__ v_pages,
     const int* __restrict__ block_table, int table_stride, const int* __restrict__ token_request,
@@ -1004,12 +1004,16 @@ __global__ __launch_bounds__(256, 2) void attention_prefill_d128_bf16_kernel(
       }
     }
   };
+  // (a kv group of five to eight heads brings as many waves, so that one walk over the keys serves them all;
+  // the first four waves bring the tiles in)
   auto fetch_keys = [&](const char* const (&kbase)[2], int stage) {      // two fetches a wave
+    if (wave >= 4) return;
 #pragma unroll
     for (int half = 0; half < 2; ++half)
       fetch_to_lds(kbase[half], key_offset, keys_address + (unsigned)(stage * KBYTES + (wave + 4 * half) * KBLOCK));
   };
   auto fetch_values = [&](const char* const (&vbase)[2], int stage) {    // two fetches a wave
+    if (wave >= 4) return;
 #pragma unroll
     for (int half = 0; half < 2; ++half)
       fetch_to_lds(vbase[half], value_offset, values_address + (unsigned)(stage * VSTAGE + half * VHALF + wave * 1024));
@@ -1312,7 +1316,7 @@ LRS_API int lrs_attention_prefill(void* out, int out_stride, const void* q, int 
   LRS_REQUIRE(window >= 0, "attention_prefill: window must be >= 0 (0 = none)");
   LRS_REQUIRE(q_stride % 8 == 0 && ((uintptr_t)q % 16) == 0 && out_stride % 4 == 0 && ((uintptr_t)out % 8) == 0,
               "attention_prefill: q rows must be 16-byte and out rows 8-byte aligned");
-  // always four waves: with fewer heads in a kv group the spare waves still help to bring tiles in
+  // four waves (with fewer heads in a kv group the spare waves still help to bring tiles in), more only below
   LRS_REQUIRE(splits >= 1 && splits <= 64 && (splits == 1 || (part_o && part_ml && tokens > 0)),
               "attention_prefill: splits=%d (1..64) need partial buffers and the number of tokens", splits);
   LRS_REQUIRE(splits == 1 || ((uintptr_t)part_o % 16) == 0, "attention_prefill: part_o must be 16-byte aligned");
@@ -1341,6 +1345,10 @@ LRS_API int lrs_attention_prefill(void* out, int out_stride, const void* q, int 
     case 96: LAUNCH(96); break;
     case 128:
       // head size 128 has a kernel of its own, whose tiles go from memory straight into LDS
+      // A kv group of five to eight heads: a wave for every head and one walk over the keys instead of two, while
+      // the launch is small (measured, 40 heads on 8: 512 tokens 28.9 -> 19.6 us, 512 tokens after 1,536 88 -> 54 us;
+      // but 2,048 tokens 113 -> 129 us: a full chip does better with the smaller workgroups, three to a unit)
+      if (nq / nkv > 4 && (int64_t)n_blocks * nkv * splits <= 2 * compute_units()) block = dim3((nq / nkv < 8 ? nq / nkv : 8) * WAVE);
       if (max_count <= 16)
         attention_prefill_d128_bf16_kernel<1><<<grid, block, 0, s>>>(
             (bf16*)out, out_stride, (const bf16*)q, q_stride, (const bf16*)k_pages, (const bf16*)v_pages, block_table, table_stride,

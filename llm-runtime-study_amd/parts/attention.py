@@ -99,17 +99,34 @@ class GQAAttention(Part):
         return max(1, min(wanted, length_class(longest) // 256, 64), -(-bound // (4096 * page_size)))
 
     @staticmethod
-    def _prefill_splits(workgroups: int, longest: int, outputs: int) -> int:
-        """Into how many workgroups the keys of every query group of a ragged step are divided: one,
-        unless the groups alone leave compute units idle and the contexts are long (a last portion of
-        a long prompt, single tokens beside a portion); then towards eight workgroups per unit, at
-        least 1,024 keys each, and partial results (float32, `outputs` values per split) of at most
-        256 MB.  Measured on MI355X at 32,768 tokens of context: 1 token 1,161 -> 57 us with 32
-        splits, 64 tokens 1,165 -> 105 us with 16, 512 tokens 1,186 -> 576 us with 8."""
+    def _prefill_splits(workgroups: int, longest: int, outputs: int, heads_per_group: int = 4) -> int:
+        """Into how many workgroups the keys of every query group of a ragged step are divided: one, unless
+        the groups alone leave compute units idle (a last portion of a prompt, a short portion after a long
+        context).  Partial results (float32, `outputs` values per split) stay within 256 MB.  Measured on
+        MI355X, 32 query heads on 8 kv heads:
+          * contexts of 16,384 tokens and more: towards eight workgroups a unit, at least 1,024 keys each
+            (32,768 tokens of context: 1 token 1,161 -> 57 us with 32 splits, 64 tokens 1,165 -> 105 us with
+            16, 512 tokens 1,186 -> 576 us with 8);
+          * shorter contexts: towards two workgroups a unit, at least 256 keys each, and none from two a unit
+            on (2,048 tokens of context: 64 tokens 42.5 -> 18.6 us with 8 splits, 256 tokens 43.2 -> 32.4 with
+            4, 512 tokens 87.5 -> 76.4 with 2, but 1,024 tokens 96.8 -> 127 and 2,032 tokens 111 -> 173 with 2:
+            what the merge reads and writes grows with the tokens, what a split saves with the context).
+        A kv group of five to eight heads walks the keys once with a wave for every head while the launch is at
+        most two workgroups a unit; that walk is short enough that one workgroup a unit is the aim (40 heads on
+        8: 512 tokens after 1,536 54 us undivided against 72 with 2; 256 tokens 51 -> 43 with 2, 128 tokens
+        after 8,064 177 -> 59 with 4, 64 tokens after 2,000 50 -> 22 with 8); from 16,384 tokens of context on the rule
+        for long contexts holds for them too (512 tokens after 32,256: 697 us undivided, 617 with 8)."""
         units = ops.compute_units()
+        within = (64 << 20) // max(outputs, 1)
         if workgroups >= 4 * units:
             return 1
-        return max(1, min(-(-8 * units // workgroups), longest // 1024, 32, (64 << 20) // max(outputs, 1)))
+        if heads_per_group > 4 and workgroups <= units and longest < 16384:
+            return max(1, min(-(-units // workgroups), longest // 256, 32, within))
+        if longest >= 16384:
+            return max(1, min(-(-8 * units // workgroups), longest // 1024, 32, within))
+        if workgroups >= 2 * units:
+            return 1
+        return max(1, min(-(-2 * units // workgroups), longest // 256, 32, within))
 
     PREPARE_INSIDE_ROWS = 16     # rows of a decode step up to which the attention kernel prepares q, k and v itself
 
@@ -184,7 +201,7 @@ class GQAAttention(Part):
             rest = ctx.memo.get("rows_after_singles")
             if rest is None:
                 rest = ctx.memo["rows_after_singles"] = (ctx.token_request[singles:], ctx.positions[singles:])
-            splits = self._prefill_splits(ctx.num_qblocks * kv_heads, longest, (t - singles) * nq * d)
+            splits = self._prefill_splits(ctx.num_qblocks * kv_heads, longest, (t - singles) * nq * d, nq // kv_heads)
             part_o = part_ml = None
             if splits > 1:
                 part_o = ctx.scratch("attn_part_o", (t - singles, nq * splits * d), torch.float32)

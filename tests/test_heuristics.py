@@ -54,8 +54,14 @@ def test_prefill_splits_only_where_groups_leave_the_chip_idle(monkeypatch):
     assert splits(256, 33216, 1 << 20) == 8             # a 512-token portion after 32,704 tokens
     assert splits(32, 32768, 1 << 20) == 32             # a 64-token portion
     assert splits(8, 32768, 1 << 16) == 32              # one token: as many as allowed
-    assert splits(8, 2048, 1 << 16) == 2                # at least 1,024 keys each
     assert splits(8, 1 << 20, 16 << 20) == 4            # partial results stay within 256 MB
+    # contexts under 16,384 tokens: towards two workgroups a unit, at least 256 keys each, none from two a unit on
+    assert splits(8, 2048, 1 << 16) == 8 and splits(32, 2064, 1 << 20) == 8 and splits(128, 2048, 1 << 20) == 4
+    assert splits(256, 2048, 1 << 20) == 2 and splits(256, 4096, 1 << 20) == 2 and splits(1016, 2047, 1 << 20) == 1
+    assert splits(64, 700, 1 << 20) == 2                # 256 keys each
+    # kv groups of five to eight heads (one walk with a wave a head): one workgroup a unit is the aim
+    assert splits(256, 8192, 1 << 20, 5) == 1 and splits(128, 2048, 1 << 20, 5) == 2 and splits(32, 2064, 1 << 20, 8) == 8
+    assert splits(512, 2048, 1 << 20, 5) == 1 and splits(256, 33216, 1 << 20, 5) == 8 and splits(512, 33216, 1 << 20, 5) == 4
 
 
 def test_shapes_of_the_kernel_for_17_to_64_rows():
