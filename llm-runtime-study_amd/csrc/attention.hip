@@ -918,8 +918,8 @@ __global__ __launch_bounds__(256, D <= 128 ? 2 : 1) void attention_prefill_bf16_
 // The wave that fetched a tile waits for its own fetches (vmcnt) before the barrier that opens the
 // tile to the others; the fetches of the tile after it stay in flight.  The fetches are written in
 // assembly because the compiler would wait for all of them before any LDS read it cannot tell apart.
-template <int QB>
-__global__ __launch_bounds__(512) void attention_prefill_d128_bf16_kernel(
+template <int QB, bool MANY_WAVES, bool IDLE_WAVES>
+__global__ __launch_bounds__(MANY_WAVES ? 512 : 256, MANY_WAVES ? 1 : 2) void attention_prefill_d128_bf16_kernel(
     bf16* __restrict__ out, int out_stride, const bf16* __restrict__ q, int q_stride,
     const bf16* __restrict__ k_pages, const bf16* __restrict__ v_pages,
     const int* __restrict__ block_table, int table_stride, const int* __restrict__ token_request,
@@ -1200,7 +1200,7 @@ __global__ __launch_bounds__(512) void attention_prefill_d128_bf16_kernel(
       if (pending == 4) fetched_then_barrier<4>();
       else if (pending == 2) fetched_then_barrier<2>();
       else fetched_then_barrier<0>();
-      scores(0, sa);
+      if (!IDLE_WAVES || active) scores(0, sa);
       asm volatile("s_barrier" ::: "memory");                  // everyone has read the first keys: their stage may be filled again
     }
     int tile = first_tile, stage = 0;                          // stage = (tile - first_tile) % 3
@@ -1228,6 +1228,13 @@ __global__ __launch_bounds__(512) void attention_prefill_d128_bf16_kernel(
     // that needs the mask, or whose weights came out too large, or one of the last three, leaves it and takes
     // the long way.  The scores of the tile at hand are in sa at the top of every turn.
     const int fast_begin = whole_begin, fast_end = whole_end < last_tile - 2 ? whole_end : last_tile - 2;
+    // A wave without a head (a kv group whose heads are no multiple of the waves: IDLE_WAVES, a kernel of its own
+    // so that the others keep their registers) only brings its share of the tiles in and keeps the workgroup's
+    // barriers: one a tile, as the others.
+    if (IDLE_WAVES && !active) {
+      while (tile <= last_tile) turn_over(ask_ahead(std::false_type{}));
+      continue;
+    }
     for (;;) {
       bool asked = false;                                      // the turn's fetches have been asked for already
       // one way out of the inner loop only, at its top, before anything of the turn has happened to the accumulators
@@ -1348,15 +1355,24 @@ LRS_API int lrs_attention_prefill(void* out, int out_stride, const void* q, int 
       // A kv group of five to eight heads: a wave for every head and one walk over the keys instead of two, while
       // the launch is small (measured, 40 heads on 8: 512 tokens 28.9 -> 19.6 us, 512 tokens after 1,536 88 -> 54 us;
       // but 2,048 tokens 113 -> 129 us: a full chip does better with the smaller workgroups, three to a unit)
-      if (nq / nkv > 4 && (int64_t)n_blocks * nkv * splits <= 2 * compute_units()) block = dim3((nq / nkv < 8 ? nq / nkv : 8) * WAVE);
-      if (max_count <= 16)
-        attention_prefill_d128_bf16_kernel<1><<<grid, block, 0, s>>>(
-            (bf16*)out, out_stride, (const bf16*)q, q_stride, (const bf16*)k_pages, (const bf16*)v_pages, block_table, table_stride,
-            token_request, positions, qblock_token0, qblock_count, n_blocks, chunk, nq, nkv, page_size, scale, window, splits, part_o, part_ml);
-      else
-        attention_prefill_d128_bf16_kernel<2><<<grid, block, 0, s>>>(
-            (bf16*)out, out_stride, (const bf16*)q, q_stride, (const bf16*)k_pages, (const bf16*)v_pages, block_table, table_stride,
-            token_request, positions, qblock_token0, qblock_count, n_blocks, chunk, nq, nkv, page_size, scale, window, splits, part_o, part_ml);
+      {
+        const bool many = nq / nkv > 4 && (int64_t)n_blocks * nkv * splits <= 2 * compute_units();
+        if (many) block = dim3((nq / nkv < 8 ? nq / nkv : 8) * WAVE);
+#define D128(QB, MANY, IDLE)                                                                                                      \
+        attention_prefill_d128_bf16_kernel<QB, MANY, IDLE><<<grid, block, 0, s>>>(                                                    \
+            (bf16*)out, out_stride, (const bf16*)q, q_stride, (const bf16*)k_pages, (const bf16*)v_pages, block_table, table_stride, \
+            token_request, positions, qblock_token0, qblock_count, n_blocks, chunk, nq, nkv, page_size, scale, window, splits, part_o, part_ml)
+#define D128_OF(QB)                                      \
+        if (many && idle) D128(QB, true, true);          \
+        else if (many) D128(QB, true, false);            \
+        else if (idle) D128(QB, false, true);            \
+        else D128(QB, false, false)
+        const bool idle = (nq / nkv) % (int)(block.x / WAVE) != 0;   // some wave of some pass has no head
+        if (max_count <= 16) { D128_OF(1); }
+        else { D128_OF(2); }
+#undef D128_OF
+#undef D128
+      }
       break;
     case 192: LAUNCH(192); break;
     default: return lrs_fail("attention_prefill: head_dim %d has no matrix-core kernel (32, 64, 96, 128, 192)", d);
