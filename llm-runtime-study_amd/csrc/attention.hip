@@ -1302,10 +1302,20 @@ static int compute_units() {
 // Largest number of tokens in one query group of lrs_attention_prefill.
 LRS_API int lrs_attention_prefill_group() { return 32; }
 
-// The group size that serves a step of `tokens` tokens best: groups of 16 while those of 32 would
-// not give every compute unit its two workgroups several times over (measured on MI355X: 16 is
-// faster up to 2,048 tokens, 32 beyond).
-LRS_API int lrs_attention_prefill_group_for(int tokens) { return tokens <= 8 * compute_units() ? 16 : 32; }
+// The group size that serves a step of `tokens` tokens best, the longest context among them being `longest`
+// (0: not known): groups of 16 while those of 32 would not give every compute unit its two workgroups several
+// times over (measured on MI355X: a fresh prompt of up to 2,048 tokens is faster with 16, longer ones with 32);
+// but groups of 32 already for 2,048 tokens behind as many or more, and for 1,024 behind three times as many: the
+// walks are long then, and a wave with 32 queries does half as much beside its products for every key (2,048
+// tokens after 2,048 / 6,144 / 30,720: 173 / 366 / 1,412 us with groups of 16, 142 / 272 / 1,071 with 32; 1,024
+// after 7,168: 204 against 181 us; 512 after 7,680 stay with 16: 117 against 140 us).
+LRS_API int lrs_attention_prefill_group_for(int tokens, int longest) {
+  const int units = compute_units();
+  if (tokens > 8 * units) return 32;
+  if (tokens >= 8 * units && longest >= 2 * tokens) return 32;
+  if (tokens >= 4 * units && longest >= 4 * tokens) return 32;
+  return 16;
+}
 
 // Any step in bf16.  qblock_token0 / qblock_count [n_blocks]: first token and number of tokens
 // (1..lrs_attention_prefill_group()) of each group of consecutive tokens of one request.

@@ -355,7 +355,7 @@ class ModelRunner:
             # after them, and count their tokens from there.
             singles = next(i for i, n in enumerate(ctx.host_q_lens) if n != 1)
             ctx.single_rows = singles
-            starts, size = cu[:ctx.R + 1], min(self.query_group, ops.attention_prefill_group(cursor - singles))
+            starts, size = cu[:ctx.R + 1], min(self.query_group, ops.attention_prefill_group(cursor - singles, ctx.max_k))
             blocks = [(int(pos[min(t0 + size, int(starts[i + 1])) - 1]), t0 - singles, min(size, int(starts[i + 1]) - t0))
                       for i in range(singles, ctx.R) for t0 in range(int(starts[i]), int(starts[i + 1]), size)]
             blocks.sort(key=lambda b: -b[0])

@@ -117,7 +117,7 @@ _SIGNATURES = {
     "lrs_gemm_lines_splits": (c_int, [c_int, c_int, c_int]),
     "lrs_gemm_lines_split_pays": (c_int, [c_int, c_int, c_int]),
     "lrs_attention_prefill_group": (c_int, []),
-    "lrs_attention_prefill_group_for": (c_int, [c_int]),
+    "lrs_attention_prefill_group_for": (c_int, [c_int, c_int]),
     "lrs_choose_tokens": (c_int, [c_void_p, c_void_p, c_int64, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p]),
     "lrs_choose_tokens_split": (c_int, [c_void_p, c_void_p, c_int64, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p]),
     "lrs_choose_tokens_static": (c_int, [c_void_p, c_void_p, c_int64, c_int, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p]),
@@ -867,12 +867,13 @@ def compute_units() -> int:
     return library().lrs_compute_units()
 
 
-def attention_prefill_group(tokens: int | None = None) -> int:
+def attention_prefill_group(tokens: int | None = None, longest: int = 0) -> int:
     """Most tokens in one query group of attention_prefill(); with `tokens`, the group size that
-    serves a step of that many tokens best (smaller groups fill the chip when there are few)."""
+    serves a step of that many tokens best (smaller groups fill the chip when there are few), given the
+    longest context (position + 1) among them, if known (larger groups pay earlier behind a long context)."""
     if tokens is None:
         return library().lrs_attention_prefill_group()
-    return library().lrs_attention_prefill_group_for(tokens)
+    return library().lrs_attention_prefill_group_for(tokens, longest)
 
 
 # --------------------------------------------------------------- sampling

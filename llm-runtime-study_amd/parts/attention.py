@@ -102,13 +102,13 @@ class GQAAttention(Part):
     def _prefill_splits(workgroups: int, longest: int, outputs: int, heads_per_group: int = 4) -> int:
         """Into how many workgroups the keys of every query group of a ragged step are divided: one, unless
         the groups alone leave compute units idle (a last portion of a prompt, a short portion after a long
-        context).  Partial results (float32, `outputs` values per split) stay within 256 MB.  Measured on
+        context), and never from two workgroups a unit on.  Partial results (float32, `outputs` values per split)
+        stay within 256 MB.  Measured on
         MI355X, 32 query heads on 8 kv heads:
           * contexts of 16,384 tokens and more: towards eight workgroups a unit, at least 1,024 keys each
             (32,768 tokens of context: 1 token 1,161 -> 57 us with 32 splits, 64 tokens 1,165 -> 105 us with
             16, 512 tokens 1,186 -> 576 us with 8);
-          * shorter contexts: towards two workgroups a unit, at least 256 keys each, and none from two a unit
-            on (2,048 tokens of context: 64 tokens 42.5 -> 18.6 us with 8 splits, 256 tokens 43.2 -> 32.4 with
+          * shorter contexts: towards two workgroups a unit, at least 256 keys each (2,048 tokens of context: 64 tokens 42.5 -> 18.6 us with 8 splits, 256 tokens 43.2 -> 32.4 with
             4, 512 tokens 87.5 -> 76.4 with 2, but 1,024 tokens 96.8 -> 127 and 2,032 tokens 111 -> 173 with 2:
             what the merge reads and writes grows with the tokens, what a split saves with the context).
         A kv group of five to eight heads walks the keys once with a wave for every head while the launch is at
@@ -118,14 +118,12 @@ class GQAAttention(Part):
         for long contexts holds for them too (512 tokens after 32,256: 697 us undivided, 617 with 8)."""
         units = ops.compute_units()
         within = (64 << 20) // max(outputs, 1)
-        if workgroups >= 4 * units:
+        if workgroups >= 2 * units:      # (2,048 tokens in groups of 32 after 30,720: 1,071 us undivided, 1,115 with 2)
             return 1
         if heads_per_group > 4 and workgroups <= units and longest < 16384:
             return max(1, min(-(-units // workgroups), longest // 256, 32, within))
         if longest >= 16384:
             return max(1, min(-(-8 * units // workgroups), longest // 1024, 32, within))
-        if workgroups >= 2 * units:
-            return 1
         return max(1, min(-(-2 * units // workgroups), longest // 256, 32, within))
 
     PREPARE_INSIDE_ROWS = 16     # rows of a decode step up to which the attention kernel prepares q, k and v itself

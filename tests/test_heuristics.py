@@ -61,7 +61,20 @@ def test_prefill_splits_only_where_groups_leave_the_chip_idle(monkeypatch):
     assert splits(64, 700, 1 << 20) == 2                # 256 keys each
     # kv groups of five to eight heads (one walk with a wave a head): one workgroup a unit is the aim
     assert splits(256, 8192, 1 << 20, 5) == 1 and splits(128, 2048, 1 << 20, 5) == 2 and splits(32, 2064, 1 << 20, 8) == 8
-    assert splits(512, 2048, 1 << 20, 5) == 1 and splits(256, 33216, 1 << 20, 5) == 8 and splits(512, 33216, 1 << 20, 5) == 4
+    assert splits(512, 2048, 1 << 20, 5) == 1 and splits(256, 33216, 1 << 20, 5) == 8 and splits(512, 33216, 1 << 20, 5) == 1
+
+
+def test_query_groups_of_32_behind_long_contexts():
+    """`lrs_attention_prefill_group_for`: 16 queries a group for fresh prompts up to 2,048 tokens, 32 beyond, and 32
+    already for portions of 2,048 (1,024) tokens whose context is twice (four times) as long."""
+    from llm_runtime_study_amd.kernels import ops
+
+    if ops.compute_units() not in (0, 256):
+        return
+    group = ops.attention_prefill_group
+    assert group(512) == 16 and group(2048) == 16 and group(2049) == 32 and group(2048, 2048) == 16
+    assert group(2048, 4096) == 32 and group(2047, 32768) == 32 and group(1024, 8192) == 32 and group(1024, 2048) == 16
+    assert group(1023, 32768) == 16 and group(512, 8192) == 16
 
 
 def test_shapes_of_the_kernel_for_17_to_64_rows():
