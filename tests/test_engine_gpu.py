@@ -298,7 +298,7 @@ def test_graphs_of_large_batches_hold_library_products(folders):
         for index in range(20):
             admit(index)
         for step in range(24):
-            if step in (3, 4, 5, 9, 10, 11, 12, 13, 14, 15, 16, 17, 18, 19, 20):     # 20 -> 35 requests: buckets 32 and 64
+            if step in (3, 4, 5, 9, 10, 11, 12, 13, 14, 15, 16, 17, 18, 19, 20):     # 20 -> 35 requests: buckets 32 and 48
                 admit(100 + step)
             if step == 22:                                                           # ... and down to 15: the own kernels' graphs
                 for index in sorted(live)[:20]:
@@ -312,13 +312,13 @@ def test_graphs_of_large_batches_hold_library_products(folders):
             assert torch.equal(a, b), f"step {step} with {len(order)} requests: graph replay differs from the eager step"
             for row, i in enumerate(order):
                 live[i] = (live[i][0], int(a[row].argmax()))
-    assert graphed.graph_replays + graphed.graph_captures == 24 and {key[0] for key in graphed._graphs} == {16, 32, 64}
+    assert graphed.graph_replays + graphed.graph_captures == 24 and {key[0] for key in graphed._graphs} == {16, 32, 48}
     graphed.drop_graphs()
 
 
 def test_graphs_of_up_to_128_rows_hold_this_packages_kernels(tmp_path):
     """A model whose matrices suit the kernel for 17..128 rows (every K a multiple of 256): batches of 40 to 100
-    requests run as graphs of 64 and 128 rows of this package's kernels alone, and every replay gives the
+    requests run as graphs of 48, 64, 96 and 128 rows of this package's kernels alone, and every replay gives the
     logits of the same step run eagerly, bit for bit; the logits agree with the float32 path."""
     from llm_runtime_study_amd.cache import CacheManager
     from llm_runtime_study_amd.config import config_from_dict
@@ -356,7 +356,7 @@ def test_graphs_of_up_to_128_rows_hold_this_packages_kernels(tmp_path):
         for index in range(40):
             admit(index)
         for step in range(12):
-            for extra in range(6 if step < 10 else 0):                 # 40 -> 100 requests: buckets 64 and 128
+            for extra in range(6 if step < 10 else 0):                 # 40 -> 100 requests: buckets 48, 64, 96 and 128
                 admit(1000 + step * 10 + extra)
             order = sorted(live)
             a = eager.step([StepEntry(live[i][0][0], [live[i][1]], [0]) for i in order]).clone()
@@ -368,7 +368,7 @@ def test_graphs_of_up_to_128_rows_hold_this_packages_kernels(tmp_path):
             assert error < 0.03, f"step {step}: bfloat16 logits are {float(error):.3f} of the float32 logits away"
             for row, i in enumerate(order):
                 live[i] = (live[i][0], int(c[row].argmax()))
-    assert graphed.graph_replays + graphed.graph_captures == 12 and {key[0] for key in graphed._graphs} == {64, 128}
+    assert graphed.graph_replays + graphed.graph_captures == 12 and {key[0] for key in graphed._graphs} == {48, 64, 96, 128}
     graphed.drop_graphs()
 
 
