@@ -179,6 +179,25 @@ def lds(args) -> None:
         print(f"lds rows {stride:3d} bytes apart: {seconds * 1e3:7.3f} ms  {per_cycle:6.1f} bytes a cycle and compute unit (at 2.4 GHz)", flush=True)
 
 
+def lines(args) -> None:
+    """What one compute unit, and many, stream from memory with 16-byte loads, by the lines that 16 neighbouring
+    lanes touch: 16 (the order of a matrix-core fragment: a lane's row is lane % 16), 2 (whole lines) or 4 (64
+    bytes of a row to four neighbouring lanes)."""
+    data = torch.randint(0, 1 << 30, (2048 << 18,), dtype=torch.int32, device="cuda")      # 2 GB, walked region by region: no call finds its bytes in a cache
+    sink = torch.zeros(256, dtype=torch.int32, device="cuda")
+    names = ("fragment order", "whole lines", "a row to four lanes")
+    for blocks in _ints(args.blocks):
+        for threads in (256, 1024):
+            for kilobytes in (256, 1024):
+                span = blocks * (kilobytes << 8)                                            # int32 elements a call
+                regions = data.numel() // span
+                for pattern in range(3):
+                    seconds = _time(lambda i: ops.probe_lines(data[(i % regions) * span:(i % regions + 1) * span], sink, blocks, threads, kilobytes << 10, pattern),
+                                    args.repeats)
+                    print(f"lines {blocks:4d} workgroups of {threads:4d} threads, {kilobytes:4d} KB each, {names[pattern]:20s}: {seconds * 1e6:7.1f} us  "
+                          f"{(kilobytes << 10) / seconds / 1e9:6.1f} GB/s a workgroup  {blocks * (kilobytes << 10) / seconds / 1e9:7.0f} GB/s", flush=True)
+
+
 def mfma(args) -> None:
     """What the matrix cores sustain alone and with vector instructions of the same wave between the products."""
     units, iters = ops.compute_units(), 4000
@@ -192,7 +211,7 @@ def mfma(args) -> None:
 
 def main(argv=None) -> int:
     parser = argparse.ArgumentParser(prog="python -m llm_runtime_study_amd.kernels.microbench", description=__doc__.split("\n\n")[0])
-    parser.add_argument("kernel", choices=["attention_prefill", "attention_decode", "gemm", "memory", "sampling", "lds", "mfma"])
+    parser.add_argument("kernel", choices=["attention_prefill", "attention_decode", "gemm", "memory", "sampling", "lds", "mfma", "lines"])
     parser.add_argument("--heads", type=int, default=32)
     parser.add_argument("--kv-heads", type=int, default=8)
     parser.add_argument("--head-dim", type=int, default=128)
@@ -213,7 +232,7 @@ def main(argv=None) -> int:
     parser.add_argument("--fragment-loads", action="store_true", help="gemm: the few-rows kernel loads weights and activations as MFMA fragments (64 bytes of 16 rows), not as whole lines")
     parser.add_argument("--mid-sweep", default="", help="gemm: also time the kernel for 17..128 rows with 4, 6 and 8 waves at these numbers of K splits")
     parser.add_argument("--megabytes", default="32,200,1200", help="memory: sizes of the buffers read")
-    parser.add_argument("--blocks", default="512,2048,8192", help="memory: numbers of workgroups")
+    parser.add_argument("--blocks", default="512,2048,8192", help="memory, lines: numbers of workgroups (lines: try 8,64,256,512)")
     parser.add_argument("--repeats", type=int, default=20)
     args = parser.parse_args(argv)
     if not torch.cuda.is_available():
@@ -221,7 +240,7 @@ def main(argv=None) -> int:
         return 2
     ops.library()
     {"attention_prefill": attention_prefill, "attention_decode": attention_decode, "gemm": gemm, "memory": memory, "sampling": sampling, "lds": lds,
-     "mfma": mfma}[args.kernel](args)
+     "mfma": mfma, "lines": lines}[args.kernel](args)
     return 0
 
 

@@ -13,7 +13,7 @@ import functools
 from dataclasses import dataclass
 import ctypes
 import struct
-from ctypes import c_char_p, c_float, c_int, c_int64, c_void_p, POINTER, byref
+from ctypes import c_char_p, c_float, c_int, c_int64, c_size_t, c_void_p, POINTER, byref
 
 import torch
 
@@ -96,6 +96,7 @@ _SIGNATURES = {
     "lrs_stream_read": (c_int, [c_void_p, c_int64, c_void_p, c_int, c_void_p]),
     "lrs_probe_lds": (c_int, [c_void_p, c_int, c_int, c_int, c_void_p]),
     "lrs_probe_mfma": (c_int, [c_void_p, c_int, c_int, c_int, c_int, c_void_p]),
+    "lrs_probe_lines": (c_int, [c_void_p, c_size_t, c_void_p, c_int, c_int, c_size_t, c_int, c_void_p]),
     "lrs_gemm_prepare": (c_int, []),
     "lrs_library_gemm_prepare": (c_int, []),
     "lrs_library_gemm": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p]),
@@ -327,6 +328,14 @@ def probe_lds(sink: torch.Tensor, blocks: int, iters: int, stride: int) -> None:
     """`blocks` workgroups read LDS `iters` x 8 times, 16 bytes a lane, rows `stride` bytes apart (microbench lds)."""
     _need(sink.dtype == torch.int32 and sink.numel() >= 256, "probe_lds: an int32 sink of 256 elements")
     _launch("lrs_probe_lds", _dev(sink, "sink"), blocks, iters, stride, _stream())
+
+
+def probe_lines(data: torch.Tensor, sink: torch.Tensor, blocks: int, threads: int, bytes_each: int, pattern: int) -> None:
+    """Measurement only: `blocks` workgroups stream `bytes_each` bytes each of `data` with 16-byte loads in the lane
+    order `pattern` (0 fragment order, 1 whole lines, 2 a row to four neighbouring lanes)."""
+    _need(sink.dtype == torch.int32 and sink.numel() >= 256, "probe_lines: an int32 sink of 256 elements")
+    _need(data.is_contiguous(), "probe_lines: data must be contiguous")
+    _launch("lrs_probe_lines", _dev(data, "data"), data.numel() * data.element_size(), _dev(sink, "sink"), blocks, threads, bytes_each, pattern, _stream())
 
 
 def probe_mfma(sink: torch.Tensor, blocks: int, iters: int, valu: int, exps: bool) -> None:
