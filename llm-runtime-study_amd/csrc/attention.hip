@@ -925,7 +925,7 @@ __global__ __launch_bounds__(MANY_WAVES ? 512 : 256, MANY_WAVES ? 1 : 2) void at
     const int* __restrict__ block_table, int table_stride, const int* __restrict__ token_request,
     const int* __restrict__ positions, const int* __restrict__ qblock_token0,
     const int* __restrict__ qblock_count, int n_blocks, int chunk, int nq, int nkv, int page_size, float scale,
-    int window, int splits, float* __restrict__ part_o, float* __restrict__ part_ml) {
+    int window, int splits, float* __restrict__ part_o, float* __restrict__ part_ml, int prepare_q, DecodePrep prep) {
   constexpr int D = 128, DS = D / 32, DB = D / 16, STAGES = 3;
   constexpr int KBLOCK = 1024 + 32, KBYTES = 8 * KBLOCK, VHALF = 16 * D * 2 + 16, VBYTES = 2 * VHALF;
   constexpr int VSTAGE = (VBYTES + 63) / 64 * 64;
@@ -1040,9 +1040,19 @@ __global__ __launch_bounds__(MANY_WAVES ? 512 : 256, MANY_WAVES ? 1 : 2) void at
       lo[b] = (window > 0 && pos[b] - window + 1 > 0) ? pos[b] - window + 1 : 0;
       run_max[b] = -INFINITY;
       run_sum[b] = 0.f;
+      if (prepare_q) {
+        // q holds the raw rows of the q/k/v product: the head is normalised and rotated here, on its way into
+        // the registers it stays in (a dead column prepares its group's first token and drops the result)
+        prepare_head<D>(qf[b], q + (int64_t)token * q_stride + (int64_t)(active ? head : head0) * D, g, prep.q_weight, prep.weight_is_f32,
+                        prep.eps, prep.cosv ? prep.cosv + (int64_t)token * (D / 2) : nullptr,
+                        prep.sinv ? prep.sinv + (int64_t)token * (D / 2) : nullptr);
 #pragma unroll
-      for (int c = 0; c < DS; ++c)
-        qf[b][c] = live[b] ? *(const bf16x8*)(q + (int64_t)token * q_stride + (int64_t)head * D + c * 32 + g * 8) : zero8;
+        for (int c = 0; c < DS; ++c) qf[b][c] = live[b] ? qf[b][c] : zero8;
+      } else {
+#pragma unroll
+        for (int c = 0; c < DS; ++c)
+          qf[b][c] = live[b] ? *(const bf16x8*)(q + (int64_t)token * q_stride + (int64_t)head * D + c * 32 + g * 8) : zero8;
+      }
 #pragma unroll
       for (int e = 0; e < DB; ++e) o[b][e] = floatx4{0.f, 0.f, 0.f, 0.f};
     }
@@ -1317,17 +1327,32 @@ LRS_API int lrs_attention_prefill_group_for(int tokens, int longest) {
   return 16;
 }
 
+// Whether lrs_attention_prefill can be given the raw q rows of the q/k/v product (prepare != 0) for this head size.
+LRS_API int lrs_attention_prefill_prepares(int d) { return d == 128; }
+
 // Any step in bf16.  qblock_token0 / qblock_count [n_blocks]: first token and number of tokens
 // (1..lrs_attention_prefill_group()) of each group of consecutive tokens of one request.
 // splits > 1: every group's keys are divided between that many workgroups; needs part_o
 // [tokens, nq, splits, d] and part_ml [tokens, nq, splits, 2] float32 and `tokens`, the step's size.
+// prepare != 0 (heads of 128 only): q holds raw rows; every query head gets its RMSNorm (q_weight [d], or null for none)
+// and the rotation of pairs (i, i + d/2) by the step's tables cosv / sinv [tokens, d/2] (null: none) on its way into the
+// kernel's registers, as lrs_qk_prep would have left it in memory; the keys and values are in the pages already.
 LRS_API int lrs_attention_prefill(void* out, int out_stride, const void* q, int q_stride, const void* k_pages,
                                   const void* v_pages, const int* block_table, int table_stride,
                                   const int* token_request, const int* positions, const int* qblock_token0,
                                   const int* qblock_count, int n_blocks, int max_count, int max_context, int nq,
                                   int nkv, int d, int page_size, float scale, int window, int tokens, int splits,
-                                  float* part_o, float* part_ml, void* stream) {
+                                  float* part_o, float* part_ml, int prepare, const void* q_weight, int w_dtype, float eps,
+                                  const float* cosv, const float* sinv, void* stream) {
   LRS_REQUIRE(n_blocks > 0 && nq > 0 && nkv > 0 && nq % nkv == 0, "attention_prefill: bad sizes blocks=%d nq=%d nkv=%d", n_blocks, nq, nkv);
+  if (prepare) {
+    LRS_REQUIRE(lrs_attention_prefill_prepares(d), "attention_prefill: only the kernel for heads of 128 prepares the queries itself, got head_dim %d", d);
+    LRS_REQUIRE(q_weight == nullptr || eps > 0.f, "attention_prefill: eps must be positive");
+    LRS_REQUIRE((cosv == nullptr) == (sinv == nullptr), "attention_prefill: cos and sin tables must come together");
+    LRS_REQUIRE((uintptr_t)q_weight % 16 == 0 && (uintptr_t)cosv % 16 == 0 && (uintptr_t)sinv % 16 == 0,
+                "attention_prefill: norm weight and rotation tables must be 16-byte aligned");
+  }
+  const DecodePrep prep{q_weight, nullptr, w_dtype == LRS_F32, eps, cosv, sinv, 0};
   LRS_REQUIRE(max_count >= 1 && max_count <= 32, "attention_prefill: query groups hold 1..32 tokens, got %d", max_count);
   LRS_REQUIRE(page_size % 16 == 0, "attention_prefill: page size %d is not a multiple of 16", page_size);
   LRS_REQUIRE(window >= 0, "attention_prefill: window must be >= 0 (0 = none)");
@@ -1371,7 +1396,8 @@ LRS_API int lrs_attention_prefill(void* out, int out_stride, const void* q, int 
 #define D128(QB, MANY, IDLE)                                                                                                      \
         attention_prefill_d128_bf16_kernel<QB, MANY, IDLE><<<grid, block, 0, s>>>(                                                    \
             (bf16*)out, out_stride, (const bf16*)q, q_stride, (const bf16*)k_pages, (const bf16*)v_pages, block_table, table_stride, \
-            token_request, positions, qblock_token0, qblock_count, n_blocks, chunk, nq, nkv, page_size, scale, window, splits, part_o, part_ml)
+            token_request, positions, qblock_token0, qblock_count, n_blocks, chunk, nq, nkv, page_size, scale, window, splits, part_o, part_ml, \
+            prepare, prep)
 #define D128_OF(QB)                                      \
         if (many && idle) D128(QB, true, true);          \
         else if (many) D128(QB, true, false);            \

@@ -226,9 +226,9 @@ __global__ void qk_prep_kernel(T* __restrict__ qkv, int row_stride, int nq, int 
                                float eps, const float* __restrict__ cosv,
                                const float* __restrict__ sinv, int rot_half,
                                T* __restrict__ k_pages, T* __restrict__ v_pages,
-                               const int* __restrict__ slots, int page_size) {
-  // v_pages == null: the values are stored by values_to_pages_kernel instead
-  const int token = blockIdx.x, head = blockIdx.y, lane = threadIdx.x;
+                               const int* __restrict__ slots, int page_size, int first_head) {
+  // v_pages == null: the values are stored by values_to_pages_kernel instead; first_head: the heads before it are left alone
+  const int token = blockIdx.x, head = blockIdx.y + first_head, lane = threadIdx.x;
   T* src = qkv + (int64_t)token * row_stride + (int64_t)head * d;
   const bool is_q = head < nq, is_k = !is_q && head < nq + nkv;
   T* dst = src;
@@ -349,7 +349,8 @@ __global__ __launch_bounds__(256) void qk_prep_vec_kernel(T* __restrict__ qkv, i
                                                           int rot_half, T* __restrict__ k_pages, T* __restrict__ v_pages,
                                                           const int* __restrict__ slots, int page_size, int prep_blocks,
                                                           const float* __restrict__ sums, int splits,
-                                                          int sum_columns) {
+                                                          int sum_columns, int first_head) {
+  // first_head: the heads before it (the q heads, or none) are left as they are.
   // sums != null: the heads come as the float32 sums that the K splits of the q/k/v product left,
   // [splits, tokens, sum_columns], added up here in split order; qkv only receives the prepared q heads.
   constexpr int VE = 16 / sizeof(T);
@@ -365,11 +366,11 @@ __global__ __launch_bounds__(256) void qk_prep_vec_kernel(T* __restrict__ qkv, i
   // fill a token's heads): the token's rotation tables and the norm weights, which every head needs again, are
   // read once a group, and all the heads' values are asked for before the first is worked on.
   constexpr int together = TOGETHER;
-  const int groups_per_token = heads / together;
+  const int groups_per_token = (heads - first_head) / together;
   const int64_t pair = (int64_t)blockIdx.x * (256 / per_head) + threadIdx.x / per_head;
   const int j = threadIdx.x % per_head;
   if (pair >= (int64_t)tokens * groups_per_token) return;   // whole groups of per_head lanes leave together
-  const int token = pair / groups_per_token, head0 = (int)(pair % groups_per_token) * together;
+  const int token = pair / groups_per_token, head0 = first_head + (int)(pair % groups_per_token) * together;
   float c[VE], sn[VE], wq[2][VE], wk[2][VE];
   if (rot_half) {
     load_floats<float, VE>(cosv + (int64_t)token * rot_half + VE * j, c);
@@ -478,11 +479,14 @@ __global__ __launch_bounds__(256) void qk_prep_vec_kernel(T* __restrict__ qkv, i
   }
 }
 
+LRS_API int lrs_compute_units();
+
 static int qk_prep_launch(void* qkv, int dtype, int tokens, int row_stride, int nq, int nkv, int d,
                           const void* q_weight, const void* k_weight, int w_dtype, float eps,
                           const float* cosv, const float* sinv, int rot_half, void* k_pages,
                           void* v_pages, const int* slots, int page_size, void* stream,
-                          const float* sums, int splits, int sum_columns) {
+                          const float* sums, int splits, int sum_columns, int skip_q = 0) {
+  LRS_REQUIRE(!skip_q || (nkv > 0 && !sums), "qk_prep: leaving the q heads alone needs k and v heads to prepare, and no sums");
   LRS_REQUIRE(tokens > 0 && nq > 0 && nkv >= 0 && d > 0, "qk_prep: bad sizes tokens=%d nq=%d nkv=%d d=%d", tokens, nq, nkv, d);
   LRS_REQUIRE(rot_half >= 0 && 2 * rot_half <= d, "qk_prep: rotary width %d exceeds head_dim %d", 2 * rot_half, d);
   LRS_REQUIRE(rot_half == 0 || (cosv && sinv), "qk_prep: rotation asked for without tables");
@@ -504,9 +508,17 @@ static int qk_prep_launch(void* qkv, int dtype, int tokens, int row_stride, int 
     const int heads = nq + (values_apart ? nkv : 2 * nkv);    // heads the (token, head) pairs run over
     // heads of one token that a group of threads takes in turn: the largest of 5, 4, 2 that divides them, for
     // steps of many tokens (a decode step has too few groups to fill the chip as it is)
-    const int together = tokens < 128 || sums ? 1 : heads % 5 == 0 ? 5 : heads % 4 == 0 ? 4 : heads % 2 == 0 ? 2 : 1;
-    const int64_t pairs = (int64_t)tokens * (heads / together);
+    const int first_head = skip_q ? nq : 0, taken = heads - first_head;
+    // ... as long as that leaves two workgroups for every compute unit
     const int per_block = 256 / per_head;
+    int together = 1;
+    if (tokens >= 128 && !sums)
+      for (int many : {5, 4, 2})
+        if (taken % many == 0 && (int64_t)tokens * (taken / many) / per_block >= 2 * lrs_compute_units()) {
+          together = many;
+          break;
+        }
+    const int64_t pairs = (int64_t)tokens * (taken / together);
     const int64_t prep_blocks = (pairs + per_block - 1) / per_block;
     const int64_t value_blocks = values_apart ? (int64_t)((tokens + 15) / 16) * nkv : 0;
     LRS_REQUIRE(prep_blocks + value_blocks < (1ll << 31), "qk_prep: %d tokens are too many for one launch", tokens);
@@ -514,7 +526,7 @@ static int qk_prep_launch(void* qkv, int dtype, int tokens, int row_stride, int 
 #define LAUNCH_VEC_OF(T, TW, TOGETHER)                                                                                   \
   qk_prep_vec_kernel<T, TW, TOGETHER><<<vgrid, 256, 0, s>>>((T*)qkv, row_stride, tokens, heads, nq, nkv, d, (const TW*)q_weight, \
                                                             (const TW*)k_weight, eps, cosv, sinv, rot_half, (T*)k_pages,   \
-                                                            (T*)v_pages, slots, page_size, (int)prep_blocks, sums, splits, sum_columns)
+                                                            (T*)v_pages, slots, page_size, (int)prep_blocks, sums, splits, sum_columns, first_head)
 #define LAUNCH_VEC(T, TW)                        \
   do {                                           \
     if (together == 5) LAUNCH_VEC_OF(T, TW, 5);  \
@@ -544,10 +556,11 @@ static int qk_prep_launch(void* qkv, int dtype, int tokens, int row_stride, int 
     v_pages = nullptr;
     grid.y = nq + nkv;
   }
+  if (skip_q) grid.y -= nq;
 #define LAUNCH(T, TW)                                                                          \
   qk_prep_kernel<T, TW><<<grid, block, 0, s>>>((T*)qkv, row_stride, nq, nkv, d, (const TW*)q_weight, \
                                                (const TW*)k_weight, eps, cosv, sinv, rot_half,  \
-                                               (T*)k_pages, (T*)v_pages, slots, page_size)
+                                               (T*)k_pages, (T*)v_pages, slots, page_size, skip_q ? nq : 0)
   if (dtype == LRS_F32 && w_dtype == LRS_F32) LAUNCH(float, float);
   else if (dtype == LRS_BF16 && w_dtype == LRS_BF16) LAUNCH(bf16, bf16);
   else if (dtype == LRS_BF16 && w_dtype == LRS_F32) LAUNCH(bf16, float);
@@ -560,9 +573,9 @@ static int qk_prep_launch(void* qkv, int dtype, int tokens, int row_stride, int 
 LRS_API int lrs_qk_prep(void* qkv, int dtype, int tokens, int row_stride, int nq, int nkv, int d,
                         const void* q_weight, const void* k_weight, int w_dtype, float eps,
                         const float* cosv, const float* sinv, int rot_half, void* k_pages,
-                        void* v_pages, const int* slots, int page_size, void* stream) {
+                        void* v_pages, const int* slots, int page_size, int skip_q, void* stream) {
   return qk_prep_launch(qkv, dtype, tokens, row_stride, nq, nkv, d, q_weight, k_weight, w_dtype, eps, cosv, sinv, rot_half, k_pages,
-                        v_pages, slots, page_size, stream, nullptr, 0, 0);
+                        v_pages, slots, page_size, stream, nullptr, 0, 0, skip_q);
 }
 
 // The same from the float32 sums that the K splits of the q/k/v product left, sums [splits, tokens, (nq + 2 nkv) d]:

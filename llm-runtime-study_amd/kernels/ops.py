@@ -76,7 +76,7 @@ _SIGNATURES = {
     "lrs_add_rmsnorm": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_float, c_void_p]),
     "lrs_rope_table": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p]),
     "lrs_qk_prep": (c_int, [c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_int, c_float,
-                            c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p]),
+                            c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p]),
     "lrs_gemm_mid_qk_prep": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p, c_int, c_float, c_int, c_int, c_int,
                                      c_void_p, c_void_p, c_int, c_float, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p]),
     "lrs_silu_mul": (c_int, [c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p]),
@@ -112,7 +112,8 @@ _SIGNATURES = {
                                      c_void_p, c_void_p, c_int, c_float, c_void_p, c_void_p, c_int, c_void_p]),
     "lrs_attention_prefill": (c_int, [c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p,
                                       c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int,
-                                      c_int, c_int, c_void_p, c_void_p, c_void_p]),
+                                      c_int, c_int, c_void_p, c_void_p, c_int, c_void_p, c_int, c_float, c_void_p, c_void_p, c_void_p]),
+    "lrs_attention_prefill_prepares": (c_int, [c_int]),
     "lrs_compute_units": (c_int, []),
     "lrs_gemm_lines_width": (c_int, [c_int, c_int, c_int]),
     "lrs_gemm_lines_splits": (c_int, [c_int, c_int, c_int]),
@@ -393,8 +394,9 @@ def rope_table(cos: torch.Tensor, sin: torch.Tensor, positions: torch.Tensor, in
 
 
 def qk_prep(qkv: torch.Tensor, nq: int, nkv: int, d: int, q_weight, k_weight, eps: float, cos, sin,
-            k_pages, v_pages, slots, page_size: int) -> None:
-    """Normalise and rotate the q and k heads of `qkv` [T, (nq+2*nkv)*d]; q in place, k and v into pages."""
+            k_pages, v_pages, slots, page_size: int, skip_q: bool = False) -> None:
+    """Normalise and rotate the q and k heads of `qkv` [T, (nq+2*nkv)*d]; q in place, k and v into pages.
+    skip_q: the q heads are left as they are (attention_prefill() with `prepare` takes them raw)."""
     tokens = qkv.shape[0]
     stride = _rows(qkv, "qkv")
     _need(qkv.shape[1] == (nq + 2 * nkv) * d, f"qk_prep: qkv width {qkv.shape[1]} is not (nq+2nkv)*d = {(nq + 2 * nkv) * d}")
@@ -417,7 +419,7 @@ def qk_prep(qkv: torch.Tensor, nq: int, nkv: int, d: int, q_weight, k_weight, ep
         None if q_weight is None else _dev(q_weight, "q_weight"), None if k_weight is None else _dev(k_weight, "k_weight"),
         dtype_code(w_dtype), eps, None if cos is None else cos.data_ptr(), None if sin is None else sin.data_ptr(), rot_half,
         None if nkv == 0 else _dev(k_pages, "k_pages"), None if nkv == 0 else _dev(v_pages, "v_pages"),
-        None if nkv == 0 else _dev(slots, "slots"), page_size, _stream())
+        None if nkv == 0 else _dev(slots, "slots"), page_size, int(bool(skip_q)), _stream())
 
 
 def gemm_mid_qk_prep_takes(dtype: torch.dtype, m: int, nq: int, nkv: int, d: int, k: int, rot_half: int,
@@ -838,13 +840,17 @@ def attention_decode(out: torch.Tensor, q: torch.Tensor, k_pages: torch.Tensor, 
 def attention_prefill(out: torch.Tensor, q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, block_table: torch.Tensor,
                       token_request: torch.Tensor, positions: torch.Tensor, qblock_token0: torch.Tensor, qblock_count: torch.Tensor,
                       nq: int, scale: float, window: int = 0, max_count: int | None = None, max_context: int | None = None,
-                      splits: int = 1, part_o: torch.Tensor | None = None, part_ml: torch.Tensor | None = None) -> None:
+                      splits: int = 1, part_o: torch.Tensor | None = None, part_ml: torch.Tensor | None = None,
+                      prepare: "DecodePrepare | None" = None) -> None:
     """attention() on matrix cores for any bfloat16 step.  qblock_token0 / qblock_count list groups of at
     most attention_prefill_group() consecutive tokens of one request that together cover every token of
     the step once; `max_count` is the largest count among them (the group limit if not given) and
     `max_context` the longest context (position + 1) of any token (what the block table can hold if not given).
     splits > 1 divides every group's keys between that many workgroups (few queries over long contexts);
-    their partial results meet in part_o [T, nq * splits * d] and part_ml [T, nq * splits * 2] float32."""
+    their partial results meet in part_o [T, nq * splits * d] and part_ml [T, nq * splits * 2] float32.
+    prepare (where attention_prefill_prepares(d)): `q` holds the raw q heads of the q/k/v product, and the kernel gives
+    them their norm and rotation itself (q_weight, eps, cos, sin of DecodePrepare; kv_heads 0: the keys and values are in
+    the pages already, from qk_prep(skip_q=True))."""
     tokens = out.shape[0]
     _need(k_pages.dim() == 4 and k_pages.is_contiguous() and v_pages.is_contiguous(), "attention_prefill: pages must be contiguous")
     _, nkv, page_size, d = k_pages.shape
@@ -862,13 +868,30 @@ def attention_prefill(out: torch.Tensor, q: torch.Tensor, k_pages: torch.Tensor,
     if splits > 1:
         _need(part_o is not None and part_o.dtype == torch.float32 and part_o.is_contiguous() and part_o.numel() >= tokens * nq * splits * d, "attention_prefill: part_o too small")
         _need(part_ml is not None and part_ml.dtype == torch.float32 and part_ml.is_contiguous() and part_ml.numel() >= tokens * nq * splits * 2, "attention_prefill: part_ml too small")
+    fused = [0, None, 0, 0.0, None, None]
+    if prepare is not None:
+        _need(attention_prefill_prepares(d), f"attention_prefill: heads of {d} dims must come prepared")
+        _need(prepare.kv_heads == 0, "attention_prefill: prepares the queries only (kv_heads must be 0)")
+        w = prepare.q_weight
+        _need(w is None or (w.numel() == d and w.is_contiguous() and prepare.eps > 0), "attention_prefill: q_weight must hold head_dim values, eps be positive")
+        for name, t in (("cos", prepare.cos), ("sin", prepare.sin)):
+            _need((t is None) == (prepare.cos is None) and (t is None or (t.dtype == torch.float32 and t.dim() == 2 and t.shape[0] >= tokens
+                                                                       and t.shape[1] == d // 2 and t.is_contiguous())),
+                  f"attention_prefill: {name} must be float32 [{tokens}, {d // 2}]")
+        fused = [1, None if w is None else _dev(w, "q_weight"), 0 if w is None else dtype_code(w.dtype), prepare.eps,
+                 None if prepare.cos is None else _dev(prepare.cos, "cos"), None if prepare.sin is None else _dev(prepare.sin, "sin")]
     _launch("lrs_attention_prefill", 
         _dev(out, "out"), _rows(out, "out"), _dev(q, "q"), _rows(q, "q"), _dev(k_pages, "k_pages"), _dev(v_pages, "v_pages"),
         _dev(block_table, "block_table"), block_table.stride(0), _dev(token_request, "token_request"), _dev(positions, "positions"),
         _dev(qblock_token0, "qblock_token0"), _dev(qblock_count, "qblock_count"), n_blocks,
         attention_prefill_group() if max_count is None else max_count,
         block_table.shape[1] * page_size if max_context is None else max_context, nq, nkv, d, page_size, scale, window,
-        tokens, splits, None if splits == 1 else _dev(part_o, "part_o"), None if splits == 1 else _dev(part_ml, "part_ml"), _stream())
+        tokens, splits, None if splits == 1 else _dev(part_o, "part_o"), None if splits == 1 else _dev(part_ml, "part_ml"), *fused, _stream())
+
+
+def attention_prefill_prepares(d: int) -> bool:
+    """Whether attention_prefill() can take raw q heads of d dims and prepare them itself."""
+    return bool(library().lrs_attention_prefill_prepares(d))
 
 
 def compute_units() -> int:

@@ -161,14 +161,21 @@ class GQAAttention(Part):
         # value itself, when the rotation covers the whole head or there is none; beyond 16 rows a kernel
         # before it does that once a token (measured: 98 against 108 us for the attention kernel at 64 rows)
         whole_head = cos is None or cos.shape[1] * 2 == d
-        prepare = None
+        prepare = queries_raw = None
         if together:
             pass
         elif decode and whole_head and ops.decode_prepare_supported(d, cos is not None) and t <= self.PREPARE_INSIDE_ROWS:
             prepare = ops.DecodePrepare(self.q_norm, self.k_norm, self.qk_norm_eps, cos, sin, nkv)
         else:
+            # a ragged step of heads of 128: the attention kernel normalises and rotates the q heads on their way into its
+            # registers, so that only the k and v heads pass through a kernel before it (a third of the rows' bytes;
+            # measured at 2,048 tokens, 32 q heads on 8: 19-22 -> 10.4 us for the kernel before attention, 66 -> 68 us
+            # for attention itself)
+            if (not decode and nkv > 0 and whole_head and ops.attention_prefill_prepares(d)
+                    and ops.attention_decode_supported(ctx.dtype, nq, kv_heads, d, group.page_size)):
+                queries_raw = ops.DecodePrepare(self.q_norm, None, self.qk_norm_eps, cos, sin, 0)
             ops.qk_prep(qkv, nq, nkv, d, self.q_norm, self.k_norm, self.qk_norm_eps, cos, sin,
-                        cache.k_pages, cache.v_pages, group.slots, group.page_size)
+                        cache.k_pages, cache.v_pages, group.slots, group.page_size, skip_q=queries_raw is not None)
         if decode:
             longest, bound = ctx.max_k, ctx.max_k_bound
             if self.window is not None:
@@ -194,11 +201,18 @@ class GQAAttention(Part):
                 if splits > 1:
                     part_o = ctx.scratch("attn_single_part_o", (singles, nq * splits * d), torch.float32)
                     part_ml = ctx.scratch("attn_single_part_ml", (singles, nq * splits * 2), torch.float32)
+                first = None
+                if queries_raw is not None:      # the decode kernel prepares the q heads of its rows likewise
+                    first = ops.DecodePrepare(self.q_norm, self.k_norm, self.qk_norm_eps, None if cos is None else cos[:singles],
+                                              None if sin is None else sin[:singles], 0)
                 ops.attention_decode(out[:singles], qkv[:singles], cache.k_pages, cache.v_pages, group.block_table, ctx.token_request,
-                                     ctx.positions, nq, self.scale, self.window or 0, splits, part_o, part_ml, ctx.max_k_bound, None, form=1)
+                                     ctx.positions, nq, self.scale, self.window or 0, splits, part_o, part_ml, ctx.max_k_bound, first, form=1)
             rest = ctx.memo.get("rows_after_singles")
             if rest is None:
                 rest = ctx.memo["rows_after_singles"] = (ctx.token_request[singles:], ctx.positions[singles:])
+            if queries_raw is not None and singles:
+                queries_raw = ops.DecodePrepare(self.q_norm, None, self.qk_norm_eps, None if cos is None else cos[singles:],
+                                                None if sin is None else sin[singles:], 0)
             splits = self._prefill_splits(ctx.num_qblocks * kv_heads, longest, (t - singles) * nq * d, nq // kv_heads)
             part_o = part_ml = None
             if splits > 1:
@@ -206,7 +220,7 @@ class GQAAttention(Part):
                 part_ml = ctx.scratch("attn_part_ml", (t - singles, nq * splits * 2), torch.float32)
             ops.attention_prefill(out[singles:], qkv[singles:], cache.k_pages, cache.v_pages, group.block_table, rest[0], rest[1],
                                   ctx.qblock_token0, ctx.qblock_count, nq, self.scale, self.window or 0, ctx.max_qblock, ctx.max_k_bound,
-                                  splits, part_o, part_ml)
+                                  splits, part_o, part_ml, queries_raw)
         else:
             ops.attention(out, qkv, cache.k_pages, cache.v_pages, group.block_table, ctx.token_request, ctx.positions,
                           nq, self.scale, self.window or 0)

@@ -633,6 +633,89 @@ def test_attention_ragged_batch(ops, dtype, nq, nkv, d, page, window):
             torch.testing.assert_close(fast.cpu().double(), want, rtol=2e-2, atol=2e-2)
 
 
+@pytest.mark.parametrize("nq,nkv,page,window,normed,rotated", [
+    (32, 8, 16, 0, True, True), (8, 1, 32, 0, True, True), (6, 2, 64, 40, True, False), (5, 1, 16, 0, False, True), (16, 1, 16, 21, True, True),
+])
+def test_attention_prefill_prepares_raw_queries(ops, nq, nkv, page, window, normed, rotated):
+    """Heads of 128: the kernel for ragged steps given the raw q heads of the q/k/v product (norm and rotation on their
+    way into its registers) against attention over queries that were normalised, rotated and rounded beforehand;
+    qk_prep(skip_q=True) beside it writes the keys and values as always and leaves the q heads as they were."""
+    dtype, d = torch.bfloat16, 128
+    g = torch.Generator().manual_seed(61)
+    requests = [(0, 19), (37, 1), (150, 1), (5, 6), (page * 3 - 1, 2), (9, 75)]
+    scale = 1 / math.sqrt(d)
+    max_blocks = max((a + b + page - 1) // page for a, b in requests)
+    n_pages = sum((a + b + page - 1) // page for a, b in requests) + 3
+    perm = torch.randperm(n_pages, generator=g).tolist()
+    table = torch.zeros(len(requests), max_blocks, dtype=torch.int32)
+    qw = (1 + 0.1 * torch.randn(d, generator=g)).to(dtype) if normed else None
+    kw = (1 + 0.1 * torch.randn(d, generator=g)).to(dtype) if normed else None
+    rot_half = d // 2 if rotated else 0
+    inv = 1.0 / (1e4 ** (torch.arange(0, d, 2, dtype=torch.float32) / d))
+    kp = torch.randn(n_pages, nkv, page, d, generator=g).to(dtype)      # slots not written hold finite junk
+    vp = torch.randn(n_pages, nkv, d, page, generator=g).to(dtype)
+    rows, slots, tok_req, tok_pos, meta, k_all, v_all = [], [], [], [], [], [], []
+    for r, (before, new) in enumerate(requests):
+        total = before + new
+        for b in range((total + page - 1) // page):
+            table[r, b] = perm.pop()
+        # what the cache holds of the request before the step, and the raw rows of the step's tokens
+        k_old = torch.randn(before, nkv, d, generator=g).to(dtype)
+        v_old = torch.randn(before, nkv, d, generator=g).to(dtype)
+        for i in range(before):
+            pg = int(table[r, i // page])
+            kp[pg, :, i % page] = k_old[i]
+            vp[pg, :, :, i % page] = v_old[i]
+        raw = (torch.randn(new, (nq + 2 * nkv) * d, generator=g) * 2).to(dtype)
+        positions = torch.arange(before, total, dtype=torch.int32)
+        want_q, want_k, want_v = _qk_prep_reference(raw, nq, nkv, d, qw, kw, 1e-6, positions, inv, rot_half)
+        rows.append((raw, want_q.to(dtype).float()))
+        k_all.append(torch.cat((k_old.float(), want_k.to(dtype).float())))
+        v_all.append(torch.cat((v_old.float(), want_v)))
+        for i in range(new):
+            slots.append(int(table[r, (before + i) // page]) * page + (before + i) % page)
+            tok_req.append(r)
+            tok_pos.append(before + i)
+            meta.append((r, before + i))
+    raw = torch.cat([a for a, _ in rows])
+    t = raw.shape[0]
+    want = _attention_reference(torch.cat([b for _, b in rows]), k_all, v_all, meta, None, nq, nkv, d, scale, window)
+    d_raw, d_kp, d_vp, d_pos = dev(raw), dev(kp), dev(vp), dev(torch.tensor(tok_pos, dtype=torch.int32))
+    cos = sin = None
+    if rotated:
+        cos = torch.empty(t, rot_half, device="cuda")
+        sin = torch.empty_like(cos)
+        ops.rope_table(cos, sin, d_pos, dev(inv))
+    ops.qk_prep(d_raw, nq, nkv, d, None if qw is None else dev(qw), None if kw is None else dev(kw), 1e-6, cos, sin, d_kp, d_vp,
+                dev(torch.tensor(slots, dtype=torch.int32)), page, skip_q=True)
+    assert torch.equal(d_raw.cpu()[:, :nq * d], raw[:, :nq * d]), "the q heads were to be left alone"
+    for i, (r, pos) in enumerate(meta):
+        pg = int(table[r, pos // page])
+        torch.testing.assert_close(d_kp[pg, :, pos % page].cpu().float(), k_all[r][pos], rtol=2e-2, atol=2e-2)
+        assert torch.equal(d_vp[pg, :, :, pos % page].cpu().float(), v_all[r][pos])
+    prepare = ops.DecodePrepare(None if qw is None else dev(qw), None, 1e-6, cos, sin, 0)
+    for size, splits in ((16, 1), (32, 1), (7, 1), (25, 3), (16, 8)):
+        blocks, at = [], 0
+        for before, new in requests:
+            blocks += [(at + i, min(size, new - i)) for i in range(0, new, size)]
+            at += new
+        blocks = blocks[::-1]
+        out = torch.empty(t, nq * d, device="cuda", dtype=dtype)
+        part_o = torch.full((t, nq * splits * d), float("nan"), device="cuda") if splits > 1 else None
+        part_ml = torch.full((t, nq * splits * 2), float("nan"), device="cuda") if splits > 1 else None
+        ops.attention_prefill(out, d_raw, d_kp, d_vp, dev(table), dev(torch.tensor(tok_req, dtype=torch.int32)), d_pos,
+                              dev(torch.tensor([b[0] for b in blocks], dtype=torch.int32)),
+                              dev(torch.tensor([b[1] for b in blocks], dtype=torch.int32)), nq, scale, window, size,
+                              splits=splits, part_o=part_o, part_ml=part_ml, prepare=prepare)
+        torch.testing.assert_close(out.cpu().double(), want, rtol=2e-2, atol=2e-2)
+    from llm_runtime_study_amd.errors import KernelError
+    with pytest.raises(KernelError):                      # only the queries: no kv heads to write
+        ops.attention_prefill(out, d_raw, d_kp, d_vp, dev(table), dev(torch.tensor(tok_req, dtype=torch.int32)), d_pos,
+                              dev(torch.tensor([0], dtype=torch.int32)), dev(torch.tensor([1], dtype=torch.int32)), nq, scale, window, 16,
+                              prepare=ops.DecodePrepare(None, None, 1e-6, cos, sin, nkv))
+    assert not ops.attention_prefill_prepares(64) and ops.attention_prefill_prepares(128)
+
+
 @pytest.mark.parametrize("nq,nkv,d,page,window,splits", [
     (8, 2, 32, 16, 0, 1), (32, 8, 128, 16, 0, 1), (32, 8, 128, 16, 0, 5), (4, 4, 64, 32, 0, 3), (16, 1, 96, 16, 0, 2),
     (6, 2, 192, 64, 0, 4), (8, 2, 32, 16, 40, 1), (8, 2, 64, 16, 100, 3), (8, 2, 32, 16, 0, 64),
@@ -978,8 +1061,8 @@ def test_filter_logits_of_a_large_vocabulary_matches_the_sort_based_rule(ops, vo
 
 @pytest.mark.gpu
 def test_the_probes_of_lds_and_matrix_rates_run_and_refuse_what_they_cannot_do(ops):
-    """`microbench lds` and `microbench mfma` are measurements, not products: here only that they launch,
-    finish and refuse parameters outside what their kernels hold."""
+    """`microbench lds`, `microbench mfma` and `microbench lines` are measurements, not products: here only that
+    they launch, finish and refuse parameters outside what their kernels hold."""
     from llm_runtime_study_amd.errors import KernelError
 
     ints = torch.zeros(256, dtype=torch.int32, device="cuda")
@@ -987,7 +1070,14 @@ def test_the_probes_of_lds_and_matrix_rates_run_and_refuse_what_they_cannot_do(o
     ops.probe_lds(ints, 8, 4, 96)
     ops.probe_mfma(floats, 8, 4, 2, True)
     ops.probe_mfma(floats, 8, 4, 0, False)
+    data = torch.zeros(3 * 8192 // 4, dtype=torch.int32, device="cuda")
+    for pattern in range(3):
+        ops.probe_lines(data, ints, 3, 256, 8192, pattern)
+    ops.probe_lines(data, ints, 1, 1024, 3 * 8192, 1)
     torch.cuda.synchronize()
+    for blocks, threads, each, pattern in ((4, 256, 8192, 0), (3, 96, 8192, 0), (3, 256, 6000, 1), (3, 256, 8192, 3)):   # beyond the data; no whole waves; no whole turns
+        with pytest.raises(KernelError):
+            ops.probe_lines(data, ints, blocks, threads, each, pattern)
     for bad in (8, 100, 1024):
         with pytest.raises(KernelError):
             ops.probe_lds(ints, 8, 4, bad)

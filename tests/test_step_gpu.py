@@ -26,6 +26,19 @@ def folder_b(tmp_path_factory):
     return folder
 
 
+@pytest.fixture(scope="module")
+def folder_heads_of_128(tmp_path_factory):
+    """Heads of 128 dims, the size whose kernel for ragged steps prepares the queries itself; kv groups of three heads
+    (a wave of the four has none), everything else small."""
+    from llm_runtime_study_amd.config import config_from_dict
+    from llm_runtime_study_amd.weights import write_model_dir
+
+    folder = tmp_path_factory.mktemp("step_heads_of_128")
+    write_model_dir(config_from_dict(dict(TINY_C, head_dim=128, num_attention_heads=6, num_key_value_heads=2, vocab_size=290)),
+                    seed=43, model_dir=folder, init="scaled")
+    return folder
+
+
 def make_runner(folder, dtype, *, pages=40, requests=4, seq=256, step_tokens=64, graph=False, page_size=16):
     from llm_runtime_study_amd.cache import CacheManager
     from llm_runtime_study_amd.engine.loading import load_model
@@ -255,14 +268,17 @@ def test_whole_prompts_through_the_own_many_rows_product(folder_b, dtype, tmp_pa
     assert checked == 300 + 150 + 2 + 130
 
 
+@pytest.mark.parametrize("model", ["b", "heads_of_128"])
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-def test_single_tokens_at_the_head_of_a_mixed_step_and_elsewhere_in_it(folder_b, dtype, tmp_path):
+def test_single_tokens_at_the_head_of_a_mixed_step_and_elsewhere_in_it(folder_b, folder_heads_of_128, model, dtype, tmp_path):
     """Decoding requests beside a prompt portion: the single tokens that a step begins with go to the
     attention kernel of decode steps, single tokens further back stay rows of the other kernel, and one
     token that is a whole portion (a request's first) is a single token like any other.  Every asked row
-    against the plain implementation."""
+    against the plain implementation.  (With heads of 128 dims both kernels take the raw q heads of the
+    q/k/v product in bfloat16 and prepare them themselves.)"""
     from llm_runtime_study_amd.engine import trace
 
+    folder_b = folder_b if model == "b" else folder_heads_of_128
     cfg, weights = plain.load_model_dir(folder_b, torch.float64)
     rng = np.random.default_rng(21)
     requests = {key: rng.integers(0, cfg["vocab_size"], n).tolist() for key, n in (("a", 45), ("b", 30), ("c", 64), ("d", 3))}
