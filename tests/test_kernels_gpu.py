@@ -879,8 +879,16 @@ def test_one_key_stands_out_in_every_attention_kernel(ops, window, planted):
     run_one_key_stands_out(ops, window, planted, 128, 32)
 
 
-def run_one_key_stands_out(ops, window, planted, d, page):
-    nq, nkv, before, new = 4, 2, 690, 10
+@pytest.mark.parametrize("window,planted", [(0, 0), (0, 32767), (0, 32768), (0, 39001), (100, 39950), (100, 39895)])
+def test_one_key_stands_out_far_back_in_a_long_context(ops, window, planted):
+    """The same ten tokens after 39,990 cached ones (2,500 pages of 16, or 625 of 64): block tables, key numbers and
+    byte offsets of a size the short tests never reach, in every attention kernel and with the keys divided."""
+    run_one_key_stands_out(ops, window, planted, 128, 16, before=39990)
+    run_one_key_stands_out(ops, window, planted, 64, 64, before=39990)
+
+
+def run_one_key_stands_out(ops, window, planted, d, page, before=690):
+    nq, nkv, new = 4, 2, 10
     length = before + new
     g = torch.Generator().manual_seed(70 + planted)
     k = (torch.randn(length, nkv, d, generator=g) * 0.1).bfloat16()
