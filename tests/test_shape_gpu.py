@@ -87,3 +87,54 @@ def test_bfloat16_path_follows_float32_at_full_layer_sizes(sizes):
     error = (exact - fast).norm(dim=1) / exact.norm(dim=1)
     assert error.max() < 2e-2, f"largest relative error of a logits row {error.max():.3g}"
     assert (exact.argmax(1) == fast.argmax(1)).float().mean() > 0.95
+
+
+@pytest.mark.parametrize("sizes", ["8b", "14b"])
+def test_a_long_prompt_in_portions_follows_the_prompt_in_one_step(sizes):
+    """17,000 tokens at the benchmark's layer sizes, and with kv groups of five heads (two layers): the prompt in one step and in portions (eight of
+    2,048, then 512 behind 16,384 tokens, where every query group's keys are divided between workgroups, then 100,
+    2 and 2) in bfloat16, both against the float32 path in one step, at places on both sides of the portions'
+    edges; then one decoded token behind the 17,000."""
+    from llm_runtime_study_amd.cache import CacheManager
+    from llm_runtime_study_amd.config import config_from_dict, spec_for
+    from llm_runtime_study_amd.engine.step import ModelRunner, StepEntry
+    from llm_runtime_study_amd.models import DecoderModel
+    from llm_runtime_study_amd.weights import random_init
+
+    cfg = config_from_dict(dict(SHAPE, **LARGER[sizes]))
+    device = torch.device("cuda", 0)
+    weights = random_init.device_weights(DecoderModel(spec_for(cfg)), 0, torch.bfloat16, device, "scaled")
+    rng = np.random.default_rng(5)
+    length = 17000
+    prompt = rng.integers(0, cfg.vocab_size, length).tolist()
+    wanted = [0, 2047, 2048, 8191, 16383, 16384, 16895, 16896, 16995, 16996, 16998, 16999]
+    portions = [2048] * 8 + [512, 100, 2, 2]
+    assert sum(portions) == length
+
+    def run(dtype, cuts):
+        model = DecoderModel(spec_for(cfg))
+        model.bind(weights, dtype)
+        cache = CacheManager(model.cache_needs(), page_size=64, num_pages=270, max_requests=2, max_seq_len=17024, dtype=dtype, device=device)
+        runner = ModelRunner(model, cache, max_step_tokens=max(cuts), dtype=dtype, device=device, use_graph=False)
+        rows, at = [], 0
+        with torch.cuda.stream(torch.cuda.Stream(device)):
+            request = cache.admit(0)
+            for n in cuts:
+                want = [p - at for p in wanted if at <= p < at + n]
+                out = runner.step([StepEntry(request, prompt[at:at + n], want)])
+                if want:
+                    rows.append(out.float().cpu())
+                at += n
+            rows.append(runner.step([StepEntry(request, [prompt[0]], [0])]).float().cpu())     # one decoded token behind the prompt
+        cache.check_invariants()
+        return torch.cat(rows)
+
+    exact = run(torch.float32, [length])
+    whole = run(torch.bfloat16, [length])
+    cut = run(torch.bfloat16, portions)
+    assert exact.shape == whole.shape == cut.shape == (len(wanted) + 1, cfg.vocab_size)
+    for name, fast in (("in one step", whole), ("in portions", cut)):
+        error = (exact - fast).norm(dim=1) / exact.norm(dim=1)
+        assert error.max() < 2e-2, f"{name}: largest relative error of a logits row {error.max():.3g} (rows {error.tolist()})"
+    between = (whole - cut).norm(dim=1) / whole.norm(dim=1)
+    assert between.max() < 1e-2, f"portions against one step: {between.tolist()}"
