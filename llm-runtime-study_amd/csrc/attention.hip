@@ -151,18 +151,13 @@ struct DecodePrep {
 // One head row, raw -> normalised and rotated, in the operand layout of the 16x16x32 products: the
 // lane holds dims c*32 + g*8 .. +8 of every 32-dim chunk c, the four lanes g = 0..3 with equal
 // lane % 16 hold one head between them.  All 64 lanes must call it together.
+// head_from_values: the same from values already in registers (a row asked for earlier, so that its trip to memory
+// ran beside other work).
 template <int D>
-__device__ __forceinline__ void prepare_head(bf16x8 (&r)[D / 32], const bf16* __restrict__ head, int g,
-                                             const void* __restrict__ weight, int weight_is_f32, float eps,
-                                             const float* __restrict__ cosrow, const float* __restrict__ sinrow) {
+__device__ __forceinline__ void head_from_values(bf16x8 (&r)[D / 32], float (&x)[D / 32][8], int g,
+                                                 const void* __restrict__ weight, int weight_is_f32, float eps,
+                                                 const float* __restrict__ cosrow, const float* __restrict__ sinrow) {
   constexpr int DS = D / 32;
-  float x[DS][8];
-#pragma unroll
-  for (int c = 0; c < DS; ++c) {
-    const bf16x8 raw = *(const bf16x8*)(head + c * 32 + g * 8);
-#pragma unroll
-    for (int j = 0; j < 8; ++j) x[c][j] = (float)raw[j];
-  }
   // weights and tables come in 16-byte loads (the host checks their alignment)
   if (weight) {
     float ss = 0.f;
@@ -209,6 +204,20 @@ __device__ __forceinline__ void prepare_head(bf16x8 (&r)[D / 32], const bf16* __
     for (int j = 0; j < 8; ++j) r[c][j] = (bf16)x[c][j];
 }
 
+template <int D>
+__device__ __forceinline__ void prepare_head(bf16x8 (&r)[D / 32], const bf16* __restrict__ head, int g,
+                                             const void* __restrict__ weight, int weight_is_f32, float eps,
+                                             const float* __restrict__ cosrow, const float* __restrict__ sinrow) {
+  float x[D / 32][8];
+#pragma unroll
+  for (int c = 0; c < D / 32; ++c) {
+    const bf16x8 raw = *(const bf16x8*)(head + c * 32 + g * 8);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) x[c][j] = (float)raw[j];
+  }
+  head_from_values<D>(r, x, g, weight, weight_is_f32, eps, cosrow, sinrow);
+}
+
 // One query token per request (a decode step).  A workgroup of four waves owns one
 // (token, kv head, split): the query heads that share the kv head (at most 16) sit in the
 // columns of the matrix-core tiles, so every key and value is loaded once for the whole
@@ -245,6 +254,22 @@ __global__ __launch_bounds__(WAVES * 64) void attention_decode_bf16_kernel(
   const int per_split = (last_tile - first_tile + splits) / splits;
   const int tile_begin = first_tile + split * per_split;
   const int tile_end = tile_begin + per_split <= last_tile + 1 ? tile_begin + per_split : last_tile + 1;
+  // PREP: the wave that may have to prepare the token's new key asks for the raw key and value rows now, before
+  // anything here waits for memory: the rows are then there when their turn comes, two trips to memory later
+  // (they are the token's own, whichever workgroup turns out to walk its position)
+  const bf16* q_row = q + (int64_t)token * q_stride;
+  bf16x8 raw_k[DS];
+  bf16 raw_v[(D + WAVE - 1) / WAVE];
+  if constexpr (PREP) {
+    if (prep.kv_columns > 0 && wave == WAVES - 1) {
+#pragma unroll
+      for (int c = 0; c < DS; ++c) raw_k[c] = *(const bf16x8*)(q_row + (int64_t)(nq + kvh) * D + c * 32 + g * 8);
+      const bf16* v_row = q_row + (int64_t)(nq + prep.kv_columns + kvh) * D;
+#pragma unroll
+      for (int n = 0; n < (D + WAVE - 1) / WAVE; ++n)
+        if (lane + n * WAVE < D) raw_v[n] = v_row[lane + n * WAVE];
+    }
+  }
 
   // the block table entries of this workgroup's tiles, in LDS: the address of a key must not
   // wait for a trip to memory of its own
@@ -294,7 +319,6 @@ __global__ __launch_bounds__(WAVES * 64) void attention_decode_bf16_kernel(
     if (tile_begin + wave < tile_end) fetch(tile_begin + wave, (bf16x8(&)[2][DS])kf_a, (bf16x8(&)[DB])vf_a);
   }
   bf16x8 qf[DS];
-  const bf16* q_row = q + (int64_t)token * q_stride;
   if (PREP) {
     const float* cosrow = prep.cosv ? prep.cosv + (int64_t)token * (D / 2) : nullptr;
     const float* sinrow = prep.sinv ? prep.sinv + (int64_t)token * (D / 2) : nullptr;
@@ -315,10 +339,16 @@ __global__ __launch_bounds__(WAVES * 64) void attention_decode_bf16_kernel(
   const bool holds_own = PREP && prep.kv_columns > 0 && tile_begin <= last_tile && last_tile < tile_end;
   if (holds_own && wave == WAVES - 1) {
     bf16x8 kn[DS];
-    prepare_head<D>(kn, q_row + (int64_t)(nq + kvh) * D, g, prep.k_weight, prep.weight_is_f32, prep.eps,
-                    prep.cosv ? prep.cosv + (int64_t)token * (D / 2) : nullptr,
-                    prep.sinv ? prep.sinv + (int64_t)token * (D / 2) : nullptr);
-    const int64_t page = table[pos / page_size];
+    float kx[DS][8];
+#pragma unroll
+    for (int c = 0; c < DS; ++c)
+#pragma unroll
+      for (int j = 0; j < 8; ++j) kx[c][j] = (float)raw_k[c][j];
+    head_from_values<D>(kn, kx, g, prep.k_weight, prep.weight_is_f32, prep.eps,
+                        prep.cosv ? prep.cosv + (int64_t)token * (D / 2) : nullptr,
+                        prep.sinv ? prep.sinv + (int64_t)token * (D / 2) : nullptr);
+    // (among this workgroup's entries, since it walks the position; they are in LDS once a barrier has been passed)
+    const int64_t page = AHEAD ? page_ids[pos / page_size - first_block] : table[pos / page_size];
     const int off = pos % page_size;
     if (col == 0) {
       bf16* kdst = k_pages + ((page * nkv + kvh) * page_size + off) * D + g * 8;
@@ -328,11 +358,14 @@ __global__ __launch_bounds__(WAVES * 64) void attention_decode_bf16_kernel(
         if (page >= 0) *(bf16x8*)(kdst + c * 32) = kn[c];
       }
     }
-    const bf16* v_row = q_row + (int64_t)(nq + prep.kv_columns + kvh) * D;
-    for (int i = lane; i < D; i += WAVE) {
-      const bf16 vn = v_row[i];
-      own_v[i] = vn;
-      if (page >= 0) v_pages[(page * nkv + kvh) * (int64_t)D * page_size + (int64_t)i * page_size + off] = vn;
+#pragma unroll
+    for (int n = 0; n < (D + WAVE - 1) / WAVE; ++n) {
+      const int i = lane + n * WAVE;
+      if (i < D) {
+        const bf16 vn = raw_v[n];
+        own_v[i] = vn;
+        if (page >= 0) v_pages[(page * nkv + kvh) * (int64_t)D * page_size + (int64_t)i * page_size + off] = vn;
+      }
     }
   }
   __syncthreads();
