@@ -203,16 +203,20 @@ class GQAAttention(Part):
                     part_ml = ctx.scratch("attn_single_part_ml", (singles, nq * splits * 2), torch.float32)
                 first = None
                 if queries_raw is not None:      # the decode kernel prepares the q heads of its rows likewise
-                    first = ops.DecodePrepare(self.q_norm, self.k_norm, self.qk_norm_eps, None if cos is None else cos[:singles],
-                                              None if sin is None else sin[:singles], 0)
+                    parted = None
+                    if cos is not None:          # the tables' rows of the single tokens and of the rest, cut once a step
+                        parted = ctx.memo.get(("rotation_rows", id(cos)))
+                        if parted is None:
+                            parted = ctx.memo[("rotation_rows", id(cos))] = (cos[:singles], sin[:singles], cos[singles:], sin[singles:])
+                    first = ops.DecodePrepare(self.q_norm, self.k_norm, self.qk_norm_eps, None if parted is None else parted[0],
+                                              None if parted is None else parted[1], 0)
                 ops.attention_decode(out[:singles], qkv[:singles], cache.k_pages, cache.v_pages, group.block_table, ctx.token_request,
                                      ctx.positions, nq, self.scale, self.window or 0, splits, part_o, part_ml, ctx.max_k_bound, first, form=1)
             rest = ctx.memo.get("rows_after_singles")
             if rest is None:
                 rest = ctx.memo["rows_after_singles"] = (ctx.token_request[singles:], ctx.positions[singles:])
-            if queries_raw is not None and singles:
-                queries_raw = ops.DecodePrepare(self.q_norm, None, self.qk_norm_eps, None if cos is None else cos[singles:],
-                                                None if sin is None else sin[singles:], 0)
+            if queries_raw is not None and singles and cos is not None:
+                queries_raw = ops.DecodePrepare(self.q_norm, None, self.qk_norm_eps, parted[2], parted[3], 0)
             splits = self._prefill_splits(ctx.num_qblocks * kv_heads, longest, (t - singles) * nq * d, nq // kv_heads)
             part_o = part_ml = None
             if splits > 1:
