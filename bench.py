@@ -28,6 +28,9 @@ FLOP_PEAK = {"bf16": 2.5e15, "fp32": 157.3e12}
 from llm_runtime_study_amd.benchmarks.shapes import QWEN3_8B, SHAPES  # noqa: E402  (layer sizes of the 8B, 14B and 32B models)
 
 FULL_LAYERS = QWEN3_8B["num_hidden_layers"]
+BENCHMARK_CONTEXT = 4096      # tokens a request's cache can hold at the least: the benchmark context of the 8B configuration
+PORTION_TOKENS = 512          # a second prefill figure: the size of a prompt portion in the serving configuration
+SIZE_KEYS = ("hidden_size", "intermediate_size", "num_attention_heads", "num_key_value_heads", "head_dim", "vocab_size")
 
 
 def parse_args():
@@ -38,6 +41,7 @@ def parse_args():
     parser.add_argument("--batch", type=int, default=8)
     parser.add_argument("--context", type=int, default=2048)
     parser.add_argument("--prefill-tokens", type=int, default=2048)
+    parser.add_argument("--max-seq-len", type=int, default=None, help="context the cache is made for: 4,096 (the benchmark context of the 8B configuration) or what the workload needs, whichever is more")
     parser.add_argument("--shape", choices=tuple(SHAPES), default="8b", help="layer sizes: Qwen3-8B (default), 14B or 32B")
     parser.add_argument("--layers", type=int, default=None, help="fewer layers than the shape has (reported in config)")
     parser.add_argument("--dtype", choices=("bfloat16", "float32"), default="bfloat16")
@@ -52,16 +56,10 @@ def parse_args():
     return parser.parse_args()
 
 
-def matrix_params_per_layer(c) -> int:
-    qkv = (c.num_attention_heads + 2 * c.num_key_value_heads) * c.head_dim * c.hidden_size
-    return qkv + c.hidden_size * c.num_attention_heads * c.head_dim + 3 * c.hidden_size * c.intermediate_size
-
-
-def prefill_flops(c, tokens: int) -> float:
-    """Matrix products of every layer for all tokens, the head for one row, causal attention."""
-    linear = 2.0 * tokens * matrix_params_per_layer(c) * c.num_hidden_layers + 2.0 * c.hidden_size * c.vocab_size
-    attention = 4.0 * (tokens * (tokens + 1) / 2) * c.num_attention_heads * c.head_dim * c.num_hidden_layers
-    return linear + attention
+def prefill_flops(model, tokens: int) -> float:
+    """Matrix products of every layer for all tokens of a prompt read from its start (each part says its own: projections,
+    causal attention), and the head for one row."""
+    return model.flops(tokens, tokens * (tokens + 1) // 2, 1)
 
 
 def decode_lead(batch: int, context: int, step_tokens: int) -> int:
@@ -127,25 +125,32 @@ def measure_decode(engine, batch: int, context: int, steps: int, warmup: int, se
 
 
 def measure_prefill(engine, tokens: int, repeats: int, seed: int):
+    """Seconds from handing the scheduler one prompt of `tokens` tokens to its first token, `repeats` times
+    (after one untimed run): admission, the step function on the whole prompt, the token's choice."""
     import numpy as np
     import torch
 
-    from llm_runtime_study_amd.engine.step import StepEntry
-
     rng = np.random.default_rng(seed)
-    runner = engine.runner
     times = []
+    scheduler = engine.create_scheduler(ignore_eos=True)
     with torch.cuda.device(engine.device), torch.cuda.stream(engine.stream):
-        for i in range(repeats + 1):
-            prompt = rng.integers(0, engine.config.vocab_size, tokens).tolist()
-            cache = runner.cache.admit(f"prefill{i}")
+        for _ in range(repeats + 1):
+            scheduler.add_request(rng.integers(0, engine.config.vocab_size, tokens).tolist(), max_new_tokens=1)
             engine.synchronize()
             started = time.perf_counter()
-            runner.step([StepEntry(cache, prompt, [tokens - 1])])
+            events = []
+            while scheduler.has_unfinished:
+                events += scheduler.step()
             engine.synchronize()
             times.append(time.perf_counter() - started)
-            runner.cache.release(cache)
+            assert len(events) == 1 and events[0][1].prompt_token_count == tokens
     return times[1:]  # the first run warms up buffers
+
+
+def prefill_entry(engine, tokens: int, dtype_name: str, seed: int) -> dict:
+    seconds = statistics.median(measure_prefill(engine, tokens, repeats=3, seed=seed))
+    return {"value": round(tokens / seconds, 1), "tokens": tokens, "ms": round(seconds * 1e3, 3),
+            "frac": round(prefill_flops(engine.model, tokens) / seconds / FLOP_PEAK[dtype_name], 4)}
 
 
 def main() -> int:
@@ -164,8 +169,12 @@ def main() -> int:
     raw = dict(SHAPES[args.shape], num_hidden_layers=args.layers)
     config = config_from_dict(raw)
     max_batch = args.batch if args.no_points else max(args.batch, 64)
-    max_seq_len = args.context + args.steps + args.warmup + decode_lead(max_batch, args.context, max(2048, args.prefill_tokens)) + max_batch + 64
-    max_seq_len = max(max_seq_len, args.prefill_tokens)
+    needed = args.context + args.steps + args.warmup + decode_lead(max_batch, args.context, max(2048, args.prefill_tokens)) + max_batch + 64
+    needed = max(needed, args.prefill_tokens + 1)
+    max_seq_len = max(needed, BENCHMARK_CONTEXT) if args.max_seq_len is None else args.max_seq_len
+    if max_seq_len < needed:
+        print(f"bench.py: --max-seq-len {max_seq_len} is less than the {needed} tokens the workload needs", file=sys.stderr)
+        return 2
     from llm_runtime_study_amd.kernels.ops import KernelChoice
 
     engine = Engine.from_config(config, seed=0, dtype=args.dtype, max_seq_len=max_seq_len, max_batch_size=max_batch,
@@ -174,9 +183,8 @@ def main() -> int:
                                 decode_steps_per_launch=args.decode_steps_per_launch)
     dtype_name = "bf16" if args.dtype == "bfloat16" else "fp32"
 
-    prefill_times = measure_prefill(engine, args.prefill_tokens, repeats=3, seed=1)
-    prefill_s = statistics.median(prefill_times)
-    flops = prefill_flops(config, args.prefill_tokens)
+    prefill = prefill_entry(engine, args.prefill_tokens, dtype_name, seed=1)
+    prefill_portion = prefill_entry(engine, PORTION_TOKENS, dtype_name, seed=5) if args.prefill_tokens != PORTION_TOKENS else prefill
 
     sampling = None
     if args.temperature > 0:
@@ -212,19 +220,16 @@ def main() -> int:
         "data": "synthetic (seeded uniform random token ids, random weights N(0, 0.02))",
         "config": {
             "model": f"Qwen3-{args.shape.upper()} shape", "layers": args.layers, "layers_of_shape": full_layers,
-            "hidden_size": config.hidden_size, "intermediate_size": config.intermediate_size,
-            "num_attention_heads": config.num_attention_heads, "num_key_value_heads": config.num_key_value_heads,
-            "head_dim": config.head_dim, "vocab_size": config.vocab_size, "global_batch": args.batch,
-            "seq_len": args.context, "new_tokens": args.steps + args.warmup, "page_size": engine.page_size,
-            "prefill_tokens": args.prefill_tokens, "hip_graph": bool(engine.runner.use_graph),
-            "decode_steps_per_launch": args.decode_steps_per_launch if engine.runner.use_graph else 1, "prefill_gemm": "own" if args.own_gemm else "hipBLASLt",
-            "parallelism": "single GPU",
+            **{key: raw[key] for key in SIZE_KEYS if key in raw},
+            "global_batch": args.batch, "seq_len": args.context, "new_tokens": args.steps + args.warmup,
+            "max_seq_len": max_seq_len, "num_pages": engine.cache_manager.groups[0].pool.num_pages, "page_size": engine.page_size,
+            "prefill_tokens": args.prefill_tokens,
+            "decode_steps_per_graph_launch": args.decode_steps_per_launch if engine.runner.use_graph else 0,
+            "prefill_gemm": "own" if args.own_gemm else "hipBLASLt", "parallelism": "single GPU",
             "sampling": "greedy" if sampling is None else f"temperature {args.temperature} top_k {args.top_k} top_p {args.top_p}",
         },
-        "prefill": {
-            "value": round(args.prefill_tokens / prefill_s, 1), "tokens": args.prefill_tokens,
-            "ms": round(prefill_s * 1e3, 3), "frac": round(flops / prefill_s / FLOP_PEAK[dtype_name], 4),
-        },
+        "prefill": prefill,
+        f"prefill_{PORTION_TOKENS}": prefill_portion,
         "roofline": {
             "bound": "hbm", "achieved": round(achieved / 1e9, 1), "peak": HBM_PEAK / 1e9, "unit": "GB/s",
             "frac": round(achieved / HBM_PEAK, 4),

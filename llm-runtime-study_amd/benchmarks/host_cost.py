@@ -107,7 +107,8 @@ def main(argv=None) -> int:
     # from the graph of the plan
     graphed = runner_like_the_engines(True)
     result["from_graph_of_plan"] = dict(measure(engine, graphed, args, rng, args.repeats, 2 + graphed.PLAN_GRAPH_AFTER),
-                                        recordings=graphed.plan_recordings, replays=graphed.plan_replays)
+                                        recordings=graphed.plan_recordings, replays=graphed.plan_replays,
+                                        graph_replays=graphed.plan_graph_replays)
     print(json.dumps(result), flush=True)
     return 0
 

@@ -722,7 +722,7 @@ __global__ void advance_decode_kernel(int* __restrict__ token_ids, int* __restri
                                       const int* __restrict__ real_rows, int rows) {
   const int t = blockIdx.x * blockDim.x + threadIdx.x;
   if (t >= rows || t >= *real_rows) return;
-  token_ids[t] = chosen[t];
+  token_ids[t] = chosen[t] >= 0 ? chosen[t] : 0;     // -1: a row whose logits were not finite (the host raises when it reads it)
   positions[t] += 1;
   seq_lens[token_request[t]] += 1;
   if (draws) draws[t] += 1;

@@ -20,14 +20,16 @@
 
 // lrs_choose_tokens_split() without its two scratch arguments: out[r] = the chosen token of row r of
 // logits [rows, vocab] (float32, row stride `row_stride`); temperature == nullptr or temperature[r] == 0
-// picks the lowest index among the largest logits, else a draw keyed by (seeds[r], counters[r]).  Each row is
+// picks the lowest index among the largest logits, else a draw keyed by (seeds[r], counters[r]).  A row that
+// holds a value that is not finite comes out as -1 (`filtered` != 0: rows of positive temperature may hold -inf,
+// as lrs_filter_logits() leaves them).  Each row is
 // cut into `parts` slices, one workgroup each; rows x parts must not exceed LRS_CHOOSE_STATIC_MAX_PARTS.
 // Results equal lrs_choose_tokens_split()'s for the same `parts`.  Every call on a GPU uses that GPU's one
 // scratch array (nothing in it needs clearing between calls): calls that overlap on one GPU race, so
 // keep them on one stream or order them yourself.  Returns 0, or 1 with a message for lrs_last_error().
 LRS_API int lrs_choose_tokens_static(int* out, const float* logits, int64_t row_stride, int rows, int vocab,
                                      const float* temperature, const uint64_t* seeds, const uint32_t* counters,
-                                     int parts, void* stream);
+                                     int parts, int filtered, void* stream);
 
 // Looks up the current device's copy of the scratch array now (otherwise the first call on a device does
 // it): call it once per device before a capture begins.  Safe to call again.

@@ -5,6 +5,11 @@
 //   keyed by (seed, draw counter, token index): the draw of a request depends on its own
 //   seed and on how many tokens it has drawn, never on the other rows of the batch.
 //   Entries equal to -inf (filtered out beforehand) are never chosen.
+//   A row that holds a value that is not finite is refused, as the reference refuses it
+//   (mini_llm/sampling.py:104-113): its token comes out as -1, which the host turns into an error.
+//   Rows that filter_logits() has been over (`filtered`, and a positive temperature) may hold -inf;
+//   NaN and +inf are refused there too, and filter_logits() leaves a NaN in a row that was not finite
+//   when it came.
 #include "common.h"
 #include "no_alloc.h"
 
@@ -35,7 +40,7 @@ __device__ __forceinline__ float exponential_variate(uint32_t seed_lo, uint32_t 
 __global__ __launch_bounds__(1024) void choose_token_kernel(
     int* __restrict__ out, const float* __restrict__ logits, int64_t row_stride, int vocab,
     const float* __restrict__ temperature, const uint64_t* __restrict__ seeds,
-    const uint32_t* __restrict__ counters) {
+    const uint32_t* __restrict__ counters, int filtered) {
   __shared__ float best_value[16];
   __shared__ int best_index[16];
   const int row = blockIdx.x, tid = threadIdx.x;
@@ -43,10 +48,13 @@ __global__ __launch_bounds__(1024) void choose_token_kernel(
   const float temp = temperature ? temperature[row] : 0.f;
   const uint64_t seed = seeds ? seeds[row] : 0;
   const uint32_t counter = counters ? counters[row] : 0;
+  const bool may_hold_minus_inf = filtered && temp > 0.f;
   float value = -INFINITY;
   int index = 0x7fffffff;
+  int bad = 0;
   for (int i = tid; i < vocab; i += blockDim.x) {
     float v = src[i];
+    if (!(fabsf(v) < INFINITY) && !(may_hold_minus_inf && v == -INFINITY)) bad = 1;
     if (temp > 0.f && v > -INFINITY)
       v = v / temp - logf(exponential_variate((uint32_t)seed, (uint32_t)(seed >> 32), counter, (uint32_t)i));
     if (v > value || (v == value && i < index)) {
@@ -68,7 +76,7 @@ __global__ __launch_bounds__(1024) void choose_token_kernel(
     best_value[wave] = value;
     best_index[wave] = index;
   }
-  __syncthreads();
+  bad = __syncthreads_or(bad);
   if (tid == 0) {
     const int waves = (blockDim.x + WAVE - 1) / WAVE;
     for (int i = 1; i < waves; ++i)
@@ -76,7 +84,7 @@ __global__ __launch_bounds__(1024) void choose_token_kernel(
         value = best_value[i];
         index = best_index[i];
       }
-    out[row] = index;
+    out[row] = bad || index == 0x7fffffff ? -1 : index;      // nothing finite to choose from is refused too
   }
 }
 
@@ -86,7 +94,7 @@ __global__ __launch_bounds__(1024) void choose_token_kernel(
 __global__ __launch_bounds__(256) void choose_token_part_kernel(
     float* __restrict__ part_value, int* __restrict__ part_index, const float* __restrict__ logits,
     int64_t row_stride, int vocab, int parts, const float* __restrict__ temperature,
-    const uint64_t* __restrict__ seeds, const uint32_t* __restrict__ counters) {
+    const uint64_t* __restrict__ seeds, const uint32_t* __restrict__ counters, int filtered) {
   __shared__ float best_value[4];
   __shared__ int best_index[4];
   const int row = blockIdx.y, part = blockIdx.x, tid = threadIdx.x;
@@ -94,12 +102,15 @@ __global__ __launch_bounds__(256) void choose_token_part_kernel(
   const float temp = temperature ? temperature[row] : 0.f;
   const uint64_t seed = seeds ? seeds[row] : 0;
   const uint32_t counter = counters ? counters[row] : 0;
+  const bool may_hold_minus_inf = filtered && temp > 0.f;
   const int per = (vocab + parts - 1) / parts;
   const int begin = part * per, end = begin + per < vocab ? begin + per : vocab;
   float value = -INFINITY;
   int index = 0x7fffffff;
+  int bad = 0;
   for (int i = begin + tid; i < end; i += 256) {
     float v = src[i];
+    if (!(fabsf(v) < INFINITY) && !(may_hold_minus_inf && v == -INFINITY)) bad = 1;
     if (temp > 0.f && v > -INFINITY)
       v = v / temp - logf(exponential_variate((uint32_t)seed, (uint32_t)(seed >> 32), counter, (uint32_t)i));
     if (v > value || (v == value && i < index)) {
@@ -120,14 +131,14 @@ __global__ __launch_bounds__(256) void choose_token_part_kernel(
     best_value[tid / WAVE] = value;
     best_index[tid / WAVE] = index;
   }
-  __syncthreads();
+  bad = __syncthreads_or(bad);
   if (tid == 0) {
     for (int i = 1; i < 4; ++i)
       if (best_value[i] > value || (best_value[i] == value && best_index[i] < index)) {
         value = best_value[i];
         index = best_index[i];
       }
-    part_value[(int64_t)row * parts + part] = value;
+    part_value[(int64_t)row * parts + part] = bad ? NAN : value;      // a NaN tells the second pass to refuse the row
     part_index[(int64_t)row * parts + part] = index;
   }
 }
@@ -137,9 +148,11 @@ __global__ void choose_token_final_kernel(int* __restrict__ out, const float* __
   const int row = blockIdx.x, lane = threadIdx.x;
   float value = -INFINITY;
   int index = 0x7fffffff;
+  bool bad = false;
   for (int i = lane; i < parts; i += WAVE) {
     const float v = part_value[(int64_t)row * parts + i];
     const int at = part_index[(int64_t)row * parts + i];
+    if (v != v) bad = true;
     if (v > value || (v == value && at < index)) {
       value = v;
       index = at;
@@ -154,19 +167,21 @@ __global__ void choose_token_final_kernel(int* __restrict__ out, const float* __
       index = oi;
     }
   }
-  if (lane == 0) out[row] = index;
+  bad = __any(bad);
+  if (lane == 0) out[row] = bad || index == 0x7fffffff ? -1 : index;
 }
 
-// out[r] = chosen token of row r.  temperature == nullptr or temperature[r] == 0: greedy.
+// out[r] = chosen token of row r, or -1 for a row that is not finite.  temperature == nullptr or temperature[r] == 0:
+// greedy.  filtered: filter_logits() has been over the rows (those of positive temperature may hold -inf).
 // part_value / part_index [rows, parts] are scratch for the two-pass form (parts > 1).
 LRS_API int lrs_choose_tokens_split(int* out, const float* logits, int64_t row_stride, int rows, int vocab,
                                     const float* temperature, const uint64_t* seeds, const uint32_t* counters,
-                                    float* part_value, int* part_index, int parts, void* stream) {
+                                    float* part_value, int* part_index, int parts, int filtered, void* stream) {
   LRS_REQUIRE(rows > 0 && vocab > 0 && parts > 0, "choose_tokens: rows=%d vocab=%d parts=%d must be positive", rows, vocab, parts);
   LRS_REQUIRE(row_stride >= vocab, "choose_tokens: row stride below vocab");
   LRS_REQUIRE(part_value && part_index, "choose_tokens: the two-pass form needs its scratch buffers");
   choose_token_part_kernel<<<dim3(parts, rows), 256, 0, (hipStream_t)stream>>>(part_value, part_index, logits, row_stride, vocab,
-                                                                               parts, temperature, seeds, counters);
+                                                                               parts, temperature, seeds, counters, filtered);
   if (lrs_check_launch("choose_tokens_part")) return 1;
   choose_token_final_kernel<<<rows, WAVE, 0, (hipStream_t)stream>>>(out, part_value, part_index, parts);
   return lrs_check_launch("choose_tokens_final");
@@ -211,7 +226,7 @@ LRS_API int lrs_choose_tokens_static_max_parts() { return LRS_CHOOSE_STATIC_MAX_
 
 LRS_API int lrs_choose_tokens_static(int* out, const float* logits, int64_t row_stride, int rows, int vocab,
                                      const float* temperature, const uint64_t* seeds, const uint32_t* counters,
-                                     int parts, void* stream) {
+                                     int parts, int filtered, void* stream) {
   LRS_REQUIRE(rows > 0 && vocab > 0 && parts > 0, "choose_tokens_static: rows=%d vocab=%d parts=%d must be positive", rows, vocab, parts);
   LRS_REQUIRE(row_stride >= vocab, "choose_tokens_static: row stride below vocab");
   LRS_REQUIRE(out && logits, "choose_tokens_static: out and logits are required");
@@ -222,7 +237,7 @@ LRS_API int lrs_choose_tokens_static(int* out, const float* logits, int64_t row_
   float* part_value = (float*)scratch;
   int* part_index = (int*)((unsigned char*)scratch + (size_t)LRS_CHOOSE_STATIC_MAX_PARTS * 4);
   choose_token_part_kernel<<<dim3(parts, rows), 256, 0, (hipStream_t)stream>>>(part_value, part_index, logits, row_stride, vocab,
-                                                                               parts, temperature, seeds, counters);
+                                                                               parts, temperature, seeds, counters, filtered);
   if (lrs_check_launch("choose_tokens_static_part")) return 1;
   choose_token_final_kernel<<<rows, WAVE, 0, (hipStream_t)stream>>>(out, part_value, part_index, parts);
   return lrs_check_launch("choose_tokens_static_final");
@@ -231,12 +246,12 @@ LRS_API int lrs_choose_tokens_static(int* out, const float* logits, int64_t row_
 // out[r] = chosen token of row r.  temperature == nullptr or temperature[r] == 0: greedy.
 LRS_API int lrs_choose_tokens(int* out, const float* logits, int64_t row_stride, int rows, int vocab,
                               const float* temperature, const uint64_t* seeds,
-                              const uint32_t* counters, void* stream) {
+                              const uint32_t* counters, int filtered, void* stream) {
   LRS_REQUIRE(rows > 0 && vocab > 0, "choose_tokens: rows=%d vocab=%d must be positive", rows, vocab);
   LRS_REQUIRE(row_stride >= vocab, "choose_tokens: row stride below vocab");
   const int threads = vocab >= 4096 ? 1024 : 256;
   choose_token_kernel<<<rows, threads, 0, (hipStream_t)stream>>>(out, logits, row_stride, vocab,
-                                                                 temperature, seeds, counters);
+                                                                 temperature, seeds, counters, filtered);
   return lrs_check_launch("choose_tokens");
 }
 
@@ -305,7 +320,6 @@ __global__ __launch_bounds__(1024) void filter_logits_kernel(float* __restrict__
   const int k = top_k ? top_k[row] : 0;
   const float p = top_p ? top_p[row] : 1.f;
   const bool use_k = k > 0 && k < vocab, use_p = p < 1.f;
-  if (!use_k && !use_p) return;
 
   // A pass over the row: body(index, logit) for each of this thread's values.  Four loads of 16 bytes are asked
   // for before any is used (a thread's loads one after the other, each waited for, were what a pass took its
@@ -334,8 +348,21 @@ __global__ __launch_bounds__(1024) void filter_logits_kernel(float* __restrict__
     for (int i = fours * 4 + tid; i < vocab; i += blockDim.x) body(i, z[i]);
   };
 
+  // Every row of positive temperature is looked over once, filtered or not: a row that is not finite as it comes
+  // (the reference refuses it, mini_llm/sampling.py:104-113) gets a NaN that the token choice after this kernel
+  // refuses, since it can no longer tell a -inf that came from one that a filter left.
   float zmax = -INFINITY;
-  walk([&](int, float v) { zmax = fmaxf(zmax, v); });
+  int bad = 0;
+  walk([&](int, float v) {
+    zmax = fmaxf(zmax, v);
+    if (!(fabsf(v) < INFINITY)) bad = 1;
+  });
+  bad = __syncthreads_or(bad);
+  if (bad) {
+    if (tid == 0) z[0] = NAN;
+    return;
+  }
+  if (!use_k && !use_p) return;
   zmax = block_max(zmax, scratch);
   const float per_temp2 = 1.4426950408889634f / temp;          // exp(x / temp) = exp2(x * this)
 

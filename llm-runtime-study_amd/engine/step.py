@@ -34,6 +34,7 @@ from ..errors import GenerationError, KVCacheError
 from ..kernels import ops
 from ..models import DecoderModel
 from ..parts.base import length_class
+from ..sampling.sampler import refuse_not_finite
 
 
 @dataclass
@@ -152,6 +153,7 @@ class ModelRunner:
         self._plans: dict[tuple, RecordedStep] = {}
         self.plan_replays = 0
         self.plan_recordings = 0
+        self.plan_graph_replays = 0     # of the replays, those made by launching the graph of a plan
         self.graph_replays = 0     # steps (or launches of several steps) served by replaying a graph
         self.graph_captures = 0    # ... and those that ran eagerly and were captured on the way
         # query groups for the ragged attention kernel: at most `query_group` consecutive tokens of one request
@@ -454,6 +456,7 @@ class ModelRunner:
                 known.graph = ops.graph_end()
             if known.graph is not None and stream != 0:
                 ops.graph_launch(known.graph)
+                self.plan_graph_replays += 1
             else:
                 ops.plan_run(known.plan)
             self.plan_replays += 1
@@ -559,7 +562,7 @@ class ModelRunner:
         sampled = sampling is not None and any(not row.config.greedy for row in sampling)
         if sampled:
             self._upload_sampling(sampling)
-        return [row[:len(entries)] for row in self._run_decode_graph(ctx, bucket, steps, sampled)]
+        return [row[:len(entries)] for row in self._run_decode_graph(ctx, bucket, steps, sampled, len(entries))]
 
     def _upload_sampling(self, sampling: Sequence) -> None:
         """Temperature, top-p, top-k, draws so far and seed of every row, in one buffer on the device
@@ -584,7 +587,8 @@ class ModelRunner:
         return (dev[:cap].view(torch.float32)[:rows], dev[cap:2 * cap].view(torch.float32)[:rows], dev[2 * cap:3 * cap][:rows],
                 dev[3 * cap:4 * cap][:rows], dev[4 * cap:6 * cap].view(torch.int64)[:rows])
 
-    def _run_decode_graph(self, ctx: StepContext, bucket: int, steps: int, sampled: bool = False) -> list[list[int]]:
+    def _run_decode_graph(self, ctx: StepContext, bucket: int, steps: int, sampled: bool = False, real: int | None = None) -> list[list[int]]:
+        real = bucket if real is None else real
         key = (bucket, length_class(ctx.max_k), steps, sampled)
         if self._chosen_dev is None:
             rows = self.MAX_DECODE_STEPS * (-(-self.max_requests // 4) * 4)
@@ -615,7 +619,10 @@ class ModelRunner:
             ops.graph_launch(graph[0])
             self.graph_replays += 1
         torch.cuda.current_stream(self.device).synchronize()
-        return [self._chosen_host[i * stride:i * stride + bucket].tolist() for i in range(steps)]
+        chosen = [self._chosen_host[i * stride:i * stride + bucket].tolist() for i in range(steps)]
+        for row in chosen:
+            refuse_not_finite(row[:real])       # a row whose logits were not finite (rows that pad the batch are not looked at)
+        return chosen
 
     def _decode_steps_on_stream(self, ctx: StepContext, steps: int, stride: int, sampled: bool) -> None:
         draws = None
@@ -628,7 +635,7 @@ class ModelRunner:
             chosen = self._chosen_dev[i * stride:i * stride + ctx.T]
             if sampled:
                 ops.filter_logits(logits, temperature, top_k, top_p)
-                ops.choose_tokens(chosen, logits, temperature, seeds, draws)
+                ops.choose_tokens(chosen, logits, temperature, seeds, draws, filtered=True)
             else:
                 ops.choose_tokens(chosen, logits)
             if i + 1 < steps:

@@ -40,7 +40,8 @@ def build_parser() -> argparse.ArgumentParser:
     return parser
 
 
-def make_runner(model_dir, dtype_name: str, max_tokens: int, page_size: int = PAGE_SIZE, library_gemm: bool = True):
+def make_runner(model_dir, dtype_name: str, max_tokens: int, page_size: int = PAGE_SIZE, library_gemm: bool = True,
+                use_graph: bool = False):
     device = resolve_device("auto")
     dtype = resolve_dtype(dtype_name)
     # a replay takes the folder as it is: tensors stored in 32-bit beside bfloat16 ones stay 32-bit
@@ -50,7 +51,8 @@ def make_runner(model_dir, dtype_name: str, max_tokens: int, page_size: int = PA
     num_pages = -(-max_tokens // page_size)
     cache = CacheManager(model.cache_needs(), page_size=page_size, num_pages=num_pages, max_requests=MAX_LIVE_REQUESTS,
                          max_seq_len=min(model.spec.max_positions, num_pages * page_size), dtype=dtype, device=device)
-    runner = ModelRunner(model, cache, max_step_tokens=num_pages * page_size, dtype=dtype, device=device, library_gemm=library_gemm)
+    runner = ModelRunner(model, cache, max_step_tokens=num_pages * page_size, dtype=dtype, device=device, library_gemm=library_gemm,
+                         use_graph=use_graph)
     return runner
 
 

@@ -120,9 +120,9 @@ _SIGNATURES = {
     "lrs_gemm_lines_split_pays": (c_int, [c_int, c_int, c_int]),
     "lrs_attention_prefill_group": (c_int, []),
     "lrs_attention_prefill_group_for": (c_int, [c_int, c_int]),
-    "lrs_choose_tokens": (c_int, [c_void_p, c_void_p, c_int64, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p]),
-    "lrs_choose_tokens_split": (c_int, [c_void_p, c_void_p, c_int64, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p]),
-    "lrs_choose_tokens_static": (c_int, [c_void_p, c_void_p, c_int64, c_int, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p]),
+    "lrs_choose_tokens": (c_int, [c_void_p, c_void_p, c_int64, c_int, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p]),
+    "lrs_choose_tokens_split": (c_int, [c_void_p, c_void_p, c_int64, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p]),
+    "lrs_choose_tokens_static": (c_int, [c_void_p, c_void_p, c_int64, c_int, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p]),
     "lrs_choose_tokens_static_init": (c_int, []),
     "lrs_choose_tokens_static_max_parts": (c_int, []),
     "lrs_filter_logits": (c_int, [c_void_p, c_int64, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p]),
@@ -913,10 +913,12 @@ _choose_scratch: dict = {}
 
 
 def choose_tokens(out: torch.Tensor, logits: torch.Tensor, temperature=None, seeds=None, counters=None,
-                  out_address: int | None = None) -> None:
+                  out_address: int | None = None, filtered: bool = False) -> None:
     """One token per row of logits into `out`, int32 [R] on the device; or, with `out_address` (from
     pinned_device_address(out)), into pinned host memory that the kernel writes directly and the
-    host reads after synchronising the stream."""
+    host reads after synchronising the stream.  A row that holds a value that is not finite gets -1
+    (the reference refuses such logits, mini_llm/sampling.py:104-113); `filtered`: filter_logits() has
+    been over the rows, so those of positive temperature may hold -inf."""
     rows, vocab = logits.shape
     _need(out.dtype == torch.int32 and out.numel() >= rows and out.is_contiguous(), "choose_tokens: out must be int32 [R]")
     stride = _rows(logits, "logits")
@@ -939,12 +941,13 @@ def choose_tokens(out: torch.Tensor, logits: torch.Tensor, temperature=None, see
             scratch = _choose_scratch[key] = (torch.empty(rows * parts, dtype=torch.float32, device=logits.device),
                                               torch.empty(rows * parts, dtype=torch.int32, device=logits.device))
         _launch("lrs_choose_tokens_split", out_pointer, _dev(logits, "logits", torch.float32), stride, rows, vocab, *args,
-                                                 _dev(scratch[0], "part_value"), _dev(scratch[1], "part_index"), parts, _stream())
+                                                 _dev(scratch[0], "part_value"), _dev(scratch[1], "part_index"), parts, int(bool(filtered)), _stream())
         return
-    _launch("lrs_choose_tokens", out_pointer, _dev(logits, "logits", torch.float32), stride, rows, vocab, *args, _stream())
+    _launch("lrs_choose_tokens", out_pointer, _dev(logits, "logits", torch.float32), stride, rows, vocab, *args, int(bool(filtered)), _stream())
 
 
-def choose_tokens_static(out: torch.Tensor, logits: torch.Tensor, parts: int, temperature=None, seeds=None, counters=None) -> None:
+def choose_tokens_static(out: torch.Tensor, logits: torch.Tensor, parts: int, temperature=None, seeds=None, counters=None,
+                         filtered: bool = False) -> None:
     """choose_tokens() in its two-pass form (`parts` slices a row) for callers that must not allocate: the
     slices' results go to a fixed array inside the library (rows * parts at most
     lrs_choose_tokens_static_max_parts()), so nothing is allocated here or there.  Calls that overlap on
@@ -958,7 +961,7 @@ def choose_tokens_static(out: torch.Tensor, logits: torch.Tensor, parts: int, te
     _launch("lrs_choose_tokens_static", 
         _dev(out, "out"), _dev(logits, "logits", torch.float32), _rows(logits, "logits"), rows, vocab,
         None if temperature is None else _dev(temperature, "temperature"), None if temperature is None else _dev(seeds, "seeds"),
-        None if temperature is None else _dev(counters, "counters"), parts, _stream())
+        None if temperature is None else _dev(counters, "counters"), parts, int(bool(filtered)), _stream())
 
 
 def filter_logits(logits: torch.Tensor, temperature: torch.Tensor, top_k: torch.Tensor | None, top_p: torch.Tensor | None) -> None:

@@ -78,6 +78,12 @@ class DecoderModel:
             total += self.embedding.numel() * self.embedding.element_size()
         return total
 
+    def flops(self, tokens: int, pairs: int, logit_rows: int = 1) -> float:
+        """Floating-point operations of the matrix products of one step of `tokens` tokens: every scheduled layer
+        (what each part says of itself, see Part.flops for `pairs`) and the head for `logit_rows` rows."""
+        total = sum(self.layers[e.layer].flops(tokens, pairs) for e in self.spec.schedule)
+        return total + 2.0 * logit_rows * self.spec.vocab_size * self.spec.hidden_size
+
     # ------------------------------------------------------------------ forward
     def forward_hidden(self, ctx) -> torch.Tensor:
         """Residual stream [T, H] float32 after the last layer (before the final norm)."""

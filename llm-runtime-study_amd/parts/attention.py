@@ -78,6 +78,12 @@ class GQAAttention(Part):
     def weight_bytes(self):
         return (self.w_qkv.numel() + self.w_o.numel()) * self.w_o.element_size()
 
+    def flops(self, tokens, pairs):
+        if self.window is not None:
+            pairs = min(pairs, tokens * self.window)
+        # the projections, then scores and weighted values: two products of head_dim per pair and query head
+        return super().flops(tokens, pairs) + 4.0 * pairs * self.num_heads * self.head_dim
+
     def cache_need(self):
         if self.kv_shared:
             return None

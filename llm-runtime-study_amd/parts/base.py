@@ -41,6 +41,7 @@ scratch arena.  The residual stream `h` is float32 in every precision mode.
 
 from __future__ import annotations
 
+import math
 from dataclasses import dataclass, field
 from typing import Any, Mapping
 
@@ -120,6 +121,14 @@ class Part:
     def weight_bytes(self) -> int:
         """Bytes of weights that one step reads (for roofline accounting)."""
         return 0
+
+    def flops(self, tokens: int, pairs: int) -> float:
+        """Floating-point operations of this part's matrix products in a step of `tokens` tokens (for roofline
+        accounting; elementwise work is left out).  `pairs` is the number of (query, earlier-or-same position)
+        pairs of the step under a causal mask: tokens * (tokens + 1) / 2 for a prompt read from its start, the
+        sum of the context lengths for decoding requests.  Only mixers that look back use it.  Unless a part says
+        otherwise: every matrix it declares in tensors() is multiplied with every token once."""
+        return 2.0 * tokens * sum(math.prod(spec.shape) for spec in self.tensors().values() if spec.role == "matrix")
 
 
 def length_class(length: int) -> int:

@@ -35,6 +35,9 @@ class PreNormBlock(Part):
     def weight_bytes(self):
         return sum(part.weight_bytes() for _, part in self._children())
 
+    def flops(self, tokens, pairs):
+        return sum(part.flops(tokens, pairs) for _, part in self._children())
+
     def cache_need(self):
         return self.mixer.cache_need()
 

@@ -34,6 +34,13 @@ class SamplingRow:
     counter: int  # tokens this request has drawn so far
 
 
+def refuse_not_finite(tokens) -> None:
+    """The kernels give -1 for a row of logits that holds a value that is not finite; the reference refuses
+    such logits with this message (mini_llm/sampling.py:104-113)."""
+    if any(token < 0 for token in tokens):
+        raise SamplingError("logits must contain only finite values")
+
+
 class Sampler:
     def __init__(self, device):
         self.device = torch.device(device)
@@ -48,7 +55,9 @@ class Sampler:
 
     def _read(self, out: torch.Tensor) -> list[int]:
         torch.cuda.current_stream(self.device).synchronize()
-        return out.tolist()
+        tokens = out.tolist()
+        refuse_not_finite(tokens)
+        return tokens
 
     def choose(self, logits: torch.Tensor, rows: list[SamplingRow]) -> list[int]:
         """One token per row of `logits` [R, V] float32 (filters the sampled rows in place)."""
@@ -65,9 +74,10 @@ class Sampler:
         temperature = torch.tensor([row.config.temperature for row in rows], dtype=torch.float32, device=self.device)
         seeds = torch.tensor([row.seed for row in rows], dtype=torch.int64, device=self.device)
         counters = torch.tensor([row.counter for row in rows], dtype=torch.int32, device=self.device)
-        if any((row.config.top_k is not None and row.config.top_k < vocab) or row.config.top_p < 1.0 for row in rows if not row.config.greedy):
+        filtered = any((row.config.top_k is not None and row.config.top_k < vocab) or row.config.top_p < 1.0 for row in rows if not row.config.greedy)
+        if filtered:
             top_k = torch.tensor([row.config.top_k or 0 for row in rows], dtype=torch.int32, device=self.device)
             top_p = torch.tensor([row.config.top_p for row in rows], dtype=torch.float32, device=self.device)
             ops.filter_logits(logits, temperature, top_k, top_p)
-        ops.choose_tokens(out, logits, temperature, seeds, counters, out_address=self._chosen_address)
+        ops.choose_tokens(out, logits, temperature, seeds, counters, out_address=self._chosen_address, filtered=filtered)
         return self._read(out)

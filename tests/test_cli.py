@@ -154,12 +154,16 @@ def test_bench_counts_the_flops_and_the_lead_of_early_requests():
 
     from llm_runtime_study_amd.config import config_from_dict
 
-    c = config_from_dict(bench.QWEN3_8B)
-    per_layer = bench.matrix_params_per_layer(c)
-    assert per_layer == (32 + 16) * 128 * 4096 + 4096 * 4096 + 3 * 4096 * 12288
+    from llm_runtime_study_amd.config import spec_for
+    from llm_runtime_study_amd.models import DecoderModel
+
+    # the model says its own operations, part by part, from the tensors it declares (nothing is allocated for that)
+    model = DecoderModel(spec_for(config_from_dict(bench.QWEN3_8B)))
+    per_layer = (32 + 16) * 128 * 4096 + 4096 * 4096 + 3 * 4096 * 12288
     linear = 2.0 * 2048 * per_layer * 36 + 2.0 * 4096 * 151936
     attention = 4.0 * (2048 * 2049 / 2) * 32 * 128 * 36
-    assert bench.prefill_flops(c, 2048) == linear + attention
+    assert bench.prefill_flops(model, 2048) == linear + attention
+    assert model.flops(8, 8 * 2049, 8) == 2.0 * 8 * per_layer * 36 + 8 * 2.0 * 4096 * 151936 + 4.0 * 8 * 2049 * 32 * 128 * 36
     # eight prompts of 2,048 tokens read one a step: the first request is seven tokens ahead of the last
     assert bench.decode_lead(8, 2048, 2048) == 7
     assert bench.decode_lead(8, 32768, 2048) == 7 * 16 and bench.decode_lead(1, 5000, 2048) == 0

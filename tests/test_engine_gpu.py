@@ -404,6 +404,34 @@ def test_sampled_tokens_do_not_depend_on_steps_per_launch(folders):
     assert replays_several < replays_single
 
 
+@pytest.mark.parametrize("graph,steps_per_launch", [(False, 1), (True, 1), (True, 4)], ids=["eager", "graph", "four-steps-a-launch"])
+def test_logits_that_are_not_finite_abort_generation(folders, graph, steps_per_launch):
+    """A request whose logits turn NaN while it decodes (the embedding row of its first generated token is
+    poisoned) beside a healthy one: the step raises the reference's error (mini_llm/sampling.py:104-113), whether
+    the host or the device chooses the tokens, every page comes back, and the engine generates again afterwards."""
+    from llm_runtime_study_amd import Engine
+    from llm_runtime_study_amd.errors import SamplingError
+
+    folder, cfg, weights = folders["c"]
+    rng = np.random.default_rng(12)
+    prompts = [rng.integers(0, cfg["vocab_size"], n).tolist() for n in (9, 14)]
+    expected = [plain_greedy(cfg, weights, p, 6) for p in prompts]
+    poisoned = expected[0][0]
+    assert poisoned not in prompts[0] + prompts[1] + expected[1]
+    engine = Engine.from_model_dir(folder, dtype="float32", max_seq_len=64, max_batch_size=2, max_num_batched_tokens=32,
+                                   use_cuda_graph=graph, decode_steps_per_launch=steps_per_launch)
+    assert engine.generate_tokens(prompts, max_new_tokens=6, ignore_eos=True) == expected
+    row = engine.model.embedding[poisoned].clone()
+    engine.model.embedding[poisoned] = float("nan")
+    with pytest.raises(SamplingError, match="only finite values"):
+        engine.generate_tokens(prompts, max_new_tokens=6, ignore_eos=True)
+    manager = engine.cache_manager
+    manager.check_invariants()
+    assert manager.active_requests == 0 and manager.used_pages() == 0
+    engine.model.embedding[poisoned] = row
+    assert engine.generate_tokens(prompts, max_new_tokens=6, ignore_eos=True) == expected
+
+
 def test_small_pool_makes_requests_wait_and_reuses_pages(folders):
     from llm_runtime_study_amd import Engine
 
@@ -542,8 +570,8 @@ def test_staggered_benchmark_runs_every_request_to_its_limit(capsys):
 @pytest.mark.gpu
 def test_host_cost_benchmark_times_the_three_ways_of_launching_a_step(capsys):
     """One layer of the 8B shape, a 64-token portion beside two decoding requests: the report holds the three
-    ways of launching, the plan is recorded once and replayed for every timed step, and the graph of the plan
-    costs the host less than the parts do."""
+    ways of launching, the plan is recorded once and replayed for every timed step, and every timed step of the
+    third way is a launch of the plan's graph."""
     import json
 
     from llm_runtime_study_amd.benchmarks import host_cost
@@ -554,7 +582,9 @@ def test_host_cost_benchmark_times_the_three_ways_of_launching_a_step(capsys):
     for way in ("through_parts", "from_plan", "from_graph_of_plan"):
         assert 0 < report[way]["host_ms"] <= report[way]["total_ms"]
     assert report["from_plan"]["replays"] >= 3 and report["from_graph_of_plan"]["replays"] >= 3
-    assert report["from_graph_of_plan"]["host_ms"] < report["through_parts"]["host_ms"]
+    # two shapes are recorded, once each: the step that reads a decoding request's context and the timed step
+    assert report["from_plan"]["recordings"] == 2 and report["from_graph_of_plan"]["recordings"] == 2
+    assert report["from_graph_of_plan"]["graph_replays"] >= 3
 
 
 def test_a_cache_pool_the_device_cannot_hold_is_refused_before_anything_is_allocated():

@@ -968,7 +968,7 @@ def test_choose_tokens_two_pass_equals_one_pass(ops):
     ops.choose_tokens(two, logits, temps, seeds, counters)
     one = torch.empty(rows, dtype=torch.int32, device="cuda")
     code = ops.library().lrs_choose_tokens(one.data_ptr(), logits.data_ptr(), vocab, rows, vocab, temps.data_ptr(), seeds.data_ptr(),
-                                           counters.data_ptr(), torch.cuda.current_stream().cuda_stream)
+                                           counters.data_ptr(), 0, torch.cuda.current_stream().cuda_stream)
     assert code == 0 and one.cpu().tolist() == two.cpu().tolist()
     assert two.cpu()[0] == logits[0].argmax().cpu() and two.cpu()[1] != logits[1].argmax().cpu()
 
@@ -982,17 +982,64 @@ def test_choose_tokens_temperature_statistics(ops):
     temps = torch.full((draws,), temperature, device="cuda")
     seeds = torch.full((draws,), 1234, dtype=torch.int64, device="cuda")
     counters = torch.arange(draws, dtype=torch.int32, device="cuda")
-    ops.choose_tokens(out, dev(logits), temps, seeds, counters)
+    ops.choose_tokens(out, dev(logits), temps, seeds, counters, filtered=True)   # -inf as a filter leaves it
     freq = torch.bincount(out.cpu().long(), minlength=vocab).float() / draws
     assert freq[-1] == 0  # a -inf logit is never drawn
     assert (freq - probs).abs().max() < 0.012
     # reproducible, and a row's draw does not depend on its neighbours
     again = torch.empty(7, dtype=torch.int32, device="cuda")
-    ops.choose_tokens(again, dev(logits[:7]), temps[:7], seeds[:7], counters[100:107].contiguous())
+    ops.choose_tokens(again, dev(logits[:7]), temps[:7], seeds[:7], counters[100:107].contiguous(), filtered=True)
     assert again.cpu().tolist() == out.cpu()[100:107].tolist()
     other = torch.empty(draws, dtype=torch.int32, device="cuda")
-    ops.choose_tokens(other, dev(logits), temps, seeds + 1, counters)
+    ops.choose_tokens(other, dev(logits), temps, seeds + 1, counters, filtered=True)
     assert (other != out).float().mean() > 0.3
+
+
+@pytest.mark.parametrize("vocab", [1000, 151936], ids=["one-pass", "two-pass"])
+def test_rows_that_are_not_finite_are_refused(ops, vocab):
+    """The reference refuses logits that hold a value that is not finite (mini_llm/sampling.py:104-113): here such a
+    row's token comes out as -1 beside healthy rows, greedy or drawn, filtered or not, and the sampler raises."""
+    from llm_runtime_study_amd.errors import SamplingError
+    from llm_runtime_study_amd.sampling import Sampler, SamplingConfig, SamplingRow
+
+    g = torch.Generator().manual_seed(21)
+    base = torch.randn(6, vocab, generator=g)
+    base[1, vocab - 3] = float("nan")
+    base[3, 17] = float("inf")
+    base[4, vocab // 2] = float("-inf")
+    base[5, :] = float("-inf")                       # nothing to choose from
+    out = torch.empty(6, dtype=torch.int32, device="cuda")
+    ops.choose_tokens(out, dev(base))
+    assert out.cpu().tolist() == [int(base[0].argmax()), -1, int(base[2].argmax()), -1, -1, -1]
+    # drawn rows without a filter: the same rows are refused
+    temps = torch.full((6,), 0.8, device="cuda")
+    seeds = torch.arange(6, dtype=torch.int64, device="cuda")
+    counters = torch.zeros(6, dtype=torch.int32, device="cuda")
+    ops.choose_tokens(out, dev(base), temps, seeds, counters)
+    got = out.cpu().tolist()
+    assert [t < 0 for t in got] == [False, True, False, True, True, True] and all(t < vocab for t in got)
+    # after filter_logits() a -inf is what a filter leaves, but the rows that came with one are still refused:
+    # the filter marks them; a greedy row among them (temperature 0) is never filtered and is looked at as it came
+    work = dev(base.clone())
+    temps = torch.tensor([0.8, 0.8, 0.0, 0.8, 0.8, 0.8], device="cuda")
+    ks = torch.tensor([5, 5, 0, 0, 5, 5], dtype=torch.int32, device="cuda")
+    ps = torch.tensor([1.0, 1.0, 1.0, 0.9, 1.0, 0.5], device="cuda")
+    ops.filter_logits(work, temps, ks, ps)
+    ops.choose_tokens(out, work, temps, seeds, counters, filtered=True)
+    got = out.cpu().tolist()
+    assert [t < 0 for t in got] == [False, True, False, True, True, True]
+    assert got[2] == int(base[2].argmax()) and got[0] in base[0].topk(5).indices.tolist()
+    assert torch.isfinite(work[0]).sum().item() == 5 and torch.isfinite(work[2]).all()
+
+    sampler = Sampler("cuda")
+    for config in (SamplingConfig(), SamplingConfig(temperature=0.8, seed=1), SamplingConfig(temperature=0.8, top_k=7, seed=1),
+                   SamplingConfig(temperature=0.8, top_p=0.9, seed=1)):
+        rows = [SamplingRow(config, 1, 0)] * 2
+        healthy = sampler.choose(dev(base[[0, 2]].clone()), rows)
+        assert all(0 <= t < vocab for t in healthy)
+        for bad in (1, 3, 4):
+            with pytest.raises(SamplingError, match="only finite values"):
+                sampler.choose(dev(base[[0, bad]].clone()), rows)
 
 
 def test_filter_logits_matches_sort_based_rule(ops):

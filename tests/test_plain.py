@@ -235,6 +235,69 @@ def test_model_invariants(cfg):
     torch.testing.assert_close(plain.qwen3_forward(wz, cfg, ids), want)
 
 
+def _one_token_by_hand(w, cfg, token, eps, parallel=False, embedding_scale=1.0):
+    """Logits of a sequence of one token, written with library routines only.  One token attends to itself with
+    weight 1, so attention is o_proj of its own value heads, each repeated for the query heads of its group: no
+    rotation, no q or k, no softmax.  mini_llm/model/qwen.py:58-72 (the block), mini_llm/model/base.py:72-89 (embedding
+    without a multiplier for this family, final norm), mini_llm/model/qwen.py:109-112 (head)."""
+    nq, nkv, d = cfg["num_attention_heads"], cfg["num_key_value_heads"], cfg["head_dim"]
+    h = embedding_scale * w["model.embed_tokens.weight"][token]
+    for i in range(cfg["num_hidden_layers"]):
+        p = f"model.layers.{i}"
+        x = F.rms_norm(h, h.shape, w[f"{p}.input_layernorm.weight"], eps)
+        v = F.linear(x, w[f"{p}.self_attn.v_proj.weight"], w.get(f"{p}.self_attn.v_proj.bias"))
+        merged = v.view(nkv, 1, d).expand(nkv, nq // nkv, d).reshape(nq * d)
+        attn = F.linear(merged, w[f"{p}.self_attn.o_proj.weight"])
+        after = h + attn
+        y = F.rms_norm(h if parallel else after, h.shape, w[f"{p}.post_attention_layernorm.weight"], eps)
+        mlp = F.linear(F.silu(F.linear(y, w[f"{p}.mlp.gate_proj.weight"])) * F.linear(y, w[f"{p}.mlp.up_proj.weight"]), w[f"{p}.mlp.down_proj.weight"])
+        h = after + mlp
+    head = w.get("lm_head.weight", w["model.embed_tokens.weight"])
+    return F.linear(F.rms_norm(h, h.shape, w["model.norm.weight"], eps), head)
+
+
+@pytest.mark.parametrize("cfg", [TINY_A, TINY_B])
+def test_one_token_reduces_to_library_routines_and_tells_the_block_readings_apart(cfg):
+    """The block is sequential (the feed-forward reads the norm of the stream the attention has already been added
+    to: the composition the reference's own test states, tests/test_qwen_model.py:93-111) and the embedding enters
+    the stream unscaled.  A block whose feed-forward read the norm of the layer's input (both branches side by side),
+    or an embedding scaled by sqrt(hidden), gives other logits by far: the norms cancel a scale inside the branches,
+    but not in the sum with their output."""
+    w = random_qwen3_weights(cfg, seed=6, dtype=torch.float64)
+    eps = cfg["rms_norm_eps"]
+    for token in (0, 5, cfg["vocab_size"] - 1):
+        got = plain.qwen3_forward(w, cfg, [token])[0]
+        torch.testing.assert_close(got, _one_token_by_hand(w, cfg, token, eps), rtol=1e-9, atol=1e-9)
+        side_by_side = _one_token_by_hand(w, cfg, token, eps, parallel=True)
+        scaled = _one_token_by_hand(w, cfg, token, eps, embedding_scale=cfg["hidden_size"] ** 0.5)
+        assert (got - side_by_side).norm() > 0.05 * got.norm() and (got - scaled).norm() > 0.05 * got.norm()
+
+
+def test_q_and_k_norms_use_the_models_eps():
+    """mini_llm/model/qwen.py:33,44-47: the per-head norms of q and k take rms_norm_eps like the other norms.  With
+    eps 0.3 a reading that hard-codes 1e-6 there is far off.  Two tokens: heads normalised by the library's rms_norm,
+    rotated (pinned above), attended by the library's causal attention."""
+    cfg = dict(TINY_A, rms_norm_eps=0.3, num_hidden_layers=1)
+    w = random_qwen3_weights(cfg, seed=8, dtype=torch.float64)
+    nq, nkv, d = cfg["num_attention_heads"], cfg["num_key_value_heads"], cfg["head_dim"]
+    x = torch.randn(2, cfg["hidden_size"], dtype=torch.float64)
+    got, _ = plain.qwen3_attention(x, w, "model.layers.0.self_attn", cfg, torch.arange(2))
+
+    def by_hand(eps):
+        p = "model.layers.0.self_attn"
+        q = F.rms_norm((x @ w[f"{p}.q_proj.weight"].T).view(2, nq, d), (d,), w[f"{p}.q_norm.weight"], eps)
+        k = F.rms_norm((x @ w[f"{p}.k_proj.weight"].T).view(2, nkv, d), (d,), w[f"{p}.k_norm.weight"], eps)
+        v = (x @ w[f"{p}.v_proj.weight"].T).view(2, nkv, d)
+        cos, sin = plain.rope_tables(torch.arange(2), d, cfg["rope_theta"], x.dtype)
+        q, k = plain.apply_rope(q.transpose(0, 1), cos, sin), plain.apply_rope(k.transpose(0, 1), cos, sin)
+        k, v = k.repeat_interleave(nq // nkv, 0), v.transpose(0, 1).repeat_interleave(nq // nkv, 0)
+        out = F.scaled_dot_product_attention(q[None], k[None], v[None], is_causal=True)[0]
+        return out.transpose(0, 1).reshape(2, nq * d) @ w[f"{p}.o_proj.weight"].T
+
+    torch.testing.assert_close(got, by_hand(0.3), rtol=1e-9, atol=1e-9)
+    assert (got[1] - by_hand(1e-6)[1]).norm() > 0.02 * got[1].norm()
+
+
 def test_tied_head_uses_embedding():
     w = random_qwen3_weights(TINY_A, seed=1, dtype=torch.float64)
     assert "lm_head.weight" not in w

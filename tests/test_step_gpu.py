@@ -315,19 +315,22 @@ def test_single_tokens_at_the_head_of_a_mixed_step_and_elsewhere_in_it(folder_b,
 
 
 # ------------------------------- one layer at the benchmark's sizes, against plain
-def test_one_layer_at_the_benchmark_sizes_against_the_plain_implementation():
+@pytest.mark.parametrize("sizes", ["8b", "14b", "32b"])
+def test_one_layer_at_the_benchmark_sizes_against_the_plain_implementation(sizes):
     """Hidden 4096, 32 query and 8 kv heads of 128 dims, feed-forward 12288, vocabulary 151936, float32,
     100 tokens in portions of 60, 39 and 1: the engine against the plain implementation itself, not against
     another precision of the engine.  The plain side computes the logits of three slices of the vocabulary
-    (its first, a middle and its last rows) to keep the float64 work small."""
+    (its first, a middle and its last rows) to keep the float64 work small.  Likewise at the layer sizes of the
+    two larger models of the family (hidden 5120 with kv groups of five and of eight query heads), on which the
+    comparison of the bfloat16 path with the float32 path at those sizes stands."""
     from llm_runtime_study_amd.cache import CacheManager
     from llm_runtime_study_amd.config import config_from_dict, spec_for
     from llm_runtime_study_amd.engine.step import ModelRunner, StepEntry
     from llm_runtime_study_amd.models import DecoderModel
     from llm_runtime_study_amd.weights import random_init
-    from tests.test_shape_gpu import SHAPE
+    from tests.test_shape_gpu import LARGER, SHAPE
 
-    raw = dict(SHAPE, num_hidden_layers=1)
+    raw = dict(SHAPE, num_hidden_layers=1, **LARGER[sizes])
     cfg = config_from_dict(raw)
     device = torch.device("cuda", 0)
     model = DecoderModel(spec_for(cfg))
@@ -412,6 +415,71 @@ def test_steps_made_again_from_a_recorded_plan_equal_steps_through_the_parts(fol
         assert torch.equal(a.k_pages, b.k_pages) and torch.equal(a.v_pages, b.v_pages)
     # a model with a part that is not known to be safe to record runs through its parts every time
     runners[0].cache.check_invariants()
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_the_graph_of_a_plan_equals_the_parts_and_the_plain_implementation(folder_b, dtype):
+    """The path steady serving runs on: a step shape that keeps coming back on a stream of its own is recorded,
+    replayed from the plan and then launched as the graph of that plan.  One mixed shape (two requests bringing a
+    single token, a third a portion of 20) comes eleven times, with other tokens, requests changing roles, contexts
+    growing, and pages that a finished request gave back and a new one took.  Every logits row equals, bit for bit,
+    that of a runner without plans through the same steps, and agrees with the plain implementation of the whole
+    sequences."""
+    from llm_runtime_study_amd.engine.step import StepEntry
+
+    cfg, weights = plain.load_model_dir(folder_b, torch.float64)
+    rng = np.random.default_rng(17)
+    vocab = TINY_B["vocab_size"]
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        runners = [make_runner(folder_b, dtype, pages=40, requests=3, seq=256, step_tokens=32) for _ in range(2)]
+        runners[1].use_plans = False
+        assert runners[0].use_plans
+        caches = [[r.cache.admit(i) for i in range(3)] for r in runners]
+        history = {0: [], 1: [], 2: []}            # request -> its tokens so far
+        names = [0, 1, 2]                          # which request sits in each of the three places
+        finished, got = {}, {}
+        rounds = runners[0].PLAN_GRAPH_AFTER + 8
+        for turn in range(rounds):
+            if turn == 6:
+                # the request in place 0 ends; a new one takes its slot and, lowest ids first, other pages than it had
+                finished[names[0]] = history.pop(names[0])
+                for runner, mine in zip(runners, caches):
+                    runner.cache.release(mine[0])
+                    mine[0] = runner.cache.admit(3)
+                names[0], history[3] = 3, []
+            singles, portion = [(turn + 0) % 3, (turn + 1) % 3], (turn + 2) % 3
+            plan = [(place, rng.integers(0, vocab, 1).tolist(), [0]) for place in singles]
+            plan.append((portion, rng.integers(0, vocab, 20).tolist(), [3, 19]))
+            outs = []
+            for runner, mine in zip(runners, caches):
+                outs.append(runner.step([StepEntry(mine[place], tokens, want) for place, tokens, want in plan]).clone())
+            assert torch.equal(outs[0], outs[1]), f"turn {turn}"
+            row = 0
+            for place, tokens, want in plan:
+                at = len(history[names[place]])
+                for w in want:
+                    got[(names[place], at + w)] = outs[0][row].cpu()
+                    row += 1
+                history[names[place]] += tokens
+        side.synchronize()
+        known = [k for k in runners[0]._plans.values() if k.graph is not None]
+        assert len(known) == 1 and runners[0].plan_recordings <= 3
+        assert runners[0].plan_graph_replays >= rounds - 3 - runners[0].PLAN_GRAPH_AFTER
+        assert runners[1].plan_replays == 0
+        for a, b in zip(runners[0].cache.layer_caches, runners[1].cache.layer_caches):
+            assert torch.equal(a.k_pages, b.k_pages) and torch.equal(a.v_pages, b.v_pages)
+    finished.update(history)
+    want = {name: plain.qwen3_forward(weights, cfg, ids) for name, ids in finished.items()}
+    assert len(got) == rounds * 4
+    for (name, position), row in got.items():
+        ref = want[name][position]
+        if dtype == torch.float32:
+            torch.testing.assert_close(row.double(), ref, rtol=1e-4, atol=1e-4, msg=lambda m: f"request {name} position {position}: {m}")
+        else:
+            err = (row.double() - ref).norm() / ref.norm()
+            assert err < 3e-2, f"request {name} position {position}: relative error {err:.3g}"
+            assert int(row.argmax()) == int(ref.argmax()) or ref.topk(2).values.diff().abs() < 0.25
 
 
 def test_a_model_with_parts_of_unknown_habits_is_never_recorded():
