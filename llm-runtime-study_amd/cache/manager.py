@@ -2,7 +2,8 @@
 fixed-size per-request state.
 
 What each schedule entry of the model keeps between steps is declared by its mixer:
-  PagedKVNeed(nkv, d, window)  keys and values of every position, or of a sliding window;
+  PagedKVNeed(nkv, d, window, dtype)  keys and values of every position, or of a sliding window, kept in `dtype`
+                               (None: the run's activation dtype);
   StateNeed(shape, dtype)      a state of fixed size;
   ("from", j)                  nothing of its own: it reads the cache of entry j;
   None                         nothing.
@@ -69,6 +70,7 @@ class RequestCache:
 class PagedGroup:
     def __init__(self, need: PagedKVNeed, entries: list[int], num_pages: int):
         self.need, self.entries = need, entries
+        self.dtype: torch.dtype | None = None       # what its pages hold: the need's own dtype, else the manager's
         self.pool = PagePool(num_pages)
         self.reserved_pages = 0
         self.k: dict[int, torch.Tensor] = {}
@@ -102,6 +104,7 @@ class CacheManager:
             if isinstance(need, PagedKVNeed):
                 if need not in by_need:
                     by_need[need] = PagedGroup(need, [], num_pages)
+                    by_need[need].dtype = need.dtype if need.dtype is not None else dtype
                     self.groups.append(by_need[need])
                 group = by_need[need]
                 group.entries.append(position)
@@ -121,8 +124,7 @@ class CacheManager:
 
         if allocate_storage and self.device.type == "cuda" and self.groups:
             # a pool the device cannot hold is refused before anything is allocated, with the numbers that decide it
-            element = torch.empty(0, dtype=dtype).element_size()
-            per_page = sum(2 * len(g.entries) * g.need.num_kv_heads * g.need.head_dim * page_size * element for g in self.groups)
+            per_page = page_size * self.bytes_per_token()
             free, _ = torch.cuda.mem_get_info(self.device)
             if (num_pages + 1) * per_page > free:
                 fits = max(free // per_page - 1, 0)
@@ -134,8 +136,8 @@ class CacheManager:
                 k_shape = (num_pages + 1, group.need.num_kv_heads, page_size, group.need.head_dim)
                 v_shape = (num_pages + 1, group.need.num_kv_heads, group.need.head_dim, page_size)
                 for position in group.entries:
-                    group.k[position] = torch.zeros(k_shape, dtype=dtype, device=self.device)
-                    group.v[position] = torch.zeros(v_shape, dtype=dtype, device=self.device)
+                    group.k[position] = torch.zeros(k_shape, dtype=group.dtype, device=self.device)
+                    group.v[position] = torch.zeros(v_shape, dtype=group.dtype, device=self.device)
                     self.layer_caches[position].k_pages = group.k[position]
                     self.layer_caches[position].v_pages = group.v[position]
 
@@ -164,8 +166,8 @@ class CacheManager:
         return max((g.pool.used_pages for g in self.groups), default=0) * self.page_size
 
     def bytes_per_token(self) -> int:
-        size = torch.empty(0, dtype=self.dtype).element_size()
-        return sum(2 * len(g.entries) * g.need.num_kv_heads * g.need.head_dim * size for g in self.groups)
+        return sum(2 * len(g.entries) * g.need.num_kv_heads * g.need.head_dim * torch.empty(0, dtype=g.dtype).element_size()
+                   for g in self.groups)
 
     def trash_page(self, group: int = 0) -> int:
         """Page that no request owns; padding rows of a padded batch write there."""

@@ -32,9 +32,15 @@ class ModelConfig(Protocol):
 
     def validate_context_length(self, max_seq_len: int) -> None: ...
 
+    def to_json_dict(self) -> dict: ...  # the config.json content that reads back as this configuration (random-weights folders)
+
 
 CONFIG_ATTRIBUTES = ("model_type", "vocab_size", "eos_token_ids")
-CONFIG_METHODS = ("from_dict", "validate_context_length")
+CONFIG_METHODS = ("from_dict", "validate_context_length", "to_json_dict")
+# Modules named here (comma-separated import paths) are imported when the registry is first used: each registers its
+# parts and architectures as it is imported, so that a program started as a process of its own (the command line,
+# bin/trace_run) knows an architecture that lives outside this package.
+PLUGINS_VARIABLE = "LLM_RUNTIME_STUDY_PLUGINS"
 
 
 def _config_fields(config_class: type) -> set:
@@ -70,6 +76,14 @@ def _load_builtin() -> None:
 
     if Qwen3Config.ARCHITECTURE not in _ARCHITECTURES:
         register_architecture(Qwen3Config.ARCHITECTURE, Qwen3Config, build_spec, chat_template=format_qwen3_chat)
+    import importlib
+    import os
+
+    for name in filter(None, (piece.strip() for piece in os.environ.get(PLUGINS_VARIABLE, "").split(","))):
+        try:
+            importlib.import_module(name)
+        except ImportError as exc:
+            raise ConfigError(f"{PLUGINS_VARIABLE} names the module {name!r}, which cannot be imported: {exc}") from exc
 
 
 def register_architecture(name: str, config_class: type, build_spec: Callable, chat_template: Callable | None = None) -> None:

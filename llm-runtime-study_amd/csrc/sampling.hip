@@ -259,6 +259,9 @@ LRS_API int lrs_choose_tokens(int* out, const float* logits, int64_t row_stride,
 // others to -inf, in place.  One workgroup per row.  Rule (the reference's): after scaling
 // by 1/temperature keep the k largest; then, in descending order, drop a token once the
 // probability mass strictly before it reaches top_p, so the token that crosses stays.
+// Values equal to a threshold are all kept: where the reference's topk and sort keep one of several equal
+// values and drop another, whichever their order of the equal ones says, both stay here (a kept set that does
+// not depend on an order of arrival).
 // Both thresholds are values of the row itself and are found without a sort, by selection over the
 // ordered bit patterns of float32, 11 + 11 + 10 bits at a time: a pass over the row counts (top-k) or
 // weighs (top-p) the values by the next digit of their pattern in LDS, the digit whose bin holds the
@@ -323,9 +326,9 @@ __global__ __launch_bounds__(1024) void filter_logits_kernel(float* __restrict__
 
   // A pass over the row: body(index, logit) for each of this thread's values.  Four loads of 16 bytes are asked
   // for before any is used (a thread's loads one after the other, each waited for, were what a pass took its
-  // time for); rows that do not begin on 16 bytes go one value at a time.  Dividing by the temperature (positive)
-  // changes no order, so the patterns compared are those of the logits themselves, and only the masses are taken
-  // of the scaled values: exp((logit - largest logit) / temperature).
+  // time for); rows that do not begin on 16 bytes go one value at a time.  The patterns compared are those of the
+  // scaled values logit / temperature, as the reference compares them: two logits whose quotients round to one
+  // float32 are a tie there and are kept or dropped together.  The masses are exp((logit - largest logit) / temperature).
   const bool in_fours = ((uintptr_t)z % 16) == 0;
   auto walk = [&](auto&& body) {
     const int fours = in_fours ? vocab / 4 : 0;
@@ -379,7 +382,7 @@ __global__ __launch_bounds__(1024) void filter_logits_kernel(float* __restrict__
       uint32_t run_bin = 0xFFFFFFFFu;                          // values that follow each other into one bin are added up first
       unsigned long long run = 0;
       walk([&](int, float v) {
-        const uint32_t key = ordered_key(v);
+        const uint32_t key = ordered_key(v / temp);
         if (MASS && key < floor) return;
         if (level == 1 && (key >> 21) != prefix) return;
         if (level == 2 && (key >> 10) != prefix) return;
@@ -418,7 +421,7 @@ __global__ __launch_bounds__(1024) void filter_logits_kernel(float* __restrict__
   if (use_k) threshold = select(std::false_type{}, (double)k, 0u, 0.f);
   if (use_p) threshold = select(std::true_type{}, 0.0, threshold, p);
   walk([&](int i, float v) {
-    if (ordered_key(v) < threshold) z[i] = -INFINITY;
+    if (ordered_key(v / temp) < threshold) z[i] = -INFINITY;
   });
 }
 

@@ -8,6 +8,7 @@ from ..config import load_config, spec_for
 from ..errors import EngineError
 from ..models import DecoderModel
 from ..weights import Checkpoint, device_weights, load
+from ..weights.random_init import TORCH_DTYPES
 
 DTYPES = {"bfloat16": torch.bfloat16, "float32": torch.float32}
 
@@ -65,6 +66,8 @@ def random_model(config, seed: int, dtype: torch.dtype, device, init: str = "nor
     """Bound model with random weights made on the device (no files)."""
     spec = spec_for(config)
     model = DecoderModel(spec)
-    store = torch.bfloat16 if spec.checkpoint_dtype != "float32" else torch.float32
-    model.bind(device_weights(model, seed, store, device, init), dtype)
+    # drawn in the precision the architecture's checkpoints are stored in, and brought to the device as a loaded
+    # checkpoint is: float16, which no kernel takes, widened to float32
+    weights = device_weights(model, seed, TORCH_DTYPES[spec.checkpoint_dtype], device, init)
+    model.bind({name: t.float() if t.dtype == torch.float16 else t for name, t in weights.items()}, dtype)
     return model

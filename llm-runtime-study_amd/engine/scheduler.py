@@ -168,7 +168,7 @@ class BatchScheduler:
                 tokens = self.sampler.choose(logits, [row for _, row in rows]) if rows else []
                 seconds = self._now() - started if started is not None else None
                 self._finish_step(rows, tokens, seconds, events)
-        except Exception:
+        except BaseException:       # an interrupt from the keyboard frees everything as well
             self.abort_all()
             raise
         return events

@@ -138,26 +138,28 @@ class ModelRunner:
         # Which matrix-product kernels this runner's steps use: a property of the runner, carried by every step's
         # context, never of the process.  Unless `kernels` says otherwise: bfloat16 products of more rows than this
         # package's kernels for few rows take go to the vendor library, if `library_gemm` allows it.
-        self.kernels = kernels if kernels is not None else ops.KernelChoice(library=library_gemm)
+        self._graphs: dict[tuple, tuple] = {}   # (bucket, length class) -> (handle, arena generation, logits tensor)
+        self._plans: dict[tuple, RecordedStep] = {}
+        self._kernels = kernels if kernels is not None else ops.KernelChoice(library=library_gemm)
         self.library_gemm = self.kernels.library
         # decode-only steps are captured in a HIP graph per padded batch size and replayed
         self.use_graph = use_graph and model.graph_safe()
-        self._graphs: dict[tuple, tuple] = {}   # (bucket, length class) -> (handle, arena generation, logits tensor)
         # Steps that are not replayed from a graph (prompt portions, mixed steps) are recorded as launch plans:
         # the first step of a shape runs through the parts as usual while every launch is written down; later
         # steps of that shape fill in the metadata and make the same launches from one call into the library.
         # A shape is what the launches' arguments depend on (see _plan_key); a plan also names addresses, so it
         # is good only while the scratch buffers stay where they are (the arena's generation).  Only models
         # whose every part launches through this package's kernels alone (`plan_safe`) are recorded.
-        self.use_plans = use_plans and getattr(model, "plan_safe", lambda: False)()
-        self._plans: dict[tuple, RecordedStep] = {}
+        self._use_plans = use_plans and getattr(model, "plan_safe", lambda: False)()
         self.plan_replays = 0
         self.plan_recordings = 0
         self.plan_graph_replays = 0     # of the replays, those made by launching the graph of a plan
         self.graph_replays = 0     # steps (or launches of several steps) served by replaying a graph
         self.graph_captures = 0    # ... and those that ran eagerly and were captured on the way
-        # query groups for the ragged attention kernel: at most `query_group` consecutive tokens of one request
-        self.query_group = ops.attention_prefill_group()   # the most; a step of few tokens uses smaller ones
+        # query groups for mixers that ask for them (the ragged attention kernel): at most `query_group` consecutive
+        # tokens of one request
+        self._query_groups = getattr(model, "wants_query_groups", lambda: True)()
+        self.query_group = ops.attention_prefill_group() if self._query_groups else 0   # the most; a step of few tokens uses smaller ones
         # The metadata of a step is one int32 buffer whose layout follows the step's own numbers of
         # tokens and requests, so that a decode step uploads a few KB whatever the limits are.  A
         # graph holds addresses inside it: steps of one padded batch size share one layout.
@@ -190,13 +192,37 @@ class ModelRunner:
             self._built.record(stream)
             self._follows_construction = {stream.cuda_stream}
 
+    # A captured graph and a recorded plan hold the kernels that were chosen when they were made, and the addresses of
+    # the weights and pages of that time: whoever changes the choice gets them made again.
+    @property
+    def kernels(self) -> "ops.KernelChoice":
+        return self._kernels
+
+    @kernels.setter
+    def kernels(self, choice: "ops.KernelChoice") -> None:
+        if choice != self._kernels:
+            self.drop_graphs()
+        self._kernels = choice
+        self.library_gemm = choice.library
+
+    @property
+    def use_plans(self) -> bool:
+        return self._use_plans
+
+    @use_plans.setter
+    def use_plans(self, wanted: bool) -> None:
+        wanted = bool(wanted) and getattr(self.model, "plan_safe", lambda: False)()
+        if wanted != self._use_plans:
+            self.drop_graphs()
+        self._use_plans = wanted
+
     def _layout(self, tokens: int, requests: int) -> tuple[dict, int]:
         """Where each array of a step of `tokens` tokens and `requests` requests lies in the metadata
         buffer: name -> (first element, elements), and the elements in all (16-byte aligned parts)."""
         known = self._layouts.get((tokens, requests))
         if known is None:
             offsets, cursor = {}, 0
-            qblocks = -(-tokens // 16) + requests
+            qblocks = -(-tokens // 16) + requests if self._query_groups else 0
             parts = [("token_ids", tokens), ("positions", tokens), ("token_request", tokens), ("logit_rows", tokens),
                      ("cu_seqlens_q", requests + 1), ("seq_lens_k", requests), ("slot_ids", requests),
                      ("qblock_token0", qblocks), ("qblock_count", qblocks), ("counts", 4)]
@@ -346,8 +372,10 @@ class ModelRunner:
             n_rows = cursor
         ctx.T, ctx.R, ctx.num_logit_rows = cursor, max(real, pad_to), n_rows
         self._host_view("counts")[0] = real          # rows that belong to requests (the others pad a graph's batch)
-        # groups of consecutive tokens of one request, the longest contexts first
-        if ctx.all_decode:
+        # groups of consecutive tokens of one request, the longest contexts first: only for mixers that ask for them
+        if not self._query_groups:
+            ctx.num_qblocks = ctx.max_qblock = 0
+        elif ctx.all_decode:
             ctx.num_qblocks, ctx.max_qblock = cursor, 1
             self._host_view("qblock_token0")[:cursor] = np.argsort(-pos[:cursor], kind="stable")
             self._host_view("qblock_count")[:cursor] = 1
@@ -416,7 +444,7 @@ class ModelRunner:
                 logits = self._step_graph(entries, bucket)
             else:
                 logits = self._step_eager(self.prepare(entries))
-        except Exception:
+        except BaseException:       # an interrupt from the keyboard in the middle of a step must leave no trace either
             ops.record_drop()
             self._undo(extended, before, states)
             raise
@@ -450,7 +478,7 @@ class ModelRunner:
                 ops.graph_begin()
                 try:
                     ops.plan_run(known.plan)
-                except Exception:
+                except BaseException:
                     ops.graph_destroy(ops.graph_end())
                     raise
                 known.graph = ops.graph_end()
@@ -468,7 +496,7 @@ class ModelRunner:
         try:
             h = self.model.forward_hidden(ctx)
             logits = self.model.logits(ctx, h) if ctx.num_logit_rows else None
-        except Exception:
+        except BaseException:
             ops.record_drop()
             raise
         plan = ops.record_end()
@@ -545,7 +573,7 @@ class ModelRunner:
                     if sampling is not None:
                         rows = [type(row)(row.config, row.seed, row.counter + len(chosen)) for row in sampling]
                 chosen += self._decode_launch(current, count, rows, bucket)
-        except Exception:
+        except BaseException:
             self._undo(entries, before, states)
             raise
         for entry in entries:

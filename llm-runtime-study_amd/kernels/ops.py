@@ -9,6 +9,7 @@ the library is missing or cannot be built; there is no fallback.
 from __future__ import annotations
 
 import functools
+import threading
 
 from dataclasses import dataclass
 import ctypes
@@ -166,7 +167,15 @@ PLAN_OPS = ("lrs_add_into", "lrs_add_rmsnorm", "lrs_advance_decode", "lrs_advanc
             "lrs_filter_logits", "lrs_gather_rows", "lrs_gemm", "lrs_gemm_mid_add_norm_begin", "lrs_gemm_mid_qk_prep", "lrs_gemm_mid_scaled",
             "lrs_gemm_norm_chain", "lrs_library_gemm", "lrs_qk_prep", "lrs_rmsnorm", "lrs_rope_table", "lrs_scale_rows", "lrs_silu_mul")
 _PLAN_INDEX = {name: index for index, name in enumerate(PLAN_OPS)}
-_recording: list | None = None
+
+
+class _Recording(threading.local):
+    """The recording that is open on this thread, if any: launches made on another thread (a second runner, a
+    sampler) are none of its business."""
+    calls: list | None = None
+
+
+_recording = _Recording()
 
 
 class Plan:
@@ -190,26 +199,23 @@ class Plan:
 
 
 def record_begin() -> None:
-    """Start writing launches down (they still run as they are made)."""
-    global _recording
-    if _recording is not None:
+    """Start writing down the launches this thread makes (they still run as they are made)."""
+    if _recording.calls is not None:
         raise KernelError("a recording of launches is already open")
-    _recording = []
+    _recording.calls = []
 
 
 def record_end() -> Plan:
     """Stop writing launches down; returns the plan of those made since record_begin()."""
-    global _recording
-    if _recording is None:
+    if _recording.calls is None:
         raise KernelError("no recording of launches is open")
-    calls, _recording = _recording, None
+    calls, _recording.calls = _recording.calls, None
     return Plan(calls)
 
 
 def record_drop() -> None:
     """Stop writing launches down and forget them (after a failure)."""
-    global _recording
-    _recording = None
+    _recording.calls = None
 
 
 def plan_run(plan: Plan) -> None:
@@ -222,10 +228,10 @@ def _launch(name: str, *args) -> None:
     code = getattr(_lib or library(), name)(*args)
     if code != 0:
         raise KernelError(library().lrs_last_error().decode())
-    if _recording is not None:
+    if _recording.calls is not None:
         if name not in _PLAN_INDEX:
             raise KernelError(f"{name} cannot be part of a recorded plan")
-        _recording.append((name, args[:-1]))
+        _recording.calls.append((name, args[:-1]))
 
 
 def loaded_library_path() -> str:

@@ -12,6 +12,7 @@ import torch
 
 from ..kernels import ops
 from ..parts import TensorSpec, create
+from ..parts.base import flops_of
 from ..parts.linear import linear
 from .spec import ModelSpec
 
@@ -22,6 +23,9 @@ class DecoderModel:
         self.spec = spec
         self.layers = [create("block", block) for block in spec.layers]
         self.final_norm = create("norm", spec.final_norm)
+        # optional parts around the stack: (part, prefix of its tensors' names)
+        self.after_embedding = None if spec.after_embedding is None else create("transform", spec.after_embedding)
+        self.after_head = None if spec.after_head is None else create("transform", spec.after_head)
         self.embedding = self.head = None
         self.dtype = None
 
@@ -34,6 +38,8 @@ class DecoderModel:
             prefix = spec.layer_prefix.format(index=index)
             out.update({f"{prefix}.{name}": t for name, t in layer.tensors().items()})
         out.update({f"{spec.final_norm_prefix}.{name}": t for name, t in self.final_norm.tensors().items()})
+        for part, prefix in self._around():
+            out.update({f"{prefix}.{name}": t for name, t in part.tensors().items()})
         out[spec.head_name] = TensorSpec((spec.vocab_size, spec.hidden_size), role="matrix", optional=spec.tie_head)
         return out
 
@@ -47,8 +53,17 @@ class DecoderModel:
         for index, layer in enumerate(self.layers):
             prefix = spec.layer_prefix.format(index=index) + "."
             layer.bind({n[len(prefix):]: t for n, t in weights.items() if n.startswith(prefix)}, dtype)
-        prefix = spec.final_norm_prefix + "."
-        self.final_norm.bind({n[len(prefix):]: t for n, t in weights.items() if n.startswith(prefix)}, dtype)
+        for part, prefix in [(self.final_norm, spec.final_norm_prefix)] + self._around():
+            prefix += "."
+            part.bind({n[len(prefix):]: t for n, t in weights.items() if n.startswith(prefix)}, dtype)
+
+    def _around(self) -> list:
+        """The optional parts after the embedding and after the head, each with the prefix of its tensors."""
+        return [(part, prefix) for part, prefix in ((self.after_embedding, self.spec.after_embedding_prefix),
+                                                    (self.after_head, self.spec.after_head_prefix)) if part is not None]
+
+    def _parts(self) -> list:
+        return self.layers + [self.final_norm] + [part for part, _ in self._around()]
 
     def cache_needs(self) -> list:
         """What each schedule entry keeps between steps: a need, ("from", entry) or None."""
@@ -63,16 +78,21 @@ class DecoderModel:
     def graph_safe(self) -> bool:
         """Whether a step launches only this library's kernels on preallocated buffers, so that it
         can be captured in a HIP graph: every part must say so itself."""
-        return all(getattr(layer, "graph_safe", False) for layer in self.layers)
+        return all(getattr(part, "graph_safe", False) for part in self._parts())
+
+    def wants_query_groups(self) -> bool:
+        """Whether any mixer reads the step's query groups (see parts/base.py); the step function builds them only then."""
+        return any(getattr(layer, "wants_query_groups", False) for layer in self.layers)
 
     def plan_safe(self) -> bool:
         """Whether a step's launches can be written down once and made again from the record: every part must
         launch through this package's kernels alone, with arguments that follow from the step's shape."""
-        return all(getattr(layer, "plan_safe", False) for layer in self.layers) and getattr(self.final_norm, "plan_safe", False)
+        return all(getattr(part, "plan_safe", False) for part in self._parts())
 
     def weight_bytes(self, with_embedding: bool = False) -> int:
         """Bytes of weights one decode step reads: every scheduled layer once, and the head."""
         total = sum(self.layers[e.layer].weight_bytes() for e in self.spec.schedule)
+        total += sum(part.weight_bytes() for part, _ in self._around())
         total += self.head.numel() * self.head.element_size()
         if with_embedding and self.head is not self.embedding:
             total += self.embedding.numel() * self.embedding.element_size()
@@ -81,7 +101,8 @@ class DecoderModel:
     def flops(self, tokens: int, pairs: int, logit_rows: int = 1) -> float:
         """Floating-point operations of the matrix products of one step of `tokens` tokens: every scheduled layer
         (what each part says of itself, see Part.flops for `pairs`) and the head for `logit_rows` rows."""
-        total = sum(self.layers[e.layer].flops(tokens, pairs) for e in self.spec.schedule)
+        total = sum(flops_of(self.layers[e.layer], tokens, pairs) for e in self.spec.schedule)
+        total += sum(flops_of(part, tokens, pairs) for part, _ in self._around())
         return total + 2.0 * logit_rows * self.spec.vocab_size * self.spec.hidden_size
 
     # ------------------------------------------------------------------ forward
@@ -89,6 +110,8 @@ class DecoderModel:
         """Residual stream [T, H] float32 after the last layer (before the final norm)."""
         h = ctx.scratch("residual", (ctx.T, self.spec.hidden_size), torch.float32)
         ops.embed(h, self.embedding, ctx.token_ids, self.spec.embedding_multiplier)
+        if self.after_embedding is not None:
+            self.after_embedding.forward(ctx, h)
         schedule = self.spec.schedule
         begun = None   # the next layer's first norm, if the product that last updated h began it
         for position, entry in enumerate(schedule):
@@ -111,4 +134,6 @@ class DecoderModel:
             x = self.final_norm.forward(ctx, h, rows=ctx.logit_rows, count=n)
         out = ctx.scratch("logits", (n, self.spec.vocab_size), torch.float32)
         linear(ctx, out, x, self.head)
+        if self.after_head is not None:
+            self.after_head.forward(ctx, out)
         return out

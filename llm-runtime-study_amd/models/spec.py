@@ -7,6 +7,11 @@ An architecture turns its typed configuration into a ModelSpec; everything after
   schedule  the order in which layers run: ScheduleEntry(layer, cache_from).  A layer may be
             named twice (same weights, a cache of its own for each run), and an entry may
             read the cache that an earlier entry writes (`cache_from` = index into schedule).
+  after_embedding, after_head
+            optional parts of the role "transform" that work in place on the float32 residual
+            stream right after the embedding (a learned or absolute position signal, a scale)
+            and on the float32 logits (a scale, a soft cap); their tensors are named
+            `<after_embedding_prefix>.<name>` and `<after_head_prefix>.<name>`.
 """
 
 from __future__ import annotations
@@ -40,6 +45,10 @@ class ModelSpec:
     final_norm_prefix: str = "model.norm"
     layer_prefix: str = "model.layers.{index}"
     checkpoint_dtype: str = "bfloat16"
+    after_embedding: PartSpec | None = None
+    after_head: PartSpec | None = None
+    after_embedding_prefix: str = "model.after_embedding"
+    after_head_prefix: str = "after_head"
     extra: dict = field(default_factory=dict, compare=False)
 
     def validate(self) -> None:

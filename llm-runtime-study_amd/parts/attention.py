@@ -28,6 +28,7 @@ class GQAAttention(Part):
     plan_safe = True   # ... and nothing but this package's kernels, with arguments that follow the step's shape alone
     takes_lazy_norm = True
     begins_next_norm = True
+    wants_query_groups = True   # ragged steps go to a kernel that walks groups of a request's consecutive tokens
 
     def __init__(self, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int, *,
                  position: PartSpec = PartSpec("none"), qk_norm: bool = False, qk_norm_eps: float = 1e-6,

@@ -14,6 +14,11 @@ Roles and what each must provide:
                  forward(ctx, x, residual, cache)       adds its output into residual (float32)
   feed_forward   forward(ctx, x, residual)              adds its output into residual (float32)
   block          forward(ctx, h, cache)                 one layer: norms, mixer, feed-forward
+  transform      forward(ctx, x)                        works in place on float32 rows: the residual stream [T, H] right
+                                                        after the embedding (ModelSpec.after_embedding: a position signal
+                                                        added there, a scale), or the logits [wanted, V] (ModelSpec.after_head:
+                                                        a scale, a soft cap).  ctx.positions / ctx.logit_rows say which
+                                                        tokens the rows belong to
 
 Optional, each announced by a class attribute (a part without it is simply given plain tensors):
 
@@ -26,6 +31,16 @@ Optional, each announced by a class attribute (a part without it is simply given
   chains_norms = True         block: forward(ctx, h, cache, normed=None, then_norm=None) takes the
                               normalised input a previous block began and may return the next one;
                               `first_norm` is the norm it applies to its input
+
+  wants_query_groups = True   mixer (a block passes it on): the step function cuts the tokens of a ragged step into
+                              query groups for it: ctx.qblock_token0 / ctx.qblock_count [ctx.num_qblocks] list groups of
+                              at most ctx.max_qblock consecutive tokens of one request, longest context first, which
+                              together cover every token once.  In a step that is not decode-only the requests at its
+                              head that bring one token each (ctx.single_rows of them; their tokens are the step's
+                              first rows) are left out of the groups, which count their tokens from the first row
+                              after them: a mixer that uses the groups serves those single rows itself (attention
+                              gives them to its kernel for decode steps).  Without the attribute nothing is built and
+                              ctx.num_qblocks is 0: a model of other mixers does not pay for it
 
 A part may also say how its steps can be run again without it (both default to no):
 
@@ -47,7 +62,7 @@ from typing import Any, Mapping
 
 import torch
 
-ROLES = ("norm", "position", "mixer", "feed_forward", "block")
+ROLES = ("norm", "position", "mixer", "feed_forward", "block", "transform")
 _REGISTRY: dict[str, dict[str, type]] = {role: {} for role in ROLES}
 
 
@@ -94,11 +109,13 @@ class TensorSpec:
 
 @dataclass(frozen=True)
 class PagedKVNeed:
-    """A mixer that keeps keys and values of every position (or of a window) in pages."""
+    """A mixer that keeps keys and values of every position (or of a window) in pages; `dtype`: what the pages
+    hold, if not the run's activation dtype."""
 
     num_kv_heads: int
     head_dim: int
     window: int | None = None
+    dtype: torch.dtype | None = None
 
 
 @dataclass(frozen=True)
@@ -129,6 +146,13 @@ class Part:
         sum of the context lengths for decoding requests.  Only mixers that look back use it.  Unless a part says
         otherwise: every matrix it declares in tensors() is multiplied with every token once."""
         return 2.0 * tokens * sum(math.prod(spec.shape) for spec in self.tensors().values() if spec.role == "matrix")
+
+
+def flops_of(part, tokens: int, pairs: int) -> float:
+    """part.flops(tokens, pairs), also for a part that does not derive from Part and says nothing of its own
+    (then: its declared matrices, each multiplied with every token once)."""
+    own = getattr(part, "flops", None)
+    return own(tokens, pairs) if own is not None else Part.flops(part, tokens, pairs)
 
 
 def length_class(length: int) -> int:

@@ -7,7 +7,7 @@ The two sums happen inside the parts, which add into the float32 residual stream
 
 from __future__ import annotations
 
-from .base import Part, PartSpec, create, register
+from .base import Part, PartSpec, create, flops_of, register
 from .linear import materialize
 
 
@@ -36,7 +36,7 @@ class PreNormBlock(Part):
         return sum(part.weight_bytes() for _, part in self._children())
 
     def flops(self, tokens, pairs):
-        return sum(part.flops(tokens, pairs) for _, part in self._children())
+        return sum(flops_of(part, tokens, pairs) for _, part in self._children())
 
     def cache_need(self):
         return self.mixer.cache_need()
@@ -48,6 +48,10 @@ class PreNormBlock(Part):
     @property
     def plan_safe(self) -> bool:
         return all(getattr(part, "plan_safe", False) for _, part in self._children())
+
+    @property
+    def wants_query_groups(self) -> bool:
+        return getattr(self.mixer, "wants_query_groups", False)
 
     chains_norms = True
 

@@ -218,3 +218,62 @@ def test_the_tile_width_of_the_many_rows_kernel_follows_the_rounds_of_the_chip()
     assert ops.gemm_split_pays(256, 5120, 5120) and not ops.gemm_split_pays(512, 5120, 5120)
     assert not ops.gemm_split_pays(256, 4096, 4096)            # 8 parts of 8 slices: too short
     assert not ops.gemm_split_pays(2048, 4096, 12288) and not ops.gemm_split_pays(512, 34816, 5120)
+
+
+def test_a_recording_of_launches_belongs_to_its_thread():
+    """Two runners stepping on two threads each write their own launches down: a recording that is open on one
+    thread is not seen, and cannot be closed, from another."""
+    import threading
+
+    import pytest
+
+    from llm_runtime_study_amd.errors import KernelError
+    from llm_runtime_study_amd.kernels import ops
+
+    ops.record_begin()
+    try:
+        with pytest.raises(KernelError, match="already open"):
+            ops.record_begin()
+        seen = {}
+
+        def other():
+            try:
+                ops.record_end()
+            except KernelError as exc:
+                seen["end"] = str(exc)
+            ops.record_begin()                       # its own, beside the first thread's
+            seen["plan"] = ops.record_end().launches
+
+        worker = threading.Thread(target=other)
+        worker.start()
+        worker.join()
+        assert "no recording" in seen["end"] and seen["plan"] == 0
+        assert ops.record_end().launches == 0        # still open here
+    finally:
+        ops.record_drop()
+
+
+def test_changing_a_runners_kernels_or_plans_forgets_what_was_recorded():
+    """A recorded plan holds the kernels that were chosen when it was made: changing the choice, or switching plans
+    off and on, on a live runner empties what it had recorded."""
+    import torch
+
+    from llm_runtime_study_amd.cache import CacheManager
+    from llm_runtime_study_amd.config import config_from_dict, spec_for
+    from llm_runtime_study_amd.engine.step import ModelRunner, RecordedStep
+    from llm_runtime_study_amd.kernels import ops
+    from llm_runtime_study_amd.models import DecoderModel
+    from tests.helpers import TINY_A
+
+    model = DecoderModel(spec_for(config_from_dict(TINY_A)))
+    cache = CacheManager(model.cache_needs(), page_size=16, num_pages=4, max_requests=2, max_seq_len=64, device="cpu", allocate_storage=False)
+    runner = ModelRunner(model, cache, max_step_tokens=16, dtype=torch.float32, device="cpu")
+    assert runner.use_plans and runner.kernels.library
+    runner._plans[("shape",)] = RecordedStep(ops.Plan([]), 0, None)
+    runner.kernels = runner.kernels                  # the same choice: nothing to forget
+    assert len(runner._plans) == 1
+    runner.kernels = ops.KernelChoice(library=False)
+    assert not runner._plans and not runner.library_gemm
+    runner._plans[("shape",)] = RecordedStep(ops.Plan([]), 0, None)
+    runner.use_plans = False
+    assert not runner._plans and not runner.use_plans

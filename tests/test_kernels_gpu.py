@@ -1063,6 +1063,38 @@ def test_filter_logits_matches_sort_based_rule(ops):
     assert torch.isfinite(got[1]).sum() == 2
 
 
+def test_filter_logits_compares_the_scaled_values(ops):
+    """The thresholds are values of logits / temperature (mini_llm/sampling.py:53-64), not of the logits: two logits
+    one step of float32 apart whose quotients round to one float32 are a tie.  At the k-th place the reference's
+    topk keeps one of the two, whichever; here both stay, and nothing else differs."""
+    from tests.plain.model import filter_logits as plain_filter
+
+    temp, k, vocab = 0.7, 6, 400
+    low = torch.tensor(1.5)
+    while True:                                       # neighbours whose quotients by the temperature are one float32
+        high = torch.nextafter(low, torch.tensor(2.0))
+        if low / temp == high / temp:
+            break
+        low = high
+    assert low != high
+    g = torch.Generator().manual_seed(5)
+    logits = torch.randn(2, vocab, generator=g).clamp(max=1.2)
+    logits[:, 10:15] = torch.tensor([3.0, 2.9, 2.8, 2.7, 2.6])      # five above the pair
+    logits[:, 200], logits[:, 300] = high, low                      # the k-th and the one after it
+    work = dev(logits.clone())
+    temps = dev(torch.tensor([temp, temp]))
+    ops.filter_logits(work, temps, dev(torch.tensor([k, 0], dtype=torch.int32)), dev(torch.tensor([1.0, 0.999])))
+    kept = torch.isfinite(work.cpu())
+    assert kept[0].sum() == k + 1 and kept[0, 200] and kept[0, 300]
+    want = torch.isfinite(plain_filter(logits[0], temp, k, 1.0))
+    assert want.sum() == k and want[200] != want[300]
+    others = torch.ones(vocab, dtype=torch.bool)
+    others[[200, 300]] = False
+    assert torch.equal(kept[0][others], want[others])
+    # the mass rule likewise: the pair is kept or dropped together
+    assert kept[1, 200] == kept[1, 300]
+
+
 @pytest.mark.parametrize("vocab", [151936, 50257, 4099])
 def test_filter_logits_of_a_large_vocabulary_matches_the_sort_based_rule(ops, vocab):
     """The selection by digits of the bit pattern, where it has something to select from: a vocabulary of the

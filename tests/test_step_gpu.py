@@ -108,11 +108,13 @@ def test_every_refusal_of_the_step_function_leaves_the_cache_alone(folder_b):
 
 
 # ------------------------------------------------------- a forward that fails
+@pytest.mark.parametrize("failure", [Failing, KeyboardInterrupt], ids=["error", "interrupt"])
 @pytest.mark.parametrize("dtype", DTYPES)
-def test_a_failing_forward_leaves_no_trace_in_a_mixed_step(folder_b, dtype):
-    """Two running requests decode beside a new request's first portion; the second layer raises.
-    Lengths, page lists, pool counts and host block tables are as before, the new request holds
-    nothing, and the same step run again gives what a runner that never failed gives."""
+def test_a_failing_forward_leaves_no_trace_in_a_mixed_step(folder_b, dtype, failure):
+    """Two running requests decode beside a new request's first portion; the second layer raises (an error, or
+    an interrupt from the keyboard, which is no Exception).  Lengths, page lists, pool counts and host block
+    tables are as before, the new request holds nothing, the recording of launches that was open is closed, and
+    the same step run again (recorded anew) gives what a runner that never failed gives."""
     from llm_runtime_study_amd.engine.step import StepEntry
 
     rng = np.random.default_rng(3)
@@ -131,16 +133,19 @@ def test_a_failing_forward_leaves_no_trace_in_a_mixed_step(folder_b, dtype):
             original = layer.forward
 
             def broken(*args, **kwargs):
-                raise Failing("the second layer fails")
+                raise failure("the second layer fails")
 
             layer.forward = broken
-            with pytest.raises(Failing):
+            with pytest.raises(failure):
                 runner.step(entries)
             layer.forward = original
+            recorded = runner.plan_recordings
             assert same(snapshot(cache, [r0, r1, r2]), before)
             assert r2.length == 0 and r2.tables == [[]] and cache.used_pages() == 3
             cache.check_invariants()
         first = runner.step(entries).clone()
+        if fail:
+            assert runner.use_plans and runner.plan_recordings == recorded + 1     # no recording was left open
         second = runner.step([StepEntry(r0, [1], [0]), StepEntry(r1, [2], [0]), StepEntry(r2, [3], [0])]).clone()
         cache.check_invariants()
         return first, second

@@ -122,6 +122,9 @@ def test_the_chat_template_comes_from_the_architecture_registry(tokenizer):
         def validate_context_length(self, max_seq_len):
             pass
 
+        def to_json_dict(self):
+            return {"architectures": ["OtherForCausalLM"]}
+
     def shout(messages, *, enable_thinking=False):
         return "".join(f"[{m.role.upper()}] {m.content}\n" for m in messages)
 
@@ -145,11 +148,11 @@ def test_a_configuration_class_must_provide_what_the_engine_reads():
         def from_dict(cls, raw):
             return cls()
 
-    with pytest.raises(ConfigError, match="lacks: eos_token_ids, validate_context_length"):
+    with pytest.raises(ConfigError, match="lacks: eos_token_ids, validate_context_length, to_json_dict"):
         register_architecture("LackingForCausalLM", Lacking, lambda config: None)
     with pytest.raises(ConfigError, match="must be callable"):
         register_architecture("X", type("C", (), {"model_type": "", "vocab_size": 1, "eos_token_ids": (), "from_dict": classmethod(lambda c, r: c()),
-                                                  "validate_context_length": lambda s, n: None}), None)
+                                                  "validate_context_length": lambda s, n: None, "to_json_dict": lambda s: {}}), None)
 
 
 # ------------------------------------------ chat messages through the scheduler
