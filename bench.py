@@ -42,6 +42,7 @@ def parse_args():
     parser.add_argument("--context", type=int, default=2048)
     parser.add_argument("--prefill-tokens", type=int, default=2048)
     parser.add_argument("--max-seq-len", type=int, default=None, help="context the cache is made for: 4,096 (the benchmark context of the 8B configuration) or what the workload needs, whichever is more")
+    parser.add_argument("--num-pages", type=int, default=None, help="pages of the cache pool (default: max-seq-len tokens for every request of the largest batch)")
     parser.add_argument("--shape", choices=tuple(SHAPES), default="8b", help="layer sizes: Qwen3-8B (default), 14B or 32B")
     parser.add_argument("--layers", type=int, default=None, help="fewer layers than the shape has (reported in config)")
     parser.add_argument("--dtype", choices=("bfloat16", "float32"), default="bfloat16")
@@ -178,7 +179,7 @@ def main() -> int:
     from llm_runtime_study_amd.kernels.ops import KernelChoice
 
     engine = Engine.from_config(config, seed=0, dtype=args.dtype, max_seq_len=max_seq_len, max_batch_size=max_batch,
-                                max_num_batched_tokens=max(2048, args.prefill_tokens), use_cuda_graph=not args.no_graph,
+                                max_num_batched_tokens=max(2048, args.prefill_tokens), use_cuda_graph=not args.no_graph, num_pages=args.num_pages,
                                 kernels=KernelChoice(library=not args.own_gemm, mid=not args.library_mid_gemm),
                                 decode_steps_per_launch=args.decode_steps_per_launch)
     dtype_name = "bf16" if args.dtype == "bfloat16" else "fp32"

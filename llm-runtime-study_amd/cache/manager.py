@@ -16,6 +16,12 @@ and one block table per request.  Pages are taken when a request grows into them
 back when the request ends, is rolled back, or (windowed groups) when every position in
 the page has left the window of all future queries.
 
+The block tables live on the device for good: one int32 array [groups, max_requests + 1, max_blocks] (row = the
+request's slot; the last row, the trash row, points at the trash page), a copy of the host's.  Whatever changes an
+entry on the host (extend, rollback, trim, release) writes the range down; the step function takes the ranges with
+table_patches() and sends the changed entries along with its step's metadata, a few integers a step however long the
+contexts may grow.  Kernels read the device array at a fixed address, with the slot of a token's request as the row.
+
 Every admitted request also holds one state slot out of `max_requests`; StateNeed entries
 keep a tensor [max_requests + 1, *shape], zeroed for the slot at admission.  The slot is also
 the request's row in the per-group host block tables.  The extra last row is the trash slot:
@@ -75,7 +81,7 @@ class PagedGroup:
         self.reserved_pages = 0
         self.k: dict[int, torch.Tensor] = {}
         self.v: dict[int, torch.Tensor] = {}
-        self.host_table: np.ndarray | None = None   # [max_requests, max_blocks] int32
+        self.host_table: np.ndarray | None = None   # [max_requests, max_blocks] int32, a view of the manager's array of all groups
 
 
 class CacheManager:
@@ -130,8 +136,17 @@ class CacheManager:
                 fits = max(free // per_page - 1, 0)
                 raise KVCacheError(f"a cache pool of {num_pages} pages of {page_size} tokens needs {(num_pages + 1) * per_page / 2**30:.1f} GiB, "
                                    f"{free / 2**30:.1f} GiB are free on {self.device}: {fits} pages ({fits * page_size} tokens) would fit")
+        # block tables of all groups, host and device: [groups, max_requests + 1, max_blocks]; the last row of a group
+        # is the trash row (rows that pad a batch read their one page there)
+        self._tables_host = np.full((len(self.groups), max_requests + 1, self.max_blocks), -1, dtype=np.int32)
+        self._dirty: list[tuple[int, int, int, int]] = []     # (group, slot, first block, end block) changed since table_patches()
         for index, group in enumerate(self.groups):
-            group.host_table = np.full((max_requests, self.max_blocks), -1, dtype=np.int32)
+            self._tables_host[index, max_requests, 0] = group.pool.num_pages          # the trash page
+            group.host_table = self._tables_host[index, :max_requests]
+        self.device_tables = None
+        if allocate_storage and self.groups:
+            self.device_tables = torch.from_numpy(self._tables_host).to(self.device)
+        for index, group in enumerate(self.groups):
             if allocate_storage:
                 k_shape = (num_pages + 1, group.need.num_kv_heads, page_size, group.need.head_dim)
                 v_shape = (num_pages + 1, group.need.num_kv_heads, group.need.head_dim, page_size)
@@ -263,6 +278,7 @@ class CacheManager:
                 table = request.tables[index]
                 pages = group.pool.allocate(count)
                 group.host_table[request.slot, len(table):len(table) + count] = pages
+                self._touch(index, request.slot, len(table), len(table) + count)
                 table.extend(pages)
         request.length = required
 
@@ -278,6 +294,7 @@ class CacheManager:
                 raise KVCacheError(f"cannot roll back to length {length}: its pages have left the window and were given back")
             extra = [page for page in table[blocks:] if page >= 0]
             group.pool.free(extra)
+            self._touch(index, request.slot, blocks, len(table))
             del table[blocks:]
             group.host_table[request.slot, blocks:] = -1
         request.length = length
@@ -299,6 +316,7 @@ class CacheManager:
                 table[b] = -1
             if dead_blocks > request.first_live[index]:
                 group.host_table[request.slot, request.first_live[index]:dead_blocks] = -1
+                self._touch(index, request.slot, request.first_live[index], dead_blocks)
                 request.first_live[index] = dead_blocks
             group.pool.free(pages)
             freed += len(pages)
@@ -314,6 +332,7 @@ class CacheManager:
             group.pool.free([page for page in request.tables[index] if page >= 0])
             group.reserved_pages -= request.reserved[index]
             group.host_table[request.slot, :] = -1
+            self._touch(index, request.slot, 0, len(request.tables[index]))
             request.tables[index] = []
         request.released = True
         request.length = 0
@@ -321,6 +340,48 @@ class CacheManager:
         heapq.heappush(self._free_slots, request.slot)
 
     # ------------------------------------------------------------ step support
+    def _touch(self, group: int, slot: int, first: int, end: int) -> None:
+        if end > first and self.device_tables is not None:
+            self._dirty.append((group, slot, first, end))
+
+    def tables_with_trash_row(self, group: int) -> np.ndarray:
+        """The group's host block table with the trash row behind the requests' rows: [max_requests + 1, max_blocks]."""
+        return self._tables_host[group]
+
+    def device_table(self, group: int) -> torch.Tensor:
+        """The group's block table on the device, int32 [max_requests + 1, max_blocks]: row = a request's slot."""
+        return self.device_tables[group]
+
+    def table_patches(self) -> tuple[np.ndarray, np.ndarray] | None:
+        """The block table entries that have changed on the host since the last call, as (offsets into the device
+        array of all groups, values), or None if there are none.  The caller writes them into the device array
+        before the next kernel reads it."""
+        if not self._dirty:
+            return None
+        dirty, self._dirty = self._dirty, []
+        rows, blocks = self.max_requests + 1, self.max_blocks
+        flat: list[int] = []
+        for g, slot, first, end in dirty:
+            base = (g * rows + slot) * blocks
+            flat.extend(range(base + first, base + end))
+        if len(dirty) > 1:
+            flat = sorted(set(flat))             # a page taken and given back again is sent once, with what the host holds now
+        offsets = np.array(flat, dtype=np.int32)
+        return offsets, self._tables_host.reshape(-1)[offsets]
+
+    def upload_tables(self) -> None:
+        """The whole host array to the device at once (for more changes than a step's metadata has room for)."""
+        self._dirty = []
+        self.device_tables.copy_(torch.from_numpy(self._tables_host))
+
+    def tables_match_device(self) -> bool:
+        """Whether the device's block tables equal the host's in every entry that is not waiting in table_patches()."""
+        expected = self._tables_host.copy()
+        got = self.device_tables.cpu().numpy().copy()
+        for g, slot, first, end in self._dirty:
+            expected[g, slot, first:end] = got[g, slot, first:end]
+        return bool((expected == got).all())
+
     def slot_of_position(self, request: RequestCache, group: int, position: int) -> int:
         """Physical slot (page * page_size + offset) of a logical position."""
         page = request.tables[group][position // self.page_size]

@@ -753,6 +753,19 @@ LRS_API int lrs_advance_slots(int* slots, const int* positions, const int* token
   return lrs_check_launch("advance_slots");
 }
 
+// dst[pairs[2 i]] = pairs[2 i + 1] for i < count: the block table entries that changed on the host since the
+// last step, written into the device's tables.  The host has checked every offset against the tables' size.
+__global__ void scatter_i32_kernel(int* __restrict__ dst, const int* __restrict__ pairs, int count) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < count) dst[pairs[2 * i]] = pairs[2 * i + 1];
+}
+
+LRS_API int lrs_scatter_i32(int* dst, const int* pairs, int count, void* stream) {
+  LRS_REQUIRE(count > 0 && dst && pairs, "scatter_i32: needs a destination, pairs and a positive count");
+  scatter_i32_kernel<<<(count + 255) / 256, 256, 0, (hipStream_t)stream>>>(dst, pairs, count);
+  return lrs_check_launch("scatter_i32");
+}
+
 LRS_API int lrs_fill_i32(int* dst, int value, int64_t n, void* stream) {
   LRS_REQUIRE(n > 0, "fill: n must be positive");
   const int blocks = (int)((n + 255) / 256 < 4096 ? (n + 255) / 256 : 4096);

@@ -10,11 +10,13 @@ are the same thing with different lengths; entries may be cut anywhere.  The run
   4. returns float32 logits at the wanted places, in entry order then `want` order,
   5. on failure rolls every cache back to its length before the step.
 
-Device metadata (all int32): token ids, positions, request row of each token, rows whose
-logits are wanted, per request cumulative query starts, context lengths and state slots,
-and per cache group the physical slot of each token and the block table rows of the batch.
-The layout has fixed offsets given the capacities, so a captured graph can be replayed
-after only the buffer's content has changed.
+Device metadata (all int32): token ids, positions, request row of each token, the state slot of
+each token's request (which is also its row in the block tables), rows whose logits are wanted,
+per request cumulative query starts, context lengths and state slots, and per cache group the
+physical slot of each token.  The block tables themselves stay on the device (cache/manager.py):
+the step sends the entries that changed since the last one behind its metadata, in the same copy,
+and a small kernel writes them in before the step's own kernels run.  The layout has fixed offsets
+given the capacities, so a captured graph can be replayed after only the buffer's content has changed.
 
 Reference: mini_llm/model/base.py:161-248 (prefill/decode as extend -> forward -> logits,
 rollback on failure); the reference runs whole prompts alone and decode tokens as a second
@@ -45,7 +47,8 @@ class StepEntry:
 
 
 class GroupStep:
-    """Per cache group view of the step metadata on the device."""
+    """Per cache group view of the step metadata on the device: the cache slot of every token of the step, and the
+    group's block table [max_requests + 1, max_blocks], whose row for a token is ctx.token_slot[token]."""
 
     def __init__(self, slots: torch.Tensor, block_table: torch.Tensor, page_size: int):
         self.slots, self.block_table, self.page_size = slots, block_table, page_size
@@ -111,7 +114,7 @@ class StepContext:
         self.host_q_lens: list[int] = []
         self.host_slots: list[int] = []
         self.host_positions: list[int] = []   # first position of each request's tokens in this step
-        self.token_ids = self.positions = self.token_request = self.logit_rows = None
+        self.token_ids = self.positions = self.token_request = self.token_slot = self.logit_rows = None
         self.cu_seqlens_q = self.seq_lens_k = self.slot_ids = self.counts = None
         self._groups: list[GroupStep] = []
 
@@ -165,7 +168,9 @@ class ModelRunner:
         # graph holds addresses inside it: steps of one padded batch size share one layout.
         self._layouts: dict[tuple[int, int], tuple[dict, int]] = {}
         self._off, self._meta_size = self._layout(max_step_tokens, self.max_requests)
-        cursor = self._meta_size
+        # behind a step's arrays: the block table entries that changed since the last step, as (offset, value) pairs
+        cursor = self._meta_size + 2 * self.TABLE_PATCHES
+        self._patches = 0
         # two pinned staging buffers used in turn: a buffer is rewritten only after the copy
         # that read it has finished
         pin = self.device.type == "cuda"
@@ -223,11 +228,11 @@ class ModelRunner:
         if known is None:
             offsets, cursor = {}, 0
             qblocks = -(-tokens // 16) + requests if self._query_groups else 0
-            parts = [("token_ids", tokens), ("positions", tokens), ("token_request", tokens), ("logit_rows", tokens),
+            parts = [("token_ids", tokens), ("positions", tokens), ("token_request", tokens), ("token_slot", tokens), ("logit_rows", tokens),
                      ("cu_seqlens_q", requests + 1), ("seq_lens_k", requests), ("slot_ids", requests),
                      ("qblock_token0", qblocks), ("qblock_count", qblocks), ("counts", 4)]
             for index in range(len(self.cache.groups)):
-                parts += [(f"slots{index}", tokens), (f"table{index}", requests * self.cache.max_blocks)]
+                parts += [(f"slots{index}", tokens)]
             for name, size in parts:
                 offsets[name] = (cursor, size)
                 cursor += -(-size // 4) * 4
@@ -253,8 +258,27 @@ class ModelRunner:
         self._host = self._hosts[self._turn]
         self._host_np = self._host.numpy()
 
+    TABLE_PATCHES = 2048     # block table entries a step's metadata has room for (more are sent as the whole tables, once)
+
+    def _stage_table_patches(self) -> None:
+        """The block table entries that changed on the host since the last step, behind the step's arrays."""
+        self._patches = 0
+        changed = self.cache.table_patches() if self.cache.device_tables is not None else None
+        if changed is None:
+            return
+        offsets, values = changed
+        if len(offsets) > self.TABLE_PATCHES:
+            self.cache.upload_tables()
+            return
+        pairs = self._host_np[self._meta_size:self._meta_size + 2 * len(offsets)]
+        pairs[0::2], pairs[1::2] = offsets, values
+        self._patches = len(offsets)
+
     def _upload(self) -> None:
-        ops.copy_h2d(self._dev, self._host, self._meta_size)
+        self._stage_table_patches()
+        ops.copy_h2d(self._dev, self._host, self._meta_size + 2 * self._patches)
+        if self._patches:
+            ops.scatter_i32(self.cache.device_tables, self._dev, self._patches, first=self._meta_size)
         if self.device.type == "cuda":
             event = self._copied[self._turn] or torch.cuda.Event()
             event.record()
@@ -308,7 +332,7 @@ class ModelRunner:
         self._next_staging()
         self._off, self._meta_size = self._layout(max(sum(len(e.tokens) for e in entries), pad_to), max(len(entries), pad_to))
         ids, pos, req, rows = (self._host_view(n) for n in ("token_ids", "positions", "token_request", "logit_rows"))
-        cu, lens, slots = (self._host_view(n) for n in ("cu_seqlens_q", "seq_lens_k", "slot_ids"))
+        cu, lens, slots, of_token = (self._host_view(n) for n in ("cu_seqlens_q", "seq_lens_k", "slot_ids", "token_slot"))
         cursor = n_rows = 0
         cu[0] = 0
         if all(len(entry.tokens) == 1 for entry in entries):
@@ -323,6 +347,7 @@ class ModelRunner:
             cu[:cursor + 1] = count
             lens[:cursor] = lengths
             slots[:cursor] = ctx.host_slots
+            of_token[:cursor] = ctx.host_slots
             wanted = [r for r, entry in enumerate(entries) for _ in entry.want]   # a place asked twice is given twice
             n_rows = len(wanted)
             rows[:n_rows] = wanted
@@ -337,6 +362,7 @@ class ModelRunner:
                 ids[cursor:cursor + n] = entry.tokens
                 pos[cursor:cursor + n] = np.arange(start, start + n, dtype=np.int32)
                 req[cursor:cursor + n] = r
+                of_token[cursor:cursor + n] = entry.cache.slot
                 for place in entry.want:
                     rows[n_rows] = cursor + place
                     n_rows += 1
@@ -366,6 +392,7 @@ class ModelRunner:
             cu[real + 1:pad_to + 1] = np.arange(cursor + 1, cursor + extra + 1, dtype=np.int32)
             lens[real:pad_to] = 1
             slots[real:pad_to] = cache.trash_slot        # their state, like their keys and values, goes where no request reads
+            of_token[cursor:cursor + extra] = cache.trash_slot   # ... and the trash row of the block tables names the trash page
             cursor += extra
         if pad_to:
             rows[:cursor] = np.arange(cursor, dtype=np.int32)
@@ -393,16 +420,10 @@ class ModelRunner:
             ctx.max_qblock = max(b[2] for b in blocks)
             self._host_view("qblock_token0")[:len(blocks)] = [b[1] for b in blocks]
             self._host_view("qblock_count")[:len(blocks)] = [b[2] for b in blocks]
-        mb = cache.max_blocks
         for index, group in enumerate(cache.groups):
-            table = self._host_view(f"table{index}").reshape(max(real, pad_to), mb)
-            table[:real] = group.host_table[ctx.host_slots]
-            if pad_to > real:
-                table[real:pad_to] = -1
-                table[real:pad_to, 0] = cache.trash_page(index)
             gslots = self._host_view(f"slots{index}")
             p = pos[:cursor]
-            pages = table[req[:cursor], p // page]
+            pages = cache.tables_with_trash_row(index)[of_token[:cursor], p // page]
             gslots[:cursor] = np.where(pages >= 0, pages * page + p % page, -1)
         self._upload()
         self.bind_views(ctx)
@@ -413,17 +434,16 @@ class ModelRunner:
         key = (ctx.T, ctx.R, ctx.num_logit_rows, ctx.num_qblocks)
         views = self._views.get(key)
         if views is None:
-            mb = self.cache.max_blocks
             if len(self._views) > 256:
                 self._views.clear()
             views = self._views[key] = (
-                self._view("token_ids", ctx.T), self._view("positions", ctx.T), self._view("token_request", ctx.T),
+                self._view("token_ids", ctx.T), self._view("positions", ctx.T), self._view("token_request", ctx.T), self._view("token_slot", ctx.T),
                 self._view("logit_rows", max(ctx.num_logit_rows, 1)), self._view("cu_seqlens_q", ctx.R + 1),
                 self._view("seq_lens_k", ctx.R), self._view("slot_ids", ctx.R), self._view("qblock_token0", ctx.num_qblocks),
                 self._view("qblock_count", ctx.num_qblocks), self._view("counts", 4),
-                [GroupStep(self._view(f"slots{i}", ctx.T), self._view(f"table{i}").view(ctx.R, mb), self.cache.page_size)
+                [GroupStep(self._view(f"slots{i}", ctx.T), self.cache.device_table(i), self.cache.page_size)
                  for i in range(len(self.cache.groups))])
-        (ctx.token_ids, ctx.positions, ctx.token_request, ctx.logit_rows, ctx.cu_seqlens_q, ctx.seq_lens_k, ctx.slot_ids,
+        (ctx.token_ids, ctx.positions, ctx.token_request, ctx.token_slot, ctx.logit_rows, ctx.cu_seqlens_q, ctx.seq_lens_k, ctx.slot_ids,
          ctx.qblock_token0, ctx.qblock_count, ctx.counts, ctx._groups) = views
 
     def step(self, entries: Sequence[StepEntry]) -> torch.Tensor | None:
@@ -669,7 +689,7 @@ class ModelRunner:
             if i + 1 < steps:
                 ops.advance_decode(ctx.token_ids, ctx.positions, ctx.token_request, ctx.seq_lens_k, chosen, ctx.counts, draws)
                 for group in ctx._groups:
-                    ops.advance_slots(group.slots, ctx.positions, ctx.token_request, group.block_table, group.page_size, ctx.counts)
+                    ops.advance_slots(group.slots, ctx.positions, ctx.token_slot, group.block_table, group.page_size, ctx.counts)
         ops.copy_to_pinned(self._chosen_host, self._chosen_dev, steps * stride)
 
     # ------------------------------------------------------------------ graphs

@@ -83,6 +83,7 @@ _SIGNATURES = {
     "lrs_silu_mul": (c_int, [c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p]),
     "lrs_add_into": (c_int, [c_void_p, c_void_p, c_int, c_int64, c_void_p]),
     "lrs_fill_i32": (c_int, [c_void_p, c_int, c_int64, c_void_p]),
+    "lrs_scatter_i32": (c_int, [c_void_p, c_void_p, c_int, c_void_p]),
     "lrs_gather_rows": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p]),
     "lrs_gemm": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p,
                          c_int, c_float, c_int, c_int, c_void_p]),
@@ -601,6 +602,15 @@ def advance_slots(slots: torch.Tensor, positions: torch.Tensor, token_request: t
 def fill_i32(dst: torch.Tensor, value: int) -> None:
     _need(dst.dtype == torch.int32 and dst.is_contiguous(), "fill_i32: int32 contiguous tensor needed")
     _launch("lrs_fill_i32", _dev(dst, "dst"), value, dst.numel(), _stream())
+
+
+def scatter_i32(dst: torch.Tensor, pairs: torch.Tensor, count: int, first: int = 0) -> None:
+    """dst.view(-1)[offset_i] = value_i for the `count` (offset, value) pairs that lie in `pairs` (int32, on the device)
+    from element `first` on.  The caller has checked that every offset lies inside dst."""
+    _need(dst.dtype == torch.int32 and dst.is_contiguous() and pairs.dtype == torch.int32 and pairs.is_contiguous()
+          and first >= 0 and first % 2 == 0 and 0 < 2 * count <= pairs.numel() - first,
+          "scatter_i32: int32 contiguous tensors and 2 * count values in pairs from an even element on needed")
+    _launch("lrs_scatter_i32", _dev(dst, "dst"), _dev(pairs, "pairs") + 4 * first, count, _stream())
 
 
 def gather_rows(out: torch.Tensor, x: torch.Tensor, rows: torch.Tensor) -> None:

@@ -192,7 +192,7 @@ class GQAAttention(Part):
             if splits > 1:
                 part_o = ctx.scratch("attn_part_o", (t, nq * splits * d), torch.float32)
                 part_ml = ctx.scratch("attn_part_ml", (t, nq * splits * 2), torch.float32)
-            ops.attention_decode(out, qkv, cache.k_pages, cache.v_pages, group.block_table, ctx.token_request, ctx.positions,
+            ops.attention_decode(out, qkv, cache.k_pages, cache.v_pages, group.block_table, ctx.token_slot, ctx.positions,
                                  nq, self.scale, self.window or 0, splits, part_o, part_ml, ctx.max_k_bound, prepare,
                                  form=1)   # the next tile on its way while one is worked on, the first one before the query is prepared (measured: 0.6 % of a step)
         elif ops.attention_decode_supported(ctx.dtype, nq, kv_heads, d, group.page_size):
@@ -217,11 +217,11 @@ class GQAAttention(Part):
                             parted = ctx.memo[("rotation_rows", id(cos))] = (cos[:singles], sin[:singles], cos[singles:], sin[singles:])
                     first = ops.DecodePrepare(self.q_norm, self.k_norm, self.qk_norm_eps, None if parted is None else parted[0],
                                               None if parted is None else parted[1], 0)
-                ops.attention_decode(out[:singles], qkv[:singles], cache.k_pages, cache.v_pages, group.block_table, ctx.token_request,
+                ops.attention_decode(out[:singles], qkv[:singles], cache.k_pages, cache.v_pages, group.block_table, ctx.token_slot,
                                      ctx.positions, nq, self.scale, self.window or 0, splits, part_o, part_ml, ctx.max_k_bound, first, form=1)
             rest = ctx.memo.get("rows_after_singles")
             if rest is None:
-                rest = ctx.memo["rows_after_singles"] = (ctx.token_request[singles:], ctx.positions[singles:])
+                rest = ctx.memo["rows_after_singles"] = (ctx.token_slot[singles:], ctx.positions[singles:])
             if queries_raw is not None and singles and cos is not None:
                 queries_raw = ops.DecodePrepare(self.q_norm, None, self.qk_norm_eps, parted[2], parted[3], 0)
             splits = self._prefill_splits(ctx.num_qblocks * kv_heads, longest, (t - singles) * nq * d, nq // kv_heads)
@@ -233,7 +233,7 @@ class GQAAttention(Part):
                                   ctx.qblock_token0, ctx.qblock_count, nq, self.scale, self.window or 0, ctx.max_qblock, ctx.max_k_bound,
                                   splits, part_o, part_ml, queries_raw)
         else:
-            ops.attention(out, qkv, cache.k_pages, cache.v_pages, group.block_table, ctx.token_request, ctx.positions,
+            ops.attention(out, qkv, cache.k_pages, cache.v_pages, group.block_table, ctx.token_slot, ctx.positions,
                           nq, self.scale, self.window or 0)
         return linear(ctx, residual, out, self.w_o, accumulate=True, then_norm=then_norm)
 

@@ -453,6 +453,7 @@ def test_small_pool_makes_requests_wait_and_reuses_pages(folders):
             most_running = max(most_running, scheduler.num_running)
             waited_for_pages |= scheduler.num_waiting > 0 and scheduler.num_running < 4
             engine.cache_manager.check_invariants()
+            assert engine.cache_manager.tables_match_device()
     assert [got[i] for i in range(len(prompts))] == expected
     assert 2 <= most_running <= 3 and waited_for_pages and engine.cache_manager.used_pages() == 0
 
@@ -489,6 +490,7 @@ def test_many_requests_through_the_scheduler_equal_each_alone(steps_per_launch):
                 for index, event in scheduler.step():
                     got[index].append(event.token_id)
                 engine.cache_manager.check_invariants()
+                assert engine.cache_manager.tables_match_device()
     assert [got[i] for i in range(len(requests))] == want
     assert engine.cache_manager.used_pages() == 0
 

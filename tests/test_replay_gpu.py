@@ -66,6 +66,7 @@ def run_replay(folder, dtype, steps, max_tokens, tmp_path, page_size=16, as_the_
         trace.replay(runner, traces.strip(steps).splitlines(), out_dir, echo=lambda _: None)
     runner.cache.check_invariants()
     assert runner.cache.active_requests == 0 and runner.cache.used_pages() == 0
+    assert runner.cache.tables_match_device()
     return out_dir
 
 

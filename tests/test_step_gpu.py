@@ -362,6 +362,47 @@ def test_one_layer_at_the_benchmark_sizes_against_the_plain_implementation(sizes
     assert want.abs().max() > 1.0
 
 
+# ------------------------------------------------ block tables that stay on the device
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_block_tables_on_the_device_follow_the_hosts(folder_b, dtype):
+    """The device keeps the block tables; a step sends only the entries that changed since the last one.  Through
+    prompts, decoding, a rollback, a release and a new request in the freed slot the device's tables equal the
+    host's after every step, also when a step has more changes than its metadata has room for (then the whole
+    tables are sent), and the logits equal those of a runner that never ran short of room."""
+    from llm_runtime_study_amd.engine.step import StepEntry
+
+    rng = np.random.default_rng(23)
+    vocab = TINY_B["vocab_size"]
+    tokens = {key: rng.integers(0, vocab, n).tolist() for key, n in (("a", 150), ("b", 40), ("c", 90))}
+    outs = []
+    for room in (2048, 3):
+        runner = make_runner(folder_b, dtype, pages=48, requests=2, seq=256, step_tokens=160, page_size=8)
+        runner.TABLE_PATCHES = room
+        cache = runner.cache
+        rows = []
+        a, b = cache.admit("a"), cache.admit("b")
+        rows.append(runner.step([StepEntry(a, tokens["a"][:100], [99]), StepEntry(b, tokens["b"][:33], [32])]).clone())
+        assert cache.tables_match_device()
+        for i in range(7):                         # b crosses a page's edge while decoding
+            rows.append(runner.step([StepEntry(a, [tokens["a"][100 + i]], [0]), StepEntry(b, [tokens["b"][33 + i]], [0])]).clone())
+            assert cache.tables_match_device()
+        cache.extend(a, 20)                        # pages taken and given back without a step between
+        cache.rollback(a, 107)
+        cache.release(b)
+        c = cache.admit("c")                       # b's slot and, lowest ids first, b's pages
+        assert c.slot == b.slot
+        rows.append(runner.step([StepEntry(a, tokens["a"][107:150], [42]), StepEntry(c, tokens["c"], [89])]).clone())
+        assert cache.tables_match_device() and not cache._dirty
+        cache.check_invariants()
+        outs.append(torch.cat(rows))
+    assert torch.equal(outs[0], outs[1])
+    cfg, weights = plain.load_model_dir(folder_b, torch.float64)
+    want_a, want_c = plain.qwen3_forward(weights, cfg, tokens["a"]), plain.qwen3_forward(weights, cfg, tokens["c"])
+    for got, want in ((outs[0][0], want_a[99]), (outs[0][-2], want_a[149]), (outs[0][-1], want_c[89])):
+        err = (got.double().cpu() - want).norm() / want.norm()
+        assert err < (1e-5 if dtype == torch.float32 else 3e-2)
+
+
 # ---------------------------------------------------------------- launch plans
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_steps_made_again_from_a_recorded_plan_equal_steps_through_the_parts(folder_b, dtype):
