@@ -532,6 +532,63 @@ __global__ void attention_merge_kernel(bf16* __restrict__ out, int out_stride, c
   }
 }
 
+// The same merge for steps of many tokens (prompt portions whose keys were divided): a thread owns four dims of one
+// (token, head) and asks for everything it needs at once, 16 bytes a load; workgroups of four waves over all of them,
+// where a workgroup a (token, head) would be tens of thousands of workgroups of two waves with a few loads each.  The
+// sums are added in split order, as attention_merge_kernel adds them: the same bits.
+template <int SPLITS>
+__global__ __launch_bounds__(256) void attention_merge_wide_kernel(bf16* __restrict__ out, int out_stride, const float* __restrict__ part_o,
+                                                                   const float* __restrict__ part_ml, int64_t quads, int nq, int d) {
+  const int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (e >= quads) return;
+  const int per_head = d / 4;
+  const int64_t pair = e / per_head;                 // token * nq + head
+  const int dim = (int)(e % per_head) * 4;
+  const int64_t base = pair * SPLITS;
+  float m[SPLITS], l[SPLITS];
+  floatx4 o[SPLITS];
+#pragma unroll
+  for (int s = 0; s < SPLITS; ++s) {
+    const float2 ml = *(const float2*)(part_ml + (base + s) * 2);
+    m[s] = ml.x;
+    l[s] = ml.y;
+    o[s] = *(const floatx4*)(part_o + (base + s) * d + dim);
+  }
+  float top = -INFINITY;
+#pragma unroll
+  for (int s = 0; s < SPLITS; ++s) top = fmaxf(top, m[s]);
+  float total = 0.f;
+  floatx4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int s = 0; s < SPLITS; ++s) {
+    const float weight = m[s] > -INFINITY ? fast_exp2(m[s] - top) : 0.f;
+    total += l[s] * weight;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) acc[i] += o[s][i] * weight;
+  }
+  const int64_t token = pair / nq, head = pair % nq;
+  bf16x4 r;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) r[i] = (bf16)(acc[i] / total);
+  *(bf16x4*)(out + token * out_stride + head * d + dim) = r;
+}
+
+static void launch_attention_merge(bf16* out, int out_stride, const float* part_o, const float* part_ml, int tokens, int nq, int d,
+                                   int splits, hipStream_t s) {
+  const bool wide = tokens >= 64 && d % 4 == 0 && out_stride % 4 == 0 && (uintptr_t)out % 8 == 0 && (uintptr_t)part_o % 16 == 0 &&
+                    (uintptr_t)part_ml % 8 == 0 && (splits == 2 || splits == 3 || splits == 4 || splits == 8);
+  if (wide) {
+    const int64_t quads = (int64_t)tokens * nq * (d / 4);
+    const int blocks = (int)((quads + 255) / 256);
+    if (splits == 2) attention_merge_wide_kernel<2><<<blocks, 256, 0, s>>>(out, out_stride, part_o, part_ml, quads, nq, d);
+    else if (splits == 3) attention_merge_wide_kernel<3><<<blocks, 256, 0, s>>>(out, out_stride, part_o, part_ml, quads, nq, d);
+    else if (splits == 4) attention_merge_wide_kernel<4><<<blocks, 256, 0, s>>>(out, out_stride, part_o, part_ml, quads, nq, d);
+    else attention_merge_wide_kernel<8><<<blocks, 256, 0, s>>>(out, out_stride, part_o, part_ml, quads, nq, d);
+  } else {
+    attention_merge_kernel<<<dim3(tokens, nq), d < 64 ? 64 : d, 0, s>>>(out, out_stride, part_o, part_ml, nq, d, splits);
+  }
+}
+
 // Decode step in bf16: one query token per request.  part_o [tokens, nq, splits, d] and part_ml
 // [tokens, nq, splits, 2] float32 are needed when splits > 1.  Returns an error for shapes the
 // matrix-core kernel does not take (the caller then uses lrs_attention).
@@ -599,7 +656,7 @@ LRS_API int lrs_attention_decode(void* out, int out_stride, float* part_o, float
 #undef ARGS
   if (lrs_check_launch("attention_decode")) return 1;
   if (splits > 1) {
-    attention_merge_kernel<<<dim3(tokens, nq), d < 64 ? 64 : d, 0, s>>>((bf16*)out, out_stride, part_o, part_ml, nq, d, splits);
+    launch_attention_merge((bf16*)out, out_stride, part_o, part_ml, tokens, nq, d, splits, s);
     return lrs_check_launch("attention_merge");
   }
   return 0;
@@ -1450,7 +1507,7 @@ LRS_API int lrs_attention_prefill(void* out, int out_stride, const void* q, int 
 #undef LAUNCH2
   if (lrs_check_launch("attention_prefill")) return 1;
   if (splits > 1) {
-    attention_merge_kernel<<<dim3(tokens, nq), d < 64 ? 64 : d, 0, s>>>((bf16*)out, out_stride, part_o, part_ml, nq, d, splits);
+    launch_attention_merge((bf16*)out, out_stride, part_o, part_ml, tokens, nq, d, splits, s);
     return lrs_check_launch("attention_merge");
   }
   return 0;

@@ -60,7 +60,7 @@ __global__ void rmsnorm_kernel(TO* __restrict__ out, float* __restrict__ x, cons
 template <typename TW, typename TO, int VEC>
 __global__ void rmsnorm_vec_kernel(TO* __restrict__ out, float* __restrict__ x, const bf16* __restrict__ add,
                                    const TW* __restrict__ weight, const int* __restrict__ rows,
-                                   int hidden, float eps) {
+                                   int hidden, float eps, const float* __restrict__ sums = nullptr, int splits = 0) {
   __shared__ float scratch[16];
   const int64_t src_row = rows ? rows[blockIdx.x] : blockIdx.x;
   floatx4* src = (floatx4*)(x + src_row * hidden);
@@ -76,6 +76,14 @@ __global__ void rmsnorm_vec_kernel(TO* __restrict__ out, float* __restrict__ x, 
         const bf16x4 y = *(const bf16x4*)(add + src_row * hidden + c * 4);
 #pragma unroll
         for (int i = 0; i < 4; ++i) v[j][i] += (float)y[i];
+        src[c] = v[j];
+      }
+      if (sums) {
+        // what the K splits of the product before left, [splits, rows, hidden], added up in split order
+        floatx4 y = floatx4{0.f, 0.f, 0.f, 0.f};
+        for (int sp = 0; sp < splits; ++sp)
+          y += *(const floatx4*)(sums + ((int64_t)sp * gridDim.x + src_row) * hidden + c * 4);
+        v[j] += y;
         src[c] = v[j];
       }
 #pragma unroll
@@ -184,6 +192,27 @@ LRS_API int lrs_split_add_norm_begin(float* x, const float* sums, int splits, co
   else if (w_dtype == LRS_BF16) split_add_norm_begin_kernel<bf16><<<grid, threads, 0, s>>>(x, sums, splits, (const bf16*)weight, (bf16*)next_x, next_sumsq, hidden);
   else return lrs_fail("split_add_norm_begin: unknown weight dtype %d", w_dtype);
   return lrs_check_launch("split_add_norm_begin");
+}
+
+// x [n_rows, hidden] float32 += the sum over `splits` of sums[split, n_rows, hidden], then out = RMSNorm(x): what
+// follows a product of many rows whose K was divided between workgroups, in one pass over the rows.
+LRS_API int lrs_split_add_rmsnorm(void* out, int out_dtype, float* x, const float* sums, int splits, const void* weight,
+                                  int w_dtype, int n_rows, int hidden, float eps, void* stream) {
+  LRS_REQUIRE(n_rows > 0 && hidden > 0 && splits > 0 && sums && out && x && weight, "split_add_rmsnorm: rows=%d hidden=%d splits=%d must be positive", n_rows, hidden, splits);
+  LRS_REQUIRE(eps > 0.f, "split_add_rmsnorm: eps must be positive");
+  LRS_REQUIRE(hidden % 4 == 0 && hidden <= 4 * 4 * 512 && ((uintptr_t)x % 16) == 0 && ((uintptr_t)sums % 16) == 0,
+              "split_add_rmsnorm: needs hidden %% 4 == 0, at most 8192 columns and 16-byte aligned rows (hidden=%d)", hidden);
+  const int threads = hidden <= 1024 ? 64 : (hidden <= 4096 ? 256 : 512);
+  hipStream_t s = (hipStream_t)stream;
+#define LAUNCH_VEC(TW, TO) \
+  rmsnorm_vec_kernel<TW, TO, 4><<<n_rows, threads, 0, s>>>((TO*)out, x, nullptr, (const TW*)weight, nullptr, hidden, eps, sums, splits)
+  if (w_dtype == LRS_F32 && out_dtype == LRS_F32) LAUNCH_VEC(float, float);
+  else if (w_dtype == LRS_BF16 && out_dtype == LRS_BF16) LAUNCH_VEC(bf16, bf16);
+  else if (w_dtype == LRS_F32 && out_dtype == LRS_BF16) LAUNCH_VEC(float, bf16);
+  else if (w_dtype == LRS_BF16 && out_dtype == LRS_F32) LAUNCH_VEC(bf16, float);
+  else return lrs_fail("split_add_rmsnorm: unknown dtypes %d/%d", w_dtype, out_dtype);
+#undef LAUNCH_VEC
+  return lrs_check_launch("split_add_rmsnorm");
 }
 
 // x [n_rows, hidden] float32 += y (bf16), then out = RMSNorm(x): see rmsnorm_kernel.

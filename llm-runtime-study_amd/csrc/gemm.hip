@@ -1252,13 +1252,35 @@ static int even_group_rows(int n) {
   return rows <= 32 ? rows : 0;
 }
 
-// Device memory for the sums of K splits, made on first use and kept (one per process: one GPU).
+// Device memory for the sums of K splits.  A caller brings its own (`workspace`, at least lrs_gemm_workspace_bytes()
+// bytes: every runner has one, so that two runners on two streams of one GPU do not write over each other's sums
+// between a product and the kernel that finishes it); a caller that brings none gets one that the process keeps, made
+// on first use, and must then keep all its products on one stream.  Which of the two an entry point uses is a matter
+// of that call alone: UseSpace notes it for the launches the call makes on its thread.
 static float* g_split_sums = nullptr;
 constexpr size_t SPLIT_SUMS_BYTES = 64u << 20;
-static float* split_sums_buffer() {
+static float* own_split_sums() {
   if (!g_split_sums && hipMalloc((void**)&g_split_sums, SPLIT_SUMS_BYTES) != hipSuccess) g_split_sums = nullptr;
   return g_split_sums;
 }
+struct SplitSpace {
+  float* sums;
+  size_t bytes;
+};
+static thread_local SplitSpace t_split_space = {nullptr, 0};
+struct UseSpace {
+  SplitSpace before;
+  UseSpace(void* workspace, int64_t bytes) : before(t_split_space) {
+    t_split_space = workspace ? SplitSpace{(float*)workspace, (size_t)bytes} : SplitSpace{own_split_sums(), SPLIT_SUMS_BYTES};
+  }
+  ~UseSpace() { t_split_space = before; }
+};
+static float* split_sums_buffer() { return t_split_space.sums; }
+static size_t split_sums_bytes() { return t_split_space.sums ? t_split_space.bytes : 0; }
+static bool workspace_ok(const void* workspace, int64_t bytes) {
+  return workspace == nullptr || (bytes >= (int64_t)SPLIT_SUMS_BYTES && (uintptr_t)workspace % 16 == 0);
+}
+LRS_API int64_t lrs_gemm_workspace_bytes() { return (int64_t)SPLIT_SUMS_BYTES; }
 
 // The kernel for 17..128 rows: which of its workgroup shapes and how many K splits.  Unless the caller's
 // choices say otherwise: the shape and split that fill a whole multiple of the compute units best, then the
@@ -1342,7 +1364,7 @@ static int launch_mid_mt(void* out, int mode, const bf16* a, const bf16* w, int 
   int waves = 4, splits = 1;
   choose_mid_shape(n, k, tune, waves, splits);
   float* sums = splits > 1 || keep_sums ? split_sums_buffer() : nullptr;
-  if ((splits > 1 || keep_sums) && (!sums || (size_t)splits * m * n * sizeof(float) > SPLIT_SUMS_BYTES)) {
+  if ((splits > 1 || keep_sums) && (!sums || (size_t)splits * m * n * sizeof(float) > split_sums_bytes())) {
     if (keep_sums) return 0;
     splits = 1, sums = nullptr;
   }
@@ -1393,7 +1415,7 @@ static void launch_skinny(void* out, int mode, const bf16* a, NormInput norm, co
     if (splits > 8) splits = 8;
     while (splits > 1 && k / splits < 512) --splits;
     float* sums = splits > 1 ? split_sums_buffer() : nullptr;
-    if (splits > 1 && (!sums || (size_t)splits * m * n * sizeof(float) > SPLIT_SUMS_BYTES)) splits = 1;
+    if (splits > 1 && (!sums || (size_t)splits * m * n * sizeof(float) > split_sums_bytes())) splits = 1;
     launch_skinny_rt<MT, (MT > 1 ? 4 : 1), NORM, SWIGLU>(out, mode, a, norm, w, bias, m, n, k, lda, ldc, s, tune, sums, splits);
     return;
   }
@@ -1426,7 +1448,7 @@ static void launch_skinny_m(void* out, int mode, const bf16* a, NormInput norm, 
 // Allocates the device memory the K-split products need, so that no later call has to (a call
 // under graph capture must not allocate).  Safe to call more than once.
 LRS_API int lrs_gemm_prepare() {
-  if (!split_sums_buffer()) return lrs_fail("gemm_prepare: could not allocate %zu bytes for split sums", SPLIT_SUMS_BYTES);
+  if (!own_split_sums()) return lrs_fail("gemm_prepare: could not allocate %zu bytes for split sums", SPLIT_SUMS_BYTES);
   return 0;
 }
 
@@ -1479,8 +1501,11 @@ static bool mid_shape_ok(const void* a, const void* w, int m, int n, int k, int 
 // [M, K], in_sumsq [in_parts, M] partial sums of h^2; row r of the result is multiplied by
 // rsqrt(sum_p in_sumsq[p, r] / K + in_eps).  swiglu as in lrs_gemm.
 LRS_API int lrs_gemm_mid_scaled(void* out, int mode, const void* a, const void* w, int m, int n, int k, int lda, int ldc,
-                                int swiglu, const float* in_sumsq, int in_parts, float in_eps, int tune, void* stream) {
+                                int swiglu, const float* in_sumsq, int in_parts, float in_eps, int tune, void* workspace,
+                                int64_t workspace_bytes, void* stream) {
   LRS_REQUIRE(tune_ok(tune), "gemm_mid_scaled: unknown choices %d", tune);
+  LRS_REQUIRE(workspace_ok(workspace, workspace_bytes), "gemm_mid_scaled: a workspace must be 16-byte aligned and hold lrs_gemm_workspace_bytes() bytes");
+  const UseSpace space(workspace, workspace_bytes);
   LRS_REQUIRE(mid_shape_ok(a, w, m, n, k, lda), "gemm_mid_scaled: takes 17..128 rows, K %% 256 == 0, N %% 16 == 0, 16-byte aligned rows (m=%d n=%d k=%d lda=%d)", m, n, k, lda);
   LRS_REQUIRE(mode >= OUT_STORE && mode <= OUT_ADD_F32 && ldc >= (swiglu ? n / 2 : n) && ldc % 4 == 0 && (uintptr_t)out % 16 == 0,
               "gemm_mid_scaled: unknown output mode %d, or an output that is not 16-byte aligned (ldc=%d)", mode, ldc);
@@ -1503,8 +1528,11 @@ extern "C" int lrs_split_add_norm_begin(float* x, const float* sums, int splits,
 // (lrs_gemm_mid_scaled) or for scale_rows.  The kernel that adds the K splits' sums spreads over rows x 1,024
 // columns, where a whole norm would have one workgroup a row.
 LRS_API int lrs_gemm_mid_add_norm_begin(float* residual, const void* a, const void* w, const void* norm_weight, int norm_weight_dtype,
-                                        void* next_x, float* next_sumsq, int m, int n, int k, int lda, int tune, void* stream) {
+                                        void* next_x, float* next_sumsq, int m, int n, int k, int lda, int tune, void* workspace,
+                                        int64_t workspace_bytes, void* stream) {
   LRS_REQUIRE(tune_ok(tune), "gemm_mid_add_norm_begin: unknown choices %d", tune);
+  LRS_REQUIRE(workspace_ok(workspace, workspace_bytes), "gemm_mid_add_norm_begin: a workspace must be 16-byte aligned and hold lrs_gemm_workspace_bytes() bytes");
+  const UseSpace space(workspace, workspace_bytes);
   LRS_REQUIRE(mid_shape_ok(a, w, m, n, k, lda) && ((uintptr_t)residual % 16 == 0), "gemm_mid_add_norm_begin: takes 17..128 rows, K %% 256 == 0, N %% 16 == 0, 16-byte aligned rows (m=%d n=%d k=%d lda=%d)", m, n, k, lda);
   LRS_REQUIRE(next_x && next_sumsq && norm_weight, "gemm_mid_add_norm_begin: needs the norm weight and the two outputs for the next norm");
   const int splits = launch_mid<false>(nullptr, OUT_STORE, (const bf16*)a, (const bf16*)w, m, n, k, lda, n, (hipStream_t)stream, tune_of(tune), true);
@@ -1526,9 +1554,11 @@ LRS_API int lrs_gemm_mid_qk_prep(void* qkv, int row_stride, const void* a, const
                                  const float* in_sumsq, int in_parts, float in_eps, int nq, int nkv, int d,
                                  const void* q_weight, const void* k_weight, int w_dtype, float eps, const float* cosv,
                                  const float* sinv, int rot_half, void* k_pages, void* v_pages, const int* slots,
-                                 int page_size, int tune, void* stream) {
+                                 int page_size, int tune, void* workspace, int64_t workspace_bytes, void* stream) {
   const int n = (nq + 2 * nkv) * d;
   LRS_REQUIRE(tune_ok(tune), "gemm_mid_qk_prep: unknown choices %d", tune);
+  LRS_REQUIRE(workspace_ok(workspace, workspace_bytes), "gemm_mid_qk_prep: a workspace must be 16-byte aligned and hold lrs_gemm_workspace_bytes() bytes");
+  const UseSpace space(workspace, workspace_bytes);
   LRS_REQUIRE(mid_shape_ok(a, w, m, n, k, lda), "gemm_mid_qk_prep: takes 17..128 rows, K %% 256 == 0, N %% 16 == 0, 16-byte aligned rows (m=%d n=%d k=%d lda=%d)", m, n, k, lda);
   LRS_REQUIRE(in_sumsq == nullptr || (in_parts > 0 && in_eps > 0.f), "gemm_mid_qk_prep: in_parts and in_eps must be positive");
   const MidScale scale{in_sumsq, in_parts, in_eps};
@@ -1588,16 +1618,51 @@ LRS_API int lrs_gemm_lines_split_pays(int m, int n, int k) {
   return m <= 256 && splits >= 2 && (k / 64 + splits - 1) / splits >= 12;
 }
 
+// Defined beside the norm kernels: x += the sum of the splits' sums, then out = RMSNorm(x), one pass over the rows.
+extern "C" int lrs_split_add_rmsnorm(void* out, int out_dtype, float* x, const float* sums, int splits, const void* weight,
+                                     int w_dtype, int n_rows, int hidden, float eps, void* stream);
+
+// A product of more than 128 bf16 rows that adds into the float32 residual stream, and the RMSNorm that follows, as two
+// kernels: residual [M, N] += a [M, K] w[N, K]^T; normed [M, N] = RMSNorm(residual) with norm_weight and eps.  The
+// product is the many-rows kernel with slices of whole lines, its K divided between workgroups as lrs_gemm_lines_splits
+// says (which must take the shape); its sums stay in the workspace, and the kernel that adds them up also adds the
+// residual, writes it back and normalises the row: no kernel of its own for the add, none for the norm.
+LRS_API int lrs_gemm_lines_add_rmsnorm(float* residual, const void* a, const void* w, int m, int n, int k, int lda,
+                                       const void* norm_weight, int norm_weight_dtype, float eps, void* normed, int normed_dtype,
+                                       void* workspace, int64_t workspace_bytes, void* stream) {
+  LRS_REQUIRE(m > 128 && n > 0 && k > 0 && lda >= k, "gemm_lines_add_rmsnorm: takes more than 128 rows and positive sizes, got m=%d n=%d k=%d lda=%d", m, n, k, lda);
+  LRS_REQUIRE(workspace_ok(workspace, workspace_bytes), "gemm_lines_add_rmsnorm: a workspace must be 16-byte aligned and hold lrs_gemm_workspace_bytes() bytes");
+  const UseSpace space(workspace, workspace_bytes);
+  const int splits = lrs_gemm_lines_splits(m, n, k);
+  LRS_REQUIRE(splits >= 1, "gemm_lines_add_rmsnorm: the divided product does not take m=%d n=%d k=%d (see lrs_gemm_lines_splits)", m, n, k);
+  LRS_REQUIRE(k % WIDE_BK == 0 && lda % 8 == 0 && n % 4 == 0 && ((uintptr_t)a % 16 == 0) && ((uintptr_t)w % 16 == 0) && ((uintptr_t)residual % 16 == 0) &&
+                  (int64_t)m * lda < (1ll << 31) && (int64_t)n * k < (1ll << 31),
+              "gemm_lines_add_rmsnorm: needs 16-byte aligned rows and sizes below 2^31 elements (m=%d n=%d k=%d lda=%d)", m, n, k, lda);
+  float* sums = split_sums_buffer();
+  LRS_REQUIRE(sums != nullptr && (size_t)splits * m * n * sizeof(float) <= split_sums_bytes(), "gemm_lines_add_rmsnorm: no room for the sums of %d K splits of %d x %d", splits, m, n);
+  LRS_REQUIRE(residual && normed && norm_weight && eps > 0.f, "gemm_lines_add_rmsnorm: needs the residual stream, the norm's weight, a positive eps and the output");
+  const int big_m = (m + 255) / 256, tiles_w = (n + 127) / 128;
+  gemm_bf16_lines_kernel<128, false, OUT_STORE_F32><<<big_m * tiles_w * splits, 512, 0, (hipStream_t)stream>>>(
+      sums, (const bf16*)a, (const bf16*)w, m, n, k, lda, n, big_m, tiles_w, splits);
+  if (int rc = lrs_check_launch("gemm_lines_add_rmsnorm")) return rc;
+  return lrs_split_add_rmsnorm(normed, normed_dtype, residual, sums, splits, norm_weight, norm_weight_dtype, m, n, eps, stream);
+}
+
 // out [M, N] (row stride ldc) = a [M, K] (row stride lda) times w[N, K]^T.
 //   norm_weight != null: `a` is the float32 residual stream [*, K]; its rows (picked through
 //     `rows` if given) are RMS-normalised with norm_weight and eps on the way in.  bf16 weights,
 //     at most 64 rows.
 //   swiglu != 0: w holds gate and up rows interleaved in groups of 8 and out is [M, N/2] with
 //     silu(gate) * up.  bf16, K % 8 == 0, no bias.
+//   workspace: device memory of lrs_gemm_workspace_bytes() bytes for the sums of K splits, the caller's own; null: the
+//     one the process keeps, which every caller that brings none shares (products on one stream only then).
 LRS_API int lrs_gemm(void* out, int mode, const void* a, const void* w, const void* bias, int dtype,
                      int m, int n, int k, int lda, int ldc, const int* rows, const void* norm_weight,
-                     int norm_weight_dtype, float eps, int swiglu, int tune_word, void* stream) {
+                     int norm_weight_dtype, float eps, int swiglu, int tune_word, void* workspace, int64_t workspace_bytes,
+                     void* stream) {
   LRS_REQUIRE(m > 0 && n > 0 && k > 0, "gemm: sizes m=%d n=%d k=%d must be positive", m, n, k);
+  LRS_REQUIRE(workspace_ok(workspace, workspace_bytes), "gemm: a workspace must be 16-byte aligned and hold lrs_gemm_workspace_bytes() bytes");
+  const UseSpace space(workspace, workspace_bytes);
   LRS_REQUIRE(tune_ok(tune_word), "gemm: unknown choices %d", tune_word);
   const GemmTune tune = tune_of(tune_word);
   LRS_REQUIRE(lda >= k && ldc >= (swiglu ? n / 2 : n), "gemm: strides lda=%d ldc=%d too small for k=%d n=%d", lda, ldc, k, n);

@@ -79,14 +79,18 @@ _SIGNATURES = {
     "lrs_qk_prep": (c_int, [c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_int, c_float,
                             c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p]),
     "lrs_gemm_mid_qk_prep": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p, c_int, c_float, c_int, c_int, c_int,
-                                     c_void_p, c_void_p, c_int, c_float, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p]),
+                                     c_void_p, c_void_p, c_int, c_float, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int,
+                                     c_void_p, c_int64, c_void_p]),
     "lrs_silu_mul": (c_int, [c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p]),
     "lrs_add_into": (c_int, [c_void_p, c_void_p, c_int, c_int64, c_void_p]),
     "lrs_fill_i32": (c_int, [c_void_p, c_int, c_int64, c_void_p]),
     "lrs_scatter_i32": (c_int, [c_void_p, c_void_p, c_int, c_void_p]),
     "lrs_gather_rows": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p]),
     "lrs_gemm": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p,
-                         c_int, c_float, c_int, c_int, c_void_p]),
+                         c_int, c_float, c_int, c_int, c_void_p, c_int64, c_void_p]),
+    "lrs_gemm_workspace_bytes": (c_int64, []),
+    "lrs_gemm_lines_add_rmsnorm": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p, c_int, c_float, c_void_p, c_int,
+                                           c_void_p, c_int64, c_void_p]),
     "lrs_gemm_norm_chain": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,
                                     c_void_p, c_int, c_float, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p]),
     "lrs_gemm_norm_chain_parts": (c_int, [c_int]),
@@ -104,8 +108,10 @@ _SIGNATURES = {
     "lrs_library_gemm": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p]),
     "lrs_host_device_pointer": (c_int, [c_void_p, POINTER(c_void_p)]),
     "lrs_gemm_mid_shape": (c_int, [c_int, c_int, c_int, c_void_p, c_void_p]),
-    "lrs_gemm_mid_scaled": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_int, c_float, c_int, c_void_p]),
-    "lrs_gemm_mid_add_norm_begin": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p]),
+    "lrs_gemm_mid_scaled": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_int, c_float, c_int,
+                                    c_void_p, c_int64, c_void_p]),
+    "lrs_gemm_mid_add_norm_begin": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int,
+                                            c_void_p, c_int64, c_void_p]),
     "lrs_norm_begin_parts": (c_int, [c_int]),
     "lrs_attention": (c_int, [c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p,
                               c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_void_p]),
@@ -165,7 +171,7 @@ def library():
 # and _SIGNATURES by kernels/plan_codegen.py, is the other side (a test keeps the two in step).
 PLAN_OPS = ("lrs_add_into", "lrs_add_rmsnorm", "lrs_advance_decode", "lrs_advance_slots", "lrs_attention", "lrs_attention_decode",
             "lrs_attention_prefill", "lrs_choose_tokens", "lrs_choose_tokens_split", "lrs_copy_to_pinned", "lrs_embed", "lrs_fill_i32",
-            "lrs_filter_logits", "lrs_gather_rows", "lrs_gemm", "lrs_gemm_mid_add_norm_begin", "lrs_gemm_mid_qk_prep", "lrs_gemm_mid_scaled",
+            "lrs_filter_logits", "lrs_gather_rows", "lrs_gemm", "lrs_gemm_lines_add_rmsnorm", "lrs_gemm_mid_add_norm_begin", "lrs_gemm_mid_qk_prep", "lrs_gemm_mid_scaled",
             "lrs_gemm_norm_chain", "lrs_library_gemm", "lrs_qk_prep", "lrs_rmsnorm", "lrs_rope_table", "lrs_scale_rows", "lrs_silu_mul")
 _PLAN_INDEX = {name: index for index, name in enumerate(PLAN_OPS)}
 
@@ -429,6 +435,22 @@ def qk_prep(qkv: torch.Tensor, nq: int, nkv: int, d: int, q_weight, k_weight, ep
         None if nkv == 0 else _dev(slots, "slots"), page_size, int(bool(skip_q)), _stream())
 
 
+@functools.lru_cache(maxsize=1)
+def gemm_workspace_bytes() -> int:
+    """Bytes of device memory a caller brings as `workspace` to the products that divide K between workgroups."""
+    return int(library().lrs_gemm_workspace_bytes())
+
+
+def _workspace(t: torch.Tensor | None, name: str) -> tuple:
+    """(address, bytes) of a caller's workspace for the sums of K splits; (None, 0): the one the process keeps, which
+    all callers that bring none share (their products must then stay on one stream)."""
+    if t is None:
+        return None, 0
+    _need(t.is_cuda and t.is_contiguous() and t.numel() * t.element_size() >= gemm_workspace_bytes(),
+          f"{name}: the workspace must be a contiguous device tensor of at least {gemm_workspace_bytes()} bytes")
+    return t.data_ptr(), t.numel() * t.element_size()
+
+
 def gemm_mid_qk_prep_takes(dtype: torch.dtype, m: int, nq: int, nkv: int, d: int, k: int, rot_half: int,
                            choice: KernelChoice = DEFAULT_CHOICE) -> bool:
     """Whether gemm_mid_qk_prep() takes the shape: bf16, 17..128 rows, heads the vector form of qk_prep takes
@@ -440,7 +462,7 @@ def gemm_mid_qk_prep_takes(dtype: torch.dtype, m: int, nq: int, nkv: int, d: int
 
 def gemm_mid_qk_prep(qkv: torch.Tensor, a: torch.Tensor, w: torch.Tensor, sumsq: torch.Tensor | None, in_eps: float, nq: int, nkv: int,
                      d: int, q_weight, k_weight, eps: float, cos, sin, k_pages, v_pages, slots, page_size: int,
-                     choice: KernelChoice = DEFAULT_CHOICE) -> None:
+                     choice: KernelChoice = DEFAULT_CHOICE, workspace: torch.Tensor | None = None) -> None:
     """The q/k/v product of 17..128 bf16 rows (a @ w.T; with `sumsq` the input is a norm begun before it, as in
     gemm_mid_scaled) and qk_prep() of its result in two kernels: the one that prepares the heads adds up the sums of
     the product's K splits itself.  q goes into `qkv` [M, (nq+2*nkv)*d], k and v into the pages."""
@@ -468,7 +490,8 @@ def gemm_mid_qk_prep(qkv: torch.Tensor, a: torch.Tensor, w: torch.Tensor, sumsq:
         None if sumsq is None else _dev(sumsq, "sumsq"), 0 if sumsq is None else sumsq.shape[0], in_eps if sumsq is not None else 0.0,
         nq, nkv, d, None if q_weight is None else _dev(q_weight, "q_weight"), None if k_weight is None else _dev(k_weight, "k_weight"),
         dtype_code(w_dtype), eps, None if cos is None else cos.data_ptr(), None if sin is None else sin.data_ptr(), rot_half,
-        _dev(k_pages, "k_pages"), _dev(v_pages, "v_pages"), _dev(slots, "slots"), page_size, choice.word, _stream())
+        _dev(k_pages, "k_pages"), _dev(v_pages, "v_pages"), _dev(slots, "slots"), page_size, choice.word,
+        *_workspace(workspace, "gemm_mid_qk_prep"), _stream())
 
 
 def silu_mul(out: torch.Tensor, gate_up: torch.Tensor, interleaved: bool = False) -> None:
@@ -537,7 +560,8 @@ def norm_begin_parts(n: int) -> int:
 
 
 def gemm_mid_add_norm_begin(residual: torch.Tensor, a: torch.Tensor, w: torch.Tensor, norm_weight: torch.Tensor,
-                            next_x: torch.Tensor, next_sumsq: torch.Tensor, choice: KernelChoice = DEFAULT_CHOICE) -> None:
+                            next_x: torch.Tensor, next_sumsq: torch.Tensor, choice: KernelChoice = DEFAULT_CHOICE,
+                            workspace: torch.Tensor | None = None) -> None:
     """residual (float32 [M, N]) += a @ w.T for 17..128 bf16 rows, and the first half of the RMSNorm that follows:
     next_x [M, N] = bf16(residual * norm_weight), next_sumsq [norm_begin_parts(N), M] = partial sums of residual^2.
     gemm_mid_scaled() (or scale_rows()) finishes the norm."""
@@ -552,11 +576,11 @@ def gemm_mid_add_norm_begin(residual: torch.Tensor, a: torch.Tensor, w: torch.Te
     _need(norm_weight.is_contiguous() and norm_weight.numel() == n, f"gemm_mid_add_norm_begin: norm weight must hold {n} values")
     _launch("lrs_gemm_mid_add_norm_begin", _dev(residual, "residual"), _dev(a, "a"), _dev(w, "w"), _dev(norm_weight, "norm_weight"),
                                                  dtype_code(norm_weight.dtype), _dev(next_x, "next_x"), _dev(next_sumsq, "next_sumsq"),
-                                                 m, n, k, _rows(a, "a"), choice.word, _stream())
+                                                 m, n, k, _rows(a, "a"), choice.word, *_workspace(workspace, "gemm_mid_add_norm_begin"), _stream())
 
 
 def gemm_mid_scaled(out: torch.Tensor, a: torch.Tensor, w: torch.Tensor, sumsq: torch.Tensor, eps: float, swiglu: bool = False,
-                    choice: KernelChoice = DEFAULT_CHOICE) -> None:
+                    choice: KernelChoice = DEFAULT_CHOICE, workspace: torch.Tensor | None = None) -> None:
     """out = (the RMSNorm that `a` and `sumsq` stand for) @ w.T for 17..128 rows: a = bf16(h * norm weight) [M, K],
     sumsq [parts, M] partial sums of h^2; row r of the product is multiplied by rsqrt(sum_p sumsq[p, r] / K + eps).
     swiglu as in gemm()."""
@@ -569,7 +593,8 @@ def gemm_mid_scaled(out: torch.Tensor, a: torch.Tensor, w: torch.Tensor, sumsq: 
     _need(sumsq.dtype == torch.float32 and sumsq.dim() == 2 and sumsq.shape[1] == m and sumsq.is_contiguous() and eps > 0, f"gemm_mid_scaled: sumsq must be float32 [parts, {m}] and eps positive")
     mode = OUT_STORE if out.dtype == torch.bfloat16 else OUT_STORE_F32
     _launch("lrs_gemm_mid_scaled", _dev(out, "out"), mode, _dev(a, "a"), _dev(w, "w"), m, n, k, _rows(a, "a"), _rows(out, "out"),
-                                         int(swiglu), _dev(sumsq, "sumsq"), sumsq.shape[0], eps, choice.word, _stream())
+                                         int(swiglu), _dev(sumsq, "sumsq"), sumsq.shape[0], eps, choice.word,
+                                         *_workspace(workspace, "gemm_mid_scaled"), _stream())
 
 
 def _int_vector(t: torch.Tensor, name: str, at_least: int) -> int:
@@ -635,8 +660,11 @@ def gemm_norm_fusion_pays(n: int) -> bool:
 
 def gemm(out: torch.Tensor, a: torch.Tensor, w: torch.Tensor, bias: torch.Tensor | None = None, accumulate: bool = False,
          swiglu: bool = False, norm_weight: torch.Tensor | None = None, eps: float = 0.0, rows: torch.Tensor | None = None,
-         count: int | None = None, choice: KernelChoice = DEFAULT_CHOICE) -> None:
+         count: int | None = None, choice: KernelChoice = DEFAULT_CHOICE, workspace: torch.Tensor | None = None) -> None:
     """out = a @ w.T (+ bias).  `accumulate` adds into a float32 `out` instead of storing.
+
+    workspace: the caller's own device memory (gemm_workspace_bytes()) for the sums of K splits, which some shapes
+    leave for a second kernel; without it the process-wide one is used, which is safe on one stream only.
 
     norm_weight: `a` is the float32 residual stream [*, K]; the product is taken of its RMSNorm
     (weight norm_weight, eps), of the `count` rows listed in `rows` if given, else of its first rows.
@@ -674,7 +702,25 @@ def gemm(out: torch.Tensor, a: torch.Tensor, w: torch.Tensor, bias: torch.Tensor
     _launch("lrs_gemm", _dev(out, "out"), mode, _dev(a, "a"), _dev(w, "w"), None if bias is None else _dev(bias, "bias"),
                               dtype_code(w.dtype), m, n, k, lda, ldc, None if rows is None else _dev(rows, "rows"),
                               None if not normed else _dev(norm_weight, "norm_weight"), dtype_code(norm_weight.dtype) if normed else 0,
-                              eps, 1 if swiglu else 0, choice.word, _stream())
+                              eps, 1 if swiglu else 0, choice.word, *_workspace(workspace, "gemm"), _stream())
+
+
+def gemm_lines_add_rmsnorm(residual: torch.Tensor, a: torch.Tensor, w: torch.Tensor, norm_weight: torch.Tensor, eps: float,
+                           normed: torch.Tensor, workspace: torch.Tensor | None = None) -> None:
+    """residual (float32 [M, N]) += a @ w.T for more than 128 bf16 rows of a shape that gemm_lines_splits() takes, and
+    normed [M, N] = RMSNorm(residual) with `norm_weight` and `eps`: the product with its K divided between workgroups,
+    and one kernel that adds up their sums, adds them to the residual stream and normalises the rows."""
+    m, k = a.shape
+    n = w.shape[0]
+    _need(a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and w.shape == (n, k) and w.is_contiguous() and m > 128
+          and gemm_lines_splits(m, n, k) >= 1, "gemm_lines_add_rmsnorm: takes bf16 products of more than 128 rows that gemm_lines_splits() takes")
+    _need(residual.dtype == torch.float32 and residual.is_contiguous() and residual.shape == (m, n), f"gemm_lines_add_rmsnorm: residual must be contiguous float32 [{m}, {n}]")
+    _need(normed.is_contiguous() and normed.shape == (m, n), f"gemm_lines_add_rmsnorm: normed must be contiguous [{m}, {n}]")
+    _need(norm_weight.is_contiguous() and norm_weight.numel() == n and eps > 0 and n % 4 == 0 and n <= 8192,
+          f"gemm_lines_add_rmsnorm: the norm weight must hold {n} values, eps be positive and N a multiple of 4 up to 8192")
+    _launch("lrs_gemm_lines_add_rmsnorm", _dev(residual, "residual"), _dev(a, "a"), _dev(w, "w"), m, n, k, _rows(a, "a"),
+            _dev(norm_weight, "norm_weight"), dtype_code(norm_weight.dtype), eps, _dev(normed, "normed"), dtype_code(normed.dtype),
+            *_workspace(workspace, "gemm_lines_add_rmsnorm"), _stream())
 
 
 def library_gemm(out: torch.Tensor, a: torch.Tensor, w: torch.Tensor) -> None:

@@ -20,7 +20,7 @@ import torch
 
 from ..kernels import ops
 from .base import PagedKVNeed, Part, PartSpec, TensorSpec, create, length_class, register
-from .linear import ScaledRows, kernels_of, linear, materialize, rows_of
+from .linear import ScaledRows, kernels_of, linear, materialize, rows_of, workspace_of
 
 
 class GQAAttention(Part):
@@ -158,7 +158,7 @@ class GQAAttention(Part):
         if together:
             ops.gemm_mid_qk_prep(qkv, plain, self.w_qkv, None if begun is None else begun.sumsq, 0.0 if begun is None else begun.eps,
                                  nq, nkv, d, self.q_norm, self.k_norm, self.qk_norm_eps, cos, sin, cache.k_pages, cache.v_pages,
-                                 group.slots, group.page_size, choice=kernels_of(ctx))
+                                 group.slots, group.page_size, choice=kernels_of(ctx), workspace=workspace_of(ctx))
         else:
             linear(ctx, qkv, x if plain is None or begun is not None else plain, self.w_qkv, self.b_qkv)
         out = ctx.scratch("attn_out", (t, nq * d), ctx.dtype)

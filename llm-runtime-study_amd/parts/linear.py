@@ -21,6 +21,9 @@ name of a route and `linear()` runs it.  The routes:
   fused_norm few rows of the float32 residual stream, normalised on the way in (gemm with norm_weight)
   mid_begin  17..128 rows adding into the residual stream and beginning the norm that follows
   mid        17..128 rows, nothing folded in (gemm picks the kernel for them)
+  split_norm more than 128 rows adding into the residual stream before an RMSNorm, of a shape whose K this package's
+             many-rows kernel divides between workgroups: the kernel that adds up their sums also adds the residual
+             and normalises the rows (gemm_lines_add_rmsnorm)
   library    more rows than these kernels are made for, if the step may use the vendor library; the
              residual add (with the norm that follows) or the gated activation take one more small kernel
   own        everything else, and every float32 product (gemm picks the kernel by shape)
@@ -76,7 +79,13 @@ def kernels_of(ctx) -> ops.KernelChoice:
     return getattr(ctx, "kernels", None) or ops.DEFAULT_CHOICE
 
 
-ROUTES = ("chain", "mid_scaled", "fused_norm", "mid_begin", "mid", "library", "own")
+def workspace_of(ctx) -> torch.Tensor:
+    """The step's own memory for the sums of products that divide K between workgroups (one per scratch arena, so two
+    runners on two streams never share one)."""
+    return ctx.scratch("gemm_split_sums", (ops.gemm_workspace_bytes() // 4,), torch.float32)
+
+
+ROUTES = ("chain", "mid_scaled", "fused_norm", "mid_begin", "mid", "split_norm", "library", "own")
 
 
 def plan(m: int, n: int, k: int, *, weight_dtype: torch.dtype, run_dtype: torch.dtype, out_dtype: torch.dtype, arrives: str,
@@ -111,7 +120,8 @@ def plan(m: int, n: int, k: int, *, weight_dtype: torch.dtype, run_dtype: torch.
     if (choice.library and bf16 and m > choice.few_rows_max and not bias and contiguous
             and (accumulate or (stores and out_contiguous))):
         if m > 128 and out_contiguous and ops.gemm_split_pays(m, n, k):
-            return "own", first            # too few tiles for the chip and a long K: divided between workgroups here
+            # too few tiles for the chip and a long K: divided between workgroups here
+            return ("split_norm" if follows and n % 4 == 0 and n <= 8192 else "own"), first
         return "library", first
     return "own", first
 
@@ -152,7 +162,7 @@ def linear(ctx, out, x, weight, bias=None, accumulate: bool = False, swiglu: boo
     if first:
         x = x.materialize(ctx)
         # a plain tensor now: its dtype and layout may send it elsewhere than was planned for the norm's own form
-        if route in ("mid", "mid_begin", "library") and not (x.dtype == torch.bfloat16 and x.is_contiguous()):
+        if route in ("mid", "mid_begin", "library", "split_norm") and not (x.dtype == torch.bfloat16 and x.is_contiguous()):
             route = "own"
     elif arrives == "tensor" and route != "own" and x.dtype != torch.bfloat16:
         route = "own"
@@ -167,7 +177,7 @@ def linear(ctx, out, x, weight, bias=None, accumulate: bool = False, swiglu: boo
                             next_weight=None if begun is None else following[0], choice=choice)
         return begun
     if route == "mid_scaled":
-        ops.gemm_mid_scaled(out, scaled.x, weight, scaled.sumsq, scaled.eps, swiglu, choice=choice)
+        ops.gemm_mid_scaled(out, scaled.x, weight, scaled.sumsq, scaled.eps, swiglu, choice=choice, workspace=workspace_of(ctx))
         return None
     if route == "fused_norm":
         ops.gemm(out, x.h, weight, bias, accumulate, swiglu, norm_weight=x.weight, eps=x.eps, rows=x.rows, count=x.count, choice=choice)
@@ -176,8 +186,12 @@ def linear(ctx, out, x, weight, bias=None, accumulate: bool = False, swiglu: boo
         # product, residual add and the first half of the norm that follows: the kernel that adds the K splits'
         # sums leaves bf16(h * norm weight) and partial sums of squares, the next product finishes
         begun = _ahead_buffers(ctx, m, n, ops.norm_begin_parts(n), following[1], "norm_begin_sumsq")
-        ops.gemm_mid_add_norm_begin(out, x, weight, following[0], begun.x, begun.sumsq, choice=choice)
+        ops.gemm_mid_add_norm_begin(out, x, weight, following[0], begun.x, begun.sumsq, choice=choice, workspace=workspace_of(ctx))
         return begun
+    if route == "split_norm":
+        normed = ctx.scratch("norm_after_add", (m, n), ctx.dtype)
+        ops.gemm_lines_add_rmsnorm(out, x, weight, following[0], following[1], normed, workspace=workspace_of(ctx))
+        return normed
     if route == "library":
         if not (accumulate or swiglu):
             ops.library_gemm(out, x, weight)                      # bfloat16, or the float32 logits of many rows
@@ -194,5 +208,6 @@ def linear(ctx, out, x, weight, bias=None, accumulate: bool = False, swiglu: boo
             return normed
         ops.add_into(out, y)
         return None
-    ops.gemm(out, x, weight, bias, accumulate, swiglu, choice=choice)     # "mid" and "own": gemm picks the kernel by shape
+    # "mid" and "own": gemm picks the kernel by shape
+    ops.gemm(out, x, weight, bias, accumulate, swiglu, choice=choice, workspace=workspace_of(ctx) if ctx.dtype == torch.bfloat16 else None)
     return None

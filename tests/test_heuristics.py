@@ -142,8 +142,10 @@ def test_the_route_of_a_product_follows_rows_dtype_and_the_runners_choices():
     # a prompt portion of a few hundred rows: too few tiles for the chip; with a long K (or up to 256 rows) this
     # package's kernel with K divided between workgroups, else the library
     if ops.compute_units() in (0, 256):
-        assert route(512, 5120, 17408, out=f32, accumulate=True, norm_follows=5120) == ("own", "")
-        assert route(512, 4096, 12288, out=f32, accumulate=True, norm_follows=4096) == ("own", "")
+        # ... whose finishing kernel also adds the residual and normalises the rows when an RMSNorm follows
+        assert route(512, 5120, 17408, out=f32, accumulate=True, norm_follows=5120) == ("split_norm", "")
+        assert route(512, 4096, 12288, out=f32, accumulate=True, norm_follows=4096) == ("split_norm", "")
+        assert route(512, 4096, 12288, out=f32, accumulate=True) == ("own", "")
         assert route(256, 7168, 5120) == ("own", "") and route(512, 7168, 5120) == ("library", "")
         assert route(512, 4096, 4096, out=f32, accumulate=True, norm_follows=4096) == ("library", "")
         assert route(512, 34816, 5120, swiglu=True) == ("library", "")

@@ -316,6 +316,40 @@ def test_gemm_of_17_to_64_rows(ops, m, n, k, waves, splits):
 
 
 @pytest.mark.parametrize("w_dtype", DTYPES)
+@pytest.mark.parametrize("m,n,k", [(512, 4096, 4096), (300, 1024, 3072), (257, 7000, 1088), (129, 512, 8192)])
+def test_product_of_many_rows_with_residual_add_and_norm_in_its_finishing_kernel(ops, w_dtype, m, n, k):
+    """residual += a w^T and the RMSNorm of the result in two kernels (K divided between workgroups or the tiles as
+    they are; the kernel that adds up the sums adds the residual and normalises), with the caller's own workspace and
+    with the one the process keeps: the same bits, and both as the plain computation."""
+    if ops.gemm_lines_splits(m, n, k) < 1:
+        pytest.skip("the divided product does not take this shape on this device")
+    g = torch.Generator().manual_seed(m + n + k)
+    a = torch.randn(m, k, generator=g).bfloat16()
+    w = (torch.randn(n, k, generator=g) / math.sqrt(k)).bfloat16()
+    res = torch.randn(m, n, generator=g)
+    nw = (1 + 0.1 * torch.randn(n, generator=g)).to(w_dtype)
+    eps = 1e-5
+    want_res = res.double() + a.double() @ w.double().T
+    want = nw.double() * want_res * torch.rsqrt(want_res.square().mean(-1, keepdim=True) + eps)
+    outs = []
+    for own in (True, False):
+        residual = dev(res.clone())
+        normed = torch.empty(m, n, device="cuda", dtype=torch.bfloat16)
+        space = torch.empty(ops.gemm_workspace_bytes() // 4, device="cuda") if own else None
+        ops.gemm_lines_add_rmsnorm(residual, dev(a), dev(w), dev(nw), eps, normed, workspace=space)
+        torch.testing.assert_close(residual.cpu().double(), want_res, rtol=1e-4, atol=1e-4)
+        close_in_norm(normed, want, rel=5e-3)
+        outs.append((residual.cpu(), normed.cpu()))
+    assert torch.equal(outs[0][0], outs[1][0]) and torch.equal(outs[0][1], outs[1][1])
+    # the same product through gemm() and the norm kernel: the residual stream bit for bit
+    residual = dev(res.clone())
+    ops.gemm(residual, dev(a), dev(w), accumulate=True)
+    assert torch.equal(residual.cpu(), outs[0][0])
+    with pytest.raises(Exception, match="workspace"):
+        ops.gemm(residual, dev(a), dev(w), accumulate=True, workspace=torch.empty(1024, device="cuda"))
+
+
+@pytest.mark.parametrize("w_dtype", DTYPES)
 @pytest.mark.parametrize("m,h,n2,k,swiglu,splits", [(17, 256, 64, 256, False, 0), (40, 512, 208, 1024, True, 2), (64, 4096, 6144, 4096, False, 0),
                                                      (100, 1024, 2048, 3328, True, 3), (128, 4096, 24576, 512, True, 0)])
 def test_gemm_of_17_to_128_rows_with_norm_taken_apart(ops, w_dtype, m, h, n2, k, swiglu, splits):
