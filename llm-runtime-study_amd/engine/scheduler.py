@@ -166,17 +166,21 @@ class BatchScheduler:
                 started = self._now()
                 logits = self.runner.step(entries)
                 tokens = self.sampler.choose(logits, [row for _, row in rows]) if rows else []
-                seconds = self._now() - started if started is not None else None
+                # reading the tokens has waited for the step; a step that samples nothing stays in flight
+                seconds = self._now(wait=False) - started if started is not None and rows else None
                 self._finish_step(rows, tokens, seconds, events)
         except BaseException:       # an interrupt from the keyboard frees everything as well
             self.abort_all()
             raise
         return events
 
-    def _now(self):
+    def _now(self, wait: bool = True):
+        """The clock for `model_seconds` (None if the scheduler was given no way to wait for the device).  wait: after
+        everything queued on the device has finished, so that the time of a step is its own."""
         if self._synchronize is None:
             return None
-        self._synchronize()
+        if wait:
+            self._synchronize()
         return time.perf_counter()
 
     def abort_all(self) -> None:
@@ -248,7 +252,7 @@ class BatchScheduler:
             chosen = self.runner.decode_steps(entries, steps, [SamplingRow(r.sampling, r.seed, r.produced) for r in running])
         else:
             chosen = self.runner.decode_steps(entries, steps)
-        seconds = (self._now() - started) / steps if started is not None else None
+        seconds = (self._now(wait=False) - started) / steps if started is not None else None     # the tokens are back: the launch has finished
         alive = running
         for tokens in chosen:
             if not alive:

@@ -28,6 +28,8 @@ from __future__ import annotations
 from dataclasses import dataclass
 from typing import Sequence
 
+import ctypes
+
 import numpy as np
 import torch
 
@@ -186,6 +188,11 @@ class ModelRunner:
         self._chosen_dev = self._chosen_host = None   # tokens chosen on the device by decode_steps()
         self._sampling_dev = self._sampling_host = None
         self._counting = np.arange(max(max_step_tokens, self.max_requests) + 1, dtype=np.int32)
+        # the staging buffer is filled by the library's host routine; False: by the Python routine it is tested against
+        self.native_prepare = True
+        self._native_layouts: dict = {}
+        self._summary = np.zeros(ops.step_prepare_summary_size(), dtype=np.int32)
+        self._table_addresses = (ctypes.c_void_p * max(len(cache.groups), 1))(*[cache.tables_with_trash_row(i).ctypes.data for i in range(len(cache.groups))])
         self.steps_run = 0
         # The weights, the cache pools and the buffers above were converted and cleared by work queued
         # on the stream that is current now.  A step on another stream waits for that work once: streams
@@ -308,9 +315,8 @@ class ModelRunner:
             if id(entry.cache) in seen:
                 raise GenerationError("a request may appear only once in a step")
             seen.add(id(entry.cache))
-            for token in entry.tokens:
-                if not 0 <= token < vocab:
-                    raise GenerationError(f"input_ids must be within vocabulary [0, {vocab})")
+            if min(entry.tokens) < 0 or max(entry.tokens) >= vocab:
+                raise GenerationError(f"input_ids must be within vocabulary [0, {vocab})")
             for place in entry.want:
                 if not 0 <= place < n:
                     raise GenerationError(f"wanted place {place} is outside the entry's {n} tokens")
@@ -331,6 +337,58 @@ class ModelRunner:
         ctx = StepContext(self)
         self._next_staging()
         self._off, self._meta_size = self._layout(max(sum(len(e.tokens) for e in entries), pad_to), max(len(entries), pad_to))
+        if self.native_prepare:
+            self._prepare_native(ctx, entries, pad_to, ahead)
+        else:
+            self._prepare_python(ctx, entries, pad_to, ahead)
+        # what kernels size their tables and choose their key splits by: an upper bound of the longest context that is
+        # the same for every step of one shape (a recorded plan holds it), the next multiple of 256
+        ctx.max_k_bound = min(-(-ctx.max_k // 256) * 256, max(cache.max_seq_len, ctx.max_k))
+        if pad_to:
+            # a graph outlives the step it is captured in: sizes that must hold for every replay are
+            # made for the longest context the cache can hold
+            ctx.max_k_bound = cache.max_seq_len
+        ctx.all_decode = ctx.max_q == 1
+        self._upload()
+        self.bind_views(ctx)
+        return ctx
+
+    def _prepare_native(self, ctx: StepContext, entries: Sequence[StepEntry], pad_to: int, ahead: int) -> None:
+        """The staging buffer filled by the library's host routine (csrc/prepare.hip) from the entries as flat arrays."""
+        count = len(entries)
+        ctx.host_slots = [entry.cache.slot for entry in entries]
+        lengths = [entry.cache.length - ahead for entry in entries]
+        ctx.host_q_lens = [len(entry.tokens) for entry in entries]
+        wants = [len(entry.want) for entry in entries]
+        if ahead and any(n != 1 for n in ctx.host_q_lens):
+            raise GenerationError("only a decode-only step can be prepared ahead of later steps")
+        flat = ctx.host_slots + lengths + ctx.host_q_lens + wants
+        for entry in entries:
+            flat += entry.tokens
+        for entry in entries:
+            flat += entry.want
+        packed = np.array(flat, dtype=np.int32)
+        tokens_at = 4 * count
+        wants_at = tokens_at + sum(ctx.host_q_lens)
+        offsets, tables = self._native_layout()
+        summary = self._summary
+        ops.step_prepare(self._host_np, offsets, count, packed, tokens_at, wants_at, pad_to, self.cache.trash_slot, tables,
+                         len(self.cache.groups), self.cache.max_blocks, self.cache.page_size, self.query_group if self._query_groups else 0, summary)
+        (ctx.T, ctx.R, ctx.num_logit_rows, ctx.num_qblocks, ctx.max_qblock, ctx.max_q, ctx.max_k, ctx.single_rows) = summary.tolist()
+        ctx.host_positions = [length - n for length, n in zip(lengths, ctx.host_q_lens)]
+
+    def _native_layout(self):
+        """The current layout's offsets in the order the host routine reads them, and the host block tables' addresses."""
+        known = self._native_layouts.get(id(self._off))
+        if known is None:
+            names = ["token_ids", "positions", "token_request", "token_slot", "logit_rows", "cu_seqlens_q", "seq_lens_k", "slot_ids",
+                     "qblock_token0", "qblock_count", "counts"] + [f"slots{i}" for i in range(len(self.cache.groups))]
+            known = self._native_layouts[id(self._off)] = np.array([self._off[name][0] for name in names], dtype=np.int64)
+        return known, self._table_addresses
+
+    def _prepare_python(self, ctx: StepContext, entries: Sequence[StepEntry], pad_to: int, ahead: int) -> None:
+        """The same in Python and numpy: the reference the host routine is tested against."""
+        cache, page = self.cache, self.cache.page_size
         ids, pos, req, rows = (self._host_view(n) for n in ("token_ids", "positions", "token_request", "logit_rows"))
         cu, lens, slots, of_token = (self._host_view(n) for n in ("cu_seqlens_q", "seq_lens_k", "slot_ids", "token_slot"))
         cursor = n_rows = 0
@@ -376,13 +434,6 @@ class ModelRunner:
         real = len(entries)
         ctx.max_q = max(ctx.host_q_lens)
         ctx.max_k = int(lens[:real].max())
-        # what kernels size their tables and choose their key splits by: an upper bound of the longest context that is
-        # the same for every step of one shape (a recorded plan holds it), the next multiple of 256
-        ctx.max_k_bound = min(-(-ctx.max_k // 256) * 256, max(self.cache.max_seq_len, ctx.max_k))
-        if pad_to:
-            # a graph outlives the step it is captured in: sizes that must hold for every replay are
-            # made for the longest context the cache can hold
-            ctx.max_k_bound = self.cache.max_seq_len
         ctx.all_decode = ctx.max_q == 1
         if pad_to > real:
             extra = pad_to - real
@@ -425,9 +476,6 @@ class ModelRunner:
             p = pos[:cursor]
             pages = cache.tables_with_trash_row(index)[of_token[:cursor], p // page]
             gslots[:cursor] = np.where(pages >= 0, pages * page + p % page, -1)
-        self._upload()
-        self.bind_views(ctx)
-        return ctx
 
     def bind_views(self, ctx: StepContext) -> None:
         """The device views of the step's arrays; steps of one shape share them (slicing is slow)."""

@@ -84,6 +84,9 @@ _SIGNATURES = {
     "lrs_silu_mul": (c_int, [c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p]),
     "lrs_add_into": (c_int, [c_void_p, c_void_p, c_int, c_int64, c_void_p]),
     "lrs_fill_i32": (c_int, [c_void_p, c_int, c_int64, c_void_p]),
+    "lrs_step_prepare": (c_int, [c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int,
+                                 c_int, c_void_p, c_int, c_int, c_int, c_void_p]),
+    "lrs_step_prepare_summary_size": (c_int, []),
     "lrs_scatter_i32": (c_int, [c_void_p, c_void_p, c_int, c_void_p]),
     "lrs_gather_rows": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p]),
     "lrs_gemm": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p,
@@ -622,6 +625,26 @@ def advance_slots(slots: torch.Tensor, positions: torch.Tensor, token_request: t
     _launch("lrs_advance_slots", _int_vector(slots, "slots", rows), _int_vector(positions, "positions", rows),
                                        _int_vector(token_request, "token_request", rows), _dev(block_table, "block_table"),
                                        block_table.stride(0), page_size, _int_vector(real_rows, "real_rows", 1), rows, _stream())
+
+
+def step_prepare_summary_size() -> int:
+    return library().lrs_step_prepare_summary_size()
+
+
+def step_prepare(meta, offsets, entries: int, packed, tokens_at: int, wants_at: int, pad_to: int, trash_slot: int, tables,
+                 groups: int, max_blocks: int, page_size: int, query_group: int, summary) -> None:
+    """Fill a step's metadata in the staging buffer `meta` (a numpy int32 view of pinned memory) on the host: see
+    csrc/prepare.hip.  `packed` (numpy int32) holds, `entries` values each, the entries' state slots, context lengths,
+    token counts and numbers of wanted places, then from `tokens_at` all tokens and from `wants_at` all wanted places;
+    `offsets` (numpy int64) where each array lies in `meta`; `tables` a ctypes array of the host block tables' addresses;
+    `summary` (numpy int32) takes T, R, logit rows, query groups, largest group, longest portion, longest context and
+    the single rows at the step's head."""
+    base = packed.ctypes.data
+    code = library().lrs_step_prepare(meta.ctypes.data, offsets.ctypes.data, entries, base, base + 4 * entries, base + 8 * entries,
+                                      base + 4 * tokens_at, base + 12 * entries, base + 4 * wants_at, pad_to, trash_slot, groups,
+                                      ctypes.cast(tables, c_void_p), max_blocks, page_size, query_group, summary.ctypes.data)
+    if code != 0:
+        raise KernelError(library().lrs_last_error().decode())
 
 
 def fill_i32(dst: torch.Tensor, value: int) -> None:

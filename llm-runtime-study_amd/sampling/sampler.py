@@ -14,6 +14,7 @@ from __future__ import annotations
 import random
 from dataclasses import dataclass
 
+import numpy as np
 import torch
 
 from ..errors import SamplingError
@@ -46,6 +47,17 @@ class Sampler:
         self.device = torch.device(device)
         self._chosen = None      # pinned host memory the kernel writes the tokens into ...
         self._chosen_address = 0  # ... and where the device sees it
+        self._settings_host = self._settings_dev = None   # the rows' sampling settings: pinned staging and its device copy
+        self._settings_cap = 0
+
+    def _settings_room(self, rows: int) -> int:
+        """Staging for `rows` rows' settings (six int32 words a row, in five arrays of `cap` rows); returns cap.  The
+        staging is written again only after the copy that last read it has finished."""
+        if self._settings_cap < rows:
+            self._settings_cap = cap = max(64, -(-rows // 4) * 4)
+            self._settings_host = torch.zeros(6 * cap, dtype=torch.int32, pin_memory=True)
+            self._settings_dev = torch.zeros(6 * cap, dtype=torch.int32, device=self.device)
+        return self._settings_cap
 
     def _result(self, rows: int) -> torch.Tensor:
         if self._chosen is None or self._chosen.numel() < rows:
@@ -71,13 +83,22 @@ class Sampler:
         if all(row.config.greedy for row in rows):
             ops.choose_tokens(out, logits, out_address=self._chosen_address)
             return self._read(out)
-        temperature = torch.tensor([row.config.temperature for row in rows], dtype=torch.float32, device=self.device)
-        seeds = torch.tensor([row.seed for row in rows], dtype=torch.int64, device=self.device)
-        counters = torch.tensor([row.counter for row in rows], dtype=torch.int32, device=self.device)
+        # temperature, top-p, top-k, draws so far and seed of every row: written into pinned memory and sent in one copy
+        # (five tensors made from Python lists would be five pageable copies, each waiting for the device)
+        n = len(rows)
+        cap = self._settings_room(n)
+        host = self._settings_host.numpy()
+        host[:cap].view(np.float32)[:n] = [row.config.temperature for row in rows]
+        host[cap:2 * cap].view(np.float32)[:n] = [row.config.top_p for row in rows]
+        host[2 * cap:3 * cap][:n] = [row.config.top_k or 0 for row in rows]
+        host[3 * cap:4 * cap][:n] = [row.counter for row in rows]
+        host[4 * cap:6 * cap].view(np.int64)[:n] = [row.seed for row in rows]
+        ops.copy_h2d(self._settings_dev, self._settings_host, 6 * cap)
+        dev = self._settings_dev
+        temperature, top_p = dev[:cap].view(torch.float32)[:n], dev[cap:2 * cap].view(torch.float32)[:n]
+        top_k, counters, seeds = dev[2 * cap:3 * cap][:n], dev[3 * cap:4 * cap][:n], dev[4 * cap:6 * cap].view(torch.int64)[:n]
         filtered = any((row.config.top_k is not None and row.config.top_k < vocab) or row.config.top_p < 1.0 for row in rows if not row.config.greedy)
         if filtered:
-            top_k = torch.tensor([row.config.top_k or 0 for row in rows], dtype=torch.int32, device=self.device)
-            top_p = torch.tensor([row.config.top_p for row in rows], dtype=torch.float32, device=self.device)
             ops.filter_logits(logits, temperature, top_k, top_p)
         ops.choose_tokens(out, logits, temperature, seeds, counters, out_address=self._chosen_address, filtered=filtered)
         return self._read(out)
