@@ -449,9 +449,17 @@ def _workspace(t: torch.Tensor | None, name: str) -> tuple:
     all callers that bring none share (their products must then stay on one stream)."""
     if t is None:
         return None, 0
+    if isinstance(t, tuple):            # (address, bytes) that workspace_address() has checked before
+        return t
     _need(t.is_cuda and t.is_contiguous() and t.numel() * t.element_size() >= gemm_workspace_bytes(),
           f"{name}: the workspace must be a contiguous device tensor of at least {gemm_workspace_bytes()} bytes")
     return t.data_ptr(), t.numel() * t.element_size()
+
+
+def workspace_address(t: torch.Tensor) -> tuple:
+    """(address, bytes) of a workspace tensor, checked once: callers that make many products a step pass this on as
+    `workspace` instead of the tensor."""
+    return _workspace(t, "workspace")
 
 
 def gemm_mid_qk_prep_takes(dtype: torch.dtype, m: int, nq: int, nkv: int, d: int, k: int, rot_half: int,

@@ -79,10 +79,16 @@ def kernels_of(ctx) -> ops.KernelChoice:
     return getattr(ctx, "kernels", None) or ops.DEFAULT_CHOICE
 
 
-def workspace_of(ctx) -> torch.Tensor:
+def workspace_of(ctx) -> tuple:
     """The step's own memory for the sums of products that divide K between workgroups (one per scratch arena, so two
     runners on two streams never share one)."""
-    return ctx.scratch("gemm_split_sums", (ops.gemm_workspace_bytes() // 4,), torch.float32)
+    memo = getattr(ctx, "memo", None)
+    known = None if memo is None else memo.get("gemm_workspace")
+    if known is None:
+        known = ops.workspace_address(ctx.scratch("gemm_split_sums", (ops.gemm_workspace_bytes() // 4,), torch.float32))
+        if memo is not None:
+            memo["gemm_workspace"] = known
+    return known
 
 
 ROUTES = ("chain", "mid_scaled", "fused_norm", "mid_begin", "mid", "split_norm", "library", "own")
