@@ -94,6 +94,34 @@ LRS_API int lrs_copy_to_pinned(void* dst_host, const void* src, int64_t bytes, v
   return lrs_check_launch("copy_to_pinned");
 }
 
+// A step's metadata from pinned host memory to the device and, in the same launch, the block table entries that
+// changed since the last step written into the device's tables: `count` (offset, value) pairs lie in the pinned buffer
+// from byte `pairs_at` on (they need not be part of what is copied); the workgroups behind those that copy read them
+// there and scatter them.  One launch where a copy and a scatter kernel would be two, each with its wait for the host.
+__global__ void copy_and_scatter_kernel(int4* __restrict__ dst, const int4* __restrict__ src, int64_t chunks, int copy_blocks,
+                                        int* __restrict__ tables, const int* __restrict__ pairs, int count) {
+  if ((int)blockIdx.x < copy_blocks) {
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < chunks; i += (int64_t)copy_blocks * blockDim.x) dst[i] = src[i];
+  } else {
+    const int i = ((int)blockIdx.x - copy_blocks) * blockDim.x + threadIdx.x;
+    if (i < count) tables[pairs[2 * i]] = pairs[2 * i + 1];
+  }
+}
+
+LRS_API int lrs_copy_h2d_scatter(void* dst, const void* src, int64_t bytes, int* tables, int64_t pairs_at, int count, void* stream) {
+  LRS_REQUIRE(bytes > 0 && bytes % 16 == 0 && (uintptr_t)dst % 16 == 0 && (uintptr_t)src % 16 == 0 && bytes <= (256 << 10),
+              "copy_h2d_scatter: %lld bytes (at most 256 KB) and both addresses must be multiples of 16", (long long)bytes);
+  LRS_REQUIRE(count > 0 && tables && pairs_at >= 0 && pairs_at % 8 == 0, "copy_h2d_scatter: needs pairs to scatter at a multiple of 8 bytes");
+  void* device_src = nullptr;
+  hipError_t err = hipHostGetDevicePointer(&device_src, const_cast<void*>(src), 0);
+  if (err != hipSuccess) return lrs_fail("hipHostGetDevicePointer: %s (is the memory pinned?)", hipGetErrorString(err));
+  const int64_t chunks = bytes / 16;
+  const int copy_blocks = (int)((chunks + 255) / 256 < 64 ? (chunks + 255) / 256 : 64);
+  copy_and_scatter_kernel<<<copy_blocks + (count + 255) / 256, 256, 0, (hipStream_t)stream>>>(
+      (int4*)dst, (const int4*)device_src, chunks, copy_blocks, tables, (const int*)((const char*)device_src + pairs_at), count);
+  return lrs_check_launch("copy_h2d_scatter");
+}
+
 LRS_API int lrs_copy_h2d(void* dst, const void* src, int64_t bytes, void* stream) {
   hipStream_t s = (hipStream_t)stream;
   if (bytes <= (256 << 10) && bytes % 16 == 0 && (uintptr_t)dst % 16 == 0 && (uintptr_t)src % 16 == 0) {

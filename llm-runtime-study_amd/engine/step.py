@@ -171,7 +171,7 @@ class ModelRunner:
         self._layouts: dict[tuple[int, int], tuple[dict, int]] = {}
         self._off, self._meta_size = self._layout(max_step_tokens, self.max_requests)
         # behind a step's arrays: the block table entries that changed since the last step, as (offset, value) pairs
-        cursor = self._meta_size + 2 * self.TABLE_PATCHES
+        cursor = self._meta_size + 2 * self.TABLE_PATCHES + 4
         self._patches = 0
         # two pinned staging buffers used in turn: a buffer is rewritten only after the copy
         # that read it has finished
@@ -283,9 +283,14 @@ class ModelRunner:
 
     def _upload(self) -> None:
         self._stage_table_patches()
-        ops.copy_h2d(self._dev, self._host, self._meta_size + 2 * self._patches)
-        if self._patches:
+        if self._patches and self._meta_size <= 65536:
+            # the same launch writes the changed block table entries, which it reads where the host put them
+            ops.copy_h2d_scatter(self._dev, self._host, self._meta_size, self.cache.device_tables, self._meta_size, self._patches)
+        elif self._patches:   # a step of tens of thousands of tokens: the runtime's copy, the pairs with it, then the scatter
+            ops.copy_h2d(self._dev, self._host, -(-(self._meta_size + 2 * self._patches) // 4) * 4)
             ops.scatter_i32(self.cache.device_tables, self._dev, self._patches, first=self._meta_size)
+        else:
+            ops.copy_h2d(self._dev, self._host, self._meta_size)
         if self.device.type == "cuda":
             event = self._copied[self._turn] or torch.cuda.Event()
             event.record()

@@ -72,6 +72,7 @@ _SIGNATURES = {
     "lrs_graph_launch": (c_int, [c_void_p, c_void_p]),
     "lrs_graph_destroy": (c_int, [c_void_p]),
     "lrs_copy_h2d": (c_int, [c_void_p, c_void_p, c_int64, c_void_p]),
+    "lrs_copy_h2d_scatter": (c_int, [c_void_p, c_void_p, c_int64, c_void_p, c_int64, c_int, c_void_p]),
     "lrs_embed": (c_int, [c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_float, c_void_p]),
     "lrs_rmsnorm": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_float, c_void_p]),
     "lrs_add_rmsnorm": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_float, c_void_p]),
@@ -332,6 +333,18 @@ def copy_h2d(dst: torch.Tensor, src: torch.Tensor, count: int) -> None:
     _need(src.device.type == "cpu" and src.is_contiguous() and dst.is_contiguous(), "copy_h2d needs a contiguous host source and a contiguous destination")
     _need(src.dtype == dst.dtype and 0 < count <= src.numel() and count <= dst.numel(), "copy_h2d: size or dtype mismatch")
     _launch("lrs_copy_h2d", _dev(dst, "dst"), src.data_ptr(), count * src.element_size(), _stream())
+
+
+def copy_h2d_scatter(dst: torch.Tensor, src: torch.Tensor, count: int, tables: torch.Tensor, pairs_at: int, pairs: int) -> None:
+    """copy_h2d() of the first `count` int32 elements (a multiple of 4) of pinned `src`, and in the same launch the `pairs`
+    (offset, value) pairs that lie in `src` from element `pairs_at` (even) on written into `tables` (int32, on the
+    device): tables.view(-1)[offset] = value.  The caller has checked the offsets."""
+    _need(src.device.type == "cpu" and src.is_contiguous() and dst.is_contiguous() and src.dtype == dst.dtype == torch.int32,
+          "copy_h2d_scatter needs contiguous int32 tensors, the source on the host")
+    _need(0 < count <= src.numel() and count <= dst.numel() and count % 4 == 0, "copy_h2d_scatter: the count must be a positive multiple of 4 inside both tensors")
+    _need(tables.dtype == torch.int32 and tables.is_contiguous() and pairs > 0 and pairs_at % 2 == 0 and pairs_at + 2 * pairs <= src.numel(),
+          "copy_h2d_scatter: int32 tables and pairs inside the source, from an even element on")
+    _launch("lrs_copy_h2d_scatter", _dev(dst, "dst"), src.data_ptr(), count * 4, _dev(tables, "tables"), pairs_at * 4, pairs, _stream())
 
 
 def stream_read(src: torch.Tensor, sink: torch.Tensor, blocks: int) -> None:
