@@ -52,6 +52,7 @@ def parse_args():
     parser.add_argument("--top-p", type=float, default=1.0, help="with --temperature: keep the likeliest tokens up to this share of the mass")
     parser.add_argument("--no-graph", action="store_true")
     parser.add_argument("--decode-steps-per-launch", type=int, default=4, help="greedy decode steps run from one graph launch (1: one step a launch)")
+    parser.add_argument("--no-launch-ahead", action="store_true", help="wait for a launch's tokens before the next launch is queued")
     parser.add_argument("--library-mid-gemm", action="store_true", help="products of 17..128 rows through the vendor library instead of this package's kernel for them")
     parser.add_argument("--own-gemm", action="store_true", help="this package's kernel also for products of many rows (default: vendor library)")
     return parser.parse_args()
@@ -69,6 +70,11 @@ def decode_lead(batch: int, context: int, step_tokens: int) -> int:
     return (batch - 1) * -(-context // step_tokens)
 
 
+def warmup_room(warmup: int, per_launch: int) -> int:
+    """Most decode steps the warm-up of measure_decode() takes (its rounds go on until no new graph is captured)."""
+    return 6 * (-(-max(warmup, 1) // per_launch) * per_launch + 2 * per_launch) + per_launch
+
+
 def measure_decode(engine, batch: int, context: int, steps: int, warmup: int, seed: int, sampling=None):
     """Prefill `batch` prompts of `context` random tokens through the scheduler, then time `steps`
     decode steps.  Returns (seconds per step list, mean context length over the timed steps)."""
@@ -84,7 +90,7 @@ def measure_decode(engine, batch: int, context: int, steps: int, warmup: int, se
     lead = decode_lead(batch, context, engine.max_num_batched_tokens)
     for _ in range(batch):
         scheduler.add_request(rng.integers(0, vocab, context).tolist(),
-                              max_new_tokens=warmup + steps + lead + batch + 8 + 2 * scheduler.decode_steps_per_launch,
+                              max_new_tokens=steps + lead + batch + 8 + warmup_room(warmup, scheduler.decode_steps_per_launch),
                               sampling=sampling if sampling is not None else SamplingConfig())
     times = []
     with torch.cuda.device(engine.device), torch.cuda.stream(engine.stream):
@@ -92,32 +98,50 @@ def measure_decode(engine, batch: int, context: int, steps: int, warmup: int, se
         produced = 0
         while produced < batch:
             produced += sum(1 for _, e in scheduler.step() if e.prompt_token_count is not None)
-        # one call of the scheduler may hold several decode steps (one graph launch): count steps, not calls
-        per_launch = scheduler.decode_steps_per_launch
+        # one call of the scheduler may hold several decode steps (one graph launch): count steps, not calls.  With
+        # launches queued ahead a call returns the tokens of the launch queued by the call before it, and queues the next:
+        # the settings below are changed so that exactly `count` steps run, none queued when the last call returns.
+        per_launch, ahead = scheduler.decode_steps_per_launch, scheduler.launch_ahead
+        runner = engine.runner
 
         def run(count: int, record: bool) -> None:
             done = 0
             while done < count:
-                scheduler.decode_steps_per_launch = min(per_launch, count - done)
+                if scheduler.steps_in_flight == 0:     # this call queues a launch and, ahead, one of the same size behind it
+                    scheduler.launch_ahead = ahead and count - done >= 2 * per_launch
+                    scheduler.decode_steps_per_launch = min(per_launch, count - done)
+                else:                                  # this call queues what may still be queued behind the launch in flight
+                    left = count - done - scheduler.steps_in_flight
+                    scheduler.launch_ahead = ahead and left > 0
+                    scheduler.decode_steps_per_launch = max(1, min(per_launch, left))
                 started = time.perf_counter()
                 events = scheduler.step()
-                engine.synchronize()
-                elapsed = time.perf_counter() - started
+                elapsed = time.perf_counter() - started                # the call returns when its launch's tokens are there
                 assert len(events) % batch == 0 and len(events) > 0
                 held = len(events) // batch
                 if record:
                     times.extend([elapsed / held] * held)
                 done += held
+            assert done == count and scheduler.steps_in_flight == 0
+            scheduler.launch_ahead, scheduler.decode_steps_per_launch = ahead, per_launch
 
-        # warm-up: at least `warmup` steps, in whole launches, and one launch of every size the timed
-        # steps will use (a graph is captured at the first launch of its size)
-        warmed = -(-max(warmup, 1) // per_launch) * per_launch
-        run(warmed, False)
+        # warm-up: at least `warmup` steps, in whole launches, until a round of launches captures no new graph (a launch
+        # that follows another, and each of the two result buffers, has a graph of its own), and one launch of every
+        # size the timed steps will use
+        warmed = 0
+        for _ in range(6):
+            captured = runner.graph_captures
+            rounds = -(-max(warmup, 1) // per_launch) * per_launch + (2 * per_launch if ahead else 0)
+            run(rounds, False)
+            warmed += rounds
+            if runner.graph_captures == captured:
+                break
         if steps % per_launch:
             run(steps % per_launch, False)
             warmed += steps % per_launch
         engine.synchronize()
         run(steps, True)
+        engine.synchronize()
         assert len(times) == steps
         scheduler.abort_all()
     # requests finished their prompts `portions` steps apart, so they are up to `lead` tokens apart in length
@@ -170,7 +194,8 @@ def main() -> int:
     raw = dict(SHAPES[args.shape], num_hidden_layers=args.layers)
     config = config_from_dict(raw)
     max_batch = args.batch if args.no_points else max(args.batch, 64)
-    needed = args.context + args.steps + args.warmup + decode_lead(max_batch, args.context, max(2048, args.prefill_tokens)) + max_batch + 64
+    needed = (args.context + args.steps + warmup_room(args.warmup, max(args.decode_steps_per_launch, 1))
+              + decode_lead(max_batch, args.context, max(2048, args.prefill_tokens)) + max_batch + 64)
     needed = max(needed, args.prefill_tokens + 1)
     max_seq_len = max(needed, BENCHMARK_CONTEXT) if args.max_seq_len is None else args.max_seq_len
     if max_seq_len < needed:
@@ -181,7 +206,7 @@ def main() -> int:
     engine = Engine.from_config(config, seed=0, dtype=args.dtype, max_seq_len=max_seq_len, max_batch_size=max_batch,
                                 max_num_batched_tokens=max(2048, args.prefill_tokens), use_cuda_graph=not args.no_graph, num_pages=args.num_pages,
                                 kernels=KernelChoice(library=not args.own_gemm, mid=not args.library_mid_gemm),
-                                decode_steps_per_launch=args.decode_steps_per_launch)
+                                decode_steps_per_launch=args.decode_steps_per_launch, launch_ahead=not args.no_launch_ahead)
     dtype_name = "bf16" if args.dtype == "bfloat16" else "fp32"
 
     prefill = prefill_entry(engine, args.prefill_tokens, dtype_name, seed=1)

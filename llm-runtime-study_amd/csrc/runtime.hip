@@ -109,8 +109,8 @@ __global__ void copy_and_scatter_kernel(int4* __restrict__ dst, const int4* __re
 }
 
 LRS_API int lrs_copy_h2d_scatter(void* dst, const void* src, int64_t bytes, int* tables, int64_t pairs_at, int count, void* stream) {
-  LRS_REQUIRE(bytes > 0 && bytes % 16 == 0 && (uintptr_t)dst % 16 == 0 && (uintptr_t)src % 16 == 0 && bytes <= (256 << 10),
-              "copy_h2d_scatter: %lld bytes (at most 256 KB) and both addresses must be multiples of 16", (long long)bytes);
+  LRS_REQUIRE(bytes >= 0 && bytes % 16 == 0 && (uintptr_t)dst % 16 == 0 && (uintptr_t)src % 16 == 0 && bytes <= (256 << 10),
+              "copy_h2d_scatter: %lld bytes (at most 256 KB; 0: nothing is copied) and both addresses must be multiples of 16", (long long)bytes);
   LRS_REQUIRE(count > 0 && tables && pairs_at >= 0 && pairs_at % 8 == 0, "copy_h2d_scatter: needs pairs to scatter at a multiple of 8 bytes");
   void* device_src = nullptr;
   hipError_t err = hipHostGetDevicePointer(&device_src, const_cast<void*>(src), 0);

@@ -33,7 +33,7 @@ class Engine:
                  cache_backend: str = "paged", use_cuda_graph: bool = True, page_size: int = DEFAULT_PAGE_SIZE,
                  max_num_batched_tokens: int | None = None, num_pages: int | None = None, tokenizer=None,
                  load_seconds: float = 0.0, library_gemm: bool = True, decode_steps_per_launch: int = 4, kernels=None,
-                 use_launch_plans: bool = True):
+                 use_launch_plans: bool = True, launch_ahead: bool = True):
         if max_batch_size <= 0:
             raise EngineError("max_batch_size must be positive")
         if cache_backend != "paged":
@@ -53,6 +53,8 @@ class Engine:
         self.library_gemm = library_gemm if kernels is None else kernels.library
         # steps outside graphs are recorded once per shape and made again from the record (see engine/step.py)
         self.use_launch_plans = use_launch_plans
+        # decode launches are queued one ahead: the device never waits for the host between them (see BatchScheduler)
+        self.launch_ahead = launch_ahead
         self.tokenizer = tokenizer
         self.load_seconds = load_seconds
         self.quantization = "dense"
@@ -129,7 +131,7 @@ class Engine:
             self.runner, self._sampler, max_batch_size=self.max_batch_size, max_seq_len=self.max_seq_len,
             max_step_tokens=self.max_num_batched_tokens, eos_token_ids=() if ignore_eos else self.config.eos_token_ids,
             vocab_size=self.config.vocab_size, tokenizer=self.tokenizer, synchronize=self.synchronize,
-            decode_steps_per_launch=self.decode_steps_per_launch if self.use_cuda_graph else 1)
+            decode_steps_per_launch=self.decode_steps_per_launch if self.use_cuda_graph else 1, launch_ahead=self.launch_ahead)
 
     def generate(self, message_batches: Sequence, *, max_new_tokens: int, sampling: SamplingConfig = SamplingConfig(),
                  enable_thinking: bool = False, ignore_eos: bool = False) -> Iterator[tuple[int, GenerationEvent]]:

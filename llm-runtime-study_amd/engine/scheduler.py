@@ -78,7 +78,7 @@ class _Running:
 class BatchScheduler:
     def __init__(self, runner, sampler, *, max_batch_size: int, max_seq_len: int, max_step_tokens: int,
                  eos_token_ids: Sequence[int] = (), vocab_size: int | None = None, tokenizer=None,
-                 synchronize: Callable[[], None] | None = None, decode_steps_per_launch: int = 1):
+                 synchronize: Callable[[], None] | None = None, decode_steps_per_launch: int = 1, launch_ahead: bool = False):
         if max_batch_size <= 0:
             raise GenerationError("max_batch_size must be positive")
         if max_seq_len <= 0 or max_seq_len > runner.cache.max_seq_len:
@@ -100,6 +100,15 @@ class BatchScheduler:
         # produced after its end-of-sequence token are dropped; a waiting request is admitted up
         # to that many steps later than it could have been.
         self.decode_steps_per_launch = decode_steps_per_launch
+        # launch_ahead: while every running request decodes, the next launch of decode steps is queued before the tokens
+        # of the one before are read, so the device goes from launch to launch without waiting for the host (which
+        # reads tokens, finishes requests and streams text meanwhile).  The tokens of a launch then come out of the
+        # step() call after the one that queued it.  A request that ends in a launch (its end-of-sequence token) has
+        # run on in the launch queued behind it; those tokens are dropped like the ones after an end-of-sequence
+        # token inside one launch, and a waiting request is admitted that much later.
+        self.launch_ahead = launch_ahead and decode_steps_per_launch > 1 and hasattr(runner, "decode_launch_begin")
+        self._in_flight = None          # (launch, the requests of its rows, when it was queued)
+        self._collected_at = 0.0
         self._ids = itertools.count()
         self._waiting: deque[_Waiting] = deque()
         self._running: list[_Running] = []
@@ -144,6 +153,11 @@ class BatchScheduler:
         return bool(self._waiting or self._running)
 
     @property
+    def steps_in_flight(self) -> int:
+        """Decode steps of the launch that has been queued and whose tokens the next step() call returns (0: none)."""
+        return 0 if self._in_flight is None else self._in_flight[0].steps
+
+    @property
     def num_waiting(self) -> int:
         return len(self._waiting)
 
@@ -156,8 +170,15 @@ class BatchScheduler:
         """Admit, run one mixed batch, sample; returns (request index, event) pairs."""
         events: list[tuple[int, GenerationEvent]] = []
         try:
+            if self._in_flight is not None:
+                self._collect(events)
+                return events
             self._admit(events)
             steps = self._decode_steps_ahead()
+            if steps > 1 and self.launch_ahead:
+                self._queue_launch(steps, None)
+                self._collect(events)
+                return events
             if steps > 1:
                 self._decode_several(steps, events)
                 return events
@@ -174,6 +195,64 @@ class BatchScheduler:
             raise
         return events
 
+    # ------------------------------------------------------ launches queued ahead
+    def _queue_launch(self, steps: int, after) -> None:
+        """Queue a launch of decode steps of every running request; `after`: (launch, requests, ...) it follows directly."""
+        running = list(self._running) if after is None else after[1]
+        entries = [StepEntry(r.cache, [r.next_token if r.next_token is not None else 0], [0]) for r in running]
+        rows = [SamplingRow(r.sampling, r.seed, r.produced) for r in running] if after is None else None
+        if after is not None and after[0].sampled:
+            rows = [SamplingRow(r.sampling, r.seed, r.produced + after[0].steps) for r in running]
+        launch = self.runner.decode_launch_begin(entries, steps, rows, after=None if after is None else after[0])
+        self._in_flight = (launch, running, time.perf_counter())
+
+    def _collect(self, events) -> None:
+        """The tokens of the launch in flight.  Before they are waited for, the launch after it is queued if no
+        request can reach its length limit inside the one in flight and nothing waits that could be admitted now."""
+        launch, running, queued_at = self._in_flight
+        following = None
+        still = {id(r) for r in self._running}
+        left = min(r.output_limit - r.produced for r in running) - launch.steps
+        # (a launch can only be followed by one of the same requests: once one of them has ended, the launch in flight
+        # is the last of its chain, and the next step starts anew with those that are left)
+        if self.launch_ahead and left >= 1 and all(id(r) in still for r in running) and not self._could_admit():
+            self._queue_launch(min(self.decode_steps_per_launch, left), self._in_flight)
+            following = self._in_flight
+        self._in_flight = None
+        try:
+            chosen = self.runner.decode_launch_end(launch)
+        except BaseException:
+            if following is not None:
+                self.runner.decode_launch_drop(following[0])
+            raise
+        now = time.perf_counter()
+        seconds = (now - max(queued_at, self._collected_at)) / launch.steps if self._synchronize is not None else None
+        self._collected_at = now                                 # a launch queued behind another began when that one's tokens were due
+        alive = [r for r in running if id(r) in still]           # a request that ended in the launch before is not looked at again
+        for tokens in chosen:
+            if not alive:
+                break
+            by_request = dict(zip(map(id, running), tokens))
+            self.step_log.append([(r.index, 1) for r in alive])
+            self._finish_step([(r, None) for r in alive], [by_request[id(r)] for r in alive], seconds, events)
+            still = {id(r) for r in self._running}
+            alive = [r for r in alive if id(r) in still]
+        if following is not None:
+            if alive:
+                self._in_flight = following
+            else:
+                self.runner.decode_launch_drop(following[0])     # every one of its requests has ended: nobody wants its tokens
+
+    def _could_admit(self) -> bool:
+        """Whether the head of the queue could be admitted right now (then decoding pauses for a step that takes it in)."""
+        if not self._waiting:
+            return False
+        head = self._waiting[0]
+        if head.output_limit == 0:
+            return True
+        lifetime = len(head.prompt) + head.output_limit
+        return len(self._running) < self.max_batch_size and self.cache.can_admit(lifetime, self.max_step_tokens)
+
     def _now(self, wait: bool = True):
         """The clock for `model_seconds` (None if the scheduler was given no way to wait for the device).  wait: after
         everything queued on the device has finished, so that the time of a step is its own."""
@@ -185,6 +264,9 @@ class BatchScheduler:
 
     def abort_all(self) -> None:
         """Release every running request's cache and drop every waiting request."""
+        in_flight, self._in_flight = self._in_flight, None
+        if in_flight is not None:
+            self.runner.decode_launch_drop(in_flight[0])
         running, self._running = self._running, []
         self._waiting.clear()
         for request in running:

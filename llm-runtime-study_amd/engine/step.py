@@ -99,6 +99,22 @@ class RecordedStep:
     graph: int | None = None             # the plan captured in a HIP graph, once the shape has come back often enough
 
 
+@dataclass
+class DecodeLaunch:
+    """Decode steps that have been queued and not yet waited for (ModelRunner.decode_launch_begin)."""
+
+    entries: list
+    steps: int
+    bucket: int
+    before: list                         # the caches' lengths before the launch
+    ctx: "StepContext"
+    sampled: bool
+    parity: int                          # which of the two result buffers its tokens go to
+    done: object                         # an event recorded behind the launch
+    serial: int
+    ended: bool = False
+
+
 class StepContext:
     """What the parts see of one step."""
 
@@ -185,7 +201,8 @@ class ModelRunner:
         self._host_np = self._host.numpy()
         self._dev = torch.zeros(cursor, dtype=torch.int32, device=self.device)
         self._views: dict[tuple, tuple] = {}
-        self._chosen_dev = self._chosen_host = None   # tokens chosen on the device by decode_steps()
+        self._chosen_devs = self._chosen_hosts = None   # tokens chosen on the device by decode_steps(): two sets, for launches that follow each other
+        self._launch_serial = 0     # counts everything that writes the device's step metadata
         self._sampling_dev = self._sampling_host = None
         self._counting = np.arange(max(max_step_tokens, self.max_requests) + 1, dtype=np.int32)
         # the staging buffer is filled by the library's host routine; False: by the Python routine it is tested against
@@ -291,6 +308,10 @@ class ModelRunner:
             ops.scatter_i32(self.cache.device_tables, self._dev, self._patches, first=self._meta_size)
         else:
             ops.copy_h2d(self._dev, self._host, self._meta_size)
+        self._launch_serial += 1          # the device's step metadata is another step's now
+        self._mark_copied()
+
+    def _mark_copied(self) -> None:
         if self.device.type == "cuda":
             event = self._copied[self._turn] or torch.cuda.Event()
             event.record()
@@ -654,6 +675,86 @@ class ModelRunner:
         self.steps_run += steps
         return chosen
 
+    # ------------------------------------------ launches that follow each other without the host between them
+    def decode_launch_begin(self, entries: Sequence[StepEntry], steps: int, sampling: Sequence | None = None,
+                            after: "DecodeLaunch | None" = None) -> "DecodeLaunch":
+        """Queue up to `steps` decode steps of `entries` (as decode_steps() would run them) and return at once;
+        decode_launch_end() waits for them and gives their tokens.
+
+        after: the launch that was begun last, with the same requests in the same order and not yet ended: this one
+        then follows it directly.  Its first tokens are the ones the device chose last (the entries' own tokens are
+        not read), and the host sends nothing but the block table entries of the new pages, so the device goes from
+        one launch to the next without waiting for the host.  A launch ends at the edge of a length class like those
+        of decode_steps(): `launch.steps` says how many steps it holds."""
+        if not 1 <= steps <= self.MAX_DECODE_STEPS:
+            raise GenerationError(f"a launch takes 1..{self.MAX_DECODE_STEPS} decode steps, got {steps}")
+        if after is None:
+            self.validate(entries)
+        elif after.serial != self._launch_serial or len(entries) != len(after.entries) or any(
+                mine.cache is not theirs.cache for mine, theirs in zip(entries, after.entries)):
+            raise GenerationError("a launch can only follow the launch begun last (no other step since), with the same requests in the same order")
+        self._follow_construction()
+        bucket = self._graph_bucket(entries)
+        if not bucket:
+            raise GenerationError("decode launches need graphs and one token per entry")
+        if sampling is not None and len(sampling) != len(entries):
+            raise GenerationError("decode launches need one sampling row per entry")
+        longest = max(entry.cache.length for entry in entries) + 1         # the longest context of the launch's first step
+        reach = length_class(longest)
+        count = min(steps, (2 * reach if reach else 256) - longest)
+        before = [entry.cache.length for entry in entries]
+        extended = []
+        try:
+            for entry in entries:
+                self.cache.extend(entry.cache, count)
+                extended.append(entry)
+            sampled = sampling is not None and any(not row.config.greedy for row in sampling)
+            if after is None:
+                ctx = self.prepare(entries, pad_to=bucket, ahead=count - 1)
+                if sampled:
+                    self._upload_sampling(sampling)
+                parity = 0
+            else:
+                # the device holds the step's metadata, moved on by the launch before; only new pages are news to it
+                if sampled != after.sampled:
+                    raise GenerationError("a launch that follows another samples as that one does")
+                ctx, parity = after.ctx, after.parity ^ 1
+                ctx.max_k = longest
+                self._next_staging()
+                self._stage_table_patches()
+                if self._patches:
+                    ops.copy_h2d_scatter(self._dev, self._host, 0, self.cache.device_tables, self._meta_size, self._patches)
+                    self._mark_copied()
+            self._launch_decode_graph(ctx, bucket, count, sampled, parity, goes_on=True, follows=after is not None)
+        except BaseException:
+            for entry, length in zip(extended, before):
+                if not entry.cache.released:
+                    self.cache.rollback(entry.cache, length)
+            raise
+        self._launch_serial += 1
+        done = torch.cuda.Event()
+        done.record()
+        return DecodeLaunch(list(entries), count, bucket, before, ctx, sampled, parity, done, self._launch_serial)
+
+    def decode_launch_end(self, launch: "DecodeLaunch") -> list[list[int]]:
+        """Wait for a launch and return its tokens [steps][entries] (a row whose logits were not finite raises)."""
+        if launch.ended:
+            raise GenerationError("this launch has been ended before")
+        launch.ended = True
+        launch.done.synchronize()
+        chosen = self._read_chosen(launch.bucket, launch.steps, len(launch.entries), launch.parity)
+        for entry in launch.entries:
+            if not entry.cache.released:
+                self.cache.trim(entry.cache)
+        self.steps_run += launch.steps
+        return [row[:len(launch.entries)] for row in chosen]
+
+    def decode_launch_drop(self, launch: "DecodeLaunch") -> None:
+        """Wait for a launch whose tokens nobody wants any more (its requests are being given up)."""
+        if not launch.ended:
+            launch.ended = True
+            launch.done.synchronize()
+
     def _decode_launch(self, entries: Sequence[StepEntry], steps: int, sampling: Sequence | None, bucket: int) -> list[list[int]]:
         """One graph launch of `steps` decode steps.  Every cache is lengthened by all `steps` positions
         first, so the block tables that the launch uploads already hold the pages of the later ones."""
@@ -689,23 +790,38 @@ class ModelRunner:
                 dev[3 * cap:4 * cap][:rows], dev[4 * cap:6 * cap].view(torch.int64)[:rows])
 
     def _run_decode_graph(self, ctx: StepContext, bucket: int, steps: int, sampled: bool = False, real: int | None = None) -> list[list[int]]:
-        real = bucket if real is None else real
-        key = (bucket, length_class(ctx.max_k), steps, sampled)
-        if self._chosen_dev is None:
+        self._launch_decode_graph(ctx, bucket, steps, sampled)
+        torch.cuda.current_stream(self.device).synchronize()
+        return self._read_chosen(bucket, steps, bucket if real is None else real)
+
+    def _read_chosen(self, bucket: int, steps: int, real: int, parity: int = 0) -> list[list[int]]:
+        stride = -(-self.max_requests // 4) * 4
+        host = self._chosen_hosts[parity]
+        chosen = [host[i * stride:i * stride + bucket].tolist() for i in range(steps)]
+        for row in chosen:
+            refuse_not_finite(row[:real])       # a row whose logits were not finite (rows that pad the batch are not looked at)
+        return chosen
+
+    def _launch_decode_graph(self, ctx: StepContext, bucket: int, steps: int, sampled: bool = False, parity: int = 0, goes_on: bool = False,
+                             follows: bool = False) -> None:
+        """Queue `steps` decode steps of the prepared batch: a replay of their graph, or, the first time, an eager run
+        that is captured on the way.  Nothing is waited for."""
+        key = (bucket, length_class(ctx.max_k), steps, sampled) + ((parity, follows) if goes_on else ())
+        if self._chosen_devs is None:
             rows = self.MAX_DECODE_STEPS * (-(-self.max_requests // 4) * 4)
-            self._chosen_dev = torch.zeros(rows, dtype=torch.int32, device=self.device)
-            self._chosen_host = torch.zeros(rows, dtype=torch.int32, pin_memory=True)
+            self._chosen_devs = [torch.zeros(rows, dtype=torch.int32, device=self.device) for _ in range(2)]
+            self._chosen_hosts = [torch.zeros(rows, dtype=torch.int32, pin_memory=True) for _ in range(2)]
         stride = -(-self.max_requests // 4) * 4                    # rows of 16 bytes and more
         graph = self._graphs.get(key)
         if graph is None or graph[1] != self.arena.generation:
             if graph is not None:
                 ops.graph_destroy(graph[0])
                 del self._graphs[key]
-            self._decode_steps_on_stream(ctx, steps, stride, sampled)   # an eager run first: it sizes every scratch buffer
+            self._decode_steps_on_stream(ctx, steps, stride, sampled, parity, goes_on, follows)   # an eager run first: it sizes every scratch buffer
             generation = self.arena.generation
             ops.graph_begin()
             try:
-                self._decode_steps_on_stream(ctx, steps, stride, sampled)
+                self._decode_steps_on_stream(ctx, steps, stride, sampled, parity, goes_on, follows)
             finally:
                 handle = ops.graph_end()
             if self.arena.generation != generation:
@@ -719,31 +835,37 @@ class ModelRunner:
         else:
             ops.graph_launch(graph[0])
             self.graph_replays += 1
-        torch.cuda.current_stream(self.device).synchronize()
-        chosen = [self._chosen_host[i * stride:i * stride + bucket].tolist() for i in range(steps)]
-        for row in chosen:
-            refuse_not_finite(row[:real])       # a row whose logits were not finite (rows that pad the batch are not looked at)
-        return chosen
 
-    def _decode_steps_on_stream(self, ctx: StepContext, steps: int, stride: int, sampled: bool) -> None:
+    def _decode_steps_on_stream(self, ctx: StepContext, steps: int, stride: int, sampled: bool, parity: int = 0, goes_on: bool = False,
+                                follows: bool = False) -> None:
+        """goes_on: tokens, positions and lengths are moved on after the last step as well, so that a launch that follows
+        this one directly finds its first step's on the device.  follows: this launch is such a one: it begins by
+        looking up the cache slots of its first positions, which may lie in pages that the host took for it only
+        after the launch before had been queued (their table entries arrive between the two).  parity: which of
+        the two result buffers the tokens go to (launches that follow each other take them in turn)."""
         draws = None
+        chosen_dev, chosen_host = self._chosen_devs[parity], self._chosen_hosts[parity]
         if sampled:
             temperature, top_p, top_k, draws, seeds = self._sampling_views(ctx.T)
+        if follows:
+            for group in ctx._groups:
+                ops.advance_slots(group.slots, ctx.positions, ctx.token_slot, group.block_table, group.page_size, ctx.counts)
         for i in range(steps):
             ctx.memo.clear()                                       # position tables are made again for the new positions
             h = self.model.forward_hidden(ctx)
             logits = self.model.logits(ctx, h)
-            chosen = self._chosen_dev[i * stride:i * stride + ctx.T]
+            chosen = chosen_dev[i * stride:i * stride + ctx.T]
             if sampled:
                 ops.filter_logits(logits, temperature, top_k, top_p)
                 ops.choose_tokens(chosen, logits, temperature, seeds, draws, filtered=True)
             else:
                 ops.choose_tokens(chosen, logits)
-            if i + 1 < steps:
+            if i + 1 < steps or goes_on:
                 ops.advance_decode(ctx.token_ids, ctx.positions, ctx.token_request, ctx.seq_lens_k, chosen, ctx.counts, draws)
+            if i + 1 < steps:
                 for group in ctx._groups:
                     ops.advance_slots(group.slots, ctx.positions, ctx.token_slot, group.block_table, group.page_size, ctx.counts)
-        ops.copy_to_pinned(self._chosen_host, self._chosen_dev, steps * stride)
+        ops.copy_to_pinned(chosen_host, chosen_dev, steps * stride)
 
     # ------------------------------------------------------------------ graphs
     GRAPH_BUCKETS = (1, 2, 4, 8, 16, 32, 48, 64, 96, 128)

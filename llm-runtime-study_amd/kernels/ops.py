@@ -341,7 +341,7 @@ def copy_h2d_scatter(dst: torch.Tensor, src: torch.Tensor, count: int, tables: t
     device): tables.view(-1)[offset] = value.  The caller has checked the offsets."""
     _need(src.device.type == "cpu" and src.is_contiguous() and dst.is_contiguous() and src.dtype == dst.dtype == torch.int32,
           "copy_h2d_scatter needs contiguous int32 tensors, the source on the host")
-    _need(0 < count <= src.numel() and count <= dst.numel() and count % 4 == 0, "copy_h2d_scatter: the count must be a positive multiple of 4 inside both tensors")
+    _need(0 <= count <= src.numel() and count <= dst.numel() and count % 4 == 0, "copy_h2d_scatter: the count must be a multiple of 4 inside both tensors (0: only the pairs)")
     _need(tables.dtype == torch.int32 and tables.is_contiguous() and pairs > 0 and pairs_at % 2 == 0 and pairs_at + 2 * pairs <= src.numel(),
           "copy_h2d_scatter: int32 tables and pairs inside the source, from an even element on")
     _launch("lrs_copy_h2d_scatter", _dev(dst, "dst"), src.data_ptr(), count * 4, _dev(tables, "tables"), pairs_at * 4, pairs, _stream())

@@ -286,3 +286,109 @@ def test_several_decode_steps_need_greedy_requests_and_room():
     assert runner.launches == [(2, [0, 1])]
     (first, second), = runner.sampling_seen
     assert first == (0.7, 11, 1) and second[0] == 0.0 and second[2] == 1
+
+
+class QueuedLaunchRunner(SeveralStepsRunner):
+    """A fake step function whose launches of decode steps can be queued and waited for later, as the real one's: a
+    launch that follows another takes its first tokens from that one (the entries' own are not read), and only the
+    launch begun last can be followed."""
+
+    def __init__(self, *args, **kwargs):
+        super().__init__(*args, **kwargs)
+        self.begun, self.ended, self.dropped, self.serial, self.open = [], [], [], 0, 0
+        self.decode_steps_sample = True
+
+    def step(self, entries):
+        assert self.open == 0, "a step ran while a launch was in flight"
+        self.serial += 1
+        return super().step(entries)
+
+    def decode_launch_begin(self, entries, steps, sampling=None, after=None):
+        if after is not None:
+            assert after["serial"] == self.serial and [e.cache for e in entries] == [e.cache for e in after["entries"]]
+        for e in entries:
+            self.cache.extend(e.cache, steps)          # a released cache would refuse
+        self.serial += 1
+        self.open += 1
+        launch = {"entries": list(entries), "steps": steps, "serial": self.serial, "follows": after is not None, "sampled": False}
+        launch = type("Launch", (), launch)() if False else _Launch(launch)
+        self.begun.append((steps, [e.cache.request_id for e in entries], after is not None))
+        return launch
+
+    def decode_launch_end(self, launch):
+        self.open -= 1
+        self.ended.append(launch.serial)
+        chosen = []
+        for _ in range(launch.steps):
+            row = []
+            for e in launch.entries:
+                k = self.produced.get(e.cache.request_id, 0)
+                self.produced[e.cache.request_id] = k + 1
+                script = self.script[e.cache.request_id]
+                row.append(script[k] if k < len(script) else 0)
+            chosen.append(row)
+        self.cache.check_invariants()
+        return chosen
+
+    def decode_launch_drop(self, launch):
+        self.open -= 1
+        self.dropped.append(launch.serial)
+
+
+class _Launch(dict):
+    __getattr__ = dict.__getitem__
+
+
+def test_launches_queued_ahead_give_the_same_events_and_end_their_chain_when_a_request_ends():
+    # request 1 meets its end-of-sequence token as its sixth token, inside the second launch
+    script = {0: list(range(10, 40)), 1: [20, 21, 22, 23, 24, 1] + [9] * 30}
+
+    def run(ahead):
+        runner = QueuedLaunchRunner(script)
+        s = scheduler(runner, decode_steps_per_launch=4, launch_ahead=ahead)
+        s.add_request([3, 4, 5], max_new_tokens=18)
+        s.add_request([6, 2], max_new_tokens=18)
+        events = [(i, e.token_id, e.token_index, e.finish_reason) for i, e in drain(s)]
+        assert runner.cache.active_requests == 0 and runner.cache.used_pages() == 0 and runner.open == 0
+        return events, runner, s
+
+    plain, _, log_plain = run(False)
+    ahead, runner, log_ahead = run(True)
+    assert sorted(plain) == sorted(ahead) and log_plain.step_log == log_ahead.step_log
+    assert [t for i, t, _, _ in ahead if i == 1] == [20, 21, 22, 23, 24, 1]
+    # Both requests have sampled once when the launches begin.  The first (tokens 2..5) is followed at once by a second
+    # (6..9) and, when the first is read, a third (10..13) behind the second.  Request 1 ends in the second; the third,
+    # already queued with it, is the last of its chain, and request 1's rows of it are dropped.  Request 0 (13 tokens
+    # so far, 5 to go) goes on alone: a launch of 4 and, behind it, one of the single token that is left.
+    assert runner.begun == [(4, [0, 1], False), (4, [0, 1], True), (4, [0, 1], True), (4, [0], False), (1, [0], True)]
+    assert runner.dropped == [] and len(runner.ended) == 5
+    assert [t for i, t, _, _ in ahead if i == 0] == list(range(10, 28))
+
+
+def test_launches_are_not_queued_ahead_past_a_length_limit_or_while_a_request_could_be_admitted():
+    script = {0: list(range(10, 40)), 1: list(range(40, 70)), 2: [7] * 10}
+    runner = QueuedLaunchRunner(script, num_pages=40)
+    s = scheduler(runner, decode_steps_per_launch=4, launch_ahead=True, max_batch_size=2)
+    s.add_request([3, 4], max_new_tokens=7)            # six tokens after the first: a launch of 4, then 2 are left
+    s.add_request([5, 6], max_new_tokens=30)
+    s.add_request([8, 9], max_new_tokens=3)            # waits for a slot
+    events = drain(s)
+    # the launch of 4 is followed by one of 2 (what request 0 has left); when request 0 ends, the waiting request
+    # could be admitted, so nothing is queued behind the launch in flight and the next step takes it in
+    assert runner.begun[:2] == [(4, [0, 1], False), (2, [0, 1], True)]
+    assert all(not follows for _, ids, follows in runner.begun[2:3])
+    assert {i for i, _ in events} == {0, 1, 2} and runner.open == 0 and runner.cache.used_pages() == 0
+    assert [e.token_id for i, e in events if i == 2] == [7, 7, 7]
+
+
+def test_a_launch_in_flight_is_waited_for_when_everything_is_given_up():
+    script = {0: list(range(10, 40)), 1: list(range(40, 70))}
+    runner = QueuedLaunchRunner(script)
+    s = scheduler(runner, decode_steps_per_launch=4, launch_ahead=True)
+    s.add_request([3, 4], max_new_tokens=20)
+    s.add_request([5, 6], max_new_tokens=20)
+    while not runner.begun:
+        s.step()
+    assert runner.open == 1                              # one launch has been read, the one behind it is in flight
+    s.abort_all()
+    assert runner.open == 0 and len(runner.dropped) == 1 and runner.cache.used_pages() == 0 and not s.has_unfinished

@@ -362,6 +362,93 @@ def test_one_layer_at_the_benchmark_sizes_against_the_plain_implementation(sizes
     assert want.abs().max() > 1.0
 
 
+# ------------------------------------------- launches that follow each other
+@pytest.mark.parametrize("sampled", [False, True], ids=["greedy", "drawn"])
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_launches_that_follow_each_other_give_the_tokens_of_single_steps(tmp_path, dtype, sampled):
+    """Launches of decode steps queued one behind the other, each begun before the one before is read (the device
+    feeds itself, the host sends only new pages' table entries), against decode_steps() one launch at a time: the
+    same tokens, across page edges and the edge of a length class (one request grows past 256 tokens), greedy and
+    with seeded draws; the caches end as long, and a step after the chain sees what it left."""
+    from llm_runtime_study_amd.config import config_from_dict
+    from llm_runtime_study_amd.engine.step import StepEntry
+    from llm_runtime_study_amd.sampling import SamplingConfig, SamplingRow
+    from llm_runtime_study_amd.weights import write_model_dir
+
+    folder = tmp_path / "model"
+    write_model_dir(config_from_dict(TINY_C), seed=47, model_dir=folder, init="scaled")
+    rng = np.random.default_rng(6)
+    prompts = [rng.integers(0, TINY_C["vocab_size"], n).tolist() for n in (242, 30, 9)]
+    configs = [SamplingConfig(temperature=0.9, top_k=40, seed=5), SamplingConfig(), SamplingConfig(temperature=0.7, top_p=0.8, seed=6)]
+
+    def rows(produced):
+        return [SamplingRow(c, c.seed or 0, produced) for c in configs] if sampled else None
+
+    def drive(chained: bool):
+        runner = make_runner(folder, dtype, pages=40, requests=3, seq=320, step_tokens=320, graph=True)
+        cache = runner.cache
+        with torch.cuda.stream(torch.cuda.Stream(runner.device)):
+            requests = [cache.admit(i) for i in range(3)]
+            first = runner.step([StepEntry(r, p, [len(p) - 1]) for r, p in zip(requests, prompts)]).argmax(-1).tolist()
+            entries = [StepEntry(r, [t], [0]) for r, t in zip(requests, first)]
+            tokens = []
+            if chained:
+                launches = [runner.decode_launch_begin(entries, 4, rows(0))]
+                for _ in range(6):
+                    launches.append(runner.decode_launch_begin(entries, 4, rows(0), after=launches[-1]))
+                    tokens += runner.decode_launch_end(launches[-2])
+                tokens += runner.decode_launch_end(launches[-1])
+                assert all(launch.ended for launch in launches) and sum(launch.steps for launch in launches) == len(tokens)
+                assert any(launch.steps < 4 for launch in launches)          # one ended at the edge of the length class
+            else:
+                while len(tokens) < 22:
+                    latest = [StepEntry(r, [t], [0]) for r, t in zip(requests, tokens[-1])] if tokens else entries
+                    tokens += runner.decode_steps(latest, min(4, 22 - len(tokens)), rows(len(tokens)))
+            lengths = [r.length - len(tokens) for r in requests]          # every cache grew by what was decoded
+            after = runner.step([StepEntry(r, [t], [0]) for r, t in zip(requests, tokens[-1])]).argmax(-1).tolist()
+            tokens = tokens[:22]
+            torch.cuda.synchronize()
+            assert cache.tables_match_device()
+            runner.drop_graphs()
+        cache.check_invariants()
+        return tokens, lengths, after
+
+    chained, chained_lengths, after_chain = drive(True)
+    single, single_lengths, _ = drive(False)
+    assert chained == single and len(chained) == 22
+    assert chained_lengths == single_lengths == [len(p) for p in prompts]
+    assert all(0 <= t < TINY_C["vocab_size"] for t in after_chain)            # a step after the chain runs on what it left
+    if sampled:
+        assert len({tuple(row) for row in chained}) > 5                      # draws, not a fixed point
+
+
+def test_a_launch_follows_only_the_launch_begun_last(folder_b):
+    from llm_runtime_study_amd.engine.step import StepEntry
+    from llm_runtime_study_amd.errors import GenerationError
+
+    runner = make_runner(folder_b, torch.float32, pages=12, graph=True)
+    cache = runner.cache
+    with torch.cuda.stream(torch.cuda.Stream(runner.device)):
+        a, b = cache.admit("a"), cache.admit("b")
+        runner.step([StepEntry(a, [3, 4, 5], []), StepEntry(b, [6], [])])
+        entries = [StepEntry(a, [7], [0]), StepEntry(b, [8], [0])]
+        first = runner.decode_launch_begin(entries, 2)
+        with pytest.raises(GenerationError, match="same requests in the same order"):
+            runner.decode_launch_begin(entries[::-1], 2, after=first)
+        assert [a.length, b.length] == [5, 3]                                # the refused launch took nothing
+        second = runner.decode_launch_begin(entries, 2, after=first)
+        tokens = runner.decode_launch_end(first) + runner.decode_launch_end(second)
+        assert len(tokens) == 4 and [a.length, b.length] == [7, 5]
+        runner.step([StepEntry(a, [tokens[-1][0]], [0])])                     # another step: the device's metadata is its own now
+        with pytest.raises(GenerationError, match="begun last"):
+            runner.decode_launch_begin(entries, 2, after=second)
+        with pytest.raises(GenerationError, match="ended before"):
+            runner.decode_launch_end(second)
+        torch.cuda.synchronize()
+        runner.drop_graphs()
+    cache.check_invariants()
+
+
 # ------------------------------------------------ block tables that stay on the device
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_block_tables_on_the_device_follow_the_hosts(folder_b, dtype):
