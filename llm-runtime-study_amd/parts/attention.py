@@ -106,7 +106,7 @@ class GQAAttention(Part):
         return max(1, min(wanted, length_class(longest) // 256, 64), -(-bound // (4096 * page_size)))
 
     @staticmethod
-    def _prefill_splits(workgroups: int, longest: int, outputs: int, heads_per_group: int = 4) -> int:
+    def _prefill_splits(workgroups: int, longest: int, outputs: int, heads_per_group: int = 4, tokens: int = 0) -> int:
         """Into how many workgroups the keys of every query group of a ragged step are divided: one, unless
         the groups alone leave compute units idle (a last portion of a prompt, a short portion after a long
         context), and never from two workgroups a unit on.  Partial results (float32, `outputs` values per split)
@@ -117,7 +117,12 @@ class GQAAttention(Part):
             16, 512 tokens 1,186 -> 576 us with 8);
           * shorter contexts: towards two workgroups a unit, at least 256 keys each (2,048 tokens of context: 64 tokens 42.5 -> 18.6 us with 8 splits, 256 tokens 43.2 -> 32.4 with
             4, 512 tokens 87.5 -> 76.4 with 2, but 1,024 tokens 96.8 -> 127 and 2,032 tokens 111 -> 173 with 2:
-            what the merge reads and writes grows with the tokens, what a split saves with the context).
+            what the merge reads and writes grows with the tokens, what a split saves with the context).  So under
+            16,384 tokens of context the keys are divided only where the longest context is at least four times the
+            step's `tokens` (undivided against 2 splits with their merge: 512 tokens after 0 / 512 / 1,024 / 1,536:
+            16.9 / 26.6 / 36.2 / 45.8 against 24.4 / 30.5 / 36.9 / 42.9 us; 256 tokens after 256 / 512 / 768 / 1,024:
+            16.5 / 21.1 / 25.7 / 30.2 against 18.8 / 20.3 / 23.1 / 25.6 us; 128 tokens after 0 / 256 / 512: 14.4 / 14.1 /
+            18.5 against 16.2 / 16.8 / 17.1 us).
         A kv group of five to eight heads walks the keys once with a wave for every head while the launch is at
         most two workgroups a unit; that walk is short enough that one workgroup a unit is the aim (40 heads on
         8: 512 tokens after 1,536 54 us undivided against 72 with 2; 256 tokens 51 -> 43 with 2, 128 tokens
@@ -126,6 +131,8 @@ class GQAAttention(Part):
         units = ops.compute_units()
         within = (64 << 20) // max(outputs, 1)
         if workgroups >= 2 * units:      # (2,048 tokens in groups of 32 after 30,720: 1,071 us undivided, 1,115 with 2)
+            return 1
+        if longest < 16384 and longest < 4 * tokens:
             return 1
         if heads_per_group > 4 and workgroups <= units and longest < 16384:
             return max(1, min(-(-units // workgroups), longest // 256, 32, within))
@@ -224,7 +231,7 @@ class GQAAttention(Part):
                 rest = ctx.memo["rows_after_singles"] = (ctx.token_slot[singles:], ctx.positions[singles:])
             if queries_raw is not None and singles and cos is not None:
                 queries_raw = ops.DecodePrepare(self.q_norm, None, self.qk_norm_eps, parted[2], parted[3], 0)
-            splits = self._prefill_splits(ctx.num_qblocks * kv_heads, longest, (t - singles) * nq * d, nq // kv_heads)
+            splits = self._prefill_splits(ctx.num_qblocks * kv_heads, longest, (t - singles) * nq * d, nq // kv_heads, t - singles)
             part_o = part_ml = None
             if splits > 1:
                 part_o = ctx.scratch("attn_part_o", (t - singles, nq * splits * d), torch.float32)

@@ -59,6 +59,10 @@ def test_prefill_splits_only_where_groups_leave_the_chip_idle(monkeypatch):
     assert splits(8, 2048, 1 << 16) == 8 and splits(32, 2064, 1 << 20) == 8 and splits(128, 2048, 1 << 20) == 4
     assert splits(256, 2048, 1 << 20) == 2 and splits(256, 4096, 1 << 20) == 2 and splits(1016, 2047, 1 << 20) == 1
     assert splits(64, 700, 1 << 20) == 2                # 256 keys each
+    # and only where the longest context is four times the step's tokens or more: the merge costs by the token
+    assert splits(256, 2048, 1 << 20, 4, 512) == 2 and splits(256, 2047, 1 << 20, 4, 512) == 1 and splits(256, 512, 1 << 20, 4, 512) == 1
+    assert splits(64, 700, 1 << 20, 4, 128) == 2 and splits(64, 384, 1 << 20, 4, 128) == 1
+    assert splits(256, 33216, 1 << 20, 4, 16384) == 8   # not a rule for long contexts
     # kv groups of five to eight heads (one walk with a wave a head): one workgroup a unit is the aim
     assert splits(256, 8192, 1 << 20, 5) == 1 and splits(128, 2048, 1 << 20, 5) == 2 and splits(32, 2064, 1 << 20, 8) == 8
     assert splits(512, 2048, 1 << 20, 5) == 1 and splits(256, 33216, 1 << 20, 5) == 8 and splits(512, 33216, 1 << 20, 5) == 1
