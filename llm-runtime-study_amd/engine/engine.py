@@ -20,7 +20,7 @@ from ..errors import EngineError
 from ..sampling import Sampler, SamplingConfig
 from ..text import TextTokenizer
 from ..config import chat_template_for, load_config
-from .loading import load_model, random_model, resolve_device, resolve_dtype
+from .loading import load_model, random_model, reserve_for, resolve_device, resolve_dtype
 from .scheduler import BatchScheduler, GenerationEvent, generate as _generate
 from .step import ModelRunner
 
@@ -74,6 +74,7 @@ class Engine:
         config = load_config(model_dir)
         config.validate_context_length(max_seq_len)
         selected_device, selected_dtype = resolve_device(device), resolve_dtype(dtype)
+        cls._reserve(config, selected_dtype, selected_device, max_seq_len, max_batch_size, options)
         config, model = load_model(model_dir, selected_dtype, selected_device, config, stored_precision)
         tokenizer = TextTokenizer.from_model_dir(model_dir, config.vocab_size, chat_template_for(config))
         engine = cls(config, model, device=selected_device, dtype=selected_dtype, max_seq_len=max_seq_len,
@@ -89,6 +90,7 @@ class Engine:
         """Random weights made on the device for `config` (a typed configuration)."""
         started = time.perf_counter()
         selected_device, selected_dtype = resolve_device(device), resolve_dtype(dtype)
+        cls._reserve(config, selected_dtype, selected_device, options.get("max_seq_len", 4096), options.get("max_batch_size", 1), options)
         model = random_model(config, seed, selected_dtype, selected_device, init)
         engine = cls(config, model, device=selected_device, dtype=selected_dtype, **options)
         engine._reload = lambda dtype: random_model(config, seed, dtype, selected_device, init)
@@ -96,13 +98,26 @@ class Engine:
         engine.load_seconds = time.perf_counter() - started
         return engine
 
+    @staticmethod
+    def _pool_pages(num_pages, max_seq_len: int, page_size: int, max_batch_size: int) -> int:
+        return num_pages or -(-max_seq_len // page_size) * max_batch_size
+
+    @classmethod
+    def _reserve(cls, config, dtype, device, max_seq_len: int, max_batch_size: int, options: dict) -> None:
+        """One segment of device memory for the weights, the cache pool and the step's buffers of the engine that
+        is about to be made (see engine/loading.py); `reserve_memory=False` among the options leaves it out."""
+        if not options.pop("reserve_memory", True) or max_batch_size <= 0:
+            return
+        page_size = options.get("page_size", DEFAULT_PAGE_SIZE)
+        reserve_for(config, dtype, device, page_size, cls._pool_pages(options.get("num_pages"), max_seq_len, page_size, max_batch_size))
+
     # ------------------------------------------------------------------ cache
     @property
     def runner(self) -> ModelRunner:
         """The step function over this engine's cache pool, made on first use: the pool holds
         max_seq_len * max_batch_size tokens unless `num_pages` says otherwise."""
         if self._runner is None:
-            pages = self.num_pages or -(-self.max_seq_len // self.page_size) * self.max_batch_size
+            pages = self._pool_pages(self.num_pages, self.max_seq_len, self.page_size, self.max_batch_size)
             cache = CacheManager(self.model.cache_needs(), page_size=self.page_size, num_pages=pages,
                                  max_requests=self.max_batch_size, max_seq_len=self.max_seq_len,
                                  dtype=self.dtype, device=self.device)

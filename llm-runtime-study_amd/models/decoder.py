@@ -12,7 +12,7 @@ import torch
 
 from ..kernels import ops
 from ..parts import TensorSpec, create
-from ..parts.base import flops_of
+from ..parts.base import flops_of, under
 from ..parts.linear import linear
 from .spec import ModelSpec
 
@@ -52,10 +52,10 @@ class DecoderModel:
         self.head = self.embedding if head is None else head.to(dtype).contiguous()
         for index, layer in enumerate(self.layers):
             prefix = spec.layer_prefix.format(index=index) + "."
-            layer.bind({n[len(prefix):]: t for n, t in weights.items() if n.startswith(prefix)}, dtype)
+            layer.bind(under(weights, prefix), dtype)
         for part, prefix in [(self.final_norm, spec.final_norm_prefix)] + self._around():
             prefix += "."
-            part.bind({n[len(prefix):]: t for n, t in weights.items() if n.startswith(prefix)}, dtype)
+            part.bind(under(weights, prefix), dtype)
 
     def _around(self) -> list:
         """The optional parts after the embedding and after the head, each with the prefix of its tensors."""

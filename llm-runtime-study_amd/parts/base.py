@@ -57,8 +57,9 @@ scratch arena.  The residual stream `h` is float32 in every precision mode.
 from __future__ import annotations
 
 import math
+from collections.abc import Mapping as MappingView
 from dataclasses import dataclass, field
-from typing import Any, Mapping
+from typing import Any, Callable, Iterable, Mapping
 
 import torch
 
@@ -81,6 +82,56 @@ def create(role: str, spec: "PartSpec"):
         known = ", ".join(sorted(_REGISTRY.get(role, {}))) or "none"
         raise KeyError(f"no {role} of kind {spec.kind!r} is registered (known: {known})") from None
     return cls(**spec.params)
+
+
+class LazyTensors(MappingView):
+    """Tensors by name, each made when it is asked for (and again at every asking: nothing is kept here).  A
+    model whose parts take their tensors one after the other then never holds a second copy of all its weights:
+    the raw tensor of a matrix lives only while the part that asked for it puts it into its own form."""
+
+    def __init__(self, names: Iterable[str], make: Callable[[str], torch.Tensor]):
+        self._names, self._make = tuple(names), make
+        self._known = frozenset(self._names)
+
+    def __getitem__(self, name: str) -> torch.Tensor:
+        if name not in self._known:
+            raise KeyError(name)
+        return self._make(name)
+
+    def __iter__(self):
+        return iter(self._names)
+
+    def __len__(self) -> int:
+        return len(self._names)
+
+    def __contains__(self, name) -> bool:
+        return name in self._known
+
+
+class Under(MappingView):
+    """The tensors of `weights` whose names begin with `prefix`, under the rest of their names.  A view: nothing
+    is looked up before it is asked for, so tensors that are made on demand (LazyTensors) stay so."""
+
+    def __init__(self, weights: Mapping[str, torch.Tensor], prefix: str):
+        self._weights, self._prefix = weights, prefix
+
+    def __getitem__(self, name: str) -> torch.Tensor:
+        return self._weights[self._prefix + name]
+
+    def __iter__(self):
+        cut = len(self._prefix)
+        return (name[cut:] for name in self._weights if name.startswith(self._prefix))
+
+    def __len__(self) -> int:
+        return sum(1 for _ in self)
+
+    def __contains__(self, name) -> bool:
+        return isinstance(name, str) and self._prefix + name in self._weights
+
+
+def under(weights: Mapping[str, torch.Tensor], prefix: str) -> Mapping[str, torch.Tensor]:
+    """What a part that owns the names under `prefix` is given to bind()."""
+    return Under(weights, prefix)
 
 
 @dataclass(frozen=True)

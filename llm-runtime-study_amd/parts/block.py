@@ -7,7 +7,7 @@ The two sums happen inside the parts, which add into the float32 residual stream
 
 from __future__ import annotations
 
-from .base import Part, PartSpec, create, flops_of, register
+from .base import Part, PartSpec, create, flops_of, register, under
 from .linear import materialize
 
 
@@ -29,8 +29,7 @@ class PreNormBlock(Part):
 
     def bind(self, weights, dtype):
         for prefix, part in self._children():
-            own = {name[len(prefix) + 1:]: t for name, t in weights.items() if name.startswith(prefix + ".")}
-            part.bind(own, dtype)
+            part.bind(under(weights, prefix + "."), dtype)
 
     def weight_bytes(self):
         return sum(part.weight_bytes() for _, part in self._children())

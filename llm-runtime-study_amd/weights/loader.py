@@ -23,7 +23,7 @@ from typing import Mapping
 import torch
 
 from ..errors import CheckpointValidationError
-from ..parts import TensorSpec
+from ..parts import LazyTensors, TensorSpec
 from .safetensors_io import Checkpoint
 
 FLOAT_DTYPES = ("F32", "BF16", "F16")
@@ -67,18 +67,20 @@ def validate(checkpoint: Checkpoint, expected: Mapping[str, TensorSpec], archite
 
 
 def load(checkpoint: Checkpoint, expected: Mapping[str, TensorSpec], architecture: str, device,
-         checkpoint_dtype: str | None = None) -> dict[str, torch.Tensor]:
+         checkpoint_dtype: str | None = None, lazy: bool = False) -> Mapping[str, torch.Tensor]:
     """Validate (see validate() for `checkpoint_dtype`), then move every expected tensor that is
-    present to `device` in its stored precision."""
+    present to `device` in its stored precision.  lazy: each tensor is read and moved when it is asked for
+    (parts.LazyTensors; the checkpoint must stay open meanwhile), so that a model which takes its tensors part
+    by part never holds the checkpoint and its own form of the weights at once."""
     validate(checkpoint, expected, architecture, checkpoint_dtype)
-    out = {}
-    for name, spec in expected.items():
-        if name not in checkpoint.manifest:
-            continue
+
+    def fetch(name: str) -> torch.Tensor:
         t = checkpoint.tensor(name)
-        if spec.dtype == "int32":
+        if expected[name].dtype == "int32":
             t = t.to(torch.int32)
         elif t.dtype == torch.float16:
             t = t.to(torch.float32)
-        out[name] = t.to(device)
-    return out
+        return t.to(device)
+
+    present = [name for name in expected if name in checkpoint.manifest]
+    return LazyTensors(present, fetch) if lazy else {name: fetch(name) for name in present}

@@ -9,8 +9,10 @@ N(0, 0.02).  init = "scaled": matrices N(0, 1/fan_in), embedding N(0, 1), norm w
 1 + N(0, 0.1), biases N(0, 0.1), which keeps every part's contribution at order one so that
 tests see faults that tiny weights would hide.
 
-`device_weights` fills tensors on the device directly (same distributions, another stream
-of numbers) for benchmark-sized models, where a file would only cost time.
+`device_weights` makes tensors on the device directly (same distributions, other numbers: every
+tensor has a generator of its own, seeded by the seed and the tensor's place in the sorted names) for
+benchmark-sized models, where a file would only cost time.  Each tensor is drawn when it is asked for,
+so a model that takes its tensors part by part never holds two copies of its weights.
 """
 
 from __future__ import annotations
@@ -22,7 +24,7 @@ import torch
 
 from ..config import spec_for
 from ..models import DecoderModel
-from ..parts import TensorSpec
+from ..parts import LazyTensors, TensorSpec
 from .safetensors_io import write_safetensors
 
 TORCH_DTYPES = {"bfloat16": torch.bfloat16, "float32": torch.float32, "float16": torch.float16}
@@ -63,11 +65,16 @@ def write_model_dir(config, seed: int, model_dir, init: str = "normal") -> Path:
     return model_dir
 
 
-def device_weights(model: DecoderModel, seed: int, dtype: torch.dtype, device, init: str = "normal") -> dict[str, torch.Tensor]:
-    generator = torch.Generator(device=device).manual_seed(seed)
+def device_weights(model: DecoderModel, seed: int, dtype: torch.dtype, device, init: str = "normal") -> LazyTensors:
     expected = model.tensors()
-    return {name: _draw(expected[name], init, generator, device).to(torch.int32 if expected[name].dtype == "int32" else dtype)
-            for name in sorted(expected) if not expected[name].optional}
+    names = [name for name in sorted(expected) if not expected[name].optional]
+    place = {name: index for index, name in enumerate(names)}
+
+    def draw(name: str) -> torch.Tensor:
+        generator = torch.Generator(device=device).manual_seed((seed << 20) + place[name])
+        return _draw(expected[name], init, generator, device).to(torch.int32 if expected[name].dtype == "int32" else dtype)
+
+    return LazyTensors(names, draw)
 
 
 def main(argv=None) -> int:

@@ -601,3 +601,38 @@ def test_a_cache_pool_the_device_cannot_hold_is_refused_before_anything_is_alloc
         CacheManager([PagedKVNeed(8, 128, None)] * 36, page_size=16, num_pages=64 * 65536, max_requests=64, max_seq_len=1 << 20,
                      dtype=torch.bfloat16, device="cuda")
     assert torch.cuda.memory_allocated() == before
+
+
+def test_one_segment_of_device_memory_is_reserved_for_an_engine_and_its_tensors_come_out_of_it(folders):
+    """engine/loading.py: the reservation is one allocation that torch's allocator keeps; what is allocated next is
+    cut out of it (torch asks the device for nothing more); an engine too small to gain reserves nothing, a size the
+    device does not have is no error, and the option switches it off."""
+    from llm_runtime_study_amd import Engine
+    from llm_runtime_study_amd.config import config_from_dict, spec_for
+    from llm_runtime_study_amd.engine import loading
+    from llm_runtime_study_amd.models import DecoderModel
+
+    tiny = config_from_dict(TINY_B)
+    model = DecoderModel(spec_for(tiny))
+    weights = sum(int(np.prod(spec.shape)) for spec in model.tensors().values())
+    pages = 2 * TINY_B["num_key_value_heads"] * TINY_B["head_dim"] * TINY_B["num_hidden_layers"] * 16 * (40 + 1)
+    assert loading.engine_bytes(model, torch.bfloat16, 16, 40) == 2 * (weights + pages)
+    assert loading.engine_bytes(model, torch.float32, 16, 40) == 4 * (weights + pages)
+    assert loading.reserve_for(tiny, torch.bfloat16, "cuda", 16, 40) == 0          # far under a gigabyte
+    assert loading.reserve_device_memory(1 << 50, "cuda") == 0                     # a petabyte: refused, nothing raised
+    torch.cuda.synchronize()
+    torch.cuda.empty_cache()
+    before = torch.cuda.memory_reserved()
+    got = loading.reserve_device_memory(1 << 30, "cuda")
+    assert got == 3 << 30 and torch.cuda.memory_reserved() == before + got         # a gigabyte and the margin, in whole gigabytes
+    first = torch.empty(700 << 20, dtype=torch.uint8, device="cuda")
+    second = torch.empty(900 << 20, dtype=torch.uint8, device="cuda")
+    assert torch.cuda.memory_reserved() == before + got                            # both were cut out of the segment
+    assert abs(first.data_ptr() - second.data_ptr()) < got
+    del first, second
+    torch.cuda.empty_cache()
+    assert torch.cuda.memory_reserved() == before
+    folder = folders["b"][0]
+    engine = Engine.from_model_dir(folder, max_seq_len=128, max_batch_size=2, reserve_memory=False)
+    assert engine.generate_tokens([[5, 6, 7]], max_new_tokens=3) == Engine.from_model_dir(
+        folder, max_seq_len=128, max_batch_size=2).generate_tokens([[5, 6, 7]], max_new_tokens=3)

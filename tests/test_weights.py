@@ -154,3 +154,55 @@ def test_file_errors(tmp_path):
     write_safetensors(tmp_path / "model.safetensors", {"a": torch.zeros(2)})
     with pytest.raises(CheckpointError, match="tensor is not in the checkpoint: b"):
         Checkpoint.from_model_dir(tmp_path).tensor("b")
+
+
+def test_lazy_load_reads_a_tensor_when_it_is_asked_for(tmp_path, monkeypatch):
+    """load(..., lazy=True): validated as a whole at once, the same tensors as the eager load, and no tensor's bytes
+    are touched before a part asks for it; views by prefix (what a model hands its parts) keep that."""
+    from llm_runtime_study_amd.parts import LazyTensors, under
+
+    config = config_from_dict(TINY_B)
+    write_model_dir(config, 3, tmp_path, init="scaled")
+    expected = expected_for(TINY_B)
+    checkpoint = Checkpoint.from_model_dir(tmp_path)
+    eager = load(checkpoint, expected, "qwen3", "cpu")
+    read = []
+    original = Checkpoint.tensor
+    monkeypatch.setattr(Checkpoint, "tensor", lambda self, name: (read.append(name), original(self, name))[1])
+    lazy = load(checkpoint, expected, "qwen3", "cpu", lazy=True)
+    assert isinstance(lazy, LazyTensors) and read == []
+    assert list(lazy) == list(eager) and len(lazy) == len(eager) and "lm_head.weight" in lazy and "nothing" not in lazy
+    layer = under(lazy, "model.layers.1.")
+    mixer = under(layer, "self_attn.")
+    assert read == [] and "q_proj.weight" in mixer and "gate_proj.weight" not in mixer
+    assert sorted(mixer) == sorted(n[len("model.layers.1.self_attn."):] for n in eager if n.startswith("model.layers.1.self_attn."))
+    assert torch.equal(mixer["q_proj.weight"], eager["model.layers.1.self_attn.q_proj.weight"])
+    assert read == ["model.layers.1.self_attn.q_proj.weight"]
+    assert mixer.get("nothing") is None and lazy.get("nothing") is None
+    with pytest.raises(KeyError):
+        lazy["nothing"]
+    assert all(torch.equal(lazy[n], eager[n]) for n in eager)
+    # a checkpoint that does not fit is refused before anything is read, lazily or not
+    read.clear()
+    with pytest.raises(CheckpointValidationError):
+        load(checkpoint, expected_for(TINY_A), "qwen3", "cpu", lazy=True)
+    assert read == []
+
+
+def test_a_model_binds_lazy_tensors_as_it_binds_a_dictionary(tmp_path):
+    """DecoderModel.bind with tensors made on demand: the same bound weights as with all of them in a dictionary."""
+    from llm_runtime_study_amd.config import spec_for
+    from llm_runtime_study_amd.models import DecoderModel
+
+    config = config_from_dict(TINY_B)
+    write_model_dir(config, 7, tmp_path, init="scaled")
+    spec = spec_for(config)
+    checkpoint = Checkpoint.from_model_dir(tmp_path)
+    one, other = DecoderModel(spec), DecoderModel(spec)
+    one.bind(load(checkpoint, one.tensors(), "qwen3", "cpu"), torch.bfloat16)
+    other.bind(load(checkpoint, other.tensors(), "qwen3", "cpu", lazy=True), torch.bfloat16)
+    assert torch.equal(one.embedding, other.embedding) and torch.equal(one.head, other.head)
+    for a, b in zip(one.layers, other.layers):
+        assert torch.equal(a.mixer.w_qkv, b.mixer.w_qkv) and torch.equal(a.mixer.b_qkv, b.mixer.b_qkv)
+        assert torch.equal(a.mixer.w_o, b.mixer.w_o) and torch.equal(a.feed_forward.down, b.feed_forward.down)
+        assert torch.equal(a.mixer_norm.weight, b.mixer_norm.weight)
