@@ -131,7 +131,9 @@ class CacheManager:
         if allocate_storage and self.device.type == "cuda" and self.groups:
             # a pool the device cannot hold is refused before anything is allocated, with the numbers that decide it
             per_page = page_size * self.bytes_per_token()
-            free, _ = torch.cuda.mem_get_info(self.device)
+            # free: what the device has left, and what torch's allocator holds without using it (an engine reserves
+            # its memory as one segment before its weights are made: the pool comes out of that)
+            free = torch.cuda.mem_get_info(self.device)[0] + torch.cuda.memory_reserved(self.device) - torch.cuda.memory_allocated(self.device)
             if (num_pages + 1) * per_page > free:
                 fits = max(free // per_page - 1, 0)
                 raise KVCacheError(f"a cache pool of {num_pages} pages of {page_size} tokens needs {(num_pages + 1) * per_page / 2**30:.1f} GiB, "
