@@ -937,11 +937,20 @@ struct MidScale {
   float eps;
 };
 
-template <int MT, int WAVES, bool SWIGLU>
+//
+// EXTRA (4 or 8 waves, up to 64 rows): the weight rows are dealt out in tiles of 16 so that every workgroup of the
+// launch has WAVES or WAVES + 1 of them (the first `extras` workgroups the one more), which lets a launch be a whole
+// multiple of the compute units whatever n is: a unit fetches at a fixed rate, so the launch takes as long as the
+// unit with the most rows.  The extra tile has no wave of its own: its k steps are dealt out over the waves (one
+// step of a slice each with eight waves, two with four), which multiply them by the activation fragments they hold
+// anyway; the waves' partial sums meet in LDS at the end, are added in wave order and written by the first MT waves.
+template <int MT, int WAVES, bool SWIGLU, bool EXTRA = false>
 __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_mid_kernel(
     void* __restrict__ out, int mode, const bf16* __restrict__ x, const bf16* __restrict__ w,
-    int m, int n, int k, int lda, int ldc, float* __restrict__ split_sums, MidScale scale) {
+    int m, int n, int k, int lda, int ldc, float* __restrict__ split_sums, MidScale scale, int extras) {
+  static_assert(!EXTRA || ((WAVES == 4 || WAVES == 8) && MT <= 4), "the extra tile needs 4 or 8 waves and at most 64 rows");
   constexpr int STEPS = 8;                         // k steps of 32 in a slice
+  constexpr int XS = EXTRA ? STEPS / WAVES : 1;    // steps of the extra tile that a wave multiplies in every slice
   constexpr int FRAGS = STEPS * MT;                // activation fragments of a slice
   constexpr int MINE = (FRAGS + WAVES - 1) / WAVES;  // of which a wave brings this many
   // LDS (dynamic: more than the 64 KB a static array may have): two buffers of activations, then a patch of
@@ -950,7 +959,10 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_mid_kernel(
   extern __shared__ __attribute__((aligned(16))) bf16x8 mid_lds[];
   const int tid = threadIdx.x, lane = tid % WAVE, wave = __builtin_amdgcn_readfirstlane(tid / WAVE);
   const int r = lane & 15, g = lane >> 4;
-  const int row0 = blockIdx.x * (16 * WAVES) + wave * 16;
+  const int tile0 = EXTRA ? (int)blockIdx.x * WAVES + ((int)blockIdx.x < extras ? (int)blockIdx.x : extras) : (int)blockIdx.x * WAVES;
+  const int row0 = (tile0 + wave) * 16;
+  const bool has_extra = EXTRA && (int)blockIdx.x < extras;        // the same for every wave of the workgroup
+  const int row_x = (tile0 + WAVES) * 16;                          // first row of the extra tile
   bf16x8* const patch = mid_lds + 2 * STEPS * MT * WAVE + wave * 256;
   const bf16* wl[2];
   int wr_off[2], rd_off[2];
@@ -1019,6 +1031,23 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_mid_kernel(
 #pragma unroll
   for (int t = 0; t < MT; ++t) acc[t] = floatx4{0.f, 0.f, 0.f, 0.f};
   bf16x8 wa[STEPS], wb[STEPS], sa[MINE], sb[MINE];
+  // the extra tile: this wave's steps of it as A fragments straight from memory (row = lane % 16, 8 k from 8 * (lane / 16))
+  floatx4 acc_x[MT];
+  bf16x8 xa[XS], xb[XS];
+  const bf16* xl = w;
+  if constexpr (EXTRA) {
+#pragma unroll
+    for (int t = 0; t < MT; ++t) acc_x[t] = floatx4{0.f, 0.f, 0.f, 0.f};
+    xl = w + (int64_t)(row_x + r < n ? row_x + r : n - 1) * k + g * 8 + wave * 32;
+  }
+  auto load_x = [&](int slice, bf16x8 (&xf)[XS]) {
+    if constexpr (EXTRA) {
+      if (has_extra) {
+#pragma unroll
+        for (int j = 0; j < XS; ++j) xf[j] = *(const bf16x8*)(xl + (int64_t)slice * 256 + j * (WAVES * 32));
+      }
+    }
+  };
   // a[2 p + h]: line p (k steps 2 p and 2 p + 1) of rows 8 h .. 8 h + 7
   auto load_w = [&](int slice, bf16x8 (&a)[STEPS]) {
 #pragma unroll
@@ -1038,7 +1067,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_mid_kernel(
   // activation fragments of a step are read from LDS while the step before is multiplied.
   const bf16x8* const frag_even = lds + place(0, 0, r, g);    // this lane's piece of a fragment in an even panel ...
   const bf16x8* const frag_odd = lds + place(1, 0, r, g) - MT * 64;   // ... and in an odd one, less the panel's own offset
-  auto compute = [&](int buf, bf16x8 (&a)[STEPS], auto reload, int next) {
+  auto compute = [&](int buf, bf16x8 (&a)[STEPS], bf16x8 (&xf)[XS], auto reload, int next) {
     constexpr bool RELOAD = decltype(reload)::value;
     const bf16x8* const even = frag_even + buf * (STEPS * MT * WAVE);
     const bf16x8* const odd = frag_odd + buf * (STEPS * MT * WAVE);
@@ -1060,14 +1089,27 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_mid_kernel(
       for (int t = 0; t < MT; ++t) b[1][t] = odd[((2 * p + 1) * MT + t) * WAVE];
 #pragma unroll
       for (int t = 0; t < MT; ++t) acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(f0, b[0][t], acc[t], 0, 0, 0);
+      if constexpr (EXTRA) {       // step 2 p of the extra tile is the business of wave 2 p % WAVES
+        if (has_extra && wave == (2 * p) % WAVES) {
+#pragma unroll
+          for (int t = 0; t < MT; ++t) acc_x[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xf[(2 * p) / WAVES], b[0][t], acc_x[t], 0, 0, 0);
+        }
+      }
       if (2 * p + 2 < STEPS) {
 #pragma unroll
         for (int t = 0; t < MT; ++t) b[0][t] = even[((2 * p + 2) * MT + t) * WAVE];
       }
 #pragma unroll
       for (int t = 0; t < MT; ++t) acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(f1, b[1][t], acc[t], 0, 0, 0);
+      if constexpr (EXTRA) {
+        if (has_extra && wave == (2 * p + 1) % WAVES) {
+#pragma unroll
+          for (int t = 0; t < MT; ++t) acc_x[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xf[(2 * p + 1) / WAVES], b[1][t], acc_x[t], 0, 0, 0);
+        }
+      }
       if constexpr (RELOAD) __builtin_amdgcn_sched_barrier(0);
     }
+    if constexpr (RELOAD) load_x(next, xf);
   };
   const std::true_type again;
   const std::false_type last;
@@ -1080,36 +1122,38 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_mid_kernel(
   if constexpr (MT <= 4) {
     if (count > 0) {
       load_w(slice_at(0), wa);
+      load_x(slice_at(0), xa);
       load_acts(slice_at(0), sa);
     }
     if (count > 1) {
       load_w(slice_at(1), wb);
+      load_x(slice_at(1), xb);
       load_acts(slice_at(1), sb);
     }
     if (count > 0) store_acts(0, sa);
     if (count > 2) load_acts(slice_at(2), sa);
     // slice c: after the barrier LDS buffer c & 1 holds it and nobody reads the other buffer any more
-    auto steady = [&](int c, bf16x8 (&a)[STEPS], bf16x8 (&st)[MINE]) {
+    auto steady = [&](int c, bf16x8 (&a)[STEPS], bf16x8 (&xf)[XS], bf16x8 (&st)[MINE]) {
       __syncthreads();
       store_acts((c & 1) ^ 1, st);                       // slice c + 1
       load_acts(slice_at(c + 3), st);
-      compute(c & 1, a, again, slice_at(c + 2));
+      compute(c & 1, a, xf, again, slice_at(c + 2));
     };
-    auto ending = [&](int c, bf16x8 (&a)[STEPS], bf16x8 (&st)[MINE]) {
+    auto ending = [&](int c, bf16x8 (&a)[STEPS], bf16x8 (&xf)[XS], bf16x8 (&st)[MINE]) {
       __syncthreads();
       if (c + 1 < count) store_acts((c & 1) ^ 1, st);
       if (c + 3 < count) load_acts(slice_at(c + 3), st);
-      if (c + 2 < count) compute(c & 1, a, again, slice_at(c + 2));
-      else compute(c & 1, a, last, 0);
+      if (c + 2 < count) compute(c & 1, a, xf, again, slice_at(c + 2));
+      else compute(c & 1, a, xf, last, 0);
     };
     for (; c + 4 < count; c += 2) {            // no branch inside: slices up to c + 4 exist
-      steady(c, wa, sb);
-      steady(c + 1, wb, sa);
+      steady(c, wa, xa, sb);
+      steady(c + 1, wb, xb, sa);
     }
     for (; c < count; c += 2) {                // the last one to four slices
-      ending(c, wa, sb);
+      ending(c, wa, xa, sb);
       if (c + 1 >= count) break;
-      ending(c + 1, wb, sa);
+      ending(c + 1, wb, xb, sa);
     }
   } else {
     if (count > 0) {
@@ -1123,16 +1167,16 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_mid_kernel(
       __syncthreads();
       store_acts((c & 1) ^ 1, sa);                       // slice c + 1
       load_acts(slice_at(c + 2), sa);
-      compute(c & 1, a, again, slice_at(c + 2));
+      compute(c & 1, a, xa, again, slice_at(c + 2));
     };
     auto ending = [&](int c, bf16x8 (&a)[STEPS]) {
       __syncthreads();
       if (c + 1 < count) store_acts((c & 1) ^ 1, sa);
       if (c + 2 < count) {
         load_acts(slice_at(c + 2), sa);
-        compute(c & 1, a, again, slice_at(c + 2));
+        compute(c & 1, a, xa, again, slice_at(c + 2));
       } else {
-        compute(c & 1, a, last, 0);
+        compute(c & 1, a, xa, last, 0);
       }
     };
     for (; c + 3 < count; c += 2) {            // no branch inside: slices up to c + 3 exist
@@ -1154,37 +1198,49 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_mid_kernel(
 #pragma unroll
     for (int t = 0; t < MT; ++t) acc[t] *= row_scales[t * 16 + r < m ? t * 16 + r : 0];
   }
-  const int gn = row0 + 4 * g;
-  if (split_sums) {
-#pragma unroll
-    for (int t = 0; t < MT; ++t) {
-      const int token = t * 16 + r;
-      if (token < m && gn < n) *(floatx4*)(split_sums + ((int64_t)blockIdx.y * m + token) * n + gn) = acc[t];
+  // one block of 16 tokens of a tile of 16 weight rows that begins at row `first`: the wave's own, or the extra one
+  auto emit_block = [&](int t, floatx4 v, int first) {
+    const int token = t * 16 + r, gn = first + 4 * g;
+    if (split_sums) {
+      if (token < m && gn < n) *(floatx4*)(split_sums + ((int64_t)blockIdx.y * m + token) * n + gn) = v;
+      return;
     }
-    return;
-  }
-#pragma unroll
-  for (int t = 0; t < MT; ++t) {
-    const int token = t * 16 + r;
     if constexpr (SWIGLU) {
-      // the 16 rows of a wave are 8 gate rows and the 8 up rows of the same features: the up values
+      // the 16 rows of a tile are 8 gate rows and the 8 up rows of the same features: the up values
       // of a lane's gate rows sit 32 lanes further on
       floatx4 up;
 #pragma unroll
-      for (int i = 0; i < 4; ++i) up[i] = __shfl(acc[t][i], (lane + 32) & 63, WAVE);
-      if (g < 2 && token < m && row0 < n) {
+      for (int i = 0; i < 4; ++i) up[i] = __shfl(v[i], (lane + 32) & 63, WAVE);
+      if (g < 2 && token < m && first < n) {
         bf16x4 y;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) y[i] = (bf16)(silu(acc[t][i]) * up[i]);
-        *(bf16x4*)((bf16*)out + (int64_t)token * ldc + row0 / 2 + 4 * g) = y;
+        for (int i = 0; i < 4; ++i) y[i] = (bf16)(silu(v[i]) * up[i]);
+        *(bf16x4*)((bf16*)out + (int64_t)token * ldc + first / 2 + 4 * g) = y;
       }
     } else if (token < m && gn < n) {
-      const floatx4 v = acc[t];
       if (mode == OUT_STORE) *(bf16x4*)((bf16*)out + (int64_t)token * ldc + gn) = bf16x4{(bf16)v[0], (bf16)v[1], (bf16)v[2], (bf16)v[3]};
       else if (mode == OUT_STORE_F32) *(floatx4*)((float*)out + (int64_t)token * ldc + gn) = v;
       else *(floatx4*)((float*)out + (int64_t)token * ldc + gn) = *(const floatx4*)((const float*)out + (int64_t)token * ldc + gn) + v;
     }
+  };
+  if constexpr (EXTRA) {
+    if (has_extra) {
+      // the waves' partial sums of the extra tile, [wave][block][lane], behind the row factors at the head of LDS
+      floatx4* const meet = (floatx4*)mid_lds + 64;
+      __syncthreads();                               // nobody reads activations any more (and the row factors are written)
+#pragma unroll
+      for (int t = 0; t < MT; ++t) meet[(wave * MT + t) * WAVE + lane] = acc_x[t];
+      __syncthreads();
+      if (wave < MT) {
+        floatx4 v = meet[wave * WAVE + lane];
+        for (int other = 1; other < WAVES; ++other) v += meet[(other * MT + wave) * WAVE + lane];
+        if (scale.sumsq) v *= ((const float*)mid_lds)[wave * 16 + r < m ? wave * 16 + r : 0];
+        emit_block(wave, v, row_x);
+      }
+    }
   }
+#pragma unroll
+  for (int t = 0; t < MT; ++t) emit_block(t, acc[t], row0);
 }
 
 // Choices a caller may make for the products (measurements and tests; a step carries its runner's).  They
@@ -1193,16 +1249,19 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_mid_kernel(
 //   bit 1      the few-rows kernel loads its weights as whole 128-byte lines where the shape allows
 //   bits 4-7   workgroup shape of the kernel for 17..128 rows: 4, 5, 6 or 8 waves (0: chosen here)
 //   bits 8-12  its number of K splits, 1..16 (0: chosen here)
+//   bits 13-14 its weight rows dealt out evenly over a whole multiple of the compute units, some workgroups with a
+//              tile more than the others (see the kernel, EXTRA): 0: where it pays (chosen here), 1: never, 2: wherever
+//              the shape allows
 struct GemmTune {
   bool mid, lines;
-  int waves, splits;
+  int waves, splits, even;
 };
 constexpr int TUNE_DEFAULT = 3;
 static bool tune_ok(int word) {
-  const int waves = (word >> 4) & 15, splits = (word >> 8) & 31;
-  return word >= 0 && (word >> 13) == 0 && (waves == 0 || waves == 4 || waves == 5 || waves == 6 || waves == 8) && splits <= 16;
+  const int waves = (word >> 4) & 15, splits = (word >> 8) & 31, even = (word >> 13) & 3;
+  return word >= 0 && (word >> 15) == 0 && (waves == 0 || waves == 4 || waves == 5 || waves == 6 || waves == 8) && splits <= 16 && even <= 2;
 }
-static GemmTune tune_of(int word) { return GemmTune{(word & 1) != 0, (word & 2) != 0, (word >> 4) & 15, (word >> 8) & 31}; }
+static GemmTune tune_of(int word) { return GemmTune{(word & 1) != 0, (word & 2) != 0, (word >> 4) & 15, (word >> 8) & 31, (word >> 13) & 3}; }
 
 // Row tiles per workgroup: more of them means each activation fragment read from L2 serves more
 // weight rows, which matters once there are several token blocks; fewer means more workgroups.
@@ -1287,7 +1346,12 @@ LRS_API int64_t lrs_gemm_workspace_bytes() { return (int64_t)SPLIT_SUMS_BYTES; }
 // fewest splits.
 LRS_API int lrs_compute_units();
 
-static void choose_mid_shape(int n, int k, GemmTune tune, int& waves, int& splits) {
+// What a launch of `groups` workgroups of `wv` tiles (16 weight rows each) costs: a compute unit fetches at a fixed
+// rate (some 45 GB/s), so the launch takes as long as the unit with the most to fetch: the tiles of its workgroups
+// and, for each of them, the activations once (`blocks` blocks of 16 tokens: as many bytes as that many tiles).
+static int mid_cost(int groups, int wv, int blocks, int units) { return (groups + units - 1) / units * (wv + blocks); }
+
+static void choose_mid_shape(int n, int k, GemmTune tune, int& waves, int& splits, int blocks = 4) {
   const int want_waves = tune.waves, want_splits = tune.splits;
   const int units = lrs_compute_units() > 0 ? lrs_compute_units() : 256, slices = k / 256;
   auto tiles_of = [&](int wv) { return (n + 16 * wv - 1) / (16 * wv); };
@@ -1296,18 +1360,25 @@ static void choose_mid_shape(int n, int k, GemmTune tune, int& waves, int& split
     waves = want_waves, splits = want_splits;
     return;
   }
-  // Measured on MI355X (Qwen3-8B shapes, 32..64 rows).  A matrix with enough rows to give every compute
-  // unit a workgroup is not divided along K: six waves (96 rows) a workgroup, or four where that fills the
-  // chip clearly better; eight waves walking many slices were a third slower (gate_up, the LM head).
-  // Five waves where the launch then takes a tenth fewer rows a compute unit (rounds of the chip times the
-  // rows of a workgroup) than with either: 34,816 rows are 363 workgroups of 96 rows or 544 of 64, two and
-  // three rounds, 192 rows a unit, but 436 of 80, two rounds, 160 (at 64 rows 89 -> 77 us).
+  // Measured on MI355X (32..64 rows).  A matrix with enough rows to give every compute unit a workgroup is not
+  // divided along K; of the workgroup shapes the one that costs least by mid_cost(): 24,576 rows are 256 workgroups
+  // of six waves (one round of the chip; 39 us at 64 rows, eight waves 192 workgroups: a third slower); 34,816 rows
+  // 436 of five (two rounds of 80 rows: 83 us at 64 rows; 363 of six 88, 544 of four 93, 272 of eight 100); 51,200
+  // rows 400 of eight (110 us; 640 of five 121, 800 of four 124, 534 of six 131).  Eight waves only while that is
+  // at most two rounds: walking many slices in many rounds they were slower than six (the LM head).  Ties go to
+  // six, five, four, eight in that order.
   if ((!want_splits || want_splits == 1) && tiles_of(6) >= units && (!want_waves || want_waves == 4 || want_waves == 5 || want_waves == 6)) {
     splits = 1;
-    waves = want_waves ? want_waves : (fill_of(tiles_of(4)) > fill_of(tiles_of(6)) + 0.08 ? 4 : 6);
+    waves = want_waves;
     if (!want_waves) {
-      auto rows_a_unit = [&](int wv) { return (tiles_of(wv) + units - 1) / units * wv; };
-      if (10 * rows_a_unit(5) <= 9 * rows_a_unit(4) && 10 * rows_a_unit(5) <= 9 * rows_a_unit(6)) waves = 5;
+      const int order[4] = {6, 5, 4, 8};
+      int best = 0;
+      for (int i = 0; i < 4; ++i) {
+        const int wv = order[i], groups = tiles_of(wv);
+        if (wv == 8 && groups > 2 * units) continue;
+        const int cost = mid_cost(groups, wv, blocks, units);
+        if (best == 0 || cost < best) best = cost, waves = wv;
+      }
     }
     return;
   }
@@ -1349,11 +1420,54 @@ static void choose_mid_shape(int n, int k, GemmTune tune, int& waves, int& split
   waves = pick->waves, splits = pick->splits;
 }
 
-// The shape the kernel for 17..128 rows takes for a matrix of n rows and k columns (for tests and reports).
+// An even deal of the weight rows for a matrix that is not divided along K (see the kernel, EXTRA): workgroups of 4
+// or 8 tiles of 16 rows, `groups` of them (a whole multiple of the compute units), the first `extras` with a tile
+// more.  What a launch costs is taken to be what its busiest compute unit fetches, in tiles: the tiles of its
+// workgroups and, for each of them, the activations once (mid_cost()), and one tile more where there are extras.  Taken
+// where that is a tenth less than for the plain shape (measured on MI355X: 34,816 x 5,120 as 256 workgroups of 8 or 9
+// tiles against 436 of 5: 66 / 68 / 71 us at 32 / 48 / 64 rows against 72 / 77 / 83; 51,200 x 5,120 as 768 of 4 or 5
+// is no better than 400 of 8: 107 / 104 / 113 against 100 / 105 / 110, and is not taken).  Returns false if there is
+// no such deal or it does not pay.
+static bool choose_mid_even(int n, int blocks, GemmTune tune, int plain_waves, int& waves, int& groups, int& extras) {
+  if (tune.even == 1 || blocks > 4) return false;
+  const int units = lrs_compute_units() > 0 ? lrs_compute_units() : 256, tiles = (n + 15) / 16;
+  const int plain_cost = mid_cost((tiles + plain_waves - 1) / plain_waves, plain_waves, blocks, units);
+  int best = 0;
+  for (int rounds = 1; rounds <= 8; ++rounds) {
+    const int g = units * rounds, wv = tiles / g;
+    if (wv != 4 && wv != 8) continue;
+    if (tune.waves && tune.waves != wv) continue;
+    const int more = tiles - g * wv;                        // 0 .. g - 1 workgroups with a tile more
+    const int cost = rounds * (wv + blocks) + (more + units - 1) / units;
+    if (best == 0 || cost < best) best = cost, waves = wv, groups = g, extras = more;
+  }
+  if (best == 0) return false;
+  return tune.even == 2 || 10 * best <= 9 * plain_cost;
+}
+
+// The shape the kernel for 17..128 rows takes for a matrix of n rows and k columns at 49..64 rows (for tests and
+// reports; lrs_gemm_mid_deal() says it for any number of rows).
 LRS_API int lrs_gemm_mid_shape(int n, int k, int tune, int* waves, int* splits) {
   LRS_REQUIRE(n > 0 && k > 0 && k % 256 == 0 && waves && splits, "gemm_mid_shape: needs n > 0 and K %% 256 == 0, got n=%d k=%d", n, k);
   LRS_REQUIRE(tune_ok(tune), "gemm_mid_shape: unknown choices %d", tune);
   choose_mid_shape(n, k, tune_of(tune), *waves, *splits);
+  return 0;
+}
+
+// How the kernel for 17..128 rows deals out a matrix of n rows and k columns for a product of m rows: waves a
+// workgroup, K splits, workgroups along n, and how many of those have a tile of 16 rows more than `waves` (0: the
+// plain deal, every workgroup 16 * waves rows).
+LRS_API int lrs_gemm_mid_deal(int m, int n, int k, int tune, int* waves, int* splits, int* groups, int* extras) {
+  LRS_REQUIRE(m > 16 && m <= 128 && n > 0 && k > 0 && k % 256 == 0 && waves && splits && groups && extras,
+              "gemm_mid_deal: needs 17..128 rows, n > 0 and K %% 256 == 0, got m=%d n=%d k=%d", m, n, k);
+  LRS_REQUIRE(tune_ok(tune), "gemm_mid_deal: unknown choices %d", tune);
+  const int blocks = m <= 32 ? 2 : m <= 48 ? 3 : m <= 64 ? 4 : m <= 96 ? 6 : 8;
+  choose_mid_shape(n, k, tune_of(tune), *waves, *splits, blocks);
+  *groups = (n + 16 * *waves - 1) / (16 * *waves);
+  *extras = 0;
+  int even_waves = 0, even_groups = 0, more = 0;
+  if (*splits == 1 && choose_mid_even(n, blocks, tune_of(tune), *waves, even_waves, even_groups, more))
+    *waves = even_waves, *groups = even_groups, *extras = more;
   return 0;
 }
 
@@ -1362,28 +1476,43 @@ LRS_API int lrs_gemm_mid_shape(int n, int k, int tune, int* waves, int* splits) 
 template <int MT, bool SWIGLU>
 static int launch_mid_mt(void* out, int mode, const bf16* a, const bf16* w, int m, int n, int k, int lda, int ldc, hipStream_t s, GemmTune tune, bool keep_sums, MidScale scale) {
   int waves = 4, splits = 1;
-  choose_mid_shape(n, k, tune, waves, splits);
+  choose_mid_shape(n, k, tune, waves, splits, MT);
   float* sums = splits > 1 || keep_sums ? split_sums_buffer() : nullptr;
   if ((splits > 1 || keep_sums) && (!sums || (size_t)splits * m * n * sizeof(float) > split_sums_bytes())) {
     if (keep_sums) return 0;
     splits = 1, sums = nullptr;
   }
-  const dim3 grid((n + 16 * waves - 1) / (16 * waves), splits);
+  dim3 grid((n + 16 * waves - 1) / (16 * waves), splits);
+  int extras = 0;
+  bool even = false;
+  if constexpr (MT <= 4) {
+    int even_waves = 0, even_groups = 0;
+    if (splits == 1 && choose_mid_even(n, MT, tune, waves, even_waves, even_groups, extras)) {
+      even = true;
+      waves = even_waves;
+      grid = dim3(even_groups, 1);
+    }
+  }
   // dynamic LDS: two activation buffers of 8 x MT KB and 4 KB a wave; more than 64 KB has to be asked for once
-#define MID_LAUNCH(WV)                                                                                              \
+#define MID_LAUNCH(WV, EXTRA)                                                                                       \
   do {                                                                                                              \
     constexpr int bytes = (2 * 8 * MT * 64 + WV * 256) * 16;                                                        \
     static bool asked = false;                                                                                      \
     if (!asked) {                                                                                                   \
-      (void)hipFuncSetAttribute((const void*)gemm_bf16_mid_kernel<MT, WV, SWIGLU>, hipFuncAttributeMaxDynamicSharedMemorySize, bytes); \
+      (void)hipFuncSetAttribute((const void*)gemm_bf16_mid_kernel<MT, WV, SWIGLU, EXTRA>, hipFuncAttributeMaxDynamicSharedMemorySize, bytes); \
       asked = true;                                                                                                 \
     }                                                                                                               \
-    gemm_bf16_mid_kernel<MT, WV, SWIGLU><<<grid, WV * 64, bytes, s>>>(out, mode, a, w, m, n, k, lda, ldc, sums, scale);    \
+    gemm_bf16_mid_kernel<MT, WV, SWIGLU, EXTRA><<<grid, WV * 64, bytes, s>>>(out, mode, a, w, m, n, k, lda, ldc, sums, scale, extras);    \
   } while (0)
-  if (waves == 4) MID_LAUNCH(4);
-  else if (waves == 5) MID_LAUNCH(5);
-  else if (waves == 6) MID_LAUNCH(6);
-  else MID_LAUNCH(8);
+  if constexpr (MT <= 4) {
+    if (even && waves == 4) MID_LAUNCH(4, true);
+    else if (even) MID_LAUNCH(8, true);
+  }
+  if (even) {
+  } else if (waves == 4) MID_LAUNCH(4, false);
+  else if (waves == 5) MID_LAUNCH(5, false);
+  else if (waves == 6) MID_LAUNCH(6, false);
+  else MID_LAUNCH(8, false);
 #undef MID_LAUNCH
   if (splits > 1 && !keep_sums) {
     const int64_t total = (int64_t)m * (SWIGLU ? n / 2 : n);

@@ -115,18 +115,22 @@ def gemm(args) -> None:
                 out = torch.empty(rows, n, device="cuda", dtype=torch.bfloat16)
                 variants = [("own", 0, 0), ("library", 0, 0), ("torch.mm", 0, 0)]
                 if args.mid_sweep and 16 < rows <= 128:
-                    variants = [(f"mid w{wv} s{sp}", wv, sp) for wv in (4, 6, 8) for sp in _ints(args.mid_sweep)] + variants
+                    # every shape with the plain deal of the weight rows; "even": dealt evenly where the shape allows
+                    variants = [(f"mid w{wv} s{sp}", wv, sp) for wv in (4, 5, 6, 8) for sp in _ints(args.mid_sweep)] + [("mid even", 0, 0)] + variants
                 for which, wv, sp in variants:
                     if which == "library":
                         call = lambda i: ops.library_gemm(out, x, weights[i % sets])
                     elif which == "torch.mm":
                         call = lambda i: torch.mm(x, weights[i % sets].t(), out=out)
                     else:
-                        choice = ops.KernelChoice(mid_waves=wv, mid_splits=sp, **base)
+                        choice = ops.KernelChoice(mid_waves=wv, mid_splits=sp, mid_even=2 if which == "mid even" else 1 if which.startswith("mid") else 0, **base)
                         call = lambda i: ops.gemm(out, x, weights[i % sets], choice=choice)
+                    note = ""
+                    if which in ("own", "mid even") and 16 < rows <= 128 and k % 256 == 0:
+                        note = "  %d waves x %d splits, %d workgroups, %d with a tile more" % ops.gemm_mid_deal(rows, n, k, choice)
                     seconds = _time(call, max(args.repeats, 2 * sets))
                     print(f"gemm {name:8s} rows={rows:5d} {which:10s} {seconds * 1e6:9.1f} us  {n * k * 2 / seconds / 1e9:8.0f} GB/s of weights  "
-                          f"{2 * rows * n * k / seconds / 1e12:8.1f} TFLOP/s", flush=True)
+                          f"{2 * rows * n * k / seconds / 1e12:8.1f} TFLOP/s{note}", flush=True)
             del weights
 
 
@@ -230,7 +234,7 @@ def main(argv=None) -> int:
     parser.add_argument("--form", default="0,1,2", help="attention_decode: 0 four waves, 1 four waves with the next tile on the way, 2 eight waves likewise")
     parser.add_argument("--rows", default="1,8,16,64,2048", help="gemm: numbers of rows")
     parser.add_argument("--fragment-loads", action="store_true", help="gemm: the few-rows kernel loads weights and activations as MFMA fragments (64 bytes of 16 rows), not as whole lines")
-    parser.add_argument("--mid-sweep", default="", help="gemm: also time the kernel for 17..128 rows with 4, 6 and 8 waves at these numbers of K splits")
+    parser.add_argument("--mid-sweep", default="", help="gemm: also time the kernel for 17..128 rows with 4, 5, 6 and 8 waves at these numbers of K splits, and with its rows dealt evenly")
     parser.add_argument("--megabytes", default="32,200,1200", help="memory: sizes of the buffers read")
     parser.add_argument("--blocks", default="512,2048,8192", help="memory, lines: numbers of workgroups (lines: try 8,64,256,512)")
     parser.add_argument("--repeats", type=int, default=20)

@@ -38,6 +38,8 @@ class KernelChoice:
                    steps, since from 17 rows on other kernels are faster; the kernels themselves take 64
     mid            the kernel for 17..128 rows may be used
     mid_waves, mid_splits   its workgroup shape (4, 5, 6 or 8 waves) and number of K splits (0: its own choice)
+    mid_even       its weight rows dealt out evenly over a whole multiple of the compute units, some workgroups with
+                   16 rows more than the others: 0 where it pays (its own choice), 1 never, 2 wherever the shape allows
     whole_lines    the few-rows kernel loads its weights as whole 128-byte lines where the shape allows
     library        bfloat16 products of more rows than these kernels are made for go to the vendor's matrix
                    library (as the reference leaves them to nn.Linear); else to this package's own kernel"""
@@ -46,6 +48,7 @@ class KernelChoice:
     mid: bool = True
     mid_waves: int = 0
     mid_splits: int = 0
+    mid_even: int = 0
     whole_lines: bool = True
     library: bool = True
 
@@ -54,11 +57,13 @@ class KernelChoice:
             raise KernelError(f"the few-rows kernel takes 1..64 rows, got few_rows_max={self.few_rows_max}")
         if self.mid_waves not in (0, 4, 5, 6, 8) or not 0 <= self.mid_splits <= 16:
             raise KernelError(f"the kernel for 17..128 rows has 4, 5, 6 or 8 waves and 1..16 K splits (0: its own choice), got {self.mid_waves} and {self.mid_splits}")
+        if self.mid_even not in (0, 1, 2):
+            raise KernelError(f"mid_even is 0 (where it pays), 1 (never) or 2 (wherever the shape allows), got {self.mid_even}")
 
     @property
     def word(self) -> int:
         """The choices a kernel launch needs, as the one integer the entry points take."""
-        return int(self.mid) | int(self.whole_lines) << 1 | self.mid_waves << 4 | self.mid_splits << 8
+        return int(self.mid) | int(self.whole_lines) << 1 | self.mid_waves << 4 | self.mid_splits << 8 | self.mid_even << 13
 
 
 DEFAULT_CHOICE = KernelChoice()
@@ -112,6 +117,7 @@ _SIGNATURES = {
     "lrs_library_gemm": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p]),
     "lrs_host_device_pointer": (c_int, [c_void_p, POINTER(c_void_p)]),
     "lrs_gemm_mid_shape": (c_int, [c_int, c_int, c_int, c_void_p, c_void_p]),
+    "lrs_gemm_mid_deal": (c_int, [c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p]),
     "lrs_gemm_mid_scaled": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_int, c_float, c_int,
                                     c_void_p, c_int64, c_void_p]),
     "lrs_gemm_mid_add_norm_begin": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int,
@@ -563,6 +569,15 @@ def gemm_mid_shape(n: int, k: int, choice: KernelChoice = DEFAULT_CHOICE) -> tup
     waves, splits = c_int(0), c_int(0)
     _check(library().lrs_gemm_mid_shape(n, k, choice.word, ctypes.addressof(waves), ctypes.addressof(splits)))
     return waves.value, splits.value
+
+
+def gemm_mid_deal(m: int, n: int, k: int, choice: KernelChoice = DEFAULT_CHOICE) -> tuple[int, int, int, int]:
+    """(waves a workgroup, K splits, workgroups along n, how many of them have 16 rows more than 16 * waves) for a
+    product of m rows (17..128) with a weight matrix [n, k]."""
+    waves, splits, groups, extras = c_int(0), c_int(0), c_int(0), c_int(0)
+    _check(library().lrs_gemm_mid_deal(m, n, k, choice.word, ctypes.addressof(waves), ctypes.addressof(splits), ctypes.addressof(groups),
+                                       ctypes.addressof(extras)))
+    return waves.value, splits.value, groups.value, extras.value
 
 
 # Rows up to which callers that may use the vendor library take this package's kernel for 17..128 rows instead.

@@ -315,6 +315,55 @@ def test_gemm_of_17_to_64_rows(ops, m, n, k, waves, splits):
     close_in_norm(gated, torch.nn.functional.silu(want[:, :inter]) * want[:, inter:])
 
 
+@pytest.mark.parametrize("m", [17, 33, 48, 64])
+@pytest.mark.parametrize("n,k,deal", [(17984, 512, (4, 256, 100)), (36848, 256, (8, 256, 255)), (37568, 768, (4, 512, 300)), (17976, 512, (4, 256, 100)),
+                                      (34816, 1024, (8, 256, 128))])
+def test_gemm_of_17_to_64_rows_with_rows_dealt_evenly(ops, m, n, k, deal):
+    """The kernel for 17..64 rows with its weight rows dealt out over a whole multiple of the compute units, some
+    workgroups with a tile more than their waves (the extra tile's k steps go round the waves and meet in LDS): every
+    output mode, the gated epilogue, a norm begun before, a ragged last tile; and the same results as the plain deal."""
+    if ops.compute_units() != 256:
+        pytest.skip("the shapes are made for 256 compute units")
+    even, plain_deal = ops.KernelChoice(mid_even=2), ops.KernelChoice(mid_even=1)
+    assert ops.gemm_mid_deal(m, n, k, even) == (deal[0], 1, deal[1], deal[2])
+    assert ops.gemm_mid_deal(m, n, k, plain_deal)[3] == 0
+    g = torch.Generator().manual_seed(m * 7 + n + k)
+    a = torch.randn(m, k, generator=g).bfloat16()
+    w = (torch.randn(n, k, generator=g) / math.sqrt(k)).bfloat16()
+    want = a.double() @ w.double().T
+    sumsq = torch.rand(3, m, generator=g) * k
+    results = {}
+    for name, choice in (("even", even), ("plain", plain_deal)):
+        stored = torch.empty(m, n, device="cuda", dtype=torch.bfloat16)
+        ops.gemm(stored, dev(a), dev(w), choice=choice)
+        wide = torch.full((m, n), 0.5, device="cuda")
+        ops.gemm(wide, dev(a), dev(w), accumulate=True, choice=choice)
+        plain = torch.empty(m, n, device="cuda")
+        ops.gemm(plain, dev(a), dev(w), choice=choice)
+        torch.testing.assert_close(stored.cpu().double(), want, rtol=1e-2, atol=1e-2)
+        torch.testing.assert_close(plain.cpu().double(), want, rtol=1e-4, atol=1e-4)
+        torch.testing.assert_close(wide.cpu().double(), want + 0.5, rtol=1e-4, atol=1e-4)
+        results[name] = [stored.cpu(), plain.cpu()]
+        if n % 16 == 0:
+            inter = n // 2
+            mixed = torch.stack((w[:inter].view(inter // 8, 8, k), w[inter:].view(inter // 8, 8, k)), 1).reshape(n, k).contiguous()
+            gated = torch.empty(m, inter, device="cuda", dtype=torch.bfloat16)
+            ops.gemm(gated, dev(a), dev(mixed), swiglu=True, choice=choice)
+            close_in_norm(gated, torch.nn.functional.silu(want[:, :inter]) * want[:, inter:])
+            # behind a norm that the product before began: rows scaled by the factor of their partial sums of squares
+            eps = 1e-5
+            factor = torch.rsqrt(sumsq.double().sum(0) / k + eps)[:, None]
+            scaled = torch.empty(m, inter, device="cuda", dtype=torch.bfloat16)
+            ops.gemm_mid_scaled(scaled, dev(a), dev(mixed), dev(sumsq), eps, swiglu=True, choice=choice)
+            y = want * factor
+            close_in_norm(scaled, torch.nn.functional.silu(y[:, :inter]) * y[:, inter:], 1e-2)
+            results[name] += [gated.cpu(), scaled.cpu()]
+    # the sums of a column are added in the same order of k either way (slices in turn, steps in turn) only within a
+    # wave; the extra tile's are added wave by wave, so its columns may differ in the last bit of the float32 sum
+    for one, other in zip(results["even"], results["plain"]):
+        torch.testing.assert_close(one.double(), other.double(), rtol=1e-2 if one.dtype == torch.bfloat16 else 1e-5, atol=1e-2 if one.dtype == torch.bfloat16 else 1e-5)
+
+
 @pytest.mark.parametrize("w_dtype", DTYPES)
 @pytest.mark.parametrize("m,n,k", [(512, 4096, 4096), (300, 1024, 3072), (257, 7000, 1088), (129, 512, 8192)])
 def test_product_of_many_rows_with_residual_add_and_norm_in_its_finishing_kernel(ops, w_dtype, m, n, k):
