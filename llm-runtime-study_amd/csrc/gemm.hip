@@ -1387,11 +1387,11 @@ static void choose_mid_shape(int n, int k, GemmTune tune, int& waves, int& split
   // among those whose workgroups still walk four slices or more (down: 8 waves x 8 splits, 6 slices each),
   // else the one with the fewest waves (o_proj: 4 waves x 4 splits); then the fewest splits.
   struct Choice { int waves, splits, len; double fill; };
-  Choice all[24];
+  Choice all[32];
   int count = 0;
   double fullest = -1.0;
-  const int shapes[3] = {4, 6, 8};
-  for (int wi = 0; wi < 3; ++wi) {
+  const int shapes[4] = {4, 5, 6, 8};
+  for (int wi = 0; wi < 4; ++wi) {
     const int wv = shapes[wi];
     if (want_waves && wv != want_waves) continue;
     for (int sp = 1; sp <= 8; ++sp) {
