@@ -458,27 +458,31 @@ def test_small_pool_makes_requests_wait_and_reuses_pages(folders):
     assert 2 <= most_running <= 3 and waited_for_pages and engine.cache_manager.used_pages() == 0
 
 
-@pytest.mark.parametrize("steps_per_launch,ahead", [(1, False), (4, False), (4, True)], ids=["one-step", "four-steps", "four-steps-queued-ahead"])
-def test_many_requests_through_the_scheduler_equal_each_alone(steps_per_launch, ahead):
+@pytest.mark.parametrize("steps_per_launch,ahead,ends", [(1, False, False), (4, False, False), (4, True, False), (4, True, True)],
+                         ids=["one-step", "four-steps", "four-steps-queued-ahead", "queued-ahead-with-ends-of-sequence"])
+def test_many_requests_through_the_scheduler_equal_each_alone(steps_per_launch, ahead, ends):
     """Forty requests of random lengths, two in three greedy and the others with seeded top-k / top-p
     sampling, arriving a few at a time into continuous batching with portions of at most 48 tokens, a
     pool of 40 pages and up to eight running: in float32 every request's tokens are exactly those it
-    produces alone, and the pool is empty at the end."""
+    produces alone, and the pool is empty at the end.  ends: a tenth of the vocabulary ends a sequence, so
+    requests end inside launches while the launch after is already queued."""
     from llm_runtime_study_amd import Engine, SamplingConfig
     from llm_runtime_study_amd.config import config_from_dict
 
-    cfg = config_from_dict(TINY_C)
+    cfg = config_from_dict(dict(TINY_C, eos_token_id=list(range(0, TINY_C["vocab_size"], 10))) if ends else TINY_C)
     rng = np.random.default_rng(5)
     requests = []
     for i in range(40):
         prompt = rng.integers(0, cfg.vocab_size, int(rng.integers(1, 120))).tolist()
         sampling = SamplingConfig() if i % 3 else SamplingConfig(temperature=0.8, top_k=20, top_p=0.9, seed=i)
-        requests.append((prompt, int(rng.integers(1, 40)), sampling))
+        requests.append((prompt, int(rng.integers(1, 40 if not ends else 90)), sampling))
     alone = Engine.from_config(cfg, seed=1, init="scaled", dtype="float32", max_seq_len=256, max_batch_size=1, decode_steps_per_launch=1, launch_ahead=False)
-    want = [alone.generate_tokens([p], max_new_tokens=n, sampling=s, ignore_eos=True)[0] for p, n, s in requests]
+    want = [alone.generate_tokens([p], max_new_tokens=n, sampling=s, ignore_eos=not ends)[0] for p, n, s in requests]
+    if ends:
+        assert sum(len(w) < n for w, (_, n, _) in zip(want, requests)) >= 10     # many do end early
     engine = Engine.from_config(cfg, seed=1, init="scaled", dtype="float32", max_seq_len=256, max_batch_size=8,
                                 max_num_batched_tokens=48, num_pages=40, decode_steps_per_launch=steps_per_launch, launch_ahead=ahead)
-    scheduler = engine.create_scheduler(ignore_eos=True)
+    scheduler = engine.create_scheduler(ignore_eos=not ends)
     got, pending = {}, list(requests)
     with torch.cuda.device(engine.device), torch.cuda.stream(engine.stream):
         while pending or scheduler.has_unfinished:
