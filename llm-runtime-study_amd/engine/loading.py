@@ -82,9 +82,7 @@ def engine_bytes(model: DecoderModel, dtype: torch.dtype, page_size: int, num_pa
 def reserve_device_memory(num_bytes: int, device) -> int:
     """Allocate one tensor of `num_bytes` and a margin (in whole gigabytes) and give it back to torch's allocator,
     which keeps the segment for the allocations that follow.  Returns the bytes reserved (0: nothing; an allocation
-    that does not fit fails cleanly).  Nothing is asked of the device first (its free memory, its size): where such a
-    query was the process's first use of the device and the allocation followed at once, the decode step came out
-    0.5 % slower than with the allocation itself as the first use, every time it was tried; why is not known."""
+    that does not fit fails cleanly)."""
     if num_bytes < RESERVE_AT_LEAST:
         return 0
     num_bytes = -(-(num_bytes + RESERVE_MARGIN) >> 30) << 30
@@ -97,7 +95,11 @@ def reserve_device_memory(num_bytes: int, device) -> int:
 
 
 def reserve_for(config, dtype: torch.dtype, device, page_size: int, num_pages: int) -> int:
-    """reserve_device_memory() for an engine of `config` that is about to be made."""
+    """reserve_device_memory() for an engine of `config` that is about to be made.  The device is initialised before
+    the engine's size is worked out, not by the allocation itself right after it: measured several times over on the
+    MI355X, a process whose first use of the device was followed at once by this allocation ran its decode steps 0.5 %
+    slower than one with a few tenths of a second of host work between the two (3.95 against 3.93 ms); why is not known."""
+    torch.cuda.init()
     return reserve_device_memory(engine_bytes(DecoderModel(spec_for(config)), dtype, page_size, num_pages), device)
 
 
