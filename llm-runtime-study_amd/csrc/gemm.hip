@@ -1346,8 +1346,9 @@ LRS_API int64_t lrs_gemm_workspace_bytes() { return (int64_t)SPLIT_SUMS_BYTES; }
 // fewest splits.
 LRS_API int lrs_compute_units();
 
-// What a launch of `groups` workgroups of `wv` tiles (16 weight rows each) costs: a compute unit fetches at a fixed
-// rate (some 45 GB/s), so the launch takes as long as the unit with the most to fetch: the tiles of its workgroups
+// What a launch of `groups` workgroups of `wv` tiles (16 weight rows each) costs: with every unit busy a compute unit
+// gets some 35-45 GB/s from the L2s (a workgroup all alone on the chip 70-75), so the launch takes as long as the
+// unit with the most to fetch: the tiles of its workgroups
 // and, for each of them, the activations once (`blocks` blocks of 16 tokens: as many bytes as that many tiles).
 static int mid_cost(int groups, int wv, int blocks, int units) { return (groups + units - 1) / units * (wv + blocks); }
 
