@@ -52,6 +52,7 @@ def parse_args():
     parser.add_argument("--top-p", type=float, default=1.0, help="with --temperature: keep the likeliest tokens up to this share of the mass")
     parser.add_argument("--no-graph", action="store_true")
     parser.add_argument("--decode-steps-per-launch", type=int, default=4, help="greedy decode steps run from one graph launch (1: one step a launch)")
+    parser.add_argument("--plain-deal", action="store_true", help="the product for 17..64 rows never deals its weight rows evenly (every workgroup 16 rows a wave)")
     parser.add_argument("--no-reserve", action="store_true", help="let every tensor be an allocation of its own instead of one segment for the engine")
     parser.add_argument("--no-launch-ahead", action="store_true", help="wait for a launch's tokens before the next launch is queued")
     parser.add_argument("--library-mid-gemm", action="store_true", help="products of 17..128 rows through the vendor library instead of this package's kernel for them")
@@ -206,7 +207,7 @@ def main() -> int:
 
     engine = Engine.from_config(config, seed=0, dtype=args.dtype, max_seq_len=max_seq_len, max_batch_size=max_batch,
                                 max_num_batched_tokens=max(2048, args.prefill_tokens), use_cuda_graph=not args.no_graph, num_pages=args.num_pages,
-                                kernels=KernelChoice(library=not args.own_gemm, mid=not args.library_mid_gemm),
+                                kernels=KernelChoice(library=not args.own_gemm, mid=not args.library_mid_gemm, mid_even=1 if args.plain_deal else 0),
                                 decode_steps_per_launch=args.decode_steps_per_launch, launch_ahead=not args.no_launch_ahead,
                                 reserve_memory=not args.no_reserve)
     dtype_name = "bf16" if args.dtype == "bfloat16" else "fp32"

@@ -938,19 +938,20 @@ struct MidScale {
 };
 
 //
-// EXTRA (4 or 8 waves, up to 64 rows): the weight rows are dealt out in tiles of 16 so that every workgroup of the
+// EXTRA (4, 6 or 8 waves, up to 64 rows): the weight rows are dealt out in tiles of 16 so that every workgroup of the
 // launch has WAVES or WAVES + 1 of them (the first `extras` workgroups the one more), which lets a launch be a whole
-// multiple of the compute units whatever n is: a unit fetches at a fixed rate, so the launch takes as long as the
-// unit with the most rows.  The extra tile has no wave of its own: its k steps are dealt out over the waves (one
-// step of a slice each with eight waves, two with four), which multiply them by the activation fragments they hold
-// anyway; the waves' partial sums meet in LDS at the end, are added in wave order and written by the first MT waves.
+// multiple of the compute units whatever n is: the launch takes as long as the unit with the most to fetch.  The
+// extra tile has no wave of its own: its k steps are dealt out over the waves (step s of a slice to wave s % WAVES:
+// one each with eight waves, two with four, one or two with six), which multiply them by the activation fragments
+// they hold anyway; the waves' partial sums meet in LDS at the end, are added in wave order and written by the
+// first MT waves.
 template <int MT, int WAVES, bool SWIGLU, bool EXTRA = false>
 __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_mid_kernel(
     void* __restrict__ out, int mode, const bf16* __restrict__ x, const bf16* __restrict__ w,
     int m, int n, int k, int lda, int ldc, float* __restrict__ split_sums, MidScale scale, int extras) {
-  static_assert(!EXTRA || ((WAVES == 4 || WAVES == 8) && MT <= 4), "the extra tile needs 4 or 8 waves and at most 64 rows");
+  static_assert(!EXTRA || ((WAVES == 4 || WAVES == 6 || WAVES == 8) && MT <= 4), "the extra tile needs 4, 6 or 8 waves and at most 64 rows");
   constexpr int STEPS = 8;                         // k steps of 32 in a slice
-  constexpr int XS = EXTRA ? STEPS / WAVES : 1;    // steps of the extra tile that a wave multiplies in every slice
+  constexpr int XS = EXTRA ? (STEPS + WAVES - 1) / WAVES : 1;    // most steps of the extra tile that a wave multiplies in a slice
   constexpr int FRAGS = STEPS * MT;                // activation fragments of a slice
   constexpr int MINE = (FRAGS + WAVES - 1) / WAVES;  // of which a wave brings this many
   // LDS (dynamic: more than the 64 KB a static array may have): two buffers of activations, then a patch of
@@ -1044,7 +1045,8 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_mid_kernel(
     if constexpr (EXTRA) {
       if (has_extra) {
 #pragma unroll
-        for (int j = 0; j < XS; ++j) xf[j] = *(const bf16x8*)(xl + (int64_t)slice * 256 + j * (WAVES * 32));
+        for (int j = 0; j < XS; ++j)
+          if (STEPS % WAVES == 0 || wave + j * WAVES < STEPS) xf[j] = *(const bf16x8*)(xl + (int64_t)slice * 256 + j * (WAVES * 32));
       }
     }
   };
@@ -1118,8 +1120,10 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_mid_kernel(
   // staging registers into the LDS buffer that slice c - 1 has left, and those of the slices after it are on
   // their way into the staging registers: two sets of them in turn (slices c + 2 and c + 3) up to 64 rows, one
   // set (slice c + 2) beyond, where registers are short.
+  // (six waves with an extra tile at 64 rows have no registers for the second set either)
+  constexpr bool TWO_SETS = MT <= 4 && !(EXTRA && WAVES == 6 && MT == 4);
   int c = 0;
-  if constexpr (MT <= 4) {
+  if constexpr (TWO_SETS) {
     if (count > 0) {
       load_w(slice_at(0), wa);
       load_x(slice_at(0), xa);
@@ -1158,35 +1162,39 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_mid_kernel(
   } else {
     if (count > 0) {
       load_w(slice_at(0), wa);
+      load_x(slice_at(0), xa);
       load_acts(slice_at(0), sa);
     }
-    if (count > 1) load_w(slice_at(1), wb);
+    if (count > 1) {
+      load_w(slice_at(1), wb);
+      load_x(slice_at(1), xb);
+    }
     if (count > 0) store_acts(0, sa);
     if (count > 1) load_acts(slice_at(1), sa);
-    auto steady = [&](int c, bf16x8 (&a)[STEPS]) {
+    auto steady = [&](int c, bf16x8 (&a)[STEPS], bf16x8 (&xf)[XS]) {
       __syncthreads();
       store_acts((c & 1) ^ 1, sa);                       // slice c + 1
       load_acts(slice_at(c + 2), sa);
-      compute(c & 1, a, xa, again, slice_at(c + 2));
+      compute(c & 1, a, xf, again, slice_at(c + 2));
     };
-    auto ending = [&](int c, bf16x8 (&a)[STEPS]) {
+    auto ending = [&](int c, bf16x8 (&a)[STEPS], bf16x8 (&xf)[XS]) {
       __syncthreads();
       if (c + 1 < count) store_acts((c & 1) ^ 1, sa);
       if (c + 2 < count) {
         load_acts(slice_at(c + 2), sa);
-        compute(c & 1, a, xa, again, slice_at(c + 2));
+        compute(c & 1, a, xf, again, slice_at(c + 2));
       } else {
-        compute(c & 1, a, xa, last, 0);
+        compute(c & 1, a, xf, last, 0);
       }
     };
     for (; c + 3 < count; c += 2) {            // no branch inside: slices up to c + 3 exist
-      steady(c, wa);
-      steady(c + 1, wb);
+      steady(c, wa, xa);
+      steady(c + 1, wb, xb);
     }
     for (; c < count; c += 2) {                // the last one to three slices
-      ending(c, wa);
+      ending(c, wa, xa);
       if (c + 1 >= count) break;
-      ending(c + 1, wb);
+      ending(c + 1, wb, xb);
     }
   }
   // accumulator layout: token = t * 16 + lane % 16, weight rows row0 + 4 * (lane / 16) + 0..3
@@ -1421,8 +1429,8 @@ static void choose_mid_shape(int n, int k, GemmTune tune, int& waves, int& split
   waves = pick->waves, splits = pick->splits;
 }
 
-// An even deal of the weight rows for a matrix that is not divided along K (see the kernel, EXTRA): workgroups of 4
-// or 8 tiles of 16 rows, `groups` of them (a whole multiple of the compute units), the first `extras` with a tile
+// An even deal of the weight rows for a matrix that is not divided along K (see the kernel, EXTRA): workgroups of 4,
+// 6 or 8 tiles of 16 rows, `groups` of them (a whole multiple of the compute units), the first `extras` with a tile
 // more.  What a launch costs is taken to be what its busiest compute unit fetches, in tiles: the tiles of its
 // workgroups and, for each of them, the activations once (mid_cost()), and one tile more where there are extras.  Taken
 // where that is a tenth less than for the plain shape (measured on MI355X: 34,816 x 5,120 as 256 workgroups of 8 or 9
@@ -1436,7 +1444,7 @@ static bool choose_mid_even(int n, int blocks, GemmTune tune, int plain_waves, i
   int best = 0;
   for (int rounds = 1; rounds <= 8; ++rounds) {
     const int g = units * rounds, wv = tiles / g;
-    if (wv != 4 && wv != 8) continue;
+    if (wv != 4 && wv != 6 && wv != 8) continue;
     if (tune.waves && tune.waves != wv) continue;
     const int more = tiles - g * wv;                        // 0 .. g - 1 workgroups with a tile more
     const int cost = rounds * (wv + blocks) + (more + units - 1) / units;
@@ -1507,6 +1515,7 @@ static int launch_mid_mt(void* out, int mode, const bf16* a, const bf16* w, int 
   } while (0)
   if constexpr (MT <= 4) {
     if (even && waves == 4) MID_LAUNCH(4, true);
+    else if (even && waves == 6) MID_LAUNCH(6, true);
     else if (even) MID_LAUNCH(8, true);
   }
   if (even) {

@@ -98,11 +98,13 @@ def test_shapes_of_the_kernel_for_17_to_64_rows():
     # 51,200 rows (the 32B feed-forward): 400 workgroups of eight waves, two rounds, fetch least for the busiest unit
     assert ops.gemm_mid_shape(51200, 5120) == (8, 1)
     # the deal of the rows for a given number of rows of the product: the 14B feed-forward evenly, 256 workgroups of 8
-    # tiles of which 128 have a ninth; the others as their shapes say
+    # tiles of which 128 have a ninth; the 32B one 512 of 6, 128 with a seventh; the LM head 1,536 of 6, 280 with a
+    # seventh; those whose rows divide evenly as their shapes say
     for m in (17, 40, 64):
-        assert ops.gemm_mid_deal(m, 34816, 5120) == (8, 1, 256, 128)
-        assert ops.gemm_mid_deal(m, 24576, 4096) == (6, 1, 256, 0) and ops.gemm_mid_deal(m, 51200, 5120) == (8, 1, 400, 0)
-        assert ops.gemm_mid_deal(m, 151936, 4096) == (6, 1, 1583, 0) and ops.gemm_mid_deal(m, 4096, 4096) == (4, 4, 64, 0)
+        assert ops.gemm_mid_deal(m, 34816, 5120) == (8, 1, 256, 128) and ops.gemm_mid_deal(m, 51200, 5120) == (6, 1, 512, 128)
+        assert ops.gemm_mid_deal(m, 24576, 4096) == (6, 1, 256, 0) and ops.gemm_mid_deal(m, 4096, 4096) == (4, 4, 64, 0)
+    assert ops.gemm_mid_deal(64, 151936, 4096) == (6, 1, 1536, 280)
+    assert ops.gemm_mid_deal(64, 51200, 5120, ops.KernelChoice(mid_even=1)) == (8, 1, 400, 0)
     assert ops.gemm_mid_deal(100, 34816, 5120)[3] == 0            # beyond 64 rows the plain deal only
     assert ops.gemm_mid_deal(64, 34816, 5120, ops.KernelChoice(mid_even=1)) == (5, 1, 436, 0)
     for n, k in ((64, 256), (208, 512), (5120, 5120), (5120, 17408), (7168, 5120), (51200, 5120), (1040, 3328)):

@@ -317,7 +317,7 @@ def test_gemm_of_17_to_64_rows(ops, m, n, k, waves, splits):
 
 @pytest.mark.parametrize("m", [17, 33, 48, 64])
 @pytest.mark.parametrize("n,k,deal", [(17984, 512, (4, 256, 100)), (36848, 256, (8, 256, 255)), (37568, 768, (4, 512, 300)), (17976, 512, (4, 256, 100)),
-                                      (34816, 1024, (8, 256, 128))])
+                                      (34816, 1024, (8, 256, 128)), (25808, 512, (6, 256, 77)), (51200, 256, (6, 512, 128))])
 def test_gemm_of_17_to_64_rows_with_rows_dealt_evenly(ops, m, n, k, deal):
     """The kernel for 17..64 rows with its weight rows dealt out over a whole multiple of the compute units, some
     workgroups with a tile more than their waves (the extra tile's k steps go round the waves and meet in LDS): every
