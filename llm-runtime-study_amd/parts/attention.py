@@ -103,6 +103,13 @@ class GQAAttention(Part):
         # to merge (2,048 tokens of context, batch 20 / 24 / 32: 37.8 / 42.0 / 52.7 us undivided against 40.1 / 45 /
         # 54.4 us with the 4 / 3 / 2 parts that two workgroups a unit would ask for; the same at 8,192 tokens)
         wanted = 1 if 8 * workgroups >= 5 * units else -(-2 * units // workgroups)
+        # between one and one and a half workgroups a unit some units have two where the others have one, and with
+        # contexts of 2,048 tokens and more the second round costs more than a merge: two parts (40 query heads on 8:
+        # batch 33 / 40 / 44 / 48 at 2,048 tokens 72.6 / 75.1 / 77.9 / 79.7 us undivided, 66.5 / 71.5 / 73.3 / 78.2 in two parts;
+        # at 4,096 tokens 140 / 144 / 148 / 151 against 122 / 129 / 134 / 144; at 1,024 tokens and from batch 52 on nothing
+        # is gained; four parts are better still up to batch 40 and worse from 44 on, and a graph serves both)
+        if units < workgroups <= units + units // 2 and length_class(longest) >= 2048:
+            wanted = 2
         return max(1, min(wanted, length_class(longest) // 256, 64), -(-bound // (4096 * page_size)))
 
     @staticmethod

@@ -25,7 +25,10 @@ def test_decode_splits_follow_the_class_not_the_length(monkeypatch):
     assert splits(8, 4096, 8192, 16) == 16 and splits(64, 2048, 4096, 16) == 8 and splits(128, 2048, 4096, 16) == 4
     # five workgroups for every eight compute units, or more: not divided
     assert splits(152, 2048, 4096, 16) == 4 and splits(160, 2048, 4096, 16) == 1 and splits(192, 8192, 8192, 16) == 1
-    for workgroups in (1, 8, 24, 64, 200):
+    # between one and one and a half workgroups a unit, from 2,048 tokens of context on: two parts
+    assert splits(256, 4000, 4096, 16) == 1 and splits(264, 4000, 4096, 16) == 2 and splits(384, 2048, 4096, 16) == 2
+    assert splits(385, 4000, 4096, 16) == 1 and splits(384, 2047, 4096, 16) == 1 and splits(512, 4000, 4096, 16) == 1
+    for workgroups in (1, 8, 24, 64, 200, 300):
         for length in range(1, 20000, 501):
             n = splits(workgroups, length, 32768, 16)
             assert n == splits(workgroups, max(length_class(length), 1), 32768, 16)   # the same all over a class
