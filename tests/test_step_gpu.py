@@ -362,6 +362,50 @@ def test_one_layer_at_the_benchmark_sizes_against_the_plain_implementation(sizes
     assert want.abs().max() > 1.0
 
 
+@pytest.mark.parametrize("sizes,batch", [("14b", 40), ("32b", 64), ("8b", 33)])
+def test_decode_steps_of_17_to_64_rows_at_the_benchmark_sizes_against_the_plain_implementation(sizes, batch):
+    """One layer at the sizes of the family's larger models in bfloat16, decode steps of 33..64 requests: the products
+    of 17..64 rows as the runner chooses them there (weight rows dealt evenly over the compute units with an extra
+    tile for some workgroups, K divided for the narrow matrices, the norms taken apart around them) and decode
+    attention over caches of different lengths, against the plain implementation on three slices of the vocabulary."""
+    from llm_runtime_study_amd.cache import CacheManager
+    from llm_runtime_study_amd.config import config_from_dict, spec_for
+    from llm_runtime_study_amd.engine.step import ModelRunner, StepEntry
+    from llm_runtime_study_amd.models import DecoderModel
+    from llm_runtime_study_amd.weights import random_init
+    from tests.test_shape_gpu import LARGER, SHAPE
+
+    raw = dict(SHAPE, num_hidden_layers=1, **LARGER[sizes])
+    cfg = config_from_dict(raw)
+    device = torch.device("cuda", 0)
+    model = DecoderModel(spec_for(cfg))
+    weights = random_init.device_weights(model, 4, torch.bfloat16, device, "scaled")
+    model.bind(weights, torch.bfloat16)
+    cache = CacheManager(model.cache_needs(), page_size=16, num_pages=2 * batch, max_requests=batch, max_seq_len=32, dtype=torch.bfloat16, device=device)
+    runner = ModelRunner(model, cache, max_step_tokens=1024, dtype=torch.bfloat16, device=device)
+    rng = np.random.default_rng(11)
+    prompts = [rng.integers(0, cfg.vocab_size, int(rng.integers(2, 13))).tolist() for _ in range(batch)]
+    decoded = [rng.integers(0, cfg.vocab_size, 3).tolist() for _ in range(batch)]
+    requests = [cache.admit(i) for i in range(batch)]
+    runner.step([StepEntry(r, p, []) for r, p in zip(requests, prompts)])
+    got = [runner.step([StepEntry(r, [d[i]], [0]) for r, d in zip(requests, decoded)]).cpu() for i in range(3)]   # [3][batch, vocab]
+    vocab = cfg.vocab_size
+    columns = torch.cat([torch.arange(0, 500), torch.arange(70000, 70500), torch.arange(vocab - 500, vocab)])
+    used = sorted({t for seq in prompts + decoded for t in seq})
+    small = {name: t.cpu().double() for name, t in weights.items() if name not in ("model.embed_tokens.weight", "lm_head.weight")}
+    small["model.embed_tokens.weight"] = weights["model.embed_tokens.weight"][torch.tensor(used, device=device)].cpu().double()
+    small["lm_head.weight"] = weights["lm_head.weight"][columns.to(device)].cpu().double()
+    worst = 0.0
+    for index, (prompt, more) in enumerate(zip(prompts, decoded)):
+        want = plain.qwen3_forward(small, raw, [used.index(t) for t in prompt + more])
+        for i in range(3):
+            ref, mine = want[len(prompt) + i], got[i][index, columns].double()
+            err = float((mine - ref).norm() / ref.norm())
+            worst = max(worst, err)
+            assert err < 3e-2, f"request {index}, decode step {i}: relative error {err:.3g}"
+    assert worst > 0
+
+
 # ------------------------------------------- launches that follow each other
 @pytest.mark.parametrize("sampled", [False, True], ids=["greedy", "drawn"])
 @pytest.mark.parametrize("dtype", DTYPES)
